@@ -1,0 +1,397 @@
+"""ctypes binding of libferrox_hip.so (see include/ferrox_hip.h) plus a small numpy-facing convenience layer.
+
+The binding is deliberately thin: `lib.fx_<name>` are the raw C entry points with argtypes set; `Context`
+wraps a `fx_ctx*` and offers upload/download and one Python method per kernel family so tests and the
+benchmark read like the C calls they make.  There is no CPU fallback: if the library cannot be loaded the
+import raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libferrox_hip.so")
+
+FX_F32, FX_F64 = 0, 1
+CONV_FWD, CONV_DGRAD, CONV_WGRAD = 0, 1, 2
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "equal": 4, "greater": 5, "greater_equal": 6, "less": 7,
+              "less_equal": 8, "min": 9, "max": 10}
+UNARY_OPS = {"neg": 0, "sqrt": 1, "exp": 2, "log": 3, "relu": 4, "sigmoid": 5, "tanh": 6, "abs": 7, "reciprocal": 8}
+SCALAR_OPS = {"add_scalar": 0, "sub_scalar": 1, "mul_scalar": 2, "div_scalar": 3, "greater_scalar": 4,
+              "greater_equal_scalar": 5, "less_equal_scalar": 6, "less_scalar": 7}
+FX_MAX_BUCKETS = 8
+
+
+class BucketConfig(C.Structure):
+    _fields_ = [("min_elems", C.c_int64), ("max_elems", C.c_int64), ("max_blocks", C.c_int64), ("to_evict", C.c_int64),
+                ("eviction_threshold_ms", C.c_int64)]
+
+
+class PoolConfig(C.Structure):
+    _fields_ = [("n_buckets", C.c_int32), ("literal_ids", C.c_int32), ("buckets", BucketConfig * FX_MAX_BUCKETS)]
+
+
+class PoolStats(C.Structure):
+    _fields_ = [(n, C.c_int64) for n in ("total_allocations", "active_allocations", "pool_hits", "pool_misses",
+                                         "underflow_misses", "allocation_counter", "active_table_len", "device_allocs",
+                                         "device_frees", "bytes_in_use", "bytes_pooled", "peak_bytes")]
+
+    def as_dict(self):
+        return {n: getattr(self, n) for n, _ in self._fields_}
+
+
+class BucketStats(C.Structure):
+    _fields_ = [(n, C.c_int64) for n in ("pooled_blocks", "total_allocations", "total_evictions", "av_allocations",
+                                         "max_allocations")]
+
+    def as_dict(self):
+        return {n: getattr(self, n) for n, _ in self._fields_}
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        from . import build as _build  # build only when nothing is built yet
+        _build.build()
+    return C.CDLL(LIB_PATH)
+
+
+lib = _load()
+
+_vp, _i64, _int, _u64 = C.c_void_p, C.c_int64, C.c_int, C.c_uint64
+
+
+def _sig(name, *argtypes, restype=C.c_int):
+    fn = getattr(lib, name)
+    fn.argtypes = list(argtypes)
+    fn.restype = restype
+    return fn
+
+
+_sig("fx_init", _int, C.POINTER(PoolConfig), C.POINTER(_vp))
+_sig("fx_destroy", _vp)
+_sig("fx_sync", _vp)
+_sig("fx_device_name", _vp, C.c_char_p, _i64)
+_sig("fx_last_error", restype=C.c_char_p)
+_sig("fx_stream", _vp, restype=_vp)
+_sig("fx_timer_start", _vp)
+_sig("fx_timer_stop", _vp, C.POINTER(C.c_float))
+_sig("fx_alloc", _vp, _int, _i64, C.POINTER(_vp), C.POINTER(_i64), C.POINTER(_u64))
+_sig("fx_free", _vp, _int, _vp, _u64)
+_sig("fx_pool_cleanup", _vp, _int)
+_sig("fx_pool_reset", _vp, _int)
+_sig("fx_pool_stats_get", _vp, _int, C.POINTER(PoolStats))
+_sig("fx_pool_bucket_stats_get", _vp, _int, _int, C.POINTER(BucketStats))
+_sig("fx_h2d", _vp, _vp, _vp, _i64)
+_sig("fx_d2h", _vp, _vp, _vp, _i64)
+_sig("fx_d2d", _vp, _vp, _vp, _i64)
+_sig("fx_conv2d_workspace_bytes", _int, _int, _int, *([_i64] * 11), restype=_i64)
+
+_CONV_INTS = [_i64] * 11
+for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
+    _sig(f"fx_fill_{_s}", _vp, _vp, _ct, _i64)
+    _sig(f"fx_materialize_{_s}", _vp, _vp, _vp, C.POINTER(_i64), C.POINTER(_i64), _int, _i64)
+    _sig(f"fx_binary_{_s}", _vp, _int, _vp, _vp, _vp, _i64)
+    for _n in ("add", "sub", "mul", "div", "equal"):
+        _sig(f"fx_{_n}_{_s}", _vp, _vp, _vp, _vp, _i64)
+    _sig(f"fx_scalar_{_s}", _vp, _int, _vp, _ct, _vp, _i64)
+    for _n in ("add_scalar", "sub_scalar", "mul_scalar", "div_scalar", "greater_scalar", "greater_equal_scalar",
+               "less_equal_scalar"):
+        _sig(f"fx_{_n}_{_s}", _vp, _vp, _ct, _vp, _i64)
+    _sig(f"fx_unary_{_s}", _vp, _int, _vp, _vp, _i64)
+    for _n in ("neg", "sqrt", "exp", "log", "relu", "sigmoid", "tanh"):
+        _sig(f"fx_{_n}_{_s}", _vp, _vp, _vp, _i64)
+    _sig(f"fx_clamp_{_s}", _vp, _vp, _ct, _ct, _vp, _i64)
+    _sig(f"fx_relu_bwd_{_s}", _vp, _vp, _vp, _vp, _i64)
+    _sig(f"fx_sigmoid_bwd_{_s}", _vp, _vp, _vp, _vp, _i64, _int)
+    _sig(f"fx_tanh_bwd_{_s}", _vp, _vp, _vp, _vp, _i64)
+    _sig(f"fx_softmax_axis_{_s}", _vp, _vp, _vp, _i64, _i64, _i64)
+    _sig(f"fx_reduce_sum_{_s}", _vp, _vp, _vp, _i64, _i64, _i64)
+    _sig(f"fx_reduce_mean_{_s}", _vp, _vp, _vp, _i64, _i64, _i64)
+    _sig(f"fx_reduce_max_{_s}", _vp, _vp, _vp, _vp, _i64, _i64, _i64)
+    _sig(f"fx_gemm_{_s}", _vp, _int, _int, _i64, _i64, _i64, _vp, _vp, _vp)
+    _sig(f"fx_im2col_{_s}", _vp, _vp, _vp, *([_i64] * 10))
+    _sig(f"fx_col2im_{_s}", _vp, _vp, _vp, *([_i64] * 10), _int)
+    _sig(f"fx_conv2d_fwd_{_s}", _vp, _vp, _vp, _vp, *_CONV_INTS, _vp, _i64)
+    _sig(f"fx_conv2d_dgrad_{_s}", _vp, _vp, _vp, _vp, *_CONV_INTS, _int, _vp, _i64)
+    _sig(f"fx_conv2d_wgrad_{_s}", _vp, _vp, _vp, _vp, *_CONV_INTS, _int, _vp, _i64)
+
+
+class FerroxHipError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"[fx error {code}] {message}")
+        self.code = code
+        self.message = message
+
+
+def check(rc):
+    if rc != 0:
+        raise FerroxHipError(rc, lib.fx_last_error().decode("utf-8", "replace"))
+
+
+def dtype_code(dtype):
+    dtype = np.dtype(dtype)
+    if dtype == np.float32:
+        return FX_F32, "f32"
+    if dtype == np.float64:
+        return FX_F64, "f64"
+    raise TypeError(f"only float32/float64 are supported, got {dtype}")
+
+
+class DeviceArray:
+    """A pool allocation with a shape (row-major).  Returned to the pool by free() or when garbage collected."""
+
+    def __init__(self, ctx, shape, dtype, ptr, granted, alloc_id):
+        self.ctx, self.shape, self.dtype = ctx, tuple(int(s) for s in shape), np.dtype(dtype)
+        self.ptr, self.granted, self.alloc_id = ptr, granted, alloc_id
+
+    @property
+    def size(self):
+        return int(np.prod(self.shape, dtype=np.int64))
+
+    @property
+    def nbytes(self):
+        return self.size * self.dtype.itemsize
+
+    def reshape(self, *shape):
+        shape = shape[0] if len(shape) == 1 and isinstance(shape[0], (tuple, list)) else shape
+        assert int(np.prod(shape, dtype=np.int64)) == self.size
+        v = DeviceArray(self.ctx, shape, self.dtype, self.ptr, self.granted, None)  # non-owning view
+        v._base = self
+        return v
+
+    def numpy(self):
+        out = np.empty(self.shape, dtype=self.dtype)
+        if self.size:
+            check(lib.fx_d2h(self.ctx.h, out.ctypes.data_as(_vp), self.ptr, self.nbytes))
+        return out
+
+    def free(self):
+        if self.alloc_id is not None and self.ptr is not None and self.ctx.h:
+            code, _ = dtype_code(self.dtype)
+            check(lib.fx_free(self.ctx.h, code, self.ptr, self.alloc_id))
+        self.ptr = None
+        self.alloc_id = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Context:
+    def __init__(self, device=0, pool_config=None):
+        h = _vp()
+        check(lib.fx_init(device, C.byref(pool_config) if pool_config is not None else None, C.byref(h)))
+        self.h = h
+
+    def close(self):
+        if self.h:
+            check(lib.fx_destroy(self.h))
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    # ---- runtime ----
+    def sync(self):
+        check(lib.fx_sync(self.h))
+
+    def device_name(self):
+        buf = C.create_string_buffer(256)
+        check(lib.fx_device_name(self.h, buf, 256))
+        return buf.value.decode()
+
+    def timer_start(self):
+        check(lib.fx_timer_start(self.h))
+
+    def timer_stop(self):
+        ms = C.c_float(0)
+        check(lib.fx_timer_stop(self.h, C.byref(ms)))
+        return ms.value
+
+    # ---- memory ----
+    def empty(self, shape, dtype=np.float32):
+        shape = (shape,) if isinstance(shape, (int, np.integer)) else tuple(shape)
+        code, _ = dtype_code(dtype)
+        n = int(np.prod(shape, dtype=np.int64))
+        ptr, granted, aid = _vp(), _i64(0), _u64(0)
+        check(lib.fx_alloc(self.h, code, n, C.byref(ptr), C.byref(granted), C.byref(aid)))
+        return DeviceArray(self, shape, dtype, ptr.value, granted.value, aid.value)
+
+    def upload(self, a):
+        a = np.ascontiguousarray(a)
+        d = self.empty(a.shape, a.dtype)
+        check(lib.fx_h2d(self.h, d.ptr, a.ctypes.data_as(_vp), a.nbytes))
+        return d
+
+    def pool_stats(self, dtype=np.float32):
+        st = PoolStats()
+        check(lib.fx_pool_stats_get(self.h, dtype_code(dtype)[0], C.byref(st)))
+        return st.as_dict()
+
+    def bucket_stats(self, bucket, dtype=np.float32):
+        st = BucketStats()
+        check(lib.fx_pool_bucket_stats_get(self.h, dtype_code(dtype)[0], bucket, C.byref(st)))
+        return st.as_dict()
+
+    def pool_cleanup(self, dtype=np.float32):
+        check(lib.fx_pool_cleanup(self.h, dtype_code(dtype)[0]))
+
+    def pool_reset(self, dtype=np.float32):
+        check(lib.fx_pool_reset(self.h, dtype_code(dtype)[0]))
+
+    # ---- kernels (each allocates its output from the pool unless `out` is given) ----
+    def _fn(self, name, dtype):
+        return getattr(lib, f"fx_{name}_{dtype_code(dtype)[1]}")
+
+    def fill(self, shape, value, dtype=np.float32):
+        o = self.empty(shape, dtype)
+        check(self._fn("fill", dtype)(self.h, o.ptr, float(value), o.size))
+        return o
+
+    def binary(self, op, a, b, out=None):
+        assert a.shape == b.shape, f"Shape mismatch: {a.shape} vs {b.shape}"
+        o = out or self.empty(a.shape, a.dtype)
+        check(self._fn("binary", a.dtype)(self.h, BINARY_OPS[op], a.ptr, b.ptr, o.ptr, a.size))
+        return o
+
+    def scalar(self, op, a, s, out=None):
+        o = out or self.empty(a.shape, a.dtype)
+        check(self._fn("scalar", a.dtype)(self.h, SCALAR_OPS[op], a.ptr, float(s), o.ptr, a.size))
+        return o
+
+    def unary(self, op, a, out=None):
+        o = out or self.empty(a.shape, a.dtype)
+        check(self._fn("unary", a.dtype)(self.h, UNARY_OPS[op], a.ptr, o.ptr, a.size))
+        return o
+
+    def clamp(self, a, lo, hi):
+        o = self.empty(a.shape, a.dtype)
+        check(self._fn("clamp", a.dtype)(self.h, a.ptr, float(lo), float(hi), o.ptr, a.size))
+        return o
+
+    def relu_bwd(self, g, x, out=None):
+        o = out or self.empty(g.shape, g.dtype)
+        check(self._fn("relu_bwd", g.dtype)(self.h, g.ptr, x.ptr, o.ptr, g.size))
+        return o
+
+    def sigmoid_bwd(self, g, s, literal, out=None):
+        o = out or self.empty(g.shape, g.dtype)
+        check(self._fn("sigmoid_bwd", g.dtype)(self.h, g.ptr, s.ptr, o.ptr, g.size, int(literal)))
+        return o
+
+    def tanh_bwd(self, g, t, out=None):
+        o = out or self.empty(g.shape, g.dtype)
+        check(self._fn("tanh_bwd", g.dtype)(self.h, g.ptr, t.ptr, o.ptr, g.size))
+        return o
+
+    def materialize(self, a, shape, strides):
+        n = int(np.prod(shape, dtype=np.int64))
+        o = self.empty(shape, a.dtype)
+        sh = (_i64 * len(shape))(*shape)
+        st = (_i64 * len(shape))(*strides)
+        check(self._fn("materialize", a.dtype)(self.h, a.ptr, o.ptr, sh, st, len(shape), n))
+        return o
+
+    @staticmethod
+    def _oai(shape, axis):
+        outer = int(np.prod(shape[:axis], dtype=np.int64))
+        inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
+        return outer, int(shape[axis]), inner
+
+    def reduce(self, kind, a, axis, want_idx=False, out=None):
+        """kind in sum/mean/max over ONE axis (keep_dims False)."""
+        outer, ax, inner = self._oai(a.shape, axis)
+        oshape = a.shape[:axis] + a.shape[axis + 1:]
+        o = out or self.empty(oshape if oshape else (1,), a.dtype)
+        if kind == "max":
+            idx = None
+            iptr = None
+            if want_idx:
+                idx = _RawI64(self, max(1, outer * inner))
+                iptr = idx.ptr
+            check(self._fn("reduce_max", a.dtype)(self.h, a.ptr, o.ptr, iptr, outer, ax, inner))
+            o.shape = oshape
+            if want_idx:
+                return o, idx.numpy().reshape(oshape)
+            return o
+        check(self._fn("reduce_" + kind, a.dtype)(self.h, a.ptr, o.ptr, outer, ax, inner))
+        o.shape = oshape
+        return o
+
+    def softmax_axis(self, a, axis):
+        outer, ax, inner = self._oai(a.shape, axis)
+        o = self.empty(a.shape, a.dtype)
+        check(self._fn("softmax_axis", a.dtype)(self.h, a.ptr, o.ptr, outer, ax, inner))
+        return o
+
+    def gemm(self, a, b, ta=False, tb=False, out=None):
+        M = a.shape[1] if ta else a.shape[0]
+        K = a.shape[0] if ta else a.shape[1]
+        N = b.shape[0] if tb else b.shape[1]
+        Kb = b.shape[1] if tb else b.shape[0]
+        if K != Kb:
+            raise FerroxHipError(1, f"Matrix multiplication shape mismatch: ({M}, {K}) @ ({Kb}, {N})")
+        o = out or self.empty((M, N), a.dtype)
+        check(self._fn("gemm", a.dtype)(self.h, int(ta), int(tb), M, N, K, a.ptr, b.ptr, o.ptr))
+        return o
+
+    def im2col(self, x, kernel, stride, padding):
+        B, Cc, H, W = x.shape
+        (kh, kw), (sh, sw), (ph, pw) = kernel, stride, padding
+        oh, ow = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+        col = self.empty((Cc * kh * kw, B * oh * ow), x.dtype)
+        check(self._fn("im2col", x.dtype)(self.h, x.ptr, col.ptr, B, Cc, H, W, kh, kw, sh, sw, ph, pw))
+        return col
+
+    def col2im(self, col, out_shape, kernel, stride, padding, layout):
+        B, Cc, H, W = out_shape
+        (kh, kw), (sh, sw), (ph, pw) = kernel, stride, padding
+        o = self.empty(out_shape, col.dtype)
+        check(self._fn("col2im", col.dtype)(self.h, col.ptr, o.ptr, B, Cc, H, W, kh, kw, sh, sw, ph, pw, layout))
+        return o
+
+    def conv2d_fwd(self, x, w, stride, padding, out=None):
+        B, Cin, H, W = x.shape
+        Cout, _, kh, kw = w.shape
+        (sh, sw), (ph, pw) = stride, padding
+        oh, ow = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+        y = out or self.empty((B, Cout, oh, ow), x.dtype)
+        check(self._fn("conv2d_fwd", x.dtype)(self.h, x.ptr, w.ptr, y.ptr, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, None, 0))
+        return y
+
+    def conv2d_dgrad(self, g, w, x_shape, stride, padding, mode=0, out=None):
+        B, Cin, H, W = x_shape
+        Cout, _, kh, kw = w.shape
+        (sh, sw), (ph, pw) = stride, padding
+        dx = out or self.empty(x_shape, g.dtype)
+        check(self._fn("conv2d_dgrad", g.dtype)(self.h, g.ptr, w.ptr, dx.ptr, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, mode,
+                                                None, 0))
+        return dx
+
+    def conv2d_wgrad(self, x, g, w_shape, stride, padding, mode=0, out=None):
+        B, Cin, H, W = x.shape
+        Cout, _, kh, kw = w_shape
+        (sh, sw), (ph, pw) = stride, padding
+        dw = out or self.empty(w_shape, x.dtype)
+        check(self._fn("conv2d_wgrad", x.dtype)(self.h, x.ptr, g.ptr, dw.ptr, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, mode,
+                                                None, 0))
+        return dw
+
+
+class _RawI64:
+    """int64 device buffer (argmax indices); carved from the f64 pool since both are 8-byte elements."""
+
+    def __init__(self, ctx, n):
+        self._a = ctx.empty((n,), np.float64)
+        self.ptr, self.n, self.ctx = self._a.ptr, n, ctx
+
+    def numpy(self):
+        out = np.empty(self.n, dtype=np.int64)
+        check(lib.fx_d2h(self.ctx.h, out.ctypes.data_as(_vp), self.ptr, out.nbytes))
+        return out

@@ -1,0 +1,66 @@
+// Shared internals of libferrox_hip.so: context object, error reporting, launch helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <cstdio>
+#include <mutex>
+#include <string>
+
+#include "../../include/ferrox_hip.h"
+
+typedef int64_t i64;
+
+namespace fx {
+
+struct Pool;  // allocator.hip
+
+void set_error(const char* fmt, ...);
+
+#define FX_HIP_CHECK(expr)                                                                                  \
+    do {                                                                                                    \
+        hipError_t _e = (expr);                                                                             \
+        if (_e != hipSuccess) {                                                                             \
+            fx::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__);       \
+            return FX_ERR_HIP;                                                                              \
+        }                                                                                                   \
+    } while (0)
+
+#define FX_REQUIRE(cond, ...)                                                                               \
+    do {                                                                                                    \
+        if (!(cond)) {                                                                                      \
+            fx::set_error(__VA_ARGS__);                                                                     \
+            return FX_ERR_INVALID;                                                                          \
+        }                                                                                                   \
+    } while (0)
+
+#define FX_CHECK_CTX(ctx) FX_REQUIRE((ctx) != nullptr, "null context")
+
+// Checks the launch itself (bad configuration shows up here, not at the next sync).
+#define FX_LAUNCH_CHECK()                                                                                   \
+    do {                                                                                                    \
+        hipError_t _e = hipGetLastError();                                                                  \
+        if (_e != hipSuccess) {                                                                             \
+            fx::set_error("kernel launch failed: %s (%s:%d)", hipGetErrorString(_e), __FILE__, __LINE__);   \
+            return FX_ERR_HIP;                                                                              \
+        }                                                                                                   \
+    } while (0)
+
+inline i64 ceil_div(i64 a, i64 b) { return (a + b - 1) / b; }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace fx
+
+struct fx_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    std::string name;
+    int num_cus = 0;
+    fx::Pool* pools[2] = {nullptr, nullptr};
+    // library-owned scratch (split-K partials, reduction partials, permuted weights); grows on demand
+    void* scratch = nullptr;
+    i64 scratch_bytes = 0;
+    std::mutex launch_mutex;
+    // returns a scratch region of at least `bytes` (256-byte aligned); nullptr + error on failure
+    void* get_scratch(i64 bytes);
+};

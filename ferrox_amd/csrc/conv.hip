@@ -1,0 +1,232 @@
+// Conv2d forward, data-gradient and weight-gradient as implicit GEMMs on the MFMA pipes.
+//
+// The reference CPU backend builds an explicit im2col matrix (925 MB for N=128,C=64,56x56,k3), multiplies, and
+// transposes or scatters the result (src/backend/storage/extensions/convolutions.rs:218-338); its CUDA backend
+// uses direct kernels (kernels/convolutions.cu).  Here the three passes are GEMMs whose operand loaders do the
+// im2col / col2im index arithmetic while filling LDS, so HBM traffic stays at the tensors themselves:
+//   fwd  : y[b,oc,l]   = sum_{c,ky,kx} w[oc,(c,ky,kx)] * x[b,c,oy*s+ky-p,ox*s+kx-p]   M=Cout N=B*oh*ow K=Cin*kh*kw
+//   dgrad: dx[b,c,p]   = sum_{oc,ky,kx} wt[c,(oc,ky,kx)] * g[b,oc,(y+p-ky)/s,(x+p-kx)/s] M=Cin  N=B*H*W   K=Cout*kh*kw
+//          (gather form of col2im: one accumulator owns each input pixel -> race-free and deterministic)
+//   wgrad: dw[oc,(c,ky,kx)] = sum_{b,l} g[b,oc,l] * x[b,c,...]                         M=Cout N=Cin*kh*kw K=B*oh*ow
+//          (split along K into fixed-order partial sums; no float atomics)
+// mode 1 reproduces the CPU backend's literal arithmetic for the gradients (see include/ferrox_hip.h).
+#include "igemm_core.hpp"
+
+namespace fx {
+int col2im_f32(fx_ctx*, const float*, float*, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, int);
+int col2im_f64(fx_ctx*, const double*, double*, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, int);
+}
+extern "C" int fx_gemm_f32(fx_ctx*, int, int, int64_t, int64_t, int64_t, const float*, const float*, float*);
+extern "C" int fx_gemm_f64(fx_ctx*, int, int, int64_t, int64_t, int64_t, const double*, const double*, double*);
+
+namespace {
+using namespace igemm;
+
+typedef Tile<128, 128, 16, 64, 64> TileM128;  // 4 waves as 2x2, 64x64 each
+typedef Tile<64, 128, 16, 64, 32> TileM64;    // 4 waves as 1x4, 64x32 each
+typedef Tile<32, 256, 16, 32, 64> TileM32;    // 4 waves as 1x4, 32x64 each
+typedef Tile<64, 64, 16, 32, 32> TileSmall;   // 4 waves as 2x2, 32x32 each
+
+int gemm_t(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const float* A, const float* B, float* C) { return fx_gemm_f32(c, ta, tb, M, N, K, A, B, C); }
+int gemm_t(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const double* A, const double* B, double* C) { return fx_gemm_f64(c, ta, tb, M, N, K, A, B, C); }
+int col2im_t(fx_ctx* c, const float* col, float* out, i64 B, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, int layout) { return fx::col2im_f32(c, col, out, B, C, H, W, kh, kw, sh, sw, ph, pw, layout); }
+int col2im_t(fx_ctx* c, const double* col, double* out, i64 B, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, int layout) { return fx::col2im_f64(c, col, out, B, C, H, W, kh, kw, sh, sw, ph, pw, layout); }
+
+struct Dims {
+    i64 B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, oh, ow;
+};
+
+int check_dims(Dims& d, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, const char* what) {
+    FX_REQUIRE(B > 0 && Cin > 0 && H > 0 && W > 0 && Cout > 0 && kh > 0 && kw > 0 && sh > 0 && sw > 0 && ph >= 0 && pw >= 0,
+               "%s: non-positive dimension", what);
+    FX_REQUIRE(H + 2 * ph >= kh && W + 2 * pw >= kw, "%s: kernel larger than padded input", what);
+    FX_REQUIRE(ph < 32768 && pw < 32768 && kh < 32768 && kw < 32768, "%s: kernel/padding too large", what);
+    d = Dims{B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, (H + 2 * ph - kh) / sh + 1, (W + 2 * pw - kw) / sw + 1};
+    const i64 lim = (1ll << 31) - 1;
+    FX_REQUIRE(B * d.oh * d.ow <= lim && B * H * W <= lim && Cin * H * W <= lim && Cout * d.oh * d.ow <= lim &&
+                   Cin * kh * kw <= lim && Cout * kh * kw <= lim,
+               "%s: a GEMM dimension or per-image plane exceeds 2^31-1", what);
+    return FX_OK;
+}
+
+// wt[c][oc*KK + r] = w[oc][c][r]
+template <typename T>
+__global__ __launch_bounds__(256) void permute_weights_kernel(const T* __restrict__ w, T* __restrict__ wt, int Cout, int Cin, int KK) {
+    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+    const i64 n = (i64)Cout * Cin * KK;
+    if (i >= n) return;
+    const int r = (int)(i % KK);
+    const i64 t = i / KK;
+    const int oc = (int)(t % Cout), c = (int)(t / Cout);
+    wt[i] = w[((i64)oc * Cin + c) * KK + r];
+}
+
+template <typename T, class Cfg>
+int fwd_tile(fx_ctx* c, const T* x, const T* w, T* y, const Dims& d) {
+    const i64 M = d.Cout, N = d.B * d.oh * d.ow, K = d.Cin * d.kh * d.kw;
+    const ConvShape s = make_shape(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
+    MatLoader<T, true> al{w, K, (int)M};
+    ConvFwdB<T> bl{x, s, (int)N};
+    NchwStore<T> ep{y, (int)d.Cout, (int)(d.oh * d.ow), (int)N, s.div_L};
+    const int kps = (int)(fx::ceil_div(K, Cfg::BK) * Cfg::BK);
+    return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
+}
+
+template <typename T>
+int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw,
+             i64 ph, i64 pw) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(x && w && y, "fx_conv2d_fwd: null pointer");
+    Dims d;
+    if (int rc = check_dims(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_fwd")) return rc;
+    std::lock_guard<std::mutex> lk(c->launch_mutex);
+    if (Cout > 64) return fwd_tile<T, TileM128>(c, x, w, y, d);
+    if (Cout > 32) return fwd_tile<T, TileM64>(c, x, w, y, d);
+    return fwd_tile<T, TileM32>(c, x, w, y, d);
+}
+
+template <typename T, class Cfg>
+int dgrad_tile(fx_ctx* c, const T* g, const T* wt, T* dx, const Dims& d) {
+    const i64 M = d.Cin, N = d.B * d.H * d.W, K = d.Cout * d.kh * d.kw;
+    const ConvShape s = make_shape(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
+    MatLoader<T, true> al{wt, K, (int)M};
+    ConvDgradB<T> bl{g, s, (int)N};
+    NchwStore<T> ep{dx, (int)d.Cin, (int)(d.H * d.W), (int)N, s.div_HW};
+    const int kps = (int)(fx::ceil_div(K, Cfg::BK) * Cfg::BK);
+    return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
+}
+
+template <typename T>
+i64 dgrad_ws_bytes(const Dims& d, int mode) {
+    if (mode == 1) return d.Cin * d.kh * d.kw * d.B * d.oh * d.ow * (i64)sizeof(T);
+    return d.Cin * d.Cout * d.kh * d.kw * (i64)sizeof(T);
+}
+
+template <typename T>
+int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw,
+               i64 ph, i64 pw, int mode, void* ws, i64 ws_bytes) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(g && w && dx, "fx_conv2d_dgrad: null pointer");
+    FX_REQUIRE(mode == 0 || mode == 1, "fx_conv2d_dgrad: mode must be 0 or 1");
+    Dims d;
+    if (int rc = check_dims(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_dgrad")) return rc;
+    const i64 need = dgrad_ws_bytes<T>(d, mode);
+    FX_REQUIRE(ws == nullptr || ws_bytes >= need, "fx_conv2d_dgrad: workspace of %lld bytes is smaller than the %lld needed",
+               (long long)ws_bytes, (long long)need);
+    if (mode == 1) {
+        // CPU-literal arithmetic: col[K, N] = W2d^T . (g read flat as [Cout, N]); col2im with the batch-major index.
+        const i64 K = Cin * kh * kw, N = B * d.oh * d.ow;
+        T* col = (T*)ws;
+        bool own = false;
+        if (!col) {
+            FX_HIP_CHECK(hipMalloc((void**)&col, (size_t)need));
+            own = true;
+        }
+        int rc = gemm_t(c, 1, 0, K, N, Cout, w, g, col);
+        if (!rc) rc = col2im_t(c, col, dx, B, Cin, H, W, kh, kw, sh, sw, ph, pw, 1);
+        if (own) {
+            (void)hipStreamSynchronize(c->stream);
+            (void)hipFree(col);
+        }
+        return rc;
+    }
+    std::lock_guard<std::mutex> lk(c->launch_mutex);
+    T* wt = (T*)(ws ? ws : c->get_scratch(need));
+    if (!wt) return FX_ERR_OOM;
+    const i64 nw = Cin * Cout * kh * kw;
+    permute_weights_kernel<T><<<dim3((unsigned)fx::ceil_div(nw, 256)), dim3(256), 0, c->stream>>>(w, wt, (int)Cout, (int)Cin, (int)(kh * kw));
+    FX_LAUNCH_CHECK();
+    if (Cin > 64) return dgrad_tile<T, TileM128>(c, g, wt, dx, d);
+    if (Cin > 32) return dgrad_tile<T, TileM64>(c, g, wt, dx, d);
+    return dgrad_tile<T, TileM32>(c, g, wt, dx, d);
+}
+
+template <typename T, class Cfg>
+void wgrad_plan(fx_ctx* c, const Dims& d, int* splits, int* kps) {
+    const i64 M = d.Cout, N = d.Cin * d.kh * d.kw, K = d.B * d.oh * d.ow;
+    const i64 tiles = fx::ceil_div(M, Cfg::BM) * fx::ceil_div(N, Cfg::BN);
+    *splits = choose_splits(tiles, K, Cfg::BK, (i64)(c ? c->num_cus : 256) * 4, kps);
+}
+
+template <typename T, class Cfg>
+int wgrad_tile(fx_ctx* c, const T* x, const T* g, T* dw, const Dims& d, int mode, void* ws) {
+    const i64 M = d.Cout, N = d.Cin * d.kh * d.kw, K = d.B * d.oh * d.ow;
+    const ConvShape s = make_shape(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
+    int splits, kps;
+    wgrad_plan<T, Cfg>(c, d, &splits, &kps);
+    T* part = dw;
+    if (splits > 1) {
+        part = (T*)(ws ? ws : c->get_scratch((i64)splits * M * N * (i64)sizeof(T)));
+        if (!part) return FX_ERR_OOM;
+    }
+    ConvWgradB<T> bl{x, s, (int)N};
+    MatStore<T> ep{part, N, M * N, (int)M, (int)N};
+    int rc;
+    if (mode == 1) {
+        MatLoader<T, true> al{g, K, (int)M};  // g read flat as [Cout, B*L] (convolutions.rs:323-326)
+        rc = launch<T, Cfg>(c, al, bl, ep, M, N, K, splits, kps);
+    } else {
+        ConvWgradA<T> al{g, s};
+        rc = launch<T, Cfg>(c, al, bl, ep, M, N, K, splits, kps);
+    }
+    if (rc || splits == 1) return rc;
+    return launch_splitk_reduce<T>(c, part, dw, M * N, splits);
+}
+
+template <typename T>
+i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d) {
+    int splits, kps;
+    if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64) wgrad_plan<T, TileM128>(c, d, &splits, &kps);
+    else wgrad_plan<T, TileSmall>(c, d, &splits, &kps);
+    return splits > 1 ? (i64)splits * d.Cout * d.Cin * d.kh * d.kw * (i64)sizeof(T) : 0;
+}
+
+template <typename T>
+int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw,
+               i64 ph, i64 pw, int mode, void* ws, i64 ws_bytes) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(x && g && dw, "fx_conv2d_wgrad: null pointer");
+    FX_REQUIRE(mode == 0 || mode == 1, "fx_conv2d_wgrad: mode must be 0 or 1");
+    Dims d;
+    if (int rc = check_dims(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_wgrad")) return rc;
+    const i64 need = wgrad_ws_bytes<T>(c, d);
+    FX_REQUIRE(ws == nullptr || ws_bytes >= need, "fx_conv2d_wgrad: workspace of %lld bytes is smaller than the %lld needed",
+               (long long)ws_bytes, (long long)need);
+    std::lock_guard<std::mutex> lk(c->launch_mutex);
+    if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64) return wgrad_tile<T, TileM128>(c, x, g, dw, d, mode, ws);
+    return wgrad_tile<T, TileSmall>(c, x, g, dw, d, mode, ws);
+}
+
+}  // namespace
+
+extern "C" int64_t fx_conv2d_workspace_bytes(int kind, int dtype, int mode, int64_t B, int64_t Cin, int64_t H, int64_t W,
+                                             int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw) {
+    Dims d;
+    if (check_dims(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_workspace_bytes")) return -1;
+    if (kind == FX_CONV_FWD) return 0;
+    if (kind == FX_CONV_DGRAD) return dtype == FX_F64 ? dgrad_ws_bytes<double>(d, mode) : dgrad_ws_bytes<float>(d, mode);
+    if (kind == FX_CONV_WGRAD) return dtype == FX_F64 ? wgrad_ws_bytes<double>(nullptr, d) : wgrad_ws_bytes<float>(nullptr, d);
+    fx::set_error("fx_conv2d_workspace_bytes: unknown kind %d", kind);
+    return -1;
+}
+
+#define FX_DEFINE_CONV(T, S)                                                                                           \
+    extern "C" int fx_conv2d_fwd_##S(fx_ctx* c, const T* x, const T* w, T* y, int64_t B, int64_t Cin, int64_t H, int64_t W, \
+                                     int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,  \
+                                     void* ws, int64_t ws_bytes) {                                                     \
+        (void)ws; (void)ws_bytes;                                                                                      \
+        return conv_fwd<T>(c, x, w, y, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw);                                    \
+    }                                                                                                                  \
+    extern "C" int fx_conv2d_dgrad_##S(fx_ctx* c, const T* g, const T* w, T* dx, int64_t B, int64_t Cin, int64_t H, int64_t W, \
+                                       int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,   \
+                                       int mode, void* ws, int64_t ws_bytes) {                                         \
+        return conv_dgrad<T>(c, g, w, dx, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, mode, ws, ws_bytes);             \
+    }                                                                                                                  \
+    extern "C" int fx_conv2d_wgrad_##S(fx_ctx* c, const T* x, const T* g, T* dw, int64_t B, int64_t Cin, int64_t H, int64_t W, \
+                                       int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,   \
+                                       int mode, void* ws, int64_t ws_bytes) {                                         \
+        return conv_wgrad<T>(c, x, g, dw, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, mode, ws, ws_bytes);             \
+    }
+
+FX_DEFINE_CONV(float, f32)
+FX_DEFINE_CONV(double, f64)

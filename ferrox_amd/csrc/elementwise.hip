@@ -1,0 +1,318 @@
+// Elementwise kernels (binary, scalar, unary, clamp, fill, fused activation gradients, materialize).
+// Replaces kernels/elementwise.cu, activations.cu (relu/sigmoid/tanh), comparison.cu, fill.cu, materialize.cu
+// of the reference with wave64 streaming kernels: 16-byte vector accesses, four independent vectors in flight per
+// thread, one pass over memory.  HBM-bound: 2 or 3 arrays of n elements per call.
+// Built with floating-point contraction off so composed expressions round op by op like the CPU backend.
+#include "common.hpp"
+
+namespace {
+
+template <typename T> struct Vec16;
+template <> struct Vec16<float> { typedef float4 type; static constexpr int N = 4; };
+template <> struct Vec16<double> { typedef double2 type; static constexpr int N = 2; };
+
+template <typename T> __device__ __forceinline__ T vget(const typename Vec16<T>::type& v, int i);
+template <> __device__ __forceinline__ float vget<float>(const float4& v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+template <> __device__ __forceinline__ double vget<double>(const double2& v, int i) { return i == 0 ? v.x : v.y; }
+template <typename T> __device__ __forceinline__ void vset(typename Vec16<T>::type& v, int i, T x);
+template <> __device__ __forceinline__ void vset<float>(float4& v, int i, float x) { if (i == 0) v.x = x; else if (i == 1) v.y = x; else if (i == 2) v.z = x; else v.w = x; }
+template <> __device__ __forceinline__ void vset<double>(double2& v, int i, double x) { if (i == 0) v.x = x; else v.y = x; }
+
+constexpr int EW_THREADS = 256;
+constexpr int EW_UNROLL = 4;
+
+// NIN = number of input arrays (0, 1 or 2).  F: T operator()(T a, T b).
+template <typename T, int NIN, class F>
+__global__ __launch_bounds__(EW_THREADS) void ew_vec_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                            T* __restrict__ out, i64 nvec, F f) {
+    typedef typename Vec16<T>::type V;
+    constexpr int N = Vec16<T>::N;
+    const V* av = reinterpret_cast<const V*>(a);
+    const V* bv = reinterpret_cast<const V*>(b);
+    V* ov = reinterpret_cast<V*>(out);
+    const i64 base = (i64)blockIdx.x * (EW_THREADS * EW_UNROLL) + threadIdx.x;
+    V ra[EW_UNROLL], rb[EW_UNROLL];
+#pragma unroll
+    for (int j = 0; j < EW_UNROLL; ++j) {
+        const i64 i = base + (i64)j * EW_THREADS;
+        if (i < nvec) {
+            if (NIN >= 1) ra[j] = av[i];
+            if (NIN >= 2) rb[j] = bv[i];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < EW_UNROLL; ++j) {
+        const i64 i = base + (i64)j * EW_THREADS;
+        if (i < nvec) {
+            V r;
+#pragma unroll
+            for (int e = 0; e < N; ++e)
+                vset<T>(r, e, f(NIN >= 1 ? vget<T>(ra[j], e) : T(0), NIN >= 2 ? vget<T>(rb[j], e) : T(0)));
+            ov[i] = r;
+        }
+    }
+}
+
+template <typename T, int NIN, class F>
+__global__ __launch_bounds__(EW_THREADS) void ew_scalar_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                               T* __restrict__ out, i64 begin, i64 n, F f) {
+    const i64 i = begin + (i64)blockIdx.x * EW_THREADS + threadIdx.x;
+    if (i < n) out[i] = f(NIN >= 1 ? a[i] : T(0), NIN >= 2 ? b[i] : T(0));
+}
+
+template <typename T, int NIN, class F>
+int launch_ew(fx_ctx* c, const T* a, const T* b, T* out, i64 n, F f, const char* what) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(n >= 0, "%s: negative element count", what);
+    if (n == 0) return FX_OK;
+    FX_REQUIRE(out != nullptr && (NIN < 1 || a != nullptr) && (NIN < 2 || b != nullptr), "%s: null pointer", what);
+    constexpr int N = Vec16<T>::N;
+    const bool vec_ok = fx::aligned16(out) && (NIN < 1 || fx::aligned16(a)) && (NIN < 2 || fx::aligned16(b));
+    i64 done = 0;
+    if (vec_ok && n >= N) {
+        const i64 nvec = n / N;
+        const i64 blocks = fx::ceil_div(nvec, (i64)EW_THREADS * EW_UNROLL);
+        FX_REQUIRE(blocks <= 0x7fffffff, "%s: too many elements", what);
+        ew_vec_kernel<T, NIN, F><<<dim3((unsigned)blocks), dim3(EW_THREADS), 0, c->stream>>>(a, b, out, nvec, f);
+        FX_LAUNCH_CHECK();
+        done = nvec * N;
+    }
+    if (done < n) {
+        const i64 blocks = fx::ceil_div(n - done, (i64)EW_THREADS);
+        FX_REQUIRE(blocks <= 0x7fffffff, "%s: too many elements", what);
+        ew_scalar_kernel<T, NIN, F><<<dim3((unsigned)blocks), dim3(EW_THREADS), 0, c->stream>>>(a, b, out, done, n, f);
+        FX_LAUNCH_CHECK();
+    }
+    return FX_OK;
+}
+
+// ---- functors -------------------------------------------------------------------------------------------
+template <typename T> __device__ __forceinline__ T dev_exp(T x);
+template <> __device__ __forceinline__ float dev_exp<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ double dev_exp<double>(double x) { return exp(x); }
+template <typename T> __device__ __forceinline__ T dev_log(T x);
+template <> __device__ __forceinline__ float dev_log<float>(float x) { return logf(x); }
+template <> __device__ __forceinline__ double dev_log<double>(double x) { return log(x); }
+template <typename T> __device__ __forceinline__ T dev_sqrt(T x);
+template <> __device__ __forceinline__ float dev_sqrt<float>(float x) { return sqrtf(x); }
+template <> __device__ __forceinline__ double dev_sqrt<double>(double x) { return sqrt(x); }
+
+template <typename T, int OP> struct BinF {
+    __device__ __forceinline__ T operator()(T x, T y) const {
+        if (OP == FX_ADD) return x + y;
+        if (OP == FX_SUB) return x - y;
+        if (OP == FX_MUL) return x * y;
+        if (OP == FX_DIV) return x / y;
+        if (OP == FX_EQUAL) return x == y ? T(1) : T(0);
+        if (OP == FX_GREATER) return x > y ? T(1) : T(0);
+        if (OP == FX_GREATER_EQUAL) return x >= y ? T(1) : T(0);
+        if (OP == FX_LESS) return x < y ? T(1) : T(0);
+        if (OP == FX_LESS_EQUAL) return x <= y ? T(1) : T(0);
+        if (OP == FX_MIN) return x <= y ? x : y;
+        return x >= y ? x : y;  // FX_MAX
+    }
+};
+
+template <typename T, int OP> struct ScalarF {
+    T s;
+    __device__ __forceinline__ T operator()(T x, T) const {
+        if (OP == FX_ADD_SCALAR) return x + s;
+        if (OP == FX_SUB_SCALAR) return x - s;
+        if (OP == FX_MUL_SCALAR) return x * s;
+        if (OP == FX_DIV_SCALAR) return x / s;
+        if (OP == FX_GREATER_SCALAR) return x > s ? T(1) : T(0);
+        if (OP == FX_GREATER_EQUAL_SCALAR) return x >= s ? T(1) : T(0);
+        if (OP == FX_LESS_EQUAL_SCALAR) return x <= s ? T(1) : T(0);
+        return x < s ? T(1) : T(0);  // FX_LESS_SCALAR
+    }
+};
+
+// tanh with the CPU backend's branches (cpu.rs:1108-1147)
+template <typename T> __device__ __forceinline__ T tanh_like_cpu(T x) {
+    if (x > T(20)) return T(1);
+    if (x < T(-20)) return T(-1);
+    if (x >= T(0)) {
+        const T e = dev_exp<T>(-x * T(2));
+        const T num = T(1) - e, den = T(1) + e;
+        return den == T(0) ? T(1) : num / den;
+    }
+    const T e = dev_exp<T>(x * T(2));
+    const T num = e - T(1), den = e + T(1);
+    return den == T(0) ? T(-1) : num / den;
+}
+
+template <typename T, int OP> struct UnaryF {
+    __device__ __forceinline__ T operator()(T x, T) const {
+        if (OP == FX_NEG) return -x;
+        if (OP == FX_SQRT) return dev_sqrt<T>(x);
+        if (OP == FX_EXP) return dev_exp<T>(x);
+        if (OP == FX_LOG) return dev_log<T>(x);
+        if (OP == FX_RELU) return x > T(0) ? x : T(0);
+        if (OP == FX_SIGMOID) return T(1) / (T(1) + dev_exp<T>(-x));
+        if (OP == FX_TANH) return tanh_like_cpu<T>(x);
+        if (OP == FX_ABS) return x < T(0) ? -x : x;
+        return T(1) / x;  // FX_RECIPROCAL
+    }
+};
+
+template <typename T> struct ClampF {
+    T lo, hi;
+    __device__ __forceinline__ T operator()(T x, T) const { return x < lo ? lo : (x > hi ? hi : x); }
+};
+template <typename T> struct FillF {
+    T v;
+    __device__ __forceinline__ T operator()(T, T) const { return v; }
+};
+template <typename T> struct ReluBwdF {  // (g, x)
+    __device__ __forceinline__ T operator()(T g, T x) const { return g * (x > T(0) ? T(1) : T(0)); }
+};
+template <typename T, int LITERAL> struct SigmoidBwdF {  // (g, s)
+    __device__ __forceinline__ T operator()(T g, T s) const {
+        const T t = LITERAL ? (s - T(1)) : (T(1) - s);
+        const T local = s * t;
+        return g * local;
+    }
+};
+template <typename T> struct TanhBwdF {  // (g, t)
+    __device__ __forceinline__ T operator()(T g, T t) const {
+        const T sq = t * t;
+        const T m = sq - T(1);
+        return g * (-m);
+    }
+};
+
+template <typename T>
+int binary_dispatch(fx_ctx* c, int op, const T* a, const T* b, T* o, i64 n) {
+    switch (op) {
+#define CASE(OP) case OP: return launch_ew<T, 2>(c, a, b, o, n, BinF<T, OP>{}, "fx_binary");
+        CASE(FX_ADD) CASE(FX_SUB) CASE(FX_MUL) CASE(FX_DIV) CASE(FX_EQUAL) CASE(FX_GREATER) CASE(FX_GREATER_EQUAL)
+        CASE(FX_LESS) CASE(FX_LESS_EQUAL) CASE(FX_MIN) CASE(FX_MAX)
+#undef CASE
+    }
+    fx::set_error("fx_binary: unknown op %d", op);
+    return FX_ERR_INVALID;
+}
+
+template <typename T>
+int scalar_dispatch(fx_ctx* c, int op, const T* a, T s, T* o, i64 n) {
+    switch (op) {
+#define CASE(OP) case OP: return launch_ew<T, 1>(c, a, (const T*)nullptr, o, n, ScalarF<T, OP>{s}, "fx_scalar");
+        CASE(FX_ADD_SCALAR) CASE(FX_SUB_SCALAR) CASE(FX_MUL_SCALAR) CASE(FX_DIV_SCALAR) CASE(FX_GREATER_SCALAR)
+        CASE(FX_GREATER_EQUAL_SCALAR) CASE(FX_LESS_EQUAL_SCALAR) CASE(FX_LESS_SCALAR)
+#undef CASE
+    }
+    fx::set_error("fx_scalar: unknown op %d", op);
+    return FX_ERR_INVALID;
+}
+
+template <typename T>
+int unary_dispatch(fx_ctx* c, int op, const T* a, T* o, i64 n) {
+    switch (op) {
+#define CASE(OP) case OP: return launch_ew<T, 1>(c, a, (const T*)nullptr, o, n, UnaryF<T, OP>{}, "fx_unary");
+        CASE(FX_NEG) CASE(FX_SQRT) CASE(FX_EXP) CASE(FX_LOG) CASE(FX_RELU) CASE(FX_SIGMOID) CASE(FX_TANH) CASE(FX_ABS)
+        CASE(FX_RECIPROCAL)
+#undef CASE
+    }
+    fx::set_error("fx_unary: unknown op %d", op);
+    return FX_ERR_INVALID;
+}
+
+// ---- materialize: gather a strided / broadcast view into contiguous memory ------------------------------
+struct ViewDesc {
+    int ndim;
+    i64 shape[8];
+    i64 stride[8];
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void materialize_kernel(const T* __restrict__ in, T* __restrict__ out, ViewDesc v, i64 n) {
+    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    i64 r = i, off = 0;
+#pragma unroll
+    for (int d = 7; d >= 0; --d) {
+        if (d < v.ndim) {
+            const i64 q = r / v.shape[d];
+            off += (r - q * v.shape[d]) * v.stride[d];
+            r = q;
+        }
+    }
+    out[i] = in[off];
+}
+
+template <typename T>
+int materialize(fx_ctx* c, const T* in, T* out, const i64* shape, const i64* strides, int ndim, i64 n) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(ndim >= 0 && ndim <= 8, "fx_materialize: ndim %d not in 0..8", ndim);
+    FX_REQUIRE(n >= 0, "fx_materialize: negative element count");
+    if (n == 0) return FX_OK;
+    FX_REQUIRE(in && out && (ndim == 0 || (shape && strides)), "fx_materialize: null pointer");
+    ViewDesc v{};
+    v.ndim = ndim;
+    i64 prod = 1;
+    for (int d = 0; d < ndim; ++d) {
+        FX_REQUIRE(shape[d] > 0 && strides[d] >= 0, "fx_materialize: bad shape/stride at dim %d", d);
+        v.shape[d] = shape[d];
+        v.stride[d] = strides[d];
+        prod *= shape[d];
+    }
+    FX_REQUIRE(prod == n, "fx_materialize: shape product %lld != n %lld", (long long)prod, (long long)n);
+    const i64 blocks = fx::ceil_div(n, 256);
+    FX_REQUIRE(blocks <= 0x7fffffff, "fx_materialize: too many elements");
+    materialize_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(in, out, v, n);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+}  // namespace
+
+#define FX_DEFINE_EW(T, S)                                                                                             \
+    extern "C" int fx_fill_##S(fx_ctx* c, T* out, T v, int64_t n) {                                                    \
+        return launch_ew<T, 0>(c, (const T*)nullptr, (const T*)nullptr, out, n, FillF<T>{v}, "fx_fill");               \
+    }                                                                                                                  \
+    extern "C" int fx_materialize_##S(fx_ctx* c, const T* in, T* out, const int64_t* sh, const int64_t* st, int nd,    \
+                                      int64_t n) {                                                                     \
+        return materialize<T>(c, in, out, sh, st, nd, n);                                                              \
+    }                                                                                                                  \
+    extern "C" int fx_binary_##S(fx_ctx* c, int op, const T* a, const T* b, T* o, int64_t n) {                         \
+        return binary_dispatch<T>(c, op, a, b, o, n);                                                                  \
+    }                                                                                                                  \
+    extern "C" int fx_add_##S(fx_ctx* c, const T* a, const T* b, T* o, int64_t n) { return binary_dispatch<T>(c, FX_ADD, a, b, o, n); } \
+    extern "C" int fx_sub_##S(fx_ctx* c, const T* a, const T* b, T* o, int64_t n) { return binary_dispatch<T>(c, FX_SUB, a, b, o, n); } \
+    extern "C" int fx_mul_##S(fx_ctx* c, const T* a, const T* b, T* o, int64_t n) { return binary_dispatch<T>(c, FX_MUL, a, b, o, n); } \
+    extern "C" int fx_div_##S(fx_ctx* c, const T* a, const T* b, T* o, int64_t n) { return binary_dispatch<T>(c, FX_DIV, a, b, o, n); } \
+    extern "C" int fx_equal_##S(fx_ctx* c, const T* a, const T* b, T* o, int64_t n) { return binary_dispatch<T>(c, FX_EQUAL, a, b, o, n); } \
+    extern "C" int fx_scalar_##S(fx_ctx* c, int op, const T* a, T s, T* o, int64_t n) {                                \
+        return scalar_dispatch<T>(c, op, a, s, o, n);                                                                  \
+    }                                                                                                                  \
+    extern "C" int fx_add_scalar_##S(fx_ctx* c, const T* a, T s, T* o, int64_t n) { return scalar_dispatch<T>(c, FX_ADD_SCALAR, a, s, o, n); } \
+    extern "C" int fx_sub_scalar_##S(fx_ctx* c, const T* a, T s, T* o, int64_t n) { return scalar_dispatch<T>(c, FX_SUB_SCALAR, a, s, o, n); } \
+    extern "C" int fx_mul_scalar_##S(fx_ctx* c, const T* a, T s, T* o, int64_t n) { return scalar_dispatch<T>(c, FX_MUL_SCALAR, a, s, o, n); } \
+    extern "C" int fx_div_scalar_##S(fx_ctx* c, const T* a, T s, T* o, int64_t n) { return scalar_dispatch<T>(c, FX_DIV_SCALAR, a, s, o, n); } \
+    extern "C" int fx_greater_scalar_##S(fx_ctx* c, const T* a, T s, T* o, int64_t n) { return scalar_dispatch<T>(c, FX_GREATER_SCALAR, a, s, o, n); } \
+    extern "C" int fx_greater_equal_scalar_##S(fx_ctx* c, const T* a, T s, T* o, int64_t n) { return scalar_dispatch<T>(c, FX_GREATER_EQUAL_SCALAR, a, s, o, n); } \
+    extern "C" int fx_less_equal_scalar_##S(fx_ctx* c, const T* a, T s, T* o, int64_t n) { return scalar_dispatch<T>(c, FX_LESS_EQUAL_SCALAR, a, s, o, n); } \
+    extern "C" int fx_unary_##S(fx_ctx* c, int op, const T* a, T* o, int64_t n) { return unary_dispatch<T>(c, op, a, o, n); } \
+    extern "C" int fx_neg_##S(fx_ctx* c, const T* a, T* o, int64_t n) { return unary_dispatch<T>(c, FX_NEG, a, o, n); } \
+    extern "C" int fx_sqrt_##S(fx_ctx* c, const T* a, T* o, int64_t n) { return unary_dispatch<T>(c, FX_SQRT, a, o, n); } \
+    extern "C" int fx_exp_##S(fx_ctx* c, const T* a, T* o, int64_t n) { return unary_dispatch<T>(c, FX_EXP, a, o, n); } \
+    extern "C" int fx_log_##S(fx_ctx* c, const T* a, T* o, int64_t n) { return unary_dispatch<T>(c, FX_LOG, a, o, n); } \
+    extern "C" int fx_relu_##S(fx_ctx* c, const T* a, T* o, int64_t n) { return unary_dispatch<T>(c, FX_RELU, a, o, n); } \
+    extern "C" int fx_sigmoid_##S(fx_ctx* c, const T* a, T* o, int64_t n) { return unary_dispatch<T>(c, FX_SIGMOID, a, o, n); } \
+    extern "C" int fx_tanh_##S(fx_ctx* c, const T* a, T* o, int64_t n) { return unary_dispatch<T>(c, FX_TANH, a, o, n); } \
+    extern "C" int fx_clamp_##S(fx_ctx* c, const T* a, T lo, T hi, T* o, int64_t n) {                                  \
+        return launch_ew<T, 1>(c, a, (const T*)nullptr, o, n, ClampF<T>{lo, hi}, "fx_clamp");                          \
+    }                                                                                                                  \
+    extern "C" int fx_relu_bwd_##S(fx_ctx* c, const T* g, const T* x, T* o, int64_t n) {                               \
+        return launch_ew<T, 2>(c, g, x, o, n, ReluBwdF<T>{}, "fx_relu_bwd");                                           \
+    }                                                                                                                  \
+    extern "C" int fx_sigmoid_bwd_##S(fx_ctx* c, const T* g, const T* s, T* o, int64_t n, int literal) {               \
+        return literal ? launch_ew<T, 2>(c, g, s, o, n, SigmoidBwdF<T, 1>{}, "fx_sigmoid_bwd")                         \
+                       : launch_ew<T, 2>(c, g, s, o, n, SigmoidBwdF<T, 0>{}, "fx_sigmoid_bwd");                        \
+    }                                                                                                                  \
+    extern "C" int fx_tanh_bwd_##S(fx_ctx* c, const T* g, const T* t, T* o, int64_t n) {                               \
+        return launch_ew<T, 2>(c, g, t, o, n, TanhBwdF<T>{}, "fx_tanh_bwd");                                           \
+    }
+
+FX_DEFINE_EW(float, f32)
+FX_DEFINE_EW(double, f64)

@@ -1,0 +1,59 @@
+// fx_gemm: C[M,N] = op(A) . op(B) on the MFMA pipes (f32: v_mfma_f32_32x32x2_f32, f64: v_mfma_f64_16x16x4_f64).
+// Replaces kernels/matmul.cu (16x16 shared-memory tiles, 75 % of threads idle) and serves MatMul::compute /
+// MatMul::gradient (src/ops/matrix.rs:17-55) without materialised transposes via the trans flags.
+// Small or skinny products are split along K into deterministic partial sums (no atomics).
+#include "igemm_core.hpp"
+
+namespace {
+using namespace igemm;
+
+typedef Tile<128, 128, 16, 64, 64> TileBig;    // 4 waves, 64x64 each
+typedef Tile<64, 64, 16, 32, 32> TileSmall;    // 4 waves, 32x32 each
+
+template <typename T, class Cfg, bool TA, bool TB>
+int run(fx_ctx* c, i64 M, i64 N, i64 K, const T* A, const T* B, T* C) {
+    // A stored [M,K] (k contiguous) unless TA ([K,M], m contiguous); B stored [K,N] (n contiguous) unless TB ([N,K]).
+    MatLoader<T, !TA> al{A, TA ? M : K, (int)M};
+    MatLoader<T, TB> bl{B, TB ? K : N, (int)N};
+    const i64 tiles = fx::ceil_div(M, Cfg::BM) * fx::ceil_div(N, Cfg::BN);
+    int kps = 0;
+    const int splits = choose_splits(tiles, K, Cfg::BK, (i64)c->num_cus * 2, &kps);
+    if (splits == 1) {
+        MatStore<T> ep{C, N, 0, (int)M, (int)N};
+        return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
+    }
+    T* part = (T*)c->get_scratch((i64)splits * M * N * (i64)sizeof(T));
+    if (!part) return FX_ERR_OOM;
+    MatStore<T> ep{part, N, M * N, (int)M, (int)N};
+    if (int rc = launch<T, Cfg>(c, al, bl, ep, M, N, K, splits, kps)) return rc;
+    return launch_splitk_reduce<T>(c, part, C, M * N, splits);
+}
+
+template <typename T, class Cfg>
+int run_trans(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B, T* C) {
+    if (!ta && !tb) return run<T, Cfg, false, false>(c, M, N, K, A, B, C);
+    if (!ta && tb) return run<T, Cfg, false, true>(c, M, N, K, A, B, C);
+    if (ta && !tb) return run<T, Cfg, true, false>(c, M, N, K, A, B, C);
+    return run<T, Cfg, true, true>(c, M, N, K, A, B, C);
+}
+
+template <typename T>
+int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B, T* C) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(M >= 0 && N >= 0 && K >= 0, "fx_gemm: negative dimension");
+    if (M == 0 || N == 0) return FX_OK;
+    FX_REQUIRE(A && B && C, "fx_gemm: null pointer");
+    FX_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "fx_gemm: dimension exceeds 2^31");
+    std::lock_guard<std::mutex> lk(c->launch_mutex);
+    if (K == 0) return launch_zero<T>(c, C, M * N);  // empty sum
+    if (M >= 128 && N >= 128) return run_trans<T, TileBig>(c, ta, tb, M, N, K, A, B, C);
+    return run_trans<T, TileSmall>(c, ta, tb, M, N, K, A, B, C);
+}
+}  // namespace
+
+extern "C" int fx_gemm_f32(fx_ctx* c, int ta, int tb, int64_t M, int64_t N, int64_t K, const float* A, const float* B, float* C) {
+    return gemm<float>(c, ta, tb, M, N, K, A, B, C);
+}
+extern "C" int fx_gemm_f64(fx_ctx* c, int ta, int tb, int64_t M, int64_t N, int64_t K, const double* A, const double* B, double* C) {
+    return gemm<double>(c, ta, tb, M, N, K, A, B, C);
+}

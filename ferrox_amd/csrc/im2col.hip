@@ -1,0 +1,134 @@
+// Explicit im2col / col2im kernels: the bit-exact-layout path of the convolution
+// (src/backend/storage/extensions/convolutions.rs:10-75 and 79-153).  The fast convolution entry points use an
+// implicit GEMM and never build the column matrix; these kernels serve callers that want the matrix itself and
+// the CPU-literal gradient mode.
+//
+// col2im is written as a GATHER: one thread owns one image pixel and adds the (at most kh*kw) column entries that
+// map to it in ascending (ky, kx) order -- the order in which the reference's scatter loop reaches that pixel --
+// so the result is race-free, deterministic and bit-identical to the CPU.
+#include "common.hpp"
+
+namespace {
+
+struct ConvGeom {
+    i64 B, C, H, W, kh, kw, sh, sw, ph, pw, oh, ow;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void im2col_kernel(const T* __restrict__ x, T* __restrict__ col, ConvGeom g) {
+    const i64 n = (i64)blockIdx.x * 256 + threadIdx.x;  // column = b*oh*ow + oy*ow + ox
+    const i64 row = blockIdx.y;                         // row = c*kh*kw + ky*kw + kx
+    const i64 N = g.B * g.oh * g.ow;
+    if (n >= N) return;
+    const i64 L = g.oh * g.ow;
+    const i64 b = n / L, l = n - b * L;
+    const i64 oy = l / g.ow, ox = l - oy * g.ow;
+    const i64 KK = g.kh * g.kw;
+    const i64 c = row / KK, r = row - c * KK;
+    const i64 ky = r / g.kw, kx = r - ky * g.kw;
+    const i64 iy = oy * g.sh + ky - g.ph, ix = ox * g.sw + kx - g.pw;
+    T v = T(0);
+    if (iy >= 0 && iy < g.H && ix >= 0 && ix < g.W) v = x[((b * g.C + c) * g.H + iy) * g.W + ix];
+    col[row * N + n] = v;
+}
+
+template <typename T, int LAYOUT>
+__global__ __launch_bounds__(256) void col2im_kernel(const T* __restrict__ col, T* __restrict__ out, ConvGeom g) {
+    const i64 idx = (i64)blockIdx.x * 256 + threadIdx.x;  // flat NCHW pixel
+    const i64 total = g.B * g.C * g.H * g.W;
+    if (idx >= total) return;
+    const i64 xw = idx % g.W;
+    i64 t = idx / g.W;
+    const i64 y = t % g.H;
+    t /= g.H;
+    const i64 c = t % g.C;
+    const i64 b = t / g.C;
+    const i64 L = g.oh * g.ow, KK = g.kh * g.kw;
+    const i64 Y = y + g.ph, X = xw + g.pw;  // position in the padded image
+    T acc = T(0);
+    for (i64 ky = 0; ky < g.kh; ++ky) {
+        const i64 ty = Y - ky;
+        if (ty < 0) break;
+        if (ty % g.sh != 0) continue;
+        const i64 cy = ty / g.sh;
+        if (cy >= g.oh) continue;
+        for (i64 kx = 0; kx < g.kw; ++kx) {
+            const i64 tx = X - kx;
+            if (tx < 0) break;
+            if (tx % g.sw != 0) continue;
+            const i64 cx = tx / g.sw;
+            if (cx >= g.ow) continue;
+            i64 ci;
+            if (LAYOUT == 1)
+                ci = b * (g.C * KK * L) + c * (KK * L) + ky * (g.kw * L) + kx * L + cy * g.ow + cx;
+            else
+                ci = (c * KK + ky * g.kw + kx) * (g.B * L) + b * L + cy * g.ow + cx;
+            acc = acc + col[ci];
+        }
+    }
+    out[idx] = acc;
+}
+
+int make_geom(ConvGeom& g, i64 B, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, const char* what) {
+    FX_REQUIRE(B > 0 && C > 0 && H > 0 && W > 0 && kh > 0 && kw > 0 && sh > 0 && sw > 0 && ph >= 0 && pw >= 0,
+               "%s: non-positive dimension", what);
+    FX_REQUIRE(H + 2 * ph >= kh && W + 2 * pw >= kw, "%s: kernel larger than padded input", what);
+    g = ConvGeom{B, C, H, W, kh, kw, sh, sw, ph, pw, (H + 2 * ph - kh) / sh + 1, (W + 2 * pw - kw) / sw + 1};
+    return FX_OK;
+}
+
+template <typename T>
+int im2col(fx_ctx* c, const T* x, T* col, i64 B, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(x && col, "fx_im2col: null pointer");
+    ConvGeom g;
+    if (int rc = make_geom(g, B, C, H, W, kh, kw, sh, sw, ph, pw, "fx_im2col")) return rc;
+    const i64 N = B * g.oh * g.ow, rows = C * kh * kw;
+    FX_REQUIRE(rows <= 65535, "fx_im2col: C*kh*kw = %lld exceeds 65535", (long long)rows);
+    FX_REQUIRE(fx::ceil_div(N, 256) <= 0x7fffffff, "fx_im2col: too many columns");
+    im2col_kernel<T><<<dim3((unsigned)fx::ceil_div(N, 256), (unsigned)rows), dim3(256), 0, c->stream>>>(x, col, g);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+template <typename T>
+int col2im(fx_ctx* c, const T* col, T* out, i64 B, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw,
+           int layout) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(col && out, "fx_col2im: null pointer");
+    FX_REQUIRE(layout == 0 || layout == 1, "fx_col2im: layout must be 0 or 1");
+    ConvGeom g;
+    if (int rc = make_geom(g, B, C, H, W, kh, kw, sh, sw, ph, pw, "fx_col2im")) return rc;
+    const i64 total = B * C * H * W;
+    FX_REQUIRE(fx::ceil_div(total, 256) <= 0x7fffffff, "fx_col2im: too many pixels");
+    const dim3 grid((unsigned)fx::ceil_div(total, 256)), block(256);
+    if (layout == 1) col2im_kernel<T, 1><<<grid, block, 0, c->stream>>>(col, out, g);
+    else col2im_kernel<T, 0><<<grid, block, 0, c->stream>>>(col, out, g);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+}  // namespace
+
+namespace fx {
+// used by the literal-mode data gradient in igemm.hip
+int col2im_f32(fx_ctx* c, const float* col, float* out, i64 B, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, int layout) {
+    return col2im<float>(c, col, out, B, C, H, W, kh, kw, sh, sw, ph, pw, layout);
+}
+int col2im_f64(fx_ctx* c, const double* col, double* out, i64 B, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, int layout) {
+    return col2im<double>(c, col, out, B, C, H, W, kh, kw, sh, sw, ph, pw, layout);
+}
+}  // namespace fx
+
+#define FX_DEFINE_IM2COL(T, S)                                                                                         \
+    extern "C" int fx_im2col_##S(fx_ctx* c, const T* x, T* col, int64_t B, int64_t C, int64_t H, int64_t W, int64_t kh, \
+                                 int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw) {                         \
+        return im2col<T>(c, x, col, B, C, H, W, kh, kw, sh, sw, ph, pw);                                               \
+    }                                                                                                                  \
+    extern "C" int fx_col2im_##S(fx_ctx* c, const T* col, T* out, int64_t B, int64_t C, int64_t H, int64_t W,          \
+                                 int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw, int layout) { \
+        return col2im<T>(c, col, out, B, C, H, W, kh, kw, sh, sw, ph, pw, layout);                                     \
+    }
+
+FX_DEFINE_IM2COL(float, f32)
+FX_DEFINE_IM2COL(double, f64)

@@ -1,0 +1,390 @@
+// Axis reductions (sum / mean / max with first-occurrence argmax) and the axis softmax.
+// Replaces kernels/reduction.cu and softmax_batch_axis of kernels/activations.cu.  The reference launches one
+// 32-lane-shuffle block per output element and walks the axis with stride `inner` (uncoalesced when inner > 1);
+// here every access is a coalesced 16-byte vector and the work is split so that thousands of wave64 blocks are in
+// flight, because these kernels are HBM-bound: sizeof(T) * (outer*axis*inner + outer*inner) bytes per call.
+//
+// Two shapes of the contiguous [outer, axis, inner] view:
+//   inner == 1 : "row" reduction.  grid (S, outer): block (s, o) reduces slice s of row o.
+//   inner  > 1 : "column" reduction.  A wave covers 64 vectors of adjacent columns; the four waves of a block
+//                take interleaved rows of the axis slice; grid (column tiles, S, outer).
+// When the axis is split (S > 1) the per-slice partials go to library scratch and a second small kernel combines
+// them in slice order; no atomics, so results are deterministic run to run.
+// Max takes strictly greater values starting from the lowest finite T (src/backend/storage/cpu.rs:1231-1234);
+// the recorded index is the first position along the axis that attains the maximum.
+#include <limits>
+
+#include "common.hpp"
+
+namespace {
+
+constexpr i64 NO_INDEX = INT64_MAX;
+
+template <typename T> struct Vec16;
+template <> struct Vec16<float> { typedef float4 type; static constexpr int N = 4; };
+template <> struct Vec16<double> { typedef double2 type; static constexpr int N = 2; };
+template <typename T> __device__ __forceinline__ T vget(const typename Vec16<T>::type& v, int i);
+template <> __device__ __forceinline__ float vget<float>(const float4& v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+template <> __device__ __forceinline__ double vget<double>(const double2& v, int i) { return i == 0 ? v.x : v.y; }
+
+template <typename T> __device__ __forceinline__ T lowest();
+template <> __device__ __forceinline__ float lowest<float>() { return -3.402823466e+38f; }
+template <> __device__ __forceinline__ double lowest<double>() { return -1.7976931348623157e+308; }
+
+__device__ __forceinline__ i64 shfl_down_i64(i64 v, int d) {
+    int lo = (int)(v & 0xffffffffll), hi = (int)(v >> 32);
+    lo = __shfl_down(lo, d, 64);
+    hi = __shfl_down(hi, d, 64);
+    return ((i64)hi << 32) | (unsigned int)lo;
+}
+__device__ __forceinline__ double shfl_down_t(double v, int d) { return __shfl_down(v, d, 64); }
+__device__ __forceinline__ float shfl_down_t(float v, int d) { return __shfl_down(v, d, 64); }
+
+// Accumulator: value (+ index when IS_MAX).  Sum ignores idx.
+template <typename T, bool IS_MAX> struct Acc {
+    T v;
+    i64 i;
+    __device__ __forceinline__ void init() { v = IS_MAX ? lowest<T>() : T(0); i = NO_INDEX; }
+    // element x at axis position p, visited in increasing p by this thread
+    __device__ __forceinline__ void take(T x, i64 p) {
+        if (IS_MAX) { if (x > v) { v = x; i = p; } }
+        else v = v + x;
+    }
+    // merge another accumulator (any order): ties go to the smaller index
+    __device__ __forceinline__ void merge(T ov, i64 oi) {
+        if (IS_MAX) { if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; } }
+        else v = v + ov;
+    }
+};
+
+template <typename T, bool IS_MAX>
+__device__ __forceinline__ void wave_reduce(Acc<T, IS_MAX>& a) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        const T ov = shfl_down_t(a.v, d);
+        i64 oi = NO_INDEX;
+        if (IS_MAX) oi = shfl_down_i64(a.i, d);
+        a.merge(ov, oi);
+    }
+}
+
+// ---- row reduction (inner == 1) ---------------------------------------------------------------------------
+// grid (S, outer), 256 threads.  Slice s covers [s*chunk, min(axis, (s+1)*chunk)).  VEC: 16-byte loads (requires
+// axis % N == 0, chunk % N == 0 and a 16-byte aligned base).  Output slot o*S + s.
+template <typename T, bool IS_MAX, bool VEC>
+__global__ __launch_bounds__(256) void row_reduce_kernel(const T* __restrict__ in, T* __restrict__ out, i64* __restrict__ idx_out,
+                                                         i64 axis, i64 chunk, T scale) {
+    constexpr int N = Vec16<T>::N;
+    typedef typename Vec16<T>::type V;
+    const i64 o = blockIdx.y, s = blockIdx.x, S = gridDim.x;
+    const i64 beg = s * chunk, end = min(axis, beg + chunk);
+    const T* row = in + o * axis;
+    Acc<T, IS_MAX> acc;
+    acc.init();
+    if (VEC) {
+        const V* rv = reinterpret_cast<const V*>(row);
+        const i64 vbeg = beg / N, vend = end / N;
+        i64 p = vbeg + threadIdx.x;
+        for (; p + 3 * 256 < vend; p += 4 * 256) {
+            V r0 = rv[p], r1 = rv[p + 256], r2 = rv[p + 512], r3 = rv[p + 768];
+#pragma unroll
+            for (int e = 0; e < N; ++e) acc.take(vget<T>(r0, e), p * N + e);
+#pragma unroll
+            for (int e = 0; e < N; ++e) acc.take(vget<T>(r1, e), (p + 256) * N + e);
+#pragma unroll
+            for (int e = 0; e < N; ++e) acc.take(vget<T>(r2, e), (p + 512) * N + e);
+#pragma unroll
+            for (int e = 0; e < N; ++e) acc.take(vget<T>(r3, e), (p + 768) * N + e);
+        }
+        for (; p < vend; p += 256) {
+            V r0 = rv[p];
+#pragma unroll
+            for (int e = 0; e < N; ++e) acc.take(vget<T>(r0, e), p * N + e);
+        }
+    } else {
+        for (i64 p = beg + threadIdx.x; p < end; p += 256) acc.take(row[p], p);
+    }
+    wave_reduce(acc);
+    __shared__ T sv[4];
+    __shared__ i64 si[4];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) { sv[wave] = acc.v; si[wave] = acc.i; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        Acc<T, IS_MAX> r;
+        r.v = sv[0]; r.i = si[0];
+        for (int w = 1; w < 4; ++w) r.merge(sv[w], si[w]);
+        const i64 slot = o * S + s;
+        out[slot] = IS_MAX ? r.v : r.v * scale;
+        if (IS_MAX && idx_out) idx_out[slot] = (S == 1 && r.i == NO_INDEX) ? 0 : r.i;
+    }
+}
+
+// Short rows: G = power of two >= axis lanes per row (G <= 64), 64/G rows per wave, 4 waves per block.
+template <typename T, bool IS_MAX>
+__global__ __launch_bounds__(256) void short_row_reduce_kernel(const T* __restrict__ in, T* __restrict__ out,
+                                                               i64* __restrict__ idx_out, i64 outer, i64 axis, int G, T scale) {
+    const int lane = threadIdx.x & 63;
+    const i64 rows_per_block = (256 / G);
+    const i64 o = (i64)blockIdx.x * rows_per_block + threadIdx.x / G;
+    const int a = threadIdx.x % G;
+    Acc<T, IS_MAX> acc;
+    acc.init();
+    if (o < outer && a < axis) acc.take(in[o * axis + a], a);
+    for (int d = G >> 1; d >= 1; d >>= 1) {
+        const T ov = shfl_down_t(acc.v, d);
+        i64 oi = NO_INDEX;
+        if (IS_MAX) oi = shfl_down_i64(acc.i, d);
+        if ((lane % G) + d < G) acc.merge(ov, oi);
+    }
+    if (a == 0 && o < outer) {
+        out[o] = IS_MAX ? acc.v : acc.v * scale;
+        if (IS_MAX && idx_out) idx_out[o] = acc.i == NO_INDEX ? 0 : acc.i;
+    }
+}
+
+// Combine S slice partials per output: one wave per output element, slices merged with the tie rule.
+template <typename T, bool IS_MAX>
+__global__ __launch_bounds__(256) void combine_rows_kernel(const T* __restrict__ pv, const i64* __restrict__ pi, T* __restrict__ out,
+                                                           i64* __restrict__ idx_out, i64 n_out, i64 S, T scale) {
+    const i64 o = (i64)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (o >= n_out) return;
+    Acc<T, IS_MAX> acc;
+    acc.init();
+    for (i64 s = lane; s < S; s += 64) acc.merge(pv[o * S + s], IS_MAX && pi ? pi[o * S + s] : NO_INDEX);
+    wave_reduce(acc);
+    if (lane == 0) {
+        out[o] = IS_MAX ? acc.v : acc.v * scale;
+        if (IS_MAX && idx_out) idx_out[o] = acc.i == NO_INDEX ? 0 : acc.i;
+    }
+}
+
+// ---- column reduction (inner > 1) -------------------------------------------------------------------------
+// grid (col tiles, S, outer), 256 threads = 4 waves.  A wave covers 64*NV adjacent columns (NV = N when VEC else 1);
+// wave w takes axis positions beg + w, beg + w + 4, ...  Output slot ((o*S + s) * inner + col).
+// FROM_PARTIAL: the input is a partial array whose index values come from `pidx` instead of the axis position.
+template <typename T, bool IS_MAX, bool VEC, bool FROM_PARTIAL>
+__global__ __launch_bounds__(256) void col_reduce_kernel(const T* __restrict__ in, const i64* __restrict__ pidx, T* __restrict__ out,
+                                                         i64* __restrict__ idx_out, i64 axis, i64 inner, i64 chunk, T scale,
+                                                         int final_pass) {
+    constexpr int N = VEC ? Vec16<T>::N : 1;
+    typedef typename Vec16<T>::type V;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const i64 col = ((i64)blockIdx.x * 64 + lane) * N;
+    const i64 s = blockIdx.y, S = gridDim.y, o = blockIdx.z;
+    const i64 beg = s * chunk, end = min(axis, beg + chunk);
+    Acc<T, IS_MAX> acc[N];
+#pragma unroll
+    for (int e = 0; e < N; ++e) acc[e].init();
+    if (col < inner) {
+        const T* base = in + (o * axis) * inner + col;
+        const i64* ibase = FROM_PARTIAL && IS_MAX ? pidx + (o * axis) * inner + col : nullptr;
+        i64 a = beg + wave;
+        if (VEC && !FROM_PARTIAL) {
+            for (; a + 12 < end; a += 16) {
+                V r0 = *reinterpret_cast<const V*>(base + a * inner);
+                V r1 = *reinterpret_cast<const V*>(base + (a + 4) * inner);
+                V r2 = *reinterpret_cast<const V*>(base + (a + 8) * inner);
+                V r3 = *reinterpret_cast<const V*>(base + (a + 12) * inner);
+#pragma unroll
+                for (int e = 0; e < N; ++e) {
+                    acc[e].take(vget<T>(r0, e), a);
+                    acc[e].take(vget<T>(r1, e), a + 4);
+                    acc[e].take(vget<T>(r2, e), a + 8);
+                    acc[e].take(vget<T>(r3, e), a + 12);
+                }
+            }
+            for (; a < end; a += 4) {
+                V r0 = *reinterpret_cast<const V*>(base + a * inner);
+#pragma unroll
+                for (int e = 0; e < N; ++e) acc[e].take(vget<T>(r0, e), a);
+            }
+        } else {
+            for (; a < end; a += 4) {
+#pragma unroll
+                for (int e = 0; e < N; ++e) {
+                    const T x = base[a * inner + e];
+                    if (FROM_PARTIAL) acc[e].merge(x, IS_MAX ? ibase[a * inner + e] : NO_INDEX);
+                    else acc[e].take(x, a);
+                }
+            }
+        }
+    }
+    __shared__ T sv[4][64 * N];
+    __shared__ i64 si[IS_MAX ? 4 : 1][IS_MAX ? 64 * N : 1];
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+        sv[wave][lane * N + e] = acc[e].v;
+        if (IS_MAX) si[wave][lane * N + e] = acc[e].i;
+    }
+    __syncthreads();
+    if (wave == 0 && col < inner) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+            Acc<T, IS_MAX> r;
+            r.v = sv[0][lane * N + e];
+            r.i = IS_MAX ? si[0][lane * N + e] : NO_INDEX;
+            for (int w = 1; w < 4; ++w) r.merge(sv[w][lane * N + e], IS_MAX ? si[w][lane * N + e] : NO_INDEX);
+            const i64 slot = (o * S + s) * inner + col + e;
+            out[slot] = IS_MAX ? r.v : r.v * scale;
+            if (IS_MAX && idx_out) idx_out[slot] = (final_pass && r.i == NO_INDEX) ? 0 : r.i;
+        }
+    }
+}
+
+template <typename T, bool IS_MAX>
+int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i64 inner, T scale, const char* what) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(outer >= 0 && axis >= 1 && inner >= 0, "%s: bad view [%lld, %lld, %lld]", what, (long long)outer,
+               (long long)axis, (long long)inner);
+    if (outer == 0 || inner == 0) return FX_OK;
+    FX_REQUIRE(in && out, "%s: null pointer", what);
+    FX_REQUIRE(outer <= 65535 * 1024ll, "%s: outer too large", what);
+    constexpr int N = Vec16<T>::N;
+    const bool want_idx = IS_MAX && idx_out != nullptr;
+    std::lock_guard<std::mutex> lk(c->launch_mutex);
+    const i64 target_blocks = (i64)c->num_cus * 8;
+
+    if (inner == 1) {
+        if (axis <= 64 && outer >= 1) {
+            int G = 1;
+            while (G < axis) G <<= 1;
+            const i64 rows_per_block = 256 / G;
+            const i64 blocks = fx::ceil_div(outer, rows_per_block);
+            FX_REQUIRE(blocks <= 0x7fffffff, "%s: too many rows", what);
+            short_row_reduce_kernel<T, IS_MAX><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(in, out, idx_out, outer, axis, G, scale);
+            FX_LAUNCH_CHECK();
+            return FX_OK;
+        }
+        FX_REQUIRE(outer <= 65535, "%s: more than 65535 long rows; reshape so that the reduced axis is not the last", what);
+        // slices: enough blocks to fill the chip, each at least 16 KiB, slice length a multiple of 1024 elements
+        i64 S = 1;
+        if (outer < target_blocks) {
+            S = std::min<i64>(fx::ceil_div(target_blocks, outer), std::max<i64>(1, axis / 4096));
+            S = std::min<i64>(S, 65535);
+        }
+        i64 chunk = fx::ceil_div(axis, S);
+        chunk = fx::ceil_div(chunk, 1024) * 1024;
+        S = fx::ceil_div(axis, chunk);
+        const bool vec = fx::aligned16(in) && (axis % N == 0);
+        T* pv = out;
+        i64* pi = idx_out;
+        if (S > 1) {
+            const i64 bytes = outer * S * (i64)(sizeof(T) + sizeof(i64));
+            char* sc = (char*)c->get_scratch(bytes);
+            if (!sc) return FX_ERR_OOM;
+            pi = (i64*)sc;
+            pv = (T*)(sc + outer * S * sizeof(i64));
+        }
+        const dim3 grid((unsigned)S, (unsigned)outer), block(256);
+        const T sc1 = S > 1 ? T(1) : scale;
+        i64* io = (S > 1 && IS_MAX) ? pi : idx_out;
+        if (vec) row_reduce_kernel<T, IS_MAX, true><<<grid, block, 0, c->stream>>>(in, pv, io, axis, chunk, sc1);
+        else row_reduce_kernel<T, IS_MAX, false><<<grid, block, 0, c->stream>>>(in, pv, io, axis, chunk, sc1);
+        FX_LAUNCH_CHECK();
+        if (S > 1) {
+            combine_rows_kernel<T, IS_MAX><<<dim3((unsigned)fx::ceil_div(outer, 4)), dim3(256), 0, c->stream>>>(
+                pv, IS_MAX ? pi : nullptr, out, idx_out, outer, S, scale);
+            FX_LAUNCH_CHECK();
+        }
+        (void)want_idx;
+        return FX_OK;
+    }
+
+    // column reduction
+    FX_REQUIRE(outer <= 65535, "%s: outer %lld exceeds 65535 for a column reduction", what, (long long)outer);
+    const bool vec = fx::aligned16(in) && (inner % N == 0);
+    const i64 cols_per_block = 64 * (vec ? N : 1);
+    const i64 tiles = fx::ceil_div(inner, cols_per_block);
+    FX_REQUIRE(tiles <= 0x7fffffff, "%s: inner too large", what);
+    i64 S = 1;
+    if (tiles * outer < target_blocks) {
+        S = std::min<i64>(fx::ceil_div(target_blocks, tiles * outer), std::max<i64>(1, axis / 32));
+        S = std::min<i64>(S, 65535);
+    }
+    i64 chunk = fx::ceil_div(axis, S);
+    chunk = fx::ceil_div(chunk, 4) * 4;
+    S = fx::ceil_div(axis, chunk);
+    if (S == 1) {
+        const dim3 grid((unsigned)tiles, 1, (unsigned)outer), block(256);
+        if (vec) col_reduce_kernel<T, IS_MAX, true, false><<<grid, block, 0, c->stream>>>(in, nullptr, out, idx_out, axis, inner, chunk, scale, 1);
+        else col_reduce_kernel<T, IS_MAX, false, false><<<grid, block, 0, c->stream>>>(in, nullptr, out, idx_out, axis, inner, chunk, scale, 1);
+        FX_LAUNCH_CHECK();
+        return FX_OK;
+    }
+    const i64 n_part = outer * S * inner;
+    const i64 bytes = n_part * (i64)(sizeof(T) + (IS_MAX ? sizeof(i64) : 0)) + 256;
+    char* sc = (char*)c->get_scratch(bytes);
+    if (!sc) return FX_ERR_OOM;
+    i64* pi = IS_MAX ? (i64*)sc : nullptr;
+    T* pv = (T*)(sc + (IS_MAX ? ((n_part * sizeof(i64) + 255) / 256) * 256 : 0));
+    {
+        const dim3 grid((unsigned)tiles, (unsigned)S, (unsigned)outer), block(256);
+        if (vec) col_reduce_kernel<T, IS_MAX, true, false><<<grid, block, 0, c->stream>>>(in, nullptr, pv, pi, axis, inner, chunk, T(1), 0);
+        else col_reduce_kernel<T, IS_MAX, false, false><<<grid, block, 0, c->stream>>>(in, nullptr, pv, pi, axis, inner, chunk, T(1), 0);
+        FX_LAUNCH_CHECK();
+    }
+    {
+        // second pass over [outer, S, inner] partials; scalar columns so that many blocks share the work
+        const i64 tiles2 = fx::ceil_div(inner, 64);
+        const dim3 grid((unsigned)tiles2, 1, (unsigned)outer), block(256);
+        col_reduce_kernel<T, IS_MAX, false, true><<<grid, block, 0, c->stream>>>(pv, pi, out, idx_out, S, inner, fx::ceil_div(S, 4) * 4, scale, 1);
+        FX_LAUNCH_CHECK();
+    }
+    return FX_OK;
+}
+
+// ---- softmax over the middle axis: cpu.rs:1037-1068 -----------------------------------------------------
+template <typename T> __device__ __forceinline__ T dev_exp(T x);
+template <> __device__ __forceinline__ float dev_exp<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ double dev_exp<double>(double x) { return exp(x); }
+
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_axis_kernel(const T* __restrict__ in, T* __restrict__ out, i64 outer, i64 axis, i64 inner) {
+    const i64 t = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (t >= outer * inner) return;
+    const i64 o = t / inner, i = t - o * inner;
+    const T* p = in + o * axis * inner + i;
+    T* q = out + o * axis * inner + i;
+    T m = lowest<T>();
+    for (i64 a = 0; a < axis; ++a) { const T x = p[a * inner]; if (x > m) m = x; }
+    T s = T(0);
+    for (i64 a = 0; a < axis; ++a) { const T e = dev_exp<T>(p[a * inner] - m); q[a * inner] = e; s = s + e; }
+    for (i64 a = 0; a < axis; ++a) q[a * inner] = q[a * inner] / s;
+}
+
+template <typename T>
+int softmax_axis(fx_ctx* c, const T* in, T* out, i64 outer, i64 axis, i64 inner) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(outer >= 0 && axis >= 1 && inner >= 0, "fx_softmax_axis: bad view");
+    if (outer == 0 || inner == 0) return FX_OK;
+    FX_REQUIRE(in && out, "fx_softmax_axis: null pointer");
+    FX_REQUIRE(in != out, "fx_softmax_axis: in-place not supported");
+    const i64 blocks = fx::ceil_div(outer * inner, 256);
+    FX_REQUIRE(blocks <= 0x7fffffff, "fx_softmax_axis: too many rows");
+    softmax_axis_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(in, out, outer, axis, inner);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+}  // namespace
+
+#define FX_DEFINE_REDUCE(T, S)                                                                                         \
+    extern "C" int fx_reduce_sum_##S(fx_ctx* c, const T* in, T* out, int64_t outer, int64_t axis, int64_t inner) {     \
+        return reduce<T, false>(c, in, out, nullptr, outer, axis, inner, T(1), "fx_reduce_sum");                       \
+    }                                                                                                                  \
+    extern "C" int fx_reduce_mean_##S(fx_ctx* c, const T* in, T* out, int64_t outer, int64_t axis, int64_t inner) {    \
+        FX_REQUIRE(axis >= 1, "fx_reduce_mean: empty axis");                                                           \
+        return reduce<T, false>(c, in, out, nullptr, outer, axis, inner, (T)(1.0 / (double)axis), "fx_reduce_mean");   \
+    }                                                                                                                  \
+    extern "C" int fx_reduce_max_##S(fx_ctx* c, const T* in, T* out, int64_t* idx, int64_t outer, int64_t axis,        \
+                                     int64_t inner) {                                                                  \
+        return reduce<T, true>(c, in, out, idx, outer, axis, inner, T(1), "fx_reduce_max");                            \
+    }                                                                                                                  \
+    extern "C" int fx_softmax_axis_##S(fx_ctx* c, const T* in, T* out, int64_t outer, int64_t axis, int64_t inner) {   \
+        return softmax_axis<T>(c, in, out, outer, axis, inner);                                                        \
+    }
+
+FX_DEFINE_REDUCE(float, f32)
+FX_DEFINE_REDUCE(double, f64)

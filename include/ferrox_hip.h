@@ -1,0 +1,224 @@
+/*
+ * ferrox_hip.h -- C ABI of libferrox_hip.so, the MI355X (gfx950) backend for Ferrox's training hot path.
+ *
+ * This is the boundary a `HipStorage<T>: StorageBackend<T>` implementation binds through FFI.  It replaces,
+ * one for one, what the reference reaches through cudarc:
+ *   - CudaContextManager  (src/backend/cuda/context.rs:30-175)   -> fx_init / fx_destroy / fx_sync / copies
+ *   - CudaMemoryPool      (src/backend/memory/cuda.rs:55-134)    -> fx_alloc / fx_free / fx_pool_*
+ *   - KernelManager::launch_* (src/backend/cuda/kernels.rs:435-1918) -> the fx_<op>_{f32,f64} kernel entry points
+ *
+ * Conventions
+ *   - Every function returns an int status: FX_OK (0) or an FX_ERR_* code; the message of the last failure on
+ *     the calling thread is available from fx_last_error().
+ *   - All tensor pointers are DEVICE pointers unless the parameter is named host_*.  Sizes and counts are
+ *     int64_t ELEMENTS unless named *_bytes.  Shapes are row-major (C order), exactly as Ferrox stores them.
+ *   - Every kernel is enqueued on the context's single compute stream and returns without waiting; call
+ *     fx_sync() (or a device-to-host copy, which waits) before reading results on the host.
+ *   - Memory handed out by the pool is NOT zeroed on reuse (as in the reference, context.rs:72-73); every
+ *     kernel here fully defines its output.
+ *   - A context may be used from several host threads; allocator calls are serialised internally and launches
+ *     are serialised per context.
+ *   - dtype suffixes: _f32 = float, _f64 = double.  The reference names its kernels `op` / `op_f64`
+ *     (src/backend/cuda/kernels.rs:283-292).
+ */
+#ifndef FERROX_HIP_H
+#define FERROX_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FX_OK 0
+#define FX_ERR_INVALID 1     /* bad argument / shape mismatch */
+#define FX_ERR_HIP 2         /* a HIP runtime call failed */
+#define FX_ERR_OOM 3         /* device allocation failed */
+#define FX_ERR_UNSUPPORTED 4 /* valid request this build does not serve */
+
+#define FX_F32 0
+#define FX_F64 1
+
+typedef struct fx_ctx fx_ctx;
+
+/* ---- allocator configuration: PoolConfig / BucketConfig, src/backend/memory/mod.rs:15-82 ---------------- */
+#define FX_MAX_BUCKETS 8
+typedef struct fx_bucket_config {
+    int64_t min_elems;              /* inclusive */
+    int64_t max_elems;              /* inclusive; INT64_MAX for "no limit" */
+    int64_t max_blocks;             /* max_allocations */
+    int64_t to_evict;               /* blocks dropped at once when the bucket is full (LRU) */
+    int64_t eviction_threshold_ms;  /* >= 0: evict blocks older than this instead of LRU; < 0: none */
+} fx_bucket_config;
+
+typedef struct fx_pool_config {
+    int32_t n_buckets;   /* 0 = PoolConfig::default() (mod.rs:50-82) */
+    int32_t literal_ids; /* 1 = keep the reference's id bookkeeping (a reused block keeps its old id, so its second
+                            release is dropped, cuda.rs:61-62,76-87); 0 = a reused block is re-registered (default) */
+    fx_bucket_config buckets[FX_MAX_BUCKETS];
+} fx_pool_config;
+
+/* PoolStats, src/backend/memory/mod.rs:195-202, plus what print_stats derives (cuda.rs:138-185) */
+typedef struct fx_pool_stats {
+    int64_t total_allocations;
+    int64_t active_allocations;
+    int64_t pool_hits;
+    int64_t pool_misses;
+    int64_t underflow_misses;
+    int64_t allocation_counter; /* CudaMemoryPool::allocation_counter */
+    int64_t active_table_len;   /* active_allocations.len() */
+    int64_t device_allocs;      /* hipMalloc calls made for this pool */
+    int64_t device_frees;       /* hipFree calls made for this pool */
+    int64_t bytes_in_use;       /* bytes currently handed out */
+    int64_t bytes_pooled;       /* bytes cached in buckets */
+    int64_t peak_bytes;         /* high-water mark of in_use + pooled */
+} fx_pool_stats;
+
+/* BucketStats, src/backend/memory/mod.rs:204-222 */
+typedef struct fx_bucket_stats {
+    int64_t pooled_blocks;
+    int64_t total_allocations;
+    int64_t total_evictions;
+    int64_t av_allocations;
+    int64_t max_allocations;
+} fx_bucket_stats;
+
+/* ---- runtime: CudaContextManager::{from_device_id, synchronize, name}, context.rs:35-59, 152-172 -------- */
+int fx_init(int device, const fx_pool_config* cfg_or_null, fx_ctx** out);
+int fx_destroy(fx_ctx* ctx);
+int fx_sync(fx_ctx* ctx);
+int fx_device_name(fx_ctx* ctx, char* buf, int64_t buf_len);
+const char* fx_last_error(void);
+/* The compute stream as a hipStream_t (for callers that enqueue their own work behind the library's). */
+void* fx_stream(fx_ctx* ctx);
+
+/* Stream timing for benchmarks (the reference times with cudaEvent pairs, kernels/benchmark.cu:575-603):
+ * fx_timer_start records an event on the compute stream, fx_timer_stop records a second one, waits for it and
+ * returns the elapsed milliseconds between the two. */
+int fx_timer_start(fx_ctx* ctx);
+int fx_timer_stop(fx_ctx* ctx, float* elapsed_ms);
+
+/* ---- allocator: CudaMemoryPool::{allocate, deallocate, cleanup, reset, stats}, memory/cuda.rs:55-134 ----- */
+/* n_elems == 0 -> FX_ERR_INVALID "Cannot allocate zero-sized CUDA memory" (cuda.rs:57-59).
+ * *granted_elems may exceed n_elems on a pool hit (the reference truncates on read-back, context.rs:410-426). */
+int fx_alloc(fx_ctx* ctx, int dtype, int64_t n_elems, void** ptr, int64_t* granted_elems, uint64_t* alloc_id);
+int fx_free(fx_ctx* ctx, int dtype, void* ptr, uint64_t alloc_id);
+int fx_pool_cleanup(fx_ctx* ctx, int dtype);
+int fx_pool_reset(fx_ctx* ctx, int dtype);
+int fx_pool_stats_get(fx_ctx* ctx, int dtype, fx_pool_stats* out);
+int fx_pool_bucket_stats_get(fx_ctx* ctx, int dtype, int bucket, fx_bucket_stats* out);
+
+/* ---- copies: host_to_device / device_to_host / device_to_device, context.rs:81-150 (synchronous) -------- */
+int fx_h2d(fx_ctx* ctx, void* dst_dev, const void* host_src, int64_t bytes);
+int fx_d2h(fx_ctx* ctx, void* host_dst, const void* src_dev, int64_t bytes);
+int fx_d2d(fx_ctx* ctx, void* dst_dev, const void* src_dev, int64_t bytes);
+
+/* ---- workspace queries ---------------------------------------------------------------------------------- */
+#define FX_CONV_FWD 0
+#define FX_CONV_DGRAD 1
+#define FX_CONV_WGRAD 2
+/* Bytes of scratch fx_conv2d_* needs for this shape.  Passing workspace == NULL to the conv entry points makes
+ * the library use (and grow) its own per-context scratch instead. */
+int64_t fx_conv2d_workspace_bytes(int kind, int dtype, int mode, int64_t B, int64_t Cin, int64_t H, int64_t W,
+                                  int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw);
+
+/* Binary / scalar / unary op selectors for the generic entry points (also exported one by one below). */
+enum fx_binary_op { FX_ADD = 0, FX_SUB = 1, FX_MUL = 2, FX_DIV = 3, FX_EQUAL = 4, FX_GREATER = 5, FX_GREATER_EQUAL = 6,
+                    FX_LESS = 7, FX_LESS_EQUAL = 8, FX_MIN = 9, FX_MAX = 10 };
+enum fx_unary_op { FX_NEG = 0, FX_SQRT = 1, FX_EXP = 2, FX_LOG = 3, FX_RELU = 4, FX_SIGMOID = 5, FX_TANH = 6, FX_ABS = 7,
+                   FX_RECIPROCAL = 8 };
+enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_DIV_SCALAR = 3, FX_GREATER_SCALAR = 4,
+                    FX_GREATER_EQUAL_SCALAR = 5, FX_LESS_EQUAL_SCALAR = 6, FX_LESS_SCALAR = 7 };
+
+#define FX_DECLARE_KERNELS(T, S)                                                                                       \
+    /* launch_fill, kernels.rs:435-448 */                                                                              \
+    int fx_fill_##S(fx_ctx* ctx, T* out, T value, int64_t n);                                                          \
+    /* launch_materialize, kernels.rs:802-830 / CudaOps::materialize, ops.rs:175-214.  shape and strides (in          \
+       elements, 0 on broadcast dims) are HOST arrays, ndim <= 8. */                                                   \
+    int fx_materialize_##S(fx_ctx* ctx, const T* in, T* out, const int64_t* host_shape, const int64_t* host_strides,   \
+                           int ndim, int64_t n);                                                                       \
+    /* launch_add/sub/mul/div/min/max + comparisons, kernels.rs:469-585, 940-1075.  Same-shape operands only           \
+       (cpu.rs:629-690).  Comparisons write 1.0 / 0.0.  a/0 follows IEEE like the CPU backend. */                      \
+    int fx_binary_##S(fx_ctx* ctx, int op, const T* a, const T* b, T* out, int64_t n);                                 \
+    int fx_add_##S(fx_ctx* ctx, const T* a, const T* b, T* out, int64_t n);                                            \
+    int fx_sub_##S(fx_ctx* ctx, const T* a, const T* b, T* out, int64_t n);                                            \
+    int fx_mul_##S(fx_ctx* ctx, const T* a, const T* b, T* out, int64_t n);                                            \
+    int fx_div_##S(fx_ctx* ctx, const T* a, const T* b, T* out, int64_t n);                                            \
+    int fx_equal_##S(fx_ctx* ctx, const T* a, const T* b, T* out, int64_t n);                                          \
+    /* scalar ops, CudaOps::{add,sub,mul,div}_scalar ops.rs:435-464 (the reference fills a full-size temp first;       \
+       here the scalar is a kernel argument) and launch_*_scalar, kernels.rs:954-1010 */                               \
+    int fx_scalar_##S(fx_ctx* ctx, int op, const T* a, T s, T* out, int64_t n);                                        \
+    int fx_add_scalar_##S(fx_ctx* ctx, const T* a, T s, T* out, int64_t n);                                            \
+    int fx_sub_scalar_##S(fx_ctx* ctx, const T* a, T s, T* out, int64_t n);                                            \
+    int fx_mul_scalar_##S(fx_ctx* ctx, const T* a, T s, T* out, int64_t n);                                            \
+    int fx_div_scalar_##S(fx_ctx* ctx, const T* a, T s, T* out, int64_t n);                                            \
+    int fx_greater_scalar_##S(fx_ctx* ctx, const T* a, T s, T* out, int64_t n);                                        \
+    int fx_greater_equal_scalar_##S(fx_ctx* ctx, const T* a, T s, T* out, int64_t n);                                  \
+    int fx_less_equal_scalar_##S(fx_ctx* ctx, const T* a, T s, T* out, int64_t n);                                     \
+    /* unary ops, kernels.rs:587-740 (abs, sqrt, exp, log, negate, sigmoid, tanh, relu).  tanh saturates to +-1        \
+       beyond |x| > 20 like cpu.rs:1112-1119. */                                                                       \
+    int fx_unary_##S(fx_ctx* ctx, int op, const T* a, T* out, int64_t n);                                              \
+    int fx_neg_##S(fx_ctx* ctx, const T* a, T* out, int64_t n);                                                        \
+    int fx_sqrt_##S(fx_ctx* ctx, const T* a, T* out, int64_t n);                                                       \
+    int fx_exp_##S(fx_ctx* ctx, const T* a, T* out, int64_t n);                                                        \
+    int fx_log_##S(fx_ctx* ctx, const T* a, T* out, int64_t n);                                                        \
+    int fx_relu_##S(fx_ctx* ctx, const T* a, T* out, int64_t n);                                                       \
+    int fx_sigmoid_##S(fx_ctx* ctx, const T* a, T* out, int64_t n);                                                    \
+    int fx_tanh_##S(fx_ctx* ctx, const T* a, T* out, int64_t n);                                                       \
+    /* launch_clamp, kernels.rs:894-917 / cpu.rs:792-805 */                                                            \
+    int fx_clamp_##S(fx_ctx* ctx, const T* a, T lo, T hi, T* out, int64_t n);                                          \
+    /* Fused activation gradients.  The reference has no backward kernels: ReLU::gradient, Sigmoid::gradient and       \
+       Tanh::gradient (src/ops/unary.rs:358-375, 254-276, 306-328) compose 2-4 storage ops.  These produce the         \
+       same values in one pass: relu: g*(x>0); tanh: g*(-(t*t-1)); sigmoid: literal=1 -> g*(s*(s-1)) (the              \
+       reference's sign), literal=0 -> g*(s*(1-s)). */                                                                 \
+    int fx_relu_bwd_##S(fx_ctx* ctx, const T* g, const T* x, T* out, int64_t n);                                       \
+    int fx_sigmoid_bwd_##S(fx_ctx* ctx, const T* g, const T* s, T* out, int64_t n, int literal);                       \
+    int fx_tanh_bwd_##S(fx_ctx* ctx, const T* g, const T* t, T* out, int64_t n);                                       \
+    /* launch_softmax_batched, kernels.rs:683-711 / cpu.rs:1037-1068: softmax over `axis` of [outer, axis, inner] */   \
+    int fx_softmax_axis_##S(fx_ctx* ctx, const T* in, T* out, int64_t outer, int64_t axis, int64_t inner);             \
+    /* launch_sum_axes / launch_max_axes / launch_*_all, kernels.rs:742-800; CudaOps::reduce_axes ops.rs:2171-2284;    \
+       cpu.rs:1183-1238.  Reduces the middle dimension of a contiguous [outer, axis, inner] view into                  \
+       [outer, inner]; "all" = (1, n, 1).  mean multiplies the sum by T(1/axis) (cpu.rs:1217-1220).  max starts        \
+       from the lowest finite T and takes strictly greater values (cpu.rs:1231-1234); idx_out (may be NULL)            \
+       receives the FIRST index along the axis that attains the maximum, as int64. */                                  \
+    int fx_reduce_sum_##S(fx_ctx* ctx, const T* in, T* out, int64_t outer, int64_t axis, int64_t inner);               \
+    int fx_reduce_mean_##S(fx_ctx* ctx, const T* in, T* out, int64_t outer, int64_t axis, int64_t inner);              \
+    int fx_reduce_max_##S(fx_ctx* ctx, const T* in, T* out, int64_t* idx_out, int64_t outer, int64_t axis,             \
+                          int64_t inner);                                                                              \
+    /* launch_matmul, kernels.rs:919-938 / cpu.rs:967-1002: C[M,N] = op(A) . op(B).  trans_a: A is stored [K,M];       \
+       trans_b: B is stored [N,K]  (lets MatMul::gradient, src/ops/matrix.rs:30-55, skip materialised transposes). */  \
+    int fx_gemm_##S(fx_ctx* ctx, int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const T* A, const T* B,    \
+                    T* C);                                                                                             \
+    /* im2col / col2im, src/backend/storage/extensions/convolutions.rs:10-75, 79-153.                                  \
+       col is [C*kh*kw, B*oh*ow] row-major.  col2im layout 0 reads it that way; layout 1 reads the buffer with the     \
+       reference's batch-major flat index (convolutions.rs:122-127).  The sum for each pixel runs over (ky, kx)        \
+       ascending, the reference's loop order, so results are bit-identical to the CPU. */                              \
+    int fx_im2col_##S(fx_ctx* ctx, const T* x, T* col, int64_t B, int64_t C, int64_t H, int64_t W, int64_t kh,         \
+                      int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw);                                     \
+    int fx_col2im_##S(fx_ctx* ctx, const T* col, T* out, int64_t B, int64_t C, int64_t H, int64_t W, int64_t kh,       \
+                      int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw, int layout);                         \
+    /* launch_conv2d_forward / launch_deconv2d / launch_cross_correlation2d, kernels.rs:1213-1256, 1340-1384,          \
+       1386-1430; CPU path convolutions.rs:218-338.  NCHW.  oh = (H+2ph-kh)/sh+1.                                      \
+       fwd:   y[B,Cout,oh,ow]   = conv(x[B,Cin,H,W], w[Cout,Cin,kh,kw])                                                \
+       dgrad: dx[B,Cin,H,W]     from g[B,Cout,oh,ow], w                                                                \
+       wgrad: dw[Cout,Cin,kh,kw] from x, g                                                                             \
+       mode 0 = the mathematical gradient (what the reference's CUDA kernels compute); mode 1 = the CPU backend's      \
+       literal arithmetic (flat reinterpretation of g as [Cout, B*L] and batch-major col2im), which equals mode 0       \
+       only for batch 1. */                                                                                            \
+    int fx_conv2d_fwd_##S(fx_ctx* ctx, const T* x, const T* w, T* y, int64_t B, int64_t Cin, int64_t H, int64_t W,     \
+                          int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,        \
+                          void* workspace, int64_t ws_bytes);                                                          \
+    int fx_conv2d_dgrad_##S(fx_ctx* ctx, const T* g, const T* w, T* dx, int64_t B, int64_t Cin, int64_t H, int64_t W,  \
+                            int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,      \
+                            int mode, void* workspace, int64_t ws_bytes);                                              \
+    int fx_conv2d_wgrad_##S(fx_ctx* ctx, const T* x, const T* g, T* dw, int64_t B, int64_t Cin, int64_t H, int64_t W,  \
+                            int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,      \
+                            int mode, void* workspace, int64_t ws_bytes);
+
+FX_DECLARE_KERNELS(float, f32)
+FX_DECLARE_KERNELS(double, f64)
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FERROX_HIP_H */

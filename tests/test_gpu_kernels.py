@@ -1,0 +1,336 @@
+"""GPU parity tests: every kernel family of libferrox_hip.so, called through the C ABI, against the CPU oracle
+on the same seeded inputs.  Bit-exact where the arithmetic order is defined (data movement, elementwise
+compositions, max/argmax); rel 1e-5 (f32) / 1e-12 (f64) against a float64/longdouble ground truth elsewhere."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [np.float32, np.float64]
+TOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float64): 1e-12}
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from ferrox_amd import capi
+    c = capi.Context(0)
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def orc():
+    import oracle
+    return oracle
+
+
+def rel_err(got, ref):
+    ref = np.asarray(ref, dtype=np.float64)
+    return np.abs(np.asarray(got, dtype=np.float64) - ref).max() / max(1e-30, np.abs(ref).max())
+
+
+# ------------------------------------------------------------------------------------------ elementwise
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n", [1, 3, 4, 1023, 1024, 4099, 1 << 20])
+def test_binary_ops_bit_exact(ctx, orc, dtype, n):
+    rng = np.random.default_rng(n)
+    a = rng.uniform(-4, 4, n).astype(dtype)
+    b = rng.uniform(-4, 4, n).astype(dtype)
+    b[::7] = a[::7]  # exercise equality
+    da, db = ctx.upload(a), ctx.upload(b)
+    for op in ("add", "sub", "mul", "div", "equal", "greater", "greater_equal", "less", "less_equal", "min", "max"):
+        got = ctx.binary(op, da, db).numpy()
+        assert np.array_equal(got, orc.binary(op, a, b)), op
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_division_by_zero_follows_ieee_like_cpu(ctx, orc, dtype):
+    a = np.array([1.0, -1.0, 0.0, 2.0], dtype)
+    b = np.array([0.0, 0.0, 0.0, 4.0], dtype)
+    got = ctx.binary("div", ctx.upload(a), ctx.upload(b)).numpy()
+    with np.errstate(all="ignore"):
+        ref = orc.binary("div", a, b)
+    assert np.array_equal(got, ref, equal_nan=True)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_scalar_and_clamp_bit_exact(ctx, orc, dtype):
+    rng = np.random.default_rng(11)
+    a = rng.uniform(-4, 4, 70001).astype(dtype)
+    da = ctx.upload(a)
+    for op, s in (("add_scalar", 1.5), ("sub_scalar", 1.0), ("mul_scalar", 0.01), ("div_scalar", 3.0), ("greater_scalar", 0.0),
+                  ("greater_equal_scalar", 1e-8), ("less_equal_scalar", 0.5), ("less_scalar", 0.0)):
+        assert np.array_equal(ctx.scalar(op, da, s).numpy(), orc.scalar(op, a, dtype(s))), op
+    lo, hi = dtype(1e-8), dtype(1.0 - 1e-8)
+    assert np.array_equal(ctx.clamp(da, lo, hi).numpy(), orc.clamp(a, lo, hi))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_unary_ops(ctx, orc, dtype):
+    rng = np.random.default_rng(12)
+    a = rng.uniform(-4, 4, 100003).astype(dtype)
+    a[:6] = [0.0, -0.0, 25.0, -25.0, 1000.0, -1000.0]
+    da = ctx.upload(a)
+    pos = ctx.upload(np.abs(a) + dtype(1e-3))
+    for op in ("neg", "relu", "abs"):  # exact ops
+        assert np.array_equal(ctx.unary(op, da).numpy(), orc.unary(op, a)), op
+    for op in ("exp", "sigmoid", "tanh"):  # libm vs device math: elementwise relative tolerance
+        with np.errstate(over="ignore"):
+            ref = orc.unary(op, a.astype(np.float64)).astype(dtype)  # overflow to inf exactly where T overflows
+        # tanh's exp-based formula (cpu.rs:1120-1146) cancels near 0 in T on CPU and GPU alike: allow a few ulp of 1.0
+        atol = 4 * np.finfo(dtype).eps if op == "tanh" else 0
+        np.testing.assert_allclose(ctx.unary(op, da).numpy(), ref, rtol=TOL[np.dtype(dtype)] * 4, atol=atol, err_msg=op)
+    for op in ("sqrt", "log", "reciprocal"):
+        ref = orc.unary(op, (np.abs(a) + dtype(1e-3)).astype(np.float64))
+        assert rel_err(ctx.unary(op, pos).numpy(), ref) <= TOL[np.dtype(dtype)] * 4, op
+    # saturation like the CPU backend (tensor.rs:2667-2729): exactly +-1 beyond |x| > 20, sigmoid -> 0 / 1
+    t = ctx.unary("tanh", da).numpy()
+    assert t[2] == 1.0 and t[3] == -1.0 and t[4] == 1.0 and t[5] == -1.0
+    s = ctx.unary("sigmoid", da).numpy()
+    assert s[4] == 1.0 and s[5] == 0.0
+
+
+def test_reference_activation_vectors(ctx, golden):
+    for key, op in (("relu", "relu"), ("sigmoid", "sigmoid"), ("tanh", "tanh"), ("neg", "neg")):
+        x, y = (np.array(v, np.float32) for v in golden[key]["arrays"])
+        got = ctx.unary(op, ctx.upload(x)).numpy()
+        np.testing.assert_allclose(got, y, atol=1e-4, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_activation_backward_bit_exact_vs_composed_cpu(ctx, orc, dtype):
+    rng = np.random.default_rng(13)
+    n = 300007
+    g = rng.uniform(-4, 4, n).astype(dtype)
+    x = rng.uniform(-4, 4, n).astype(dtype)
+    x[:3] = [0.0, -0.0, 1e-30]
+    dg, dx = ctx.upload(g), ctx.upload(x)
+    assert np.array_equal(ctx.relu_bwd(dg, dx).numpy(), orc.relu_bwd(g, x))
+    s = orc.unary("sigmoid", x)
+    t = orc.unary("tanh", x)
+    ds, dt = ctx.upload(s), ctx.upload(t)
+    for lit in (0, 1):
+        assert np.array_equal(ctx.sigmoid_bwd(dg, ds, lit).numpy(), orc.sigmoid_bwd(g, s, lit))
+    assert np.array_equal(ctx.tanh_bwd(dg, dt).numpy(), orc.tanh_bwd(g, t))
+    # the fused kernels equal the reference's op-by-op composition run on the GPU (src/ops/unary.rs:358-375)
+    mask = ctx.scalar("greater_scalar", dx, 0.0)
+    assert np.array_equal(ctx.binary("mul", dg, mask).numpy(), ctx.relu_bwd(dg, dx).numpy())
+    # correct-mode sigmoid gradient against the closed form in float64
+    ref = g.astype(np.float64) * s.astype(np.float64) * (1 - s.astype(np.float64))
+    assert rel_err(ctx.sigmoid_bwd(dg, ds, 0).numpy(), ref) <= TOL[np.dtype(dtype)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_fill_and_materialize(ctx, orc, dtype):
+    assert np.array_equal(ctx.fill((3, 5, 7), 2.5, dtype).numpy(), np.full((3, 5, 7), 2.5, dtype))
+    rng = np.random.default_rng(14)
+    bias = rng.standard_normal(32).astype(dtype)
+    # bias [C] -> [1,C,1,1] -> broadcast [B,C,H,W]  (src/nn/layers/utils.rs:6-42)
+    got = ctx.materialize(ctx.upload(bias), (4, 32, 5, 6), (0, 1, 0, 0)).numpy()
+    assert np.array_equal(got, np.broadcast_to(bias.reshape(1, 32, 1, 1), (4, 32, 5, 6)))
+    assert np.array_equal(got, orc.materialize(bias, (4, 32, 5, 6), (0, 1, 0, 0)))
+    m = rng.standard_normal((37, 53)).astype(dtype)
+    got = ctx.materialize(ctx.upload(m), (53, 37), (1, 53)).numpy()  # transpose
+    assert np.array_equal(got, m.T)
+
+
+# ------------------------------------------------------------------------------------------ im2col / col2im
+GEOMS = [  # B, C, H, W, k, s, p
+    (1, 1, 5, 5, 3, 1, 1), (2, 3, 8, 7, 3, 1, 1), (3, 2, 9, 9, 3, 2, 1), (2, 2, 6, 6, 2, 2, 0), (2, 3, 7, 5, 1, 1, 0),
+    (32, 1, 28, 28, 3, 1, 1), (4, 3, 32, 32, 3, 1, 1), (4, 32, 32, 32, 3, 2, 1),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_im2col_col2im_bit_exact(ctx, orc, dtype):
+    rng = np.random.default_rng(20)
+    for (B, Cc, H, W, k, s, p) in GEOMS:
+        x = rng.uniform(-1, 1, (B, Cc, H, W)).astype(dtype)
+        col = ctx.im2col(ctx.upload(x), (k, k), (s, s), (p, p))
+        ref = orc.im2col(x, (k, k), (s, s), (p, p))
+        assert np.array_equal(col.numpy(), ref), (B, Cc, H, W, k, s, p)
+        c2 = rng.standard_normal(ref.shape).astype(dtype)
+        dc2 = ctx.upload(c2)
+        for layout in (0, 1):
+            got = ctx.col2im(dc2, x.shape, (k, k), (s, s), (p, p), layout).numpy()
+            assert np.array_equal(got, orc.col2im(c2, x.shape, (k, k), (s, s), (p, p), layout)), (layout, B, Cc, H, W, k, s, p)
+
+
+def test_im2col_rectangular(ctx, orc):
+    rng = np.random.default_rng(21)
+    x = rng.uniform(-1, 1, (2, 2, 9, 6)).astype(np.float32)
+    for k, s, p in [((3, 2), (2, 1), (1, 0)), ((1, 3), (1, 2), (0, 1)), ((2, 2), (1, 1), (2, 2))]:
+        assert np.array_equal(ctx.im2col(ctx.upload(x), k, s, p).numpy(), orc.im2col(x, k, s, p))
+
+
+# ------------------------------------------------------------------------------------------ reductions
+RED_SHAPES = [(2, 2), (7, 13), (256, 10), (64, 1000), (3, 5, 7), (16, 32, 8, 8), (1, 70001), (5000, 33), (300, 4100), (2049, 515)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_reduce_every_axis(ctx, orc, dtype):
+    rng = np.random.default_rng(30)
+    tol = TOL[np.dtype(dtype)]
+    for shape in RED_SHAPES:
+        x = rng.standard_normal(shape).astype(dtype)
+        dx = ctx.upload(x)
+        for axis in range(len(shape)):
+            truth = x.astype(np.longdouble).sum(axis=axis)
+            bound = tol * np.abs(x).astype(np.float64).sum(axis=axis).max()
+            got = ctx.reduce("sum", dx, axis).numpy()
+            assert np.abs(got - truth).max() <= bound, ("sum", shape, axis)
+            # and against the oracle's CPU summation order, relative to the same scale
+            assert np.abs(got - orc.reduce_axis("sum", x, axis)).max() <= 2 * bound
+            got = ctx.reduce("mean", dx, axis).numpy()
+            assert np.abs(got - truth / shape[axis]).max() <= bound / shape[axis] + tol * np.abs(truth / shape[axis]).max()
+            v, i = ctx.reduce("max", dx, axis, want_idx=True)
+            rv, ri = orc.reduce_axis("max", x, axis, want_idx=True)
+            assert np.array_equal(v.numpy(), rv), ("max", shape, axis)
+            assert np.array_equal(i, ri) and np.array_equal(i, np.argmax(x, axis=axis)), ("argmax", shape, axis)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_reduce_all_and_ties(ctx, orc, dtype):
+    rng = np.random.default_rng(31)
+    x = rng.integers(-3, 4, (1 << 21) + 5).astype(dtype)  # many ties: first occurrence must win
+    dx = ctx.upload(x)
+    v, i = ctx.reduce("max", dx, 0, want_idx=True)
+    assert v.numpy().item() == x.max() and i.item() == int(np.argmax(x))
+    assert ctx.reduce("sum", dx, 0).numpy().item() == x.astype(np.float64).sum()  # small integers: exact in any order
+    y = rng.integers(-2, 3, (513, 1031)).astype(dtype)
+    dy = ctx.upload(y)
+    for axis in (0, 1):
+        v, i = ctx.reduce("max", dy, axis, want_idx=True)
+        assert np.array_equal(i, np.argmax(y, axis=axis)) and np.array_equal(v.numpy(), y.max(axis=axis))
+        assert np.array_equal(ctx.reduce("sum", dy, axis).numpy(), y.sum(axis=axis))
+
+
+def test_reduce_max_identity_and_nan(ctx, orc):
+    lowest = np.finfo(np.float32).min
+    x = np.array([[-np.inf, -np.inf, -np.inf], [np.nan, 1.0, 2.0], [lowest, lowest, -np.inf]], np.float32)
+    v, i = ctx.reduce("max", ctx.upload(x), 1, want_idx=True)
+    rv, ri = orc.reduce_axis("max", x, 1, want_idx=True)
+    assert np.array_equal(v.numpy(), rv) and np.array_equal(i, ri)
+    assert v.numpy()[0] == lowest and i[0] == 0 and i[1] == 2
+
+
+def test_reference_reduction_vectors(ctx, golden):
+    up = lambda k: ctx.upload(np.array(golden[k]["arrays"][0], np.float32).reshape(2, 2))  # noqa: E731
+    flat = lambda d: d.reshape(4)  # noqa: E731
+    assert ctx.reduce("sum", flat(up("sum_all")), 0).numpy().item() == golden["sum_all"]["arrays"][1][0]
+    assert ctx.reduce("sum", up("sum_axis0"), 0).numpy().tolist() == golden["sum_axis0"]["arrays"][1]
+    assert ctx.reduce("mean", flat(up("mean_all")), 0).numpy().item() == golden["mean_all"]["arrays"][1][0]
+    assert ctx.reduce("mean", up("mean_axis1"), 1).numpy().tolist() == golden["mean_axis1"]["arrays"][1]
+    assert ctx.reduce("max", flat(up("max_all")), 0).numpy().item() == golden["max_all"]["arrays"][1][0]
+    assert ctx.reduce("max", up("max_axis0"), 0).numpy().tolist() == golden["max_axis0"]["arrays"][1]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_softmax_axis(ctx, orc, golden, dtype):
+    rng = np.random.default_rng(32)
+    for shape, axis in (((256, 10), 1), ((4, 7, 5), 1), ((6, 9), 0)):
+        x = (rng.standard_normal(shape) * 3).astype(dtype)
+        got = ctx.softmax_axis(ctx.upload(x), axis).numpy()
+        assert rel_err(got, orc.softmax_axis(x.astype(np.float64), axis)) <= TOL[np.dtype(dtype)] * 4
+    for key, shape, axis in (("softmax_axis1", (2, 3), 1), ("softmax_axis0", (2, 2), 0)):
+        x, y = (np.array(v, dtype) for v in golden[key]["arrays"])
+        got = ctx.softmax_axis(ctx.upload(x.reshape(shape)), axis).numpy().ravel()
+        np.testing.assert_allclose(got, y, atol=1e-3, rtol=0)
+
+
+# ------------------------------------------------------------------------------------------ GEMM
+GEMM_SHAPES = [(2, 2, 2), (1, 1, 1), (5, 7, 3), (64, 64, 64), (128, 128, 16), (130, 257, 75), (256, 256, 784), (256, 10, 128),
+               (256, 10, 16384), (16384, 10, 256), (256, 16384, 10), (300, 200, 1000)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_all_transposes(ctx, orc, golden, dtype):
+    rng = np.random.default_rng(40)
+    tol = TOL[np.dtype(dtype)]
+    for (M, N, K) in GEMM_SHAPES:
+        a = rng.standard_normal((M, K)).astype(dtype)
+        b = rng.standard_normal((K, N)).astype(dtype)
+        truth = a.astype(np.float64) @ b.astype(np.float64)
+        scale = (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)).max()
+        for ta in (False, True):
+            for tb in (False, True):
+                da = ctx.upload(a.T if ta else a)
+                db = ctx.upload(b.T if tb else b)
+                got = ctx.gemm(da, db, ta, tb).numpy()
+                assert np.abs(got - truth).max() <= tol * scale, (M, N, K, ta, tb)
+    a, b, c = (np.array(v, dtype).reshape(2, 2) for v in golden["matmul"]["arrays"])
+    assert np.array_equal(ctx.gemm(ctx.upload(a), ctx.upload(b)).numpy(), c)
+    got = ctx.gemm(ctx.upload(rng.standard_normal((64, 64)).astype(dtype)), ctx.upload(np.eye(64, dtype=dtype))).numpy()
+    assert got.shape == (64, 64)
+
+
+def test_gemm_shape_mismatch_message(ctx):
+    from ferrox_amd.capi import FerroxHipError
+    a = ctx.upload(np.zeros((2, 3), np.float32))
+    b = ctx.upload(np.zeros((4, 5), np.float32))
+    with pytest.raises(FerroxHipError, match=r"Matrix multiplication shape mismatch: \(2, 3\) @ \(4, 5\)"):
+        ctx.gemm(a, b)
+
+
+# ------------------------------------------------------------------------------------------ convolution
+CONV_CASES = [  # B, Cin, H, W, Cout, k, s, p
+    (1, 1, 5, 5, 1, 3, 1, 1), (1, 3, 5, 5, 4, 3, 1, 1), (2, 3, 8, 8, 4, 3, 1, 1), (3, 2, 9, 7, 5, 3, 2, 1), (2, 4, 6, 6, 3, 1, 1, 0),
+    (32, 1, 28, 28, 8, 3, 1, 1), (8, 3, 32, 32, 32, 3, 1, 1), (8, 32, 32, 32, 64, 3, 2, 1), (2, 64, 56, 56, 128, 3, 1, 1),
+    (2, 70, 13, 11, 130, 3, 1, 1), (2, 3, 7, 7, 2, 2, 2, 0),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_conv2d_fwd_dgrad_wgrad_vs_oracle(ctx, orc, dtype):
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(50)
+    tol = TOL[np.dtype(dtype)]
+    for (B, Cin, H, W, Cout, k, s, p) in CONV_CASES:
+        x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(dtype)
+        w = (rng.standard_normal((Cout, Cin, k, k)) * np.sqrt(2.0 / (Cin * k * k))).astype(dtype)
+        oh, ow = orc.out_hw(H, W, k, k, s, s, p, p)
+        g = rng.standard_normal((B, Cout, oh, ow)).astype(dtype)
+        dx_, dw_, dg_ = ctx.upload(x), ctx.upload(w), ctx.upload(g)
+        y = ctx.conv2d_fwd(dx_, dw_, (s, s), (p, p)).numpy()
+        dxg = ctx.conv2d_dgrad(dg_, dw_, x.shape, (s, s), (p, p), 0).numpy()
+        dwg = ctx.conv2d_wgrad(dx_, dg_, w.shape, (s, s), (p, p), 0).numpy()
+        # float64 ground truth from torch (the textbook routine) with |.|-scaled bounds
+        tx = torch.from_numpy(x).double().requires_grad_(True)
+        tw = torch.from_numpy(w).double().requires_grad_(True)
+        ty = F.conv2d(tx, tw, stride=s, padding=p)
+        ty.backward(torch.from_numpy(g).double())
+        ay = F.conv2d(tx.detach().abs(), tw.detach().abs(), stride=s, padding=p).max().item()
+        case = (B, Cin, H, W, Cout, k, s, p)
+        assert np.abs(y - ty.detach().numpy()).max() <= tol * ay, ("fwd", case)
+        assert rel_err(dxg, tx.grad.numpy()) <= tol * 8, ("dgrad", case)
+        assert rel_err(dwg, tw.grad.numpy()) <= tol * 8, ("wgrad", case)
+        # and against the CPU oracle (restated reference algorithm), both gradient modes
+        assert rel_err(y, orc.conv2d_fwd(x, w, (s, s), (p, p))) <= tol * 8
+        assert rel_err(dxg, orc.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), 0)) <= tol * 8
+        assert rel_err(dwg, orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 0)) <= tol * 8
+        if B * Cin * H * W <= 200000:
+            lit_dx = ctx.conv2d_dgrad(dg_, dw_, x.shape, (s, s), (p, p), 1).numpy()
+            lit_dw = ctx.conv2d_wgrad(dx_, dg_, w.shape, (s, s), (p, p), 1).numpy()
+            assert rel_err(lit_dx, orc.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), 1)) <= tol * 8, ("literal dgrad", case)
+            assert rel_err(lit_dw, orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 1)) <= tol * 8, ("literal wgrad", case)
+
+
+def test_conv2d_reference_vectors(ctx, golden):
+    for key in ("conv2d_test", "conv2d_simple_forward", "conv2d_edge_cases"):
+        gv = golden[key]
+        x = np.array(gv["x"], np.float32).reshape(gv["x_shape"])
+        w = np.array(gv["w"], np.float32).reshape(gv["w_shape"])
+        y = ctx.conv2d_fwd(ctx.upload(x), ctx.upload(w), tuple(gv["stride"]), tuple(gv["padding"])).numpy()
+        assert list(y.shape) == gv["y_shape"]
+        np.testing.assert_allclose(y.ravel(), np.array(gv["y"], np.float32), atol=gv["tol"], rtol=0)
+
+
+def test_conv2d_run_to_run_determinism(ctx):
+    rng = np.random.default_rng(51)
+    x = ctx.upload(rng.uniform(-1, 1, (4, 16, 20, 20)).astype(np.float32))
+    w = ctx.upload(rng.standard_normal((24, 16, 3, 3)).astype(np.float32))
+    g = ctx.upload(rng.standard_normal((4, 24, 20, 20)).astype(np.float32))
+    a = [ctx.conv2d_dgrad(g, w, x.shape, (1, 1), (1, 1)).numpy(), ctx.conv2d_wgrad(x, g, w.shape, (1, 1), (1, 1)).numpy()]
+    b = [ctx.conv2d_dgrad(g, w, x.shape, (1, 1), (1, 1)).numpy(), ctx.conv2d_wgrad(x, g, w.shape, (1, 1), (1, 1)).numpy()]
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
