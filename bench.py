@@ -1,0 +1,207 @@
+#!/usr/bin/env python3
+"""Benchmark of the Ferrox-on-MI355X hot path.  Prints ONE JSON line.
+
+Primary workload (config C3 of BASELINE.json): a single Conv2d layer, f32, input N=128, C_in=64, 56x56, U(-1,1);
+C_out=128, 3x3, stride 1, pad 1, Kaiming-normal weights; upstream gradient N(0,1).  One "step" is one forward +
+one data-gradient + one weight-gradient pass.  `value` is the conv fwd+bwd throughput in TFLOP/s, counting the
+algorithmic 2*Cout*(Cin*kh*kw)*(B*oh*ow) FLOP per pass, with all tensors resident in HBM before timing starts.
+
+Also measured in the same run and reported under "also": the bandwidth kernels of config C4 (sum/mean/max over
+axis 0, axis 1 and all elements of [8192,8192] f32 and f64; add/mul and ReLU/sigmoid/tanh backward on 2^28 f32).
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--skip-also]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_F32_MFMA_TFLOPS = 157.3
+PEAK_F64_MFMA_TFLOPS = 78.6
+PEAK_HBM_GBS = 8000.0
+
+C3 = dict(B=128, Cin=64, H=56, W=56, Cout=128, k=3, s=1, p=1)
+
+
+def time_stream(ctx, fn, iters, warmup):
+    """Average milliseconds per call of fn, measured with HIP events on the stream the kernels run on."""
+    for _ in range(warmup):
+        fn()
+    ctx.sync()
+    ctx.timer_start()
+    for _ in range(iters):
+        fn()
+    return ctx.timer_stop() / iters
+
+
+def bench_conv(ctx, steps, warmup, dtype=np.float32, B=None):
+    c = dict(C3)
+    if B is not None:
+        c["B"] = B
+    B, Cin, H, W, Cout, k, s, p = (c[n] for n in ("B", "Cin", "H", "W", "Cout", "k", "s", "p"))
+    x = ctx.uniform((B, Cin, H, W), 3, -1.0, 1.0, dtype)
+    w = ctx.normal((Cout, Cin, k, k), 33, 0.0, (2.0 / (Cin * k * k)) ** 0.5, dtype)
+    g = ctx.normal((B, Cout, H, W), 333, 0.0, 1.0, dtype)
+    y = ctx.empty((B, Cout, H, W), dtype)
+    dx = ctx.empty(x.shape, dtype)
+    dw = ctx.empty(w.shape, dtype)
+    flop = 2.0 * Cout * Cin * k * k * B * H * W
+    passes = {
+        "fwd": lambda: ctx.conv2d_fwd(x, w, (s, s), (p, p), out=y),
+        "dgrad": lambda: ctx.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), out=dx),
+        "wgrad": lambda: ctx.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), out=dw),
+    }
+    per_pass = {}
+    for name, fn in passes.items():
+        ms = time_stream(ctx, fn, steps, warmup)
+        per_pass[name] = {"ms": ms, "tflops": flop / ms / 1e9}
+
+    def step():
+        for fn in passes.values():
+            fn()
+
+    # the timed region of the headline number: exactly `steps` steps between two synchronisations
+    for _ in range(warmup):
+        step()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    ctx.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return {"flop_per_pass": flop, "per_pass": per_pass, "ms_per_step": wall_ms, "tflops": 3 * flop / wall_ms / 1e9}
+
+
+def bench_bandwidth(ctx, iters=20, warmup=3):
+    from ferrox_amd import capi
+    out = {"reductions": {}, "elementwise": {}}
+    for dtype in (np.float32, np.float64):
+        sfx = capi.dtype_code(dtype)[1]
+        a = ctx.normal((8192, 8192), 4, 0.0, 1.0, dtype)
+        res = ctx.empty((8192,), dtype)
+        idx = ctx.empty((8192,), np.float64)  # int64 argmax indices (8 bytes each)
+        for kind in ("sum", "mean", "max"):
+            for axis, view in (("0", (1, 8192, 8192)), ("1", (8192, 8192, 1)), ("all", (1, 8192 * 8192, 1))):
+                n_out = view[0] * view[2]
+                if kind == "max":
+                    fn = lambda: capi.check(getattr(capi.lib, f"fx_reduce_max_{sfx}")(ctx.h, a.ptr, res.ptr, idx.ptr, *view))  # noqa: E731
+                    nbytes = a.dtype.itemsize * (a.size + n_out) + 8 * n_out
+                else:
+                    fn = lambda: capi.check(getattr(capi.lib, f"fx_reduce_{kind}_{sfx}")(ctx.h, a.ptr, res.ptr, *view))  # noqa: E731
+                    nbytes = a.dtype.itemsize * (a.size + n_out)
+                ms = time_stream(ctx, fn, iters, warmup)
+                out["reductions"][f"{kind}_axis{axis}_{sfx}"] = {"us": ms * 1e3, "GBps": nbytes / ms / 1e6,
+                                                                 "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+        del a, res, idx
+    n = 1 << 28
+    g = ctx.uniform((n,), 7, -4.0, 4.0)
+    x = ctx.uniform((n,), 8, -4.0, 4.0)
+    s = ctx.unary("sigmoid", x)
+    t = ctx.unary("tanh", x)
+    o = ctx.empty((n,))
+    cases = {
+        "add": lambda: ctx.binary("add", g, x, out=o),
+        "mul": lambda: ctx.binary("mul", g, x, out=o),
+        "relu_bwd": lambda: ctx.relu_bwd(g, x, out=o),
+        "sigmoid_bwd": lambda: ctx.sigmoid_bwd(g, s, 0, out=o),
+        "tanh_bwd": lambda: ctx.tanh_bwd(g, t, out=o),
+    }
+    for name, fn in cases.items():
+        ms = time_stream(ctx, fn, 10, 2)
+        nbytes = 3 * 4 * n
+        out["elementwise"][f"{name}_f32"] = {"ms": ms, "GBps": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    return out
+
+
+def cpu_baseline_conv(batch=8, reps=1):
+    """The CPU oracle (a restatement of Ferrox's ndarray path: im2col + single-thread GEMM + col2im) timed on this
+    host, on a batch slice of the same layer; one thread, like the reference."""
+    import oracle as orc
+    c = dict(C3, B=batch)
+    B, Cin, H, W, Cout, k, s, p = (c[n] for n in ("B", "Cin", "H", "W", "Cout", "k", "s", "p"))
+    rng = np.random.default_rng(3)
+    x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, k, k)) * (2.0 / (Cin * k * k)) ** 0.5).astype(np.float32)
+    g = rng.standard_normal((B, Cout, H, W)).astype(np.float32)
+    flop = 3 * 2.0 * Cout * Cin * k * k * B * H * W
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        orc.conv2d_fwd(x, w, (s, s), (p, p))
+        orc.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), 0)
+        orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 0)
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": flop / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"same layer at batch {B} of 128 (fwd+dgrad+wgrad, {reps} rep(s), {dt:.2f} s per rep), f32, "
+                      f"im2col + blocked single-thread GEMM + col2im as in the reference CPU backend",
+            "host_cpu": _cpu_model()}
+
+
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip() + f" ({os.cpu_count()} logical cores visible)"
+    except OSError:
+        pass
+    return "unknown"
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--skip-also", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (the hot path has no cross-GPU exchange built); use --gpus 1")
+
+    from ferrox_amd import capi
+    ctx = capi.Context(0)
+    conv = bench_conv(ctx, args.steps, args.warmup)
+    dominant = max(conv["per_pass"], key=lambda k: conv["per_pass"][k]["ms"])
+    dom = conv["per_pass"][dominant]
+    result = {
+        "metric": "conv fwd+bwd TFLOP/s",
+        "value": conv["tflops"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": conv["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "C3: Conv2d N=128 Cin=64 56x56 -> Cout=128 3x3 s1 p1, f32; step = fwd + dgrad + wgrad",
+                   "flop_per_step": 3 * conv["flop_per_pass"], "device": ctx.device_name()},
+        "roofline": {"bound": "mfma", "kernel": f"igemm_kernel<float> conv {dominant}", "achieved": dom["tflops"],
+                     "peak": PEAK_F32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": dom["tflops"] / PEAK_F32_MFMA_TFLOPS,
+                     "traffic": None, "avg_launch_ms": dom["ms"]},
+        "conv_passes": {k: {"ms": v["ms"], "tflops": v["tflops"], "frac_mfma_f32": v["tflops"] / PEAK_F32_MFMA_TFLOPS}
+                        for k, v in conv["per_pass"].items()},
+    }
+    if not args.skip_also:
+        c64 = bench_conv(ctx, max(3, args.steps // 4), 1, np.float64, B=64)
+        result["also"] = {
+            "conv_f64_batch64": {k: {"ms": v["ms"], "tflops": v["tflops"], "frac_mfma_f64": v["tflops"] / PEAK_F64_MFMA_TFLOPS}
+                                 for k, v in c64["per_pass"].items()},
+        }
+        result["also"].update(bench_bandwidth(ctx))
+    ctx.close()
+    if not args.skip_cpu:
+        result["cpu_baseline"] = cpu_baseline_conv()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -90,6 +90,8 @@ _sig("fx_conv2d_workspace_bytes", _int, _int, _int, *([_i64] * 11), restype=_i64
 _CONV_INTS = [_i64] * 11
 for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_fill_{_s}", _vp, _vp, _ct, _i64)
+    _sig(f"fx_fill_uniform_{_s}", _vp, _vp, _i64, _u64, _ct, _ct)
+    _sig(f"fx_fill_normal_{_s}", _vp, _vp, _i64, _u64, _ct, _ct)
     _sig(f"fx_materialize_{_s}", _vp, _vp, _vp, C.POINTER(_i64), C.POINTER(_i64), _int, _i64)
     _sig(f"fx_binary_{_s}", _vp, _int, _vp, _vp, _vp, _i64)
     for _n in ("add", "sub", "mul", "div", "equal"):
@@ -252,6 +254,16 @@ class Context:
     def fill(self, shape, value, dtype=np.float32):
         o = self.empty(shape, dtype)
         check(self._fn("fill", dtype)(self.h, o.ptr, float(value), o.size))
+        return o
+
+    def uniform(self, shape, seed, lo, hi, dtype=np.float32):
+        o = self.empty(shape, dtype)
+        check(self._fn("fill_uniform", dtype)(self.h, o.ptr, o.size, seed, float(lo), float(hi)))
+        return o
+
+    def normal(self, shape, seed, mean=0.0, std=1.0, dtype=np.float32):
+        o = self.empty(shape, dtype)
+        check(self._fn("fill_normal", dtype)(self.h, o.ptr, o.size, seed, float(mean), float(std)))
         return o
 
     def binary(self, op, a, b, out=None):

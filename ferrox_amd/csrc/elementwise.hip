@@ -264,9 +264,54 @@ int materialize(fx_ctx* c, const T* in, T* out, const i64* shape, const i64* str
     return FX_OK;
 }
 
+// ---- synthetic data: counter-based generator (splitmix64 of seed + index), identical for any launch shape ----
+__device__ __forceinline__ uint64_t splitmix64(uint64_t x) {
+    x += 0x9e3779b97f4a7c15ull;
+    x = (x ^ (x >> 30)) * 0xbf58476d1ce4e5b9ull;
+    x = (x ^ (x >> 27)) * 0x94d049bb133111ebull;
+    return x ^ (x >> 31);
+}
+// u in [0,1) with 53 (double) or 24 (float) random bits
+template <typename T> __device__ __forceinline__ T unit_uniform(uint64_t z);
+template <> __device__ __forceinline__ double unit_uniform<double>(uint64_t z) { return (double)(z >> 11) * (1.0 / 9007199254740992.0); }
+template <> __device__ __forceinline__ float unit_uniform<float>(uint64_t z) { return (float)(z >> 40) * (1.0f / 16777216.0f); }
+
+template <typename T, bool NORMAL>
+__global__ __launch_bounds__(256) void random_fill_kernel(T* __restrict__ out, i64 n, uint64_t seed, T a, T b) {
+    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    if (!NORMAL) {
+        out[i] = a + (b - a) * unit_uniform<T>(splitmix64(seed + (uint64_t)i));
+    } else {  // Box-Muller; a = mean, b = std
+        const double u1 = unit_uniform<double>(splitmix64(seed + 2 * (uint64_t)i));
+        const double u2 = unit_uniform<double>(splitmix64(seed + 2 * (uint64_t)i + 1));
+        const double r = sqrt(-2.0 * log(1.0 - u1));
+        out[i] = (T)((double)a + (double)b * r * cos(6.283185307179586 * u2));
+    }
+}
+
+template <typename T, bool NORMAL>
+int random_fill(fx_ctx* c, T* out, i64 n, uint64_t seed, T a, T b) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(n >= 0, "fx_fill_random: negative element count");
+    if (n == 0) return FX_OK;
+    FX_REQUIRE(out != nullptr, "fx_fill_random: null pointer");
+    const i64 blocks = fx::ceil_div(n, 256);
+    FX_REQUIRE(blocks <= 0x7fffffff, "fx_fill_random: too many elements");
+    random_fill_kernel<T, NORMAL><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(out, n, seed, a, b);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
 }  // namespace
 
 #define FX_DEFINE_EW(T, S)                                                                                             \
+    extern "C" int fx_fill_uniform_##S(fx_ctx* c, T* out, int64_t n, uint64_t seed, T lo, T hi) {                      \
+        return random_fill<T, false>(c, out, n, seed, lo, hi);                                                         \
+    }                                                                                                                  \
+    extern "C" int fx_fill_normal_##S(fx_ctx* c, T* out, int64_t n, uint64_t seed, T mean, T std) {                    \
+        return random_fill<T, true>(c, out, n, seed, mean, std);                                                       \
+    }                                                                                                                  \
     extern "C" int fx_fill_##S(fx_ctx* c, T* out, T v, int64_t n) {                                                    \
         return launch_ew<T, 0>(c, (const T*)nullptr, (const T*)nullptr, out, n, FillF<T>{v}, "fx_fill");               \
     }                                                                                                                  \

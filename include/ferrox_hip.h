@@ -133,6 +133,11 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
 #define FX_DECLARE_KERNELS(T, S)                                                                                       \
     /* launch_fill, kernels.rs:435-448 */                                                                              \
     int fx_fill_##S(fx_ctx* ctx, T* out, T value, int64_t n);                                                          \
+    /* launch_fill_random, kernels.rs:450-467 (kernels/fill.cu:7-21 hashes seed+idx with xorshift32 into U(-1,1)).     \
+       Here: splitmix64(seed + i) -> lo + (hi-lo)*u, u in [0,1) with 24/53 random bits; reproducible on the host        \
+       with integer arithmetic.  The normal variant applies Box-Muller to hashes 2i and 2i+1. */                       \
+    int fx_fill_uniform_##S(fx_ctx* ctx, T* out, int64_t n, uint64_t seed, T lo, T hi);                                \
+    int fx_fill_normal_##S(fx_ctx* ctx, T* out, int64_t n, uint64_t seed, T mean, T std);                              \
     /* launch_materialize, kernels.rs:802-830 / CudaOps::materialize, ops.rs:175-214.  shape and strides (in          \
        elements, 0 on broadcast dims) are HOST arrays, ndim <= 8. */                                                   \
     int fx_materialize_##S(fx_ctx* ctx, const T* in, T* out, const int64_t* host_shape, const int64_t* host_strides,   \
