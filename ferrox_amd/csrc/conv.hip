@@ -10,6 +10,8 @@
 //   wgrad: dw[oc,(c,ky,kx)] = sum_{b,l} g[b,oc,l] * x[b,c,...]                         M=Cout N=Cin*kh*kw K=B*oh*ow
 //          (split along K into fixed-order partial sums; no float atomics)
 // mode 1 reproduces the CPU backend's literal arithmetic for the gradients (see include/ferrox_hip.h).
+#include <cstdlib>
+
 #include "igemm_core.hpp"
 
 namespace fx {
@@ -26,6 +28,13 @@ typedef Tile<128, 128, 16, 64, 64> TileM128;  // 4 waves as 2x2, 64x64 each
 typedef Tile<64, 128, 16, 64, 32> TileM64;    // 4 waves as 1x4, 64x32 each
 typedef Tile<32, 256, 16, 32, 64> TileM32;    // 4 waves as 1x4, 32x64 each
 typedef Tile<64, 64, 16, 32, 32> TileSmall;   // 4 waves as 2x2, 32x32 each
+// tuning variants
+typedef Tile<128, 128, 32, 64, 64> TileM128K32;
+typedef Tile<64, 256, 16, 64, 64> TileM64N256;
+typedef Tile<64, 256, 32, 64, 64> TileM64N256K32;
+typedef Tile<128, 192, 16, 64, 96> TileN192;
+typedef Tile<128, 192, 32, 64, 96> TileN192K32;
+static int variant() { const char* v = getenv("FX_CONV_VARIANT"); return v ? atoi(v) : 0; }
 
 int gemm_t(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const float* A, const float* B, float* C) { return fx_gemm_f32(c, ta, tb, M, N, K, A, B, C); }
 int gemm_t(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const double* A, const double* B, double* C) { return fx_gemm_f64(c, ta, tb, M, N, K, A, B, C); }
@@ -36,6 +45,7 @@ struct Dims {
     i64 B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, oh, ow;
 };
 
+template <typename T>
 int check_dims(Dims& d, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, const char* what) {
     FX_REQUIRE(B > 0 && Cin > 0 && H > 0 && W > 0 && Cout > 0 && kh > 0 && kw > 0 && sh > 0 && sw > 0 && ph >= 0 && pw >= 0,
                "%s: non-positive dimension", what);
@@ -46,51 +56,87 @@ int check_dims(Dims& d, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, 
     FX_REQUIRE(B * d.oh * d.ow <= lim && B * H * W <= lim && Cin * H * W <= lim && Cout * d.oh * d.ow <= lim &&
                    Cin * kh * kw <= lim && Cout * kh * kw <= lim,
                "%s: a GEMM dimension or per-image plane exceeds 2^31-1", what);
+    if (B * Cin * H * W * (i64)sizeof(T) > lim || B * Cout * d.oh * d.ow * (i64)sizeof(T) > lim) {
+        fx::set_error("%s: tensors of 2 GiB or more are not supported by this build", what);
+        return FX_ERR_UNSUPPORTED;
+    }
     return FX_OK;
 }
 
-// wt[c][oc*KK + r] = w[oc][c][r]
+// Weight re-layouts feeding the A operand (w is [Cout][Cin][KK], KK = kh*kw):
+//  mode 0: out[oc][r*Cin + c]   = w[oc][c][r]   forward, K ordered (ky,kx) outer / channel inner
+//  mode 1: out[c][oc*KK + r]    = w[oc][c][r]   data gradient, K ordered like the reference (oc,ky,kx)
+//  mode 2: out[c][r*Cout + oc]  = w[oc][c][r]   data gradient, K ordered (ky,kx) outer / out-channel inner
 template <typename T>
-__global__ __launch_bounds__(256) void permute_weights_kernel(const T* __restrict__ w, T* __restrict__ wt, int Cout, int Cin, int KK) {
+__global__ __launch_bounds__(256) void permute_weights_kernel(const T* __restrict__ w, T* __restrict__ out, int Cout, int Cin, int KK, int mode) {
     const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
     const i64 n = (i64)Cout * Cin * KK;
     if (i >= n) return;
-    const int r = (int)(i % KK);
-    const i64 t = i / KK;
-    const int oc = (int)(t % Cout), c = (int)(t / Cout);
-    wt[i] = w[((i64)oc * Cin + c) * KK + r];
+    int oc, c, r;
+    if (mode == 0) { c = (int)(i % Cin); const i64 t = i / Cin; r = (int)(t % KK); oc = (int)(t / KK); }
+    else if (mode == 1) { r = (int)(i % KK); const i64 t = i / KK; oc = (int)(t % Cout); c = (int)(t / Cout); }
+    else { oc = (int)(i % Cout); const i64 t = i / Cout; r = (int)(t % KK); c = (int)(t / KK); }
+    out[i] = w[((i64)oc * Cin + c) * KK + r];
 }
 
-template <typename T, class Cfg>
+template <typename T>
+int permute_weights(fx_ctx* c, const T* w, T* out, const Dims& d, int mode) {
+    const i64 nw = d.Cin * d.Cout * d.kh * d.kw;
+    permute_weights_kernel<T><<<dim3((unsigned)fx::ceil_div(nw, 256)), dim3(256), 0, c->stream>>>(w, out, (int)d.Cout, (int)d.Cin, (int)(d.kh * d.kw), mode);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+constexpr int CONV_BK = 16;  // slab depth of every conv tile; the (ky,kx)-outer K order needs channels % CONV_BK == 0
+
+template <typename T, class Cfg, bool FAST>
 int fwd_tile(fx_ctx* c, const T* x, const T* w, T* y, const Dims& d) {
+    static_assert(Cfg::BK == CONV_BK || !FAST || Cfg::BK == 32, "unexpected slab depth");
     const i64 M = d.Cout, N = d.B * d.oh * d.ow, K = d.Cin * d.kh * d.kw;
     const ConvShape s = make_shape(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
     MatLoader<T, true> al{w, K, (int)M};
-    ConvFwdB<T> bl{x, s, (int)N};
+    ConvFwdB<T, FAST> bl{x, s, (int)N};
     NchwStore<T> ep{y, (int)d.Cout, (int)(d.oh * d.ow), (int)N, s.div_L};
     const int kps = (int)(fx::ceil_div(K, Cfg::BK) * Cfg::BK);
     return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
 }
 
 template <typename T>
+i64 fwd_ws_bytes(const Dims& d) {
+    return d.Cin % CONV_BK == 0 ? d.Cin * d.Cout * d.kh * d.kw * (i64)sizeof(T) : 0;
+}
+
+template <typename T>
 int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw,
-             i64 ph, i64 pw) {
+             i64 ph, i64 pw, void* ws, i64 ws_bytes) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(x && w && y, "fx_conv2d_fwd: null pointer");
     Dims d;
-    if (int rc = check_dims(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_fwd")) return rc;
+    if (int rc = check_dims<T>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_fwd")) return rc;
+    const i64 need = fwd_ws_bytes<T>(d);
+    FX_REQUIRE(ws == nullptr || ws_bytes >= need, "fx_conv2d_fwd: workspace of %lld bytes is smaller than the %lld needed",
+               (long long)ws_bytes, (long long)need);
     std::lock_guard<std::mutex> lk(c->launch_mutex);
-    if (Cout > 64) return fwd_tile<T, TileM128>(c, x, w, y, d);
-    if (Cout > 32) return fwd_tile<T, TileM64>(c, x, w, y, d);
-    return fwd_tile<T, TileM32>(c, x, w, y, d);
+    if (need > 0) {
+        T* wp = (T*)(ws ? ws : c->get_scratch(need));
+        if (!wp) return FX_ERR_OOM;
+        if (int rc = permute_weights<T>(c, w, wp, d, 0)) return rc;
+        if constexpr (sizeof(T) == 4) if (Cout > 64 && Cin % 32 == 0 && variant() == 1) return fwd_tile<T, TileM128K32, true>(c, x, wp, y, d);
+        if (Cout > 64) return fwd_tile<T, TileM128, true>(c, x, wp, y, d);
+        if (Cout > 32) return fwd_tile<T, TileM64, true>(c, x, wp, y, d);
+        return fwd_tile<T, TileM32, true>(c, x, wp, y, d);
+    }
+    if (Cout > 64) return fwd_tile<T, TileM128, false>(c, x, w, y, d);
+    if (Cout > 32) return fwd_tile<T, TileM64, false>(c, x, w, y, d);
+    return fwd_tile<T, TileM32, false>(c, x, w, y, d);
 }
 
-template <typename T, class Cfg>
+template <typename T, class Cfg, bool FAST>
 int dgrad_tile(fx_ctx* c, const T* g, const T* wt, T* dx, const Dims& d) {
     const i64 M = d.Cin, N = d.B * d.H * d.W, K = d.Cout * d.kh * d.kw;
     const ConvShape s = make_shape(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
     MatLoader<T, true> al{wt, K, (int)M};
-    ConvDgradB<T> bl{g, s, (int)N};
+    ConvDgradB<T, FAST> bl{g, s, (int)N};
     NchwStore<T> ep{dx, (int)d.Cin, (int)(d.H * d.W), (int)N, s.div_HW};
     const int kps = (int)(fx::ceil_div(K, Cfg::BK) * Cfg::BK);
     return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
@@ -109,7 +155,7 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
     FX_REQUIRE(g && w && dx, "fx_conv2d_dgrad: null pointer");
     FX_REQUIRE(mode == 0 || mode == 1, "fx_conv2d_dgrad: mode must be 0 or 1");
     Dims d;
-    if (int rc = check_dims(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_dgrad")) return rc;
+    if (int rc = check_dims<T>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_dgrad")) return rc;
     const i64 need = dgrad_ws_bytes<T>(d, mode);
     FX_REQUIRE(ws == nullptr || ws_bytes >= need, "fx_conv2d_dgrad: workspace of %lld bytes is smaller than the %lld needed",
                (long long)ws_bytes, (long long)need);
@@ -133,12 +179,18 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
     std::lock_guard<std::mutex> lk(c->launch_mutex);
     T* wt = (T*)(ws ? ws : c->get_scratch(need));
     if (!wt) return FX_ERR_OOM;
-    const i64 nw = Cin * Cout * kh * kw;
-    permute_weights_kernel<T><<<dim3((unsigned)fx::ceil_div(nw, 256)), dim3(256), 0, c->stream>>>(w, wt, (int)Cout, (int)Cin, (int)(kh * kw));
-    FX_LAUNCH_CHECK();
-    if (Cin > 64) return dgrad_tile<T, TileM128>(c, g, wt, dx, d);
-    if (Cin > 32) return dgrad_tile<T, TileM64>(c, g, wt, dx, d);
-    return dgrad_tile<T, TileM32>(c, g, wt, dx, d);
+    if (Cout % CONV_BK == 0) {
+        if (int rc = permute_weights<T>(c, w, wt, d, 2)) return rc;
+        if constexpr (sizeof(T) == 4) if (Cin > 32 && variant() == 1) return dgrad_tile<T, TileM64N256, true>(c, g, wt, dx, d);
+        if constexpr (sizeof(T) == 4) if (Cin > 32 && Cout % 32 == 0 && variant() == 2) return dgrad_tile<T, TileM64N256K32, true>(c, g, wt, dx, d);
+        if (Cin > 64) return dgrad_tile<T, TileM128, true>(c, g, wt, dx, d);
+        if (Cin > 32) return dgrad_tile<T, TileM64, true>(c, g, wt, dx, d);
+        return dgrad_tile<T, TileM32, true>(c, g, wt, dx, d);
+    }
+    if (int rc = permute_weights<T>(c, w, wt, d, 1)) return rc;
+    if (Cin > 64) return dgrad_tile<T, TileM128, false>(c, g, wt, dx, d);
+    if (Cin > 32) return dgrad_tile<T, TileM64, false>(c, g, wt, dx, d);
+    return dgrad_tile<T, TileM32, false>(c, g, wt, dx, d);
 }
 
 template <typename T, class Cfg>
@@ -188,11 +240,14 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
     FX_REQUIRE(x && g && dw, "fx_conv2d_wgrad: null pointer");
     FX_REQUIRE(mode == 0 || mode == 1, "fx_conv2d_wgrad: mode must be 0 or 1");
     Dims d;
-    if (int rc = check_dims(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_wgrad")) return rc;
+    if (int rc = check_dims<T>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_wgrad")) return rc;
     const i64 need = wgrad_ws_bytes<T>(c, d);
     FX_REQUIRE(ws == nullptr || ws_bytes >= need, "fx_conv2d_wgrad: workspace of %lld bytes is smaller than the %lld needed",
                (long long)ws_bytes, (long long)need);
     std::lock_guard<std::mutex> lk(c->launch_mutex);
+    if constexpr (sizeof(T) == 4) if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64 && variant() == 1) return wgrad_tile<T, TileM128K32>(c, x, g, dw, d, mode, ws);
+    if constexpr (sizeof(T) == 4) if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64 && variant() == 2) return wgrad_tile<T, TileN192>(c, x, g, dw, d, mode, ws);
+    if constexpr (sizeof(T) == 4) if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64 && variant() == 3) return wgrad_tile<T, TileN192K32>(c, x, g, dw, d, mode, ws);
     if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64) return wgrad_tile<T, TileM128>(c, x, g, dw, d, mode, ws);
     return wgrad_tile<T, TileSmall>(c, x, g, dw, d, mode, ws);
 }
@@ -202,8 +257,10 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
 extern "C" int64_t fx_conv2d_workspace_bytes(int kind, int dtype, int mode, int64_t B, int64_t Cin, int64_t H, int64_t W,
                                              int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw) {
     Dims d;
-    if (check_dims(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_workspace_bytes")) return -1;
-    if (kind == FX_CONV_FWD) return 0;
+    if (dtype == FX_F64 ? check_dims<double>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_workspace_bytes")
+                        : check_dims<float>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_workspace_bytes"))
+        return -1;
+    if (kind == FX_CONV_FWD) return dtype == FX_F64 ? fwd_ws_bytes<double>(d) : fwd_ws_bytes<float>(d);
     if (kind == FX_CONV_DGRAD) return dtype == FX_F64 ? dgrad_ws_bytes<double>(d, mode) : dgrad_ws_bytes<float>(d, mode);
     if (kind == FX_CONV_WGRAD) return dtype == FX_F64 ? wgrad_ws_bytes<double>(nullptr, d) : wgrad_ws_bytes<float>(nullptr, d);
     fx::set_error("fx_conv2d_workspace_bytes: unknown kind %d", kind);
@@ -214,8 +271,7 @@ extern "C" int64_t fx_conv2d_workspace_bytes(int kind, int dtype, int mode, int6
     extern "C" int fx_conv2d_fwd_##S(fx_ctx* c, const T* x, const T* w, T* y, int64_t B, int64_t Cin, int64_t H, int64_t W, \
                                      int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,  \
                                      void* ws, int64_t ws_bytes) {                                                     \
-        (void)ws; (void)ws_bytes;                                                                                      \
-        return conv_fwd<T>(c, x, w, y, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw);                                    \
+        return conv_fwd<T>(c, x, w, y, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, ws, ws_bytes);                      \
     }                                                                                                                  \
     extern "C" int fx_conv2d_dgrad_##S(fx_ctx* c, const T* g, const T* w, T* dx, int64_t B, int64_t Cin, int64_t H, int64_t W, \
                                        int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,   \

@@ -44,6 +44,8 @@ int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B,
     if (M == 0 || N == 0) return FX_OK;
     FX_REQUIRE(A && B && C, "fx_gemm: null pointer");
     FX_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "fx_gemm: dimension exceeds 2^31");
+    // 32-bit byte offsets inside one 128-row tile of a k-contiguous operand
+    FX_REQUIRE(K * 128 * (i64)sizeof(T) < (1ll << 32), "fx_gemm: K = %lld is too large for this build", (long long)K);
     std::lock_guard<std::mutex> lk(c->launch_mutex);
     if (K == 0) return launch_zero<T>(c, C, M * N);  // empty sum
     if (M >= 128 && N >= 128) return run_trans<T, TileBig>(c, ta, tb, M, N, K, A, B, C);

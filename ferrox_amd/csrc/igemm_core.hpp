@@ -8,14 +8,21 @@
 //     v_mfma_f64_16x16x4_f64;
 //   - the epilogue scatters accumulators to their final layout (row-major matrix, NCHW tensor, or split-K
 //     partial).
-// Global loads for slab i+1 are issued before the MFMA loop of slab i, so their latency hides behind the matrix
-// pipe; two or more blocks are resident per CU so one block's barriers overlap another block's MFMAs.
-// Index arithmetic uses 32-bit tile coordinates (hosts check M, N, K < 2^31) and 64-bit addresses.
+// Loaders are branch-free: an element outside the operand (padding ring, ragged tile edge, K tail) is fetched
+// from a clamped in-range address and replaced by zero afterwards, so all global loads of a slab sit in one basic
+// block and can be scheduled behind the MFMA stream.  Addresses are a wave-uniform 64-bit base plus a 32-bit byte
+// offset per lane (hosts check that the addressed tensor is below 2 GiB and M, N, K below 2^31).
+// Global loads for slab i+1 are issued before the MFMA loop of slab i; LDS is double-buffered so there is one
+// barrier per slab; several blocks are resident per CU so one block's barrier overlaps another block's MFMAs.
 #pragma once
-#include <climits>
 #include <algorithm>
+#include <climits>
 
 #include "common.hpp"
+
+#ifndef FX_KPAD
+#define FX_KPAD 2
+#endif
 
 namespace igemm {
 
@@ -33,6 +40,11 @@ struct FastDiv {
     }
     __device__ __forceinline__ uint32_t div(uint32_t n) const { return (uint32_t)(((uint64_t)__umulhi(n, m) + n) >> s); }
 };
+
+// Load from a wave-uniform base plus a 32-bit unsigned byte offset.
+template <typename T> __device__ __forceinline__ T ldg(const T* base, uint32_t byteoff) {
+    return *reinterpret_cast<const T*>(reinterpret_cast<const char*>(base) + byteoff);
+}
 
 template <typename T> struct Mfma;
 template <> struct Mfma<float> {
@@ -63,7 +75,7 @@ template <int BM_, int BN_, int BK_, int WM_, int WN_> struct Tile {
 template <int BMN, int BK, int NT, bool KMAJOR> struct SlabMap {
     static constexpr int CNT = BMN * BK / NT;
     static constexpr int STEP = KMAJOR ? NT / BK : NT / BMN;
-    static constexpr int LD = KMAJOR ? BMN + 1 : BMN;  // LDS row pitch; +1 spreads the transposing writes over banks
+    static constexpr int LD = KMAJOR ? BMN + FX_KPAD : BMN;  // LDS row pitch; the pad spreads the transposing writes over banks
     static_assert(BMN * BK % NT == 0, "slab must divide evenly over the block");
     static_assert(KMAJOR ? (NT % BK == 0) : (NT % BMN == 0 && BMN % 64 == 0), "unsupported tile/thread shape");
     static __device__ __forceinline__ int k_of(int tid, int i) { return KMAJOR ? tid % BK : tid / BMN + i * STEP; }
@@ -83,25 +95,49 @@ template <typename T, bool KMAJOR_> struct MatLoader {
     int MN;
     template <int BMN, int BK, int NT> struct Dev {
         typedef SlabMap<BMN, BK, NT, KMAJOR_> Map;
-        const T* p; i64 ld; int MN, origin, tid;
-        __device__ __forceinline__ Dev(const MatLoader& L, int origin_, int tid_) : p(L.p), ld(L.ld), MN(L.MN), origin(origin_), tid(tid_) {}
-        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) const {
+        const T* base;          // wave-uniform: first row (KMAJOR) / first column (otherwise) of this block's tile
+        i64 ld;
+        uint32_t off[KMAJOR_ ? Map::CNT : 1];  // byte offsets from base (rows clamped into the matrix)
+        uint32_t okmask;        // bit i: register i addresses a row/column inside the matrix
+        int klane, krow;
+        __device__ __forceinline__ Dev(const MatLoader& L, int origin, int tid) : ld(L.ld) {
+            okmask = 0;
             if (KMAJOR_) {
-                const int k = k0 + tid % BK;
-                const bool kok = k < kend;
+                base = L.p + (i64)origin * L.ld;
+                klane = tid % BK;
+                krow = 0;
 #pragma unroll
                 for (int i = 0; i < Map::CNT; ++i) {
-                    const int mn = origin + Map::mn_of(tid, i);
-                    r[i] = (kok && mn < MN) ? p[(i64)mn * ld + k] : T(0);
+                    const int r = Map::mn_of(tid, i);
+                    const bool ok = origin + r < L.MN;
+                    okmask |= ok ? (1u << i) : 0u;
+                    off[i] = (uint32_t)(((ok ? r : 0) * (uint32_t)L.ld + klane) * sizeof(T));
                 }
             } else {
-                const int mn = origin + tid % BMN;
-                const bool ok = mn < MN;
-                const int krow = __builtin_amdgcn_readfirstlane(tid / BMN);
+                base = L.p + origin;
+                const int r = tid % BMN;
+                const bool ok = origin + r < L.MN;
+                okmask = ok ? ~0u : 0u;
+                off[0] = (uint32_t)((ok ? r : 0) * sizeof(T));
+                klane = 0;
+                krow = __builtin_amdgcn_readfirstlane(tid / BMN);
+            }
+        }
+        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) const {
+            if (KMAJOR_) {
+                const bool kok = k0 + klane < kend;
+                const T* b = base + k0;  // uniform
+#pragma unroll
+                for (int i = 0; i < Map::CNT; ++i) r[i] = ldg(b, kok ? off[i] : 0u);
+#pragma unroll
+                for (int i = 0; i < Map::CNT; ++i) r[i] = (kok && ((okmask >> i) & 1u)) ? r[i] : T(0);
+            } else {
 #pragma unroll
                 for (int i = 0; i < Map::CNT; ++i) {
-                    const int k = k0 + krow + i * Map::STEP;
-                    r[i] = (ok && k < kend) ? p[(i64)k * ld + mn] : T(0);
+                    const int k = k0 + krow + i * Map::STEP;       // uniform
+                    const int kc = min(k, kend - 1);               // clamped row stays inside the split
+                    r[i] = ldg(base + (i64)kc * ld, off[0]);
+                    r[i] = (k < kend && okmask) ? r[i] : T(0);
                 }
             }
         }
@@ -111,86 +147,126 @@ template <typename T, bool KMAJOR_> struct MatLoader {
 // ---- convolution geometry shared by the conv loaders -------------------------------------------------------
 struct ConvShape {
     int B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, oh, ow;
-    FastDiv div_L, div_ow, div_KK, div_kw, div_HW, div_W, div_sh, div_sw;
+    FastDiv div_L, div_ow, div_KK, div_kw, div_HW, div_W, div_sh, div_sw, div_Cin, div_Cout;
 };
 
-// Forward B operand: B(k = (c,ky,kx), n = (b,oy,ox)) = x[b, c, oy*sh + ky - ph, ox*sw + kx - pw] (0 outside).
+// Forward B operand: B(k, n = (b,oy,ox)) = x[b, c, oy*sh + ky - ph, ox*sw + kx - pw] (0 outside the image).
 // Contiguous along n.  The pixel of a thread is fixed for the whole kernel; k is wave-uniform.
-template <typename T> struct ConvFwdB {
+//  FAST  : k = (ky*kw + kx)*Cin + c with Cin % BK == 0 (the host permutes the weights to match): all BK rows of a
+//          slab share (ky,kx), so the bounds test is done once per slab and rows differ by a uniform H*W stride.
+//  !FAST : k = (c*kh + ky)*kw + kx as in the reference im2col; every row decodes its own (c,ky,kx).
+template <typename T, bool FAST> struct ConvFwdB {
     static constexpr bool KMAJOR = false;
     const T* x;
     ConvShape s;
     int N;
     template <int BMN, int BK, int NT> struct Dev {
         typedef SlabMap<BMN, BK, NT, false> Map;
-        const T* base; const ConvShape& s; int iy0, ix0, krow; bool ok;
-        __device__ __forceinline__ Dev(const ConvFwdB& L, int origin, int tid) : s(L.s) {
+        const T* x; const ConvShape& s; int pix, iy0, ix0, krow; bool ok;
+        __device__ __forceinline__ Dev(const ConvFwdB& L, int origin, int tid) : x(L.x), s(L.s) {
             const int n = origin + tid % BMN;
             ok = n < L.N;
             const uint32_t nn = ok ? n : 0;
             const uint32_t b = s.div_L.div(nn), l = nn - b * (s.oh * s.ow);
             const uint32_t oy = s.div_ow.div(l), ox = l - oy * s.ow;
-            base = L.x + (i64)b * s.Cin * s.H * s.W;
             iy0 = (int)oy * s.sh - s.ph;
             ix0 = (int)ox * s.sw - s.pw;
+            pix = (((int)b * s.Cin * s.H + iy0) * s.W + ix0) * (int)sizeof(T);  // signed byte offset of tap (c=0,ky=0,kx=0)
             krow = __builtin_amdgcn_readfirstlane(tid / BMN);
         }
         __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) const {
-            const int KK = s.kh * s.kw;
+            const int HW = s.H * s.W;
+            if (FAST) {
+                const uint32_t kyx = s.div_Cin.div(k0), c0 = k0 - kyx * s.Cin;
+                const uint32_t ky = s.div_kw.div(kyx), kx = kyx - ky * s.kw;
+                const bool in = ok && (unsigned)(iy0 + (int)ky) < (unsigned)s.H && (unsigned)(ix0 + (int)kx) < (unsigned)s.W;
+                const int uni = (((int)c0 + krow) * HW + (int)ky * s.W + (int)kx) * (int)sizeof(T);
+                const uint32_t v = in ? (uint32_t)(pix + uni) : 0u;
 #pragma unroll
-            for (int i = 0; i < Map::CNT; ++i) {
-                const int k = k0 + krow + i * Map::STEP;
-                const uint32_t c = s.div_KK.div(k), rr = k - c * KK;
-                const uint32_t ky = s.div_kw.div(rr), kx = rr - ky * s.kw;
-                const int iy = iy0 + (int)ky, ix = ix0 + (int)kx;
-                const bool in = ok && k < kend && (unsigned)iy < (unsigned)s.H && (unsigned)ix < (unsigned)s.W;
-                r[i] = in ? base[((int)c * s.H + iy) * s.W + ix] : T(0);
+                for (int i = 0; i < Map::CNT; ++i) r[i] = ldg(x, v + (uint32_t)(i * Map::STEP * HW * (int)sizeof(T)));
+#pragma unroll
+                for (int i = 0; i < Map::CNT; ++i) r[i] = in ? r[i] : T(0);
+            } else {
+                const int KK = s.kh * s.kw;
+                bool in[Map::CNT];
+#pragma unroll
+                for (int i = 0; i < Map::CNT; ++i) {
+                    const int k = k0 + krow + i * Map::STEP;
+                    const uint32_t c = s.div_KK.div(k), rr = k - c * KK;
+                    const uint32_t ky = s.div_kw.div(rr), kx = rr - ky * s.kw;
+                    in[i] = ok && k < kend && (unsigned)(iy0 + (int)ky) < (unsigned)s.H && (unsigned)(ix0 + (int)kx) < (unsigned)s.W;
+                    const int uni = ((int)c * HW + (int)ky * s.W + (int)kx) * (int)sizeof(T);
+                    r[i] = ldg(x, in[i] ? (uint32_t)(pix + uni) : 0u);
+                }
+#pragma unroll
+                for (int i = 0; i < Map::CNT; ++i) r[i] = in[i] ? r[i] : T(0);
             }
         }
     };
 };
 
-// Data-gradient B operand: B(k = (oc,ky,kx), n = (b,y,x)) = g[b, oc, (y+ph-ky)/sh, (x+pw-kx)/sw] when both
-// quotients are exact and inside the output plane, else 0.  This is the gather form of col2im: every input pixel
-// is owned by exactly one accumulator, so there are no races and no atomics.
-template <typename T> struct ConvDgradB {
+// Data-gradient B operand: B(k, n = (b,y,x)) = g[b, oc, (y+ph-ky)/sh, (x+pw-kx)/sw] when both quotients are exact
+// and inside the output plane, else 0.  This is the gather form of col2im: every input pixel is owned by exactly
+// one accumulator, so there are no races and no atomics.
+//  FAST  : k = (ky*kw + kx)*Cout + oc with Cout % BK == 0;  !FAST : k = (oc*kh + ky)*kw + kx.
+template <typename T, bool FAST> struct ConvDgradB {
     static constexpr bool KMAJOR = false;
     const T* g;
     ConvShape s;
     int N;  // B*H*W
     template <int BMN, int BK, int NT> struct Dev {
         typedef SlabMap<BMN, BK, NT, false> Map;
-        const T* base; const ConvShape& s; int yp, xp, krow; bool ok;
-        __device__ __forceinline__ Dev(const ConvDgradB& L, int origin, int tid) : s(L.s) {
+        const T* g; const ConvShape& s; int img, yp, xp, krow; bool ok;
+        __device__ __forceinline__ Dev(const ConvDgradB& L, int origin, int tid) : g(L.g), s(L.s) {
             const int n = origin + tid % BMN;
             ok = n < L.N;
             const uint32_t nn = ok ? n : 0;
             const uint32_t b = s.div_HW.div(nn), p = nn - b * (s.H * s.W);
             const uint32_t y = s.div_W.div(p), x = p - y * s.W;
-            base = L.g + (i64)b * s.Cout * s.oh * s.ow;
+            img = (int)b * s.Cout * s.oh * s.ow * (int)sizeof(T);
             yp = (int)y + s.ph;
             xp = (int)x + s.pw;
             krow = __builtin_amdgcn_readfirstlane(tid / BMN);
         }
+        // byte offset of g[b, 0, cy, cx] for tap (ky,kx); `in` false when the tap does not reach the output plane
+        __device__ __forceinline__ int tap(int ky, int kx, bool& in) const {
+            const int ty = yp - ky, tx = xp - kx;
+            in = ok && ty >= 0 && tx >= 0;
+            int cy = ty, cx = tx;
+            if (!(s.sh == 1 && s.sw == 1)) {
+                cy = (int)s.div_sh.div(in ? (uint32_t)ty : 0u);
+                cx = (int)s.div_sw.div(in ? (uint32_t)tx : 0u);
+                in = in && cy * s.sh == ty && cx * s.sw == tx;
+            }
+            in = in && cy < s.oh && cx < s.ow;
+            return img + (cy * s.ow + cx) * (int)sizeof(T);
+        }
         __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) const {
-            const int KK = s.kh * s.kw;
-            const bool unit = (s.sh == 1 && s.sw == 1);
+            const int L = s.oh * s.ow;
+            if (FAST) {
+                const uint32_t kyx = s.div_Cout.div(k0), oc0 = k0 - kyx * s.Cout;
+                const uint32_t ky = s.div_kw.div(kyx), kx = kyx - ky * s.kw;
+                bool in;
+                const int t = tap((int)ky, (int)kx, in);
+                const uint32_t v = in ? (uint32_t)(t + ((int)oc0 + krow) * L * (int)sizeof(T)) : 0u;
 #pragma unroll
-            for (int i = 0; i < Map::CNT; ++i) {
-                const int k = k0 + krow + i * Map::STEP;
-                const uint32_t oc = s.div_KK.div(k), rr = k - oc * KK;
-                const uint32_t ky = s.div_kw.div(rr), kx = rr - ky * s.kw;
-                const int ty = yp - (int)ky, tx = xp - (int)kx;
-                bool in = ok && k < kend && ty >= 0 && tx >= 0;
-                int cy = ty, cx = tx;
-                if (!unit) {
-                    const uint32_t uy = in ? (uint32_t)ty : 0u, ux = in ? (uint32_t)tx : 0u;
-                    cy = (int)s.div_sh.div(uy);
-                    cx = (int)s.div_sw.div(ux);
-                    in = in && (cy * s.sh == ty) && (cx * s.sw == tx);
+                for (int i = 0; i < Map::CNT; ++i) r[i] = ldg(g, v + (uint32_t)(i * Map::STEP * L * (int)sizeof(T)));
+#pragma unroll
+                for (int i = 0; i < Map::CNT; ++i) r[i] = in ? r[i] : T(0);
+            } else {
+                const int KK = s.kh * s.kw;
+                bool in[Map::CNT];
+#pragma unroll
+                for (int i = 0; i < Map::CNT; ++i) {
+                    const int k = k0 + krow + i * Map::STEP;
+                    const uint32_t oc = s.div_KK.div(k), rr = k - oc * KK;
+                    const uint32_t ky = s.div_kw.div(rr), kx = rr - ky * s.kw;
+                    const int t = tap((int)ky, (int)kx, in[i]);
+                    in[i] = in[i] && k < kend;
+                    r[i] = ldg(g, in[i] ? (uint32_t)(t + (int)oc * L * (int)sizeof(T)) : 0u);
                 }
-                in = in && cy < s.oh && cx < s.ow;
-                r[i] = in ? base[((int)oc * s.oh + cy) * s.ow + cx] : T(0);
+#pragma unroll
+                for (int i = 0; i < Map::CNT; ++i) r[i] = in[i] ? r[i] : T(0);
             }
         }
     };
@@ -203,20 +279,32 @@ template <typename T> struct ConvWgradA {
     ConvShape s;
     template <int BMN, int BK, int NT> struct Dev {
         typedef SlabMap<BMN, BK, NT, true> Map;
-        const T* g; const ConvShape& s; int origin, tid;
-        __device__ __forceinline__ Dev(const ConvWgradA& L, int origin_, int tid_) : g(L.g), s(L.s), origin(origin_), tid(tid_) {}
-        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) const {
-            const int k = k0 + tid % BK;
-            const bool kok = k < kend;
-            const int L = s.oh * s.ow;
-            const uint32_t kk = kok ? k : 0;
-            const uint32_t b = s.div_L.div(kk), l = kk - b * L;
-            const T* p = g + (i64)b * s.Cout * L + l;
+        const T* g; const ConvShape& s; int klane;
+        uint32_t moff[Map::CNT];  // oc * L * sizeof(T), oc clamped into range
+        uint32_t okmask;
+        __device__ __forceinline__ Dev(const ConvWgradA& L, int origin, int tid) : g(L.g), s(L.s) {
+            klane = tid % BK;
+            okmask = 0;
+            const int Lp = s.oh * s.ow;
 #pragma unroll
             for (int i = 0; i < Map::CNT; ++i) {
                 const int m = origin + Map::mn_of(tid, i);
-                r[i] = (kok && m < s.Cout) ? p[(i64)m * L] : T(0);
+                const bool ok = m < s.Cout;
+                okmask |= ok ? (1u << i) : 0u;
+                moff[i] = (uint32_t)((ok ? m : 0) * Lp * (int)sizeof(T));
             }
+        }
+        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) const {
+            const int k = k0 + klane;
+            const bool kok = k < kend;
+            const int L = s.oh * s.ow;
+            const uint32_t kk = kok ? k : (uint32_t)k0;  // k0 < kend always
+            const uint32_t b = s.div_L.div(kk), l = kk - b * L;
+            const uint32_t v = (b * (uint32_t)s.Cout * L + l) * (uint32_t)sizeof(T);
+#pragma unroll
+            for (int i = 0; i < Map::CNT; ++i) r[i] = ldg(g, v + moff[i]);
+#pragma unroll
+            for (int i = 0; i < Map::CNT; ++i) r[i] = (kok && ((okmask >> i) & 1u)) ? r[i] : T(0);
         }
     };
 };
@@ -230,10 +318,11 @@ template <typename T> struct ConvWgradB {
     int N;  // Cin*kh*kw
     template <int BMN, int BK, int NT> struct Dev {
         typedef SlabMap<BMN, BK, NT, true> Map;
-        const T* x; const ConvShape& s; int tid;
-        int off[Map::CNT];   // c*H*W + (ky-ph)*W + (kx-pw)
+        const T* x; const ConvShape& s; int klane;
+        int off[Map::CNT];   // (c*H*W + (ky-ph)*W + (kx-pw)) * sizeof(T)
         int kyx[Map::CNT];   // (ky-ph) << 16 | ((kx-pw) & 0xffff); INT_MIN when the column is out of range
-        __device__ __forceinline__ Dev(const ConvWgradB& L, int origin, int tid_) : x(L.x), s(L.s), tid(tid_) {
+        __device__ __forceinline__ Dev(const ConvWgradB& L, int origin, int tid) : x(L.x), s(L.s) {
+            klane = tid % BK;
             const int KK = s.kh * s.kw;
 #pragma unroll
             for (int i = 0; i < Map::CNT; ++i) {
@@ -242,8 +331,8 @@ template <typename T> struct ConvWgradB {
                     const uint32_t c = s.div_KK.div(n), rr = n - c * KK;
                     const uint32_t ky = s.div_kw.div(rr), kx = rr - ky * s.kw;
                     const int dy = (int)ky - s.ph, dx = (int)kx - s.pw;
-                    off[i] = ((int)c * s.H + dy) * s.W + dx;
-                    kyx[i] = (dy << 16) | (dx & 0xffff);
+                    off[i] = (((int)c * s.H + dy) * s.W + dx) * (int)sizeof(T);
+                    kyx[i] = (int)(((uint32_t)dy << 16) | ((uint32_t)dx & 0xffffu));
                 } else {
                     off[i] = 0;
                     kyx[i] = INT_MIN;
@@ -251,46 +340,51 @@ template <typename T> struct ConvWgradB {
             }
         }
         __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) const {
-            const int k = k0 + tid % BK;
+            const int k = k0 + klane;
             const bool kok = k < kend;
-            const uint32_t kk = kok ? k : 0;
+            const uint32_t kk = kok ? k : (uint32_t)k0;
             const int L = s.oh * s.ow;
             const uint32_t b = s.div_L.div(kk), l = kk - b * L;
             const uint32_t oy = s.div_ow.div(l), ox = l - oy * s.ow;
             const int y0 = (int)oy * s.sh, x0 = (int)ox * s.sw;
-            const T* p = x + (i64)b * s.Cin * s.H * s.W + y0 * s.W + x0;
+            const int pix = (((int)b * s.Cin * s.H + y0) * s.W + x0) * (int)sizeof(T);
+            bool in[Map::CNT];
 #pragma unroll
             for (int i = 0; i < Map::CNT; ++i) {
                 const int dy = kyx[i] >> 16, dx = (int)(short)(kyx[i] & 0xffff);
-                const bool in = kok && kyx[i] != INT_MIN && (unsigned)(y0 + dy) < (unsigned)s.H && (unsigned)(x0 + dx) < (unsigned)s.W;
-                r[i] = in ? p[off[i]] : T(0);
+                in[i] = kok && kyx[i] != INT_MIN && (unsigned)(y0 + dy) < (unsigned)s.H && (unsigned)(x0 + dx) < (unsigned)s.W;
+                r[i] = ldg(x, in[i] ? (uint32_t)(pix + off[i]) : 0u);
             }
+#pragma unroll
+            for (int i = 0; i < Map::CNT; ++i) r[i] = in[i] ? r[i] : T(0);
         }
     };
 };
 
 // ---- epilogues ---------------------------------------------------------------------------------------------
+// An epilogue maps a column n to a base pointer (col) and stores row m at q[m * row_stride].
 // Row-major matrix (also used for split-K partials: split z goes to p + z*split_stride).
 template <typename T> struct MatStore {
     T* p;
     i64 ld, split_stride;
     int M, N;
-    struct Col { T* q; };
-    __device__ __forceinline__ Col col(int n, int split) const { return Col{n < N ? p + (i64)split * split_stride + n : nullptr}; }
-    __device__ __forceinline__ void put(const Col& c, int m, T v) const { if (c.q && m < M) c.q[(i64)m * ld] = v; }
+    __device__ __forceinline__ int rows() const { return M; }
+    __device__ __forceinline__ int cols() const { return N; }
+    __device__ __forceinline__ i64 row_stride() const { return ld; }
+    __device__ __forceinline__ T* col(int n, int split) const { return p + (i64)split * split_stride + n; }
 };
 // NCHW tensor: row m = channel, column n = (b, l) -> p[(b*C + m)*L + l].
 template <typename T> struct NchwStore {
     T* p;
     int C, L, N;
     FastDiv div_L;
-    struct Col { T* q; };
-    __device__ __forceinline__ Col col(int n, int) const {
-        if (n >= N) return Col{nullptr};
+    __device__ __forceinline__ int rows() const { return C; }
+    __device__ __forceinline__ int cols() const { return N; }
+    __device__ __forceinline__ i64 row_stride() const { return L; }
+    __device__ __forceinline__ T* col(int n, int) const {
         const uint32_t b = div_L.div(n), l = n - b * L;
-        return Col{p + (i64)b * C * L + l};
+        return p + (i64)b * C * L + l;
     }
-    __device__ __forceinline__ void put(const Col& c, int m, T v) const { if (c.q && m < C) c.q[(i64)m * L] = v; }
 };
 
 // ---- the kernel -------------------------------------------------------------------------------------------
@@ -306,8 +400,10 @@ __global__ __launch_bounds__(Cfg::NT) void igemm_kernel(AL al, BL bl, EP ep, int
     typedef typename ADev::Map AMap;
     typedef typename BDev::Map BMap;
 
-    __shared__ T As[BK * AMap::LD];
-    __shared__ T Bs[BK * BMap::LD];
+    // Two LDS stages: while the MFMA loop reads stage `cur`, the next slab (already in registers) is written to the
+    // other stage, so one barrier per slab suffices.
+    __shared__ T As[2][BK * AMap::LD];
+    __shared__ T Bs[2][BK * BMap::LD];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bm = blockIdx.y * BM, bn = blockIdx.x * BN, split = blockIdx.z;
@@ -328,49 +424,84 @@ __global__ __launch_bounds__(Cfg::NT) void igemm_kernel(AL al, BL bl, EP ep, int
     T ra[AMap::CNT], rb[BMap::CNT];
     ad.load(kbeg, kend, ra);
     bd.load(kbeg, kend, rb);
+    AMap::store(As[0], ra, tid);
+    BMap::store(Bs[0], rb, tid);
+    __syncthreads();
 
     const int lrow = lane / MF::BLK, lcol = lane % MF::BLK;
+    int cur = 0;
     for (int k0 = kbeg; k0 < kend; k0 += BK) {
-        __syncthreads();  // everyone is done reading the previous slab
-        AMap::store(As, ra, tid);
-        BMap::store(Bs, rb, tid);
-        __syncthreads();
-        if (k0 + BK < kend) {  // prefetch the next slab; latency hides behind the MFMA loop below
+        const bool more = k0 + BK < kend;
+        if (more) {  // global loads for the next slab fly while this slab is multiplied
             ad.load(k0 + BK, kend, ra);
             bd.load(k0 + BK, kend, rb);
         }
+        const T* Ac = As[cur] + lrow * AMap::LD + wm0 + lcol;
+        const T* Bc = Bs[cur] + lrow * BMap::LD + wn0 + lcol;
 #pragma unroll
         for (int kk = 0; kk < BK; kk += MF::KSTEP) {
             T a[TM], b[TN];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) a[i] = As[(kk + lrow) * AMap::LD + wm0 + i * MF::BLK + lcol];
+            for (int i = 0; i < TM; ++i) a[i] = Ac[kk * AMap::LD + i * MF::BLK];
 #pragma unroll
-            for (int j = 0; j < TN; ++j) b[j] = Bs[(kk + lrow) * BMap::LD + wn0 + j * MF::BLK + lcol];
+            for (int j = 0; j < TN; ++j) b[j] = Bc[kk * BMap::LD + j * MF::BLK];
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) acc[i][j] = MF::mma(a[i], b[j], acc[i][j]);
         }
+        if (more) {
+            AMap::store(As[cur ^ 1], ra, tid);
+            BMap::store(Bs[cur ^ 1], rb, tid);
+        }
+        __syncthreads();
+        cur ^= 1;
     }
 
+    const int M = ep.rows(), N = ep.cols();
+    const i64 rs = ep.row_stride();
+    if (bm + BM <= M && bn + BN <= N) {  // interior tile: no edge tests
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int n = bn + wn0 + j * MF::BLK + lcol;
-        const typename EP::Col cc = ep.col(n, split);
+        for (int j = 0; j < TN; ++j) {
+            T* q = ep.col(bn + wn0 + j * MF::BLK + lcol, split) + (i64)(bm + wm0) * rs;
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int e = 0; e < MF::NACC; ++e) ep.put(cc, bm + wm0 + i * MF::BLK + MF::row(e, lane), acc[i][j][e]);
+                for (int e = 0; e < MF::NACC; ++e) q[(i64)(i * MF::BLK + MF::row(e, lane)) * rs] = acc[i][j][e];
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = bn + wn0 + j * MF::BLK + lcol;
+            if (n < N) {
+                T* q = ep.col(n, split);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int e = 0; e < MF::NACC; ++e) {
+                        const int m = bm + wm0 + i * MF::BLK + MF::row(e, lane);
+                        if (m < M) q[(i64)m * rs] = acc[i][j][e];
+                    }
+            }
+        }
     }
 }
 
-// Sums split-K partials in split order (deterministic) into the final buffer.
+// Sums split-K partials in split order (deterministic) into the final buffer; 8 independent loads in flight.
 template <typename T>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const T* __restrict__ part, T* __restrict__ out, i64 n, int splits) {
     const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
-    T s = part[i];
-    for (int z = 1; z < splits; ++z) s = s + part[(i64)z * n + i];
+    T s = T(0);
+    int z = 0;
+    for (; z + 8 <= splits; z += 8) {
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = part[(i64)(z + u) * n + i];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s = s + v[u];
+    }
+    for (; z < splits; ++z) s = s + part[(i64)z * n + i];
     out[i] = s;
 }
 
@@ -378,6 +509,7 @@ template <typename T, class Cfg, class AL, class BL, class EP>
 int launch(fx_ctx* c, const AL& al, const BL& bl, const EP& ep, i64 M, i64 N, i64 K, int splits, int kps) {
     const i64 gx = fx::ceil_div(N, Cfg::BN), gy = fx::ceil_div(M, Cfg::BM);
     FX_REQUIRE(gx <= 0x7fffffff && gy <= 65535 && splits >= 1 && splits <= 65535, "implicit GEMM grid out of range");
+    FX_REQUIRE(K >= 1, "implicit GEMM needs K >= 1");
     igemm_kernel<T, Cfg, AL, BL, EP><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)splits), dim3(Cfg::NT), 0, c->stream>>>(
         al, bl, ep, (int)K, kps);
     FX_LAUNCH_CHECK();
@@ -428,6 +560,8 @@ inline ConvShape make_shape(i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 
     s.div_W = FastDiv((uint32_t)W);
     s.div_sh = FastDiv((uint32_t)sh);
     s.div_sw = FastDiv((uint32_t)sw);
+    s.div_Cin = FastDiv((uint32_t)Cin);
+    s.div_Cout = FastDiv((uint32_t)Cout);
     return s;
 }
 
