@@ -34,6 +34,8 @@ typedef Tile<64, 256, 16, 64, 64> TileM64N256;
 typedef Tile<64, 256, 32, 64, 64> TileM64N256K32;
 typedef Tile<128, 192, 16, 64, 96> TileN192;
 typedef Tile<128, 192, 32, 64, 96> TileN192K32;
+typedef Tile<128, 64, 16, 64, 32> TileN64;
+typedef Tile<128, 64, 32, 64, 32> TileN64K32;
 static int variant() { const char* v = getenv("FX_CONV_VARIANT"); return v ? atoi(v) : 0; }
 
 int gemm_t(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const float* A, const float* B, float* C) { return fx_gemm_f32(c, ta, tb, M, N, K, A, B, C); }
@@ -246,8 +248,8 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
                (long long)ws_bytes, (long long)need);
     std::lock_guard<std::mutex> lk(c->launch_mutex);
     if constexpr (sizeof(T) == 4) if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64 && variant() == 1) return wgrad_tile<T, TileM128K32>(c, x, g, dw, d, mode, ws);
-    if constexpr (sizeof(T) == 4) if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64 && variant() == 2) return wgrad_tile<T, TileN192>(c, x, g, dw, d, mode, ws);
-    if constexpr (sizeof(T) == 4) if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64 && variant() == 3) return wgrad_tile<T, TileN192K32>(c, x, g, dw, d, mode, ws);
+    if constexpr (sizeof(T) == 4) if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64 && variant() == 2) return wgrad_tile<T, TileN64>(c, x, g, dw, d, mode, ws);
+    if constexpr (sizeof(T) == 4) if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64 && variant() == 3) return wgrad_tile<T, TileN64K32>(c, x, g, dw, d, mode, ws);
     if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64) return wgrad_tile<T, TileM128>(c, x, g, dw, d, mode, ws);
     return wgrad_tile<T, TileSmall>(c, x, g, dw, d, mode, ws);
 }

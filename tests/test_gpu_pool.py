@@ -1,0 +1,142 @@
+"""The hipMalloc caching allocator behind fx_alloc/fx_free, replaying the traces of tests/test_pool_oracle.py on
+the GPU and checking every counter against the oracle state machine step by step."""
+import ctypes as C
+import random
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def make_cfg(capi, buckets, literal):
+    cfg = capi.PoolConfig()
+    cfg.n_buckets = len(buckets)
+    cfg.literal_ids = int(literal)
+    for i, (lo, hi, cap, ev, th) in enumerate(buckets):
+        cfg.buckets[i] = capi.BucketConfig(lo, hi, cap, ev, th)
+    return cfg
+
+
+class GpuPool:
+    """fx_alloc/fx_free through the raw C ABI, f32 pool."""
+
+    def __init__(self, capi, buckets, literal):
+        self.capi = capi
+        self.ctx = capi.Context(0, make_cfg(capi, buckets, literal) if buckets is not None else None)
+
+    def alloc(self, n):
+        capi = self.capi
+        ptr, granted, aid = C.c_void_p(), C.c_int64(0), C.c_uint64(0)
+        capi.check(capi.lib.fx_alloc(self.ctx.h, capi.FX_F32, n, C.byref(ptr), C.byref(granted), C.byref(aid)))
+        return ptr.value, granted.value, aid.value
+
+    def free(self, ptr, aid):
+        self.capi.check(self.capi.lib.fx_free(self.ctx.h, self.capi.FX_F32, ptr, aid))
+
+    def stats(self):
+        return self.ctx.pool_stats()
+
+    def close(self):
+        self.ctx.close()
+
+
+SMALL = [(1, 10, 3, 2, -1), (11, 100, 2, 1, -1)]
+KEYS = ("total_allocations", "active_allocations", "pool_hits", "pool_misses", "underflow_misses", "active_table_len",
+        "device_allocs", "device_frees")
+
+
+@pytest.mark.parametrize("literal", [True, False])
+def test_random_trace_matches_oracle_counters(literal):
+    import oracle as orc
+    from ferrox_amd import capi
+    rng = random.Random(7)
+    gp = GpuPool(capi, SMALL, literal)
+    op = orc.Pool(SMALL, literal=literal)
+    live = []  # (ptr, granted, gpu_id, oracle_id)
+    try:
+        for step in range(400):
+            if live and rng.random() < 0.5:
+                ptr, granted, gid, oid = live.pop(rng.randrange(len(live)))
+                gp.free(ptr, gid)
+                op.free(granted, oid)
+            else:
+                n = rng.choice([1, 2, 5, 9, 10, 11, 40, 100])
+                ptr, granted, gid = gp.alloc(n)
+                og, oid = op.alloc(n)
+                assert (granted, gid) == (og, oid), step
+                live.append((ptr, granted, gid, oid))
+            gs, os_ = gp.stats(), op.stats()
+            assert {k: gs[k] for k in KEYS} == {k: os_[k] for k in KEYS}, step
+            for b in range(2):
+                gb, ob = gp.ctx.bucket_stats(b), op.bucket_stats(b)
+                assert (gb["pooled_blocks"], gb["total_allocations"], gb["total_evictions"], gb["av_allocations"],
+                        gb["max_allocations"]) == (ob["pooled"], ob["total_allocations"], ob["total_evictions"],
+                                                   ob["av_allocations"], ob["max_allocations"]), (step, b)
+    finally:
+        gp.close()
+
+
+def test_zero_size_and_unroutable_size_are_errors():
+    from ferrox_amd import capi
+    gp = GpuPool(capi, SMALL, False)
+    try:
+        with pytest.raises(capi.FerroxHipError, match="Cannot allocate zero-sized CUDA memory"):
+            gp.alloc(0)
+        with pytest.raises(capi.FerroxHipError, match="No bucket configured for allocation size 101"):
+            gp.alloc(101)
+        with pytest.raises(capi.FerroxHipError, match="not owned by this pool"):
+            gp.free(12345, 1)
+    finally:
+        gp.close()
+
+
+def test_default_config_hit_rate_in_a_training_like_loop():
+    """Steady-state reuse with the default buckets: released in reverse creation order (LIFO) every request is a
+    hit after the first pass; released in creation order the reference's pop-most-recent policy produces underflow
+    misses inside a bucket, exactly as the oracle state machine predicts."""
+    import oracle as orc
+    from ferrox_amd import capi
+    sizes = [10, 256 * 10, 256 * 128, 256 * 256, 784 * 256, 256 * 16384]
+    ctx = capi.Context(0)
+    try:
+        for it in range(20):
+            bufs = [ctx.empty((n,)) for n in sizes]
+            for b in reversed(bufs):
+                b.free()
+        st = ctx.pool_stats()
+        assert st["pool_misses"] == len(sizes) and st["pool_hits"] == 19 * len(sizes) and st["underflow_misses"] == 0
+        assert st["device_allocs"] == len(sizes) and st["bytes_in_use"] == 0
+        ctx.pool_cleanup()
+        st = ctx.pool_stats()
+        assert st["bytes_pooled"] == 0 and st["device_frees"] == len(sizes)
+    finally:
+        ctx.close()
+    ctx = capi.Context(0)
+    op = orc.Pool(literal=False)
+    try:
+        for it in range(10):
+            bufs = [ctx.empty((n,)) for n in sizes]
+            obufs = [op.alloc(n) for n in sizes]
+            for b, (og, oid) in zip(bufs, obufs):
+                assert b.granted == og
+                b.free()
+                op.free(og, oid)
+        gs, os_ = ctx.pool_stats(), op.stats()
+        assert {k: gs[k] for k in KEYS} == {k: os_[k] for k in KEYS}
+        assert gs["underflow_misses"] > 0
+    finally:
+        ctx.close()
+
+
+def test_reused_block_is_not_zeroed_but_usable():
+    from ferrox_amd import capi
+    with capi.Context(0) as ctx:
+        a = ctx.upload(np.arange(1000, dtype=np.float32))
+        ptr = a.ptr
+        a.free()
+        b = ctx.empty((1000,))
+        assert b.ptr == ptr                          # LIFO reuse of the most recently returned block
+        assert np.array_equal(b.numpy(), np.arange(1000, dtype=np.float32))  # dirty on purpose (context.rs:72-73)
+        c = ctx.fill((1000,), 3.0)
+        assert np.all(c.numpy() == 3.0)
