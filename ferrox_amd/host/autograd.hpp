@@ -1,0 +1,600 @@
+// Host-side callers of the storage backend, mirrored from the reference so that one training step issues the same
+// sequence of storage calls (and therefore the same kernels and pool traffic) as Ferrox does:
+//   Operator<T>          src/ops/mod.rs:16-49  and the operators of src/ops/{basic,matrix,unary,reduction,reshape,
+//                        comparison,batched}.rs that the MLP / CNN configs exercise
+//   AutoFerroxEngine<T>  src/graph/mod.rs:341-997  (eager tape: apply_operation, backward, accumulate_gradient)
+//   Linear, Conv2d, ReLU, Flatten   src/nn/layers/{linear,conv2d,activation,pooling}.rs
+//   CCELoss              src/nn/losses/classification.rs:191-257
+//   SGD, Adam            src/nn/optim/{sgd,adam}.rs
+// With `literal_engine` the engine also performs the reference's per-node deep clone in backward_node
+// (src/graph/mod.rs:735-751: get_node_owned clones the node and its tensor just to read its inputs); without it
+// that redundant device copy is skipped.  Everything else is issued exactly as the reference issues it.
+#pragma once
+#include <cmath>
+#include <functional>
+#include <map>
+#include <set>
+
+#include "hip_storage.hpp"
+
+namespace ferrox {
+
+template <typename T> using TensorRefs = std::vector<const HipStorage<T>*>;
+
+// ---- Operator: src/ops/mod.rs:16-49 ---------------------------------------------------------------------------
+template <typename T> struct Operator {
+    virtual ~Operator() = default;
+    virtual Tensor<T> compute(const TensorRefs<T>& inputs) const = 0;
+    virtual std::vector<Tensor<T>> gradient(Tensor<T> grad_output, const TensorRefs<T>& inputs, const HipStorage<T>* output) const = 0;
+    virtual size_t num_inputs() const = 0;
+    virtual bool cache_output() const { return false; }
+    virtual const char* name() const = 0;
+};
+
+// reduce_gradient_for_broadcasting, src/ops/basic.rs:10-53
+template <typename T> void reduce_gradient_for_broadcasting(Tensor<T>& grad, const Shape& target) {
+    const Shape& gs = grad->shape();
+    if (gs == target) return;
+    std::vector<size_t> axes;
+    size_t ti = target.size();
+    for (size_t i = gs.size(); i-- > 0;) {
+        if (ti == 0) axes.push_back(i);
+        else {
+            --ti;
+            if (target[ti] == 1 && gs[i] > 1) axes.push_back(i);
+        }
+    }
+    if (!axes.empty()) grad = grad->sum(&axes, false);
+    if (grad->shape() != target) grad->reshape(target);
+}
+
+// expand_reduction, src/ops/reduction.rs:9-50
+template <typename T> Tensor<T> expand_reduction(Tensor<T> g, const std::vector<size_t>* axes, const Shape& input_shape) {
+    if (axes) {
+        std::vector<size_t> sorted = *axes;
+        std::sort(sorted.begin(), sorted.end());
+        if (sorted.empty()) return g;
+        for (size_t a : sorted) g->unsqueeze(a);
+        if (g->shape() != input_shape) g->broadcast_to(input_shape);
+        return g;
+    }
+    const T scalar = g->first();  // device -> host round trip, as in the reference
+    return HipStorage<T>::full(input_shape, scalar);
+}
+
+template <typename T> struct Add : Operator<T> {  // src/ops/basic.rs:57-130
+    Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->add(*in[1]); }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        Tensor<T> g1 = g->clone_storage();
+        Tensor<T> g2 = std::move(g);
+        reduce_gradient_for_broadcasting(g1, in[0]->shape());
+        reduce_gradient_for_broadcasting(g2, in[1]->shape());
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(g1));
+        r.push_back(std::move(g2));
+        return r;
+    }
+    size_t num_inputs() const override { return 2; }
+    const char* name() const override { return "Add"; }
+};
+
+template <typename T> struct Mul : Operator<T> {  // src/ops/basic.rs:175-215
+    Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->mul(*in[1]); }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        Tensor<T> g1 = g->mul(*in[1]);
+        Tensor<T> g2 = g->mul(*in[0]);
+        reduce_gradient_for_broadcasting(g1, in[0]->shape());
+        reduce_gradient_for_broadcasting(g2, in[1]->shape());
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(g1));
+        r.push_back(std::move(g2));
+        return r;
+    }
+    size_t num_inputs() const override { return 2; }
+    const char* name() const override { return "Mul"; }
+};
+
+template <typename T> struct MatMul : Operator<T> {  // src/ops/matrix.rs:17-64
+    Tensor<T> compute(const TensorRefs<T>& in) const override {
+        if (in[0]->ndim() != 2 || in[1]->ndim() != 2) throw Error("MatMul requires 2D tensors (matrices)");
+        return in[0]->matmul(*in[1]);
+    }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        Tensor<T> bt = in[1]->clone_storage();
+        bt->transpose(nullptr);
+        Tensor<T> ga = g->matmul(*bt);
+        Tensor<T> at = in[0]->clone_storage();
+        at->transpose(nullptr);
+        Tensor<T> gb = at->matmul(*g);
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(ga));
+        r.push_back(std::move(gb));
+        return r;
+    }
+    size_t num_inputs() const override { return 2; }
+    const char* name() const override { return "MatMul"; }
+};
+
+template <typename T> struct Transpose : Operator<T> {  // src/ops/matrix.rs:66-125 (axes = None)
+    Tensor<T> compute(const TensorRefs<T>& in) const override {
+        Tensor<T> r = in[0]->clone_storage();
+        r->transpose(nullptr);
+        return r;
+    }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>&, const HipStorage<T>*) const override {
+        g->transpose(nullptr);
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(g));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    const char* name() const override { return "Transpose"; }
+};
+
+template <typename T> struct ReLUOp : Operator<T> {  // src/ops/unary.rs:340-384
+    Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->relu(); }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        Tensor<T> mask = in[0]->greater_scalar(T(0));
+        std::vector<Tensor<T>> r;
+        r.push_back(g->mul(*mask));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    const char* name() const override { return "ReLU"; }
+};
+
+template <typename T> struct Log : Operator<T> {  // src/ops/unary.rs:60-95
+    Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->log(); }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        std::vector<Tensor<T>> r;
+        r.push_back(g->div(*in[0]));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    const char* name() const override { return "Log"; }
+};
+
+template <typename T> struct Neg : Operator<T> {  // src/ops/unary.rs:196-236
+    Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->neg(); }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>&, const HipStorage<T>*) const override {
+        std::vector<Tensor<T>> r;
+        r.push_back(g->neg());
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    const char* name() const override { return "Neg"; }
+};
+
+template <typename T> struct Clamp : Operator<T> {  // src/ops/comparison.rs:250-297
+    T lo, hi;
+    Clamp(T lo_, T hi_) : lo(lo_), hi(hi_) {}
+    Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->clamp(lo, hi); }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        Tensor<T> a = in[0]->greater_equal_scalar(lo);
+        Tensor<T> b = in[0]->less_equal_scalar(hi);
+        Tensor<T> m = a->mul(*b);
+        std::vector<Tensor<T>> r;
+        r.push_back(g->mul(*m));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    const char* name() const override { return "Clamp"; }
+};
+
+template <typename T> struct Softmax : Operator<T> {  // src/ops/batched.rs:4-131 (axis = Some(axis))
+    size_t axis;
+    explicit Softmax(size_t a) : axis(a) {}
+    Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->softmax_batched(axis); }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out) const override {
+        Tensor<T> recomputed;
+        if (!out) {
+            recomputed = compute(in);
+            out = recomputed.get();
+        }
+        if (out->shape() != g->shape()) throw Error("Softmax gradient: shape mismatch");
+        Tensor<T> prod = g->mul(*out);
+        std::vector<size_t> ax{axis};
+        Tensor<T> sum_prod = prod->sum(&ax, true);
+        sum_prod->broadcast_to(out->shape());
+        Tensor<T> diff = g->sub(*sum_prod);
+        std::vector<Tensor<T>> r;
+        r.push_back(out->mul(*diff));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    bool cache_output() const override { return true; }
+    const char* name() const override { return "Softmax"; }
+};
+
+template <typename T> struct Sum : Operator<T> {  // src/ops/reduction.rs:52-140
+    bool has_axes;
+    std::vector<size_t> axes;
+    bool keep_dims;
+    Sum(bool keep) : has_axes(false), keep_dims(keep) {}
+    Sum(std::vector<size_t> a, bool keep) : has_axes(true), axes(std::move(a)), keep_dims(keep) {}
+    Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->sum(has_axes ? &axes : nullptr, keep_dims); }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        const Shape& is = in[0]->shape();
+        Tensor<T> e = (keep_dims && has_axes) ? std::move(g) : expand_reduction<T>(std::move(g), has_axes ? &axes : nullptr, is);
+        if (e->shape() != is) e->broadcast_to(is);
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(e));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    const char* name() const override { return "Sum"; }
+};
+
+template <typename T> struct Mean : Operator<T> {  // src/ops/reduction.rs:141-230 (Mean::new(): all axes, keep_dims false)
+    bool has_axes = false;
+    std::vector<size_t> axes;
+    bool keep_dims = false;
+    Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->mean(has_axes ? &axes : nullptr, keep_dims); }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        const Shape& is = in[0]->shape();
+        double n = 1;
+        if (has_axes) for (size_t a : axes) n *= (double)is[a];
+        else n = (double)numel(is);
+        Tensor<T> scaled = g->mul_scalar((T)(1.0 / n));
+        Tensor<T> e = (keep_dims && has_axes) ? std::move(scaled) : expand_reduction<T>(std::move(scaled), has_axes ? &axes : nullptr, is);
+        if (e->shape() != is) e->broadcast_to(is);
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(e));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    const char* name() const override { return "Mean"; }
+};
+
+template <typename T> struct Reshape : Operator<T> {  // src/ops/reshape.rs:4-55
+    Shape new_shape;
+    explicit Reshape(Shape s) : new_shape(std::move(s)) {}
+    Tensor<T> compute(const TensorRefs<T>& in) const override {
+        Tensor<T> r = in[0]->clone_storage();
+        r->reshape(new_shape);
+        return r;
+    }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        g->reshape(in[0]->shape());
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(g));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    const char* name() const override { return "Reshape"; }
+};
+
+template <typename T> struct BroadcastTo : Operator<T> {  // src/ops/reshape.rs:57-115
+    Shape target;
+    explicit BroadcastTo(Shape s) : target(std::move(s)) {}
+    Tensor<T> compute(const TensorRefs<T>& in) const override {
+        Tensor<T> r = in[0]->clone_storage();
+        r->broadcast_to(target);
+        return r;
+    }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        reduce_gradient_for_broadcasting(g, in[0]->shape());
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(g));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    const char* name() const override { return "BroadcastTo"; }
+};
+
+template <typename T> struct Conv2dOp : Operator<T> {  // src/ops/batched.rs:133-230
+    std::pair<size_t, size_t> stride, padding;
+    Conv2dOp(std::pair<size_t, size_t> s, std::pair<size_t, size_t> p) : stride(s), padding(p) {}
+    Tensor<T> compute(const TensorRefs<T>& in) const override {
+        if (in[0]->ndim() != 4) throw Error("Conv2d input must be 4D [batch_size, in_channels, height, width]");
+        if (in[1]->ndim() != 4) throw Error("Conv2d filter must be 4D [out_channels, in_channels, kernel_height, kernel_width]");
+        if (in[0]->shape()[1] != in[1]->shape()[1]) {
+            std::ostringstream m;
+            m << "Input channels " << in[0]->shape()[1] << " don't match filter channels " << in[1]->shape()[1];
+            throw Error(m.str());
+        }
+        return in[0]->conv2d(*in[1], stride, padding);
+    }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        Tensor<T> gi = g->deconv2d(*in[1], in[0]->shape(), stride, padding);
+        Tensor<T> gf = in[0]->cross_correlation2d(*g, in[1]->shape(), stride, padding);
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(gi));
+        r.push_back(std::move(gf));
+        return r;
+    }
+    size_t num_inputs() const override { return 2; }
+    const char* name() const override { return "Conv2d"; }
+};
+
+// ---- AutoFerroxEngine: src/graph/mod.rs:341-997 (eager mode) -------------------------------------------------
+using NodeId = size_t;
+
+template <typename T> class AutoFerroxEngine {
+    struct Node {
+        Tensor<T> tensor;
+        std::unique_ptr<Operator<T>> op;  // null for leaves
+        std::vector<NodeId> inputs;
+        bool requires_grad = false;
+        bool is_leaf() const { return !op; }
+        bool is_parameter() const { return is_leaf() && requires_grad; }
+    };
+
+  public:
+    explicit AutoFerroxEngine(bool literal_engine = true) : literal_(literal_engine) {}
+
+    NodeId create_variable(Tensor<T> t, bool requires_grad) {  // :403-408
+        const NodeId id = next_id_++;
+        Node n;
+        n.tensor = std::move(t);
+        n.requires_grad = requires_grad;
+        nodes_[id] = std::move(n);
+        return id;
+    }
+    NodeId apply_operation(std::unique_ptr<Operator<T>> op, std::vector<NodeId> input_ids) {  // :622-679
+        if (input_ids.size() != op->num_inputs()) {
+            std::ostringstream m;
+            m << "Operation " << op->name() << " expects " << op->num_inputs() << " inputs, got " << input_ids.size();
+            throw Error(m.str());
+        }
+        TensorRefs<T> in = collect(input_ids);
+        Tensor<T> result = op->compute(in);
+        const NodeId id = next_id_++;
+        Node n;
+        n.tensor = std::move(result);
+        n.op = std::move(op);
+        n.inputs = std::move(input_ids);
+        n.requires_grad = true;
+        nodes_[id] = std::move(n);
+        return id;
+    }
+    const HipStorage<T>* get_tensor(NodeId id) const {
+        auto it = nodes_.find(id);
+        return it == nodes_.end() ? nullptr : it->second.tensor.get();
+    }
+    const HipStorage<T>* get_gradient(NodeId id) const {  // :394-396
+        auto it = grads_.find(id);
+        return it == grads_.end() ? nullptr : it->second.get();
+    }
+    void zero_gradients() { grads_.clear(); }  // :838-840
+    void update_parameter(NodeId id, Tensor<T> t) {  // :845-866
+        auto it = nodes_.find(id);
+        if (it == nodes_.end()) throw Error("Node " + std::to_string(id) + " not found");
+        if (!it->second.is_parameter()) throw Error("Can only update parameter nodes (leaf nodes with requires_grad)");
+        it->second.tensor = std::move(t);
+    }
+    void backward(NodeId loss_id) {  // :700-733
+        const HipStorage<T>* loss = get_tensor(loss_id);
+        if (!loss) throw Error("Loss node not found");
+        grads_[loss_id] = HipStorage<T>::ones(loss->shape());
+        std::set<NodeId> visited;
+        std::vector<NodeId> topo;
+        topological_sort(loss_id, visited, topo);
+        for (auto it = topo.rbegin(); it != topo.rend(); ++it) backward_node(*it);
+        cleanup();
+    }
+    size_t num_nodes() const { return nodes_.size(); }
+
+  private:
+    TensorRefs<T> collect(const std::vector<NodeId>& ids) const {  // collect_nodes_data, :575-585
+        TensorRefs<T> r;
+        for (NodeId id : ids) {
+            const HipStorage<T>* t = get_tensor(id);
+            if (!t) throw Error("[ERROR] Node " + std::to_string(id) + " not found!");
+            r.push_back(t);
+        }
+        return r;
+    }
+    void topological_sort(NodeId id, std::set<NodeId>& visited, std::vector<NodeId>& order) const {  // :786-808
+        if (visited.count(id)) return;
+        visited.insert(id);
+        auto it = nodes_.find(id);
+        if (it != nodes_.end())
+            for (NodeId in : it->second.inputs) topological_sort(in, visited, order);
+        order.push_back(id);
+    }
+    void backward_node(NodeId id) {  // :743-783
+        auto git = grads_.find(id);
+        if (git == grads_.end()) return;
+        Tensor<T> grad_output = std::move(git->second);
+        grads_.erase(git);
+        Node& node = nodes_.at(id);
+        Tensor<T> literal_copy;
+        if (literal_ && node.tensor) literal_copy = node.tensor->clone_storage();  // get_node_owned's deep clone, :735-751
+        if (node.is_leaf()) {
+            grads_[id] = std::move(grad_output);
+            return;
+        }
+        TensorRefs<T> in = collect(node.inputs);
+        std::vector<Tensor<T>> gs = node.op->gradient(std::move(grad_output), in, node.tensor.get());
+        for (size_t i = 0; i < node.inputs.size(); ++i) accumulate_gradient(node.inputs[i], std::move(gs[i]));
+    }
+    void accumulate_gradient(NodeId id, Tensor<T> g) {  // :681-698
+        auto it = grads_.find(id);
+        if (it != grads_.end()) it->second = it->second->add(*g);
+        else grads_[id] = std::move(g);
+    }
+    void cleanup() {  // :587-620: everything that is not a parameter goes away, with its gradient
+        for (auto it = nodes_.begin(); it != nodes_.end();) {
+            if (!it->second.is_parameter()) {
+                grads_.erase(it->first);
+                it = nodes_.erase(it);
+            } else ++it;
+        }
+    }
+
+    bool literal_;
+    NodeId next_id_ = 0;
+    std::map<NodeId, Node> nodes_;
+    std::map<NodeId, Tensor<T>> grads_;
+};
+
+// ---- layers: src/nn/layers ------------------------------------------------------------------------------------
+template <typename T> struct Module {
+    virtual ~Module() = default;
+    virtual NodeId forward(AutoFerroxEngine<T>& g, NodeId input) = 0;
+    virtual std::vector<NodeId> parameters() const { return {}; }
+};
+
+// reshape_and_broadcast, src/nn/layers/utils.rs:6-42
+template <typename T> NodeId reshape_and_broadcast(NodeId input, NodeId target, AutoFerroxEngine<T>& g) {
+    const Shape ts = g.get_tensor(target)->shape();
+    const Shape is = g.get_tensor(input)->shape();
+    NodeId res = input;
+    if (is.size() == 1) {
+        Shape ns = ts.size() == 4 ? Shape{1, is[0], 1, 1} : Shape{1, is[0]};
+        res = g.apply_operation(std::make_unique<Reshape<T>>(ns), {input});
+    }
+    if (is != ts) return g.apply_operation(std::make_unique<BroadcastTo<T>>(ts), {res});
+    return res;
+}
+
+template <typename T> struct Linear : Module<T> {  // src/nn/layers/linear.rs:152-308; weight is [out_features, in_features]
+    size_t in_features, out_features;
+    NodeId weight = 0, bias = 0;
+    bool has_bias = true;
+    Linear(AutoFerroxEngine<T>& g, size_t in, size_t out, const T* w, const T* b) : in_features(in), out_features(out) {
+        weight = g.create_variable(HipStorage<T>::from_vec(w, {out, in}), true);  // Linear::from_tensors, linear.rs:78-119
+        has_bias = b != nullptr;
+        if (has_bias) bias = g.create_variable(HipStorage<T>::from_vec(b, {out}), true);
+    }
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
+        const Shape& s = g.get_tensor(input)->shape();
+        if (s.size() != 1 && s.size() != 2)
+            throw Error("Linear layer only supports 1D or 2D inputs, got shape " + fmt_shape(s));
+        if (s.back() != in_features) {
+            std::ostringstream m;
+            m << "Input shape " << fmt_shape(s) << " doesn't match expected last dimension " << in_features;
+            throw Error(m.str());
+        }
+        const NodeId wt = g.apply_operation(std::make_unique<Transpose<T>>(), {weight});
+        const NodeId lin = g.apply_operation(std::make_unique<MatMul<T>>(), {input, wt});
+        if (!has_bias) return lin;
+        const Shape rs = g.get_tensor(lin)->shape();
+        if (g.get_tensor(bias)->shape() != rs) {
+            const NodeId bb = g.apply_operation(std::make_unique<BroadcastTo<T>>(rs), {bias});
+            return g.apply_operation(std::make_unique<Add<T>>(), {lin, bb});
+        }
+        return g.apply_operation(std::make_unique<Add<T>>(), {lin, bias});
+    }
+    std::vector<NodeId> parameters() const override { return has_bias ? std::vector<NodeId>{weight, bias} : std::vector<NodeId>{weight}; }
+};
+
+template <typename T> struct Conv2d : Module<T> {  // src/nn/layers/conv2d.rs:135-243
+    size_t in_channels, out_channels;
+    std::pair<size_t, size_t> kernel, stride, padding;
+    NodeId weight = 0, bias = 0;
+    bool has_bias = true;
+    Conv2d(AutoFerroxEngine<T>& g, size_t cin, size_t cout, size_t k, size_t s, size_t p, const T* w, const T* b)
+        : in_channels(cin), out_channels(cout), kernel(k, k), stride(s, s), padding(p, p) {
+        weight = g.create_variable(HipStorage<T>::from_vec(w, {cout, cin, k, k}), true);
+        has_bias = b != nullptr;
+        if (has_bias) bias = g.create_variable(HipStorage<T>::from_vec(b, {cout}), true);
+    }
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
+        const Shape& s = g.get_tensor(input)->shape();
+        if (s.size() != 4) throw Error("Conv2d requires 4D input [batch, channels, height, width], got shape " + fmt_shape(s));
+        if (s[1] != in_channels) {
+            std::ostringstream m;
+            m << "Input channels " << s[1] << " don't match layer channels " << in_channels;
+            throw Error(m.str());
+        }
+        const NodeId conv = g.apply_operation(std::make_unique<Conv2dOp<T>>(stride, padding), {input, weight});
+        if (!has_bias) return conv;
+        const NodeId bb = reshape_and_broadcast<T>(bias, conv, g);
+        return g.apply_operation(std::make_unique<Add<T>>(), {conv, bb});
+    }
+    std::vector<NodeId> parameters() const override { return has_bias ? std::vector<NodeId>{weight, bias} : std::vector<NodeId>{weight}; }
+};
+
+template <typename T> struct ReLU : Module<T> {  // src/nn/layers/activation.rs:47-80
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override { return g.apply_operation(std::make_unique<ReLUOp<T>>(), {input}); }
+};
+
+template <typename T> struct Flatten : Module<T> {  // src/nn/layers/pooling.rs:100-140 (batch-first)
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
+        const Shape& s = g.get_tensor(input)->shape();
+        size_t rest = 1;
+        for (size_t i = 1; i < s.size(); ++i) rest *= s[i];
+        return g.apply_operation(std::make_unique<Reshape<T>>(Shape{s[0], rest}), {input});
+    }
+};
+
+// ---- CCELoss (softmax cross-entropy, mean reduction): src/nn/losses/classification.rs:191-257 -------------------
+template <typename T> NodeId cce_loss(AutoFerroxEngine<T>& g, NodeId predictions, NodeId targets) {
+    const NodeId probs_raw = g.apply_operation(std::make_unique<Softmax<T>>(1), {predictions});
+    const NodeId probs = g.apply_operation(std::make_unique<Clamp<T>>((T)1e-8, (T)(1.0 - 1e-8)), {probs_raw});
+    const NodeId logp = g.apply_operation(std::make_unique<Log<T>>(), {probs});
+    const NodeId tl = g.apply_operation(std::make_unique<Mul<T>>(), {targets, logp});
+    const NodeId ce = g.apply_operation(std::make_unique<Sum<T>>(std::vector<size_t>{1}, true), {tl});
+    const NodeId neg = g.apply_operation(std::make_unique<Neg<T>>(), {ce});
+    return g.apply_operation(std::make_unique<Mean<T>>(), {neg});
+}
+
+// ---- optimizers: src/nn/optim ---------------------------------------------------------------------------------
+template <typename T> struct Optimizer {
+    virtual ~Optimizer() = default;
+    virtual void step(AutoFerroxEngine<T>& g) = 0;
+    std::vector<NodeId> params;
+};
+
+template <typename T> struct SGD : Optimizer<T> {  // src/nn/optim/sgd.rs:116-245 (momentum 0, weight decay 0 path)
+    T lr;
+    explicit SGD(T lr_) : lr(lr_) {}
+    void step(AutoFerroxEngine<T>& g) override {
+        for (NodeId p : this->params) {
+            const HipStorage<T>* grad = g.get_gradient(p);
+            if (!grad) continue;
+            const HipStorage<T>* w = g.get_tensor(p);
+            Tensor<T> effective = grad->clone_storage();  // apply_weight_decay with rate 0 returns grad.clone()
+            Tensor<T> scaled = effective->mul_scalar(lr); // apply_lr
+            g.update_parameter(p, w->sub(*scaled));
+        }
+    }
+};
+
+template <typename T> struct Adam : Optimizer<T> {  // src/nn/optim/adam.rs:110-358 (no amsgrad)
+    T lr, beta1, beta2, eps, weight_decay;
+    long step_count = 0;
+    std::map<NodeId, Tensor<T>> m1, m2;
+    Adam(T lr_, T b1, T b2, T eps_, T wd) : lr(lr_), beta1(b1), beta2(b2), eps(eps_), weight_decay(wd) {}
+    void step(AutoFerroxEngine<T>& g) override {
+        step_count += 1;
+        const T stepf = (T)step_count;
+        const T b1p = std::max((T)std::pow(beta1, stepf), (T)1e-8), b2p = std::max((T)std::pow(beta2, stepf), (T)1e-8);
+        const T bc1 = T(1) - b1p, bc2 = T(1) - b2p;
+        for (NodeId p : this->params) {
+            const HipStorage<T>* grad = g.get_gradient(p);
+            if (!grad) continue;
+            Tensor<T> w = g.get_tensor(p)->clone_storage();  // adam.rs:299-302 clones the parameter
+            if (!m1.count(p)) m1[p] = HipStorage<T>::zeros(w->shape());
+            {  // first moment: beta1*m + (1-beta1)*g
+                Tensor<T> a = m1[p]->mul_scalar(beta1), b = grad->mul_scalar(T(1) - beta1);
+                m1[p] = a->add(*b);
+            }
+            if (!m2.count(p)) m2[p] = HipStorage<T>::zeros(w->shape());
+            {  // second moment: beta2*v + (1-beta2)*g*g
+                Tensor<T> gg = grad->mul(*grad);
+                Tensor<T> a = m2[p]->mul_scalar(beta2), b = gg->mul_scalar(T(1) - beta2);
+                m2[p] = a->add(*b);
+            }
+            Tensor<T> second = m2[p]->clone_storage();  // take_current_buffer clones
+            Tensor<T> t1 = second->div_scalar(bc2);
+            Tensor<T> t2 = t1->sqrt();
+            Tensor<T> denom = t2->add_scalar(eps);
+            Tensor<T> first = m1[p]->clone_storage();
+            Tensor<T> u1 = first->div_scalar(bc1);
+            Tensor<T> u2 = u1->div(*denom);
+            Tensor<T> update = u2->mul_scalar(lr);
+            Tensor<T> nw;
+            if (weight_decay != T(0)) {
+                Tensor<T> wd = w->mul_scalar(weight_decay * lr);
+                Tensor<T> s1 = w->sub(*update);
+                nw = s1->sub(*wd);
+            } else nw = w->sub(*update);
+            g.update_parameter(p, std::move(nw));
+        }
+    }
+};
+
+}  // namespace ferrox

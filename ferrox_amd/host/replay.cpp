@@ -1,0 +1,210 @@
+// Replay harness: drives the mirrored Ferrox host stack (autograd.hpp) through a C ABI so that tests and the
+// benchmark can run the MLP / CNN training configs end to end against libferrox_hip.so.
+// One training step follows examples/common/training.rs:33-81 of the reference:
+//   zero_gradients -> create_variable(inputs.clone()), create_variable(targets.clone()) (:125-126) ->
+//   model.forward -> loss.forward -> loss.clone().first() (device->host sync) -> backward -> optimizer.step
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <sstream>
+
+#include "autograd.hpp"
+
+using namespace ferrox;
+
+namespace {
+thread_local std::string g_err;
+
+struct ModelBase {
+    virtual ~ModelBase() = default;
+    virtual int num_params() const = 0;
+    virtual int64_t param_numel(int i) const = 0;
+    virtual void set_batch(const void* x, const Shape& xs, const void* y, const Shape& ys) = 0;
+    virtual double train_step() = 0;
+    virtual void get_param(int i, void* host) const = 0;
+    virtual void get_grad(int i, void* host) const = 0;
+    virtual void forward_only(void* host_out) = 0;
+    virtual int64_t output_numel() = 0;
+};
+
+std::vector<std::string> split(const std::string& s, char sep) {
+    std::vector<std::string> out;
+    std::stringstream ss(s);
+    std::string item;
+    while (std::getline(ss, item, sep)) {
+        size_t a = item.find_first_not_of(" \t\n"), b = item.find_last_not_of(" \t\n");
+        if (a != std::string::npos) out.push_back(item.substr(a, b - a + 1));
+    }
+    return out;
+}
+
+template <typename T> struct Model : ModelBase {
+    AutoFerroxEngine<T> graph;
+    std::vector<std::unique_ptr<Module<T>>> layers;
+    std::vector<NodeId> params;
+    std::unique_ptr<Optimizer<T>> opt;
+    Tensor<T> x, y;
+
+    Model(const std::string& spec, const std::string& optspec, bool literal, const void* const* pv, int np) : graph(literal) {
+        int pi = 0;
+        auto next = [&]() -> const T* {
+            if (pi >= np) throw Error("not enough parameter arrays for the layer spec");
+            return static_cast<const T*>(pv[pi++]);
+        };
+        for (const std::string& tok : split(spec, ';')) {
+            std::stringstream ss(tok);
+            std::string kind;
+            ss >> kind;
+            if (kind == "linear") {
+                size_t in, out;
+                ss >> in >> out;
+                const T* w = next();
+                const T* b = next();
+                layers.push_back(std::make_unique<Linear<T>>(graph, in, out, w, b));
+            } else if (kind == "conv") {
+                size_t cin, cout, k, s, p;
+                ss >> cin >> cout >> k >> s >> p;
+                const T* w = next();
+                const T* b = next();
+                layers.push_back(std::make_unique<Conv2d<T>>(graph, cin, cout, k, s, p, w, b));
+            } else if (kind == "relu") layers.push_back(std::make_unique<ReLU<T>>());
+            else if (kind == "flatten") layers.push_back(std::make_unique<Flatten<T>>());
+            else throw Error("unknown layer '" + kind + "'");
+            for (NodeId p : layers.back()->parameters()) params.push_back(p);
+        }
+        std::stringstream os(optspec);
+        std::string kind;
+        os >> kind;
+        if (kind == "sgd") {
+            double lr = 0.01;
+            os >> lr;
+            opt = std::make_unique<SGD<T>>((T)lr);
+        } else if (kind == "adam") {
+            double lr = 1e-3, b1 = 0.9, b2 = 0.999, eps = 1e-8, wd = 0;
+            os >> lr >> b1 >> b2 >> eps >> wd;
+            opt = std::make_unique<Adam<T>>((T)lr, (T)b1, (T)b2, (T)eps, (T)wd);
+        } else throw Error("unknown optimizer '" + kind + "'");
+        opt->params = params;
+    }
+    int num_params() const override { return (int)params.size(); }
+    int64_t param_numel(int i) const override { return (int64_t)graph.get_tensor(params.at(i))->size(); }
+    void set_batch(const void* xv, const Shape& xs, const void* yv, const Shape& ys) override {
+        x = HipStorage<T>::from_vec(static_cast<const T*>(xv), xs);
+        y = HipStorage<T>::from_vec(static_cast<const T*>(yv), ys);
+    }
+    NodeId forward(NodeId in) {
+        for (auto& l : layers) in = l->forward(graph, in);
+        return in;
+    }
+    double train_step() override {
+        if (!x || !y) throw Error("set_batch was not called");
+        graph.zero_gradients();
+        const NodeId xin = graph.create_variable(x->clone_storage(), false);
+        const NodeId yin = graph.create_variable(y->clone_storage(), false);
+        const NodeId pred = forward(xin);
+        const NodeId loss = cce_loss<T>(graph, pred, yin);
+        const T lv = graph.get_tensor(loss)->clone_storage()->first();
+        graph.backward(loss);
+        opt->step(graph);
+        return (double)lv;
+    }
+    void get_param(int i, void* host) const override {
+        std::vector<T> v = graph.get_tensor(params.at(i))->to_vec();
+        std::memcpy(host, v.data(), v.size() * sizeof(T));
+    }
+    void get_grad(int i, void* host) const override {
+        const HipStorage<T>* g = graph.get_gradient(params.at(i));
+        if (!g) throw Error("no gradient for parameter " + std::to_string(i));
+        std::vector<T> v = g->to_vec();
+        std::memcpy(host, v.data(), v.size() * sizeof(T));
+    }
+    int64_t output_numel() override {
+        const NodeId xin = graph.create_variable(x->clone_storage(), false);
+        const NodeId pred = forward(xin);
+        return (int64_t)graph.get_tensor(pred)->size();
+    }
+    void forward_only(void* host_out) override {
+        const NodeId xin = graph.create_variable(x->clone_storage(), false);
+        const NodeId pred = forward(xin);
+        std::vector<T> v = graph.get_tensor(pred)->to_vec();
+        std::memcpy(host_out, v.data(), v.size() * sizeof(T));
+    }
+};
+
+template <typename F> int guarded(F&& f) {
+    try {
+        f();
+        return 0;
+    } catch (const std::exception& e) {
+        g_err = e.what();
+        return 1;
+    }
+}
+}  // namespace
+
+extern "C" {
+
+const char* fxh_last_error(void) { return g_err.c_str(); }
+
+int fxh_init(int device, int conv_grad_mode, const fx_pool_config* cfg) {
+    return guarded([&] {
+        BackendManager::get().init(device, cfg);
+        BackendManager::get().conv_grad_mode = conv_grad_mode;
+    });
+}
+void fxh_shutdown(void) { BackendManager::get().shutdown(); }
+
+void* fxh_model_create(int dtype, const char* spec, const char* optimizer, int literal_engine, const void* const* params, int n_params) {
+    ModelBase* m = nullptr;
+    const int rc = guarded([&] {
+        if (dtype == FX_F32) m = new Model<float>(spec, optimizer, literal_engine != 0, params, n_params);
+        else if (dtype == FX_F64) m = new Model<double>(spec, optimizer, literal_engine != 0, params, n_params);
+        else throw Error("unknown dtype");
+    });
+    return rc ? nullptr : m;
+}
+void fxh_model_destroy(void* m) { delete static_cast<ModelBase*>(m); }
+int fxh_model_num_params(void* m) { return static_cast<ModelBase*>(m)->num_params(); }
+int64_t fxh_model_param_numel(void* m, int i) {
+    int64_t n = -1;
+    guarded([&] { n = static_cast<ModelBase*>(m)->param_numel(i); });
+    return n;
+}
+int fxh_model_set_batch(void* m, const void* x, const int64_t* xshape, int xnd, const void* y, const int64_t* yshape, int ynd) {
+    return guarded([&] {
+        Shape xs(xshape, xshape + xnd), ys(yshape, yshape + ynd);
+        static_cast<ModelBase*>(m)->set_batch(x, xs, y, ys);
+    });
+}
+int fxh_model_train_step(void* m, double* loss) {
+    return guarded([&] { *loss = static_cast<ModelBase*>(m)->train_step(); });
+}
+// n steps back to back; wall time covers forward + backward + optimizer step of every step and one final sync
+int fxh_model_train_steps(void* m, int n, double* last_loss, double* total_ms) {
+    return guarded([&] {
+        fx_ok(fx_sync(BackendManager::get().ctx()));
+        const auto t0 = std::chrono::steady_clock::now();
+        for (int i = 0; i < n; ++i) *last_loss = static_cast<ModelBase*>(m)->train_step();
+        fx_ok(fx_sync(BackendManager::get().ctx()));
+        *total_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+    });
+}
+int fxh_model_get_param(void* m, int i, void* host) {
+    return guarded([&] { static_cast<ModelBase*>(m)->get_param(i, host); });
+}
+int fxh_model_get_grad(void* m, int i, void* host) {
+    return guarded([&] { static_cast<ModelBase*>(m)->get_grad(i, host); });
+}
+int64_t fxh_model_output_numel(void* m) {
+    int64_t n = -1;
+    guarded([&] { n = static_cast<ModelBase*>(m)->output_numel(); });
+    return n;
+}
+int fxh_model_forward(void* m, void* host_out) {
+    return guarded([&] { static_cast<ModelBase*>(m)->forward_only(host_out); });
+}
+int fxh_pool_stats(int dtype, fx_pool_stats* out) {
+    return guarded([&] { fx_ok(fx_pool_stats_get(BackendManager::get().ctx(), dtype, out)); });
+}
+
+}  // extern "C"

@@ -1,0 +1,115 @@
+"""ctypes binding of libferrox_host.so: the C++ mirror of Ferrox's host stack (HipStorage, autograd tape, layers,
+loss, optimizers) with a small C harness to run whole training steps through the C ABI of libferrox_hip.so."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+from . import capi
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libferrox_host.so")
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        subprocess.check_call(["make", "-C", os.path.join(_HERE, "host"), "-s"])
+    return C.CDLL(LIB_PATH)
+
+
+lib = _load()
+lib.fxh_last_error.restype = C.c_char_p
+lib.fxh_init.argtypes = [C.c_int, C.c_int, C.POINTER(capi.PoolConfig)]
+lib.fxh_model_create.restype = C.c_void_p
+lib.fxh_model_create.argtypes = [C.c_int, C.c_char_p, C.c_char_p, C.c_int, C.POINTER(C.c_void_p), C.c_int]
+lib.fxh_model_destroy.argtypes = [C.c_void_p]
+lib.fxh_model_num_params.argtypes = [C.c_void_p]
+lib.fxh_model_param_numel.argtypes = [C.c_void_p, C.c_int]
+lib.fxh_model_param_numel.restype = C.c_int64
+lib.fxh_model_set_batch.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_int64), C.c_int, C.c_void_p, C.POINTER(C.c_int64), C.c_int]
+lib.fxh_model_train_step.argtypes = [C.c_void_p, C.POINTER(C.c_double)]
+lib.fxh_model_train_steps.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
+lib.fxh_model_get_param.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
+lib.fxh_model_get_grad.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
+lib.fxh_model_output_numel.argtypes = [C.c_void_p]
+lib.fxh_model_output_numel.restype = C.c_int64
+lib.fxh_model_forward.argtypes = [C.c_void_p, C.c_void_p]
+lib.fxh_pool_stats.argtypes = [C.c_int, C.POINTER(capi.PoolStats)]
+
+
+class HostError(RuntimeError):
+    pass
+
+
+def _check(rc):
+    if rc != 0:
+        raise HostError(lib.fxh_last_error().decode("utf-8", "replace"))
+
+
+def init(device=0, conv_grad_mode=0, pool_config=None):
+    _check(lib.fxh_init(device, conv_grad_mode, C.byref(pool_config) if pool_config is not None else None))
+
+
+def shutdown():
+    lib.fxh_shutdown()
+
+
+def pool_stats(dtype=np.float32):
+    st = capi.PoolStats()
+    _check(lib.fxh_pool_stats(capi.dtype_code(dtype)[0], C.byref(st)))
+    return st.as_dict()
+
+
+class Model:
+    """spec: 'conv CIN COUT K S P; relu; flatten; linear IN OUT; ...'  optimizer: 'sgd LR' | 'adam LR B1 B2 EPS WD'."""
+
+    def __init__(self, spec, params, optimizer, dtype=np.float32, literal_engine=True):
+        self.dtype = np.dtype(dtype)
+        self._params = [np.ascontiguousarray(p, dtype=self.dtype) for p in params]
+        self.shapes = [p.shape for p in self._params]
+        arr = (C.c_void_p * len(params))(*[p.ctypes.data for p in self._params])
+        self.h = lib.fxh_model_create(capi.dtype_code(dtype)[0], spec.encode(), optimizer.encode(), int(literal_engine), arr,
+                                      len(params))
+        if not self.h:
+            raise HostError(lib.fxh_last_error().decode("utf-8", "replace"))
+
+    def close(self):
+        if self.h:
+            lib.fxh_model_destroy(self.h)
+            self.h = None
+
+    def set_batch(self, x, y):
+        x = np.ascontiguousarray(x, dtype=self.dtype)
+        y = np.ascontiguousarray(y, dtype=self.dtype)
+        xs = (C.c_int64 * x.ndim)(*x.shape)
+        ys = (C.c_int64 * y.ndim)(*y.shape)
+        _check(lib.fxh_model_set_batch(self.h, x.ctypes.data, xs, x.ndim, y.ctypes.data, ys, y.ndim))
+
+    def train_step(self):
+        loss = C.c_double(0)
+        _check(lib.fxh_model_train_step(self.h, C.byref(loss)))
+        return loss.value
+
+    def train_steps(self, n):
+        loss, ms = C.c_double(0), C.c_double(0)
+        _check(lib.fxh_model_train_steps(self.h, n, C.byref(loss), C.byref(ms)))
+        return loss.value, ms.value
+
+    def param(self, i):
+        out = np.empty(self.shapes[i], self.dtype)
+        _check(lib.fxh_model_get_param(self.h, i, out.ctypes.data))
+        return out
+
+    def grad(self, i):
+        out = np.empty(self.shapes[i], self.dtype)
+        _check(lib.fxh_model_get_grad(self.h, i, out.ctypes.data))
+        return out
+
+    def forward(self):
+        n = lib.fxh_model_output_numel(self.h)
+        if n < 0:
+            raise HostError(lib.fxh_last_error().decode("utf-8", "replace"))
+        out = np.empty(n, self.dtype)
+        _check(lib.fxh_model_forward(self.h, out.ctypes.data))
+        return out

@@ -4,3 +4,4 @@ Importable only from tests/, __graft_entry__.smoke() and bench.py's cpu_baseline
 The product package (ferrox_amd) never imports this module.
 """
 from .binding import *  # noqa: F401,F403
+from . import train  # noqa: F401

@@ -1,0 +1,164 @@
+"""CPU oracle for one Ferrox training step (test infrastructure only).
+
+Restates, operator by operator and in the reference's order, what `AutoFerroxEngine` + the `nn` layers do for a
+Sequential model of Linear / Conv2d / ReLU / Flatten layers with the softmax cross-entropy loss and SGD or Adam,
+using the oracle's C primitives for every storage op so that each intermediate is rounded to the tensor dtype
+exactly where the CPU backend rounds it.  References (Ferrox repository paths):
+  layers     src/nn/layers/linear.rs:183-279, conv2d.rs:168-214, utils.rs:6-42, activation.rs:47-80, pooling.rs:100-140
+  loss       src/nn/losses/classification.rs:191-257
+  gradients  src/ops/{basic.rs:10-215, matrix.rs:17-125, unary.rs:60-95,196-236,340-384, comparison.rs:250-297,
+             reduction.rs:9-230, reshape.rs:4-115, batched.rs:41-131,154-217}
+  optimizers src/nn/optim/sgd.rs:116-245, adam.rs:110-358
+`conv_mode` 0 uses the mathematical conv gradients (what the GPU path computes), 1 the CPU backend's literal ones.
+"""
+import numpy as np
+
+from . import binding as orc
+
+
+def _bcast(b, shape):
+    """Reshape [C] -> [1,C,1,1] / [1,C] and materialise to `shape` (utils.rs:6-42, BroadcastTo)."""
+    if len(shape) == 4:
+        return orc.materialize(b, shape, (0, 1, 0, 0))
+    return orc.materialize(b, shape, (0, 1))
+
+
+class Sequential:
+    def __init__(self, spec, params, dtype, conv_mode=0):
+        self.dtype = np.dtype(dtype)
+        self.conv_mode = conv_mode
+        self.layers = []
+        self.params = [np.ascontiguousarray(p, dtype=self.dtype).copy() for p in params]
+        pi = 0
+        for tok in [t.strip() for t in spec.split(";") if t.strip()]:
+            parts = tok.split()
+            kind = parts[0]
+            if kind == "linear":
+                self.layers.append(("linear", pi, pi + 1))
+                pi += 2
+            elif kind == "conv":
+                _, cin, cout, k, s, p = parts
+                self.layers.append(("conv", pi, pi + 1, (int(s), int(s)), (int(p), int(p))))
+                pi += 2
+            elif kind in ("relu", "flatten"):
+                self.layers.append((kind,))
+            else:
+                raise ValueError(kind)
+        assert pi == len(self.params)
+
+    # ---- forward, recording what backward needs ----
+    def forward(self, x):
+        tape = []
+        h = np.ascontiguousarray(x, dtype=self.dtype)
+        for layer in self.layers:
+            kind = layer[0]
+            if kind == "linear":
+                w, b = self.params[layer[1]], self.params[layer[2]]
+                wt = np.ascontiguousarray(w.T)                      # Transpose op (owned copy)
+                lin = orc.gemm(h, wt)                               # MatMul
+                out = orc.binary("add", lin, _bcast(b, lin.shape))  # BroadcastTo + Add
+                tape.append(("linear", layer, h, wt))
+                h = out
+            elif kind == "conv":
+                w, b = self.params[layer[1]], self.params[layer[2]]
+                y = orc.conv2d_fwd(h, w, layer[3], layer[4])
+                out = orc.binary("add", y, _bcast(b, y.shape))
+                tape.append(("conv", layer, h))
+                h = out
+            elif kind == "relu":
+                tape.append(("relu", h))
+                h = orc.unary("relu", h)
+            else:
+                tape.append(("flatten", h.shape))
+                h = h.reshape(h.shape[0], -1)
+        return h, tape
+
+    def loss_and_grads(self, x, y):
+        dt = self.dtype.type
+        pred, tape = self.forward(x)
+        y = np.ascontiguousarray(y, dtype=self.dtype)
+        # CCELoss forward
+        s = orc.softmax_axis(pred, 1)
+        c = orc.clamp(s, dt(1e-8), dt(1.0 - 1e-8))
+        lp = orc.unary("log", c)
+        tl = orc.binary("mul", y, lp)
+        ce = orc.reduce("sum", tl, [1], keep_dims=True)
+        neg = orc.unary("neg", ce)
+        loss = orc.reduce("mean", neg)
+        # backward, op by op
+        g = np.ones((), self.dtype)
+        g = orc.scalar("mul_scalar", g.reshape(1), dt(1.0 / neg.size)).reshape(())       # Mean::gradient scale
+        g = np.full(neg.shape, g.item(), self.dtype)                                      # expand_reduction(None) -> full
+        g = orc.unary("neg", g)                                                           # Neg
+        g = orc.materialize(g, tl.shape, (1, 0))                                          # Sum(keep_dims): broadcast_to
+        g = orc.binary("mul", g, y)                                                       # Mul: grad wrt log-probs
+        g = orc.binary("div", g, c)                                                       # Log
+        m = orc.binary("mul", orc.scalar("greater_equal_scalar", s, dt(1e-8)),
+                       orc.scalar("less_equal_scalar", s, dt(1.0 - 1e-8)))
+        g = orc.binary("mul", g, m)                                                       # Clamp
+        prod = orc.binary("mul", g, s)                                                    # Softmax batch gradient
+        sp = orc.reduce("sum", prod, [1], keep_dims=True)
+        diff = orc.binary("sub", g, orc.materialize(sp, s.shape, (1, 0)))
+        g = orc.binary("mul", s, diff)
+        grads = [None] * len(self.params)
+        for rec in reversed(tape):
+            kind = rec[0]
+            if kind == "linear":
+                _, layer, h, wt = rec
+                grads[layer[2]] = orc.reduce("sum", g, [0])                               # bias: sum over batch axis
+                ga = orc.gemm(g, np.ascontiguousarray(wt.T))                              # grad . B^T (materialised)
+                gb = orc.gemm(np.ascontiguousarray(h.T), g)                               # A^T . grad
+                grads[layer[1]] = np.ascontiguousarray(gb.T)                              # Transpose::gradient
+                g = ga
+            elif kind == "conv":
+                _, layer, h = rec
+                w = self.params[layer[1]]
+                grads[layer[2]] = orc.reduce("sum", g, [3, 2, 0])                         # bias: axes (3,2,0)
+                gi = orc.conv2d_dgrad(g, w, h.shape, layer[3], layer[4], self.conv_mode)
+                grads[layer[1]] = orc.conv2d_wgrad(h, g, w.shape, layer[3], layer[4], self.conv_mode)
+                g = gi
+            elif kind == "relu":
+                g = orc.binary("mul", g, orc.scalar("greater_scalar", rec[1], dt(0)))
+            else:
+                g = g.reshape(rec[1])
+        return loss.item(), grads
+
+
+class SGD:
+    def __init__(self, lr):
+        self.lr = lr
+
+    def step(self, model, grads):
+        dt = model.dtype.type
+        for i, g in enumerate(grads):
+            model.params[i] = orc.binary("sub", model.params[i], orc.scalar("mul_scalar", g, dt(self.lr)))
+
+
+class Adam:
+    def __init__(self, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0):
+        self.lr, self.b1, self.b2, self.eps, self.wd = lr, beta1, beta2, eps, weight_decay
+        self.t = 0
+        self.m, self.v = {}, {}
+
+    def step(self, model, grads):
+        dt = model.dtype.type
+        self.t += 1
+        b1, b2 = dt(self.b1), dt(self.b2)
+        bc1 = dt(1) - max(dt(np.power(b1, dt(self.t))), dt(1e-8))      # adam.rs:110-126
+        bc2 = dt(1) - max(dt(np.power(b2, dt(self.t))), dt(1e-8))
+        for i, g in enumerate(grads):
+            w = model.params[i]
+            m = self.m.get(i, np.zeros_like(w))
+            v = self.v.get(i, np.zeros_like(w))
+            m = orc.binary("add", orc.scalar("mul_scalar", m, b1), orc.scalar("mul_scalar", g, dt(1) - b1))
+            v = orc.binary("add", orc.scalar("mul_scalar", v, b2),
+                           orc.scalar("mul_scalar", orc.binary("mul", g, g), dt(1) - b2))
+            self.m[i], self.v[i] = m, v
+            denom = orc.scalar("add_scalar", orc.unary("sqrt", orc.scalar("div_scalar", v, bc2)), dt(self.eps))
+            upd = orc.scalar("mul_scalar", orc.binary("div", orc.scalar("div_scalar", m, bc1), denom), dt(self.lr))
+            if self.wd != 0:
+                wdt = orc.scalar("mul_scalar", w, dt(self.wd) * dt(self.lr))
+                w = orc.binary("sub", orc.binary("sub", w, upd), wdt)
+            else:
+                w = orc.binary("sub", w, upd)
+            model.params[i] = w

