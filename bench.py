@@ -119,7 +119,87 @@ def bench_bandwidth(ctx, iters=20, warmup=3):
     return out
 
 
-def cpu_baseline_conv(batch=8, reps=1):
+TRAIN_CONFIGS = {
+    "C5_cnn": dict(spec="conv 3 32 3 1 1; relu; conv 32 64 3 2 1; relu; flatten; linear 16384 10", in_shape=(256, 3, 32, 32),
+                   classes=10, opt="adam 0.001 0.9 0.999 1e-08 0", seed=5),
+    "C2_mlp": dict(spec="linear 784 256; relu; linear 256 128; relu; linear 128 10", in_shape=(256, 784), classes=10,
+                   opt="sgd 0.01", seed=2),
+}
+
+
+def make_train_problem(cfg, dtype):
+    """Kaiming-uniform weights U(+-sqrt(6/fan_in)), zero biases, N(0,1) inputs, uniform one-hot labels."""
+    rng = np.random.default_rng(cfg["seed"])
+    params = []
+    for tok in [t.strip() for t in cfg["spec"].split(";") if t.strip()]:
+        p = tok.split()
+        if p[0] == "linear":
+            i, o = int(p[1]), int(p[2])
+            params += [rng.uniform(-1, 1, (o, i)).astype(dtype) * dtype(np.sqrt(6.0 / i)), np.zeros(o, dtype)]
+        elif p[0] == "conv":
+            ci, co, k = int(p[1]), int(p[2]), int(p[3])
+            params += [rng.uniform(-1, 1, (co, ci, k, k)).astype(dtype) * dtype(np.sqrt(6.0 / (ci * k * k))), np.zeros(co, dtype)]
+    x = rng.standard_normal(cfg["in_shape"]).astype(dtype)
+    y = np.eye(cfg["classes"], dtype=dtype)[rng.integers(0, cfg["classes"], cfg["in_shape"][0])]
+    return params, x, y
+
+
+def reference_pool_config():
+    """PoolConfig::default() of the reference (src/backend/memory/mod.rs:50-82) with its allocation policy."""
+    from ferrox_amd import capi
+    cfg = capi.PoolConfig()
+    cfg.n_buckets, cfg.literal_ids, cfg.best_fit = 4, 0, 0
+    for i, b in enumerate([(1, 1024, 500, 50, -1), (1025, 262144, 50, 15, -1), (262145, 16777216, 10, 5, -1),
+                           (16777217, 2**62, 2, 2, -1)]):
+        cfg.buckets[i] = capi.BucketConfig(*b)
+    return cfg
+
+
+def bench_train_steps(steps=30, warmup=5, cpu=True, reference_pool=False):
+    """Full training steps (forward + backward + optimizer step, allocations from the pool) through the mirrored
+    Ferrox host stack; imgs/sec = batch / wall time per step with one final synchronisation."""
+    from ferrox_amd import host_api
+    host_api.init(0, 0, reference_pool_config() if reference_pool else None)
+    out = {}
+    for name, cfg in TRAIN_CONFIGS.items():
+        for dtype in (np.float32, np.float64):
+            if name == "C2_mlp" and dtype == np.float64:
+                continue
+            params, x, y = make_train_problem(cfg, dtype)
+            key = f"{name}_{np.dtype(dtype).name}"
+            out[key] = {"batch": int(x.shape[0])}
+            for literal in (True, False):
+                m = host_api.Model(cfg["spec"], params, cfg["opt"], dtype, literal_engine=literal)
+                m.set_batch(x, y)
+                m.train_steps(warmup)
+                st0 = host_api.pool_stats(dtype)
+                loss, ms = m.train_steps(steps)
+                st1 = host_api.pool_stats(dtype)
+                req = (st1["pool_hits"] + st1["pool_misses"]) - (st0["pool_hits"] + st0["pool_misses"])
+                out[key]["engine_literal" if literal else "engine_without_node_clones"] = {
+                    "ms_per_step": ms / steps, "imgs_per_s": x.shape[0] / (ms / steps / 1e3), "final_loss": loss,
+                    "pool_requests_per_step": req / steps,
+                    "pool_hit_rate": (st1["pool_hits"] - st0["pool_hits"]) / max(1, req),
+                    "pool_underflow_misses": st1["underflow_misses"] - st0["underflow_misses"]}
+                m.close()
+            if cpu:
+                from oracle import train as otrain
+                ref = otrain.Sequential(cfg["spec"], params, dtype)
+                kind, *nums = cfg["opt"].split()
+                opt = otrain.SGD(float(nums[0])) if kind == "sgd" else otrain.Adam(*[float(v) for v in nums])
+                n_cpu = 3
+                t0 = time.perf_counter()
+                for _ in range(n_cpu):
+                    _, grads = ref.loss_and_grads(x, y)
+                    opt.step(ref, grads)
+                dt = (time.perf_counter() - t0) / n_cpu
+                out[key]["cpu_baseline"] = {"value": x.shape[0] / dt, "unit": "imgs/s", "cores": 1, "kind": "port",
+                                            "sample": f"{n_cpu} full steps of the same config, {dt:.2f} s per step"}
+    host_api.shutdown()
+    return out
+
+
+def cpu_baseline_conv(batch=32, reps=4):
     """The CPU oracle (a restatement of Ferrox's ndarray path: im2col + single-thread GEMM + col2im) timed on this
     host, on a batch slice of the same layer; one thread, like the reference."""
     import oracle as orc
@@ -198,6 +278,9 @@ def main():
         }
         result["also"].update(bench_bandwidth(ctx))
     ctx.close()
+    if not args.skip_also:
+        result["also"]["train_step"] = bench_train_steps(cpu=not args.skip_cpu)
+        result["also"]["train_step_reference_pool_config"] = bench_train_steps(cpu=False, reference_pool=True)
     if not args.skip_cpu:
         result["cpu_baseline"] = cpu_baseline_conv()
     print(json.dumps(result))

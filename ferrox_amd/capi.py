@@ -29,7 +29,8 @@ class BucketConfig(C.Structure):
 
 
 class PoolConfig(C.Structure):
-    _fields_ = [("n_buckets", C.c_int32), ("literal_ids", C.c_int32), ("buckets", BucketConfig * FX_MAX_BUCKETS)]
+    _fields_ = [("n_buckets", C.c_int32), ("literal_ids", C.c_int32), ("best_fit", C.c_int32), ("reserved", C.c_int32),
+                ("buckets", BucketConfig * FX_MAX_BUCKETS)]
 
 
 class PoolStats(C.Structure):

@@ -43,6 +43,7 @@ struct Pool {
     std::mutex mu;
     int elem_size = 4;
     int literal_ids = 0;
+    int best_fit = 0;
     hipStream_t stream = nullptr;  // work that may still touch a block is queued here
     std::vector<Bucket> buckets;
     std::unordered_map<uint64_t, int> active;         // allocation id -> bucket index
@@ -100,13 +101,17 @@ Pool* pool_create(const fx_pool_config* cfg, int elem_size, hipStream_t stream) 
     p->elem_size = elem_size;
     p->stream = stream;
     fx_pool_config def{};
-    if (!cfg || cfg->n_buckets == 0) {  // PoolConfig::default, mod.rs:50-82
+    if (!cfg || cfg->n_buckets == 0) {
+        // The four size classes of PoolConfig::default (mod.rs:50-82) with block counts sized for 288 GB of HBM:
+        // the reference's 500/50/10/2 blocks (chosen for a 4-8 GB card) evict and re-allocate on every step of
+        // the CNN config, where more than ten 1-32 MiB activations are alive at once.
         def.n_buckets = 4;
         def.literal_ids = cfg ? cfg->literal_ids : 0;
-        def.buckets[0] = {1, 1024, 500, 50, -1};
-        def.buckets[1] = {1025, 262144, 50, 15, -1};
-        def.buckets[2] = {262145, 16777216, 10, 5, -1};
-        def.buckets[3] = {16777217, INT64_MAX, 2, 2, -1};
+        def.best_fit = cfg ? cfg->best_fit : 1;
+        def.buckets[0] = {1, 1024, 4096, 512, -1};
+        def.buckets[1] = {1025, 262144, 1024, 128, -1};
+        def.buckets[2] = {262145, 16777216, 256, 32, -1};
+        def.buckets[3] = {16777217, INT64_MAX, 16, 4, -1};
         cfg = &def;
     }
     if (cfg->n_buckets < 0 || cfg->n_buckets > FX_MAX_BUCKETS) {
@@ -115,6 +120,7 @@ Pool* pool_create(const fx_pool_config* cfg, int elem_size, hipStream_t stream) 
         return nullptr;
     }
     p->literal_ids = cfg->literal_ids;
+    p->best_fit = cfg->best_fit;
     for (int i = 0; i < cfg->n_buckets; ++i) {
         Bucket b;
         b.cfg = cfg->buckets[i];
@@ -167,8 +173,14 @@ int fx_alloc(fx_ctx* c, int dtype, int64_t n, void** ptr, int64_t* granted, uint
     p->active[id] = bi;
     Bucket& b = p->buckets[bi];
     if (!b.blocks.empty()) {
-        Block blk = b.blocks.back();
-        b.blocks.pop_back();
+        size_t pick = b.blocks.size() - 1;  // reference policy: the most recently returned block
+        if (p->best_fit) {                   // smallest block that fits; ties go to the most recently returned
+            i64 best = -1;
+            for (size_t i = b.blocks.size(); i-- > 0;)
+                if (b.blocks[i].elems >= n && (best < 0 || b.blocks[i].elems < best)) { best = b.blocks[i].elems; pick = i; }
+        }
+        Block blk = b.blocks[pick];
+        b.blocks.erase(b.blocks.begin() + pick);
         if (blk.elems >= n) {
             p->st.pool_hits += 1;
             p->st.active_allocations += 1;

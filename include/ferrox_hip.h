@@ -52,9 +52,16 @@ typedef struct fx_bucket_config {
 } fx_bucket_config;
 
 typedef struct fx_pool_config {
-    int32_t n_buckets;   /* 0 = PoolConfig::default() (mod.rs:50-82) */
+    int32_t n_buckets;   /* 0 = the library default: the four size classes of PoolConfig::default() (mod.rs:50-82:
+                            <=1024, <=262144, <=16777216, larger) holding 4096/1024/256/16 blocks instead of the
+                            reference's 500/50/10/2, which were sized for a 4-8 GB card */
     int32_t literal_ids; /* 1 = keep the reference's id bookkeeping (a reused block keeps its old id, so its second
                             release is dropped, cuda.rs:61-62,76-87); 0 = a reused block is re-registered (default) */
+    int32_t best_fit;    /* 0 = the reference's policy: only the most recently returned block of the bucket is tried
+                            (cuda.rs:79-92), a too-small one is an underflow miss; 1 = the smallest pooled block of the
+                            bucket that is large enough is taken (most recent among equals), which removes most
+                            underflow misses.  fx_init(cfg = NULL) uses best_fit = 1, literal_ids = 0. */
+    int32_t reserved;
     fx_bucket_config buckets[FX_MAX_BUCKETS];
 } fx_pool_config;
 

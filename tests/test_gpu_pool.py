@@ -13,6 +13,7 @@ def make_cfg(capi, buckets, literal):
     cfg = capi.PoolConfig()
     cfg.n_buckets = len(buckets)
     cfg.literal_ids = int(literal)
+    cfg.best_fit = 0   # the reference's pop-most-recent policy, which is what the oracle state machine restates
     for i, (lo, hi, cap, ev, th) in enumerate(buckets):
         cfg.buckets[i] = capi.BucketConfig(lo, hi, cap, ev, th)
     return cfg
@@ -110,9 +111,10 @@ def test_default_config_hit_rate_in_a_training_like_loop():
         ctx.pool_cleanup()
         st = ctx.pool_stats()
         assert st["bytes_pooled"] == 0 and st["device_frees"] == len(sizes)
+        assert [ctx.bucket_stats(b)["max_allocations"] for b in range(4)] == [4096, 1024, 256, 16]
     finally:
         ctx.close()
-    ctx = capi.Context(0)
+    ctx = capi.Context(0, make_cfg(capi, orc.DEFAULT_BUCKETS, False))
     op = orc.Pool(literal=False)
     try:
         for it in range(10):
@@ -125,6 +127,17 @@ def test_default_config_hit_rate_in_a_training_like_loop():
         gs, os_ = ctx.pool_stats(), op.stats()
         assert {k: gs[k] for k in KEYS} == {k: os_[k] for k in KEYS}
         assert gs["underflow_misses"] > 0
+    finally:
+        ctx.close()
+    # the library default (best fit inside the bucket) serves the same creation-order loop without underflows
+    ctx = capi.Context(0)
+    try:
+        for it in range(10):
+            bufs = [ctx.empty((n,)) for n in sizes]
+            for b in bufs:
+                b.free()
+        st = ctx.pool_stats()
+        assert st["underflow_misses"] == 0 and st["pool_misses"] == len(sizes) and st["pool_hits"] == 9 * len(sizes)
     finally:
         ctx.close()
 
