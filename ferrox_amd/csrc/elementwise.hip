@@ -20,8 +20,18 @@ template <> __device__ __forceinline__ void vset<double>(double2& v, int i, doub
 
 constexpr int EW_THREADS = 256;
 constexpr int EW_UNROLL = 4;
+constexpr i64 EW_STREAM_BYTES = 128ll << 20;  // arrays at least this large are streamed past the caches
+
+typedef float nt_f4 __attribute__((ext_vector_type(4)));
+typedef double nt_d2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float4 nt_load(const float4* p) { const nt_f4 v = __builtin_nontemporal_load(reinterpret_cast<const nt_f4*>(p)); return float4{v.x, v.y, v.z, v.w}; }
+__device__ __forceinline__ double2 nt_load(const double2* p) { const nt_d2 v = __builtin_nontemporal_load(reinterpret_cast<const nt_d2*>(p)); return double2{v.x, v.y}; }
+__device__ __forceinline__ void nt_store(float4 r, float4* p) { const nt_f4 v = {r.x, r.y, r.z, r.w}; __builtin_nontemporal_store(v, reinterpret_cast<nt_f4*>(p)); }
+__device__ __forceinline__ void nt_store(double2 r, double2* p) { const nt_d2 v = {r.x, r.y}; __builtin_nontemporal_store(v, reinterpret_cast<nt_d2*>(p)); }
 
 // NIN = number of input arrays (0, 1 or 2).  F: T operator()(T a, T b).
+// Cached variant (small arrays: the consumer kernel finds the data in L2 / Infinity Cache): four 16-byte vectors in
+// flight per thread.
 template <typename T, int NIN, class F>
 __global__ __launch_bounds__(EW_THREADS) void ew_vec_kernel(const T* __restrict__ a, const T* __restrict__ b,
                                                             T* __restrict__ out, i64 nvec, F f) {
@@ -53,6 +63,24 @@ __global__ __launch_bounds__(EW_THREADS) void ew_vec_kernel(const T* __restrict_
     }
 }
 
+// Streaming variant (large arrays): one 16-byte vector per thread, non-temporal loads and stores, many small waves.
+// Measured on MI355X for c = a + b over 2^28 floats: 6.4 TB/s against 5.65 TB/s for the cached variant.
+template <typename T, int NIN, class F>
+__global__ __launch_bounds__(EW_THREADS) void ew_stream_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                               T* __restrict__ out, i64 nvec, F f) {
+    typedef typename Vec16<T>::type V;
+    constexpr int N = Vec16<T>::N;
+    const i64 i = (i64)blockIdx.x * EW_THREADS + threadIdx.x;
+    if (i >= nvec) return;
+    V ra, rb;
+    if (NIN >= 1) ra = nt_load(reinterpret_cast<const V*>(a) + i);
+    if (NIN >= 2) rb = nt_load(reinterpret_cast<const V*>(b) + i);
+    V r;
+#pragma unroll
+    for (int e = 0; e < N; ++e) vset<T>(r, e, f(NIN >= 1 ? vget<T>(ra, e) : T(0), NIN >= 2 ? vget<T>(rb, e) : T(0)));
+    nt_store(r, reinterpret_cast<V*>(out) + i);
+}
+
 template <typename T, int NIN, class F>
 __global__ __launch_bounds__(EW_THREADS) void ew_scalar_kernel(const T* __restrict__ a, const T* __restrict__ b,
                                                                T* __restrict__ out, i64 begin, i64 n, F f) {
@@ -71,9 +99,14 @@ int launch_ew(fx_ctx* c, const T* a, const T* b, T* out, i64 n, F f, const char*
     i64 done = 0;
     if (vec_ok && n >= N) {
         const i64 nvec = n / N;
-        const i64 blocks = fx::ceil_div(nvec, (i64)EW_THREADS * EW_UNROLL);
-        FX_REQUIRE(blocks <= 0x7fffffff, "%s: too many elements", what);
-        ew_vec_kernel<T, NIN, F><<<dim3((unsigned)blocks), dim3(EW_THREADS), 0, c->stream>>>(a, b, out, nvec, f);
+        if (n * (i64)sizeof(T) >= EW_STREAM_BYTES) {
+            const i64 blocks = fx::ceil_div(nvec, (i64)EW_THREADS);
+            FX_REQUIRE(blocks <= 0x7fffffff, "%s: too many elements", what);
+            ew_stream_kernel<T, NIN, F><<<dim3((unsigned)blocks), dim3(EW_THREADS), 0, c->stream>>>(a, b, out, nvec, f);
+        } else {
+            const i64 blocks = fx::ceil_div(nvec, (i64)EW_THREADS * EW_UNROLL);
+            ew_vec_kernel<T, NIN, F><<<dim3((unsigned)blocks), dim3(EW_THREADS), 0, c->stream>>>(a, b, out, nvec, f);
+        }
         FX_LAUNCH_CHECK();
         done = nvec * N;
     }

@@ -12,6 +12,7 @@
 // them in slice order; no atomics, so results are deterministic run to run.
 // Max takes strictly greater values starting from the lowest finite T (src/backend/storage/cpu.rs:1231-1234);
 // the recorded index is the first position along the axis that attains the maximum.
+#include <cstdlib>
 #include <limits>
 
 #include "common.hpp"
@@ -19,6 +20,7 @@
 namespace {
 
 constexpr i64 NO_INDEX = INT64_MAX;
+constexpr i64 STREAM_BYTES = 320ll << 20;  // inputs that cannot stay in the 256 MiB Infinity Cache are read with cache-bypassing loads
 
 template <typename T> struct Vec16;
 template <> struct Vec16<float> { typedef float4 type; static constexpr int N = 4; };
@@ -26,6 +28,20 @@ template <> struct Vec16<double> { typedef double2 type; static constexpr int N 
 template <typename T> __device__ __forceinline__ T vget(const typename Vec16<T>::type& v, int i);
 template <> __device__ __forceinline__ float vget<float>(const float4& v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
 template <> __device__ __forceinline__ double vget<double>(const double2& v, int i) { return i == 0 ? v.x : v.y; }
+
+// 16-byte load that bypasses the caches when STREAM is set (inputs much larger than L2 are read exactly once)
+typedef float nt_f4 __attribute__((ext_vector_type(4)));
+typedef double nt_d2 __attribute__((ext_vector_type(2)));
+template <bool STREAM> __device__ __forceinline__ float4 ld16(const float4* p) {
+    if (!STREAM) return *p;
+    const nt_f4 v = __builtin_nontemporal_load(reinterpret_cast<const nt_f4*>(p));
+    return float4{v.x, v.y, v.z, v.w};
+}
+template <bool STREAM> __device__ __forceinline__ double2 ld16(const double2* p) {
+    if (!STREAM) return *p;
+    const nt_d2 v = __builtin_nontemporal_load(reinterpret_cast<const nt_d2*>(p));
+    return double2{v.x, v.y};
+}
 
 template <typename T> __device__ __forceinline__ T lowest();
 template <> __device__ __forceinline__ float lowest<float>() { return -3.402823466e+38f; }
@@ -71,7 +87,7 @@ __device__ __forceinline__ void wave_reduce(Acc<T, IS_MAX>& a) {
 // ---- row reduction (inner == 1) ---------------------------------------------------------------------------
 // grid (S, outer), 256 threads.  Slice s covers [s*chunk, min(axis, (s+1)*chunk)).  VEC: 16-byte loads (requires
 // axis % N == 0, chunk % N == 0 and a 16-byte aligned base).  Output slot o*S + s.
-template <typename T, bool IS_MAX, bool VEC>
+template <typename T, bool IS_MAX, bool VEC, bool STREAM>
 __global__ __launch_bounds__(256) void row_reduce_kernel(const T* __restrict__ in, T* __restrict__ out, i64* __restrict__ idx_out,
                                                          i64 axis, i64 chunk, T scale) {
     constexpr int N = Vec16<T>::N;
@@ -86,7 +102,7 @@ __global__ __launch_bounds__(256) void row_reduce_kernel(const T* __restrict__ i
         const i64 vbeg = beg / N, vend = end / N;
         i64 p = vbeg + threadIdx.x;
         for (; p + 3 * 256 < vend; p += 4 * 256) {
-            V r0 = rv[p], r1 = rv[p + 256], r2 = rv[p + 512], r3 = rv[p + 768];
+            V r0 = ld16<STREAM>(rv + p), r1 = ld16<STREAM>(rv + p + 256), r2 = ld16<STREAM>(rv + p + 512), r3 = ld16<STREAM>(rv + p + 768);
 #pragma unroll
             for (int e = 0; e < N; ++e) acc.take(vget<T>(r0, e), p * N + e);
 #pragma unroll
@@ -97,7 +113,7 @@ __global__ __launch_bounds__(256) void row_reduce_kernel(const T* __restrict__ i
             for (int e = 0; e < N; ++e) acc.take(vget<T>(r3, e), (p + 768) * N + e);
         }
         for (; p < vend; p += 256) {
-            V r0 = rv[p];
+            V r0 = ld16<STREAM>(rv + p);
 #pragma unroll
             for (int e = 0; e < N; ++e) acc.take(vget<T>(r0, e), p * N + e);
         }
@@ -143,35 +159,45 @@ __global__ __launch_bounds__(256) void short_row_reduce_kernel(const T* __restri
     }
 }
 
-// Combine S slice partials per output: one wave per output element, slices merged with the tie rule.
+// Combine S slice partials per output: one 256-thread block per output element, slices merged with the tie rule.
 template <typename T, bool IS_MAX>
 __global__ __launch_bounds__(256) void combine_rows_kernel(const T* __restrict__ pv, const i64* __restrict__ pi, T* __restrict__ out,
                                                            i64* __restrict__ idx_out, i64 n_out, i64 S, T scale) {
-    const i64 o = (i64)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63;
-    if (o >= n_out) return;
+    const i64 o = blockIdx.x;
     Acc<T, IS_MAX> acc;
     acc.init();
-    for (i64 s = lane; s < S; s += 64) acc.merge(pv[o * S + s], IS_MAX && pi ? pi[o * S + s] : NO_INDEX);
+    for (i64 s = threadIdx.x; s < S; s += 256) acc.merge(pv[o * S + s], IS_MAX && pi ? pi[o * S + s] : NO_INDEX);
     wave_reduce(acc);
-    if (lane == 0) {
-        out[o] = IS_MAX ? acc.v : acc.v * scale;
-        if (IS_MAX && idx_out) idx_out[o] = acc.i == NO_INDEX ? 0 : acc.i;
+    __shared__ T sv[4];
+    __shared__ i64 si[4];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) { sv[wave] = acc.v; si[wave] = acc.i; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        Acc<T, IS_MAX> r;
+        r.v = sv[0]; r.i = si[0];
+        for (int w = 1; w < 4; ++w) r.merge(sv[w], si[w]);
+        out[o] = IS_MAX ? r.v : r.v * scale;
+        if (IS_MAX && idx_out) idx_out[o] = r.i == NO_INDEX ? 0 : r.i;
     }
 }
 
 // ---- column reduction (inner > 1) -------------------------------------------------------------------------
-// grid (col tiles, S, outer), 256 threads = 4 waves.  A wave covers 64*NV adjacent columns (NV = N when VEC else 1);
-// wave w takes axis positions beg + w, beg + w + 4, ...  Output slot ((o*S + s) * inner + col).
+// grid (col tiles, S, outer), 256 threads = 4 waves arranged as CW waves side by side x (4/CW) waves over rows.
+// A wave covers 64*NV adjacent columns (NV = N when VEC else 1), so a block reads CW*64*NV contiguous elements of
+// each row it visits (4 KiB at CW = 4 with 16-byte vectors); waves sharing columns take interleaved axis positions
+// and are merged through LDS.  Output slot ((o*S + s) * inner + col).
 // FROM_PARTIAL: the input is a partial array whose index values come from `pidx` instead of the axis position.
-template <typename T, bool IS_MAX, bool VEC, bool FROM_PARTIAL>
+template <typename T, bool IS_MAX, bool VEC, bool FROM_PARTIAL, int CW, bool STREAM>
 __global__ __launch_bounds__(256) void col_reduce_kernel(const T* __restrict__ in, const i64* __restrict__ pidx, T* __restrict__ out,
                                                          i64* __restrict__ idx_out, i64 axis, i64 inner, i64 chunk, T scale,
                                                          int final_pass) {
     constexpr int N = VEC ? Vec16<T>::N : 1;
+    constexpr int RW = 4 / CW;
     typedef typename Vec16<T>::type V;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const i64 col = ((i64)blockIdx.x * 64 + lane) * N;
+    const int wc = wave % CW, wr = wave / CW;
+    const i64 col = (((i64)blockIdx.x * CW + wc) * 64 + lane) * N;
     const i64 s = blockIdx.y, S = gridDim.y, o = blockIdx.z;
     const i64 beg = s * chunk, end = min(axis, beg + chunk);
     Acc<T, IS_MAX> acc[N];
@@ -180,28 +206,24 @@ __global__ __launch_bounds__(256) void col_reduce_kernel(const T* __restrict__ i
     if (col < inner) {
         const T* base = in + (o * axis) * inner + col;
         const i64* ibase = FROM_PARTIAL && IS_MAX ? pidx + (o * axis) * inner + col : nullptr;
-        i64 a = beg + wave;
+        i64 a = beg + wr;
         if (VEC && !FROM_PARTIAL) {
-            for (; a + 12 < end; a += 16) {
-                V r0 = *reinterpret_cast<const V*>(base + a * inner);
-                V r1 = *reinterpret_cast<const V*>(base + (a + 4) * inner);
-                V r2 = *reinterpret_cast<const V*>(base + (a + 8) * inner);
-                V r3 = *reinterpret_cast<const V*>(base + (a + 12) * inner);
+            for (; a + 7 * RW < end; a += 8 * RW) {
+                V r[8];
 #pragma unroll
-                for (int e = 0; e < N; ++e) {
-                    acc[e].take(vget<T>(r0, e), a);
-                    acc[e].take(vget<T>(r1, e), a + 4);
-                    acc[e].take(vget<T>(r2, e), a + 8);
-                    acc[e].take(vget<T>(r3, e), a + 12);
-                }
+                for (int u = 0; u < 8; ++u) r[u] = ld16<STREAM>(reinterpret_cast<const V*>(base + (a + u * RW) * inner));
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+#pragma unroll
+                    for (int e = 0; e < N; ++e) acc[e].take(vget<T>(r[u], e), a + u * RW);
             }
-            for (; a < end; a += 4) {
-                V r0 = *reinterpret_cast<const V*>(base + a * inner);
+            for (; a < end; a += RW) {
+                V r0 = ld16<STREAM>(reinterpret_cast<const V*>(base + a * inner));
 #pragma unroll
                 for (int e = 0; e < N; ++e) acc[e].take(vget<T>(r0, e), a);
             }
         } else {
-            for (; a < end; a += 4) {
+            for (; a < end; a += RW) {
 #pragma unroll
                 for (int e = 0; e < N; ++e) {
                     const T x = base[a * inner + e];
@@ -211,26 +233,32 @@ __global__ __launch_bounds__(256) void col_reduce_kernel(const T* __restrict__ i
             }
         }
     }
-    __shared__ T sv[4][64 * N];
-    __shared__ i64 si[IS_MAX ? 4 : 1][IS_MAX ? 64 * N : 1];
-#pragma unroll
-    for (int e = 0; e < N; ++e) {
-        sv[wave][lane * N + e] = acc[e].v;
-        if (IS_MAX) si[wave][lane * N + e] = acc[e].i;
-    }
-    __syncthreads();
-    if (wave == 0 && col < inner) {
+    __shared__ T sv[RW][CW * 64 * N];
+    __shared__ i64 si[IS_MAX ? RW : 1][IS_MAX ? CW * 64 * N : 1];
+    const int sl = (wc * 64 + lane) * N;
+    if (RW > 1) {
 #pragma unroll
         for (int e = 0; e < N; ++e) {
-            Acc<T, IS_MAX> r;
-            r.v = sv[0][lane * N + e];
-            r.i = IS_MAX ? si[0][lane * N + e] : NO_INDEX;
-            for (int w = 1; w < 4; ++w) r.merge(sv[w][lane * N + e], IS_MAX ? si[w][lane * N + e] : NO_INDEX);
+            sv[wr][sl + e] = acc[e].v;
+            if (IS_MAX) si[wr][sl + e] = acc[e].i;
+        }
+        __syncthreads();
+    }
+    if (wr == 0 && col < inner) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+            Acc<T, IS_MAX> r = acc[e];
+            for (int w = 1; w < RW; ++w) r.merge(sv[w][sl + e], IS_MAX ? si[w][sl + e] : NO_INDEX);
             const i64 slot = (o * S + s) * inner + col + e;
             out[slot] = IS_MAX ? r.v : r.v * scale;
             if (IS_MAX && idx_out) idx_out[slot] = (final_pass && r.i == NO_INDEX) ? 0 : r.i;
         }
     }
+}
+
+template <typename T, bool IS_MAX, bool VEC, int CW, bool STREAM>
+void launch_col(fx_ctx* c, dim3 grid, const T* in, T* out, i64* idx_out, i64 axis, i64 inner, i64 chunk, T scale, int final_pass) {
+    col_reduce_kernel<T, IS_MAX, VEC, false, CW, STREAM><<<grid, dim3(256), 0, c->stream>>>(in, nullptr, out, idx_out, axis, inner, chunk, scale, final_pass);
 }
 
 template <typename T, bool IS_MAX>
@@ -260,8 +288,9 @@ int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i6
         FX_REQUIRE(outer <= 65535, "%s: more than 65535 long rows; reshape so that the reduced axis is not the last", what);
         // slices: enough blocks to fill the chip, each at least 16 KiB, slice length a multiple of 1024 elements
         i64 S = 1;
-        if (outer < target_blocks) {
-            S = std::min<i64>(fx::ceil_div(target_blocks, outer), std::max<i64>(1, axis / 4096));
+        const i64 row_want = (i64)c->num_cus * 3;  // measured on 2^26 elements: 2-4 blocks per CU is fastest
+        if (outer < row_want) {
+            S = std::min<i64>(fx::ceil_div(row_want, outer), std::max<i64>(1, axis / 4096));
             S = std::min<i64>(S, 65535);
         }
         i64 chunk = fx::ceil_div(axis, S);
@@ -280,11 +309,13 @@ int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i6
         const dim3 grid((unsigned)S, (unsigned)outer), block(256);
         const T sc1 = S > 1 ? T(1) : scale;
         i64* io = (S > 1 && IS_MAX) ? pi : idx_out;
-        if (vec) row_reduce_kernel<T, IS_MAX, true><<<grid, block, 0, c->stream>>>(in, pv, io, axis, chunk, sc1);
-        else row_reduce_kernel<T, IS_MAX, false><<<grid, block, 0, c->stream>>>(in, pv, io, axis, chunk, sc1);
+        const bool stream = outer * axis * (i64)sizeof(T) >= STREAM_BYTES;
+        if (vec && stream) row_reduce_kernel<T, IS_MAX, true, true><<<grid, block, 0, c->stream>>>(in, pv, io, axis, chunk, sc1);
+        else if (vec) row_reduce_kernel<T, IS_MAX, true, false><<<grid, block, 0, c->stream>>>(in, pv, io, axis, chunk, sc1);
+        else row_reduce_kernel<T, IS_MAX, false, false><<<grid, block, 0, c->stream>>>(in, pv, io, axis, chunk, sc1);
         FX_LAUNCH_CHECK();
         if (S > 1) {
-            combine_rows_kernel<T, IS_MAX><<<dim3((unsigned)fx::ceil_div(outer, 4)), dim3(256), 0, c->stream>>>(
+            combine_rows_kernel<T, IS_MAX><<<dim3((unsigned)outer), dim3(256), 0, c->stream>>>(
                 pv, IS_MAX ? pi : nullptr, out, idx_out, outer, S, scale);
             FX_LAUNCH_CHECK();
         }
@@ -295,41 +326,47 @@ int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i6
     // column reduction
     FX_REQUIRE(outer <= 65535, "%s: outer %lld exceeds 65535 for a column reduction", what, (long long)outer);
     const bool vec = fx::aligned16(in) && (inner % N == 0);
-    const i64 cols_per_block = 64 * (vec ? N : 1);
+    const bool stream = outer * axis * inner * (i64)sizeof(T) >= STREAM_BYTES;
+    const int NV = vec ? N : 1;
+    const bool wide = vec && inner >= 4 * 64 * NV;  // four waves side by side: 4 KiB contiguous per row and block
+    const i64 cols_per_block = (wide ? 4 : 1) * 64 * NV;
     const i64 tiles = fx::ceil_div(inner, cols_per_block);
     FX_REQUIRE(tiles <= 0x7fffffff, "%s: inner too large", what);
     i64 S = 1;
-    if (tiles * outer < target_blocks) {
-        S = std::min<i64>(fx::ceil_div(target_blocks, tiles * outer), std::max<i64>(1, axis / 32));
+    // measured on [8192,8192]: about 0.75 blocks per CU (each keeping 32 KiB of loads in flight) is fastest
+    const i64 want = wide ? (i64)c->num_cus * 3 / 4 : target_blocks;
+    if (tiles * outer < want) {
+        S = std::min<i64>(fx::ceil_div(want, tiles * outer), std::max<i64>(1, axis / 32));
         S = std::min<i64>(S, 65535);
     }
     i64 chunk = fx::ceil_div(axis, S);
     chunk = fx::ceil_div(chunk, 4) * 4;
     S = fx::ceil_div(axis, chunk);
-    if (S == 1) {
-        const dim3 grid((unsigned)tiles, 1, (unsigned)outer), block(256);
-        if (vec) col_reduce_kernel<T, IS_MAX, true, false><<<grid, block, 0, c->stream>>>(in, nullptr, out, idx_out, axis, inner, chunk, scale, 1);
-        else col_reduce_kernel<T, IS_MAX, false, false><<<grid, block, 0, c->stream>>>(in, nullptr, out, idx_out, axis, inner, chunk, scale, 1);
-        FX_LAUNCH_CHECK();
-        return FX_OK;
-    }
-    const i64 n_part = outer * S * inner;
-    const i64 bytes = n_part * (i64)(sizeof(T) + (IS_MAX ? sizeof(i64) : 0)) + 256;
-    char* sc = (char*)c->get_scratch(bytes);
-    if (!sc) return FX_ERR_OOM;
-    i64* pi = IS_MAX ? (i64*)sc : nullptr;
-    T* pv = (T*)(sc + (IS_MAX ? ((n_part * sizeof(i64) + 255) / 256) * 256 : 0));
-    {
-        const dim3 grid((unsigned)tiles, (unsigned)S, (unsigned)outer), block(256);
-        if (vec) col_reduce_kernel<T, IS_MAX, true, false><<<grid, block, 0, c->stream>>>(in, nullptr, pv, pi, axis, inner, chunk, T(1), 0);
-        else col_reduce_kernel<T, IS_MAX, false, false><<<grid, block, 0, c->stream>>>(in, nullptr, pv, pi, axis, inner, chunk, T(1), 0);
-        FX_LAUNCH_CHECK();
+    T* pv = out;
+    i64* pi = idx_out;
+    if (S > 1) {
+        const i64 n_part = outer * S * inner;
+        const i64 bytes = n_part * (i64)(sizeof(T) + (IS_MAX ? sizeof(i64) : 0)) + 256;
+        char* sc = (char*)c->get_scratch(bytes);
+        if (!sc) return FX_ERR_OOM;
+        pi = IS_MAX ? (i64*)sc : nullptr;
+        pv = (T*)(sc + (IS_MAX ? ((n_part * sizeof(i64) + 255) / 256) * 256 : 0));
     }
     {
+        const dim3 grid((unsigned)tiles, (unsigned)S, (unsigned)outer);
+        const T sc1 = S > 1 ? T(1) : scale;
+        const int fin = S > 1 ? 0 : 1;
+        if (wide && stream) launch_col<T, IS_MAX, true, 4, true>(c, grid, in, pv, pi, axis, inner, chunk, sc1, fin);
+        else if (wide) launch_col<T, IS_MAX, true, 4, false>(c, grid, in, pv, pi, axis, inner, chunk, sc1, fin);
+        else if (vec) launch_col<T, IS_MAX, true, 1, false>(c, grid, in, pv, pi, axis, inner, chunk, sc1, fin);
+        else launch_col<T, IS_MAX, false, 1, false>(c, grid, in, pv, pi, axis, inner, chunk, sc1, fin);
+        FX_LAUNCH_CHECK();
+    }
+    if (S > 1) {
         // second pass over [outer, S, inner] partials; scalar columns so that many blocks share the work
         const i64 tiles2 = fx::ceil_div(inner, 64);
         const dim3 grid((unsigned)tiles2, 1, (unsigned)outer), block(256);
-        col_reduce_kernel<T, IS_MAX, false, true><<<grid, block, 0, c->stream>>>(pv, pi, out, idx_out, S, inner, fx::ceil_div(S, 4) * 4, scale, 1);
+        col_reduce_kernel<T, IS_MAX, false, true, 1, false><<<grid, block, 0, c->stream>>>(pv, pi, out, idx_out, S, inner, fx::ceil_div(S, 4) * 4, scale, 1);
         FX_LAUNCH_CHECK();
     }
     return FX_OK;
