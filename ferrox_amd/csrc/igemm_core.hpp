@@ -99,6 +99,7 @@ template <typename T, bool KMAJOR_> struct MatLoader {
         i64 ld;
         uint32_t off[KMAJOR_ ? Map::CNT : 1];  // byte offsets from base (rows clamped into the matrix)
         uint32_t okmask;        // bit i: register i addresses a row/column inside the matrix
+        uint32_t live;          // validity of the slab in flight, consumed by mask()
         int klane, krow;
         __device__ __forceinline__ Dev(const MatLoader& L, int origin, int tid) : ld(L.ld) {
             okmask = 0;
@@ -123,23 +124,29 @@ template <typename T, bool KMAJOR_> struct MatLoader {
                 krow = __builtin_amdgcn_readfirstlane(tid / BMN);
             }
         }
-        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) const {
+        // load() only issues the global loads (from clamped addresses); mask() zeroes what lay outside the operand.
+        // The kernel calls mask() after the MFMA loop, so the loads stay in flight behind the matrix work.
+        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) {
             if (KMAJOR_) {
                 const bool kok = k0 + klane < kend;
+                live = kok ? okmask : 0u;
                 const T* b = base + k0;  // uniform
 #pragma unroll
                 for (int i = 0; i < Map::CNT; ++i) r[i] = ldg(b, kok ? off[i] : 0u);
-#pragma unroll
-                for (int i = 0; i < Map::CNT; ++i) r[i] = (kok && ((okmask >> i) & 1u)) ? r[i] : T(0);
             } else {
+                live = 0;
 #pragma unroll
                 for (int i = 0; i < Map::CNT; ++i) {
                     const int k = k0 + krow + i * Map::STEP;       // uniform
                     const int kc = min(k, kend - 1);               // clamped row stays inside the split
                     r[i] = ldg(base + (i64)kc * ld, off[0]);
-                    r[i] = (k < kend && okmask) ? r[i] : T(0);
+                    live |= (k < kend && okmask) ? (1u << i) : 0u;
                 }
             }
+        }
+        __device__ __forceinline__ void mask(T (&r)[Map::CNT]) const {
+#pragma unroll
+            for (int i = 0; i < Map::CNT; ++i) r[i] = ((live >> i) & 1u) ? r[i] : T(0);
         }
     };
 };
@@ -162,7 +169,7 @@ template <typename T, bool FAST> struct ConvFwdB {
     int N;
     template <int BMN, int BK, int NT> struct Dev {
         typedef SlabMap<BMN, BK, NT, false> Map;
-        const T* x; const ConvShape& s; int pix, iy0, ix0, krow; bool ok;
+        const T* x; const ConvShape& s; int pix, iy0, ix0, krow; bool ok; uint32_t live;
         __device__ __forceinline__ Dev(const ConvFwdB& L, int origin, int tid) : x(L.x), s(L.s) {
             const int n = origin + tid % BMN;
             ok = n < L.N;
@@ -174,33 +181,35 @@ template <typename T, bool FAST> struct ConvFwdB {
             pix = (((int)b * s.Cin * s.H + iy0) * s.W + ix0) * (int)sizeof(T);  // signed byte offset of tap (c=0,ky=0,kx=0)
             krow = __builtin_amdgcn_readfirstlane(tid / BMN);
         }
-        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) const {
+        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) {
             const int HW = s.H * s.W;
             if (FAST) {
                 const uint32_t kyx = s.div_Cin.div(k0), c0 = k0 - kyx * s.Cin;
                 const uint32_t ky = s.div_kw.div(kyx), kx = kyx - ky * s.kw;
                 const bool in = ok && (unsigned)(iy0 + (int)ky) < (unsigned)s.H && (unsigned)(ix0 + (int)kx) < (unsigned)s.W;
+                live = in ? ~0u : 0u;
                 const int uni = (((int)c0 + krow) * HW + (int)ky * s.W + (int)kx) * (int)sizeof(T);
                 const uint32_t v = in ? (uint32_t)(pix + uni) : 0u;
 #pragma unroll
                 for (int i = 0; i < Map::CNT; ++i) r[i] = ldg(x, v + (uint32_t)(i * Map::STEP * HW * (int)sizeof(T)));
-#pragma unroll
-                for (int i = 0; i < Map::CNT; ++i) r[i] = in ? r[i] : T(0);
             } else {
                 const int KK = s.kh * s.kw;
-                bool in[Map::CNT];
+                live = 0;
 #pragma unroll
                 for (int i = 0; i < Map::CNT; ++i) {
                     const int k = k0 + krow + i * Map::STEP;
                     const uint32_t c = s.div_KK.div(k), rr = k - c * KK;
                     const uint32_t ky = s.div_kw.div(rr), kx = rr - ky * s.kw;
-                    in[i] = ok && k < kend && (unsigned)(iy0 + (int)ky) < (unsigned)s.H && (unsigned)(ix0 + (int)kx) < (unsigned)s.W;
+                    const bool in = ok && k < kend && (unsigned)(iy0 + (int)ky) < (unsigned)s.H && (unsigned)(ix0 + (int)kx) < (unsigned)s.W;
+                    live |= in ? (1u << i) : 0u;
                     const int uni = ((int)c * HW + (int)ky * s.W + (int)kx) * (int)sizeof(T);
-                    r[i] = ldg(x, in[i] ? (uint32_t)(pix + uni) : 0u);
+                    r[i] = ldg(x, in ? (uint32_t)(pix + uni) : 0u);
                 }
-#pragma unroll
-                for (int i = 0; i < Map::CNT; ++i) r[i] = in[i] ? r[i] : T(0);
             }
+        }
+        __device__ __forceinline__ void mask(T (&r)[Map::CNT]) const {
+#pragma unroll
+            for (int i = 0; i < Map::CNT; ++i) r[i] = ((live >> i) & 1u) ? r[i] : T(0);
         }
     };
 };
@@ -216,7 +225,7 @@ template <typename T, bool FAST> struct ConvDgradB {
     int N;  // B*H*W
     template <int BMN, int BK, int NT> struct Dev {
         typedef SlabMap<BMN, BK, NT, false> Map;
-        const T* g; const ConvShape& s; int img, yp, xp, krow; bool ok;
+        const T* g; const ConvShape& s; int img, yp, xp, krow; bool ok; uint32_t live;
         __device__ __forceinline__ Dev(const ConvDgradB& L, int origin, int tid) : g(L.g), s(L.s) {
             const int n = origin + tid % BMN;
             ok = n < L.N;
@@ -241,33 +250,36 @@ template <typename T, bool FAST> struct ConvDgradB {
             in = in && cy < s.oh && cx < s.ow;
             return img + (cy * s.ow + cx) * (int)sizeof(T);
         }
-        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) const {
+        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) {
             const int L = s.oh * s.ow;
             if (FAST) {
                 const uint32_t kyx = s.div_Cout.div(k0), oc0 = k0 - kyx * s.Cout;
                 const uint32_t ky = s.div_kw.div(kyx), kx = kyx - ky * s.kw;
                 bool in;
                 const int t = tap((int)ky, (int)kx, in);
+                live = in ? ~0u : 0u;
                 const uint32_t v = in ? (uint32_t)(t + ((int)oc0 + krow) * L * (int)sizeof(T)) : 0u;
 #pragma unroll
                 for (int i = 0; i < Map::CNT; ++i) r[i] = ldg(g, v + (uint32_t)(i * Map::STEP * L * (int)sizeof(T)));
-#pragma unroll
-                for (int i = 0; i < Map::CNT; ++i) r[i] = in ? r[i] : T(0);
             } else {
                 const int KK = s.kh * s.kw;
-                bool in[Map::CNT];
+                live = 0;
 #pragma unroll
                 for (int i = 0; i < Map::CNT; ++i) {
                     const int k = k0 + krow + i * Map::STEP;
                     const uint32_t oc = s.div_KK.div(k), rr = k - oc * KK;
                     const uint32_t ky = s.div_kw.div(rr), kx = rr - ky * s.kw;
-                    const int t = tap((int)ky, (int)kx, in[i]);
-                    in[i] = in[i] && k < kend;
-                    r[i] = ldg(g, in[i] ? (uint32_t)(t + (int)oc * L * (int)sizeof(T)) : 0u);
+                    bool in;
+                    const int t = tap((int)ky, (int)kx, in);
+                    in = in && k < kend;
+                    live |= in ? (1u << i) : 0u;
+                    r[i] = ldg(g, in ? (uint32_t)(t + (int)oc * L * (int)sizeof(T)) : 0u);
                 }
-#pragma unroll
-                for (int i = 0; i < Map::CNT; ++i) r[i] = in[i] ? r[i] : T(0);
             }
+        }
+        __device__ __forceinline__ void mask(T (&r)[Map::CNT]) const {
+#pragma unroll
+            for (int i = 0; i < Map::CNT; ++i) r[i] = ((live >> i) & 1u) ? r[i] : T(0);
         }
     };
 };
@@ -281,7 +293,7 @@ template <typename T> struct ConvWgradA {
         typedef SlabMap<BMN, BK, NT, true> Map;
         const T* g; const ConvShape& s; int klane;
         uint32_t moff[Map::CNT];  // oc * L * sizeof(T), oc clamped into range
-        uint32_t okmask;
+        uint32_t okmask, live;
         __device__ __forceinline__ Dev(const ConvWgradA& L, int origin, int tid) : g(L.g), s(L.s) {
             klane = tid % BK;
             okmask = 0;
@@ -294,17 +306,20 @@ template <typename T> struct ConvWgradA {
                 moff[i] = (uint32_t)((ok ? m : 0) * Lp * (int)sizeof(T));
             }
         }
-        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) const {
+        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) {
             const int k = k0 + klane;
             const bool kok = k < kend;
+            live = kok ? okmask : 0u;
             const int L = s.oh * s.ow;
             const uint32_t kk = kok ? k : (uint32_t)k0;  // k0 < kend always
             const uint32_t b = s.div_L.div(kk), l = kk - b * L;
             const uint32_t v = (b * (uint32_t)s.Cout * L + l) * (uint32_t)sizeof(T);
 #pragma unroll
             for (int i = 0; i < Map::CNT; ++i) r[i] = ldg(g, v + moff[i]);
+        }
+        __device__ __forceinline__ void mask(T (&r)[Map::CNT]) const {
 #pragma unroll
-            for (int i = 0; i < Map::CNT; ++i) r[i] = (kok && ((okmask >> i) & 1u)) ? r[i] : T(0);
+            for (int i = 0; i < Map::CNT; ++i) r[i] = ((live >> i) & 1u) ? r[i] : T(0);
         }
     };
 };
@@ -318,7 +333,7 @@ template <typename T> struct ConvWgradB {
     int N;  // Cin*kh*kw
     template <int BMN, int BK, int NT> struct Dev {
         typedef SlabMap<BMN, BK, NT, true> Map;
-        const T* x; const ConvShape& s; int klane;
+        const T* x; const ConvShape& s; int klane; uint32_t live;
         int off[Map::CNT];   // (c*H*W + (ky-ph)*W + (kx-pw)) * sizeof(T)
         int kyx[Map::CNT];   // (ky-ph) << 16 | ((kx-pw) & 0xffff); INT_MIN when the column is out of range
         __device__ __forceinline__ Dev(const ConvWgradB& L, int origin, int tid) : x(L.x), s(L.s) {
@@ -339,7 +354,7 @@ template <typename T> struct ConvWgradB {
                 }
             }
         }
-        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) const {
+        __device__ __forceinline__ void load(int k0, int kend, T (&r)[Map::CNT]) {
             const int k = k0 + klane;
             const bool kok = k < kend;
             const uint32_t kk = kok ? k : (uint32_t)k0;
@@ -348,15 +363,18 @@ template <typename T> struct ConvWgradB {
             const uint32_t oy = s.div_ow.div(l), ox = l - oy * s.ow;
             const int y0 = (int)oy * s.sh, x0 = (int)ox * s.sw;
             const int pix = (((int)b * s.Cin * s.H + y0) * s.W + x0) * (int)sizeof(T);
-            bool in[Map::CNT];
+            live = 0;
 #pragma unroll
             for (int i = 0; i < Map::CNT; ++i) {
                 const int dy = kyx[i] >> 16, dx = (int)(short)(kyx[i] & 0xffff);
-                in[i] = kok && kyx[i] != INT_MIN && (unsigned)(y0 + dy) < (unsigned)s.H && (unsigned)(x0 + dx) < (unsigned)s.W;
-                r[i] = ldg(x, in[i] ? (uint32_t)(pix + off[i]) : 0u);
+                const bool in = kok && kyx[i] != INT_MIN && (unsigned)(y0 + dy) < (unsigned)s.H && (unsigned)(x0 + dx) < (unsigned)s.W;
+                live |= in ? (1u << i) : 0u;
+                r[i] = ldg(x, in ? (uint32_t)(pix + off[i]) : 0u);
             }
+        }
+        __device__ __forceinline__ void mask(T (&r)[Map::CNT]) const {
 #pragma unroll
-            for (int i = 0; i < Map::CNT; ++i) r[i] = in[i] ? r[i] : T(0);
+            for (int i = 0; i < Map::CNT; ++i) r[i] = ((live >> i) & 1u) ? r[i] : T(0);
         }
     };
 };
@@ -424,11 +442,14 @@ __global__ __launch_bounds__(Cfg::NT) void igemm_kernel(AL al, BL bl, EP ep, int
     T ra[AMap::CNT], rb[BMap::CNT];
     ad.load(kbeg, kend, ra);
     bd.load(kbeg, kend, rb);
+    ad.mask(ra);
+    bd.mask(rb);
     AMap::store(As[0], ra, tid);
     BMap::store(Bs[0], rb, tid);
     __syncthreads();
 
     const int lrow = lane / MF::BLK, lcol = lane % MF::BLK;
+    constexpr int STORE_AT = (BK / MF::KSTEP * 3 / 4) * MF::KSTEP;  // k-step at which the prefetched slab goes to LDS
     int cur = 0;
     for (int k0 = kbeg; k0 < kend; k0 += BK) {
         const bool more = k0 + BK < kend;
@@ -440,6 +461,16 @@ __global__ __launch_bounds__(Cfg::NT) void igemm_kernel(AL al, BL bl, EP ep, int
         const T* Bc = Bs[cur] + lrow * BMap::LD + wn0 + lcol;
 #pragma unroll
         for (int kk = 0; kk < BK; kk += MF::KSTEP) {
+            if (kk == STORE_AT && more) {
+                // The next slab's loads were issued a half slab of MFMAs ago; writing them to the other LDS stage
+                // here lets the LDS stores drain under the remaining MFMAs instead of after them.
+                __builtin_amdgcn_sched_barrier(0);
+                ad.mask(ra);
+                bd.mask(rb);
+                AMap::store(As[cur ^ 1], ra, tid);
+                BMap::store(Bs[cur ^ 1], rb, tid);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             T a[TM], b[TN];
 #pragma unroll
             for (int i = 0; i < TM; ++i) a[i] = Ac[kk * AMap::LD + i * MF::BLK];
@@ -449,10 +480,6 @@ __global__ __launch_bounds__(Cfg::NT) void igemm_kernel(AL al, BL bl, EP ep, int
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) acc[i][j] = MF::mma(a[i], b[j], acc[i][j]);
-        }
-        if (more) {
-            AMap::store(As[cur ^ 1], ra, tid);
-            BMap::store(Bs[cur ^ 1], rb, tid);
         }
         __syncthreads();
         cur ^= 1;
