@@ -13,6 +13,7 @@
 #include <cstdlib>
 
 #include "igemm_core.hpp"
+#include "wgrad_patch.hpp"
 
 namespace fx {
 int col2im_f32(fx_ctx*, const float*, float*, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, int);
@@ -228,7 +229,18 @@ int wgrad_tile(fx_ctx* c, const T* x, const T* g, T* dw, const Dims& d, int mode
 }
 
 template <typename T>
-i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d) {
+wgp::Plan patch_plan(fx_ctx* c, const Dims& d, int mode) {
+    if constexpr (sizeof(T) == 4) {
+        if (mode == 0 && variant() != 9)
+            return wgp::make_plan(c ? c->num_cus : 256, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
+    }
+    return wgp::Plan();
+}
+
+template <typename T>
+i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
+    const wgp::Plan pl = patch_plan<T>(c, d, mode);
+    if (pl.ok) return wgp::workspace_bytes(pl, d.Cout, d.Cin);
     int splits, kps;
     if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64) wgrad_plan<T, TileM128>(c, d, &splits, &kps);
     else wgrad_plan<T, TileSmall>(c, d, &splits, &kps);
@@ -243,13 +255,18 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
     FX_REQUIRE(mode == 0 || mode == 1, "fx_conv2d_wgrad: mode must be 0 or 1");
     Dims d;
     if (int rc = check_dims<T>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_wgrad")) return rc;
-    const i64 need = wgrad_ws_bytes<T>(c, d);
+    const i64 need = wgrad_ws_bytes<T>(c, d, mode);
     FX_REQUIRE(ws == nullptr || ws_bytes >= need, "fx_conv2d_wgrad: workspace of %lld bytes is smaller than the %lld needed",
                (long long)ws_bytes, (long long)need);
     std::lock_guard<std::mutex> lk(c->launch_mutex);
-    if constexpr (sizeof(T) == 4) if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64 && variant() == 1) return wgrad_tile<T, TileM128K32>(c, x, g, dw, d, mode, ws);
-    if constexpr (sizeof(T) == 4) if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64 && variant() == 2) return wgrad_tile<T, TileN64>(c, x, g, dw, d, mode, ws);
-    if constexpr (sizeof(T) == 4) if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64 && variant() == 3) return wgrad_tile<T, TileN64K32>(c, x, g, dw, d, mode, ws);
+    if constexpr (sizeof(T) == 4) {
+        const wgp::Plan pl = patch_plan<T>(c, d, mode);
+        if (pl.ok) {
+            float* part = (float*)(ws ? ws : c->get_scratch(need));
+            if (!part) return FX_ERR_OOM;
+            return wgp::run(c, pl, x, g, dw, part, Cin, H, W, Cout, sh, sw, ph, pw, d.oh, d.ow);
+        }
+    }
     if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64) return wgrad_tile<T, TileM128>(c, x, g, dw, d, mode, ws);
     return wgrad_tile<T, TileSmall>(c, x, g, dw, d, mode, ws);
 }
@@ -264,7 +281,7 @@ extern "C" int64_t fx_conv2d_workspace_bytes(int kind, int dtype, int mode, int6
         return -1;
     if (kind == FX_CONV_FWD) return dtype == FX_F64 ? fwd_ws_bytes<double>(d) : fwd_ws_bytes<float>(d);
     if (kind == FX_CONV_DGRAD) return dtype == FX_F64 ? dgrad_ws_bytes<double>(d, mode) : dgrad_ws_bytes<float>(d, mode);
-    if (kind == FX_CONV_WGRAD) return dtype == FX_F64 ? wgrad_ws_bytes<double>(nullptr, d) : wgrad_ws_bytes<float>(nullptr, d);
+    if (kind == FX_CONV_WGRAD) return dtype == FX_F64 ? wgrad_ws_bytes<double>(nullptr, d, mode) : wgrad_ws_bytes<float>(nullptr, d, mode);
     fx::set_error("fx_conv2d_workspace_bytes: unknown kind %d", kind);
     return -1;
 }

@@ -316,6 +316,47 @@ def test_conv2d_fwd_dgrad_wgrad_vs_oracle(ctx, orc, dtype):
             assert rel_err(lit_dw, orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 1)) <= tol * 8, ("literal wgrad", case)
 
 
+# 3x3 weight gradients that take the LDS-patch kernel (Cin % 32 == 0, even output width, Cout >= 32) in its
+# variants: 64/128-row tiles, ragged Cout, several rows per stage, strides, asymmetric padding, scalar loads
+# (W % 4 != 0), and a split count that does not divide the stages.  B, Cin, H, W, Cout, (sh, sw), (ph, pw)
+WGRAD_PATCH_CASES = [
+    (3, 32, 12, 10, 40, (1, 1), (1, 1)), (2, 64, 9, 14, 72, (1, 1), (0, 0)), (5, 32, 15, 18, 33, (1, 1), (1, 1)),
+    (2, 32, 17, 16, 64, (2, 1), (1, 1)), (2, 96, 16, 16, 160, (2, 2), (1, 1)), (3, 32, 11, 12, 48, (1, 2), (2, 0)),
+    (1, 32, 8, 6, 32, (1, 1), (1, 2)), (37, 32, 6, 8, 32, (1, 1), (1, 1)), (2, 32, 7, 62, 130, (3, 1), (1, 1)),
+    (21, 32, 29, 56, 32, (1, 1), (1, 1)),
+]
+
+
+def test_conv2d_wgrad_patch_kernel_shapes(ctx, orc):
+    import torch
+    from ferrox_amd import capi
+    import torch.nn.functional as F
+    rng = np.random.default_rng(57)
+    tol = TOL[np.dtype(np.float32)]
+    for (B, Cin, H, W, Cout, st, pd) in WGRAD_PATCH_CASES:
+        x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(np.float32)
+        oh, ow = orc.out_hw(H, W, 3, 3, st[0], st[1], pd[0], pd[1])
+        g = rng.standard_normal((B, Cout, oh, ow)).astype(np.float32)
+        dx_, dg_ = ctx.upload(x), ctx.upload(g)
+        dw = ctx.conv2d_wgrad(dx_, dg_, (Cout, Cin, 3, 3), st, pd, 0).numpy()
+        tw = torch.zeros((Cout, Cin, 3, 3), dtype=torch.float64, requires_grad=True)
+        F.conv2d(torch.from_numpy(x).double(), tw, stride=st, padding=pd).backward(torch.from_numpy(g).double())
+        case = (B, Cin, H, W, Cout, st, pd)
+        assert rel_err(dw, tw.grad.numpy()) <= tol * 8, case
+        assert rel_err(dw, orc.conv2d_wgrad(x, g, (Cout, Cin, 3, 3), st, pd, 0)) <= tol * 8, case
+        # same bits on a second run and with a caller-provided workspace of exactly the advertised size
+        assert np.array_equal(dw, ctx.conv2d_wgrad(dx_, dg_, (Cout, Cin, 3, 3), st, pd, 0).numpy()), case
+        need = capi.lib.fx_conv2d_workspace_bytes(capi.CONV_WGRAD, capi.FX_F32, 0, B, Cin, H, W, Cout, 3, 3, st[0], st[1], pd[0], pd[1])
+        assert need > 0
+        ws = ctx.empty((need // 4,), np.float32)
+        out = ctx.empty((Cout, Cin, 3, 3), np.float32)
+        capi.check(capi.lib.fx_conv2d_wgrad_f32(ctx.h, dx_.ptr, dg_.ptr, out.ptr, B, Cin, H, W, Cout, 3, 3, st[0], st[1],
+                                                pd[0], pd[1], 0, ws.ptr, need))
+        assert np.array_equal(dw, out.numpy()), case
+        assert capi.lib.fx_conv2d_wgrad_f32(ctx.h, dx_.ptr, dg_.ptr, out.ptr, B, Cin, H, W, Cout, 3, 3, st[0], st[1],
+                                            pd[0], pd[1], 0, ws.ptr, need - 4) != 0
+
+
 def test_conv2d_reference_vectors(ctx, golden):
     for key in ("conv2d_test", "conv2d_simple_forward", "conv2d_edge_cases"):
         gv = golden[key]
