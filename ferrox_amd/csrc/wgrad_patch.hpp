@@ -4,12 +4,14 @@
 // (the product the reference forms as grad_out_2d . im2col(x)^T, src/backend/storage/extensions/convolutions.rs:296-338).
 //
 // One stage = R output rows of one image.  A block copies, per stage,
-//   Gs[oc][pixel]      BM output-channel rows of g, pixels contiguous as in memory  (pitch GP,    GP % 32 == 1)
+//   Gs[oc][pixel]      BM output-channel rows of g, pixels contiguous as in memory  (pitch GP,    GP % 32 == 4)
 //   Xs[c][row][col]    32 input-channel planes of the zero-padded rows those pixels touch (pitch PLANE % 32 == 1)
 // and every wave then runs 9 accumulator blocks of 32(oc) x 32(c), one per filter tap: the MFMA A operand of lane l
 // is Gs[oc = l%32][pixel + l/32], the B operand of tap (ky,kx) is Xs[c = l%32][that pixel shifted by (ky,kx)].
-// The odd pitches put the 32 lanes of a half-wave on 32 different LDS banks for both reads.  The patch is
-// loaded once and serves all nine taps, so no im2col gather or bounds test is left in the MFMA loop.
+// The odd plane pitch puts the 32 lanes of a half-wave on 32 different LDS banks for the nine B reads of a step;
+// the single A read takes a 4-way conflict in exchange for 16-byte aligned rows (one 128-bit LDS store per
+// float4 of g).  The patch is loaded once and serves all nine taps, so no im2col gather or bounds test is left
+// in the MFMA loop.
 // The pixel range is split over blockIdx.z into partial sums kept tap-major ([oc][tap][c], coalesced stores);
 // a second kernel adds the partials in split order and writes dw in its [oc][c][tap] order.
 #pragma once
@@ -24,6 +26,16 @@ constexpr int KH = 3, KW = 3, KK = 9, CT = 32;  // filter taps; input channels p
 constexpr size_t LDS_BUDGET = 72 * 1024;        // per block, so that two blocks share a CU
 constexpr int SLACK = 64;                       // floats behind the last plane that the look-ahead read may touch
 
+// 16-byte load from global memory at a wave-uniform base plus a 32-bit byte offset (never a FLAT access, so it
+// does not tie up the LDS counter that the MFMA loop waits on).
+__device__ __forceinline__ float4 ldg4(const float* base, uint32_t byteoff) {
+    typedef __attribute__((address_space(1))) const char gchar;
+    typedef float v4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(1))) const v4 gv4;
+    const v4 v = *(gv4*)((gchar*)base + byteoff);
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+
 struct Params {
     const float* x;
     const float* g;
@@ -36,14 +48,21 @@ struct Params {
 };
 
 
-// PREF: the next stage's global loads are issued before the MFMA loop of the current stage and parked in
-// registers, NG float4 of g and NX float4 of x per thread (needs VEC); otherwise a stage is loaded, then used.
-template <int WM, bool VEC, int NG, int NX>
+constexpr int LPR = 16;  // lanes that share one row of a staged operand in the prefetching variant
+
+// XR > 0 selects the prefetching variant: the next stage's global loads are issued before the MFMA loop of the
+// current stage and held in registers until that loop is done.  It needs WM == 4, VEC, rows of at most
+// 4*LPR floats (Kst <= 64, W <= 64) and exactly XR patch rows; thread t then owns float4 column t % 16 of rows
+// t/16 + 16u, so every address is a per-thread constant plus a wave-uniform step and a stage costs a handful of
+// vector instructions outside the MFMAs.  XR == 0: a stage is loaded, stored to LDS, then used.
+template <int WM, bool VEC, int XR>
 __global__ __launch_bounds__(64 * WM, 2) void wgrad_patch_kernel(const Params p) {
-    constexpr bool PREF = NG > 0;
-    static_assert(VEC || !PREF, "prefetch needs the vector path");
+    constexpr bool PREF = XR > 0;
+    static_assert(!PREF || (VEC && WM == 4), "prefetch needs the vector path and 256 threads");
     constexpr int NT = 64 * WM, BM = 32 * WM;
-    extern __shared__ float smem[];
+    constexpr int RPP = NT / LPR;                     // rows covered by one pass of the block
+    constexpr int NG = BM / RPP, NXC = CT / RPP, NX = NXC * (PREF ? XR : 1);
+    extern __shared__ __align__(16) float smem[];
     float* Gs = smem;
     float* Xs = smem + BM * p.GP;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
@@ -60,9 +79,7 @@ __global__ __launch_bounds__(64 * WM, 2) void wgrad_patch_kernel(const Params p)
         for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
     __syncthreads();
 
-    float4 gv[PREF ? NG : 1], xv[PREF ? NX : 1];
     const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-
     auto stage_ptrs = [&](int s, const float*& gsrc, const float*& xsrc, int& iy0) {
         const int b = (int)p.div_spi.div((uint32_t)s);
         const int oy0 = (s - b * p.spi) * p.R;
@@ -70,56 +87,86 @@ __global__ __launch_bounds__(64 * WM, 2) void wgrad_patch_kernel(const Params p)
         gsrc = p.g + ((i64)b * p.Cout + oc0) * L + (i64)oy0 * p.ow;
         xsrc = p.x + ((i64)b * p.Cin + c0) * p.H * p.W;
     };
-    auto g_load4 = [&](const float* gsrc, int i) {
-        const int row = (int)p.div_g4.div((uint32_t)i), q = i - row * k4;
-        return (i < ng4 && oc0 + row < p.Cout) ? *reinterpret_cast<const float4*>(gsrc + (i64)row * L + 4 * q) : zero4;
-    };
-    auto g_store4 = [&](int i, const float4& v) {
-        if (i < ng4) {
-            const int row = (int)p.div_g4.div((uint32_t)i), q = i - row * k4;
-            float* d = Gs + row * p.GP + 4 * q;
-            d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
-        }
-    };
-    auto x_load4 = [&](const float* xsrc, int iy0, int i) {
-        const int c = (int)p.div_xc.div((uint32_t)i), rem = i - c * (p.PR * w4);
-        const int r = (int)p.div_xr.div((uint32_t)rem), q = rem - r * w4;
-        const int iy = iy0 + r;
-        return (i < nx4 && iy >= 0 && iy < p.H) ? *reinterpret_cast<const float4*>(xsrc + ((i64)c * p.H + iy) * p.W + 4 * q) : zero4;
-    };
-    auto x_store4 = [&](int i, const float4& v) {
-        if (i < nx4) {
-            const int c = (int)p.div_xc.div((uint32_t)i), rem = i - c * (p.PR * w4);
-            const int r = (int)p.div_xr.div((uint32_t)rem), q = rem - r * w4;
-            float* d = Xs + c * p.PLANE + r * p.PW + p.pw + 4 * q;
-            d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
-        }
-    };
+
+    // ---- prefetching variant: registers of the stage in flight and the per-thread constants of its addresses
+    float4 gv[PREF ? NG : 1], xv[PREF ? NX : 1];
+    const int pq = tid & (LPR - 1), prow = tid / LPR;
+    const bool g_lane = pq < k4, x_lane = pq < w4;
+    const bool full_m = oc0 + BM <= p.Cout;
+    const uint32_t g_off = g_lane ? (uint32_t)(prow * L + 4 * pq) * 4u : 0u;
+    const uint32_t x_off = x_lane ? (uint32_t)(prow * p.H * p.W + 4 * pq) * 4u : 0u;
+    const int g_dst0 = prow * p.GP + 4 * pq;
+    const int x_dst0 = BM * p.GP + prow * p.PLANE + p.pw + 4 * pq;
+    uint32_t x_rows = 0;  // bit r: patch row r of the stage in flight lies inside the image
     auto prefetch = [&](int s) {
         const float *gsrc, *xsrc;
-        int iy0, t0 = tid;
-        asm volatile("" : "+v"(t0));  // keeps the per-stage index arithmetic out of long-lived registers
+        int iy0;
         stage_ptrs(s, gsrc, xsrc, iy0);
 #pragma unroll
-        for (int u = 0; u < NG; ++u) gv[PREF ? u : 0] = g_load4(gsrc, t0 + u * NT);
+        for (int u = 0; u < NG; ++u) {
+            const bool ok = full_m || oc0 + prow + u * RPP < p.Cout;
+            gv[PREF ? u : 0] = ldg4(gsrc + (i64)u * RPP * L, ok ? g_off : 0u);
+        }
+        x_rows = 0;
 #pragma unroll
-        for (int u = 0; u < NX; ++u) xv[PREF ? u : 0] = x_load4(xsrc, iy0, t0 + u * NT);
+        for (int r = 0; r < XR; ++r) {
+            const int iy = iy0 + r;
+            if (iy >= 0 && iy < p.H) {  // wave-uniform
+                x_rows |= 1u << r;
+#pragma unroll
+                for (int cu = 0; cu < NXC; ++cu)
+                    xv[PREF ? r * NXC + cu : 0] = ldg4(xsrc + ((i64)cu * RPP * p.H + iy) * p.W, x_off);
+            }
+        }
     };
     auto park = [&]() {
-        int t0 = tid;
-        asm volatile("" : "+v"(t0));
+        int gd = g_dst0, xd = x_dst0;
+        asm volatile("" : "+v"(gd), "+v"(xd));  // recompute the row addresses here instead of keeping 14 of them alive
+        float* const g_dst = smem + gd;
+        float* const x_dst = smem + xd;
+        if (g_lane) {
 #pragma unroll
-        for (int u = 0; u < NG; ++u) g_store4(t0 + u * NT, gv[PREF ? u : 0]);
+            for (int u = 0; u < NG; ++u) {
+                const bool ok = full_m || oc0 + prow + u * RPP < p.Cout;
+                const float4 v = ok ? gv[PREF ? u : 0] : zero4;
+                float* d = g_dst + u * RPP * p.GP;
+                d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+            }
+        }
+        if (x_lane) {
 #pragma unroll
-        for (int u = 0; u < NX; ++u) x_store4(t0 + u * NT, xv[PREF ? u : 0]);
+            for (int r = 0; r < XR; ++r) {
+                const bool ok = (x_rows >> r) & 1;  // wave-uniform
+#pragma unroll
+                for (int cu = 0; cu < NXC; ++cu) {
+                    const float4 v = ok ? xv[PREF ? r * NXC + cu : 0] : zero4;
+                    float* d = x_dst + cu * RPP * p.PLANE + r * p.PW;
+                    d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+                }
+            }
+        }
     };
+
+    // ---- plain variant
     auto stage_direct = [&](int s) {
         const float *gsrc, *xsrc;
         int iy0;
         stage_ptrs(s, gsrc, xsrc, iy0);
         if constexpr (VEC) {
-            for (int i = tid; i < ng4; i += NT) g_store4(i, g_load4(gsrc, i));
-            for (int i = tid; i < nx4; i += NT) x_store4(i, x_load4(xsrc, iy0, i));
+            for (int i = tid; i < ng4; i += NT) {
+                const int row = (int)p.div_g4.div((uint32_t)i), q = i - row * k4;
+                const float4 v = oc0 + row < p.Cout ? ldg4(gsrc, (uint32_t)(row * L + 4 * q) * 4u) : zero4;
+                float* d = Gs + row * p.GP + 4 * q;
+                d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+            }
+            for (int i = tid; i < nx4; i += NT) {
+                const int c = (int)p.div_xc.div((uint32_t)i), rem = i - c * (p.PR * w4);
+                const int r = (int)p.div_xr.div((uint32_t)rem), q = rem - r * w4;
+                const int iy = iy0 + r;
+                const float4 v = iy >= 0 && iy < p.H ? ldg4(xsrc, (uint32_t)((c * p.H + iy) * p.W + 4 * q) * 4u) : zero4;
+                float* d = Xs + c * p.PLANE + r * p.PW + p.pw + 4 * q;
+                d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+            }
         } else {
             for (int i = tid; i < BM * p.Kst; i += NT) {
                 const int row = (int)p.div_kst.div((uint32_t)i), q = i - row * p.Kst;
@@ -185,7 +232,11 @@ __global__ __launch_bounds__(64 * WM, 2) void wgrad_patch_kernel(const Params p)
         for (int s = s_beg; s < s_end; ++s) {
             const bool more = s + 1 < s_end;
             if (more) prefetch(s + 1);
+            // The other block on this CU may be staging: its address arithmetic must not win the issue slot over
+            // this wave's MFMAs, so the MFMA loop runs at raised wave priority.
+            __builtin_amdgcn_s_setprio(3);
             compute();
+            __builtin_amdgcn_s_setprio(0);
             __syncthreads();
             if (more) park();
             __syncthreads();
@@ -237,6 +288,7 @@ struct Plan {
 };
 
 inline int odd_pitch(int n) { return (n + 30) / 32 * 32 + 1; }  // smallest pitch >= n with pitch % 32 == 1
+inline int g_pitch(int n) { return odd_pitch(n); }    // smallest pitch >= n with pitch % 32 == 4
 
 inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, i64 oh, i64 ow) {
     Plan pl;
@@ -248,7 +300,7 @@ inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 k
     for (int R = 1; R <= oh; ++R) {
         if (oh % R) continue;
         const int PR = (int)((R - 1) * sh + kh), PW = (int)(W + 2 * pw);
-        const size_t smem = ((size_t)BM * odd_pitch((int)(R * ow)) + (size_t)CT * odd_pitch(PR * PW) + SLACK) * sizeof(float);
+        const size_t smem = ((size_t)BM * g_pitch((int)(R * ow)) + (size_t)CT * odd_pitch(PR * PW) + SLACK) * sizeof(float);
         if (smem > LDS_BUDGET) break;
         best = R;
         if (R * ow >= 48) break;
@@ -259,7 +311,7 @@ inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 k
     pl.PW = (int)(W + 2 * pw);
     pl.PLANE = odd_pitch(pl.PR * pl.PW);
     pl.Kst = (int)(best * ow);
-    pl.GP = odd_pitch(pl.Kst);
+    pl.GP = g_pitch(pl.Kst);
     pl.smem = ((size_t)BM * pl.GP + (size_t)CT * pl.PLANE + SLACK) * sizeof(float);
     // the last tap of the last pixel of a stage must stay inside the plane
     if ((pl.PR - 1) * pl.PW + (ow - 1) * sw + kw - 1 >= pl.PLANE) return pl;
@@ -295,25 +347,20 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
     p.part_stride = Cout * Cin * KK;
     const int BM = 32 * pl.WM;
     const dim3 grid((unsigned)(Cin / CT), (unsigned)fx::ceil_div(Cout, (i64)BM), (unsigned)pl.splits);
-#define FX_WGP_LAUNCH(WMV, VECV, NGV, NXV)                                                                            \
+#define FX_WGP_LAUNCH(WMV, VECV, XRV)                                                                                 \
     do {                                                                                                              \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_patch_kernel<WMV, VECV, NGV, NXV>,      \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_patch_kernel<WMV, VECV, XRV>,           \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
         FX_HIP_CHECK(attr);                                                                                           \
-        wgrad_patch_kernel<WMV, VECV, NGV, NXV><<<grid, dim3(64 * WMV), pl.smem, c->stream>>>(p);                     \
+        wgrad_patch_kernel<WMV, VECV, XRV><<<grid, dim3(64 * WMV), pl.smem, c->stream>>>(p);                          \
     } while (0)
-#define FX_WGP_DISPATCH(WMV)                                                                                          \
-    do {                                                                                                              \
-        if (vec && ng <= 4 && nx <= 4) FX_WGP_LAUNCH(WMV, true, 4, 4);                                                \
-        else if (vec && ng <= 7 && nx <= 6) FX_WGP_LAUNCH(WMV, true, 7, 6);                                           \
-        else if (vec) FX_WGP_LAUNCH(WMV, true, 0, 0);                                                                 \
-        else FX_WGP_LAUNCH(WMV, false, 0, 0);                                                                         \
-    } while (0)
-    const int NT = 64 * pl.WM;  // float4 loads per thread and stage: ng of g, nx of x
-    const i64 ng = fx::ceil_div((i64)BM * (pl.Kst / 4), (i64)NT), nx = fx::ceil_div((i64)CT * pl.PR * (W / 4), (i64)NT);
-    if (pl.WM == 4) FX_WGP_DISPATCH(4);
-    else FX_WGP_DISPATCH(2);
-#undef FX_WGP_DISPATCH
+    const bool pref = vec && pl.WM == 4 && pl.Kst <= 4 * LPR && W <= 4 * LPR;
+    if (pref && pl.PR == 3) FX_WGP_LAUNCH(4, true, 3);
+    else if (pref && pl.PR == 4) FX_WGP_LAUNCH(4, true, 4);
+    else if (pl.WM == 4 && vec) FX_WGP_LAUNCH(4, true, 0);
+    else if (pl.WM == 4) FX_WGP_LAUNCH(4, false, 0);
+    else if (vec) FX_WGP_LAUNCH(2, true, 0);
+    else FX_WGP_LAUNCH(2, false, 0);
 #undef FX_WGP_LAUNCH
     FX_LAUNCH_CHECK();
     const int n = (int)p.part_stride;

@@ -323,7 +323,8 @@ WGRAD_PATCH_CASES = [
     (3, 32, 12, 10, 40, (1, 1), (1, 1)), (2, 64, 9, 14, 72, (1, 1), (0, 0)), (5, 32, 15, 18, 33, (1, 1), (1, 1)),
     (2, 32, 17, 16, 64, (2, 1), (1, 1)), (2, 96, 16, 16, 160, (2, 2), (1, 1)), (3, 32, 11, 12, 48, (1, 2), (2, 0)),
     (1, 32, 8, 6, 32, (1, 1), (1, 2)), (37, 32, 6, 8, 32, (1, 1), (1, 1)), (2, 32, 7, 62, 130, (3, 1), (1, 1)),
-    (21, 32, 29, 56, 32, (1, 1), (1, 1)),
+    (21, 32, 29, 56, 32, (1, 1), (1, 1)), (2, 32, 10, 56, 100, (1, 1), (1, 1)), (3, 64, 28, 28, 96, (1, 1), (1, 1)),
+    (2, 32, 16, 16, 128, (1, 1), (1, 1)), (2, 32, 9, 64, 128, (1, 1), (0, 1)),
 ]
 
 
