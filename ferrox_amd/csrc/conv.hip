@@ -14,6 +14,7 @@
 
 #include "igemm_core.hpp"
 #include "wgrad_patch.hpp"
+#include "conv_patch.hpp"
 
 namespace fx {
 int col2im_f32(fx_ctx*, const float*, float*, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, int);
@@ -105,7 +106,27 @@ int fwd_tile(fx_ctx* c, const T* x, const T* w, T* y, const Dims& d) {
 }
 
 template <typename T>
-i64 fwd_ws_bytes(const Dims& d) {
+cpk::Plan fwd_patch_plan(fx_ctx* c, const Dims& d) {
+    if constexpr (sizeof(T) == 4) {
+        if (variant() != 9) return cpk::make_plan(c ? c->num_cus : 256, d.B, d.Cin, d.H, d.W, d.Cout, d.oh, d.ow, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
+    }
+    return cpk::Plan();
+}
+
+// The stride-1 data gradient is a forward pass over grad_out with padding k-1-p.
+template <typename T>
+cpk::Plan dgrad_patch_plan(fx_ctx* c, const Dims& d, int mode) {
+    if constexpr (sizeof(T) == 4) {
+        if (mode == 0 && variant() != 9 && d.sh == 1 && d.sw == 1 && d.ph <= 2 && d.pw <= 2)
+            return cpk::make_plan(c ? c->num_cus : 256, d.B, d.Cout, d.oh, d.ow, d.Cin, d.H, d.W, d.kh, d.kw, 1, 1, 2 - d.ph, 2 - d.pw);
+    }
+    return cpk::Plan();
+}
+
+template <typename T>
+i64 fwd_ws_bytes(fx_ctx* c, const Dims& d) {
+    const cpk::Plan pl = fwd_patch_plan<T>(c, d);
+    if (pl.ok) return cpk::workspace_bytes(pl, d.Cout);
     return d.Cin % CONV_BK == 0 ? d.Cin * d.Cout * d.kh * d.kw * (i64)sizeof(T) : 0;
 }
 
@@ -116,10 +137,18 @@ int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64
     FX_REQUIRE(x && w && y, "fx_conv2d_fwd: null pointer");
     Dims d;
     if (int rc = check_dims<T>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_fwd")) return rc;
-    const i64 need = fwd_ws_bytes<T>(d);
+    const i64 need = fwd_ws_bytes<T>(c, d);
     FX_REQUIRE(ws == nullptr || ws_bytes >= need, "fx_conv2d_fwd: workspace of %lld bytes is smaller than the %lld needed",
                (long long)ws_bytes, (long long)need);
     std::lock_guard<std::mutex> lk(c->launch_mutex);
+    if constexpr (sizeof(T) == 4) {
+        const cpk::Plan pl = fwd_patch_plan<T>(c, d);
+        if (pl.ok) {
+            float* wimg = (float*)(ws ? ws : c->get_scratch(need));
+            if (!wimg) return FX_ERR_OOM;
+            return cpk::run(c, pl, x, w, y, wimg, 0, Cout, Cin, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw);
+        }
+    }
     if (need > 0) {
         T* wp = (T*)(ws ? ws : c->get_scratch(need));
         if (!wp) return FX_ERR_OOM;
@@ -146,8 +175,10 @@ int dgrad_tile(fx_ctx* c, const T* g, const T* wt, T* dx, const Dims& d) {
 }
 
 template <typename T>
-i64 dgrad_ws_bytes(const Dims& d, int mode) {
+i64 dgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     if (mode == 1) return d.Cin * d.kh * d.kw * d.B * d.oh * d.ow * (i64)sizeof(T);
+    const cpk::Plan pl = dgrad_patch_plan<T>(c, d, mode);
+    if (pl.ok) return cpk::workspace_bytes(pl, d.Cin);
     return d.Cin * d.Cout * d.kh * d.kw * (i64)sizeof(T);
 }
 
@@ -159,7 +190,7 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
     FX_REQUIRE(mode == 0 || mode == 1, "fx_conv2d_dgrad: mode must be 0 or 1");
     Dims d;
     if (int rc = check_dims<T>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_dgrad")) return rc;
-    const i64 need = dgrad_ws_bytes<T>(d, mode);
+    const i64 need = dgrad_ws_bytes<T>(c, d, mode);
     FX_REQUIRE(ws == nullptr || ws_bytes >= need, "fx_conv2d_dgrad: workspace of %lld bytes is smaller than the %lld needed",
                (long long)ws_bytes, (long long)need);
     if (mode == 1) {
@@ -182,6 +213,10 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
     std::lock_guard<std::mutex> lk(c->launch_mutex);
     T* wt = (T*)(ws ? ws : c->get_scratch(need));
     if (!wt) return FX_ERR_OOM;
+    if constexpr (sizeof(T) == 4) {
+        const cpk::Plan pl = dgrad_patch_plan<T>(c, d, mode);
+        if (pl.ok) return cpk::run(c, pl, g, w, dx, wt, 1, Cout, Cin, B, Cout, d.oh, d.ow, Cin, H, W, 1, 1, 2 - ph, 2 - pw);
+    }
     if (Cout % CONV_BK == 0) {
         if (int rc = permute_weights<T>(c, w, wt, d, 2)) return rc;
         if constexpr (sizeof(T) == 4) if (Cin > 32 && variant() == 1) return dgrad_tile<T, TileM64N256, true>(c, g, wt, dx, d);
@@ -279,8 +314,8 @@ extern "C" int64_t fx_conv2d_workspace_bytes(int kind, int dtype, int mode, int6
     if (dtype == FX_F64 ? check_dims<double>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_workspace_bytes")
                         : check_dims<float>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_workspace_bytes"))
         return -1;
-    if (kind == FX_CONV_FWD) return dtype == FX_F64 ? fwd_ws_bytes<double>(d) : fwd_ws_bytes<float>(d);
-    if (kind == FX_CONV_DGRAD) return dtype == FX_F64 ? dgrad_ws_bytes<double>(d, mode) : dgrad_ws_bytes<float>(d, mode);
+    if (kind == FX_CONV_FWD) return dtype == FX_F64 ? fwd_ws_bytes<double>(nullptr, d) : fwd_ws_bytes<float>(nullptr, d);
+    if (kind == FX_CONV_DGRAD) return dtype == FX_F64 ? dgrad_ws_bytes<double>(nullptr, d, mode) : dgrad_ws_bytes<float>(nullptr, d, mode);
     if (kind == FX_CONV_WGRAD) return dtype == FX_F64 ? wgrad_ws_bytes<double>(nullptr, d, mode) : wgrad_ws_bytes<float>(nullptr, d, mode);
     fx::set_error("fx_conv2d_workspace_bytes: unknown kind %d", kind);
     return -1;

@@ -1,0 +1,283 @@
+// 3x3 convolution forward (f32) with the input patch and the weights staged in LDS; the stride-1 data gradient
+// runs through the same kernel as a forward pass over grad_out with flipped, transposed weights.
+//
+// y[b][m][oy][ox] = sum over (c, ky, kx) of wgt[m][c][ky][kx] * in[b][c][oy*sh+ky-ph][ox*sw+kx-pw]
+// (the product the reference forms as filter_2d . im2col(x), src/backend/storage/extensions/convolutions.rs:218-290).
+//
+// A block (4 waves, WM along the output channels) owns BM = 32*WM output channels x 32*TN*(4/WM) consecutive
+// output pixels of one image and walks the input channels in chunks of 8 (one stage each).  Per stage it holds in LDS
+//   Ws[m][tap*8 + c]   the weights of the chunk, pitch 73 (odd: the 32 lanes of an A read hit 32 banks)
+//   Xs[c][row][col]    the zero-padded input rows under the pixel tile, plane pitch odd for the same reason
+// so each of the nine taps reads the same patch at a shifted address and no im2col index arithmetic or bounds
+// test is left in the MFMA loop.  Ws arrives as a ready-made image (built once per call by wimg_kernel), so its
+// staging is a straight 16-byte copy; the patch rows use the regular thread-to-row map of the weight-gradient
+// kernel.  The next stage's global loads are issued before the MFMA loop of the current one.
+#pragma once
+#include "wgrad_patch.hpp"
+
+namespace cpk {
+using igemm::FastDiv;
+using igemm::f32x16;
+using wgp::ldg4;
+
+constexpr int CC = 8, NT = 256, KK = 9;
+constexpr int WPITCH = KK * CC + 1;         // 73
+constexpr int NXP = 4, MAX_PR = 2 * NXP;    // patch rows are staged two per pass
+constexpr int LPR = 16;                     // lanes per patch row: W <= 64
+constexpr int SLACK = 16;
+constexpr size_t LDS_BUDGET = 72 * 1024;
+
+struct Params {
+    const float* x;
+    const float* wimg;
+    float* y;
+    int C, H, W, M, OH, OW, sh, sw, ph, pw;
+    int PR, PW, PLANE, L, tpi, nchunks;
+    FastDiv div_tpi, div_ow;
+};
+
+// Weight images: out[mt][ch][m][tap*8 + cc], zero in column 72 and in rows past the last output channel.
+//   flip == 0 (forward):        wgt[m][c][tap]   = w[oc = m][c][tap]
+//   flip == 1 (data gradient):  wgt[m][c][tap]   = w[oc = c][cin = m][8 - tap]
+__global__ __launch_bounds__(256) void wimg_kernel(const float* __restrict__ w, float* __restrict__ out, int Cout, int Cin, int M,
+                                                   int BM, int nchunks, int flip, i64 n) {
+    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int col = (int)(i % WPITCH);
+    i64 r = i / WPITCH;
+    const int m = (int)(r % BM);
+    r /= BM;
+    const int ch = (int)(r % nchunks), mt = (int)(r / nchunks);
+    const int mm = mt * BM + m;
+    float v = 0.f;
+    if (col < KK * CC && mm < M) {
+        const int t = col / CC, c = ch * CC + col % CC;
+        v = flip ? w[((i64)c * Cin + mm) * KK + (KK - 1 - t)] : w[((i64)mm * Cin + c) * KK + t];
+    }
+    out[i] = v;
+}
+
+template <int WM, int TN>
+__global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
+    constexpr int BM = 32 * WM, WN = 4 / WM, NPIX = 32 * TN * WN;
+    constexpr int WIMG = BM * WPITCH;             // floats in one weight image
+    constexpr int NW = (WIMG / 4 + NT - 1) / NT;  // float4 of the image per thread (the last one only partly used)
+    extern __shared__ __align__(16) float smem[];
+    float* Ws = smem;
+    float* Xs = smem + WIMG;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
+    const int b = (int)p.div_tpi.div(blockIdx.x);
+    const int wm = wave % WM, wn = wave / WM;
+    const int pix0 = ((int)blockIdx.x - b * p.tpi) * NPIX;
+    const int wpix0 = pix0 + wn * 32 * TN;  // first pixel of this wave's columns
+    const int m0 = blockIdx.y * BM;
+    const int py0 = (int)p.div_ow.div((uint32_t)pix0);
+    const int iy_base = py0 * p.sh - p.ph;
+
+    for (int i = tid; i < CC * p.PLANE + SLACK; i += NT) Xs[i] = 0.f;  // the padding columns stay zero from here on
+    int boff[TN];  // LDS offset of this lane's pixel in acc block j (plus the plane of its channel of the pair)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int pi = wpix0 + j * 32 + l32;
+        const int py = (int)p.div_ow.div((uint32_t)pi), px = pi - py * p.OW;
+        boff[j] = (pi < p.L ? (py - py0) * p.sh * p.PW + px * p.sw : 0) + half * p.PLANE;
+    }
+    f32x16 acc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+    __syncthreads();
+
+    // staging: thread t copies float4 t + 256u of the weight image and owns float4 column t % 16 of patch rows
+    // 2u + rp of channel (t / 16) % 8, where rp = t / 128 is uniform over a wave.
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int pq = tid & (LPR - 1), xc = (tid >> 4) & (CC - 1), rp = tid >> 7;
+    const bool x_lane = pq < (p.W >> 2);
+    const uint32_t x_off = x_lane ? (uint32_t)(xc * p.H * p.W + 4 * pq) * 4u : 0u;
+    const int x_dst0 = WIMG + xc * p.PLANE + p.pw + 4 * pq;
+    const float* const wsrc0 = p.wimg + (i64)blockIdx.y * p.nchunks * WIMG;
+    const float* const xsrc0 = p.x + (i64)b * p.C * p.H * p.W;
+    float4 wv[NW], xv[NXP];
+    auto prefetch = [&](int ch) {
+        const float* wsrc = wsrc0 + (i64)ch * WIMG;
+#pragma unroll
+        for (int u = 0; u < NW; ++u) {
+            const int idx = tid + u * NT;
+            wv[u] = ldg4(wsrc, (uint32_t)((u + 1) * NT <= WIMG / 4 || idx < WIMG / 4 ? idx : 0) * 16u);
+        }
+        const float* xsrc = xsrc0 + (i64)ch * CC * p.H * p.W;
+#pragma unroll
+        for (int u = 0; u < NXP; ++u) {
+            const int r = 2 * u + rp, iy = iy_base + r;
+            if (r < p.PR && iy >= 0 && iy < p.H) xv[u] = ldg4(xsrc + (i64)iy * p.W, x_off);  // wave-uniform test
+            else xv[u] = zero4;
+        }
+    };
+    auto park = [&]() {
+        int xd = x_dst0, wd = tid;
+        asm volatile("" : "+v"(xd), "+v"(wd));  // recompute the addresses here instead of keeping them alive
+#pragma unroll
+        for (int u = 0; u < NW; ++u) {
+            const int idx = wd + u * NT;
+            if ((u + 1) * NT <= WIMG / 4 || idx < WIMG / 4) *reinterpret_cast<float4*>(Ws + 4 * idx) = wv[u];
+        }
+        if (x_lane) {
+#pragma unroll
+            for (int u = 0; u < NXP; ++u) {
+                const int r = 2 * u + rp;
+                if (r < p.PR) {  // wave-uniform
+                    const float4 v = xv[u];
+                    float* d = smem + xd + r * p.PW;
+                    d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+                }
+            }
+        }
+    };
+
+    // One stage: 9 taps x 4 channel pairs, fully unrolled; two register sets alternate so that the LDS reads of
+    // step i+1 are in flight while the MFMAs of step i run.
+    const float* const wa = Ws + (wm * 32 + l32) * WPITCH + half;
+    auto compute = [&]() {
+        float a0, b0[TN], a1, b1[TN];
+        const float* xrow[3] = {Xs, Xs + p.PW, Xs + 2 * p.PW};
+#pragma unroll
+        for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(boff[j]));  // form the 12 x TN read addresses per stage, not once
+        auto rd = [&](float& a, float (&bv)[TN], int step) {
+            const int t = step >> 2, cp = step & 3, ky = t / 3, kx = t % 3;
+            a = wa[t * CC + 2 * cp];
+            const float* src = xrow[ky] + 2 * cp * p.PLANE + kx;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) bv[j] = src[boff[j]];
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto mma = [&](float a, const float (&bv)[TN]) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, bv[j], acc[j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        rd(a0, b0, 0);
+#pragma unroll
+        for (int step = 0; step < KK * 4; step += 2) {
+            rd(a1, b1, step + 1);
+            mma(a0, b0);
+            if (step + 2 < KK * 4) rd(a0, b0, step + 2);
+            mma(a1, b1);
+        }
+    };
+
+    prefetch(0);
+    park();
+    __syncthreads();
+    for (int ch = 0; ch < p.nchunks; ++ch) {
+        const bool more = ch + 1 < p.nchunks;
+        if (more) prefetch(ch + 1);
+        __builtin_amdgcn_s_setprio(3);  // a co-resident block that is staging must not delay these MFMAs
+        compute();
+        __builtin_amdgcn_s_setprio(0);
+        __syncthreads();
+        if (more) park();
+        __syncthreads();
+    }
+
+    float* out = p.y + (i64)b * p.M * p.L;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int pi = wpix0 + j * 32 + l32;
+        if (pi < p.L) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int m = m0 + wm * 32 + igemm::Mfma<float>::row(e, lane);
+                if (m < p.M) out[(i64)m * p.L + pi] = acc[j][e];
+            }
+        }
+    }
+}
+
+struct Plan {
+    bool ok = false;
+    int WM = 4, TN = 0, PR = 0, PW = 0, PLANE = 0, tpi = 0, mtiles = 0, nchunks = 0;
+    size_t smem = 0;
+    int bm() const { return 32 * WM; }
+    int npix() const { return 32 * TN * (4 / WM); }
+    i64 wimg() const { return (i64)bm() * WPITCH; }
+};
+
+// C input channels of H x W, M output channels of OH x OW (already the dimensions of the pass that runs).
+// Among the tile shapes whose patch fits, takes the one with the least (rounds of co-resident blocks) x (work of
+// a block): padded pixels, padded channels and a nearly empty last round all cost MFMA time.
+inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph,
+                      i64 pw) {
+    Plan pl;
+    if (kh != 3 || kw != 3 || C % CC != 0 || W % 4 != 0 || W > 4 * LPR || sh > 8 || sw > 8) return pl;
+    const i64 L = OH * OW, slots = 2 * (i64)std::max(1, num_cus);
+    static const int shapes[8][2] = {{4, 8}, {4, 7}, {4, 6}, {4, 5}, {4, 4}, {2, 4}, {2, 3}, {2, 2}};
+    i64 best_cost = -1;
+    for (const auto& sp : shapes) {
+        const int wm = sp[0], tn = sp[1];
+        const i64 bm = 32 * wm, np = 32 * tn * (4 / wm), tiles = fx::ceil_div(L, np), mtiles = fx::ceil_div(M, bm);
+        const i64 rows = std::min<i64>(OH, (np - 1) / OW + 2), PR = (rows - 1) * sh + 3;
+        if (PR > MAX_PR) continue;
+        const i64 cost = fx::ceil_div(B * tiles * mtiles, slots) * np * bm;
+        if (best_cost < 0 || cost < best_cost) {
+            best_cost = cost;
+            pl.WM = wm;
+            pl.TN = tn;
+            pl.PR = (int)PR;
+            pl.tpi = (int)tiles;
+        }
+    }
+    if (best_cost < 0) return pl;
+    pl.PW = (int)(W + 2 * pw);
+    pl.PLANE = wgp::odd_pitch(pl.PR * pl.PW);
+    pl.smem = ((size_t)pl.wimg() + (size_t)CC * pl.PLANE + SLACK) * sizeof(float);
+    pl.mtiles = (int)fx::ceil_div(M, (i64)pl.bm());
+    pl.nchunks = (int)(C / CC);
+    if (pl.smem > LDS_BUDGET || B * pl.tpi > 0x7fffffff || pl.mtiles > 65535) return pl;
+    pl.ok = true;
+    return pl;
+}
+
+// Sized for 128-row images whatever tile was picked, so the figure does not depend on the CU count behind the plan.
+inline i64 workspace_bytes(const Plan& pl, i64 M) { return fx::ceil_div(M, (i64)128) * 128 * WPITCH * pl.nchunks * (i64)sizeof(float); }
+
+// w is the reference's [Cout][Cin][3][3] filter; flip selects the data-gradient image.
+inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float* y, float* wimg, int flip, i64 Cout, i64 Cin, i64 B,
+               i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw) {
+    const i64 n = (i64)pl.mtiles * pl.nchunks * pl.wimg();
+    wimg_kernel<<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(w, wimg, (int)Cout, (int)Cin, (int)M, pl.bm(),
+                                                                                  pl.nchunks, flip, n);
+    FX_LAUNCH_CHECK();
+    Params p;
+    p.x = x; p.wimg = wimg; p.y = y;
+    p.C = (int)C; p.H = (int)H; p.W = (int)W; p.M = (int)M; p.OH = (int)OH; p.OW = (int)OW;
+    p.sh = (int)sh; p.sw = (int)sw; p.ph = (int)ph; p.pw = (int)pw;
+    p.PR = pl.PR; p.PW = pl.PW; p.PLANE = pl.PLANE; p.L = (int)(OH * OW); p.tpi = pl.tpi; p.nchunks = pl.nchunks;
+    p.div_tpi = FastDiv((uint32_t)pl.tpi);
+    p.div_ow = FastDiv((uint32_t)OW);
+    const dim3 grid((unsigned)(B * pl.tpi), (unsigned)pl.mtiles);
+#define FX_CPK_LAUNCH(WMV, TNV)                                                                                       \
+    case WMV * 16 + TNV: {                                                                                            \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV>,                  \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
+        FX_HIP_CHECK(attr);                                                                                           \
+        conv_patch_kernel<WMV, TNV><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                                       \
+        break;                                                                                                        \
+    }
+    switch (pl.WM * 16 + pl.TN) {
+        FX_CPK_LAUNCH(4, 4)
+        FX_CPK_LAUNCH(4, 5)
+        FX_CPK_LAUNCH(4, 6)
+        FX_CPK_LAUNCH(4, 7)
+        FX_CPK_LAUNCH(4, 8)
+        FX_CPK_LAUNCH(2, 2)
+        FX_CPK_LAUNCH(2, 3)
+        FX_CPK_LAUNCH(2, 4)
+        default: FX_REQUIRE(false, "conv patch kernel: unexpected tile %d x %d", pl.WM, pl.TN);
+    }
+#undef FX_CPK_LAUNCH
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+}  // namespace cpk

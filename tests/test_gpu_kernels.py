@@ -358,6 +358,55 @@ def test_conv2d_wgrad_patch_kernel_shapes(ctx, orc):
                                             pd[0], pd[1], 0, ws.ptr, need - 4) != 0
 
 
+# 3x3 forward / stride-1 data-gradient shapes that take the LDS-patch kernel (channels % 8 == 0, W % 4 == 0,
+# W <= 64): 64- and 128-row tiles, ragged channel counts, ragged last pixel tile, paddings 0..2 (the data gradient
+# then runs with padding 2..0), a strided forward, the widest supported row.  B, Cin, H, W, Cout, (sh, sw), (ph, pw)
+CONV_PATCH_CASES = [
+    (2, 8, 6, 12, 16, (1, 1), (1, 1)), (3, 16, 8, 36, 100, (1, 1), (0, 0)), (2, 24, 4, 8, 136, (1, 1), (2, 2)),
+    (2, 64, 28, 28, 64, (1, 1), (1, 1)), (1, 8, 64, 64, 32, (1, 1), (1, 1)), (2, 16, 6, 16, 40, (2, 2), (1, 1)),
+    (2, 8, 5, 12, 24, (1, 1), (0, 1)), (5, 72, 6, 40, 200, (1, 1), (1, 1)), (2, 128, 6, 8, 72, (1, 1), (1, 0)),
+    (2, 8, 12, 12, 16, (1, 1), (1, 1)),
+]
+
+
+def test_conv2d_patch_kernel_shapes(ctx, orc):
+    import torch
+    import torch.nn.functional as F
+    from ferrox_amd import capi
+    rng = np.random.default_rng(58)
+    tol = TOL[np.dtype(np.float32)]
+    for (B, Cin, H, W, Cout, st, pd) in CONV_PATCH_CASES:
+        case = (B, Cin, H, W, Cout, st, pd)
+        x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(np.float32)
+        w = (rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9))).astype(np.float32)
+        oh, ow = orc.out_hw(H, W, 3, 3, st[0], st[1], pd[0], pd[1])
+        g = rng.standard_normal((B, Cout, oh, ow)).astype(np.float32)
+        dx_, dw_, dg_ = ctx.upload(x), ctx.upload(w), ctx.upload(g)
+        y = ctx.conv2d_fwd(dx_, dw_, st, pd).numpy()
+        dxg = ctx.conv2d_dgrad(dg_, dw_, x.shape, st, pd, 0).numpy()
+        tx = torch.from_numpy(x).double().requires_grad_(True)
+        tw = torch.from_numpy(w).double()
+        ty = F.conv2d(tx, tw, stride=st, padding=pd)
+        ty.backward(torch.from_numpy(g).double())
+        ay = F.conv2d(tx.detach().abs(), tw.abs(), stride=st, padding=pd).max().item()
+        assert np.abs(y - ty.detach().numpy()).max() <= tol * ay, ("fwd", case)
+        assert rel_err(dxg, tx.grad.numpy()) <= tol * 8, ("dgrad", case)
+        assert rel_err(y, orc.conv2d_fwd(x, w, st, pd)) <= tol * 8, ("fwd vs oracle", case)
+        assert rel_err(dxg, orc.conv2d_dgrad(g, w, x.shape, st, pd, 0)) <= tol * 8, ("dgrad vs oracle", case)
+        # caller-provided workspaces of exactly the advertised size give the same bits
+        dims = (B, Cin, H, W, Cout, 3, 3, st[0], st[1], pd[0], pd[1])
+        for kind, fn, a, b_, ref, shape in (
+                (capi.CONV_FWD, capi.lib.fx_conv2d_fwd_f32, dx_, dw_, y, y.shape),
+                (capi.CONV_DGRAD, capi.lib.fx_conv2d_dgrad_f32, dg_, dw_, dxg, x.shape)):
+            need = capi.lib.fx_conv2d_workspace_bytes(kind, capi.FX_F32, 0, *dims)
+            assert need >= 0, case
+            ws = ctx.empty((max(need, 4) // 4,), np.float32)
+            out = ctx.empty(shape, np.float32)
+            extra = () if kind == capi.CONV_FWD else (0,)
+            capi.check(fn(ctx.h, a.ptr, b_.ptr, out.ptr, *dims, *extra, ws.ptr, need))
+            assert np.array_equal(out.numpy(), ref), (kind, case)
+
+
 def test_conv2d_reference_vectors(ctx, golden):
     for key in ("conv2d_test", "conv2d_simple_forward", "conv2d_edge_cases"):
         gv = golden[key]
