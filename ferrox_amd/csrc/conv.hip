@@ -30,20 +30,15 @@ typedef Tile<128, 128, 16, 64, 64> TileM128;  // 4 waves as 2x2, 64x64 each
 typedef Tile<64, 128, 16, 64, 32> TileM64;    // 4 waves as 1x4, 64x32 each
 typedef Tile<32, 256, 16, 32, 64> TileM32;    // 4 waves as 1x4, 32x64 each
 typedef Tile<64, 64, 16, 32, 32> TileSmall;   // 4 waves as 2x2, 32x32 each
-// tuning variants
-typedef Tile<128, 128, 32, 64, 64> TileM128K32;
-typedef Tile<64, 256, 16, 64, 64> TileM64N256;
-typedef Tile<64, 256, 32, 64, 64> TileM64N256K32;
-typedef Tile<128, 192, 16, 64, 96> TileN192;
-typedef Tile<128, 192, 32, 64, 96> TileN192K32;
-typedef Tile<128, 64, 16, 64, 32> TileN64;
-typedef Tile<128, 64, 32, 64, 32> TileN64K32;
-static int variant() { const char* v = getenv("FX_CONV_VARIANT"); return v ? atoi(v) : 0; }
+// FX_CONV_GENERIC=1 in the environment sends every shape to the implicit-GEMM kernels (A/B timing, debugging).
+static bool generic_only() { const char* v = getenv("FX_CONV_GENERIC"); return v && atoi(v) != 0; }
 
 int gemm_t(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const float* A, const float* B, float* C) { return fx_gemm_f32(c, ta, tb, M, N, K, A, B, C); }
 int gemm_t(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const double* A, const double* B, double* C) { return fx_gemm_f64(c, ta, tb, M, N, K, A, B, C); }
 int col2im_t(fx_ctx* c, const float* col, float* out, i64 B, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, int layout) { return fx::col2im_f32(c, col, out, B, C, H, W, kh, kw, sh, sw, ph, pw, layout); }
 int col2im_t(fx_ctx* c, const double* col, double* out, i64 B, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, int layout) { return fx::col2im_f64(c, col, out, B, C, H, W, kh, kw, sh, sw, ph, pw, layout); }
+
+inline bool aligned16(const void* a, const void* b) { return (((uintptr_t)a | (uintptr_t)b) & 15) == 0; }
 
 struct Dims {
     i64 B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, oh, ow;
@@ -108,7 +103,7 @@ int fwd_tile(fx_ctx* c, const T* x, const T* w, T* y, const Dims& d) {
 template <typename T>
 cpk::Plan fwd_patch_plan(fx_ctx* c, const Dims& d) {
     if constexpr (sizeof(T) == 4) {
-        if (variant() != 9) return cpk::make_plan(c ? c->num_cus : 256, d.B, d.Cin, d.H, d.W, d.Cout, d.oh, d.ow, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
+        if (!generic_only()) return cpk::make_plan(c ? c->num_cus : 256, d.B, d.Cin, d.H, d.W, d.Cout, d.oh, d.ow, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
     }
     return cpk::Plan();
 }
@@ -117,7 +112,7 @@ cpk::Plan fwd_patch_plan(fx_ctx* c, const Dims& d) {
 template <typename T>
 cpk::Plan dgrad_patch_plan(fx_ctx* c, const Dims& d, int mode) {
     if constexpr (sizeof(T) == 4) {
-        if (mode == 0 && variant() != 9 && d.sh == 1 && d.sw == 1 && d.ph <= 2 && d.pw <= 2)
+        if (mode == 0 && !generic_only() && d.sh == 1 && d.sw == 1 && d.ph <= 2 && d.pw <= 2)
             return cpk::make_plan(c ? c->num_cus : 256, d.B, d.Cout, d.oh, d.ow, d.Cin, d.H, d.W, d.kh, d.kw, 1, 1, 2 - d.ph, 2 - d.pw);
     }
     return cpk::Plan();
@@ -125,9 +120,10 @@ cpk::Plan dgrad_patch_plan(fx_ctx* c, const Dims& d, int mode) {
 
 template <typename T>
 i64 fwd_ws_bytes(fx_ctx* c, const Dims& d) {
+    // enough for either kernel: a misaligned tensor sends a patch-kernel shape to the implicit GEMM
     const cpk::Plan pl = fwd_patch_plan<T>(c, d);
-    if (pl.ok) return cpk::workspace_bytes(pl, d.Cout);
-    return d.Cin % CONV_BK == 0 ? d.Cin * d.Cout * d.kh * d.kw * (i64)sizeof(T) : 0;
+    const i64 generic = d.Cin % CONV_BK == 0 ? d.Cin * d.Cout * d.kh * d.kw * (i64)sizeof(T) : 0;
+    return pl.ok ? std::max(generic, cpk::workspace_bytes(pl, d.Cout)) : generic;
 }
 
 template <typename T>
@@ -143,17 +139,16 @@ int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64
     std::lock_guard<std::mutex> lk(c->launch_mutex);
     if constexpr (sizeof(T) == 4) {
         const cpk::Plan pl = fwd_patch_plan<T>(c, d);
-        if (pl.ok) {
+        if (pl.ok && aligned16(x, ws)) {
             float* wimg = (float*)(ws ? ws : c->get_scratch(need));
             if (!wimg) return FX_ERR_OOM;
             return cpk::run(c, pl, x, w, y, wimg, 0, Cout, Cin, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw);
         }
     }
-    if (need > 0) {
+    if (d.Cin % CONV_BK == 0) {
         T* wp = (T*)(ws ? ws : c->get_scratch(need));
         if (!wp) return FX_ERR_OOM;
         if (int rc = permute_weights<T>(c, w, wp, d, 0)) return rc;
-        if constexpr (sizeof(T) == 4) if (Cout > 64 && Cin % 32 == 0 && variant() == 1) return fwd_tile<T, TileM128K32, true>(c, x, wp, y, d);
         if (Cout > 64) return fwd_tile<T, TileM128, true>(c, x, wp, y, d);
         if (Cout > 32) return fwd_tile<T, TileM64, true>(c, x, wp, y, d);
         return fwd_tile<T, TileM32, true>(c, x, wp, y, d);
@@ -178,8 +173,8 @@ template <typename T>
 i64 dgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     if (mode == 1) return d.Cin * d.kh * d.kw * d.B * d.oh * d.ow * (i64)sizeof(T);
     const cpk::Plan pl = dgrad_patch_plan<T>(c, d, mode);
-    if (pl.ok) return cpk::workspace_bytes(pl, d.Cin);
-    return d.Cin * d.Cout * d.kh * d.kw * (i64)sizeof(T);
+    const i64 generic = d.Cin * d.Cout * d.kh * d.kw * (i64)sizeof(T);
+    return pl.ok ? std::max(generic, cpk::workspace_bytes(pl, d.Cin)) : generic;
 }
 
 template <typename T>
@@ -215,12 +210,10 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
     if (!wt) return FX_ERR_OOM;
     if constexpr (sizeof(T) == 4) {
         const cpk::Plan pl = dgrad_patch_plan<T>(c, d, mode);
-        if (pl.ok) return cpk::run(c, pl, g, w, dx, wt, 1, Cout, Cin, B, Cout, d.oh, d.ow, Cin, H, W, 1, 1, 2 - ph, 2 - pw);
+        if (pl.ok && aligned16(g, wt)) return cpk::run(c, pl, g, w, dx, wt, 1, Cout, Cin, B, Cout, d.oh, d.ow, Cin, H, W, 1, 1, 2 - ph, 2 - pw);
     }
     if (Cout % CONV_BK == 0) {
         if (int rc = permute_weights<T>(c, w, wt, d, 2)) return rc;
-        if constexpr (sizeof(T) == 4) if (Cin > 32 && variant() == 1) return dgrad_tile<T, TileM64N256, true>(c, g, wt, dx, d);
-        if constexpr (sizeof(T) == 4) if (Cin > 32 && Cout % 32 == 0 && variant() == 2) return dgrad_tile<T, TileM64N256K32, true>(c, g, wt, dx, d);
         if (Cin > 64) return dgrad_tile<T, TileM128, true>(c, g, wt, dx, d);
         if (Cin > 32) return dgrad_tile<T, TileM64, true>(c, g, wt, dx, d);
         return dgrad_tile<T, TileM32, true>(c, g, wt, dx, d);
@@ -266,7 +259,7 @@ int wgrad_tile(fx_ctx* c, const T* x, const T* g, T* dw, const Dims& d, int mode
 template <typename T>
 wgp::Plan patch_plan(fx_ctx* c, const Dims& d, int mode) {
     if constexpr (sizeof(T) == 4) {
-        if (mode == 0 && variant() != 9)
+        if (mode == 0 && !generic_only())
             return wgp::make_plan(c ? c->num_cus : 256, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
     }
     return wgp::Plan();
@@ -275,11 +268,11 @@ wgp::Plan patch_plan(fx_ctx* c, const Dims& d, int mode) {
 template <typename T>
 i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     const wgp::Plan pl = patch_plan<T>(c, d, mode);
-    if (pl.ok) return wgp::workspace_bytes(pl, d.Cout, d.Cin);
     int splits, kps;
     if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64) wgrad_plan<T, TileM128>(c, d, &splits, &kps);
     else wgrad_plan<T, TileSmall>(c, d, &splits, &kps);
-    return splits > 1 ? (i64)splits * d.Cout * d.Cin * d.kh * d.kw * (i64)sizeof(T) : 0;
+    const i64 generic = splits > 1 ? (i64)splits * d.Cout * d.Cin * d.kh * d.kw * (i64)sizeof(T) : 0;
+    return pl.ok ? std::max(generic, wgp::workspace_bytes(pl, d.Cout, d.Cin)) : generic;
 }
 
 template <typename T>
@@ -296,7 +289,7 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
     std::lock_guard<std::mutex> lk(c->launch_mutex);
     if constexpr (sizeof(T) == 4) {
         const wgp::Plan pl = patch_plan<T>(c, d, mode);
-        if (pl.ok) {
+        if (pl.ok && aligned16(x, g) && aligned16(ws, ws)) {
             float* part = (float*)(ws ? ws : c->get_scratch(need));
             if (!part) return FX_ERR_OOM;
             return wgp::run(c, pl, x, g, dw, part, Cin, H, W, Cout, sh, sw, ph, pw, d.oh, d.ow);

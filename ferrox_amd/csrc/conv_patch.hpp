@@ -217,7 +217,7 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
         const int wm = sp[0], tn = sp[1];
         const i64 bm = 32 * wm, np = 32 * tn * (4 / wm), tiles = fx::ceil_div(L, np), mtiles = fx::ceil_div(M, bm);
         const i64 rows = std::min<i64>(OH, (np - 1) / OW + 2), PR = (rows - 1) * sh + 3;
-        if (PR > MAX_PR) continue;
+        if (PR > MAX_PR || mtiles * bm * 4 > M * 5) continue;  // no more than a quarter of the rows may be padding
         const i64 cost = fx::ceil_div(B * tiles * mtiles, slots) * np * bm;
         if (best_cost < 0 || cost < best_cost) {
             best_cost = cost;

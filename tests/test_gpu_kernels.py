@@ -316,15 +316,16 @@ def test_conv2d_fwd_dgrad_wgrad_vs_oracle(ctx, orc, dtype):
             assert rel_err(lit_dw, orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 1)) <= tol * 8, ("literal wgrad", case)
 
 
-# 3x3 weight gradients that take the LDS-patch kernel (Cin % 32 == 0, even output width, Cout >= 32) in its
-# variants: 64/128-row tiles, ragged Cout, several rows per stage, strides, asymmetric padding, scalar loads
-# (W % 4 != 0), and a split count that does not divide the stages.  B, Cin, H, W, Cout, (sh, sw), (ph, pw)
+# 3x3 weight gradients around the LDS-patch kernel (taken when Cin % 32 == 0, Cout > 64, W % 4 == 0, W <= 64, even
+# output width): ragged Cout, one and two output rows per stage, strides, asymmetric padding, the widest row, and
+# neighbours that fall back to the implicit GEMM (Cout <= 64, W % 4 != 0).  B, Cin, H, W, Cout, (sh, sw), (ph, pw)
 WGRAD_PATCH_CASES = [
     (3, 32, 12, 10, 40, (1, 1), (1, 1)), (2, 64, 9, 14, 72, (1, 1), (0, 0)), (5, 32, 15, 18, 33, (1, 1), (1, 1)),
     (2, 32, 17, 16, 64, (2, 1), (1, 1)), (2, 96, 16, 16, 160, (2, 2), (1, 1)), (3, 32, 11, 12, 48, (1, 2), (2, 0)),
     (1, 32, 8, 6, 32, (1, 1), (1, 2)), (37, 32, 6, 8, 32, (1, 1), (1, 1)), (2, 32, 7, 62, 130, (3, 1), (1, 1)),
     (21, 32, 29, 56, 32, (1, 1), (1, 1)), (2, 32, 10, 56, 100, (1, 1), (1, 1)), (3, 64, 28, 28, 96, (1, 1), (1, 1)),
-    (2, 32, 16, 16, 128, (1, 1), (1, 1)), (2, 32, 9, 64, 128, (1, 1), (0, 1)),
+    (2, 32, 16, 16, 128, (1, 1), (1, 1)), (2, 32, 9, 64, 128, (1, 1), (0, 1)), (40, 64, 14, 14, 200, (1, 1), (1, 1)),
+    (3, 32, 12, 20, 96, (1, 2), (2, 0)), (2, 32, 8, 24, 65, (2, 2), (0, 0)),
 ]
 
 
@@ -348,14 +349,15 @@ def test_conv2d_wgrad_patch_kernel_shapes(ctx, orc):
         # same bits on a second run and with a caller-provided workspace of exactly the advertised size
         assert np.array_equal(dw, ctx.conv2d_wgrad(dx_, dg_, (Cout, Cin, 3, 3), st, pd, 0).numpy()), case
         need = capi.lib.fx_conv2d_workspace_bytes(capi.CONV_WGRAD, capi.FX_F32, 0, B, Cin, H, W, Cout, 3, 3, st[0], st[1], pd[0], pd[1])
-        assert need > 0
-        ws = ctx.empty((need // 4,), np.float32)
+        assert need >= 0
+        ws = ctx.empty((max(need, 4) // 4,), np.float32)
         out = ctx.empty((Cout, Cin, 3, 3), np.float32)
         capi.check(capi.lib.fx_conv2d_wgrad_f32(ctx.h, dx_.ptr, dg_.ptr, out.ptr, B, Cin, H, W, Cout, 3, 3, st[0], st[1],
                                                 pd[0], pd[1], 0, ws.ptr, need))
         assert np.array_equal(dw, out.numpy()), case
-        assert capi.lib.fx_conv2d_wgrad_f32(ctx.h, dx_.ptr, dg_.ptr, out.ptr, B, Cin, H, W, Cout, 3, 3, st[0], st[1],
-                                            pd[0], pd[1], 0, ws.ptr, need - 4) != 0
+        if need > 0:
+            assert capi.lib.fx_conv2d_wgrad_f32(ctx.h, dx_.ptr, dg_.ptr, out.ptr, B, Cin, H, W, Cout, 3, 3, st[0], st[1],
+                                                pd[0], pd[1], 0, ws.ptr, need - 4) != 0
 
 
 # 3x3 forward / stride-1 data-gradient shapes that take the LDS-patch kernel (channels % 8 == 0, W % 4 == 0,
@@ -405,6 +407,34 @@ def test_conv2d_patch_kernel_shapes(ctx, orc):
             extra = () if kind == capi.CONV_FWD else (0,)
             capi.check(fn(ctx.h, a.ptr, b_.ptr, out.ptr, *dims, *extra, ws.ptr, need))
             assert np.array_equal(out.numpy(), ref), (kind, case)
+
+
+def test_conv2d_misaligned_tensors_match_aligned(ctx):
+    """Tensors that are only 4-byte aligned (a view into a larger buffer) cannot use the 16-byte loads of the
+    patch kernels; the library must fall back and give the implicit-GEMM result, not fault or misread."""
+    from ferrox_amd import capi
+    rng = np.random.default_rng(59)
+    B, Cin, H, W, Cout = 2, 32, 10, 56, 100
+    x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, 3, 3)) * 0.06).astype(np.float32)
+    g = rng.standard_normal((B, Cout, H, W)).astype(np.float32)
+    dims = (B, Cin, H, W, Cout, 3, 3, 1, 1, 1, 1)
+
+    def shifted(a):  # device copy of `a` that starts 4 bytes into its allocation
+        buf = ctx.upload(np.concatenate([np.zeros(1, np.float32), a.ravel()]))
+        return buf, buf.ptr + 4
+
+    (xb, xp), (gb, gp) = shifted(x), shifted(g)
+    dw_, dx_al, dg_al = ctx.upload(w), ctx.upload(x), ctx.upload(g)
+    y, dx, dwt = ctx.empty(g.shape, np.float32), ctx.empty(x.shape, np.float32), ctx.empty(w.shape, np.float32)
+    capi.check(capi.lib.fx_conv2d_fwd_f32(ctx.h, xp, dw_.ptr, y.ptr, *dims, None, 0))
+    capi.check(capi.lib.fx_conv2d_dgrad_f32(ctx.h, gp, dw_.ptr, dx.ptr, *dims, 0, None, 0))
+    capi.check(capi.lib.fx_conv2d_wgrad_f32(ctx.h, xp, gp, dwt.ptr, *dims, 0, None, 0))
+    tol = TOL[np.dtype(np.float32)] * 8
+    assert rel_err(y.numpy(), ctx.conv2d_fwd(dx_al, dw_, (1, 1), (1, 1)).numpy()) <= tol
+    assert rel_err(dx.numpy(), ctx.conv2d_dgrad(dg_al, dw_, x.shape, (1, 1), (1, 1), 0).numpy()) <= tol
+    assert rel_err(dwt.numpy(), ctx.conv2d_wgrad(dx_al, dg_al, w.shape, (1, 1), (1, 1), 0).numpy()) <= tol
+    del xb, gb
 
 
 def test_conv2d_reference_vectors(ctx, golden):
