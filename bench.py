@@ -9,7 +9,7 @@ algorithmic 2*Cout*(Cin*kh*kw)*(B*oh*ow) FLOP per pass, with all tensors residen
 Also measured in the same run and reported under "also": the bandwidth kernels of config C4 (sum/mean/max over
 axis 0, axis 1 and all elements of [8192,8192] f32 and f64; add/mul and ReLU/sigmoid/tanh backward on 2^28 f32).
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--skip-also]
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--skip-also] [--skip-train]
 """
 import argparse
 import json
@@ -42,6 +42,12 @@ def time_stream(ctx, fn, iters, warmup):
 
 CONV_KERNELS = {"fwd": "cpk::conv_patch_kernel (conv fwd pass)", "dgrad": "cpk::conv_patch_kernel (conv dgrad pass)",
                 "wgrad": "wgp::wgrad_patch_kernel + wgrad_patch_reduce_kernel (conv wgrad pass)"}
+
+
+# HBM-side bytes per launch of the main kernel of each C3 pass: rocprofv3 FETCH_SIZE + WRITE_SIZE per dispatch,
+# scaled by what the same counters read for the streaming add kernel of known size (x2.000 and x1.000); the
+# summary with the commands is profiles/conv_c3_f32_hbm_traffic.txt.
+CONV_C3_TRAFFIC_BYTES = {"fwd": 446.3e6, "dgrad": 684.4e6, "wgrad": 964.9e6}
 
 
 def bench_conv(ctx, steps, warmup, dtype=np.float32, B=None):
@@ -249,6 +255,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-also", action="store_true")
+    ap.add_argument("--skip-train", action="store_true", help="leave the train-step section out of `also` (short profiler runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the hot path has no cross-GPU exchange built); use --gpus 1")
@@ -275,7 +282,8 @@ def main():
                    "flop_per_step": 3 * conv["flop_per_pass"], "device": ctx.device_name()},
         "roofline": {"bound": "mfma", "kernel": CONV_KERNELS[dominant], "achieved": dom["tflops"],
                      "peak": PEAK_F32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": dom["tflops"] / PEAK_F32_MFMA_TFLOPS,
-                     "traffic": None, "avg_launch_ms": dom["ms"]},
+                     "traffic": CONV_C3_TRAFFIC_BYTES[dominant], "traffic_unit": "bytes per launch",
+                     "algorithmic_bytes": 308.6e6, "avg_launch_ms": dom["ms"]},
         "conv_passes": {k: {"ms": v["ms"], "tflops": v["tflops"], "frac_mfma_f32": v["tflops"] / PEAK_F32_MFMA_TFLOPS}
                         for k, v in conv["per_pass"].items()},
     }
@@ -287,7 +295,7 @@ def main():
         }
         result["also"].update(bench_bandwidth(ctx))
     ctx.close()
-    if not args.skip_also:
+    if not args.skip_also and not args.skip_train:
         result["also"]["train_step"] = bench_train_steps(cpu=not args.skip_cpu)
         result["also"]["train_step_reference_pool_config"] = bench_train_steps(cpu=False, reference_pool=True)
     if not args.skip_cpu:
