@@ -273,6 +273,81 @@ __global__ __launch_bounds__(256) void materialize_kernel(const T* __restrict__ 
     out[i] = in[off];
 }
 
+// Collapsed view of at most 4 dims whose innermost dim is contiguous (stride 1) or broadcast (stride 0) with an
+// extent that is a multiple of the 16-byte vector: 32-bit index arithmetic with multiply-shift division.
+struct U32Div {
+    uint32_t d, m, s;
+    __device__ __forceinline__ uint32_t div(uint32_t n) const { return (uint32_t)(((uint64_t)__umulhi(n, m) + n) >> s); }
+};
+static U32Div make_u32div(uint32_t d) {
+    U32Div r;
+    r.d = d;
+    r.s = 0;
+    while ((1ull << r.s) < d) ++r.s;
+    r.m = (uint32_t)((((1ull << 32) * ((1ull << r.s) - d)) / d) + 1);
+    return r;
+}
+struct FastView {
+    U32Div inner4;      // vectors along the innermost dim
+    int inner_stride;   // 0 or 1
+    U32Div ext[3];      // outer dims, innermost of them first (extent 1 when absent)
+    i64 stride[3];
+};
+
+struct CollapsedView {
+    int nd;
+    U32Div ext[8];  // innermost first
+    i64 stride[8];
+};
+
+// Any collapsed view below 2^31 elements, one element per thread.
+template <typename T>
+__global__ __launch_bounds__(256) void materialize_u32_kernel(const T* __restrict__ in, T* __restrict__ out, CollapsedView v, i64 n) {
+    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    uint32_t r = (uint32_t)i;
+    i64 off = 0;
+#pragma unroll
+    for (int d = 0; d < 8; ++d) {
+        if (d < v.nd) {
+            const uint32_t q = v.ext[d].div(r);
+            off += (i64)(r - q * v.ext[d].d) * v.stride[d];
+            r = q;
+        }
+    }
+    out[i] = in[off];
+}
+
+template <typename T, bool SRC_VEC>
+__global__ __launch_bounds__(256) void materialize_vec_kernel(const T* __restrict__ in, T* __restrict__ out, FastView v, i64 nv) {
+    constexpr int V = 16 / (int)sizeof(T);
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= nv) return;
+    uint32_t r = (uint32_t)i;
+    uint32_t q = v.inner4.div(r);
+    i64 off = (i64)(r - q * v.inner4.d) * V * v.inner_stride;
+    r = q;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+        q = v.ext[d].div(r);
+        off += (i64)(r - q * v.ext[d].d) * v.stride[d];
+        r = q;
+    }
+    vec_t o;
+    if (SRC_VEC) {
+        o = *reinterpret_cast<const vec_t*>(in + off);
+    } else if (v.inner_stride == 0) {
+        const T x = in[off];
+#pragma unroll
+        for (int u = 0; u < V; ++u) o[u] = x;
+    } else {
+#pragma unroll
+        for (int u = 0; u < V; ++u) o[u] = in[off + u];
+    }
+    *reinterpret_cast<vec_t*>(out + i * V) = o;
+}
+
 template <typename T>
 int materialize(fx_ctx* c, const T* in, T* out, const i64* shape, const i64* strides, int ndim, i64 n) {
     FX_CHECK_CTX(c);
@@ -290,8 +365,53 @@ int materialize(fx_ctx* c, const T* in, T* out, const i64* shape, const i64* str
         prod *= shape[d];
     }
     FX_REQUIRE(prod == n, "fx_materialize: shape product %lld != n %lld", (long long)prod, (long long)n);
+    // Collapse the view: drop extent-1 dims, merge neighbours that walk memory as one dim (or are both broadcast).
+    i64 cs[8], ct[8];
+    int nd = 0;
+    for (int d = 0; d < ndim; ++d) {
+        if (shape[d] == 1) continue;
+        if (nd > 0 && ct[nd - 1] == strides[d] * shape[d]) {
+            cs[nd - 1] *= shape[d];
+            ct[nd - 1] = strides[d];
+        } else {
+            cs[nd] = shape[d];
+            ct[nd] = strides[d];
+            ++nd;
+        }
+    }
+    constexpr int V = 16 / (int)sizeof(T);
+    if (nd >= 1 && nd <= 4 && n < (1ll << 31) && cs[nd - 1] % V == 0 && (ct[nd - 1] == 0 || ct[nd - 1] == 1) &&
+        ((uintptr_t)out & 15) == 0) {
+        // vector path: one thread writes V consecutive outputs of the innermost collapsed dim
+        bool src_vec = ct[nd - 1] == 1 && ((uintptr_t)in & 15) == 0;
+        FastView fv{};
+        fv.inner4 = make_u32div((uint32_t)(cs[nd - 1] / V));
+        fv.inner_stride = (int)ct[nd - 1];
+        for (int d = 0; d < 3; ++d) {
+            const int src = nd - 2 - d;  // outer dims, innermost of them first
+            fv.ext[d] = make_u32div((uint32_t)(src >= 0 ? cs[src] : 1));
+            fv.stride[d] = src >= 0 ? ct[src] : 0;
+            if (src >= 0 && ct[src] % V != 0) src_vec = false;
+        }
+        const i64 nv = n / V, blocks = fx::ceil_div(nv, 256);
+        if (src_vec) materialize_vec_kernel<T, true><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(in, out, fv, nv);
+        else materialize_vec_kernel<T, false><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(in, out, fv, nv);
+        FX_LAUNCH_CHECK();
+        return FX_OK;
+    }
     const i64 blocks = fx::ceil_div(n, 256);
     FX_REQUIRE(blocks <= 0x7fffffff, "fx_materialize: too many elements");
+    if (n < (1ll << 31)) {
+        CollapsedView cv{};
+        cv.nd = nd;
+        for (int d = 0; d < nd; ++d) {
+            cv.ext[d] = make_u32div((uint32_t)cs[nd - 1 - d]);
+            cv.stride[d] = ct[nd - 1 - d];
+        }
+        materialize_u32_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(in, out, cv, n);
+        FX_LAUNCH_CHECK();
+        return FX_OK;
+    }
     materialize_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(in, out, v, n);
     FX_LAUNCH_CHECK();
     return FX_OK;

@@ -543,9 +543,45 @@ int launch(fx_ctx* c, const AL& al, const BL& bl, const EP& ep, i64 M, i64 N, i6
     return FX_OK;
 }
 
+// Same sum for few outputs and many splits: G threads share one output, thread g adds splits g, g+G, ... in
+// order, then the G partial sums are added in order of g.  The grouping depends only on (n, splits), so the
+// result is reproducible run to run; it differs from the single-chain order by rounding only.
+template <typename T, int G>
+__global__ __launch_bounds__(256) void splitk_reduce_grouped_kernel(const T* __restrict__ part, T* __restrict__ out, i64 n, int splits) {
+    constexpr int COLS = 256 / G;
+    __shared__ T sm[G][COLS];
+    const int col = threadIdx.x % COLS, g = threadIdx.x / COLS;
+    const i64 i = (i64)blockIdx.x * COLS + col;
+    T s = T(0);
+    if (i < n) {
+        int z = g;
+        for (; z + 7 * G < splits; z += 8 * G) {
+            T v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = part[(i64)(z + u * G) * n + i];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s = s + v[u];
+        }
+        for (; z < splits; z += G) s = s + part[(i64)z * n + i];
+    }
+    sm[g][col] = s;
+    __syncthreads();
+    if (g == 0 && i < n) {
+        T t = sm[0][col];
+#pragma unroll
+        for (int u = 1; u < G; ++u) t = t + sm[u][col];
+        out[i] = t;
+    }
+}
+
 template <typename T>
 int launch_splitk_reduce(fx_ctx* c, const T* part, T* out, i64 n, int splits) {
-    splitk_reduce_kernel<T><<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(part, out, n, splits);
+    if (splits >= 128 && n <= (1 << 16))
+        splitk_reduce_grouped_kernel<T, 16><<<dim3((unsigned)fx::ceil_div(n, 16)), dim3(256), 0, c->stream>>>(part, out, n, splits);
+    else if (splits >= 32 && n <= (1 << 18))
+        splitk_reduce_grouped_kernel<T, 4><<<dim3((unsigned)fx::ceil_div(n, 64)), dim3(256), 0, c->stream>>>(part, out, n, splits);
+    else
+        splitk_reduce_kernel<T><<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(part, out, n, splits);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

@@ -134,6 +134,38 @@ def test_fill_and_materialize(ctx, orc, dtype):
     assert np.array_equal(got, m.T)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_materialize_views_bit_exact(ctx, dtype):
+    """Broadcasts, permutations, slices-with-step and 5..8-dim views against numpy's as_strided (element strides):
+    covers the vector kernel (contiguous or broadcast inner dim, aligned and misaligned source), the 32-bit
+    one-element kernel and the collapse of mergeable dims."""
+    from numpy.lib.stride_tricks import as_strided
+    rng = np.random.default_rng(15)
+    base = rng.standard_normal(40000).astype(dtype)
+    dbase = ctx.upload(base)
+    item = base.itemsize
+    views = [
+        ((256, 32, 8, 8), (0, 1, 0, 0)),          # bias broadcast, inner dims merge to one broadcast dim
+        ((64, 128), (0, 1)), ((128, 64), (1, 0)),  # row / column broadcast
+        ((100, 64), (1, 100)), ((37, 53), (53, 1)), ((53, 37), (1, 53)),  # transposes and identity
+        ((6, 5, 4, 8), (160, 8, 40, 1)),           # permute with contiguous inner dim
+        ((3, 4, 5, 6), (1, 3, 12, 60)),            # full reversal of a [6,5,4,3] tensor
+        ((7, 12), (24, 2)), ((5, 9, 4), (0, 4, 1)), ((2, 3, 1, 4, 1, 5), (60, 20, 0, 5, 0, 1)),
+        ((2, 2, 2, 2, 2, 2, 2, 4), (512, 1024, 64, 128, 16, 32, 4, 1)), ((1,), (0,)), ((9,), (3,)), ((16,), (0,)),
+    ]
+    for shape, strides in views:
+        want = np.ascontiguousarray(as_strided(base, shape, tuple(s_ * item for s_ in strides)))
+        got = ctx.materialize(dbase, shape, strides).numpy()
+        assert np.array_equal(got, want), (shape, strides)
+    # a source that is only element-aligned (view starting one element into the buffer)
+    from ferrox_amd import capi
+    shape, strides = (32, 64), (64, 1)
+    out = ctx.empty(shape, dtype)
+    sh, st = (capi._i64 * 2)(*shape), (capi._i64 * 2)(*strides)
+    capi.check(ctx._fn("materialize", np.dtype(dtype))(ctx.h, dbase.ptr + item, out.ptr, sh, st, 2, 32 * 64))
+    assert np.array_equal(out.numpy(), base[1:1 + 2048].reshape(shape))
+
+
 # ------------------------------------------------------------------------------------------ im2col / col2im
 GEOMS = [  # B, C, H, W, k, s, p
     (1, 1, 5, 5, 3, 1, 1), (2, 3, 8, 7, 3, 1, 1), (3, 2, 9, 9, 3, 2, 1), (2, 2, 6, 6, 2, 2, 0), (2, 3, 7, 5, 1, 1, 0),
