@@ -169,6 +169,67 @@ int dgrad_tile(fx_ctx* c, const T* g, const T* wt, T* dx, const Dims& d) {
     return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
 }
 
+// Data gradient for at most 4 input channels (the first layer of an image network): the implicit GEMM would pad
+// Cin = 3 to a 32-row tile and run at 10 % useful work.  One thread owns one input pixel and all its channels and
+// gathers over (tap, oc); the filters sit in LDS as wl[tap][oc][4] so one 16-byte broadcast read feeds the channel
+// FMAs, and lanes walk consecutive x, so every grad_out load is a contiguous 256-byte row segment.
+template <typename T>
+__global__ __launch_bounds__(256) void dgrad_small_cin_kernel(const T* __restrict__ g, const T* __restrict__ w, T* __restrict__ dx,
+                                                              ConvShape s, int npix) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* wl = reinterpret_cast<T*>(smem_raw);
+    const int KK = s.kh * s.kw;
+    for (int i = threadIdx.x; i < KK * s.Cout * 4; i += 256) {
+        const int c = i & 3, oc = (i >> 2) % s.Cout, t = (i >> 2) / s.Cout;
+        wl[i] = c < s.Cin ? w[((i64)oc * s.Cin + c) * KK + t] : T(0);
+    }
+    __syncthreads();
+    const int n = blockIdx.x * 256 + threadIdx.x;
+    if (n >= npix) return;
+    const uint32_t b = s.div_HW.div((uint32_t)n), rem = n - b * (s.H * s.W);
+    const uint32_t y = s.div_W.div(rem), x = rem - y * s.W;
+    const int L = s.oh * s.ow;
+    const T* gb = g + (i64)b * s.Cout * L;
+    T acc[4] = {T(0), T(0), T(0), T(0)};
+    for (int ky = 0; ky < s.kh; ++ky) {
+        const int ty = (int)y + s.ph - ky;
+        if (ty < 0) continue;
+        const uint32_t oy = s.div_sh.div((uint32_t)ty);
+        if ((int)(oy * s.sh) != ty || (int)oy >= s.oh) continue;
+        for (int kx = 0; kx < s.kw; ++kx) {
+            const int tx = (int)x + s.pw - kx;
+            if (tx < 0) continue;
+            const uint32_t ox = s.div_sw.div((uint32_t)tx);
+            if ((int)(ox * s.sw) != tx || (int)ox >= s.ow) continue;
+            const T* gp = gb + oy * s.ow + ox;
+            const T* wt = wl + (ky * s.kw + kx) * s.Cout * 4;
+#pragma unroll 4
+            for (int oc = 0; oc < s.Cout; ++oc) {
+                const T gv = gp[(i64)oc * L];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) acc[c] += gv * wt[oc * 4 + c];
+            }
+        }
+    }
+    T* o = dx + (i64)b * s.Cin * s.H * s.W + rem;
+    for (int c = 0; c < s.Cin; ++c) o[(i64)c * s.H * s.W] = acc[c];
+}
+
+template <typename T>
+bool dgrad_small_cin_ok(const Dims& d) {
+    return d.Cin <= 4 && d.kh * d.kw * d.Cout * 4 * (i64)sizeof(T) <= 48 * 1024 && !generic_only();
+}
+
+template <typename T>
+int dgrad_small_cin(fx_ctx* c, const T* g, const T* w, T* dx, const Dims& d) {
+    const ConvShape s = make_shape(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
+    const i64 npix = d.B * d.H * d.W;
+    const size_t smem = (size_t)(d.kh * d.kw * d.Cout * 4) * sizeof(T);
+    dgrad_small_cin_kernel<T><<<dim3((unsigned)fx::ceil_div(npix, 256)), dim3(256), smem, c->stream>>>(g, w, dx, s, (int)npix);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
 template <typename T>
 i64 dgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     if (mode == 1) return d.Cin * d.kh * d.kw * d.B * d.oh * d.ow * (i64)sizeof(T);
@@ -205,6 +266,7 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
         }
         return rc;
     }
+    if (dgrad_small_cin_ok<T>(d)) return dgrad_small_cin<T>(c, g, w, dx, d);
     std::lock_guard<std::mutex> lk(c->launch_mutex);
     T* wt = (T*)(ws ? ws : c->get_scratch(need));
     if (!wt) return FX_ERR_OOM;
