@@ -131,6 +131,19 @@ def bench_bandwidth(ctx, iters=20, warmup=3):
         ms = time_stream(ctx, fn, 10, 2)
         nbytes = 3 * 4 * n
         out["elementwise"][f"{name}_f32"] = {"ms": ms, "GBps": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    # the same gradients composed op by op as the reference's operators do (ops/unary.rs:254-375): more array passes
+    # over HBM for the same algorithmic 3 arrays; GB/s below is still algorithmic bytes / time
+    t1, t2 = ctx.empty((n,)), ctx.empty((n,))
+    composed = {
+        "relu_bwd": lambda: (ctx.scalar("greater_scalar", x, 0.0, out=t1), ctx.binary("mul", g, t1, out=o)),
+        "sigmoid_bwd": lambda: (ctx.scalar("sub_scalar", s, 1.0, out=t1), ctx.binary("mul", s, t1, out=t2), ctx.binary("mul", g, t2, out=o)),
+        "tanh_bwd": lambda: (ctx.binary("mul", t, t, out=t1), ctx.scalar("sub_scalar", t1, 1.0, out=t2), ctx.unary("neg", t2, out=t1),
+                             ctx.binary("mul", g, t1, out=o)),
+    }
+    for name, fn in composed.items():
+        ms = time_stream(ctx, fn, 5, 1)
+        nbytes = 3 * 4 * n
+        out["elementwise"][f"{name}_composed_f32"] = {"ms": ms, "GBps_algorithmic": nbytes / ms / 1e6}
     return out
 
 
@@ -231,10 +244,36 @@ def cpu_baseline_conv(batch=32, reps=4):
         orc.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), 0)
         orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 0)
     dt = (time.perf_counter() - t0) / reps
-    return {"value": flop / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
-            "sample": f"same layer at batch {B} of 128 (fwd+dgrad+wgrad, {reps} rep(s), {dt:.2f} s per rep), f32, "
-                      f"im2col + blocked single-thread GEMM + col2im as in the reference CPU backend",
-            "host_cpu": _cpu_model()}
+    out = {"value": flop / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+           "sample": f"same layer at batch {B} of 128 (fwd+dgrad+wgrad, {reps} rep(s), {dt:.2f} s per rep), f32, "
+                     f"im2col + blocked single-thread GEMM + col2im as in the reference CPU backend",
+           "host_cpu": _cpu_model()}
+    out["torch_cpu_comparator"] = _torch_cpu_conv(x, w, g, s, p, flop)
+    return out
+
+
+def _torch_cpu_conv(x, w, g, s, p, flop):
+    """A tuned CPU library on the same slice (fwd + autograd backward), 1 thread and all threads: an upper-bound
+    comparator for the CPU column, not the reference's algorithm."""
+    import torch
+    import torch.nn.functional as F
+    res = {}
+    keep = torch.get_num_threads()
+    for label, nt in (("1_thread", 1), ("all_threads", keep)):
+        torch.set_num_threads(nt)
+        tx = torch.from_numpy(x).requires_grad_(True)
+        tw = torch.from_numpy(w).requires_grad_(True)
+        tg = torch.from_numpy(g)
+        best = None
+        for _ in range(2):
+            t0 = time.perf_counter()
+            F.conv2d(tx, tw, stride=s, padding=p).backward(tg)
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+            tx.grad = tw.grad = None
+        res[label] = {"threads": nt, "tflops": flop / best / 1e12, "s_per_rep": best}
+    torch.set_num_threads(keep)
+    return res
 
 
 def _cpu_model():
