@@ -118,6 +118,12 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_conv2d_fwd_{_s}", _vp, _vp, _vp, _vp, *_CONV_INTS, _vp, _i64)
     _sig(f"fx_conv2d_dgrad_{_s}", _vp, _vp, _vp, _vp, *_CONV_INTS, _int, _vp, _i64)
     _sig(f"fx_conv2d_wgrad_{_s}", _vp, _vp, _vp, _vp, *_CONV_INTS, _int, _vp, _i64)
+    _sig(f"fx_bias_act_{_s}", _vp, _vp, _vp, _i64, _i64, _i64, _int)
+    _sig(f"fx_bias_grad_{_s}", _vp, _vp, _vp, _i64, _i64, _i64)
+    _sig(f"fx_softmax_ce_fwd_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64)
+    _sig(f"fx_softmax_ce_bwd_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64)
+    _sig(f"fx_adam_step_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, *([_ct] * 7))
+    _sig(f"fx_sgd_step_{_s}", _vp, _vp, _vp, _i64, _ct)
 
 
 class FerroxHipError(RuntimeError):
@@ -386,6 +392,35 @@ class Context:
         check(self._fn("conv2d_dgrad", g.dtype)(self.h, g.ptr, w.ptr, dx.ptr, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, mode,
                                                 None, 0))
         return dx
+
+    # ---- fused sequences
+    def bias_act(self, y, bias, outer, C, inner, act=0):
+        """In place: y[o, c, i] += bias[c], then ReLU when act == 1."""
+        check(self._fn("bias_act", y.dtype)(self.h, y.ptr, bias.ptr, outer, C, inner, act))
+        return y
+
+    def bias_grad(self, g, outer, C, inner):
+        o = self.empty((C,), g.dtype)
+        check(self._fn("bias_grad", g.dtype)(self.h, g.ptr, o.ptr, outer, C, inner))
+        return o
+
+    def softmax_ce_fwd(self, logits, targets):
+        B, Cc = logits.shape
+        probs, loss = self.empty((B, Cc), logits.dtype), self.empty((1,), logits.dtype)
+        check(self._fn("softmax_ce_fwd", logits.dtype)(self.h, logits.ptr, targets.ptr, probs.ptr, loss.ptr, B, Cc))
+        return probs, loss
+
+    def softmax_ce_bwd(self, probs, targets, grad_loss):
+        B, Cc = probs.shape
+        d = self.empty((B, Cc), probs.dtype)
+        check(self._fn("softmax_ce_bwd", probs.dtype)(self.h, probs.ptr, targets.ptr, grad_loss.ptr, d.ptr, B, Cc))
+        return d
+
+    def adam_step(self, p, g, m, v, lr, beta1, beta2, eps, wd, bc1, bc2):
+        check(self._fn("adam_step", p.dtype)(self.h, p.ptr, g.ptr, m.ptr, v.ptr, p.size, lr, beta1, beta2, eps, wd, bc1, bc2))
+
+    def sgd_step(self, p, g, lr):
+        check(self._fn("sgd_step", p.dtype)(self.h, p.ptr, g.ptr, p.size, lr))
 
     def conv2d_wgrad(self, x, g, w_shape, stride, padding, mode=0, out=None):
         B, Cin, H, W = x.shape

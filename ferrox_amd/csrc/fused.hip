@@ -1,0 +1,307 @@
+// Fused entry points for sequences that the reference composes from many small operators; each keeps the
+// composed path's arithmetic (same operations in the same order per element; this file is built without a*b+c
+// contraction) so that results equal the composed path bit for bit wherever no reduction order is involved.
+//   bias_act      y += bias[c] (then ReLU)      replaces Reshape + BroadcastTo + Add (+ ReLU): nn/layers/utils.rs:6-42,
+//                                               conv2d.rs:203-213, linear.rs:262-279, ops/unary.rs:340-356
+//   bias_grad     db[c] = sum_{o,i} g[o,c,i]    replaces reduce_gradient_for_broadcasting (ops/basic.rs:10-53)
+//   softmax_ce    loss and d loss / d logits    replaces the 7 forward / 7 backward ops of CCELoss
+//                                               (nn/losses/classification.rs:191-257, ops/batched.rs:106-131)
+//   adam_step     in-place Adam update          replaces ~14 kernels per parameter (nn/optim/adam.rs:288-358)
+//   sgd_step      in-place p -= lr*g            replaces nn/optim/sgd.rs:210-245 (momentum 0, weight decay 0)
+#include "common.hpp"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ T dev_exp(T x);
+template <> __device__ __forceinline__ float dev_exp<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ double dev_exp<double>(double x) { return exp(x); }
+template <typename T> __device__ __forceinline__ T dev_log(T x);
+template <> __device__ __forceinline__ float dev_log<float>(float x) { return logf(x); }
+template <> __device__ __forceinline__ double dev_log<double>(double x) { return log(x); }
+template <typename T> __device__ __forceinline__ T dev_sqrt(T x);
+template <> __device__ __forceinline__ float dev_sqrt<float>(float x) { return sqrtf(x); }
+template <> __device__ __forceinline__ double dev_sqrt<double>(double x) { return sqrt(x); }
+template <typename T> __device__ __forceinline__ T lowest();
+template <> __device__ __forceinline__ float lowest<float>() { return -3.402823466e+38f; }
+template <> __device__ __forceinline__ double lowest<double>() { return -1.7976931348623157e+308; }
+
+// ---- bias add (+ ReLU), in place: y viewed as [outer, C, inner] ---------------------------------------------------
+// VEC: inner is a multiple of the 16-byte vector and y is 16-byte aligned, so one thread owns one vector (one channel).
+template <typename T, bool VEC, bool RELU>
+__global__ __launch_bounds__(256) void bias_act_kernel(T* __restrict__ y, const T* __restrict__ bias, i64 n, uint32_t C, uint32_t inner) {
+    constexpr int V = VEC ? 16 / (int)sizeof(T) : 1;
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    const i64 i = ((i64)blockIdx.x * 256 + threadIdx.x) * V;
+    if (i >= n) return;
+    const T b = bias[(i / inner) % C];
+    vec_t v = *reinterpret_cast<vec_t*>(y + i);
+#pragma unroll
+    for (int u = 0; u < V; ++u) {
+        T r = v[u] + b;
+        if (RELU) r = r > T(0) ? r : T(0);  // ReLU as in the forward kernel: x > 0 ? x : 0
+        v[u] = r;
+    }
+    *reinterpret_cast<vec_t*>(y + i) = v;
+}
+
+template <typename T>
+int bias_act(fx_ctx* c, T* y, const T* bias, i64 outer, i64 C, i64 inner, int act) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(outer >= 0 && C >= 1 && inner >= 1, "fx_bias_act: bad view");
+    FX_REQUIRE(act == 0 || act == 1, "fx_bias_act: act must be 0 (none) or 1 (relu)");
+    const i64 n = outer * C * inner;
+    if (n == 0) return FX_OK;
+    FX_REQUIRE(y && bias, "fx_bias_act: null pointer");
+    FX_REQUIRE(C < (1ll << 31) && inner < (1ll << 31), "fx_bias_act: view too large");
+    constexpr int V = 16 / (int)sizeof(T);
+    const bool vec = inner % V == 0 && ((uintptr_t)y & 15) == 0;
+    const i64 threads = vec ? n / V : n, blocks = fx::ceil_div(threads, 256);
+    FX_REQUIRE(blocks <= 0x7fffffff, "fx_bias_act: too many elements");
+    const dim3 grid((unsigned)blocks), blk(256);
+    if (vec) {
+        if (act) bias_act_kernel<T, true, true><<<grid, blk, 0, c->stream>>>(y, bias, n, (uint32_t)C, (uint32_t)inner);
+        else bias_act_kernel<T, true, false><<<grid, blk, 0, c->stream>>>(y, bias, n, (uint32_t)C, (uint32_t)inner);
+    } else {
+        if (act) bias_act_kernel<T, false, true><<<grid, blk, 0, c->stream>>>(y, bias, n, (uint32_t)C, (uint32_t)inner);
+        else bias_act_kernel<T, false, false><<<grid, blk, 0, c->stream>>>(y, bias, n, (uint32_t)C, (uint32_t)inner);
+    }
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+// ---- bias gradient: out[c] = sum over (o, i) of g[o, c, i] --------------------------------------------------------
+// Stage 1: block (c, slice) sums rows o of its slice, each thread running over i and o in a fixed pattern, then a
+// fixed-order tree; stage 2 adds the slice partials in slice order.  Deterministic for a given (outer, C, inner).
+template <typename T>
+__global__ __launch_bounds__(256) void bias_grad_partial_kernel(const T* __restrict__ g, T* __restrict__ part, i64 outer, i64 C,
+                                                                i64 inner, i64 rows_per_slice) {
+    __shared__ T sm[256];
+    const i64 c = blockIdx.x, slice = blockIdx.y;
+    const i64 o0 = slice * rows_per_slice, o1 = min(outer, o0 + rows_per_slice);
+    T s = T(0);
+    if (inner >= 64) {  // threads run along i (contiguous), rows one after the other
+        for (i64 o = o0; o < o1; ++o) {
+            const T* p = g + (o * C + c) * inner;
+            for (i64 i = threadIdx.x; i < inner; i += 256) s = s + p[i];
+        }
+    } else {  // short rows: threads run over (o, i) pairs
+        const i64 total = (o1 - o0) * inner;
+        for (i64 t = threadIdx.x; t < total; t += 256) {
+            const i64 o = o0 + t / inner, i = t % inner;
+            s = s + g[(o * C + c) * inner + i];
+        }
+    }
+    sm[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) sm[threadIdx.x] = sm[threadIdx.x] + sm[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) part[slice * C + c] = sm[0];
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bias_grad_final_kernel(const T* __restrict__ part, T* __restrict__ out, i64 C, int slices) {
+    const i64 c = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    T s = T(0);
+    for (int z = 0; z < slices; ++z) s = s + part[(i64)z * C + c];
+    out[c] = s;
+}
+
+template <typename T>
+int bias_grad(fx_ctx* c, const T* g, T* out, i64 outer, i64 C, i64 inner) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(outer >= 1 && C >= 1 && inner >= 1, "fx_bias_grad: bad view");
+    FX_REQUIRE(g && out, "fx_bias_grad: null pointer");
+    FX_REQUIRE(C <= 0x7fffffff, "fx_bias_grad: too many channels");
+    // enough blocks to fill the chip, at least 8 rows (or 16k elements) per block
+    i64 slices = std::max<i64>(1, std::min<i64>((i64)c->num_cus * 4 / C, 65535));
+    const i64 min_rows = std::max<i64>(1, 16384 / inner);
+    slices = std::max<i64>(1, std::min<i64>(slices, outer / min_rows));
+    const i64 rps = fx::ceil_div(outer, slices);
+    slices = fx::ceil_div(outer, rps);
+    std::lock_guard<std::mutex> lk(c->launch_mutex);
+    T* part = out;
+    if (slices > 1) {
+        part = (T*)c->get_scratch(slices * C * (i64)sizeof(T));
+        if (!part) return FX_ERR_OOM;
+    }
+    bias_grad_partial_kernel<T><<<dim3((unsigned)C, (unsigned)slices), dim3(256), 0, c->stream>>>(g, part, outer, C, inner, rps);
+    FX_LAUNCH_CHECK();
+    if (slices > 1) {
+        bias_grad_final_kernel<T><<<dim3((unsigned)fx::ceil_div(C, (i64)256)), dim3(256), 0, c->stream>>>(part, out, C, (int)slices);
+        FX_LAUNCH_CHECK();
+    }
+    return FX_OK;
+}
+
+// ---- softmax cross-entropy with mean reduction -------------------------------------------------------------------
+// forward, one thread per row, classes walked in order (as softmax_batched and the row sum do):
+//   s = exp(x - max) / sum;  p = clamp(s, 1e-8, 1 - 1e-8);  row = -(sum_c y*log(p));  loss = (sum_b row) * (1/B)
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_ce_rows_kernel(const T* __restrict__ x, const T* __restrict__ y, T* __restrict__ probs,
+                                                              T* __restrict__ rowloss, i64 B, i64 C, T lo, T hi) {
+    const i64 b = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (b >= B) return;
+    const T* xr = x + b * C;
+    const T* yr = y + b * C;
+    T* pr = probs + b * C;
+    T m = lowest<T>();
+    for (i64 k = 0; k < C; ++k) { const T v = xr[k]; if (v > m) m = v; }
+    T s = T(0);
+    for (i64 k = 0; k < C; ++k) { const T e = dev_exp<T>(xr[k] - m); pr[k] = e; s = s + e; }
+    T acc = T(0);
+    for (i64 k = 0; k < C; ++k) {
+        const T sm = pr[k] / s;
+        pr[k] = sm;
+        T p = sm;
+        if (p < lo) p = lo;
+        if (p > hi) p = hi;
+        acc = acc + yr[k] * dev_log<T>(p);
+    }
+    rowloss[b] = -acc;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void mean_rows_kernel(const T* __restrict__ rowloss, T* __restrict__ loss, i64 B, T inv) {
+    __shared__ T sm[256];
+    T s = T(0);
+    for (i64 i = threadIdx.x; i < B; i += 256) s = s + rowloss[i];
+    sm[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) sm[threadIdx.x] = sm[threadIdx.x] + sm[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) loss[0] = sm[0] * inv;
+}
+
+template <typename T>
+int softmax_ce_fwd(fx_ctx* c, const T* logits, const T* targets, T* probs, T* loss, i64 B, i64 C) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(B >= 1 && C >= 1, "fx_softmax_ce_fwd: bad shape");
+    FX_REQUIRE(logits && targets && probs && loss, "fx_softmax_ce_fwd: null pointer");
+    std::lock_guard<std::mutex> lk(c->launch_mutex);
+    T* rowloss = (T*)c->get_scratch(B * (i64)sizeof(T));
+    if (!rowloss) return FX_ERR_OOM;
+    softmax_ce_rows_kernel<T><<<dim3((unsigned)fx::ceil_div(B, (i64)256)), dim3(256), 0, c->stream>>>(
+        logits, targets, probs, rowloss, B, C, (T)1e-8, (T)(1.0 - 1e-8));
+    FX_LAUNCH_CHECK();
+    mean_rows_kernel<T><<<dim3(1), dim3(256), 0, c->stream>>>(rowloss, loss, B, (T)(1.0 / (double)B));
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+// backward: upstream g (one element on the device) -> d logits, the composed chain evaluated per row:
+//   d_tl = (-(g * (1/B)));  d_logp = d_tl * y;  d_p = d_logp / p;  d_s = d_p * (s >= lo) * (s <= hi);
+//   d_x = s * (d_s - sum_c(d_s * s))
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_ce_bwd_kernel(const T* __restrict__ probs, const T* __restrict__ y,
+                                                             const T* __restrict__ gup, T* __restrict__ dx, i64 B, i64 C, T inv, T lo, T hi) {
+    const i64 b = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (b >= B) return;
+    const T* sr = probs + b * C;
+    const T* yr = y + b * C;
+    T* dr = dx + b * C;
+    const T dtl = -(gup[0] * inv);
+    T dot = T(0);
+    for (i64 k = 0; k < C; ++k) {
+        const T s = sr[k];
+        T p = s;
+        if (p < lo) p = lo;
+        if (p > hi) p = hi;
+        const T dp = (dtl * yr[k]) / p;
+        const T ds = (dp * (s >= lo ? T(1) : T(0))) * (s <= hi ? T(1) : T(0));
+        dr[k] = ds;
+        dot = dot + ds * s;
+    }
+    for (i64 k = 0; k < C; ++k) dr[k] = sr[k] * (dr[k] - dot);
+}
+
+template <typename T>
+int softmax_ce_bwd(fx_ctx* c, const T* probs, const T* targets, const T* gup, T* dlogits, i64 B, i64 C) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(B >= 1 && C >= 1, "fx_softmax_ce_bwd: bad shape");
+    FX_REQUIRE(probs && targets && gup && dlogits, "fx_softmax_ce_bwd: null pointer");
+    softmax_ce_bwd_kernel<T><<<dim3((unsigned)fx::ceil_div(B, (i64)256)), dim3(256), 0, c->stream>>>(
+        probs, targets, gup, dlogits, B, C, (T)(1.0 / (double)B), (T)1e-8, (T)(1.0 - 1e-8));
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+// ---- optimizers, in place ----------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void adam_step_kernel(T* __restrict__ p, const T* __restrict__ g, T* __restrict__ m, T* __restrict__ v,
+                                                        i64 n, T lr, T beta1, T beta2, T eps, T wd, T bc1, T bc2) {
+    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const T gi = g[i], w = p[i];
+    const T m1 = m[i] * beta1 + gi * (T(1) - beta1);
+    const T m2 = v[i] * beta2 + (gi * gi) * (T(1) - beta2);
+    m[i] = m1;
+    v[i] = m2;
+    const T denom = dev_sqrt<T>(m2 / bc2) + eps;
+    const T update = ((m1 / bc1) / denom) * lr;
+    T nw = w - update;
+    if (wd != T(0)) nw = nw - w * (wd * lr);
+    p[i] = nw;
+}
+
+template <typename T>
+int adam_step(fx_ctx* c, T* p, const T* g, T* m, T* v, i64 n, T lr, T beta1, T beta2, T eps, T wd, T bc1, T bc2) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(n >= 0, "fx_adam_step: negative element count");
+    if (n == 0) return FX_OK;
+    FX_REQUIRE(p && g && m && v, "fx_adam_step: null pointer");
+    const i64 blocks = fx::ceil_div(n, (i64)256);
+    FX_REQUIRE(blocks <= 0x7fffffff, "fx_adam_step: too many elements");
+    adam_step_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(p, g, m, v, n, lr, beta1, beta2, eps, wd, bc1, bc2);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void sgd_step_kernel(T* __restrict__ p, const T* __restrict__ g, i64 n, T lr) {
+    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = p[i] - g[i] * lr;
+}
+
+template <typename T>
+int sgd_step(fx_ctx* c, T* p, const T* g, i64 n, T lr) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(n >= 0, "fx_sgd_step: negative element count");
+    if (n == 0) return FX_OK;
+    FX_REQUIRE(p && g, "fx_sgd_step: null pointer");
+    const i64 blocks = fx::ceil_div(n, (i64)256);
+    FX_REQUIRE(blocks <= 0x7fffffff, "fx_sgd_step: too many elements");
+    sgd_step_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(p, g, n, lr);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+}  // namespace
+
+#define FX_DEFINE_FUSED(T, S)                                                                                          \
+    extern "C" int fx_bias_act_##S(fx_ctx* c, T* y, const T* bias, int64_t outer, int64_t C, int64_t inner, int act) { \
+        return bias_act<T>(c, y, bias, outer, C, inner, act);                                                          \
+    }                                                                                                                  \
+    extern "C" int fx_bias_grad_##S(fx_ctx* c, const T* g, T* out, int64_t outer, int64_t C, int64_t inner) {          \
+        return bias_grad<T>(c, g, out, outer, C, inner);                                                               \
+    }                                                                                                                  \
+    extern "C" int fx_softmax_ce_fwd_##S(fx_ctx* c, const T* logits, const T* targets, T* probs, T* loss, int64_t B,   \
+                                         int64_t C) {                                                                  \
+        return softmax_ce_fwd<T>(c, logits, targets, probs, loss, B, C);                                               \
+    }                                                                                                                  \
+    extern "C" int fx_softmax_ce_bwd_##S(fx_ctx* c, const T* probs, const T* targets, const T* gup, T* dlogits,        \
+                                         int64_t B, int64_t C) {                                                       \
+        return softmax_ce_bwd<T>(c, probs, targets, gup, dlogits, B, C);                                               \
+    }                                                                                                                  \
+    extern "C" int fx_adam_step_##S(fx_ctx* c, T* p, const T* g, T* m, T* v, int64_t n, T lr, T beta1, T beta2, T eps, \
+                                    T wd, T bc1, T bc2) {                                                              \
+        return adam_step<T>(c, p, g, m, v, n, lr, beta1, beta2, eps, wd, bc1, bc2);                                    \
+    }                                                                                                                  \
+    extern "C" int fx_sgd_step_##S(fx_ctx* c, T* p, const T* g, int64_t n, T lr) { return sgd_step<T>(c, p, g, n, lr); }
+
+FX_DEFINE_FUSED(float, f32)
+FX_DEFINE_FUSED(double, f64)

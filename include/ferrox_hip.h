@@ -225,7 +225,30 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
                             int mode, void* workspace, int64_t ws_bytes);                                              \
     int fx_conv2d_wgrad_##S(fx_ctx* ctx, const T* x, const T* g, T* dw, int64_t B, int64_t Cin, int64_t H, int64_t W,  \
                             int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,      \
-                            int mode, void* workspace, int64_t ws_bytes);
+                            int mode, void* workspace, int64_t ws_bytes);                                              \
+    /* ---- fused sequences (optional: every one equals a chain of the entry points above) ----                        \
+       Bias add, in place, on y viewed as [outer, C, inner] (conv: outer = B, inner = oh*ow; linear: outer = B,        \
+       inner = 1), act 0 = none, 1 = ReLU.  Replaces Reshape + BroadcastTo + Add (+ ReLU) of                           \
+       src/nn/layers/utils.rs:6-42, conv2d.rs:203-213, linear.rs:262-279; same values bit for bit. */                  \
+    int fx_bias_act_##S(fx_ctx* ctx, T* y, const T* bias, int64_t outer, int64_t C, int64_t inner, int act);           \
+    /* Bias gradient out[c] = sum over (o, i) of g[o, c, i]: reduce_gradient_for_broadcasting,                         \
+       src/ops/basic.rs:10-53 (three axis sums for a conv bias) in one pass; fixed summation order per shape. */       \
+    int fx_bias_grad_##S(fx_ctx* ctx, const T* g, T* out, int64_t outer, int64_t C, int64_t inner);                    \
+    /* CCELoss with mean reduction, src/nn/losses/classification.rs:191-257: probs[B,C] = softmax(logits) (kept for    \
+       the backward), loss[1] = mean_b( -sum_c targets*log(clamp(probs, 1e-8, 1-1e-8)) ).  bwd: d logits from the      \
+       upstream gradient of the loss (1 element on the device) through Mean, Neg, Sum, Mul, Log, Clamp and the         \
+       softmax Jacobian (src/ops/batched.rs:106-131). */                                                               \
+    int fx_softmax_ce_fwd_##S(fx_ctx* ctx, const T* logits, const T* targets, T* probs, T* loss, int64_t B, int64_t C); \
+    int fx_softmax_ce_bwd_##S(fx_ctx* ctx, const T* probs, const T* targets, const T* grad_loss, T* dlogits, int64_t B, \
+                              int64_t C);                                                                              \
+    /* Adam::step for one parameter, in place on p, m, v (src/nn/optim/adam.rs:288-358, no amsgrad):                   \
+       m = m*b1 + g*(1-b1); v = v*b2 + (g*g)*(1-b2); p = p - ((m/bc1)/(sqrt(v/bc2)+eps))*lr [- p*(wd*lr)], with        \
+       bc1 = 1-max(b1^t,1e-8), bc2 = 1-max(b2^t,1e-8) computed by the caller (adam.rs:110-126).  Same operations in    \
+       the same order as the composed kernels: bit-identical results. */                                               \
+    int fx_adam_step_##S(fx_ctx* ctx, T* p, const T* g, T* m, T* v, int64_t n, T lr, T beta1, T beta2, T eps,          \
+                         T weight_decay, T bc1, T bc2);                                                                \
+    /* SGD::step without momentum or weight decay, src/nn/optim/sgd.rs:210-245: p = p - g*lr, in place. */             \
+    int fx_sgd_step_##S(fx_ctx* ctx, T* p, const T* g, int64_t n, T lr);
 
 FX_DECLARE_KERNELS(float, f32)
 FX_DECLARE_KERNELS(double, f64)

@@ -23,6 +23,64 @@ def _bcast(b, shape):
     return orc.materialize(b, shape, (0, 1))
 
 
+def softmax_ce_forward(pred, y):
+    """CCELoss forward (classification.rs:191-257): returns (loss as a 0-d array, softmax probabilities)."""
+    dt = pred.dtype.type
+    s = orc.softmax_axis(pred, 1)
+    c = orc.clamp(s, dt(1e-8), dt(1.0 - 1e-8))
+    lp = orc.unary("log", c)
+    tl = orc.binary("mul", y, lp)
+    ce = orc.reduce("sum", tl, [1], keep_dims=True)
+    neg = orc.unary("neg", ce)
+    return orc.reduce("mean", neg), s
+
+
+def softmax_ce_backward(s, y, g_loss):
+    """Gradient of the loss w.r.t. the logits from the upstream gradient of the (scalar) loss, op by op."""
+    dt = s.dtype.type
+    B = s.shape[0]
+    c = orc.clamp(s, dt(1e-8), dt(1.0 - 1e-8))
+    g = orc.scalar("mul_scalar", np.asarray(g_loss, s.dtype).reshape(1), dt(1.0 / B)).reshape(())   # Mean::gradient scale
+    g = np.full((B, 1), g.item(), s.dtype)                                            # expand_reduction(None) -> full
+    g = orc.unary("neg", g)                                                           # Neg
+    g = orc.materialize(g, s.shape, (1, 0))                                           # Sum(keep_dims): broadcast_to
+    g = orc.binary("mul", g, y)                                                       # Mul: grad wrt log-probs
+    g = orc.binary("div", g, c)                                                       # Log
+    m = orc.binary("mul", orc.scalar("greater_equal_scalar", s, dt(1e-8)),
+                   orc.scalar("less_equal_scalar", s, dt(1.0 - 1e-8)))
+    g = orc.binary("mul", g, m)                                                       # Clamp
+    prod = orc.binary("mul", g, s)                                                    # Softmax batch gradient
+    sp = orc.reduce("sum", prod, [1], keep_dims=True)
+    diff = orc.binary("sub", g, orc.materialize(sp, s.shape, (1, 0)))
+    return orc.binary("mul", s, diff)
+
+
+def bias_act(y, b, relu=False):
+    """Reshape + BroadcastTo + Add (+ ReLU) of a per-channel bias on [B,C] or [B,C,H,W] (utils.rs:6-42)."""
+    out = orc.binary("add", y, _bcast(b, y.shape))
+    return orc.unary("relu", out) if relu else out
+
+
+def bias_grad(g):
+    """reduce_gradient_for_broadcasting (ops/basic.rs:10-53): axes (3,2,0) for a conv bias, (0) for a linear one."""
+    return orc.reduce("sum", g, [3, 2, 0] if g.ndim == 4 else [0])
+
+
+def adam_update(w, g, m, v, lr, b1, b2, eps, wd, bc1, bc2):
+    """One Adam::step for one parameter (adam.rs:288-358); every scalar already in the tensor dtype."""
+    dt = w.dtype.type
+    m = orc.binary("add", orc.scalar("mul_scalar", m, b1), orc.scalar("mul_scalar", g, dt(1) - b1))
+    v = orc.binary("add", orc.scalar("mul_scalar", v, b2), orc.scalar("mul_scalar", orc.binary("mul", g, g), dt(1) - b2))
+    denom = orc.scalar("add_scalar", orc.unary("sqrt", orc.scalar("div_scalar", v, bc2)), eps)
+    upd = orc.scalar("mul_scalar", orc.binary("div", orc.scalar("div_scalar", m, bc1), denom), lr)
+    if wd != 0:
+        wdt = orc.scalar("mul_scalar", w, wd * lr)
+        w = orc.binary("sub", orc.binary("sub", w, upd), wdt)
+    else:
+        w = orc.binary("sub", w, upd)
+    return w, m, v
+
+
 class Sequential:
     def __init__(self, spec, params, dtype, conv_mode=0):
         self.dtype = np.dtype(dtype)
@@ -77,29 +135,8 @@ class Sequential:
         dt = self.dtype.type
         pred, tape = self.forward(x)
         y = np.ascontiguousarray(y, dtype=self.dtype)
-        # CCELoss forward
-        s = orc.softmax_axis(pred, 1)
-        c = orc.clamp(s, dt(1e-8), dt(1.0 - 1e-8))
-        lp = orc.unary("log", c)
-        tl = orc.binary("mul", y, lp)
-        ce = orc.reduce("sum", tl, [1], keep_dims=True)
-        neg = orc.unary("neg", ce)
-        loss = orc.reduce("mean", neg)
-        # backward, op by op
-        g = np.ones((), self.dtype)
-        g = orc.scalar("mul_scalar", g.reshape(1), dt(1.0 / neg.size)).reshape(())       # Mean::gradient scale
-        g = np.full(neg.shape, g.item(), self.dtype)                                      # expand_reduction(None) -> full
-        g = orc.unary("neg", g)                                                           # Neg
-        g = orc.materialize(g, tl.shape, (1, 0))                                          # Sum(keep_dims): broadcast_to
-        g = orc.binary("mul", g, y)                                                       # Mul: grad wrt log-probs
-        g = orc.binary("div", g, c)                                                       # Log
-        m = orc.binary("mul", orc.scalar("greater_equal_scalar", s, dt(1e-8)),
-                       orc.scalar("less_equal_scalar", s, dt(1.0 - 1e-8)))
-        g = orc.binary("mul", g, m)                                                       # Clamp
-        prod = orc.binary("mul", g, s)                                                    # Softmax batch gradient
-        sp = orc.reduce("sum", prod, [1], keep_dims=True)
-        diff = orc.binary("sub", g, orc.materialize(sp, s.shape, (1, 0)))
-        g = orc.binary("mul", s, diff)
+        loss, s = softmax_ce_forward(pred, y)
+        g = softmax_ce_backward(s, y, np.ones((), self.dtype))
         grads = [None] * len(self.params)
         for rec in reversed(tape):
             kind = rec[0]
@@ -150,15 +187,6 @@ class Adam:
             w = model.params[i]
             m = self.m.get(i, np.zeros_like(w))
             v = self.v.get(i, np.zeros_like(w))
-            m = orc.binary("add", orc.scalar("mul_scalar", m, b1), orc.scalar("mul_scalar", g, dt(1) - b1))
-            v = orc.binary("add", orc.scalar("mul_scalar", v, b2),
-                           orc.scalar("mul_scalar", orc.binary("mul", g, g), dt(1) - b2))
+            w, m, v = adam_update(w, g, m, v, dt(self.lr), b1, b2, dt(self.eps), dt(self.wd), bc1, bc2)
             self.m[i], self.v[i] = m, v
-            denom = orc.scalar("add_scalar", orc.unary("sqrt", orc.scalar("div_scalar", v, bc2)), dt(self.eps))
-            upd = orc.scalar("mul_scalar", orc.binary("div", orc.scalar("div_scalar", m, bc1), denom), dt(self.lr))
-            if self.wd != 0:
-                wdt = orc.scalar("mul_scalar", w, dt(self.wd) * dt(self.lr))
-                w = orc.binary("sub", orc.binary("sub", w, upd), wdt)
-            else:
-                w = orc.binary("sub", w, upd)
             model.params[i] = w

@@ -1,0 +1,117 @@
+"""Fused entry points (bias add + ReLU, bias gradient, softmax cross-entropy, Adam / SGD step) against the same
+sequences composed op by op from the CPU oracle's primitives.  Where no reduction is involved the fused kernel
+performs the composed path's operations in the same order, so the comparison is bit-exact."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [np.float32, np.float64]
+TOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float64): 1e-12}
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from ferrox_amd import capi
+    c = capi.Context(0)
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def train():
+    import oracle.train as t
+    return t
+
+
+def rel_err(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-300)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_bias_act_bit_exact(ctx, train, dtype):
+    rng = np.random.default_rng(70)
+    for shape in [(4, 10), (256, 10), (3, 7, 5, 6), (2, 32, 8, 8), (5, 3, 1, 9), (1, 1, 1, 1), (2, 5, 4, 4)]:
+        y = rng.standard_normal(shape).astype(dtype)
+        b = rng.standard_normal(shape[1]).astype(dtype)
+        inner = int(np.prod(shape[2:], dtype=np.int64))
+        for act in (0, 1):
+            got = ctx.bias_act(ctx.upload(y), ctx.upload(b), shape[0], shape[1], inner, act).numpy()
+            assert np.array_equal(got, train.bias_act(y, b, relu=bool(act))), (shape, act)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_bias_grad_vs_oracle_and_float64(ctx, train, dtype):
+    rng = np.random.default_rng(71)
+    tol = TOL[np.dtype(dtype)]
+    for shape in [(256, 10), (7, 3), (256, 32, 32, 32), (64, 64, 16, 16), (3, 5, 7, 9), (1, 4, 2, 2), (1000, 1, 3, 3)]:
+        g = rng.standard_normal(shape).astype(dtype)
+        inner = int(np.prod(shape[2:], dtype=np.int64))
+        got = ctx.bias_grad(ctx.upload(g), shape[0], shape[1], inner).numpy()
+        axes = (0,) if g.ndim == 2 else (0, 2, 3)
+        truth = g.astype(np.float64).sum(axis=axes)
+        scale = np.abs(g.astype(np.float64)).sum(axis=axes).max()
+        assert np.abs(got - truth).max() <= tol * scale, shape
+        assert np.abs(got - train.bias_grad(g)).max() <= 2 * tol * scale, shape
+        # same bits on a second run
+        assert np.array_equal(got, ctx.bias_grad(ctx.upload(g), shape[0], shape[1], inner).numpy())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_softmax_ce_fwd_bwd_vs_oracle(ctx, train, dtype):
+    import torch
+    rng = np.random.default_rng(72)
+    tol = TOL[np.dtype(dtype)]
+    for (B, C) in [(256, 10), (1, 1), (3, 2), (300, 17), (5, 1000)]:
+        x = (rng.standard_normal((B, C)) * 3).astype(dtype)
+        if B >= 3:
+            x[0, 0] = 60.0   # saturates: the other classes' probabilities fall under the 1e-8 clamp
+            x[1] = 0.0       # uniform row
+        y = np.eye(C, dtype=dtype)[rng.integers(0, C, B)]
+        if B >= 3:
+            y[0] = 0
+            y[0, C - 1] = 1  # target on a clamped class: the gradient must vanish there (f64) like the composed path
+        probs, loss = ctx.softmax_ce_fwd(ctx.upload(x), ctx.upload(y))
+        ol, os_ = train.softmax_ce_forward(x, y)
+        # same operations in the same order as the library's softmax kernel; exp differs from the CPU libm by rounding
+        assert np.array_equal(probs.numpy(), ctx.softmax_axis(ctx.upload(x), 1).numpy()), (B, C)
+        assert np.abs(probs.numpy() - os_).max() <= 4 * tol, (B, C)
+        assert abs(loss.numpy()[0] - ol.item()) <= 4 * tol * max(1.0, abs(ol.item())), (B, C)
+        gl = np.array([0.75], dtype)
+        d = ctx.softmax_ce_bwd(probs, ctx.upload(y), ctx.upload(gl)).numpy()
+        od = train.softmax_ce_backward(probs.numpy(), y, gl[0])
+        assert np.abs(d - od).max() <= 8 * tol * max(np.abs(od).max(), 1e-30), (B, C)
+        # textbook check where the clamp is inactive: torch log_softmax in float64
+        if C > 1 and B < 3:
+            tx = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
+            tl = -(torch.from_numpy(y.astype(np.float64)) * torch.log_softmax(tx, 1)).sum(1).mean()
+            tl.backward()
+            assert abs(loss.numpy()[0] - tl.item()) <= 1e-4 * max(1, abs(tl.item()))
+            assert np.abs(d - 0.75 * tx.grad.numpy()).max() <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_adam_and_sgd_step_bit_exact(ctx, train, dtype):
+    rng = np.random.default_rng(73)
+    dt = np.dtype(dtype).type
+    for n in (1, 10, 864, 18432, 163840):
+        for wd in (0.0, 0.01):
+            w = rng.standard_normal(n).astype(dtype)
+            m = (rng.standard_normal(n) * 0.1).astype(dtype)
+            v = (rng.random(n) * 0.01).astype(dtype)
+            dw, dm, dv = ctx.upload(w), ctx.upload(m), ctx.upload(v)
+            for t in (1, 2, 3):
+                g = rng.standard_normal(n).astype(dtype)
+                b1, b2 = dt(0.9), dt(0.999)
+                bc1 = dt(1) - max(dt(np.power(b1, dt(t))), dt(1e-8))
+                bc2 = dt(1) - max(dt(np.power(b2, dt(t))), dt(1e-8))
+                w, m, v = train.adam_update(w, g, m, v, dt(1e-3), b1, b2, dt(1e-8), dt(wd), bc1, bc2)
+                ctx.adam_step(dw, ctx.upload(g), dm, dv, 1e-3, 0.9, 0.999, 1e-8, wd, float(bc1), float(bc2))
+                assert np.array_equal(dw.numpy(), w) and np.array_equal(dm.numpy(), m) and np.array_equal(dv.numpy(), v), (n, wd, t)
+    import oracle as orc
+    w = rng.standard_normal(1000).astype(dtype)
+    g = rng.standard_normal(1000).astype(dtype)
+    dw = ctx.upload(w)
+    ctx.sgd_step(dw, ctx.upload(g), 0.01)
+    assert np.array_equal(dw.numpy(), orc.binary("sub", w, orc.scalar("mul_scalar", g, dt(0.01))))
