@@ -196,15 +196,20 @@ def bench_train_steps(steps=30, warmup=5, cpu=True, reference_pool=False):
             params, x, y = make_train_problem(cfg, dtype)
             key = f"{name}_{np.dtype(dtype).name}"
             out[key] = {"batch": int(x.shape[0])}
-            for literal in (True, False):
-                m = host_api.Model(cfg["spec"], params, cfg["opt"], dtype, literal_engine=literal)
+            # engine_literal: the reference's op sequence as is; engine_without_node_clones: the same minus the
+            # engine's per-node deep clones; engine_fused: fused layers, loss and optimizer (extra entry points)
+            for label, literal, fused in (("engine_literal", True, False), ("engine_without_node_clones", False, False),
+                                          ("engine_fused", False, True)):
+                if fused and reference_pool:
+                    continue
+                m = host_api.Model(cfg["spec"], params, cfg["opt"], dtype, literal_engine=literal, fused=fused)
                 m.set_batch(x, y)
                 m.train_steps(warmup)
                 st0 = host_api.pool_stats(dtype)
                 loss, ms = m.train_steps(steps)
                 st1 = host_api.pool_stats(dtype)
                 req = (st1["pool_hits"] + st1["pool_misses"]) - (st0["pool_hits"] + st0["pool_misses"])
-                out[key]["engine_literal" if literal else "engine_without_node_clones"] = {
+                out[key][label] = {
                     "ms_per_step": ms / steps, "imgs_per_s": x.shape[0] / (ms / steps / 1e3), "final_loss": loss,
                     "pool_requests_per_step": req / steps,
                     "pool_hit_rate": (st1["pool_hits"] - st0["pool_hits"]) / max(1, req),

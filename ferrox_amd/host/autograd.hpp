@@ -26,6 +26,12 @@ template <typename T> struct Operator {
     virtual ~Operator() = default;
     virtual Tensor<T> compute(const TensorRefs<T>& inputs) const = 0;
     virtual std::vector<Tensor<T>> gradient(Tensor<T> grad_output, const TensorRefs<T>& inputs, const HipStorage<T>* output) const = 0;
+    // `needs[i]` tells whether input i takes part in differentiation.  The reference's operators always return
+    // every gradient, which is what the default does; fused operators may return a null entry where needs[i] is false.
+    virtual std::vector<Tensor<T>> gradient_needs(Tensor<T> grad_output, const TensorRefs<T>& inputs, const HipStorage<T>* output,
+                                                  const std::vector<bool>&) const {
+        return gradient(std::move(grad_output), inputs, output);
+    }
     virtual size_t num_inputs() const = 0;
     virtual bool cache_output() const { return false; }
     virtual const char* name() const = 0;
@@ -356,6 +362,11 @@ template <typename T> class AutoFerroxEngine {
         auto it = grads_.find(id);
         return it == grads_.end() ? nullptr : it->second.get();
     }
+    HipStorage<T>* mutable_tensor(NodeId id) {  // in-place parameter updates of the fused optimizers
+        auto it = nodes_.find(id);
+        if (it == nodes_.end() || !it->second.is_parameter()) throw Error("Can only update parameter nodes (leaf nodes with requires_grad)");
+        return it->second.tensor.get();
+    }
     void zero_gradients() { grads_.clear(); }  // :838-840
     void update_parameter(NodeId id, Tensor<T> t) {  // :845-866
         auto it = nodes_.find(id);
@@ -406,8 +417,11 @@ template <typename T> class AutoFerroxEngine {
             return;
         }
         TensorRefs<T> in = collect(node.inputs);
-        std::vector<Tensor<T>> gs = node.op->gradient(std::move(grad_output), in, node.tensor.get());
-        for (size_t i = 0; i < node.inputs.size(); ++i) accumulate_gradient(node.inputs[i], std::move(gs[i]));
+        std::vector<bool> needs;
+        for (NodeId i : node.inputs) needs.push_back(nodes_.at(i).requires_grad);
+        std::vector<Tensor<T>> gs = node.op->gradient_needs(std::move(grad_output), in, node.tensor.get(), needs);
+        for (size_t i = 0; i < node.inputs.size(); ++i)
+            if (gs[i]) accumulate_gradient(node.inputs[i], std::move(gs[i]));
     }
     void accumulate_gradient(NodeId id, Tensor<T> g) {  // :681-698
         auto it = grads_.find(id);

@@ -1,0 +1,195 @@
+// Fused variants of the layers, the loss and the optimizers: what Ferrox's nn layer code looks like once it calls
+// the fused entry points of include/ferrox_hip.h instead of composing every step from storage ops.  They plug
+// into the same AutoFerroxEngine as graph operators; values equal the composed path (same arithmetic per element,
+// reductions to tolerance).
+//   Linear   : x.W^T through the transposed-operand GEMM (no Transpose node, linear.rs:225-228), bias (+ReLU) in
+//              place; backward dX = G.W, dW = G^T.X directly in W's layout (matrix.rs:30-55 materialises two
+//              transposes and Transpose::gradient a third), db in one pass (basic.rs:10-53 takes one per axis)
+//   Conv2d   : conv, bias (+ReLU) in place (conv2d.rs:203-213 materialises the broadcast bias first); backward
+//              skips the data gradient of an input that needs none (the first layer)
+//   CCELoss  : one forward and one backward kernel (classification.rs:191-257 builds 7 nodes)
+//   Adam/SGD : one in-place kernel per parameter (adam.rs:288-358 runs ~14 and clones the parameter and moments)
+#pragma once
+#include "autograd.hpp"
+
+namespace ferrox {
+
+template <typename T> struct FusedApi;
+#define FERROX_FUSED_API(T, S)                                                                                         \
+    template <> struct FusedApi<T> {                                                                                   \
+        static int bias_act(fx_ctx* c, T* y, const T* b, int64_t o, int64_t C, int64_t i, int act) { return fx_bias_act_##S(c, y, b, o, C, i, act); } \
+        static int bias_grad(fx_ctx* c, const T* g, T* out, int64_t o, int64_t C, int64_t i) { return fx_bias_grad_##S(c, g, out, o, C, i); } \
+        static int sce_fwd(fx_ctx* c, const T* x, const T* y, T* p, T* l, int64_t B, int64_t C) { return fx_softmax_ce_fwd_##S(c, x, y, p, l, B, C); } \
+        static int sce_bwd(fx_ctx* c, const T* p, const T* y, const T* g, T* d, int64_t B, int64_t C) { return fx_softmax_ce_bwd_##S(c, p, y, g, d, B, C); } \
+        static int adam(fx_ctx* c, T* p, const T* g, T* m, T* v, int64_t n, T lr, T b1, T b2, T eps, T wd, T bc1, T bc2) { \
+            return fx_adam_step_##S(c, p, g, m, v, n, lr, b1, b2, eps, wd, bc1, bc2);                                  \
+        }                                                                                                              \
+        static int sgd(fx_ctx* c, T* p, const T* g, int64_t n, T lr) { return fx_sgd_step_##S(c, p, g, n, lr); }       \
+        static int relu_bwd(fx_ctx* c, const T* g, const T* x, T* o, int64_t n) { return fx_relu_bwd_##S(c, g, x, o, n); } \
+    };
+FERROX_FUSED_API(float, f32)
+FERROX_FUSED_API(double, f64)
+#undef FERROX_FUSED_API
+
+inline fx_ctx* fused_ctx() { return BackendManager::get().ctx(); }
+
+// g * (y > 0): the ReLU mask taken from the activation's OUTPUT (y > 0 exactly when its input was > 0)
+template <typename T> Tensor<T> relu_mask_grad(const HipStorage<T>& g, const HipStorage<T>& y) {
+    Tensor<T> r = HipStorage<T>::alloc(g.shape());
+    fx_ok(FusedApi<T>::relu_bwd(fused_ctx(), g.data(), y.data(), r->data(), (int64_t)g.size()));
+    return r;
+}
+
+template <typename T> struct LinearFusedOp : Operator<T> {  // inputs: x [B, in], W [out, in], b [out]
+    bool relu;
+    explicit LinearFusedOp(bool relu_) : relu(relu_) {}
+    Tensor<T> compute(const TensorRefs<T>& in) const override {
+        const Shape &xs = in[0]->shape(), &ws = in[1]->shape();
+        if (xs.size() != 2 || ws.size() != 2 || xs[1] != ws[1]) throw Error("Linear: input " + fmt_shape(xs) + " vs weight " + fmt_shape(ws));
+        Tensor<T> y = HipStorage<T>::alloc({xs[0], ws[0]});
+        fx_ok(Api<T>::gemm(fused_ctx(), 0, 1, (int64_t)xs[0], (int64_t)ws[0], (int64_t)xs[1], in[0]->data(), in[1]->data(), y->data()));
+        fx_ok(FusedApi<T>::bias_act(fused_ctx(), y->data(), in[2]->data(), (int64_t)xs[0], (int64_t)ws[0], 1, relu ? 1 : 0));
+        return y;
+    }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out) const override {
+        return gradient_needs(std::move(g), in, out, {true, true, true});
+    }
+    std::vector<Tensor<T>> gradient_needs(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out,
+                                          const std::vector<bool>& needs) const override {
+        const Shape &xs = in[0]->shape(), &ws = in[1]->shape();
+        const int64_t B = (int64_t)xs[0], I = (int64_t)xs[1], O = (int64_t)ws[0];
+        if (relu) g = relu_mask_grad<T>(*g, *out);
+        std::vector<Tensor<T>> r(3);
+        if (needs[0]) {
+            r[0] = HipStorage<T>::alloc(xs);
+            fx_ok(Api<T>::gemm(fused_ctx(), 0, 0, B, I, O, g->data(), in[1]->data(), r[0]->data()));
+        }
+        r[1] = HipStorage<T>::alloc(ws);
+        fx_ok(Api<T>::gemm(fused_ctx(), 1, 0, O, I, B, g->data(), in[0]->data(), r[1]->data()));
+        r[2] = HipStorage<T>::alloc({ws[0]});
+        fx_ok(FusedApi<T>::bias_grad(fused_ctx(), g->data(), r[2]->data(), B, O, 1));
+        return r;
+    }
+    size_t num_inputs() const override { return 3; }
+    const char* name() const override { return "LinearFused"; }
+};
+
+template <typename T> struct Conv2dFusedOp : Operator<T> {  // inputs: x [B,Cin,H,W], W [Cout,Cin,kh,kw], b [Cout]
+    std::pair<size_t, size_t> stride, padding;
+    bool relu;
+    Conv2dFusedOp(std::pair<size_t, size_t> s, std::pair<size_t, size_t> p, bool relu_) : stride(s), padding(p), relu(relu_) {}
+    Tensor<T> compute(const TensorRefs<T>& in) const override {
+        Tensor<T> y = in[0]->conv2d(*in[1], stride, padding);
+        const Shape& ys = y->shape();
+        fx_ok(FusedApi<T>::bias_act(fused_ctx(), y->data(), in[2]->data(), (int64_t)ys[0], (int64_t)ys[1], (int64_t)(ys[2] * ys[3]),
+                                    relu ? 1 : 0));
+        return y;
+    }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out) const override {
+        return gradient_needs(std::move(g), in, out, {true, true, true});
+    }
+    std::vector<Tensor<T>> gradient_needs(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out,
+                                          const std::vector<bool>& needs) const override {
+        if (relu) g = relu_mask_grad<T>(*g, *out);
+        const Shape& gs = g->shape();
+        std::vector<Tensor<T>> r(3);
+        if (needs[0]) r[0] = g->deconv2d(*in[1], in[0]->shape(), stride, padding);
+        r[1] = in[0]->cross_correlation2d(*g, in[1]->shape(), stride, padding);
+        r[2] = HipStorage<T>::alloc({gs[1]});
+        fx_ok(FusedApi<T>::bias_grad(fused_ctx(), g->data(), r[2]->data(), (int64_t)gs[0], (int64_t)gs[1], (int64_t)(gs[2] * gs[3])));
+        return r;
+    }
+    size_t num_inputs() const override { return 3; }
+    const char* name() const override { return "Conv2dFused"; }
+};
+
+template <typename T> struct SoftmaxCEOp : Operator<T> {  // inputs: logits [B,C], targets [B,C]; output: scalar loss
+    mutable Tensor<T> probs;  // kept for the backward pass
+    Tensor<T> compute(const TensorRefs<T>& in) const override {
+        const Shape& s = in[0]->shape();
+        if (s.size() != 2 || in[1]->shape() != s) throw Error("CCELoss: predictions " + fmt_shape(s) + " vs targets " + fmt_shape(in[1]->shape()));
+        probs = HipStorage<T>::alloc(s);
+        Tensor<T> loss = HipStorage<T>::alloc({});
+        fx_ok(FusedApi<T>::sce_fwd(fused_ctx(), in[0]->data(), in[1]->data(), probs->data(), loss->data(), (int64_t)s[0], (int64_t)s[1]));
+        return loss;
+    }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        const Shape& s = in[0]->shape();
+        std::vector<Tensor<T>> r(2);
+        r[0] = HipStorage<T>::alloc(s);
+        fx_ok(FusedApi<T>::sce_bwd(fused_ctx(), probs->data(), in[1]->data(), g->data(), r[0]->data(), (int64_t)s[0], (int64_t)s[1]));
+        return r;  // no gradient for the targets
+    }
+    size_t num_inputs() const override { return 2; }
+    const char* name() const override { return "SoftmaxCE"; }
+};
+
+template <typename T> struct LinearFused : Module<T> {
+    size_t in_features, out_features;
+    NodeId weight = 0, bias = 0;
+    bool relu;
+    LinearFused(AutoFerroxEngine<T>& g, size_t in, size_t out, const T* w, const T* b, bool relu_) : in_features(in), out_features(out), relu(relu_) {
+        weight = g.create_variable(HipStorage<T>::from_vec(w, {out, in}), true);
+        bias = g.create_variable(HipStorage<T>::from_vec(b, {out}), true);
+    }
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
+        return g.apply_operation(std::make_unique<LinearFusedOp<T>>(relu), {input, weight, bias});
+    }
+    std::vector<NodeId> parameters() const override { return {weight, bias}; }
+};
+
+template <typename T> struct Conv2dFused : Module<T> {
+    std::pair<size_t, size_t> stride, padding;
+    NodeId weight = 0, bias = 0;
+    bool relu;
+    Conv2dFused(AutoFerroxEngine<T>& g, size_t cin, size_t cout, size_t k, size_t s, size_t p, const T* w, const T* b, bool relu_)
+        : stride(s, s), padding(p, p), relu(relu_) {
+        weight = g.create_variable(HipStorage<T>::from_vec(w, {cout, cin, k, k}), true);
+        bias = g.create_variable(HipStorage<T>::from_vec(b, {cout}), true);
+    }
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
+        return g.apply_operation(std::make_unique<Conv2dFusedOp<T>>(stride, padding, relu), {input, weight, bias});
+    }
+    std::vector<NodeId> parameters() const override { return {weight, bias}; }
+};
+
+template <typename T> NodeId cce_loss_fused(AutoFerroxEngine<T>& g, NodeId predictions, NodeId targets) {
+    return g.apply_operation(std::make_unique<SoftmaxCEOp<T>>(), {predictions, targets});
+}
+
+template <typename T> struct SGDFused : Optimizer<T> {
+    T lr;
+    explicit SGDFused(T lr_) : lr(lr_) {}
+    void step(AutoFerroxEngine<T>& g) override {
+        for (NodeId p : this->params) {
+            const HipStorage<T>* grad = g.get_gradient(p);
+            if (!grad) continue;
+            HipStorage<T>* w = g.mutable_tensor(p);
+            fx_ok(FusedApi<T>::sgd(fused_ctx(), w->data(), grad->data(), (int64_t)w->size(), lr));
+        }
+    }
+};
+
+template <typename T> struct AdamFused : Optimizer<T> {
+    T lr, beta1, beta2, eps, weight_decay;
+    long step_count = 0;
+    std::map<NodeId, Tensor<T>> m1, m2;
+    AdamFused(T lr_, T b1, T b2, T eps_, T wd) : lr(lr_), beta1(b1), beta2(b2), eps(eps_), weight_decay(wd) {}
+    void step(AutoFerroxEngine<T>& g) override {
+        step_count += 1;
+        const T stepf = (T)step_count;
+        const T b1p = std::max((T)std::pow(beta1, stepf), (T)1e-8), b2p = std::max((T)std::pow(beta2, stepf), (T)1e-8);
+        const T bc1 = T(1) - b1p, bc2 = T(1) - b2p;
+        for (NodeId p : this->params) {
+            const HipStorage<T>* grad = g.get_gradient(p);
+            if (!grad) continue;
+            HipStorage<T>* w = g.mutable_tensor(p);
+            if (!m1.count(p)) m1[p] = HipStorage<T>::zeros(w->shape());
+            if (!m2.count(p)) m2[p] = HipStorage<T>::zeros(w->shape());
+            fx_ok(FusedApi<T>::adam(fused_ctx(), w->data(), grad->data(), m1[p]->data(), m2[p]->data(), (int64_t)w->size(), lr, beta1,
+                                    beta2, eps, weight_decay, bc1, bc2));
+        }
+    }
+};
+
+}  // namespace ferrox

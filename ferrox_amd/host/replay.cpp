@@ -8,7 +8,7 @@
 #include <cstdlib>
 #include <sstream>
 
-#include "autograd.hpp"
+#include "fused.hpp"
 
 using namespace ferrox;
 
@@ -45,28 +45,42 @@ template <typename T> struct Model : ModelBase {
     std::unique_ptr<Optimizer<T>> opt;
     Tensor<T> x, y;
 
-    Model(const std::string& spec, const std::string& optspec, bool literal, const void* const* pv, int np) : graph(literal) {
+    bool fused = false;
+
+    // engine: 0 = reference op sequence without the per-node deep clones, 1 = reference op sequence as is,
+    //         2 = fused layers / loss / optimizers
+    Model(const std::string& spec, const std::string& optspec, int engine, const void* const* pv, int np)
+        : graph(engine == 1), fused(engine == 2) {
         int pi = 0;
         auto next = [&]() -> const T* {
             if (pi >= np) throw Error("not enough parameter arrays for the layer spec");
             return static_cast<const T*>(pv[pi++]);
         };
-        for (const std::string& tok : split(spec, ';')) {
-            std::stringstream ss(tok);
+        const std::vector<std::string> toks = split(spec, ';');
+        for (size_t ti = 0; ti < toks.size(); ++ti) {
+            std::stringstream ss(toks[ti]);
             std::string kind;
             ss >> kind;
+            // fused mode folds a ReLU that directly follows a linear / conv layer into that layer
+            const bool relu_next = fused && ti + 1 < toks.size() && toks[ti + 1] == "relu";
             if (kind == "linear") {
                 size_t in, out;
                 ss >> in >> out;
                 const T* w = next();
                 const T* b = next();
-                layers.push_back(std::make_unique<Linear<T>>(graph, in, out, w, b));
+                if (fused) {
+                    layers.push_back(std::make_unique<LinearFused<T>>(graph, in, out, w, b, relu_next));
+                    if (relu_next) ++ti;
+                } else layers.push_back(std::make_unique<Linear<T>>(graph, in, out, w, b));
             } else if (kind == "conv") {
                 size_t cin, cout, k, s, p;
                 ss >> cin >> cout >> k >> s >> p;
                 const T* w = next();
                 const T* b = next();
-                layers.push_back(std::make_unique<Conv2d<T>>(graph, cin, cout, k, s, p, w, b));
+                if (fused) {
+                    layers.push_back(std::make_unique<Conv2dFused<T>>(graph, cin, cout, k, s, p, w, b, relu_next));
+                    if (relu_next) ++ti;
+                } else layers.push_back(std::make_unique<Conv2d<T>>(graph, cin, cout, k, s, p, w, b));
             } else if (kind == "relu") layers.push_back(std::make_unique<ReLU<T>>());
             else if (kind == "flatten") layers.push_back(std::make_unique<Flatten<T>>());
             else throw Error("unknown layer '" + kind + "'");
@@ -78,11 +92,13 @@ template <typename T> struct Model : ModelBase {
         if (kind == "sgd") {
             double lr = 0.01;
             os >> lr;
-            opt = std::make_unique<SGD<T>>((T)lr);
+            if (fused) opt = std::make_unique<SGDFused<T>>((T)lr);
+            else opt = std::make_unique<SGD<T>>((T)lr);
         } else if (kind == "adam") {
             double lr = 1e-3, b1 = 0.9, b2 = 0.999, eps = 1e-8, wd = 0;
             os >> lr >> b1 >> b2 >> eps >> wd;
-            opt = std::make_unique<Adam<T>>((T)lr, (T)b1, (T)b2, (T)eps, (T)wd);
+            if (fused) opt = std::make_unique<AdamFused<T>>((T)lr, (T)b1, (T)b2, (T)eps, (T)wd);
+            else opt = std::make_unique<Adam<T>>((T)lr, (T)b1, (T)b2, (T)eps, (T)wd);
         } else throw Error("unknown optimizer '" + kind + "'");
         opt->params = params;
     }
@@ -102,7 +118,7 @@ template <typename T> struct Model : ModelBase {
         const NodeId xin = graph.create_variable(x->clone_storage(), false);
         const NodeId yin = graph.create_variable(y->clone_storage(), false);
         const NodeId pred = forward(xin);
-        const NodeId loss = cce_loss<T>(graph, pred, yin);
+        const NodeId loss = fused ? cce_loss_fused<T>(graph, pred, yin) : cce_loss<T>(graph, pred, yin);
         const T lv = graph.get_tensor(loss)->clone_storage()->first();
         graph.backward(loss);
         opt->step(graph);
@@ -154,11 +170,11 @@ int fxh_init(int device, int conv_grad_mode, const fx_pool_config* cfg) {
 }
 void fxh_shutdown(void) { BackendManager::get().shutdown(); }
 
-void* fxh_model_create(int dtype, const char* spec, const char* optimizer, int literal_engine, const void* const* params, int n_params) {
+void* fxh_model_create(int dtype, const char* spec, const char* optimizer, int literal_engine /* engine mode 0, 1 or 2 */, const void* const* params, int n_params) {
     ModelBase* m = nullptr;
     const int rc = guarded([&] {
-        if (dtype == FX_F32) m = new Model<float>(spec, optimizer, literal_engine != 0, params, n_params);
-        else if (dtype == FX_F64) m = new Model<double>(spec, optimizer, literal_engine != 0, params, n_params);
+        if (dtype == FX_F32) m = new Model<float>(spec, optimizer, literal_engine, params, n_params);
+        else if (dtype == FX_F64) m = new Model<double>(spec, optimizer, literal_engine, params, n_params);
         else throw Error("unknown dtype");
     });
     return rc ? nullptr : m;

@@ -64,12 +64,13 @@ def pool_stats(dtype=np.float32):
 class Model:
     """spec: 'conv CIN COUT K S P; relu; flatten; linear IN OUT; ...'  optimizer: 'sgd LR' | 'adam LR B1 B2 EPS WD'."""
 
-    def __init__(self, spec, params, optimizer, dtype=np.float32, literal_engine=True):
+    def __init__(self, spec, params, optimizer, dtype=np.float32, literal_engine=True, fused=False):
+        """literal_engine: keep the reference engine's per-node deep clones; fused: fused layers, loss and optimizer."""
         self.dtype = np.dtype(dtype)
         self._params = [np.ascontiguousarray(p, dtype=self.dtype) for p in params]
         self.shapes = [p.shape for p in self._params]
         arr = (C.c_void_p * len(params))(*[p.ctypes.data for p in self._params])
-        self.h = lib.fxh_model_create(capi.dtype_code(dtype)[0], spec.encode(), optimizer.encode(), int(literal_engine), arr,
+        self.h = lib.fxh_model_create(capi.dtype_code(dtype)[0], spec.encode(), optimizer.encode(), 2 if fused else int(literal_engine), arr,
                                       len(params))
         if not self.h:
             raise HostError(lib.fxh_last_error().decode("utf-8", "replace"))

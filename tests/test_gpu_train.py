@@ -54,18 +54,21 @@ CASES = [
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
-@pytest.mark.parametrize("literal_engine", [True, False])
-def test_train_step_matches_oracle(host, case, dtype, literal_engine):
+@pytest.mark.parametrize("engine", ["literal", "lean", "fused"])
+def test_train_step_matches_oracle(host, case, dtype, engine):
+    """engine: the reference's op sequence with / without its per-node clones, or the fused layers, loss and
+    optimizer; all three must reproduce the composed CPU oracle."""
     from oracle import train as otrain
     name, spec, in_shape, ncls, optspec, steps = case
-    if not literal_engine and name.endswith(("c2", "c5")) and dtype == np.float64:
+    literal_engine = engine == "literal"
+    if engine == "lean" and name.endswith(("c2", "c5")) and dtype == np.float64:
         pytest.skip("covered by the literal-engine run")
     tol = TOL[np.dtype(dtype)]
     params, x, y = kaiming_uniform_problem(spec, in_shape, ncls, 5, dtype)
     ref = otrain.Sequential(spec, params, dtype, conv_mode=0)
     kind, *nums = optspec.split()
     ropt = otrain.SGD(float(nums[0])) if kind == "sgd" else otrain.Adam(*[float(v) for v in nums])
-    model = host.Model(spec, params, optspec, dtype, literal_engine=literal_engine)
+    model = host.Model(spec, params, optspec, dtype, literal_engine=literal_engine, fused=engine == "fused")
     try:
         model.set_batch(x, y)
         for step in range(steps):
