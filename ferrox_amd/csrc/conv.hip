@@ -169,6 +169,75 @@ int dgrad_tile(fx_ctx* c, const T* g, const T* wt, T* dx, const Dims& d) {
     return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
 }
 
+// Strided data gradient by pixel classes.  An input pixel (y, x) only receives taps with ky = (y+ph) mod sh and
+// kx = (x+pw) mod sw (mod the strides), so the gather over all kh*kw taps multiplies mostly zeros (3 of 4 for a
+// 3x3 stride-2 layer).  Pixels are grouped by (ry, rx) = ((y+ph) % sh, (x+pw) % sw); each class is a dense
+// stride-1 correlation of grad_out with the sub-filter w[.., ry + jy*sh, rx + jx*sw] (flipped), written to the
+// class's sub-grid of dx.  One implicit GEMM per class, with exactly the useful multiply-adds.
+//   out[c][yy][xx] = sum_{j'y, j'x, oc} g[oc][yy - pad_y + j'y][xx - pad_x + j'x] * wcls[c][(j'y, j'x, oc)]
+template <typename T>
+__global__ __launch_bounds__(256) void permute_weights_class_kernel(const T* __restrict__ w, T* __restrict__ out, int Cout, int Cin, int kh,
+                                                                    int kw, int ry, int rx, int sh, int sw, int nky, int nkx) {
+    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+    const i64 n = (i64)Cin * nky * nkx * Cout;
+    if (i >= n) return;
+    const int oc = (int)(i % Cout);
+    i64 t = i / Cout;
+    const int jx = (int)(t % nkx);
+    t /= nkx;
+    const int jy = (int)(t % nky), c = (int)(t / nky);
+    const int ky = ry + (nky - 1 - jy) * sh, kx = rx + (nkx - 1 - jx) * sw;
+    out[i] = w[(((i64)oc * Cin + c) * kh + ky) * kw + kx];
+}
+
+template <typename T, class Cfg>
+int dgrad_class_tile(fx_ctx* c, const T* g, const T* wcls, T* dx, const Dims& d, const ConvShape& s, int Hy, int Wx, int y0, int x0) {
+    const i64 M = d.Cin, N = d.B * Hy * Wx, K = (i64)s.kh * s.kw * d.Cout;
+    MatLoader<T, true> al{wcls, K, (int)M};
+    ConvFwdB<T, true> bl{g, s, (int)N};
+    NchwSubgridStore<T> ep{dx, (int)d.Cin, (int)d.H, (int)d.W, Hy, Wx, y0, x0, (int)d.sh, (int)d.sw, (int)N,
+                           FastDiv((uint32_t)(Hy * Wx)), FastDiv((uint32_t)Wx)};
+    const int kps = (int)(fx::ceil_div(K, Cfg::BK) * Cfg::BK);
+    return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
+}
+
+template <typename T>
+bool dgrad_classes_ok(const Dims& d) {
+    return (d.sh > 1 || d.sw > 1) && d.kh >= d.sh && d.kw >= d.sw && d.Cout % CONV_BK == 0 && !generic_only();
+}
+
+template <typename T>
+int dgrad_classes(fx_ctx* c, const T* g, const T* w, T* dx, T* wt, const Dims& d) {
+    T* wcls = wt;
+    for (int ry = 0; ry < d.sh; ++ry)
+        for (int rx = 0; rx < d.sw; ++rx) {
+            const int y0 = (int)(((ry - d.ph) % d.sh + d.sh) % d.sh), x0 = (int)(((rx - d.pw) % d.sw + d.sw) % d.sw);
+            if (y0 >= d.H || x0 >= d.W) continue;  // no pixel of this class
+            const int Hy = (int)((d.H - y0 + d.sh - 1) / d.sh), Wx = (int)((d.W - x0 + d.sw - 1) / d.sw);
+            const int nky = (int)((d.kh - ry + d.sh - 1) / d.sh), nkx = (int)((d.kw - rx + d.sw - 1) / d.sw);
+            const int dy0 = (int)((y0 + d.ph - ry) / d.sh), dx0 = (int)((x0 + d.pw - rx) / d.sw);
+            const i64 nw = d.Cin * nky * nkx * d.Cout;
+            permute_weights_class_kernel<T><<<dim3((unsigned)fx::ceil_div(nw, 256)), dim3(256), 0, c->stream>>>(
+                w, wcls, (int)d.Cout, (int)d.Cin, (int)d.kh, (int)d.kw, ry, rx, (int)d.sh, (int)d.sw, nky, nkx);
+            FX_LAUNCH_CHECK();
+            // the class as a forward stride-1 correlation: input = grad_out [B, Cout, oh, ow], kernel nky x nkx
+            ConvShape s = make_shape(d.B, d.Cout, d.oh, d.ow, d.Cin, nky, nkx, 1, 1, 0, 0);
+            s.ph = (nky - 1) - dy0;
+            s.pw = (nkx - 1) - dx0;
+            s.oh = Hy;
+            s.ow = Wx;
+            s.div_L = FastDiv((uint32_t)(Hy * Wx));
+            s.div_ow = FastDiv((uint32_t)Wx);
+            int rc;
+            if (d.Cin > 64) rc = dgrad_class_tile<T, TileM128>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0);
+            else if (d.Cin > 32) rc = dgrad_class_tile<T, TileM64>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0);
+            else rc = dgrad_class_tile<T, TileM32>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0);
+            if (rc) return rc;
+            wcls += nw;
+        }
+    return FX_OK;
+}
+
 // Data gradient for at most 4 input channels (the first layer of an image network): the implicit GEMM would pad
 // Cin = 3 to a 32-row tile and run at 10 % useful work.  One thread owns one input pixel and all its channels and
 // gathers over (tap, oc); the filters sit in LDS as wl[tap][oc][4] so one 16-byte broadcast read feeds the channel
@@ -274,6 +343,7 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
         const cpk::Plan pl = dgrad_patch_plan<T>(c, d, mode);
         if (pl.ok && aligned16(g, wt)) return cpk::run(c, pl, g, w, dx, wt, 1, Cout, Cin, B, Cout, d.oh, d.ow, Cin, H, W, 1, 1, 2 - ph, 2 - pw);
     }
+    if (dgrad_classes_ok<T>(d)) return dgrad_classes<T>(c, g, w, dx, wt, d);
     if (Cout % CONV_BK == 0) {
         if (int rc = permute_weights<T>(c, w, wt, d, 2)) return rc;
         if (Cin > 64) return dgrad_tile<T, TileM128, true>(c, g, wt, dx, d);

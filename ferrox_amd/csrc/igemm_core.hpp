@@ -405,6 +405,22 @@ template <typename T> struct NchwStore {
     }
 };
 
+// A strided sub-grid of an NCHW tensor [.., C, H, W]: column n = (b, yy, xx) over a [Hs, Ws] grid lands on pixel
+// (y0 + yy*sy, x0 + xx*sx); row m = channel.
+template <typename T> struct NchwSubgridStore {
+    T* p;
+    int C, H, W, Hs, Ws, y0, x0, sy, sx, N;
+    FastDiv div_grid, div_ws;
+    __device__ __forceinline__ int rows() const { return C; }
+    __device__ __forceinline__ int cols() const { return N; }
+    __device__ __forceinline__ i64 row_stride() const { return (i64)H * W; }
+    __device__ __forceinline__ T* col(int n, int) const {
+        const uint32_t b = div_grid.div(n), l = n - b * (Hs * Ws);
+        const uint32_t yy = div_ws.div(l), xx = l - yy * Ws;
+        return p + ((i64)b * C * H + (y0 + (int)yy * sy)) * W + (x0 + (int)xx * sx);
+    }
+};
+
 // ---- the kernel -------------------------------------------------------------------------------------------
 // grid (N tiles, M tiles, K splits).  Split z covers k in [z*kps, min(K, (z+1)*kps)), kps a multiple of BK.
 template <typename T, class Cfg, class AL, class BL, class EP>

@@ -441,6 +441,35 @@ def test_conv2d_patch_kernel_shapes(ctx, orc):
             assert np.array_equal(out.numpy(), ref), (kind, case)
 
 
+# Strided data gradients, computed per pixel class (Cout % 16 == 0, kernel >= stride) and by the all-taps gather
+# otherwise: odd sizes, classes without pixels, kernel == stride, stride 3, 5x5, asymmetric stride and padding.
+# B, Cin, H, W, Cout, (kh, kw), (sh, sw), (ph, pw)
+STRIDED_DGRAD_CASES = [
+    (3, 5, 9, 7, 16, (3, 3), (2, 2), (1, 1)), (2, 32, 32, 32, 64, (3, 3), (2, 2), (1, 1)), (2, 40, 11, 13, 32, (3, 3), (2, 1), (1, 0)),
+    (2, 3, 8, 8, 16, (2, 2), (2, 2), (0, 0)), (2, 70, 10, 9, 48, (3, 3), (3, 3), (1, 1)), (1, 8, 12, 12, 16, (5, 5), (2, 2), (2, 2)),
+    (2, 4, 1, 9, 16, (3, 3), (2, 2), (1, 1)), (2, 130, 7, 6, 32, (3, 3), (1, 2), (0, 1)), (2, 6, 9, 9, 24, (3, 3), (2, 2), (1, 1)),
+    (1, 2, 5, 5, 16, (3, 3), (2, 2), (0, 0)),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_conv2d_strided_dgrad_vs_torch_and_oracle(ctx, orc, dtype):
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(60)
+    tol = TOL[np.dtype(dtype)]
+    for (B, Cin, H, W, Cout, k, st, pd) in STRIDED_DGRAD_CASES:
+        case = (B, Cin, H, W, Cout, k, st, pd)
+        oh, ow = orc.out_hw(H, W, k[0], k[1], st[0], st[1], pd[0], pd[1])
+        w = (rng.standard_normal((Cout, Cin, k[0], k[1])) * np.sqrt(2.0 / (Cin * k[0] * k[1]))).astype(dtype)
+        g = rng.standard_normal((B, Cout, oh, ow)).astype(dtype)
+        dx = ctx.conv2d_dgrad(ctx.upload(g), ctx.upload(w), (B, Cin, H, W), st, pd, 0).numpy()
+        tx = torch.zeros((B, Cin, H, W), dtype=torch.float64, requires_grad=True)
+        F.conv2d(tx, torch.from_numpy(w).double(), stride=st, padding=pd).backward(torch.from_numpy(g).double())
+        assert rel_err(dx, tx.grad.numpy()) <= tol * 8, case
+        assert rel_err(dx, orc.conv2d_dgrad(g, w, (B, Cin, H, W), st, pd, 0)) <= tol * 8, case
+
+
 def test_conv2d_misaligned_tensors_match_aligned(ctx):
     """Tensors that are only 4-byte aligned (a view into a larger buffer) cannot use the 16-byte loads of the
     patch kernels; the library must fall back and give the implicit-GEMM result, not fault or misread."""
