@@ -79,7 +79,27 @@ __global__ __launch_bounds__(256) void bias_grad_partial_kernel(const T* __restr
     const i64 c = blockIdx.x, slice = blockIdx.y;
     const i64 o0 = slice * rows_per_slice, o1 = min(outer, o0 + rows_per_slice);
     T s = T(0);
-    if (inner >= 64) {  // threads run along i (contiguous), rows one after the other
+    constexpr int V = 16 / (int)sizeof(T);
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    if (inner >= 64 && inner % V == 0 && ((uintptr_t)g & 15) == 0) {
+        // threads run along i in 16-byte vectors, four rows in flight; one running sum per vector lane
+        vec_t acc = vec_t(T(0));
+        const i64 nv = inner / V;
+        i64 o = o0;
+        for (; o + 4 <= o1; o += 4) {
+            for (i64 i = threadIdx.x; i < nv; i += 256) {
+                vec_t v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = reinterpret_cast<const vec_t*>(g + ((o + u) * C + c) * inner)[i];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) acc = acc + v[u];
+            }
+        }
+        for (; o < o1; ++o)
+            for (i64 i = threadIdx.x; i < nv; i += 256) acc = acc + reinterpret_cast<const vec_t*>(g + (o * C + c) * inner)[i];
+#pragma unroll
+        for (int u = 0; u < V; ++u) s = s + acc[u];
+    } else if (inner >= 64) {  // threads run along i (contiguous), rows one after the other
         for (i64 o = o0; o < o1; ++o) {
             const T* p = g + (o * C + c) * inner;
             for (i64 i = threadIdx.x; i < inner; i += 256) s = s + p[i];
