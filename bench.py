@@ -183,7 +183,7 @@ def reference_pool_config():
     return cfg
 
 
-def bench_train_steps(steps=30, warmup=5, cpu=True, reference_pool=False):
+def bench_train_steps(steps=30, warmup=5, cpu=True, reference_pool=False, only=None):
     """Full training steps (forward + backward + optimizer step, allocations from the pool) through the mirrored
     Ferrox host stack; imgs/sec = batch / wall time per step with one final synchronisation."""
     from ferrox_amd import host_api
@@ -193,6 +193,8 @@ def bench_train_steps(steps=30, warmup=5, cpu=True, reference_pool=False):
         for dtype in (np.float32, np.float64):
             if name == "C2_mlp" and dtype == np.float64:
                 continue
+            if only and (only[0] != name or only[1] != np.dtype(dtype).name):
+                continue
             params, x, y = make_train_problem(cfg, dtype)
             key = f"{name}_{np.dtype(dtype).name}"
             out[key] = {"batch": int(x.shape[0])}
@@ -200,7 +202,7 @@ def bench_train_steps(steps=30, warmup=5, cpu=True, reference_pool=False):
             # engine's per-node deep clones; engine_fused: fused layers, loss and optimizer (extra entry points)
             for label, literal, fused in (("engine_literal", True, False), ("engine_without_node_clones", False, False),
                                           ("engine_fused", False, True)):
-                if fused and reference_pool:
+                if (fused and reference_pool) or (only and only[2] != label):
                     continue
                 m = host_api.Model(cfg["spec"], params, cfg["opt"], dtype, literal_engine=literal, fused=fused)
                 m.set_batch(x, y)
@@ -300,9 +302,16 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-also", action="store_true")
     ap.add_argument("--skip-train", action="store_true", help="leave the train-step section out of `also` (short profiler runs)")
+    ap.add_argument("--train-only", nargs="?", const="all", default=None, metavar="CONFIG,DTYPE,ENGINE",
+                    help="run only the train-step section and print it (profiler runs); optional filter such as "
+                         "C5_cnn,float32,engine_fused")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the hot path has no cross-GPU exchange built); use --gpus 1")
+    if args.train_only:
+        only = None if args.train_only == "all" else tuple(args.train_only.split(","))
+        print(json.dumps({"train_step": bench_train_steps(cpu=False, only=only)}))
+        return
 
     from ferrox_amd import capi
     ctx = capi.Context(0)
