@@ -30,6 +30,7 @@ typedef Tile<128, 128, 16, 64, 64> TileM128;  // 4 waves as 2x2, 64x64 each
 typedef Tile<64, 128, 16, 64, 32> TileM64;    // 4 waves as 1x4, 64x32 each
 typedef Tile<32, 256, 16, 32, 64> TileM32;    // 4 waves as 1x4, 32x64 each
 typedef Tile<64, 64, 16, 32, 32> TileSmall;   // 4 waves as 2x2, 32x32 each
+typedef Tile<32, 32, 16, 32, 32> TileTiny;    // one wave: first-layer weight gradients (Cout <= 32, Cin*kh*kw <= 32)
 // FX_CONV_GENERIC=1 in the environment sends every shape to the implicit-GEMM kernels (A/B timing, debugging).
 static bool generic_only() { const char* v = getenv("FX_CONV_GENERIC"); return v && atoi(v) != 0; }
 
@@ -402,6 +403,7 @@ i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     const wgp::Plan pl = patch_plan<T>(c, d, mode);
     int splits, kps;
     if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64) wgrad_plan<T, TileM128>(c, d, &splits, &kps);
+    else if (d.Cout <= 32 && d.Cin * d.kh * d.kw <= 32) wgrad_plan<T, TileTiny>(c, d, &splits, &kps);
     else wgrad_plan<T, TileSmall>(c, d, &splits, &kps);
     const i64 generic = splits > 1 ? (i64)splits * d.Cout * d.Cin * d.kh * d.kw * (i64)sizeof(T) : 0;
     return pl.ok ? std::max(generic, wgp::workspace_bytes(pl, d.Cout, d.Cin)) : generic;
@@ -428,6 +430,7 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
         }
     }
     if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64) return wgrad_tile<T, TileM128>(c, x, g, dw, d, mode, ws);
+    if (d.Cout <= 32 && d.Cin * d.kh * d.kw <= 32) return wgrad_tile<T, TileTiny>(c, x, g, dw, d, mode, ws);
     return wgrad_tile<T, TileSmall>(c, x, g, dw, d, mode, ws);
 }
 
