@@ -87,6 +87,19 @@ int permute_weights(fx_ctx* c, const T* w, T* out, const Dims& d, int mode) {
     return FX_OK;
 }
 
+// Tile for an [M x N] implicit GEMM without split-K: the widest tile that fits M, stepped down while the grid
+// would leave CUs idle (a 14x14 layer at batch 32 has only 98 tiles of 128x128).  Returns 128, 64, 32 or 0 (64x64).
+inline int pick_tile(fx_ctx* c, i64 M, i64 N) {
+    const i64 cus = c ? c->num_cus : 256;
+    if (M > 64) {
+        if (fx::ceil_div(M, (i64)128) * fx::ceil_div(N, (i64)128) >= cus) return 128;
+        if (fx::ceil_div(M, (i64)64) * fx::ceil_div(N, (i64)128) >= cus) return 64;
+        return 0;
+    }
+    if (M > 32) return fx::ceil_div(N, (i64)128) >= cus ? 64 : 0;
+    return 32;
+}
+
 constexpr int CONV_BK = 16;  // slab depth of every conv tile; the (ky,kx)-outer K order needs channels % CONV_BK == 0
 
 template <typename T, class Cfg, bool FAST>
@@ -150,13 +163,19 @@ int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64
         T* wp = (T*)(ws ? ws : c->get_scratch(need));
         if (!wp) return FX_ERR_OOM;
         if (int rc = permute_weights<T>(c, w, wp, d, 0)) return rc;
-        if (Cout > 64) return fwd_tile<T, TileM128, true>(c, x, wp, y, d);
-        if (Cout > 32) return fwd_tile<T, TileM64, true>(c, x, wp, y, d);
-        return fwd_tile<T, TileM32, true>(c, x, wp, y, d);
+        switch (pick_tile(c, Cout, B * d.oh * d.ow)) {
+            case 128: return fwd_tile<T, TileM128, true>(c, x, wp, y, d);
+            case 64: return fwd_tile<T, TileM64, true>(c, x, wp, y, d);
+            case 32: return fwd_tile<T, TileM32, true>(c, x, wp, y, d);
+            default: return fwd_tile<T, TileSmall, true>(c, x, wp, y, d);
+        }
     }
-    if (Cout > 64) return fwd_tile<T, TileM128, false>(c, x, w, y, d);
-    if (Cout > 32) return fwd_tile<T, TileM64, false>(c, x, w, y, d);
-    return fwd_tile<T, TileM32, false>(c, x, w, y, d);
+    switch (pick_tile(c, Cout, B * d.oh * d.ow)) {
+        case 128: return fwd_tile<T, TileM128, false>(c, x, w, y, d);
+        case 64: return fwd_tile<T, TileM64, false>(c, x, w, y, d);
+        case 32: return fwd_tile<T, TileM32, false>(c, x, w, y, d);
+        default: return fwd_tile<T, TileSmall, false>(c, x, w, y, d);
+    }
 }
 
 template <typename T, class Cfg, bool FAST>
@@ -230,9 +249,12 @@ int dgrad_classes(fx_ctx* c, const T* g, const T* w, T* dx, T* wt, const Dims& d
             s.div_L = FastDiv((uint32_t)(Hy * Wx));
             s.div_ow = FastDiv((uint32_t)Wx);
             int rc;
-            if (d.Cin > 64) rc = dgrad_class_tile<T, TileM128>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0);
-            else if (d.Cin > 32) rc = dgrad_class_tile<T, TileM64>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0);
-            else rc = dgrad_class_tile<T, TileM32>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0);
+            switch (pick_tile(c, d.Cin, d.B * Hy * Wx)) {
+                case 128: rc = dgrad_class_tile<T, TileM128>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0); break;
+                case 64: rc = dgrad_class_tile<T, TileM64>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0); break;
+                case 32: rc = dgrad_class_tile<T, TileM32>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0); break;
+                default: rc = dgrad_class_tile<T, TileSmall>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0); break;
+            }
             if (rc) return rc;
             wcls += nw;
         }
@@ -347,14 +369,20 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
     if (dgrad_classes_ok<T>(d)) return dgrad_classes<T>(c, g, w, dx, wt, d);
     if (Cout % CONV_BK == 0) {
         if (int rc = permute_weights<T>(c, w, wt, d, 2)) return rc;
-        if (Cin > 64) return dgrad_tile<T, TileM128, true>(c, g, wt, dx, d);
-        if (Cin > 32) return dgrad_tile<T, TileM64, true>(c, g, wt, dx, d);
-        return dgrad_tile<T, TileM32, true>(c, g, wt, dx, d);
+        switch (pick_tile(c, Cin, B * H * W)) {
+            case 128: return dgrad_tile<T, TileM128, true>(c, g, wt, dx, d);
+            case 64: return dgrad_tile<T, TileM64, true>(c, g, wt, dx, d);
+            case 32: return dgrad_tile<T, TileM32, true>(c, g, wt, dx, d);
+            default: return dgrad_tile<T, TileSmall, true>(c, g, wt, dx, d);
+        }
     }
     if (int rc = permute_weights<T>(c, w, wt, d, 1)) return rc;
-    if (Cin > 64) return dgrad_tile<T, TileM128, false>(c, g, wt, dx, d);
-    if (Cin > 32) return dgrad_tile<T, TileM64, false>(c, g, wt, dx, d);
-    return dgrad_tile<T, TileM32, false>(c, g, wt, dx, d);
+    switch (pick_tile(c, Cin, B * H * W)) {
+        case 128: return dgrad_tile<T, TileM128, false>(c, g, wt, dx, d);
+        case 64: return dgrad_tile<T, TileM64, false>(c, g, wt, dx, d);
+        case 32: return dgrad_tile<T, TileM32, false>(c, g, wt, dx, d);
+        default: return dgrad_tile<T, TileSmall, false>(c, g, wt, dx, d);
+    }
 }
 
 template <typename T, class Cfg>
