@@ -95,7 +95,7 @@ def bench_conv(ctx, steps, warmup, dtype=np.float32, B=None):
 
 def bench_bandwidth(ctx, iters=20, warmup=3):
     from ferrox_amd import capi
-    out = {"reductions": {}, "elementwise": {}}
+    out = {"reductions": {}, "elementwise": {}, "pooling": {}}
     for dtype in (np.float32, np.float64):
         sfx = capi.dtype_code(dtype)[1]
         a = ctx.normal((8192, 8192), 4, 0.0, 1.0, dtype)
@@ -131,6 +131,29 @@ def bench_bandwidth(ctx, iters=20, warmup=3):
         ms = time_stream(ctx, fn, 10, 2)
         nbytes = 3 * 4 * n
         out["elementwise"][f"{name}_f32"] = {"ms": ms, "GBps": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    # pooling and its gradient on [128, 64, 112, 112] f32, 2x2 stride 2: algorithmic bytes = input + output (forward),
+    # grad_out + input + pooled + grad_in (max gradient), grad_out + grad_in (avg gradient)
+    del g, x, s, t, o
+    pshape, k2 = (128, 64, 112, 112), ((2, 2), (2, 2), (0, 0))
+    px = ctx.uniform(pshape, 9, -1.0, 1.0)
+    n_in, n_out = px.size, px.size // 4
+    out["pooling"] = {}
+    for name, is_max in (("maxpool2d", True), ("avgpool2d", False)):
+        pooled = ctx.pool2d(px, *k2, is_max)
+        pg = ctx.uniform(pooled.shape, 10, -1.0, 1.0)
+        ms = time_stream(ctx, lambda: ctx.pool2d(px, *k2, is_max), 10, 2)
+        nbytes = 4 * (n_in + n_out)
+        out["pooling"][f"{name}_f32"] = {"ms": ms, "GBps": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+        ms = time_stream(ctx, lambda: ctx.unpool2d(pg, px, pooled, *k2, is_max), 10, 2)
+        nbytes = 4 * ((2 * n_in + 2 * n_out) if is_max else (n_in + n_out))
+        out["pooling"][f"{name}_grad_f32"] = {"ms": ms, "GBps": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+        del pooled, pg
+    del px
+    g = ctx.uniform((n,), 7, -4.0, 4.0)
+    x = ctx.uniform((n,), 8, -4.0, 4.0)
+    s = ctx.unary("sigmoid", x)
+    t = ctx.unary("tanh", x)
+    o = ctx.empty((n,))
     # the same gradients composed op by op as the reference's operators do (ops/unary.rs:254-375): more array passes
     # over HBM for the same algorithmic 3 arrays; GB/s below is still algorithmic bytes / time
     t1, t2 = ctx.empty((n,)), ctx.empty((n,))

@@ -16,10 +16,11 @@ LIB_PATH = os.path.join(_HERE, "libferrox_hip.so")
 FX_F32, FX_F64 = 0, 1
 CONV_FWD, CONV_DGRAD, CONV_WGRAD = 0, 1, 2
 BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "equal": 4, "greater": 5, "greater_equal": 6, "less": 7,
-              "less_equal": 8, "min": 9, "max": 10}
-UNARY_OPS = {"neg": 0, "sqrt": 1, "exp": 2, "log": 3, "relu": 4, "sigmoid": 5, "tanh": 6, "abs": 7, "reciprocal": 8}
+              "less_equal": 8, "min": 9, "max": 10, "pow": 11}
+UNARY_OPS = {"neg": 0, "sqrt": 1, "exp": 2, "log": 3, "relu": 4, "sigmoid": 5, "tanh": 6, "abs": 7, "reciprocal": 8,
+             "sign": 9, "logical_not": 10}
 SCALAR_OPS = {"add_scalar": 0, "sub_scalar": 1, "mul_scalar": 2, "div_scalar": 3, "greater_scalar": 4,
-              "greater_equal_scalar": 5, "less_equal_scalar": 6, "less_scalar": 7}
+              "greater_equal_scalar": 5, "less_equal_scalar": 6, "less_scalar": 7, "pow_scalar": 8}
 FX_MAX_BUCKETS = 8
 
 
@@ -112,6 +113,12 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_reduce_sum_{_s}", _vp, _vp, _vp, _i64, _i64, _i64)
     _sig(f"fx_reduce_mean_{_s}", _vp, _vp, _vp, _i64, _i64, _i64)
     _sig(f"fx_reduce_max_{_s}", _vp, _vp, _vp, _vp, _i64, _i64, _i64)
+    _sig(f"fx_reduce_min_{_s}", _vp, _vp, _vp, _vp, _i64, _i64, _i64)
+    _sig(f"fx_in_range_{_s}", _vp, _vp, _ct, _ct, _vp, _i64)
+    _sig(f"fx_maxpool2d_{_s}", _vp, _vp, _vp, *([_i64] * 10))
+    _sig(f"fx_avgpool2d_{_s}", _vp, _vp, _vp, *([_i64] * 10))
+    _sig(f"fx_max_unpool2d_{_s}", _vp, _vp, _vp, _vp, _vp, *([_i64] * 10))
+    _sig(f"fx_avg_unpool2d_{_s}", _vp, _vp, _vp, *([_i64] * 10))
     _sig(f"fx_gemm_{_s}", _vp, _int, _int, _i64, _i64, _i64, _vp, _vp, _vp)
     _sig(f"fx_im2col_{_s}", _vp, _vp, _vp, *([_i64] * 10))
     _sig(f"fx_col2im_{_s}", _vp, _vp, _vp, *([_i64] * 10), _int)
@@ -289,6 +296,28 @@ class Context:
         check(self._fn("unary", a.dtype)(self.h, UNARY_OPS[op], a.ptr, o.ptr, a.size))
         return o
 
+    def in_range(self, a, lo, hi):
+        o = self.empty(a.shape, a.dtype)
+        check(self._fn("in_range", a.dtype)(self.h, a.ptr, float(lo), float(hi), o.ptr, a.size))
+        return o
+
+    def pool2d(self, x, kernel, stride, padding, is_max):
+        N, Cc, H, W = x.shape
+        (kh, kw), (sh, sw), (ph, pw) = kernel, stride, padding
+        o = self.empty((N, Cc, (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1), x.dtype)
+        check(self._fn("maxpool2d" if is_max else "avgpool2d", x.dtype)(self.h, x.ptr, o.ptr, N, Cc, H, W, kh, kw, sh, sw, ph, pw))
+        return o
+
+    def unpool2d(self, grad_out, x, pooled, kernel, stride, padding, is_max):
+        N, Cc, H, W = x.shape
+        (kh, kw), (sh, sw), (ph, pw) = kernel, stride, padding
+        gi = self.empty(x.shape, x.dtype)
+        if is_max:
+            check(self._fn("max_unpool2d", x.dtype)(self.h, grad_out.ptr, x.ptr, pooled.ptr, gi.ptr, N, Cc, H, W, kh, kw, sh, sw, ph, pw))
+        else:
+            check(self._fn("avg_unpool2d", x.dtype)(self.h, grad_out.ptr, gi.ptr, N, Cc, H, W, kh, kw, sh, sw, ph, pw))
+        return gi
+
     def clamp(self, a, lo, hi):
         o = self.empty(a.shape, a.dtype)
         check(self._fn("clamp", a.dtype)(self.h, a.ptr, float(lo), float(hi), o.ptr, a.size))
@@ -328,13 +357,13 @@ class Context:
         outer, ax, inner = self._oai(a.shape, axis)
         oshape = a.shape[:axis] + a.shape[axis + 1:]
         o = out or self.empty(oshape if oshape else (1,), a.dtype)
-        if kind == "max":
+        if kind in ("max", "min"):
             idx = None
             iptr = None
             if want_idx:
                 idx = _RawI64(self, max(1, outer * inner))
                 iptr = idx.ptr
-            check(self._fn("reduce_max", a.dtype)(self.h, a.ptr, o.ptr, iptr, outer, ax, inner))
+            check(self._fn("reduce_" + kind, a.dtype)(self.h, a.ptr, o.ptr, iptr, outer, ax, inner))
             o.shape = oshape
             if want_idx:
                 return o, idx.numpy().reshape(oshape)

@@ -130,6 +130,10 @@ template <typename T> __device__ __forceinline__ T dev_sqrt(T x);
 template <> __device__ __forceinline__ float dev_sqrt<float>(float x) { return sqrtf(x); }
 template <> __device__ __forceinline__ double dev_sqrt<double>(double x) { return sqrt(x); }
 
+template <typename T> __device__ __forceinline__ T dev_pow(T x, T y);
+template <> __device__ __forceinline__ float dev_pow<float>(float x, float y) { return powf(x, y); }
+template <> __device__ __forceinline__ double dev_pow<double>(double x, double y) { return pow(x, y); }
+
 template <typename T, int OP> struct BinF {
     __device__ __forceinline__ T operator()(T x, T y) const {
         if (OP == FX_ADD) return x + y;
@@ -142,6 +146,7 @@ template <typename T, int OP> struct BinF {
         if (OP == FX_LESS) return x < y ? T(1) : T(0);
         if (OP == FX_LESS_EQUAL) return x <= y ? T(1) : T(0);
         if (OP == FX_MIN) return x <= y ? x : y;
+        if (OP == FX_POW) return dev_pow<T>(x, y);
         return x >= y ? x : y;  // FX_MAX
     }
 };
@@ -156,6 +161,7 @@ template <typename T, int OP> struct ScalarF {
         if (OP == FX_GREATER_SCALAR) return x > s ? T(1) : T(0);
         if (OP == FX_GREATER_EQUAL_SCALAR) return x >= s ? T(1) : T(0);
         if (OP == FX_LESS_EQUAL_SCALAR) return x <= s ? T(1) : T(0);
+        if (OP == FX_POW_SCALAR) return dev_pow<T>(x, s);
         return x < s ? T(1) : T(0);  // FX_LESS_SCALAR
     }
 };
@@ -184,6 +190,8 @@ template <typename T, int OP> struct UnaryF {
         if (OP == FX_SIGMOID) return T(1) / (T(1) + dev_exp<T>(-x));
         if (OP == FX_TANH) return tanh_like_cpu<T>(x);
         if (OP == FX_ABS) return x < T(0) ? -x : x;
+        if (OP == FX_SIGN) return x > T(0) ? T(1) : (x < T(0) ? T(-1) : T(0));
+        if (OP == FX_LOGICAL_NOT) return x == T(0) ? T(1) : T(0);
         return T(1) / x;  // FX_RECIPROCAL
     }
 };
@@ -191,6 +199,10 @@ template <typename T, int OP> struct UnaryF {
 template <typename T> struct ClampF {
     T lo, hi;
     __device__ __forceinline__ T operator()(T x, T) const { return x < lo ? lo : (x > hi ? hi : x); }
+};
+template <typename T> struct InRangeF {
+    T lo, hi;
+    __device__ __forceinline__ T operator()(T x, T) const { return (x >= lo && x <= hi) ? T(1) : T(0); }
 };
 template <typename T> struct FillF {
     T v;
@@ -219,7 +231,7 @@ int binary_dispatch(fx_ctx* c, int op, const T* a, const T* b, T* o, i64 n) {
     switch (op) {
 #define CASE(OP) case OP: return launch_ew<T, 2>(c, a, b, o, n, BinF<T, OP>{}, "fx_binary");
         CASE(FX_ADD) CASE(FX_SUB) CASE(FX_MUL) CASE(FX_DIV) CASE(FX_EQUAL) CASE(FX_GREATER) CASE(FX_GREATER_EQUAL)
-        CASE(FX_LESS) CASE(FX_LESS_EQUAL) CASE(FX_MIN) CASE(FX_MAX)
+        CASE(FX_LESS) CASE(FX_LESS_EQUAL) CASE(FX_MIN) CASE(FX_MAX) CASE(FX_POW)
 #undef CASE
     }
     fx::set_error("fx_binary: unknown op %d", op);
@@ -231,7 +243,7 @@ int scalar_dispatch(fx_ctx* c, int op, const T* a, T s, T* o, i64 n) {
     switch (op) {
 #define CASE(OP) case OP: return launch_ew<T, 1>(c, a, (const T*)nullptr, o, n, ScalarF<T, OP>{s}, "fx_scalar");
         CASE(FX_ADD_SCALAR) CASE(FX_SUB_SCALAR) CASE(FX_MUL_SCALAR) CASE(FX_DIV_SCALAR) CASE(FX_GREATER_SCALAR)
-        CASE(FX_GREATER_EQUAL_SCALAR) CASE(FX_LESS_EQUAL_SCALAR) CASE(FX_LESS_SCALAR)
+        CASE(FX_GREATER_EQUAL_SCALAR) CASE(FX_LESS_EQUAL_SCALAR) CASE(FX_LESS_SCALAR) CASE(FX_POW_SCALAR)
 #undef CASE
     }
     fx::set_error("fx_scalar: unknown op %d", op);
@@ -243,7 +255,7 @@ int unary_dispatch(fx_ctx* c, int op, const T* a, T* o, i64 n) {
     switch (op) {
 #define CASE(OP) case OP: return launch_ew<T, 1>(c, a, (const T*)nullptr, o, n, UnaryF<T, OP>{}, "fx_unary");
         CASE(FX_NEG) CASE(FX_SQRT) CASE(FX_EXP) CASE(FX_LOG) CASE(FX_RELU) CASE(FX_SIGMOID) CASE(FX_TANH) CASE(FX_ABS)
-        CASE(FX_RECIPROCAL)
+        CASE(FX_RECIPROCAL) CASE(FX_SIGN) CASE(FX_LOGICAL_NOT)
 #undef CASE
     }
     fx::set_error("fx_unary: unknown op %d", op);
@@ -500,6 +512,9 @@ int random_fill(fx_ctx* c, T* out, i64 n, uint64_t seed, T a, T b) {
     extern "C" int fx_tanh_##S(fx_ctx* c, const T* a, T* o, int64_t n) { return unary_dispatch<T>(c, FX_TANH, a, o, n); } \
     extern "C" int fx_clamp_##S(fx_ctx* c, const T* a, T lo, T hi, T* o, int64_t n) {                                  \
         return launch_ew<T, 1>(c, a, (const T*)nullptr, o, n, ClampF<T>{lo, hi}, "fx_clamp");                          \
+    }                                                                                                                  \
+    extern "C" int fx_in_range_##S(fx_ctx* c, const T* a, T lo, T hi, T* o, int64_t n) {                               \
+        return launch_ew<T, 1>(c, a, (const T*)nullptr, o, n, InRangeF<T>{lo, hi}, "fx_in_range");                     \
     }                                                                                                                  \
     extern "C" int fx_relu_bwd_##S(fx_ctx* c, const T* g, const T* x, T* o, int64_t n) {                               \
         return launch_ew<T, 2>(c, g, x, o, n, ReluBwdF<T>{}, "fx_relu_bwd");                                           \

@@ -56,24 +56,28 @@ __device__ __forceinline__ i64 shfl_down_i64(i64 v, int d) {
 __device__ __forceinline__ double shfl_down_t(double v, int d) { return __shfl_down(v, d, 64); }
 __device__ __forceinline__ float shfl_down_t(float v, int d) { return __shfl_down(v, d, 64); }
 
-// Accumulator: value (+ index when IS_MAX).  Sum ignores idx.
-template <typename T, bool IS_MAX> struct Acc {
+// Accumulator: value (+ index for the extrema).  IS_MAX: 0 = sum (ignores idx), 1 = maximum, 2 = minimum.
+// The extrema start from the lowest / highest finite T and take strictly greater / smaller values
+// (cpu.rs:1231-1234, 1240-1252), so the first position attaining the extremum wins.
+template <typename T, int IS_MAX> struct Acc {
     T v;
     i64 i;
-    __device__ __forceinline__ void init() { v = IS_MAX ? lowest<T>() : T(0); i = NO_INDEX; }
+    __device__ __forceinline__ void init() { v = IS_MAX == 1 ? lowest<T>() : IS_MAX == 2 ? -lowest<T>() : T(0); i = NO_INDEX; }
     // element x at axis position p, visited in increasing p by this thread
     __device__ __forceinline__ void take(T x, i64 p) {
-        if (IS_MAX) { if (x > v) { v = x; i = p; } }
+        if (IS_MAX == 1) { if (x > v) { v = x; i = p; } }
+        else if (IS_MAX == 2) { if (x < v) { v = x; i = p; } }
         else v = v + x;
     }
     // merge another accumulator (any order): ties go to the smaller index
     __device__ __forceinline__ void merge(T ov, i64 oi) {
-        if (IS_MAX) { if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; } }
+        if (IS_MAX == 1) { if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; } }
+        else if (IS_MAX == 2) { if (ov < v || (ov == v && oi < i)) { v = ov; i = oi; } }
         else v = v + ov;
     }
 };
 
-template <typename T, bool IS_MAX>
+template <typename T, int IS_MAX>
 __device__ __forceinline__ void wave_reduce(Acc<T, IS_MAX>& a) {
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) {
@@ -87,7 +91,7 @@ __device__ __forceinline__ void wave_reduce(Acc<T, IS_MAX>& a) {
 // ---- row reduction (inner == 1) ---------------------------------------------------------------------------
 // grid (S, outer), 256 threads.  Slice s covers [s*chunk, min(axis, (s+1)*chunk)).  VEC: 16-byte loads (requires
 // axis % N == 0, chunk % N == 0 and a 16-byte aligned base).  Output slot o*S + s.
-template <typename T, bool IS_MAX, bool VEC, bool STREAM>
+template <typename T, int IS_MAX, bool VEC, bool STREAM>
 __global__ __launch_bounds__(256) void row_reduce_kernel(const T* __restrict__ in, T* __restrict__ out, i64* __restrict__ idx_out,
                                                          i64 axis, i64 chunk, T scale) {
     constexpr int N = Vec16<T>::N;
@@ -137,7 +141,7 @@ __global__ __launch_bounds__(256) void row_reduce_kernel(const T* __restrict__ i
 }
 
 // Short rows: G = power of two >= axis lanes per row (G <= 64), 64/G rows per wave, 4 waves per block.
-template <typename T, bool IS_MAX>
+template <typename T, int IS_MAX>
 __global__ __launch_bounds__(256) void short_row_reduce_kernel(const T* __restrict__ in, T* __restrict__ out,
                                                                i64* __restrict__ idx_out, i64 outer, i64 axis, int G, T scale) {
     const int lane = threadIdx.x & 63;
@@ -160,7 +164,7 @@ __global__ __launch_bounds__(256) void short_row_reduce_kernel(const T* __restri
 }
 
 // Combine S slice partials per output: one 256-thread block per output element, slices merged with the tie rule.
-template <typename T, bool IS_MAX>
+template <typename T, int IS_MAX>
 __global__ __launch_bounds__(256) void combine_rows_kernel(const T* __restrict__ pv, const i64* __restrict__ pi, T* __restrict__ out,
                                                            i64* __restrict__ idx_out, i64 n_out, i64 S, T scale) {
     const i64 o = blockIdx.x;
@@ -188,7 +192,7 @@ __global__ __launch_bounds__(256) void combine_rows_kernel(const T* __restrict__
 // each row it visits (4 KiB at CW = 4 with 16-byte vectors); waves sharing columns take interleaved axis positions
 // and are merged through LDS.  Output slot ((o*S + s) * inner + col).
 // FROM_PARTIAL: the input is a partial array whose index values come from `pidx` instead of the axis position.
-template <typename T, bool IS_MAX, bool VEC, bool FROM_PARTIAL, int CW, bool STREAM>
+template <typename T, int IS_MAX, bool VEC, bool FROM_PARTIAL, int CW, bool STREAM>
 __global__ __launch_bounds__(256) void col_reduce_kernel(const T* __restrict__ in, const i64* __restrict__ pidx, T* __restrict__ out,
                                                          i64* __restrict__ idx_out, i64 axis, i64 inner, i64 chunk, T scale,
                                                          int final_pass) {
@@ -256,12 +260,12 @@ __global__ __launch_bounds__(256) void col_reduce_kernel(const T* __restrict__ i
     }
 }
 
-template <typename T, bool IS_MAX, bool VEC, int CW, bool STREAM>
+template <typename T, int IS_MAX, bool VEC, int CW, bool STREAM>
 void launch_col(fx_ctx* c, dim3 grid, const T* in, T* out, i64* idx_out, i64 axis, i64 inner, i64 chunk, T scale, int final_pass) {
     col_reduce_kernel<T, IS_MAX, VEC, false, CW, STREAM><<<grid, dim3(256), 0, c->stream>>>(in, nullptr, out, idx_out, axis, inner, chunk, scale, final_pass);
 }
 
-template <typename T, bool IS_MAX>
+template <typename T, int IS_MAX>
 int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i64 inner, T scale, const char* what) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(outer >= 0 && axis >= 1 && inner >= 0, "%s: bad view [%lld, %lld, %lld]", what, (long long)outer,
@@ -391,6 +395,36 @@ __global__ __launch_bounds__(256) void softmax_axis_kernel(const T* __restrict__
     for (i64 a = 0; a < axis; ++a) q[a * inner] = q[a * inner] / s;
 }
 
+// Long contiguous rows (inner == 1, e.g. the whole-tensor softmax of cpu.rs:1018-1036 viewed as one row): one block per
+// row; maximum, sum of exponentials and the division each run block-wide.  The sum is a fixed tree (reproducible),
+// not the one-thread running sum of the kernel above.
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_row_kernel(const T* __restrict__ in, T* __restrict__ out, i64 axis) {
+    __shared__ T sm[256];
+    const T* p = in + (i64)blockIdx.x * axis;
+    T* q = out + (i64)blockIdx.x * axis;
+    T m = lowest<T>();
+    for (i64 a = threadIdx.x; a < axis; a += 256) { const T x = p[a]; if (x > m) m = x; }
+    sm[threadIdx.x] = m;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w && sm[threadIdx.x + w] > sm[threadIdx.x]) sm[threadIdx.x] = sm[threadIdx.x + w];
+        __syncthreads();
+    }
+    m = sm[0];
+    __syncthreads();
+    T s = T(0);
+    for (i64 a = threadIdx.x; a < axis; a += 256) { const T e = dev_exp<T>(p[a] - m); q[a] = e; s = s + e; }
+    sm[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) sm[threadIdx.x] = sm[threadIdx.x] + sm[threadIdx.x + w];
+        __syncthreads();
+    }
+    s = sm[0];
+    for (i64 a = threadIdx.x; a < axis; a += 256) q[a] = q[a] / s;
+}
+
 template <typename T>
 int softmax_axis(fx_ctx* c, const T* in, T* out, i64 outer, i64 axis, i64 inner) {
     FX_CHECK_CTX(c);
@@ -398,6 +432,11 @@ int softmax_axis(fx_ctx* c, const T* in, T* out, i64 outer, i64 axis, i64 inner)
     if (outer == 0 || inner == 0) return FX_OK;
     FX_REQUIRE(in && out, "fx_softmax_axis: null pointer");
     FX_REQUIRE(in != out, "fx_softmax_axis: in-place not supported");
+    if (inner == 1 && axis >= 2048 && outer <= 0x7fffffff) {
+        softmax_row_kernel<T><<<dim3((unsigned)outer), dim3(256), 0, c->stream>>>(in, out, axis);
+        FX_LAUNCH_CHECK();
+        return FX_OK;
+    }
     const i64 blocks = fx::ceil_div(outer * inner, 256);
     FX_REQUIRE(blocks <= 0x7fffffff, "fx_softmax_axis: too many rows");
     softmax_axis_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(in, out, outer, axis, inner);
@@ -417,7 +456,11 @@ int softmax_axis(fx_ctx* c, const T* in, T* out, i64 outer, i64 axis, i64 inner)
     }                                                                                                                  \
     extern "C" int fx_reduce_max_##S(fx_ctx* c, const T* in, T* out, int64_t* idx, int64_t outer, int64_t axis,        \
                                      int64_t inner) {                                                                  \
-        return reduce<T, true>(c, in, out, idx, outer, axis, inner, T(1), "fx_reduce_max");                            \
+        return reduce<T, 1>(c, in, out, idx, outer, axis, inner, T(1), "fx_reduce_max");                               \
+    }                                                                                                                  \
+    extern "C" int fx_reduce_min_##S(fx_ctx* c, const T* in, T* out, int64_t* idx, int64_t outer, int64_t axis,        \
+                                     int64_t inner) {                                                                  \
+        return reduce<T, 2>(c, in, out, idx, outer, axis, inner, T(1), "fx_reduce_min");                               \
     }                                                                                                                  \
     extern "C" int fx_softmax_axis_##S(fx_ctx* c, const T* in, T* out, int64_t outer, int64_t axis, int64_t inner) {   \
         return softmax_axis<T>(c, in, out, outer, axis, inner);                                                        \

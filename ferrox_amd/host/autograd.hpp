@@ -313,6 +313,31 @@ template <typename T> struct Conv2dOp : Operator<T> {  // src/ops/batched.rs:133
     const char* name() const override { return "Conv2d"; }
 };
 
+// MaxPool2D / AvgPool2D: src/ops/pooling.rs:12-230 (square window, one stride, zero padding; the output is cached
+// because the max gradient needs to know which positions were selected)
+template <typename T> struct Pool2dOp : Operator<T> {
+    bool is_max;
+    size_t kernel, stride, padding;
+    Pool2dOp(bool mx, size_t k, size_t s, size_t p) : is_max(mx), kernel(k), stride(s), padding(p) {}
+    Tensor<T> compute(const TensorRefs<T>& in) const override {
+        return is_max ? in[0]->maxpool2d(kernel, stride, padding) : in[0]->avgpool2d(kernel, stride, padding);
+    }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out) const override {
+        if (in[0]->ndim() != 4) throw Error(std::string(is_max ? "MaxPool2D" : "AvgPool2D") + " requires 4D input tensor [N, C, H, W]");
+        Tensor<T> recomputed;
+        if (!out) {
+            recomputed = compute(in);
+            out = recomputed.get();
+        }
+        std::vector<Tensor<T>> r;
+        r.push_back(is_max ? g->max_unpool2d(*in[0], *out, kernel, stride, padding) : g->avg_unpool2d(*in[0], *out, kernel, stride, padding));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    bool cache_output() const override { return true; }
+    const char* name() const override { return is_max ? "MaxPool2D" : "AvgPool2D"; }
+};
+
 // ---- AutoFerroxEngine: src/graph/mod.rs:341-997 (eager mode) -------------------------------------------------
 using NodeId = size_t;
 
@@ -523,6 +548,15 @@ template <typename T> struct Conv2d : Module<T> {  // src/nn/layers/conv2d.rs:13
 
 template <typename T> struct ReLU : Module<T> {  // src/nn/layers/activation.rs:47-80
     NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override { return g.apply_operation(std::make_unique<ReLUOp<T>>(), {input}); }
+};
+
+template <typename T> struct Pool2d : Module<T> {  // nn::MaxPool2d / AvgPool2d, src/nn/layers/pooling.rs
+    bool is_max;
+    size_t kernel, stride, padding;
+    Pool2d(bool mx, size_t k, size_t s, size_t p) : is_max(mx), kernel(k), stride(s), padding(p) {}
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
+        return g.apply_operation(std::make_unique<Pool2dOp<T>>(is_max, kernel, stride, padding), {input});
+    }
 };
 
 template <typename T> struct Flatten : Module<T> {  // src/nn/layers/pooling.rs:100-140 (batch-first)

@@ -81,6 +81,16 @@ template <typename T> struct Api;
         static int scalar(fx_ctx* c, int op, const T* a, T s, T* o, int64_t n) { return fx_scalar_##S(c, op, a, s, o, n); } \
         static int unary(fx_ctx* c, int op, const T* a, T* o, int64_t n) { return fx_unary_##S(c, op, a, o, n); }      \
         static int clamp(fx_ctx* c, const T* a, T lo, T hi, T* o, int64_t n) { return fx_clamp_##S(c, a, lo, hi, o, n); } \
+        static int in_range(fx_ctx* c, const T* a, T lo, T hi, T* o, int64_t n) { return fx_in_range_##S(c, a, lo, hi, o, n); } \
+        static int rmin(fx_ctx* c, const T* i, T* o, int64_t ou, int64_t ax, int64_t in) { return fx_reduce_min_##S(c, i, o, nullptr, ou, ax, in); } \
+        static int pool(fx_ctx* c, bool mx, const T* i, T* o, const int64_t* d) {                                      \
+            return mx ? fx_maxpool2d_##S(c, i, o, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9])          \
+                      : fx_avgpool2d_##S(c, i, o, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9]);         \
+        }                                                                                                              \
+        static int unpool(fx_ctx* c, bool mx, const T* g, const T* x, const T* p, T* gi, const int64_t* d) {           \
+            return mx ? fx_max_unpool2d_##S(c, g, x, p, gi, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9]) \
+                      : fx_avg_unpool2d_##S(c, g, gi, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9]);     \
+        }                                                                                                              \
         static int softmax(fx_ctx* c, const T* i, T* o, int64_t ou, int64_t ax, int64_t in) { return fx_softmax_axis_##S(c, i, o, ou, ax, in); } \
         static int rsum(fx_ctx* c, const T* i, T* o, int64_t ou, int64_t ax, int64_t in) { return fx_reduce_sum_##S(c, i, o, ou, ax, in); } \
         static int rmean(fx_ctx* c, const T* i, T* o, int64_t ou, int64_t ax, int64_t in) { return fx_reduce_mean_##S(c, i, o, ou, ax, in); } \
@@ -166,6 +176,24 @@ template <typename T> class HipStorage {
     Ptr mul(const HipStorage& o) const { return binary(FX_MUL, o, "multiplication"); }
     Ptr div(const HipStorage& o) const { return binary(FX_DIV, o, "division"); }
     Ptr equal(const HipStorage& o) const { return binary(FX_EQUAL, o, "comparison"); }
+    Ptr min(const HipStorage& o) const { return binary(FX_MIN, o, "min operation"); }          // cpu.rs:692-715
+    Ptr max(const HipStorage& o) const { return binary(FX_MAX, o, "max operation"); }          // cpu.rs:717-740
+    Ptr greater(const HipStorage& o) const { return binary(FX_GREATER, o, "comparison"); }     // cpu.rs:865-885
+    Ptr greater_equal(const HipStorage& o) const { return binary(FX_GREATER_EQUAL, o, "comparison"); }
+    Ptr less(const HipStorage& o) const { return binary(FX_LESS, o, "comparison"); }
+    Ptr less_equal(const HipStorage& o) const { return binary(FX_LESS_EQUAL, o, "comparison"); }
+    Ptr powf(const HipStorage& o) const { return binary(FX_POW, o, "powf"); }                  // cpu.rs:1152-1172
+    Ptr power_scalar(T s) const { return scalar(FX_POW_SCALAR, s); }                           // cpu.rs:1174-1181
+    Ptr less_scalar(T s) const { return scalar(FX_LESS_SCALAR, s); }
+    Ptr abs() const { return unary(FX_ABS); }
+    Ptr reciprocal() const { return unary(FX_RECIPROCAL); }
+    Ptr sign() const { return unary(FX_SIGN); }                                               // cpu.rs:949-965
+    Ptr logical_not() const { return unary(FX_LOGICAL_NOT); }                                 // cpu.rs:920-931
+    Ptr in_range(T lo, T hi) const {                                                          // cpu.rs:933-947
+        Ptr r = alloc(shape_);
+        fx_ok(Api<T>::in_range(ctx(), ptr_, lo, hi, r->ptr_, (int64_t)size()));
+        return r;
+    }
     Ptr add_scalar(T s) const { return scalar(FX_ADD_SCALAR, s); }
     Ptr sub_scalar(T s) const { return scalar(FX_SUB_SCALAR, s); }
     Ptr mul_scalar(T s) const { return scalar(FX_MUL_SCALAR, s); }
@@ -224,10 +252,36 @@ template <typename T> class HipStorage {
         return r;
     }
 
+    Ptr softmax() const {  // whole tensor as one row, cpu.rs:1018-1036
+        Ptr r = alloc(shape_);
+        fx_ok(Api<T>::softmax(ctx(), ptr_, r->ptr_, 1, (int64_t)size(), 1));
+        return r;
+    }
+
+    // ---- pooling and its gradients: storage/mod.rs:328-420, extensions/pooling.rs; storage/cuda.rs:1127-1290 ----
+    Ptr maxpool2d(size_t k, size_t s, size_t p) const { return pool2d(true, k, s, p, "Maxpool2d"); }
+    Ptr avgpool2d(size_t k, size_t s, size_t p) const { return pool2d(false, k, s, p, "Avgpool2d"); }
+    Ptr maxpool1d(size_t k, size_t s, size_t p) const { return pool1d(true, k, s, p, "Maxpool1d"); }
+    Ptr avgpool1d(size_t k, size_t s, size_t p) const { return pool1d(false, k, s, p, "Avgpool1d"); }
+    // self is the upstream gradient; original_input / pooled_output as in the trait
+    Ptr max_unpool2d(const HipStorage& original_input, const HipStorage& pooled_output, size_t k, size_t s, size_t p) const {
+        return unpool(true, original_input, &pooled_output, k, k, s, s, p, p);
+    }
+    Ptr avg_unpool2d(const HipStorage& original_input, const HipStorage& pooled_output, size_t k, size_t s, size_t p) const {
+        return unpool(false, original_input, &pooled_output, k, k, s, s, p, p);
+    }
+    Ptr max_unpool1d(const HipStorage& original_input, const HipStorage& pooled_output, size_t k, size_t s, size_t p) const {
+        return unpool(true, original_input, &pooled_output, 1, k, 1, s, 0, p);
+    }
+    Ptr avg_unpool1d(const HipStorage& original_input, const HipStorage& pooled_output, size_t k, size_t s, size_t p) const {
+        return unpool(false, original_input, &pooled_output, 1, k, 1, s, 0, p);
+    }
+
     // ---- reductions: cpu.rs:60-130, 1183-1238; CudaOps::reduce_axes cuda/ops.rs:2171-2284 ---------------------
     // axes == nullptr reduces everything to a 0-dimensional result (or all-ones shape with keep_dims).
     Ptr sum(const std::vector<size_t>* axes, bool keep_dims) const { return reduce(0, axes, keep_dims); }
     Ptr max_reduce(const std::vector<size_t>* axes, bool keep_dims) const { return reduce(2, axes, keep_dims); }
+    Ptr min_reduce(const std::vector<size_t>* axes, bool keep_dims) const { return reduce(3, axes, keep_dims); }  // cpu.rs:1240-1252
     Ptr mean(const std::vector<size_t>* axes, bool keep_dims) const {  // sum * T(1/n), cpu.rs:1193-1221
         Ptr s = reduce(0, axes, keep_dims);
         double n = 1;
@@ -391,11 +445,39 @@ template <typename T> class HipStorage {
         std::swap(granted_, r->granted_);
         shape_ = ns;
     }
-    // kind 0 sum, 2 max.  One kernel per axis, axes in descending order, temporaries between steps
+    Ptr pool2d(bool is_max, size_t k, size_t s, size_t p, const char* what) const {
+        if (ndim() != 4) throw Error(std::string(what) + " requires 4D tensor [N, C, H, W]");
+        const int64_t d[10] = {(int64_t)shape_[0], (int64_t)shape_[1], (int64_t)shape_[2], (int64_t)shape_[3], (int64_t)k, (int64_t)k,
+                               (int64_t)s, (int64_t)s, (int64_t)p, (int64_t)p};
+        Ptr r = alloc({shape_[0], shape_[1], (shape_[2] + 2 * p - k) / s + 1, (shape_[3] + 2 * p - k) / s + 1});
+        fx_ok(Api<T>::pool(ctx(), is_max, ptr_, r->ptr_, d));
+        return r;
+    }
+    Ptr pool1d(bool is_max, size_t k, size_t s, size_t p, const char* what) const {  // [N, C, L] = H of 1, window 1 x k
+        if (ndim() != 3) throw Error(std::string(what) + " requires 3D tensor [N, C, L]");
+        const int64_t d[10] = {(int64_t)shape_[0], (int64_t)shape_[1], 1, (int64_t)shape_[2], 1, (int64_t)k, 1, (int64_t)s, 0, (int64_t)p};
+        Ptr r = alloc({shape_[0], shape_[1], (shape_[2] + 2 * p - k) / s + 1});
+        fx_ok(Api<T>::pool(ctx(), is_max, ptr_, r->ptr_, d));
+        return r;
+    }
+    Ptr unpool(bool is_max, const HipStorage& x, const HipStorage* pooled, size_t kh, size_t kw, size_t sh, size_t sw, size_t ph,
+               size_t pw) const {
+        const bool one_d = x.ndim() == 3;
+        if (!one_d && (x.ndim() != 4 || ndim() != 4)) throw Error("Unpool2D requires 4D tensors [N, C, H, W]");
+        if (one_d && ndim() != 3) throw Error("Unpool1D requires 3D tensors [N, C, L]");
+        const Shape& xs = x.shape_;
+        const int64_t d[10] = {(int64_t)xs[0], (int64_t)xs[1], one_d ? 1 : (int64_t)xs[2], (int64_t)xs[one_d ? 2 : 3], (int64_t)kh,
+                               (int64_t)kw, (int64_t)sh, (int64_t)sw, (int64_t)ph, (int64_t)pw};
+        Ptr r = alloc(xs);
+        fx_ok(Api<T>::unpool(ctx(), is_max, ptr_, x.ptr_, pooled ? pooled->ptr_ : nullptr, r->ptr_, d));
+        return r;
+    }
+    // kind 0 sum, 2 max, 3 min.  One kernel per axis, axes in descending order, temporaries between steps
     // (CudaOps::reduce_axes, cuda/ops.rs:2171-2284; the CPU backend uses the same order, cpu.rs:85-95).
     Ptr reduce(int kind, const std::vector<size_t>* axes, bool keep_dims) const {
         auto launch = [&](const T* in, T* out, int64_t outer, int64_t ax, int64_t inner) {
-            fx_ok(kind == 0 ? Api<T>::rsum(ctx(), in, out, outer, ax, inner) : Api<T>::rmax(ctx(), in, out, outer, ax, inner));
+            fx_ok(kind == 0 ? Api<T>::rsum(ctx(), in, out, outer, ax, inner)
+                  : kind == 2 ? Api<T>::rmax(ctx(), in, out, outer, ax, inner) : Api<T>::rmin(ctx(), in, out, outer, ax, inner));
         };
         if (!axes) {
             Shape fs = keep_dims ? Shape(ndim(), 1) : Shape{};

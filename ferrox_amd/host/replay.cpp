@@ -81,6 +81,10 @@ template <typename T> struct Model : ModelBase {
                     layers.push_back(std::make_unique<Conv2dFused<T>>(graph, cin, cout, k, s, p, w, b, relu_next));
                     if (relu_next) ++ti;
                 } else layers.push_back(std::make_unique<Conv2d<T>>(graph, cin, cout, k, s, p, w, b));
+            } else if (kind == "maxpool" || kind == "avgpool") {
+                size_t k, st, p;
+                ss >> k >> st >> p;
+                layers.push_back(std::make_unique<Pool2d<T>>(kind == "maxpool", k, st, p));
             } else if (kind == "relu") layers.push_back(std::make_unique<ReLU<T>>());
             else if (kind == "flatten") layers.push_back(std::make_unique<Flatten<T>>());
             else throw Error("unknown layer '" + kind + "'");

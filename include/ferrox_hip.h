@@ -131,11 +131,11 @@ int64_t fx_conv2d_workspace_bytes(int kind, int dtype, int mode, int64_t B, int6
 
 /* Binary / scalar / unary op selectors for the generic entry points (also exported one by one below). */
 enum fx_binary_op { FX_ADD = 0, FX_SUB = 1, FX_MUL = 2, FX_DIV = 3, FX_EQUAL = 4, FX_GREATER = 5, FX_GREATER_EQUAL = 6,
-                    FX_LESS = 7, FX_LESS_EQUAL = 8, FX_MIN = 9, FX_MAX = 10 };
+                    FX_LESS = 7, FX_LESS_EQUAL = 8, FX_MIN = 9, FX_MAX = 10, FX_POW = 11 };
 enum fx_unary_op { FX_NEG = 0, FX_SQRT = 1, FX_EXP = 2, FX_LOG = 3, FX_RELU = 4, FX_SIGMOID = 5, FX_TANH = 6, FX_ABS = 7,
-                   FX_RECIPROCAL = 8 };
+                   FX_RECIPROCAL = 8, FX_SIGN = 9, FX_LOGICAL_NOT = 10 };
 enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_DIV_SCALAR = 3, FX_GREATER_SCALAR = 4,
-                    FX_GREATER_EQUAL_SCALAR = 5, FX_LESS_EQUAL_SCALAR = 6, FX_LESS_SCALAR = 7 };
+                    FX_GREATER_EQUAL_SCALAR = 5, FX_LESS_EQUAL_SCALAR = 6, FX_LESS_SCALAR = 7, FX_POW_SCALAR = 8 };
 
 #define FX_DECLARE_KERNELS(T, S)                                                                                       \
     /* launch_fill, kernels.rs:435-448 */                                                                              \
@@ -179,6 +179,10 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
     int fx_tanh_##S(fx_ctx* ctx, const T* a, T* out, int64_t n);                                                       \
     /* launch_clamp, kernels.rs:894-917 / cpu.rs:792-805 */                                                            \
     int fx_clamp_##S(fx_ctx* ctx, const T* a, T lo, T hi, T* out, int64_t n);                                          \
+    /* in_range, cpu.rs:933-947: 1 where lo <= a <= hi, else 0.  (min/max/greater/less... of two tensors, sign,        \
+       logical_not, powf and power_scalar -- cpu.rs:692-740, 815-965, 1152-1182 -- go through the fx_binary /          \
+       fx_unary / fx_scalar selectors.) */                                                                             \
+    int fx_in_range_##S(fx_ctx* ctx, const T* a, T lo, T hi, T* out, int64_t n);                                       \
     /* Fused activation gradients.  The reference has no backward kernels: ReLU::gradient, Sigmoid::gradient and       \
        Tanh::gradient (src/ops/unary.rs:358-375, 254-276, 306-328) compose 2-4 storage ops.  These produce the         \
        same values in one pass: relu: g*(x>0); tanh: g*(-(t*t-1)); sigmoid: literal=1 -> g*(s*(s-1)) (the              \
@@ -196,6 +200,9 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
     int fx_reduce_sum_##S(fx_ctx* ctx, const T* in, T* out, int64_t outer, int64_t axis, int64_t inner);               \
     int fx_reduce_mean_##S(fx_ctx* ctx, const T* in, T* out, int64_t outer, int64_t axis, int64_t inner);              \
     int fx_reduce_max_##S(fx_ctx* ctx, const T* in, T* out, int64_t* idx_out, int64_t outer, int64_t axis,             \
+                          int64_t inner);                                                                              \
+    /* min_reduce, cpu.rs:1240-1252: starts from the highest finite T, takes strictly smaller values; idx_out as above. */ \
+    int fx_reduce_min_##S(fx_ctx* ctx, const T* in, T* out, int64_t* idx_out, int64_t outer, int64_t axis,             \
                           int64_t inner);                                                                              \
     /* launch_matmul, kernels.rs:919-938 / cpu.rs:967-1002: C[M,N] = op(A) . op(B).  trans_a: A is stored [K,M];       \
        trans_b: B is stored [N,K]  (lets MatMul::gradient, src/ops/matrix.rs:30-55, skip materialised transposes). */  \
@@ -226,6 +233,21 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
     int fx_conv2d_wgrad_##S(fx_ctx* ctx, const T* x, const T* g, T* dw, int64_t B, int64_t Cin, int64_t H, int64_t W,  \
                             int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,      \
                             int mode, void* workspace, int64_t ws_bytes);                                              \
+    /* maxpool2d / avgpool2d and their gradients max_unpool2d / avg_unpool2d, storage/mod.rs:328-420 ->                \
+       extensions/pooling.rs:154-229, 339-418 (launch_maxpool2d... kernels.rs; kernels/convolutions.cu:671-1222).      \
+       NCHW, out is [N, C, (H+2ph-kh)/sh+1, (W+2pw-kw)/sw+1]; the reference's square window / single stride is         \
+       kh == kw, sh == sw; the 1-D calls ([N, C, L]) are H = 1, kh = 1, sh = 1, ph = 0.  Bit-identical to the CPU      \
+       loops: max from the lowest finite T with strict >, avg over the in-bounds count, max gradient where             \
+       |in - pooled| < 1e-8, avg gradient scaled by T(1.0f / float(kh*kw)). */                                         \
+    int fx_maxpool2d_##S(fx_ctx* ctx, const T* in, T* out, int64_t N, int64_t C, int64_t H, int64_t W, int64_t kh,     \
+                         int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw);                                  \
+    int fx_avgpool2d_##S(fx_ctx* ctx, const T* in, T* out, int64_t N, int64_t C, int64_t H, int64_t W, int64_t kh,     \
+                         int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw);                                  \
+    int fx_max_unpool2d_##S(fx_ctx* ctx, const T* grad_out, const T* in, const T* pooled, T* grad_in, int64_t N,       \
+                            int64_t C, int64_t H, int64_t W, int64_t kh, int64_t kw, int64_t sh, int64_t sw,           \
+                            int64_t ph, int64_t pw);                                                                   \
+    int fx_avg_unpool2d_##S(fx_ctx* ctx, const T* grad_out, T* grad_in, int64_t N, int64_t C, int64_t H, int64_t W,    \
+                            int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw);                   \
     /* ---- fused sequences (optional: every one equals a chain of the entry points above) ----                        \
        Bias add, in place, on y viewed as [outer, C, inner] (conv: outer = B, inner = oh*ow; linear: outer = B,        \
        inner = 1), act 0 = none, 1 = ReLU.  Replaces Reshape + BroadcastTo + Add (+ ReLU) of                           \

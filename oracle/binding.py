@@ -13,10 +13,11 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libferrox_oracle.so")
 
 BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "equal": 4, "greater": 5, "greater_equal": 6, "less": 7,
-              "less_equal": 8, "min": 9, "max": 10}
-UNARY_OPS = {"neg": 0, "sqrt": 1, "exp": 2, "log": 3, "relu": 4, "sigmoid": 5, "tanh": 6, "abs": 7, "reciprocal": 8}
+              "less_equal": 8, "min": 9, "max": 10, "pow": 11}
+UNARY_OPS = {"neg": 0, "sqrt": 1, "exp": 2, "log": 3, "relu": 4, "sigmoid": 5, "tanh": 6, "abs": 7, "reciprocal": 8,
+             "sign": 9, "logical_not": 10}
 SCALAR_OPS = {"add_scalar": 0, "sub_scalar": 1, "mul_scalar": 2, "div_scalar": 3, "greater_scalar": 4,
-              "greater_equal_scalar": 5, "less_equal_scalar": 6, "less_scalar": 7}
+              "greater_equal_scalar": 5, "less_equal_scalar": 6, "less_scalar": 7, "pow_scalar": 8}
 
 
 def build():
@@ -190,9 +191,9 @@ def reduce_axis(kind, x, axis, want_idx=False):
     outer, ax, inner = _oai(x.shape, axis)
     out_shape = x.shape[:axis] + x.shape[axis + 1:]
     out = np.empty(out_shape, dtype=x.dtype)
-    if kind == "max":
+    if kind in ("max", "min"):
         idx = np.empty(out_shape, dtype=np.int64)
-        _fn("orc_reduce_max", x.dtype)(_p(x), _i64(outer), _i64(ax), _i64(inner), _p(out), _p(idx))
+        _fn("orc_reduce_" + kind, x.dtype)(_p(x), _i64(outer), _i64(ax), _i64(inner), _p(out), _p(idx))
         return (out, idx) if want_idx else out
     _fn("orc_reduce_" + kind, x.dtype)(_p(x), _i64(outer), _i64(ax), _i64(inner), _p(out))
     return out
@@ -217,6 +218,42 @@ def reduce(kind, x, axes=None, keep_dims=False):
             fs[a] = 1
         r = r.reshape(fs)
     return r
+
+
+def in_range(a, lo, hi):
+    a = _c(a)
+    o = np.empty_like(a)
+    _, ct = _sfx(a.dtype)
+    _fn("orc_in_range", a.dtype)(_p(a), ct(lo), ct(hi), _p(o), _i64(a.size))
+    return o
+
+
+def softmax_all(x):
+    """Whole-tensor softmax (cpu.rs:1018-1036): the tensor as one row."""
+    x = _c(x)
+    return softmax_axis(x.reshape(1, -1), 1).reshape(x.shape)
+
+
+def pool2d(x, kernel, stride, padding, is_max):
+    """maxpool2d / avgpool2d (extensions/pooling.rs:154-229) on [N,C,H,W]."""
+    x = _c(x)
+    N, Cc, H, W = x.shape
+    (kh, kw), (sh, sw), (ph, pw) = kernel, stride, padding
+    oh, ow = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    out = np.empty((N, Cc, oh, ow), x.dtype)
+    _fn("orc_pool2d", x.dtype)(_p(x), _p(out), *[_i64(v) for v in (N, Cc, H, W, kh, kw, sh, sw, ph, pw)], C.c_int(int(is_max)))
+    return out
+
+
+def unpool2d(grad_out, x, pooled, kernel, stride, padding, is_max):
+    """max_unpool2d / avg_unpool2d (extensions/pooling.rs:339-418): gradient w.r.t. the pooling input."""
+    x, grad_out, pooled = _c(x), _c(grad_out), _c(pooled)
+    N, Cc, H, W = x.shape
+    (kh, kw), (sh, sw), (ph, pw) = kernel, stride, padding
+    gin = np.empty_like(x)
+    _fn("orc_unpool2d", x.dtype)(_p(grad_out), _p(x), _p(pooled), _p(gin), *[_i64(v) for v in (N, Cc, H, W, kh, kw, sh, sw, ph, pw)],
+                                 C.c_int(int(is_max)))
+    return gin
 
 
 def softmax_axis(x, axis):

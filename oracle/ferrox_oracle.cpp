@@ -183,9 +183,9 @@ void conv2d_wgrad(const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, i64 W, i
 // Elementwise: src/backend/storage/cpu.rs:629-690 (binary), :741-767 (scalar, neg), :792-813 (clamp, sqrt),
 // :829-918 (comparisons -> 1.0/0.0), :1004-1016 sigmoid, :1070-1100 relu/exp/log, :1102-1150 tanh.
 // ---------------------------------------------------------------------------------------------
-enum { B_ADD = 0, B_SUB = 1, B_MUL = 2, B_DIV = 3, B_EQUAL = 4, B_GREATER = 5, B_GE = 6, B_LESS = 7, B_LE = 8, B_MIN = 9, B_MAX = 10 };
-enum { U_NEG = 0, U_SQRT = 1, U_EXP = 2, U_LOG = 3, U_RELU = 4, U_SIGMOID = 5, U_TANH = 6, U_ABS = 7, U_RECIP = 8 };
-enum { S_ADD = 0, S_SUB = 1, S_MUL = 2, S_DIV = 3, S_GREATER = 4, S_GE = 5, S_LE = 6, S_LESS = 7 };
+enum { B_ADD = 0, B_SUB = 1, B_MUL = 2, B_DIV = 3, B_EQUAL = 4, B_GREATER = 5, B_GE = 6, B_LESS = 7, B_LE = 8, B_MIN = 9, B_MAX = 10, B_POW = 11 };
+enum { U_NEG = 0, U_SQRT = 1, U_EXP = 2, U_LOG = 3, U_RELU = 4, U_SIGMOID = 5, U_TANH = 6, U_ABS = 7, U_RECIP = 8, U_SIGN = 9, U_NOT = 10 };
+enum { S_ADD = 0, S_SUB = 1, S_MUL = 2, S_DIV = 3, S_GREATER = 4, S_GE = 5, S_LE = 6, S_LESS = 7, S_POW = 8 };
 
 template <typename T>
 T tanh_ref(T x) {  // cpu.rs:1108-1147
@@ -218,6 +218,7 @@ void binary(int op, const T* a, const T* b, T* o, i64 n) {
             case B_LE: r = x <= y ? T(1) : T(0); break;
             case B_MIN: r = x <= y ? x : y; break;   // cpu.rs:708
             case B_MAX: r = x >= y ? x : y; break;   // cpu.rs:732
+            case B_POW: r = std::pow(x, y); break;   // cpu.rs:1152-1172
             default: r = T(0);
         }
         o[i] = r;
@@ -238,6 +239,7 @@ void scalar_op(int op, const T* a, T s, T* o, i64 n) {
             case S_GE: r = x >= s ? T(1) : T(0); break;
             case S_LE: r = x <= s ? T(1) : T(0); break;
             case S_LESS: r = x < s ? T(1) : T(0); break;
+            case S_POW: r = std::pow(x, s); break;   // cpu.rs:1174-1181
             default: r = T(0);
         }
         o[i] = r;
@@ -259,6 +261,8 @@ void unary(int op, const T* a, T* o, i64 n) {
             case U_TANH: r = tanh_ref(x); break;
             case U_ABS: r = std::fabs(x); break;
             case U_RECIP: r = T(1) / x; break;
+            case U_SIGN: r = x > T(0) ? T(1) : (x < T(0) ? -T(1) : T(0)); break;  // cpu.rs:949-965
+            case U_NOT: r = x == T(0) ? T(1) : T(0); break;                       // cpu.rs:920-931
             default: r = T(0);
         }
         o[i] = r;
@@ -375,6 +379,86 @@ void softmax_axis(const T* x, i64 outer, i64 axis, i64 inner, T* out) {
             }
 }
 
+template <typename T>
+void reduce_min_axis(const T* x, i64 outer, i64 axis, i64 inner, T* out, i64* idx) {  // cpu.rs:1240-1252
+    const T highest = std::numeric_limits<T>::max();  // FerroxN::max_value
+    for (i64 o = 0; o < outer; ++o)
+        for (i64 i = 0; i < inner; ++i) {
+            T acc = highest;
+            i64 am = 0;
+            for (i64 a = 0; a < axis; ++a) {
+                const T v = x[(o * axis + a) * inner + i];
+                if (v < acc) { acc = v; am = a; }
+            }
+            out[o * inner + i] = acc;
+            if (idx) idx[o * inner + i] = am;
+        }
+}
+
+template <typename T>
+void in_range(const T* a, T lo, T hi, T* o, i64 n) {  // cpu.rs:933-947
+    for (i64 i = 0; i < n; ++i) o[i] = (a[i] >= lo && a[i] <= hi) ? T(1) : T(0);
+}
+
+// pool2d_impl, extensions/pooling.rs:154-229 with MaxPoolOp / AvgPoolOp (:25-64); separate window / stride / padding
+// per dimension so that the 1-D variant (:231-287) is H = 1 with a 1 x k window.
+template <typename T>
+void pool2d(const T* in, T* out, i64 N, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, int is_max) {
+    const i64 oh = (H + 2 * ph - kh) / sh + 1, ow = (W + 2 * pw - kw) / sw + 1;
+    for (i64 b = 0; b < N; ++b)
+        for (i64 c = 0; c < C; ++c)
+            for (i64 oy = 0; oy < oh; ++oy)
+                for (i64 ox = 0; ox < ow; ++ox) {
+                    const i64 hs = oy * sh - ph, ws = ox * sw - pw;
+                    T acc = is_max ? std::numeric_limits<T>::lowest() : T(0);
+                    int count = 0;
+                    for (i64 ky = 0; ky < kh; ++ky)
+                        for (i64 kx = 0; kx < kw; ++kx) {
+                            const i64 y = hs + ky, x = ws + kx;
+                            if (y >= 0 && y < H && x >= 0 && x < W) {
+                                const T v = in[((b * C + c) * H + y) * W + x];
+                                if (is_max) { if (v > acc) acc = v; }
+                                else { acc += v; count += 1; }
+                            }
+                        }
+                    if (!is_max) acc = count > 0 ? acc / (T)count : T(0);
+                    out[((b * C + c) * oh + oy) * ow + ox] = acc;
+                }
+}
+
+// unpool2d_impl, extensions/pooling.rs:339-418 with MaxUnpoolOp / AvgUnpoolOp (:88-148): for every input position a
+// scan over ALL output windows in (out_h, out_w) order, as the reference does.
+template <typename T>
+void unpool2d(const T* gout, const T* in, const T* pooled, T* gin, i64 N, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i64 sw,
+              i64 ph, i64 pw, int is_max) {
+    const i64 oh = (H + 2 * ph - kh) / sh + 1, ow = (W + 2 * pw - kw) / sw + 1;
+    const float kernel_area = (float)(kh * kw);
+    const T eps = (T)1e-8f;                      // FerroxN::from_f32(1e-8)
+    const T scale = (T)(1.0f / kernel_area);     // FerroxN::from_f32(1.0 / kernel_area)
+    for (i64 b = 0; b < N; ++b)
+        for (i64 c = 0; c < C; ++c)
+            for (i64 y = 0; y < H; ++y)
+                for (i64 x = 0; x < W; ++x) {
+                    const i64 ii = ((b * C + c) * H + y) * W + x;
+                    T acc = T(0);
+                    for (i64 oy = 0; oy < oh; ++oy)
+                        for (i64 ox = 0; ox < ow; ++ox) {
+                            const i64 hs = oy * sh - ph, ws = ox * sw - pw;
+                            if (y >= hs && y < hs + kh && x >= ws && x < ws + kw) {
+                                const i64 oi = ((b * C + c) * oh + oy) * ow + ox;
+                                if (is_max) {
+                                    const T o = in[ii], pv = pooled[oi];
+                                    const T diff = o > pv ? o - pv : pv - o;
+                                    if (diff < eps) acc += gout[oi];
+                                } else {
+                                    acc += gout[oi] * scale;
+                                }
+                            }
+                        }
+                    gin[ii] = acc;
+                }
+}
+
 // materialize a strided/broadcast view into contiguous memory: cpu.rs:510-562 (broadcast_to, transpose -> to_owned)
 template <typename T>
 void materialize(const T* x, T* out, const i64* shape, const i64* strides, int ndim, i64 n) {
@@ -441,6 +525,18 @@ void materialize(const T* x, T* out, const i64* shape, const i64* strides, int n
     }                                                                                                                  \
     extern "C" void orc_reduce_max_##S(const T* x, i64 outer, i64 axis, i64 inner, T* out, i64* idx) {                \
         reduce_max_axis<T>(x, outer, axis, inner, out, idx);                                                           \
+    }                                                                                                                  \
+    extern "C" void orc_reduce_min_##S(const T* x, i64 outer, i64 axis, i64 inner, T* out, i64* idx) {                \
+        reduce_min_axis<T>(x, outer, axis, inner, out, idx);                                                           \
+    }                                                                                                                  \
+    extern "C" void orc_in_range_##S(const T* a, T lo, T hi, T* o, i64 n) { in_range<T>(a, lo, hi, o, n); }           \
+    extern "C" void orc_pool2d_##S(const T* in, T* out, i64 N, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i64 sw,   \
+                                   i64 ph, i64 pw, int is_max) {                                                       \
+        pool2d<T>(in, out, N, C, H, W, kh, kw, sh, sw, ph, pw, is_max);                                               \
+    }                                                                                                                  \
+    extern "C" void orc_unpool2d_##S(const T* gout, const T* in, const T* pooled, T* gin, i64 N, i64 C, i64 H, i64 W, \
+                                     i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, int is_max) {                     \
+        unpool2d<T>(gout, in, pooled, gin, N, C, H, W, kh, kw, sh, sw, ph, pw, is_max);                               \
     }                                                                                                                  \
     extern "C" void orc_softmax_axis_##S(const T* x, i64 outer, i64 axis, i64 inner, T* out) {                        \
         softmax_axis<T>(x, outer, axis, inner, out);                                                                   \

@@ -98,6 +98,9 @@ class Sequential:
                 _, cin, cout, k, s, p = parts
                 self.layers.append(("conv", pi, pi + 1, (int(s), int(s)), (int(p), int(p))))
                 pi += 2
+            elif kind in ("maxpool", "avgpool"):
+                _, k, st, p = parts
+                self.layers.append((kind, (int(k), int(k)), (int(st), int(st)), (int(p), int(p))))
             elif kind in ("relu", "flatten"):
                 self.layers.append((kind,))
             else:
@@ -122,6 +125,10 @@ class Sequential:
                 y = orc.conv2d_fwd(h, w, layer[3], layer[4])
                 out = orc.binary("add", y, _bcast(b, y.shape))
                 tape.append(("conv", layer, h))
+                h = out
+            elif kind in ("maxpool", "avgpool"):
+                out = orc.pool2d(h, layer[1], layer[2], layer[3], kind == "maxpool")      # ops/pooling.rs:38-48, 150-162
+                tape.append((kind, layer, h, out))
                 h = out
             elif kind == "relu":
                 tape.append(("relu", h))
@@ -154,6 +161,9 @@ class Sequential:
                 gi = orc.conv2d_dgrad(g, w, h.shape, layer[3], layer[4], self.conv_mode)
                 grads[layer[1]] = orc.conv2d_wgrad(h, g, w.shape, layer[3], layer[4], self.conv_mode)
                 g = gi
+            elif kind in ("maxpool", "avgpool"):
+                _, layer, h, out = rec
+                g = orc.unpool2d(g, h, out, layer[1], layer[2], layer[3], kind == "maxpool")
             elif kind == "relu":
                 g = orc.binary("mul", g, orc.scalar("greater_scalar", rec[1], dt(0)))
             else:

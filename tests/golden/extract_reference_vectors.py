@@ -54,7 +54,11 @@ def main(ref):
                     ("matmul", "matrix_multiply"), ("sum_all", "sum_all_elements"), ("sum_axis0", "sum_along_axes"),
                     ("mean_all", "mean_all_elements"), ("mean_axis1", "mean_along_axes"), ("max_all", "max_all_elements"),
                     ("max_axis0", "max_along_axes"), ("softmax_axis1", "softmax_last_axis"),
-                    ("softmax_axis0", "softmax_first_axis"), ("neg", "neg_function")]:
+                    ("softmax_axis0", "softmax_first_axis"), ("neg", "neg_function"), ("min_all", "min_all_elements"),
+                    ("min_axis1", "min_along_axes"), ("max_elementwise", "max_elementwise"),
+                    ("min_elementwise", "min_elementwise"), ("reciprocal", "reciprocal_operation"),
+                    ("maxpool1d", "test_maxpool1d_forward"), ("avgpool1d", "test_avgpool1d_forward"),
+                    ("maxpool2d", "test_maxpool2d_forward"), ("avgpool2d", "test_avgpool2d_forward")]:
         arrs = simple(fn, 1)
         out[key] = {"source": f"src/ops/mod.rs fn {fn}", "arrays": arrs}
 

@@ -8,6 +8,7 @@ pytestmark = pytest.mark.gpu
 
 MLP_SMALL = "linear 20 16; relu; linear 16 12; relu; linear 12 5"
 CNN_SMALL = "conv 3 4 3 1 1; relu; conv 4 6 3 2 1; relu; flatten; linear 96 5"
+CNN_POOL = "conv 3 8 3 1 1; relu; maxpool 2 2 0; conv 8 8 3 1 1; relu; avgpool 3 2 1; flatten; linear 128 5"
 MLP_C2 = "linear 784 256; relu; linear 256 128; relu; linear 128 10"
 CNN_C5 = "conv 3 32 3 1 1; relu; conv 32 64 3 2 1; relu; flatten; linear 16384 10"
 TOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float64): 1e-12}
@@ -47,6 +48,7 @@ def close(got, ref, tol):
 CASES = [
     ("mlp_small", MLP_SMALL, (9, 20), 5, "sgd 0.01", 3),
     ("cnn_small", CNN_SMALL, (5, 3, 8, 8), 5, "adam 0.001 0.9 0.999 1e-08 0", 3),
+    ("cnn_pool", CNN_POOL, (4, 3, 16, 16), 5, "sgd 0.05", 2),
     ("mlp_c2", MLP_C2, (256, 784), 10, "sgd 0.01", 1),
     ("cnn_c5", CNN_C5, (256, 3, 32, 32), 10, "adam 0.001 0.9 0.999 1e-08 0", 1),
 ]

@@ -118,3 +118,80 @@ def test_materialize_and_clamp_and_scalar():
     assert orc.clamp(x, 1e-8, 1 - 1e-8).tolist() == [np.float32(1e-8), np.float32(1e-8), 0.5, 1.0, 1.0]  # f32: 1-1e-8 == 1
     assert orc.scalar("greater_equal_scalar", x, 0.5).tolist() == [0, 0, 1, 1, 1]
     assert orc.binary("equal", x, x[::-1].copy()).tolist() == [0, 0, 1, 0, 0]
+
+
+# ---- oracle functions added for the rest of the storage trait: pinned by the reference's vectors, numpy and torch ----
+def test_min_minmax_elementwise_reciprocal_reference_vectors(golden):
+    import oracle as orc
+    a = np.array(golden["min_all"]["arrays"][0], np.float32).reshape(2, 2)
+    assert orc.reduce("min", a).item() == golden["min_all"]["arrays"][1][0]
+    assert orc.reduce("min", a, [1]).tolist() == golden["min_axis1"]["arrays"][1]
+    for key, op in (("max_elementwise", "max"), ("min_elementwise", "min")):
+        x, y, want = (np.array(v, np.float32) for v in golden[key]["arrays"])
+        assert np.array_equal(orc.binary(op, x, y), want)
+    x, want = (np.array(v, np.float32) for v in golden["reciprocal"]["arrays"])
+    assert np.array_equal(orc.unary("reciprocal", x), want)
+
+
+def test_pooling_reference_vectors(golden):
+    import oracle as orc
+    for key, is_max in (("maxpool1d", True), ("avgpool1d", False)):
+        x, want = (np.array(v, np.float32) for v in golden[key]["arrays"])
+        got = orc.pool2d(x.reshape(1, 1, 1, 6), (1, 2), (1, 2), (0, 0), is_max)  # [N,C,L] as H = 1
+        assert np.array_equal(got.ravel(), want)
+    for key, is_max in (("maxpool2d", True), ("avgpool2d", False)):
+        x, want = (np.array(v, np.float32) for v in golden[key]["arrays"])
+        assert np.array_equal(orc.pool2d(x.reshape(1, 1, 4, 4), (2, 2), (2, 2), (0, 0), is_max).ravel(), want)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_pooling_vs_torch(dtype):
+    """torch as the independent routine: max_pool2d (pads with -inf: same winners), avg_pool2d with
+    count_include_pad=False for the forward (the reference divides by the in-bounds count) and with
+    count_include_pad=True for the backward (the reference's gradient scale is 1/kernel_area for every window)."""
+    import oracle as orc
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(30)
+    for (N, Cc, H, W, k, s, p) in [(2, 3, 8, 8, 2, 2, 0), (1, 2, 7, 9, 3, 2, 1), (2, 1, 6, 5, 3, 1, 1), (1, 1, 5, 5, 2, 1, 0), (1, 2, 9, 9, 3, 3, 1)]:
+        x = rng.standard_normal((N, Cc, H, W)).astype(dtype)  # no ties
+        tx = torch.from_numpy(x).double().requires_grad_(True)
+        mp = F.max_pool2d(tx, k, s, p)
+        g = rng.standard_normal(tuple(mp.shape)).astype(dtype)
+        mp.backward(torch.from_numpy(g).double())
+        omp = orc.pool2d(x, (k, k), (s, s), (p, p), True)
+        assert np.array_equal(omp, mp.detach().numpy().astype(dtype))
+        got = orc.unpool2d(g, x, omp, (k, k), (s, s), (p, p), True)
+        assert np.allclose(got, tx.grad.numpy(), rtol=1e-6 if dtype == np.float32 else 1e-14, atol=1e-6 if dtype == np.float32 else 1e-14)
+        ap = F.avg_pool2d(torch.from_numpy(x).double(), k, s, p, count_include_pad=False).numpy()
+        oap = orc.pool2d(x, (k, k), (s, s), (p, p), False)
+        assert np.allclose(oap, ap, rtol=1e-5 if dtype == np.float32 else 1e-13, atol=1e-6 if dtype == np.float32 else 1e-14)
+        tx2 = torch.from_numpy(x).double().requires_grad_(True)
+        F.avg_pool2d(tx2, k, s, p, count_include_pad=True).backward(torch.from_numpy(g).double())
+        got = orc.unpool2d(g, x, oap, (k, k), (s, s), (p, p), False)
+        # the reference rounds 1/kernel_area to f32 first, for f64 tensors too (pooling.rs:138): 1/9 is then off by 3e-9 relative
+        assert np.allclose(got, tx2.grad.numpy(), rtol=1e-5 if dtype == np.float32 else 1e-7, atol=1e-6 if dtype == np.float32 else 1e-8)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_sign_not_in_range_pow_min_softmax_all_vs_numpy(dtype):
+    import oracle as orc
+    rng = np.random.default_rng(31)
+    a = rng.standard_normal(1000).astype(dtype)
+    a[::9] = 0
+    assert np.array_equal(orc.unary("sign", a), np.sign(a))
+    assert np.array_equal(orc.unary("logical_not", a), (a == 0).astype(dtype))
+    assert np.array_equal(orc.in_range(a, -0.5, 0.25), ((a >= dtype(-0.5)) & (a <= dtype(0.25))).astype(dtype))
+    b = np.abs(a) + dtype(0.1)
+    e = rng.uniform(-2, 3, 1000).astype(dtype)
+    tol = 1e-6 if dtype == np.float32 else 1e-14
+    assert np.allclose(orc.binary("pow", b, e), np.power(b.astype(np.float64), e.astype(np.float64)), rtol=tol)
+    assert np.allclose(orc.scalar("pow_scalar", b, 2.5), np.power(b.astype(np.float64), 2.5), rtol=tol)
+    m = rng.standard_normal((6, 7, 5)).astype(dtype)
+    m[2, 3, 1] = m[2, 5, 1] = -9.0  # tie: the first index wins
+    for ax in range(3):
+        v, i = orc.reduce_axis("min", m, ax, want_idx=True)
+        assert np.array_equal(v, m.min(axis=ax)) and np.array_equal(i, m.argmin(axis=ax))
+    x = (rng.standard_normal((3, 40)) * 4).astype(dtype)
+    e64 = np.exp(x.astype(np.float64) - x.max())
+    assert np.allclose(orc.softmax_all(x), e64 / e64.sum(), rtol=1e-5 if dtype == np.float32 else 1e-13)
