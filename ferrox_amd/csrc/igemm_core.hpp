@@ -33,7 +33,7 @@ typedef double f64x4 __attribute__((ext_vector_type(4)));
 struct FastDiv {
     uint32_t d, m, s;
     FastDiv() : d(1), m(1), s(0) {}
-    explicit FastDiv(uint32_t d_) : d(d_) {
+    explicit FastDiv(uint32_t d_) : d(d_ ? d_ : 1) {  // a zero divisor (an empty extent that is never indexed) acts as 1
         s = 0;
         while ((1ull << s) < d) ++s;
         m = (uint32_t)((((1ull << 32) * ((1ull << s) - d)) / d) + 1);

@@ -470,6 +470,43 @@ def test_conv2d_strided_dgrad_vs_torch_and_oracle(ctx, orc, dtype):
         assert rel_err(dx, orc.conv2d_dgrad(g, w, (B, Cin, H, W), st, pd, 0)) <= tol * 8, case
 
 
+@pytest.mark.parametrize("seed", [61, 62, 63, 64])
+def test_conv2d_random_shapes_all_paths_vs_torch(ctx, seed):
+    """Seeded random 3x3 / 1x1 / 5x5 shapes biased towards the dispatch boundaries of the conv kernels (channel counts
+    around multiples of 8 / 16 / 32 / 64, widths around 64 and multiples of 4, strides 1-3, paddings 0-2): forward,
+    data gradient and weight gradient against torch in float64."""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(seed)
+    tol = TOL[np.dtype(np.float32)] * 8
+    chans = [1, 3, 4, 8, 16, 24, 32, 40, 64, 65, 72, 96, 128, 136]
+    widths = [4, 6, 8, 12, 14, 16, 20, 28, 30, 32, 36, 56, 60, 64, 66, 68]
+    for it in range(70):
+        Cin, Cout = int(rng.choice(chans)), int(rng.choice(chans))
+        k = int(rng.choice([3, 3, 3, 3, 1, 5]))
+        sh, sw = int(rng.choice([1, 1, 1, 2, 3])), int(rng.choice([1, 1, 1, 2, 3]))
+        ph, pw = int(rng.integers(0, 3)), int(rng.integers(0, 3))
+        W = int(rng.choice(widths))
+        H = int(rng.choice([1, 2, 3, 5, 8, 9, 14, 28])) if rng.random() < 0.7 else W
+        B = int(rng.choice([1, 2, 3, 5]))
+        if H + 2 * ph < k or W + 2 * pw < k or B * Cin * H * W > 1_500_000 or B * Cout * H * W > 3_000_000:
+            continue
+        case = (it, B, Cin, H, W, Cout, k, (sh, sw), (ph, pw))
+        x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(np.float32)
+        w = (rng.standard_normal((Cout, Cin, k, k)) * np.sqrt(2.0 / (Cin * k * k))).astype(np.float32)
+        tx = torch.from_numpy(x).double().requires_grad_(True)
+        tw = torch.from_numpy(w).double().requires_grad_(True)
+        ty = F.conv2d(tx, tw, stride=(sh, sw), padding=(ph, pw))
+        g = rng.standard_normal(tuple(ty.shape)).astype(np.float32)
+        ty.backward(torch.from_numpy(g).double())
+        dx_, dw_, dg_ = ctx.upload(x), ctx.upload(w), ctx.upload(g)
+        y = ctx.conv2d_fwd(dx_, dw_, (sh, sw), (ph, pw)).numpy()
+        ay = F.conv2d(tx.detach().abs(), tw.detach().abs(), stride=(sh, sw), padding=(ph, pw)).max().item()
+        assert np.abs(y - ty.detach().numpy()).max() <= tol * max(ay, 1e-30), ("fwd", case)
+        assert rel_err(ctx.conv2d_dgrad(dg_, dw_, x.shape, (sh, sw), (ph, pw), 0).numpy(), tx.grad.numpy()) <= tol, ("dgrad", case)
+        assert rel_err(ctx.conv2d_wgrad(dx_, dg_, w.shape, (sh, sw), (ph, pw), 0).numpy(), tw.grad.numpy()) <= tol, ("wgrad", case)
+
+
 def test_conv2d_misaligned_tensors_match_aligned(ctx):
     """Tensors that are only 4-byte aligned (a view into a larger buffer) cannot use the 16-byte loads of the
     patch kernels; the library must fall back and give the implicit-GEMM result, not fault or misread."""
