@@ -470,15 +470,15 @@ def test_conv2d_strided_dgrad_vs_torch_and_oracle(ctx, orc, dtype):
         assert rel_err(dx, orc.conv2d_dgrad(g, w, (B, Cin, H, W), st, pd, 0)) <= tol * 8, case
 
 
-@pytest.mark.parametrize("seed", [61, 62, 63, 64])
-def test_conv2d_random_shapes_all_paths_vs_torch(ctx, seed):
+@pytest.mark.parametrize("seed,dtype", [(61, np.float32), (62, np.float32), (63, np.float32), (64, np.float32), (65, np.float64), (66, np.float64)])
+def test_conv2d_random_shapes_all_paths_vs_torch(ctx, seed, dtype):
     """Seeded random 3x3 / 1x1 / 5x5 shapes biased towards the dispatch boundaries of the conv kernels (channel counts
     around multiples of 8 / 16 / 32 / 64, widths around 64 and multiples of 4, strides 1-3, paddings 0-2): forward,
     data gradient and weight gradient against torch in float64."""
     import torch
     import torch.nn.functional as F
     rng = np.random.default_rng(seed)
-    tol = TOL[np.dtype(np.float32)] * 8
+    tol = TOL[np.dtype(dtype)] * 8
     chans = [1, 3, 4, 8, 16, 24, 32, 40, 64, 65, 72, 96, 128, 136]
     widths = [4, 6, 8, 12, 14, 16, 20, 28, 30, 32, 36, 56, 60, 64, 66, 68]
     for it in range(70):
@@ -492,12 +492,12 @@ def test_conv2d_random_shapes_all_paths_vs_torch(ctx, seed):
         if H + 2 * ph < k or W + 2 * pw < k or B * Cin * H * W > 1_500_000 or B * Cout * H * W > 3_000_000:
             continue
         case = (it, B, Cin, H, W, Cout, k, (sh, sw), (ph, pw))
-        x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(np.float32)
-        w = (rng.standard_normal((Cout, Cin, k, k)) * np.sqrt(2.0 / (Cin * k * k))).astype(np.float32)
+        x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(dtype)
+        w = (rng.standard_normal((Cout, Cin, k, k)) * np.sqrt(2.0 / (Cin * k * k))).astype(dtype)
         tx = torch.from_numpy(x).double().requires_grad_(True)
         tw = torch.from_numpy(w).double().requires_grad_(True)
         ty = F.conv2d(tx, tw, stride=(sh, sw), padding=(ph, pw))
-        g = rng.standard_normal(tuple(ty.shape)).astype(np.float32)
+        g = rng.standard_normal(tuple(ty.shape)).astype(dtype)
         ty.backward(torch.from_numpy(g).double())
         dx_, dw_, dg_ = ctx.upload(x), ctx.upload(w), ctx.upload(g)
         y = ctx.conv2d_fwd(dx_, dw_, (sh, sw), (ph, pw)).numpy()
