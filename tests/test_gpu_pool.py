@@ -153,3 +153,52 @@ def test_reused_block_is_not_zeroed_but_usable():
         assert np.array_equal(b.numpy(), np.arange(1000, dtype=np.float32))  # dirty on purpose (context.rs:72-73)
         c = ctx.fill((1000,), 3.0)
         assert np.all(c.numpy() == 3.0)
+
+
+def test_entry_points_are_thread_safe():
+    """Ferrox's own tests run on parallel threads against one process-wide backend (manager.rs:343-353): calls from
+    several threads into one context - pool traffic plus kernels that share the library scratch (split-K partial
+    sums, weight images, reduction partials) - must give the single-threaded results bit for bit."""
+    import threading
+    from ferrox_amd import capi
+    ctx = capi.Context(0)
+    try:
+        rng = np.random.default_rng(90)
+        x = rng.uniform(-1, 1, (4, 32, 12, 56)).astype(np.float32)
+        w = (rng.standard_normal((96, 32, 3, 3)) * 0.06).astype(np.float32)
+        g = rng.standard_normal((4, 96, 12, 56)).astype(np.float32)
+        m = rng.standard_normal((512, 2048)).astype(np.float32)
+        dx_, dw_, dg_, dm_ = ctx.upload(x), ctx.upload(w), ctx.upload(g), ctx.upload(m)
+
+        def work():
+            y = ctx.conv2d_fwd(dx_, dw_, (1, 1), (1, 1)).numpy()
+            dw = ctx.conv2d_wgrad(dx_, dg_, w.shape, (1, 1), (1, 1)).numpy()
+            dxx = ctx.conv2d_dgrad(dg_, dw_, x.shape, (1, 1), (1, 1)).numpy()
+            s0 = ctx.reduce("sum", dm_, 0).numpy()
+            mx = ctx.reduce("max", dm_, 1).numpy()
+            bg = ctx.bias_grad(dg_, 4, 96, 12 * 56).numpy()
+            return y, dw, dxx, s0, mx, bg
+
+        want = work()
+        results, errors = {}, []
+
+        def runner(i):
+            try:
+                for _ in range(6):
+                    results[i] = work()
+            except Exception as e:  # noqa: BLE001
+                errors.append(repr(e))
+
+        threads = [threading.Thread(target=runner, args=(i,)) for i in range(6)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        assert not errors, errors
+        for i, got in results.items():
+            for a, b in zip(got, want):
+                assert np.array_equal(a, b), i
+        st = ctx.pool_stats(np.float32)
+        assert st["active_allocations"] >= 4
+    finally:
+        ctx.close()
