@@ -90,7 +90,16 @@ def bench_conv(ctx, steps, warmup, dtype=np.float32, B=None):
     for name, fn in passes.items():
         ms = time_stream(ctx, fn, steps, warmup)
         per_pass[name] = {"ms": ms, "tflops": flop / ms / 1e9}
-    return {"flop_per_pass": flop, "per_pass": per_pass, "ms_per_step": wall_ms, "tflops": 3 * flop / wall_ms / 1e9}
+    res = {"flop_per_pass": flop, "per_pass": per_pass, "ms_per_step": wall_ms, "tflops": 3 * flop / wall_ms / 1e9}
+    if dtype == np.float32 and B == C3["B"]:
+        # forward + bias + ReLU: in the conv kernel's store (one pass over y) vs conv, then an in-place bias/ReLU pass
+        from ferrox_amd import capi
+        bias = ctx.normal((Cout,), 34, 0.0, 0.1, dtype)
+        dims = (B, Cin, H, W, Cout, k, k, s, s, p, p)
+        fused = lambda: capi.check(capi.lib.fx_conv2d_fwd_bias_act_f32(ctx.h, x.ptr, w.ptr, bias.ptr, y.ptr, *dims, 1, None, 0))  # noqa: E731
+        two = lambda: (ctx.conv2d_fwd(x, w, (s, s), (p, p), out=y), ctx.bias_act(y, bias, B, Cout, H * W, 1))  # noqa: E731
+        res["fwd_bias_relu"] = {"epilogue_ms": time_stream(ctx, fused, steps, warmup), "two_call_ms": time_stream(ctx, two, steps, warmup)}
+    return res
 
 
 def bench_bandwidth(ctx, iters=20, warmup=3):
@@ -362,6 +371,7 @@ def main():
                      "algorithmic_bytes": 308.6e6, "avg_launch_ms": dom["ms"]},
         "conv_passes": {k: {"ms": v["ms"], "tflops": v["tflops"], "frac_mfma_f32": v["tflops"] / PEAK_F32_MFMA_TFLOPS}
                         for k, v in conv["per_pass"].items()},
+        "conv_fwd_bias_relu": conv.get("fwd_bias_relu"),
     }
     if not args.skip_also:
         c64 = bench_conv(ctx, max(3, args.steps // 4), 1, np.float64, B=64)

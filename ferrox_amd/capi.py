@@ -126,6 +126,8 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_conv2d_dgrad_{_s}", _vp, _vp, _vp, _vp, *_CONV_INTS, _int, _vp, _i64)
     _sig(f"fx_conv2d_wgrad_{_s}", _vp, _vp, _vp, _vp, *_CONV_INTS, _int, _vp, _i64)
     _sig(f"fx_bias_act_{_s}", _vp, _vp, _vp, _i64, _i64, _i64, _int)
+    _sig(f"fx_conv2d_fwd_bias_act_{_s}", _vp, _vp, _vp, _vp, _vp, *_CONV_INTS, _int, _vp, _i64)
+    _sig(f"fx_gemm_bias_act_{_s}", _vp, _int, _int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _int)
     _sig(f"fx_bias_grad_{_s}", _vp, _vp, _vp, _i64, _i64, _i64)
     _sig(f"fx_softmax_ce_fwd_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64)
     _sig(f"fx_softmax_ce_bwd_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64)

@@ -103,13 +103,13 @@ inline int pick_tile(fx_ctx* c, i64 M, i64 N) {
 constexpr int CONV_BK = 16;  // slab depth of every conv tile; the (ky,kx)-outer K order needs channels % CONV_BK == 0
 
 template <typename T, class Cfg, bool FAST>
-int fwd_tile(fx_ctx* c, const T* x, const T* w, T* y, const Dims& d) {
+int fwd_tile(fx_ctx* c, const T* x, const T* w, T* y, const Dims& d, const T* bias, int relu) {
     static_assert(Cfg::BK == CONV_BK || !FAST || Cfg::BK == 32, "unexpected slab depth");
     const i64 M = d.Cout, N = d.B * d.oh * d.ow, K = d.Cin * d.kh * d.kw;
     const ConvShape s = make_shape(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
     MatLoader<T, true> al{w, K, (int)M};
     ConvFwdB<T, FAST> bl{x, s, (int)N};
-    NchwStore<T> ep{y, (int)d.Cout, (int)(d.oh * d.ow), (int)N, s.div_L};
+    NchwStore<T> ep{y, (int)d.Cout, (int)(d.oh * d.ow), (int)N, s.div_L, bias, relu};
     const int kps = (int)(fx::ceil_div(K, Cfg::BK) * Cfg::BK);
     return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
 }
@@ -142,7 +142,7 @@ i64 fwd_ws_bytes(fx_ctx* c, const Dims& d) {
 
 template <typename T>
 int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw,
-             i64 ph, i64 pw, void* ws, i64 ws_bytes) {
+             i64 ph, i64 pw, void* ws, i64 ws_bytes, const T* bias = nullptr, int relu = 0) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(x && w && y, "fx_conv2d_fwd: null pointer");
     Dims d;
@@ -156,7 +156,7 @@ int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64
         if (pl.ok && aligned16(x, ws)) {
             float* wimg = (float*)(ws ? ws : c->get_scratch(need));
             if (!wimg) return FX_ERR_OOM;
-            return cpk::run(c, pl, x, w, y, wimg, 0, Cout, Cin, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw);
+            return cpk::run(c, pl, x, w, y, wimg, 0, Cout, Cin, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw, bias, relu);
         }
     }
     if (d.Cin % CONV_BK == 0) {
@@ -164,17 +164,17 @@ int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64
         if (!wp) return FX_ERR_OOM;
         if (int rc = permute_weights<T>(c, w, wp, d, 0)) return rc;
         switch (pick_tile(c, Cout, B * d.oh * d.ow)) {
-            case 128: return fwd_tile<T, TileM128, true>(c, x, wp, y, d);
-            case 64: return fwd_tile<T, TileM64, true>(c, x, wp, y, d);
-            case 32: return fwd_tile<T, TileM32, true>(c, x, wp, y, d);
-            default: return fwd_tile<T, TileSmall, true>(c, x, wp, y, d);
+            case 128: return fwd_tile<T, TileM128, true>(c, x, wp, y, d, bias, relu);
+            case 64: return fwd_tile<T, TileM64, true>(c, x, wp, y, d, bias, relu);
+            case 32: return fwd_tile<T, TileM32, true>(c, x, wp, y, d, bias, relu);
+            default: return fwd_tile<T, TileSmall, true>(c, x, wp, y, d, bias, relu);
         }
     }
     switch (pick_tile(c, Cout, B * d.oh * d.ow)) {
-        case 128: return fwd_tile<T, TileM128, false>(c, x, w, y, d);
-        case 64: return fwd_tile<T, TileM64, false>(c, x, w, y, d);
-        case 32: return fwd_tile<T, TileM32, false>(c, x, w, y, d);
-        default: return fwd_tile<T, TileSmall, false>(c, x, w, y, d);
+        case 128: return fwd_tile<T, TileM128, false>(c, x, w, y, d, bias, relu);
+        case 64: return fwd_tile<T, TileM64, false>(c, x, w, y, d, bias, relu);
+        case 32: return fwd_tile<T, TileM32, false>(c, x, w, y, d, bias, relu);
+        default: return fwd_tile<T, TileSmall, false>(c, x, w, y, d, bias, relu);
     }
 }
 
@@ -482,6 +482,13 @@ extern "C" int64_t fx_conv2d_workspace_bytes(int kind, int dtype, int mode, int6
                                      int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,  \
                                      void* ws, int64_t ws_bytes) {                                                     \
         return conv_fwd<T>(c, x, w, y, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, ws, ws_bytes);                      \
+    }                                                                                                                  \
+    extern "C" int fx_conv2d_fwd_bias_act_##S(fx_ctx* c, const T* x, const T* w, const T* bias, T* y, int64_t B, int64_t Cin,  \
+                                              int64_t H, int64_t W, int64_t Cout, int64_t kh, int64_t kw, int64_t sh,     \
+                                              int64_t sw, int64_t ph, int64_t pw, int act, void* ws, int64_t ws_bytes) { \
+        FX_REQUIRE(bias != nullptr, "fx_conv2d_fwd_bias_act: null bias");                                              \
+        FX_REQUIRE(act == 0 || act == 1, "fx_conv2d_fwd_bias_act: act must be 0 (none) or 1 (relu)");                  \
+        return conv_fwd<T>(c, x, w, y, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, ws, ws_bytes, bias, act);           \
     }                                                                                                                  \
     extern "C" int fx_conv2d_dgrad_##S(fx_ctx* c, const T* g, const T* w, T* dx, int64_t B, int64_t Cin, int64_t H, int64_t W, \
                                        int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,   \

@@ -31,6 +31,8 @@ struct Params {
     const float* x;
     const float* wimg;
     float* y;
+    const float* bias;  // optional, per output channel; with relu != 0 the sum is clamped at 0 afterwards
+    int relu;
     int C, H, W, M, OH, OW, sh, sw, ph, pw;
     int PR, PW, PLANE, L, tpi, nchunks;
     FastDiv div_tpi, div_ow;
@@ -57,7 +59,7 @@ __global__ __launch_bounds__(256) void wimg_kernel(const float* __restrict__ w, 
     out[i] = v;
 }
 
-template <int WM, int TN>
+template <int WM, int TN, bool BIAS>
 __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
     constexpr int BM = 32 * WM, WN = 4 / WM, NPIX = 32 * TN * WN;
     constexpr int WIMG = BM * WPITCH;             // floats in one weight image
@@ -181,6 +183,12 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
     }
 
     float* out = p.y + (i64)b * p.M * p.L;
+    float bv[16];  // bias of the 16 output channels this lane stores: 16 independent loads (row clamped, no branches)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const int m = m0 + wm * 32 + igemm::Mfma<float>::row(e, lane);
+        bv[e] = BIAS ? p.bias[m < p.M ? m : p.M - 1] : 0.f;
+    }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int pi = wpix0 + j * 32 + l32;
@@ -188,7 +196,14 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int m = m0 + wm * 32 + igemm::Mfma<float>::row(e, lane);
-                if (m < p.M) out[(i64)m * p.L + pi] = acc[j][e];
+                if (m < p.M) {
+                    float v = acc[j][e];
+                    if (BIAS) {
+                        v = v + bv[e];
+                        if (p.relu) v = v > 0.f ? v : 0.f;
+                    }
+                    out[(i64)m * p.L + pi] = v;
+                }
             }
         }
     }
@@ -243,13 +258,13 @@ inline i64 workspace_bytes(const Plan& pl, i64 M) { return fx::ceil_div(M, (i64)
 
 // w is the reference's [Cout][Cin][3][3] filter; flip selects the data-gradient image.
 inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float* y, float* wimg, int flip, i64 Cout, i64 Cin, i64 B,
-               i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw) {
+               i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw, const float* bias = nullptr, int relu = 0) {
     const i64 n = (i64)pl.mtiles * pl.nchunks * pl.wimg();
     wimg_kernel<<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(w, wimg, (int)Cout, (int)Cin, (int)M, pl.bm(),
                                                                                   pl.nchunks, flip, n);
     FX_LAUNCH_CHECK();
     Params p;
-    p.x = x; p.wimg = wimg; p.y = y;
+    p.x = x; p.wimg = wimg; p.y = y; p.bias = bias; p.relu = relu;
     p.C = (int)C; p.H = (int)H; p.W = (int)W; p.M = (int)M; p.OH = (int)OH; p.OW = (int)OW;
     p.sh = (int)sh; p.sw = (int)sw; p.ph = (int)ph; p.pw = (int)pw;
     p.PR = pl.PR; p.PW = pl.PW; p.PLANE = pl.PLANE; p.L = (int)(OH * OW); p.tpi = pl.tpi; p.nchunks = pl.nchunks;
@@ -258,10 +273,14 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
     const dim3 grid((unsigned)(B * pl.tpi), (unsigned)pl.mtiles);
 #define FX_CPK_LAUNCH(WMV, TNV)                                                                                       \
     case WMV * 16 + TNV: {                                                                                            \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV>,                  \
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
-        FX_HIP_CHECK(attr);                                                                                           \
-        conv_patch_kernel<WMV, TNV><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                                       \
+        static const hipError_t attr0 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, false>,          \
+                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
+        static const hipError_t attr1 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, true>,           \
+                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
+        FX_HIP_CHECK(attr0);                                                                                          \
+        FX_HIP_CHECK(attr1);                                                                                          \
+        if (bias) conv_patch_kernel<WMV, TNV, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                       \
+        else conv_patch_kernel<WMV, TNV, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                           \
         break;                                                                                                        \
     }
     switch (pl.WM * 16 + pl.TN) {

@@ -4,14 +4,20 @@
 // Small or skinny products are split along K into deterministic partial sums (no atomics).
 #include "igemm_core.hpp"
 
+extern "C" int fx_bias_act_f32(fx_ctx*, float*, const float*, int64_t, int64_t, int64_t, int);
+extern "C" int fx_bias_act_f64(fx_ctx*, double*, const double*, int64_t, int64_t, int64_t, int);
+
 namespace {
 using namespace igemm;
+
+int bias_act_t(fx_ctx* c, float* y, const float* b, i64 rows, i64 cols, int act) { return fx_bias_act_f32(c, y, b, rows, cols, 1, act); }
+int bias_act_t(fx_ctx* c, double* y, const double* b, i64 rows, i64 cols, int act) { return fx_bias_act_f64(c, y, b, rows, cols, 1, act); }
 
 typedef Tile<128, 128, 16, 64, 64> TileBig;    // 4 waves, 64x64 each
 typedef Tile<64, 64, 16, 32, 32> TileSmall;    // 4 waves, 32x32 each
 
 template <typename T, class Cfg, bool TA, bool TB>
-int run(fx_ctx* c, i64 M, i64 N, i64 K, const T* A, const T* B, T* C) {
+int run(fx_ctx* c, i64 M, i64 N, i64 K, const T* A, const T* B, T* C, const T* bias, int relu, bool* bias_pending) {
     // A stored [M,K] (k contiguous) unless TA ([K,M], m contiguous); B stored [K,N] (n contiguous) unless TB ([N,K]).
     MatLoader<T, !TA> al{A, TA ? M : K, (int)M};
     MatLoader<T, TB> bl{B, TB ? K : N, (int)N};
@@ -19,9 +25,10 @@ int run(fx_ctx* c, i64 M, i64 N, i64 K, const T* A, const T* B, T* C) {
     int kps = 0;
     const int splits = choose_splits(tiles, K, Cfg::BK, (i64)c->num_cus * 2, &kps);
     if (splits == 1) {
-        MatStore<T> ep{C, N, 0, (int)M, (int)N};
+        MatStore<T> ep{C, N, 0, (int)M, (int)N, bias, relu};  // bias (+ReLU) in the epilogue
         return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
     }
+    *bias_pending = bias != nullptr;  // split-K: the caller adds the bias after the ordered sum
     T* part = (T*)c->get_scratch((i64)splits * M * N * (i64)sizeof(T));
     if (!part) return FX_ERR_OOM;
     MatStore<T> ep{part, N, M * N, (int)M, (int)N};
@@ -30,15 +37,15 @@ int run(fx_ctx* c, i64 M, i64 N, i64 K, const T* A, const T* B, T* C) {
 }
 
 template <typename T, class Cfg>
-int run_trans(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B, T* C) {
-    if (!ta && !tb) return run<T, Cfg, false, false>(c, M, N, K, A, B, C);
-    if (!ta && tb) return run<T, Cfg, false, true>(c, M, N, K, A, B, C);
-    if (ta && !tb) return run<T, Cfg, true, false>(c, M, N, K, A, B, C);
-    return run<T, Cfg, true, true>(c, M, N, K, A, B, C);
+int run_trans(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B, T* C, const T* bias, int relu, bool* pend) {
+    if (!ta && !tb) return run<T, Cfg, false, false>(c, M, N, K, A, B, C, bias, relu, pend);
+    if (!ta && tb) return run<T, Cfg, false, true>(c, M, N, K, A, B, C, bias, relu, pend);
+    if (ta && !tb) return run<T, Cfg, true, false>(c, M, N, K, A, B, C, bias, relu, pend);
+    return run<T, Cfg, true, true>(c, M, N, K, A, B, C, bias, relu, pend);
 }
 
 template <typename T>
-int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B, T* C) {
+int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B, T* C, const T* bias = nullptr, int relu = 0) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(M >= 0 && N >= 0 && K >= 0, "fx_gemm: negative dimension");
     if (M == 0 || N == 0) return FX_OK;
@@ -46,10 +53,18 @@ int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B,
     FX_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "fx_gemm: dimension exceeds 2^31");
     // 32-bit byte offsets inside one 128-row tile of a k-contiguous operand
     FX_REQUIRE(K * 128 * (i64)sizeof(T) < (1ll << 32), "fx_gemm: K = %lld is too large for this build", (long long)K);
-    std::lock_guard<std::mutex> lk(c->launch_mutex);
-    if (K == 0) return launch_zero<T>(c, C, M * N);  // empty sum
-    if (M >= 128 && N >= 128) return run_trans<T, TileBig>(c, ta, tb, M, N, K, A, B, C);
-    return run_trans<T, TileSmall>(c, ta, tb, M, N, K, A, B, C);
+    bool pending = false;
+    {
+        std::lock_guard<std::mutex> lk(c->launch_mutex);
+        int rc;
+        if (K == 0) {  // empty sum
+            rc = launch_zero<T>(c, C, M * N);
+            pending = bias != nullptr;
+        } else if (M >= 128 && N >= 128) rc = run_trans<T, TileBig>(c, ta, tb, M, N, K, A, B, C, bias, relu, &pending);
+        else rc = run_trans<T, TileSmall>(c, ta, tb, M, N, K, A, B, C, bias, relu, &pending);
+        if (rc) return rc;
+    }
+    return pending ? bias_act_t(c, C, bias, M, N, relu) : FX_OK;
 }
 }  // namespace
 
@@ -58,4 +73,17 @@ extern "C" int fx_gemm_f32(fx_ctx* c, int ta, int tb, int64_t M, int64_t N, int6
 }
 extern "C" int fx_gemm_f64(fx_ctx* c, int ta, int tb, int64_t M, int64_t N, int64_t K, const double* A, const double* B, double* C) {
     return gemm<double>(c, ta, tb, M, N, K, A, B, C);
+}
+// C = act(op(A).op(B) + bias[n]): the bias add (and ReLU) ride in the GEMM's store unless the product was split along K.
+extern "C" int fx_gemm_bias_act_f32(fx_ctx* c, int ta, int tb, int64_t M, int64_t N, int64_t K, const float* A, const float* B,
+                                    const float* bias, float* C, int act) {
+    FX_REQUIRE(bias != nullptr, "fx_gemm_bias_act: null bias");
+    FX_REQUIRE(act == 0 || act == 1, "fx_gemm_bias_act: act must be 0 (none) or 1 (relu)");
+    return gemm<float>(c, ta, tb, M, N, K, A, B, C, bias, act);
+}
+extern "C" int fx_gemm_bias_act_f64(fx_ctx* c, int ta, int tb, int64_t M, int64_t N, int64_t K, const double* A, const double* B,
+                                    const double* bias, double* C, int act) {
+    FX_REQUIRE(bias != nullptr, "fx_gemm_bias_act: null bias");
+    FX_REQUIRE(act == 0 || act == 1, "fx_gemm_bias_act: act must be 0 (none) or 1 (relu)");
+    return gemm<double>(c, ta, tb, M, N, K, A, B, C, bias, act);
 }

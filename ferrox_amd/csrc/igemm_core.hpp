@@ -380,22 +380,41 @@ template <typename T> struct ConvWgradB {
 };
 
 // ---- epilogues ---------------------------------------------------------------------------------------------
-// An epilogue maps a column n to a base pointer (col) and stores row m at q[m * row_stride].
-// Row-major matrix (also used for split-K partials: split z goes to p + z*split_stride).
+// An epilogue maps a column n to a base pointer (col) and stores row m at q[m * row_stride]; xform(m, n, v) is
+// applied to every stored value (identity unless a bias vector is attached: v + bias, then ReLU when relu != 0).
+// Row-major matrix (also used for split-K partials: split z goes to p + z*split_stride).  bias is per column n.
 template <typename T> struct MatStore {
     T* p;
     i64 ld, split_stride;
     int M, N;
+    const T* bias = nullptr;
+    int relu = 0;
     __device__ __forceinline__ int rows() const { return M; }
     __device__ __forceinline__ int cols() const { return N; }
     __device__ __forceinline__ i64 row_stride() const { return ld; }
     __device__ __forceinline__ T* col(int n, int split) const { return p + (i64)split * split_stride + n; }
+    __device__ __forceinline__ T xform(int, int n, T v) const {
+        if (bias) {
+            v = v + bias[n];
+            if (relu) v = v > T(0) ? v : T(0);
+        }
+        return v;
+    }
 };
 // NCHW tensor: row m = channel, column n = (b, l) -> p[(b*C + m)*L + l].
-template <typename T> struct NchwStore {
+template <typename T> struct NchwStore {  // bias is per row m (channel)
     T* p;
     int C, L, N;
     FastDiv div_L;
+    const T* bias = nullptr;
+    int relu = 0;
+    __device__ __forceinline__ T xform(int m, int, T v) const {
+        if (bias) {
+            v = v + bias[m];
+            if (relu) v = v > T(0) ? v : T(0);
+        }
+        return v;
+    }
     __device__ __forceinline__ int rows() const { return C; }
     __device__ __forceinline__ int cols() const { return N; }
     __device__ __forceinline__ i64 row_stride() const { return L; }
@@ -411,6 +430,7 @@ template <typename T> struct NchwSubgridStore {
     T* p;
     int C, H, W, Hs, Ws, y0, x0, sy, sx, N;
     FastDiv div_grid, div_ws;
+    __device__ __forceinline__ T xform(int, int, T v) const { return v; }
     __device__ __forceinline__ int rows() const { return C; }
     __device__ __forceinline__ int cols() const { return N; }
     __device__ __forceinline__ i64 row_stride() const { return (i64)H * W; }
@@ -506,11 +526,15 @@ __global__ __launch_bounds__(Cfg::NT) void igemm_kernel(AL al, BL bl, EP ep, int
     if (bm + BM <= M && bn + BN <= N) {  // interior tile: no edge tests
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            T* q = ep.col(bn + wn0 + j * MF::BLK + lcol, split) + (i64)(bm + wm0) * rs;
+            const int n = bn + wn0 + j * MF::BLK + lcol;
+            T* q = ep.col(n, split) + (i64)(bm + wm0) * rs;
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int e = 0; e < MF::NACC; ++e) q[(i64)(i * MF::BLK + MF::row(e, lane)) * rs] = acc[i][j][e];
+                for (int e = 0; e < MF::NACC; ++e) {
+                    const int r = i * MF::BLK + MF::row(e, lane);
+                    q[(i64)r * rs] = ep.xform(bm + wm0 + r, n, acc[i][j][e]);
+                }
         }
     } else {
 #pragma unroll
@@ -523,7 +547,7 @@ __global__ __launch_bounds__(Cfg::NT) void igemm_kernel(AL al, BL bl, EP ep, int
 #pragma unroll
                     for (int e = 0; e < MF::NACC; ++e) {
                         const int m = bm + wm0 + i * MF::BLK + MF::row(e, lane);
-                        if (m < M) q[(i64)m * rs] = acc[i][j][e];
+                        if (m < M) q[(i64)m * rs] = ep.xform(m, n, acc[i][j][e]);
                     }
             }
         }

@@ -26,6 +26,12 @@ template <typename T> struct FusedApi;
         }                                                                                                              \
         static int sgd(fx_ctx* c, T* p, const T* g, int64_t n, T lr) { return fx_sgd_step_##S(c, p, g, n, lr); }       \
         static int relu_bwd(fx_ctx* c, const T* g, const T* x, T* o, int64_t n) { return fx_relu_bwd_##S(c, g, x, o, n); } \
+        static int gemm_bias(fx_ctx* c, int ta, int tb, int64_t M, int64_t N, int64_t K, const T* A, const T* B, const T* b, T* C, int act) { \
+            return fx_gemm_bias_act_##S(c, ta, tb, M, N, K, A, B, b, C, act);                                          \
+        }                                                                                                              \
+        static int conv_bias(fx_ctx* c, const T* x, const T* w, const T* b, T* y, const int64_t* d, int act) {         \
+            return fx_conv2d_fwd_bias_act_##S(c, x, w, b, y, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9], d[10], act, nullptr, 0); \
+        }                                                                                                              \
     };
 FERROX_FUSED_API(float, f32)
 FERROX_FUSED_API(double, f64)
@@ -47,8 +53,8 @@ template <typename T> struct LinearFusedOp : Operator<T> {  // inputs: x [B, in]
         const Shape &xs = in[0]->shape(), &ws = in[1]->shape();
         if (xs.size() != 2 || ws.size() != 2 || xs[1] != ws[1]) throw Error("Linear: input " + fmt_shape(xs) + " vs weight " + fmt_shape(ws));
         Tensor<T> y = HipStorage<T>::alloc({xs[0], ws[0]});
-        fx_ok(Api<T>::gemm(fused_ctx(), 0, 1, (int64_t)xs[0], (int64_t)ws[0], (int64_t)xs[1], in[0]->data(), in[1]->data(), y->data()));
-        fx_ok(FusedApi<T>::bias_act(fused_ctx(), y->data(), in[2]->data(), (int64_t)xs[0], (int64_t)ws[0], 1, relu ? 1 : 0));
+        fx_ok(FusedApi<T>::gemm_bias(fused_ctx(), 0, 1, (int64_t)xs[0], (int64_t)ws[0], (int64_t)xs[1], in[0]->data(), in[1]->data(),
+                                     in[2]->data(), y->data(), relu ? 1 : 0));
         return y;
     }
     std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out) const override {
@@ -79,10 +85,13 @@ template <typename T> struct Conv2dFusedOp : Operator<T> {  // inputs: x [B,Cin,
     bool relu;
     Conv2dFusedOp(std::pair<size_t, size_t> s, std::pair<size_t, size_t> p, bool relu_) : stride(s), padding(p), relu(relu_) {}
     Tensor<T> compute(const TensorRefs<T>& in) const override {
-        Tensor<T> y = in[0]->conv2d(*in[1], stride, padding);
-        const Shape& ys = y->shape();
-        fx_ok(FusedApi<T>::bias_act(fused_ctx(), y->data(), in[2]->data(), (int64_t)ys[0], (int64_t)ys[1], (int64_t)(ys[2] * ys[3]),
-                                    relu ? 1 : 0));
+        const Shape &xs = in[0]->shape(), &ws = in[1]->shape();
+        if (xs.size() != 4 || ws.size() != 4 || xs[1] != ws[1]) throw Error("Conv2d: input " + fmt_shape(xs) + " vs filter " + fmt_shape(ws));
+        const int64_t d[11] = {(int64_t)xs[0], (int64_t)xs[1], (int64_t)xs[2], (int64_t)xs[3], (int64_t)ws[0], (int64_t)ws[2], (int64_t)ws[3],
+                               (int64_t)stride.first, (int64_t)stride.second, (int64_t)padding.first, (int64_t)padding.second};
+        Tensor<T> y = HipStorage<T>::alloc({xs[0], ws[0], (xs[2] + 2 * padding.first - ws[2]) / stride.first + 1,
+                                            (xs[3] + 2 * padding.second - ws[3]) / stride.second + 1});
+        fx_ok(FusedApi<T>::conv_bias(fused_ctx(), in[0]->data(), in[1]->data(), in[2]->data(), y->data(), d, relu ? 1 : 0));
         return y;
     }
     std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out) const override {

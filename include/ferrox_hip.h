@@ -253,6 +253,14 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
        inner = 1), act 0 = none, 1 = ReLU.  Replaces Reshape + BroadcastTo + Add (+ ReLU) of                           \
        src/nn/layers/utils.rs:6-42, conv2d.rs:203-213, linear.rs:262-279; same values bit for bit. */                  \
     int fx_bias_act_##S(fx_ctx* ctx, T* y, const T* bias, int64_t outer, int64_t C, int64_t inner, int act);           \
+    /* The same bias add (+ ReLU) carried in the store of the producing kernel: fx_conv2d_fwd / fx_gemm followed by     \
+       fx_bias_act, in one pass over the output (bias per output channel for the conv, per column of C for the GEMM);   \
+       bit-identical to the two-call sequence. */                                                                      \
+    int fx_conv2d_fwd_bias_act_##S(fx_ctx* ctx, const T* x, const T* w, const T* bias, T* y, int64_t B, int64_t Cin,   \
+                                   int64_t H, int64_t W, int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, \
+                                   int64_t ph, int64_t pw, int act, void* workspace, int64_t ws_bytes);                \
+    int fx_gemm_bias_act_##S(fx_ctx* ctx, int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const T* A,       \
+                             const T* B, const T* bias, T* C, int act);                                                \
     /* Bias gradient out[c] = sum over (o, i) of g[o, c, i]: reduce_gradient_for_broadcasting,                         \
        src/ops/basic.rs:10-53 (three axis sums for a conv bias) in one pass; fixed summation order per shape. */       \
     int fx_bias_grad_##S(fx_ctx* ctx, const T* g, T* out, int64_t outer, int64_t C, int64_t inner);                    \

@@ -115,3 +115,34 @@ def test_adam_and_sgd_step_bit_exact(ctx, train, dtype):
     dw = ctx.upload(w)
     ctx.sgd_step(dw, ctx.upload(g), 0.01)
     assert np.array_equal(dw.numpy(), orc.binary("sub", w, orc.scalar("mul_scalar", g, dt(0.01))))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_conv_and_gemm_with_bias_epilogue_equal_two_call_sequence(ctx, dtype):
+    """fx_conv2d_fwd_bias_act / fx_gemm_bias_act must give the bits of fx_conv2d_fwd / fx_gemm followed by fx_bias_act,
+    on every conv path (LDS-patch, implicit GEMM, strided) and on plain and split-K GEMMs."""
+    from ferrox_amd import capi
+    rng = np.random.default_rng(74)
+    sfx = capi.dtype_code(dtype)[1]
+    for (B, Cin, H, W, Cout, k, s, p) in [(2, 32, 8, 56, 96, 3, 1, 1), (2, 16, 6, 16, 40, 3, 1, 1), (3, 3, 9, 9, 8, 3, 1, 1),
+                                          (2, 64, 14, 14, 130, 3, 2, 1), (2, 8, 7, 7, 5, 1, 1, 0)]:
+        x = ctx.upload(rng.uniform(-1, 1, (B, Cin, H, W)).astype(dtype))
+        w = ctx.upload((rng.standard_normal((Cout, Cin, k, k)) * 0.1).astype(dtype))
+        b = ctx.upload(rng.standard_normal(Cout).astype(dtype))
+        dims = (B, Cin, H, W, Cout, k, k, s, s, p, p)
+        for act in (0, 1):
+            y2 = ctx.conv2d_fwd(x, w, (s, s), (p, p))
+            ctx.bias_act(y2, b, B, Cout, y2.shape[2] * y2.shape[3], act)
+            y1 = ctx.empty(y2.shape, dtype)
+            capi.check(getattr(capi.lib, f"fx_conv2d_fwd_bias_act_{sfx}")(ctx.h, x.ptr, w.ptr, b.ptr, y1.ptr, *dims, act, None, 0))
+            assert np.array_equal(y1.numpy(), y2.numpy()), (dims, act)
+    for (M, N, K, ta, tb) in [(256, 256, 784, 0, 1), (256, 10, 16384, 0, 1), (130, 70, 33, 0, 0), (512, 384, 256, 1, 0), (5, 3, 2, 0, 0)]:
+        a = ctx.upload(rng.standard_normal((K, M) if ta else (M, K)).astype(dtype))
+        bm = ctx.upload(rng.standard_normal((N, K) if tb else (K, N)).astype(dtype))
+        bias = ctx.upload(rng.standard_normal(N).astype(dtype))
+        for act in (0, 1):
+            c2 = ctx.gemm(a, bm, bool(ta), bool(tb))
+            ctx.bias_act(c2, bias, M, N, 1, act)
+            c1 = ctx.empty((M, N), dtype)
+            capi.check(getattr(capi.lib, f"fx_gemm_bias_act_{sfx}")(ctx.h, ta, tb, M, N, K, a.ptr, bm.ptr, bias.ptr, c1.ptr, act))
+            assert np.array_equal(c1.numpy(), c2.numpy()), (M, N, K, ta, tb, act)
