@@ -18,7 +18,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # Files whose composed expressions must round op by op like the CPU backend (no a*b+c contraction).
-NO_CONTRACT = {"elementwise.hip", "reduce.hip", "im2col.hip", "fused.hip", "pooling.hip"}
+NO_CONTRACT = {"elementwise.hip", "reduce.hip", "im2col.hip", "fused.hip", "pooling.hip", "batchnorm.hip"}
 
 
 def sources():

@@ -114,7 +114,12 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_reduce_mean_{_s}", _vp, _vp, _vp, _i64, _i64, _i64)
     _sig(f"fx_reduce_max_{_s}", _vp, _vp, _vp, _vp, _i64, _i64, _i64)
     _sig(f"fx_reduce_min_{_s}", _vp, _vp, _vp, _vp, _i64, _i64, _i64)
+    _sig(f"fx_reduce_prod_{_s}", _vp, _vp, _vp, _i64, _i64, _i64)
     _sig(f"fx_in_range_{_s}", _vp, _vp, _ct, _ct, _vp, _i64)
+    _sig(f"fx_batchnorm_stats_{_s}", _vp, _vp, _vp, _vp, _vp, _vp, C.c_double, _i64, _i64, _i64)
+    _sig(f"fx_batchnorm_fwd_{_s}", _vp, _vp, _vp, _vp, _vp, _vp, C.c_double, _vp, _i64, _i64, _i64)
+    _sig(f"fx_batchnorm_bwd_{_s}", _vp, _vp, _vp, _vp, _vp, _vp, C.c_double, _vp, _vp, _vp, _i64, _i64, _i64, _int)
+    _sig(f"fx_dropout_{_s}", _vp, _vp, _vp, _vp, _i64, C.c_double, _u64)
     _sig(f"fx_maxpool2d_{_s}", _vp, _vp, _vp, *([_i64] * 10))
     _sig(f"fx_avgpool2d_{_s}", _vp, _vp, _vp, *([_i64] * 10))
     _sig(f"fx_max_unpool2d_{_s}", _vp, _vp, _vp, _vp, _vp, *([_i64] * 10))
@@ -355,7 +360,7 @@ class Context:
         return outer, int(shape[axis]), inner
 
     def reduce(self, kind, a, axis, want_idx=False, out=None):
-        """kind in sum/mean/max over ONE axis (keep_dims False)."""
+        """kind in sum/mean/max/min/prod over ONE axis (keep_dims False)."""
         outer, ax, inner = self._oai(a.shape, axis)
         oshape = a.shape[:axis] + a.shape[axis + 1:]
         o = out or self.empty(oshape if oshape else (1,), a.dtype)
@@ -429,6 +434,46 @@ class Context:
         """In place: y[o, c, i] += bias[c], then ReLU when act == 1."""
         check(self._fn("bias_act", y.dtype)(self.h, y.ptr, bias.ptr, outer, C, inner, act))
         return y
+
+    @staticmethod
+    def _channel_view(shape):
+        """[N, C, ...] -> (outer, C, inner) of the channel axis."""
+        inner = 1
+        for d in shape[2:]:
+            inner *= d
+        return shape[0], shape[1], inner
+
+    def batchnorm_stats(self, x, running_mean=None, running_var=None, momentum=0.1):
+        """Per-channel mean and biased variance of x [N, C, ...]; updates the running arrays in place when given."""
+        outer, Cc, inner = self._channel_view(x.shape)
+        mean, var = self.empty((Cc,), x.dtype), self.empty((Cc,), x.dtype)
+        check(self._fn("batchnorm_stats", x.dtype)(self.h, x.ptr, mean.ptr, var.ptr,
+                                                   running_mean.ptr if running_mean is not None else None,
+                                                   running_var.ptr if running_var is not None else None,
+                                                   float(momentum), outer, Cc, inner))
+        return mean, var
+
+    def batchnorm_fwd(self, x, mean, var, gamma, beta, eps):
+        outer, Cc, inner = self._channel_view(x.shape)
+        y = self.empty(x.shape, x.dtype)
+        check(self._fn("batchnorm_fwd", x.dtype)(self.h, x.ptr, mean.ptr, var.ptr, gamma.ptr, beta.ptr, float(eps), y.ptr,
+                                                 outer, Cc, inner))
+        return y
+
+    def batchnorm_bwd(self, dy, x, mean, var, gamma, eps, batch_stats=True, need_dx=True):
+        outer, Cc, inner = self._channel_view(x.shape)
+        dx = self.empty(x.shape, x.dtype) if need_dx else None
+        dgamma, dbeta = self.empty((Cc,), x.dtype), self.empty((Cc,), x.dtype)
+        check(self._fn("batchnorm_bwd", x.dtype)(self.h, dy.ptr, x.ptr, mean.ptr, var.ptr, gamma.ptr, float(eps),
+                                                 dx.ptr if need_dx else None, dgamma.ptr, dbeta.ptr, outer, Cc, inner,
+                                                 1 if batch_stats else 0))
+        return dx, dgamma, dbeta
+
+    def dropout(self, x, p, seed):
+        """Returns (y, mask): mask = 1/(1-p) or 0 from splitmix64(seed + i), y = x*mask."""
+        mask, y = self.empty(x.shape, x.dtype), self.empty(x.shape, x.dtype)
+        check(self._fn("dropout", x.dtype)(self.h, x.ptr, mask.ptr, y.ptr, x.size, float(p), int(seed)))
+        return y, mask
 
     def bias_grad(self, g, outer, C, inner):
         o = self.empty((C,), g.dtype)

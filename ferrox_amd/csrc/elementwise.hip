@@ -468,9 +468,52 @@ int random_fill(fx_ctx* c, T* out, i64 n, uint64_t seed, T a, T b) {
     return FX_OK;
 }
 
+// ---- inverted dropout: nn/layers/dropout.rs:56-136 draws one f64 uniform per element, keeps it when u < 1 - p and
+// writes mask = 1/(1-p) (cast to T) or 0, then multiplies.  The reference's generator is unseeded; here element i
+// takes the 53-bit uniform of splitmix64(seed + i), so a mask can be rebuilt on the host.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void dropout_kernel(const T* __restrict__ x, T* __restrict__ mask, T* __restrict__ y, i64 n,
+                                                      uint64_t seed, double keep, T scale) {
+    constexpr int V = VEC ? 16 / (int)sizeof(T) : 1;
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    const i64 i = ((i64)blockIdx.x * 256 + threadIdx.x) * V;
+    if (i >= n) return;
+    const vec_t v = *reinterpret_cast<const vec_t*>(x + i);
+    vec_t m, r;
+#pragma unroll
+    for (int u = 0; u < V; ++u) {
+        m[u] = unit_uniform<double>(splitmix64(seed + (uint64_t)(i + u))) < keep ? scale : T(0);
+        r[u] = v[u] * m[u];
+    }
+    *reinterpret_cast<vec_t*>(mask + i) = m;
+    *reinterpret_cast<vec_t*>(y + i) = r;
+}
+
+template <typename T>
+int dropout(fx_ctx* c, const T* x, T* mask, T* y, i64 n, double p, uint64_t seed) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(n >= 0, "fx_dropout: negative element count");
+    FX_REQUIRE(p >= 0.0 && p < 1.0, "fx_dropout: p must be in [0, 1)");
+    if (n == 0) return FX_OK;
+    FX_REQUIRE(x && mask && y, "fx_dropout: null pointer");
+    constexpr int V = 16 / (int)sizeof(T);
+    const bool vec = n % V == 0 && fx::aligned16(x) && fx::aligned16(mask) && fx::aligned16(y);
+    const i64 blocks = fx::ceil_div(vec ? n / V : n, 256);
+    FX_REQUIRE(blocks <= 0x7fffffff, "fx_dropout: too many elements");
+    const double keep = 1.0 - p;
+    const T scale = (T)(1.0 / keep);
+    if (vec) dropout_kernel<T, true><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(x, mask, y, n, seed, keep, scale);
+    else dropout_kernel<T, false><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(x, mask, y, n, seed, keep, scale);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
 }  // namespace
 
 #define FX_DEFINE_EW(T, S)                                                                                             \
+    extern "C" int fx_dropout_##S(fx_ctx* c, const T* x, T* mask, T* y, int64_t n, double p, uint64_t seed) {          \
+        return dropout<T>(c, x, mask, y, n, p, seed);                                                                  \
+    }                                                                                                                  \
     extern "C" int fx_fill_uniform_##S(fx_ctx* c, T* out, int64_t n, uint64_t seed, T lo, T hi) {                      \
         return random_fill<T, false>(c, out, n, seed, lo, hi);                                                         \
     }                                                                                                                  \

@@ -56,23 +56,27 @@ __device__ __forceinline__ i64 shfl_down_i64(i64 v, int d) {
 __device__ __forceinline__ double shfl_down_t(double v, int d) { return __shfl_down(v, d, 64); }
 __device__ __forceinline__ float shfl_down_t(float v, int d) { return __shfl_down(v, d, 64); }
 
-// Accumulator: value (+ index for the extrema).  IS_MAX: 0 = sum (ignores idx), 1 = maximum, 2 = minimum.
+// Accumulator: value (+ index for the extrema).  IS_MAX: 0 = sum (ignores idx), 1 = maximum, 2 = minimum,
+// 3 = product (ignores idx; kernels/reduction.cu:232-301 starts from 1 and multiplies).
+#define EXTREMUM(M) ((M) == 1 || (M) == 2)
 // The extrema start from the lowest / highest finite T and take strictly greater / smaller values
 // (cpu.rs:1231-1234, 1240-1252), so the first position attaining the extremum wins.
 template <typename T, int IS_MAX> struct Acc {
     T v;
     i64 i;
-    __device__ __forceinline__ void init() { v = IS_MAX == 1 ? lowest<T>() : IS_MAX == 2 ? -lowest<T>() : T(0); i = NO_INDEX; }
+    __device__ __forceinline__ void init() { v = IS_MAX == 1 ? lowest<T>() : IS_MAX == 2 ? -lowest<T>() : IS_MAX == 3 ? T(1) : T(0); i = NO_INDEX; }
     // element x at axis position p, visited in increasing p by this thread
     __device__ __forceinline__ void take(T x, i64 p) {
         if (IS_MAX == 1) { if (x > v) { v = x; i = p; } }
         else if (IS_MAX == 2) { if (x < v) { v = x; i = p; } }
+        else if (IS_MAX == 3) v = v * x;
         else v = v + x;
     }
     // merge another accumulator (any order): ties go to the smaller index
     __device__ __forceinline__ void merge(T ov, i64 oi) {
         if (IS_MAX == 1) { if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; } }
         else if (IS_MAX == 2) { if (ov < v || (ov == v && oi < i)) { v = ov; i = oi; } }
+        else if (IS_MAX == 3) v = v * ov;
         else v = v + ov;
     }
 };
@@ -83,7 +87,7 @@ __device__ __forceinline__ void wave_reduce(Acc<T, IS_MAX>& a) {
     for (int d = 32; d >= 1; d >>= 1) {
         const T ov = shfl_down_t(a.v, d);
         i64 oi = NO_INDEX;
-        if (IS_MAX) oi = shfl_down_i64(a.i, d);
+        if (EXTREMUM(IS_MAX)) oi = shfl_down_i64(a.i, d);
         a.merge(ov, oi);
     }
 }
@@ -135,8 +139,8 @@ __global__ __launch_bounds__(256) void row_reduce_kernel(const T* __restrict__ i
         r.v = sv[0]; r.i = si[0];
         for (int w = 1; w < 4; ++w) r.merge(sv[w], si[w]);
         const i64 slot = o * S + s;
-        out[slot] = IS_MAX ? r.v : r.v * scale;
-        if (IS_MAX && idx_out) idx_out[slot] = (S == 1 && r.i == NO_INDEX) ? 0 : r.i;
+        out[slot] = EXTREMUM(IS_MAX) ? r.v : r.v * scale;
+        if (EXTREMUM(IS_MAX) && idx_out) idx_out[slot] = (S == 1 && r.i == NO_INDEX) ? 0 : r.i;
     }
 }
 
@@ -154,12 +158,12 @@ __global__ __launch_bounds__(256) void short_row_reduce_kernel(const T* __restri
     for (int d = G >> 1; d >= 1; d >>= 1) {
         const T ov = shfl_down_t(acc.v, d);
         i64 oi = NO_INDEX;
-        if (IS_MAX) oi = shfl_down_i64(acc.i, d);
+        if (EXTREMUM(IS_MAX)) oi = shfl_down_i64(acc.i, d);
         if ((lane % G) + d < G) acc.merge(ov, oi);
     }
     if (a == 0 && o < outer) {
-        out[o] = IS_MAX ? acc.v : acc.v * scale;
-        if (IS_MAX && idx_out) idx_out[o] = acc.i == NO_INDEX ? 0 : acc.i;
+        out[o] = EXTREMUM(IS_MAX) ? acc.v : acc.v * scale;
+        if (EXTREMUM(IS_MAX) && idx_out) idx_out[o] = acc.i == NO_INDEX ? 0 : acc.i;
     }
 }
 
@@ -170,7 +174,7 @@ __global__ __launch_bounds__(256) void combine_rows_kernel(const T* __restrict__
     const i64 o = blockIdx.x;
     Acc<T, IS_MAX> acc;
     acc.init();
-    for (i64 s = threadIdx.x; s < S; s += 256) acc.merge(pv[o * S + s], IS_MAX && pi ? pi[o * S + s] : NO_INDEX);
+    for (i64 s = threadIdx.x; s < S; s += 256) acc.merge(pv[o * S + s], EXTREMUM(IS_MAX) && pi ? pi[o * S + s] : NO_INDEX);
     wave_reduce(acc);
     __shared__ T sv[4];
     __shared__ i64 si[4];
@@ -181,8 +185,8 @@ __global__ __launch_bounds__(256) void combine_rows_kernel(const T* __restrict__
         Acc<T, IS_MAX> r;
         r.v = sv[0]; r.i = si[0];
         for (int w = 1; w < 4; ++w) r.merge(sv[w], si[w]);
-        out[o] = IS_MAX ? r.v : r.v * scale;
-        if (IS_MAX && idx_out) idx_out[o] = r.i == NO_INDEX ? 0 : r.i;
+        out[o] = EXTREMUM(IS_MAX) ? r.v : r.v * scale;
+        if (EXTREMUM(IS_MAX) && idx_out) idx_out[o] = r.i == NO_INDEX ? 0 : r.i;
     }
 }
 
@@ -209,7 +213,7 @@ __global__ __launch_bounds__(256) void col_reduce_kernel(const T* __restrict__ i
     for (int e = 0; e < N; ++e) acc[e].init();
     if (col < inner) {
         const T* base = in + (o * axis) * inner + col;
-        const i64* ibase = FROM_PARTIAL && IS_MAX ? pidx + (o * axis) * inner + col : nullptr;
+        const i64* ibase = FROM_PARTIAL && EXTREMUM(IS_MAX) ? pidx + (o * axis) * inner + col : nullptr;
         i64 a = beg + wr;
         if (VEC && !FROM_PARTIAL) {
             for (; a + 7 * RW < end; a += 8 * RW) {
@@ -231,20 +235,20 @@ __global__ __launch_bounds__(256) void col_reduce_kernel(const T* __restrict__ i
 #pragma unroll
                 for (int e = 0; e < N; ++e) {
                     const T x = base[a * inner + e];
-                    if (FROM_PARTIAL) acc[e].merge(x, IS_MAX ? ibase[a * inner + e] : NO_INDEX);
+                    if (FROM_PARTIAL) acc[e].merge(x, EXTREMUM(IS_MAX) ? ibase[a * inner + e] : NO_INDEX);
                     else acc[e].take(x, a);
                 }
             }
         }
     }
     __shared__ T sv[RW][CW * 64 * N];
-    __shared__ i64 si[IS_MAX ? RW : 1][IS_MAX ? CW * 64 * N : 1];
+    __shared__ i64 si[EXTREMUM(IS_MAX) ? RW : 1][EXTREMUM(IS_MAX) ? CW * 64 * N : 1];
     const int sl = (wc * 64 + lane) * N;
     if (RW > 1) {
 #pragma unroll
         for (int e = 0; e < N; ++e) {
             sv[wr][sl + e] = acc[e].v;
-            if (IS_MAX) si[wr][sl + e] = acc[e].i;
+            if (EXTREMUM(IS_MAX)) si[wr][sl + e] = acc[e].i;
         }
         __syncthreads();
     }
@@ -252,10 +256,10 @@ __global__ __launch_bounds__(256) void col_reduce_kernel(const T* __restrict__ i
 #pragma unroll
         for (int e = 0; e < N; ++e) {
             Acc<T, IS_MAX> r = acc[e];
-            for (int w = 1; w < RW; ++w) r.merge(sv[w][sl + e], IS_MAX ? si[w][sl + e] : NO_INDEX);
+            for (int w = 1; w < RW; ++w) r.merge(sv[w][sl + e], EXTREMUM(IS_MAX) ? si[w][sl + e] : NO_INDEX);
             const i64 slot = (o * S + s) * inner + col + e;
-            out[slot] = IS_MAX ? r.v : r.v * scale;
-            if (IS_MAX && idx_out) idx_out[slot] = (final_pass && r.i == NO_INDEX) ? 0 : r.i;
+            out[slot] = EXTREMUM(IS_MAX) ? r.v : r.v * scale;
+            if (EXTREMUM(IS_MAX) && idx_out) idx_out[slot] = (final_pass && r.i == NO_INDEX) ? 0 : r.i;
         }
     }
 }
@@ -274,7 +278,7 @@ int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i6
     FX_REQUIRE(in && out, "%s: null pointer", what);
     FX_REQUIRE(outer <= 65535 * 1024ll, "%s: outer too large", what);
     constexpr int N = Vec16<T>::N;
-    const bool want_idx = IS_MAX && idx_out != nullptr;
+    const bool want_idx = EXTREMUM(IS_MAX) && idx_out != nullptr;
     std::lock_guard<std::mutex> lk(c->launch_mutex);
     const i64 target_blocks = (i64)c->num_cus * 8;
 
@@ -312,7 +316,7 @@ int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i6
         }
         const dim3 grid((unsigned)S, (unsigned)outer), block(256);
         const T sc1 = S > 1 ? T(1) : scale;
-        i64* io = (S > 1 && IS_MAX) ? pi : idx_out;
+        i64* io = (S > 1 && EXTREMUM(IS_MAX)) ? pi : idx_out;
         const bool stream = outer * axis * (i64)sizeof(T) >= STREAM_BYTES;
         if (vec && stream) row_reduce_kernel<T, IS_MAX, true, true><<<grid, block, 0, c->stream>>>(in, pv, io, axis, chunk, sc1);
         else if (vec) row_reduce_kernel<T, IS_MAX, true, false><<<grid, block, 0, c->stream>>>(in, pv, io, axis, chunk, sc1);
@@ -320,7 +324,7 @@ int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i6
         FX_LAUNCH_CHECK();
         if (S > 1) {
             combine_rows_kernel<T, IS_MAX><<<dim3((unsigned)outer), dim3(256), 0, c->stream>>>(
-                pv, IS_MAX ? pi : nullptr, out, idx_out, outer, S, scale);
+                pv, EXTREMUM(IS_MAX) ? pi : nullptr, out, idx_out, outer, S, scale);
             FX_LAUNCH_CHECK();
         }
         (void)want_idx;
@@ -350,11 +354,11 @@ int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i6
     i64* pi = idx_out;
     if (S > 1) {
         const i64 n_part = outer * S * inner;
-        const i64 bytes = n_part * (i64)(sizeof(T) + (IS_MAX ? sizeof(i64) : 0)) + 256;
+        const i64 bytes = n_part * (i64)(sizeof(T) + (EXTREMUM(IS_MAX) ? sizeof(i64) : 0)) + 256;
         char* sc = (char*)c->get_scratch(bytes);
         if (!sc) return FX_ERR_OOM;
-        pi = IS_MAX ? (i64*)sc : nullptr;
-        pv = (T*)(sc + (IS_MAX ? ((n_part * sizeof(i64) + 255) / 256) * 256 : 0));
+        pi = EXTREMUM(IS_MAX) ? (i64*)sc : nullptr;
+        pv = (T*)(sc + (EXTREMUM(IS_MAX) ? ((n_part * sizeof(i64) + 255) / 256) * 256 : 0));
     }
     {
         const dim3 grid((unsigned)tiles, (unsigned)S, (unsigned)outer);
@@ -461,6 +465,9 @@ int softmax_axis(fx_ctx* c, const T* in, T* out, i64 outer, i64 axis, i64 inner)
     extern "C" int fx_reduce_min_##S(fx_ctx* c, const T* in, T* out, int64_t* idx, int64_t outer, int64_t axis,        \
                                      int64_t inner) {                                                                  \
         return reduce<T, 2>(c, in, out, idx, outer, axis, inner, T(1), "fx_reduce_min");                               \
+    }                                                                                                                  \
+    extern "C" int fx_reduce_prod_##S(fx_ctx* c, const T* in, T* out, int64_t outer, int64_t axis, int64_t inner) {    \
+        return reduce<T, 3>(c, in, out, nullptr, outer, axis, inner, T(1), "fx_reduce_prod");                          \
     }                                                                                                                  \
     extern "C" int fx_softmax_axis_##S(fx_ctx* c, const T* in, T* out, int64_t outer, int64_t axis, int64_t inner) {   \
         return softmax_axis<T>(c, in, out, outer, axis, inner);                                                        \

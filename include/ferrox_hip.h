@@ -204,6 +204,8 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
     /* min_reduce, cpu.rs:1240-1252: starts from the highest finite T, takes strictly smaller values; idx_out as above. */ \
     int fx_reduce_min_##S(fx_ctx* ctx, const T* in, T* out, int64_t* idx_out, int64_t outer, int64_t axis,             \
                           int64_t inner);                                                                              \
+    /* reduce_prod_all / reduce_prod_axes, kernels/reduction.cu:232-301, 348-360: product along the axis, from 1. */    \
+    int fx_reduce_prod_##S(fx_ctx* ctx, const T* in, T* out, int64_t outer, int64_t axis, int64_t inner);              \
     /* launch_matmul, kernels.rs:919-938 / cpu.rs:967-1002: C[M,N] = op(A) . op(B).  trans_a: A is stored [K,M];       \
        trans_b: B is stored [N,K]  (lets MatMul::gradient, src/ops/matrix.rs:30-55, skip materialised transposes). */  \
     int fx_gemm_##S(fx_ctx* ctx, int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const T* A, const T* B,    \
@@ -261,6 +263,24 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
                                    int64_t ph, int64_t pw, int act, void* workspace, int64_t ws_bytes);                \
     int fx_gemm_bias_act_##S(fx_ctx* ctx, int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const T* A,       \
                              const T* B, const T* bias, T* C, int act);                                                \
+    /* BatchNorm, src/nn/layers/norm.rs:127-336, on x viewed as [outer, C, inner] ([N,C,H,W]: outer = N, inner = H*W;   \
+       [N,F]: C = F, inner = 1).  stats: mean[C] and biased variance[C] of every channel in one read of x (the         \
+       reference's Mean, Sub, Mul, Mean chain), and, when the pointers are not NULL, the running update                \
+       running = running*(1-momentum) + batch*momentum (norm.rs:144-161).  fwd: y = ((x-mean)/sqrt(var+eps))*gamma     \
+       + beta, the composed operations in the composed order, bit-identical to them given mean and var (pass the       \
+       running statistics for inference, norm.rs:261-290).  bwd: dgamma[C], dbeta[C] and, unless dx is NULL, dx;       \
+       batch_stats 1 = mean/var came from this batch (gradient flows through them), 0 = fixed statistics. */           \
+    int fx_batchnorm_stats_##S(fx_ctx* ctx, const T* x, T* mean, T* var, T* running_mean, T* running_var,              \
+                               double momentum, int64_t outer, int64_t C, int64_t inner);                              \
+    int fx_batchnorm_fwd_##S(fx_ctx* ctx, const T* x, const T* mean, const T* var, const T* gamma, const T* beta,      \
+                             double eps, T* y, int64_t outer, int64_t C, int64_t inner);                               \
+    int fx_batchnorm_bwd_##S(fx_ctx* ctx, const T* dy, const T* x, const T* mean, const T* var, const T* gamma,        \
+                             double eps, T* dx, T* dgamma, T* dbeta, int64_t outer, int64_t C, int64_t inner,          \
+                             int batch_stats);                                                                         \
+    /* Dropout::forward in training, src/nn/layers/dropout.rs:56-136: mask[i] = 1/(1-p) where u_i < 1-p, else 0, and    \
+       y = x*mask; u_i is the 53-bit uniform of splitmix64(seed + i) (the reference's generator is unseeded), 0 <= p    \
+       < 1.  The gradient is fx_mul(grad, mask). */                                                                    \
+    int fx_dropout_##S(fx_ctx* ctx, const T* x, T* mask, T* y, int64_t n, double p, uint64_t seed);                    \
     /* Bias gradient out[c] = sum over (o, i) of g[o, c, i]: reduce_gradient_for_broadcasting,                         \
        src/ops/basic.rs:10-53 (three axis sums for a conv bias) in one pass; fixed summation order per shape. */       \
     int fx_bias_grad_##S(fx_ctx* ctx, const T* g, T* out, int64_t outer, int64_t C, int64_t inner);                    \

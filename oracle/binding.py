@@ -186,7 +186,7 @@ def _oai(shape, axis):
 
 
 def reduce_axis(kind, x, axis, want_idx=False):
-    """kind in {'sum','mean','max'} over ONE axis of a contiguous array (keep_dims False)."""
+    """kind in {'sum','mean','max','min','prod'} over ONE axis of a contiguous array (keep_dims False)."""
     x = _c(x)
     outer, ax, inner = _oai(x.shape, axis)
     out_shape = x.shape[:axis] + x.shape[axis + 1:]
@@ -218,6 +218,25 @@ def reduce(kind, x, axes=None, keep_dims=False):
             fs[a] = 1
         r = r.reshape(fs)
     return r
+
+
+def splitmix64_uniform(seed, n):
+    """u_i in [0,1), i < n: the top 53 bits of splitmix64(seed + i) (Steele, Lea & Flood 2014) as a float64."""
+    with np.errstate(over="ignore"):
+        z = np.uint64(seed) + np.arange(n, dtype=np.uint64) + np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        z = z ^ (z >> np.uint64(31))
+    return (z >> np.uint64(11)).astype(np.float64) * (1.0 / 9007199254740992.0)
+
+
+def dropout_mask(shape, p, seed, dtype):
+    """create_dropout_mask (nn/layers/dropout.rs:56-82): one f64 uniform per element, keep when u < 1 - p,
+    mask = T(1/(1-p)) or 0.  The reference draws from an unseeded generator; element i takes splitmix64(seed + i)."""
+    n = int(np.prod(shape))
+    keep = 1.0 - p
+    u = splitmix64_uniform(seed, n)
+    return np.where(u < keep, np.dtype(dtype).type(1.0 / keep), np.dtype(dtype).type(0)).astype(dtype).reshape(shape)
 
 
 def in_range(a, lo, hi):

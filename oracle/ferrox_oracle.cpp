@@ -395,6 +395,19 @@ void reduce_min_axis(const T* x, i64 outer, i64 axis, i64 inner, T* out, i64* id
         }
 }
 
+// Product along the axis, from 1, positions in increasing order.  The reference has no CPU product; this restates the
+// per-output arithmetic of kernels/reduction.cu:263-301 (prod = 1; prod *= input[...]) without its 32-lane tree, so
+// the device result is compared to tolerance, never bit for bit.
+template <typename T>
+void reduce_prod_axis(const T* x, i64 outer, i64 axis, i64 inner, T* out) {
+    for (i64 o = 0; o < outer; ++o)
+        for (i64 i = 0; i < inner; ++i) {
+            T acc = T(1);
+            for (i64 a = 0; a < axis; ++a) acc = acc * x[(o * axis + a) * inner + i];
+            out[o * inner + i] = acc;
+        }
+}
+
 template <typename T>
 void in_range(const T* a, T lo, T hi, T* o, i64 n) {  // cpu.rs:933-947
     for (i64 i = 0; i < n; ++i) o[i] = (a[i] >= lo && a[i] <= hi) ? T(1) : T(0);
@@ -525,6 +538,9 @@ void materialize(const T* x, T* out, const i64* shape, const i64* strides, int n
     }                                                                                                                  \
     extern "C" void orc_reduce_max_##S(const T* x, i64 outer, i64 axis, i64 inner, T* out, i64* idx) {                \
         reduce_max_axis<T>(x, outer, axis, inner, out, idx);                                                           \
+    }                                                                                                                  \
+    extern "C" void orc_reduce_prod_##S(const T* x, i64 outer, i64 axis, i64 inner, T* out) {                         \
+        reduce_prod_axis<T>(x, outer, axis, inner, out);                                                               \
     }                                                                                                                  \
     extern "C" void orc_reduce_min_##S(const T* x, i64 outer, i64 axis, i64 inner, T* out, i64* idx) {                \
         reduce_min_axis<T>(x, outer, axis, inner, out, idx);                                                           \

@@ -1,10 +1,11 @@
 """CPU oracle for one Ferrox training step (test infrastructure only).
 
 Restates, operator by operator and in the reference's order, what `AutoFerroxEngine` + the `nn` layers do for a
-Sequential model of Linear / Conv2d / ReLU / Flatten layers with the softmax cross-entropy loss and SGD or Adam,
+Sequential model of Linear / Conv2d / ReLU / Flatten / pooling / BatchNorm / GlobalAvgPool2d / Dropout layers with the softmax cross-entropy loss and SGD or Adam,
 using the oracle's C primitives for every storage op so that each intermediate is rounded to the tensor dtype
 exactly where the CPU backend rounds it.  References (Ferrox repository paths):
-  layers     src/nn/layers/linear.rs:183-279, conv2d.rs:168-214, utils.rs:6-42, activation.rs:47-80, pooling.rs:100-140
+  layers     src/nn/layers/linear.rs:183-279, conv2d.rs:168-214, utils.rs:6-42, activation.rs:47-80, pooling.rs:100-140,
+             604-623, norm.rs:127-336, dropout.rs:56-136
   loss       src/nn/losses/classification.rs:191-257
   gradients  src/ops/{basic.rs:10-215, matrix.rs:17-125, unary.rs:60-95,196-236,340-384, comparison.rs:250-297,
              reduction.rs:9-230, reshape.rs:4-115, batched.rs:41-131,154-217}
@@ -81,12 +82,68 @@ def adam_update(w, g, m, v, lr, b1, b2, eps, wd, bc1, bc2):
     return w, m, v
 
 
+def batchnorm_forward(x, gamma, beta, eps, training=True, running_mean=None, running_var=None):
+    """BatchNorm::forward (nn/layers/norm.rs:167-336), operator by operator.  Training: statistics of the batch over
+    axes (0,2,3) / (0); AddScalar and Sqrt run on the full-size broadcast variance (norm.rs:228-236, 298-311).
+    Inference: the running statistics, Sqrt on [C] then broadcast (norm.rs:261-290).  Returns (out, tape record,
+    batch mean or None, batch variance or None)."""
+    dt = x.dtype.type
+    axes = [0, 2, 3] if x.ndim == 4 else [0]
+    if training:
+        mean = orc.reduce("mean", x, axes)
+        cen = orc.binary("sub", x, _bcast(mean, x.shape))
+        var = orc.reduce("mean", orc.binary("mul", cen, cen), axes)
+        std = orc.unary("sqrt", orc.scalar("add_scalar", _bcast(var, x.shape), dt(eps)))
+    else:
+        mean = var = None
+        cen = orc.binary("sub", x, _bcast(running_mean, x.shape))
+        std = _bcast(orc.unary("sqrt", orc.scalar("add_scalar", running_var, dt(eps))), x.shape)
+    normalized = orc.binary("div", cen, std)
+    wb = _bcast(gamma, x.shape)
+    out = orc.binary("add", orc.binary("mul", normalized, wb), _bcast(beta, x.shape))
+    return out, (cen, std, normalized, wb, training), mean, var
+
+
+def batchnorm_running_update(running, batch, momentum):
+    """update_running_stats (norm.rs:127-164): running*(1-momentum) + batch*momentum, the biased batch variance."""
+    dt = running.dtype.type
+    return orc.binary("add", orc.scalar("mul_scalar", running, dt(1.0 - momentum)), orc.scalar("mul_scalar", batch, dt(momentum)))
+
+
+def batchnorm_backward(g, rec):
+    """Gradients (dx, dgamma, dbeta) in the order AutoFerroxEngine::backward visits the nodes (graph/mod.rs:700-783:
+    reverse of the depth-first post-order): Add, Mul, Div, Sqrt, AddScalar, BroadcastTo, Mean, Mul(centered, centered)
+    twice into `centered`, Sub, BroadcastTo, Mean into x."""
+    cen, std, normalized, wb, training = rec
+    dt = g.dtype.type
+    red = (lambda t: orc.reduce("sum", t, [3, 2, 0])) if g.ndim == 4 else (lambda t: orc.reduce("sum", t, [0]))
+    dbeta = red(g)                                                         # Add -> BroadcastTo -> Reshape
+    g_norm = orc.binary("mul", g, wb)                                      # Mul::gradient, input 0
+    dgamma = red(orc.binary("mul", g, normalized))                         # input 1 -> BroadcastTo -> Reshape
+    d_cen = orc.binary("div", g_norm, std)                                 # Div::gradient, input 0 (ops/basic.rs:253)
+    if not training:
+        return d_cen, dgamma, dbeta
+    n = float(cen.size // dbeta.size)
+    g_std = orc.binary("mul", g_norm, orc.unary("neg", orc.binary("div", normalized, std)))      # basic.rs:256-257
+    g_vpe = orc.binary("div", g_std, orc.scalar("mul_scalar", std, dt(2.0)))                      # Sqrt, unary.rs:138-140
+    g_var = red(g_vpe)                                                     # AddScalar passes; BroadcastTo sums; Reshape
+    g_sq = _bcast(orc.scalar("mul_scalar", g_var, dt(1.0 / n)), cen.shape)  # Mean::gradient, reduction.rs:178-194
+    a = orc.binary("mul", g_sq, cen)                                       # Mul(centered, centered): both inputs
+    d_cen = orc.binary("add", orc.binary("add", d_cen, a), a)              # accumulate_gradient, graph/mod.rs:681-690
+    g_mean = red(orc.unary("neg", d_cen))                                  # Sub input 1 -> BroadcastTo -> Reshape
+    dx = orc.binary("add", d_cen, _bcast(orc.scalar("mul_scalar", g_mean, dt(1.0 / n)), cen.shape))
+    return dx, dgamma, dbeta
+
+
 class Sequential:
     def __init__(self, spec, params, dtype, conv_mode=0):
         self.dtype = np.dtype(dtype)
         self.conv_mode = conv_mode
         self.layers = []
         self.params = [np.ascontiguousarray(p, dtype=self.dtype).copy() for p in params]
+        self.training = True
+        self.running = {}     # layer index -> [running_mean, running_var]  (zeros / ones, norm.rs:75-84)
+        self.dropout_calls = 0
         pi = 0
         for tok in [t.strip() for t in spec.split(";") if t.strip()]:
             parts = tok.split()
@@ -101,7 +158,16 @@ class Sequential:
             elif kind in ("maxpool", "avgpool"):
                 _, k, st, p = parts
                 self.layers.append((kind, (int(k), int(k)), (int(st), int(st)), (int(p), int(p))))
-            elif kind in ("relu", "flatten"):
+            elif kind == "bn":              # bn C eps momentum
+                cfeat = int(parts[1])
+                eps = float(parts[2]) if len(parts) > 2 else 1e-5
+                mom = float(parts[3]) if len(parts) > 3 else 0.1
+                self.running[len(self.layers)] = [np.zeros(cfeat, self.dtype), np.ones(cfeat, self.dtype)]
+                self.layers.append(("bn", pi, pi + 1, eps, mom))
+                pi += 2
+            elif kind == "dropout":         # dropout p seed
+                self.layers.append(("dropout", float(parts[1]), int(parts[2])))
+            elif kind in ("relu", "flatten", "gap"):
                 self.layers.append((kind,))
             else:
                 raise ValueError(kind)
@@ -133,6 +199,27 @@ class Sequential:
             elif kind == "relu":
                 tape.append(("relu", h))
                 h = orc.unary("relu", h)
+            elif kind == "bn":
+                li = self.layers.index(layer)
+                rm, rv = self.running[li]
+                out, rec, mean, var = batchnorm_forward(h, self.params[layer[1]], self.params[layer[2]], layer[3],
+                                                        self.training, rm, rv)
+                if self.training:
+                    self.running[li] = [batchnorm_running_update(rm, mean, layer[4]),
+                                        batchnorm_running_update(rv, var, layer[4])]
+                tape.append(("bn", layer, rec))
+                h = out
+            elif kind == "gap":             # GlobalAvgPool2d(flatten = false): Mean over axes (2,3), keep_dims (pooling.rs:604-623)
+                tape.append(("gap", h.shape))
+                h = orc.reduce("mean", h, [2, 3], keep_dims=True)
+            elif kind == "dropout":         # dropout.rs:100-136; call k of a run uses seed + k * 2^32
+                if self.training and layer[1] != 0.0:
+                    mask = orc.dropout_mask(h.shape, layer[1], layer[2] + (self.dropout_calls << 32), self.dtype)
+                    self.dropout_calls += 1
+                    tape.append(("dropout", mask))
+                    h = orc.binary("mul", h, mask)
+                else:
+                    tape.append(("dropout", None))
             else:
                 tape.append(("flatten", h.shape))
                 h = h.reshape(h.shape[0], -1)
@@ -166,6 +253,16 @@ class Sequential:
                 g = orc.unpool2d(g, h, out, layer[1], layer[2], layer[3], kind == "maxpool")
             elif kind == "relu":
                 g = orc.binary("mul", g, orc.scalar("greater_scalar", rec[1], dt(0)))
+            elif kind == "bn":
+                _, layer, brec = rec
+                g, grads[layer[1]], grads[layer[2]] = batchnorm_backward(g, brec)
+            elif kind == "gap":
+                shape = rec[1]
+                g = orc.scalar("mul_scalar", g, dt(1.0 / float(shape[2] * shape[3])))     # Mean::gradient, keep_dims
+                g = orc.materialize(g, shape, (shape[1], 1, 0, 0))
+            elif kind == "dropout":
+                if rec[1] is not None:
+                    g = orc.binary("mul", g, rec[1])                                      # Mul::gradient wrt the input
             else:
                 g = g.reshape(rec[1])
         return loss.item(), grads
