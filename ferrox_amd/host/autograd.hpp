@@ -100,6 +100,77 @@ template <typename T> struct Mul : Operator<T> {  // src/ops/basic.rs:175-215
     const char* name() const override { return "Mul"; }
 };
 
+template <typename T> struct Sub : Operator<T> {  // src/ops/basic.rs:130-169
+    Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->sub(*in[1]); }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        Tensor<T> g2 = g->neg();
+        Tensor<T> g1 = std::move(g);
+        reduce_gradient_for_broadcasting(g1, in[0]->shape());
+        reduce_gradient_for_broadcasting(g2, in[1]->shape());
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(g1));
+        r.push_back(std::move(g2));
+        return r;
+    }
+    size_t num_inputs() const override { return 2; }
+    const char* name() const override { return "Sub"; }
+};
+
+template <typename T> struct Div : Operator<T> {  // src/ops/basic.rs:221-272 (output cached: the gradient reuses x/y)
+    Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->div(*in[1]); }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out) const override {
+        Tensor<T> recomputed;
+        if (!out) {
+            recomputed = compute(in);
+            out = recomputed.get();
+        }
+        Tensor<T> g1 = g->div(*in[1]);
+        reduce_gradient_for_broadcasting(g1, in[0]->shape());
+        Tensor<T> q = out->div(*in[1]);
+        Tensor<T> nq = q->neg();
+        Tensor<T> g2 = g->mul(*nq);
+        reduce_gradient_for_broadcasting(g2, in[1]->shape());
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(g1));
+        r.push_back(std::move(g2));
+        return r;
+    }
+    size_t num_inputs() const override { return 2; }
+    bool cache_output() const override { return true; }
+    const char* name() const override { return "Div"; }
+};
+
+template <typename T> struct AddScalar : Operator<T> {  // src/ops/scalar.rs (AddScalar): the gradient passes through
+    T scalar;
+    explicit AddScalar(T s) : scalar(s) {}
+    Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->add_scalar(scalar); }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>&, const HipStorage<T>*) const override {
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(g));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    const char* name() const override { return "AddScalar"; }
+};
+
+template <typename T> struct Sqrt : Operator<T> {  // src/ops/unary.rs:107-151: g / (2 * sqrt(x)), from the cached output
+    Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->sqrt(); }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out) const override {
+        Tensor<T> recomputed;
+        if (!out) {
+            recomputed = compute(in);
+            out = recomputed.get();
+        }
+        Tensor<T> den = out->mul_scalar(T(2));
+        std::vector<Tensor<T>> r;
+        r.push_back(g->div(*den));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    bool cache_output() const override { return true; }
+    const char* name() const override { return "Sqrt"; }
+};
+
 template <typename T> struct MatMul : Operator<T> {  // src/ops/matrix.rs:17-64
     Tensor<T> compute(const TensorRefs<T>& in) const override {
         if (in[0]->ndim() != 2 || in[1]->ndim() != 2) throw Error("MatMul requires 2D tensors (matrices)");
@@ -235,6 +306,8 @@ template <typename T> struct Mean : Operator<T> {  // src/ops/reduction.rs:141-2
     bool has_axes = false;
     std::vector<size_t> axes;
     bool keep_dims = false;
+    Mean() = default;
+    Mean(std::vector<size_t> a, bool keep) : has_axes(true), axes(std::move(a)), keep_dims(keep) {}  // Mean::along_axes
     Tensor<T> compute(const TensorRefs<T>& in) const override { return in[0]->mean(has_axes ? &axes : nullptr, keep_dims); }
     std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
         const Shape& is = in[0]->shape();
@@ -473,6 +546,9 @@ template <typename T> struct Module {
     virtual ~Module() = default;
     virtual NodeId forward(AutoFerroxEngine<T>& g, NodeId input) = 0;
     virtual std::vector<NodeId> parameters() const { return {}; }
+    virtual void set_training(bool) {}
+    // tensors that are not parameters but persist across steps (BatchNorm's running statistics)
+    virtual std::vector<const HipStorage<T>*> state() const { return {}; }
 };
 
 // reshape_and_broadcast, src/nn/layers/utils.rs:6-42
@@ -565,6 +641,116 @@ template <typename T> struct Flatten : Module<T> {  // src/nn/layers/pooling.rs:
         size_t rest = 1;
         for (size_t i = 1; i < s.size(); ++i) rest *= s[i];
         return g.apply_operation(std::make_unique<Reshape<T>>(Shape{s[0], rest}), {input});
+    }
+};
+
+// BatchNorm composed from graph operators exactly as src/nn/layers/norm.rs:167-336 does (weight = gamma, bias = beta,
+// running statistics updated outside the graph with the biased batch variance, norm.rs:127-164).
+template <typename T> struct BatchNorm : Module<T> {
+    size_t num_features;
+    double eps, momentum;
+    bool track_running_stats = true, training = true;
+    NodeId weight = 0, bias = 0;
+    Tensor<T> running_mean, running_var;
+    size_t num_batches_tracked = 0;
+    BatchNorm(AutoFerroxEngine<T>& g, size_t c, double eps_, double mom, const T* w, const T* b) : num_features(c), eps(eps_), momentum(mom) {
+        weight = g.create_variable(HipStorage<T>::from_vec(w, {c}), true);
+        bias = g.create_variable(HipStorage<T>::from_vec(b, {c}), true);
+        running_mean = HipStorage<T>::zeros({c});  // norm.rs:75-84
+        running_var = HipStorage<T>::ones({c});
+    }
+    void set_training(bool t) override { training = t; }
+    std::vector<NodeId> parameters() const override { return {weight, bias}; }
+    std::vector<const HipStorage<T>*> state() const override { return {running_mean.get(), running_var.get()}; }
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
+        if (g.get_tensor(input)->ndim() < 2) throw Error("BatchNorm requires at least 2D input [batch_size, features]");
+        return (training || !track_running_stats) ? forward_training(g, input) : forward_inference(g, input);
+    }
+
+  private:
+    void update_running_stats(const HipStorage<T>& batch_mean, const HipStorage<T>& batch_var) {  // norm.rs:127-164
+        if (!track_running_stats || !training) return;
+        const T mom = (T)momentum, om = (T)(1.0 - momentum);
+        ++num_batches_tracked;
+        {
+            Tensor<T> a = running_mean->mul_scalar(om), b = batch_mean.mul_scalar(mom);
+            running_mean = a->add(*b);
+        }
+        {
+            Tensor<T> a = running_var->mul_scalar(om), b = batch_var.mul_scalar(mom);
+            running_var = a->add(*b);
+        }
+    }
+    NodeId forward_training(AutoFerroxEngine<T>& g, NodeId input) {  // norm.rs:192-259
+        const std::vector<size_t> axes = g.get_tensor(input)->ndim() == 4 ? std::vector<size_t>{0, 2, 3} : std::vector<size_t>{0};
+        const NodeId batch_mean = g.apply_operation(std::make_unique<Mean<T>>(axes, false), {input});
+        const NodeId mean_b = reshape_and_broadcast<T>(batch_mean, input, g);
+        const NodeId centered = g.apply_operation(std::make_unique<Sub<T>>(), {input, mean_b});
+        const NodeId sq = g.apply_operation(std::make_unique<Mul<T>>(), {centered, centered});
+        const NodeId variance = g.apply_operation(std::make_unique<Mean<T>>(axes, false), {sq});
+        const NodeId var_b = reshape_and_broadcast<T>(variance, input, g);
+        if (track_running_stats) update_running_stats(*g.get_tensor(batch_mean), *g.get_tensor(variance));
+        return finish(g, centered, var_b);
+    }
+    NodeId forward_inference(AutoFerroxEngine<T>& g, NodeId input) {  // norm.rs:261-290
+        const NodeId rm = g.create_variable(running_mean->clone_storage(), false);
+        const NodeId rv = g.create_variable(running_var->clone_storage(), false);
+        const NodeId mean_b = reshape_and_broadcast<T>(rm, input, g);
+        const NodeId centered = g.apply_operation(std::make_unique<Sub<T>>(), {input, mean_b});
+        return finish(g, centered, rv);
+    }
+    NodeId finish(AutoFerroxEngine<T>& g, NodeId centered, NodeId variance) {  // norm.rs:292-336
+        const NodeId vpe = g.apply_operation(std::make_unique<AddScalar<T>>((T)eps), {variance});
+        const NodeId sd = g.apply_operation(std::make_unique<Sqrt<T>>(), {vpe});
+        const NodeId sd_b = reshape_and_broadcast<T>(sd, centered, g);
+        const NodeId normalized = g.apply_operation(std::make_unique<Div<T>>(), {centered, sd_b});
+        const NodeId w_b = reshape_and_broadcast<T>(weight, normalized, g);
+        const NodeId scaled = g.apply_operation(std::make_unique<Mul<T>>(), {normalized, w_b});
+        const NodeId b_b = reshape_and_broadcast<T>(bias, normalized, g);
+        return g.apply_operation(std::make_unique<Add<T>>(), {scaled, b_b});
+    }
+};
+
+// GlobalAvgPool2d(flatten = false), src/nn/layers/pooling.rs:604-623: Mean over axes (2, 3) with keep_dims
+template <typename T> struct GlobalAvgPool2d : Module<T> {
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
+        if (g.get_tensor(input)->ndim() != 4) throw Error("GlobalAvgPool2d requires 4D input [batch, channels, height, width]");
+        return g.apply_operation(std::make_unique<Mean<T>>(std::vector<size_t>{2, 3}, true), {input});
+    }
+};
+
+// splitmix64 (Steele, Lea & Flood): element i of a dropout mask takes the 53-bit uniform of splitmix64(seed + i),
+// the same stream as fx_dropout, so host-built and device-built masks agree.
+inline double splitmix64_uniform(uint64_t x) {
+    x += 0x9e3779b97f4a7c15ull;
+    x = (x ^ (x >> 30)) * 0xbf58476d1ce4e5b9ull;
+    x = (x ^ (x >> 27)) * 0x94d049bb133111ebull;
+    x ^= x >> 31;
+    return (double)(x >> 11) * (1.0 / 9007199254740992.0);
+}
+
+// Dropout, src/nn/layers/dropout.rs:56-136: the mask is drawn on the host, one f64 uniform per element, uploaded as
+// a constant node and multiplied in.  (The reference's generator is unseeded; call k here uses seed + k * 2^32.)
+template <typename T> struct Dropout : Module<T> {
+    double p;
+    uint64_t seed, calls = 0;
+    bool training = true;
+    Dropout(double p_, uint64_t seed_) : p(p_), seed(seed_) {
+        if (!(p >= 0.0 && p <= 1.0)) throw Error("Dropout probability must be between 0.0 and 1.0");
+    }
+    void set_training(bool t) override { training = t; }
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
+        if (!training || p == 0.0) return input;
+        const Shape shape = g.get_tensor(input)->shape();
+        if (p == 1.0) return g.create_variable(HipStorage<T>::zeros(shape), false);
+        const size_t n = numel(shape);
+        const double keep = 1.0 - p;
+        const T scale = (T)(1.0 / keep);
+        std::vector<T> mask(n);
+        const uint64_t s = seed + (calls++ << 32);
+        for (size_t i = 0; i < n; ++i) mask[i] = splitmix64_uniform(s + i) < keep ? scale : T(0);
+        const NodeId m = g.create_variable(HipStorage<T>::from_vec(mask.data(), shape), false);
+        return g.apply_operation(std::make_unique<Mul<T>>(), {input, m});
     }
 };
 

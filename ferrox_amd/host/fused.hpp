@@ -8,6 +8,8 @@
 //   Conv2d   : conv, bias (+ReLU) in place (conv2d.rs:203-213 materialises the broadcast bias first); backward
 //              skips the data gradient of an input that needs none (the first layer)
 //   CCELoss  : one forward and one backward kernel (classification.rs:191-257 builds 7 nodes)
+//   BatchNorm: statistics (+ running update), normalise and backward kernels (norm.rs:192-336 builds ~15 nodes);
+//              GlobalAvgPool2d as one reduction; Dropout with the mask drawn on the device
 //   Adam/SGD : one in-place kernel per parameter (adam.rs:288-358 runs ~14 and clones the parameter and moments)
 #pragma once
 #include "autograd.hpp"
@@ -32,6 +34,18 @@ template <typename T> struct FusedApi;
         static int conv_bias(fx_ctx* c, const T* x, const T* w, const T* b, T* y, const int64_t* d, int act) {         \
             return fx_conv2d_fwd_bias_act_##S(c, x, w, b, y, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9], d[10], act, nullptr, 0); \
         }                                                                                                              \
+        static int bn_stats(fx_ctx* c, const T* x, T* m, T* v, T* rm, T* rv, double mom, int64_t o, int64_t C, int64_t i) { \
+            return fx_batchnorm_stats_##S(c, x, m, v, rm, rv, mom, o, C, i);                                           \
+        }                                                                                                              \
+        static int bn_fwd(fx_ctx* c, const T* x, const T* m, const T* v, const T* g, const T* b, double eps, T* y, int64_t o, int64_t C, int64_t i) { \
+            return fx_batchnorm_fwd_##S(c, x, m, v, g, b, eps, y, o, C, i);                                            \
+        }                                                                                                              \
+        static int bn_bwd(fx_ctx* c, const T* dy, const T* x, const T* m, const T* v, const T* g, double eps, T* dx, T* dg, T* db, \
+                          int64_t o, int64_t C, int64_t i, int batch_stats) {                                         \
+            return fx_batchnorm_bwd_##S(c, dy, x, m, v, g, eps, dx, dg, db, o, C, i, batch_stats);                     \
+        }                                                                                                              \
+        static int dropout(fx_ctx* c, const T* x, T* mask, T* y, int64_t n, double p, uint64_t seed) { return fx_dropout_##S(c, x, mask, y, n, p, seed); } \
+        static int rmean(fx_ctx* c, const T* i, T* o, int64_t ou, int64_t ax, int64_t in) { return fx_reduce_mean_##S(c, i, o, ou, ax, in); } \
     };
 FERROX_FUSED_API(float, f32)
 FERROX_FUSED_API(double, f64)
@@ -160,6 +174,148 @@ template <typename T> struct Conv2dFused : Module<T> {
         return g.apply_operation(std::make_unique<Conv2dFusedOp<T>>(stride, padding, relu), {input, weight, bias});
     }
     std::vector<NodeId> parameters() const override { return {weight, bias}; }
+};
+
+// BatchNorm as three kernels (statistics + running update, normalise, backward) instead of ~15 graph nodes.
+// inputs: x [N, C, ...], gamma [C], beta [C].  The module's running statistics are updated in place by the
+// statistics kernel (training) or read (inference).
+template <typename T> struct BatchNormFusedOp : Operator<T> {
+    double eps, momentum;
+    bool batch_stats;                         // training (or no running statistics): statistics of this batch
+    HipStorage<T>*running_mean, *running_var;  // owned by the module; null when not tracked
+    mutable Tensor<T> mean, var;               // batch statistics, kept for the backward pass
+    BatchNormFusedOp(double eps_, double mom, bool batch, HipStorage<T>* rm, HipStorage<T>* rv)
+        : eps(eps_), momentum(mom), batch_stats(batch), running_mean(rm), running_var(rv) {}
+    static void view(const Shape& s, int64_t& outer, int64_t& C, int64_t& inner) {
+        outer = (int64_t)s[0];
+        C = (int64_t)s[1];
+        inner = 1;
+        for (size_t i = 2; i < s.size(); ++i) inner *= (int64_t)s[i];
+    }
+    Tensor<T> compute(const TensorRefs<T>& in) const override {
+        const Shape& xs = in[0]->shape();
+        if (xs.size() < 2) throw Error("BatchNorm requires at least 2D input [batch_size, features]");
+        int64_t outer, C, inner;
+        view(xs, outer, C, inner);
+        const T *m, *v;
+        if (batch_stats) {
+            mean = HipStorage<T>::alloc({(size_t)C});
+            var = HipStorage<T>::alloc({(size_t)C});
+            fx_ok(FusedApi<T>::bn_stats(fused_ctx(), in[0]->data(), mean->data(), var->data(), running_mean ? running_mean->data() : nullptr,
+                                        running_var ? running_var->data() : nullptr, momentum, outer, C, inner));
+            m = mean->data();
+            v = var->data();
+        } else {
+            m = running_mean->data();
+            v = running_var->data();
+        }
+        Tensor<T> y = HipStorage<T>::alloc(xs);
+        fx_ok(FusedApi<T>::bn_fwd(fused_ctx(), in[0]->data(), m, v, in[1]->data(), in[2]->data(), eps, y->data(), outer, C, inner));
+        return y;
+    }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out) const override {
+        return gradient_needs(std::move(g), in, out, {true, true, true});
+    }
+    std::vector<Tensor<T>> gradient_needs(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*, const std::vector<bool>& needs) const override {
+        const Shape& xs = in[0]->shape();
+        int64_t outer, C, inner;
+        view(xs, outer, C, inner);
+        std::vector<Tensor<T>> r(3);
+        if (needs[0]) r[0] = HipStorage<T>::alloc(xs);
+        r[1] = HipStorage<T>::alloc({(size_t)C});
+        r[2] = HipStorage<T>::alloc({(size_t)C});
+        const T* m = batch_stats ? mean->data() : running_mean->data();
+        const T* v = batch_stats ? var->data() : running_var->data();
+        fx_ok(FusedApi<T>::bn_bwd(fused_ctx(), g->data(), in[0]->data(), m, v, in[1]->data(), eps, needs[0] ? r[0]->data() : nullptr,
+                                  r[1]->data(), r[2]->data(), outer, C, inner, batch_stats ? 1 : 0));
+        return r;
+    }
+    size_t num_inputs() const override { return 3; }
+    const char* name() const override { return "BatchNormFused"; }
+};
+
+template <typename T> struct BatchNormFused : Module<T> {
+    double eps, momentum;
+    bool track_running_stats = true, training = true;
+    NodeId weight = 0, bias = 0;
+    Tensor<T> running_mean, running_var;
+    BatchNormFused(AutoFerroxEngine<T>& g, size_t c, double eps_, double mom, const T* w, const T* b) : eps(eps_), momentum(mom) {
+        weight = g.create_variable(HipStorage<T>::from_vec(w, {c}), true);
+        bias = g.create_variable(HipStorage<T>::from_vec(b, {c}), true);
+        running_mean = HipStorage<T>::zeros({c});
+        running_var = HipStorage<T>::ones({c});
+    }
+    void set_training(bool t) override { training = t; }
+    std::vector<NodeId> parameters() const override { return {weight, bias}; }
+    std::vector<const HipStorage<T>*> state() const override { return {running_mean.get(), running_var.get()}; }
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
+        const bool batch = training || !track_running_stats;
+        const bool update = training && track_running_stats;
+        return g.apply_operation(std::make_unique<BatchNormFusedOp<T>>(eps, momentum, batch, (update || !batch) ? running_mean.get() : nullptr,
+                                                                       (update || !batch) ? running_var.get() : nullptr),
+                                 {input, weight, bias});
+    }
+};
+
+// GlobalAvgPool2d as one reduction over the contiguous H*W run of every (n, c) instead of one per axis
+template <typename T> struct GlobalAvgPoolFusedOp : Operator<T> {
+    Tensor<T> compute(const TensorRefs<T>& in) const override {
+        const Shape& s = in[0]->shape();
+        if (s.size() != 4) throw Error("GlobalAvgPool2d requires 4D input [batch, channels, height, width]");
+        Tensor<T> y = HipStorage<T>::alloc({s[0], s[1], 1, 1});
+        fx_ok(FusedApi<T>::rmean(fused_ctx(), in[0]->data(), y->data(), (int64_t)(s[0] * s[1]), (int64_t)(s[2] * s[3]), 1));
+        return y;
+    }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {  // Mean::gradient
+        const Shape& s = in[0]->shape();
+        Tensor<T> e = g->mul_scalar((T)(1.0 / (double)(s[2] * s[3])));
+        e->broadcast_to(s);
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(e));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    const char* name() const override { return "GlobalAvgPoolFused"; }
+};
+template <typename T> struct GlobalAvgPoolFused : Module<T> {
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
+        return g.apply_operation(std::make_unique<GlobalAvgPoolFusedOp<T>>(), {input});
+    }
+};
+
+// Dropout with the mask drawn on the device (same stream as the host-built mask of Dropout)
+template <typename T> struct DropoutFusedOp : Operator<T> {
+    double p;
+    uint64_t seed;
+    mutable Tensor<T> mask;
+    DropoutFusedOp(double p_, uint64_t s) : p(p_), seed(s) {}
+    Tensor<T> compute(const TensorRefs<T>& in) const override {
+        mask = HipStorage<T>::alloc(in[0]->shape());
+        Tensor<T> y = HipStorage<T>::alloc(in[0]->shape());
+        fx_ok(FusedApi<T>::dropout(fused_ctx(), in[0]->data(), mask->data(), y->data(), (int64_t)in[0]->size(), p, seed));
+        return y;
+    }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>&, const HipStorage<T>*) const override {
+        std::vector<Tensor<T>> r;
+        r.push_back(g->mul(*mask));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    const char* name() const override { return "DropoutFused"; }
+};
+template <typename T> struct DropoutFused : Module<T> {
+    double p;
+    uint64_t seed, calls = 0;
+    bool training = true;
+    DropoutFused(double p_, uint64_t seed_) : p(p_), seed(seed_) {
+        if (!(p >= 0.0 && p <= 1.0)) throw Error("Dropout probability must be between 0.0 and 1.0");
+    }
+    void set_training(bool t) override { training = t; }
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
+        if (!training || p == 0.0) return input;
+        if (p == 1.0) return g.create_variable(HipStorage<T>::zeros(g.get_tensor(input)->shape()), false);
+        return g.apply_operation(std::make_unique<DropoutFusedOp<T>>(p, seed + (calls++ << 32)), {input});
+    }
 };
 
 template <typename T> NodeId cce_loss_fused(AutoFerroxEngine<T>& g, NodeId predictions, NodeId targets) {

@@ -25,6 +25,10 @@ struct ModelBase {
     virtual void get_grad(int i, void* host) const = 0;
     virtual void forward_only(void* host_out) = 0;
     virtual int64_t output_numel() = 0;
+    virtual void set_training(bool t) = 0;
+    virtual int num_state() const = 0;
+    virtual int64_t state_numel(int i) const = 0;
+    virtual void get_state(int i, void* host) const = 0;
 };
 
 std::vector<std::string> split(const std::string& s, char sep) {
@@ -85,6 +89,25 @@ template <typename T> struct Model : ModelBase {
                 size_t k, st, p;
                 ss >> k >> st >> p;
                 layers.push_back(std::make_unique<Pool2d<T>>(kind == "maxpool", k, st, p));
+            } else if (kind == "bn") {  // bn C [eps [momentum]]
+                size_t c;
+                double eps = 1e-5, mom = 0.1;
+                ss >> c;
+                if (!(ss >> eps)) eps = 1e-5;
+                else if (!(ss >> mom)) mom = 0.1;
+                const T* w = next();
+                const T* b = next();
+                if (fused) layers.push_back(std::make_unique<BatchNormFused<T>>(graph, c, eps, mom, w, b));
+                else layers.push_back(std::make_unique<BatchNorm<T>>(graph, c, eps, mom, w, b));
+            } else if (kind == "gap") {
+                if (fused) layers.push_back(std::make_unique<GlobalAvgPoolFused<T>>());
+                else layers.push_back(std::make_unique<GlobalAvgPool2d<T>>());
+            } else if (kind == "dropout") {  // dropout p seed
+                double p = 0.5;
+                uint64_t seed = 0;
+                ss >> p >> seed;
+                if (engine == 1) layers.push_back(std::make_unique<Dropout<T>>(p, seed));
+                else layers.push_back(std::make_unique<DropoutFused<T>>(p, seed));
             } else if (kind == "relu") layers.push_back(std::make_unique<ReLU<T>>());
             else if (kind == "flatten") layers.push_back(std::make_unique<Flatten<T>>());
             else throw Error("unknown layer '" + kind + "'");
@@ -105,6 +128,21 @@ template <typename T> struct Model : ModelBase {
             else opt = std::make_unique<Adam<T>>((T)lr, (T)b1, (T)b2, (T)eps, (T)wd);
         } else throw Error("unknown optimizer '" + kind + "'");
         opt->params = params;
+    }
+    void set_training(bool t) override {
+        for (auto& l : layers) l->set_training(t);
+    }
+    std::vector<const HipStorage<T>*> all_state() const {
+        std::vector<const HipStorage<T>*> r;
+        for (auto& l : layers)
+            for (const HipStorage<T>* s : l->state()) r.push_back(s);
+        return r;
+    }
+    int num_state() const override { return (int)all_state().size(); }
+    int64_t state_numel(int i) const override { return (int64_t)all_state().at(i)->size(); }
+    void get_state(int i, void* host) const override {
+        std::vector<T> v = all_state().at(i)->to_vec();
+        std::memcpy(host, v.data(), v.size() * sizeof(T));
     }
     int num_params() const override { return (int)params.size(); }
     int64_t param_numel(int i) const override { return (int64_t)graph.get_tensor(params.at(i))->size(); }
@@ -222,6 +260,20 @@ int64_t fxh_model_output_numel(void* m) {
 }
 int fxh_model_forward(void* m, void* host_out) {
     return guarded([&] { static_cast<ModelBase*>(m)->forward_only(host_out); });
+}
+// training / evaluation mode of every layer (BatchNorm statistics, Dropout), Module::set_training
+int fxh_model_set_training(void* m, int training) {
+    return guarded([&] { static_cast<ModelBase*>(m)->set_training(training != 0); });
+}
+// persistent non-parameter tensors in layer order (BatchNorm: running mean, running variance)
+int fxh_model_num_state(void* m) { return static_cast<ModelBase*>(m)->num_state(); }
+int64_t fxh_model_state_numel(void* m, int i) {
+    int64_t n = -1;
+    guarded([&] { n = static_cast<ModelBase*>(m)->state_numel(i); });
+    return n;
+}
+int fxh_model_get_state(void* m, int i, void* host) {
+    return guarded([&] { static_cast<ModelBase*>(m)->get_state(i, host); });
 }
 int fxh_pool_stats(int dtype, fx_pool_stats* out) {
     return guarded([&] { fx_ok(fx_pool_stats_get(BackendManager::get().ctx(), dtype, out)); });

@@ -35,6 +35,11 @@ lib.fxh_model_get_grad.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
 lib.fxh_model_output_numel.argtypes = [C.c_void_p]
 lib.fxh_model_output_numel.restype = C.c_int64
 lib.fxh_model_forward.argtypes = [C.c_void_p, C.c_void_p]
+lib.fxh_model_set_training.argtypes = [C.c_void_p, C.c_int]
+lib.fxh_model_num_state.argtypes = [C.c_void_p]
+lib.fxh_model_state_numel.argtypes = [C.c_void_p, C.c_int]
+lib.fxh_model_state_numel.restype = C.c_int64
+lib.fxh_model_get_state.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
 lib.fxh_pool_stats.argtypes = [C.c_int, C.POINTER(capi.PoolStats)]
 
 
@@ -62,7 +67,8 @@ def pool_stats(dtype=np.float32):
 
 
 class Model:
-    """spec: 'conv CIN COUT K S P; relu; flatten; linear IN OUT; ...'  optimizer: 'sgd LR' | 'adam LR B1 B2 EPS WD'."""
+    """spec: 'conv CIN COUT K S P; bn C EPS MOMENTUM; relu; maxpool K S P; gap; flatten; linear IN OUT; dropout P SEED; ...'
+    optimizer: 'sgd LR' | 'adam LR B1 B2 EPS WD'."""
 
     def __init__(self, spec, params, optimizer, dtype=np.float32, literal_engine=True, fused=False):
         """literal_engine: keep the reference engine's per-node deep clones; fused: fused layers, loss and optimizer."""
@@ -105,6 +111,19 @@ class Model:
     def grad(self, i):
         out = np.empty(self.shapes[i], self.dtype)
         _check(lib.fxh_model_get_grad(self.h, i, out.ctypes.data))
+        return out
+
+    def set_training(self, training):
+        """Module::set_training on every layer (BatchNorm statistics, Dropout)."""
+        _check(lib.fxh_model_set_training(self.h, 1 if training else 0))
+
+    def state(self):
+        """Persistent non-parameter tensors in layer order (BatchNorm: running mean, running variance)."""
+        out = []
+        for i in range(lib.fxh_model_num_state(self.h)):
+            a = np.empty(lib.fxh_model_state_numel(self.h, i), self.dtype)
+            _check(lib.fxh_model_get_state(self.h, i, a.ctypes.data))
+            out.append(a)
         return out
 
     def forward(self):
