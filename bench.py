@@ -158,6 +158,33 @@ def bench_bandwidth(ctx, iters=20, warmup=3):
         out["pooling"][f"{name}_grad_f32"] = {"ms": ms, "GBps": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
         del pooled, pg
     del px
+    # BatchNorm on [256, 128, 56, 56] f32 (411 MB per array, larger than the last-level cache) and dropout on 2^28:
+    # algorithmic bytes = x (statistics), x + y (forward), 2 reads of (dy, x) + dx (backward), x + mask + y (dropout)
+    out["normalisation"] = {}
+    bshape = (256, 128, 56, 56)
+    bx = ctx.normal(bshape, 13, 0.5, 2.0)
+    bg = ctx.normal(bshape, 14, 0.0, 1.0)
+    gamma, beta = ctx.fill((128,), 1.0), ctx.fill((128,), 0.0)
+    mean, var = ctx.batchnorm_stats(bx)
+    by, bdx, dgm, dbt = ctx.empty(bshape), ctx.empty(bshape), ctx.empty((128,)), ctx.empty((128,))
+    view = (256, 128, 56 * 56)
+    bn_cases = {
+        "batchnorm_stats": (1, lambda: capi.check(capi.lib.fx_batchnorm_stats_f32(ctx.h, bx.ptr, mean.ptr, var.ptr, None, None, 0.1, *view))),
+        "batchnorm_fwd": (2, lambda: capi.check(capi.lib.fx_batchnorm_fwd_f32(ctx.h, bx.ptr, mean.ptr, var.ptr, gamma.ptr, beta.ptr,
+                                                                            1e-5, by.ptr, *view))),
+        "batchnorm_bwd": (5, lambda: capi.check(capi.lib.fx_batchnorm_bwd_f32(ctx.h, bg.ptr, bx.ptr, mean.ptr, var.ptr, gamma.ptr, 1e-5,
+                                                                            bdx.ptr, dgm.ptr, dbt.ptr, *view, 1))),
+    }
+    for name, (passes, fn) in bn_cases.items():
+        ms = time_stream(ctx, fn, 10, 2)
+        nbytes = passes * 4 * bx.size
+        out["normalisation"][f"{name}_f32"] = {"ms": ms, "GBps": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    del bx, bg, by, bdx
+    dxx = ctx.uniform((n,), 15, -1.0, 1.0)
+    dm, dy_ = ctx.empty((n,)), ctx.empty((n,))
+    ms = time_stream(ctx, lambda: capi.check(capi.lib.fx_dropout_f32(ctx.h, dxx.ptr, dm.ptr, dy_.ptr, n, 0.3, 99)), 10, 2)
+    out["normalisation"]["dropout_f32"] = {"ms": ms, "GBps": 3 * 4 * n / ms / 1e6, "frac_hbm": 3 * 4 * n / ms / 1e6 / PEAK_HBM_GBS}
+    del dxx, dm, dy_
     g = ctx.uniform((n,), 7, -4.0, 4.0)
     x = ctx.uniform((n,), 8, -4.0, 4.0)
     s = ctx.unary("sigmoid", x)
@@ -184,6 +211,10 @@ TRAIN_CONFIGS = {
                    classes=10, opt="adam 0.001 0.9 0.999 1e-08 0", seed=5),
     "C2_mlp": dict(spec="linear 784 256; relu; linear 256 128; relu; linear 128 10", in_shape=(256, 784), classes=10,
                    opt="sgd 0.01", seed=2),
+    # CNNClassifier of the reference's examples (examples/common/models.rs:200-318) for 32x32 RGB images
+    "cnn_classifier": dict(spec="conv 3 32 3 1 1; bn 32 0.001 0.1; relu; conv 32 64 3 1 1; bn 64 0.001 0.1; relu; gap; flatten; "
+                                "linear 64 64; relu; dropout 0.3 23; linear 64 10", in_shape=(256, 3, 32, 32), classes=10,
+                           opt="adam 0.001 0.9 0.999 1e-08 0", seed=6),
 }
 
 
@@ -199,6 +230,8 @@ def make_train_problem(cfg, dtype):
         elif p[0] == "conv":
             ci, co, k = int(p[1]), int(p[2]), int(p[3])
             params += [rng.uniform(-1, 1, (co, ci, k, k)).astype(dtype) * dtype(np.sqrt(6.0 / (ci * k * k))), np.zeros(co, dtype)]
+        elif p[0] == "bn":  # weight ones, bias zeros (nn/layers/norm.rs:62-100)
+            params += [np.ones(int(p[1]), dtype), np.zeros(int(p[1]), dtype)]
     x = rng.standard_normal(cfg["in_shape"]).astype(dtype)
     y = np.eye(cfg["classes"], dtype=dtype)[rng.integers(0, cfg["classes"], cfg["in_shape"][0])]
     return params, x, y
@@ -223,7 +256,7 @@ def bench_train_steps(steps=30, warmup=5, cpu=True, reference_pool=False, only=N
     out = {}
     for name, cfg in TRAIN_CONFIGS.items():
         for dtype in (np.float32, np.float64):
-            if name == "C2_mlp" and dtype == np.float64:
+            if name in ("C2_mlp", "cnn_classifier") and dtype == np.float64:
                 continue
             if only and (only[0] != name or only[1] != np.dtype(dtype).name):
                 continue
@@ -254,7 +287,7 @@ def bench_train_steps(steps=30, warmup=5, cpu=True, reference_pool=False, only=N
                 ref = otrain.Sequential(cfg["spec"], params, dtype)
                 kind, *nums = cfg["opt"].split()
                 opt = otrain.SGD(float(nums[0])) if kind == "sgd" else otrain.Adam(*[float(v) for v in nums])
-                n_cpu = 3
+                n_cpu = 1 if name == "cnn_classifier" else 3
                 t0 = time.perf_counter()
                 for _ in range(n_cpu):
                     _, grads = ref.loss_and_grads(x, y)

@@ -109,8 +109,12 @@ int fwd_tile(fx_ctx* c, const T* x, const T* w, T* y, const Dims& d, const T* bi
     const ConvShape s = make_shape(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
     MatLoader<T, true> al{w, K, (int)M};
     ConvFwdB<T, FAST> bl{x, s, (int)N};
-    NchwStore<T> ep{y, (int)d.Cout, (int)(d.oh * d.ow), (int)N, s.div_L, bias, relu};
     const int kps = (int)(fx::ceil_div(K, Cfg::BK) * Cfg::BK);
+    if (bias) {
+        NchwStore<T, true> ep{y, (int)d.Cout, (int)(d.oh * d.ow), (int)N, s.div_L, bias, relu};
+        return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
+    }
+    NchwStore<T> ep{y, (int)d.Cout, (int)(d.oh * d.ow), (int)N, s.div_L};
     return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
 }
 

@@ -25,7 +25,11 @@ int run(fx_ctx* c, i64 M, i64 N, i64 K, const T* A, const T* B, T* C, const T* b
     int kps = 0;
     const int splits = choose_splits(tiles, K, Cfg::BK, (i64)c->num_cus * 2, &kps);
     if (splits == 1) {
-        MatStore<T> ep{C, N, 0, (int)M, (int)N, bias, relu};  // bias (+ReLU) in the epilogue
+        if (bias) {  // bias (+ReLU) in the epilogue
+            MatStore<T, true> ep{C, N, 0, (int)M, (int)N, bias, relu};
+            return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
+        }
+        MatStore<T> ep{C, N, 0, (int)M, (int)N};
         return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
     }
     *bias_pending = bias != nullptr;  // split-K: the caller adds the bias after the ordered sum

@@ -381,9 +381,10 @@ template <typename T> struct ConvWgradB {
 
 // ---- epilogues ---------------------------------------------------------------------------------------------
 // An epilogue maps a column n to a base pointer (col) and stores row m at q[m * row_stride]; xform(m, n, v) is
-// applied to every stored value (identity unless a bias vector is attached: v + bias, then ReLU when relu != 0).
+// applied to every stored value: identity, or with BIAS (a compile-time switch, so that the plain kernels carry no
+// trace of it) v + bias, then ReLU when relu != 0.
 // Row-major matrix (also used for split-K partials: split z goes to p + z*split_stride).  bias is per column n.
-template <typename T> struct MatStore {
+template <typename T, bool BIAS = false> struct MatStore {
     T* p;
     i64 ld, split_stride;
     int M, N;
@@ -394,7 +395,7 @@ template <typename T> struct MatStore {
     __device__ __forceinline__ i64 row_stride() const { return ld; }
     __device__ __forceinline__ T* col(int n, int split) const { return p + (i64)split * split_stride + n; }
     __device__ __forceinline__ T xform(int, int n, T v) const {
-        if (bias) {
+        if constexpr (BIAS) {
             v = v + bias[n];
             if (relu) v = v > T(0) ? v : T(0);
         }
@@ -402,14 +403,14 @@ template <typename T> struct MatStore {
     }
 };
 // NCHW tensor: row m = channel, column n = (b, l) -> p[(b*C + m)*L + l].
-template <typename T> struct NchwStore {  // bias is per row m (channel)
+template <typename T, bool BIAS = false> struct NchwStore {  // bias is per row m (channel)
     T* p;
     int C, L, N;
     FastDiv div_L;
     const T* bias = nullptr;
     int relu = 0;
     __device__ __forceinline__ T xform(int m, int, T v) const {
-        if (bias) {
+        if constexpr (BIAS) {
             v = v + bias[m];
             if (relu) v = v > T(0) ? v : T(0);
         }
