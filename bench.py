@@ -171,8 +171,8 @@ def bench_bandwidth(ctx, iters=20, warmup=3):
     bn_cases = {
         "batchnorm_stats": (1, lambda: capi.check(capi.lib.fx_batchnorm_stats_f32(ctx.h, bx.ptr, mean.ptr, var.ptr, None, None, 0.1, *view))),
         "batchnorm_fwd": (2, lambda: capi.check(capi.lib.fx_batchnorm_fwd_f32(ctx.h, bx.ptr, mean.ptr, var.ptr, gamma.ptr, beta.ptr,
-                                                                            1e-5, by.ptr, *view))),
-        "batchnorm_bwd": (5, lambda: capi.check(capi.lib.fx_batchnorm_bwd_f32(ctx.h, bg.ptr, bx.ptr, mean.ptr, var.ptr, gamma.ptr, 1e-5,
+                                                                            1e-5, by.ptr, *view, 0))),
+        "batchnorm_bwd": (5, lambda: capi.check(capi.lib.fx_batchnorm_bwd_f32(ctx.h, bg.ptr, bx.ptr, None, mean.ptr, var.ptr, gamma.ptr, 1e-5,
                                                                             bdx.ptr, dgm.ptr, dbt.ptr, *view, 1))),
     }
     for name, (passes, fn) in bn_cases.items():

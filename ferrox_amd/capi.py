@@ -117,8 +117,8 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_reduce_prod_{_s}", _vp, _vp, _vp, _i64, _i64, _i64)
     _sig(f"fx_in_range_{_s}", _vp, _vp, _ct, _ct, _vp, _i64)
     _sig(f"fx_batchnorm_stats_{_s}", _vp, _vp, _vp, _vp, _vp, _vp, C.c_double, _i64, _i64, _i64)
-    _sig(f"fx_batchnorm_fwd_{_s}", _vp, _vp, _vp, _vp, _vp, _vp, C.c_double, _vp, _i64, _i64, _i64)
-    _sig(f"fx_batchnorm_bwd_{_s}", _vp, _vp, _vp, _vp, _vp, _vp, C.c_double, _vp, _vp, _vp, _i64, _i64, _i64, _int)
+    _sig(f"fx_batchnorm_fwd_{_s}", _vp, _vp, _vp, _vp, _vp, _vp, C.c_double, _vp, _i64, _i64, _i64, _int)
+    _sig(f"fx_batchnorm_bwd_{_s}", _vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_double, _vp, _vp, _vp, _i64, _i64, _i64, _int)
     _sig(f"fx_dropout_{_s}", _vp, _vp, _vp, _vp, _i64, C.c_double, _u64)
     _sig(f"fx_maxpool2d_{_s}", _vp, _vp, _vp, *([_i64] * 10))
     _sig(f"fx_avgpool2d_{_s}", _vp, _vp, _vp, *([_i64] * 10))
@@ -453,18 +453,20 @@ class Context:
                                                    float(momentum), outer, Cc, inner))
         return mean, var
 
-    def batchnorm_fwd(self, x, mean, var, gamma, beta, eps):
+    def batchnorm_fwd(self, x, mean, var, gamma, beta, eps, relu=False):
         outer, Cc, inner = self._channel_view(x.shape)
         y = self.empty(x.shape, x.dtype)
         check(self._fn("batchnorm_fwd", x.dtype)(self.h, x.ptr, mean.ptr, var.ptr, gamma.ptr, beta.ptr, float(eps), y.ptr,
-                                                 outer, Cc, inner))
+                                                 outer, Cc, inner, 1 if relu else 0))
         return y
 
-    def batchnorm_bwd(self, dy, x, mean, var, gamma, eps, batch_stats=True, need_dx=True):
+    def batchnorm_bwd(self, dy, x, mean, var, gamma, eps, batch_stats=True, need_dx=True, y_act=None):
+        """y_act: the output of batchnorm_fwd(relu=True); dy is then masked where it is zero."""
         outer, Cc, inner = self._channel_view(x.shape)
         dx = self.empty(x.shape, x.dtype) if need_dx else None
         dgamma, dbeta = self.empty((Cc,), x.dtype), self.empty((Cc,), x.dtype)
-        check(self._fn("batchnorm_bwd", x.dtype)(self.h, dy.ptr, x.ptr, mean.ptr, var.ptr, gamma.ptr, float(eps),
+        check(self._fn("batchnorm_bwd", x.dtype)(self.h, dy.ptr, x.ptr, y_act.ptr if y_act is not None else None,
+                                                 mean.ptr, var.ptr, gamma.ptr, float(eps),
                                                  dx.ptr if need_dx else None, dgamma.ptr, dbeta.ptr, outer, Cc, inner,
                                                  1 if batch_stats else 0))
         return dx, dgamma, dbeta

@@ -6,6 +6,7 @@
 //   fwd     y = ((x - mean) / sqrt(var + eps)) * gamma + beta, the composed operations in the composed order
 //           (this file is built without a*b+c contraction), so y equals the composed path bit for bit given mean/var
 //   bwd     two reads of (dy, x): channel sums, then dx = (gamma/std) * (dy - mean(dy) - xc * mean(dy*xc)/std^2)
+//   A ReLU that follows the layer can ride along: fwd applies it in the store, bwd masks dy where the activation is 0.
 // All three are HBM-bound: sizeof(T) * n * {1, 2, 5} bytes.
 //
 // Moments are combined with the pairwise update of Chan, Golub & LeVeque (count, mean, M2): every thread folds
@@ -148,20 +149,27 @@ __global__ __launch_bounds__(256) void bn_stats_column_kernel(const T* __restric
     p[0] = acc.n; p[1] = acc.mean; p[2] = acc.m2;
 }
 
-// one thread per channel: merges `slices` x `per_channel` partial triples in (slice, column) order
+// one wave per channel: lane l folds partial triples l, l + 64, ... (in (slice, column) order), then the lanes merge in a
+// fixed shuffle tree
 template <typename T>
-__global__ __launch_bounds__(256) void bn_stats_final_kernel(const T* __restrict__ part, T* __restrict__ mean, T* __restrict__ var,
-                                                             T* __restrict__ run_mean, T* __restrict__ run_var, T mom, T one_minus_mom,
-                                                             i64 C, i64 per_channel, int slices) {
-    const i64 c = (i64)blockIdx.x * 256 + threadIdx.x;
-    if (c >= C) return;
+__global__ __launch_bounds__(64) void bn_stats_final_kernel(const T* __restrict__ part, T* __restrict__ mean, T* __restrict__ var,
+                                                            T* __restrict__ run_mean, T* __restrict__ run_var, T mom, T one_minus_mom,
+                                                            i64 C, i64 per_channel, int slices) {
+    const i64 c = blockIdx.x;
+    const i64 count = (i64)slices * per_channel;
     Moments<T> acc;
     acc.init();
-    for (int z = 0; z < slices; ++z)
-        for (i64 j = 0; j < per_channel; ++j) {
-            const T* p = part + (((i64)z * C + c) * per_channel + j) * 3;
-            acc.merge_any(p[0], p[1], p[2]);
-        }
+    for (i64 k = threadIdx.x; k < count; k += 64) {
+        const i64 z = k / per_channel, j = k - z * per_channel;
+        const T* p = part + ((z * C + c) * per_channel + j) * 3;
+        acc.merge_any(p[0], p[1], p[2]);
+    }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) {
+        const T on = __shfl_down(acc.n, d, 64), om = __shfl_down(acc.mean, d, 64), o2 = __shfl_down(acc.m2, d, 64);
+        if ((int)threadIdx.x + d < 64) acc.merge_any(on, om, o2);
+    }
+    if (threadIdx.x != 0) return;
     const T m = acc.mean, v = acc.m2 / acc.n;
     mean[c] = m;
     var[c] = v;
@@ -213,14 +221,14 @@ int bn_stats(fx_ctx* c, const T* x, T* mean, T* var, T* run_mean, T* run_var, do
         bn_stats_column_kernel<T><<<dim3((unsigned)col_blocks, (unsigned)sp.slices), dim3(256), 0, c->stream>>>(x, part, outer, Q, sp.rows_per_slice);
     }
     FX_LAUNCH_CHECK();
-    bn_stats_final_kernel<T><<<dim3((unsigned)fx::ceil_div(C, (i64)256)), dim3(256), 0, c->stream>>>(
+    bn_stats_final_kernel<T><<<dim3((unsigned)C), dim3(64), 0, c->stream>>>(
         part, mean, var, run_mean, run_var, (T)momentum, (T)(1.0 - momentum), C, per_channel, (int)sp.slices);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
 
 // ---- forward: y = ((x - mean) / sqrt(var + eps)) * gamma + beta ------------------------------------------------------
-template <typename T, bool VEC>
+template <typename T, bool VEC, bool RELU>
 __global__ __launch_bounds__(256) void bn_fwd_kernel(const T* __restrict__ x, const T* __restrict__ mean, const T* __restrict__ var,
                                                      const T* __restrict__ gamma, const T* __restrict__ beta, T eps, T* __restrict__ y,
                                                      i64 n, uint32_t C, uint32_t inner) {
@@ -232,15 +240,20 @@ __global__ __launch_bounds__(256) void bn_fwd_kernel(const T* __restrict__ x, co
     const T m = mean[c], sd = dev_sqrt<T>(var[c] + eps), g = gamma[c], b = beta[c];
     vec_t v = *reinterpret_cast<const vec_t*>(x + i);
 #pragma unroll
-    for (int u = 0; u < V; ++u) v[u] = ((v[u] - m) / sd) * g + b;
+    for (int u = 0; u < V; ++u) {
+        T r = ((v[u] - m) / sd) * g + b;
+        if (RELU) r = r > T(0) ? r : T(0);  // ReLU as the forward kernel does it: x > 0 ? x : 0
+        v[u] = r;
+    }
     *reinterpret_cast<vec_t*>(y + i) = v;
 }
 
 template <typename T>
 int bn_fwd(fx_ctx* c, const T* x, const T* mean, const T* var, const T* gamma, const T* beta, double eps, T* y, i64 outer, i64 C,
-           i64 inner) {
+           i64 inner, int act) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(outer >= 0 && C >= 1 && inner >= 1, "fx_batchnorm_fwd: bad view");
+    FX_REQUIRE(act == 0 || act == 1, "fx_batchnorm_fwd: act must be 0 (none) or 1 (relu)");
     const i64 n = outer * C * inner;
     if (n == 0) return FX_OK;
     FX_REQUIRE(x && mean && var && gamma && beta && y, "fx_batchnorm_fwd: null pointer");
@@ -249,17 +262,23 @@ int bn_fwd(fx_ctx* c, const T* x, const T* mean, const T* var, const T* gamma, c
     const bool vec = inner % V == 0 && fx::aligned16(x) && fx::aligned16(y);
     const i64 blocks = fx::ceil_div(vec ? n / V : n, 256);
     FX_REQUIRE(blocks <= 0x7fffffff, "fx_batchnorm_fwd: too many elements");
-    if (vec) bn_fwd_kernel<T, true><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(x, mean, var, gamma, beta, (T)eps, y, n, (uint32_t)C, (uint32_t)inner);
-    else bn_fwd_kernel<T, false><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(x, mean, var, gamma, beta, (T)eps, y, n, (uint32_t)C, (uint32_t)inner);
+    const dim3 grid((unsigned)blocks), blk(256);
+    const T e = (T)eps;
+    const uint32_t Cu = (uint32_t)C, iu = (uint32_t)inner;
+    if (vec && act) bn_fwd_kernel<T, true, true><<<grid, blk, 0, c->stream>>>(x, mean, var, gamma, beta, e, y, n, Cu, iu);
+    else if (vec) bn_fwd_kernel<T, true, false><<<grid, blk, 0, c->stream>>>(x, mean, var, gamma, beta, e, y, n, Cu, iu);
+    else if (act) bn_fwd_kernel<T, false, true><<<grid, blk, 0, c->stream>>>(x, mean, var, gamma, beta, e, y, n, Cu, iu);
+    else bn_fwd_kernel<T, false, false><<<grid, blk, 0, c->stream>>>(x, mean, var, gamma, beta, e, y, n, Cu, iu);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
 
 // ---- backward, stage 1: per (slice, column) sums of dy and dy * (x - mean) -------------------------------------------
-template <typename T, bool VEC>
+// MASK: dy is the gradient of relu(y); yact holds relu(y) and dy counts only where yact > 0 (ReLU::gradient, unary.rs:358-375).
+template <typename T, bool VEC, bool MASK>
 __global__ __launch_bounds__(256) void bn_bwd_sums_planar_kernel(const T* __restrict__ dy, const T* __restrict__ x,
-                                                                 const T* __restrict__ mean, T* __restrict__ part, i64 outer, i64 C,
-                                                                 i64 inner, i64 rows_per_slice) {
+                                                                 const T* __restrict__ yact, const T* __restrict__ mean,
+                                                                 T* __restrict__ part, i64 outer, i64 C, i64 inner, i64 rows_per_slice) {
     constexpr int V = VEC ? 16 / (int)sizeof(T) : 1;
     typedef T vec_t __attribute__((ext_vector_type(V)));
     __shared__ T sm[2][256];
@@ -277,6 +296,11 @@ __global__ __launch_bounds__(256) void bn_bwd_sums_planar_kernel(const T* __rest
             const i64 off = (w.o * C + c) * inner + w.iv * V;
             g[u] = *reinterpret_cast<const vec_t*>(dy + off);
             v[u] = *reinterpret_cast<const vec_t*>(x + off);
+            if (MASK) {
+                const vec_t a = *reinterpret_cast<const vec_t*>(yact + off);
+#pragma unroll
+                for (int e = 0; e < V; ++e) g[u][e] = a[e] > T(0) ? g[u][e] : T(0);
+            }
             w.step();
         }
 #pragma unroll
@@ -288,7 +312,13 @@ __global__ __launch_bounds__(256) void bn_bwd_sums_planar_kernel(const T* __rest
     }
     for (; q < pairs; q += 256) {
         const i64 off = (w.o * C + c) * inner + w.iv * V;
-        const vec_t g = *reinterpret_cast<const vec_t*>(dy + off), v = *reinterpret_cast<const vec_t*>(x + off);
+        vec_t g = *reinterpret_cast<const vec_t*>(dy + off);
+        const vec_t v = *reinterpret_cast<const vec_t*>(x + off);
+        if (MASK) {
+            const vec_t a = *reinterpret_cast<const vec_t*>(yact + off);
+#pragma unroll
+            for (int e = 0; e < V; ++e) g[e] = a[e] > T(0) ? g[e] : T(0);
+        }
         w.step();
         s1 = s1 + g;
 #pragma unroll
@@ -314,15 +344,16 @@ __global__ __launch_bounds__(256) void bn_bwd_sums_planar_kernel(const T* __rest
 
 template <typename T>
 __global__ __launch_bounds__(256) void bn_bwd_sums_column_kernel(const T* __restrict__ dy, const T* __restrict__ x,
-                                                                 const T* __restrict__ mean, T* __restrict__ part, i64 outer, i64 Q,
-                                                                 uint32_t inner, i64 rows_per_slice) {
+                                                                 const T* __restrict__ yact, const T* __restrict__ mean,
+                                                                 T* __restrict__ part, i64 outer, i64 Q, uint32_t inner, i64 rows_per_slice) {
     const i64 col = (i64)blockIdx.x * 256 + threadIdx.x, slice = blockIdx.y;
     if (col >= Q) return;
     const i64 o0 = slice * rows_per_slice, o1 = min(outer, o0 + rows_per_slice);
     const T m = mean[col / inner];
     T a = T(0), b = T(0);
     for (i64 o = o0; o < o1; ++o) {
-        const T g = dy[o * Q + col];
+        T g = dy[o * Q + col];
+        if (yact) g = yact[o * Q + col] > T(0) ? g : T(0);
         a = a + g;
         b = dev_fma(g, x[o * Q + col] - m, b);
     }
@@ -330,22 +361,28 @@ __global__ __launch_bounds__(256) void bn_bwd_sums_column_kernel(const T* __rest
     p[0] = a; p[1] = b;
 }
 
-// one thread per channel: dbeta, dgamma and the coefficients of the dx kernel (coef[0..C) = gamma/std,
-// coef[C..2C) = mean(dy), coef[2C..3C) = mean(dy*xc)/std^2)
+// one wave per channel: dbeta, dgamma and the coefficients of the dx kernel (coef[0..C) = gamma/std,
+// coef[C..2C) = mean(dy), coef[2C..3C) = mean(dy*xc)/std^2); partials summed lane-strided, then a fixed shuffle tree
 template <typename T>
-__global__ __launch_bounds__(256) void bn_bwd_final_kernel(const T* __restrict__ part, const T* __restrict__ var,
-                                                           const T* __restrict__ gamma, T eps, T* __restrict__ dgamma,
-                                                           T* __restrict__ dbeta, T* __restrict__ coef, T count, i64 C, i64 per_channel,
-                                                           int slices) {
-    const i64 c = (i64)blockIdx.x * 256 + threadIdx.x;
-    if (c >= C) return;
+__global__ __launch_bounds__(64) void bn_bwd_final_kernel(const T* __restrict__ part, const T* __restrict__ var,
+                                                          const T* __restrict__ gamma, T eps, T* __restrict__ dgamma,
+                                                          T* __restrict__ dbeta, T* __restrict__ coef, T count, i64 C, i64 per_channel,
+                                                          int slices) {
+    const i64 c = blockIdx.x;
+    const i64 np = (i64)slices * per_channel;
     T a = T(0), b = T(0);
-    for (int z = 0; z < slices; ++z)
-        for (i64 j = 0; j < per_channel; ++j) {
-            const T* p = part + (((i64)z * C + c) * per_channel + j) * 2;
-            a = a + p[0];
-            b = b + p[1];
-        }
+    for (i64 k = threadIdx.x; k < np; k += 64) {
+        const i64 z = k / per_channel, j = k - z * per_channel;
+        const T* p = part + ((z * C + c) * per_channel + j) * 2;
+        a = a + p[0];
+        b = b + p[1];
+    }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) {
+        const T oa = __shfl_down(a, d, 64), ob = __shfl_down(b, d, 64);
+        if ((int)threadIdx.x + d < 64) { a = a + oa; b = b + ob; }
+    }
+    if (threadIdx.x != 0) return;
     const T sd = dev_sqrt<T>(var[c] + eps);
     dbeta[c] = a;
     dgamma[c] = b / sd;
@@ -355,17 +392,23 @@ __global__ __launch_bounds__(256) void bn_bwd_final_kernel(const T* __restrict__
 }
 
 // stage 2, batch statistics: dx = (dy - k1 - (x - mean) * k2) * (gamma/std)
-template <typename T, bool VEC>
-__global__ __launch_bounds__(256) void bn_bwd_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ mean,
-                                                        const T* __restrict__ coef, T* __restrict__ dx, i64 n, uint32_t C,
-                                                        uint32_t inner) {
+template <typename T, bool VEC, bool MASK>
+__global__ __launch_bounds__(256) void bn_bwd_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ yact,
+                                                        const T* __restrict__ mean, const T* __restrict__ coef, T* __restrict__ dx, i64 n,
+                                                        uint32_t C, uint32_t inner) {
     constexpr int V = VEC ? 16 / (int)sizeof(T) : 1;
     typedef T vec_t __attribute__((ext_vector_type(V)));
     const i64 i = ((i64)blockIdx.x * 256 + threadIdx.x) * V;
     if (i >= n) return;
     const uint32_t c = (uint32_t)((i / inner) % C);
     const T m = mean[c], a = coef[c], k1 = coef[C + c], k2 = coef[2 * C + c];
-    const vec_t g = *reinterpret_cast<const vec_t*>(dy + i), v = *reinterpret_cast<const vec_t*>(x + i);
+    vec_t g = *reinterpret_cast<const vec_t*>(dy + i);
+    const vec_t v = *reinterpret_cast<const vec_t*>(x + i);
+    if (MASK) {
+        const vec_t ya = *reinterpret_cast<const vec_t*>(yact + i);
+#pragma unroll
+        for (int u = 0; u < V; ++u) g[u] = ya[u] > T(0) ? g[u] : T(0);
+    }
     vec_t r;
 #pragma unroll
     for (int u = 0; u < V; ++u) r[u] = ((g[u] - k1) - (v[u] - m) * k2) * a;
@@ -373,10 +416,10 @@ __global__ __launch_bounds__(256) void bn_bwd_dx_kernel(const T* __restrict__ dy
 }
 
 // stage 2, fixed (running) statistics: dx = (dy * gamma) / std, the composed Mul and Div gradients in their order
-template <typename T, bool VEC>
-__global__ __launch_bounds__(256) void bn_bwd_dx_fixed_kernel(const T* __restrict__ dy, const T* __restrict__ var,
-                                                              const T* __restrict__ gamma, T eps, T* __restrict__ dx, i64 n, uint32_t C,
-                                                              uint32_t inner) {
+template <typename T, bool VEC, bool MASK>
+__global__ __launch_bounds__(256) void bn_bwd_dx_fixed_kernel(const T* __restrict__ dy, const T* __restrict__ yact,
+                                                              const T* __restrict__ var, const T* __restrict__ gamma, T eps,
+                                                              T* __restrict__ dx, i64 n, uint32_t C, uint32_t inner) {
     constexpr int V = VEC ? 16 / (int)sizeof(T) : 1;
     typedef T vec_t __attribute__((ext_vector_type(V)));
     const i64 i = ((i64)blockIdx.x * 256 + threadIdx.x) * V;
@@ -384,14 +427,19 @@ __global__ __launch_bounds__(256) void bn_bwd_dx_fixed_kernel(const T* __restric
     const uint32_t c = (uint32_t)((i / inner) % C);
     const T sd = dev_sqrt<T>(var[c] + eps), gm = gamma[c];
     vec_t g = *reinterpret_cast<const vec_t*>(dy + i);
+    if (MASK) {
+        const vec_t ya = *reinterpret_cast<const vec_t*>(yact + i);
+#pragma unroll
+        for (int u = 0; u < V; ++u) g[u] = ya[u] > T(0) ? g[u] : T(0);
+    }
 #pragma unroll
     for (int u = 0; u < V; ++u) g[u] = (g[u] * gm) / sd;
     *reinterpret_cast<vec_t*>(dx + i) = g;
 }
 
 template <typename T>
-int bn_bwd(fx_ctx* c, const T* dy, const T* x, const T* mean, const T* var, const T* gamma, double eps, T* dx, T* dgamma, T* dbeta,
-           i64 outer, i64 C, i64 inner, int batch_stats) {
+int bn_bwd(fx_ctx* c, const T* dy, const T* x, const T* yact, const T* mean, const T* var, const T* gamma, double eps, T* dx, T* dgamma,
+           T* dbeta, i64 outer, i64 C, i64 inner, int batch_stats) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(outer >= 1 && C >= 1 && inner >= 1, "fx_batchnorm_bwd: bad view");
     FX_REQUIRE(dy && x && mean && var && gamma && dgamma && dbeta, "fx_batchnorm_bwd: null pointer");
@@ -421,28 +469,36 @@ int bn_bwd(fx_ctx* c, const T* dy, const T* x, const T* mean, const T* var, cons
     T* coef = (T*)(sc + coef_off);
     if (planar) {
         const dim3 grid((unsigned)C, (unsigned)sp.slices);
-        if (inner % V == 0 && fx::aligned16(x) && fx::aligned16(dy))
-            bn_bwd_sums_planar_kernel<T, true><<<grid, dim3(256), 0, c->stream>>>(dy, x, mean, part, outer, C, inner, sp.rows_per_slice);
-        else bn_bwd_sums_planar_kernel<T, false><<<grid, dim3(256), 0, c->stream>>>(dy, x, mean, part, outer, C, inner, sp.rows_per_slice);
+        const bool v16 = inner % V == 0 && fx::aligned16(x) && fx::aligned16(dy) && (!yact || fx::aligned16(yact));
+        const i64 rps = sp.rows_per_slice;
+        if (v16 && yact) bn_bwd_sums_planar_kernel<T, true, true><<<grid, dim3(256), 0, c->stream>>>(dy, x, yact, mean, part, outer, C, inner, rps);
+        else if (v16) bn_bwd_sums_planar_kernel<T, true, false><<<grid, dim3(256), 0, c->stream>>>(dy, x, yact, mean, part, outer, C, inner, rps);
+        else if (yact) bn_bwd_sums_planar_kernel<T, false, true><<<grid, dim3(256), 0, c->stream>>>(dy, x, yact, mean, part, outer, C, inner, rps);
+        else bn_bwd_sums_planar_kernel<T, false, false><<<grid, dim3(256), 0, c->stream>>>(dy, x, yact, mean, part, outer, C, inner, rps);
     } else {
         bn_bwd_sums_column_kernel<T><<<dim3((unsigned)col_blocks, (unsigned)sp.slices), dim3(256), 0, c->stream>>>(
-            dy, x, mean, part, outer, Q, (uint32_t)inner, sp.rows_per_slice);
+            dy, x, yact, mean, part, outer, Q, (uint32_t)inner, sp.rows_per_slice);
     }
     FX_LAUNCH_CHECK();
-    bn_bwd_final_kernel<T><<<dim3((unsigned)fx::ceil_div(C, (i64)256)), dim3(256), 0, c->stream>>>(
+    bn_bwd_final_kernel<T><<<dim3((unsigned)C), dim3(64), 0, c->stream>>>(
         part, var, gamma, (T)eps, dgamma, dbeta, coef, (T)(outer * inner), C, per_channel, (int)sp.slices);
     FX_LAUNCH_CHECK();
     if (!dx) return FX_OK;
-    const bool vec = inner % V == 0 && fx::aligned16(x) && fx::aligned16(dy) && fx::aligned16(dx);
+    const bool vec = inner % V == 0 && fx::aligned16(x) && fx::aligned16(dy) && fx::aligned16(dx) && (!yact || fx::aligned16(yact));
     const i64 blocks = fx::ceil_div(vec ? n / V : n, 256);
     FX_REQUIRE(blocks <= 0x7fffffff, "fx_batchnorm_bwd: too many elements");
     const dim3 grid((unsigned)blocks), blk(256);
+    const uint32_t Cu = (uint32_t)C, iu = (uint32_t)inner;
     if (batch_stats) {
-        if (vec) bn_bwd_dx_kernel<T, true><<<grid, blk, 0, c->stream>>>(dy, x, mean, coef, dx, n, (uint32_t)C, (uint32_t)inner);
-        else bn_bwd_dx_kernel<T, false><<<grid, blk, 0, c->stream>>>(dy, x, mean, coef, dx, n, (uint32_t)C, (uint32_t)inner);
+        if (vec && yact) bn_bwd_dx_kernel<T, true, true><<<grid, blk, 0, c->stream>>>(dy, x, yact, mean, coef, dx, n, Cu, iu);
+        else if (vec) bn_bwd_dx_kernel<T, true, false><<<grid, blk, 0, c->stream>>>(dy, x, yact, mean, coef, dx, n, Cu, iu);
+        else if (yact) bn_bwd_dx_kernel<T, false, true><<<grid, blk, 0, c->stream>>>(dy, x, yact, mean, coef, dx, n, Cu, iu);
+        else bn_bwd_dx_kernel<T, false, false><<<grid, blk, 0, c->stream>>>(dy, x, yact, mean, coef, dx, n, Cu, iu);
     } else {
-        if (vec) bn_bwd_dx_fixed_kernel<T, true><<<grid, blk, 0, c->stream>>>(dy, var, gamma, (T)eps, dx, n, (uint32_t)C, (uint32_t)inner);
-        else bn_bwd_dx_fixed_kernel<T, false><<<grid, blk, 0, c->stream>>>(dy, var, gamma, (T)eps, dx, n, (uint32_t)C, (uint32_t)inner);
+        if (vec && yact) bn_bwd_dx_fixed_kernel<T, true, true><<<grid, blk, 0, c->stream>>>(dy, yact, var, gamma, (T)eps, dx, n, Cu, iu);
+        else if (vec) bn_bwd_dx_fixed_kernel<T, true, false><<<grid, blk, 0, c->stream>>>(dy, yact, var, gamma, (T)eps, dx, n, Cu, iu);
+        else if (yact) bn_bwd_dx_fixed_kernel<T, false, true><<<grid, blk, 0, c->stream>>>(dy, yact, var, gamma, (T)eps, dx, n, Cu, iu);
+        else bn_bwd_dx_fixed_kernel<T, false, false><<<grid, blk, 0, c->stream>>>(dy, yact, var, gamma, (T)eps, dx, n, Cu, iu);
     }
     FX_LAUNCH_CHECK();
     return FX_OK;
@@ -456,13 +512,14 @@ int bn_bwd(fx_ctx* c, const T* dy, const T* x, const T* mean, const T* var, cons
         return bn_stats<T>(c, x, mean, var, running_mean, running_var, momentum, outer, C, inner);                     \
     }                                                                                                                  \
     extern "C" int fx_batchnorm_fwd_##S(fx_ctx* c, const T* x, const T* mean, const T* var, const T* gamma,            \
-                                        const T* beta, double eps, T* y, int64_t outer, int64_t C, int64_t inner) {    \
-        return bn_fwd<T>(c, x, mean, var, gamma, beta, eps, y, outer, C, inner);                                       \
+                                        const T* beta, double eps, T* y, int64_t outer, int64_t C, int64_t inner,      \
+                                        int act) {                                                                     \
+        return bn_fwd<T>(c, x, mean, var, gamma, beta, eps, y, outer, C, inner, act);                                  \
     }                                                                                                                  \
-    extern "C" int fx_batchnorm_bwd_##S(fx_ctx* c, const T* dy, const T* x, const T* mean, const T* var,               \
-                                        const T* gamma, double eps, T* dx, T* dgamma, T* dbeta, int64_t outer,         \
-                                        int64_t C, int64_t inner, int batch_stats) {                                   \
-        return bn_bwd<T>(c, dy, x, mean, var, gamma, eps, dx, dgamma, dbeta, outer, C, inner, batch_stats);            \
+    extern "C" int fx_batchnorm_bwd_##S(fx_ctx* c, const T* dy, const T* x, const T* y_act, const T* mean,             \
+                                        const T* var, const T* gamma, double eps, T* dx, T* dgamma, T* dbeta,          \
+                                        int64_t outer, int64_t C, int64_t inner, int batch_stats) {                    \
+        return bn_bwd<T>(c, dy, x, y_act, mean, var, gamma, eps, dx, dgamma, dbeta, outer, C, inner, batch_stats);     \
     }
 
 FX_DEFINE_BN(float, f32)

@@ -37,12 +37,12 @@ template <typename T> struct FusedApi;
         static int bn_stats(fx_ctx* c, const T* x, T* m, T* v, T* rm, T* rv, double mom, int64_t o, int64_t C, int64_t i) { \
             return fx_batchnorm_stats_##S(c, x, m, v, rm, rv, mom, o, C, i);                                           \
         }                                                                                                              \
-        static int bn_fwd(fx_ctx* c, const T* x, const T* m, const T* v, const T* g, const T* b, double eps, T* y, int64_t o, int64_t C, int64_t i) { \
-            return fx_batchnorm_fwd_##S(c, x, m, v, g, b, eps, y, o, C, i);                                            \
+        static int bn_fwd(fx_ctx* c, const T* x, const T* m, const T* v, const T* g, const T* b, double eps, T* y, int64_t o, int64_t C, int64_t i, int act) { \
+            return fx_batchnorm_fwd_##S(c, x, m, v, g, b, eps, y, o, C, i, act);                                       \
         }                                                                                                              \
-        static int bn_bwd(fx_ctx* c, const T* dy, const T* x, const T* m, const T* v, const T* g, double eps, T* dx, T* dg, T* db, \
+        static int bn_bwd(fx_ctx* c, const T* dy, const T* x, const T* ya, const T* m, const T* v, const T* g, double eps, T* dx, T* dg, T* db, \
                           int64_t o, int64_t C, int64_t i, int batch_stats) {                                         \
-            return fx_batchnorm_bwd_##S(c, dy, x, m, v, g, eps, dx, dg, db, o, C, i, batch_stats);                     \
+            return fx_batchnorm_bwd_##S(c, dy, x, ya, m, v, g, eps, dx, dg, db, o, C, i, batch_stats);                 \
         }                                                                                                              \
         static int dropout(fx_ctx* c, const T* x, T* mask, T* y, int64_t n, double p, uint64_t seed) { return fx_dropout_##S(c, x, mask, y, n, p, seed); } \
         static int rmean(fx_ctx* c, const T* i, T* o, int64_t ou, int64_t ax, int64_t in) { return fx_reduce_mean_##S(c, i, o, ou, ax, in); } \
@@ -181,11 +181,12 @@ template <typename T> struct Conv2dFused : Module<T> {
 // statistics kernel (training) or read (inference).
 template <typename T> struct BatchNormFusedOp : Operator<T> {
     double eps, momentum;
-    bool batch_stats;                         // training (or no running statistics): statistics of this batch
+    bool relu;                                 // the ReLU that follows the layer, applied in the same kernels
+    bool batch_stats;                          // training (or no running statistics): statistics of this batch
     HipStorage<T>*running_mean, *running_var;  // owned by the module; null when not tracked
     mutable Tensor<T> mean, var;               // batch statistics, kept for the backward pass
-    BatchNormFusedOp(double eps_, double mom, bool batch, HipStorage<T>* rm, HipStorage<T>* rv)
-        : eps(eps_), momentum(mom), batch_stats(batch), running_mean(rm), running_var(rv) {}
+    BatchNormFusedOp(double eps_, double mom, bool relu_, bool batch, HipStorage<T>* rm, HipStorage<T>* rv)
+        : eps(eps_), momentum(mom), relu(relu_), batch_stats(batch), running_mean(rm), running_var(rv) {}
     static void view(const Shape& s, int64_t& outer, int64_t& C, int64_t& inner) {
         outer = (int64_t)s[0];
         C = (int64_t)s[1];
@@ -210,36 +211,42 @@ template <typename T> struct BatchNormFusedOp : Operator<T> {
             v = running_var->data();
         }
         Tensor<T> y = HipStorage<T>::alloc(xs);
-        fx_ok(FusedApi<T>::bn_fwd(fused_ctx(), in[0]->data(), m, v, in[1]->data(), in[2]->data(), eps, y->data(), outer, C, inner));
+        fx_ok(FusedApi<T>::bn_fwd(fused_ctx(), in[0]->data(), m, v, in[1]->data(), in[2]->data(), eps, y->data(), outer, C, inner, relu ? 1 : 0));
         return y;
     }
     std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out) const override {
         return gradient_needs(std::move(g), in, out, {true, true, true});
     }
-    std::vector<Tensor<T>> gradient_needs(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*, const std::vector<bool>& needs) const override {
+    std::vector<Tensor<T>> gradient_needs(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out, const std::vector<bool>& needs) const override {
         const Shape& xs = in[0]->shape();
         int64_t outer, C, inner;
         view(xs, outer, C, inner);
+        Tensor<T> recomputed;
+        if (relu && !out) {
+            recomputed = compute(in);
+            out = recomputed.get();
+        }
         std::vector<Tensor<T>> r(3);
         if (needs[0]) r[0] = HipStorage<T>::alloc(xs);
         r[1] = HipStorage<T>::alloc({(size_t)C});
         r[2] = HipStorage<T>::alloc({(size_t)C});
         const T* m = batch_stats ? mean->data() : running_mean->data();
         const T* v = batch_stats ? var->data() : running_var->data();
-        fx_ok(FusedApi<T>::bn_bwd(fused_ctx(), g->data(), in[0]->data(), m, v, in[1]->data(), eps, needs[0] ? r[0]->data() : nullptr,
+        fx_ok(FusedApi<T>::bn_bwd(fused_ctx(), g->data(), in[0]->data(), relu ? out->data() : nullptr, m, v, in[1]->data(), eps, needs[0] ? r[0]->data() : nullptr,
                                   r[1]->data(), r[2]->data(), outer, C, inner, batch_stats ? 1 : 0));
         return r;
     }
     size_t num_inputs() const override { return 3; }
+    bool cache_output() const override { return relu; }
     const char* name() const override { return "BatchNormFused"; }
 };
 
 template <typename T> struct BatchNormFused : Module<T> {
     double eps, momentum;
-    bool track_running_stats = true, training = true;
+    bool track_running_stats = true, training = true, relu = false;
     NodeId weight = 0, bias = 0;
     Tensor<T> running_mean, running_var;
-    BatchNormFused(AutoFerroxEngine<T>& g, size_t c, double eps_, double mom, const T* w, const T* b) : eps(eps_), momentum(mom) {
+    BatchNormFused(AutoFerroxEngine<T>& g, size_t c, double eps_, double mom, const T* w, const T* b, bool relu_) : eps(eps_), momentum(mom), relu(relu_) {
         weight = g.create_variable(HipStorage<T>::from_vec(w, {c}), true);
         bias = g.create_variable(HipStorage<T>::from_vec(b, {c}), true);
         running_mean = HipStorage<T>::zeros({c});
@@ -251,7 +258,7 @@ template <typename T> struct BatchNormFused : Module<T> {
     NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
         const bool batch = training || !track_running_stats;
         const bool update = training && track_running_stats;
-        return g.apply_operation(std::make_unique<BatchNormFusedOp<T>>(eps, momentum, batch, (update || !batch) ? running_mean.get() : nullptr,
+        return g.apply_operation(std::make_unique<BatchNormFusedOp<T>>(eps, momentum, relu, batch, (update || !batch) ? running_mean.get() : nullptr,
                                                                        (update || !batch) ? running_var.get() : nullptr),
                                  {input, weight, bias});
     }

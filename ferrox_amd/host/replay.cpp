@@ -65,7 +65,7 @@ template <typename T> struct Model : ModelBase {
             std::stringstream ss(toks[ti]);
             std::string kind;
             ss >> kind;
-            // fused mode folds a ReLU that directly follows a linear / conv layer into that layer
+            // fused mode folds a ReLU that directly follows a linear / conv / batch-norm layer into that layer
             const bool relu_next = fused && ti + 1 < toks.size() && toks[ti + 1] == "relu";
             if (kind == "linear") {
                 size_t in, out;
@@ -97,7 +97,10 @@ template <typename T> struct Model : ModelBase {
                 else if (!(ss >> mom)) mom = 0.1;
                 const T* w = next();
                 const T* b = next();
-                if (fused) layers.push_back(std::make_unique<BatchNormFused<T>>(graph, c, eps, mom, w, b));
+                if (fused) {
+                    layers.push_back(std::make_unique<BatchNormFused<T>>(graph, c, eps, mom, w, b, relu_next));
+                    if (relu_next) ++ti;
+                }
                 else layers.push_back(std::make_unique<BatchNorm<T>>(graph, c, eps, mom, w, b));
             } else if (kind == "gap") {
                 if (fused) layers.push_back(std::make_unique<GlobalAvgPoolFused<T>>());

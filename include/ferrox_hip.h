@@ -268,15 +268,18 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
        reference's Mean, Sub, Mul, Mean chain), and, when the pointers are not NULL, the running update                \
        running = running*(1-momentum) + batch*momentum (norm.rs:144-161).  fwd: y = ((x-mean)/sqrt(var+eps))*gamma     \
        + beta, the composed operations in the composed order, bit-identical to them given mean and var (pass the       \
-       running statistics for inference, norm.rs:261-290).  bwd: dgamma[C], dbeta[C] and, unless dx is NULL, dx;       \
-       batch_stats 1 = mean/var came from this batch (gradient flows through them), 0 = fixed statistics. */           \
+       running statistics for inference, norm.rs:261-290); act 1 applies the ReLU that follows the layer in the        \
+       reference's models (activation.rs:47-80) in the same store.  bwd: dgamma[C], dbeta[C] and, unless dx is NULL,   \
+       dx; batch_stats 1 = mean/var came from this batch (gradient flows through them), 0 = fixed statistics;          \
+       y_act NULL, or the output of the act = 1 forward: dy is then the gradient of that output and counts only       \
+       where y_act > 0 (ReLU::gradient, ops/unary.rs:358-375). */                                                      \
     int fx_batchnorm_stats_##S(fx_ctx* ctx, const T* x, T* mean, T* var, T* running_mean, T* running_var,              \
                                double momentum, int64_t outer, int64_t C, int64_t inner);                              \
     int fx_batchnorm_fwd_##S(fx_ctx* ctx, const T* x, const T* mean, const T* var, const T* gamma, const T* beta,      \
-                             double eps, T* y, int64_t outer, int64_t C, int64_t inner);                               \
-    int fx_batchnorm_bwd_##S(fx_ctx* ctx, const T* dy, const T* x, const T* mean, const T* var, const T* gamma,        \
-                             double eps, T* dx, T* dgamma, T* dbeta, int64_t outer, int64_t C, int64_t inner,          \
-                             int batch_stats);                                                                         \
+                             double eps, T* y, int64_t outer, int64_t C, int64_t inner, int act);                      \
+    int fx_batchnorm_bwd_##S(fx_ctx* ctx, const T* dy, const T* x, const T* y_act, const T* mean, const T* var,        \
+                             const T* gamma, double eps, T* dx, T* dgamma, T* dbeta, int64_t outer, int64_t C,         \
+                             int64_t inner, int batch_stats);                                                          \
     /* Dropout::forward in training, src/nn/layers/dropout.rs:56-136: mask[i] = 1/(1-p) where u_i < 1-p, else 0, and    \
        y = x*mask; u_i is the 53-bit uniform of splitmix64(seed + i) (the reference's generator is unseeded), 0 <= p    \
        < 1.  The gradient is fx_mul(grad, mask). */                                                                    \

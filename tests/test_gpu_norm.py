@@ -115,6 +115,41 @@ def test_batchnorm_backward_matches_composed_autograd(ctx, orc, dtype):
         assert np.array_equal(dg2.numpy(), dg.numpy()) and np.array_equal(db2.numpy(), db.numpy())
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_batchnorm_with_folded_relu_equals_batchnorm_then_relu(ctx, orc, dtype):
+    """act = 1 / y_act: the ReLU layer that follows BatchNorm in the reference's models, in the same kernels."""
+    import oracle.train as tr
+    rng = np.random.default_rng(96)
+    tol = TOL[np.dtype(dtype)]
+    for shape in BN_SHAPES:
+        C = shape[1]
+        x = (rng.standard_normal(shape) * 2 + 0.5).astype(dtype)
+        g = rng.standard_normal(shape).astype(dtype)
+        gamma, beta = rng.uniform(0.5, 1.5, C).astype(dtype), rng.standard_normal(C).astype(dtype)
+        pre, rec, mean, var = tr.batchnorm_forward(x, gamma, beta, 1e-3)
+        dmean, dvar, dgam, dbet = ctx.upload(mean), ctx.upload(var), ctx.upload(gamma), ctx.upload(beta)
+        y = ctx.batchnorm_fwd(ctx.upload(x), dmean, dvar, dgam, dbet, 1e-3, relu=True)
+        assert np.array_equal(y.numpy(), orc.unary("relu", pre)), shape
+        g_pre = orc.binary("mul", g, orc.scalar("greater_scalar", pre, dtype(0)))       # ReLU::gradient
+        rdx, rdg, rdb = tr.batchnorm_backward(g_pre, rec)
+        dx, dg, db = ctx.batchnorm_bwd(ctx.upload(g), ctx.upload(x), dmean, dvar, dgam, 1e-3, y_act=y)
+        scale = float(np.abs(g).max() * np.abs(gamma).max() / np.sqrt(var.min() + 1e-3))
+        n = x.size // C
+        assert float(np.abs(dx.numpy() - rdx).max()) <= 8 * tol * scale, shape
+        assert float(np.abs(dg.numpy() - rdg).max()) <= tol * n * 4 and float(np.abs(db.numpy() - rdb).max()) <= tol * n * 4, shape
+        # the same through the unfused pair of calls: identical bits (same kernels, mask applied at load)
+        dx2, dg2, db2 = ctx.batchnorm_bwd(ctx.upload(g_pre), ctx.upload(x), dmean, dvar, dgam, 1e-3)
+        assert np.array_equal(dx.numpy(), dx2.numpy()) and np.array_equal(dg.numpy(), dg2.numpy()) and np.array_equal(db.numpy(), db2.numpy())
+        rm, rv = rng.standard_normal(C).astype(dtype), rng.uniform(0.5, 2, C).astype(dtype)
+        pre, rec, _, _ = tr.batchnorm_forward(x, gamma, beta, 1e-3, False, rm, rv)
+        y = ctx.batchnorm_fwd(ctx.upload(x), ctx.upload(rm), ctx.upload(rv), dgam, dbet, 1e-3, relu=True)
+        assert np.array_equal(y.numpy(), orc.unary("relu", pre)), shape
+        g_pre = orc.binary("mul", g, orc.scalar("greater_scalar", pre, dtype(0)))
+        rdx, _, _ = tr.batchnorm_backward(g_pre, rec)
+        dx, _, _ = ctx.batchnorm_bwd(ctx.upload(g), ctx.upload(x), ctx.upload(rm), ctx.upload(rv), dgam, 1e-3, batch_stats=False, y_act=y)
+        assert np.array_equal(dx.numpy(), rdx), shape
+
+
 def test_batchnorm_full_size_properties(ctx):
     """[256, 32, 32, 32] f32 (the first activation of the CNN configuration): normalised output has zero mean and unit
     variance per channel; dx sums to zero against 1 and against x - mean."""
