@@ -138,6 +138,9 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_softmax_ce_bwd_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64)
     _sig(f"fx_adam_step_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, *([_ct] * 7))
     _sig(f"fx_sgd_step_{_s}", _vp, _vp, _vp, _i64, _ct)
+    _sig(f"fx_adam_step_multi_{_s}", _vp, _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_i64),
+         *([_ct] * 7))
+    _sig(f"fx_sgd_step_multi_{_s}", _vp, _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_i64), _ct)
 
 
 class FerroxHipError(RuntimeError):
@@ -496,6 +499,22 @@ class Context:
 
     def adam_step(self, p, g, m, v, lr, beta1, beta2, eps, wd, bc1, bc2):
         check(self._fn("adam_step", p.dtype)(self.h, p.ptr, g.ptr, m.ptr, v.ptr, p.size, lr, beta1, beta2, eps, wd, bc1, bc2))
+
+    def adam_step_multi(self, ps, gs, ms, vs, lr, beta1, beta2, eps, wd, bc1, bc2):
+        """One launch for a list of parameters (in place on ps, ms, vs)."""
+        k = len(ps)
+        tab = lambda arrs: (C.c_void_p * k)(*[a.ptr for a in arrs])  # noqa: E731
+        ns = (C.c_int64 * k)(*[a.size for a in ps])
+        dt = ps[0].dtype if k else np.float32
+        check(self._fn("adam_step_multi", dt)(self.h, k, tab(ps), tab(gs), tab(ms), tab(vs), ns, float(lr), float(beta1),
+                                              float(beta2), float(eps), float(wd), float(bc1), float(bc2)))
+
+    def sgd_step_multi(self, ps, gs, lr):
+        k = len(ps)
+        tab = lambda arrs: (C.c_void_p * k)(*[a.ptr for a in arrs])  # noqa: E731
+        ns = (C.c_int64 * k)(*[a.size for a in ps])
+        dt = ps[0].dtype if k else np.float32
+        check(self._fn("sgd_step_multi", dt)(self.h, k, tab(ps), tab(gs), ns, float(lr)))
 
     def sgd_step(self, p, g, lr):
         check(self._fn("sgd_step", p.dtype)(self.h, p.ptr, g.ptr, p.size, lr))

@@ -252,10 +252,7 @@ int softmax_ce_bwd(fx_ctx* c, const T* probs, const T* targets, const T* gup, T*
 
 // ---- optimizers, in place ----------------------------------------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(256) void adam_step_kernel(T* __restrict__ p, const T* __restrict__ g, T* __restrict__ m, T* __restrict__ v,
-                                                        i64 n, T lr, T beta1, T beta2, T eps, T wd, T bc1, T bc2) {
-    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
+__device__ __forceinline__ void adam_element(T* p, const T* g, T* m, T* v, i64 i, T lr, T beta1, T beta2, T eps, T wd, T bc1, T bc2) {
     const T gi = g[i], w = p[i];
     const T m1 = m[i] * beta1 + gi * (T(1) - beta1);
     const T m2 = v[i] * beta2 + (gi * gi) * (T(1) - beta2);
@@ -266,6 +263,66 @@ __global__ __launch_bounds__(256) void adam_step_kernel(T* __restrict__ p, const
     T nw = w - update;
     if (wd != T(0)) nw = nw - w * (wd * lr);
     p[i] = nw;
+}
+
+// Every parameter of a model in one launch: the tensor table travels in the kernel arguments (no device-side
+// table to upload); block b belongs to the tensor t with first[t] <= b < first[t+1].
+constexpr int MULTI_MAX = 24;
+template <typename T> struct MultiTensors {
+    T* p[MULTI_MAX];
+    const T* g[MULTI_MAX];
+    T* m[MULTI_MAX];
+    T* v[MULTI_MAX];
+    i64 n[MULTI_MAX];
+    unsigned first[MULTI_MAX + 1];
+    int count;
+};
+
+template <typename T, bool ADAM>
+__global__ __launch_bounds__(256) void multi_step_kernel(const MultiTensors<T> tt, T lr, T beta1, T beta2, T eps, T wd, T bc1, T bc2) {
+    int t = 0;
+    while (t + 1 < tt.count && blockIdx.x >= tt.first[t + 1]) ++t;  // wave-uniform
+    const i64 i = (i64)(blockIdx.x - tt.first[t]) * 256 + threadIdx.x;
+    if (i >= tt.n[t]) return;
+    if (ADAM) adam_element<T>(tt.p[t], tt.g[t], tt.m[t], tt.v[t], i, lr, beta1, beta2, eps, wd, bc1, bc2);
+    else tt.p[t][i] = tt.p[t][i] - tt.g[t][i] * lr;
+}
+
+template <typename T, bool ADAM>
+int multi_step(fx_ctx* c, int count, T* const* p, const T* const* g, T* const* m, T* const* v, const int64_t* n, T lr, T beta1, T beta2,
+               T eps, T wd, T bc1, T bc2, const char* what) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(count >= 0, "%s: negative tensor count", what);
+    FX_REQUIRE(count == 0 || (p && g && n && (!ADAM || (m && v))), "%s: null table", what);
+    for (int base = 0; base < count; base += MULTI_MAX) {
+        MultiTensors<T> tt;
+        tt.count = 0;
+        i64 blocks = 0;
+        for (int k = base; k < count && tt.count < MULTI_MAX; ++k) {
+            FX_REQUIRE(n[k] >= 0, "%s: negative element count", what);
+            if (n[k] == 0) continue;
+            FX_REQUIRE(p[k] && g[k] && (!ADAM || (m[k] && v[k])), "%s: null pointer in tensor %d", what, k);
+            const int t = tt.count++;
+            tt.p[t] = p[k]; tt.g[t] = g[k];
+            tt.m[t] = ADAM ? m[k] : nullptr; tt.v[t] = ADAM ? v[k] : nullptr;
+            tt.n[t] = n[k];
+            tt.first[t] = (unsigned)blocks;
+            blocks += fx::ceil_div(n[k], (i64)256);
+            FX_REQUIRE(blocks <= 0x7fffffff, "%s: too many elements", what);
+        }
+        if (tt.count == 0) continue;
+        tt.first[tt.count] = (unsigned)blocks;
+        multi_step_kernel<T, ADAM><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(tt, lr, beta1, beta2, eps, wd, bc1, bc2);
+        FX_LAUNCH_CHECK();
+    }
+    return FX_OK;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void adam_step_kernel(T* __restrict__ p, const T* __restrict__ g, T* __restrict__ m, T* __restrict__ v,
+                                                        i64 n, T lr, T beta1, T beta2, T eps, T wd, T bc1, T bc2) {
+    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) adam_element<T>(p, g, m, v, i, lr, beta1, beta2, eps, wd, bc1, bc2);
 }
 
 template <typename T>
@@ -321,7 +378,17 @@ int sgd_step(fx_ctx* c, T* p, const T* g, i64 n, T lr) {
                                     T wd, T bc1, T bc2) {                                                              \
         return adam_step<T>(c, p, g, m, v, n, lr, beta1, beta2, eps, wd, bc1, bc2);                                    \
     }                                                                                                                  \
-    extern "C" int fx_sgd_step_##S(fx_ctx* c, T* p, const T* g, int64_t n, T lr) { return sgd_step<T>(c, p, g, n, lr); }
+    extern "C" int fx_sgd_step_##S(fx_ctx* c, T* p, const T* g, int64_t n, T lr) { return sgd_step<T>(c, p, g, n, lr); } \
+    extern "C" int fx_adam_step_multi_##S(fx_ctx* c, int count, T* const* p, const T* const* g, T* const* m,           \
+                                          T* const* v, const int64_t* n, T lr, T beta1, T beta2, T eps, T wd, T bc1,   \
+                                          T bc2) {                                                                     \
+        return multi_step<T, true>(c, count, p, g, m, v, n, lr, beta1, beta2, eps, wd, bc1, bc2, "fx_adam_step_multi"); \
+    }                                                                                                                  \
+    extern "C" int fx_sgd_step_multi_##S(fx_ctx* c, int count, T* const* p, const T* const* g, const int64_t* n,       \
+                                         T lr) {                                                                       \
+        return multi_step<T, false>(c, count, p, g, nullptr, nullptr, n, lr, T(0), T(0), T(0), T(0), T(1), T(1),       \
+                                    "fx_sgd_step_multi");                                                              \
+    }
 
 FX_DEFINE_FUSED(float, f32)
 FX_DEFINE_FUSED(double, f64)

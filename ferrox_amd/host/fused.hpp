@@ -10,7 +10,8 @@
 //   CCELoss  : one forward and one backward kernel (classification.rs:191-257 builds 7 nodes)
 //   BatchNorm: statistics (+ running update), normalise and backward kernels (norm.rs:192-336 builds ~15 nodes);
 //              GlobalAvgPool2d as one reduction; Dropout with the mask drawn on the device
-//   Adam/SGD : one in-place kernel per parameter (adam.rs:288-358 runs ~14 and clones the parameter and moments)
+//   Adam/SGD : one in-place launch for all parameters (adam.rs:288-358 runs ~14 kernels per parameter and clones the
+//              parameter and moments)
 #pragma once
 #include "autograd.hpp"
 
@@ -27,6 +28,11 @@ template <typename T> struct FusedApi;
             return fx_adam_step_##S(c, p, g, m, v, n, lr, b1, b2, eps, wd, bc1, bc2);                                  \
         }                                                                                                              \
         static int sgd(fx_ctx* c, T* p, const T* g, int64_t n, T lr) { return fx_sgd_step_##S(c, p, g, n, lr); }       \
+        static int adam_multi(fx_ctx* c, int k, T* const* p, const T* const* g, T* const* m, T* const* v, const int64_t* n, T lr, T b1, T b2, \
+                              T eps, T wd, T bc1, T bc2) {                                                             \
+            return fx_adam_step_multi_##S(c, k, p, g, m, v, n, lr, b1, b2, eps, wd, bc1, bc2);                         \
+        }                                                                                                              \
+        static int sgd_multi(fx_ctx* c, int k, T* const* p, const T* const* g, const int64_t* n, T lr) { return fx_sgd_step_multi_##S(c, k, p, g, n, lr); } \
         static int relu_bwd(fx_ctx* c, const T* g, const T* x, T* o, int64_t n) { return fx_relu_bwd_##S(c, g, x, o, n); } \
         static int gemm_bias(fx_ctx* c, int ta, int tb, int64_t M, int64_t N, int64_t K, const T* A, const T* B, const T* b, T* C, int act) { \
             return fx_gemm_bias_act_##S(c, ta, tb, M, N, K, A, B, b, C, act);                                          \
@@ -332,13 +338,19 @@ template <typename T> NodeId cce_loss_fused(AutoFerroxEngine<T>& g, NodeId predi
 template <typename T> struct SGDFused : Optimizer<T> {
     T lr;
     explicit SGDFused(T lr_) : lr(lr_) {}
-    void step(AutoFerroxEngine<T>& g) override {
+    void step(AutoFerroxEngine<T>& g) override {  // every parameter in one launch
+        std::vector<T*> ps;
+        std::vector<const T*> gs;
+        std::vector<int64_t> ns;
         for (NodeId p : this->params) {
             const HipStorage<T>* grad = g.get_gradient(p);
             if (!grad) continue;
             HipStorage<T>* w = g.mutable_tensor(p);
-            fx_ok(FusedApi<T>::sgd(fused_ctx(), w->data(), grad->data(), (int64_t)w->size(), lr));
+            ps.push_back(w->data());
+            gs.push_back(grad->data());
+            ns.push_back((int64_t)w->size());
         }
+        fx_ok(FusedApi<T>::sgd_multi(fused_ctx(), (int)ps.size(), ps.data(), gs.data(), ns.data(), lr));
     }
 };
 
@@ -352,15 +364,23 @@ template <typename T> struct AdamFused : Optimizer<T> {
         const T stepf = (T)step_count;
         const T b1p = std::max((T)std::pow(beta1, stepf), (T)1e-8), b2p = std::max((T)std::pow(beta2, stepf), (T)1e-8);
         const T bc1 = T(1) - b1p, bc2 = T(1) - b2p;
+        std::vector<T*> ps, ms, vs;  // every parameter in one launch
+        std::vector<const T*> gs;
+        std::vector<int64_t> ns;
         for (NodeId p : this->params) {
             const HipStorage<T>* grad = g.get_gradient(p);
             if (!grad) continue;
             HipStorage<T>* w = g.mutable_tensor(p);
             if (!m1.count(p)) m1[p] = HipStorage<T>::zeros(w->shape());
             if (!m2.count(p)) m2[p] = HipStorage<T>::zeros(w->shape());
-            fx_ok(FusedApi<T>::adam(fused_ctx(), w->data(), grad->data(), m1[p]->data(), m2[p]->data(), (int64_t)w->size(), lr, beta1,
-                                    beta2, eps, weight_decay, bc1, bc2));
+            ps.push_back(w->data());
+            gs.push_back(grad->data());
+            ms.push_back(m1[p]->data());
+            vs.push_back(m2[p]->data());
+            ns.push_back((int64_t)w->size());
         }
+        fx_ok(FusedApi<T>::adam_multi(fused_ctx(), (int)ps.size(), ps.data(), gs.data(), ms.data(), vs.data(), ns.data(), lr, beta1, beta2,
+                                      eps, weight_decay, bc1, bc2));
     }
 };
 

@@ -301,7 +301,13 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
     int fx_adam_step_##S(fx_ctx* ctx, T* p, const T* g, T* m, T* v, int64_t n, T lr, T beta1, T beta2, T eps,          \
                          T weight_decay, T bc1, T bc2);                                                                \
     /* SGD::step without momentum or weight decay, src/nn/optim/sgd.rs:210-245: p = p - g*lr, in place. */             \
-    int fx_sgd_step_##S(fx_ctx* ctx, T* p, const T* g, int64_t n, T lr);
+    int fx_sgd_step_##S(fx_ctx* ctx, T* p, const T* g, int64_t n, T lr);                                               \
+    /* The same updates for `count` parameters in one launch (the optimizers' loop over parameters,                    \
+       adam.rs:288-358 / sgd.rs:210-245): p, g, m, v, n are HOST arrays of `count` device pointers / element counts;   \
+       element arithmetic and results are those of fx_adam_step / fx_sgd_step. */                                      \
+    int fx_adam_step_multi_##S(fx_ctx* ctx, int count, T* const* p, const T* const* g, T* const* m, T* const* v,       \
+                               const int64_t* n, T lr, T beta1, T beta2, T eps, T weight_decay, T bc1, T bc2);         \
+    int fx_sgd_step_multi_##S(fx_ctx* ctx, int count, T* const* p, const T* const* g, const int64_t* n, T lr);
 
 FX_DECLARE_KERNELS(float, f32)
 FX_DECLARE_KERNELS(double, f64)

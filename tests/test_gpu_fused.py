@@ -118,6 +118,38 @@ def test_adam_and_sgd_step_bit_exact(ctx, train, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_multi_tensor_adam_and_sgd_equal_the_per_tensor_calls(ctx, dtype):
+    """fx_adam_step_multi / fx_sgd_step_multi: one launch for a parameter list, bits of the per-tensor entry points;
+    30 tensors exceed one launch's table (24), sizes include 1 and a non-multiple of the block."""
+    rng = np.random.default_rng(75)
+    sizes = [1, 10, 864, 32, 18432, 64, 163840, 10, 255, 256, 257] + [int(v) for v in rng.integers(1, 3000, 19)]
+    arrs = lambda scale: [(rng.standard_normal(n) * scale).astype(dtype) for n in sizes]  # noqa: E731
+    w, g, m = arrs(1.0), arrs(1.0), arrs(0.1)
+    v = [np.abs(a) * 0.01 for a in arrs(1.0)]
+    for wd in (0.0, 0.01):
+        single = [[ctx.upload(a) for a in grp] for grp in (w, m, v)]
+        multi = [[ctx.upload(a) for a in grp] for grp in (w, m, v)]
+        dg = [ctx.upload(a) for a in g]
+        for t in (1, 2):
+            bc1, bc2 = 1 - 0.9 ** t, 1 - 0.999 ** t
+            for i in range(len(sizes)):
+                ctx.adam_step(single[0][i], dg[i], single[1][i], single[2][i], 1e-3, 0.9, 0.999, 1e-8, wd, bc1, bc2)
+            ctx.adam_step_multi(multi[0], dg, multi[1], multi[2], 1e-3, 0.9, 0.999, 1e-8, wd, bc1, bc2)
+            for grp_s, grp_m in zip(single, multi):
+                for a, b in zip(grp_s, grp_m):
+                    assert np.array_equal(a.numpy(), b.numpy()), (wd, t, a.size)
+    sw, mw = [ctx.upload(a) for a in w], [ctx.upload(a) for a in w]
+    dg = [ctx.upload(a) for a in g]
+    for i in range(len(sizes)):
+        ctx.sgd_step(sw[i], dg[i], 0.05)
+    ctx.sgd_step_multi(mw, dg, 0.05)
+    for a, b in zip(sw, mw):
+        assert np.array_equal(a.numpy(), b.numpy()), a.size
+    ctx.adam_step_multi([], [], [], [], 1e-3, 0.9, 0.999, 1e-8, 0.0, 0.1, 0.001)   # empty list: nothing to do
+    ctx.sgd_step_multi([], [], 0.05)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_conv_and_gemm_with_bias_epilogue_equal_two_call_sequence(ctx, dtype):
     """fx_conv2d_fwd_bias_act / fx_gemm_bias_act must give the bits of fx_conv2d_fwd / fx_gemm followed by fx_bias_act,
     on every conv path (LDS-patch, implicit GEMM, strided) and on plain and split-K GEMMs."""
