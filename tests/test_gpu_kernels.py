@@ -348,9 +348,10 @@ def test_conv2d_fwd_dgrad_wgrad_vs_oracle(ctx, orc, dtype):
             assert rel_err(lit_dw, orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 1)) <= tol * 8, ("literal wgrad", case)
 
 
-# 3x3 weight gradients around the LDS-patch kernel (taken when Cin % 32 == 0, Cout > 64, W % 4 == 0, W <= 64, even
-# output width): ragged Cout, one and two output rows per stage, strides, asymmetric padding, the widest row, and
-# neighbours that fall back to the implicit GEMM (Cout <= 64, W % 4 != 0).  B, Cin, H, W, Cout, (sh, sw), (ph, pw)
+# 3x3 weight gradients around the LDS-patch kernel (taken when Cin % 32 == 0, Cout > 32, W % 4 == 0, W <= 64, even
+# output width; up to 64 output channels the waves also split the input channels (Cin % 64 == 0) or the pixel rows
+# (output width % 4 == 0)): ragged Cout, one and two output rows per stage, strides, asymmetric padding, the widest
+# row, and neighbours that fall back to the implicit GEMM (Cout <= 32, W % 4 != 0).  B, Cin, H, W, Cout, (sh, sw), (ph, pw)
 WGRAD_PATCH_CASES = [
     (3, 32, 12, 10, 40, (1, 1), (1, 1)), (2, 64, 9, 14, 72, (1, 1), (0, 0)), (5, 32, 15, 18, 33, (1, 1), (1, 1)),
     (2, 32, 17, 16, 64, (2, 1), (1, 1)), (2, 96, 16, 16, 160, (2, 2), (1, 1)), (3, 32, 11, 12, 48, (1, 2), (2, 0)),
@@ -358,6 +359,9 @@ WGRAD_PATCH_CASES = [
     (21, 32, 29, 56, 32, (1, 1), (1, 1)), (2, 32, 10, 56, 100, (1, 1), (1, 1)), (3, 64, 28, 28, 96, (1, 1), (1, 1)),
     (2, 32, 16, 16, 128, (1, 1), (1, 1)), (2, 32, 9, 64, 128, (1, 1), (0, 1)), (40, 64, 14, 14, 200, (1, 1), (1, 1)),
     (3, 32, 12, 20, 96, (1, 2), (2, 0)), (2, 32, 8, 24, 65, (2, 2), (0, 0)),
+    (2, 64, 12, 56, 64, (1, 1), (1, 1)), (3, 64, 10, 32, 64, (1, 1), (1, 1)), (4, 128, 8, 16, 48, (1, 1), (1, 1)),
+    (2, 32, 12, 32, 64, (1, 1), (1, 1)), (2, 32, 16, 32, 64, (2, 2), (1, 1)), (3, 64, 9, 24, 40, (1, 2), (1, 1)),
+    (5, 32, 6, 64, 33, (1, 1), (1, 1)), (2, 96, 8, 8, 64, (1, 1), (1, 1)), (2, 64, 7, 12, 56, (1, 1), (0, 0)),
 ]
 
 
