@@ -199,30 +199,26 @@ int dgrad_tile(fx_ctx* c, const T* g, const T* wt, T* dx, const Dims& d) {
 // stride-1 correlation of grad_out with the sub-filter w[.., ry + jy*sh, rx + jx*sw] (flipped), written to the
 // class's sub-grid of dx.  One implicit GEMM per class, with exactly the useful multiply-adds.
 //   out[c][yy][xx] = sum_{j'y, j'x, oc} g[oc][yy - pad_y + j'y][xx - pad_x + j'x] * wcls[c][(j'y, j'x, oc)]
+constexpr int MAX_CLASSES = 4;  // sh * sw pixel classes handled in one launch (stride 2 in both directions)
+struct ClassPerm {
+    int ry[MAX_CLASSES], rx[MAX_CLASSES], nky[MAX_CLASSES], nkx[MAX_CLASSES];
+    i64 offset[MAX_CLASSES], n[MAX_CLASSES];
+};
+// Sub-filters of all classes, one launch: blockIdx.y = class; out[offset + ((c*nky + jy)*nkx + jx)*Cout + oc].
 template <typename T>
 __global__ __launch_bounds__(256) void permute_weights_class_kernel(const T* __restrict__ w, T* __restrict__ out, int Cout, int Cin, int kh,
-                                                                    int kw, int ry, int rx, int sh, int sw, int nky, int nkx) {
+                                                                    int kw, int sh, int sw, const ClassPerm cp) {
+    const int z = blockIdx.y;
     const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
-    const i64 n = (i64)Cin * nky * nkx * Cout;
-    if (i >= n) return;
+    if (i >= cp.n[z]) return;
+    const int nky = cp.nky[z], nkx = cp.nkx[z];
     const int oc = (int)(i % Cout);
     i64 t = i / Cout;
     const int jx = (int)(t % nkx);
     t /= nkx;
     const int jy = (int)(t % nky), c = (int)(t / nky);
-    const int ky = ry + (nky - 1 - jy) * sh, kx = rx + (nkx - 1 - jx) * sw;
-    out[i] = w[(((i64)oc * Cin + c) * kh + ky) * kw + kx];
-}
-
-template <typename T, class Cfg>
-int dgrad_class_tile(fx_ctx* c, const T* g, const T* wcls, T* dx, const Dims& d, const ConvShape& s, int Hy, int Wx, int y0, int x0) {
-    const i64 M = d.Cin, N = d.B * Hy * Wx, K = (i64)s.kh * s.kw * d.Cout;
-    MatLoader<T, true> al{wcls, K, (int)M};
-    ConvFwdB<T, true> bl{g, s, (int)N};
-    NchwSubgridStore<T> ep{dx, (int)d.Cin, (int)d.H, (int)d.W, Hy, Wx, y0, x0, (int)d.sh, (int)d.sw, (int)N,
-                           FastDiv((uint32_t)(Hy * Wx)), FastDiv((uint32_t)Wx)};
-    const int kps = (int)(fx::ceil_div(K, Cfg::BK) * Cfg::BK);
-    return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
+    const int ky = cp.ry[z] + (nky - 1 - jy) * sh, kx = cp.rx[z] + (nkx - 1 - jx) * sw;
+    out[cp.offset[z] + i] = w[(((i64)oc * Cin + c) * kh + ky) * kw + kx];
 }
 
 template <typename T>
@@ -230,9 +226,26 @@ bool dgrad_classes_ok(const Dims& d) {
     return (d.sh > 1 || d.sw > 1) && d.kh >= d.sh && d.kw >= d.sw && d.Cout % CONV_BK == 0 && !generic_only();
 }
 
-template <typename T>
-int dgrad_classes(fx_ctx* c, const T* g, const T* w, T* dx, T* wt, const Dims& d) {
-    T* wcls = wt;
+// One class = one forward stride-1 correlation over grad_out with the class's sub-filter, stored to the class's
+// sub-grid of dx.  Classes go out MAX_CLASSES per launch (blockIdx.z = class): each alone is a small GEMM (a quarter
+// of the pixels for stride 2) that fills only part of the chip.
+template <typename T, class Cfg>
+int dgrad_classes_tile(fx_ctx* c, const T* g, const T* w, T* dx, T* wt, const Dims& d) {
+    typedef igemm::MultiProblem<MatLoader<T, true>, ConvFwdB<T, true>, NchwSubgridStore<T>, MAX_CLASSES> MP;
+    MP mp;
+    ClassPerm cp;
+    int count = 0;
+    i64 woff = 0, max_n = 0;
+    auto flush = [&]() -> int {
+        if (count == 0) return FX_OK;
+        permute_weights_class_kernel<T><<<dim3((unsigned)fx::ceil_div(max_n, 256), (unsigned)count), dim3(256), 0, c->stream>>>(
+            w, wt, (int)d.Cout, (int)d.Cin, (int)d.kh, (int)d.kw, (int)d.sh, (int)d.sw, cp);
+        FX_LAUNCH_CHECK();
+        const int rc = igemm::launch_multi<T, Cfg>(c, mp, count);
+        count = 0;
+        max_n = 0;
+        return rc;
+    };
     for (int ry = 0; ry < d.sh; ++ry)
         for (int rx = 0; rx < d.sw; ++rx) {
             const int y0 = (int)(((ry - d.ph) % d.sh + d.sh) % d.sh), x0 = (int)(((rx - d.pw) % d.sw + d.sw) % d.sw);
@@ -241,9 +254,6 @@ int dgrad_classes(fx_ctx* c, const T* g, const T* w, T* dx, T* wt, const Dims& d
             const int nky = (int)((d.kh - ry + d.sh - 1) / d.sh), nkx = (int)((d.kw - rx + d.sw - 1) / d.sw);
             const int dy0 = (int)((y0 + d.ph - ry) / d.sh), dx0 = (int)((x0 + d.pw - rx) / d.sw);
             const i64 nw = d.Cin * nky * nkx * d.Cout;
-            permute_weights_class_kernel<T><<<dim3((unsigned)fx::ceil_div(nw, 256)), dim3(256), 0, c->stream>>>(
-                w, wcls, (int)d.Cout, (int)d.Cin, (int)d.kh, (int)d.kw, ry, rx, (int)d.sh, (int)d.sw, nky, nkx);
-            FX_LAUNCH_CHECK();
             // the class as a forward stride-1 correlation: input = grad_out [B, Cout, oh, ow], kernel nky x nkx
             ConvShape s = make_shape(d.B, d.Cout, d.oh, d.ow, d.Cin, nky, nkx, 1, 1, 0, 0);
             s.ph = (nky - 1) - dy0;
@@ -252,17 +262,35 @@ int dgrad_classes(fx_ctx* c, const T* g, const T* w, T* dx, T* wt, const Dims& d
             s.ow = Wx;
             s.div_L = FastDiv((uint32_t)(Hy * Wx));
             s.div_ow = FastDiv((uint32_t)Wx);
-            int rc;
-            switch (pick_tile(c, d.Cin, d.B * Hy * Wx)) {
-                case 128: rc = dgrad_class_tile<T, TileM128>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0); break;
-                case 64: rc = dgrad_class_tile<T, TileM64>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0); break;
-                case 32: rc = dgrad_class_tile<T, TileM32>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0); break;
-                default: rc = dgrad_class_tile<T, TileSmall>(c, g, wcls, dx, d, s, Hy, Wx, y0, x0); break;
-            }
-            if (rc) return rc;
-            wcls += nw;
+            const i64 M = d.Cin, N = d.B * Hy * Wx, K = (i64)nky * nkx * d.Cout;
+            const int z = count++;
+            cp.ry[z] = ry; cp.rx[z] = rx; cp.nky[z] = nky; cp.nkx[z] = nkx; cp.offset[z] = woff; cp.n[z] = nw;
+            max_n = std::max(max_n, nw);
+            mp.al[z] = MatLoader<T, true>{wt + woff, K, (int)M};
+            mp.bl[z] = ConvFwdB<T, true>{g, s, (int)N};
+            mp.ep[z] = NchwSubgridStore<T>{dx, (int)d.Cin, (int)d.H, (int)d.W, Hy, Wx, y0, x0, (int)d.sh, (int)d.sw, (int)N,
+                                          FastDiv((uint32_t)(Hy * Wx)), FastDiv((uint32_t)Wx)};
+            mp.K[z] = (int)K;
+            mp.kps[z] = (int)(fx::ceil_div(K, Cfg::BK) * Cfg::BK);
+            mp.tiles_n[z] = (int)fx::ceil_div(N, Cfg::BN);
+            mp.tiles_m[z] = (int)fx::ceil_div(M, Cfg::BM);
+            woff += nw;
+            if (count == MAX_CLASSES)
+                if (int rc = flush()) return rc;
         }
-    return FX_OK;
+    return flush();
+}
+
+template <typename T>
+int dgrad_classes(fx_ctx* c, const T* g, const T* w, T* dx, T* wt, const Dims& d) {
+    // tile from the largest class; all classes of one call share it
+    const i64 Hy = fx::ceil_div(d.H, d.sh), Wx = fx::ceil_div(d.W, d.sw);
+    switch (pick_tile(c, d.Cin, d.B * Hy * Wx * std::min<i64>(MAX_CLASSES, d.sh * d.sw))) {
+        case 128: return dgrad_classes_tile<T, TileM128>(c, g, w, dx, wt, d);
+        case 64: return dgrad_classes_tile<T, TileM64>(c, g, w, dx, wt, d);
+        case 32: return dgrad_classes_tile<T, TileM32>(c, g, w, dx, wt, d);
+        default: return dgrad_classes_tile<T, TileSmall>(c, g, w, dx, wt, d);
+    }
 }
 
 // Data gradient for at most 4 input channels (the first layer of an image network): the implicit GEMM would pad

@@ -444,8 +444,9 @@ template <typename T> struct NchwSubgridStore {
 
 // ---- the kernel -------------------------------------------------------------------------------------------
 // grid (N tiles, M tiles, K splits).  Split z covers k in [z*kps, min(K, (z+1)*kps)), kps a multiple of BK.
+// The tile program; (tile_n, tile_m, split) normally come from blockIdx.
 template <typename T, class Cfg, class AL, class BL, class EP>
-__global__ __launch_bounds__(Cfg::NT) void igemm_kernel(AL al, BL bl, EP ep, int K, int kps) {
+__device__ __forceinline__ void igemm_tile(const AL& al, const BL& bl, const EP& ep, int K, int kps, int tile_n, int tile_m, int split) {
     typedef Mfma<T> MF;
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT;
     constexpr int TM = Cfg::WM / MF::BLK, TN = Cfg::WN / MF::BLK;
@@ -461,7 +462,7 @@ __global__ __launch_bounds__(Cfg::NT) void igemm_kernel(AL al, BL bl, EP ep, int
     __shared__ T Bs[2][BK * BMap::LD];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int bm = blockIdx.y * BM, bn = blockIdx.x * BN, split = blockIdx.z;
+    const int bm = tile_m * BM, bn = tile_n * BN;
     const int kbeg = split * kps, kend = min(K, kbeg + kps);
     const int wm0 = (wave / Cfg::WAVES_N) * Cfg::WM, wn0 = (wave % Cfg::WAVES_N) * Cfg::WN;
 
@@ -555,6 +556,26 @@ __global__ __launch_bounds__(Cfg::NT) void igemm_kernel(AL al, BL bl, EP ep, int
     }
 }
 
+template <typename T, class Cfg, class AL, class BL, class EP>
+__global__ __launch_bounds__(Cfg::NT) void igemm_kernel(AL al, BL bl, EP ep, int K, int kps) {
+    igemm_tile<T, Cfg, AL, BL, EP>(al, bl, ep, K, kps, blockIdx.x, blockIdx.y, blockIdx.z);
+}
+
+// Up to NP independent problems of one kind in a single launch (blockIdx.z picks the problem, no K split): used where
+// one operator decomposes into a few small GEMMs that would each leave most of the chip idle.
+template <class AL, class BL, class EP, int NP> struct MultiProblem {
+    AL al[NP];
+    BL bl[NP];
+    EP ep[NP];
+    int K[NP], kps[NP], tiles_n[NP], tiles_m[NP];
+};
+template <typename T, class Cfg, class AL, class BL, class EP, int NP>
+__global__ __launch_bounds__(Cfg::NT) void igemm_multi_kernel(const MultiProblem<AL, BL, EP, NP> mp) {
+    const int z = blockIdx.z;  // wave-uniform: the kernel arguments are read with scalar loads
+    if ((int)blockIdx.x >= mp.tiles_n[z] || (int)blockIdx.y >= mp.tiles_m[z]) return;
+    igemm_tile<T, Cfg, AL, BL, EP>(mp.al[z], mp.bl[z], mp.ep[z], mp.K[z], mp.kps[z], blockIdx.x, blockIdx.y, 0);
+}
+
 // Sums split-K partials in split order (deterministic) into the final buffer; 8 independent loads in flight.
 template <typename T>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const T* __restrict__ part, T* __restrict__ out, i64 n, int splits) {
@@ -580,6 +601,20 @@ int launch(fx_ctx* c, const AL& al, const BL& bl, const EP& ep, i64 M, i64 N, i6
     FX_REQUIRE(K >= 1, "implicit GEMM needs K >= 1");
     igemm_kernel<T, Cfg, AL, BL, EP><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)splits), dim3(Cfg::NT), 0, c->stream>>>(
         al, bl, ep, (int)K, kps);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+template <typename T, class Cfg, class AL, class BL, class EP, int NP>
+int launch_multi(fx_ctx* c, const MultiProblem<AL, BL, EP, NP>& mp, int count) {
+    int gx = 0, gy = 0;
+    for (int z = 0; z < count; ++z) {
+        FX_REQUIRE(mp.K[z] >= 1, "implicit GEMM needs K >= 1");
+        gx = std::max(gx, mp.tiles_n[z]);
+        gy = std::max(gy, mp.tiles_m[z]);
+    }
+    FX_REQUIRE(count >= 1 && count <= NP && gx >= 1 && gy >= 1 && gy <= 65535, "implicit GEMM grid out of range");
+    igemm_multi_kernel<T, Cfg, AL, BL, EP, NP><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)count), dim3(Cfg::NT), 0, c->stream>>>(mp);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

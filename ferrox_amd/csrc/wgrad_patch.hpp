@@ -96,8 +96,11 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
         const float* xsrc = p.x + ((i64)b * p.Cin + c0) * p.H * p.W;
 #pragma unroll
         for (int u = 0; u < NG; ++u) {
+            // rows past the last output channel are never loaded: a pass of 16 rows that starts past it reads row oc0
+            // instead (block-uniform choice), a thread whose own row is past it reads the first row of its pass
+            const bool pass_in = full_m || oc0 + u * RPP < p.Cout;
             const bool ok = full_m || oc0 + prow + u * RPP < p.Cout;
-            gv[u] = ldg4(gsrc + (i64)u * RPP * L, ok ? g_off : 0u);
+            gv[u] = ldg4(pass_in ? gsrc + (i64)u * RPP * L : gsrc, ok ? g_off : 0u);
         }
 #pragma unroll
         for (int r = 0; r < XR; ++r) {

@@ -362,6 +362,9 @@ WGRAD_PATCH_CASES = [
     (2, 64, 12, 56, 64, (1, 1), (1, 1)), (3, 64, 10, 32, 64, (1, 1), (1, 1)), (4, 128, 8, 16, 48, (1, 1), (1, 1)),
     (2, 32, 12, 32, 64, (1, 1), (1, 1)), (2, 32, 16, 32, 64, (2, 2), (1, 1)), (3, 64, 9, 24, 40, (1, 2), (1, 1)),
     (5, 32, 6, 64, 33, (1, 1), (1, 1)), (2, 96, 8, 8, 64, (1, 1), (1, 1)), (2, 64, 7, 12, 56, (1, 1), (0, 0)),
+    # ragged output-channel counts in the last image: the 16-row staging passes past the last channel must not be read
+    (1, 32, 6, 24, 40, (1, 1), (1, 1)), (2, 64, 6, 28, 49, (1, 1), (1, 1)), (1, 32, 4, 32, 97, (1, 1), (1, 1)),
+    (3, 32, 8, 12, 72, (1, 1), (1, 1)), (2, 32, 8, 16, 150, (1, 1), (1, 1)), (1, 64, 5, 56, 36, (1, 1), (1, 1)),
 ]
 
 
