@@ -407,6 +407,13 @@ CONV_PATCH_CASES = [
     (2, 64, 28, 28, 64, (1, 1), (1, 1)), (1, 8, 64, 64, 32, (1, 1), (1, 1)), (2, 16, 6, 16, 40, (2, 2), (1, 1)),
     (2, 8, 5, 12, 24, (1, 1), (0, 1)), (5, 72, 6, 40, 200, (1, 1), (1, 1)), (2, 128, 6, 8, 72, (1, 1), (1, 0)),
     (2, 8, 12, 12, 16, (1, 1), (1, 1)),
+    # output-channel counts within a quarter of a 64 / 128 tile (the planner refuses more padding), one per tile shape
+    # of the forward kernel on a 256-CU device: 2x2, 2x3, 2x4, 4x4, 4x5, 4x6, 4x7, 4x8
+    (2, 8, 6, 12, 60, (1, 1), (1, 1)), (3, 16, 8, 36, 120, (1, 1), (0, 0)), (2, 24, 4, 8, 104, (1, 1), (2, 2)),
+    (1, 8, 64, 64, 52, (1, 1), (1, 1)), (2, 16, 6, 16, 60, (2, 2), (1, 1)), (2, 128, 6, 8, 120, (1, 1), (1, 0)),
+    (2, 8, 9, 64, 128, (2, 1), (1, 1)), (128, 8, 8, 40, 120, (1, 1), (1, 1)), (32, 8, 56, 56, 64, (1, 1), (1, 1)),
+    (16, 8, 56, 56, 120, (1, 1), (1, 1)), (128, 8, 8, 40, 250, (1, 1), (1, 1)), (96, 8, 12, 48, 384, (1, 1), (1, 1)),
+    (32, 8, 56, 56, 120, (1, 1), (1, 1)), (128, 8, 16, 64, 120, (1, 1), (1, 1)),
 ]
 
 
