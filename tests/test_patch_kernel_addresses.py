@@ -1,0 +1,148 @@
+"""Host-side bounds check of the LDS-patch convolution kernels' global loads (CPU only, no GPU).
+
+The staging code of ferrox_amd/csrc/wgrad_patch.hpp and conv_patch.hpp computes every global address as a
+wave-uniform base plus a per-thread offset; lanes and 16-row passes that fall outside the tile's data are redirected to
+an address that is known to be mapped.  This file restates that address arithmetic (and the planners that pick the
+tile) and walks it for every thread of every block for the shapes of the GPU tests: each 16-byte load must lie inside
+its tensor.  It guards the fix of an over-read: passes of grad_out rows that start past the last output channel used to
+be read up to 53 KB past the end of the tensor in the last image.
+"""
+import pytest
+
+LPR, NT, RPP = 16, 256, 16
+def _odd_pitch_w(n): return (n + 30) // 32 * 32 + 1
+def wgrad_plan(num_cus, B, Cin, H, W, Cout, sh, sw, ph, pw, oh, ow):
+    if Cin % 32 or Cout <= 32 or ow % 2 or W % 4 or W > 64 or sh > 8 or sw > 8: return None
+    WMO, WC, WK = 4, 1, 1
+    if Cout <= 64:
+        WMO = 2
+        if Cin % 64 == 0: WC = 2
+        elif ow % 4 == 0: WK = 2
+        else: return None
+    BM, CT = 32 * WMO, 32 * WC
+    max_pr = 3 if WC == 2 else 4
+    best = 0
+    for R in range(1, oh + 1):
+        if oh % R or R * ow > 64 or (R - 1) * sh + 3 > max_pr: continue
+        if (R * ow) % 4 == 0: best = R
+    if not best or best * ow < 24: return None
+    PR = (best - 1) * sh + 3
+    return dict(R=best, PR=PR, BM=BM, CT=CT, Kst=best * ow, stages=B * (oh // best), spi=oh // best)
+def wgrad_loads_in_bounds(B, Cin, H, W, Cout, st, pd):
+    sh, sw = st; ph, pw = pd
+    oh, ow = (H + 2 * ph - 3) // sh + 1, (W + 2 * pw - 3) // sw + 1
+    pl = wgrad_plan(256, B, Cin, H, W, Cout, sh, sw, ph, pw, oh, ow)
+    if pl is None: return "generic"
+    L = oh * ow
+    gsize, xsize = B * Cout * L, B * Cin * H * W
+    k4, w4 = pl["Kst"] // 4, W // 4
+    NG, NXC = pl["BM"] // RPP, pl["CT"] // RPP
+    for s in range(pl["stages"]):
+        b = s // pl["spi"]; oy0 = (s - b * pl["spi"]) * pl["R"]; iy0 = oy0 * sh - ph
+        for oc0 in range(0, Cout, pl["BM"]):
+            full_m = oc0 + pl["BM"] <= Cout
+            gsrc = (b * Cout + oc0) * L + oy0 * ow
+            for tid in range(NT):
+                pq, prow = tid % LPR, tid // LPR
+                g_off = (prow * L + 4 * pq) if pq < k4 else 0
+                for u in range(NG):
+                    ok = full_m or oc0 + prow + u * RPP < Cout
+                    pass_in = full_m or oc0 + u * RPP < Cout
+                    base = gsrc + u * RPP * L if pass_in else gsrc
+                    a = base + (g_off if ok else 0)
+                    assert 0 <= a and a + 4 <= gsize, ("g", (B, Cin, H, W, Cout, st, pd), s, oc0, tid, u, a, gsize)
+        for c0 in range(0, Cin, pl["CT"]):
+            xsrc = (b * Cin + c0) * H * W
+            for tid in range(NT):
+                pq, prow = tid % LPR, tid // LPR
+                x_off = (prow * H * W + 4 * pq) if pq < w4 else 0
+                for r in range(pl["PR"]):
+                    iy = iy0 + r
+                    if not (0 <= iy < H): continue
+                    for cu in range(NXC):
+                        a = xsrc + (cu * RPP * H + iy) * W + x_off
+                        assert 0 <= a and a + 4 <= xsize, ("x", (B, Cin, H, W, Cout, st, pd), a, xsize)
+    return "patch"
+
+CC, KK, WPITCH, NXP = 8, 9, 73, 4
+MAX_PR = 2 * NXP
+def _ceil_div(a, b): return (a + b - 1) // b
+def _odd_pitch_c(n): return (n + 30) // 32 * 32 + 1
+def fwd_plan(num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
+    if C % CC or W % 4 or W > 4 * LPR or sh > 8 or sw > 8: return None
+    L, slots = OH * OW, 2 * num_cus
+    best = None
+    for wm, tn in [(4, 8), (4, 7), (4, 6), (4, 5), (4, 4), (2, 4), (2, 3), (2, 2)]:
+        bm, np_ = 32 * wm, 32 * tn * (4 // wm)
+        tiles, mtiles = _ceil_div(L, np_), _ceil_div(M, bm)
+        rows = min(OH, (np_ - 1) // OW + 2); PR = (rows - 1) * sh + 3
+        if PR > MAX_PR or mtiles * bm * 4 > M * 5: continue
+        cost = _ceil_div(B * tiles * mtiles, slots) * np_ * bm
+        if best is None or cost < best[0]: best = (cost, wm, tn, PR, tiles)
+    if best is None: return None
+    _, wm, tn, PR, tiles = best
+    PW = W + 2 * pw; PLANE = _odd_pitch_c(PR * PW)
+    bm = 32 * wm
+    smem = (bm * WPITCH + CC * PLANE + 16) * 4
+    if smem > 72 * 1024: return None
+    return dict(WM=wm, TN=tn, PR=PR, tpi=tiles, mtiles=_ceil_div(M, bm), nchunks=C // CC, BM=bm, NPIX=32 * tn * (4 // wm))
+def fwd_loads_in_bounds(B, C, H, W, M, sh, sw, ph, pw):
+    OH, OW = (H + 2 * ph - 3) // sh + 1, (W + 2 * pw - 3) // sw + 1
+    pl = fwd_plan(256, B, C, H, W, M, OH, OW, sh, sw, ph, pw)
+    if pl is None: return "generic"
+    WIMG = pl["BM"] * WPITCH
+    NW = (WIMG // 4 + NT - 1) // NT
+    wbuf = pl["mtiles"] * pl["nchunks"] * WIMG          # floats written by wimg_kernel
+    xsize = B * C * H * W
+    for b in (0, B - 1):
+        for tile in range(pl["tpi"]):
+            pix0 = tile * pl["NPIX"]; py0 = pix0 // OW; iy_base = py0 * sh - ph
+            for my in range(pl["mtiles"]):
+                for ch in range(pl["nchunks"]):
+                    wsrc = my * pl["nchunks"] * WIMG + ch * WIMG
+                    xsrc = b * C * H * W + ch * CC * H * W
+                    for tid in range(NT):
+                        for u in range(NW):
+                            idx = tid + u * NT
+                            idx = idx if ((u + 1) * NT <= WIMG // 4 or idx < WIMG // 4) else 0
+                            a = wsrc + idx * 4
+                            assert 0 <= a and a + 4 <= wbuf, ("w", a, wbuf)
+                        pq, xc, rp = tid & 15, (tid >> 4) & 7, tid >> 7
+                        x_off = (xc * H * W + 4 * pq) if pq < (W >> 2) else 0
+                        for u in range(NXP):
+                            r = 2 * u + rp; iy = iy_base + r
+                            if r < pl["PR"] and 0 <= iy < H:
+                                a = xsrc + iy * W + x_off
+                                assert 0 <= a and a + 4 <= xsize, ("x", (B, C, H, W, M), a, xsize)
+    return "patch %dx%d ok" % (pl["WM"], pl["TN"])
+
+
+WGRAD_SHAPES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw): every wave layout, ragged output-channel counts
+    (2, 32, 10, 56, 100, (1, 1), (1, 1)), (3, 64, 28, 28, 96, (1, 1), (1, 1)), (2, 32, 16, 16, 128, (1, 1), (1, 1)),
+    (2, 32, 9, 64, 128, (1, 1), (0, 1)), (2, 64, 12, 56, 64, (1, 1), (1, 1)), (3, 64, 10, 32, 64, (1, 1), (1, 1)),
+    (2, 32, 12, 32, 64, (1, 1), (1, 1)), (5, 32, 6, 64, 33, (1, 1), (1, 1)), (1, 32, 6, 24, 40, (1, 1), (1, 1)),
+    (2, 64, 6, 28, 49, (1, 1), (1, 1)), (1, 32, 4, 32, 97, (1, 1), (1, 1)), (3, 32, 8, 12, 72, (1, 1), (1, 1)),
+    (2, 32, 8, 16, 150, (1, 1), (1, 1)), (1, 64, 5, 56, 36, (1, 1), (1, 1)), (2, 32, 8, 56, 65, (2, 1), (1, 1)),
+]
+FWD_SHAPES = [  # B, C, H, W, M, (sh, sw), (ph, pw): one per tile shape on a 256-CU device, ragged M, strides, paddings
+    (2, 64, 28, 28, 64, (1, 1), (1, 1)), (2, 8, 6, 12, 60, (1, 1), (1, 1)), (3, 16, 8, 36, 120, (1, 1), (0, 0)),
+    (2, 24, 4, 8, 104, (1, 1), (2, 2)), (1, 8, 64, 64, 52, (1, 1), (1, 1)), (2, 16, 6, 16, 60, (2, 2), (1, 1)),
+    (2, 8, 9, 64, 128, (2, 1), (1, 1)), (128, 8, 8, 40, 120, (1, 1), (1, 1)), (32, 8, 56, 56, 64, (1, 1), (1, 1)),
+    (16, 8, 56, 56, 120, (1, 1), (1, 1)), (128, 8, 8, 40, 250, (1, 1), (1, 1)), (96, 8, 12, 48, 384, (1, 1), (1, 1)),
+    (32, 8, 56, 56, 120, (1, 1), (1, 1)), (128, 8, 16, 64, 120, (1, 1), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", WGRAD_SHAPES, ids=str)
+def test_weight_gradient_patch_kernel_loads_stay_inside_the_tensors(case):
+    B = min(case[0], 3)  # the first and the last images are the ones at the tensor ends
+    assert wgrad_loads_in_bounds(B, *case[1:]) == "patch", "the shape must exercise the patch kernel"
+
+
+@pytest.mark.parametrize("case", FWD_SHAPES, ids=str)
+def test_forward_patch_kernel_loads_stay_inside_the_tensors(case):
+    B, C, H, W, M, st, pd = case
+    assert fwd_loads_in_bounds(B, C, H, W, M, st[0], st[1], pd[0], pd[1]).startswith("patch")
+    if st == (1, 1):  # the data gradient runs the same kernel over grad_out with padding 2 - p and channels swapped
+        OH, OW = H + 2 * pd[0] - 2, W + 2 * pd[1] - 2
+        fwd_loads_in_bounds(B, M, OH, OW, C, 1, 1, 2 - pd[0], 2 - pd[1])
