@@ -16,6 +16,7 @@
 #include <set>
 
 #include "hip_storage.hpp"
+#include "state_dict.hpp"
 
 namespace ferrox {
 
@@ -766,11 +767,78 @@ template <typename T> NodeId cce_loss(AutoFerroxEngine<T>& g, NodeId predictions
 }
 
 // ---- optimizers: src/nn/optim ---------------------------------------------------------------------------------
-template <typename T> struct Optimizer {
+template <typename T> struct Optimizer {  // trait Optimizer, src/nn/optim/mod.rs:328-378
     virtual ~Optimizer() = default;
     virtual void step(AutoFerroxEngine<T>& g) = 0;
-    std::vector<NodeId> params;
+    virtual OptimizerStateDict state_dict() const = 0;
+    virtual void load_state_dict(const OptimizerStateDict& sd) = 0;
+    std::vector<NodeId> params;  // the "default" parameter group (Adam::new / SGD::new create exactly one)
+
+  protected:
+    void save_groups(OptimizerStateDict& sd) const {  // add_parameter_group, mod.rs:304-311 (HashSet order is arbitrary: sorted here)
+        SerializableParameterGroup g;
+        g.params.assign(params.begin(), params.end());
+        std::sort(g.params.begin(), g.params.end());
+        g.name = "default";
+        sd.parameter_groups.push_back(std::move(g));
+    }
+    void load_groups(const OptimizerStateDict& sd) {  // param_groups.clear(); push every saved group
+        std::vector<NodeId> restored;
+        for (const auto& g : sd.parameter_groups) restored.insert(restored.end(), g.params.begin(), g.params.end());
+        params = std::move(restored);
+    }
+    static T hyper(const OptimizerStateDict& sd, const char* name, T current) {
+        auto it = sd.hyperparameters.find(name);
+        return it == sd.hyperparameters.end() ? current : (T)it->second;
+    }
 };
+
+// Adam::state_dict / load_state_dict, src/nn/optim/adam.rs:391-556 (no amsgrad), shared by the composed and the fused optimizer
+template <typename T, class Opt> OptimizerStateDict adam_state_dict(const Opt& o) {
+    OptimizerStateDict sd;
+    sd.optimizer_type = "Adam";
+    sd.step_count = (uint64_t)o.step_count;
+    sd.hyperparameters["lr"] = (double)o.lr;
+    sd.hyperparameters["beta1"] = (double)o.beta1;
+    sd.hyperparameters["beta2"] = (double)o.beta2;
+    sd.hyperparameters["eps"] = (double)o.eps;
+    sd.hyperparameters["weight_decay"] = (double)o.weight_decay;
+    sd.hyperparameters["amsgrad"] = 0.0;
+    for (const auto& kv : o.m1) sd.template add_buffer<T>(kv.first, *kv.second, "first_moment");
+    for (const auto& kv : o.m2) sd.template add_buffer<T>(kv.first, *kv.second, "second_moment");
+    return sd;
+}
+template <typename T, class Opt> void adam_load_state_dict(Opt& o, const OptimizerStateDict& sd) {
+    if (sd.optimizer_type != "Adam") throw Error("Type mismatch: Expected Adam state dict, got " + sd.optimizer_type);
+    o.m1.clear();
+    o.m2.clear();
+    o.step_count = (long)sd.step_count;
+    for (const auto& kv : sd.parameter_buffers) {
+        const TensorBuffer& b = kv.second;
+        if (b.buffer_type == "first_moment") o.m1[b.node_id] = b.template to_tensor<T>();
+        else if (b.buffer_type == "second_moment") o.m2[b.node_id] = b.template to_tensor<T>();
+    }
+}
+
+// SGD::state_dict / load_state_dict, src/nn/optim/sgd.rs:278-360 (momentum 0: no buffers)
+template <typename T, class Opt> OptimizerStateDict sgd_state_dict(const Opt& o) {
+    OptimizerStateDict sd;
+    sd.optimizer_type = "SGD";
+    sd.step_count = 0;
+    sd.hyperparameters["lr"] = (double)o.lr;
+    sd.hyperparameters["momentum"] = 0.0;
+    sd.hyperparameters["weight_decay"] = 0.0;
+    sd.hyperparameters["nesterov"] = 0.0;
+    SerializableParameterGroup g;
+    g.params.assign(o.params.begin(), o.params.end());
+    std::sort(g.params.begin(), g.params.end());
+    g.name = "default";
+    sd.parameter_groups.push_back(std::move(g));
+    return sd;
+}
+inline void sgd_check(const OptimizerStateDict& sd) {
+    if (sd.optimizer_type != "SGD") throw Error("Type mismatch: Expected SGD state dict, got " + sd.optimizer_type);
+}
 
 template <typename T> struct SGD : Optimizer<T> {  // src/nn/optim/sgd.rs:116-245 (momentum 0, weight decay 0 path)
     T lr;
@@ -784,6 +852,12 @@ template <typename T> struct SGD : Optimizer<T> {  // src/nn/optim/sgd.rs:116-24
             Tensor<T> scaled = effective->mul_scalar(lr); // apply_lr
             g.update_parameter(p, w->sub(*scaled));
         }
+    }
+    OptimizerStateDict state_dict() const override { return sgd_state_dict<T>(*this); }
+    void load_state_dict(const OptimizerStateDict& sd) override {
+        sgd_check(sd);
+        lr = this->hyper(sd, "lr", lr);
+        this->load_groups(sd);
     }
 };
 
@@ -828,6 +902,20 @@ template <typename T> struct Adam : Optimizer<T> {  // src/nn/optim/adam.rs:110-
             } else nw = w->sub(*update);
             g.update_parameter(p, std::move(nw));
         }
+    }
+    OptimizerStateDict state_dict() const override {
+        OptimizerStateDict sd = adam_state_dict<T>(*this);
+        this->save_groups(sd);
+        return sd;
+    }
+    void load_state_dict(const OptimizerStateDict& sd) override {
+        adam_load_state_dict<T>(*this, sd);
+        lr = this->hyper(sd, "lr", lr);
+        beta1 = this->hyper(sd, "beta1", beta1);
+        beta2 = this->hyper(sd, "beta2", beta2);
+        eps = this->hyper(sd, "eps", eps);
+        weight_decay = this->hyper(sd, "weight_decay", weight_decay);
+        this->load_groups(sd);
     }
 };
 

@@ -352,6 +352,12 @@ template <typename T> struct SGDFused : Optimizer<T> {
         }
         fx_ok(FusedApi<T>::sgd_multi(fused_ctx(), (int)ps.size(), ps.data(), gs.data(), ns.data(), lr));
     }
+    OptimizerStateDict state_dict() const override { return sgd_state_dict<T>(*this); }
+    void load_state_dict(const OptimizerStateDict& sd) override {
+        sgd_check(sd);
+        lr = this->hyper(sd, "lr", lr);
+        this->load_groups(sd);
+    }
 };
 
 template <typename T> struct AdamFused : Optimizer<T> {
@@ -381,6 +387,20 @@ template <typename T> struct AdamFused : Optimizer<T> {
         }
         fx_ok(FusedApi<T>::adam_multi(fused_ctx(), (int)ps.size(), ps.data(), gs.data(), ms.data(), vs.data(), ns.data(), lr, beta1, beta2,
                                       eps, weight_decay, bc1, bc2));
+    }
+    OptimizerStateDict state_dict() const override {
+        OptimizerStateDict sd = adam_state_dict<T>(*this);
+        this->save_groups(sd);
+        return sd;
+    }
+    void load_state_dict(const OptimizerStateDict& sd) override {
+        adam_load_state_dict<T>(*this, sd);
+        lr = this->hyper(sd, "lr", lr);
+        beta1 = this->hyper(sd, "beta1", beta1);
+        beta2 = this->hyper(sd, "beta2", beta2);
+        eps = this->hyper(sd, "eps", eps);
+        weight_decay = this->hyper(sd, "weight_decay", weight_decay);
+        this->load_groups(sd);
     }
 };
 

@@ -29,6 +29,8 @@ struct ModelBase {
     virtual int num_state() const = 0;
     virtual int64_t state_numel(int i) const = 0;
     virtual void get_state(int i, void* host) const = 0;
+    virtual std::vector<uint8_t> optimizer_state() const = 0;
+    virtual void load_optimizer_state(const uint8_t* data, size_t n) = 0;
 };
 
 std::vector<std::string> split(const std::string& s, char sep) {
@@ -147,6 +149,8 @@ template <typename T> struct Model : ModelBase {
         std::vector<T> v = all_state().at(i)->to_vec();
         std::memcpy(host, v.data(), v.size() * sizeof(T));
     }
+    std::vector<uint8_t> optimizer_state() const override { return opt->state_dict().save_to_bytes(); }
+    void load_optimizer_state(const uint8_t* data, size_t n) override { opt->load_state_dict(OptimizerStateDict::load_from_bytes(data, n)); }
     int num_params() const override { return (int)params.size(); }
     int64_t param_numel(int i) const override { return (int64_t)graph.get_tensor(params.at(i))->size(); }
     void set_batch(const void* xv, const Shape& xs, const void* yv, const Shape& ys) override {
@@ -277,6 +281,24 @@ int64_t fxh_model_state_numel(void* m, int i) {
 }
 int fxh_model_get_state(void* m, int i, void* host) {
     return guarded([&] { static_cast<ModelBase*>(m)->get_state(i, host); });
+}
+// Optimizer::state_dict().save_to_bytes(): the moments are copied from the device; *bytes is malloc'ed, release it with fxh_free
+int fxh_model_optimizer_state(void* m, uint8_t** bytes, int64_t* len) {
+    return guarded([&] {
+        const std::vector<uint8_t> v = static_cast<ModelBase*>(m)->optimizer_state();
+        *bytes = static_cast<uint8_t*>(std::malloc(v.size() ? v.size() : 1));
+        if (!*bytes) throw Error("out of host memory");
+        std::memcpy(*bytes, v.data(), v.size());
+        *len = (int64_t)v.size();
+    });
+}
+void fxh_free(void* p) { std::free(p); }
+// OptimizerStateDict::load_from_bytes + Optimizer::load_state_dict
+int fxh_model_load_optimizer_state(void* m, const uint8_t* bytes, int64_t len) {
+    return guarded([&] {
+        if (len < 0 || (!bytes && len)) throw Error("bad buffer");
+        static_cast<ModelBase*>(m)->load_optimizer_state(bytes, (size_t)len);
+    });
 }
 int fxh_pool_stats(int dtype, fx_pool_stats* out) {
     return guarded([&] { fx_ok(fx_pool_stats_get(BackendManager::get().ctx(), dtype, out)); });

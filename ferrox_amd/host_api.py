@@ -40,6 +40,10 @@ lib.fxh_model_num_state.argtypes = [C.c_void_p]
 lib.fxh_model_state_numel.argtypes = [C.c_void_p, C.c_int]
 lib.fxh_model_state_numel.restype = C.c_int64
 lib.fxh_model_get_state.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
+lib.fxh_model_optimizer_state.argtypes = [C.c_void_p, C.POINTER(C.c_void_p), C.POINTER(C.c_int64)]
+lib.fxh_free.argtypes = [C.c_void_p]
+lib.fxh_free.restype = None
+lib.fxh_model_load_optimizer_state.argtypes = [C.c_void_p, C.c_char_p, C.c_int64]
 lib.fxh_pool_stats.argtypes = [C.c_int, C.POINTER(capi.PoolStats)]
 
 
@@ -125,6 +129,18 @@ class Model:
             _check(lib.fxh_model_get_state(self.h, i, a.ctypes.data))
             out.append(a)
         return out
+
+    def optimizer_state(self):
+        """The optimizer's state dictionary as bytes in the reference's file format (moments copied from the device)."""
+        p, n = C.c_void_p(), C.c_int64(0)
+        _check(lib.fxh_model_optimizer_state(self.h, C.byref(p), C.byref(n)))
+        try:
+            return C.string_at(p, n.value)
+        finally:
+            lib.fxh_free(p)
+
+    def load_optimizer_state(self, data):
+        _check(lib.fxh_model_load_optimizer_state(self.h, data, len(data)))
 
     def forward(self):
         n = lib.fxh_model_output_numel(self.h)
