@@ -103,7 +103,9 @@ def bench_conv(ctx, steps, warmup, dtype=np.float32, B=None):
 
 
 def bench_bandwidth(ctx, iters=20, warmup=3):
+    import ctypes
     from ferrox_amd import capi
+    C_i64 = ctypes.c_int64
     out = {"reductions": {}, "elementwise": {}, "pooling": {}}
     for dtype in (np.float32, np.float64):
         sfx = capi.dtype_code(dtype)[1]
@@ -185,6 +187,48 @@ def bench_bandwidth(ctx, iters=20, warmup=3):
     ms = time_stream(ctx, lambda: capi.check(capi.lib.fx_dropout_f32(ctx.h, dxx.ptr, dm.ptr, dy_.ptr, n, 0.3, 99)), 10, 2)
     out["normalisation"]["dropout_f32"] = {"ms": ms, "GBps": 3 * 4 * n / ms / 1e6, "frac_hbm": 3 * 4 * n / ms / 1e6 / PEAK_HBM_GBS}
     del dxx, dm, dy_
+    # explicit im2col / col2im (the reference's convolution path materialises the column matrix; here they exist for
+    # parity and for callers that want the matrix) at the second conv layer of the CNN configuration, and the two
+    # materialisations the layers issue most: a channel bias broadcast to [N,C,H,W] and a 2-D transpose.
+    # Algorithmic bytes: column matrix + image (im2col, col2im); output (+ the small input) for the broadcast; 2 arrays.
+    out["data_movement"] = {}
+    ishape = (256, 32, 32, 32)
+    ix = ctx.uniform(ishape, 16, -1.0, 1.0)
+    col = ctx.im2col(ix, (3, 3), (2, 2), (1, 1))
+    dims = (256, 32, 32, 32, 3, 3, 2, 2, 1, 1)
+    back = ctx.empty(ishape)
+    dm_cases = {
+        "im2col_c5_conv2": (4 * (col.size + ix.size), lambda: capi.check(capi.lib.fx_im2col_f32(ctx.h, ix.ptr, col.ptr, *dims))),
+        "col2im_c5_conv2": (4 * (col.size + ix.size), lambda: capi.check(capi.lib.fx_col2im_f32(ctx.h, col.ptr, back.ptr, *dims, 0))),
+    }
+    bias = ctx.uniform((128,), 17, -1.0, 1.0)
+    bshape2 = (256, 128, 56, 56)
+    bout = ctx.empty(bshape2)
+    sh4, st4 = (C_i64 * 4)(*bshape2), (C_i64 * 4)(0, 1, 0, 0)
+    dm_cases["broadcast_bias_to_nchw"] = (4 * bout.size, lambda: capi.check(capi.lib.fx_materialize_f32(ctx.h, bias.ptr, bout.ptr, sh4, st4, 4, bout.size)))
+    tin = ctx.uniform((8192, 8192), 18, -1.0, 1.0)
+    tout = ctx.empty((8192, 8192))
+    sh2, st2 = (C_i64 * 2)(8192, 8192), (C_i64 * 2)(1, 8192)
+    dm_cases["transpose_8192x8192"] = (2 * 4 * tin.size, lambda: capi.check(capi.lib.fx_materialize_f32(ctx.h, tin.ptr, tout.ptr, sh2, st2, 2, tin.size)))
+    for name, (nbytes, fn) in dm_cases.items():
+        ms = time_stream(ctx, fn, 10, 2)
+        out["data_movement"][f"{name}_f32"] = {"ms": ms, "GBps": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    del ix, col, back, bias, bout, tin, tout
+    # GEMMs of the MLP / CNN configurations (forward and the two backward products) and one large square product
+    out["gemm"] = {}
+    for name, (M, N, K, ta, tb) in {"c2_fc1_fwd": (256, 256, 784, 0, 1), "c2_fc1_dx": (256, 784, 256, 0, 0), "c2_fc1_dw": (256, 784, 256, 1, 0),
+                                    "c5_fc_fwd": (256, 10, 16384, 0, 1), "c5_fc_dw": (10, 16384, 256, 1, 0),
+                                    "square_4096": (4096, 4096, 4096, 0, 0)}.items():
+        for dtype in (np.float32, np.float64):
+            sfx = capi.dtype_code(dtype)[1]
+            a = ctx.uniform((K, M) if ta else (M, K), 19, -1.0, 1.0, dtype)
+            b = ctx.uniform((N, K) if tb else (K, N), 20, -1.0, 1.0, dtype)
+            c = ctx.empty((M, N), dtype)
+            fn = lambda: capi.check(getattr(capi.lib, f"fx_gemm_{sfx}")(ctx.h, ta, tb, M, N, K, a.ptr, b.ptr, c.ptr))  # noqa: E731
+            ms = time_stream(ctx, fn, 20, 3)
+            peak = PEAK_F32_MFMA_TFLOPS if dtype == np.float32 else PEAK_F64_MFMA_TFLOPS
+            out["gemm"][f"{name}_{sfx}"] = {"us": ms * 1e3, "tflops": 2.0 * M * N * K / ms / 1e9, "frac_mfma": 2.0 * M * N * K / ms / 1e9 / peak}
+            del a, b, c
     g = ctx.uniform((n,), 7, -4.0, 4.0)
     x = ctx.uniform((n,), 8, -4.0, 4.0)
     s = ctx.unary("sigmoid", x)

@@ -360,6 +360,29 @@ __global__ __launch_bounds__(256) void materialize_vec_kernel(const T* __restric
     *reinterpret_cast<vec_t*>(out + i * V) = o;
 }
 
+// Transposed innermost pair: out[b][i][j] = in[b*sb + i + j*ld] (the view a 2-D transpose, or a batch of them, leaves
+// behind).  64 x 64 tiles through LDS so that both the reads (along i) and the writes (along j) are contiguous;
+// the 65-float pitch keeps the column reads of the tile on distinct banks.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_tile_kernel(const T* __restrict__ in, T* __restrict__ out, i64 I, i64 J, i64 ld, i64 sb) {
+    __shared__ T tile[64][65];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const i64 j0 = (i64)blockIdx.x * 64, i0 = (i64)blockIdx.y * 64, b = blockIdx.z;
+    const T* src = in + b * sb;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const i64 j = j0 + ty + 4 * r, i = i0 + tx;
+        if (j < J && i < I) tile[ty + 4 * r][tx] = src[j * ld + i];
+    }
+    __syncthreads();
+    T* dst = out + b * I * J;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const i64 i = i0 + ty + 4 * r, j = j0 + tx;
+        if (i < I && j < J) dst[i * J + j] = tile[tx][ty + 4 * r];
+    }
+}
+
 template <typename T>
 int materialize(fx_ctx* c, const T* in, T* out, const i64* shape, const i64* strides, int ndim, i64 n) {
     FX_CHECK_CTX(c);
@@ -392,6 +415,16 @@ int materialize(fx_ctx* c, const T* in, T* out, const i64* shape, const i64* str
         }
     }
     constexpr int V = 16 / (int)sizeof(T);
+    if ((nd == 2 || nd == 3) && ct[nd - 2] == 1 && ct[nd - 1] > 1 && cs[nd - 2] >= 16 && cs[nd - 1] >= 16) {
+        const i64 I = cs[nd - 2], J = cs[nd - 1], Bn = nd == 3 ? cs[0] : 1;
+        const i64 gx = fx::ceil_div(J, 64), gy = fx::ceil_div(I, 64);
+        if (gx <= 0x7fffffff && gy <= 65535 && Bn <= 65535) {
+            transpose_tile_kernel<T><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)Bn), dim3(256), 0, c->stream>>>(
+                in, out, I, J, ct[nd - 1], nd == 3 ? ct[0] : 0);
+            FX_LAUNCH_CHECK();
+            return FX_OK;
+        }
+    }
     if (nd >= 1 && nd <= 4 && n < (1ll << 31) && cs[nd - 1] % V == 0 && (ct[nd - 1] == 0 || ct[nd - 1] == 1) &&
         ((uintptr_t)out & 15) == 0) {
         // vector path: one thread writes V consecutive outputs of the innermost collapsed dim

@@ -77,6 +77,95 @@ int make_geom(ConvGeom& g, i64 B, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i
     return FX_OK;
 }
 
+// ---- 32-bit variants (every tensor below 2^31 elements): multiply-shift divisions, no 64-bit index arithmetic ------
+// n / d for 32-bit n by multiply-shift (d fixed per launch)
+struct U32Div {
+    uint32_t d, m, s;
+    __device__ __forceinline__ uint32_t div(uint32_t n) const { return (uint32_t)(((uint64_t)__umulhi(n, m) + n) >> s); }
+};
+U32Div make_div(uint32_t d) {
+    U32Div r;
+    r.d = d;
+    r.s = 0;
+    while ((1ull << r.s) < d) ++r.s;
+    r.m = (uint32_t)((((1ull << 32) * ((1ull << r.s) - d)) / d) + 1);
+    return r;
+}
+struct Geom32 {
+    int B, C, H, W, kh, kw, sh, sw, ph, pw, oh, ow;
+    U32Div div_L, div_ow, div_KK, div_kw, div_W, div_H, div_C, div_sh, div_sw;
+};
+
+// One thread writes V consecutive columns of one row of the column matrix (one 16-byte store when V > 1); the row's
+// (c, ky, kx) is block-uniform (blockIdx.y), the first column is decoded once and the rest follow by increments.
+template <typename T, int V>
+__global__ __launch_bounds__(256) void im2col32_kernel(const T* __restrict__ x, T* __restrict__ col, Geom32 g, uint32_t N) {
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    const uint32_t n0 = (blockIdx.x * 256u + threadIdx.x) * V;
+    if (n0 >= N) return;
+    const uint32_t row = blockIdx.y;
+    const uint32_t c = g.div_KK.div(row), r = row - c * (uint32_t)(g.kh * g.kw);
+    const uint32_t ky = g.div_kw.div(r), kx = r - ky * (uint32_t)g.kw;
+    const uint32_t L = (uint32_t)(g.oh * g.ow);
+    uint32_t b = g.div_L.div(n0), l = n0 - b * L;
+    uint32_t oy = g.div_ow.div(l), ox = l - oy * (uint32_t)g.ow;
+    vec_t v;
+#pragma unroll
+    for (int u = 0; u < V; ++u) {
+        const int iy = (int)(oy * g.sh + ky) - g.ph, ix = (int)(ox * g.sw + kx) - g.pw;
+        T e = T(0);
+        if (n0 + u < N && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W) e = x[((i64)(b * g.C + c) * g.H + iy) * g.W + ix];
+        v[u] = e;
+        if (++ox == (uint32_t)g.ow) {
+            ox = 0;
+            if (++oy == (uint32_t)g.oh) { oy = 0; ++b; }
+        }
+    }
+    *reinterpret_cast<vec_t*>(col + (i64)row * N + n0) = v;
+}
+
+// The gather of col2im_kernel with 32-bit indices: the taps that reach a pixel are ky = (Y mod sh) + j*sh, visited in
+// ascending order with cy = Y/sh - j (the same order and operands as the 64-bit kernel, so the same bits).
+template <typename T, int LAYOUT>
+__global__ __launch_bounds__(256) void col2im32_kernel(const T* __restrict__ col, T* __restrict__ out, Geom32 g, uint32_t total) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= total) return;
+    uint32_t t = g.div_W.div(idx);
+    const uint32_t xw = idx - t * (uint32_t)g.W;
+    const uint32_t t2 = g.div_H.div(t), y = t - t2 * (uint32_t)g.H;
+    const uint32_t b = g.div_C.div(t2), c = t2 - b * (uint32_t)g.C;
+    const uint32_t L = (uint32_t)(g.oh * g.ow), KK = (uint32_t)(g.kh * g.kw);
+    const uint32_t Y = y + (uint32_t)g.ph, X = xw + (uint32_t)g.pw;
+    const uint32_t qy = g.div_sh.div(Y), ry = Y - qy * (uint32_t)g.sh;
+    const uint32_t qx = g.div_sw.div(X), rx = X - qx * (uint32_t)g.sw;
+    const i64 base = LAYOUT == 1 ? (i64)(b * g.C + c) * KK * L : (i64)c * KK * ((i64)g.B * L) + (i64)b * L;
+    const i64 tap_stride = LAYOUT == 1 ? (i64)L : (i64)g.B * L;
+    T acc = T(0);
+    int cy = (int)qy;
+    for (int ky = (int)ry; ky < g.kh && cy >= 0; ky += g.sh, --cy) {
+        if (cy >= g.oh) continue;
+        int cx = (int)qx;
+        for (int kx = (int)rx; kx < g.kw && cx >= 0; kx += g.sw, --cx) {
+            if (cx >= g.ow) continue;
+            acc = acc + col[base + (i64)(ky * g.kw + kx) * tap_stride + cy * g.ow + cx];
+        }
+    }
+    out[idx] = acc;
+}
+
+bool geom32(Geom32& q, const ConvGeom& g) {
+    const i64 N = g.B * g.oh * g.ow, rows = g.C * g.kh * g.kw;
+    const i64 lim = 0x7fffffff;
+    if (g.B * g.C * g.H * g.W > lim || N > lim - 4 || g.H + 2 * g.ph > lim || g.W + 2 * g.pw > lim) return false;
+    q.B = (int)g.B; q.C = (int)g.C; q.H = (int)g.H; q.W = (int)g.W; q.kh = (int)g.kh; q.kw = (int)g.kw;
+    q.sh = (int)g.sh; q.sw = (int)g.sw; q.ph = (int)g.ph; q.pw = (int)g.pw; q.oh = (int)g.oh; q.ow = (int)g.ow;
+    q.div_L = make_div((uint32_t)(g.oh * g.ow)); q.div_ow = make_div((uint32_t)g.ow);
+    q.div_KK = make_div((uint32_t)(g.kh * g.kw)); q.div_kw = make_div((uint32_t)g.kw);
+    q.div_W = make_div((uint32_t)g.W); q.div_H = make_div((uint32_t)g.H); q.div_C = make_div((uint32_t)g.C);
+    q.div_sh = make_div((uint32_t)g.sh); q.div_sw = make_div((uint32_t)g.sw);
+    return true;
+}
+
 template <typename T>
 int im2col(fx_ctx* c, const T* x, T* col, i64 B, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw) {
     FX_CHECK_CTX(c);
@@ -86,6 +175,16 @@ int im2col(fx_ctx* c, const T* x, T* col, i64 B, i64 C, i64 H, i64 W, i64 kh, i6
     const i64 N = B * g.oh * g.ow, rows = C * kh * kw;
     FX_REQUIRE(rows <= 65535, "fx_im2col: C*kh*kw = %lld exceeds 65535", (long long)rows);
     FX_REQUIRE(fx::ceil_div(N, 256) <= 0x7fffffff, "fx_im2col: too many columns");
+    Geom32 q;
+    if (geom32(q, g)) {
+        constexpr int V = 16 / (int)sizeof(T);
+        if (N % V == 0 && fx::aligned16(col))
+            im2col32_kernel<T, V><<<dim3((unsigned)fx::ceil_div(N / V, 256), (unsigned)rows), dim3(256), 0, c->stream>>>(x, col, q, (uint32_t)N);
+        else
+            im2col32_kernel<T, 1><<<dim3((unsigned)fx::ceil_div(N, 256), (unsigned)rows), dim3(256), 0, c->stream>>>(x, col, q, (uint32_t)N);
+        FX_LAUNCH_CHECK();
+        return FX_OK;
+    }
     im2col_kernel<T><<<dim3((unsigned)fx::ceil_div(N, 256), (unsigned)rows), dim3(256), 0, c->stream>>>(x, col, g);
     FX_LAUNCH_CHECK();
     return FX_OK;
@@ -102,6 +201,13 @@ int col2im(fx_ctx* c, const T* col, T* out, i64 B, i64 C, i64 H, i64 W, i64 kh, 
     const i64 total = B * C * H * W;
     FX_REQUIRE(fx::ceil_div(total, 256) <= 0x7fffffff, "fx_col2im: too many pixels");
     const dim3 grid((unsigned)fx::ceil_div(total, 256)), block(256);
+    Geom32 q;
+    if (geom32(q, g)) {
+        if (layout == 1) col2im32_kernel<T, 1><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
+        else col2im32_kernel<T, 0><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
+        FX_LAUNCH_CHECK();
+        return FX_OK;
+    }
     if (layout == 1) col2im_kernel<T, 1><<<grid, block, 0, c->stream>>>(col, out, g);
     else col2im_kernel<T, 0><<<grid, block, 0, c->stream>>>(col, out, g);
     FX_LAUNCH_CHECK();

@@ -152,6 +152,9 @@ def test_materialize_views_bit_exact(ctx, dtype):
         ((3, 4, 5, 6), (1, 3, 12, 60)),            # full reversal of a [6,5,4,3] tensor
         ((7, 12), (24, 2)), ((5, 9, 4), (0, 4, 1)), ((2, 3, 1, 4, 1, 5), (60, 20, 0, 5, 0, 1)),
         ((2, 2, 2, 2, 2, 2, 2, 4), (512, 1024, 64, 128, 16, 32, 4, 1)), ((1,), (0,)), ((9,), (3,)), ((16,), (0,)),
+        # the LDS-tiled transpose: ragged tiles, a batch of transposes, a padded leading dimension, a broadcast batch
+        ((130, 67), (1, 130)), ((5, 70, 33), (2310, 1, 70)), ((40, 50), (1, 64)), ((4, 30, 20), (0, 1, 30)), ((16, 16), (1, 16)),
+        ((15, 64), (1, 15)), ((3, 17, 19), (400, 1, 21)),
     ]
     for shape, strides in views:
         want = np.ascontiguousarray(as_strided(base, shape, tuple(s_ * item for s_ in strides)))
