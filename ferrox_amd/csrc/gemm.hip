@@ -2,7 +2,9 @@
 // Replaces kernels/matmul.cu (16x16 shared-memory tiles, 75 % of threads idle) and serves MatMul::compute /
 // MatMul::gradient (src/ops/matrix.rs:17-55) without materialised transposes via the trans flags.
 // Small or skinny products are split along K into deterministic partial sums (no atomics).
-#include "igemm_core.hpp"
+#include <cstdlib>
+
+#include "gemm_lds.hpp"
 
 extern "C" int fx_bias_act_f32(fx_ctx*, float*, const float*, int64_t, int64_t, int64_t, int);
 extern "C" int fx_bias_act_f64(fx_ctx*, double*, const double*, int64_t, int64_t, int64_t, int);
@@ -61,7 +63,15 @@ int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B,
     {
         std::lock_guard<std::mutex> lk(c->launch_mutex);
         int rc;
-        if (K == 0) {  // empty sum
+        bool lds_path = false;
+        if constexpr (sizeof(T) == 4) {
+            static const bool generic_only = std::getenv("FX_GEMM_GENERIC") != nullptr;  // A/B timing switch
+            const glk::Plan pl = glk::make_plan(c->num_cus, ta != 0, tb != 0, M, N, K, ta ? M : K, tb ? K : N);
+            lds_path = pl.ok && !generic_only && fx::aligned16(A) && fx::aligned16(B) && fx::aligned16(C);
+            if (lds_path) rc = glk::run(c, pl, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu);
+        }
+        if (lds_path) {
+        } else if (K == 0) {  // empty sum
             rc = launch_zero<T>(c, C, M * N);
             pending = bias != nullptr;
         } else if (M >= 128 && N >= 128) rc = run_trans<T, TileBig>(c, ta, tb, M, N, K, A, B, C, bias, relu, &pending);

@@ -63,6 +63,16 @@ template <> struct Mfma<double> {
 };
 
 // Block tile BM x BN x BK computed by (BM/WM) x (BN/WN) waves, each owning a WM x WN sub-tile.
+// 16-byte load from global memory at a wave-uniform base plus a 32-bit byte offset (never a FLAT access, so it
+// does not tie up the LDS counter that the MFMA loop waits on).
+__device__ __forceinline__ float4 ldg4(const float* base, uint32_t byteoff) {
+    typedef __attribute__((address_space(1))) const char gchar;
+    typedef float v4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(1))) const v4 gv4;
+    const v4 v = *(gv4*)((gchar*)base + byteoff);
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+
 template <int BM_, int BN_, int BK_, int WM_, int WN_> struct Tile {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
     static constexpr int WAVES_M = BM / WM, WAVES_N = BN / WN;

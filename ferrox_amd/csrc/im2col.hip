@@ -154,7 +154,7 @@ __global__ __launch_bounds__(256) void col2im32_kernel(const T* __restrict__ col
 }
 
 bool geom32(Geom32& q, const ConvGeom& g) {
-    const i64 N = g.B * g.oh * g.ow, rows = g.C * g.kh * g.kw;
+    const i64 N = g.B * g.oh * g.ow;
     const i64 lim = 0x7fffffff;
     if (g.B * g.C * g.H * g.W > lim || N > lim - 4 || g.H + 2 * g.ph > lim || g.W + 2 * g.pw > lim) return false;
     q.B = (int)g.B; q.C = (int)g.C; q.H = (int)g.H; q.W = (int)g.W; q.kh = (int)g.kh; q.kw = (int)g.kw;

@@ -34,15 +34,7 @@ constexpr int LPR = 16, RPP = NT / LPR;     // lanes per staged row, rows covere
 constexpr int SLACK = 64;                   // floats behind the last plane that the look-ahead read may touch
 constexpr size_t LDS_BUDGET = 72 * 1024;    // per block, so that two blocks share a CU
 
-// 16-byte load from global memory at a wave-uniform base plus a 32-bit byte offset (never a FLAT access, so it
-// does not tie up the LDS counter that the MFMA loop waits on).
-__device__ __forceinline__ float4 ldg4(const float* base, uint32_t byteoff) {
-    typedef __attribute__((address_space(1))) const char gchar;
-    typedef float v4 __attribute__((ext_vector_type(4)));
-    typedef __attribute__((address_space(1))) const v4 gv4;
-    const v4 v = *(gv4*)((gchar*)base + byteoff);
-    return make_float4(v.x, v.y, v.z, v.w);
-}
+using igemm::ldg4;
 
 struct Params {
     const float* x;

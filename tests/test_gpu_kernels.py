@@ -299,6 +299,36 @@ def test_gemm_all_transposes(ctx, orc, golden, dtype):
     assert got.shape == (64, 64)
 
 
+# Products large enough for the LDS-slab f32 kernel on a 256-CU device (at least 384 tiles of 128 x 128, K % 64 == 0):
+# exact tiles, ragged M and N (rows / columns past the matrix are re-read, never stored), N below one tile.
+GEMM_LDS_SHAPES = [(2560, 2560, 128), (2500, 2436, 192), (4096, 3200, 64 * 3), (49152, 100, 128), (128 * 50, 1024 + 4, 256)]
+
+
+def test_gemm_lds_kernel_shapes_all_transposes_and_bias(ctx):
+    from ferrox_amd import capi
+    rng = np.random.default_rng(41)
+    tol = TOL[np.dtype(np.float32)]
+    for (M, N, K) in GEMM_LDS_SHAPES:
+        a = rng.standard_normal((M, K)).astype(np.float32)
+        b = rng.standard_normal((K, N)).astype(np.float32)
+        truth = a.astype(np.float64) @ b.astype(np.float64)
+        scale = (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)).max()
+        bias = rng.standard_normal(N).astype(np.float32)
+        dbias = ctx.upload(bias)
+        for ta in (False, True):
+            for tb in (False, True):
+                da = ctx.upload(np.ascontiguousarray(a.T) if ta else a)
+                db = ctx.upload(np.ascontiguousarray(b.T) if tb else b)
+                got = ctx.gemm(da, db, ta, tb)
+                assert np.abs(got.numpy() - truth).max() <= tol * scale, (M, N, K, ta, tb)
+                # same bits run to run, and the bias (+ReLU) epilogue equals the two-call sequence
+                assert np.array_equal(ctx.gemm(da, db, ta, tb).numpy(), got.numpy()), (M, N, K, ta, tb)
+                fused = ctx.empty((M, N), np.float32)
+                capi.check(capi.lib.fx_gemm_bias_act_f32(ctx.h, int(ta), int(tb), M, N, K, da.ptr, db.ptr, dbias.ptr, fused.ptr, 1))
+                ctx.bias_act(got, dbias, M, N, 1, act=1)
+                assert np.array_equal(fused.numpy(), got.numpy()), (M, N, K, ta, tb)
+
+
 def test_gemm_shape_mismatch_message(ctx):
     from ferrox_amd.capi import FerroxHipError
     a = ctx.upload(np.zeros((2, 3), np.float32))
