@@ -35,6 +35,7 @@ struct Params {
     int relu;
     int C, H, W, M, OH, OW, sh, sw, ph, pw;
     int PR, PW, PLANE, L, tpi, nchunks;
+    int xcd_chunk;  // gridDim.x / 8 when that divides: workgroup ids go to the 8 XCDs round-robin, see the kernel
     FastDiv div_tpi, div_ow;
 };
 
@@ -68,9 +69,13 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
     float* Ws = smem;
     float* Xs = smem + WIMG;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
-    const int b = (int)p.div_tpi.div(blockIdx.x);
+    // XCD x takes the contiguous range [x * chunk, (x+1) * chunk) of (image, pixel tile) pairs, so neighbouring tiles
+    // of an image (which share input rows) and the weight images meet in one L2
+    int bx = blockIdx.x;
+    if (p.xcd_chunk) bx = (bx & 7) * p.xcd_chunk + (bx >> 3);
+    const int b = (int)p.div_tpi.div((uint32_t)bx);
     const int wm = wave % WM, wn = wave / WM;
-    const int pix0 = ((int)blockIdx.x - b * p.tpi) * NPIX;
+    const int pix0 = (bx - b * p.tpi) * NPIX;
     const int wpix0 = pix0 + wn * 32 * TN;  // first pixel of this wave's columns
     const int m0 = blockIdx.y * BM;
     const int py0 = (int)p.div_ow.div((uint32_t)pix0);
@@ -271,6 +276,7 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
     p.div_tpi = FastDiv((uint32_t)pl.tpi);
     p.div_ow = FastDiv((uint32_t)OW);
     const dim3 grid((unsigned)(B * pl.tpi), (unsigned)pl.mtiles);
+    p.xcd_chunk = (B * pl.tpi) % 8 == 0 ? (int)(B * pl.tpi / 8) : 0;
 #define FX_CPK_LAUNCH(WMV, TNV)                                                                                       \
     case WMV * 16 + TNV: {                                                                                            \
         static const hipError_t attr0 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, false>,          \

@@ -43,6 +43,7 @@ struct Params {
     int Cin, H, W, Cout, oh, ow, sh, sw, ph, pw;
     int R, PW, PLANE, GP, Kst;  // rows per stage, patch width, plane pitch, g pitch, pixels per stage
     int stages, sps, spi;       // all stages, stages per split, stages per image
+    int xcd_chunk;              // blocks / 8 when that divides (see the kernel), else 0
     FastDiv div_spi;
     i64 part_stride;
 };
@@ -58,7 +59,18 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
     float* Gs = smem;
     float* Xs = smem + BM * p.GP;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
-    const int c0 = blockIdx.x * CT, oc0 = blockIdx.y * BM;
+    // Workgroup ids go to the 8 XCDs round-robin; remapped so that each XCD takes a contiguous range of
+    // (split, oc tile, channel tile) triples: the channel tiles of one split read the same rows of g through one L2.
+    int bxi = blockIdx.x, byi = blockIdx.y, bzi = blockIdx.z;
+    if (p.xcd_chunk) {
+        const int lin = bxi + gridDim.x * (byi + gridDim.y * bzi);
+        const int id = (lin & 7) * p.xcd_chunk + (lin >> 3);
+        bxi = id % gridDim.x;
+        const int rest = id / gridDim.x;
+        byi = rest % gridDim.y;
+        bzi = rest / gridDim.y;
+    }
+    const int c0 = bxi * CT, oc0 = byi * BM;
     const int L = p.oh * p.ow;
     const int k4 = p.Kst >> 2, w4 = p.W >> 2;
 
@@ -168,7 +180,7 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
         }
     };
 
-    const int s_beg = blockIdx.z * p.sps, s_end = min(p.stages, s_beg + p.sps);
+    const int s_beg = bzi * p.sps, s_end = min(p.stages, s_beg + p.sps);
     if (s_beg < s_end) {
         prefetch(s_beg);
         park();
@@ -187,7 +199,7 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
         __syncthreads();
     }
 
-    float* out = p.part + ((i64)blockIdx.z * WK + wk) * p.part_stride;
+    float* out = p.part + ((i64)bzi * WK + wk) * p.part_stride;
     const int ldo = KK * p.Cin;
 #pragma unroll
     for (int t = 0; t < KK; ++t)
@@ -314,6 +326,8 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
     p.div_spi = FastDiv((uint32_t)p.spi);
     p.part_stride = Cout * Cin * KK;
     const dim3 grid((unsigned)(Cin / pl.ct()), (unsigned)fx::ceil_div(Cout, (i64)pl.bm()), (unsigned)pl.splits);
+    const i64 blocks = (i64)grid.x * grid.y * grid.z;
+    p.xcd_chunk = blocks % 8 == 0 && blocks <= 0x7fffffff ? (int)(blocks / 8) : 0;
 #define FX_WGP_LAUNCH(XRV, A, B_, C_)                                                                                 \
     do {                                                                                                              \
         static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_patch_kernel<XRV, A, B_, C_>,           \
