@@ -204,3 +204,33 @@ def test_reduce_prod_within_tolerance(ctx, orc, dtype):
     z = np.ones((4, 100), dtype)
     z[2, 17] = 0
     assert np.array_equal(ctx.reduce("prod", ctx.upload(z), 1).numpy(), np.array([1, 1, 0, 1], dtype))
+
+
+def test_new_entry_points_reject_bad_arguments(ctx):
+    """Argument checks run on the host before any launch: null pointers, empty or negative views, bad flags."""
+    from ferrox_amd import capi
+    from ferrox_amd.capi import FerroxHipError
+    x = ctx.fill((4, 3, 5, 5), 1.0)
+    v3 = ctx.fill((3,), 1.0)
+    lib, h = capi.lib, ctx.h
+
+    def fails(rc, text):
+        with pytest.raises(FerroxHipError, match=text):
+            capi.check(rc)
+
+    fails(lib.fx_batchnorm_stats_f32(h, None, v3.ptr, v3.ptr, None, None, 0.1, 4, 3, 25), "null pointer")
+    fails(lib.fx_batchnorm_stats_f32(h, x.ptr, v3.ptr, v3.ptr, None, None, 0.1, 0, 3, 25), "bad view")
+    fails(lib.fx_batchnorm_fwd_f32(h, x.ptr, v3.ptr, v3.ptr, v3.ptr, None, 1e-5, x.ptr, 4, 3, 25, 0), "null pointer")
+    fails(lib.fx_batchnorm_fwd_f32(h, x.ptr, v3.ptr, v3.ptr, v3.ptr, v3.ptr, 1e-5, x.ptr, 4, 3, 25, 2), "act must be")
+    fails(lib.fx_batchnorm_bwd_f32(h, x.ptr, x.ptr, None, v3.ptr, v3.ptr, v3.ptr, 1e-5, x.ptr, v3.ptr, None, 4, 3, 25, 1), "null pointer")
+    fails(lib.fx_batchnorm_bwd_f32(h, x.ptr, x.ptr, None, v3.ptr, v3.ptr, v3.ptr, 1e-5, x.ptr, v3.ptr, v3.ptr, 4, 3, 25, 7), "batch_stats")
+    fails(lib.fx_dropout_f32(h, x.ptr, x.ptr, x.ptr, 300, 1.0, 1), r"p must be in \[0, 1\)")
+    fails(lib.fx_dropout_f32(h, x.ptr, None, x.ptr, 300, 0.5, 1), "null pointer")
+    fails(lib.fx_reduce_prod_f32(h, x.ptr, None, 4, 75, 1), "null pointer")
+    import ctypes as C
+    tab = (C.c_void_p * 2)(x.ptr, None)
+    ns = (C.c_int64 * 2)(300, 300)
+    fails(lib.fx_adam_step_multi_f32(h, 2, tab, tab, tab, tab, ns, 1e-3, 0.9, 0.999, 1e-8, 0.0, 0.1, 0.001), "null pointer in tensor 1")
+    fails(lib.fx_sgd_step_multi_f32(h, -1, tab, tab, ns, 0.1), "negative tensor count")
+    assert lib.fx_dropout_f32(h, x.ptr, x.ptr, x.ptr, 0, 0.5, 1) == 0          # nothing to do is not an error
+    assert lib.fx_batchnorm_fwd_f32(h, None, None, None, None, None, 1e-5, None, 0, 3, 25, 0) == 0

@@ -169,6 +169,8 @@ def test_entry_points_are_thread_safe():
         g = rng.standard_normal((4, 96, 12, 56)).astype(np.float32)
         m = rng.standard_normal((512, 2048)).astype(np.float32)
         dx_, dw_, dg_, dm_ = ctx.upload(x), ctx.upload(w), ctx.upload(g), ctx.upload(m)
+        dgam0 = ctx.upload(np.ones(96, np.float32))
+        dgs_ = ctx.upload(rng.standard_normal((4, 96, 6, 28)).astype(np.float32))
 
         def work():
             y = ctx.conv2d_fwd(dx_, dw_, (1, 1), (1, 1)).numpy()
@@ -177,7 +179,11 @@ def test_entry_points_are_thread_safe():
             s0 = ctx.reduce("sum", dm_, 0).numpy()
             mx = ctx.reduce("max", dm_, 1).numpy()
             bg = ctx.bias_grad(dg_, 4, 96, 12 * 56).numpy()
-            return y, dw, dxx, s0, mx, bg
+            mean, var = ctx.batchnorm_stats(dg_)                      # partial moments in the shared scratch
+            _, dgam, dbet = ctx.batchnorm_bwd(dg_, dg_, mean, var, dgam0, 1e-5, need_dx=False)
+            sdx = ctx.conv2d_dgrad(dgs_, dw_, x.shape, (2, 2), (1, 1)).numpy()   # class sub-filters in the scratch
+            mm = ctx.gemm(dm_, dm_, False, True).numpy()                # split-K partial sums
+            return y, dw, dxx, s0, mx, bg, mean.numpy(), var.numpy(), dgam.numpy(), dbet.numpy(), sdx, mm
 
         want = work()
         results, errors = {}, []
