@@ -134,6 +134,7 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_conv2d_fwd_bias_act_{_s}", _vp, _vp, _vp, _vp, _vp, *_CONV_INTS, _int, _vp, _i64)
     _sig(f"fx_gemm_bias_act_{_s}", _vp, _int, _int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _int)
     _sig(f"fx_bias_grad_{_s}", _vp, _vp, _vp, _i64, _i64, _i64)
+    _sig(f"fx_relu_bwd_bias_grad_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64)
     _sig(f"fx_softmax_ce_fwd_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64)
     _sig(f"fx_softmax_ce_bwd_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64)
     _sig(f"fx_adam_step_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, *([_ct] * 7))
@@ -484,6 +485,12 @@ class Context:
         o = self.empty((C,), g.dtype)
         check(self._fn("bias_grad", g.dtype)(self.h, g.ptr, o.ptr, outer, C, inner))
         return o
+
+    def relu_bwd_bias_grad(self, g, y, outer, C, inner):
+        """(g * (y > 0), its per-channel sum) in one pass."""
+        gm, db = self.empty(g.shape, g.dtype), self.empty((C,), g.dtype)
+        check(self._fn("relu_bwd_bias_grad", g.dtype)(self.h, g.ptr, y.ptr, gm.ptr, db.ptr, outer, C, inner))
+        return gm, db
 
     def softmax_ce_fwd(self, logits, targets):
         B, Cc = logits.shape

@@ -120,6 +120,55 @@ __global__ __launch_bounds__(256) void bias_grad_partial_kernel(const T* __restr
     if (threadIdx.x == 0) part[slice * C + c] = sm[0];
 }
 
+// The same reduction fused with the ReLU gradient that precedes it in a conv / linear layer with a folded activation:
+// gm = (y > 0 ? g : 0) is written out (the weight and data gradients read it) and summed per channel in one pass.
+template <typename T>
+__global__ __launch_bounds__(256) void relu_bias_grad_partial_kernel(const T* __restrict__ g, const T* __restrict__ y, T* __restrict__ gm,
+                                                                     T* __restrict__ part, i64 outer, i64 C, i64 inner, i64 rows_per_slice) {
+    __shared__ T sm[256];
+    const i64 c = blockIdx.x, slice = blockIdx.y;
+    const i64 o0 = slice * rows_per_slice, o1 = min(outer, o0 + rows_per_slice);
+    T s = T(0);
+    constexpr int V = 16 / (int)sizeof(T);
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    if (inner % V == 0 && ((uintptr_t)g & 15) == 0 && ((uintptr_t)y & 15) == 0 && ((uintptr_t)gm & 15) == 0) {
+        // threads walk the (row, vector) pairs of the slice, so every thread is busy whatever `inner` is
+        vec_t acc = vec_t(T(0));
+        const i64 nv = inner / V, pairs = (o1 - o0) * nv;
+        i64 o = o0 + threadIdx.x / nv, iv = threadIdx.x % nv;  // pair q = (row, vector); stepped without a division per load
+        const i64 dq = 256 / nv, dr = 256 % nv;
+        for (i64 q = threadIdx.x; q < pairs; q += 256) {
+            const i64 off = (o * C + c) * inner + iv * V;
+            o += dq;
+            iv += dr;
+            if (iv >= nv) { iv -= nv; ++o; }
+            vec_t gv = *reinterpret_cast<const vec_t*>(g + off);
+            const vec_t yv = *reinterpret_cast<const vec_t*>(y + off);
+#pragma unroll
+            for (int u = 0; u < V; ++u) gv[u] = gv[u] * (yv[u] > T(0) ? T(1) : T(0));  // ReluBwdF of the elementwise kernel
+            *reinterpret_cast<vec_t*>(gm + off) = gv;
+            acc = acc + gv;
+        }
+#pragma unroll
+        for (int u = 0; u < V; ++u) s = s + acc[u];
+    } else {
+        const i64 total = (o1 - o0) * inner;
+        for (i64 t = threadIdx.x; t < total; t += 256) {
+            const i64 off = ((o0 + t / inner) * C + c) * inner + t % inner;
+            const T v = g[off] * (y[off] > T(0) ? T(1) : T(0));
+            gm[off] = v;
+            s = s + v;
+        }
+    }
+    sm[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) sm[threadIdx.x] = sm[threadIdx.x] + sm[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) part[slice * C + c] = sm[0];
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void bias_grad_final_kernel(const T* __restrict__ part, T* __restrict__ out, i64 C, int slices) {
     const i64 c = (i64)blockIdx.x * 256 + threadIdx.x;
@@ -129,11 +178,12 @@ __global__ __launch_bounds__(256) void bias_grad_final_kernel(const T* __restric
     out[c] = s;
 }
 
+// y != nullptr: the fused ReLU-gradient form (gm receives the masked gradient)
 template <typename T>
-int bias_grad(fx_ctx* c, const T* g, T* out, i64 outer, i64 C, i64 inner) {
+int bias_grad(fx_ctx* c, const T* g, T* out, i64 outer, i64 C, i64 inner, const T* y = nullptr, T* gm = nullptr) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(outer >= 1 && C >= 1 && inner >= 1, "fx_bias_grad: bad view");
-    FX_REQUIRE(g && out, "fx_bias_grad: null pointer");
+    FX_REQUIRE(g && out && (y == nullptr) == (gm == nullptr), "fx_bias_grad: null pointer");
     FX_REQUIRE(C <= 0x7fffffff, "fx_bias_grad: too many channels");
     // enough blocks to fill the chip, at least 8 rows (or 16k elements) per block
     i64 slices = std::max<i64>(1, std::min<i64>((i64)c->num_cus * 4 / C, 65535));
@@ -147,7 +197,8 @@ int bias_grad(fx_ctx* c, const T* g, T* out, i64 outer, i64 C, i64 inner) {
         part = (T*)c->get_scratch(slices * C * (i64)sizeof(T));
         if (!part) return FX_ERR_OOM;
     }
-    bias_grad_partial_kernel<T><<<dim3((unsigned)C, (unsigned)slices), dim3(256), 0, c->stream>>>(g, part, outer, C, inner, rps);
+    if (y) relu_bias_grad_partial_kernel<T><<<dim3((unsigned)C, (unsigned)slices), dim3(256), 0, c->stream>>>(g, y, gm, part, outer, C, inner, rps);
+    else bias_grad_partial_kernel<T><<<dim3((unsigned)C, (unsigned)slices), dim3(256), 0, c->stream>>>(g, part, outer, C, inner, rps);
     FX_LAUNCH_CHECK();
     if (slices > 1) {
         bias_grad_final_kernel<T><<<dim3((unsigned)fx::ceil_div(C, (i64)256)), dim3(256), 0, c->stream>>>(part, out, C, (int)slices);
@@ -365,6 +416,11 @@ int sgd_step(fx_ctx* c, T* p, const T* g, i64 n, T lr) {
     }                                                                                                                  \
     extern "C" int fx_bias_grad_##S(fx_ctx* c, const T* g, T* out, int64_t outer, int64_t C, int64_t inner) {          \
         return bias_grad<T>(c, g, out, outer, C, inner);                                                               \
+    }                                                                                                                  \
+    extern "C" int fx_relu_bwd_bias_grad_##S(fx_ctx* c, const T* g, const T* y, T* gm, T* dbias, int64_t outer,        \
+                                             int64_t C, int64_t inner) {                                               \
+        FX_REQUIRE(y && gm, "fx_relu_bwd_bias_grad: null pointer");                                                    \
+        return bias_grad<T>(c, g, dbias, outer, C, inner, y, gm);                                                      \
     }                                                                                                                  \
     extern "C" int fx_softmax_ce_fwd_##S(fx_ctx* c, const T* logits, const T* targets, T* probs, T* loss, int64_t B,   \
                                          int64_t C) {                                                                  \

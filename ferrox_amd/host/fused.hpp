@@ -34,6 +34,9 @@ template <typename T> struct FusedApi;
         }                                                                                                              \
         static int sgd_multi(fx_ctx* c, int k, T* const* p, const T* const* g, const int64_t* n, T lr) { return fx_sgd_step_multi_##S(c, k, p, g, n, lr); } \
         static int relu_bwd(fx_ctx* c, const T* g, const T* x, T* o, int64_t n) { return fx_relu_bwd_##S(c, g, x, o, n); } \
+        static int relu_bias_grad(fx_ctx* c, const T* g, const T* y, T* gm, T* db, int64_t o, int64_t C, int64_t i) {  \
+            return fx_relu_bwd_bias_grad_##S(c, g, y, gm, db, o, C, i);                                                \
+        }                                                                                                              \
         static int gemm_bias(fx_ctx* c, int ta, int tb, int64_t M, int64_t N, int64_t K, const T* A, const T* B, const T* b, T* C, int act) { \
             return fx_gemm_bias_act_##S(c, ta, tb, M, N, K, A, B, b, C, act);                                          \
         }                                                                                                              \
@@ -84,16 +87,19 @@ template <typename T> struct LinearFusedOp : Operator<T> {  // inputs: x [B, in]
                                           const std::vector<bool>& needs) const override {
         const Shape &xs = in[0]->shape(), &ws = in[1]->shape();
         const int64_t B = (int64_t)xs[0], I = (int64_t)xs[1], O = (int64_t)ws[0];
-        if (relu) g = relu_mask_grad<T>(*g, *out);
         std::vector<Tensor<T>> r(3);
+        r[2] = HipStorage<T>::alloc({ws[0]});
+        if (relu) {  // mask and bias gradient in one pass over g
+            Tensor<T> gm = HipStorage<T>::alloc(g->shape());
+            fx_ok(FusedApi<T>::relu_bias_grad(fused_ctx(), g->data(), out->data(), gm->data(), r[2]->data(), B, O, 1));
+            g = std::move(gm);
+        } else fx_ok(FusedApi<T>::bias_grad(fused_ctx(), g->data(), r[2]->data(), B, O, 1));
         if (needs[0]) {
             r[0] = HipStorage<T>::alloc(xs);
             fx_ok(Api<T>::gemm(fused_ctx(), 0, 0, B, I, O, g->data(), in[1]->data(), r[0]->data()));
         }
         r[1] = HipStorage<T>::alloc(ws);
         fx_ok(Api<T>::gemm(fused_ctx(), 1, 0, O, I, B, g->data(), in[0]->data(), r[1]->data()));
-        r[2] = HipStorage<T>::alloc({ws[0]});
-        fx_ok(FusedApi<T>::bias_grad(fused_ctx(), g->data(), r[2]->data(), B, O, 1));
         return r;
     }
     size_t num_inputs() const override { return 3; }
@@ -119,13 +125,17 @@ template <typename T> struct Conv2dFusedOp : Operator<T> {  // inputs: x [B,Cin,
     }
     std::vector<Tensor<T>> gradient_needs(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>* out,
                                           const std::vector<bool>& needs) const override {
-        if (relu) g = relu_mask_grad<T>(*g, *out);
-        const Shape& gs = g->shape();
+        const Shape gs = g->shape();
         std::vector<Tensor<T>> r(3);
+        r[2] = HipStorage<T>::alloc({gs[1]});
+        if (relu) {  // mask and bias gradient in one pass over g
+            Tensor<T> gm = HipStorage<T>::alloc(gs);
+            fx_ok(FusedApi<T>::relu_bias_grad(fused_ctx(), g->data(), out->data(), gm->data(), r[2]->data(), (int64_t)gs[0], (int64_t)gs[1],
+                                              (int64_t)(gs[2] * gs[3])));
+            g = std::move(gm);
+        } else fx_ok(FusedApi<T>::bias_grad(fused_ctx(), g->data(), r[2]->data(), (int64_t)gs[0], (int64_t)gs[1], (int64_t)(gs[2] * gs[3])));
         if (needs[0]) r[0] = g->deconv2d(*in[1], in[0]->shape(), stride, padding);
         r[1] = in[0]->cross_correlation2d(*g, in[1]->shape(), stride, padding);
-        r[2] = HipStorage<T>::alloc({gs[1]});
-        fx_ok(FusedApi<T>::bias_grad(fused_ctx(), g->data(), r[2]->data(), (int64_t)gs[0], (int64_t)gs[1], (int64_t)(gs[2] * gs[3])));
         return r;
     }
     size_t num_inputs() const override { return 3; }

@@ -131,6 +131,15 @@ template <typename T> class HipStorage {
         s->ptr_ = static_cast<T*>(p);
         return s;
     }
+    // A storage that aliases another one's device memory without owning it (the caller keeps the original alive):
+    // used by the fused training loop for the batch, which the reference clones every step (training.rs:125-126).
+    static Ptr borrow(const HipStorage& src) {
+        Ptr s(new HipStorage());
+        s->shape_ = src.shape_;
+        s->ptr_ = src.ptr_;
+        s->borrowed_ = true;
+        return s;
+    }
     static Ptr full(const Shape& shape, T value) {
         Ptr s = alloc(shape);
         fx_ok(Api<T>::fill(ctx(), s->ptr_, value, (int64_t)s->size()));
@@ -407,7 +416,7 @@ template <typename T> class HipStorage {
     HipStorage() = default;
     static fx_ctx* ctx() { return BackendManager::get().ctx(); }
     void release() {
-        if (ptr_ && BackendManager::get().has_hip()) fx_free(ctx(), Api<T>::dtype, ptr_, id_);
+        if (ptr_ && !borrowed_ && BackendManager::get().has_hip()) fx_free(ctx(), Api<T>::dtype, ptr_, id_);
         ptr_ = nullptr;
     }
     static void oai(const Shape& s, size_t axis, int64_t& outer, int64_t& ax, int64_t& inner) {
@@ -443,6 +452,7 @@ template <typename T> class HipStorage {
         std::swap(ptr_, r->ptr_);
         std::swap(id_, r->id_);
         std::swap(granted_, r->granted_);
+        std::swap(borrowed_, r->borrowed_);
         shape_ = ns;
     }
     Ptr pool2d(bool is_max, size_t k, size_t s, size_t p, const char* what) const {
@@ -517,6 +527,7 @@ template <typename T> class HipStorage {
     T* ptr_ = nullptr;
     uint64_t id_ = 0;
     int64_t granted_ = 0;
+    bool borrowed_ = false;
 };
 
 // Tensor<T> (src/backend/tensor.rs:20-26) is a device tag plus a boxed storage; every method forwards to the

@@ -164,8 +164,9 @@ template <typename T> struct Model : ModelBase {
     double train_step() override {
         if (!x || !y) throw Error("set_batch was not called");
         graph.zero_gradients();
-        const NodeId xin = graph.create_variable(x->clone_storage(), false);
-        const NodeId yin = graph.create_variable(y->clone_storage(), false);
+        // the reference clones the batch every step (training.rs:125-126); the fused engine reads it in place
+        const NodeId xin = graph.create_variable(fused ? HipStorage<T>::borrow(*x) : x->clone_storage(), false);
+        const NodeId yin = graph.create_variable(fused ? HipStorage<T>::borrow(*y) : y->clone_storage(), false);
         const NodeId pred = forward(xin);
         const NodeId loss = fused ? cce_loss_fused<T>(graph, pred, yin) : cce_loss<T>(graph, pred, yin);
         const T lv = graph.get_tensor(loss)->clone_storage()->first();

@@ -287,6 +287,12 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
     /* Bias gradient out[c] = sum over (o, i) of g[o, c, i]: reduce_gradient_for_broadcasting,                         \
        src/ops/basic.rs:10-53 (three axis sums for a conv bias) in one pass; fixed summation order per shape. */       \
     int fx_bias_grad_##S(fx_ctx* ctx, const T* g, T* out, int64_t outer, int64_t C, int64_t inner);                    \
+    /* ReLU::gradient (ops/unary.rs:358-375, mask taken from the activation's output y: y > 0 exactly when its input   \
+       was) followed by that bias gradient, in one pass: gm = g * (y > 0) is written for the weight / data gradients   \
+       and dbias[c] = sum of gm over (o, i).  gm has the bits of fx_relu_bwd(g, y); dbias is summed in a fixed order   \
+       of its own (equal to fx_bias_grad(gm) up to rounding). */                                                       \
+    int fx_relu_bwd_bias_grad_##S(fx_ctx* ctx, const T* g, const T* y, T* gm, T* dbias, int64_t outer, int64_t C,      \
+                                  int64_t inner);                                                                      \
     /* CCELoss with mean reduction, src/nn/losses/classification.rs:191-257: probs[B,C] = softmax(logits) (kept for    \
        the backward), loss[1] = mean_b( -sum_c targets*log(clamp(probs, 1e-8, 1-1e-8)) ).  bwd: d logits from the      \
        upstream gradient of the loss (1 element on the device) through Mean, Neg, Sum, Mul, Log, Clamp and the         \

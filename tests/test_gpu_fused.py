@@ -118,6 +118,29 @@ def test_adam_and_sgd_step_bit_exact(ctx, train, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_relu_gradient_with_bias_gradient_in_one_pass(ctx, train, dtype):
+    """fx_relu_bwd_bias_grad: the masked gradient has the bits of fx_relu_bwd, the channel sums agree with the oracle's
+    three-axis sum and with fx_bias_grad of the masked gradient to tolerance."""
+    import oracle as orc
+    rng = np.random.default_rng(76)
+    tol = TOL[np.dtype(dtype)]
+    for shape in [(4, 3, 5, 5), (8, 32, 16, 16), (256, 10), (7, 5, 1, 3), (64, 64, 8, 8), (3, 6, 4, 4), (130, 257)]:
+        g = rng.standard_normal(shape).astype(dtype)
+        y = np.maximum(rng.standard_normal(shape), 0).astype(dtype)       # an activation output: zeros where it was clipped
+        outer, C = shape[0], shape[1]
+        inner = int(np.prod(shape[2:])) if len(shape) > 2 else 1
+        dg, dy = ctx.upload(g), ctx.upload(y)
+        gm, db = ctx.relu_bwd_bias_grad(dg, dy, outer, C, inner)
+        want_gm = orc.binary("mul", g, orc.scalar("greater_scalar", y, dtype(0)))
+        assert np.array_equal(gm.numpy(), want_gm), shape
+        assert np.array_equal(gm.numpy(), ctx.relu_bwd(dg, dy).numpy()), shape
+        want_db = train.bias_grad(want_gm.reshape(shape if len(shape) == 4 else shape))
+        mag = np.abs(want_gm.astype(np.float64)).reshape(outer, C, inner).sum(axis=(0, 2)).max()
+        assert np.abs(db.numpy() - want_db).max() <= tol * max(mag, 1e-30), shape
+        assert np.abs(db.numpy() - ctx.bias_grad(gm, outer, C, inner).numpy()).max() <= tol * max(mag, 1e-30), shape
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_multi_tensor_adam_and_sgd_equal_the_per_tensor_calls(ctx, dtype):
     """fx_adam_step_multi / fx_sgd_step_multi: one launch for a parameter list, bits of the per-tensor entry points;
     30 tensors exceed one launch's table (24), sizes include 1 and a non-multiple of the block."""
