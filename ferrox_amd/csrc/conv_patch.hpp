@@ -22,7 +22,7 @@ using wgp::ldg4;
 
 constexpr int CC = 8, NT = 256, KK = 9;
 constexpr int WPITCH = KK * CC + 1;         // 73
-constexpr int NXP = 4, MAX_PR = 2 * NXP;    // patch rows are staged two per pass
+constexpr int NXP_SHORT = 4, NXP_TALL = 10;  // patch rows are staged two per pass: up to 8 rows, or 20 (strided layers)
 constexpr int LPR = 16;                     // lanes per patch row: W <= 64
 constexpr int SLACK = 16;
 constexpr size_t LDS_BUDGET = 72 * 1024;
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void wimg_kernel(const float* __restrict__ w, 
     out[i] = v;
 }
 
-template <int WM, int TN, bool BIAS>
+template <int WM, int TN, bool BIAS, int NXP>
 __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
     constexpr int BM = 32 * WM, WN = 4 / WM, NPIX = 32 * TN * WN;
     constexpr int WIMG = BM * WPITCH;             // floats in one weight image
@@ -217,6 +217,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
 struct Plan {
     bool ok = false;
     int WM = 4, TN = 0, PR = 0, PW = 0, PLANE = 0, tpi = 0, mtiles = 0, nchunks = 0;
+    bool tall = false;  // more than 8 patch rows: the NXP_TALL instantiation
     size_t smem = 0;
     int bm() const { return 32 * WM; }
     int npix() const { return 32 * TN * (4 / WM); }
@@ -236,8 +237,10 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
     for (const auto& sp : shapes) {
         const int wm = sp[0], tn = sp[1];
         const i64 bm = 32 * wm, np = 32 * tn * (4 / wm), tiles = fx::ceil_div(L, np), mtiles = fx::ceil_div(M, bm);
-        const i64 rows = std::min<i64>(OH, (np - 1) / OW + 2), PR = (rows - 1) * sh + 3;
-        if (PR > MAX_PR || mtiles * bm * 4 > M * 5) continue;  // no more than a quarter of the rows may be padding
+        // output rows under a tile: tiles that start on a row boundary cover exactly np / OW rows
+        const i64 rows = std::min<i64>(OH, np % OW == 0 ? np / OW : (np - 1) / OW + 2), PR = (rows - 1) * sh + 3;
+        const bool tall_ok = wm == 2 || tn <= 6;  // instantiated tall variants
+        if (PR > 2 * NXP_TALL || (PR > 2 * NXP_SHORT && !tall_ok) || mtiles * bm * 4 > M * 5) continue;  // at most a quarter of the rows may be padding
         const i64 cost = fx::ceil_div(B * tiles * mtiles, slots) * np * bm;
         if (best_cost < 0 || cost < best_cost) {
             best_cost = cost;
@@ -248,6 +251,7 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
         }
     }
     if (best_cost < 0) return pl;
+    pl.tall = pl.PR > 2 * NXP_SHORT;
     pl.PW = (int)(W + 2 * pw);
     pl.PLANE = wgp::odd_pitch(pl.PR * pl.PW);
     pl.smem = ((size_t)pl.wimg() + (size_t)CC * pl.PLANE + SLACK) * sizeof(float);
@@ -277,29 +281,39 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
     p.div_ow = FastDiv((uint32_t)OW);
     const dim3 grid((unsigned)(B * pl.tpi), (unsigned)pl.mtiles);
     p.xcd_chunk = (B * pl.tpi) % 8 == 0 ? (int)(B * pl.tpi / 8) : 0;
-#define FX_CPK_LAUNCH(WMV, TNV)                                                                                       \
-    case WMV * 16 + TNV: {                                                                                            \
-        static const hipError_t attr0 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, false>,          \
+#define FX_CPK_LAUNCH_N(WMV, TNV, NXPV)                                                                              \
+    {                                                                                                                 \
+        static const hipError_t attr0 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, false, NXPV>,    \
                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
-        static const hipError_t attr1 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, true>,           \
+        static const hipError_t attr1 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, true, NXPV>,     \
                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
         FX_HIP_CHECK(attr0);                                                                                          \
         FX_HIP_CHECK(attr1);                                                                                          \
-        if (bias) conv_patch_kernel<WMV, TNV, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                       \
-        else conv_patch_kernel<WMV, TNV, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                           \
-        break;                                                                                                        \
+        if (bias) conv_patch_kernel<WMV, TNV, true, NXPV><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                 \
+        else conv_patch_kernel<WMV, TNV, false, NXPV><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                     \
     }
+#define FX_CPK_LAUNCH(WMV, TNV)                                                                                       \
+    case WMV * 16 + TNV:                                                                                              \
+        if (pl.tall) FX_CPK_LAUNCH_N(WMV, TNV, NXP_TALL) else FX_CPK_LAUNCH_N(WMV, TNV, NXP_SHORT)                    \
+        break;
+#define FX_CPK_LAUNCH_SHORT(WMV, TNV)                                                                                 \
+    case WMV * 16 + TNV:                                                                                              \
+        FX_REQUIRE(!pl.tall, "conv patch kernel: no tall variant of tile %d x %d", WMV, TNV);                        \
+        FX_CPK_LAUNCH_N(WMV, TNV, NXP_SHORT)                                                                          \
+        break;
     switch (pl.WM * 16 + pl.TN) {
         FX_CPK_LAUNCH(4, 4)
         FX_CPK_LAUNCH(4, 5)
         FX_CPK_LAUNCH(4, 6)
-        FX_CPK_LAUNCH(4, 7)
-        FX_CPK_LAUNCH(4, 8)
+        FX_CPK_LAUNCH_SHORT(4, 7)
+        FX_CPK_LAUNCH_SHORT(4, 8)
         FX_CPK_LAUNCH(2, 2)
         FX_CPK_LAUNCH(2, 3)
         FX_CPK_LAUNCH(2, 4)
         default: FX_REQUIRE(false, "conv patch kernel: unexpected tile %d x %d", pl.WM, pl.TN);
     }
+#undef FX_CPK_LAUNCH_N
+#undef FX_CPK_LAUNCH_SHORT
 #undef FX_CPK_LAUNCH
     FX_LAUNCH_CHECK();
     return FX_OK;

@@ -447,6 +447,9 @@ CONV_PATCH_CASES = [
     (2, 8, 9, 64, 128, (2, 1), (1, 1)), (128, 8, 8, 40, 120, (1, 1), (1, 1)), (32, 8, 56, 56, 64, (1, 1), (1, 1)),
     (16, 8, 56, 56, 120, (1, 1), (1, 1)), (128, 8, 8, 40, 250, (1, 1), (1, 1)), (96, 8, 12, 48, 384, (1, 1), (1, 1)),
     (32, 8, 56, 56, 120, (1, 1), (1, 1)), (128, 8, 16, 64, 120, (1, 1), (1, 1)),
+    # strided layers: up to 20 patch rows under a tile
+    (8, 32, 32, 32, 64, (2, 2), (1, 1)), (4, 64, 56, 56, 128, (2, 2), (1, 1)), (2, 16, 30, 40, 60, (2, 1), (1, 1)),
+    (2, 8, 17, 24, 128, (3, 3), (1, 1)), (64, 16, 28, 28, 128, (2, 2), (1, 1)),
 ]
 
 

@@ -64,8 +64,8 @@ def wgrad_loads_in_bounds(B, Cin, H, W, Cout, st, pd):
                         assert 0 <= a and a + 4 <= xsize, ("x", (B, Cin, H, W, Cout, st, pd), a, xsize)
     return "patch"
 
-CC, KK, WPITCH, NXP = 8, 9, 73, 4
-MAX_PR = 2 * NXP
+CC, KK, WPITCH = 8, 9, 73
+NXP_SHORT, NXP_TALL = 4, 10
 def _ceil_div(a, b): return (a + b - 1) // b
 def _odd_pitch_c(n): return (n + 30) // 32 * 32 + 1
 def fwd_plan(num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
@@ -75,8 +75,9 @@ def fwd_plan(num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
     for wm, tn in [(4, 8), (4, 7), (4, 6), (4, 5), (4, 4), (2, 4), (2, 3), (2, 2)]:
         bm, np_ = 32 * wm, 32 * tn * (4 // wm)
         tiles, mtiles = _ceil_div(L, np_), _ceil_div(M, bm)
-        rows = min(OH, (np_ - 1) // OW + 2); PR = (rows - 1) * sh + 3
-        if PR > MAX_PR or mtiles * bm * 4 > M * 5: continue
+        rows = min(OH, np_ // OW if np_ % OW == 0 else (np_ - 1) // OW + 2); PR = (rows - 1) * sh + 3
+        tall_ok = wm == 2 or tn <= 6
+        if PR > 2 * NXP_TALL or (PR > 2 * NXP_SHORT and not tall_ok) or mtiles * bm * 4 > M * 5: continue
         cost = _ceil_div(B * tiles * mtiles, slots) * np_ * bm
         if best is None or cost < best[0]: best = (cost, wm, tn, PR, tiles)
     if best is None: return None
@@ -85,7 +86,8 @@ def fwd_plan(num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
     bm = 32 * wm
     smem = (bm * WPITCH + CC * PLANE + 16) * 4
     if smem > 72 * 1024: return None
-    return dict(WM=wm, TN=tn, PR=PR, tpi=tiles, mtiles=_ceil_div(M, bm), nchunks=C // CC, BM=bm, NPIX=32 * tn * (4 // wm))
+    return dict(WM=wm, TN=tn, PR=PR, tpi=tiles, mtiles=_ceil_div(M, bm), nchunks=C // CC, BM=bm, NPIX=32 * tn * (4 // wm),
+                NXP=NXP_TALL if PR > 2 * NXP_SHORT else NXP_SHORT)
 def fwd_loads_in_bounds(B, C, H, W, M, sh, sw, ph, pw):
     OH, OW = (H + 2 * ph - 3) // sh + 1, (W + 2 * pw - 3) // sw + 1
     pl = fwd_plan(256, B, C, H, W, M, OH, OW, sh, sw, ph, pw)
@@ -109,7 +111,7 @@ def fwd_loads_in_bounds(B, C, H, W, M, sh, sw, ph, pw):
                             assert 0 <= a and a + 4 <= wbuf, ("w", a, wbuf)
                         pq, xc, rp = tid & 15, (tid >> 4) & 7, tid >> 7
                         x_off = (xc * H * W + 4 * pq) if pq < (W >> 2) else 0
-                        for u in range(NXP):
+                        for u in range(pl["NXP"]):
                             r = 2 * u + rp; iy = iy_base + r
                             if r < pl["PR"] and 0 <= iy < H:
                                 a = xsrc + iy * W + x_off
@@ -130,6 +132,9 @@ FWD_SHAPES = [  # B, C, H, W, M, (sh, sw), (ph, pw): one per tile shape on a 256
     (2, 8, 9, 64, 128, (2, 1), (1, 1)), (128, 8, 8, 40, 120, (1, 1), (1, 1)), (32, 8, 56, 56, 64, (1, 1), (1, 1)),
     (16, 8, 56, 56, 120, (1, 1), (1, 1)), (128, 8, 8, 40, 250, (1, 1), (1, 1)), (96, 8, 12, 48, 384, (1, 1), (1, 1)),
     (32, 8, 56, 56, 120, (1, 1), (1, 1)), (128, 8, 16, 64, 120, (1, 1), (1, 1)),
+    # strided layers: more than 8 patch rows under a tile
+    (8, 32, 32, 32, 64, (2, 2), (1, 1)), (4, 64, 56, 56, 128, (2, 2), (1, 1)), (2, 16, 30, 40, 60, (2, 1), (1, 1)),
+    (2, 8, 17, 24, 128, (3, 3), (1, 1)), (64, 64, 56, 56, 128, (2, 2), (1, 1)),
 ]
 
 
