@@ -169,10 +169,18 @@ template <typename T> struct Model : ModelBase {
         const NodeId yin = graph.create_variable(fused ? HipStorage<T>::borrow(*y) : y->clone_storage(), false);
         const NodeId pred = forward(xin);
         const NodeId loss = fused ? cce_loss_fused<T>(graph, pred, yin) : cce_loss<T>(graph, pred, yin);
-        const T lv = graph.get_tensor(loss)->clone_storage()->first();
+        if (!fused) {
+            const T lv = graph.get_tensor(loss)->clone_storage()->first();  // device -> host: the GPU drains here (training.rs:60-64)
+            graph.backward(loss);
+            opt->step(graph);
+            return (double)lv;
+        }
+        // fused engine: the loss is copied aside and read after the backward pass and the update are enqueued, so the
+        // device never waits for the host in the middle of a step
+        Tensor<T> lcopy = graph.get_tensor(loss)->clone_storage();
         graph.backward(loss);
         opt->step(graph);
-        return (double)lv;
+        return (double)lcopy->first();
     }
     void get_param(int i, void* host) const override {
         std::vector<T> v = graph.get_tensor(params.at(i))->to_vec();
