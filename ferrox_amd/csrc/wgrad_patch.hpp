@@ -292,6 +292,8 @@ inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 k
         if ((R * ow) % 4 == 0) best = R;
     }
     // measured at [256,32,32,32] -> 64, stride 2 (16 pixels per stage): 0.063 ms here against 0.050 ms for the implicit GEMM
+    // (and with two output rows over five patch rows per stage: 0.063 against 0.053 ms there, 0.192 against 0.156 ms at
+    // [128,64,56,56] -> 128 stride 2: a strided patch stages four input values per output pixel)
     if (!best || best * ow < 24) return pl;
     pl.R = best;
     pl.PR = (int)((best - 1) * sh + kh);

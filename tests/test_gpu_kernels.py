@@ -329,6 +329,42 @@ def test_gemm_lds_kernel_shapes_all_transposes_and_bias(ctx):
                 assert np.array_equal(fused.numpy(), got.numpy()), (M, N, K, ta, tb)
 
 
+# products with one dimension of at most 16 (a classifier head and its two gradients, in the layouts the Linear layer
+# produces): (kind, M, N, K) with kind naming the thin dimension -- n: A [M,K], B stored [N,K]; k: both plain; m: A
+# stored [K,M].  They run as ragged MFMA tiles split along K, with the bias added after the ordered sum.
+GEMM_THIN_SHAPES = [
+    ("n", 256, 10, 16384), ("n", 37, 1, 1024), ("n", 130, 16, 2052), ("n", 2050, 7, 1536), ("n", 16, 13, 4096),
+    ("k", 256, 16384, 10), ("k", 19, 1028, 1), ("k", 300, 4096, 16), ("k", 17, 2052, 7),
+    ("m", 10, 16384, 256), ("m", 1, 1024, 16), ("m", 16, 1028, 1000), ("m", 7, 2052, 33), ("m", 13, 65536, 40),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_with_one_thin_dimension(ctx, dtype):
+    from ferrox_amd import capi
+    rng = np.random.default_rng(43)
+    tol = TOL[np.dtype(dtype)]
+    sfx = "f32" if dtype == np.float32 else "f64"
+    for (kind, M, N, K) in GEMM_THIN_SHAPES:
+        ta, tb = kind == "m", kind == "n"
+        a = rng.standard_normal((M, K)).astype(dtype)
+        b = rng.standard_normal((K, N)).astype(dtype)
+        truth = a.astype(np.float64) @ b.astype(np.float64)
+        scale = (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)).max()
+        da = ctx.upload(np.ascontiguousarray(a.T) if ta else a)
+        db = ctx.upload(np.ascontiguousarray(b.T) if tb else b)
+        got = ctx.gemm(da, db, ta, tb)
+        assert np.abs(got.numpy() - truth).max() <= tol * scale, (kind, M, N, K)
+        assert np.array_equal(ctx.gemm(da, db, ta, tb).numpy(), got.numpy()), (kind, M, N, K)
+        bias = rng.standard_normal(N).astype(dtype)
+        dbias = ctx.upload(bias)
+        fused = ctx.empty((M, N), dtype)
+        capi.check(getattr(capi.lib, "fx_gemm_bias_act_" + sfx)(ctx.h, int(ta), int(tb), M, N, K, da.ptr, db.ptr, dbias.ptr,
+                                                                 fused.ptr, 1))
+        ctx.bias_act(got, dbias, M, N, 1, act=1)
+        assert np.array_equal(fused.numpy(), got.numpy()), (kind, M, N, K)
+
+
 def test_gemm_shape_mismatch_message(ctx):
     from ferrox_amd.capi import FerroxHipError
     a = ctx.upload(np.zeros((2, 3), np.float32))
@@ -398,6 +434,9 @@ WGRAD_PATCH_CASES = [
     # ragged output-channel counts in the last image: the 16-row staging passes past the last channel must not be read
     (1, 32, 6, 24, 40, (1, 1), (1, 1)), (2, 64, 6, 28, 49, (1, 1), (1, 1)), (1, 32, 4, 32, 97, (1, 1), (1, 1)),
     (3, 32, 8, 12, 72, (1, 1), (1, 1)), (2, 32, 8, 16, 150, (1, 1), (1, 1)), (1, 64, 5, 56, 36, (1, 1), (1, 1)),
+    # strided layers (implicit GEMM)
+    (3, 32, 32, 32, 64, (2, 2), (1, 1)), (2, 64, 56, 56, 128, (2, 2), (1, 1)), (2, 32, 16, 24, 70, (2, 1), (1, 1)),
+    (2, 32, 13, 32, 48, (2, 2), (0, 1)),
 ]
 
 
