@@ -47,7 +47,8 @@ struct Pool {
     hipStream_t stream = nullptr;  // work that may still touch a block is queued here
     std::vector<Bucket> buckets;
     std::unordered_map<uint64_t, int> active;         // allocation id -> bucket index
-    std::unordered_map<void*, i64> live;              // every device block this pool owns -> elems
+    struct Live { i64 elems; bool held; };            // held: handed to a caller (not sitting in a bucket)
+    std::unordered_map<void*, Live> live;             // every device block this pool owns
     uint64_t counter = 0, seq = 0;
     fx_pool_stats st{};
 };
@@ -159,6 +160,7 @@ int fx_alloc(fx_ctx* c, int dtype, int64_t n, void** ptr, int64_t* granted, uint
     FX_REQUIRE(ptr && granted && id_out, "fx_alloc: null output");
     FX_REQUIRE(n != 0, "Cannot allocate zero-sized CUDA memory");
     FX_REQUIRE(n > 0, "fx_alloc: negative size");
+    FX_REQUIRE(n <= (INT64_MAX >> 4), "fx_alloc: %lld elements exceed the address space", (long long)n);
     std::lock_guard<std::mutex> lk(p->mu);
     p->counter += 1;
     const uint64_t id = p->counter;
@@ -187,6 +189,7 @@ int fx_alloc(fx_ctx* c, int dtype, int64_t n, void** ptr, int64_t* granted, uint
             if (!p->literal_ids) blk.id = id;
             p->st.bytes_pooled -= blk.elems * p->elem_size;
             p->st.bytes_in_use += blk.elems * p->elem_size;
+            p->live[blk.ptr].held = true;
             *ptr = blk.ptr; *granted = blk.elems; *id_out = blk.id;
             return FX_OK;
         }
@@ -206,7 +209,7 @@ int fx_alloc(fx_ctx* c, int dtype, int64_t n, void** ptr, int64_t* granted, uint
         set_error("Failed to allocate GPU memory: %s (%lld elements)", hipGetErrorString(e), (long long)n);
         return FX_ERR_OOM;
     }
-    p->live[d] = n;
+    p->live[d] = Pool::Live{n, true};
     p->st.device_allocs += 1;
     p->st.pool_misses += 1;  // update_stats, cuda.rs:188-192
     p->st.total_allocations += 1;
@@ -225,7 +228,9 @@ int fx_free(fx_ctx* c, int dtype, void* ptr, uint64_t id) {
     std::lock_guard<std::mutex> lk(p->mu);
     auto lv = p->live.find(ptr);
     FX_REQUIRE(lv != p->live.end(), "fx_free: pointer %p is not owned by this pool", ptr);
-    const i64 elems = lv->second;
+    FX_REQUIRE(lv->second.held, "fx_free: pointer %p was already released", ptr);
+    lv->second.held = false;
+    const i64 elems = lv->second.elems;
     p->st.bytes_in_use -= elems * p->elem_size;
     auto it = p->active.find(id);
     if (it != p->active.end()) {

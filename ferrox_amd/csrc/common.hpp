@@ -15,6 +15,7 @@ namespace fx {
 struct Pool;  // allocator.hip
 
 void set_error(const char* fmt, ...);
+int bind_device(int device);  // runtime.hip
 
 #define FX_HIP_CHECK(expr)                                                                                  \
     do {                                                                                                    \
@@ -33,7 +34,13 @@ void set_error(const char* fmt, ...);
         }                                                                                                   \
     } while (0)
 
-#define FX_CHECK_CTX(ctx) FX_REQUIRE((ctx) != nullptr, "null context")
+// Every entry point starts here: a valid context, and its device current on the calling thread (the current device is
+// per thread in HIP; a context created on one thread may be used from any other).
+#define FX_CHECK_CTX(ctx)                                                                                   \
+    do {                                                                                                    \
+        FX_REQUIRE((ctx) != nullptr, "null context");                                                       \
+        if (int _rc = fx::bind_device((ctx)->device)) return _rc;                                           \
+    } while (0)
 
 // Checks the launch itself (bad configuration shows up here, not at the next sync).
 #define FX_LAUNCH_CHECK()                                                                                   \

@@ -14,6 +14,12 @@ void set_error(const char* fmt, ...) {
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
 }
+int bind_device(int device) {
+    int cur = -1;
+    if (hipGetDevice(&cur) == hipSuccess && cur == device) return FX_OK;
+    FX_HIP_CHECK(hipSetDevice(device));
+    return FX_OK;
+}
 Pool* pool_create(const fx_pool_config* cfg, int elem_size, hipStream_t stream);
 void pool_destroy(Pool* p);
 }  // namespace fx
@@ -58,14 +64,22 @@ int fx_init(int device, const fx_pool_config* cfg, fx_ctx** out) {
     c->device = device;
     c->name = prop.name[0] ? prop.name : prop.gcnArchName;
     c->num_cus = prop.multiProcessorCount;
-    FX_HIP_CHECK(hipStreamCreate(&c->stream));
-    FX_HIP_CHECK(hipEventCreate(&c->ev_start));
-    FX_HIP_CHECK(hipEventCreate(&c->ev_stop));
-    c->pools[FX_F32] = fx::pool_create(cfg, 4, c->stream);
-    c->pools[FX_F64] = fx::pool_create(cfg, 8, c->stream);
-    if (!c->pools[0] || !c->pools[1]) {
+    hipError_t e = hipStreamCreate(&c->stream);
+    if (e == hipSuccess) e = hipEventCreate(&c->ev_start);
+    if (e == hipSuccess) e = hipEventCreate(&c->ev_stop);
+    if (e == hipSuccess) {
+        c->pools[FX_F32] = fx::pool_create(cfg, 4, c->stream);
+        c->pools[FX_F64] = fx::pool_create(cfg, 8, c->stream);
+    }
+    if (e != hipSuccess || !c->pools[0] || !c->pools[1]) {
+        if (e != hipSuccess) fx::set_error("fx_init: %s", hipGetErrorString(e));  // else pool_create has set the message
+        fx::pool_destroy(c->pools[0]);
+        fx::pool_destroy(c->pools[1]);
+        if (c->ev_start) (void)hipEventDestroy(c->ev_start);
+        if (c->ev_stop) (void)hipEventDestroy(c->ev_stop);
+        if (c->stream) (void)hipStreamDestroy(c->stream);
         delete c;
-        return FX_ERR_INVALID;
+        return e != hipSuccess ? FX_ERR_HIP : FX_ERR_INVALID;
     }
     *out = c;
     return FX_OK;

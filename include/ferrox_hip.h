@@ -17,7 +17,7 @@
  *   - Memory handed out by the pool is NOT zeroed on reuse (as in the reference, context.rs:72-73); every
  *     kernel here fully defines its output.
  *   - A context may be used from several host threads; allocator calls are serialised internally and launches
- *     are serialised per context.
+ *     are serialised per context.  Every entry point makes the context's device current on the calling thread.
  *   - dtype suffixes: _f32 = float, _f64 = double.  The reference names its kernels `op` / `op_f64`
  *     (src/backend/cuda/kernels.rs:283-292).
  */
@@ -109,6 +109,7 @@ int fx_timer_stop(fx_ctx* ctx, float* elapsed_ms);
 /* n_elems == 0 -> FX_ERR_INVALID "Cannot allocate zero-sized CUDA memory" (cuda.rs:57-59).
  * *granted_elems may exceed n_elems on a pool hit (the reference truncates on read-back, context.rs:410-426). */
 int fx_alloc(fx_ctx* ctx, int dtype, int64_t n_elems, void** ptr, int64_t* granted_elems, uint64_t* alloc_id);
+/* A pointer the pool does not own, or one that was already released, is an error (FX_ERR_INVALID). */
 int fx_free(fx_ctx* ctx, int dtype, void* ptr, uint64_t alloc_id);
 int fx_pool_cleanup(fx_ctx* ctx, int dtype);
 int fx_pool_reset(fx_ctx* ctx, int dtype);

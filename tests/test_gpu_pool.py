@@ -88,6 +88,16 @@ def test_zero_size_and_unroutable_size_are_errors():
             gp.alloc(101)
         with pytest.raises(capi.FerroxHipError, match="not owned by this pool"):
             gp.free(12345, 1)
+        with pytest.raises(capi.FerroxHipError, match="exceed the address space"):
+            gp.alloc(1 << 62)
+        # a second release of the same block is refused instead of freeing memory that sits in the pool
+        ptr, _, aid = gp.alloc(7)
+        gp.free(ptr, aid)
+        with pytest.raises(capi.FerroxHipError, match="already released"):
+            gp.free(ptr, aid)
+        again, _, aid2 = gp.alloc(7)
+        assert again == ptr   # the block is still pooled and usable
+        gp.free(again, aid2)
     finally:
         gp.close()
 
