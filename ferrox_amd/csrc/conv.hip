@@ -14,6 +14,7 @@
 
 #include "igemm_core.hpp"
 #include "wgrad_patch.hpp"
+#include "conv_smallc.hpp"
 #include "conv_patch.hpp"
 
 namespace fx {
@@ -118,6 +119,15 @@ int fwd_tile(fx_ctx* c, const T* x, const T* w, T* y, const Dims& d, const T* bi
     return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
 }
 
+// Image layers (at most 4 input channels forward, 3 for the weight gradient), f32 3x3.
+template <typename T>
+csc::Plan smallc_plan(fx_ctx* c, const Dims& d, bool wgrad) {
+    if constexpr (sizeof(T) == 4) {
+        if (!generic_only()) return csc::make_plan(c ? c->num_cus : 256, wgrad, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
+    }
+    return csc::Plan();
+}
+
 template <typename T>
 cpk::Plan fwd_patch_plan(fx_ctx* c, const Dims& d) {
     if constexpr (sizeof(T) == 4) {
@@ -156,6 +166,8 @@ int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64
                (long long)ws_bytes, (long long)need);
     std::lock_guard<std::mutex> lk(c->launch_mutex);
     if constexpr (sizeof(T) == 4) {
+        const csc::Plan sp = smallc_plan<T>(c, d, false);
+        if (sp.ok && aligned16(x, x)) return csc::run_fwd(c, sp, x, w, y, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw, bias, relu);
         const cpk::Plan pl = fwd_patch_plan<T>(c, d);
         if (pl.ok && aligned16(x, ws)) {
             float* wimg = (float*)(ws ? ws : c->get_scratch(need));
@@ -465,7 +477,11 @@ i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64) wgrad_plan<T, TileM128>(c, d, &splits, &kps);
     else if (d.Cout <= 32 && d.Cin * d.kh * d.kw <= 32) wgrad_plan<T, TileTiny>(c, d, &splits, &kps);
     else wgrad_plan<T, TileSmall>(c, d, &splits, &kps);
-    const i64 generic = splits > 1 ? (i64)splits * d.Cout * d.Cin * d.kh * d.kw * (i64)sizeof(T) : 0;
+    i64 generic = splits > 1 ? (i64)splits * d.Cout * d.Cin * d.kh * d.kw * (i64)sizeof(T) : 0;
+    if (mode == 0) {
+        const csc::Plan sp = smallc_plan<T>(c, d, true);
+        if (sp.ok) generic = std::max(generic, csc::wgrad_workspace_bytes(sp, d.Cout, d.Cin));
+    }
     return pl.ok ? std::max(generic, wgp::workspace_bytes(pl, d.Cout, d.Cin)) : generic;
 }
 
@@ -482,6 +498,15 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
                (long long)ws_bytes, (long long)need);
     std::lock_guard<std::mutex> lk(c->launch_mutex);
     if constexpr (sizeof(T) == 4) {
+        const csc::Plan sp = mode == 0 ? smallc_plan<T>(c, d, true) : csc::Plan();
+        if (sp.ok && aligned16(x, g)) {
+            float* part = nullptr;
+            if (sp.splits > 1) {
+                part = (float*)(ws ? ws : c->get_scratch(need));
+                if (!part) return FX_ERR_OOM;
+            }
+            return csc::run_wgrad(c, sp, x, g, dw, part, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw);
+        }
         const wgp::Plan pl = patch_plan<T>(c, d, mode);
         if (pl.ok && aligned16(x, g) && aligned16(ws, ws)) {
             float* part = (float*)(ws ? ws : c->get_scratch(need));

@@ -1,0 +1,278 @@
+// 3x3 convolution over very few input channels (f32; an image layer: 1 to 4 channels forward, 1 to 3 for the weight
+// gradient), the first layer of every network of the reference's examples (examples/common/models.rs:200-318; the
+// product itself is conv2d_impl / cross_correlation2d_impl, src/backend/storage/extensions/convolutions.rs:218-338).
+//
+// With K = Cin*9 <= 36 the general kernels spend their time gathering a K x pixels operand whose rows are mostly
+// padding of the 16-deep slabs.  Here a block copies the input rows under 256 consecutive output pixels of one image
+// into LDS once, zero padded ([c][row][col]); the MFMA operand of lane l for reduction index k is then one LDS read at
+// (pixel offset) + (tap offset of k), both cheap to form:
+//   forward   y[oc][pixel] = sum_k w[oc][k] * patch(pixel, k)          A = w (registers, read in its natural [oc][c*9+t]
+//             order, no re-layout pass), B = patch; one 32(oc) x 32(pixel) accumulator per 32 pixels, K/2 MFMAs each.
+//   wgrad     dw[oc][k] = sum_pixel g[oc][pixel] * patch(pixel, k)     A = g staged as Gs[oc][pixel] (odd pitch),
+//             B = patch with n = k; each wave reduces a quarter of the tile's pixels into one 32 x 32 accumulator, the
+//             four are added through LDS at the end, blocks over disjoint pixel ranges leave partial sums that
+//             the split-K reduction adds in order.
+// Both are bound by the activation tensor they write / read (33.5 MB at [256,32,32,32]), not by the MFMA pipe.
+#pragma once
+#include "igemm_core.hpp"
+
+namespace csc {
+using igemm::FastDiv;
+using igemm::f32x16;
+
+constexpr int NT = 256, NPIX = 256, KK = 9;
+constexpr int GP = NPIX + 1;                 // pitch of Gs: odd, so 32 output channels land on 32 banks
+constexpr size_t LDS_LIMIT = 60 * 1024;
+
+struct Geometry {
+    int C, H, W, Cout, OH, OW, sh, sw, ph, pw;
+    int PR, PW, PLANE;   // patch rows, padded row width, floats per channel plane
+    int tpi;             // tiles of NPIX pixels per image
+    FastDiv div_tpi, div_ow, div_w4, div_pr;
+};
+
+struct FwdParams {
+    const float* x;
+    const float* w;
+    float* y;
+    const float* bias;
+    int relu;
+    Geometry g;
+};
+
+struct WgradParams {
+    const float* x;
+    const float* g;
+    float* part;
+    int stages, sps;     // B * tpi, stages per block
+    i64 part_stride;     // Cout * C * 9
+    Geometry q;
+};
+
+// Copies the rows under tile `tile` of image b into the patch (rows outside the image become zero; the padding
+// columns are zeroed by the caller once and never written).
+__device__ __forceinline__ void stage_patch(const Geometry& g, const float* __restrict__ x, float* patch, int b, int iy0, int tid) {
+    const int W4 = g.W >> 2, items = g.C * g.PR * W4;
+    for (int i = tid; i < items; i += NT) {
+        const int rc = (int)g.div_w4.div((uint32_t)i), q = i - rc * W4;
+        const int c = (int)g.div_pr.div((uint32_t)rc), r = rc - c * g.PR;
+        const int iy = iy0 + r;
+        const bool ok = iy >= 0 && iy < g.H;
+        const float4 v = *reinterpret_cast<const float4*>(x + (((i64)b * g.C + c) * g.H + (ok ? iy : 0)) * g.W + 4 * q);
+        float* d = patch + c * g.PLANE + r * g.PW + g.pw + 4 * q;
+        d[0] = ok ? v.x : 0.f; d[1] = ok ? v.y : 0.f; d[2] = ok ? v.z : 0.f; d[3] = ok ? v.w : 0.f;
+    }
+}
+
+// tap offset of reduction index k = c*9 + ky*3 + kx inside the patch (0 for the padding indices k >= K)
+__device__ __forceinline__ int tap_offset(const Geometry& g, int k) {
+    if (k >= g.C * KK) return 0;
+    const int c = k / KK, t = k - c * KK, ky = t / 3, kx = t - ky * 3;
+    return c * g.PLANE + ky * g.PW + kx;
+}
+
+// KS = ceil(Cin * 9 / 2) MFMA steps.  grid = (B * tiles per image, ceil(Cout / 32)).
+template <int KS, bool BIAS>
+__global__ __launch_bounds__(NT) void fwd_kernel(const FwdParams p) {
+    extern __shared__ __align__(16) float patch[];
+    const Geometry& g = p.g;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
+    const int b = (int)g.div_tpi.div(blockIdx.x), tile = (int)blockIdx.x - b * g.tpi;
+    const int m0 = blockIdx.y * 32;
+    const int L = g.OH * g.OW, K = g.C * KK;
+    const int pix0 = tile * NPIX, py0 = (int)g.div_ow.div((uint32_t)pix0), iy0 = py0 * g.sh - g.ph;
+
+    // the weight loads are in flight while the patch is staged; they are first used after the second barrier
+    float wraw[KS];
+    int koff[KS];
+    const bool m_ok = m0 + l32 < g.Cout;
+    const float* wrow = p.w + (i64)(m_ok ? m0 + l32 : 0) * K;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        const int k = 2 * s + half;
+        wraw[s] = wrow[k < K ? k : 0];
+        koff[s] = tap_offset(g, k);
+    }
+    for (int i = tid; i < g.C * g.PLANE; i += NT) patch[i] = 0.f;
+    __syncthreads();
+    stage_patch(g, p.x, patch, b, iy0, tid);
+    __syncthreads();
+    float wreg[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) wreg[s] = m_ok && 2 * s + half < K ? wraw[s] : 0.f;
+
+    float* yb = p.y + (i64)b * g.Cout * L;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+        const int pbase = pix0 + (wave * 2 + blk) * 32;
+        if (pbase >= L) break;  // wave-uniform
+        const int pp = pbase + l32, pc = min(pp, L - 1);
+        const int oy = (int)g.div_ow.div((uint32_t)pc), ox = pc - oy * g.OW;
+        const float* src = patch + (oy - py0) * g.sh * g.PW + ox * g.sw;
+        f32x16 acc;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wreg[s], src[koff[s]], acc, 0, 0, 0);
+        if (pp < L) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int ch = m0 + igemm::Mfma<float>::row(e, lane);
+                if (ch < g.Cout) {
+                    float v = acc[e];
+                    if constexpr (BIAS) {
+                        v += p.bias[ch];
+                        if (p.relu) v = v > 0.f ? v : 0.f;
+                    }
+                    yb[(i64)ch * L + pp] = v;
+                }
+            }
+        }
+    }
+}
+
+// grid = (splits, ceil(Cout / 32)); block z takes stages [z * sps, (z + 1) * sps), a stage being one tile of one image.
+// Needs C * 9 <= 32 and (OH * OW) % 4 == 0.
+__global__ __launch_bounds__(NT, 2) void wgrad_kernel(const WgradParams p) {
+    extern __shared__ __align__(16) float smem[];
+    const Geometry& g = p.q;
+    float* Gs = smem;                 // [32][GP]
+    float* patch = smem + 32 * GP;    // [C][PR][PW]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
+    const int m0 = blockIdx.y * 32, z = blockIdx.x;
+    const int L = g.OH * g.OW, K = g.C * KK;
+    const int toff = tap_offset(g, l32);
+    f32x16 acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+    for (int i = tid; i < g.C * g.PLANE; i += NT) patch[i] = 0.f;
+
+    const int s_end = min(p.stages, (z + 1) * p.sps);
+    const int gq = tid & 63, gr = tid >> 6;  // float4 column and first row of this thread in Gs
+    for (int s = z * p.sps; s < s_end; ++s) {
+        const int b = (int)g.div_tpi.div((uint32_t)s), tile = s - b * g.tpi;
+        const int pix0 = tile * NPIX, py0 = (int)g.div_ow.div((uint32_t)pix0), iy0 = py0 * g.sh - g.ph;
+        __syncthreads();  // the previous stage's reads are done (and the zero fill before the first)
+        const bool col_ok = pix0 + 4 * gq < L;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int row = gr + 4 * u;
+            const bool ok = col_ok && m0 + row < g.Cout;
+            const float4 v = *reinterpret_cast<const float4*>(p.g + ((i64)b * g.Cout + (ok ? m0 + row : 0)) * L + (ok ? pix0 + 4 * gq : 0));
+            float* d = Gs + row * GP + 4 * gq;
+            d[0] = ok ? v.x : 0.f; d[1] = ok ? v.y : 0.f; d[2] = ok ? v.z : 0.f; d[3] = ok ? v.w : 0.f;
+        }
+        stage_patch(g, p.x, patch, b, iy0, tid);
+        __syncthreads();
+        const float* ga = Gs + l32 * GP + wave * 64 + half;
+        const int pw0 = pix0 + wave * 64 + half;
+#pragma unroll 4
+        for (int st = 0; st < 32; ++st) {
+            const int pc = min(pw0 + 2 * st, L - 1);  // past the end g is zero; the patch read only has to be in range
+            const int oy = (int)g.div_ow.div((uint32_t)pc), ox = pc - oy * g.OW;
+            const float bv = patch[(oy - py0) * g.sh * g.PW + ox * g.sw + toff];
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ga[2 * st], bv, acc, 0, 0, 0);
+        }
+    }
+    // the four waves hold sums over different pixels: add them in wave order
+    __syncthreads();
+    float* red = smem;  // [4][16][64]
+#pragma unroll
+    for (int e = 0; e < 16; ++e) red[(wave * 16 + e) * 64 + lane] = acc[e];
+    __syncthreads();
+    float* out = p.part + (i64)z * p.part_stride;
+    for (int i = tid; i < 16 * 64; i += NT) {
+        const int e = i >> 6, ln = i & 63;
+        const float v = ((red[i] + red[1024 + i]) + red[2048 + i]) + red[3072 + i];
+        const int m = m0 + igemm::Mfma<float>::row(e, ln), n = ln & 31;
+        if (m < g.Cout && n < K) out[(i64)m * K + n] = v;
+    }
+}
+
+struct Plan {
+    bool ok = false;
+    int PR = 0, PW = 0, PLANE = 0, tpi = 0;
+    int splits = 1, sps = 1, stages = 0;  // weight gradient only
+    size_t smem = 0;
+};
+
+inline Plan make_plan(int num_cus, bool wgrad, i64 B, i64 C, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw,
+                      i64 OH, i64 OW) {
+    Plan pl;
+    const i64 L = OH * OW;
+    if (kh != 3 || kw != 3 || W % 4 != 0 || sh > 8 || sw > 8 || ph > 8 || pw > 8) return pl;
+    if (wgrad ? (C * KK > 32 || L % 4 != 0) : C > 4) return pl;
+    const i64 rows = std::min<i64>(OH, NPIX % OW == 0 ? NPIX / OW : (NPIX - 1) / OW + 2);
+    pl.PR = (int)((rows - 1) * sh + 3);
+    // wide images: a tile of 256 pixels covers about one output row and would stage five or seven input rows (measured
+    // at 3 x 224 x 224 -> 64: 0.300 ms here against 0.245 ms for the implicit GEMM, 0.074 against 0.059 ms at stride 2)
+    if (OW > 64 || (i64)pl.PR * OW > 2 * (i64)NPIX * sh) return pl;
+    pl.PW = (int)(W + 2 * pw);
+    pl.PLANE = pl.PR * pl.PW;
+    pl.tpi = (int)fx::ceil_div(L, (i64)NPIX);
+    pl.smem = ((size_t)C * pl.PLANE + (wgrad ? (size_t)32 * GP : 0)) * sizeof(float);
+    if (pl.smem > LDS_LIMIT || B * pl.tpi > 0x7fffffff) return pl;
+    if (wgrad) {
+        pl.stages = (int)(B * pl.tpi);
+        const i64 mblocks = fx::ceil_div(Cout, (i64)32);
+        const i64 splits = std::max<i64>(1, std::min<i64>(pl.stages, 4 * (i64)num_cus / mblocks));
+        pl.sps = (int)fx::ceil_div((i64)pl.stages, splits);
+        pl.splits = (int)fx::ceil_div((i64)pl.stages, (i64)pl.sps);
+        if (mblocks > 65535) return pl;
+    } else if (fx::ceil_div(Cout, (i64)32) > 65535) {
+        return pl;
+    }
+    pl.ok = true;
+    return pl;
+}
+
+inline i64 wgrad_workspace_bytes(const Plan& pl, i64 Cout, i64 C) { return pl.splits > 1 ? (i64)pl.splits * Cout * C * KK * (i64)sizeof(float) : 0; }
+
+inline Geometry make_geometry(const Plan& pl, i64 C, i64 H, i64 W, i64 Cout, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw) {
+    Geometry g;
+    g.C = (int)C; g.H = (int)H; g.W = (int)W; g.Cout = (int)Cout; g.OH = (int)OH; g.OW = (int)OW;
+    g.sh = (int)sh; g.sw = (int)sw; g.ph = (int)ph; g.pw = (int)pw;
+    g.PR = pl.PR; g.PW = pl.PW; g.PLANE = pl.PLANE; g.tpi = pl.tpi;
+    g.div_tpi = FastDiv((uint32_t)pl.tpi); g.div_ow = FastDiv((uint32_t)OW);
+    g.div_w4 = FastDiv((uint32_t)(W / 4)); g.div_pr = FastDiv((uint32_t)pl.PR);
+    return g;
+}
+
+// x and y's base addresses must be 16-byte aligned (x for the vector loads).
+inline int run_fwd(fx_ctx* c, const Plan& pl, const float* x, const float* w, float* y, i64 B, i64 C, i64 H, i64 W, i64 Cout, i64 OH,
+                   i64 OW, i64 sh, i64 sw, i64 ph, i64 pw, const float* bias, int relu) {
+    FwdParams p;
+    p.x = x; p.w = w; p.y = y; p.bias = bias; p.relu = relu;
+    p.g = make_geometry(pl, C, H, W, Cout, OH, OW, sh, sw, ph, pw);
+    const dim3 grid((unsigned)(B * pl.tpi), (unsigned)fx::ceil_div(Cout, (i64)32));
+#define FX_CSC_FWD(KSV)                                                                                 \
+    do {                                                                                                \
+        if (bias) fwd_kernel<KSV, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                     \
+        else fwd_kernel<KSV, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                         \
+    } while (0)
+    switch ((int)C) {
+        case 1: FX_CSC_FWD(5); break;
+        case 2: FX_CSC_FWD(9); break;
+        case 3: FX_CSC_FWD(14); break;
+        default: FX_CSC_FWD(18); break;
+    }
+#undef FX_CSC_FWD
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+// x, g and part 16-byte aligned.  part holds splits x [Cout][C*9] partial sums (unused when splits == 1).
+inline int run_wgrad(fx_ctx* c, const Plan& pl, const float* x, const float* g, float* dw, float* part, i64 C, i64 H, i64 W, i64 Cout,
+                     i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw) {
+    WgradParams p;
+    p.x = x; p.g = g; p.part = pl.splits > 1 ? part : dw;
+    p.stages = pl.stages; p.sps = pl.sps; p.part_stride = Cout * C * KK;
+    p.q = make_geometry(pl, C, H, W, Cout, OH, OW, sh, sw, ph, pw);
+    const dim3 grid((unsigned)pl.splits, (unsigned)fx::ceil_div(Cout, (i64)32));
+    wgrad_kernel<<<grid, dim3(NT), pl.smem, c->stream>>>(p);
+    FX_LAUNCH_CHECK();
+    if (pl.splits > 1) return igemm::launch_splitk_reduce<float>(c, part, dw, p.part_stride, pl.splits);
+    return FX_OK;
+}
+
+}  // namespace csc

@@ -530,6 +530,59 @@ def test_conv2d_patch_kernel_shapes(ctx, orc):
             assert np.array_equal(out.numpy(), ref), (kind, case)
 
 
+# Image layers (at most 4 input channels forward, 3 for the weight gradient; W % 4 == 0): the LDS-patch kernels for
+# few channels.  Ragged Cout, tiles that end inside a row, strides, wide rows, padding 0 and 2, one-channel MNIST shape.
+SMALLC_CASES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw)
+    (4, 3, 32, 32, 32, (1, 1), (1, 1)), (5, 1, 28, 28, 8, (1, 1), (1, 1)), (3, 3, 10, 12, 40, (1, 1), (0, 0)),
+    (2, 2, 17, 20, 33, (2, 2), (1, 1)), (2, 3, 7, 8, 5, (3, 1), (1, 1)), (1, 3, 40, 36, 64, (1, 1), (1, 1)),
+    (1, 3, 66, 64, 16, (2, 2), (1, 1)), (2, 1, 5, 4, 70, (1, 1), (2, 2)), (1, 3, 19, 60, 8, (1, 1), (1, 1)),
+    (1, 3, 20, 224, 16, (2, 2), (1, 1)), (1, 4, 10, 64, 16, (1, 2), (2, 0)), (3, 3, 9, 12, 40, (1, 1), (0, 0)), (37, 3, 16, 16, 32, (1, 1), (1, 1)),
+]
+
+
+def test_conv2d_image_layer_kernels(ctx, orc):
+    import torch
+    import torch.nn.functional as F
+    from ferrox_amd import capi
+    rng = np.random.default_rng(59)
+    tol = TOL[np.dtype(np.float32)]
+    for (B, Cin, H, W, Cout, st, pd) in SMALLC_CASES:
+        case = (B, Cin, H, W, Cout, st, pd)
+        x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(np.float32)
+        w = (rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9))).astype(np.float32)
+        bias = rng.standard_normal(Cout).astype(np.float32)
+        oh, ow = orc.out_hw(H, W, 3, 3, st[0], st[1], pd[0], pd[1])
+        g = rng.standard_normal((B, Cout, oh, ow)).astype(np.float32)
+        dx_, dw_, dg_, db_ = ctx.upload(x), ctx.upload(w), ctx.upload(g), ctx.upload(bias)
+        y = ctx.conv2d_fwd(dx_, dw_, st, pd).numpy()
+        gw = ctx.conv2d_wgrad(dx_, dg_, w.shape, st, pd, 0).numpy()
+        tx = torch.from_numpy(x).double()
+        tw = torch.from_numpy(w).double().requires_grad_(True)
+        ty = F.conv2d(tx, tw, stride=st, padding=pd)
+        ty.backward(torch.from_numpy(g).double())
+        ay = F.conv2d(tx.abs(), tw.detach().abs(), stride=st, padding=pd).max().item()
+        assert np.abs(y - ty.detach().numpy()).max() <= tol * ay, ("fwd", case)
+        assert rel_err(gw, tw.grad.numpy()) <= tol * 8, ("wgrad", case)
+        assert rel_err(y, orc.conv2d_fwd(x, w, st, pd)) <= tol * 8, ("fwd vs oracle", case)
+        assert rel_err(gw, orc.conv2d_wgrad(x, g, w.shape, st, pd, 0)) <= tol * 8, ("wgrad vs oracle", case)
+        # same bits on a second run; bias + ReLU in the store equals the separate pass
+        assert np.array_equal(ctx.conv2d_fwd(dx_, dw_, st, pd).numpy(), y), case
+        assert np.array_equal(ctx.conv2d_wgrad(dx_, dg_, w.shape, st, pd, 0).numpy(), gw), case
+        dims = (B, Cin, H, W, Cout, 3, 3, st[0], st[1], pd[0], pd[1])
+        fused = ctx.empty(y.shape, np.float32)
+        capi.check(capi.lib.fx_conv2d_fwd_bias_act_f32(ctx.h, dx_.ptr, dw_.ptr, db_.ptr, fused.ptr, *dims, 1, None, 0))
+        two = ctx.conv2d_fwd(dx_, dw_, st, pd)
+        ctx.bias_act(two, db_, B, Cout, oh * ow, act=1)
+        assert np.array_equal(fused.numpy(), two.numpy()), ("bias+relu", case)
+        # a caller-provided workspace of exactly the advertised size
+        need = capi.lib.fx_conv2d_workspace_bytes(capi.CONV_WGRAD, capi.FX_F32, 0, *dims)
+        assert need >= 0
+        ws = ctx.empty((max(need, 4) // 4,), np.float32)
+        out = ctx.empty(w.shape, np.float32)
+        capi.check(capi.lib.fx_conv2d_wgrad_f32(ctx.h, dx_.ptr, dg_.ptr, out.ptr, *dims, 0, ws.ptr, need))
+        assert np.array_equal(out.numpy(), gw), case
+
+
 # Strided data gradients, computed per pixel class (Cout % 16 == 0, kernel >= stride) and by the all-taps gather
 # otherwise: odd sizes, classes without pixels, kernel == stride, stride 3, 5x5, asymmetric stride and padding.
 # B, Cin, H, W, Cout, (kh, kw), (sh, sw), (ph, pw)

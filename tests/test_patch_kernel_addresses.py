@@ -119,6 +119,115 @@ def fwd_loads_in_bounds(B, C, H, W, M, sh, sw, ph, pw):
     return "patch %dx%d ok" % (pl["WM"], pl["TN"])
 
 
+# ---- conv_smallc.hpp: image layers (few input channels), forward and weight gradient ------------------------------------
+SC_NPIX, SC_GP = 256, 257
+def smallc_plan(wgrad, B, C, H, W, Cout, sh, sw, ph, pw, OH, OW, num_cus=256):
+    L = OH * OW
+    if W % 4 or sh > 8 or sw > 8 or ph > 8 or pw > 8: return None
+    if (C * 9 > 32 or L % 4) if wgrad else C > 4: return None
+    rows = min(OH, SC_NPIX // OW if SC_NPIX % OW == 0 else (SC_NPIX - 1) // OW + 2)
+    PR, PW = (rows - 1) * sh + 3, W + 2 * pw
+    if OW > 64 or PR * OW > 2 * SC_NPIX * sh: return None
+    pl = dict(PR=PR, PW=PW, PLANE=PR * PW, tpi=_ceil_div(L, SC_NPIX))
+    if (C * pl["PLANE"] + (32 * SC_GP if wgrad else 0)) * 4 > 60 * 1024: return None
+    if wgrad:
+        stages, mblocks = B * pl["tpi"], _ceil_div(Cout, 32)
+        splits = max(1, min(stages, 4 * num_cus // mblocks))
+        pl["sps"] = _ceil_div(stages, splits); pl["splits"] = _ceil_div(stages, pl["sps"]); pl["stages"] = stages
+    return pl
+def smallc_tap(C, PLANE, PW, k):
+    if k >= C * 9: return 0
+    c, t = divmod(k, 9); ky, kx = divmod(t, 3)
+    return c * PLANE + ky * PW + kx
+def smallc_stage_in_bounds(pl, b, C, H, W, pw, iy0, xsize):
+    W4 = W // 4
+    for i in range(C * pl["PR"] * W4):
+        rc, q = divmod(i, W4); c, r = divmod(rc, pl["PR"])
+        iy = iy0 + r; ok = 0 <= iy < H
+        a = ((b * C + c) * H + (iy if ok else 0)) * W + 4 * q
+        assert 0 <= a and a + 4 <= xsize, ("x", a, xsize)
+        d = c * pl["PLANE"] + r * pl["PW"] + pw + 4 * q
+        assert 0 <= d and d + 4 <= C * pl["PLANE"], ("patch write", d)
+def smallc_loads_in_bounds(wgrad, B, C, H, W, Cout, st, pd):
+    sh, sw = st; ph, pw = pd
+    OH, OW = (H + 2 * ph - 3) // sh + 1, (W + 2 * pw - 3) // sw + 1
+    pl = smallc_plan(wgrad, B, C, H, W, Cout, sh, sw, ph, pw, OH, OW)
+    if pl is None: return "generic"
+    L, K = OH * OW, C * 9
+    xsize, ysize, wsize = B * C * H * W, B * Cout * L, Cout * K
+    KS = {1: 5, 2: 9, 3: 14, 4: 18}[C]
+    plane_all = C * pl["PLANE"]
+    for b in range(B):
+        for tile in range(pl["tpi"]):
+            pix0 = tile * SC_NPIX; py0 = pix0 // OW; iy0 = py0 * sh - ph
+            smallc_stage_in_bounds(pl, b, C, H, W, pw, iy0, xsize)
+            for m0 in range(0, Cout, 32):
+                if not wgrad:
+                    for l32 in range(32):
+                        m_ok = m0 + l32 < Cout
+                        for k in range(2 * KS):
+                            a = (m0 + l32 if m_ok else 0) * K + (k if k < K else 0)
+                            assert 0 <= a < wsize, ("w", a)
+                    for pb in range(8):
+                        pbase = pix0 + pb * 32
+                        if pbase >= L: break
+                        for l32 in range(32):
+                            pp = pbase + l32; pc = min(pp, L - 1); oy, ox = divmod(pc, OW)
+                            assert (oy - py0) * sh + 2 < pl["PR"], "patch rows"
+                            base = (oy - py0) * sh * pl["PW"] + ox * sw
+                            for k in range(2 * KS):
+                                idx = base + smallc_tap(C, pl["PLANE"], pl["PW"], k)
+                                assert 0 <= idx < plane_all, ("patch read", idx)
+                            if pp < L:
+                                for ch in range(m0, min(m0 + 32, Cout)):
+                                    a = (b * Cout + ch) * L + pp
+                                    assert 0 <= a < ysize
+                else:
+                    for tid in range(256):
+                        gq, gr = tid & 63, tid >> 6
+                        col_ok = pix0 + 4 * gq < L
+                        for u in range(8):
+                            row = gr + 4 * u; ok = col_ok and m0 + row < Cout
+                            a = (b * Cout + (m0 + row if ok else 0)) * L + (pix0 + 4 * gq if ok else 0)
+                            assert 0 <= a and a + 4 <= ysize, ("g", a, ysize)
+                            assert row * SC_GP + 4 * gq + 4 <= 32 * SC_GP
+                    for wave in range(4):
+                        for half in range(2):
+                            for stp in range(32):
+                                pl_ = wave * 64 + half + 2 * stp
+                                assert pl_ < SC_NPIX
+                                pc = min(pix0 + pl_, L - 1); oy, ox = divmod(pc, OW)
+                                assert (oy - py0) * sh + 2 < pl["PR"], "patch rows"
+                                base = (oy - py0) * sh * pl["PW"] + ox * sw
+                                for n in range(32):
+                                    idx = base + smallc_tap(C, pl["PLANE"], pl["PW"], n)
+                                    assert 0 <= idx < plane_all, ("patch read", idx)
+    if wgrad:
+        assert pl["splits"] * pl["sps"] >= pl["stages"] and (pl["splits"] - 1) * pl["sps"] < pl["stages"]
+    return "smallc"
+
+
+SMALLC_SHAPES = [  # B, C, H, W, Cout, (sh, sw), (ph, pw)
+    (2, 3, 32, 32, 32, (1, 1), (1, 1)), (2, 1, 28, 28, 8, (1, 1), (1, 1)), (3, 3, 9, 12, 40, (1, 1), (0, 0)),
+    (2, 2, 17, 20, 33, (2, 2), (1, 1)), (2, 3, 7, 8, 5, (3, 1), (1, 1)), (1, 3, 40, 36, 64, (1, 1), (1, 1)),
+    (1, 3, 66, 64, 16, (2, 2), (1, 1)), (2, 1, 5, 4, 70, (1, 1), (2, 2)), (1, 3, 19, 60, 8, (1, 1), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", SMALLC_SHAPES, ids=str)
+def test_image_layer_kernels_stay_inside_their_tensors_and_the_patch(case):
+    B, C, H, W, Cout, (sh, sw), (ph, pw) = case
+    L = ((H + 2 * ph - 3) // sh + 1) * ((W + 2 * pw - 3) // sw + 1)
+    assert smallc_loads_in_bounds(False, *case) == "smallc"
+    assert smallc_loads_in_bounds(True, *case) == ("smallc" if L % 4 == 0 else "generic")  # whole float4 groups of grad_out
+
+
+def test_image_layer_forward_takes_four_channels_and_the_weight_gradient_does_not():
+    case = (1, 4, 10, 64, 16, (1, 2), (2, 0))
+    assert smallc_loads_in_bounds(False, *case) == "smallc"
+    assert smallc_loads_in_bounds(True, *case) == "generic"
+
+
 WGRAD_SHAPES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw): every wave layout, ragged output-channel counts
     (2, 32, 10, 56, 100, (1, 1), (1, 1)), (3, 64, 28, 28, 96, (1, 1), (1, 1)), (2, 32, 16, 16, 128, (1, 1), (1, 1)),
     (2, 32, 9, 64, 128, (1, 1), (0, 1)), (2, 64, 12, 56, 64, (1, 1), (1, 1)), (3, 64, 10, 32, 64, (1, 1), (1, 1)),
