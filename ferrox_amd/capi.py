@@ -187,6 +187,14 @@ class DeviceArray:
         v._base = self
         return v
 
+    def rows(self, lo, hi):
+        """Non-owning view of the slices lo:hi along the first axis."""
+        assert 0 <= lo <= hi <= self.shape[0]
+        inner = int(np.prod(self.shape[1:], dtype=np.int64))
+        v = DeviceArray(self.ctx, (hi - lo,) + self.shape[1:], self.dtype, self.ptr + lo * inner * self.dtype.itemsize, 0, None)
+        v._base = self
+        return v
+
     def numpy(self):
         out = np.empty(self.shape, dtype=self.dtype)
         if self.size:

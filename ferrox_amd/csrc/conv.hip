@@ -44,6 +44,7 @@ inline bool aligned16(const void* a, const void* b) { return (((uintptr_t)a | (u
 
 struct Dims {
     i64 B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, oh, ow;
+    i64 bc;  // images per launch: the kernels index one launch's tensors with 32-bit byte offsets and pixel numbers
 };
 
 template <typename T>
@@ -52,15 +53,17 @@ int check_dims(Dims& d, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, 
                "%s: non-positive dimension", what);
     FX_REQUIRE(H + 2 * ph >= kh && W + 2 * pw >= kw, "%s: kernel larger than padded input", what);
     FX_REQUIRE(ph < 32768 && pw < 32768 && kh < 32768 && kw < 32768, "%s: kernel/padding too large", what);
-    d = Dims{B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, (H + 2 * ph - kh) / sh + 1, (W + 2 * pw - kw) / sw + 1};
+    d = Dims{B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, (H + 2 * ph - kh) / sh + 1, (W + 2 * pw - kw) / sw + 1, 0};
     const i64 lim = (1ll << 31) - 1;
-    FX_REQUIRE(B * d.oh * d.ow <= lim && B * H * W <= lim && Cin * H * W <= lim && Cout * d.oh * d.ow <= lim &&
-                   Cin * kh * kw <= lim && Cout * kh * kw <= lim,
-               "%s: a GEMM dimension or per-image plane exceeds 2^31-1", what);
-    if (B * Cin * H * W * (i64)sizeof(T) > lim || B * Cout * d.oh * d.ow * (i64)sizeof(T) > lim) {
-        fx::set_error("%s: tensors of 2 GiB or more are not supported by this build", what);
+    FX_REQUIRE(Cin * kh * kw <= lim && Cout * kh * kw <= lim, "%s: a GEMM dimension exceeds 2^31-1", what);
+    // A batch whose tensors reach 2 GiB runs as several launches over slices of the batch (images are independent in
+    // the forward pass and the data gradient; the weight gradient adds the slices' results in order).
+    const i64 per_image = std::max(Cin * H * W, Cout * d.oh * d.ow) * (i64)sizeof(T);
+    if (per_image > lim) {
+        fx::set_error("%s: one image of 2 GiB or more is not supported by this build", what);
         return FX_ERR_UNSUPPORTED;
     }
+    d.bc = std::min(B, lim / per_image);
     return FX_OK;
 }
 
@@ -161,6 +164,15 @@ int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64
     FX_REQUIRE(x && w && y, "fx_conv2d_fwd: null pointer");
     Dims d;
     if (int rc = check_dims<T>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_fwd")) return rc;
+    if (d.B > d.bc) {  // slices of the batch, one launch sequence each
+        for (i64 b0 = 0; b0 < B; b0 += d.bc) {
+            const i64 nb = std::min(d.bc, B - b0);
+            if (int rc = conv_fwd<T>(c, x + b0 * Cin * H * W, w, y + b0 * Cout * d.oh * d.ow, nb, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw,
+                                     ws, ws_bytes, bias, relu))
+                return rc;
+        }
+        return FX_OK;
+    }
     const i64 need = fwd_ws_bytes<T>(c, d);
     FX_REQUIRE(ws == nullptr || ws_bytes >= need, "fx_conv2d_fwd: workspace of %lld bytes is smaller than the %lld needed",
                (long long)ws_bytes, (long long)need);
@@ -382,6 +394,19 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
     FX_REQUIRE(mode == 0 || mode == 1, "fx_conv2d_dgrad: mode must be 0 or 1");
     Dims d;
     if (int rc = check_dims<T>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_dgrad")) return rc;
+    if (d.B > d.bc) {
+        if (mode != 0) {  // the CPU-literal arithmetic reads grad_out flat across the whole batch
+            fx::set_error("fx_conv2d_dgrad: mode 1 does not support tensors of 2 GiB or more");
+            return FX_ERR_UNSUPPORTED;
+        }
+        for (i64 b0 = 0; b0 < B; b0 += d.bc) {
+            const i64 nb = std::min(d.bc, B - b0);
+            if (int rc = conv_dgrad<T>(c, g + b0 * Cout * d.oh * d.ow, w, dx + b0 * Cin * H * W, nb, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw,
+                                       mode, ws, ws_bytes))
+                return rc;
+        }
+        return FX_OK;
+    }
     const i64 need = dgrad_ws_bytes<T>(c, d, mode);
     FX_REQUIRE(ws == nullptr || ws_bytes >= need, "fx_conv2d_dgrad: workspace of %lld bytes is smaller than the %lld needed",
                (long long)ws_bytes, (long long)need);
@@ -493,6 +518,30 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
     FX_REQUIRE(mode == 0 || mode == 1, "fx_conv2d_wgrad: mode must be 0 or 1");
     Dims d;
     if (int rc = check_dims<T>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_wgrad")) return rc;
+    if (d.B > d.bc) {
+        if (mode != 0) {
+            fx::set_error("fx_conv2d_wgrad: mode 1 does not support tensors of 2 GiB or more");
+            return FX_ERR_UNSUPPORTED;
+        }
+        // one weight gradient per slice of the batch, then their sum in slice order (a rare, large case: the buffer for
+        // the slices' results is allocated and released here)
+        const i64 nchunks = fx::ceil_div(B, d.bc), nw = Cout * Cin * kh * kw;
+        T* tmp = nullptr;
+        FX_HIP_CHECK(hipMalloc((void**)&tmp, (size_t)(nchunks * nw) * sizeof(T)));
+        int rc = FX_OK;
+        for (i64 i = 0; i < nchunks && !rc; ++i) {
+            const i64 b0 = i * d.bc, nb = std::min(d.bc, B - b0);
+            rc = conv_wgrad<T>(c, x + b0 * Cin * H * W, g + b0 * Cout * d.oh * d.ow, tmp + i * nw, nb, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw,
+                               mode, ws, ws_bytes);
+        }
+        if (!rc) {
+            std::lock_guard<std::mutex> lk(c->launch_mutex);
+            rc = launch_splitk_reduce<T>(c, tmp, dw, nw, (int)nchunks);
+        }
+        (void)hipStreamSynchronize(c->stream);
+        (void)hipFree(tmp);
+        return rc;
+    }
     const i64 need = wgrad_ws_bytes<T>(c, d, mode);
     FX_REQUIRE(ws == nullptr || ws_bytes >= need, "fx_conv2d_wgrad: workspace of %lld bytes is smaller than the %lld needed",
                (long long)ws_bytes, (long long)need);
@@ -527,11 +576,25 @@ extern "C" int64_t fx_conv2d_workspace_bytes(int kind, int dtype, int mode, int6
     if (dtype == FX_F64 ? check_dims<double>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_workspace_bytes")
                         : check_dims<float>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_workspace_bytes"))
         return -1;
-    if (kind == FX_CONV_FWD) return dtype == FX_F64 ? fwd_ws_bytes<double>(nullptr, d) : fwd_ws_bytes<float>(nullptr, d);
-    if (kind == FX_CONV_DGRAD) return dtype == FX_F64 ? dgrad_ws_bytes<double>(nullptr, d, mode) : dgrad_ws_bytes<float>(nullptr, d, mode);
-    if (kind == FX_CONV_WGRAD) return dtype == FX_F64 ? wgrad_ws_bytes<double>(nullptr, d, mode) : wgrad_ws_bytes<float>(nullptr, d, mode);
-    fx::set_error("fx_conv2d_workspace_bytes: unknown kind %d", kind);
-    return -1;
+    auto need_of = [&](const Dims& q) -> i64 {
+        if (kind == FX_CONV_FWD) return dtype == FX_F64 ? fwd_ws_bytes<double>(nullptr, q) : fwd_ws_bytes<float>(nullptr, q);
+        if (kind == FX_CONV_DGRAD) return dtype == FX_F64 ? dgrad_ws_bytes<double>(nullptr, q, mode) : dgrad_ws_bytes<float>(nullptr, q, mode);
+        return dtype == FX_F64 ? wgrad_ws_bytes<double>(nullptr, q, mode) : wgrad_ws_bytes<float>(nullptr, q, mode);
+    };
+    if (kind != FX_CONV_FWD && kind != FX_CONV_DGRAD && kind != FX_CONV_WGRAD) {
+        fx::set_error("fx_conv2d_workspace_bytes: unknown kind %d", kind);
+        return -1;
+    }
+    if (d.B <= d.bc) return need_of(d);
+    // a batch that runs as slices: the largest need of a full slice and of the remainder
+    Dims q = d;
+    q.B = d.bc;
+    i64 need = need_of(q);
+    if (d.B % d.bc) {
+        q.B = q.bc = d.B % d.bc;
+        need = std::max(need, need_of(q));
+    }
+    return need;
 }
 
 #define FX_DEFINE_CONV(T, S)                                                                                           \

@@ -127,3 +127,42 @@ def test_c4_elementwise_full_size(ctx):
         assert np.array_equal(sb[sl], orc.sigmoid_bwd(g[sl], s[sl], 0))
         assert np.array_equal(tb[sl], orc.tanh_bwd(g[sl], t[sl]))
         assert np.abs(s[sl] - orc.unary("sigmoid", x[sl])).max() <= 1.2e-7   # expf differs from libm by an ulp at most
+
+
+def test_convolution_over_tensors_beyond_2_gib(ctx):
+    """Tensors of 2 GiB or more run as slices of the batch: forward and data gradient are checked on the images either
+    side of the slice boundary, the weight gradient against the ordered sum of two halves that each fit one launch."""
+    import torch
+    import torch.nn.functional as F
+    B, Cin, H, W, Cout = 2300, 16, 128, 128, 16           # 2.41 GB per activation tensor; one launch takes 2047 images
+    st, pd = (1, 1), (1, 1)
+    per_image = Cin * H * W * 4
+    cut = (2 ** 31 - 1) // per_image
+    assert cut < B
+    dx = ctx.uniform((B, Cin, H, W), 11, -1.0, 1.0)
+    dw = ctx.normal((Cout, Cin, 3, 3), 12, 0.0, float(np.sqrt(2.0 / (Cin * 9))))
+    dg = ctx.normal((B, Cout, H, W), 13, 0.0, 1.0)
+    y = ctx.conv2d_fwd(dx, dw, st, pd)
+    gx = ctx.conv2d_dgrad(dg, dw, (B, Cin, H, W), st, pd, 0)
+    w = torch.from_numpy(dw.numpy()).double()
+    for b in (0, cut - 1, cut, B - 1):
+        xb = torch.from_numpy(dx.rows(b, b + 1).numpy()).double().requires_grad_(True)
+        gb = torch.from_numpy(dg.rows(b, b + 1).numpy()).double()
+        ref = F.conv2d(xb, w, stride=st, padding=pd)
+        ref.backward(gb)
+        mag = F.conv2d(xb.detach().abs(), w.abs(), stride=st, padding=pd).max().item()
+        assert np.abs(y.rows(b, b + 1).numpy() - ref.detach().numpy()).max() <= 1e-5 * mag, ("fwd", b)
+        gmag = F.conv_transpose2d(gb.abs(), w.abs(), stride=st, padding=pd).max().item()
+        assert np.abs(gx.rows(b, b + 1).numpy() - xb.grad.numpy()).max() <= 1e-5 * gmag, ("dgrad", b)
+    gw = ctx.conv2d_wgrad(dx, dg, (Cout, Cin, 3, 3), st, pd, 0).numpy()
+    half = B // 2
+    parts = [ctx.conv2d_wgrad(dx.rows(lo, hi), dg.rows(lo, hi), (Cout, Cin, 3, 3), st, pd, 0).numpy().astype(np.float64)
+             for lo, hi in ((0, half), (half, B))]
+    ref = parts[0] + parts[1]
+    # sums of 37.7 million products each: the two groupings differ by rounding only
+    assert np.abs(gw - ref).max() <= 1e-5 * np.abs(ref).max() + 1e-3
+    assert np.array_equal(gw, ctx.conv2d_wgrad(dx, dg, (Cout, Cin, 3, 3), st, pd, 0).numpy())
+    # the CPU-literal gradient modes read the batch as one flat matrix and refuse such sizes
+    from ferrox_amd.capi import FerroxHipError
+    with pytest.raises(FerroxHipError, match="mode 1 does not support tensors of 2 GiB or more"):
+        ctx.conv2d_wgrad(dx, dg, (Cout, Cin, 3, 3), st, pd, 1)
