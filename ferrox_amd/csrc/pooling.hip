@@ -7,6 +7,8 @@
 //   unpool  grad_in[n,c,y,x] = sum over the windows (oy, ox ascending) that contain (y, x) of
 //           max: grad_out where |in - pooled| < 1e-8;   avg: grad_out * T(1.0f / float(kh*kw)).
 // Same operations in the same order as the CPU loops -> bit-identical (this file is built without contraction).
+#include <algorithm>
+
 #include "common.hpp"
 
 namespace {
@@ -173,11 +175,18 @@ int check_pool(PoolShape& s, i64 N, i64 C, i64 H, i64 W, i64 kh, i64 kw, i64 sh,
     s.div_oh = make_div((uint32_t)s.oh);
     s.div_sh = make_div((uint32_t)sh);
     s.div_sw = make_div((uint32_t)sw);
-    if (N * C * H * W >= (1ll << 31)) {
-        fx::set_error("%s: tensors of 2^31 elements or more are not supported by this build", what);
+    if (std::max(H * W, (i64)s.oh * s.ow) >= (1ll << 31)) {
+        fx::set_error("%s: planes of 2^31 elements or more are not supported by this build", what);
         return FX_ERR_UNSUPPORTED;
     }
     return FX_OK;
+}
+
+// The kernels number the elements of one launch with 32 bits.  Planes (image x channel) are independent, so a larger
+// tensor runs as several launches over ranges of planes; returns how many planes one launch may take.
+inline i64 planes_per_launch(const PoolShape& s, i64 planes) {
+    const i64 per = std::max((i64)s.H * s.W, (i64)s.oh * s.ow);
+    return std::min<i64>(planes, (((i64)1 << 31) - 1) / per);
 }
 
 template <typename T, bool IS_MAX>
@@ -186,6 +195,13 @@ int pool2d(fx_ctx* c, const T* in, T* out, i64 N, i64 C, i64 H, i64 W, i64 kh, i
     FX_REQUIRE(in && out, "%s: null pointer", what);
     PoolShape s;
     if (int rc = check_pool<T>(s, N, C, H, W, kh, kw, sh, sw, ph, pw, what)) return rc;
+    const i64 planes = N * C, ppl = planes_per_launch(s, planes);
+    if (planes > ppl) {
+        for (i64 p0 = 0; p0 < planes; p0 += ppl)
+            if (int rc = pool2d<T, IS_MAX>(c, in + p0 * H * W, out + p0 * s.oh * s.ow, std::min(ppl, planes - p0), 1, H, W, kh, kw, sh, sw, ph, pw, what))
+                return rc;
+        return FX_OK;
+    }
     const i64 n_out = N * C * s.oh * s.ow, blocks = fx::ceil_div(n_out, (i64)256);
     if (n_out == 0) return FX_OK;
     if (kh == 2 && kw == 2 && sh == 2 && sw == 2 && ph == 0 && pw == 0 && W % 2 == 0 && ((uintptr_t)in % (2 * sizeof(T))) == 0)
@@ -203,6 +219,16 @@ int unpool2d(fx_ctx* c, const T* gout, const T* in, const T* pooled, T* gin, i64
     FX_REQUIRE(gout && gin && (!IS_MAX || (in && pooled)), "%s: null pointer", what);
     PoolShape s;
     if (int rc = check_pool<T>(s, N, C, H, W, kh, kw, sh, sw, ph, pw, what)) return rc;
+    const i64 planes = N * C, ppl = planes_per_launch(s, planes);
+    if (planes > ppl) {
+        for (i64 p0 = 0; p0 < planes; p0 += ppl) {
+            const i64 oi = p0 * H * W, oo = p0 * s.oh * s.ow;
+            if (int rc = unpool2d<T, IS_MAX>(c, gout + oo, in ? in + oi : nullptr, pooled ? pooled + oo : nullptr, gin + oi,
+                                             std::min(ppl, planes - p0), 1, H, W, kh, kw, sh, sw, ph, pw, what))
+                return rc;
+        }
+        return FX_OK;
+    }
     const i64 n_in = N * C * H * W, blocks = fx::ceil_div(n_in, (i64)256);
     const float area = (float)(kh * kw);  // kernel_area is an f32 in the reference, for f64 tensors too (pooling.rs:361, 138)
     const T scale = (T)(1.0f / area);

@@ -166,3 +166,22 @@ def test_convolution_over_tensors_beyond_2_gib(ctx):
     from ferrox_amd.capi import FerroxHipError
     with pytest.raises(FerroxHipError, match="mode 1 does not support tensors of 2 GiB or more"):
         ctx.conv2d_wgrad(dx, dg, (Cout, Cin, 3, 3), st, pd, 1)
+
+
+def test_pooling_over_tensors_beyond_2_pow_31_elements(ctx):
+    """One launch numbers its elements with 32 bits; larger tensors run as ranges of (image, channel) planes.  Checked
+    on the images around the range boundary (plane 32767 of 256 x 256 elements lies inside image 2047)."""
+    import oracle as orc
+    N, Cc, H, W = 2100, 16, 256, 256                      # 2.2e9 elements, 8.8 GB
+    dx = ctx.uniform((N, Cc, H, W), 21, -1.0, 1.0)
+    dg = ctx.normal((N, Cc, H // 2, W // 2), 22, 0.0, 1.0)
+    pooled = ctx.pool2d(dx, (2, 2), (2, 2), (0, 0), True)
+    gin = ctx.unpool2d(dg, dx, pooled, (2, 2), (2, 2), (0, 0), True)
+    avg = ctx.pool2d(dx, (3, 3), (2, 2), (1, 1), False)
+    for b in (0, 2047, 2048, N - 1):
+        x = dx.rows(b, b + 1).numpy()
+        g = dg.rows(b, b + 1).numpy()
+        want = orc.pool2d(x, (2, 2), (2, 2), (0, 0), True)
+        assert np.array_equal(pooled.rows(b, b + 1).numpy(), want), ("max", b)
+        assert np.array_equal(gin.rows(b, b + 1).numpy(), orc.unpool2d(g, x, want, (2, 2), (2, 2), (0, 0), True)), ("unpool", b)
+        assert np.array_equal(avg.rows(b, b + 1).numpy(), orc.pool2d(x, (3, 3), (2, 2), (1, 1), False)), ("avg", b)
