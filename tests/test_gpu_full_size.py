@@ -185,3 +185,16 @@ def test_pooling_over_tensors_beyond_2_pow_31_elements(ctx):
         assert np.array_equal(pooled.rows(b, b + 1).numpy(), want), ("max", b)
         assert np.array_equal(gin.rows(b, b + 1).numpy(), orc.unpool2d(g, x, want, (2, 2), (2, 2), (0, 0), True)), ("unpool", b)
         assert np.array_equal(avg.rows(b, b + 1).numpy(), orc.pool2d(x, (3, 3), (2, 2), (1, 1), False)), ("avg", b)
+
+
+def test_batchnorm_statistics_over_more_than_2_pow_24_samples_per_channel(ctx):
+    """f32 sample counts above 2^24 are only weights of the pairwise merge; mean and variance stay at float accuracy."""
+    outer, Cc, inner = 48, 3, 1 << 20                      # 50.3 million samples per channel
+    dx = ctx.normal((outer, Cc, inner), 31, 3.0, 2.0)
+    mean, var = ctx.batchnorm_stats(dx)
+    x = dx.numpy().astype(np.float64)
+    m, v = x.mean(axis=(0, 2)), x.var(axis=(0, 2))
+    assert np.abs(mean.numpy() - m).max() <= 1e-5 * np.abs(m).max()
+    assert np.abs(var.numpy() - v).max() <= 1e-5 * v.max()
+    mean2, var2 = ctx.batchnorm_stats(dx)
+    assert np.array_equal(mean.numpy(), mean2.numpy()) and np.array_equal(var.numpy(), var2.numpy())
