@@ -4,7 +4,7 @@
 // y[b][m][oy][ox] = sum over (c, ky, kx) of wgt[m][c][ky][kx] * in[b][c][oy*sh+ky-ph][ox*sw+kx-pw]
 // (the product the reference forms as filter_2d . im2col(x), src/backend/storage/extensions/convolutions.rs:218-290).
 //
-// A block (4 waves, WM along the output channels) owns BM = 32*WM output channels x 32*TN*(4/WM) consecutive
+// A block (4 waves, WM = 4, 2 or 1 along the output channels) owns BM = 32*WM output channels x 32*TN*(4/WM) consecutive
 // output pixels of one image and walks the input channels in chunks of 8 (one stage each).  Per stage it holds in LDS
 //   Ws[m][tap*8 + c]   the weights of the chunk, pitch 73 (odd: the 32 lanes of an A read hit 32 banks)
 //   Xs[c][row][col]    the zero-padded input rows under the pixel tile, plane pitch odd for the same reason
@@ -232,14 +232,14 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
     Plan pl;
     if (kh != 3 || kw != 3 || C % CC != 0 || W % 4 != 0 || W > 4 * LPR || sh > 8 || sw > 8) return pl;
     const i64 L = OH * OW, slots = 2 * (i64)std::max(1, num_cus);
-    static const int shapes[8][2] = {{4, 8}, {4, 7}, {4, 6}, {4, 5}, {4, 4}, {2, 4}, {2, 3}, {2, 2}};
+    static const int shapes[11][2] = {{4, 8}, {4, 7}, {4, 6}, {4, 5}, {4, 4}, {2, 4}, {2, 3}, {2, 2}, {1, 4}, {1, 3}, {1, 2}};
     i64 best_cost = -1;
     for (const auto& sp : shapes) {
         const int wm = sp[0], tn = sp[1];
         const i64 bm = 32 * wm, np = 32 * tn * (4 / wm), tiles = fx::ceil_div(L, np), mtiles = fx::ceil_div(M, bm);
         // output rows under a tile: tiles that start on a row boundary cover exactly np / OW rows
         const i64 rows = std::min<i64>(OH, np % OW == 0 ? np / OW : (np - 1) / OW + 2), PR = (rows - 1) * sh + 3;
-        const bool tall_ok = wm == 2 || tn <= 6;  // instantiated tall variants
+        const bool tall_ok = wm <= 2 || tn <= 6;  // instantiated tall variants
         if (PR > 2 * NXP_TALL || (PR > 2 * NXP_SHORT && !tall_ok) || mtiles * bm * 4 > M * 5) continue;  // at most a quarter of the rows may be padding
         const i64 cost = fx::ceil_div(B * tiles * mtiles, slots) * np * bm;
         if (best_cost < 0 || cost < best_cost) {
@@ -310,6 +310,9 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
         FX_CPK_LAUNCH(2, 2)
         FX_CPK_LAUNCH(2, 3)
         FX_CPK_LAUNCH(2, 4)
+        FX_CPK_LAUNCH(1, 2)
+        FX_CPK_LAUNCH(1, 3)
+        FX_CPK_LAUNCH(1, 4)
         default: FX_REQUIRE(false, "conv patch kernel: unexpected tile %d x %d", pl.WM, pl.TN);
     }
 #undef FX_CPK_LAUNCH_N

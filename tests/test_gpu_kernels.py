@@ -489,6 +489,9 @@ CONV_PATCH_CASES = [
     # strided layers: up to 20 patch rows under a tile
     (8, 32, 32, 32, 64, (2, 2), (1, 1)), (4, 64, 56, 56, 128, (2, 2), (1, 1)), (2, 16, 30, 40, 60, (2, 1), (1, 1)),
     (2, 8, 17, 24, 128, (3, 3), (1, 1)), (64, 16, 28, 28, 128, (2, 2), (1, 1)),
+    # 32 channels out (forward) or in (data gradient): one block of channels, four waves along the pixels (1x2, 1x3, 1x4)
+    (64, 64, 32, 32, 32, (1, 1), (1, 1)), (3, 16, 9, 20, 30, (1, 1), (1, 1)), (64, 8, 16, 32, 32, (2, 1), (1, 1)),
+    (2, 8, 6, 8, 27, (1, 1), (0, 0)), (64, 32, 32, 32, 64, (1, 1), (1, 1)), (40, 32, 16, 16, 24, (1, 1), (1, 1)),
 ]
 
 

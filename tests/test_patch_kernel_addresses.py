@@ -72,11 +72,11 @@ def fwd_plan(num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
     if C % CC or W % 4 or W > 4 * LPR or sh > 8 or sw > 8: return None
     L, slots = OH * OW, 2 * num_cus
     best = None
-    for wm, tn in [(4, 8), (4, 7), (4, 6), (4, 5), (4, 4), (2, 4), (2, 3), (2, 2)]:
+    for wm, tn in [(4, 8), (4, 7), (4, 6), (4, 5), (4, 4), (2, 4), (2, 3), (2, 2), (1, 4), (1, 3), (1, 2)]:
         bm, np_ = 32 * wm, 32 * tn * (4 // wm)
         tiles, mtiles = _ceil_div(L, np_), _ceil_div(M, bm)
         rows = min(OH, np_ // OW if np_ % OW == 0 else (np_ - 1) // OW + 2); PR = (rows - 1) * sh + 3
-        tall_ok = wm == 2 or tn <= 6
+        tall_ok = wm <= 2 or tn <= 6
         if PR > 2 * NXP_TALL or (PR > 2 * NXP_SHORT and not tall_ok) or mtiles * bm * 4 > M * 5: continue
         cost = _ceil_div(B * tiles * mtiles, slots) * np_ * bm
         if best is None or cost < best[0]: best = (cost, wm, tn, PR, tiles)
@@ -244,6 +244,8 @@ FWD_SHAPES = [  # B, C, H, W, M, (sh, sw), (ph, pw): one per tile shape on a 256
     # strided layers: more than 8 patch rows under a tile
     (8, 32, 32, 32, 64, (2, 2), (1, 1)), (4, 64, 56, 56, 128, (2, 2), (1, 1)), (2, 16, 30, 40, 60, (2, 1), (1, 1)),
     (2, 8, 17, 24, 128, (3, 3), (1, 1)), (64, 64, 56, 56, 128, (2, 2), (1, 1)),
+    # 32 output channels: one block of channels, four waves along the pixels
+    (256, 64, 32, 32, 32, (1, 1), (1, 1)), (3, 16, 9, 20, 30, (1, 1), (1, 1)), (64, 8, 16, 32, 32, (2, 1), (1, 1)), (2, 8, 6, 8, 27, (1, 1), (0, 0)),
 ]
 
 
