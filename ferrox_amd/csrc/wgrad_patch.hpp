@@ -7,9 +7,10 @@
 //   Gs[oc][pixel]      BM output-channel rows of g, pixels contiguous as in memory  (pitch GP,    GP % 32 == 1)
 //   Xs[c][row][col]    CT input-channel planes of the zero-padded rows those pixels touch (pitch PLANE % 32 == 1)
 // The four waves are laid out WMO x WC x WK: WMO blocks of 32 output channels (BM = 32 WMO), WC blocks of 32 input
-// channels (CT = 32 WC) and WK segments of every pixel row (each segment ends in its own partial sum):
+// channels (CT = 32 WC) and WK segments of every pixel row (the segments' sums are added at the end of the block):
 //   4 x 1 x 1  more than 64 output channels;   2 x 2 x 1  up to 64, input channels a multiple of 64;
-//   2 x 1 x 2  up to 64 output channels, input channels a multiple of 32.
+//   2 x 1 x 2  up to 64 output channels, input channels a multiple of 32;
+//   1 x 2 x 2  up to 32 output channels, input channels a multiple of 64;   1 x 1 x 4  up to 32, a multiple of 32.
 // Every wave then runs 9 accumulator blocks of 32(oc) x 32(c), one per filter tap: the MFMA A operand of lane l
 // is Gs[oc = l%32][pixel + l/32], the B operand of tap (ky,kx) is Xs[c = l%32][that pixel shifted by (ky,kx)].
 // The odd pitches put the 32 lanes of a half-wave on 32 different LDS banks for both reads.  The patch is loaded
@@ -20,7 +21,7 @@
 // Staging: thread t owns float4 column t % 16 of rows t/16 + 16u of either operand, so every address is a
 // per-thread constant plus a wave-uniform step.  The next stage's global loads are issued before the MFMA loop of
 // the current stage and held in registers until that loop is done.  That fixes the shapes served here (rows of at
-// most 64 floats, 3 or 4 patch rows, more than 32 output channels); the implicit-GEMM kernel takes the rest.
+// most 64 floats, 3 or 4 patch rows); the implicit-GEMM kernel takes the rest.
 #pragma once
 #include "igemm_core.hpp"
 
@@ -199,7 +200,29 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
         __syncthreads();
     }
 
-    float* out = p.part + ((i64)bzi * WK + wk) * p.part_stride;
+    // The WK waves that split the pixel rows hold partial sums of the same outputs: added here in order of wk, tap by
+    // tap through LDS (the stage buffers are free after the loop's last barrier), so a block leaves one partial sum.
+    if constexpr (WK > 1) {
+        float* red = smem;  // [4 waves][16][64]
+#pragma unroll
+        for (int t = 0; t < KK; ++t) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) red[(wave * 16 + e) * 64 + lane] = acc[t][e];
+            __syncthreads();
+            if (wk == 0) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    float v = acc[t][e];
+#pragma unroll
+                    for (int q = 1; q < WK; ++q) v = v + red[((wave + q * WMO * WC) * 16 + e) * 64 + lane];
+                    acc[t][e] = v;
+                }
+            }
+            __syncthreads();
+        }
+        if (wk != 0) return;
+    }
+    float* out = p.part + (i64)bzi * p.part_stride;
     const int ldo = KK * p.Cin;
 #pragma unroll
     for (int t = 0; t < KK; ++t)
@@ -270,31 +293,45 @@ struct Plan {
     size_t smem = 0;
     int bm() const { return 32 * WMO; }
     int ct() const { return 32 * WC; }
-    int partials() const { return splits * WK; }
+    int partials() const { return splits; }
 };
 
 inline int odd_pitch(int n) { return (n + 30) / 32 * 32 + 1; }  // smallest pitch >= n with pitch % 32 == 1
 
 inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, i64 oh, i64 ow) {
     Plan pl;
-    if (kh != KH || kw != KW || Cin % 32 != 0 || Cout <= 32 || ow % 2 != 0 || W % 4 != 0 || W > 4 * LPR || sh > 8 || sw > 8) return pl;
-    if (Cout <= 64) {  // two blocks of output channels; the other two waves take more input channels or split the rows
-        pl.WMO = 2;
-        if (Cin % 64 == 0) pl.WC = 2;
-        else if (ow % 4 == 0) pl.WK = 2;
-        else return pl;
+    if (kh != KH || kw != KW || Cin % 32 != 0 || ow % 2 != 0 || W % 4 != 0 || W > 4 * LPR || sh > 8 || sw > 8) return pl;
+    // Wave layouts that fit the channel counts, the preferred one first.  Up to 32 output channels: one block of them, the
+    // four waves split the input channels and / or the rows; up to 64: two blocks, the other two waves take more input
+    // channels or split the rows.  A layout with 64 input channels per block holds only 3 patch rows (64 channel planes x
+    // 4 rows would not fit the register file while in flight), which on narrow maps leaves stages too short: then the
+    // next layout is tried.
+    int cand[2][3], ncand = 0;
+    auto add = [&](int a, int b, int c) { cand[ncand][0] = a; cand[ncand][1] = b; cand[ncand][2] = c; ++ncand; };
+    if (Cout <= 32) {
+        if (Cin % 64 == 0 && ow % 4 == 0) add(1, 2, 2);
+        if (ow % 8 == 0) add(1, 1, 4);
+    } else if (Cout <= 64) {
+        if (Cin % 64 == 0) add(2, 2, 1);
+        if (ow % 4 == 0) add(2, 1, 2);
+    } else {
+        add(4, 1, 1);
     }
-    const i64 BM = pl.bm(), CT = pl.ct();
-    const i64 max_pr = pl.WC == 2 ? 3 : 4;  // 64 channel planes x 4 rows would not fit the register file while in flight
     int best = 0;  // the most rows per stage that keep a stage within 64 pixels and max_pr patch rows
-    for (int R = 1; R <= oh; ++R) {
-        if (oh % R || R * ow > 4 * LPR || (R - 1) * sh + kh > max_pr) continue;
-        if ((R * ow) % 4 == 0) best = R;
+    for (int k = 0; k < ncand && !best; ++k) {
+        pl.WMO = cand[k][0]; pl.WC = cand[k][1]; pl.WK = cand[k][2];
+        const i64 max_pr = pl.WC == 2 ? 3 : 4;
+        for (int R = 1; R <= oh; ++R) {
+            if (oh % R || R * ow > 4 * LPR || (R - 1) * sh + kh > max_pr) continue;
+            if ((R * ow) % 4 == 0) best = R;
+        }
+        // measured at [256,32,32,32] -> 64, stride 2 (16 pixels per stage): 0.063 ms here against 0.050 ms for the implicit GEMM
+        // (and with two output rows over five patch rows per stage: 0.063 against 0.053 ms there, 0.192 against 0.156 ms at
+        // [128,64,56,56] -> 128 stride 2: a strided patch stages four input values per output pixel)
+        if (best * ow < 24) best = 0;
     }
-    // measured at [256,32,32,32] -> 64, stride 2 (16 pixels per stage): 0.063 ms here against 0.050 ms for the implicit GEMM
-    // (and with two output rows over five patch rows per stage: 0.063 against 0.053 ms there, 0.192 against 0.156 ms at
-    // [128,64,56,56] -> 128 stride 2: a strided patch stages four input values per output pixel)
-    if (!best || best * ow < 24) return pl;
+    if (!best) return pl;
+    const i64 BM = pl.bm(), CT = pl.ct();
     pl.R = best;
     pl.PR = (int)((best - 1) * sh + kh);
     pl.PW = (int)(W + 2 * pw);
@@ -302,11 +339,14 @@ inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 k
     pl.Kst = (int)(best * ow);
     pl.GP = odd_pitch(pl.Kst);
     pl.smem = ((size_t)BM * pl.GP + (size_t)CT * pl.PLANE + SLACK) * sizeof(float);
+    if (pl.WK > 1) pl.smem = std::max<size_t>(pl.smem, 4 * 16 * 64 * sizeof(float));  // the closing sum over the row segments
     if (pl.smem > LDS_BUDGET) return pl;
     pl.stages = (int)(B * (oh / best));
     const i64 tiles = (Cin / CT) * fx::ceil_div(Cout, BM);
     const i64 want = (i64)num_cus * 2;
-    const i64 splits = std::max<i64>(1, std::min<i64>(want / tiles, pl.stages));
+    // at least four stages per block where there are that many: a block's partial sum (and its closing sum over the row
+    // segments) is paid once per block
+    const i64 splits = std::max<i64>(1, std::min<i64>(want / tiles, std::max<i64>(1, pl.stages / 4)));
     pl.sps = (int)fx::ceil_div((i64)pl.stages, splits);
     pl.splits = (int)fx::ceil_div((i64)pl.stages, (i64)pl.sps);
     if (pl.splits > 65535 || tiles > 65535 || Cout * Cin * KK > 0x7fffffff) return pl;
@@ -343,6 +383,9 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
     else if (layout == 221 && pl.PR == 3) FX_WGP_LAUNCH(3, 2, 2, 1);
     else if (layout == 212 && pl.PR == 3) FX_WGP_LAUNCH(3, 2, 1, 2);
     else if (layout == 212) FX_WGP_LAUNCH(4, 2, 1, 2);
+    else if (layout == 122) FX_WGP_LAUNCH(3, 1, 2, 2);
+    else if (layout == 114 && pl.PR == 3) FX_WGP_LAUNCH(3, 1, 1, 4);
+    else if (layout == 114) FX_WGP_LAUNCH(4, 1, 1, 4);
     else FX_REQUIRE(false, "wgrad patch kernel: unexpected wave layout %d", layout);
 #undef FX_WGP_LAUNCH
     FX_LAUNCH_CHECK();

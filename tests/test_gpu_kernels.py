@@ -434,6 +434,10 @@ WGRAD_PATCH_CASES = [
     # ragged output-channel counts in the last image: the 16-row staging passes past the last channel must not be read
     (1, 32, 6, 24, 40, (1, 1), (1, 1)), (2, 64, 6, 28, 49, (1, 1), (1, 1)), (1, 32, 4, 32, 97, (1, 1), (1, 1)),
     (3, 32, 8, 12, 72, (1, 1), (1, 1)), (2, 32, 8, 16, 150, (1, 1), (1, 1)), (1, 64, 5, 56, 36, (1, 1), (1, 1)),
+    # at most 32 output channels: wave layouts 1 x 2 x 2 and 1 x 1 x 4, ragged counts
+    (2, 64, 8, 32, 32, (1, 1), (1, 1)), (3, 32, 8, 32, 32, (1, 1), (1, 1)), (2, 64, 6, 28, 20, (1, 1), (1, 1)), (2, 32, 10, 24, 7, (1, 1), (1, 1)),
+    (2, 96, 12, 16, 17, (1, 1), (1, 1)), (33, 32, 16, 16, 32, (1, 1), (1, 1)), (2, 128, 16, 16, 32, (1, 1), (1, 1)),
+    (3, 128, 16, 16, 64, (1, 1), (1, 1)),
     # strided layers (implicit GEMM)
     (3, 32, 32, 32, 64, (2, 2), (1, 1)), (2, 64, 56, 56, 128, (2, 2), (1, 1)), (2, 32, 16, 24, 70, (2, 1), (1, 1)),
     (2, 32, 13, 32, 48, (2, 2), (0, 1)),

@@ -12,20 +12,26 @@ import pytest
 LPR, NT, RPP = 16, 256, 16
 def _odd_pitch_w(n): return (n + 30) // 32 * 32 + 1
 def wgrad_plan(num_cus, B, Cin, H, W, Cout, sh, sw, ph, pw, oh, ow):
-    if Cin % 32 or Cout <= 32 or ow % 2 or W % 4 or W > 64 or sh > 8 or sw > 8: return None
-    WMO, WC, WK = 4, 1, 1
-    if Cout <= 64:
-        WMO = 2
-        if Cin % 64 == 0: WC = 2
-        elif ow % 4 == 0: WK = 2
-        else: return None
-    BM, CT = 32 * WMO, 32 * WC
-    max_pr = 3 if WC == 2 else 4
+    if Cin % 32 or ow % 2 or W % 4 or W > 64 or sh > 8 or sw > 8: return None
+    cand = []
+    if Cout <= 32:
+        if Cin % 64 == 0 and ow % 4 == 0: cand.append((1, 2, 2))
+        if ow % 8 == 0: cand.append((1, 1, 4))
+    elif Cout <= 64:
+        if Cin % 64 == 0: cand.append((2, 2, 1))
+        if ow % 4 == 0: cand.append((2, 1, 2))
+    else:
+        cand.append((4, 1, 1))
     best = 0
-    for R in range(1, oh + 1):
-        if oh % R or R * ow > 64 or (R - 1) * sh + 3 > max_pr: continue
-        if (R * ow) % 4 == 0: best = R
-    if not best or best * ow < 24: return None
+    for WMO, WC, WK in cand:
+        BM, CT = 32 * WMO, 32 * WC
+        max_pr = 3 if WC == 2 else 4
+        for R in range(1, oh + 1):
+            if oh % R or R * ow > 64 or (R - 1) * sh + 3 > max_pr: continue
+            if (R * ow) % 4 == 0: best = R
+        if best * ow < 24: best = 0
+        if best: break
+    if not best: return None
     PR = (best - 1) * sh + 3
     return dict(R=best, PR=PR, BM=BM, CT=CT, Kst=best * ow, stages=B * (oh // best), spi=oh // best)
 def wgrad_loads_in_bounds(B, Cin, H, W, Cout, st, pd):
@@ -234,6 +240,9 @@ WGRAD_SHAPES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw): every wave layout, r
     (2, 32, 12, 32, 64, (1, 1), (1, 1)), (5, 32, 6, 64, 33, (1, 1), (1, 1)), (1, 32, 6, 24, 40, (1, 1), (1, 1)),
     (2, 64, 6, 28, 49, (1, 1), (1, 1)), (1, 32, 4, 32, 97, (1, 1), (1, 1)), (3, 32, 8, 12, 72, (1, 1), (1, 1)),
     (2, 32, 8, 16, 150, (1, 1), (1, 1)), (1, 64, 5, 56, 36, (1, 1), (1, 1)), (2, 32, 8, 56, 65, (2, 1), (1, 1)),
+    # at most 32 output channels: 1 x 2 x 2 and 1 x 1 x 4, ragged counts
+    (2, 64, 8, 32, 32, (1, 1), (1, 1)), (3, 32, 8, 32, 32, (1, 1), (1, 1)), (2, 64, 6, 28, 20, (1, 1), (1, 1)), (2, 32, 10, 24, 7, (1, 1), (1, 1)),
+    (2, 96, 12, 16, 17, (1, 1), (1, 1)), (2, 128, 16, 16, 32, (1, 1), (1, 1)), (2, 128, 16, 16, 64, (1, 1), (1, 1)),
 ]
 FWD_SHAPES = [  # B, C, H, W, M, (sh, sw), (ph, pw): one per tile shape on a 256-CU device, ragged M, strides, paddings
     (2, 64, 28, 28, 64, (1, 1), (1, 1)), (2, 8, 6, 12, 60, (1, 1), (1, 1)), (3, 16, 8, 36, 120, (1, 1), (0, 0)),
