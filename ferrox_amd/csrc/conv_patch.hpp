@@ -240,7 +240,7 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
         // output rows under a tile: tiles that start on a row boundary cover exactly np / OW rows
         const i64 rows = std::min<i64>(OH, np % OW == 0 ? np / OW : (np - 1) / OW + 2), PR = (rows - 1) * sh + 3;
         const bool tall_ok = wm <= 2 || tn <= 6;  // instantiated tall variants
-        if (PR > 2 * NXP_TALL || (PR > 2 * NXP_SHORT && !tall_ok) || mtiles * bm * 4 > M * 5) continue;  // at most a quarter of the rows may be padding
+        if (PR > 2 * NXP_TALL || (PR > 2 * NXP_SHORT && !tall_ok) || mtiles * bm > M * 2) continue;  // at most half of the rows may be padding
         const i64 cost = fx::ceil_div(B * tiles * mtiles, slots) * np * bm;
         if (best_cost < 0 || cost < best_cost) {
             best_cost = cost;

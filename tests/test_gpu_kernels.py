@@ -483,7 +483,7 @@ CONV_PATCH_CASES = [
     (2, 64, 28, 28, 64, (1, 1), (1, 1)), (1, 8, 64, 64, 32, (1, 1), (1, 1)), (2, 16, 6, 16, 40, (2, 2), (1, 1)),
     (2, 8, 5, 12, 24, (1, 1), (0, 1)), (5, 72, 6, 40, 200, (1, 1), (1, 1)), (2, 128, 6, 8, 72, (1, 1), (1, 0)),
     (2, 8, 12, 12, 16, (1, 1), (1, 1)),
-    # output-channel counts within a quarter of a 64 / 128 tile (the planner refuses more padding), one per tile shape
+    # ragged output-channel counts, one per tile shape
     # of the forward kernel on a 256-CU device: 2x2, 2x3, 2x4, 4x4, 4x5, 4x6, 4x7, 4x8
     (2, 8, 6, 12, 60, (1, 1), (1, 1)), (3, 16, 8, 36, 120, (1, 1), (0, 0)), (2, 24, 4, 8, 104, (1, 1), (2, 2)),
     (1, 8, 64, 64, 52, (1, 1), (1, 1)), (2, 16, 6, 16, 60, (2, 2), (1, 1)), (2, 128, 6, 8, 120, (1, 1), (1, 0)),
@@ -496,6 +496,9 @@ CONV_PATCH_CASES = [
     # 32 channels out (forward) or in (data gradient): one block of channels, four waves along the pixels (1x2, 1x3, 1x4)
     (64, 64, 32, 32, 32, (1, 1), (1, 1)), (3, 16, 9, 20, 30, (1, 1), (1, 1)), (64, 8, 16, 32, 32, (2, 1), (1, 1)),
     (2, 8, 6, 8, 27, (1, 1), (0, 0)), (64, 32, 32, 32, 64, (1, 1), (1, 1)), (40, 32, 16, 16, 24, (1, 1), (1, 1)),
+    # up to half of a tile's channel rows are padding
+    (3, 16, 8, 32, 16, (1, 1), (1, 1)), (2, 8, 12, 28, 40, (1, 1), (1, 1)), (16, 8, 56, 56, 72, (1, 1), (1, 1)), (3, 24, 9, 12, 17, (1, 1), (1, 1)),
+    (4, 48, 16, 16, 64, (1, 1), (1, 1)),
 ]
 
 

@@ -83,7 +83,7 @@ def fwd_plan(num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
         tiles, mtiles = _ceil_div(L, np_), _ceil_div(M, bm)
         rows = min(OH, np_ // OW if np_ % OW == 0 else (np_ - 1) // OW + 2); PR = (rows - 1) * sh + 3
         tall_ok = wm <= 2 or tn <= 6
-        if PR > 2 * NXP_TALL or (PR > 2 * NXP_SHORT and not tall_ok) or mtiles * bm * 4 > M * 5: continue
+        if PR > 2 * NXP_TALL or (PR > 2 * NXP_SHORT and not tall_ok) or mtiles * bm > M * 2: continue
         cost = _ceil_div(B * tiles * mtiles, slots) * np_ * bm
         if best is None or cost < best[0]: best = (cost, wm, tn, PR, tiles)
     if best is None: return None
@@ -255,6 +255,8 @@ FWD_SHAPES = [  # B, C, H, W, M, (sh, sw), (ph, pw): one per tile shape on a 256
     (2, 8, 17, 24, 128, (3, 3), (1, 1)), (64, 64, 56, 56, 128, (2, 2), (1, 1)),
     # 32 output channels: one block of channels, four waves along the pixels
     (256, 64, 32, 32, 32, (1, 1), (1, 1)), (3, 16, 9, 20, 30, (1, 1), (1, 1)), (64, 8, 16, 32, 32, (2, 1), (1, 1)), (2, 8, 6, 8, 27, (1, 1), (0, 0)),
+    # up to half of a tile's channel rows are padding
+    (2, 16, 8, 32, 16, (1, 1), (1, 1)), (2, 8, 12, 28, 40, (1, 1), (1, 1)), (128, 8, 56, 56, 72, (1, 1), (1, 1)), (3, 24, 9, 12, 17, (1, 1), (1, 1)),
 ]
 
 
