@@ -438,6 +438,9 @@ WGRAD_PATCH_CASES = [
     (2, 64, 8, 32, 32, (1, 1), (1, 1)), (3, 32, 8, 32, 32, (1, 1), (1, 1)), (2, 64, 6, 28, 20, (1, 1), (1, 1)), (2, 32, 10, 24, 7, (1, 1), (1, 1)),
     (2, 96, 12, 16, 17, (1, 1), (1, 1)), (33, 32, 16, 16, 32, (1, 1), (1, 1)), (2, 128, 16, 16, 32, (1, 1), (1, 1)),
     (3, 128, 16, 16, 64, (1, 1), (1, 1)),
+    # input channels that do not fill the last block of 32 (their LDS planes stay zero)
+    (2, 16, 8, 32, 32, (1, 1), (1, 1)), (3, 48, 8, 32, 30, (1, 1), (1, 1)), (2, 24, 12, 24, 20, (1, 1), (1, 1)), (2, 40, 6, 16, 13, (1, 1), (1, 1)),
+    (1, 33, 8, 24, 16, (1, 1), (1, 1)), (2, 17, 6, 32, 32, (1, 1), (1, 1)), (3, 48, 8, 32, 64, (1, 1), (1, 1)),
     # strided layers (implicit GEMM)
     (3, 32, 32, 32, 64, (2, 2), (1, 1)), (2, 64, 56, 56, 128, (2, 2), (1, 1)), (2, 32, 16, 24, 70, (2, 1), (1, 1)),
     (2, 32, 13, 32, 48, (2, 2), (0, 1)),

@@ -12,7 +12,8 @@ import pytest
 LPR, NT, RPP = 16, 256, 16
 def _odd_pitch_w(n): return (n + 30) // 32 * 32 + 1
 def wgrad_plan(num_cus, B, Cin, H, W, Cout, sh, sw, ph, pw, oh, ow):
-    if Cin % 32 or ow % 2 or W % 4 or W > 64 or sh > 8 or sw > 8: return None
+    if Cin % 32 and (Cout > 32 or (Cin + 31) // 32 * 32 > 2 * Cin): return None
+    if ow % 2 or W % 4 or W > 64 or sh > 8 or sw > 8: return None
     cand = []
     if Cout <= 32:
         if Cin % 64 == 0 and ow % 4 == 0: cand.append((1, 2, 2))
@@ -59,15 +60,21 @@ def wgrad_loads_in_bounds(B, Cin, H, W, Cout, st, pd):
                     assert 0 <= a and a + 4 <= gsize, ("g", (B, Cin, H, W, Cout, st, pd), s, oc0, tid, u, a, gsize)
         for c0 in range(0, Cin, pl["CT"]):
             xsrc = (b * Cin + c0) * H * W
+            full_c = c0 + pl["CT"] <= Cin
             for tid in range(NT):
                 pq, prow = tid % LPR, tid // LPR
                 x_off = (prow * H * W + 4 * pq) if pq < w4 else 0
+                x_off0 = 4 * pq if pq < w4 else 0
                 for r in range(pl["PR"]):
                     iy = iy0 + r
                     if not (0 <= iy < H): continue
                     for cu in range(NXC):
-                        a = xsrc + (cu * RPP * H + iy) * W + x_off
+                        pass_in = full_c or c0 + cu * RPP < Cin
+                        ok = full_c or c0 + prow + cu * RPP < Cin
+                        a = xsrc + ((cu * RPP if pass_in else 0) * H + iy) * W + (x_off if ok else x_off0)
                         assert 0 <= a and a + 4 <= xsize, ("x", (B, Cin, H, W, Cout, st, pd), a, xsize)
+                        if ok and pq < w4:  # the plane read is the one the lane parks
+                            assert a == ((b * Cin + c0 + cu * RPP + prow) * H + iy) * W + 4 * pq
     return "patch"
 
 CC, KK, WPITCH = 8, 9, 73
@@ -243,6 +250,9 @@ WGRAD_SHAPES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw): every wave layout, r
     # at most 32 output channels: 1 x 2 x 2 and 1 x 1 x 4, ragged counts
     (2, 64, 8, 32, 32, (1, 1), (1, 1)), (3, 32, 8, 32, 32, (1, 1), (1, 1)), (2, 64, 6, 28, 20, (1, 1), (1, 1)), (2, 32, 10, 24, 7, (1, 1), (1, 1)),
     (2, 96, 12, 16, 17, (1, 1), (1, 1)), (2, 128, 16, 16, 32, (1, 1), (1, 1)), (2, 128, 16, 16, 64, (1, 1), (1, 1)),
+    # input channels that do not fill the last block of 32
+    (2, 16, 8, 32, 32, (1, 1), (1, 1)), (3, 48, 8, 32, 30, (1, 1), (1, 1)), (2, 24, 12, 24, 20, (1, 1), (1, 1)), (2, 40, 6, 16, 13, (1, 1), (1, 1)),
+    (1, 33, 8, 24, 16, (1, 1), (1, 1)), (2, 17, 6, 32, 32, (1, 1), (1, 1)),
 ]
 FWD_SHAPES = [  # B, C, H, W, M, (sh, sw), (ph, pw): one per tile shape on a 256-CU device, ragged M, strides, paddings
     (2, 64, 28, 28, 64, (1, 1), (1, 1)), (2, 8, 6, 12, 60, (1, 1), (1, 1)), (3, 16, 8, 36, 120, (1, 1), (0, 0)),
