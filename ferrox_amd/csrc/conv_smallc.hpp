@@ -52,14 +52,15 @@ struct WgradParams {
 // Copies the rows under tile `tile` of image b into the patch (rows outside the image become zero; the padding
 // columns are zeroed by the caller once and never written).
 __device__ __forceinline__ void stage_patch(const Geometry& g, const float* __restrict__ x, float* patch, int b, int iy0, int tid) {
-    const int W4 = g.W >> 2, items = g.C * g.PR * W4;
+    // ceil(W / 4) vectors per row; the last one is moved back to end with the row (overlapping its neighbour)
+    const int W4 = (g.W + 3) >> 2, items = g.C * g.PR * W4;
     for (int i = tid; i < items; i += NT) {
-        const int rc = (int)g.div_w4.div((uint32_t)i), q = i - rc * W4;
+        const int rc = (int)g.div_w4.div((uint32_t)i), q = min(4 * (i - rc * W4), g.W - 4);
         const int c = (int)g.div_pr.div((uint32_t)rc), r = rc - c * g.PR;
         const int iy = iy0 + r;
         const bool ok = iy >= 0 && iy < g.H;
-        const float4 v = *reinterpret_cast<const float4*>(x + (((i64)b * g.C + c) * g.H + (ok ? iy : 0)) * g.W + 4 * q);
-        float* d = patch + c * g.PLANE + r * g.PW + g.pw + 4 * q;
+        const float4 v = *reinterpret_cast<const float4*>(x + (((i64)b * g.C + c) * g.H + (ok ? iy : 0)) * g.W + q);
+        float* d = patch + c * g.PLANE + r * g.PW + g.pw + q;
         d[0] = ok ? v.x : 0.f; d[1] = ok ? v.y : 0.f; d[2] = ok ? v.z : 0.f; d[3] = ok ? v.w : 0.f;
     }
 }
@@ -200,7 +201,7 @@ inline Plan make_plan(int num_cus, bool wgrad, i64 B, i64 C, i64 H, i64 W, i64 C
                       i64 OH, i64 OW) {
     Plan pl;
     const i64 L = OH * OW;
-    if (kh != 3 || kw != 3 || W % 4 != 0 || sh > 8 || sw > 8 || ph > 8 || pw > 8) return pl;
+    if (kh != 3 || kw != 3 || W < 4 || sh > 8 || sw > 8 || ph > 8 || pw > 8) return pl;
     if (wgrad ? (C * KK > 32 || L % 4 != 0) : C > 4) return pl;
     const i64 rows = std::min<i64>(OH, NPIX % OW == 0 ? NPIX / OW : (NPIX - 1) / OW + 2);
     pl.PR = (int)((rows - 1) * sh + 3);
@@ -234,7 +235,7 @@ inline Geometry make_geometry(const Plan& pl, i64 C, i64 H, i64 W, i64 Cout, i64
     g.sh = (int)sh; g.sw = (int)sw; g.ph = (int)ph; g.pw = (int)pw;
     g.PR = pl.PR; g.PW = pl.PW; g.PLANE = pl.PLANE; g.tpi = pl.tpi;
     g.div_tpi = FastDiv((uint32_t)pl.tpi); g.div_ow = FastDiv((uint32_t)OW);
-    g.div_w4 = FastDiv((uint32_t)(W / 4)); g.div_pr = FastDiv((uint32_t)pl.PR);
+    g.div_w4 = FastDiv((uint32_t)((W + 3) / 4)); g.div_pr = FastDiv((uint32_t)pl.PR);
     return g;
 }
 

@@ -488,20 +488,23 @@ CONV_PATCH_CASES = [
     (2, 8, 12, 12, 16, (1, 1), (1, 1)),
     # ragged output-channel counts, one per tile shape
     # of the forward kernel on a 256-CU device: 2x2, 2x3, 2x4, 4x4, 4x5, 4x6, 4x7, 4x8
-    (2, 8, 6, 12, 60, (1, 1), (1, 1)), (3, 16, 8, 36, 120, (1, 1), (0, 0)), (2, 24, 4, 8, 104, (1, 1), (2, 2)),
-    (1, 8, 64, 64, 52, (1, 1), (1, 1)), (2, 16, 6, 16, 60, (2, 2), (1, 1)), (2, 128, 6, 8, 120, (1, 1), (1, 0)),
+    (2, 8, 6, 12, 60, (1, 1), (1, 1)), (3, 16, 8, 36, 120, (1, 1), (0, 0)), (2, 24, 6, 8, 104, (1, 1), (2, 2)),
+    (1, 8, 64, 64, 52, (1, 1), (1, 1)), (2, 16, 15, 18, 60, (2, 2), (1, 1)), (2, 128, 6, 8, 120, (1, 1), (1, 0)),
     (2, 8, 9, 64, 128, (2, 1), (1, 1)), (128, 8, 8, 40, 120, (1, 1), (1, 1)), (32, 8, 56, 56, 64, (1, 1), (1, 1)),
     (16, 8, 56, 56, 120, (1, 1), (1, 1)), (128, 8, 8, 40, 250, (1, 1), (1, 1)), (96, 8, 12, 48, 384, (1, 1), (1, 1)),
     (32, 8, 56, 56, 120, (1, 1), (1, 1)), (128, 8, 16, 64, 120, (1, 1), (1, 1)),
     # strided layers: up to 20 patch rows under a tile
     (8, 32, 32, 32, 64, (2, 2), (1, 1)), (4, 64, 56, 56, 128, (2, 2), (1, 1)), (2, 16, 30, 40, 60, (2, 1), (1, 1)),
-    (2, 8, 17, 24, 128, (3, 3), (1, 1)), (64, 16, 28, 28, 128, (2, 2), (1, 1)),
+    (2, 8, 16, 34, 128, (3, 3), (1, 1)), (64, 16, 28, 28, 128, (2, 2), (1, 1)),
     # 32 channels out (forward) or in (data gradient): one block of channels, four waves along the pixels (1x2, 1x3, 1x4)
     (64, 64, 32, 32, 32, (1, 1), (1, 1)), (3, 16, 9, 20, 30, (1, 1), (1, 1)), (64, 8, 16, 32, 32, (2, 1), (1, 1)),
-    (2, 8, 6, 8, 27, (1, 1), (0, 0)), (64, 32, 32, 32, 64, (1, 1), (1, 1)), (40, 32, 16, 16, 24, (1, 1), (1, 1)),
+    (2, 8, 18, 10, 27, (1, 1), (0, 0)), (64, 32, 32, 32, 64, (1, 1), (1, 1)), (40, 32, 16, 16, 24, (1, 1), (1, 1)),
     # up to half of a tile's channel rows are padding
-    (3, 16, 8, 32, 16, (1, 1), (1, 1)), (2, 8, 12, 28, 40, (1, 1), (1, 1)), (16, 8, 56, 56, 72, (1, 1), (1, 1)), (3, 24, 9, 12, 17, (1, 1), (1, 1)),
+    (3, 16, 8, 32, 16, (1, 1), (1, 1)), (2, 8, 12, 28, 40, (1, 1), (1, 1)), (16, 8, 56, 56, 72, (1, 1), (1, 1)), (3, 24, 12, 12, 17, (1, 1), (1, 1)),
     (4, 48, 16, 16, 64, (1, 1), (1, 1)),
+    # row lengths that are not multiples of four floats (the last vector of a row is moved back to end with the row)
+    (3, 8, 14, 14, 64, (1, 1), (1, 1)), (2, 16, 10, 7, 32, (1, 1), (1, 1)), (2, 8, 9, 30, 128, (1, 1), (0, 0)), (2, 8, 15, 18, 40, (2, 2), (1, 1)),
+    (2, 8, 6, 63, 64, (1, 1), (1, 1)), (64, 64, 14, 14, 128, (1, 1), (1, 1)),
 ]
 
 
@@ -550,6 +553,8 @@ SMALLC_CASES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw)
     (2, 2, 17, 20, 33, (2, 2), (1, 1)), (2, 3, 7, 8, 5, (3, 1), (1, 1)), (1, 3, 40, 36, 64, (1, 1), (1, 1)),
     (1, 3, 66, 64, 16, (2, 2), (1, 1)), (2, 1, 5, 4, 70, (1, 1), (2, 2)), (1, 3, 19, 60, 8, (1, 1), (1, 1)),
     (1, 3, 20, 224, 16, (2, 2), (1, 1)), (1, 4, 10, 64, 16, (1, 2), (2, 0)), (3, 3, 9, 12, 40, (1, 1), (0, 0)), (37, 3, 16, 16, 32, (1, 1), (1, 1)),
+    # row lengths that are not multiples of four floats
+    (2, 3, 14, 14, 32, (1, 1), (1, 1)), (2, 1, 9, 7, 16, (1, 1), (1, 1)), (2, 3, 12, 30, 8, (1, 1), (1, 1)), (3, 1, 8, 5, 8, (1, 1), (1, 1)),
 ]
 
 

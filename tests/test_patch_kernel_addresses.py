@@ -58,13 +58,17 @@ def wgrad_loads_in_bounds(B, Cin, H, W, Cout, st, pd):
                     base = gsrc + u * RPP * L if pass_in else gsrc
                     a = base + (g_off if ok else 0)
                     assert 0 <= a and a + 4 <= gsize, ("g", (B, Cin, H, W, Cout, st, pd), s, oc0, tid, u, a, gsize)
+                    if ok and pq < k4:  # the four floats are pixels of this stage in the lane's own channel row
+                        row0 = (b * Cout + oc0 + prow + u * RPP) * L + oy0 * ow
+                        assert row0 <= a and a + 4 <= row0 + pl["Kst"]
         for c0 in range(0, Cin, pl["CT"]):
             xsrc = (b * Cin + c0) * H * W
             full_c = c0 + pl["CT"] <= Cin
             for tid in range(NT):
                 pq, prow = tid % LPR, tid // LPR
-                x_off = (prow * H * W + 4 * pq) if pq < w4 else 0
-                x_off0 = 4 * pq if pq < w4 else 0
+                xcol = 4 * pq
+                x_off = (prow * H * W + xcol) if pq < w4 else 0
+                x_off0 = xcol if pq < w4 else 0
                 for r in range(pl["PR"]):
                     iy = iy0 + r
                     if not (0 <= iy < H): continue
@@ -74,7 +78,7 @@ def wgrad_loads_in_bounds(B, Cin, H, W, Cout, st, pd):
                         a = xsrc + ((cu * RPP if pass_in else 0) * H + iy) * W + (x_off if ok else x_off0)
                         assert 0 <= a and a + 4 <= xsize, ("x", (B, Cin, H, W, Cout, st, pd), a, xsize)
                         if ok and pq < w4:  # the plane read is the one the lane parks
-                            assert a == ((b * Cin + c0 + cu * RPP + prow) * H + iy) * W + 4 * pq
+                            assert a == ((b * Cin + c0 + cu * RPP + prow) * H + iy) * W + xcol and xcol + 4 <= W
     return "patch"
 
 CC, KK, WPITCH = 8, 9, 73
@@ -82,7 +86,7 @@ NXP_SHORT, NXP_TALL = 4, 10
 def _ceil_div(a, b): return (a + b - 1) // b
 def _odd_pitch_c(n): return (n + 30) // 32 * 32 + 1
 def fwd_plan(num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
-    if C % CC or W % 4 or W > 4 * LPR or sh > 8 or sw > 8: return None
+    if C % CC or W < 4 or W > 4 * LPR or sh > 8 or sw > 8: return None
     L, slots = OH * OW, 2 * num_cus
     best = None
     for wm, tn in [(4, 8), (4, 7), (4, 6), (4, 5), (4, 4), (2, 4), (2, 3), (2, 2), (1, 4), (1, 3), (1, 2)]:
@@ -90,7 +94,7 @@ def fwd_plan(num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
         tiles, mtiles = _ceil_div(L, np_), _ceil_div(M, bm)
         rows = min(OH, np_ // OW if np_ % OW == 0 else (np_ - 1) // OW + 2); PR = (rows - 1) * sh + 3
         tall_ok = wm <= 2 or tn <= 6
-        if PR > 2 * NXP_TALL or (PR > 2 * NXP_SHORT and not tall_ok) or mtiles * bm > M * 2: continue
+        if PR > 2 * NXP_TALL or (PR > 2 * NXP_SHORT and not tall_ok) or mtiles * bm > M * 2 or tiles * np_ > L * 2: continue
         cost = _ceil_div(B * tiles * mtiles, slots) * np_ * bm
         if best is None or cost < best[0]: best = (cost, wm, tn, PR, tiles)
     if best is None: return None
@@ -123,12 +127,15 @@ def fwd_loads_in_bounds(B, C, H, W, M, sh, sw, ph, pw):
                             a = wsrc + idx * 4
                             assert 0 <= a and a + 4 <= wbuf, ("w", a, wbuf)
                         pq, xc, rp = tid & 15, (tid >> 4) & 7, tid >> 7
-                        x_off = (xc * H * W + 4 * pq) if pq < (W >> 2) else 0
+                        x_off = (xc * H * W + min(4 * pq, W - 4)) if pq < ((W + 3) >> 2) else 0
                         for u in range(pl["NXP"]):
                             r = 2 * u + rp; iy = iy_base + r
                             if r < pl["PR"] and 0 <= iy < H:
                                 a = xsrc + iy * W + x_off
                                 assert 0 <= a and a + 4 <= xsize, ("x", (B, C, H, W, M), a, xsize)
+                                if pq < ((W + 3) >> 2):  # the four floats lie inside row iy of channel xc
+                                    row0 = ((b * C + ch * CC + xc) * H + iy) * W
+                                    assert row0 <= a and a + 4 <= row0 + W
     return "patch %dx%d ok" % (pl["WM"], pl["TN"])
 
 
@@ -136,7 +143,7 @@ def fwd_loads_in_bounds(B, C, H, W, M, sh, sw, ph, pw):
 SC_NPIX, SC_GP = 256, 257
 def smallc_plan(wgrad, B, C, H, W, Cout, sh, sw, ph, pw, OH, OW, num_cus=256):
     L = OH * OW
-    if W % 4 or sh > 8 or sw > 8 or ph > 8 or pw > 8: return None
+    if W < 4 or sh > 8 or sw > 8 or ph > 8 or pw > 8: return None
     if (C * 9 > 32 or L % 4) if wgrad else C > 4: return None
     rows = min(OH, SC_NPIX // OW if SC_NPIX % OW == 0 else (SC_NPIX - 1) // OW + 2)
     PR, PW = (rows - 1) * sh + 3, W + 2 * pw
@@ -153,13 +160,14 @@ def smallc_tap(C, PLANE, PW, k):
     c, t = divmod(k, 9); ky, kx = divmod(t, 3)
     return c * PLANE + ky * PW + kx
 def smallc_stage_in_bounds(pl, b, C, H, W, pw, iy0, xsize):
-    W4 = W // 4
+    W4 = (W + 3) // 4
     for i in range(C * pl["PR"] * W4):
         rc, q = divmod(i, W4); c, r = divmod(rc, pl["PR"])
+        q = min(4 * q, W - 4)
         iy = iy0 + r; ok = 0 <= iy < H
-        a = ((b * C + c) * H + (iy if ok else 0)) * W + 4 * q
+        a = ((b * C + c) * H + (iy if ok else 0)) * W + q
         assert 0 <= a and a + 4 <= xsize, ("x", a, xsize)
-        d = c * pl["PLANE"] + r * pl["PW"] + pw + 4 * q
+        d = c * pl["PLANE"] + r * pl["PW"] + pw + q
         assert 0 <= d and d + 4 <= C * pl["PLANE"], ("patch write", d)
 def smallc_loads_in_bounds(wgrad, B, C, H, W, Cout, st, pd):
     sh, sw = st; ph, pw = pd
@@ -224,6 +232,7 @@ SMALLC_SHAPES = [  # B, C, H, W, Cout, (sh, sw), (ph, pw)
     (2, 3, 32, 32, 32, (1, 1), (1, 1)), (2, 1, 28, 28, 8, (1, 1), (1, 1)), (3, 3, 9, 12, 40, (1, 1), (0, 0)),
     (2, 2, 17, 20, 33, (2, 2), (1, 1)), (2, 3, 7, 8, 5, (3, 1), (1, 1)), (1, 3, 40, 36, 64, (1, 1), (1, 1)),
     (1, 3, 66, 64, 16, (2, 2), (1, 1)), (2, 1, 5, 4, 70, (1, 1), (2, 2)), (1, 3, 19, 60, 8, (1, 1), (1, 1)),
+    (2, 3, 14, 14, 32, (1, 1), (1, 1)), (2, 1, 9, 7, 16, (1, 1), (1, 1)), (2, 3, 12, 30, 8, (1, 1), (1, 1)),
 ]
 
 
@@ -256,17 +265,20 @@ WGRAD_SHAPES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw): every wave layout, r
 ]
 FWD_SHAPES = [  # B, C, H, W, M, (sh, sw), (ph, pw): one per tile shape on a 256-CU device, ragged M, strides, paddings
     (2, 64, 28, 28, 64, (1, 1), (1, 1)), (2, 8, 6, 12, 60, (1, 1), (1, 1)), (3, 16, 8, 36, 120, (1, 1), (0, 0)),
-    (2, 24, 4, 8, 104, (1, 1), (2, 2)), (1, 8, 64, 64, 52, (1, 1), (1, 1)), (2, 16, 6, 16, 60, (2, 2), (1, 1)),
+    (2, 24, 6, 8, 104, (1, 1), (2, 2)), (1, 8, 64, 64, 52, (1, 1), (1, 1)), (2, 16, 15, 18, 60, (2, 2), (1, 1)),
     (2, 8, 9, 64, 128, (2, 1), (1, 1)), (128, 8, 8, 40, 120, (1, 1), (1, 1)), (32, 8, 56, 56, 64, (1, 1), (1, 1)),
     (16, 8, 56, 56, 120, (1, 1), (1, 1)), (128, 8, 8, 40, 250, (1, 1), (1, 1)), (96, 8, 12, 48, 384, (1, 1), (1, 1)),
     (32, 8, 56, 56, 120, (1, 1), (1, 1)), (128, 8, 16, 64, 120, (1, 1), (1, 1)),
     # strided layers: more than 8 patch rows under a tile
     (8, 32, 32, 32, 64, (2, 2), (1, 1)), (4, 64, 56, 56, 128, (2, 2), (1, 1)), (2, 16, 30, 40, 60, (2, 1), (1, 1)),
-    (2, 8, 17, 24, 128, (3, 3), (1, 1)), (64, 64, 56, 56, 128, (2, 2), (1, 1)),
+    (2, 8, 16, 34, 128, (3, 3), (1, 1)), (64, 64, 56, 56, 128, (2, 2), (1, 1)),
     # 32 output channels: one block of channels, four waves along the pixels
-    (256, 64, 32, 32, 32, (1, 1), (1, 1)), (3, 16, 9, 20, 30, (1, 1), (1, 1)), (64, 8, 16, 32, 32, (2, 1), (1, 1)), (2, 8, 6, 8, 27, (1, 1), (0, 0)),
+    (256, 64, 32, 32, 32, (1, 1), (1, 1)), (3, 16, 9, 20, 30, (1, 1), (1, 1)), (64, 8, 16, 32, 32, (2, 1), (1, 1)), (2, 8, 18, 10, 27, (1, 1), (0, 0)),
     # up to half of a tile's channel rows are padding
-    (2, 16, 8, 32, 16, (1, 1), (1, 1)), (2, 8, 12, 28, 40, (1, 1), (1, 1)), (128, 8, 56, 56, 72, (1, 1), (1, 1)), (3, 24, 9, 12, 17, (1, 1), (1, 1)),
+    (2, 16, 8, 32, 16, (1, 1), (1, 1)), (2, 8, 12, 28, 40, (1, 1), (1, 1)), (128, 8, 56, 56, 72, (1, 1), (1, 1)), (3, 24, 12, 12, 17, (1, 1), (1, 1)),
+    # row lengths that are not multiples of four floats
+    (3, 8, 14, 14, 64, (1, 1), (1, 1)), (2, 16, 10, 7, 32, (1, 1), (1, 1)), (2, 8, 9, 30, 128, (1, 1), (0, 0)), (2, 8, 15, 18, 40, (2, 2), (1, 1)),
+    (2, 8, 6, 63, 64, (1, 1), (1, 1)),
 ]
 
 
