@@ -329,7 +329,7 @@ inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 k
     } else {
         add(4, 1, 1);
     }
-    int best = 0;  // the most rows per stage that keep a stage within 64 pixels and max_pr patch rows
+    int best = 0;  // the most rows per stage that keep a stage within 64 pixels, max_pr patch rows and the LDS budget
     for (int k = 0; k < ncand && !best; ++k) {
         pl.WMO = cand[k][0]; pl.WC = cand[k][1]; pl.WK = cand[k][2];
         const i64 max_pr = pl.WC == 2 ? 3 : 4;
@@ -341,18 +341,19 @@ inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 k
         // (and with two output rows over five patch rows per stage: 0.063 against 0.053 ms there, 0.192 against 0.156 ms at
         // [128,64,56,56] -> 128 stride 2: a strided patch stages four input values per output pixel)
         if (best * ow < 24) best = 0;
+        if (!best) continue;
+        pl.R = best;
+        pl.PR = (int)((best - 1) * sh + kh);
+        pl.PW = (int)(W + 2 * pw);
+        pl.PLANE = odd_pitch(pl.PR * pl.PW);
+        pl.Kst = (int)(best * ow);
+        pl.GP = odd_pitch(pl.Kst);
+        pl.smem = ((size_t)pl.bm() * pl.GP + (size_t)pl.ct() * pl.PLANE + SLACK) * sizeof(float);
+        if (pl.WK > 1) pl.smem = std::max<size_t>(pl.smem, 4 * 16 * 64 * sizeof(float));  // the closing sum over the row segments
+        if (pl.smem > LDS_BUDGET) best = 0;  // 64 planes of 3 x 66 floats: the next layout holds 32 planes
     }
     if (!best) return pl;
     const i64 BM = pl.bm(), CT = pl.ct();
-    pl.R = best;
-    pl.PR = (int)((best - 1) * sh + kh);
-    pl.PW = (int)(W + 2 * pw);
-    pl.PLANE = odd_pitch(pl.PR * pl.PW);
-    pl.Kst = (int)(best * ow);
-    pl.GP = odd_pitch(pl.Kst);
-    pl.smem = ((size_t)BM * pl.GP + (size_t)CT * pl.PLANE + SLACK) * sizeof(float);
-    if (pl.WK > 1) pl.smem = std::max<size_t>(pl.smem, 4 * 16 * 64 * sizeof(float));  // the closing sum over the row segments
-    if (pl.smem > LDS_BUDGET) return pl;
     pl.stages = (int)(B * (oh / best));
     const i64 tiles = fx::ceil_div(Cin, CT) * fx::ceil_div(Cout, BM);
     const i64 want = (i64)num_cus * 2;

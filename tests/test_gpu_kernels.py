@@ -441,6 +441,8 @@ WGRAD_PATCH_CASES = [
     # input channels that do not fill the last block of 32 (their LDS planes stay zero)
     (2, 16, 8, 32, 32, (1, 1), (1, 1)), (3, 48, 8, 32, 30, (1, 1), (1, 1)), (2, 24, 12, 24, 20, (1, 1), (1, 1)), (2, 40, 6, 16, 13, (1, 1), (1, 1)),
     (1, 33, 8, 24, 16, (1, 1), (1, 1)), (2, 17, 6, 32, 32, (1, 1), (1, 1)), (3, 48, 8, 32, 64, (1, 1), (1, 1)),
+    # 64-wide rows with 64 x 64 channels (the 64-plane layout exceeds the LDS budget)
+    (2, 64, 8, 64, 64, (1, 1), (1, 1)), (2, 64, 8, 64, 32, (1, 1), (1, 1)),
     # strided layers (implicit GEMM)
     (3, 32, 32, 32, 64, (2, 2), (1, 1)), (2, 64, 56, 56, 128, (2, 2), (1, 1)), (2, 32, 16, 24, 70, (2, 1), (1, 1)),
     (2, 32, 13, 32, 48, (2, 2), (0, 1)),

@@ -31,6 +31,11 @@ def wgrad_plan(num_cus, B, Cin, H, W, Cout, sh, sw, ph, pw, oh, ow):
             if oh % R or R * ow > 64 or (R - 1) * sh + 3 > max_pr: continue
             if (R * ow) % 4 == 0: best = R
         if best * ow < 24: best = 0
+        if best:
+            PR = (best - 1) * sh + 3
+            smem = (BM * _odd_pitch_w(best * ow) + CT * _odd_pitch_w(PR * (W + 2 * pw)) + 64) * 4
+            if WK > 1: smem = max(smem, 4 * 16 * 64 * 4)
+            if smem > 72 * 1024: best = 0
         if best: break
     if not best: return None
     PR = (best - 1) * sh + 3
@@ -262,6 +267,8 @@ WGRAD_SHAPES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw): every wave layout, r
     # input channels that do not fill the last block of 32
     (2, 16, 8, 32, 32, (1, 1), (1, 1)), (3, 48, 8, 32, 30, (1, 1), (1, 1)), (2, 24, 12, 24, 20, (1, 1), (1, 1)), (2, 40, 6, 16, 13, (1, 1), (1, 1)),
     (1, 33, 8, 24, 16, (1, 1), (1, 1)), (2, 17, 6, 32, 32, (1, 1), (1, 1)),
+    # 64 x 64 channels at 64-wide rows: the 64-plane layout exceeds the LDS budget, the 32-plane one is taken
+    (2, 64, 8, 64, 64, (1, 1), (1, 1)), (2, 64, 8, 64, 32, (1, 1), (1, 1)),
 ]
 FWD_SHAPES = [  # B, C, H, W, M, (sh, sw), (ph, pw): one per tile shape on a 256-CU device, ragged M, strides, paddings
     (2, 64, 28, 28, 64, (1, 1), (1, 1)), (2, 8, 6, 12, 60, (1, 1), (1, 1)), (3, 16, 8, 36, 120, (1, 1), (0, 0)),
