@@ -37,6 +37,9 @@ struct Params {
     int PR, PW, PLANE, L, tpi, nchunks;
     int xcd_chunk;  // gridDim.x / 8 when that divides: workgroup ids go to the 8 XCDs round-robin, see the kernel
     FastDiv div_tpi, div_ow;
+    // small maps (MULTI): a tile holds nimg whole images, image i in patch rows [i * RPI, (i + 1) * RPI)
+    int nimg, RPI, B;
+    FastDiv div_L, div_rpi;
 };
 
 // Weight images: out[mt][ch][m][tap*8 + cc], zero in column 72 and in rows past the last output channel.
@@ -60,7 +63,9 @@ __global__ __launch_bounds__(256) void wimg_kernel(const float* __restrict__ w, 
     out[i] = v;
 }
 
-template <int WM, int TN, bool BIAS, int NXP>
+// MULTI: maps of at most 64 pixels.  A tile is then nimg whole images stacked in the patch, each with its own zero
+// rows above and below, so that the 128 pixels of the smallest tile are not mostly padding.
+template <int WM, int TN, bool BIAS, int NXP, bool MULTI = false>
 __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
     constexpr int BM = 32 * WM, WN = 4 / WM, NPIX = 32 * TN * WN;
     constexpr int WIMG = BM * WPITCH;             // floats in one weight image
@@ -73,9 +78,9 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
     // of an image (which share input rows) and the weight images meet in one L2
     int bx = blockIdx.x;
     if (p.xcd_chunk) bx = (bx & 7) * p.xcd_chunk + (bx >> 3);
-    const int b = (int)p.div_tpi.div((uint32_t)bx);
+    const int b = MULTI ? bx * p.nimg : (int)p.div_tpi.div((uint32_t)bx);  // (first) image of the tile
     const int wm = wave % WM, wn = wave / WM;
-    const int pix0 = (bx - b * p.tpi) * NPIX;
+    const int pix0 = MULTI ? 0 : (bx - b * p.tpi) * NPIX;
     const int wpix0 = pix0 + wn * 32 * TN;  // first pixel of this wave's columns
     const int m0 = blockIdx.y * BM;
     const int py0 = (int)p.div_ow.div((uint32_t)pix0);
@@ -86,8 +91,15 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int pi = wpix0 + j * 32 + l32;
-        const int py = (int)p.div_ow.div((uint32_t)pi), px = pi - py * p.OW;
-        boff[j] = (pi < p.L ? (py - py0) * p.sh * p.PW + px * p.sw : 0) + half * p.PLANE;
+        if constexpr (MULTI) {
+            const int img = (int)p.div_L.div((uint32_t)pi), rem = pi - img * p.L;
+            const int py = (int)p.div_ow.div((uint32_t)rem), px = rem - py * p.OW;
+            const bool valid = img < p.nimg && b + img < p.B;
+            boff[j] = (valid ? (img * p.RPI + py * p.sh) * p.PW + px * p.sw : 0) + half * p.PLANE;
+        } else {
+            const int py = (int)p.div_ow.div((uint32_t)pi), px = pi - py * p.OW;
+            boff[j] = (pi < p.L ? (py - py0) * p.sh * p.PW + px * p.sw : 0) + half * p.PLANE;
+        }
     }
     f32x16 acc[TN];
 #pragma unroll
@@ -119,9 +131,16 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
         const float* xsrc = xsrc0 + (i64)ch * CC * p.H * p.W;
 #pragma unroll
         for (int u = 0; u < NXP; ++u) {
-            const int r = 2 * u + rp, iy = iy_base + r;
-            if (r < p.PR && iy >= 0 && iy < p.H) xv[u] = ldg4(xsrc + (i64)iy * p.W, x_off);  // wave-uniform test
-            else xv[u] = zero4;
+            const int r = 2 * u + rp;
+            if constexpr (MULTI) {
+                const int img = (int)p.div_rpi.div((uint32_t)r), iy = r - img * p.RPI - p.ph;
+                if (r < p.PR && iy >= 0 && iy < p.H && b + img < p.B) xv[u] = ldg4(xsrc + ((i64)img * p.C * p.H + iy) * p.W, x_off);
+                else xv[u] = zero4;
+            } else {
+                const int iy = iy_base + r;
+                if (r < p.PR && iy >= 0 && iy < p.H) xv[u] = ldg4(xsrc + (i64)iy * p.W, x_off);  // wave-uniform test
+                else xv[u] = zero4;
+            }
         }
     };
     auto park = [&]() {
@@ -199,8 +218,16 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
     }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-        const int pi = wpix0 + j * 32 + l32;
-        if (pi < p.L) {
+        int pi = wpix0 + j * 32 + l32;
+        bool valid = pi < p.L;
+        float* oj = out;
+        if constexpr (MULTI) {
+            const int img = (int)p.div_L.div((uint32_t)pi);
+            valid = img < p.nimg && b + img < p.B;
+            pi -= img * p.L;
+            oj = out + (i64)(valid ? img : 0) * p.M * p.L;
+        }
+        if (valid) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int m = m0 + wm * 32 + igemm::Mfma<float>::row(e, lane);
@@ -210,7 +237,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
                         v = v + bv[e];
                         if (p.relu) v = v > 0.f ? v : 0.f;
                     }
-                    out[(i64)m * p.L + pi] = v;
+                    oj[(i64)m * p.L + pi] = v;
                 }
             }
         }
@@ -221,6 +248,7 @@ struct Plan {
     bool ok = false;
     int WM = 4, TN = 0, PR = 0, PW = 0, PLANE = 0, tpi = 0, mtiles = 0, nchunks = 0;
     bool tall = false;  // more than 8 patch rows: the NXP_TALL instantiation
+    int nimg = 0, RPI = 0;  // small maps: images per tile and patch rows per image (0: one image per tile)
     size_t smem = 0;
     int bm() const { return 32 * WM; }
     int npix() const { return 32 * TN * (4 / WM); }
@@ -235,6 +263,28 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
     Plan pl;
     if (kh != 3 || kw != 3 || C % CC != 0 || W < 4 || W > 4 * LPR || sh > 8 || sw > 8) return pl;
     const i64 L = OH * OW, slots = 2 * (i64)std::max(1, num_cus);
+    // Maps of at most 64 pixels: a 128-pixel tile takes as many whole images as fit its pixels and the 20 patch rows
+    // (8 x 8 and 7 x 7 maps: two images), provided that fills at least half of the tile.
+    const i64 RPI = (OH - 1) * sh + 3;
+    if (L <= 64 && B >= 2) {
+        const i64 nimg = std::min<i64>(std::min<i64>(128 / L, 2 * NXP_TALL / RPI), B);
+        const int wm = M > 64 ? 4 : 2;
+        const i64 bm = 32 * wm, mtiles = fx::ceil_div(M, bm);
+        if (nimg >= 2 && nimg * L >= 64 && mtiles * bm <= M * 2 && mtiles <= 65535) {
+            pl.WM = wm; pl.TN = wm == 4 ? 4 : 2;
+            pl.nimg = (int)nimg; pl.RPI = (int)RPI;
+            pl.PR = (int)(nimg * RPI);
+            pl.tall = true;
+            pl.tpi = 1;
+            pl.PW = (int)(W + 2 * pw);
+            pl.PLANE = wgp::odd_pitch(pl.PR * pl.PW);
+            pl.smem = ((size_t)pl.wimg() + (size_t)CC * pl.PLANE + SLACK) * sizeof(float);
+            pl.mtiles = (int)mtiles;
+            pl.nchunks = (int)(C / CC);
+            pl.ok = pl.smem <= LDS_BUDGET;
+            return pl;
+        }
+    }
     static const int shapes[11][2] = {{4, 8}, {4, 7}, {4, 6}, {4, 5}, {4, 4}, {2, 4}, {2, 3}, {2, 2}, {1, 4}, {1, 3}, {1, 2}};
     i64 best_cost = -1;
     for (const auto& sp : shapes) {
@@ -284,8 +334,29 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
     p.PR = pl.PR; p.PW = pl.PW; p.PLANE = pl.PLANE; p.L = (int)(OH * OW); p.tpi = pl.tpi; p.nchunks = pl.nchunks;
     p.div_tpi = FastDiv((uint32_t)pl.tpi);
     p.div_ow = FastDiv((uint32_t)OW);
-    const dim3 grid((unsigned)(B * pl.tpi), (unsigned)pl.mtiles);
-    p.xcd_chunk = (B * pl.tpi) % 8 == 0 ? (int)(B * pl.tpi / 8) : 0;
+    p.nimg = pl.nimg; p.RPI = pl.RPI; p.B = (int)B;
+    p.div_L = FastDiv((uint32_t)(OH * OW));
+    p.div_rpi = FastDiv((uint32_t)std::max(1, pl.RPI));
+    const i64 gx = pl.nimg ? fx::ceil_div(B, (i64)pl.nimg) : B * pl.tpi;
+    const dim3 grid((unsigned)gx, (unsigned)pl.mtiles);
+    p.xcd_chunk = gx % 8 == 0 ? (int)(gx / 8) : 0;
+    if (pl.nimg) {
+#define FX_CPK_LAUNCH_MULTI(WMV, TNV)                                                                                \
+    {                                                                                                                 \
+        static const hipError_t attr0 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, false, NXP_TALL, true>, \
+                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
+        static const hipError_t attr1 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, true, NXP_TALL, true>, \
+                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
+        FX_HIP_CHECK(attr0);                                                                                          \
+        FX_HIP_CHECK(attr1);                                                                                          \
+        if (bias) conv_patch_kernel<WMV, TNV, true, NXP_TALL, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);       \
+        else conv_patch_kernel<WMV, TNV, false, NXP_TALL, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);           \
+    }
+        if (pl.WM == 4) FX_CPK_LAUNCH_MULTI(4, 4) else FX_CPK_LAUNCH_MULTI(2, 2)
+#undef FX_CPK_LAUNCH_MULTI
+        FX_LAUNCH_CHECK();
+        return FX_OK;
+    }
 #define FX_CPK_LAUNCH_N(WMV, TNV, NXPV)                                                                              \
     {                                                                                                                 \
         static const hipError_t attr0 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, false, NXPV>,    \

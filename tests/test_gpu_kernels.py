@@ -507,6 +507,9 @@ CONV_PATCH_CASES = [
     # row lengths that are not multiples of four floats (the last vector of a row is moved back to end with the row)
     (3, 8, 14, 14, 64, (1, 1), (1, 1)), (2, 16, 10, 7, 32, (1, 1), (1, 1)), (2, 8, 9, 30, 128, (1, 1), (0, 0)), (2, 8, 15, 18, 40, (2, 2), (1, 1)),
     (2, 8, 6, 63, 64, (1, 1), (1, 1)), (64, 64, 14, 14, 128, (1, 1), (1, 1)),
+    # maps of at most 64 pixels: whole images stacked in one tile (odd batches: the last tile holds one image)
+    (5, 16, 8, 8, 128, (1, 1), (1, 1)), (3, 8, 7, 7, 64, (1, 1), (1, 1)), (7, 8, 6, 6, 40, (1, 1), (1, 1)), (4, 8, 6, 10, 200, (1, 1), (0, 1)),
+    (33, 64, 8, 8, 64, (1, 1), (1, 1)), (9, 16, 8, 8, 100, (1, 1), (0, 0)),
 ]
 
 

@@ -93,6 +93,16 @@ def _odd_pitch_c(n): return (n + 30) // 32 * 32 + 1
 def fwd_plan(num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
     if C % CC or W < 4 or W > 4 * LPR or sh > 8 or sw > 8: return None
     L, slots = OH * OW, 2 * num_cus
+    RPI = (OH - 1) * sh + 3
+    if L <= 64 and B >= 2:  # small maps: whole images stacked in one tile
+        nimg = min(128 // L, 2 * NXP_TALL // RPI, B)
+        wm = 4 if M > 64 else 2
+        bm = 32 * wm; mtiles = _ceil_div(M, bm)
+        if nimg >= 2 and nimg * L >= 64 and mtiles * bm <= M * 2:
+            PR = nimg * RPI; PW = W + 2 * pw; PLANE = _odd_pitch_c(PR * PW)
+            if (bm * WPITCH + CC * PLANE + 16) * 4 > 72 * 1024: return None
+            return dict(WM=wm, TN=4 if wm == 4 else 2, PR=PR, tpi=1, mtiles=mtiles, nchunks=C // CC, BM=bm, NPIX=128, NXP=NXP_TALL,
+                        nimg=nimg, RPI=RPI, PW=PW, PLANE=PLANE)
     best = None
     for wm, tn in [(4, 8), (4, 7), (4, 6), (4, 5), (4, 4), (2, 4), (2, 3), (2, 2), (1, 4), (1, 3), (1, 2)]:
         bm, np_ = 32 * wm, 32 * tn * (4 // wm)
@@ -110,10 +120,35 @@ def fwd_plan(num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
     if smem > 72 * 1024: return None
     return dict(WM=wm, TN=tn, PR=PR, tpi=tiles, mtiles=_ceil_div(M, bm), nchunks=C // CC, BM=bm, NPIX=32 * tn * (4 // wm),
                 NXP=NXP_TALL if PR > 2 * NXP_SHORT else NXP_SHORT)
+def fwd_multi_loads_in_bounds(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
+    L, xsize, ysize = OH * OW, B * C * H * W, B * M * OH * OW
+    nimg, RPI, PR, PW = pl["nimg"], pl["RPI"], pl["PR"], pl["PW"]
+    for bx in range(_ceil_div(B, nimg)):
+        b0 = bx * nimg
+        for ch in range(pl["nchunks"]):
+            for tid in range(NT):
+                pq, xc, rp = tid & 15, (tid >> 4) & 7, tid >> 7
+                lane_in = pq < ((W + 3) >> 2)
+                x_off = (xc * H * W + min(4 * pq, W - 4)) if lane_in else 0
+                for u in range(pl["NXP"]):
+                    r = 2 * u + rp; img = r // RPI; iy = r - img * RPI - ph
+                    if r < PR and 0 <= iy < H and b0 + img < B:
+                        a = (b0 * C + ch * CC) * H * W + (img * C * H + iy) * W + x_off
+                        assert 0 <= a and a + 4 <= xsize, ("x", a, xsize)
+                        if lane_in:
+                            row0 = (((b0 + img) * C + ch * CC + xc) * H + iy) * W
+                            assert row0 <= a and a + 4 <= row0 + W
+        for pi in range(pl["NPIX"]):  # LDS offsets of the pixels and the addresses they are stored to
+            img, rem = divmod(pi, L); py, px = divmod(rem, OW)
+            if img < nimg and b0 + img < B:
+                assert (img * RPI + py * sh + 2) * PW + px * sw + 2 < PR * PW <= pl["PLANE"]
+                assert ((b0 + img) * M + (M - 1)) * L + rem < ysize
+    return "patch multi %dx%d ok" % (pl["WM"], pl["TN"])
 def fwd_loads_in_bounds(B, C, H, W, M, sh, sw, ph, pw):
     OH, OW = (H + 2 * ph - 3) // sh + 1, (W + 2 * pw - 3) // sw + 1
     pl = fwd_plan(256, B, C, H, W, M, OH, OW, sh, sw, ph, pw)
     if pl is None: return "generic"
+    if pl.get("nimg"): return fwd_multi_loads_in_bounds(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw)
     WIMG = pl["BM"] * WPITCH
     NW = (WIMG // 4 + NT - 1) // NT
     wbuf = pl["mtiles"] * pl["nchunks"] * WIMG          # floats written by wimg_kernel
@@ -286,6 +321,9 @@ FWD_SHAPES = [  # B, C, H, W, M, (sh, sw), (ph, pw): one per tile shape on a 256
     # row lengths that are not multiples of four floats
     (3, 8, 14, 14, 64, (1, 1), (1, 1)), (2, 16, 10, 7, 32, (1, 1), (1, 1)), (2, 8, 9, 30, 128, (1, 1), (0, 0)), (2, 8, 15, 18, 40, (2, 2), (1, 1)),
     (2, 8, 6, 63, 64, (1, 1), (1, 1)),
+    # maps of at most 64 pixels: whole images stacked in one tile (odd batch: the last tile holds one image)
+    (5, 16, 8, 8, 128, (1, 1), (1, 1)), (3, 8, 7, 7, 64, (1, 1), (1, 1)), (7, 8, 6, 6, 40, (1, 1), (1, 1)), (4, 8, 6, 10, 200, (1, 1), (0, 1)),
+    (5, 8, 16, 16, 64, (2, 2), (1, 1)), (2, 8, 8, 8, 33, (1, 1), (2, 2)),
 ]
 
 
