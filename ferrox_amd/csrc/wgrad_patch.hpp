@@ -92,7 +92,10 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
     const uint32_t g_off = g_lane ? (uint32_t)(prow * L + 4 * pq) * 4u : 0u;
     const uint32_t x_off = x_lane ? (uint32_t)(prow * p.H * p.W + 4 * pq) * 4u : 0u;
     const uint32_t x_off0 = x_lane ? (uint32_t)(4 * pq) * 4u : 0u;  // the same columns in the first plane of a pass
-    const bool full_c = c0 + CT <= p.Cin;
+    // ragged input-channel counts come only with the one-channel-block layouts; elsewhere this folds to a constant and the
+    // staging code carries no channel tests (they cost the 128-row layout a fifth of its speed in registers)
+    constexpr bool RAGGED_C = WMO == 1;
+    const bool full_c = !RAGGED_C || c0 + CT <= p.Cin;
     const int g_dst0 = prow * p.GP + 4 * pq;
     const int x_dst0 = BM * p.GP + prow * p.PLANE + p.pw + 4 * pq;
     auto prefetch = [&](int s) {
@@ -236,7 +239,7 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             const int oc = oc0 + wmo * 32 + igemm::Mfma<float>::row(e, lane);
-            if (oc < p.Cout && c0 + wc * 32 + l32 < p.Cin) out[(i64)oc * ldo + t * p.Cin + c0 + wc * 32 + l32] = acc[t][e];
+            if (oc < p.Cout && (!RAGGED_C || c0 + wc * 32 + l32 < p.Cin)) out[(i64)oc * ldo + t * p.Cin + c0 + wc * 32 + l32] = acc[t][e];
         }
 }
 
