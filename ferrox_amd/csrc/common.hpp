@@ -1,7 +1,9 @@
 // Shared internals of libferrox_hip.so: context object, error reporting, launch helpers.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <array>
 #include <cstdint>
+#include <map>
 #include <cstdio>
 #include <mutex>
 #include <string>
@@ -68,6 +70,9 @@ struct fx_ctx {
     void* scratch = nullptr;
     i64 scratch_bytes = 0;
     std::mutex launch_mutex;
+    // tile shape that measured fastest per convolution layer shape (conv_patch.hpp); used under launch_mutex
+    std::map<std::array<i64, 14>, int> conv_tile_cache;
+    hipEvent_t ev_tune[2] = {nullptr, nullptr};
     // returns a scratch region of at least `bytes` (256-byte aligned); nullptr + error on failure
     void* get_scratch(i64 bytes);
 };

@@ -13,6 +13,9 @@
 // staging is a straight 16-byte copy; the patch rows use the regular thread-to-row map of the weight-gradient
 // kernel.  The next stage's global loads are issued before the MFMA loop of the current one.
 #pragma once
+#include <array>
+#include <cstdlib>
+
 #include "wgrad_patch.hpp"
 
 namespace cpk {
@@ -249,11 +252,37 @@ struct Plan {
     int WM = 4, TN = 0, PR = 0, PW = 0, PLANE = 0, tpi = 0, mtiles = 0, nchunks = 0;
     bool tall = false;  // more than 8 patch rows: the NXP_TALL instantiation
     int nimg = 0, RPI = 0;  // small maps: images per tile and patch rows per image (0: one image per tile)
+    i64 cost = 0;           // modelled cost: rounds of co-resident blocks x MFMA work of a block
     size_t smem = 0;
     int bm() const { return 32 * WM; }
     int npix() const { return 32 * TN * (4 / WM); }
     i64 wimg() const { return (i64)bm() * WPITCH; }
 };
+
+// The plan for one tile shape (wm x tn); false when the shape does not fit this layer.
+inline bool shape_plan(Plan& pl, int wm, int tn, int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph,
+                       i64 pw) {
+    const i64 L = OH * OW, slots = 2 * (i64)std::max(1, num_cus);
+    const i64 bm = 32 * wm, np = 32 * tn * (4 / wm), tiles = fx::ceil_div(L, np), mtiles = fx::ceil_div(M, bm);
+    // output rows under a tile: tiles that start on a row boundary cover exactly np / OW rows
+    const i64 rows = std::min<i64>(OH, np % OW == 0 ? np / OW : (np - 1) / OW + 2), PR = (rows - 1) * sh + 3;
+    const bool tall_ok = wm <= 2 || tn <= 6;  // instantiated tall variants
+    // at most half of the channel rows and half of the pixels of an image's tiles may be padding (measured at 7 x 7 maps,
+    // 49 pixels under a 128-pixel tile: 0.084 ms against 0.061 ms for the implicit GEMM at [256,128,7,7] -> 128)
+    if (PR > 2 * NXP_TALL || (PR > 2 * NXP_SHORT && !tall_ok) || mtiles * bm > M * 2 || tiles * np > L * 2) return false;
+    pl = Plan();
+    pl.WM = wm; pl.TN = tn; pl.PR = (int)PR; pl.tpi = (int)tiles;
+    pl.cost = fx::ceil_div(B * tiles * mtiles, slots) * np * bm;
+    pl.tall = pl.PR > 2 * NXP_SHORT;
+    pl.PW = (int)(W + 2 * pw);
+    pl.PLANE = wgp::odd_pitch(pl.PR * pl.PW);
+    pl.smem = ((size_t)pl.wimg() + (size_t)CC * pl.PLANE + SLACK) * sizeof(float);
+    pl.mtiles = (int)mtiles;
+    pl.nchunks = (int)(C / CC);
+    if (pl.smem > LDS_BUDGET || B * pl.tpi > 0x7fffffff || pl.mtiles > 65535) return false;
+    pl.ok = true;
+    return true;
+}
 
 // C input channels of H x W, M output channels of OH x OW (already the dimensions of the pass that runs).
 // Among the tile shapes whose patch fits, takes the one with the least (rounds of co-resident blocks) x (work of
@@ -262,7 +291,7 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
                       i64 pw) {
     Plan pl;
     if (kh != 3 || kw != 3 || C % CC != 0 || W < 4 || W > 4 * LPR || sh > 8 || sw > 8) return pl;
-    const i64 L = OH * OW, slots = 2 * (i64)std::max(1, num_cus);
+    const i64 L = OH * OW;
     // Maps of at most 64 pixels: a 128-pixel tile takes as many whole images as fit its pixels and the 20 patch rows
     // (8 x 8 and 7 x 7 maps: two images), provided that fills at least half of the tile.
     const i64 RPI = (OH - 1) * sh + 3;
@@ -286,43 +315,39 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
         }
     }
     static const int shapes[11][2] = {{4, 8}, {4, 7}, {4, 6}, {4, 5}, {4, 4}, {2, 4}, {2, 3}, {2, 2}, {1, 4}, {1, 3}, {1, 2}};
-    i64 best_cost = -1;
+    Plan best;
     for (const auto& sp : shapes) {
-        const int wm = sp[0], tn = sp[1];
-        const i64 bm = 32 * wm, np = 32 * tn * (4 / wm), tiles = fx::ceil_div(L, np), mtiles = fx::ceil_div(M, bm);
-        // output rows under a tile: tiles that start on a row boundary cover exactly np / OW rows
-        const i64 rows = std::min<i64>(OH, np % OW == 0 ? np / OW : (np - 1) / OW + 2), PR = (rows - 1) * sh + 3;
-        const bool tall_ok = wm <= 2 || tn <= 6;  // instantiated tall variants
-        // at most half of the channel rows and half of the pixels of an image's tiles may be padding (measured at 7 x 7 maps,
-        // 49 pixels under a 128-pixel tile: 0.084 ms against 0.061 ms for the implicit GEMM at [256,128,7,7] -> 128)
-        if (PR > 2 * NXP_TALL || (PR > 2 * NXP_SHORT && !tall_ok) || mtiles * bm > M * 2 || tiles * np > L * 2) continue;
-        const i64 cost = fx::ceil_div(B * tiles * mtiles, slots) * np * bm;
-        if (best_cost < 0 || cost < best_cost) {
-            best_cost = cost;
-            pl.WM = wm;
-            pl.TN = tn;
-            pl.PR = (int)PR;
-            pl.tpi = (int)tiles;
-        }
+        Plan q;
+        if (shape_plan(q, sp[0], sp[1], num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw) && (!best.ok || q.cost < best.cost)) best = q;
     }
-    if (best_cost < 0) return pl;
-    pl.tall = pl.PR > 2 * NXP_SHORT;
-    pl.PW = (int)(W + 2 * pw);
-    pl.PLANE = wgp::odd_pitch(pl.PR * pl.PW);
-    pl.smem = ((size_t)pl.wimg() + (size_t)CC * pl.PLANE + SLACK) * sizeof(float);
-    pl.mtiles = (int)fx::ceil_div(M, (i64)pl.bm());
-    pl.nchunks = (int)(C / CC);
-    if (pl.smem > LDS_BUDGET || B * pl.tpi > 0x7fffffff || pl.mtiles > 65535) return pl;
-    pl.ok = true;
-    return pl;
+    return best;
+}
+
+// Every tile shape whose modelled cost is within 1.5 x of the best one: the candidates that run() times once per layer
+// shape (the model counts MFMA work and rounds of blocks; staging, weight-image size and LDS traffic per MFMA differ
+// between shapes by more than that: measured spreads of 25 % and more between shapes of equal modelled cost).
+inline int candidates(Plan (&out)[11], int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw) {
+    static const int shapes[11][2] = {{4, 8}, {4, 7}, {4, 6}, {4, 5}, {4, 4}, {2, 4}, {2, 3}, {2, 2}, {1, 4}, {1, 3}, {1, 2}};
+    Plan all[11];
+    int n = 0;
+    i64 best = -1;
+    for (const auto& sp : shapes)
+        if (shape_plan(all[n], sp[0], sp[1], num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw)) {
+            if (best < 0 || all[n].cost < best) best = all[n].cost;
+            ++n;
+        }
+    int m = 0;
+    for (int k = 0; k < n; ++k)
+        if (all[k].cost * 2 <= best * 3) out[m++] = all[k];
+    return m;
 }
 
 // Sized for 128-row images whatever tile was picked, so the figure does not depend on the CU count behind the plan.
 inline i64 workspace_bytes(const Plan& pl, i64 M) { return fx::ceil_div(M, (i64)128) * 128 * WPITCH * pl.nchunks * (i64)sizeof(float); }
 
 // w is the reference's [Cout][Cin][3][3] filter; flip selects the data-gradient image.
-inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float* y, float* wimg, int flip, i64 Cout, i64 Cin, i64 B,
-               i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw, const float* bias = nullptr, int relu = 0) {
+inline int launch_plan(fx_ctx* c, const Plan& pl, const float* x, const float* w, float* y, float* wimg, int flip, i64 Cout, i64 Cin, i64 B,
+                       i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw, const float* bias, int relu) {
     const i64 n = (i64)pl.mtiles * pl.nchunks * pl.wimg();
     wimg_kernel<<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(w, wimg, (int)Cout, (int)Cin, (int)M, pl.bm(),
                                                                                   pl.nchunks, flip, n);
@@ -396,6 +421,52 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
 #undef FX_CPK_LAUNCH
     FX_LAUNCH_CHECK();
     return FX_OK;
+}
+
+// Runs the layer with the tile shape that measured fastest for this layer shape on this device.  The first call for a
+// shape times the candidate shapes (each writes the same, complete output: the order of every output's sum does not depend
+// on the tile shape) and remembers the winner in the context; FX_CONV_TUNE=0 keeps the modelled choice.
+inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float* y, float* wimg, int flip, i64 Cout, i64 Cin, i64 B,
+               i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw, const float* bias = nullptr, int relu = 0) {
+    static const bool tune = [] { const char* v = getenv("FX_CONV_TUNE"); return !(v && atoi(v) == 0); }();
+    if (!tune || pl.nimg) return launch_plan(c, pl, x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu);
+    const std::array<i64, 14> key = {flip, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias ? 1 : 0, relu};
+    Plan cand[11];
+    const int n = candidates(cand, c->num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw);
+    auto it = c->conv_tile_cache.find(key);
+    if (it == c->conv_tile_cache.end()) {
+        int best = -1;
+        if (n > 1) {
+            if (!c->ev_tune[0]) {
+                FX_HIP_CHECK(hipEventCreate(&c->ev_tune[0]));
+                FX_HIP_CHECK(hipEventCreate(&c->ev_tune[1]));
+            }
+            // the modelled choice stays unless another shape is at least 3 % faster (timer noise between equals)
+            int model = 0;
+            for (int k = 1; k < n; ++k)
+                if (cand[k].cost < cand[model].cost) model = k;
+            float ms_of[11];
+            for (int k = 0; k < n; ++k) {
+                if (int rc = launch_plan(c, cand[k], x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu)) return rc;
+                FX_HIP_CHECK(hipEventRecord(c->ev_tune[0], c->stream));
+                for (int rep = 0; rep < 3; ++rep)
+                    if (int rc = launch_plan(c, cand[k], x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu)) return rc;
+                FX_HIP_CHECK(hipEventRecord(c->ev_tune[1], c->stream));
+                FX_HIP_CHECK(hipEventSynchronize(c->ev_tune[1]));
+                FX_HIP_CHECK(hipEventElapsedTime(&ms_of[k], c->ev_tune[0], c->ev_tune[1]));
+            }
+            best = model;
+            for (int k = 0; k < n; ++k)
+                if (ms_of[k] < 0.97f * ms_of[best]) best = k;
+        }
+        const int code = best >= 0 ? cand[best].WM * 16 + cand[best].TN : pl.WM * 16 + pl.TN;
+        it = c->conv_tile_cache.emplace(key, code).first;
+        if (best >= 0 && best == n - 1) return FX_OK;  // the last candidate timed is the winner: its output stands
+    }
+    for (int k = 0; k < n; ++k)
+        if (cand[k].WM * 16 + cand[k].TN == it->second)
+            return launch_plan(c, cand[k], x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu);
+    return launch_plan(c, pl, x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu);
 }
 
 }  // namespace cpk

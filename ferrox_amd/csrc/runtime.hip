@@ -94,6 +94,8 @@ int fx_destroy(fx_ctx* c) {
     if (c->scratch) (void)hipFree(c->scratch);
     (void)hipEventDestroy(c->ev_start);
     (void)hipEventDestroy(c->ev_stop);
+    for (hipEvent_t e : c->ev_tune)
+        if (e) (void)hipEventDestroy(e);
     (void)hipStreamDestroy(c->stream);
     delete c;
     return FX_OK;

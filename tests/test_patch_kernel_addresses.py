@@ -101,25 +101,21 @@ def fwd_plan(num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
         if nimg >= 2 and nimg * L >= 64 and mtiles * bm <= M * 2:
             PR = nimg * RPI; PW = W + 2 * pw; PLANE = _odd_pitch_c(PR * PW)
             if (bm * WPITCH + CC * PLANE + 16) * 4 > 72 * 1024: return None
-            return dict(WM=wm, TN=4 if wm == 4 else 2, PR=PR, tpi=1, mtiles=mtiles, nchunks=C // CC, BM=bm, NPIX=128, NXP=NXP_TALL,
-                        nimg=nimg, RPI=RPI, PW=PW, PLANE=PLANE)
-    best = None
+            return [dict(WM=wm, TN=4 if wm == 4 else 2, PR=PR, tpi=1, mtiles=mtiles, nchunks=C // CC, BM=bm, NPIX=128, NXP=NXP_TALL,
+                         nimg=nimg, RPI=RPI, PW=PW, PLANE=PLANE, cost=0)]
+    plans = []
     for wm, tn in [(4, 8), (4, 7), (4, 6), (4, 5), (4, 4), (2, 4), (2, 3), (2, 2), (1, 4), (1, 3), (1, 2)]:
         bm, np_ = 32 * wm, 32 * tn * (4 // wm)
         tiles, mtiles = _ceil_div(L, np_), _ceil_div(M, bm)
         rows = min(OH, np_ // OW if np_ % OW == 0 else (np_ - 1) // OW + 2); PR = (rows - 1) * sh + 3
         tall_ok = wm <= 2 or tn <= 6
         if PR > 2 * NXP_TALL or (PR > 2 * NXP_SHORT and not tall_ok) or mtiles * bm > M * 2 or tiles * np_ > L * 2: continue
+        PW = W + 2 * pw; PLANE = _odd_pitch_c(PR * PW)
+        if (bm * WPITCH + CC * PLANE + 16) * 4 > 72 * 1024: continue
         cost = _ceil_div(B * tiles * mtiles, slots) * np_ * bm
-        if best is None or cost < best[0]: best = (cost, wm, tn, PR, tiles)
-    if best is None: return None
-    _, wm, tn, PR, tiles = best
-    PW = W + 2 * pw; PLANE = _odd_pitch_c(PR * PW)
-    bm = 32 * wm
-    smem = (bm * WPITCH + CC * PLANE + 16) * 4
-    if smem > 72 * 1024: return None
-    return dict(WM=wm, TN=tn, PR=PR, tpi=tiles, mtiles=_ceil_div(M, bm), nchunks=C // CC, BM=bm, NPIX=32 * tn * (4 // wm),
-                NXP=NXP_TALL if PR > 2 * NXP_SHORT else NXP_SHORT)
+        plans.append(dict(WM=wm, TN=tn, PR=PR, tpi=tiles, mtiles=mtiles, nchunks=C // CC, BM=bm, NPIX=np_, cost=cost,
+                          NXP=NXP_TALL if PR > 2 * NXP_SHORT else NXP_SHORT))
+    return plans or None
 def fwd_multi_loads_in_bounds(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
     L, xsize, ysize = OH * OW, B * C * H * W, B * M * OH * OW
     nimg, RPI, PR, PW = pl["nimg"], pl["RPI"], pl["PR"], pl["PW"]
@@ -146,8 +142,11 @@ def fwd_multi_loads_in_bounds(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
     return "patch multi %dx%d ok" % (pl["WM"], pl["TN"])
 def fwd_loads_in_bounds(B, C, H, W, M, sh, sw, ph, pw):
     OH, OW = (H + 2 * ph - 3) // sh + 1, (W + 2 * pw - 3) // sw + 1
-    pl = fwd_plan(256, B, C, H, W, M, OH, OW, sh, sw, ph, pw)
-    if pl is None: return "generic"
+    plans = fwd_plan(256, B, C, H, W, M, OH, OW, sh, sw, ph, pw)
+    if plans is None: return "generic"
+    # every tile shape that fits is walked: the library times the candidates once per layer shape and keeps the fastest
+    return " ".join(fwd_shape_loads_in_bounds(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw) for pl in plans)
+def fwd_shape_loads_in_bounds(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
     if pl.get("nimg"): return fwd_multi_loads_in_bounds(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw)
     WIMG = pl["BM"] * WPITCH
     NW = (WIMG // 4 + NT - 1) // NT
