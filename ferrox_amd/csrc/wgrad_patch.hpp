@@ -45,17 +45,23 @@ struct Params {
     int R, PW, PLANE, GP, Kst;  // rows per stage, patch width, plane pitch, g pitch, pixels per stage
     int stages, sps, spi;       // all stages, stages per split, stages per image
     int xcd_chunk;              // blocks / 8 when that divides (see the kernel), else 0
-    FastDiv div_spi;
+    int XRn;                    // NARROW kernels: patch rows per stage (a whole image)
+    FastDiv div_spi, div_xr;
     i64 part_stride;
 };
 
 // XR = patch rows per stage = (R - 1) * sh + 3; WMO x WC x WK = wave layout (see the top of the file).
-template <int XR, int WMO, int WC, int WK>
+// NARROW (maps of at most 64 pixels with rows of at most 16 floats, XR unused): a stage is one whole image, and the patch is
+// staged by (channel, row) pairs, 4 lanes per row and 64 pairs per pass, instead of 16 lanes per row: with 8-float rows
+// the regular map would leave 14 of 16 lanes idle and could hold only 4 of the image's 10 patch rows.
+template <int XR, int WMO, int WC, int WK, bool NARROW = false>
 __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
     static_assert(WMO * WC * WK == 4, "four waves");
+    static_assert(!NARROW || WC == 1, "narrow staging holds 32 channel planes");
     constexpr int BM = 32 * WMO, CT = 32 * WC;
     constexpr int NG = BM / RPP, NXC = CT / RPP;
-    constexpr int NX = NXC * XR;
+    constexpr int NXN = 5;  // NARROW: passes of 64 (channel, row) pairs; 32 channels x at most 10 rows
+    constexpr int NX = NARROW ? NXN : NXC * XR;
     extern __shared__ __align__(16) float smem[];
     float* Gs = smem;
     float* Xs = smem + BM * p.GP;
@@ -92,12 +98,16 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
     const uint32_t g_off = g_lane ? (uint32_t)(prow * L + 4 * pq) * 4u : 0u;
     const uint32_t x_off = x_lane ? (uint32_t)(prow * p.H * p.W + 4 * pq) * 4u : 0u;
     const uint32_t x_off0 = x_lane ? (uint32_t)(4 * pq) * 4u : 0u;  // the same columns in the first plane of a pass
-    // ragged input-channel counts come only with the one-channel-block layouts; elsewhere this folds to a constant and the
+    // ragged input-channel counts come only with the 1 x 1 x 4 layout; elsewhere this folds to a constant and the
     // staging code carries no channel tests (they cost the 128-row layout a fifth of its speed in registers)
-    constexpr bool RAGGED_C = WMO == 1;
+    constexpr bool RAGGED_C = WMO == 1 && WC == 1;  // 1 x 1 x 4: the only layout the planner gives ragged counts to
     const bool full_c = !RAGGED_C || c0 + CT <= p.Cin;
     const int g_dst0 = prow * p.GP + 4 * pq;
     const int x_dst0 = BM * p.GP + prow * p.PLANE + p.pw + 4 * pq;
+    // NARROW: float4 column and first (channel, row) pair of this thread
+    const int npq = tid & 3, npp = tid >> 2;
+    const bool nx_lane = npq < ((p.W + 3) >> 2);
+    const int nxcol = min(4 * npq, p.W - 4), npairs = CT * p.XRn;
     auto prefetch = [&](int s) {
         const int b = (int)p.div_spi.div((uint32_t)s);
         const int oy0 = (s - b * p.spi) * p.R;
@@ -112,8 +122,17 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
             const bool ok = full_m || oc0 + prow + u * RPP < p.Cout;
             gv[u] = ldg4(pass_in ? gsrc + (i64)u * RPP * L : gsrc, ok ? g_off : 0u);
         }
+        if constexpr (NARROW) {
 #pragma unroll
-        for (int r = 0; r < XR; ++r) {
+            for (int u = 0; u < NXN; ++u) {
+                const int pair = u * 64 + npp;
+                const int c = (int)p.div_xr.div((uint32_t)pair), iy = iy0 + pair - c * p.XRn;
+                const bool ok = nx_lane && pair < npairs && iy >= 0 && iy < p.H && (full_c || c0 + c < p.Cin);
+                xv[u] = ldg4(xsrc, ok ? (uint32_t)((c * p.H + iy) * p.W + nxcol) * 4u : 0u);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < (NARROW ? 0 : XR); ++r) {
             const int iy = iy0 + r;
             const bool row_ok = iy >= 0 && iy < p.H;  // wave-uniform
 #pragma unroll
@@ -139,7 +158,21 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
                 d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
             }
         }
-        if (x_lane) {
+        if constexpr (NARROW) {
+            if (nx_lane) {
+#pragma unroll
+                for (int u = 0; u < NXN; ++u) {
+                    const int pair = u * 64 + npp;
+                    const int c = (int)p.div_xr.div((uint32_t)pair), r = pair - c * p.XRn, iy = r - p.ph;
+                    if (pair < npairs && (full_c || c0 + c < p.Cin)) {  // rows above and below the image are written as zeros
+                        const float4 v = iy >= 0 && iy < p.H ? xv[u] : zero4;
+                        float* d = Xs + c * p.PLANE + r * p.PW + p.pw + nxcol;
+                        d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+                    }
+                }
+            }
+        }
+        if (!NARROW && x_lane) {
 #pragma unroll
             for (int r = 0; r < XR; ++r)
 #pragma unroll
@@ -300,6 +333,7 @@ struct Plan {
     bool ok = false;
     int R = 1, PR = 0, PW = 0, PLANE = 0, GP = 0, Kst = 0, splits = 1, sps = 1, stages = 0;
     int WMO = 4, WC = 1, WK = 1;  // wave layout
+    bool narrow = false;          // whole-image stages with the (channel, row) pair staging
     size_t smem = 0;
     int bm() const { return 32 * WMO; }
     int ct() const { return 32 * WC; }
@@ -355,7 +389,27 @@ inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 k
         if (pl.WK > 1) pl.smem = std::max<size_t>(pl.smem, 4 * 16 * 64 * sizeof(float));  // the closing sum over the row segments
         if (pl.smem > LDS_BUDGET) best = 0;  // 64 planes of 3 x 66 floats: the next layout holds 32 planes
     }
-    if (!best) return pl;
+    if (!best) {
+        // maps of at most 64 pixels with rows of at most 16 floats: one whole image per stage (NARROW kernels)
+        const i64 L = oh * ow, XRn = (oh - 1) * sh + kh;
+        pl.WC = 1;
+        if (Cout > 64) { pl.WMO = 4; pl.WK = 1; }
+        else if (Cout > 32 && ow % 4 == 0) { pl.WMO = 2; pl.WK = 2; }
+        else if (Cout <= 32 && ow % 8 == 0) { pl.WMO = 1; pl.WK = 4; }
+        else return pl;
+        if (W > 16 || L > 4 * LPR || L < 24 || L % 4 != 0 || XRn > 10) return pl;
+        pl.narrow = true;
+        best = (int)oh;
+        pl.R = best;
+        pl.PR = (int)XRn;
+        pl.PW = (int)(W + 2 * pw);
+        pl.PLANE = odd_pitch(pl.PR * pl.PW);
+        pl.Kst = (int)L;
+        pl.GP = odd_pitch(pl.Kst);
+        pl.smem = ((size_t)pl.bm() * pl.GP + (size_t)pl.ct() * pl.PLANE + SLACK) * sizeof(float);
+        if (pl.WK > 1) pl.smem = std::max<size_t>(pl.smem, 4 * 16 * 64 * sizeof(float));
+        if (pl.smem > LDS_BUDGET) return pl;
+    }
     const i64 BM = pl.bm(), CT = pl.ct();
     pl.stages = (int)(B * (oh / best));
     const i64 tiles = fx::ceil_div(Cin, CT) * fx::ceil_div(Cout, BM);
@@ -382,6 +436,8 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
     p.R = pl.R; p.PW = pl.PW; p.PLANE = pl.PLANE; p.GP = pl.GP; p.Kst = pl.Kst;
     p.stages = pl.stages; p.sps = pl.sps; p.spi = (int)(oh / pl.R);
     p.div_spi = FastDiv((uint32_t)p.spi);
+    p.XRn = pl.PR;
+    p.div_xr = FastDiv((uint32_t)pl.PR);
     p.part_stride = Cout * Cin * KK;
     const dim3 grid((unsigned)fx::ceil_div(Cin, (i64)pl.ct()), (unsigned)fx::ceil_div(Cout, (i64)pl.bm()), (unsigned)pl.splits);
     const i64 blocks = (i64)grid.x * grid.y * grid.z;
@@ -394,7 +450,18 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
         wgrad_patch_kernel<XRV, A, B_, C_><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                                \
     } while (0)
     const int layout = pl.WMO * 100 + pl.WC * 10 + pl.WK;
-    if (layout == 411 && pl.PR == 3) FX_WGP_LAUNCH(3, 4, 1, 1);
+#define FX_WGP_LAUNCH_NARROW(A, C_)                                                                                   \
+    do {                                                                                                              \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_patch_kernel<0, A, 1, C_, true>,        \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
+        FX_HIP_CHECK(attr);                                                                                           \
+        wgrad_patch_kernel<0, A, 1, C_, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                             \
+    } while (0)
+    if (pl.narrow && layout == 411) FX_WGP_LAUNCH_NARROW(4, 1);
+    else if (pl.narrow && layout == 212) FX_WGP_LAUNCH_NARROW(2, 2);
+    else if (pl.narrow && layout == 114) FX_WGP_LAUNCH_NARROW(1, 4);
+    else if (pl.narrow) FX_REQUIRE(false, "wgrad patch kernel: unexpected narrow layout %d", layout);
+    else if (layout == 411 && pl.PR == 3) FX_WGP_LAUNCH(3, 4, 1, 1);
     else if (layout == 411) FX_WGP_LAUNCH(4, 4, 1, 1);
     else if (layout == 221 && pl.PR == 3) FX_WGP_LAUNCH(3, 2, 2, 1);
     else if (layout == 212 && pl.PR == 3) FX_WGP_LAUNCH(3, 2, 1, 2);
@@ -404,6 +471,7 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
     else if (layout == 114) FX_WGP_LAUNCH(4, 1, 1, 4);
     else FX_REQUIRE(false, "wgrad patch kernel: unexpected wave layout %d", layout);
 #undef FX_WGP_LAUNCH
+#undef FX_WGP_LAUNCH_NARROW
     FX_LAUNCH_CHECK();
     const int n = (int)p.part_stride;
     const FastDiv div_row((uint32_t)(KK * Cin)), div_cin((uint32_t)Cin);

@@ -443,6 +443,9 @@ WGRAD_PATCH_CASES = [
     (1, 33, 8, 24, 16, (1, 1), (1, 1)), (2, 17, 6, 32, 32, (1, 1), (1, 1)), (3, 48, 8, 32, 64, (1, 1), (1, 1)),
     # 64-wide rows with 64 x 64 channels (the 64-plane layout exceeds the LDS budget)
     (2, 64, 8, 64, 64, (1, 1), (1, 1)), (2, 64, 8, 64, 32, (1, 1), (1, 1)),
+    # narrow maps: one whole image per stage, (channel, row) pair staging
+    (3, 64, 8, 8, 128, (1, 1), (1, 1)), (2, 32, 8, 8, 64, (1, 1), (1, 1)), (2, 96, 8, 8, 20, (1, 1), (1, 1)), (2, 32, 6, 8, 100, (1, 1), (1, 1)),
+    (3, 64, 4, 16, 72, (1, 1), (1, 1)), (2, 48, 8, 8, 24, (1, 1), (1, 1)), (70, 128, 8, 8, 128, (1, 1), (1, 1)),
     # strided layers (implicit GEMM)
     (3, 32, 32, 32, 64, (2, 2), (1, 1)), (2, 64, 56, 56, 128, (2, 2), (1, 1)), (2, 32, 16, 24, 70, (2, 1), (1, 1)),
     (2, 32, 13, 32, 48, (2, 2), (0, 1)),

@@ -37,9 +37,17 @@ def wgrad_plan(num_cus, B, Cin, H, W, Cout, sh, sw, ph, pw, oh, ow):
             if WK > 1: smem = max(smem, 4 * 16 * 64 * 4)
             if smem > 72 * 1024: best = 0
         if best: break
-    if not best: return None
+    if not best:
+        # maps of at most 64 pixels with rows of at most 16 floats: one whole image per stage, (channel, row) pair staging
+        L, XRn = oh * ow, (oh - 1) * sh + 3
+        if Cout > 64: WMO, WK = 4, 1
+        elif Cout > 32 and ow % 4 == 0: WMO, WK = 2, 2
+        elif Cout <= 32 and ow % 8 == 0: WMO, WK = 1, 4
+        else: return None
+        if W > 16 or L > 64 or L < 24 or L % 4 or XRn > 10: return None
+        return dict(R=oh, PR=XRn, BM=32 * WMO, CT=32, Kst=L, stages=B, spi=1, narrow=True)
     PR = (best - 1) * sh + 3
-    return dict(R=best, PR=PR, BM=BM, CT=CT, Kst=best * ow, stages=B * (oh // best), spi=oh // best)
+    return dict(R=best, PR=PR, BM=BM, CT=CT, Kst=best * ow, stages=B * (oh // best), spi=oh // best, narrow=False)
 def wgrad_loads_in_bounds(B, Cin, H, W, Cout, st, pd):
     sh, sw = st; ph, pw = pd
     oh, ow = (H + 2 * ph - 3) // sh + 1, (W + 2 * pw - 3) // sw + 1
@@ -66,7 +74,25 @@ def wgrad_loads_in_bounds(B, Cin, H, W, Cout, st, pd):
                     if ok and pq < k4:  # the four floats are pixels of this stage in the lane's own channel row
                         row0 = (b * Cout + oc0 + prow + u * RPP) * L + oy0 * ow
                         assert row0 <= a and a + 4 <= row0 + pl["Kst"]
-        for c0 in range(0, Cin, pl["CT"]):
+        for c0 in (range(0, Cin, pl["CT"]) if pl["narrow"] else ()):
+            xsrc = (b * Cin + c0) * H * W
+            full_c = c0 + pl["CT"] <= Cin
+            PW = W + 2 * pw; PLANE = _odd_pitch_w(pl["PR"] * PW)
+            for tid in range(NT):
+                npq, npp = tid & 3, tid >> 2
+                lane_in = npq < ((W + 3) >> 2); col = min(4 * npq, W - 4)
+                for u in range(5):
+                    pair = u * 64 + npp; c, r = divmod(pair, pl["PR"]); iy = iy0 + r
+                    ok = lane_in and pair < pl["CT"] * pl["PR"] and 0 <= iy < H and (full_c or c0 + c < Cin)
+                    a = xsrc + (((c * H + iy) * W + col) if ok else 0)
+                    assert 0 <= a and a + 4 <= xsize, ("x narrow", a, xsize)
+                    if ok:
+                        row0 = ((b * Cin + c0 + c) * H + iy) * W
+                        assert row0 <= a and a + 4 <= row0 + W
+                    if lane_in and pair < pl["CT"] * pl["PR"] and (full_c or c0 + c < Cin):
+                        d = c * PLANE + r * PW + pw + col
+                        assert 0 <= d and d + 4 <= pl["CT"] * PLANE, ("Xs narrow", d)
+        for c0 in (() if pl["narrow"] else range(0, Cin, pl["CT"])):
             xsrc = (b * Cin + c0) * H * W
             full_c = c0 + pl["CT"] <= Cin
             for tid in range(NT):
@@ -303,6 +329,9 @@ WGRAD_SHAPES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw): every wave layout, r
     (1, 33, 8, 24, 16, (1, 1), (1, 1)), (2, 17, 6, 32, 32, (1, 1), (1, 1)),
     # 64 x 64 channels at 64-wide rows: the 64-plane layout exceeds the LDS budget, the 32-plane one is taken
     (2, 64, 8, 64, 64, (1, 1), (1, 1)), (2, 64, 8, 64, 32, (1, 1), (1, 1)),
+    # narrow maps: one whole image per stage
+    (3, 64, 8, 8, 128, (1, 1), (1, 1)), (2, 32, 8, 8, 64, (1, 1), (1, 1)), (2, 96, 8, 8, 20, (1, 1), (1, 1)), (2, 32, 6, 8, 100, (1, 1), (1, 1)),
+    (3, 64, 4, 16, 72, (1, 1), (1, 1)), (2, 48, 8, 8, 24, (1, 1), (1, 1)),
 ]
 FWD_SHAPES = [  # B, C, H, W, M, (sh, sw), (ph, pw): one per tile shape on a 256-CU device, ragged M, strides, paddings
     (2, 64, 28, 28, 64, (1, 1), (1, 1)), (2, 8, 6, 12, 60, (1, 1), (1, 1)), (3, 16, 8, 36, 120, (1, 1), (0, 0)),
