@@ -47,7 +47,7 @@ CONV_KERNELS = {"fwd": "cpk::conv_patch_kernel (conv fwd pass)", "dgrad": "cpk::
 # HBM-side bytes per launch of the main kernel of each C3 pass: rocprofv3 FETCH_SIZE + WRITE_SIZE per dispatch,
 # scaled by what the same counters read for the streaming add kernel of known size (x2.000 and x1.000); the
 # summary with the commands is profiles/conv_c3_f32_hbm_traffic.txt.
-CONV_C3_TRAFFIC_BYTES = {"fwd": 322.1e6, "dgrad": 319.5e6, "wgrad": 506.4e6}
+CONV_C3_TRAFFIC_BYTES = {"fwd": 322.1e6, "dgrad": 319.0e6, "wgrad": 518.4e6}
 
 
 def bench_conv(ctx, steps, warmup, dtype=np.float32, B=None):

@@ -441,7 +441,7 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
                 FX_HIP_CHECK(hipEventCreate(&c->ev_tune[0]));
                 FX_HIP_CHECK(hipEventCreate(&c->ev_tune[1]));
             }
-            // the modelled choice stays unless another shape is at least 3 % faster (timer noise between equals)
+            // the modelled choice stays unless another shape is at least 5 % faster (timer noise between equals)
             int model = 0;
             for (int k = 1; k < n; ++k)
                 if (cand[k].cost < cand[model].cost) model = k;
@@ -457,7 +457,7 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
             }
             best = model;
             for (int k = 0; k < n; ++k)
-                if (ms_of[k] < 0.97f * ms_of[best]) best = k;
+                if (ms_of[k] < 0.95f * ms_of[best]) best = k;
         }
         const int code = best >= 0 ? cand[best].WM * 16 + cand[best].TN : pl.WM * 16 + pl.TN;
         it = c->conv_tile_cache.emplace(key, code).first;
