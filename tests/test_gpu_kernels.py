@@ -609,6 +609,40 @@ def test_conv2d_image_layer_kernels(ctx, orc):
         assert np.array_equal(out.numpy(), gw), case
 
 
+def test_conv2d_tile_shape_timing_does_not_change_the_bits(ctx, tmp_path):
+    """The forward / data-gradient patch kernel times its candidate tile shapes on the first call of a layer shape.  Every
+    shape adds the terms of an output in the same order, so a process that keeps the modelled shape (FX_CONV_TUNE=0) must
+    produce the same bits as this one, whatever shape won here."""
+    import os
+    import subprocess
+    import sys
+    cases = [(32, 64, 56, 56, 128), (64, 64, 32, 32, 64), (128, 32, 16, 16, 64)]
+    script = tmp_path / "untuned.py"
+    script.write_text(
+        "import sys, numpy as np\n"
+        "sys.path.insert(0, %r)\n"
+        "from ferrox_amd import capi\n"
+        "ctx = capi.Context(0)\n"
+        "for i, (B, Cin, H, W, Cout) in enumerate(%r):\n"
+        "    x = ctx.uniform((B, Cin, H, W), 71 + i, -1.0, 1.0)\n"
+        "    w = ctx.normal((Cout, Cin, 3, 3), 81 + i, 0.0, 0.05)\n"
+        "    g = ctx.normal((B, Cout, H, W), 91 + i, 0.0, 1.0)\n"
+        "    np.save(%r + '/y%%d.npy' %% i, ctx.conv2d_fwd(x, w, (1, 1), (1, 1)).numpy())\n"
+        "    np.save(%r + '/d%%d.npy' %% i, ctx.conv2d_dgrad(g, w, (B, Cin, H, W), (1, 1), (1, 1), 0).numpy())\n"
+        "ctx.close()\n" % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))), cases, str(tmp_path), str(tmp_path)))
+    env = dict(os.environ, FX_CONV_TUNE="0")
+    subprocess.run([sys.executable, str(script)], check=True, env=env, timeout=240)
+    for i, (B, Cin, H, W, Cout) in enumerate(cases):
+        x = ctx.uniform((B, Cin, H, W), 71 + i, -1.0, 1.0)
+        w = ctx.normal((Cout, Cin, 3, 3), 81 + i, 0.0, 0.05)
+        g = ctx.normal((B, Cout, H, W), 91 + i, 0.0, 1.0)
+        y = ctx.conv2d_fwd(x, w, (1, 1), (1, 1)).numpy()
+        d = ctx.conv2d_dgrad(g, w, (B, Cin, H, W), (1, 1), (1, 1), 0).numpy()
+        assert np.array_equal(y, np.load(tmp_path / ("y%d.npy" % i))), ("fwd", cases[i])
+        assert np.array_equal(d, np.load(tmp_path / ("d%d.npy" % i))), ("dgrad", cases[i])
+        assert np.array_equal(y, ctx.conv2d_fwd(x, w, (1, 1), (1, 1)).numpy())
+
+
 # Strided data gradients, computed per pixel class (Cout % 16 == 0, kernel >= stride) and by the all-taps gather
 # otherwise: odd sizes, classes without pixels, kernel == stride, stride 3, 5x5, asymmetric stride and padding.
 # B, Cin, H, W, Cout, (kh, kw), (sh, sw), (ph, pw)
