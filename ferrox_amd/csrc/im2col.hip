@@ -110,6 +110,21 @@ __global__ __launch_bounds__(256) void im2col32_kernel(const T* __restrict__ x, 
     uint32_t b = g.div_L.div(n0), l = n0 - b * L;
     uint32_t oy = g.div_ow.div(l), ox = l - oy * (uint32_t)g.ow;
     vec_t v;
+    if (ox + V <= (uint32_t)g.ow && n0 + V <= N) {
+        // the V columns lie in one output row: one source row, consecutive taps; clamped loads and selects, no branches
+        const int iy = (int)(oy * g.sh + ky) - g.ph, ix0 = (int)(ox * g.sw + kx) - g.pw;
+        const bool row_ok = iy >= 0 && iy < g.H;
+        const T* src = x + ((b * (uint32_t)g.C + c) * (uint32_t)g.H + (uint32_t)(row_ok ? iy : 0)) * (uint32_t)g.W;
+#pragma unroll
+        for (int u = 0; u < V; ++u) {
+            const int ix = ix0 + u * g.sw;
+            const bool ok = row_ok && ix >= 0 && ix < g.W;
+            const T e = src[ok ? ix : 0];
+            v[u] = ok ? e : T(0);
+        }
+        *reinterpret_cast<vec_t*>(col + (i64)row * N + n0) = v;
+        return;
+    }
 #pragma unroll
     for (int u = 0; u < V; ++u) {
         const int iy = (int)(oy * g.sh + ky) - g.ph, ix = (int)(ox * g.sw + kx) - g.pw;
@@ -122,6 +137,46 @@ __global__ __launch_bounds__(256) void im2col32_kernel(const T* __restrict__ x, 
         }
     }
     *reinterpret_cast<vec_t*>(col + (i64)row * N + n0) = v;
+}
+
+// 3 x 3 windows at horizontal stride SW (1 or 2): one thread writes V consecutive columns of ALL nine rows of one input
+// channel.  Per window row it loads the (V - 1) SW + 3 input values under its columns once (clamped loads and selects) and
+// stores the three shifted vectors, so the index arithmetic and the reads are shared by nine outputs.  The V columns lie in
+// one output row (ow % V == 0); blockIdx.y is the channel.
+template <typename T, int V, int SW>
+__global__ __launch_bounds__(256) void im2col32_w3_kernel(const T* __restrict__ x, T* __restrict__ col, Geom32 g, uint32_t N) {
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    const uint32_t n0 = (blockIdx.x * 256u + threadIdx.x) * V;
+    if (n0 >= N) return;
+    const uint32_t c = blockIdx.y;
+    const uint32_t L = (uint32_t)(g.oh * g.ow);
+    const uint32_t b = g.div_L.div(n0), l = n0 - b * L;
+    const uint32_t oy = g.div_ow.div(l), ox = l - oy * (uint32_t)g.ow;
+    const int ix0 = (int)ox * SW - g.pw;
+    const T* plane = x + (b * (uint32_t)g.C + c) * (uint32_t)(g.H * g.W);
+    T* dst = col + (i64)(c * 9u) * N + n0;
+#pragma unroll
+    for (int ky = 0; ky < 3; ++ky) {
+        const int iy = (int)(oy * g.sh) + ky - g.ph;
+        const bool row_ok = iy >= 0 && iy < g.H;
+        const T* src = plane + (uint32_t)(row_ok ? iy : 0) * (uint32_t)g.W;
+        constexpr int NB = (V - 1) * SW + 3;
+        T buf[NB];
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            const int ix = ix0 + j;
+            const bool ok = row_ok && ix >= 0 && ix < g.W;
+            const T e = src[ok ? ix : 0];
+            buf[j] = ok ? e : T(0);
+        }
+#pragma unroll
+        for (int kx = 0; kx < 3; ++kx) {
+            vec_t v;
+#pragma unroll
+            for (int u = 0; u < V; ++u) v[u] = buf[u * SW + kx];
+            *reinterpret_cast<vec_t*>(dst + (i64)(ky * 3 + kx) * N) = v;
+        }
+    }
 }
 
 // The gather of col2im_kernel with 32-bit indices: the taps that reach a pixel are ky = (Y mod sh) + j*sh, visited in
@@ -153,6 +208,37 @@ __global__ __launch_bounds__(256) void col2im32_kernel(const T* __restrict__ col
     out[idx] = acc;
 }
 
+// Stride 1 with a compile-time window: every tap of a pixel is one clamped load and a select (same taps in the same
+// order as the loop above, so the same bits; a tap that falls outside the column matrix adds nothing).
+template <typename T, int LAYOUT, int KH, int KW>
+__global__ __launch_bounds__(256) void col2im32_s1_kernel(const T* __restrict__ col, T* __restrict__ out, Geom32 g, uint32_t total) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= total) return;
+    uint32_t t = g.div_W.div(idx);
+    const uint32_t xw = idx - t * (uint32_t)g.W;
+    const uint32_t t2 = g.div_H.div(t), y = t - t2 * (uint32_t)g.H;
+    const uint32_t b = g.div_C.div(t2), c = t2 - b * (uint32_t)g.C;
+    const uint32_t L = (uint32_t)(g.oh * g.ow);
+    constexpr uint32_t KK = KH * KW;
+    const int Y = (int)y + g.ph, X = (int)xw + g.pw;
+    const i64 tap_stride = LAYOUT == 1 ? (i64)L : (i64)g.B * L;
+    const T* base = col + (LAYOUT == 1 ? (i64)(b * g.C + c) * KK * L : (i64)c * KK * ((i64)g.B * L) + (i64)b * L);
+    T acc = T(0);
+#pragma unroll
+    for (int ky = 0; ky < KH; ++ky) {
+        const int cy = Y - ky;
+        const bool row_ok = cy >= 0 && cy < g.oh;
+#pragma unroll
+        for (int kx = 0; kx < KW; ++kx) {
+            const int cx = X - kx;
+            const bool ok = row_ok && cx >= 0 && cx < g.ow;
+            const T v = base[(i64)(ky * KW + kx) * tap_stride + (ok ? cy * g.ow + cx : 0)];
+            acc = ok ? acc + v : acc;
+        }
+    }
+    out[idx] = acc;
+}
+
 bool geom32(Geom32& q, const ConvGeom& g) {
     const i64 N = g.B * g.oh * g.ow;
     const i64 lim = 0x7fffffff;
@@ -178,7 +264,11 @@ int im2col(fx_ctx* c, const T* x, T* col, i64 B, i64 C, i64 H, i64 W, i64 kh, i6
     Geom32 q;
     if (geom32(q, g)) {
         constexpr int V = 16 / (int)sizeof(T);
-        if (N % V == 0 && fx::aligned16(col))
+        if (kh == 3 && kw == 3 && sw == 1 && g.ow % V == 0 && fx::aligned16(col))
+            im2col32_w3_kernel<T, V, 1><<<dim3((unsigned)fx::ceil_div(N / V, 256), (unsigned)C), dim3(256), 0, c->stream>>>(x, col, q, (uint32_t)N);
+        else if (kh == 3 && kw == 3 && sw == 2 && g.ow % V == 0 && fx::aligned16(col))
+            im2col32_w3_kernel<T, V, 2><<<dim3((unsigned)fx::ceil_div(N / V, 256), (unsigned)C), dim3(256), 0, c->stream>>>(x, col, q, (uint32_t)N);
+        else if (N % V == 0 && fx::aligned16(col))
             im2col32_kernel<T, V><<<dim3((unsigned)fx::ceil_div(N / V, 256), (unsigned)rows), dim3(256), 0, c->stream>>>(x, col, q, (uint32_t)N);
         else
             im2col32_kernel<T, 1><<<dim3((unsigned)fx::ceil_div(N, 256), (unsigned)rows), dim3(256), 0, c->stream>>>(x, col, q, (uint32_t)N);
@@ -203,7 +293,10 @@ int col2im(fx_ctx* c, const T* col, T* out, i64 B, i64 C, i64 H, i64 W, i64 kh, 
     const dim3 grid((unsigned)fx::ceil_div(total, 256)), block(256);
     Geom32 q;
     if (geom32(q, g)) {
-        if (layout == 1) col2im32_kernel<T, 1><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
+        const bool s1_3x3 = kh == 3 && kw == 3 && sh == 1 && sw == 1;
+        if (s1_3x3 && layout == 1) col2im32_s1_kernel<T, 1, 3, 3><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
+        else if (s1_3x3) col2im32_s1_kernel<T, 0, 3, 3><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
+        else if (layout == 1) col2im32_kernel<T, 1><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
         else col2im32_kernel<T, 0><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
         FX_LAUNCH_CHECK();
         return FX_OK;
