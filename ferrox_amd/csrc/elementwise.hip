@@ -383,6 +383,42 @@ __global__ __launch_bounds__(256) void transpose_tile_kernel(const T* __restrict
     }
 }
 
+// The same tiles with 16-byte global accesses (both extents, the source pitch and the batch pitch multiples of the vector
+// length, 16-byte aligned pointers): a thread moves V consecutive elements per access, the transposition happens in the LDS
+// tile, whose reads and writes stay at two lanes per bank.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_tile_vec_kernel(const T* __restrict__ in, T* __restrict__ out, i64 I, i64 J, i64 ld, i64 sb) {
+    constexpr int V = 16 / (int)sizeof(T), VPR = 64 / V, RPP = 256 / VPR;  // vectors per tile row, rows per pass
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    __shared__ T tile[64][65];
+    const int vx = threadIdx.x % VPR, vy = threadIdx.x / VPR;
+    const i64 j0 = (i64)blockIdx.x * 64, i0 = (i64)blockIdx.y * 64, b = blockIdx.z;
+    const T* src = in + b * sb;
+#pragma unroll
+    for (int r = 0; r < 64 / RPP; ++r) {
+        const int jl = vy + RPP * r;
+        const i64 j = j0 + jl, i = i0 + vx * V;
+        if (j < J && i < I) {
+            const vec_t v = *reinterpret_cast<const vec_t*>(src + j * ld + i);
+#pragma unroll
+            for (int e = 0; e < V; ++e) tile[jl][vx * V + e] = v[e];
+        }
+    }
+    __syncthreads();
+    T* dst = out + b * I * J;
+#pragma unroll
+    for (int r = 0; r < 64 / RPP; ++r) {
+        const int il = vy + RPP * r;
+        const i64 i = i0 + il, j = j0 + vx * V;
+        if (i < I && j < J) {
+            vec_t v;
+#pragma unroll
+            for (int e = 0; e < V; ++e) v[e] = tile[vx * V + e][il];
+            *reinterpret_cast<vec_t*>(dst + i * J + j) = v;
+        }
+    }
+}
+
 template <typename T>
 int materialize(fx_ctx* c, const T* in, T* out, const i64* shape, const i64* strides, int ndim, i64 n) {
     FX_CHECK_CTX(c);
@@ -419,8 +455,12 @@ int materialize(fx_ctx* c, const T* in, T* out, const i64* shape, const i64* str
         const i64 I = cs[nd - 2], J = cs[nd - 1], Bn = nd == 3 ? cs[0] : 1;
         const i64 gx = fx::ceil_div(J, 64), gy = fx::ceil_div(I, 64);
         if (gx <= 0x7fffffff && gy <= 65535 && Bn <= 65535) {
-            transpose_tile_kernel<T><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)Bn), dim3(256), 0, c->stream>>>(
-                in, out, I, J, ct[nd - 1], nd == 3 ? ct[0] : 0);
+            const i64 ld = ct[nd - 1], sb = nd == 3 ? ct[0] : 0;
+            constexpr i64 VT = 16 / (i64)sizeof(T);
+            if (I % VT == 0 && J % VT == 0 && ld % VT == 0 && sb % VT == 0 && (((uintptr_t)in | (uintptr_t)out) & 15) == 0)
+                transpose_tile_vec_kernel<T><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)Bn), dim3(256), 0, c->stream>>>(in, out, I, J, ld, sb);
+            else
+                transpose_tile_kernel<T><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)Bn), dim3(256), 0, c->stream>>>(in, out, I, J, ld, sb);
             FX_LAUNCH_CHECK();
             return FX_OK;
         }
