@@ -208,10 +208,11 @@ __global__ __launch_bounds__(256) void col2im32_kernel(const T* __restrict__ col
     out[idx] = acc;
 }
 
-// Stride 1 with a compile-time window: every tap of a pixel is one clamped load and a select (same taps in the same
-// order as the loop above, so the same bits; a tap that falls outside the column matrix adds nothing).
-template <typename T, int LAYOUT, int KH, int KW>
-__global__ __launch_bounds__(256) void col2im32_s1_kernel(const T* __restrict__ col, T* __restrict__ out, Geom32 g, uint32_t total) {
+// Compile-time window and strides: the taps that reach a pixel are ky = (Y mod SH) + j SH with cy = Y / SH - j, j below
+// ceil(KH / SH), and likewise along x -- the loop of the kernel above, unrolled, every tap one clamped load and a select
+// (same taps in the same order, so the same bits; a tap outside the window or the column matrix adds nothing).
+template <typename T, int LAYOUT, int KH, int KW, int SH, int SW>
+__global__ __launch_bounds__(256) void col2im32_fixed_kernel(const T* __restrict__ col, T* __restrict__ out, Geom32 g, uint32_t total) {
     const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
     if (idx >= total) return;
     uint32_t t = g.div_W.div(idx);
@@ -220,19 +221,21 @@ __global__ __launch_bounds__(256) void col2im32_s1_kernel(const T* __restrict__ 
     const uint32_t b = g.div_C.div(t2), c = t2 - b * (uint32_t)g.C;
     const uint32_t L = (uint32_t)(g.oh * g.ow);
     constexpr uint32_t KK = KH * KW;
+    constexpr int NJH = (KH + SH - 1) / SH, NJW = (KW + SW - 1) / SW;
     const int Y = (int)y + g.ph, X = (int)xw + g.pw;
+    const int qy = Y / SH, ry = Y - qy * SH, qx = X / SW, rx = X - qx * SW;
     const i64 tap_stride = LAYOUT == 1 ? (i64)L : (i64)g.B * L;
     const T* base = col + (LAYOUT == 1 ? (i64)(b * g.C + c) * KK * L : (i64)c * KK * ((i64)g.B * L) + (i64)b * L);
     T acc = T(0);
 #pragma unroll
-    for (int ky = 0; ky < KH; ++ky) {
-        const int cy = Y - ky;
-        const bool row_ok = cy >= 0 && cy < g.oh;
+    for (int jy = 0; jy < NJH; ++jy) {
+        const int ky = ry + jy * SH, cy = qy - jy;
+        const bool row_ok = ky < KH && cy >= 0 && cy < g.oh;
 #pragma unroll
-        for (int kx = 0; kx < KW; ++kx) {
-            const int cx = X - kx;
-            const bool ok = row_ok && cx >= 0 && cx < g.ow;
-            const T v = base[(i64)(ky * KW + kx) * tap_stride + (ok ? cy * g.ow + cx : 0)];
+        for (int jx = 0; jx < NJW; ++jx) {
+            const int kx = rx + jx * SW, cx = qx - jx;
+            const bool ok = row_ok && kx < KW && cx >= 0 && cx < g.ow;
+            const T v = base[(ok ? (i64)(ky * KW + kx) * tap_stride + cy * g.ow + cx : (i64)0)];
             acc = ok ? acc + v : acc;
         }
     }
@@ -293,9 +296,11 @@ int col2im(fx_ctx* c, const T* col, T* out, i64 B, i64 C, i64 H, i64 W, i64 kh, 
     const dim3 grid((unsigned)fx::ceil_div(total, 256)), block(256);
     Geom32 q;
     if (geom32(q, g)) {
-        const bool s1_3x3 = kh == 3 && kw == 3 && sh == 1 && sw == 1;
-        if (s1_3x3 && layout == 1) col2im32_s1_kernel<T, 1, 3, 3><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
-        else if (s1_3x3) col2im32_s1_kernel<T, 0, 3, 3><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
+        const bool k3 = kh == 3 && kw == 3, s1 = k3 && sh == 1 && sw == 1, s2 = k3 && sh == 2 && sw == 2;
+        if (s1 && layout == 1) col2im32_fixed_kernel<T, 1, 3, 3, 1, 1><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
+        else if (s1) col2im32_fixed_kernel<T, 0, 3, 3, 1, 1><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
+        else if (s2 && layout == 1) col2im32_fixed_kernel<T, 1, 3, 3, 2, 2><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
+        else if (s2) col2im32_fixed_kernel<T, 0, 3, 3, 2, 2><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
         else if (layout == 1) col2im32_kernel<T, 1><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
         else col2im32_kernel<T, 0><<<grid, block, 0, c->stream>>>(col, out, q, (uint32_t)total);
         FX_LAUNCH_CHECK();
