@@ -162,12 +162,29 @@ __global__ __launch_bounds__(256) void im2col32_w3_kernel(const T* __restrict__ 
         const T* src = plane + (uint32_t)(row_ok ? iy : 0) * (uint32_t)g.W;
         constexpr int NB = (V - 1) * SW + 3;
         T buf[NB];
+        if (ix0 >= 0 && ix0 + NB <= g.W) {
+            // all NB values lie inside the row: V-wide loads at element alignment (the hardware takes unaligned vectors)
+            typedef T vecu_t __attribute__((ext_vector_type(V), aligned(sizeof(T))));
+            constexpr int NV = NB / V, REST = NB - NV * V;
 #pragma unroll
-        for (int j = 0; j < NB; ++j) {
-            const int ix = ix0 + j;
-            const bool ok = row_ok && ix >= 0 && ix < g.W;
-            const T e = src[ok ? ix : 0];
-            buf[j] = ok ? e : T(0);
+            for (int q = 0; q < NV; ++q) {
+                const vecu_t v = *reinterpret_cast<const vecu_t*>(src + ix0 + q * V);
+#pragma unroll
+                for (int e = 0; e < V; ++e) buf[q * V + e] = row_ok ? v[e] : T(0);
+            }
+#pragma unroll
+            for (int e = 0; e < REST; ++e) {
+                const T v = src[ix0 + NV * V + e];
+                buf[NV * V + e] = row_ok ? v : T(0);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                const int ix = ix0 + j;
+                const bool ok = row_ok && ix >= 0 && ix < g.W;
+                const T e = src[ok ? ix : 0];
+                buf[j] = ok ? e : T(0);
+            }
         }
 #pragma unroll
         for (int kx = 0; kx < 3; ++kx) {
