@@ -403,6 +403,40 @@ def _cpu_model():
     return "unknown"
 
 
+def bench_conv_sweep():
+    """3x3, stride 1, padding 1, f32: TFLOP/s of the three passes over channel counts and map sizes (batch sized to a few
+    GFLOP per pass).  Timed with the library's event timer on its own stream, 20 runs after 3 warm-up runs each."""
+    from ferrox_amd import capi
+    ctx = capi.Context(0)
+
+    def timed(fn, runs=20, warm=3):
+        for _ in range(warm):
+            fn()
+        ctx.sync()
+        ctx.timer_start()
+        for _ in range(runs):
+            fn()
+        return ctx.timer_stop() / runs
+
+    out = {}
+    for hw, batch in ((64, 64), (32, 128), (16, 256), (8, 512)):
+        for cin in (32, 64, 128, 256):
+            for cout in (32, 64, 128, 256):
+                x = ctx.uniform((batch, cin, hw, hw), 1, -1.0, 1.0)
+                g = ctx.normal((batch, cout, hw, hw), 2, 0.0, 1.0)
+                w = ctx.normal((cout, cin, 3, 3), 3, 0.0, 0.05)
+                y, dx, dw = ctx.empty(g.shape), ctx.empty(x.shape), ctx.empty(w.shape)
+                gflop = 2.0 * cout * cin * 9 * batch * hw * hw / 1e9
+                ms = (timed(lambda: ctx.conv2d_fwd(x, w, (1, 1), (1, 1), out=y)),
+                      timed(lambda: ctx.conv2d_dgrad(g, w, x.shape, (1, 1), (1, 1), 0, out=dx)),
+                      timed(lambda: ctx.conv2d_wgrad(x, g, w.shape, (1, 1), (1, 1), 0, out=dw)))
+                out[f"B{batch}_{cin}to{cout}_{hw}x{hw}"] = [round(gflop / m, 1) for m in ms]
+                for a in (x, g, w, y, dx, dw):
+                    a.free()
+    ctx.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -414,9 +448,15 @@ def main():
     ap.add_argument("--train-only", nargs="?", const="all", default=None, metavar="CONFIG,DTYPE,ENGINE",
                     help="run only the train-step section and print it (profiler runs); optional filter such as "
                          "C5_cnn,float32,engine_fused")
+    ap.add_argument("--conv-sweep", action="store_true",
+                    help="run only a sweep of 3x3 stride-1 f32 layer shapes (Cin, Cout in 32..256; 8x8..64x64 maps) and print "
+                         "TFLOP/s per pass as one JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the hot path has no cross-GPU exchange built); use --gpus 1")
+    if args.conv_sweep:
+        print(json.dumps({"conv_sweep_tflops_fwd_dgrad_wgrad": bench_conv_sweep()}))
+        return
     if args.train_only:
         only = None if args.train_only == "all" else tuple(args.train_only.split(","))
         print(json.dumps({"train_step": bench_train_steps(cpu=False, only=only)}))
