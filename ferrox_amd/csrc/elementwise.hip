@@ -367,7 +367,9 @@ template <typename T>
 __global__ __launch_bounds__(256) void transpose_tile_kernel(const T* __restrict__ in, T* __restrict__ out, i64 I, i64 J, i64 ld, i64 sb) {
     __shared__ T tile[64][65];
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    const i64 j0 = (i64)blockIdx.x * 64, i0 = (i64)blockIdx.y * 64, b = blockIdx.z;
+    // diagonal order: the blocks that run together read source rows of different tile columns, so a power-of-two pitch does
+    // not send all of them to the same memory channels
+    const i64 j0 = (i64)((blockIdx.x + blockIdx.y) % gridDim.x) * 64, i0 = (i64)blockIdx.y * 64, b = blockIdx.z;
     const T* src = in + b * sb;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -392,7 +394,9 @@ __global__ __launch_bounds__(256) void transpose_tile_vec_kernel(const T* __rest
     typedef T vec_t __attribute__((ext_vector_type(V)));
     __shared__ T tile[64][65];
     const int vx = threadIdx.x % VPR, vy = threadIdx.x / VPR;
-    const i64 j0 = (i64)blockIdx.x * 64, i0 = (i64)blockIdx.y * 64, b = blockIdx.z;
+    // diagonal order: the blocks that run together read source rows of different tile columns, so a power-of-two pitch does
+    // not send all of them to the same memory channels
+    const i64 j0 = (i64)((blockIdx.x + blockIdx.y) % gridDim.x) * 64, i0 = (i64)blockIdx.y * 64, b = blockIdx.z;
     const T* src = in + b * sb;
 #pragma unroll
     for (int r = 0; r < 64 / RPP; ++r) {
