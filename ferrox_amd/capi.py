@@ -143,6 +143,9 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
          *([_ct] * 7))
     _sig(f"fx_sgd_step_multi_{_s}", _vp, _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_i64), _ct)
 
+_sig("fx_reduce_max_noalloc_f32", _vp, _vp, _vp, _vp, _i64, _i64, _i64)
+NOALLOC_SCRATCH_BYTES = 4 << 20
+
 
 class FerroxHipError(RuntimeError):
     def __init__(self, code, message):
@@ -390,6 +393,11 @@ class Context:
         check(self._fn("reduce_" + kind, a.dtype)(self.h, a.ptr, o.ptr, outer, ax, inner))
         o.shape = oshape
         return o
+
+    def reduce_max_noalloc(self, a, axis, out, idx):
+        """fx_reduce_max_noalloc_f32 into caller-provided `out` (values) and `idx` (a _RawI64 or None)."""
+        outer, ax, inner = self._oai(a.shape, axis)
+        check(lib.fx_reduce_max_noalloc_f32(self.h, a.ptr, out.ptr, idx.ptr if idx is not None else None, outer, ax, inner))
 
     def softmax_axis(self, a, axis):
         outer, ax, inner = self._oai(a.shape, axis)

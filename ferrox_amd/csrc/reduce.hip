@@ -269,8 +269,31 @@ void launch_col(fx_ctx* c, dim3 grid, const T* in, T* out, i64* idx_out, i64 axi
     col_reduce_kernel<T, IS_MAX, VEC, false, CW, STREAM><<<grid, dim3(256), 0, c->stream>>>(in, nullptr, out, idx_out, axis, inner, chunk, scale, final_pass);
 }
 
+// Where the slice partials of a split reduction live: the context's growing scratch allocation, or, for the entry
+// point that must not allocate, a fixed region of `fixed_bytes` (a request beyond it is refused).
+struct PartialSpace {
+    char* fixed = nullptr;
+    i64 fixed_bytes = 0;
+    // returns nullptr with the error message and *rc set
+    char* get(fx_ctx* c, i64 bytes, const char* what, int* rc) const {
+        if (fixed) {
+            if (bytes > fixed_bytes) {
+                fx::set_error("%s: this shape needs %lld bytes of slice partials, the fixed scratch holds %lld", what,
+                              (long long)bytes, (long long)fixed_bytes);
+                *rc = FX_ERR_UNSUPPORTED;
+                return nullptr;
+            }
+            return fixed;
+        }
+        char* p = (char*)c->get_scratch(bytes);
+        if (!p) *rc = FX_ERR_OOM;
+        return p;
+    }
+};
+
 template <typename T, int IS_MAX>
-int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i64 inner, T scale, const char* what) {
+int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i64 inner, T scale, const char* what,
+           const PartialSpace& space = PartialSpace()) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(outer >= 0 && axis >= 1 && inner >= 0, "%s: bad view [%lld, %lld, %lld]", what, (long long)outer,
                (long long)axis, (long long)inner);
@@ -309,8 +332,9 @@ int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i6
         i64* pi = idx_out;
         if (S > 1) {
             const i64 bytes = outer * S * (i64)(sizeof(T) + sizeof(i64));
-            char* sc = (char*)c->get_scratch(bytes);
-            if (!sc) return FX_ERR_OOM;
+            int rc = FX_OK;
+            char* sc = space.get(c, bytes, what, &rc);
+            if (!sc) return rc;
             pi = (i64*)sc;
             pv = (T*)(sc + outer * S * sizeof(i64));
         }
@@ -355,8 +379,9 @@ int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i6
     if (S > 1) {
         const i64 n_part = outer * S * inner;
         const i64 bytes = n_part * (i64)(sizeof(T) + (EXTREMUM(IS_MAX) ? sizeof(i64) : 0)) + 256;
-        char* sc = (char*)c->get_scratch(bytes);
-        if (!sc) return FX_ERR_OOM;
+        int rc = FX_OK;
+        char* sc = space.get(c, bytes, what, &rc);
+        if (!sc) return rc;
         pi = EXTREMUM(IS_MAX) ? (i64*)sc : nullptr;
         pv = (T*)(sc + (EXTREMUM(IS_MAX) ? ((n_part * sizeof(i64) + 255) / 256) * 256 : 0));
     }
@@ -449,6 +474,39 @@ int softmax_axis(fx_ctx* c, const T* in, T* out, i64 outer, i64 axis, i64 inner)
 }
 
 }  // namespace
+
+// ---- the entry point that allocates nothing ---------------------------------------------------------------
+// Slice partials of fx_reduce_max_noalloc_f32 live in this array instead of the context's hipMalloc'ed scratch.
+// Every device the library is loaded on holds its own copy at its own address; host code uses the address
+// hipGetSymbolAddress returned for the device, never the array's name.
+static __device__ __align__(256) unsigned char scratch[FX_NOALLOC_SCRATCH_BYTES];
+
+namespace fx {
+constexpr int MAX_DEVICES = 64;
+static char* g_static_scratch[MAX_DEVICES] = {};
+static std::mutex g_static_scratch_mutex;
+// Called by fx_init with `device` current: resolves this device's copy of the array once.
+int static_scratch_init(int device) {
+    if (device < 0 || device >= MAX_DEVICES) return FX_OK;  // the no-alloc entry point refuses such a device itself
+    std::lock_guard<std::mutex> lk(g_static_scratch_mutex);
+    if (g_static_scratch[device]) return FX_OK;
+    void* p = nullptr;
+    FX_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    g_static_scratch[device] = (char*)p;
+    return FX_OK;
+}
+}  // namespace fx
+
+extern "C" int fx_reduce_max_noalloc_f32(fx_ctx* c, const float* in, float* out, int64_t* idx, int64_t outer, int64_t axis,
+                                         int64_t inner) {
+    FX_REQUIRE(c != nullptr, "null context");
+    FX_REQUIRE(c->device >= 0 && c->device < fx::MAX_DEVICES && fx::g_static_scratch[c->device] != nullptr,
+               "fx_reduce_max_noalloc: no fixed scratch was resolved for device %d", c->device);
+    PartialSpace space;
+    space.fixed = fx::g_static_scratch[c->device];
+    space.fixed_bytes = FX_NOALLOC_SCRATCH_BYTES;
+    return reduce<float, 1>(c, in, out, idx, outer, axis, inner, 1.0f, "fx_reduce_max_noalloc", space);
+}
 
 #define FX_DEFINE_REDUCE(T, S)                                                                                         \
     extern "C" int fx_reduce_sum_##S(fx_ctx* c, const T* in, T* out, int64_t outer, int64_t axis, int64_t inner) {     \

@@ -21,6 +21,7 @@ int bind_device(int device) {
     return FX_OK;
 }
 Pool* pool_create(const fx_pool_config* cfg, int elem_size, hipStream_t stream);
+int static_scratch_init(int device);  // reduce.hip
 void pool_destroy(Pool* p);
 }  // namespace fx
 
@@ -60,6 +61,7 @@ int fx_init(int device, const fx_pool_config* cfg, fx_ctx** out) {
         fx::set_error("fx_init: this library holds gfx950 code only; device %d is %s", device, prop.gcnArchName);
         return FX_ERR_UNSUPPORTED;
     }
+    if (int rc = fx::static_scratch_init(device)) return rc;
     fx_ctx* c = new fx_ctx();
     c->device = device;
     c->name = prop.name[0] ? prop.name : prop.gcnArchName;

@@ -319,6 +319,20 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
 FX_DECLARE_KERNELS(float, f32)
 FX_DECLARE_KERNELS(double, f64)
 
+/* ---- an entry point that allocates nothing ---------------------------------------------------------------
+ * No counterpart in the reference.  It is for callers that cannot allocate device memory at the time of the call:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same arguments, kernels and
+ * results (bit for bit) as fx_reduce_max_f32, but the partial maxima / indices of a reduction whose axis is split
+ * across blocks go to a fixed array of FX_NOALLOC_SCRATCH_BYTES inside the library's device image (resolved once per
+ * device by fx_init) instead of the context's growing hipMalloc'ed scratch.  A shape whose partials do not fit
+ * returns FX_ERR_UNSUPPORTED with the sizes in the message ([8192, 8192] along either axis or as one run needs at
+ * most 2.4 MB).  Nothing in the array has to start at zero (every partial is written before it is read), so it
+ * is never cleared; all calls on one GPU share it, so calls that overlap on one GPU -- two contexts, or two
+ * streams -- race and must be serialised by the caller. */
+#define FX_NOALLOC_SCRATCH_BYTES (4 << 20)
+int fx_reduce_max_noalloc_f32(fx_ctx* ctx, const float* in, float* out, int64_t* idx_out, int64_t outer, int64_t axis,
+                              int64_t inner);
+
 #ifdef __cplusplus
 }
 #endif

@@ -13,7 +13,8 @@ def declared_symbols():
     plain = set(re.findall(r"\b(fx_[a-z0-9_]+)\s*\(", text.split("#define FX_DECLARE_KERNELS")[0]))
     macro_body = text.split("#define FX_DECLARE_KERNELS")[1].split("FX_DECLARE_KERNELS(float")[0]
     templ = set(re.findall(r"\b(fx_[a-z0-9_]+)_##S\s*\(", macro_body))
-    syms = set(plain)
+    tail = text.split("FX_DECLARE_KERNELS(double, f64)")[1]
+    syms = set(plain) | set(re.findall(r"\b(fx_[a-z0-9_]+)\s*\(", tail))
     for s in ("f32", "f64"):
         syms |= {f"{t}_{s}" for t in templ}
     return syms
@@ -24,6 +25,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(capi.LIB_PATH)
     syms = declared_symbols()
     assert len(syms) > 90
+    assert "fx_reduce_max_noalloc_f32" in syms
     missing = [s for s in sorted(syms) if not hasattr(lib, s)]
     assert not missing, missing
 
