@@ -20,7 +20,10 @@ struct ModelBase {
     virtual int num_params() const = 0;
     virtual int64_t param_numel(int i) const = 0;
     virtual void set_batch(const void* x, const Shape& xs, const void* y, const Shape& ys) = 0;
-    virtual double train_step() = 0;
+    virtual double train_step(bool optimizer_step = true) = 0;
+    virtual void configure(int loss_kind, bool input_requires_grad) = 0;
+    virtual int64_t input_numel() const = 0;
+    virtual void get_input_grad(void* host) const = 0;
     virtual void get_param(int i, void* host) const = 0;
     virtual void get_grad(int i, void* host) const = 0;
     virtual void forward_only(void* host_out) = 0;
@@ -52,6 +55,13 @@ template <typename T> struct Model : ModelBase {
     Tensor<T> x, y;
 
     bool fused = false;
+    // loss: 0 = CCELoss on (prediction, targets); 1 = Sum over every element of the prediction (the reference's
+    // plumbing check: relu(conv(x) + b).sum().backward(), Sum::new() of src/ops/reduction.rs:52-140)
+    int loss_kind = 0;
+    // the batch enters the graph as a leaf that requires a gradient (create_variable(x, true)), kept across steps
+    bool input_requires_grad = false;
+    bool have_input_node = false;
+    NodeId input_node = 0;
 
     // engine: 0 = reference op sequence without the per-node deep clones, 1 = reference op sequence as is,
     //         2 = fused layers / loss / optimizers
@@ -156,30 +166,56 @@ template <typename T> struct Model : ModelBase {
     void set_batch(const void* xv, const Shape& xs, const void* yv, const Shape& ys) override {
         x = HipStorage<T>::from_vec(static_cast<const T*>(xv), xs);
         y = HipStorage<T>::from_vec(static_cast<const T*>(yv), ys);
+        if (have_input_node) graph.update_parameter(input_node, x->clone_storage());
+    }
+    void configure(int kind, bool in_grad) override {
+        if (kind != 0 && kind != 1) throw Error("unknown loss kind");
+        loss_kind = kind;
+        input_requires_grad = in_grad;
+    }
+    int64_t input_numel() const override { return x ? (int64_t)x->size() : -1; }
+    void get_input_grad(void* host) const override {
+        const HipStorage<T>* g = have_input_node ? graph.get_gradient(input_node) : nullptr;
+        if (!g) throw Error("no gradient for the input (configure the model with input_requires_grad and run a backward pass)");
+        std::vector<T> v = g->to_vec();
+        std::memcpy(host, v.data(), v.size() * sizeof(T));
     }
     NodeId forward(NodeId in) {
         for (auto& l : layers) in = l->forward(graph, in);
         return in;
     }
-    double train_step() override {
+    double train_step(bool optimizer_step) override {
         if (!x || !y) throw Error("set_batch was not called");
         graph.zero_gradients();
-        // the reference clones the batch every step (training.rs:125-126); the fused engine reads it in place
-        const NodeId xin = graph.create_variable(fused ? HipStorage<T>::borrow(*x) : x->clone_storage(), false);
-        const NodeId yin = graph.create_variable(fused ? HipStorage<T>::borrow(*y) : y->clone_storage(), false);
+        NodeId xin;
+        if (input_requires_grad) {
+            if (!have_input_node) {
+                input_node = graph.create_variable(x->clone_storage(), true);
+                have_input_node = true;
+            }
+            xin = input_node;
+        } else {
+            // the reference clones the batch every step (training.rs:125-126); the fused engine reads it in place
+            xin = graph.create_variable(fused ? HipStorage<T>::borrow(*x) : x->clone_storage(), false);
+        }
         const NodeId pred = forward(xin);
-        const NodeId loss = fused ? cce_loss_fused<T>(graph, pred, yin) : cce_loss<T>(graph, pred, yin);
+        NodeId loss;
+        if (loss_kind == 1) loss = graph.apply_operation(std::make_unique<Sum<T>>(false), {pred});
+        else {
+            const NodeId yin = graph.create_variable(fused ? HipStorage<T>::borrow(*y) : y->clone_storage(), false);
+            loss = fused ? cce_loss_fused<T>(graph, pred, yin) : cce_loss<T>(graph, pred, yin);
+        }
         if (!fused) {
             const T lv = graph.get_tensor(loss)->clone_storage()->first();  // device -> host: the GPU drains here (training.rs:60-64)
             graph.backward(loss);
-            opt->step(graph);
+            if (optimizer_step) opt->step(graph);
             return (double)lv;
         }
         // fused engine: the loss is copied aside and read after the backward pass and the update are enqueued, so the
         // device never waits for the host in the middle of a step
         Tensor<T> lcopy = graph.get_tensor(loss)->clone_storage();
         graph.backward(loss);
-        opt->step(graph);
+        if (optimizer_step) opt->step(graph);
         return (double)lcopy->first();
     }
     void get_param(int i, void* host) const override {
@@ -227,6 +263,13 @@ int fxh_init(int device, int conv_grad_mode, const fx_pool_config* cfg) {
     });
 }
 void fxh_shutdown(void) { BackendManager::get().shutdown(); }
+// 0 = mathematical conv gradients, 1 = the CPU backend's literal arithmetic; read by every later deconv2d / cross_correlation2d
+int fxh_set_conv_grad_mode(int mode) {
+    return guarded([&] {
+        if (mode != 0 && mode != 1) throw Error("conv gradient mode must be 0 or 1");
+        BackendManager::get().conv_grad_mode = mode;
+    });
+}
 
 void* fxh_model_create(int dtype, const char* spec, const char* optimizer, int literal_engine /* engine mode 0, 1 or 2 */, const void* const* params, int n_params) {
     ModelBase* m = nullptr;
@@ -251,14 +294,26 @@ int fxh_model_set_batch(void* m, const void* x, const int64_t* xshape, int xnd, 
     });
 }
 int fxh_model_train_step(void* m, double* loss) {
-    return guarded([&] { *loss = static_cast<ModelBase*>(m)->train_step(); });
+    return guarded([&] { *loss = static_cast<ModelBase*>(m)->train_step(true); });
+}
+// loss_kind 0 = CCELoss, 1 = Sum over the prediction; input_requires_grad: the batch is a leaf with a gradient
+int fxh_model_configure(void* m, int loss_kind, int input_requires_grad) {
+    return guarded([&] { static_cast<ModelBase*>(m)->configure(loss_kind, input_requires_grad != 0); });
+}
+// zero_gradients -> forward -> loss -> backward, no optimizer step
+int fxh_model_backward(void* m, double* loss) {
+    return guarded([&] { *loss = static_cast<ModelBase*>(m)->train_step(false); });
+}
+int64_t fxh_model_input_numel(void* m) { return static_cast<ModelBase*>(m)->input_numel(); }
+int fxh_model_get_input_grad(void* m, void* host) {
+    return guarded([&] { static_cast<ModelBase*>(m)->get_input_grad(host); });
 }
 // n steps back to back; wall time covers forward + backward + optimizer step of every step and one final sync
 int fxh_model_train_steps(void* m, int n, double* last_loss, double* total_ms) {
     return guarded([&] {
         fx_ok(fx_sync(BackendManager::get().ctx()));
         const auto t0 = std::chrono::steady_clock::now();
-        for (int i = 0; i < n; ++i) *last_loss = static_cast<ModelBase*>(m)->train_step();
+        for (int i = 0; i < n; ++i) *last_loss = static_cast<ModelBase*>(m)->train_step(true);
         fx_ok(fx_sync(BackendManager::get().ctx()));
         *total_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     });

@@ -44,6 +44,12 @@ lib.fxh_model_optimizer_state.argtypes = [C.c_void_p, C.POINTER(C.c_void_p), C.P
 lib.fxh_free.argtypes = [C.c_void_p]
 lib.fxh_free.restype = None
 lib.fxh_model_load_optimizer_state.argtypes = [C.c_void_p, C.c_char_p, C.c_int64]
+lib.fxh_set_conv_grad_mode.argtypes = [C.c_int]
+lib.fxh_model_configure.argtypes = [C.c_void_p, C.c_int, C.c_int]
+lib.fxh_model_backward.argtypes = [C.c_void_p, C.POINTER(C.c_double)]
+lib.fxh_model_input_numel.argtypes = [C.c_void_p]
+lib.fxh_model_input_numel.restype = C.c_int64
+lib.fxh_model_get_input_grad.argtypes = [C.c_void_p, C.c_void_p]
 lib.fxh_pool_stats.argtypes = [C.c_int, C.POINTER(capi.PoolStats)]
 
 
@@ -58,6 +64,11 @@ def _check(rc):
 
 def init(device=0, conv_grad_mode=0, pool_config=None):
     _check(lib.fxh_init(device, conv_grad_mode, C.byref(pool_config) if pool_config is not None else None))
+
+
+def set_conv_grad_mode(mode):
+    """0 = mathematical conv gradients (default), 1 = the CPU backend's literal arithmetic."""
+    _check(lib.fxh_set_conv_grad_mode(int(mode)))
 
 
 def shutdown():
@@ -101,6 +112,22 @@ class Model:
         loss = C.c_double(0)
         _check(lib.fxh_model_train_step(self.h, C.byref(loss)))
         return loss.value
+
+    def configure(self, loss="cce", input_requires_grad=False):
+        """loss: 'cce' (softmax cross-entropy against the targets) or 'sum' (sum of every element of the prediction)."""
+        _check(lib.fxh_model_configure(self.h, {"cce": 0, "sum": 1}[loss], int(input_requires_grad)))
+
+    def backward(self):
+        """zero_gradients, forward, loss, backward -- no optimizer step.  Returns the loss."""
+        loss = C.c_double(0)
+        _check(lib.fxh_model_backward(self.h, C.byref(loss)))
+        return loss.value
+
+    def input_grad(self, shape):
+        out = np.empty(shape, self.dtype)
+        assert out.size == lib.fxh_model_input_numel(self.h)
+        _check(lib.fxh_model_get_input_grad(self.h, out.ctypes.data))
+        return out
 
     def train_steps(self, n):
         loss, ms = C.c_double(0), C.c_double(0)

@@ -10,8 +10,11 @@
 //   im2col, col2im(layout 0/1)    : closed form + brute force + window-count identities (tests/test_oracle_*.py)
 //   conv2d forward                : reference-held PyTorch vector src/ops/mod.rs:743-801 and torch CPU conv2d
 //   conv2d dgrad/wgrad "correct"  : torch.autograd of conv2d (equals the reference CUDA kernels)
-//   conv2d dgrad/wgrad "literal"  : PARITY UNPINNED for batch > 1 (no reference test holds values; equality
-//                                   with the correct mode at batch 1 is the only check)
+//   conv2d dgrad/wgrad "literal"  : for batch > 1, rebuilt from independent routines: numpy float64 matmul on the flat
+//                                   [Cout, B*L] re-read of grad_output, torch unfold as im2col, torch fold on the
+//                                   batch-major [B, C*kh*kw, L] re-read of the column matrix (the two re-reads are
+//                                   the only thing taken from convolutions.rs:122-127, 292-293, 323-326); equality
+//                                   with the correct mode at batch 1 and, for the weight gradient, at Cout = 1
 //   gemm                          : 2x2 vectors src/ops/mod.rs:516-529, numpy float64 matmul
 //   reductions                    : 2x2 vectors src/ops/mod.rs:544-618, numpy; summation ORDER at real
 //                                   sizes is PARITY UNPINNED (ndarray/matrixmultiply sources are not in the

@@ -225,12 +225,20 @@ class Sequential:
                 h = h.reshape(h.shape[0], -1)
         return h, tape
 
-    def loss_and_grads(self, x, y):
+    def loss_and_grads(self, x, y, loss_kind="cce", want_input_grad=False):
+        """loss_kind 'cce': CCELoss against y.  'sum': Sum::new() over every element of the prediction
+        (ops/reduction.rs:52-140: every axis from last to first, cpu.rs:1183-1211; its gradient is
+        expand_reduction(None) = full(input_shape, grad.first()), reduction.rs:9-50).
+        want_input_grad: also return the gradient that reaches the batch (a leaf created with requires_grad)."""
         dt = self.dtype.type
         pred, tape = self.forward(x)
-        y = np.ascontiguousarray(y, dtype=self.dtype)
-        loss, s = softmax_ce_forward(pred, y)
-        g = softmax_ce_backward(s, y, np.ones((), self.dtype))
+        if loss_kind == "sum":
+            loss = orc.reduce("sum", pred)
+            g = np.full(pred.shape, dt(1), self.dtype)
+        else:
+            y = np.ascontiguousarray(y, dtype=self.dtype)
+            loss, s = softmax_ce_forward(pred, y)
+            g = softmax_ce_backward(s, y, np.ones((), self.dtype))
         grads = [None] * len(self.params)
         for rec in reversed(tape):
             kind = rec[0]
@@ -265,6 +273,8 @@ class Sequential:
                     g = orc.binary("mul", g, rec[1])                                      # Mul::gradient wrt the input
             else:
                 g = g.reshape(rec[1])
+        if want_input_grad:
+            return loss.item(), grads, g
         return loss.item(), grads
 
 

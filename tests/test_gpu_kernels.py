@@ -410,7 +410,7 @@ def test_conv2d_fwd_dgrad_wgrad_vs_oracle(ctx, orc, dtype):
         assert rel_err(y, orc.conv2d_fwd(x, w, (s, s), (p, p))) <= tol * 8
         assert rel_err(dxg, orc.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), 0)) <= tol * 8
         assert rel_err(dwg, orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 0)) <= tol * 8
-        if B * Cin * H * W <= 200000:
+        if True:  # the CPU backend's literal gradients at every shape
             lit_dx = ctx.conv2d_dgrad(dg_, dw_, x.shape, (s, s), (p, p), 1).numpy()
             lit_dw = ctx.conv2d_wgrad(dx_, dg_, w.shape, (s, s), (p, p), 1).numpy()
             assert rel_err(lit_dx, orc.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), 1)) <= tol * 8, ("literal dgrad", case)

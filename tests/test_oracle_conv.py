@@ -148,3 +148,68 @@ def test_conv1d_analogue_vector_from_dev_notes():
     for mode in (0, 1):  # batch 1: literal and correct modes must agree
         assert orc.conv2d_wgrad(x, g, w.shape, (1, 1), (0, 0), mode).ravel().tolist() == [20.0, 15.0, 15.0]
         assert orc.conv2d_dgrad(g, w, x.shape, (1, 1), (0, 0), mode).ravel().tolist() == [1.0, 1.5, 0.5, -0.5, -1.0]
+
+
+LITERAL_CASES = [  # B, Cin, H, W, Cout, k, s, p
+    (2, 2, 5, 5, 3, 3, 1, 1), (3, 3, 8, 6, 4, 3, 1, 1), (2, 3, 9, 7, 5, 3, 2, 1), (3, 1, 7, 7, 2, 2, 2, 0),
+    (2, 4, 6, 6, 3, 1, 1, 0), (4, 1, 28, 28, 8, 3, 1, 1),
+]
+
+
+@pytest.mark.parametrize("case", LITERAL_CASES)
+def test_literal_grads_batch_gt1_vs_composed_torch_and_numpy(case):
+    """The CPU backend's literal gradients for batch > 1, rebuilt from independent routines.
+
+    Only the two flat reinterpretations are taken from the reference: grad_output [B, OC, oh, ow] is re-read as a
+    row-major [OC, B*L] matrix (convolutions.rs:292-293, 323-326) and the column matrix [C*kh*kw, B*L] produced by the
+    product is re-read by col2im with a batch-major flat index, i.e. as [B, C*kh*kw, L] (convolutions.rs:122-127).
+    Everything else is numpy's float64 matmul and torch's unfold / fold.  A wrong stride, a transposed operand or a
+    channel-major read of the column matrix fails this comparison (the last check below makes sure the literal result
+    is NOT the mathematical gradient, so the test cannot pass by accident through the correct path)."""
+    B, Cin, H, W, Cout, k, s, p = case
+    rng = np.random.default_rng(100 + B * 7 + Cin)
+    x = rng.uniform(-1, 1, (B, Cin, H, W))
+    w = rng.standard_normal((Cout, Cin, k, k)) * np.sqrt(2.0 / (Cin * k * k))
+    oh, ow = orc.out_hw(H, W, k, k, s, s, p, p)
+    L = oh * ow
+    g = rng.standard_normal((B, Cout, oh, ow))
+    g2d = g.reshape(Cout, B * L)                      # the flat reinterpretation
+    w2d = w.reshape(Cout, Cin * k * k)
+
+    # weight gradient: g2d . im2col(x)^T, with torch.unfold as the independent im2col
+    unf = F.unfold(torch.from_numpy(x), k, padding=p, stride=s).numpy()        # [B, CKK, L]
+    col = unf.transpose(1, 0, 2).reshape(Cin * k * k, B * L)                    # [CKK, (b, l)]
+    dw_ref = (g2d @ col.T).reshape(w.shape)
+    dw = orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 1)
+    np.testing.assert_allclose(dw, dw_ref, rtol=0, atol=1e-12 * max(1.0, np.abs(dw_ref).max()))
+
+    # data gradient: fold of (w2d^T . g2d) re-read batch-major
+    colm = (w2d.T @ g2d).reshape(-1)                                            # row-major [CKK, B*L], flattened
+    dx_ref = F.fold(torch.from_numpy(colm.reshape(B, Cin * k * k, L).copy()), (H, W), k, padding=p, stride=s).numpy()
+    dx = orc.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), 1)
+    np.testing.assert_allclose(dx, dx_ref, rtol=0, atol=1e-12 * max(1.0, np.abs(dx_ref).max()))
+
+    # float32 follows the same path within its own rounding
+    dw32 = orc.conv2d_wgrad(x.astype(np.float32), g.astype(np.float32), w.shape, (s, s), (p, p), 1)
+    dx32 = orc.conv2d_dgrad(g.astype(np.float32), w.astype(np.float32), x.shape, (s, s), (p, p), 1)
+    assert np.abs(dw32 - dw_ref).max() <= 1e-5 * max(1.0, np.abs(dw_ref).max())
+    assert np.abs(dx32 - dx_ref).max() <= 1e-5 * max(1.0, np.abs(dx_ref).max())
+
+    # and it is not the mathematical gradient (batch > 1), so the literal path really is a different function
+    if Cout > 1:
+        assert np.abs(dw - orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 0)).max() > 1e-3
+    assert np.abs(dx - orc.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), 0)).max() > 1e-3
+
+
+def test_literal_wgrad_equals_correct_for_one_output_channel():
+    """With Cout = 1 the flat [OC, B*L] re-read of grad_output is the identity, so the literal weight gradient is the
+    mathematical one for any batch (torch.autograd as the independent value)."""
+    rng = np.random.default_rng(9)
+    x = rng.uniform(-1, 1, (3, 2, 6, 6))
+    w = rng.standard_normal((1, 2, 3, 3))
+    tx, tw = torch.from_numpy(x), torch.from_numpy(w).requires_grad_(True)
+    ty = F.conv2d(tx, tw, stride=1, padding=1)
+    g = rng.standard_normal(tuple(ty.shape))
+    ty.backward(torch.from_numpy(g))
+    dw = orc.conv2d_wgrad(x, g, w.shape, (1, 1), (1, 1), 1)
+    np.testing.assert_allclose(dw, tw.grad.numpy(), rtol=0, atol=1e-12)

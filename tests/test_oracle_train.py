@@ -95,3 +95,51 @@ def test_sgd_and_adam_closed_forms():
         tw.grad = torch.tensor(g)
         topt.step()
     np.testing.assert_allclose(m.params[0], tw.detach().numpy(), rtol=0, atol=1e-9)
+
+
+def c1_problem(dtype, batch=32, seed=1):
+    """The conv plumbing configuration: x U(-1,1) [B,1,28,28], Kaiming-normal W [8,1,3,3] (std = sqrt(2/9)), zero bias."""
+    rng = np.random.default_rng(seed)
+    x = rng.uniform(-1, 1, (batch, 1, 28, 28)).astype(dtype)
+    w = (rng.standard_normal((8, 1, 3, 3)) * np.sqrt(2.0 / 9.0)).astype(dtype)
+    return x, w, np.zeros(8, dtype)
+
+
+C1 = "conv 1 8 3 1 1; relu"
+
+
+@pytest.mark.parametrize("dtype,tol", [(np.float64, 1e-12), (np.float32, 1e-5)])
+def test_c1_relu_sum_backward_matches_torch(dtype, tol):
+    """sum(relu(conv(x) + b)).backward(): loss, input, weight and bias gradients against torch autograd (float64)."""
+    x, w, b = c1_problem(dtype)
+    model = otrain.Sequential(C1, [w, b], dtype, conv_mode=0)
+    loss, grads, gx = model.loss_and_grads(x, None, loss_kind="sum", want_input_grad=True)
+    tx = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    tw = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+    tb = torch.tensor(b, dtype=torch.float64, requires_grad=True)
+    tl = F.relu(F.conv2d(tx, tw, tb, stride=1, padding=1)).sum()
+    tl.backward()
+    assert abs(loss - tl.item()) <= tol * abs(tl.item())
+    for got, ref in ((gx, tx.grad), (grads[0], tw.grad), (grads[1], tb.grad)):
+        ref = ref.numpy()
+        assert got.shape == ref.shape
+        assert np.abs(got - ref).max() <= tol * max(1.0, np.abs(ref).max())
+
+
+def test_c1_literal_mode_gradients_composed():
+    """The same graph with the CPU backend's literal conv gradients (batch 32): bias gradient and loss are unchanged,
+    the input / weight gradients equal the flat-reinterpretation composition built from torch unfold / fold."""
+    x, w, b = c1_problem(np.float64)
+    model = otrain.Sequential(C1, [w, b], np.float64, conv_mode=1)
+    loss, grads, gx = model.loss_and_grads(x, None, loss_kind="sum", want_input_grad=True)
+    ref0 = otrain.Sequential(C1, [w, b], np.float64, conv_mode=0)
+    loss0, grads0, _ = ref0.loss_and_grads(x, None, loss_kind="sum", want_input_grad=True)
+    assert loss == loss0 and np.array_equal(grads[1], grads0[1])
+    B, L = 32, 28 * 28
+    pre = F.conv2d(torch.tensor(x), torch.tensor(w), torch.tensor(b), padding=1)
+    g = (pre > 0).double().numpy()                                 # d sum(relu(pre)) / d pre
+    g2d = g.reshape(8, B * L)
+    col = F.unfold(torch.tensor(x), 3, padding=1).numpy().transpose(1, 0, 2).reshape(9, B * L)
+    np.testing.assert_allclose(grads[0], (g2d @ col.T).reshape(w.shape), rtol=0, atol=1e-9)
+    colm = (w.reshape(8, 9).T @ g2d).reshape(B, 9, L)
+    np.testing.assert_allclose(gx, F.fold(torch.tensor(colm.copy()), (28, 28), 3, padding=1).numpy(), rtol=0, atol=1e-11)
