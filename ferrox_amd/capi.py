@@ -142,6 +142,12 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_adam_step_multi_{_s}", _vp, _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_i64),
          *([_ct] * 7))
     _sig(f"fx_sgd_step_multi_{_s}", _vp, _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_i64), _ct)
+    _sig(f"fx_adam_amsgrad_step_{_s}", _vp, _vp, _vp, _vp, _vp, _vp, _i64, *([_ct] * 7))
+    _sig(f"fx_sgd_momentum_step_{_s}", _vp, _vp, _vp, _vp, _i64, _ct, _ct, _ct, _int)
+    _sig(f"fx_adam_amsgrad_step_multi_{_s}", _vp, _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
+         C.POINTER(_vp), C.POINTER(_i64), *([_ct] * 7))
+    _sig(f"fx_sgd_momentum_step_multi_{_s}", _vp, _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_i64),
+         _ct, _ct, _ct, _int)
 
 _sig("fx_reduce_max_noalloc_f32", _vp, _vp, _vp, _vp, _i64, _i64, _i64)
 NOALLOC_SCRATCH_BYTES = 4 << 20
@@ -538,6 +544,14 @@ class Context:
         ns = (C.c_int64 * k)(*[a.size for a in ps])
         dt = ps[0].dtype if k else np.float32
         check(self._fn("sgd_step_multi", dt)(self.h, k, tab(ps), tab(gs), ns, float(lr)))
+
+    def adam_amsgrad_step(self, p, g, m, v, vmax, lr, beta1, beta2, eps, wd, bc1, bc2):
+        check(self._fn("adam_amsgrad_step", p.dtype)(self.h, p.ptr, g.ptr, m.ptr, v.ptr, vmax.ptr, p.size, lr, beta1, beta2, eps,
+                                                     wd, bc1, bc2))
+
+    def sgd_momentum_step(self, p, g, buf, lr, momentum, wd, nesterov):
+        check(self._fn("sgd_momentum_step", p.dtype)(self.h, p.ptr, g.ptr, buf.ptr if buf is not None else None, p.size, lr,
+                                                     momentum, wd, int(nesterov)))
 
     def sgd_step(self, p, g, lr):
         check(self._fn("sgd_step", p.dtype)(self.h, p.ptr, g.ptr, p.size, lr))

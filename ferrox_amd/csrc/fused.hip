@@ -7,7 +7,8 @@
 //   softmax_ce    loss and d loss / d logits    replaces the 7 forward / 7 backward ops of CCELoss
 //                                               (nn/losses/classification.rs:191-257, ops/batched.rs:106-131)
 //   adam_step     in-place Adam update          replaces ~14 kernels per parameter (nn/optim/adam.rs:288-358)
-//   sgd_step      in-place p -= lr*g            replaces nn/optim/sgd.rs:210-245 (momentum 0, weight decay 0)
+//   sgd_step      in-place SGD update (plain, or with L2 weight decay / momentum / Nesterov)   replaces nn/optim/sgd.rs:128-245
+//   adam_amsgrad  Adam with the running maximum of the second moment (adam.rs:203-221)
 #include "common.hpp"
 
 namespace {
@@ -302,18 +303,49 @@ int softmax_ce_bwd(fx_ctx* c, const T* probs, const T* targets, const T* gup, T*
 }
 
 // ---- optimizers, in place ----------------------------------------------------------------------------------------
+// Element updates in the composed kernels' operation order (this file is built without a*b+c contraction), so the
+// results have the bits of the op-by-op path.
+//   Adam  (nn/optim/adam.rs:136-358): m = m*b1 + g*(1-b1); v = v*b2 + (g*g)*(1-b2); AMSGrad: vmax = max(vmax, v)
+//         (cpu.rs:717-739: a >= b ? a : b) and vmax takes v's place below; p = p - ((m/bc1)/(sqrt(v/bc2)+eps))*lr
+//         [- p*(wd*lr)]
+//   SGD   (nn/optim/sgd.rs:128-245): e = g [+ p*wd]; momentum != 0: buf = buf*mu + e, u = nesterov ? buf*mu + e : buf;
+//         else u = e; p = p - u*lr
+template <typename T> struct OptHyper {
+    T lr, beta1, beta2, eps, wd, bc1, bc2;  // SGD: beta1 = momentum
+    int flag;                               // Adam: amsgrad; SGD: nesterov
+};
+
 template <typename T>
-__device__ __forceinline__ void adam_element(T* p, const T* g, T* m, T* v, i64 i, T lr, T beta1, T beta2, T eps, T wd, T bc1, T bc2) {
+__device__ __forceinline__ void adam_element(T* p, const T* g, T* m, T* v, T* vmax, i64 i, const OptHyper<T>& h) {
     const T gi = g[i], w = p[i];
-    const T m1 = m[i] * beta1 + gi * (T(1) - beta1);
-    const T m2 = v[i] * beta2 + (gi * gi) * (T(1) - beta2);
+    const T m1 = m[i] * h.beta1 + gi * (T(1) - h.beta1);
+    T m2 = v[i] * h.beta2 + (gi * gi) * (T(1) - h.beta2);
     m[i] = m1;
     v[i] = m2;
-    const T denom = dev_sqrt<T>(m2 / bc2) + eps;
-    const T update = ((m1 / bc1) / denom) * lr;
+    if (vmax) {
+        const T old = vmax[i];
+        m2 = old >= m2 ? old : m2;
+        vmax[i] = m2;
+    }
+    const T denom = dev_sqrt<T>(m2 / h.bc2) + h.eps;
+    const T update = ((m1 / h.bc1) / denom) * h.lr;
     T nw = w - update;
-    if (wd != T(0)) nw = nw - w * (wd * lr);
+    if (h.wd != T(0)) nw = nw - w * (h.wd * h.lr);
     p[i] = nw;
+}
+
+template <typename T>
+__device__ __forceinline__ void sgd_element(T* p, const T* g, T* buf, i64 i, const OptHyper<T>& h) {
+    const T w = p[i];
+    T e = g[i];
+    if (h.wd != T(0)) e = e + w * h.wd;
+    T u = e;
+    if (buf) {  // momentum != 0
+        const T b = buf[i] * h.beta1 + e;
+        buf[i] = b;
+        u = h.flag ? b * h.beta1 + e : b;
+    }
+    p[i] = w - u * h.lr;
 }
 
 // Every parameter of a model in one launch: the tensor table travels in the kernel arguments (no device-side
@@ -322,26 +354,28 @@ constexpr int MULTI_MAX = 24;
 template <typename T> struct MultiTensors {
     T* p[MULTI_MAX];
     const T* g[MULTI_MAX];
-    T* m[MULTI_MAX];
-    T* v[MULTI_MAX];
+    T* m[MULTI_MAX];   // Adam: first moment; SGD: momentum buffer (null without momentum)
+    T* v[MULTI_MAX];   // Adam: second moment
+    T* x[MULTI_MAX];   // Adam with AMSGrad: running maximum of the second moment (null otherwise)
     i64 n[MULTI_MAX];
     unsigned first[MULTI_MAX + 1];
     int count;
 };
 
 template <typename T, bool ADAM>
-__global__ __launch_bounds__(256) void multi_step_kernel(const MultiTensors<T> tt, T lr, T beta1, T beta2, T eps, T wd, T bc1, T bc2) {
+__global__ __launch_bounds__(256) void multi_step_kernel(const MultiTensors<T> tt, const OptHyper<T> h) {
     int t = 0;
     while (t + 1 < tt.count && blockIdx.x >= tt.first[t + 1]) ++t;  // wave-uniform
     const i64 i = (i64)(blockIdx.x - tt.first[t]) * 256 + threadIdx.x;
     if (i >= tt.n[t]) return;
-    if (ADAM) adam_element<T>(tt.p[t], tt.g[t], tt.m[t], tt.v[t], i, lr, beta1, beta2, eps, wd, bc1, bc2);
-    else tt.p[t][i] = tt.p[t][i] - tt.g[t][i] * lr;
+    if (ADAM) adam_element<T>(tt.p[t], tt.g[t], tt.m[t], tt.v[t], tt.x[t], i, h);
+    else sgd_element<T>(tt.p[t], tt.g[t], tt.m[t], i, h);
 }
 
+// m / v / x: tables that may be null as a whole (SGD without momentum; Adam without AMSGrad)
 template <typename T, bool ADAM>
-int multi_step(fx_ctx* c, int count, T* const* p, const T* const* g, T* const* m, T* const* v, const int64_t* n, T lr, T beta1, T beta2,
-               T eps, T wd, T bc1, T bc2, const char* what) {
+int multi_step(fx_ctx* c, int count, T* const* p, const T* const* g, T* const* m, T* const* v, T* const* x, const int64_t* n,
+               const OptHyper<T>& h, const char* what) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(count >= 0, "%s: negative tensor count", what);
     FX_REQUIRE(count == 0 || (p && g && n && (!ADAM || (m && v))), "%s: null table", what);
@@ -349,13 +383,13 @@ int multi_step(fx_ctx* c, int count, T* const* p, const T* const* g, T* const* m
         MultiTensors<T> tt;
         tt.count = 0;
         i64 blocks = 0;
-        for (int k = base; k < count && tt.count < MULTI_MAX; ++k) {
+        for (int k = base; k < count && k < base + MULTI_MAX; ++k) {
             FX_REQUIRE(n[k] >= 0, "%s: negative element count", what);
             if (n[k] == 0) continue;
-            FX_REQUIRE(p[k] && g[k] && (!ADAM || (m[k] && v[k])), "%s: null pointer in tensor %d", what, k);
+            FX_REQUIRE(p[k] && g[k] && (!m || m[k]) && (!v || v[k]) && (!x || x[k]), "%s: null pointer in tensor %d", what, k);
             const int t = tt.count++;
             tt.p[t] = p[k]; tt.g[t] = g[k];
-            tt.m[t] = ADAM ? m[k] : nullptr; tt.v[t] = ADAM ? v[k] : nullptr;
+            tt.m[t] = m ? m[k] : nullptr; tt.v[t] = v ? v[k] : nullptr; tt.x[t] = x ? x[k] : nullptr;
             tt.n[t] = n[k];
             tt.first[t] = (unsigned)blocks;
             blocks += fx::ceil_div(n[k], (i64)256);
@@ -363,49 +397,36 @@ int multi_step(fx_ctx* c, int count, T* const* p, const T* const* g, T* const* m
         }
         if (tt.count == 0) continue;
         tt.first[tt.count] = (unsigned)blocks;
-        multi_step_kernel<T, ADAM><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(tt, lr, beta1, beta2, eps, wd, bc1, bc2);
+        multi_step_kernel<T, ADAM><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(tt, h);
         FX_LAUNCH_CHECK();
     }
     return FX_OK;
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void adam_step_kernel(T* __restrict__ p, const T* __restrict__ g, T* __restrict__ m, T* __restrict__ v,
-                                                        i64 n, T lr, T beta1, T beta2, T eps, T wd, T bc1, T bc2) {
-    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) adam_element<T>(p, g, m, v, i, lr, beta1, beta2, eps, wd, bc1, bc2);
+int adam_hyper(OptHyper<T>& h, T lr, T beta1, T beta2, T eps, T wd, T bc1, T bc2, int amsgrad) {
+    h.lr = lr; h.beta1 = beta1; h.beta2 = beta2; h.eps = eps; h.wd = wd; h.bc1 = bc1; h.bc2 = bc2; h.flag = amsgrad;
+    return FX_OK;
 }
-
 template <typename T>
-int adam_step(fx_ctx* c, T* p, const T* g, T* m, T* v, i64 n, T lr, T beta1, T beta2, T eps, T wd, T bc1, T bc2) {
-    FX_CHECK_CTX(c);
-    FX_REQUIRE(n >= 0, "fx_adam_step: negative element count");
-    if (n == 0) return FX_OK;
-    FX_REQUIRE(p && g && m && v, "fx_adam_step: null pointer");
-    const i64 blocks = fx::ceil_div(n, (i64)256);
-    FX_REQUIRE(blocks <= 0x7fffffff, "fx_adam_step: too many elements");
-    adam_step_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(p, g, m, v, n, lr, beta1, beta2, eps, wd, bc1, bc2);
-    FX_LAUNCH_CHECK();
+int sgd_hyper(OptHyper<T>& h, T lr, T momentum, T wd, int nesterov, bool have_buf, const char* what) {
+    FX_REQUIRE((momentum != T(0)) == have_buf, "%s: a momentum buffer goes with a nonzero momentum, and only with one", what);
+    h.lr = lr; h.beta1 = momentum; h.beta2 = T(0); h.eps = T(0); h.wd = wd; h.bc1 = T(1); h.bc2 = T(1); h.flag = nesterov;
     return FX_OK;
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void sgd_step_kernel(T* __restrict__ p, const T* __restrict__ g, i64 n, T lr) {
-    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) p[i] = p[i] - g[i] * lr;
+int adam_step(fx_ctx* c, T* p, const T* g, T* m, T* v, T* vmax, i64 n, T lr, T beta1, T beta2, T eps, T wd, T bc1, T bc2, const char* what) {
+    OptHyper<T> h;
+    adam_hyper(h, lr, beta1, beta2, eps, wd, bc1, bc2, vmax != nullptr);
+    return multi_step<T, true>(c, 1, &p, &g, &m, &v, vmax ? &vmax : nullptr, &n, h, what);
 }
 
 template <typename T>
-int sgd_step(fx_ctx* c, T* p, const T* g, i64 n, T lr) {
-    FX_CHECK_CTX(c);
-    FX_REQUIRE(n >= 0, "fx_sgd_step: negative element count");
-    if (n == 0) return FX_OK;
-    FX_REQUIRE(p && g, "fx_sgd_step: null pointer");
-    const i64 blocks = fx::ceil_div(n, (i64)256);
-    FX_REQUIRE(blocks <= 0x7fffffff, "fx_sgd_step: too many elements");
-    sgd_step_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(p, g, n, lr);
-    FX_LAUNCH_CHECK();
-    return FX_OK;
+int sgd_step(fx_ctx* c, T* p, const T* g, T* buf, i64 n, T lr, T momentum, T wd, int nesterov, const char* what) {
+    OptHyper<T> h;
+    if (int rc = sgd_hyper(h, lr, momentum, wd, nesterov, buf != nullptr, what)) return rc;
+    return multi_step<T, false>(c, 1, &p, &g, buf ? &buf : nullptr, nullptr, nullptr, &n, h, what);
 }
 
 }  // namespace
@@ -432,18 +453,51 @@ int sgd_step(fx_ctx* c, T* p, const T* g, i64 n, T lr) {
     }                                                                                                                  \
     extern "C" int fx_adam_step_##S(fx_ctx* c, T* p, const T* g, T* m, T* v, int64_t n, T lr, T beta1, T beta2, T eps, \
                                     T wd, T bc1, T bc2) {                                                              \
-        return adam_step<T>(c, p, g, m, v, n, lr, beta1, beta2, eps, wd, bc1, bc2);                                    \
+        FX_REQUIRE(n == 0 || (p && g && m && v), "fx_adam_step: null pointer");                                        \
+        return adam_step<T>(c, p, g, m, v, nullptr, n, lr, beta1, beta2, eps, wd, bc1, bc2, "fx_adam_step");           \
     }                                                                                                                  \
-    extern "C" int fx_sgd_step_##S(fx_ctx* c, T* p, const T* g, int64_t n, T lr) { return sgd_step<T>(c, p, g, n, lr); } \
+    extern "C" int fx_adam_amsgrad_step_##S(fx_ctx* c, T* p, const T* g, T* m, T* v, T* vmax, int64_t n, T lr, T beta1, \
+                                            T beta2, T eps, T wd, T bc1, T bc2) {                                      \
+        FX_REQUIRE(n == 0 || (p && g && m && v && vmax), "fx_adam_amsgrad_step: null pointer");                        \
+        return adam_step<T>(c, p, g, m, v, vmax, n, lr, beta1, beta2, eps, wd, bc1, bc2, "fx_adam_amsgrad_step");      \
+    }                                                                                                                  \
+    extern "C" int fx_sgd_step_##S(fx_ctx* c, T* p, const T* g, int64_t n, T lr) {                                     \
+        FX_REQUIRE(n == 0 || (p && g), "fx_sgd_step: null pointer");                                                   \
+        return sgd_step<T>(c, p, g, nullptr, n, lr, T(0), T(0), 0, "fx_sgd_step");                                     \
+    }                                                                                                                  \
+    extern "C" int fx_sgd_momentum_step_##S(fx_ctx* c, T* p, const T* g, T* buf, int64_t n, T lr, T momentum,          \
+                                            T weight_decay, int nesterov) {                                            \
+        FX_REQUIRE(n == 0 || (p && g), "fx_sgd_momentum_step: null pointer");                                          \
+        return sgd_step<T>(c, p, g, buf, n, lr, momentum, weight_decay, nesterov, "fx_sgd_momentum_step");             \
+    }                                                                                                                  \
     extern "C" int fx_adam_step_multi_##S(fx_ctx* c, int count, T* const* p, const T* const* g, T* const* m,           \
                                           T* const* v, const int64_t* n, T lr, T beta1, T beta2, T eps, T wd, T bc1,   \
                                           T bc2) {                                                                     \
-        return multi_step<T, true>(c, count, p, g, m, v, n, lr, beta1, beta2, eps, wd, bc1, bc2, "fx_adam_step_multi"); \
+        OptHyper<T> h;                                                                                                 \
+        adam_hyper(h, lr, beta1, beta2, eps, wd, bc1, bc2, 0);                                                         \
+        return multi_step<T, true>(c, count, p, g, m, v, nullptr, n, h, "fx_adam_step_multi");                         \
+    }                                                                                                                  \
+    extern "C" int fx_adam_amsgrad_step_multi_##S(fx_ctx* c, int count, T* const* p, const T* const* g, T* const* m,   \
+                                                  T* const* v, T* const* vmax, const int64_t* n, T lr, T beta1,        \
+                                                  T beta2, T eps, T wd, T bc1, T bc2) {                                \
+        FX_REQUIRE(count == 0 || vmax, "fx_adam_amsgrad_step_multi: null table");                                      \
+        OptHyper<T> h;                                                                                                 \
+        adam_hyper(h, lr, beta1, beta2, eps, wd, bc1, bc2, 1);                                                         \
+        return multi_step<T, true>(c, count, p, g, m, v, vmax, n, h, "fx_adam_amsgrad_step_multi");                    \
     }                                                                                                                  \
     extern "C" int fx_sgd_step_multi_##S(fx_ctx* c, int count, T* const* p, const T* const* g, const int64_t* n,       \
                                          T lr) {                                                                       \
-        return multi_step<T, false>(c, count, p, g, nullptr, nullptr, n, lr, T(0), T(0), T(0), T(0), T(1), T(1),       \
-                                    "fx_sgd_step_multi");                                                              \
+        OptHyper<T> h;                                                                                                 \
+        sgd_hyper(h, lr, T(0), T(0), 0, false, "fx_sgd_step_multi");                                                   \
+        return multi_step<T, false>(c, count, p, g, nullptr, nullptr, nullptr, n, h, "fx_sgd_step_multi");             \
+    }                                                                                                                  \
+    extern "C" int fx_sgd_momentum_step_multi_##S(fx_ctx* c, int count, T* const* p, const T* const* g, T* const* buf, \
+                                                  const int64_t* n, T lr, T momentum, T weight_decay, int nesterov) {  \
+        FX_REQUIRE(count == 0 || (momentum != T(0)) == (buf != nullptr),                                               \
+                   "fx_sgd_momentum_step_multi: a momentum buffer table goes with a nonzero momentum, and only with one"); \
+        OptHyper<T> h;                                                                                                 \
+        sgd_hyper(h, lr, momentum, weight_decay, nesterov, momentum != T(0), "fx_sgd_momentum_step_multi");            \
+        return multi_step<T, false>(c, count, p, g, buf, nullptr, nullptr, n, h, "fx_sgd_momentum_step_multi");        \
     }
 
 FX_DEFINE_FUSED(float, f32)

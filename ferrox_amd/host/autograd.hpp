@@ -13,6 +13,7 @@
 #include <cmath>
 #include <functional>
 #include <map>
+#include <optional>
 #include <set>
 
 #include "hip_storage.hpp"
@@ -467,6 +468,12 @@ template <typename T> class AutoFerroxEngine {
         return it->second.tensor.get();
     }
     void zero_gradients() { grads_.clear(); }  // :838-840
+    void clear_gradient(NodeId id) { grads_.erase(id); }  // :858-860
+    void set_gradient(NodeId id, Tensor<T> g) { grads_[id] = std::move(g); }
+    void clip_gradient(NodeId id, T coef) {  // :875-881
+        auto it = grads_.find(id);
+        if (it != grads_.end()) it->second = it->second->mul_scalar(coef);
+    }
     void update_parameter(NodeId id, Tensor<T> t) {  // :845-866
         auto it = nodes_.find(id);
         if (it == nodes_.end()) throw Error("Node " + std::to_string(id) + " not found");
@@ -767,33 +774,90 @@ template <typename T> NodeId cce_loss(AutoFerroxEngine<T>& g, NodeId predictions
 }
 
 // ---- optimizers: src/nn/optim ---------------------------------------------------------------------------------
+// ParameterGroup, src/nn/optim/mod.rs:203-258.  The reference keeps the ids in a HashSet (iteration order arbitrary);
+// here they are kept unique in insertion order.
+template <typename T> struct ParameterGroup {
+    std::vector<NodeId> params;
+    std::optional<T> lr, weight_decay, momentum;
+    std::string name;
+    explicit ParameterGroup(std::string n = "default") : name(std::move(n)) {}
+    void add_param(NodeId id) {
+        if (std::find(params.begin(), params.end(), id) == params.end()) params.push_back(id);
+    }
+    SerializableParameterGroup to_serializable() const {  // From<&ParameterGroup>, mod.rs:189-201 (ids sorted: a HashSet has no order)
+        SerializableParameterGroup g;
+        g.params.assign(params.begin(), params.end());
+        std::sort(g.params.begin(), g.params.end());
+        if (lr) g.lr = (double)*lr;
+        if (weight_decay) g.weight_decay = (double)*weight_decay;
+        if (momentum) g.momentum = (double)*momentum;
+        g.name = name;
+        return g;
+    }
+    static ParameterGroup from_serializable(const SerializableParameterGroup& s) {  // mod.rs:241-257
+        ParameterGroup g(s.name);
+        for (size_t id : s.params) g.add_param(id);
+        if (s.lr) g.lr = (T)*s.lr;
+        if (s.weight_decay) g.weight_decay = (T)*s.weight_decay;
+        if (s.momentum) g.momentum = (T)*s.momentum;
+        return g;
+    }
+};
+
 template <typename T> struct Optimizer {  // trait Optimizer, src/nn/optim/mod.rs:328-378
     virtual ~Optimizer() = default;
     virtual void step(AutoFerroxEngine<T>& g) = 0;
     virtual OptimizerStateDict state_dict() const = 0;
     virtual void load_state_dict(const OptimizerStateDict& sd) = 0;
-    std::vector<NodeId> params;  // the "default" parameter group (Adam::new / SGD::new create exactly one)
+    virtual T get_lr() const = 0;
+    virtual void set_lr(T lr) = 0;
+    std::vector<ParameterGroup<T>> param_groups;  // new() creates the "default" group
+
+    void add_param(size_t group, NodeId id) { param_groups.at(group).add_param(id); }
+    void add_param_group(ParameterGroup<T> group) {
+        if (group.params.empty()) throw Error("Invalid parameter group configuration");
+        param_groups.push_back(std::move(group));
+    }
+    // every node id held by some group
+    std::set<NodeId> all_params() const {
+        std::set<NodeId> r;
+        for (const auto& g : param_groups) r.insert(g.params.begin(), g.params.end());
+        return r;
+    }
 
   protected:
-    void save_groups(OptimizerStateDict& sd) const {  // add_parameter_group, mod.rs:304-311 (HashSet order is arbitrary: sorted here)
-        SerializableParameterGroup g;
-        g.params.assign(params.begin(), params.end());
-        std::sort(g.params.begin(), g.params.end());
-        g.name = "default";
-        sd.parameter_groups.push_back(std::move(g));
+    void save_groups(OptimizerStateDict& sd) const {  // add_parameter_group, mod.rs:304-311
+        for (const auto& g : param_groups) sd.parameter_groups.push_back(g.to_serializable());
     }
     void load_groups(const OptimizerStateDict& sd) {  // param_groups.clear(); push every saved group
-        std::vector<NodeId> restored;
-        for (const auto& g : sd.parameter_groups) restored.insert(restored.end(), g.params.begin(), g.params.end());
-        params = std::move(restored);
+        param_groups.clear();
+        for (const auto& g : sd.parameter_groups) param_groups.push_back(ParameterGroup<T>::from_serializable(g));
     }
     static T hyper(const OptimizerStateDict& sd, const char* name, T current) {
         auto it = sd.hyperparameters.find(name);
         return it == sd.hyperparameters.end() ? current : (T)it->second;
     }
+    // Restores the buffers of one kind.  The reference inserts whatever the file holds; a buffer for a node that no
+    // restored group names could never be used again and a buffer of another shape would be read past its end by a
+    // fused update, so both are errors here.
+    void load_buffers(const OptimizerStateDict& sd, const char* type, std::map<NodeId, Tensor<T>>& into) const {
+        const std::set<NodeId> known = all_params();
+        for (const auto& kv : sd.parameter_buffers) {
+            const TensorBuffer& b = kv.second;
+            if (b.buffer_type != type) continue;
+            if (!known.count(b.node_id))
+                throw Error("optimizer state: buffer '" + std::string(type) + "' names node " + std::to_string(b.node_id) + ", which is in no parameter group");
+            into[b.node_id] = b.template to_tensor<T>();
+        }
+    }
+    static void check_buffer(const HipStorage<T>& buf, const HipStorage<T>& w, const char* type, NodeId id) {
+        if (buf.shape() != w.shape())
+            throw Error("optimizer state: buffer '" + std::string(type) + "' of node " + std::to_string(id) + " has shape " + fmt_shape(buf.shape()) +
+                        ", the parameter has " + fmt_shape(w.shape()));
+    }
 };
 
-// Adam::state_dict / load_state_dict, src/nn/optim/adam.rs:391-556 (no amsgrad), shared by the composed and the fused optimizer
+// Adam::state_dict / load_state_dict, src/nn/optim/adam.rs:391-556, shared by the composed and the fused optimizer
 template <typename T, class Opt> OptimizerStateDict adam_state_dict(const Opt& o) {
     OptimizerStateDict sd;
     sd.optimizer_type = "Adam";
@@ -803,104 +867,184 @@ template <typename T, class Opt> OptimizerStateDict adam_state_dict(const Opt& o
     sd.hyperparameters["beta2"] = (double)o.beta2;
     sd.hyperparameters["eps"] = (double)o.eps;
     sd.hyperparameters["weight_decay"] = (double)o.weight_decay;
-    sd.hyperparameters["amsgrad"] = 0.0;
+    sd.hyperparameters["amsgrad"] = o.amsgrad ? 1.0 : 0.0;
     for (const auto& kv : o.m1) sd.template add_buffer<T>(kv.first, *kv.second, "first_moment");
     for (const auto& kv : o.m2) sd.template add_buffer<T>(kv.first, *kv.second, "second_moment");
+    if (o.amsgrad)
+        for (const auto& kv : o.mmax) sd.template add_buffer<T>(kv.first, *kv.second, "max_second_moment");
     return sd;
 }
-template <typename T, class Opt> void adam_load_state_dict(Opt& o, const OptimizerStateDict& sd) {
-    if (sd.optimizer_type != "Adam") throw Error("Type mismatch: Expected Adam state dict, got " + sd.optimizer_type);
-    o.m1.clear();
-    o.m2.clear();
-    o.step_count = (long)sd.step_count;
-    for (const auto& kv : sd.parameter_buffers) {
-        const TensorBuffer& b = kv.second;
-        if (b.buffer_type == "first_moment") o.m1[b.node_id] = b.template to_tensor<T>();
-        else if (b.buffer_type == "second_moment") o.m2[b.node_id] = b.template to_tensor<T>();
+
+// bias corrections, adam.rs:110-126
+template <typename T> void adam_bias_corrections(T beta1, T beta2, long step_count, T& bc1, T& bc2) {
+    const T stepf = (T)step_count;
+    const T b1p = std::max((T)std::pow(beta1, stepf), (T)1e-8), b2p = std::max((T)std::pow(beta2, stepf), (T)1e-8);
+    bc1 = T(1) - b1p;
+    bc2 = T(1) - b2p;
+}
+
+template <typename T> struct SGD : Optimizer<T> {  // src/nn/optim/sgd.rs:11-360
+    T lr, momentum, weight_decay;
+    bool nesterov;
+    std::map<NodeId, Tensor<T>> momentum_buffers;
+    explicit SGD(T lr_, T momentum_ = T(0), T wd = T(0), bool nesterov_ = false)  // SGD::new, sgd.rs:28-45
+        : lr(lr_), momentum(momentum_), weight_decay(wd), nesterov(nesterov_) {
+        ParameterGroup<T> g("default");
+        g.lr = lr;
+        g.weight_decay = weight_decay;
+        g.momentum = momentum;
+        this->param_groups.push_back(std::move(g));
     }
-}
-
-// SGD::state_dict / load_state_dict, src/nn/optim/sgd.rs:278-360 (momentum 0: no buffers)
-template <typename T, class Opt> OptimizerStateDict sgd_state_dict(const Opt& o) {
-    OptimizerStateDict sd;
-    sd.optimizer_type = "SGD";
-    sd.step_count = 0;
-    sd.hyperparameters["lr"] = (double)o.lr;
-    sd.hyperparameters["momentum"] = 0.0;
-    sd.hyperparameters["weight_decay"] = 0.0;
-    sd.hyperparameters["nesterov"] = 0.0;
-    SerializableParameterGroup g;
-    g.params.assign(o.params.begin(), o.params.end());
-    std::sort(g.params.begin(), g.params.end());
-    g.name = "default";
-    sd.parameter_groups.push_back(std::move(g));
-    return sd;
-}
-inline void sgd_check(const OptimizerStateDict& sd) {
-    if (sd.optimizer_type != "SGD") throw Error("Type mismatch: Expected SGD state dict, got " + sd.optimizer_type);
-}
-
-template <typename T> struct SGD : Optimizer<T> {  // src/nn/optim/sgd.rs:116-245 (momentum 0, weight decay 0 path)
-    T lr;
-    explicit SGD(T lr_) : lr(lr_) {}
-    void step(AutoFerroxEngine<T>& g) override {
-        for (NodeId p : this->params) {
-            const HipStorage<T>* grad = g.get_gradient(p);
-            if (!grad) continue;
-            const HipStorage<T>* w = g.get_tensor(p);
-            Tensor<T> effective = grad->clone_storage();  // apply_weight_decay with rate 0 returns grad.clone()
-            Tensor<T> scaled = effective->mul_scalar(lr); // apply_lr
-            g.update_parameter(p, w->sub(*scaled));
+    T get_lr() const override { return lr; }
+    void set_lr(T v) override {  // sgd.rs:271-276
+        lr = v;
+        for (auto& g : this->param_groups) g.lr = v;
+    }
+    // clip_grad_norm, sgd.rs:56-101: global L2 norm over every group's gradients (one host read per parameter);
+    // when it exceeds max_norm every gradient is scaled by max_norm / norm (engine.clip_gradient).
+    T clip_grad_norm(AutoFerroxEngine<T>& g, T max_norm) {
+        T total_sq = T(0);
+        for (const auto& group : this->param_groups)
+            for (NodeId p : group.params)
+                if (const HipStorage<T>* grad = g.get_gradient(p)) {
+                    Tensor<T> sq = grad->mul(*grad);
+                    total_sq += sq->sum(nullptr, false)->first();
+                }
+        const T total = std::sqrt(total_sq);
+        if (total > max_norm) {
+            const T coef = max_norm / total;
+            for (const auto& group : this->param_groups)
+                for (NodeId p : group.params) g.clip_gradient(p, coef);
+        }
+        return total;
+    }
+    void step(AutoFerroxEngine<T>& g) override {  // sgd.rs:210-245
+        for (const auto& group : this->param_groups) {
+            const T glr = group.lr.value_or(lr), gwd = group.weight_decay.value_or(weight_decay), gmom = group.momentum.value_or(momentum);
+            for (NodeId p : group.params) {
+                const HipStorage<T>* grad = g.get_gradient(p);
+                if (!grad) continue;
+                const HipStorage<T>* w = g.get_tensor(p);
+                if (!w) throw Error("Parameter not found for node " + std::to_string(p));
+                Tensor<T> effective;  // apply_weight_decay, sgd.rs:117-134 (rate 0 returns grad.clone())
+                if (gwd == T(0)) effective = grad->clone_storage();
+                else {
+                    Tensor<T> term = w->mul_scalar(gwd);
+                    effective = grad->add(*term);
+                }
+                Tensor<T> nw;
+                if (gmom != T(0)) {  // compute_update, sgd.rs:173-206
+                    auto it = momentum_buffers.find(p);
+                    if (it == momentum_buffers.end()) it = momentum_buffers.emplace(p, HipStorage<T>::zeros(w->shape())).first;
+                    else this->check_buffer(*it->second, *w, "momentum", p);
+                    {
+                        Tensor<T> scaled = it->second->mul_scalar(gmom);
+                        it->second = scaled->add(*effective);
+                    }
+                    if (nesterov) {
+                        Tensor<T> look = it->second->mul_scalar(gmom);
+                        Tensor<T> update = look->add(*effective);
+                        nw = apply_lr(glr, *w, *update);
+                    } else nw = apply_lr(glr, *w, *it->second);
+                } else nw = apply_lr(glr, *w, *effective);
+                g.update_parameter(p, std::move(nw));
+            }
         }
     }
-    OptimizerStateDict state_dict() const override { return sgd_state_dict<T>(*this); }
-    void load_state_dict(const OptimizerStateDict& sd) override {
-        sgd_check(sd);
+    OptimizerStateDict state_dict() const override {  // sgd.rs:278-322
+        OptimizerStateDict sd;
+        sd.optimizer_type = "SGD";
+        sd.step_count = 0;
+        sd.hyperparameters["lr"] = (double)lr;
+        sd.hyperparameters["momentum"] = (double)momentum;
+        sd.hyperparameters["weight_decay"] = (double)weight_decay;
+        sd.hyperparameters["nesterov"] = nesterov ? 1.0 : 0.0;
+        this->save_groups(sd);
+        for (const auto& kv : momentum_buffers) sd.template add_buffer<T>(kv.first, *kv.second, "momentum");
+        return sd;
+    }
+    void load_state_dict(const OptimizerStateDict& sd) override {  // sgd.rs:324-360
+        if (sd.optimizer_type != "SGD") throw Error("Type mismatch: Expected SGD state dict, got " + sd.optimizer_type);
+        momentum_buffers.clear();
         lr = this->hyper(sd, "lr", lr);
+        momentum = this->hyper(sd, "momentum", momentum);
+        weight_decay = this->hyper(sd, "weight_decay", weight_decay);
+        auto it = sd.hyperparameters.find("nesterov");
+        if (it != sd.hyperparameters.end()) nesterov = it->second > 0.5;
         this->load_groups(sd);
+        this->load_buffers(sd, "momentum", momentum_buffers);
+    }
+
+  protected:
+    static Tensor<T> apply_lr(T glr, const HipStorage<T>& w, const HipStorage<T>& update) {  // sgd.rs:136-150
+        Tensor<T> scaled = update.mul_scalar(glr);
+        return w.sub(*scaled);
     }
 };
 
-template <typename T> struct Adam : Optimizer<T> {  // src/nn/optim/adam.rs:110-358 (no amsgrad)
+template <typename T> struct Adam : Optimizer<T> {  // src/nn/optim/adam.rs:11-556
     T lr, beta1, beta2, eps, weight_decay;
+    bool amsgrad;
     long step_count = 0;
-    std::map<NodeId, Tensor<T>> m1, m2;
-    Adam(T lr_, T b1, T b2, T eps_, T wd) : lr(lr_), beta1(b1), beta2(b2), eps(eps_), weight_decay(wd) {}
-    void step(AutoFerroxEngine<T>& g) override {
+    std::map<NodeId, Tensor<T>> m1, m2, mmax;
+    Adam(T lr_, T b1, T b2, T eps_, T wd, bool amsgrad_ = false)  // Adam::new, adam.rs:40-62
+        : lr(lr_), beta1(b1), beta2(b2), eps(eps_), weight_decay(wd), amsgrad(amsgrad_) {
+        ParameterGroup<T> g("default");
+        g.lr = lr;
+        g.weight_decay = weight_decay;
+        this->param_groups.push_back(std::move(g));
+    }
+    T get_lr() const override { return lr; }
+    void set_lr(T v) override {
+        lr = v;
+        for (auto& g : this->param_groups) g.lr = v;
+    }
+    void step(AutoFerroxEngine<T>& g) override {  // adam.rs:288-358
         step_count += 1;
-        const T stepf = (T)step_count;
-        const T b1p = std::max((T)std::pow(beta1, stepf), (T)1e-8), b2p = std::max((T)std::pow(beta2, stepf), (T)1e-8);
-        const T bc1 = T(1) - b1p, bc2 = T(1) - b2p;
-        for (NodeId p : this->params) {
-            const HipStorage<T>* grad = g.get_gradient(p);
-            if (!grad) continue;
-            Tensor<T> w = g.get_tensor(p)->clone_storage();  // adam.rs:299-302 clones the parameter
-            if (!m1.count(p)) m1[p] = HipStorage<T>::zeros(w->shape());
-            {  // first moment: beta1*m + (1-beta1)*g
-                Tensor<T> a = m1[p]->mul_scalar(beta1), b = grad->mul_scalar(T(1) - beta1);
-                m1[p] = a->add(*b);
+        T bc1, bc2;
+        adam_bias_corrections(beta1, beta2, step_count, bc1, bc2);
+        for (const auto& group : this->param_groups) {
+            const T glr = group.lr.value_or(lr), gwd = group.weight_decay.value_or(weight_decay);
+            for (NodeId p : group.params) {
+                const HipStorage<T>* grad = g.get_gradient(p);
+                if (!grad) continue;
+                if (!g.get_tensor(p)) throw Error("Parameter not found for node " + std::to_string(p));
+                Tensor<T> w = g.get_tensor(p)->clone_storage();  // adam.rs:299-302 clones the parameter
+                if (!m1.count(p)) m1[p] = HipStorage<T>::zeros(w->shape());
+                else this->check_buffer(*m1[p], *w, "first_moment", p);
+                {  // first moment: beta1*m + (1-beta1)*g
+                    Tensor<T> a = m1[p]->mul_scalar(beta1), b = grad->mul_scalar(T(1) - beta1);
+                    m1[p] = a->add(*b);
+                }
+                if (!m2.count(p)) m2[p] = HipStorage<T>::zeros(w->shape());
+                else this->check_buffer(*m2[p], *w, "second_moment", p);
+                {  // second moment: beta2*v + (1-beta2)*g*g
+                    Tensor<T> gg = grad->mul(*grad);
+                    Tensor<T> a = m2[p]->mul_scalar(beta2), b = gg->mul_scalar(T(1) - beta2);
+                    m2[p] = a->add(*b);
+                }
+                Tensor<T> second;
+                if (amsgrad) {  // running maximum of the second moment, adam.rs:203-221
+                    if (!mmax.count(p)) mmax[p] = HipStorage<T>::zeros(w->shape());
+                    else this->check_buffer(*mmax[p], *w, "max_second_moment", p);
+                    mmax[p] = mmax[p]->max(*m2[p]);
+                    second = mmax[p]->clone_storage();
+                } else second = m2[p]->clone_storage();  // take_current_buffer clones
+                Tensor<T> t1 = second->div_scalar(bc2);
+                Tensor<T> t2 = t1->sqrt();
+                Tensor<T> denom = t2->add_scalar(eps);
+                Tensor<T> first = m1[p]->clone_storage();
+                Tensor<T> u1 = first->div_scalar(bc1);
+                Tensor<T> u2 = u1->div(*denom);
+                Tensor<T> update = u2->mul_scalar(glr);
+                Tensor<T> nw;
+                if (gwd != T(0)) {  // decoupled weight decay, adam.rs:259-282
+                    Tensor<T> wd = w->mul_scalar(gwd * glr);
+                    Tensor<T> s1 = w->sub(*update);
+                    nw = s1->sub(*wd);
+                } else nw = w->sub(*update);
+                g.update_parameter(p, std::move(nw));
             }
-            if (!m2.count(p)) m2[p] = HipStorage<T>::zeros(w->shape());
-            {  // second moment: beta2*v + (1-beta2)*g*g
-                Tensor<T> gg = grad->mul(*grad);
-                Tensor<T> a = m2[p]->mul_scalar(beta2), b = gg->mul_scalar(T(1) - beta2);
-                m2[p] = a->add(*b);
-            }
-            Tensor<T> second = m2[p]->clone_storage();  // take_current_buffer clones
-            Tensor<T> t1 = second->div_scalar(bc2);
-            Tensor<T> t2 = t1->sqrt();
-            Tensor<T> denom = t2->add_scalar(eps);
-            Tensor<T> first = m1[p]->clone_storage();
-            Tensor<T> u1 = first->div_scalar(bc1);
-            Tensor<T> u2 = u1->div(*denom);
-            Tensor<T> update = u2->mul_scalar(lr);
-            Tensor<T> nw;
-            if (weight_decay != T(0)) {
-                Tensor<T> wd = w->mul_scalar(weight_decay * lr);
-                Tensor<T> s1 = w->sub(*update);
-                nw = s1->sub(*wd);
-            } else nw = w->sub(*update);
-            g.update_parameter(p, std::move(nw));
         }
     }
     OptimizerStateDict state_dict() const override {
@@ -908,14 +1052,26 @@ template <typename T> struct Adam : Optimizer<T> {  // src/nn/optim/adam.rs:110-
         this->save_groups(sd);
         return sd;
     }
-    void load_state_dict(const OptimizerStateDict& sd) override {
-        adam_load_state_dict<T>(*this, sd);
-        lr = this->hyper(sd, "lr", lr);
-        beta1 = this->hyper(sd, "beta1", beta1);
-        beta2 = this->hyper(sd, "beta2", beta2);
-        eps = this->hyper(sd, "eps", eps);
-        weight_decay = this->hyper(sd, "weight_decay", weight_decay);
-        this->load_groups(sd);
+    void load_state_dict(const OptimizerStateDict& sd) override { adam_load(*this, sd); }
+
+    // Adam::load_state_dict, adam.rs:463-556 (shared with the fused optimizer)
+    template <class Opt> static void adam_load(Opt& o, const OptimizerStateDict& sd) {
+        if (sd.optimizer_type != "Adam") throw Error("Type mismatch: Expected Adam state dict, got " + sd.optimizer_type);
+        o.m1.clear();
+        o.m2.clear();
+        o.mmax.clear();
+        o.step_count = (long)sd.step_count;
+        o.lr = Optimizer<T>::hyper(sd, "lr", o.lr);
+        o.beta1 = Optimizer<T>::hyper(sd, "beta1", o.beta1);
+        o.beta2 = Optimizer<T>::hyper(sd, "beta2", o.beta2);
+        o.eps = Optimizer<T>::hyper(sd, "eps", o.eps);
+        o.weight_decay = Optimizer<T>::hyper(sd, "weight_decay", o.weight_decay);
+        auto it = sd.hyperparameters.find("amsgrad");
+        if (it != sd.hyperparameters.end()) o.amsgrad = it->second > 0.5;
+        o.load_groups(sd);
+        o.load_buffers(sd, "first_moment", o.m1);
+        o.load_buffers(sd, "second_moment", o.m2);
+        if (o.amsgrad) o.load_buffers(sd, "max_second_moment", o.mmax);
     }
 };
 

@@ -33,6 +33,13 @@ template <typename T> struct FusedApi;
             return fx_adam_step_multi_##S(c, k, p, g, m, v, n, lr, b1, b2, eps, wd, bc1, bc2);                         \
         }                                                                                                              \
         static int sgd_multi(fx_ctx* c, int k, T* const* p, const T* const* g, const int64_t* n, T lr) { return fx_sgd_step_multi_##S(c, k, p, g, n, lr); } \
+        static int sgd_momentum_multi(fx_ctx* c, int k, T* const* p, const T* const* g, T* const* b, const int64_t* n, T lr, T mom, T wd, int nes) { \
+            return fx_sgd_momentum_step_multi_##S(c, k, p, g, b, n, lr, mom, wd, nes);                                 \
+        }                                                                                                              \
+        static int adam_amsgrad_multi(fx_ctx* c, int k, T* const* p, const T* const* g, T* const* m, T* const* v, T* const* x, const int64_t* n, \
+                                      T lr, T b1, T b2, T eps, T wd, T bc1, T bc2) {                                   \
+            return fx_adam_amsgrad_step_multi_##S(c, k, p, g, m, v, x, n, lr, b1, b2, eps, wd, bc1, bc2);              \
+        }                                                                                                              \
         static int relu_bwd(fx_ctx* c, const T* g, const T* x, T* o, int64_t n) { return fx_relu_bwd_##S(c, g, x, o, n); } \
         static int relu_bias_grad(fx_ctx* c, const T* g, const T* y, T* gm, T* db, int64_t o, int64_t C, int64_t i) {  \
             return fx_relu_bwd_bias_grad_##S(c, g, y, gm, db, o, C, i);                                                \
@@ -345,72 +352,79 @@ template <typename T> NodeId cce_loss_fused(AutoFerroxEngine<T>& g, NodeId predi
     return g.apply_operation(std::make_unique<SoftmaxCEOp<T>>(), {predictions, targets});
 }
 
-template <typename T> struct SGDFused : Optimizer<T> {
-    T lr;
-    explicit SGDFused(T lr_) : lr(lr_) {}
-    void step(AutoFerroxEngine<T>& g) override {  // every parameter in one launch
-        std::vector<T*> ps;
-        std::vector<const T*> gs;
-        std::vector<int64_t> ns;
-        for (NodeId p : this->params) {
-            const HipStorage<T>* grad = g.get_gradient(p);
-            if (!grad) continue;
-            HipStorage<T>* w = g.mutable_tensor(p);
-            ps.push_back(w->data());
-            gs.push_back(grad->data());
-            ns.push_back((int64_t)w->size());
+// SGD with every parameter of a group updated in one launch (fx_sgd_step_multi / fx_sgd_momentum_step_multi); same
+// hyper-parameters, groups, buffers, state dictionary and element arithmetic as SGD<T>.
+template <typename T> struct SGDFused : SGD<T> {
+    explicit SGDFused(T lr_, T momentum_ = T(0), T wd = T(0), bool nesterov_ = false) : SGD<T>(lr_, momentum_, wd, nesterov_) {}
+    void step(AutoFerroxEngine<T>& g) override {
+        for (const auto& group : this->param_groups) {
+            const T glr = group.lr.value_or(this->lr), gwd = group.weight_decay.value_or(this->weight_decay),
+                    gmom = group.momentum.value_or(this->momentum);
+            std::vector<T*> ps, bufs;
+            std::vector<const T*> gs;
+            std::vector<int64_t> ns;
+            for (NodeId p : group.params) {
+                const HipStorage<T>* grad = g.get_gradient(p);
+                if (!grad) continue;
+                HipStorage<T>* w = g.mutable_tensor(p);
+                if (grad->shape() != w->shape()) throw Error("Shape mismatch for GPU subtraction: " + fmt_shape(w->shape()) + " vs " + fmt_shape(grad->shape()));
+                if (gmom != T(0)) {
+                    auto it = this->momentum_buffers.find(p);
+                    if (it == this->momentum_buffers.end()) it = this->momentum_buffers.emplace(p, HipStorage<T>::zeros(w->shape())).first;
+                    else this->check_buffer(*it->second, *w, "momentum", p);
+                    bufs.push_back(it->second->data());
+                }
+                ps.push_back(w->data());
+                gs.push_back(grad->data());
+                ns.push_back((int64_t)w->size());
+            }
+            if (ps.empty()) continue;
+            if (gmom == T(0) && gwd == T(0)) fx_ok(FusedApi<T>::sgd_multi(fused_ctx(), (int)ps.size(), ps.data(), gs.data(), ns.data(), glr));
+            else
+                fx_ok(FusedApi<T>::sgd_momentum_multi(fused_ctx(), (int)ps.size(), ps.data(), gs.data(), gmom != T(0) ? bufs.data() : nullptr, ns.data(),
+                                                      glr, gmom, gwd, this->nesterov ? 1 : 0));
         }
-        fx_ok(FusedApi<T>::sgd_multi(fused_ctx(), (int)ps.size(), ps.data(), gs.data(), ns.data(), lr));
-    }
-    OptimizerStateDict state_dict() const override { return sgd_state_dict<T>(*this); }
-    void load_state_dict(const OptimizerStateDict& sd) override {
-        sgd_check(sd);
-        lr = this->hyper(sd, "lr", lr);
-        this->load_groups(sd);
     }
 };
 
-template <typename T> struct AdamFused : Optimizer<T> {
-    T lr, beta1, beta2, eps, weight_decay;
-    long step_count = 0;
-    std::map<NodeId, Tensor<T>> m1, m2;
-    AdamFused(T lr_, T b1, T b2, T eps_, T wd) : lr(lr_), beta1(b1), beta2(b2), eps(eps_), weight_decay(wd) {}
+// Adam with every parameter of a group updated in one launch (fx_adam_step_multi / fx_adam_amsgrad_step_multi)
+template <typename T> struct AdamFused : Adam<T> {
+    AdamFused(T lr_, T b1, T b2, T eps_, T wd, bool amsgrad_ = false) : Adam<T>(lr_, b1, b2, eps_, wd, amsgrad_) {}
     void step(AutoFerroxEngine<T>& g) override {
-        step_count += 1;
-        const T stepf = (T)step_count;
-        const T b1p = std::max((T)std::pow(beta1, stepf), (T)1e-8), b2p = std::max((T)std::pow(beta2, stepf), (T)1e-8);
-        const T bc1 = T(1) - b1p, bc2 = T(1) - b2p;
-        std::vector<T*> ps, ms, vs;  // every parameter in one launch
-        std::vector<const T*> gs;
-        std::vector<int64_t> ns;
-        for (NodeId p : this->params) {
-            const HipStorage<T>* grad = g.get_gradient(p);
-            if (!grad) continue;
-            HipStorage<T>* w = g.mutable_tensor(p);
-            if (!m1.count(p)) m1[p] = HipStorage<T>::zeros(w->shape());
-            if (!m2.count(p)) m2[p] = HipStorage<T>::zeros(w->shape());
-            ps.push_back(w->data());
-            gs.push_back(grad->data());
-            ms.push_back(m1[p]->data());
-            vs.push_back(m2[p]->data());
-            ns.push_back((int64_t)w->size());
+        this->step_count += 1;
+        T bc1, bc2;
+        adam_bias_corrections(this->beta1, this->beta2, this->step_count, bc1, bc2);
+        for (const auto& group : this->param_groups) {
+            const T glr = group.lr.value_or(this->lr), gwd = group.weight_decay.value_or(this->weight_decay);
+            std::vector<T*> ps, ms, vs, xs;
+            std::vector<const T*> gs;
+            std::vector<int64_t> ns;
+            auto buffer = [&](std::map<NodeId, Tensor<T>>& table, NodeId p, const HipStorage<T>& w, const char* type) {
+                auto it = table.find(p);
+                if (it == table.end()) it = table.emplace(p, HipStorage<T>::zeros(w.shape())).first;
+                else this->check_buffer(*it->second, w, type, p);
+                return it->second->data();
+            };
+            for (NodeId p : group.params) {
+                const HipStorage<T>* grad = g.get_gradient(p);
+                if (!grad) continue;
+                HipStorage<T>* w = g.mutable_tensor(p);
+                if (grad->shape() != w->shape()) throw Error("Shape mismatch for GPU subtraction: " + fmt_shape(w->shape()) + " vs " + fmt_shape(grad->shape()));
+                ms.push_back(buffer(this->m1, p, *w, "first_moment"));
+                vs.push_back(buffer(this->m2, p, *w, "second_moment"));
+                if (this->amsgrad) xs.push_back(buffer(this->mmax, p, *w, "max_second_moment"));
+                ps.push_back(w->data());
+                gs.push_back(grad->data());
+                ns.push_back((int64_t)w->size());
+            }
+            if (ps.empty()) continue;
+            if (this->amsgrad)
+                fx_ok(FusedApi<T>::adam_amsgrad_multi(fused_ctx(), (int)ps.size(), ps.data(), gs.data(), ms.data(), vs.data(), xs.data(), ns.data(), glr,
+                                                      this->beta1, this->beta2, this->eps, gwd, bc1, bc2));
+            else
+                fx_ok(FusedApi<T>::adam_multi(fused_ctx(), (int)ps.size(), ps.data(), gs.data(), ms.data(), vs.data(), ns.data(), glr, this->beta1,
+                                              this->beta2, this->eps, gwd, bc1, bc2));
         }
-        fx_ok(FusedApi<T>::adam_multi(fused_ctx(), (int)ps.size(), ps.data(), gs.data(), ms.data(), vs.data(), ns.data(), lr, beta1, beta2,
-                                      eps, weight_decay, bc1, bc2));
-    }
-    OptimizerStateDict state_dict() const override {
-        OptimizerStateDict sd = adam_state_dict<T>(*this);
-        this->save_groups(sd);
-        return sd;
-    }
-    void load_state_dict(const OptimizerStateDict& sd) override {
-        adam_load_state_dict<T>(*this, sd);
-        lr = this->hyper(sd, "lr", lr);
-        beta1 = this->hyper(sd, "beta1", beta1);
-        beta2 = this->hyper(sd, "beta2", beta2);
-        eps = this->hyper(sd, "eps", eps);
-        weight_decay = this->hyper(sd, "weight_decay", weight_decay);
-        this->load_groups(sd);
     }
 };
 

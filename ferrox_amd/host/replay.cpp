@@ -22,6 +22,7 @@ struct ModelBase {
     virtual void set_batch(const void* x, const Shape& xs, const void* y, const Shape& ys) = 0;
     virtual double train_step(bool optimizer_step = true) = 0;
     virtual void configure(int loss_kind, bool input_requires_grad) = 0;
+    virtual void add_param_group(const int* idx, int n, double lr, double wd, double mom) = 0;
     virtual int64_t input_numel() const = 0;
     virtual void get_input_grad(void* host) const = 0;
     virtual void get_param(int i, void* host) const = 0;
@@ -131,18 +132,36 @@ template <typename T> struct Model : ModelBase {
         std::stringstream os(optspec);
         std::string kind;
         os >> kind;
-        if (kind == "sgd") {
-            double lr = 0.01;
+        if (kind == "sgd") {  // sgd LR [MOMENTUM [WEIGHT_DECAY [NESTEROV]]]
+            double lr = 0.01, mom = 0, wd = 0;
+            int nesterov = 0;
             os >> lr;
-            if (fused) opt = std::make_unique<SGDFused<T>>((T)lr);
-            else opt = std::make_unique<SGD<T>>((T)lr);
-        } else if (kind == "adam") {
+            if (os >> mom && os >> wd) os >> nesterov;
+            if (fused) opt = std::make_unique<SGDFused<T>>((T)lr, (T)mom, (T)wd, nesterov != 0);
+            else opt = std::make_unique<SGD<T>>((T)lr, (T)mom, (T)wd, nesterov != 0);
+        } else if (kind == "adam") {  // adam LR B1 B2 EPS WEIGHT_DECAY [AMSGRAD]
             double lr = 1e-3, b1 = 0.9, b2 = 0.999, eps = 1e-8, wd = 0;
+            int amsgrad = 0;
             os >> lr >> b1 >> b2 >> eps >> wd;
-            if (fused) opt = std::make_unique<AdamFused<T>>((T)lr, (T)b1, (T)b2, (T)eps, (T)wd);
-            else opt = std::make_unique<Adam<T>>((T)lr, (T)b1, (T)b2, (T)eps, (T)wd);
+            if (!(os >> amsgrad)) amsgrad = 0;
+            if (fused) opt = std::make_unique<AdamFused<T>>((T)lr, (T)b1, (T)b2, (T)eps, (T)wd, amsgrad != 0);
+            else opt = std::make_unique<Adam<T>>((T)lr, (T)b1, (T)b2, (T)eps, (T)wd, amsgrad != 0);
         } else throw Error("unknown optimizer '" + kind + "'");
-        opt->params = params;
+        for (NodeId p : params) opt->add_param(0, p);  // initialize_model, examples/common/training.rs:18-29
+    }
+    // Moves the listed parameters (indices into the model's parameter list) out of their groups into a new group with
+    // its own lr / weight decay / momentum (NaN = not set: the optimizer's value applies), ParameterGroup of optim/mod.rs:203-258.
+    void add_param_group(const int* idx, int n, double lr, double wd, double mom) override {
+        ParameterGroup<T> group("group" + std::to_string(opt->param_groups.size()));
+        for (int k = 0; k < n; ++k) {
+            const NodeId id = params.at((size_t)idx[k]);
+            for (auto& g : opt->param_groups) g.params.erase(std::remove(g.params.begin(), g.params.end(), id), g.params.end());
+            group.add_param(id);
+        }
+        if (lr == lr) group.lr = (T)lr;
+        if (wd == wd) group.weight_decay = (T)wd;
+        if (mom == mom) group.momentum = (T)mom;
+        opt->add_param_group(std::move(group));
     }
     void set_training(bool t) override {
         for (auto& l : layers) l->set_training(t);
@@ -303,6 +322,10 @@ int fxh_model_configure(void* m, int loss_kind, int input_requires_grad) {
 // zero_gradients -> forward -> loss -> backward, no optimizer step
 int fxh_model_backward(void* m, double* loss) {
     return guarded([&] { *loss = static_cast<ModelBase*>(m)->train_step(false); });
+}
+// parameters idx[0..n) leave their groups for a new one; lr / weight_decay / momentum are NaN where the group sets none
+int fxh_model_add_param_group(void* m, const int* idx, int n, double lr, double weight_decay, double momentum) {
+    return guarded([&] { static_cast<ModelBase*>(m)->add_param_group(idx, n, lr, weight_decay, momentum); });
 }
 int64_t fxh_model_input_numel(void* m) { return static_cast<ModelBase*>(m)->input_numel(); }
 int fxh_model_get_input_grad(void* m, void* host) {

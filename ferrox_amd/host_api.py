@@ -47,6 +47,7 @@ lib.fxh_model_load_optimizer_state.argtypes = [C.c_void_p, C.c_char_p, C.c_int64
 lib.fxh_set_conv_grad_mode.argtypes = [C.c_int]
 lib.fxh_model_configure.argtypes = [C.c_void_p, C.c_int, C.c_int]
 lib.fxh_model_backward.argtypes = [C.c_void_p, C.POINTER(C.c_double)]
+lib.fxh_model_add_param_group.argtypes = [C.c_void_p, C.POINTER(C.c_int), C.c_int, C.c_double, C.c_double, C.c_double]
 lib.fxh_model_input_numel.argtypes = [C.c_void_p]
 lib.fxh_model_input_numel.restype = C.c_int64
 lib.fxh_model_get_input_grad.argtypes = [C.c_void_p, C.c_void_p]
@@ -83,7 +84,7 @@ def pool_stats(dtype=np.float32):
 
 class Model:
     """spec: 'conv CIN COUT K S P; bn C EPS MOMENTUM; relu; maxpool K S P; gap; flatten; linear IN OUT; dropout P SEED; ...'
-    optimizer: 'sgd LR' | 'adam LR B1 B2 EPS WD'."""
+    optimizer: 'sgd LR [MOMENTUM [WEIGHT_DECAY [NESTEROV]]]' | 'adam LR B1 B2 EPS WD [AMSGRAD]'."""
 
     def __init__(self, spec, params, optimizer, dtype=np.float32, literal_engine=True, fused=False):
         """literal_engine: keep the reference engine's per-node deep clones; fused: fused layers, loss and optimizer."""
@@ -116,6 +117,14 @@ class Model:
     def configure(self, loss="cce", input_requires_grad=False):
         """loss: 'cce' (softmax cross-entropy against the targets) or 'sum' (sum of every element of the prediction)."""
         _check(lib.fxh_model_configure(self.h, {"cce": 0, "sum": 1}[loss], int(input_requires_grad)))
+
+    def add_param_group(self, indices, lr=None, weight_decay=None, momentum=None):
+        """Moves the parameters `indices` into a new optimizer group with its own lr / weight decay / momentum
+        (None = the optimizer's value)."""
+        nan = float("nan")
+        arr = (C.c_int * len(indices))(*indices)
+        _check(lib.fxh_model_add_param_group(self.h, arr, len(indices), nan if lr is None else lr,
+                                             nan if weight_decay is None else weight_decay, nan if momentum is None else momentum))
 
     def backward(self):
         """zero_gradients, forward, loss, backward -- no optimizer step.  Returns the loss."""

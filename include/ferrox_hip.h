@@ -307,14 +307,29 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
        the same order as the composed kernels: bit-identical results. */                                               \
     int fx_adam_step_##S(fx_ctx* ctx, T* p, const T* g, T* m, T* v, int64_t n, T lr, T beta1, T beta2, T eps,          \
                          T weight_decay, T bc1, T bc2);                                                                \
+    /* The same step with AMSGrad (adam.rs:203-221, 326-338): vmax = max(vmax, v) elementwise (a >= b ? a : b,         \
+       cpu.rs:717-739) after v is updated, and vmax takes v's place in the denominator; in place on vmax too. */        \
+    int fx_adam_amsgrad_step_##S(fx_ctx* ctx, T* p, const T* g, T* m, T* v, T* vmax, int64_t n, T lr, T beta1, T beta2, \
+                                 T eps, T weight_decay, T bc1, T bc2);                                                 \
     /* SGD::step without momentum or weight decay, src/nn/optim/sgd.rs:210-245: p = p - g*lr, in place. */             \
     int fx_sgd_step_##S(fx_ctx* ctx, T* p, const T* g, int64_t n, T lr);                                               \
-    /* The same updates for `count` parameters in one launch (the optimizers' loop over parameters,                    \
-       adam.rs:288-358 / sgd.rs:210-245): p, g, m, v, n are HOST arrays of `count` device pointers / element counts;   \
-       element arithmetic and results are those of fx_adam_step / fx_sgd_step. */                                      \
+    /* SGD::step in full (sgd.rs:128-245): e = g + p*weight_decay when weight_decay != 0 (L2, apply_weight_decay);     \
+       momentum != 0: buf = buf*momentum + e (update_momentum_buffer; a new buffer starts at zero) and the update is   \
+       buf, or buf*momentum + e with nesterov; p = p - update*lr.  buf must be NULL exactly when momentum == 0.        \
+       Composed order, bit-identical to the op-by-op path. */                                                          \
+    int fx_sgd_momentum_step_##S(fx_ctx* ctx, T* p, const T* g, T* buf, int64_t n, T lr, T momentum, T weight_decay,   \
+                                 int nesterov);                                                                        \
+    /* The same updates for `count` parameters in one launch (the optimizers' loop over a parameter group,             \
+       adam.rs:288-358 / sgd.rs:210-245): p, g, m, v, vmax, buf, n are HOST arrays of `count` device pointers /        \
+       element counts; element arithmetic and results are those of the one-tensor calls. */                            \
     int fx_adam_step_multi_##S(fx_ctx* ctx, int count, T* const* p, const T* const* g, T* const* m, T* const* v,       \
                                const int64_t* n, T lr, T beta1, T beta2, T eps, T weight_decay, T bc1, T bc2);         \
-    int fx_sgd_step_multi_##S(fx_ctx* ctx, int count, T* const* p, const T* const* g, const int64_t* n, T lr);
+    int fx_adam_amsgrad_step_multi_##S(fx_ctx* ctx, int count, T* const* p, const T* const* g, T* const* m,            \
+                                       T* const* v, T* const* vmax, const int64_t* n, T lr, T beta1, T beta2, T eps,   \
+                                       T weight_decay, T bc1, T bc2);                                                  \
+    int fx_sgd_step_multi_##S(fx_ctx* ctx, int count, T* const* p, const T* const* g, const int64_t* n, T lr);         \
+    int fx_sgd_momentum_step_multi_##S(fx_ctx* ctx, int count, T* const* p, const T* const* g, T* const* buf,          \
+                                       const int64_t* n, T lr, T momentum, T weight_decay, int nesterov);
 
 FX_DECLARE_KERNELS(float, f32)
 FX_DECLARE_KERNELS(double, f64)

@@ -67,19 +67,24 @@ def bias_grad(g):
     return orc.reduce("sum", g, [3, 2, 0] if g.ndim == 4 else [0])
 
 
-def adam_update(w, g, m, v, lr, b1, b2, eps, wd, bc1, bc2):
-    """One Adam::step for one parameter (adam.rs:288-358); every scalar already in the tensor dtype."""
+def adam_update(w, g, m, v, lr, b1, b2, eps, wd, bc1, bc2, vmax=None):
+    """One Adam::step for one parameter (adam.rs:288-358); every scalar already in the tensor dtype.  vmax: the AMSGrad
+    running maximum of the second moment (adam.rs:203-221) or None.  Returns (w, m, v, vmax)."""
     dt = w.dtype.type
     m = orc.binary("add", orc.scalar("mul_scalar", m, b1), orc.scalar("mul_scalar", g, dt(1) - b1))
     v = orc.binary("add", orc.scalar("mul_scalar", v, b2), orc.scalar("mul_scalar", orc.binary("mul", g, g), dt(1) - b2))
-    denom = orc.scalar("add_scalar", orc.unary("sqrt", orc.scalar("div_scalar", v, bc2)), eps)
+    second = v
+    if vmax is not None:
+        vmax = orc.binary("max", vmax, v)
+        second = vmax
+    denom = orc.scalar("add_scalar", orc.unary("sqrt", orc.scalar("div_scalar", second, bc2)), eps)
     upd = orc.scalar("mul_scalar", orc.binary("div", orc.scalar("div_scalar", m, bc1), denom), lr)
     if wd != 0:
         wdt = orc.scalar("mul_scalar", w, wd * lr)
         w = orc.binary("sub", orc.binary("sub", w, upd), wdt)
     else:
         w = orc.binary("sub", w, upd)
-    return w, m, v
+    return w, m, v, vmax
 
 
 def batchnorm_forward(x, gamma, beta, eps, training=True, running_mean=None, running_var=None):
@@ -279,20 +284,43 @@ class Sequential:
 
 
 class SGD:
-    def __init__(self, lr):
-        self.lr = lr
+    """SGD::step (sgd.rs:116-245): L2 weight decay folded into the gradient, momentum buffer buf = buf*mu + e, Nesterov
+    update buf*mu + e, p = p - update*lr.  `groups` maps a parameter index to (lr, weight_decay, momentum) overrides
+    (None = the optimizer's value), the ParameterGroup options of optim/mod.rs:203-258."""
+
+    def __init__(self, lr, momentum=0.0, weight_decay=0.0, nesterov=False, groups=None):
+        self.lr, self.momentum, self.wd, self.nesterov = lr, momentum, weight_decay, bool(nesterov)
+        self.groups = groups or {}
+        self.buf = {}
 
     def step(self, model, grads):
         dt = model.dtype.type
         for i, g in enumerate(grads):
-            model.params[i] = orc.binary("sub", model.params[i], orc.scalar("mul_scalar", g, dt(self.lr)))
+            glr, gwd, gmom = self.groups.get(i, (None, None, None))
+            lr = dt(self.lr if glr is None else glr)
+            wd = dt(self.wd if gwd is None else gwd)
+            mom = dt(self.momentum if gmom is None else gmom)
+            w = model.params[i]
+            e = g if wd == 0 else orc.binary("add", g, orc.scalar("mul_scalar", w, wd))
+            if mom != 0:
+                b = self.buf.get(i, np.zeros_like(w))
+                b = orc.binary("add", orc.scalar("mul_scalar", b, mom), e)
+                self.buf[i] = b
+                upd = orc.binary("add", orc.scalar("mul_scalar", b, mom), e) if self.nesterov else b
+            else:
+                upd = e
+            model.params[i] = orc.binary("sub", w, orc.scalar("mul_scalar", upd, lr))
 
 
 class Adam:
-    def __init__(self, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0):
+    """Adam::step (adam.rs:110-358); amsgrad keeps vmax = max(vmax, v) (a >= b ? a : b) and divides by it."""
+
+    def __init__(self, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0, amsgrad=False, groups=None):
         self.lr, self.b1, self.b2, self.eps, self.wd = lr, beta1, beta2, eps, weight_decay
+        self.amsgrad = bool(amsgrad)
+        self.groups = groups or {}
         self.t = 0
-        self.m, self.v = {}, {}
+        self.m, self.v, self.vmax = {}, {}, {}
 
     def step(self, model, grads):
         dt = model.dtype.type
@@ -301,9 +329,15 @@ class Adam:
         bc1 = dt(1) - max(dt(np.power(b1, dt(self.t))), dt(1e-8))      # adam.rs:110-126
         bc2 = dt(1) - max(dt(np.power(b2, dt(self.t))), dt(1e-8))
         for i, g in enumerate(grads):
+            glr, gwd, _ = self.groups.get(i, (None, None, None))
+            lr = dt(self.lr if glr is None else glr)
+            wd = dt(self.wd if gwd is None else gwd)
             w = model.params[i]
             m = self.m.get(i, np.zeros_like(w))
             v = self.v.get(i, np.zeros_like(w))
-            w, m, v = adam_update(w, g, m, v, dt(self.lr), b1, b2, dt(self.eps), dt(self.wd), bc1, bc2)
+            vmax = self.vmax.get(i, np.zeros_like(w)) if self.amsgrad else None
+            w, m, v, vmax = adam_update(w, g, m, v, lr, b1, b2, dt(self.eps), wd, bc1, bc2, vmax)
             self.m[i], self.v[i] = m, v
+            if self.amsgrad:
+                self.vmax[i] = vmax
             model.params[i] = w

@@ -106,7 +106,7 @@ def test_adam_and_sgd_step_bit_exact(ctx, train, dtype):
                 b1, b2 = dt(0.9), dt(0.999)
                 bc1 = dt(1) - max(dt(np.power(b1, dt(t))), dt(1e-8))
                 bc2 = dt(1) - max(dt(np.power(b2, dt(t))), dt(1e-8))
-                w, m, v = train.adam_update(w, g, m, v, dt(1e-3), b1, b2, dt(1e-8), dt(wd), bc1, bc2)
+                w, m, v, _ = train.adam_update(w, g, m, v, dt(1e-3), b1, b2, dt(1e-8), dt(wd), bc1, bc2)
                 ctx.adam_step(dw, ctx.upload(g), dm, dv, 1e-3, 0.9, 0.999, 1e-8, wd, float(bc1), float(bc2))
                 assert np.array_equal(dw.numpy(), w) and np.array_equal(dm.numpy(), m) and np.array_equal(dv.numpy(), v), (n, wd, t)
     import oracle as orc
@@ -115,6 +115,51 @@ def test_adam_and_sgd_step_bit_exact(ctx, train, dtype):
     dw = ctx.upload(w)
     ctx.sgd_step(dw, ctx.upload(g), 0.01)
     assert np.array_equal(dw.numpy(), orc.binary("sub", w, orc.scalar("mul_scalar", g, dt(0.01))))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sgd_momentum_and_adam_amsgrad_steps_bit_exact(ctx, train, dtype):
+    """fx_sgd_momentum_step (L2 weight decay, momentum, Nesterov) and fx_adam_amsgrad_step against the oracle's op-by-op
+    optimizers, several steps in a row so the buffers carry over; and the buffer / momentum pairing is enforced."""
+    from ferrox_amd.capi import FerroxHipError
+
+    class One:  # the oracle optimizers update `model.params`
+        def __init__(self, w):
+            self.params, self.dtype = [w], np.dtype(dtype)
+
+    rng = np.random.default_rng(77)
+    dt = np.dtype(dtype).type
+    for n in (1, 257, 18432):
+        for mom, wd, nes in ((0.9, 0.0, False), (0.9, 5e-4, True), (0.0, 1e-2, False), (0.5, 0.1, False)):
+            w = rng.standard_normal(n).astype(dtype)
+            model, opt = One(w.copy()), train.SGD(0.05, mom, wd, nes)
+            dw = ctx.upload(w)
+            dbuf = ctx.fill((n,), 0.0, dtype) if mom != 0 else None
+            for t in range(3):
+                g = rng.standard_normal(n).astype(dtype)
+                opt.step(model, [g])
+                ctx.sgd_momentum_step(dw, ctx.upload(g), dbuf, 0.05, mom, wd, nes)
+                assert np.array_equal(dw.numpy(), model.params[0]), (n, mom, wd, nes, t)
+                if mom != 0:
+                    assert np.array_equal(dbuf.numpy(), opt.buf[0]), (n, mom, wd, nes, t)
+        for wd in (0.0, 0.01):
+            w = rng.standard_normal(n).astype(dtype)
+            model, opt = One(w.copy()), train.Adam(1e-3, 0.9, 0.999, 1e-8, wd, amsgrad=True)
+            dw, dm, dv, dx = ctx.upload(w), ctx.fill((n,), 0.0, dtype), ctx.fill((n,), 0.0, dtype), ctx.fill((n,), 0.0, dtype)
+            for t, scale in enumerate((3.0, 0.1, 1.0, 0.01), start=1):
+                g = (rng.standard_normal(n) * scale).astype(dtype)
+                opt.step(model, [g])
+                bc1 = dt(1) - max(dt(np.power(dt(0.9), dt(t))), dt(1e-8))
+                bc2 = dt(1) - max(dt(np.power(dt(0.999), dt(t))), dt(1e-8))
+                ctx.adam_amsgrad_step(dw, ctx.upload(g), dm, dv, dx, 1e-3, 0.9, 0.999, 1e-8, wd, float(bc1), float(bc2))
+                assert np.array_equal(dw.numpy(), model.params[0]), (n, wd, t)
+                assert np.array_equal(dx.numpy(), opt.vmax[0]) and np.array_equal(dv.numpy(), opt.v[0]), (n, wd, t)
+            assert np.any(opt.vmax[0] > opt.v[0])
+    w = ctx.fill((8,), 1.0, dtype)
+    with pytest.raises(FerroxHipError, match="momentum buffer"):
+        ctx.sgd_momentum_step(w, w, None, 0.1, 0.9, 0.0, False)
+    with pytest.raises(FerroxHipError, match="momentum buffer"):
+        ctx.sgd_momentum_step(w, w, w, 0.1, 0.0, 0.0, False)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -98,6 +98,9 @@ def test_state_dict_errors_follow_the_reference(host):
         sd = bc.decode_state_dict(sgd.optimizer_state())
         assert sd["optimizer_type"] == "SGD" and sd["step_count"] == 0 and sd["parameter_buffers"] == {}
         assert sd["hyperparameters"] == {"lr": float(np.float32(0.05)), "momentum": 0.0, "weight_decay": 0.0, "nesterov": 0.0}
+        # SGD::new stores the optimizer's values in its default group (sgd.rs:28-45)
+        grp = sd["parameter_groups"][0]
+        assert (grp["lr"], grp["weight_decay"], grp["momentum"]) == (float(np.float32(0.05)), 0.0, 0.0)
         with pytest.raises(host.HostError, match="Expected Adam state dict, got SGD"):
             adam.load_optimizer_state(sgd.optimizer_state())
         with pytest.raises(host.HostError, match="Expected SGD state dict, got Adam"):
@@ -113,3 +116,79 @@ def test_state_dict_errors_follow_the_reference(host):
     finally:
         for m in (adam, sgd, adam64):
             m.close()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("optspec,kinds", [("sgd 0.05 0.9 0.0005 1", ["momentum"]),
+                                           ("adam 0.001 0.9 0.999 1e-08 0.01 1", ["first_moment", "second_moment", "max_second_moment"])])
+def test_momentum_and_amsgrad_buffers_are_saved_and_resume_bit_exactly(host, dtype, fused, optspec, kinds):
+    """SGD's momentum buffers (sgd.rs:278-360) and Adam's AMSGrad maxima (adam.rs:448-461, 540-553) go through the state
+    dictionary: a fresh model built with other hyper-parameters continues exactly like the uninterrupted one."""
+    from oracle import bincode2 as bc
+    params, x, y = problem(dtype, seed=13)
+    a = host.Model(SPEC, params, optspec, dtype, literal_engine=False, fused=fused)
+    other = "sgd 0.5" if optspec.startswith("sgd") else "adam 0.5 0.5 0.5 0.5 0"
+    b = None
+    try:
+        a.add_param_group([4, 5], 0.02, 0.0, None)
+        a.set_batch(x, y)
+        for _ in range(3):
+            a.train_step()
+        raw = a.optimizer_state()
+        sd = bc.decode_state_dict(raw)
+        assert sorted({v["buffer_type"] for v in sd["parameter_buffers"].values()}) == sorted(kinds)
+        assert len(sd["parameter_buffers"]) == 6 * len(kinds)
+        assert [g["name"] for g in sd["parameter_groups"]] == ["default", "group1"]
+        assert len(sd["parameter_groups"][0]["params"]) == 4 and len(sd["parameter_groups"][1]["params"]) == 2
+        assert sd["parameter_groups"][1]["lr"] == float(dtype(0.02)) and sd["parameter_groups"][1]["momentum"] is None
+        assert bc.encode_state_dict(sd) == raw
+        b = host.Model(SPEC, [a.param(i) for i in range(6)], other, dtype, literal_engine=False, fused=fused)
+        b.load_optimizer_state(raw)
+        b.set_batch(x, y)
+        for _ in range(2):
+            assert a.train_step() == b.train_step()
+        for i in range(6):
+            assert np.array_equal(a.param(i), b.param(i)), i
+        assert b.optimizer_state() == a.optimizer_state()
+    finally:
+        a.close()
+        if b is not None:
+            b.close()
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_state_from_another_model_is_refused(host, fused):
+    """A state dictionary whose buffers do not belong to this model's parameters: a node id that no restored group names is
+    refused when the state is loaded; a buffer of another shape when the parameter is next updated (the fused update
+    would otherwise read and write past the end of the buffer)."""
+    from oracle import bincode2 as bc
+    params, x, y = problem(np.float32, seed=17)
+    m = host.Model(SPEC, params, ADAM, np.float32, literal_engine=False, fused=fused)
+    try:
+        m.set_batch(x, y)
+        m.train_step()
+        good = m.optimizer_state()
+        sd = bc.decode_state_dict(good)
+        ids = sd["parameter_groups"][0]["params"]
+        # (a) a buffer names a node that is in no group
+        bad = bc.decode_state_dict(good)
+        key = f"{ids[0]}_first_moment"
+        buf = bad["parameter_buffers"].pop(key)
+        buf["node_id"] = 9999
+        bad["parameter_buffers"]["9999_first_moment"] = buf
+        with pytest.raises(host.HostError, match="names node 9999, which is in no parameter group"):
+            m.load_optimizer_state(bc.encode_state_dict(bad))
+        # (b) the moments of the first conv weight [4,3,3,3] and of its bias [4] trade places
+        bad = bc.decode_state_dict(good)
+        for kind in ("first_moment", "second_moment"):
+            b0, b1 = bad["parameter_buffers"][f"{ids[0]}_{kind}"], bad["parameter_buffers"][f"{ids[1]}_{kind}"]
+            b0["node_id"], b1["node_id"] = ids[1], ids[0]
+            bad["parameter_buffers"][f"{ids[0]}_{kind}"], bad["parameter_buffers"][f"{ids[1]}_{kind}"] = b1, b0
+        m.load_optimizer_state(bc.encode_state_dict(bad))
+        with pytest.raises(host.HostError, match=r"buffer 'first_moment' of node \d+ has shape \[4\], the parameter has \[4, 3, 3, 3\]"):
+            m.train_step()
+        m.load_optimizer_state(good)          # the model recovers with a matching state
+        m.train_step()
+    finally:
+        m.close()

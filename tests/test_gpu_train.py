@@ -74,7 +74,22 @@ CASES = [
     ("cnn_cls", CNN_CLS, (64, 3, 32, 32), 10, "adam 0.001 0.9 0.999 1e-08 0", 1),
     ("mlp_c2", MLP_C2, (256, 784), 10, "sgd 0.01", 1),
     ("cnn_c5", CNN_C5, (256, 3, 32, 32), 10, "adam 0.001 0.9 0.999 1e-08 0", 1),
+    # the optimizer options of the reference's training example (examples/common/training.rs:99-111)
+    ("mlp_small_momentum", MLP_SMALL, (9, 20), 5, "sgd 0.05 0.9 0 0", 3),
+    ("cnn_small_nesterov_wd", CNN_SMALL, (5, 3, 8, 8), 5, "sgd 0.05 0.9 0.0005 1", 3),
+    ("cnn_small_amsgrad_wd", CNN_SMALL, (5, 3, 8, 8), 5, "adam 0.001 0.9 0.999 1e-08 0.01 1", 3),
 ]
+
+
+def oracle_optimizer(optspec, groups=None):
+    from oracle import train as otrain
+    kind, *nums = optspec.split()
+    v = [float(t) for t in nums]
+    if kind == "sgd":
+        v += [0.0] * (4 - len(v))
+        return otrain.SGD(v[0], v[1], v[2], bool(v[3]), groups=groups)
+    v += [0.0] * (6 - len(v))
+    return otrain.Adam(v[0], v[1], v[2], v[3], v[4], bool(v[5]), groups=groups)
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
@@ -91,7 +106,7 @@ def test_train_step_matches_oracle(host, case, dtype, engine):
     params, x, y = kaiming_uniform_problem(spec, in_shape, ncls, 5, dtype)
     ref = otrain.Sequential(spec, params, dtype, conv_mode=0)
     kind, *nums = optspec.split()
-    ropt = otrain.SGD(float(nums[0])) if kind == "sgd" else otrain.Adam(*[float(v) for v in nums])
+    ropt = oracle_optimizer(optspec)
     model = host.Model(spec, params, optspec, dtype, literal_engine=literal_engine, fused=engine == "fused")
     try:
         model.set_batch(x, y)
@@ -152,6 +167,38 @@ def test_train_step_with_cpu_literal_conv_gradients(host, case, dtype, engine):
     finally:
         model.close()
         host.set_conv_grad_mode(0)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("optspec", ["sgd 0.05 0.9 0.0005 0", "adam 0.001 0.9 0.999 1e-08 0.01 0"])
+@pytest.mark.parametrize("engine", ["literal", "fused"])
+def test_parameter_group_overrides(host, dtype, optspec, engine):
+    """The last layer's weight and bias move into a group with its own lr / weight decay (and no momentum for SGD):
+    ParameterGroup, src/nn/optim/mod.rs:203-258, read by sgd.rs:103-114 / adam.rs:128-134."""
+    from oracle import train as otrain
+    tol = TOL[np.dtype(dtype)]
+    params, x, y = kaiming_uniform_problem(MLP_SMALL, (9, 20), 5, 21, dtype)
+    override = (0.2, 0.0, 0.0) if optspec.startswith("sgd") else (0.01, 0.0, None)
+    ref = otrain.Sequential(MLP_SMALL, params, dtype)
+    ropt = oracle_optimizer(optspec, groups={4: override, 5: override})
+    model = host.Model(MLP_SMALL, params, optspec, dtype, literal_engine=engine == "literal", fused=engine == "fused")
+    try:
+        model.add_param_group([4, 5], *override)
+        model.set_batch(x, y)
+        for step in range(3):
+            _, rgrads = ref.loss_and_grads(x, y)
+            ropt.step(ref, rgrads)
+            model.train_step()
+        for i, rp in enumerate(ref.params):
+            if optspec.startswith("sgd"):
+                assert close(model.param(i), rp, tol * 64), i
+            else:
+                assert np.abs(model.param(i).astype(np.float64) - rp).max() <= 0.05 * (0.01 if i >= 4 else 0.001) * 3, i
+        # the override took effect: the grouped parameters moved on the group's scale, not the optimizer's
+        moved = np.abs(model.param(4) - params[4]).max()
+        assert moved > (0.02 if optspec.startswith("adam") else 0.0)
+    finally:
+        model.close()
 
 
 C1_SPEC = "conv 1 8 3 1 1; relu"

@@ -143,3 +143,49 @@ def test_c1_literal_mode_gradients_composed():
     np.testing.assert_allclose(grads[0], (g2d @ col.T).reshape(w.shape), rtol=0, atol=1e-9)
     colm = (w.reshape(8, 9).T @ g2d).reshape(B, 9, L)
     np.testing.assert_allclose(gx, F.fold(torch.tensor(colm.copy()), (28, 28), 3, padding=1).numpy(), rtol=0, atol=1e-11)
+
+
+@pytest.mark.parametrize("momentum,wd,nesterov", [(0.9, 0.0, False), (0.9, 5e-4, False), (0.9, 5e-4, True), (0.0, 1e-2, False)])
+def test_sgd_momentum_weight_decay_nesterov_match_torch(momentum, wd, nesterov):
+    """SGD::step in full (sgd.rs:116-245) against torch.optim.SGD (dampening 0: the same recurrences) over several steps."""
+    rng = np.random.default_rng(3)
+    w0 = rng.standard_normal((4, 3))
+    gs = [rng.standard_normal((4, 3)) for _ in range(6)]
+    m = otrain.Sequential("linear 3 4", [w0, np.zeros(4)], np.float64)
+    opt = otrain.SGD(0.05, momentum, wd, nesterov)
+    tw = torch.tensor(w0, requires_grad=True)
+    topt = torch.optim.SGD([tw], lr=0.05, momentum=momentum, weight_decay=wd, nesterov=nesterov)
+    for g in gs:
+        opt.step(m, [g, np.zeros(4)])
+        tw.grad = torch.tensor(g)
+        topt.step()
+        np.testing.assert_allclose(m.params[0], tw.detach().numpy(), rtol=0, atol=1e-13)
+
+
+def test_adam_amsgrad_and_decoupled_weight_decay_match_torch():
+    """AMSGrad (adam.rs:203-221) against torch.optim.Adam(amsgrad=True); the decoupled weight decay against AdamW.
+    Gradients shrink over the steps so that the running maximum differs from the current second moment."""
+    rng = np.random.default_rng(4)
+    w0 = rng.standard_normal((5, 2))
+    gs = [rng.standard_normal((5, 2)) * s for s in (3.0, 0.1, 0.05, 2.0, 0.01, 0.01)]
+    for amsgrad, wd in ((True, 0.0), (False, 0.1), (True, 0.1)):
+        m = otrain.Sequential("linear 2 5", [w0, np.zeros(5)], np.float64)
+        opt = otrain.Adam(1e-2, 0.9, 0.999, 1e-8, wd, amsgrad)
+        tw = torch.tensor(w0, requires_grad=True)
+        topt = torch.optim.AdamW([tw], lr=1e-2, eps=1e-8, weight_decay=wd, amsgrad=amsgrad)
+        for g in gs:
+            opt.step(m, [g, np.zeros(5)])
+            tw.grad = torch.tensor(g)
+            topt.step()
+            np.testing.assert_allclose(m.params[0], tw.detach().numpy(), rtol=0, atol=1e-9)
+        if amsgrad:
+            assert np.all(opt.vmax[0] >= opt.v[0]) and np.any(opt.vmax[0] > opt.v[0])
+
+
+def test_parameter_group_overrides():
+    """A group's lr / weight decay / momentum replace the optimizer's for its parameters only (mod.rs:203-258,
+    sgd.rs:103-114): closed forms for one step."""
+    m = otrain.Sequential("linear 1 1", [np.array([[2.0]]), np.array([1.0])], np.float64)
+    otrain.SGD(0.1, groups={1: (0.5, 0.25, None)}).step(m, [np.array([[1.0]]), np.array([1.0])])
+    assert m.params[0].item() == pytest.approx(2.0 - 0.1 * 1.0, abs=1e-15)
+    assert m.params[1].item() == pytest.approx(1.0 - 0.5 * (1.0 + 0.25 * 1.0), abs=1e-15)
