@@ -149,6 +149,7 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_sgd_momentum_step_multi_{_s}", _vp, _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_i64),
          _ct, _ct, _ct, _int)
 
+_sig("fx_conv2d_tune_f32", _vp, _int, *([_i64] * 11), _int, _int)
 _sig("fx_reduce_max_noalloc_f32", _vp, _vp, _vp, _vp, _i64, _i64, _i64)
 NOALLOC_SCRATCH_BYTES = 4 << 20
 
@@ -445,6 +446,13 @@ class Context:
         y = out or self.empty((B, Cout, oh, ow), x.dtype)
         check(self._fn("conv2d_fwd", x.dtype)(self.h, x.ptr, w.ptr, y.ptr, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, None, 0))
         return y
+
+    def conv2d_tune(self, kind, x_shape, w_shape, stride, padding, with_bias=False, act=0):
+        """Times the tile shapes of the f32 3x3 forward (kind CONV_FWD) / data-gradient (CONV_DGRAD) kernel for this layer now."""
+        B, Cin, H, W = x_shape
+        Cout, _, kh, kw = w_shape
+        (sh, sw), (ph, pw) = stride, padding
+        check(lib.fx_conv2d_tune_f32(self.h, kind, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, int(with_bias), int(act)))
 
     def conv2d_dgrad(self, g, w, x_shape, stride, padding, mode=0, out=None):
         B, Cin, H, W = x_shape

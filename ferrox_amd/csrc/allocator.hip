@@ -58,8 +58,13 @@ static uint64_t now_ms() {
     return (uint64_t)duration_cast<milliseconds>(system_clock::now().time_since_epoch()).count();
 }
 
-static void device_free(Pool* p, const Block& b) {
-    (void)hipStreamSynchronize(p->stream);  // kernels already queued may still use the block
+// `drained`: one stream wait covers every block freed in the same batch -- the blocks sit in the pool, so only work
+// queued before the batch began can still touch them -- and the caller keeps one flag per batch.
+static void device_free(Pool* p, const Block& b, bool& drained) {
+    if (!drained) {
+        (void)hipStreamSynchronize(p->stream);  // kernels already queued may still use the block
+        drained = true;
+    }
     (void)hipFree(b.ptr);
     p->live.erase(b.ptr);
     p->st.device_frees += 1;
@@ -69,13 +74,14 @@ static void device_free(Pool* p, const Block& b) {
 // PoolBucket::return_allocation, mod.rs:263-288
 static void bucket_return(Pool* p, Bucket& b, Block blk) {
     const i64 cur = (i64)b.blocks.size();
+    bool drained = false;
     if (cur >= b.cfg.max_blocks) {
         if (b.cfg.eviction_threshold_ms >= 0) {  // evict_older_than, mod.rs:307-320
             const uint64_t now = now_ms();
             std::vector<Block> keep;
             for (auto& x : b.blocks) {
                 if ((now > x.ts_ms ? now - x.ts_ms : 0) <= (uint64_t)b.cfg.eviction_threshold_ms) keep.push_back(x);
-                else device_free(p, x);
+                else device_free(p, x, drained);
             }
             b.blocks.swap(keep);
         } else {  // evict_lru, mod.rs:291-305
@@ -84,7 +90,7 @@ static void bucket_return(Pool* p, Bucket& b, Block blk) {
                 std::stable_sort(b.blocks.begin(), b.blocks.end(), [](const Block& x, const Block& y) {
                     return x.ts_ms != y.ts_ms ? x.ts_ms < y.ts_ms : x.seq < y.seq;
                 });
-                for (i64 i = 0; i < n; ++i) device_free(p, b.blocks[i]);
+                for (i64 i = 0; i < n; ++i) device_free(p, b.blocks[i], drained);
                 b.blocks.erase(b.blocks.begin(), b.blocks.begin() + n);
             }
         }
@@ -200,7 +206,8 @@ int fx_alloc(fx_ctx* c, int dtype, int64_t n, void** ptr, int64_t* granted, uint
     hipError_t e = hipMalloc(&d, (size_t)n * (size_t)p->elem_size);
     if (e != hipSuccess) {
         // one retry after releasing everything cached
-        for (auto& bk : p->buckets) { for (auto& x : bk.blocks) device_free(p, x); bk.blocks.clear(); }
+        bool drained = false;
+        for (auto& bk : p->buckets) { for (auto& x : bk.blocks) device_free(p, x, drained); bk.blocks.clear(); }
         e = hipMalloc(&d, (size_t)n * (size_t)p->elem_size);
     }
     if (e != hipSuccess) {
@@ -243,7 +250,8 @@ int fx_free(fx_ctx* c, int dtype, void* ptr, uint64_t id) {
     } else {
         // unknown id: the reference drops the allocation, i.e. frees the device memory
         p->st.bytes_pooled += elems * p->elem_size;  // device_free subtracts it again
-        device_free(p, Block{ptr, elems, id, 0, 0});
+        bool drained = false;
+        device_free(p, Block{ptr, elems, id, 0, 0}, drained);
     }
     note_peak(p);
     return FX_OK;
@@ -255,7 +263,8 @@ int fx_pool_cleanup(fx_ctx* c, int dtype) {  // cuda.rs:113-119
     FX_REQUIRE(p != nullptr, "fx_pool_cleanup: unknown dtype %d", dtype);
     FX_HIP_CHECK(hipStreamSynchronize(c->stream));
     std::lock_guard<std::mutex> lk(p->mu);
-    for (auto& b : p->buckets) { for (auto& x : b.blocks) device_free(p, x); b.blocks.clear(); }
+    bool drained = false;  // waits once more under the lock: another thread may have returned a block since the wait above
+    for (auto& b : p->buckets) { for (auto& x : b.blocks) device_free(p, x, drained); b.blocks.clear(); }
     return FX_OK;
 }
 
@@ -265,7 +274,8 @@ int fx_pool_reset(fx_ctx* c, int dtype) {  // cuda.rs:125-133
     FX_REQUIRE(p != nullptr, "fx_pool_reset: unknown dtype %d", dtype);
     FX_HIP_CHECK(hipStreamSynchronize(c->stream));
     std::lock_guard<std::mutex> lk(p->mu);
-    for (auto& b : p->buckets) { for (auto& x : b.blocks) device_free(p, x); b.blocks.clear(); }
+    bool drained = false;  // waits once more under the lock: another thread may have returned a block since the wait above
+    for (auto& b : p->buckets) { for (auto& x : b.blocks) device_free(p, x, drained); b.blocks.clear(); }
     p->active.clear();
     p->counter = 0;
     const i64 in_use = p->st.bytes_in_use, allocs = p->st.device_allocs, frees = p->st.device_frees;

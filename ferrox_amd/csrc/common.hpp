@@ -72,6 +72,7 @@ struct fx_ctx {
     std::mutex launch_mutex;
     // tile shape that measured fastest per convolution layer shape (conv_patch.hpp); used under launch_mutex
     std::map<std::array<i64, 14>, int> conv_tile_cache;
+    bool conv_retune = false;  // set by fx_conv2d_tune around its call: time the shapes again even when the cache has an entry
     hipEvent_t ev_tune[2] = {nullptr, nullptr};
     // returns a scratch region of at least `bytes` (256-byte aligned); nullptr + error on failure
     void* get_scratch(i64 bytes);

@@ -597,6 +597,47 @@ extern "C" int64_t fx_conv2d_workspace_bytes(int kind, int dtype, int mode, int6
     return need;
 }
 
+// Pays the tile-shape timing of fx_conv2d_fwd / fx_conv2d_dgrad up front, on temporary zero-filled tensors of the layer's
+// shape (allocated and released here; this entry point synchronises).
+extern "C" int fx_conv2d_tune_f32(fx_ctx* c, int kind, int64_t B, int64_t Cin, int64_t H, int64_t W, int64_t Cout, int64_t kh,
+                                  int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw, int with_bias, int act) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(kind == FX_CONV_FWD || kind == FX_CONV_DGRAD || kind == FX_CONV_WGRAD, "fx_conv2d_tune: unknown kind %d", kind);
+    FX_REQUIRE(act == 0 || act == 1, "fx_conv2d_tune: act must be 0 (none) or 1 (relu)");
+    Dims d;
+    if (int rc = check_dims<float>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_tune")) return rc;
+    if (kind == FX_CONV_WGRAD) return FX_OK;  // the weight-gradient kernels take their shape from the cost model alone
+    const i64 nb = std::min(d.B, d.bc);       // a batch that runs as slices is timed at the slice size
+    const i64 nx = nb * Cin * H * W, ny = nb * Cout * d.oh * d.ow, nw = Cout * Cin * kh * kw;
+    float *x = nullptr, *y = nullptr, *w = nullptr, *bias = nullptr;
+    auto release = [&] {
+        (void)hipStreamSynchronize(c->stream);
+        for (float* p : {x, y, w, bias})
+            if (p) (void)hipFree(p);
+    };
+    hipError_t e = hipMalloc((void**)&x, (size_t)nx * 4);
+    if (e == hipSuccess) e = hipMalloc((void**)&y, (size_t)ny * 4);
+    if (e == hipSuccess) e = hipMalloc((void**)&w, (size_t)nw * 4);
+    if (e == hipSuccess && with_bias) e = hipMalloc((void**)&bias, (size_t)Cout * 4);
+    if (e == hipSuccess) e = hipMemsetAsync(x, 0, (size_t)nx * 4, c->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(y, 0, (size_t)ny * 4, c->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(w, 0, (size_t)nw * 4, c->stream);
+    if (e == hipSuccess && bias) e = hipMemsetAsync(bias, 0, (size_t)Cout * 4, c->stream);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        release();
+        fx::set_error("fx_conv2d_tune: temporary tensors: %s", hipGetErrorString(e));
+        return e == hipErrorOutOfMemory ? FX_ERR_OOM : FX_ERR_HIP;
+    }
+    c->conv_retune = true;
+    int rc;
+    if (kind == FX_CONV_FWD) rc = conv_fwd<float>(c, x, w, y, nb, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, nullptr, 0, bias, act);
+    else rc = conv_dgrad<float>(c, y, w, x, nb, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, 0, nullptr, 0);
+    c->conv_retune = false;
+    release();
+    return rc;
+}
+
 #define FX_DEFINE_CONV(T, S)                                                                                           \
     extern "C" int fx_conv2d_fwd_##S(fx_ctx* c, const T* x, const T* w, T* y, int64_t B, int64_t Cin, int64_t H, int64_t W, \
                                      int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,  \

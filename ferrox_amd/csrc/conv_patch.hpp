@@ -424,17 +424,41 @@ inline int launch_plan(fx_ctx* c, const Plan& pl, const float* x, const float* w
 }
 
 // Runs the layer with the tile shape that measured fastest for this layer shape on this device.  The first call for a
-// shape times the candidate shapes (each writes the same, complete output: the order of every output's sum does not depend
-// on the tile shape) and remembers the winner in the context; FX_CONV_TUNE=0 keeps the modelled choice.
+// layer (filter, map and channel sizes, stride, padding, epilogue) and batch size class (floor(log2(B)): a ragged last batch
+// shares the class of its neighbours or costs one more timing, never one per distinct size) times the candidate shapes (each
+// writes the same, complete output: the order of every output's sum does not depend on the tile shape) and remembers the
+// winner in the context; fx_conv2d_tune times again whatever the cache holds.  Nothing is timed when the output overlaps an operand (the repeated launches would read
+// what an earlier one wrote), and FX_CONV_TUNE=0 keeps the modelled choice everywhere.
+inline int batch_class(i64 B) {
+    int k = 0;
+    while ((i64(2) << k) <= B) ++k;
+    return k;
+}
+inline bool ranges_overlap(const void* a, i64 a_bytes, const void* b, i64 b_bytes) {
+    const uintptr_t a0 = (uintptr_t)a, b0 = (uintptr_t)b;
+    return a0 < b0 + (uintptr_t)b_bytes && b0 < a0 + (uintptr_t)a_bytes;
+}
 inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float* y, float* wimg, int flip, i64 Cout, i64 Cin, i64 B,
                i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw, const float* bias = nullptr, int relu = 0) {
     static const bool tune = [] { const char* v = getenv("FX_CONV_TUNE"); return !(v && atoi(v) == 0); }();
     if (!tune || pl.nimg) return launch_plan(c, pl, x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu);
-    const std::array<i64, 14> key = {flip, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias ? 1 : 0, relu};
+    const std::array<i64, 14> key = {flip, batch_class(B), C, H, W, M, OH, OW, sh, sw, ph, pw, bias ? 1 : 0, relu};
     Plan cand[11];
     const int n = candidates(cand, c->num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw);
     auto it = c->conv_tile_cache.find(key);
+    if (c->conv_tile_cache.size() > 4096) {  // layer shapes of a process are few; a runaway caller does not grow the table for ever
+        c->conv_tile_cache.clear();
+        it = c->conv_tile_cache.end();
+    }
+    if (it != c->conv_tile_cache.end() && c->conv_retune) {
+        c->conv_tile_cache.erase(it);
+        it = c->conv_tile_cache.end();
+    }
     if (it == c->conv_tile_cache.end()) {
+        const i64 y_bytes = B * M * OH * OW * 4;
+        if (ranges_overlap(y, y_bytes, x, B * C * H * W * 4) || ranges_overlap(y, y_bytes, w, Cout * Cin * 9 * 4) ||
+            (bias && ranges_overlap(y, y_bytes, bias, M * 4)))
+            return launch_plan(c, pl, x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu);
         int best = -1, n_last = n - 1;  // n_last: the candidate launched last
         if (n > 1) {
             if (!c->ev_tune[0]) {

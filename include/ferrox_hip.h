@@ -130,6 +130,20 @@ int fx_d2d(fx_ctx* ctx, void* dst_dev, const void* src_dev, int64_t bytes);
 int64_t fx_conv2d_workspace_bytes(int kind, int dtype, int mode, int64_t B, int64_t Cin, int64_t H, int64_t W,
                                   int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw);
 
+/* Tile-shape timing of the 3x3 f32 convolutions.  fx_conv2d_fwd_f32 (and its bias variant) and fx_conv2d_dgrad_f32 pick
+ * the tile shape of their LDS-patch kernel by measurement: the FIRST call for a layer (filter / map / channel sizes,
+ * stride, padding, epilogue) and batch size class floor(log2(B)) launches every near-tied shape a few times on the
+ * caller's own tensors and waits for the stream once per shape (about 4 launches per shape, up to 11 shapes), then
+ * remembers the winner in the context; every later call is one asynchronous launch.  All shapes write the same complete
+ * output with the same bits, so only latency differs.  The output must not overlap an operand (then nothing is timed and
+ * the modelled shape is used).  FX_CONV_TUNE=0 in the environment switches the timing off.  fx_conv2d_tune_f32 pays that
+ * cost up front for a layer (kind FX_CONV_FWD or FX_CONV_DGRAD; FX_CONV_WGRAD is accepted and has nothing to time), on
+ * temporary zero-filled tensors it allocates and frees itself; it synchronises the stream.  with_bias / act select the
+ * epilogue of fx_conv2d_fwd_bias_act (both 0 for plain fx_conv2d_fwd).  No counterpart in the reference (its kernels have
+ * one fixed launch geometry, src/backend/cuda/ops.rs:57-118). */
+int fx_conv2d_tune_f32(fx_ctx* ctx, int kind, int64_t B, int64_t Cin, int64_t H, int64_t W, int64_t Cout, int64_t kh,
+                       int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw, int with_bias, int act);
+
 /* Binary / scalar / unary op selectors for the generic entry points (also exported one by one below). */
 enum fx_binary_op { FX_ADD = 0, FX_SUB = 1, FX_MUL = 2, FX_DIV = 3, FX_EQUAL = 4, FX_GREATER = 5, FX_GREATER_EQUAL = 6,
                     FX_LESS = 7, FX_LESS_EQUAL = 8, FX_MIN = 9, FX_MAX = 10, FX_POW = 11 };

@@ -609,6 +609,28 @@ def test_conv2d_image_layer_kernels(ctx, orc):
         assert np.array_equal(out.numpy(), gw), case
 
 
+def test_conv2d_tune_up_front_and_ragged_batch(ctx, orc):
+    """fx_conv2d_tune_f32 pays the tile timing for a layer before its first use; a ragged batch of the same size class and
+    one of another class run afterwards, all against the oracle.  An output that overlaps an operand is not timed."""
+    from ferrox_amd import capi
+    rng = np.random.default_rng(61)
+    Cin, H, W, Cout = 64, 16, 16, 64
+    w = (rng.standard_normal((Cout, Cin, 3, 3)) * 0.05).astype(np.float32)
+    dw = ctx.upload(w)
+    for kind in (capi.CONV_FWD, capi.CONV_DGRAD, capi.CONV_WGRAD):
+        ctx.conv2d_tune(kind, (40, Cin, H, W), w.shape, (1, 1), (1, 1))
+    ctx.conv2d_tune(capi.CONV_FWD, (40, Cin, H, W), w.shape, (1, 1), (1, 1), with_bias=True, act=1)
+    for B in (40, 37, 9):
+        x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(np.float32)
+        g = rng.standard_normal((B, Cout, H, W)).astype(np.float32)
+        y = ctx.conv2d_fwd(ctx.upload(x), dw, (1, 1), (1, 1)).numpy()
+        d = ctx.conv2d_dgrad(ctx.upload(g), dw, x.shape, (1, 1), (1, 1), 0).numpy()
+        assert rel_err(y, orc.conv2d_fwd(x, w, (1, 1), (1, 1))) <= 8e-5 / 8
+        assert rel_err(d, orc.conv2d_dgrad(g, w, x.shape, (1, 1), (1, 1), 0)) <= 8e-5 / 8
+    with pytest.raises(capi.FerroxHipError, match="unknown kind"):
+        ctx.conv2d_tune(7, (4, Cin, H, W), w.shape, (1, 1), (1, 1))
+
+
 def test_conv2d_tile_shape_timing_does_not_change_the_bits(ctx, tmp_path):
     """The forward / data-gradient patch kernel times its candidate tile shapes on the first call of a layer shape.  Every
     shape adds the terms of an output in the same order, so a process that keeps the modelled shape (FX_CONV_TUNE=0) must
