@@ -27,6 +27,7 @@ PEAK_F64_MFMA_TFLOPS = 78.6
 PEAK_HBM_GBS = 8000.0
 
 C3 = dict(B=128, Cin=64, H=56, W=56, Cout=128, k=3, s=1, p=1)
+PRIMING_STEPS = 20  # untimed steps before the `--warmup` steps of the headline measurement
 
 
 def time_stream(ctx, fn, iters, warmup):
@@ -44,10 +45,35 @@ CONV_KERNELS = {"fwd": "cpk::conv_patch_kernel (conv fwd pass)", "dgrad": "cpk::
                 "wgrad": "wgp::wgrad_patch_kernel + wgrad_patch_reduce_kernel (conv wgrad pass)"}
 
 
-# HBM-side bytes per launch of the main kernel of each C3 pass: rocprofv3 FETCH_SIZE + WRITE_SIZE per dispatch,
-# scaled by what the same counters read for the streaming add kernel of known size (x2.000 and x1.000); the
-# summary with the commands is profiles/conv_c3_f32_hbm_traffic.txt.
-CONV_C3_TRAFFIC_BYTES = {"fwd": 322.1e6, "dgrad": 319.0e6, "wgrad": 518.4e6}
+def profile_traffic(path, row):
+    """HBM-side bytes per launch of a kernel from a committed rocprofv3 counter summary under profiles/: the row that
+    starts with `row`, column "total MB" (FETCH_SIZE + WRITE_SIZE per dispatch, each scaled by what the same counter reads
+    for a streaming kernel of known size; the file states the commands and the factors).  Returns (bytes or None, source
+    label with the file's content hash, so a line can be traced to the summary it was taken from)."""
+    import hashlib
+    full = os.path.join(ROOT, path)
+    try:
+        text = open(full).read()
+    except OSError:
+        return None, f"{path} (missing)"
+    label = f"{path} sha1:{hashlib.sha1(text.encode()).hexdigest()[:12]}"
+    header = None
+    for line in text.splitlines():
+        cells = [c.strip() for c in line.split("|")]
+        if len(cells) < 3:
+            continue
+        if "total MB" in cells:
+            header = cells
+        elif header and cells[0] == row and len(cells) == len(header):
+            try:
+                return float(cells[header.index("total MB")]) * 1e6, label
+            except ValueError:
+                return None, label
+    return None, label
+
+
+CONV_C3_TRAFFIC_FILE = "profiles/conv_c3_f32_hbm_traffic.txt"
+C4_TRAFFIC_FILE = "profiles/c4_bandwidth_kernels_hbm_traffic.txt"
 
 
 def bench_conv(ctx, steps, warmup, dtype=np.float32, B=None):
@@ -72,8 +98,8 @@ def bench_conv(ctx, steps, warmup, dtype=np.float32, B=None):
             fn()
 
     # Clocks and caches settle over the first few tens of milliseconds of MFMA load; these priming steps are untimed
-    # and come on top of the `warmup` steps of the contract.
-    for _ in range(20):
+    # and come on top of the `warmup` steps of the contract (reported as "priming_steps" in the output line).
+    for _ in range(PRIMING_STEPS):
         step()
     # the timed region of the headline number: exactly `steps` steps between two synchronisations
     for _ in range(warmup):
@@ -102,49 +128,116 @@ def bench_conv(ctx, steps, warmup, dtype=np.float32, B=None):
     return res
 
 
-def bench_bandwidth(ctx, iters=20, warmup=3):
-    import ctypes
+REDUCE_VIEWS = (("0", (1, 8192, 8192)), ("1", (8192, 8192, 1)), ("all", (1, 8192 * 8192, 1)))
+ROTATE = 4  # distinct inputs a reduction cycles through: 4 x 256 MiB (f32) can not stay in the 256 MiB last-level cache
+
+
+def c4_reduction_cases(ctx, dtype, rotate):
+    """The nine reductions of config C4 on [8192, 8192] of one dtype: (name, algorithmic bytes, call) where call(j) reduces
+    input j % rotate.  Algorithmic bytes = sizeof(T) * (8192^2 + outputs) + 8 * outputs for the int64 argmax indices."""
+    import ctypes  # noqa: F401
     from ferrox_amd import capi
-    C_i64 = ctypes.c_int64
-    out = {"reductions": {}, "elementwise": {}, "pooling": {}}
-    for dtype in (np.float32, np.float64):
-        sfx = capi.dtype_code(dtype)[1]
-        a = ctx.normal((8192, 8192), 4, 0.0, 1.0, dtype)
-        res = ctx.empty((8192,), dtype)
-        idx = ctx.empty((8192,), np.float64)  # int64 argmax indices (8 bytes each)
-        for kind in ("sum", "mean", "max"):
-            for axis, view in (("0", (1, 8192, 8192)), ("1", (8192, 8192, 1)), ("all", (1, 8192 * 8192, 1))):
-                n_out = view[0] * view[2]
-                if kind == "max":
-                    fn = lambda: capi.check(getattr(capi.lib, f"fx_reduce_max_{sfx}")(ctx.h, a.ptr, res.ptr, idx.ptr, *view))  # noqa: E731
-                    nbytes = a.dtype.itemsize * (a.size + n_out) + 8 * n_out
-                else:
-                    fn = lambda: capi.check(getattr(capi.lib, f"fx_reduce_{kind}_{sfx}")(ctx.h, a.ptr, res.ptr, *view))  # noqa: E731
-                    nbytes = a.dtype.itemsize * (a.size + n_out)
-                ms = time_stream(ctx, fn, iters, warmup)
-                out["reductions"][f"{kind}_axis{axis}_{sfx}"] = {"us": ms * 1e3, "GBps": nbytes / ms / 1e6,
-                                                                 "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
-        del a, res, idx
+    sfx = capi.dtype_code(dtype)[1]
+    ins = [ctx.normal((8192, 8192), 4 + j, 0.0, 1.0, dtype) for j in range(rotate)]
+    res = ctx.empty((8192,), dtype)
+    idx = ctx.empty((8192,), np.float64)  # int64 argmax indices (8 bytes each)
+    cases = []
+    for kind in ("sum", "mean", "max"):
+        for axis, view in REDUCE_VIEWS:
+            n_out = view[0] * view[2]
+            if kind == "max":
+                f = getattr(capi.lib, f"fx_reduce_max_{sfx}")
+                call = lambda j, f=f, view=view: capi.check(f(ctx.h, ins[j % rotate].ptr, res.ptr, idx.ptr, *view))  # noqa: E731
+                nbytes = ins[0].dtype.itemsize * (ins[0].size + n_out) + 8 * n_out
+            else:
+                f = getattr(capi.lib, f"fx_reduce_{kind}_{sfx}")
+                call = lambda j, f=f, view=view: capi.check(f(ctx.h, ins[j % rotate].ptr, res.ptr, *view))  # noqa: E731
+                nbytes = ins[0].dtype.itemsize * (ins[0].size + n_out)
+            cases.append((f"{kind}_axis{axis}_{sfx}", nbytes, call))
+    return cases, (ins, res, idx)
+
+
+def c4_elementwise_cases(ctx):
+    """add / mul and the fused ReLU / sigmoid / tanh gradients on 2^28 f32: 3 arrays of 1 GiB per call."""
     n = 1 << 28
     g = ctx.uniform((n,), 7, -4.0, 4.0)
     x = ctx.uniform((n,), 8, -4.0, 4.0)
     s = ctx.unary("sigmoid", x)
     t = ctx.unary("tanh", x)
     o = ctx.empty((n,))
-    cases = {
-        "add": lambda: ctx.binary("add", g, x, out=o),
-        "mul": lambda: ctx.binary("mul", g, x, out=o),
-        "relu_bwd": lambda: ctx.relu_bwd(g, x, out=o),
-        "sigmoid_bwd": lambda: ctx.sigmoid_bwd(g, s, 0, out=o),
-        "tanh_bwd": lambda: ctx.tanh_bwd(g, t, out=o),
-    }
-    for name, fn in cases.items():
-        ms = time_stream(ctx, fn, 10, 2)
-        nbytes = 3 * 4 * n
-        out["elementwise"][f"{name}_f32"] = {"ms": ms, "GBps": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    cases = [
+        ("add_f32", 3 * 4 * n, lambda j: ctx.binary("add", g, x, out=o)),
+        ("mul_f32", 3 * 4 * n, lambda j: ctx.binary("mul", g, x, out=o)),
+        ("relu_bwd_f32", 3 * 4 * n, lambda j: ctx.relu_bwd(g, x, out=o)),
+        ("sigmoid_bwd_f32", 3 * 4 * n, lambda j: ctx.sigmoid_bwd(g, s, 0, out=o)),
+        ("tanh_bwd_f32", 3 * 4 * n, lambda j: ctx.tanh_bwd(g, t, out=o)),
+    ]
+    return cases, (g, x, s, t, o)
+
+
+def time_cycling(ctx, call, iters, warmup, rotate=1):
+    """Average ms per call; call(j) receives a running index so that consecutive calls may take different inputs."""
+    k = [0]
+
+    def fn():
+        call(k[0])
+        k[0] += 1
+    return time_stream(ctx, fn, iters, warmup)
+
+
+def bench_c4_profile(ctx, iters=4):
+    """Profiler mode: every C4 kernel `iters` times on rotating inputs, cases separated by a one-element fill (a marker
+    dispatch a counter trace can be split on).  Prints the order of the cases."""
+    from ferrox_amd import capi
+    marker = ctx.empty((1,))
+    order = []
+
+    def run_case(name, nbytes, call):
+        capi.check(capi.lib.fx_fill_f32(ctx.h, marker.ptr, float(len(order)), 1))
+        for j in range(iters):
+            call(j)
+        order.append({"case": name, "algorithmic_bytes": nbytes, "calls": iters})
+
+    for dtype in (np.float32, np.float64):
+        cases, keep = c4_reduction_cases(ctx, dtype, ROTATE)
+        for c in cases:
+            run_case(*c)
+        ctx.sync()
+        del cases, keep
+    cases, keep = c4_elementwise_cases(ctx)
+    for c in cases:
+        run_case(*c)
+    capi.check(capi.lib.fx_fill_f32(ctx.h, marker.ptr, -1.0, 1))
+    ctx.sync()
+    return order
+
+
+def bench_bandwidth(ctx, iters=20, warmup=3):
+    import ctypes
+    from ferrox_amd import capi
+    C_i64 = ctypes.c_int64
+    out = {"reductions": {}, "elementwise": {}, "pooling": {}}
+    # Reductions: `us_same_input` re-reads one buffer (an 8192^2 f32 matrix is exactly the size of the 256 MiB last-level
+    # cache, so part of it is served from there); `us` cycles through ROTATE distinct inputs, which no cache can hold:
+    # that is the figure quoted against the HBM peak.
+    for dtype in (np.float32, np.float64):
+        cases, keep = c4_reduction_cases(ctx, dtype, ROTATE)
+        for name, nbytes, call in cases:
+            same = time_cycling(ctx, lambda j: call(0), iters, warmup)
+            ms = time_cycling(ctx, call, iters, warmup + ROTATE)
+            out["reductions"][name] = {"us": ms * 1e3, "GBps": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS,
+                                       "us_same_input": same * 1e3, "GBps_same_input": nbytes / same / 1e6,
+                                       "algorithmic_bytes": nbytes, "inputs_cycled": ROTATE}
+        del cases, keep
+    cases, keep = c4_elementwise_cases(ctx)
+    for name, nbytes, call in cases:
+        ms = time_cycling(ctx, call, 10, 2)
+        out["elementwise"][name] = {"ms": ms, "GBps": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS,
+                                    "algorithmic_bytes": nbytes}
+    del cases, keep
+    n = 1 << 28
     # pooling and its gradient on [128, 64, 112, 112] f32, 2x2 stride 2: algorithmic bytes = input + output (forward),
     # grad_out + input + pooled + grad_in (max gradient), grad_out + grad_in (avg gradient)
-    del g, x, s, t, o
     pshape, k2 = (128, 64, 112, 112), ((2, 2), (2, 2), (0, 0))
     px = ctx.uniform(pshape, 9, -1.0, 1.0)
     n_in, n_out = px.size, px.size // 4
@@ -279,6 +372,15 @@ def make_train_problem(cfg, dtype):
     x = rng.standard_normal(cfg["in_shape"]).astype(dtype)
     y = np.eye(cfg["classes"], dtype=dtype)[rng.integers(0, cfg["classes"], cfg["in_shape"][0])]
     return params, x, y
+
+
+def c5_step_flop(batch=256):
+    """Algorithmic FLOP of one C5 training step: 2*M*N*K per product; conv1 3->32 on 32x32 (forward + weight gradient: its
+    input needs no gradient), conv2 32->64 stride 2 -> 16x16 and the 16384->10 classifier (forward + both gradients)."""
+    conv1 = 2.0 * 32 * 27 * batch * 32 * 32
+    conv2 = 2.0 * 64 * 288 * batch * 16 * 16
+    fc = 2.0 * batch * 10 * 16384
+    return 2 * conv1 + 3 * conv2 + 3 * fc
 
 
 def reference_pool_config():
@@ -448,6 +550,9 @@ def main():
     ap.add_argument("--train-only", nargs="?", const="all", default=None, metavar="CONFIG,DTYPE,ENGINE",
                     help="run only the train-step section and print it (profiler runs); optional filter such as "
                          "C5_cnn,float32,engine_fused")
+    ap.add_argument("--c4-profile", action="store_true",
+                    help="run only the C4 bandwidth kernels, 4 calls each on rotating inputs with marker dispatches between "
+                         "the cases, and print the case order (for rocprofv3 counter runs)")
     ap.add_argument("--conv-sweep", action="store_true",
                     help="run only a sweep of 3x3 stride-1 f32 layer shapes (Cin, Cout in 32..256; 8x8..64x64 maps) and print "
                          "TFLOP/s per pass as one JSON line")
@@ -456,6 +561,11 @@ def main():
         sys.exit("bench.py: this build runs on exactly one GPU (the hot path has no cross-GPU exchange built); use --gpus 1")
     if args.conv_sweep:
         print(json.dumps({"conv_sweep_tflops_fwd_dgrad_wgrad": bench_conv_sweep()}))
+        return
+    if args.c4_profile:
+        from ferrox_amd import capi
+        with capi.Context(0) as ctx:
+            print(json.dumps({"c4_profile_order": bench_c4_profile(ctx)}))
         return
     if args.train_only:
         only = None if args.train_only == "all" else tuple(args.train_only.split(","))
@@ -467,6 +577,7 @@ def main():
     conv = bench_conv(ctx, args.steps, args.warmup)
     dominant = max(conv["per_pass"], key=lambda k: conv["per_pass"][k]["ms"])
     dom = conv["per_pass"][dominant]
+    traffic, traffic_src = profile_traffic(CONV_C3_TRAFFIC_FILE, dominant)
     result = {
         "metric": "conv fwd+bwd TFLOP/s",
         "value": conv["tflops"],
@@ -474,6 +585,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "priming_steps": PRIMING_STEPS,
         "ms_per_step": conv["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
@@ -484,23 +596,42 @@ def main():
                    "flop_per_step": 3 * conv["flop_per_pass"], "device": ctx.device_name()},
         "roofline": {"bound": "mfma", "kernel": CONV_KERNELS[dominant], "achieved": dom["tflops"],
                      "peak": PEAK_F32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": dom["tflops"] / PEAK_F32_MFMA_TFLOPS,
-                     "traffic": CONV_C3_TRAFFIC_BYTES[dominant], "traffic_unit": "bytes per launch",
+                     "traffic": traffic, "traffic_unit": "bytes per launch", "traffic_source": traffic_src,
                      "algorithmic_bytes": 308.6e6, "avg_launch_ms": dom["ms"]},
         "conv_passes": {k: {"ms": v["ms"], "tflops": v["tflops"], "frac_mfma_f32": v["tflops"] / PEAK_F32_MFMA_TFLOPS}
                         for k, v in conv["per_pass"].items()},
         "conv_fwd_bias_relu": conv.get("fwd_bias_relu"),
     }
     if not args.skip_also:
-        c64 = bench_conv(ctx, max(3, args.steps // 4), 1, np.float64, B=64)
+        c64 = bench_conv(ctx, max(3, args.steps // 4), 1, np.float64, B=C3["B"])
         result["also"] = {
-            "conv_f64_batch64": {k: {"ms": v["ms"], "tflops": v["tflops"], "frac_mfma_f64": v["tflops"] / PEAK_F64_MFMA_TFLOPS}
-                                 for k, v in c64["per_pass"].items()},
+            "conv_f64": {k: {"ms": v["ms"], "tflops": v["tflops"], "frac_mfma_f64": v["tflops"] / PEAK_F64_MFMA_TFLOPS}
+                         for k, v in c64["per_pass"].items()},
         }
         result["also"].update(bench_bandwidth(ctx))
+        # second BASELINE metric: the slowest C4 bandwidth kernel against the HBM peak (reductions on rotating inputs)
+        worst_name, worst = min([kv for kv in list(result["also"]["reductions"].items()) + list(result["also"]["elementwise"].items())
+                                 if "frac_hbm" in kv[1]], key=lambda kv: kv[1]["frac_hbm"])
+        w_traffic, w_src = profile_traffic(C4_TRAFFIC_FILE, worst_name)
+        w_ms = worst["us"] / 1e3 if "us" in worst else worst["ms"]
+        result["also"]["roofline_c4_worst"] = {
+            "bound": "hbm", "kernel": worst_name, "achieved": worst["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": worst["frac_hbm"], "traffic": w_traffic, "traffic_unit": "bytes per launch", "traffic_source": w_src,
+            "algorithmic_bytes": worst["algorithmic_bytes"], "avg_launch_ms": w_ms}
     ctx.close()
     if not args.skip_also and not args.skip_train:
         result["also"]["train_step"] = bench_train_steps(cpu=not args.skip_cpu)
         result["also"]["train_step_reference_pool_config"] = bench_train_steps(cpu=False, reference_pool=True)
+        # third BASELINE metric: the CNN training step (fused engine) -- algorithmic FLOP of its three GEMM-shaped layers
+        # (forward, data gradient where one is needed, weight gradient) over the step's wall time, against the f32 MFMA peak
+        c5 = result["also"]["train_step"].get("C5_cnn_float32", {}).get("engine_fused")
+        if c5:
+            flop = c5_step_flop()
+            tfl = flop / (c5["ms_per_step"] * 1e-3) / 1e12
+            result["also"]["roofline_c5_train_step"] = {
+                "bound": "mfma", "kernel": "C5 CNN train step, fused engine (all kernels of the step)", "achieved": tfl,
+                "peak": PEAK_F32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": tfl / PEAK_F32_MFMA_TFLOPS, "traffic": None,
+                "algorithmic_flop": flop, "avg_launch_ms": c5["ms_per_step"], "imgs_per_s": c5["imgs_per_s"]}
     if not args.skip_cpu:
         result["cpu_baseline"] = cpu_baseline_conv()
     print(json.dumps(result))
