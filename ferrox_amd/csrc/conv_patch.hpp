@@ -14,6 +14,7 @@
 // kernel.  The next stage's global loads are issued before the MFMA loop of the current one.
 #pragma once
 #include <array>
+#include <cstdio>
 #include <cstdlib>
 
 #include "wgrad_patch.hpp"
@@ -26,9 +27,15 @@ using wgp::ldg4;
 constexpr int CC = 8, NT = 256, KK = 9;
 constexpr int WPITCH = KK * CC + 1;         // 73
 constexpr int NXP_SHORT = 4, NXP_TALL = 10;  // patch rows are staged two per pass: up to 8 rows, or 20 (strided layers)
+constexpr int NXP_PERSIST = 6;              // persistent variant: up to 12 patch rows
 constexpr int LPR = 16;                     // lanes per patch row: W <= 64
 constexpr int SLACK = 16;
 constexpr size_t LDS_BUDGET = 72 * 1024;
+// persistent variant: fixed plane pitch (1 mod 4) and buffer size, so that buffer, channel pair and tap column are all
+// part of the 16-bit immediate offset of an LDS read: 2 x (8 x 1149 + 16) x 4 bytes = 73664 <= LDS_BUDGET
+constexpr int PPLANE = 1149, PBUF = CC * PPLANE + SLACK;
+constexpr size_t PP_LDS = 2 * (size_t)PBUF * sizeof(float);
+static_assert(PP_LDS <= LDS_BUDGET && (PBUF + 6 * PPLANE + 2) * 4 < 65536 && PPLANE % 4 == 1, "persistent patch buffers");
 
 struct Params {
     const float* x;
@@ -43,6 +50,9 @@ struct Params {
     // small maps (MULTI): a tile holds nimg whole images, image i in patch rows [i * RPI, (i + 1) * RPI)
     int nimg, RPI, B;
     FastDiv div_L, div_rpi;
+    // persistent variant: all tiles (mtiles x B x tpi), floats per patch buffer, B * tpi
+    int ntiles, bufsz, bt;
+    FastDiv div_bt;
 };
 
 // Weight images: out[mt][ch][m][tap*8 + cc], zero in column 72 and in rows past the last output channel.
@@ -154,7 +164,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
             const int idx = wd + u * NT;
             if ((u + 1) * NT <= WIMG / 4 || idx < WIMG / 4) *reinterpret_cast<float4*>(Ws + 4 * idx) = wv[u];
         }
-        if (x_lane) {
+        if (x_lane && !(p.relu & 4096)) {
 #pragma unroll
             for (int u = 0; u < NXP; ++u) {
                 const int r = 2 * u + rp;
@@ -247,6 +257,262 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
     }
 }
 
+
+// ---- persistent variant ------------------------------------------------------------------------------------------
+// The kernel above pays, per stage, for parking a 37 KB weight image in LDS between two barriers and, per tile, for a
+// prologue (first loads exposed) and an epilogue (a block's slot waits for its stores): measured on the 128 x 64 x 56 x 56 -> 128
+// layer, 6.5 % of the time goes to staging and 4 % to the stores.  This variant removes both:
+//   * the weights never touch LDS: every lane loads the 36 A values of its output-channel row for a stage as nine 16-byte
+//     global loads from an image laid out in MFMA operand order ([32-row block][chunk][tap][lane][channel pair]), one stage
+//     ahead, into one of two register sets;
+//   * the patch is double-buffered in LDS, so a stage has ONE barrier and the next patch is written while other waves still
+//     compute; its row pitch is padded so that the 32 pixels of an MFMA operand read fall on 32 different banks also when
+//     the run wraps to the next output row (pitch - OW = 32);
+//   * blocks are persistent (two per CU) and walk their tiles with the stage pipeline running across tile boundaries: the
+//     loads for a tile's first stage are issued during the previous tile's last stage, and the stores of a finished tile
+//     drain while the next one computes.
+// Weight images: out[mb][ch][tap][lane][e] = wgt[m = mb*32 + lane%32][c = ch*8 + 2e + lane/32][tap], zero in rows past M
+// (wgt as for wimg_kernel: the filter, or the flipped transposed filter of the data gradient).
+__global__ __launch_bounds__(256) void wimg2_kernel(const float* __restrict__ w, float* __restrict__ out, int Cout, int Cin, int M,
+                                                    int nchunks, int flip, i64 n) {
+    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int e = (int)(i & 3), lane = (int)((i >> 2) & 63);
+    i64 r = i >> 8;
+    const int t = (int)(r % KK);
+    r /= KK;
+    const int ch = (int)(r % nchunks), mb = (int)(r / nchunks);
+    const int mm = mb * 32 + (lane & 31), c = ch * CC + 2 * e + (lane >> 5);
+    float v = 0.f;
+    if (mm < M) v = flip ? w[((i64)c * Cin + mm) * KK + (KK - 1 - t)] : w[((i64)mm * Cin + c) * KK + t];
+    out[i] = v;
+}
+
+__device__ __forceinline__ float f4sel(const float4& v, int e) { return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w; }
+
+template <int WM, int TN, bool BIAS>
+__global__ __launch_bounds__(NT, 1) void conv_patch_persist_kernel(const Params p) {
+    constexpr int BM = 32 * WM, WN = 4 / WM, NPIX = 32 * TN * WN, NXP = NXP_PERSIST;
+    constexpr int AIMG = KK * 64 * 4;  // floats of one (32-row block, chunk) weight image
+    extern __shared__ __align__(16) float smem[];
+    const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
+    // in a scalar register: what derives from the wave index (rows, pointers, tests) stays on the scalar unit
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WM, wn = wave / WM;
+    // this block's tiles: XCD x (workgroup ids go to the 8 XCDs round-robin) owns the contiguous range [x*chunk, (x+1)*chunk)
+    // and deals it to its blocks, so neighbouring tiles of an image are in flight together behind one L2
+    int q, qstep, qend;
+    if (p.xcd_chunk) {
+        const int x = blockIdx.x & 7;
+        q = x * p.xcd_chunk + (blockIdx.x >> 3);
+        qstep = gridDim.x >> 3;
+        qend = (x + 1) * p.xcd_chunk;
+    } else {
+        q = blockIdx.x;
+        qstep = gridDim.x;
+        qend = p.ntiles;
+    }
+    if (q >= qend) return;
+    // One wave per SIMD owns all 512 registers of a lane: the compiler splits them into 256 + 256 once a function touches
+    // the accumulation registers, and then keeps the MFMA accumulators there.
+    {
+        int z = 0;
+        asm volatile("; accumulators in AGPRs %0" : "+a"(z));
+    }
+    for (int i = tid; i < 2 * PBUF; i += NT) smem[i] = 0.f;  // the padding columns of both buffers stay zero from here on
+
+    // geometry of a tile
+    int b, m0, pix0, iy_base, py0, mb;
+    auto geo = [&](int qq) __attribute__((always_inline)) {
+        const int mt = (int)p.div_bt.div((uint32_t)qq), rem = qq - mt * p.bt;
+        b = (int)p.div_tpi.div((uint32_t)rem);
+        pix0 = (rem - b * p.tpi) * NPIX;
+        py0 = (int)p.div_ow.div((uint32_t)pix0);
+        iy_base = py0 * p.sh - p.ph;
+        m0 = mt * BM;
+        mb = mt * WM + wm;
+    };
+    // byte offsets into a patch buffer of this lane's B operands, one set per filter row: everything else about a read
+    // (buffer, channel pair, filter column) is a compile-time constant and rides in the instruction's offset field
+    int boff[3][TN];
+    auto set_boff = [&]() __attribute__((always_inline)) {
+        const int wpix0 = pix0 + wn * 32 * TN;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int pi = wpix0 + j * 32 + l32;
+            const int py = (int)p.div_ow.div((uint32_t)pi), px = pi - py * p.OW;
+            const int o = (pi < p.L ? (py - py0) * p.sh * p.PW + px * p.sw : 0) + half * PPLANE;
+#pragma unroll
+            for (int ky = 0; ky < 3; ++ky) boff[ky][j] = (o + ky * p.PW) * 4;
+        }
+    };
+    f32x16 acc[TN];
+    auto zero_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+    };
+
+    // staging: thread t owns float4 column t % 16 of patch rows 2u + rp of channel (t / 16) % 8, rp = t / 128
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int pq = tid & (LPR - 1), xc = (tid >> 4) & (CC - 1), rp = wave >> 1;  // rp scalar: row tests and row pointers stay on the SALU
+    const bool x_lane = pq < ((p.W + 3) >> 2);
+    const int xcol = min(4 * pq, p.W - 4);
+    const uint32_t x_off = x_lane ? (uint32_t)(xc * p.H * p.W + xcol) * 4u : 0u;
+    const int x_dst0 = xc * PPLANE + p.pw + xcol;
+    float4 Av[2][KK], xv[NXP];
+    // loads of stage (tile geometry in b / iy_base / mb, chunk ch): the A values into register set SET, the patch rows into xv
+    auto prefetch = [&](auto set_c, int ch) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_c)::value;
+        const float* asrc = p.wimg + ((i64)mb * p.nchunks + ch) * AIMG;
+#pragma unroll
+        for (int u = 0; u < KK; ++u) Av[SET][u] = ldg4(asrc + u * 256, (uint32_t)lane * 16u);
+        const float* xsrc = p.x + ((i64)b * p.C + (i64)ch * CC) * p.H * p.W;
+#pragma unroll
+        for (int u = 0; u < NXP; ++u) {
+            const int r = 2 * u + rp, iy = iy_base + r;
+            if (r < p.PR && iy >= 0 && iy < p.H) xv[u] = ldg4(xsrc + (i64)iy * p.W, x_off);  // scalar test
+            else xv[u] = zero4;
+        }
+    };
+    auto park = [&](int buf) __attribute__((always_inline)) {
+        int xd = x_dst0 + buf * PBUF;
+        asm volatile("" : "+v"(xd));
+        if (x_lane) {
+#pragma unroll
+            for (int u = 0; u < NXP; ++u) {
+                const int r = 2 * u + rp;
+                if (r < p.PR) {  // scalar test
+                    const float4 v = xv[u];
+                    float* d = smem + xd + r * p.PW;
+                    d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+                }
+            }
+        }
+    };
+    // One stage: 9 taps x 4 channel pairs, fully unrolled; two B register sets alternate so that the LDS reads of step i+1
+    // are in flight while the MFMAs of step i run.  The A value of step (tap t, pair cp) is component cp of Av[SET][t].
+    auto compute = [&](auto set_c) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_c)::value;
+        float b0[TN], b1[TN];
+#pragma unroll
+        for (int ky = 0; ky < 3; ++ky)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(boff[ky][j]));
+        auto rd = [&](float (&bv)[TN], int step) __attribute__((always_inline)) {
+            const int t = step >> 2, cp = step & 3, ky = t / 3, kx = t % 3;
+            const int imm = (SET * PBUF + 2 * cp * PPLANE + kx) * 4;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) bv[j] = *(const float*)((const char*)smem + boff[ky][j] + imm);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto mma = [&](const float (&bv)[TN], int step) __attribute__((always_inline)) {
+            const float a = f4sel(Av[SET][step >> 2], step & 3);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, bv[j], acc[j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        rd(b0, 0);
+#pragma unroll
+        for (int step = 0; step < KK * 4; step += 2) {
+            rd(b1, step + 1);
+            mma(b0, step);
+            if (step + 2 < KK * 4) rd(b0, step + 2);
+            mma(b1, step + 1);
+        }
+    };
+    // The stores of a tile: a scalar base per accumulator row (SALU) and one 32-bit lane offset per pixel block, so that
+    // a store costs no vector ALU work; tiles that reach past the last output channel or pixel take the checked path.
+    auto store_tile = [&]() __attribute__((always_inline)) {
+        typedef __attribute__((address_space(1))) char gchar;
+        typedef __attribute__((address_space(1))) float gfloat;
+        const int mw = m0 + wm * 32;  // scalar
+        float* const out = p.y + ((i64)b * p.M + mw) * p.L;
+        const int wpix0 = pix0 + wn * 32 * TN;
+        float bv[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int m = mw + igemm::Mfma<float>::row(e, lane);
+            bv[e] = BIAS ? p.bias[m < p.M ? m : p.M - 1] : 0.f;
+        }
+        auto rows = [&](auto checked_c) __attribute__((always_inline)) {
+            constexpr bool CHECKED = decltype(checked_c)::value;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int pi = wpix0 + j * 32 + l32;
+                const uint32_t lo = (uint32_t)(4 * half * p.L + pi) * 4u;
+                if (!CHECKED || pi < p.L) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int ru = 8 * (e / 4) + e % 4;  // row(e, lane) = ru + 4 * half
+                        if (!CHECKED || mw + ru + 4 * half < p.M) {
+                            float v = acc[j][e];
+                            if (BIAS) {
+                                v = v + bv[e];
+                                if (p.relu) v = v > 0.f ? v : 0.f;
+                            }
+                            float* rowp = out + (i64)ru * p.L;
+                            asm volatile("" : "+s"(rowp));  // keeps the row base apart from the lane offset: scalar base + 32-bit offset
+                            *(gfloat*)((gchar*)rowp + lo) = v;
+                        }
+                    }
+                }
+            }
+        };
+        if (mw + 32 <= p.M && wpix0 + 32 * TN <= p.L) rows(std::false_type());
+        else rows(std::true_type());
+    };
+
+    int ch = 0;
+    geo(q);
+    prefetch(std::integral_constant<int, 0>(), 0);
+    set_boff();
+    zero_acc();
+    __syncthreads();  // the zero fill is complete before the first patch lands on it
+    park(0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0) on every path into the loop (see the end of a stage)
+    __syncthreads();
+    // stage with register / LDS set SET; returns false after the block's last stage
+    auto stage = [&](auto set_c) __attribute__((always_inline)) -> bool {
+        constexpr int SET = decltype(set_c)::value;
+        const bool last_ch = ch + 1 == p.nchunks;
+        const int nq = last_ch ? q + qstep : q, nch = last_ch ? 0 : ch + 1;
+        const bool more = nq < qend;
+        // the finished tile's coordinates are needed by its stores after the next tile's have been formed for the loads
+        const int cb = b, cm0 = m0, cpix0 = pix0;
+        if (more) {
+            if (last_ch) geo(nq);
+            prefetch(std::integral_constant<int, SET ^ 1>(), nch);
+        }
+        compute(set_c);
+        // The MFMAs issued last are still running while the patch is parked and the tile stored: a wave's matrix
+        // instructions complete in the background of its own later instructions.
+        if (more) park(SET ^ 1);
+        // Parking waited for the newest loads, so every load has landed; saying so here, BEFORE the stores, keeps the
+        // compiler from guarding the next stage's first MFMAs with waits and leaves the stores to drain under them.
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), other counters untouched
+        if (last_ch) {
+            const int nb = b, nm0 = m0, npix0 = pix0;
+            b = cb; m0 = cm0; pix0 = cpix0;
+            store_tile();
+            b = nb; m0 = nm0; pix0 = npix0;
+            if (more) {
+                set_boff();
+                zero_acc();
+            }
+        }
+        __syncthreads();
+        q = nq;
+        ch = nch;
+        return more;
+    };
+    while (true) {
+        if (!stage(std::integral_constant<int, 0>())) break;
+        if (!stage(std::integral_constant<int, 1>())) break;
+    }
+}
+
 struct Plan {
     bool ok = false;
     int WM = 4, TN = 0, PR = 0, PW = 0, PLANE = 0, tpi = 0, mtiles = 0, nchunks = 0;
@@ -254,6 +520,7 @@ struct Plan {
     int nimg = 0, RPI = 0;  // small maps: images per tile and patch rows per image (0: one image per tile)
     i64 cost = 0;           // modelled cost: rounds of co-resident blocks x MFMA work of a block
     size_t smem = 0;
+    bool persist = false;  // a plan for conv_patch_persist_kernel (persist_plan); PW is then its padded row pitch
     int bm() const { return 32 * WM; }
     int npix() const { return 32 * TN * (4 / WM); }
     i64 wimg() const { return (i64)bm() * WPITCH; }
@@ -280,6 +547,42 @@ inline bool shape_plan(Plan& pl, int wm, int tn, int num_cus, i64 B, i64 C, i64 
     pl.mtiles = (int)mtiles;
     pl.nchunks = (int)(C / CC);
     if (pl.smem > LDS_BUDGET || B * pl.tpi > 0x7fffffff || pl.mtiles > 65535) return false;
+    pl.ok = true;
+    return true;
+}
+
+// Tile shapes of the persistent variant (wm x tn).
+constexpr int N_PSHAPES = 6;
+static const int PSHAPES[N_PSHAPES][2] = {{4, 10}, {4, 7}, {4, 5}, {2, 8}, {2, 5}, {2, 3}};
+inline bool persist_enabled() {
+    static const bool on = [] { const char* v = getenv("FX_CPK_PERSIST"); return v && atoi(v) != 0; }();  // off unless asked for
+    return on;
+}
+// The plan of the persistent variant for one tile shape; false when the shape does not fit this layer.
+inline bool persist_plan(Plan& pl, int wm, int tn, int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph,
+                         i64 pw) {
+    const i64 L = OH * OW, slots = std::max(1, num_cus);
+    const i64 bm = 32 * wm, np = 32 * tn * (4 / wm), tiles = fx::ceil_div(L, np), mtiles = fx::ceil_div(M, bm);
+    const i64 rows = std::min<i64>(OH, np % OW == 0 ? np / OW : (np - 1) / OW + 2), PR = (rows - 1) * sh + 3;
+    if (!persist_enabled() || PR > 2 * NXP_PERSIST || mtiles * bm > M * 2 || tiles * np > L * 2 || B * tiles * mtiles > 0x7fffffff) return false;
+    // patch row pitch: with unit column stride a run of 32 pixels that wraps to the next output row must continue 32
+    // words further on (sh * pitch - OW a multiple of 32), else two of its lanes share a bank; the plain pitch when that
+    // does not fit the plane.
+    i64 pw2 = W + 2 * pw;
+    if (sw == 1) {
+        i64 padded = pw2;
+        while ((sh * padded - OW) % 32 != 0) ++padded;
+        if (PR * padded <= PPLANE) pw2 = padded;
+    }
+    if (PR * pw2 > PPLANE) return false;
+    pl = Plan();
+    pl.persist = true;
+    pl.WM = wm; pl.TN = tn; pl.PR = (int)PR; pl.tpi = (int)tiles; pl.PW = (int)pw2; pl.PLANE = PPLANE;
+    pl.mtiles = (int)mtiles;
+    pl.nchunks = (int)(C / CC);
+    // one block per CU with the matrix pipes to itself: twice the rate of a block of the one-tile kernel, which shares them
+    pl.cost = fx::ceil_div(B * tiles * mtiles, slots) * np * bm / 2;
+    pl.smem = PP_LDS;
     pl.ok = true;
     return true;
 }
@@ -316,6 +619,10 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
     }
     static const int shapes[11][2] = {{4, 8}, {4, 7}, {4, 6}, {4, 5}, {4, 4}, {2, 4}, {2, 3}, {2, 2}, {1, 4}, {1, 3}, {1, 2}};
     Plan best;
+    for (const auto& sp : PSHAPES) {
+        Plan q;
+        if (persist_plan(q, sp[0], sp[1], num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw) && (!best.ok || q.cost < best.cost)) best = q;
+    }
     for (const auto& sp : shapes) {
         Plan q;
         if (shape_plan(q, sp[0], sp[1], num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw) && (!best.ok || q.cost < best.cost)) best = q;
@@ -326,11 +633,17 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
 // Every tile shape whose modelled cost is within 1.5 x of the best one: the candidates that run() times once per layer
 // shape (the model counts MFMA work and rounds of blocks; staging, weight-image size and LDS traffic per MFMA differ
 // between shapes by more than that: measured spreads of 25 % and more between shapes of equal modelled cost).
-inline int candidates(Plan (&out)[11], int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw) {
+constexpr int MAX_CAND = 11 + N_PSHAPES;
+inline int candidates(Plan (&out)[MAX_CAND], int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw) {
     static const int shapes[11][2] = {{4, 8}, {4, 7}, {4, 6}, {4, 5}, {4, 4}, {2, 4}, {2, 3}, {2, 2}, {1, 4}, {1, 3}, {1, 2}};
-    Plan all[11];
+    Plan all[MAX_CAND];
     int n = 0;
     i64 best = -1;
+    for (const auto& sp : PSHAPES)
+        if (persist_plan(all[n], sp[0], sp[1], num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw)) {
+            if (best < 0 || all[n].cost < best) best = all[n].cost;
+            ++n;
+        }
     for (const auto& sp : shapes)
         if (shape_plan(all[n], sp[0], sp[1], num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw)) {
             if (best < 0 || all[n].cost < best) best = all[n].cost;
@@ -341,13 +654,66 @@ inline int candidates(Plan (&out)[11], int num_cus, i64 B, i64 C, i64 H, i64 W, 
         if (all[k].cost * 2 <= best * 3) out[m++] = all[k];
     return m;
 }
+inline int plan_code(const Plan& pl) { return pl.WM * 16 + pl.TN + (pl.persist ? 256 : 0); }
 
 // Sized for 128-row images whatever tile was picked, so the figure does not depend on the CU count behind the plan.
 inline i64 workspace_bytes(const Plan& pl, i64 M) { return fx::ceil_div(M, (i64)128) * 128 * WPITCH * pl.nchunks * (i64)sizeof(float); }
 
 // w is the reference's [Cout][Cin][3][3] filter; flip selects the data-gradient image.
+// The persistent variant for plan pl (pl.persist).
+inline int launch_persist(fx_ctx* c, const Plan& pl, const float* x, const float* w, float* y, float* wimg, int flip, i64 Cout, i64 Cin,
+                          i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw, const float* bias, int relu) {
+    const i64 mblocks = (i64)pl.mtiles * pl.WM;
+    const i64 n = mblocks * pl.nchunks * KK * 64 * 4;
+    wimg2_kernel<<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(w, wimg, (int)Cout, (int)Cin, (int)M, pl.nchunks, flip, n);
+    FX_LAUNCH_CHECK();
+    Params p;
+    p.x = x; p.wimg = wimg; p.y = y; p.bias = bias; p.relu = relu;
+    p.C = (int)C; p.H = (int)H; p.W = (int)W; p.M = (int)M; p.OH = (int)OH; p.OW = (int)OW;
+    p.sh = (int)sh; p.sw = (int)sw; p.ph = (int)ph; p.pw = (int)pw;
+    p.PR = pl.PR; p.PW = pl.PW; p.PLANE = PPLANE; p.L = (int)(OH * OW); p.tpi = pl.tpi; p.nchunks = pl.nchunks;
+    p.div_tpi = FastDiv((uint32_t)pl.tpi);
+    p.div_ow = FastDiv((uint32_t)OW);
+    p.nimg = 0; p.RPI = 0; p.B = (int)B;
+    p.bt = (int)(B * pl.tpi);
+    p.ntiles = (int)(B * pl.tpi * pl.mtiles);
+    p.bufsz = PBUF;
+    p.div_bt = FastDiv((uint32_t)p.bt);
+    int nblk = std::min(p.ntiles, std::max(1, c->num_cus));  // one block per CU
+    p.xcd_chunk = 0;
+    if (p.ntiles % 8 == 0 && nblk >= 8) {
+        nblk -= nblk % 8;
+        p.xcd_chunk = p.ntiles / 8;
+    }
+    const dim3 grid((unsigned)nblk);
+#define FX_CPK_PERSIST(WMV, TNV)                                                                                      \
+    case WMV * 16 + TNV: {                                                                                            \
+        static const hipError_t attr0 = hipFuncSetAttribute((const void*)conv_patch_persist_kernel<WMV, TNV, false>,  \
+                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)PP_LDS); \
+        static const hipError_t attr1 = hipFuncSetAttribute((const void*)conv_patch_persist_kernel<WMV, TNV, true>,   \
+                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)PP_LDS); \
+        FX_HIP_CHECK(attr0);                                                                                          \
+        FX_HIP_CHECK(attr1);                                                                                          \
+        if (bias) conv_patch_persist_kernel<WMV, TNV, true><<<grid, dim3(NT), PP_LDS, c->stream>>>(p);                  \
+        else conv_patch_persist_kernel<WMV, TNV, false><<<grid, dim3(NT), PP_LDS, c->stream>>>(p);                      \
+    } break;
+    switch (pl.WM * 16 + pl.TN) {
+        FX_CPK_PERSIST(4, 10)
+        FX_CPK_PERSIST(4, 7)
+        FX_CPK_PERSIST(4, 5)
+        FX_CPK_PERSIST(2, 8)
+        FX_CPK_PERSIST(2, 5)
+        FX_CPK_PERSIST(2, 3)
+        default: FX_REQUIRE(false, "conv patch kernel (persistent): unexpected tile %d x %d", pl.WM, pl.TN);
+    }
+#undef FX_CPK_PERSIST
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
 inline int launch_plan(fx_ctx* c, const Plan& pl, const float* x, const float* w, float* y, float* wimg, int flip, i64 Cout, i64 Cin, i64 B,
                        i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw, const float* bias, int relu) {
+    if (pl.persist) return launch_persist(c, pl, x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu);
     const i64 n = (i64)pl.mtiles * pl.nchunks * pl.wimg();
     wimg_kernel<<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(w, wimg, (int)Cout, (int)Cin, (int)M, pl.bm(),
                                                                                   pl.nchunks, flip, n);
@@ -443,7 +809,7 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
     static const bool tune = [] { const char* v = getenv("FX_CONV_TUNE"); return !(v && atoi(v) == 0); }();
     if (!tune || pl.nimg) return launch_plan(c, pl, x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu);
     const std::array<i64, 14> key = {flip, batch_class(B), C, H, W, M, OH, OW, sh, sw, ph, pw, bias ? 1 : 0, relu};
-    Plan cand[11];
+    Plan cand[MAX_CAND];
     const int n = candidates(cand, c->num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw);
     auto it = c->conv_tile_cache.find(key);
     if (c->conv_tile_cache.size() > 4096) {  // layer shapes of a process are few; a runaway caller does not grow the table for ever
@@ -469,7 +835,7 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
             int model = 0;
             for (int k = 1; k < n; ++k)
                 if (cand[k].cost < cand[model].cost) model = k;
-            float ms_of[11];
+            float ms_of[MAX_CAND];
             auto time_one = [&](int k, float* ms) -> int {  // one warm-up launch, then three timed ones
                 if (int rc = launch_plan(c, cand[k], x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu)) return rc;
                 FX_HIP_CHECK(hipEventRecord(c->ev_tune[0], c->stream));
@@ -485,6 +851,12 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
             best = model;
             for (int k = 0; k < n; ++k)
                 if (ms_of[k] < 0.95f * ms_of[best]) best = k;
+            static const bool verbose = [] { const char* v = getenv("FX_CONV_VERBOSE"); return v && atoi(v) != 0; }();
+            if (verbose)
+                for (int k = 0; k < n; ++k)
+                    fprintf(stderr, "[ferrox_hip] conv3x3 %s C=%lld %lldx%lld M=%lld: tile %dx%d%s %.4f ms%s%s\n", flip ? "dgrad" : "fwd", (long long)C,
+                            (long long)H, (long long)W, (long long)M, cand[k].WM, cand[k].TN, cand[k].persist ? " persistent" : "", ms_of[k] / 3,
+                            k == model ? " (model)" : "", k == best ? " (fastest)" : "");
             if (best != model) {  // a challenger has to win a second time against the modelled shape
                 float again_model = 0.f, again_best = 0.f;
                 if (int rc = time_one(model, &again_model)) return rc;
@@ -493,12 +865,12 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
                 if (!(again_best < 0.95f * again_model)) best = model;
             }
         }
-        const int code = best >= 0 ? cand[best].WM * 16 + cand[best].TN : pl.WM * 16 + pl.TN;
+        const int code = plan_code(best >= 0 ? cand[best] : pl);
         it = c->conv_tile_cache.emplace(key, code).first;
         if (best >= 0 && best == n_last) return FX_OK;  // the candidate launched last is the winner: its output stands
     }
     for (int k = 0; k < n; ++k)
-        if (cand[k].WM * 16 + cand[k].TN == it->second)
+        if (plan_code(cand[k]) == it->second)
             return launch_plan(c, cand[k], x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu);
     return launch_plan(c, pl, x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu);
 }

@@ -114,6 +114,7 @@ def wgrad_loads_in_bounds(B, Cin, H, W, Cout, st, pd):
 
 CC, KK, WPITCH = 8, 9, 73
 NXP_SHORT, NXP_TALL = 4, 10
+PPLANE = 1149   # fixed plane pitch of the persistent variant
 def _ceil_div(a, b): return (a + b - 1) // b
 def _odd_pitch_c(n): return (n + 30) // 32 * 32 + 1
 def fwd_plan(num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
@@ -171,7 +172,10 @@ def fwd_loads_in_bounds(B, C, H, W, M, sh, sw, ph, pw):
     plans = fwd_plan(256, B, C, H, W, M, OH, OW, sh, sw, ph, pw)
     if plans is None: return "generic"
     # every tile shape that fits is walked: the library times the candidates once per layer shape and keeps the fastest
-    return " ".join(fwd_shape_loads_in_bounds(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw) for pl in plans)
+    out = [fwd_shape_loads_in_bounds(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw) for pl in plans]
+    if not plans[0].get("nimg"):
+        out += [persist_walk(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw) for pl in persist_plans(B, C, H, W, M, OH, OW, sh, sw, ph, pw)]
+    return " ".join(out)
 def fwd_shape_loads_in_bounds(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
     if pl.get("nimg"): return fwd_multi_loads_in_bounds(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw)
     WIMG = pl["BM"] * WPITCH
@@ -202,6 +206,74 @@ def fwd_shape_loads_in_bounds(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
                                     row0 = ((b * C + ch * CC + xc) * H + iy) * W
                                     assert row0 <= a and a + 4 <= row0 + W
     return "patch %dx%d ok" % (pl["WM"], pl["TN"])
+
+
+NXP_PERSIST = 6
+def persist_plans(B, C, H, W, M, OH, OW, sh, sw, ph, pw):
+    """The tile shapes of conv_patch_persist_kernel that fit a layer (persist_plan)."""
+    L, plans = OH * OW, []
+    for wm, tn in [(4, 10), (4, 7), (4, 5), (2, 8), (2, 5), (2, 3)]:
+        bm, np_ = 32 * wm, 32 * tn * (4 // wm)
+        tiles, mtiles = _ceil_div(L, np_), _ceil_div(M, bm)
+        rows = min(OH, np_ // OW if np_ % OW == 0 else (np_ - 1) // OW + 2); PR = (rows - 1) * sh + 3
+        if PR > 2 * NXP_PERSIST or mtiles * bm > M * 2 or tiles * np_ > L * 2: continue
+        pw2 = W + 2 * pw
+        if sw == 1:
+            padded = pw2
+            while (sh * padded - OW) % 32: padded += 1
+            if PR * padded <= PPLANE: pw2 = padded
+        if PR * pw2 > PPLANE: continue
+        plans.append(dict(WM=wm, TN=tn, PR=PR, tpi=tiles, mtiles=mtiles, nchunks=C // CC, BM=bm, NPIX=np_, PW=pw2))
+    return plans
+def persist_walk(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw, num_cus=256):
+    """conv_patch_persist_kernel: the blocks' tile sequences cover every tile exactly once; weight-image, input and output
+    addresses and the LDS offsets of every tile stay inside their buffers."""
+    PW, PLANE, bufsz = pl["PW"], PPLANE, CC * PPLANE + 16
+    assert PLANE % 4 == 1 and PLANE >= pl["PR"] * PW and PW >= W + 2 * pw and pl["PR"] <= 2 * NXP_PERSIST
+    L, WM, TN, NPIX = OH * OW, pl["WM"], pl["TN"], pl["NPIX"]
+    bt = B * pl["tpi"]; ntiles = bt * pl["mtiles"]
+    nblk = min(ntiles, num_cus); chunk = 0          # one block per CU
+    if ntiles % 8 == 0 and nblk >= 8:
+        nblk -= nblk % 8; chunk = ntiles // 8
+    seen = [0] * ntiles
+    for bid in range(nblk):
+        if chunk: x = bid & 7; q, step, end = x * chunk + (bid >> 3), nblk >> 3, (x + 1) * chunk
+        else: q, step, end = bid, nblk, ntiles
+        while q < end:
+            seen[q] += 1; q += step
+    assert all(v == 1 for v in seen), "tiles visited %s" % sorted(set(seen))
+    wbuf2 = pl["mtiles"] * WM * pl["nchunks"] * KK * 64 * 4            # floats written by wimg2_kernel
+    assert wbuf2 * 4 <= _ceil_div(M, 128) * 128 * WPITCH * pl["nchunks"] * 4   # the workspace the entry point asks for
+    xsize, ysize = B * C * H * W, B * M * L
+    tiles = sorted({0, 1, pl["tpi"] - 1, pl["tpi"], bt - 1, ntiles - 1, ntiles // 2} & set(range(ntiles)))
+    for q in tiles:
+        mt, rem = divmod(q, bt); b, t = divmod(rem, pl["tpi"])
+        pix0 = t * NPIX; py0 = pix0 // OW; iy_base = py0 * sh - ph; m0 = mt * pl["BM"]
+        for wm in range(WM):
+            for ch in (0, pl["nchunks"] - 1):
+                a = ((mt * WM + wm) * pl["nchunks"] + ch) * KK * 64 * 4 + (8 * 64 + 63) * 4
+                assert a + 4 <= wbuf2, ("A", a, wbuf2)
+        for ch in (0, pl["nchunks"] - 1):
+            for tid in range(NT):
+                pq, xc, rp = tid & 15, (tid >> 4) & 7, tid >> 7
+                lane_in = pq < ((W + 3) >> 2); xcol = min(4 * pq, W - 4)
+                for u in range(NXP_PERSIST):
+                    r = 2 * u + rp; iy = iy_base + r
+                    if r < pl["PR"] and 0 <= iy < H:
+                        a = ((b * C + ch * CC) * H + iy) * W + ((xc * H * W + xcol) if lane_in else 0)
+                        assert 0 <= a and a + 4 <= xsize, ("x", a, xsize)
+                    if r < pl["PR"] and lane_in:
+                        d = xc * PLANE + pw + xcol + r * PW
+                        assert 0 <= d and d + 4 <= CC * PLANE, ("park", d)
+        for pi in range(pix0, pix0 + NPIX):
+            if pi >= L: continue
+            py, px = divmod(pi, OW)
+            off = (py - py0) * sh * PW + px * sw + 7 * PLANE + 2 * PW + 2   # last channel pair, last tap
+            assert 0 <= (py - py0) * sh + 2 < pl["PR"] and px * sw + 2 < PW and off < CC * PLANE, ("B read", off)
+            assert (bufsz + 6 * PLANE + 2) * 4 < 65536   # buffer + channel pair + filter column ride in a read's 16-bit offset field
+            assert 2 * bufsz * 4 <= 72 * 1024            # two buffers
+            assert (b * M + min(M, m0 + pl["BM"]) - 1) * L + pi < ysize
+    return "persist %dx%d ok" % (WM, TN)
 
 
 # ---- conv_smallc.hpp: image layers (few input channels), forward and weight gradient ------------------------------------
