@@ -208,11 +208,11 @@ def fwd_shape_loads_in_bounds(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw):
     return "patch %dx%d ok" % (pl["WM"], pl["TN"])
 
 
-NXP_PERSIST = 6
+NXP_PERSIST = 5
 def persist_plans(B, C, H, W, M, OH, OW, sh, sw, ph, pw):
     """The tile shapes of conv_patch_persist_kernel that fit a layer (persist_plan)."""
     L, plans = OH * OW, []
-    for wm, tn in [(4, 10), (4, 7), (4, 5), (2, 8), (2, 5), (2, 3)]:
+    for wm, tn in [(4, 5), (4, 4), (2, 5), (2, 4), (2, 3)]:
         bm, np_ = 32 * wm, 32 * tn * (4 // wm)
         tiles, mtiles = _ceil_div(L, np_), _ceil_div(M, bm)
         rows = min(OH, np_ // OW if np_ % OW == 0 else (np_ - 1) // OW + 2); PR = (rows - 1) * sh + 3
@@ -232,7 +232,7 @@ def persist_walk(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw, num_cus=256):
     assert PLANE % 4 == 1 and PLANE >= pl["PR"] * PW and PW >= W + 2 * pw and pl["PR"] <= 2 * NXP_PERSIST
     L, WM, TN, NPIX = OH * OW, pl["WM"], pl["TN"], pl["NPIX"]
     bt = B * pl["tpi"]; ntiles = bt * pl["mtiles"]
-    nblk = min(ntiles, num_cus); chunk = 0          # one block per CU
+    nblk = min(ntiles, 2 * num_cus); chunk = 0      # two blocks per CU
     if ntiles % 8 == 0 and nblk >= 8:
         nblk -= nblk % 8; chunk = ntiles // 8
     seen = [0] * ntiles
