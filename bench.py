@@ -41,7 +41,7 @@ def time_stream(ctx, fn, iters, warmup):
     return ctx.timer_stop() / iters
 
 
-CONV_KERNELS = {"fwd": "cpk::conv_patch_kernel (conv fwd pass)", "dgrad": "cpk::conv_patch_kernel (conv dgrad pass)",
+CONV_KERNELS = {"fwd": "cpk::conv_patch_persist_kernel (conv fwd pass)", "dgrad": "cpk::conv_patch_persist_kernel (conv dgrad pass)",
                 "wgrad": "wgp::wgrad_patch_kernel + wgrad_patch_reduce_kernel (conv wgrad pass)"}
 
 

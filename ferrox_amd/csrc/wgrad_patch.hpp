@@ -54,7 +54,8 @@ struct Params {
 // NARROW (maps of at most 64 pixels with rows of at most 16 floats, XR unused): a stage is one whole image, and the patch is
 // staged by (channel, row) pairs, 4 lanes per row and 64 pairs per pass, instead of 16 lanes per row: with 8-float rows
 // the regular map would leave 14 of 16 lanes idle and could hold only 4 of the image's 10 patch rows.
-template <int XR, int WMO, int WC, int WK, bool NARROW = false>
+// PAIRS > 0 (unit column stride, a wave's row segment = 2 PAIRS pixels): the pixel loop of a row is unrolled, see compute.
+template <int XR, int WMO, int WC, int WK, bool NARROW = false, int PAIRS = 0>
 __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
     static_assert(WMO * WC * WK == 4, "four waves");
     static_assert(!NARROW || WC == 1, "narrow staging holds 32 channel planes");
@@ -65,7 +66,8 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
     extern __shared__ __align__(16) float smem[];
     float* Gs = smem;
     float* Xs = smem + BM * p.GP;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
+    const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register, with everything derived from it
     // Workgroup ids go to the 8 XCDs round-robin; remapped so that each XCD takes a contiguous range of
     // (split, oc tile, channel tile) triples: the channel tiles of one split read the same rows of g through one L2.
     int bxi = blockIdx.x, byi = blockIdx.y, bzi = blockIdx.z;
@@ -194,6 +196,43 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
     // the next pair are read from LDS into the other set.  The reads past the end of a row land in the pitch
     // padding or in the slack behind the planes and are never used.
     auto compute = [&]() {
+        if constexpr (PAIRS > 0) {
+            // Unit column stride and a row segment of 2 PAIRS pixels, unrolled: every LDS address is a row pointer plus an
+            // immediate, and of the three patch columns under a pixel pair the last one is the next pair's first, so a
+            // pair costs 7 LDS reads (1 of g, 3 middle, 3 new right columns) for its 9 MFMAs and no address arithmetic.
+            for (int r = 0; r < p.R; ++r) {
+                const float* gr = ga + r * p.ow;
+                const float* xk[KH];
+                xk[0] = xb + r * p.sh * p.PW;
+                xk[1] = xk[0] + p.PW;
+                xk[2] = xk[1] + p.PW;
+                float a[PAIRS], mid[PAIRS][KH], col[PAIRS + 1][KH];
+                auto rd = [&](int j) __attribute__((always_inline)) {
+                    a[j] = gr[2 * j];
+#pragma unroll
+                    for (int ky = 0; ky < KH; ++ky) {
+                        mid[j][ky] = xk[ky][2 * j + 1];
+                        col[j + 1][ky] = xk[ky][2 * j + 2];
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                };
+#pragma unroll
+                for (int ky = 0; ky < KH; ++ky) col[0][ky] = xk[ky][0];
+                rd(0);
+#pragma unroll
+                for (int j = 0; j < PAIRS; ++j) {
+                    if (j + 1 < PAIRS) rd(j + 1);
+#pragma unroll
+                    for (int ky = 0; ky < KH; ++ky) {
+                        acc[ky * KW + 0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], col[j][ky], acc[ky * KW + 0], 0, 0, 0);
+                        acc[ky * KW + 1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], mid[j][ky], acc[ky * KW + 1], 0, 0, 0);
+                        acc[ky * KW + 2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], col[j + 1][ky], acc[ky * KW + 2], 0, 0, 0);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            return;
+        }
         for (int r = 0; r < p.R; ++r) {
             const float* gr = ga + r * p.ow;
             const float* x0 = xb + r * p.sh * p.PW;
@@ -450,6 +489,15 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
         wgrad_patch_kernel<XRV, A, B_, C_><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                                \
     } while (0)
     const int layout = pl.WMO * 100 + pl.WC * 10 + pl.WK;
+    // pixel pairs of a wave's row segment when the unrolled pixel loop applies (unit column stride), else 0
+    const int pairs = sw == 1 && !pl.narrow && (ow / pl.WK) % 2 == 0 ? (int)(ow / pl.WK / 2) : 0;
+#define FX_WGP_LAUNCH_PAIRS(XRV, A, B_, C_, PV)                                                                       \
+    do {                                                                                                              \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_patch_kernel<XRV, A, B_, C_, false, PV>, \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
+        FX_HIP_CHECK(attr);                                                                                           \
+        wgrad_patch_kernel<XRV, A, B_, C_, false, PV><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                     \
+    } while (0)
 #define FX_WGP_LAUNCH_NARROW(A, C_)                                                                                   \
     do {                                                                                                              \
         static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_patch_kernel<0, A, 1, C_, true>,        \
@@ -461,6 +509,9 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
     else if (pl.narrow && layout == 212) FX_WGP_LAUNCH_NARROW(2, 2);
     else if (pl.narrow && layout == 114) FX_WGP_LAUNCH_NARROW(1, 4);
     else if (pl.narrow) FX_REQUIRE(false, "wgrad patch kernel: unexpected narrow layout %d", layout);
+    else if (layout == 411 && pl.PR == 3 && pairs == 28) FX_WGP_LAUNCH_PAIRS(3, 4, 1, 1, 28);
+    else if (layout == 411 && pl.PR == 4 && pairs == 14) FX_WGP_LAUNCH_PAIRS(4, 4, 1, 1, 14);
+    else if (layout == 221 && pl.PR == 3 && pairs == 28) FX_WGP_LAUNCH_PAIRS(3, 2, 2, 1, 28);
     else if (layout == 411 && pl.PR == 3) FX_WGP_LAUNCH(3, 4, 1, 1);
     else if (layout == 411) FX_WGP_LAUNCH(4, 4, 1, 1);
     else if (layout == 221 && pl.PR == 3) FX_WGP_LAUNCH(3, 2, 2, 1);
@@ -471,6 +522,7 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
     else if (layout == 114) FX_WGP_LAUNCH(4, 1, 1, 4);
     else FX_REQUIRE(false, "wgrad patch kernel: unexpected wave layout %d", layout);
 #undef FX_WGP_LAUNCH
+#undef FX_WGP_LAUNCH_PAIRS
 #undef FX_WGP_LAUNCH_NARROW
     FX_LAUNCH_CHECK();
     const int n = (int)p.part_stride;
