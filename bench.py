@@ -411,11 +411,14 @@ def bench_train_steps(steps=30, warmup=5, cpu=True, reference_pool=False, only=N
             out[key] = {"batch": int(x.shape[0])}
             # engine_literal: the reference's op sequence as is; engine_without_node_clones: the same minus the
             # engine's per-node deep clones; engine_fused: fused layers, loss and optimizer (extra entry points)
+            # engine_fused_graph: the fused step recorded once into a HIP graph and replayed (one submission per step)
             for label, literal, fused in (("engine_literal", True, False), ("engine_without_node_clones", False, False),
-                                          ("engine_fused", False, True)):
+                                          ("engine_fused", False, True), ("engine_fused_graph", False, True)):
                 if (fused and reference_pool) or (only and only[2] != label):
                     continue
                 m = host_api.Model(cfg["spec"], params, cfg["opt"], dtype, literal_engine=literal, fused=fused)
+                if label == "engine_fused_graph":
+                    m.enable_graph()
                 m.set_batch(x, y)
                 m.train_steps(warmup)
                 st0 = host_api.pool_stats(dtype)
@@ -427,6 +430,8 @@ def bench_train_steps(steps=30, warmup=5, cpu=True, reference_pool=False, only=N
                     "pool_requests_per_step": req / steps,
                     "pool_hit_rate": (st1["pool_hits"] - st0["pool_hits"]) / max(1, req),
                     "pool_underflow_misses": st1["underflow_misses"] - st0["underflow_misses"]}
+                if label == "engine_fused_graph":
+                    out[key][label]["graph"] = m.graph_info()  # kernel_nodes 0: the model has a Dropout layer and stayed eager
                 m.close()
             if cpu:
                 from oracle import train as otrain

@@ -149,6 +149,17 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_sgd_momentum_step_multi_{_s}", _vp, _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_i64),
          _ct, _ct, _ct, _int)
 
+    _sig(f"fx_adam_step_multi_bc_{_s}", _vp, _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
+         C.POINTER(_i64), *([_ct] * 5), _vp)
+
+_sig("fx_graph_begin", _vp)
+_sig("fx_graph_end", _vp, C.POINTER(_vp))
+_sig("fx_graph_launch", _vp, _vp)
+_sig("fx_graph_info", _vp, C.POINTER(_i64), C.POINTER(_i64), C.POINTER(_i64))
+_sig("fx_graph_destroy", _vp, _vp)
+_sig("fx_host_alloc", _vp, _i64, C.POINTER(_vp))
+_sig("fx_host_free", _vp, _vp)
+_sig("fx_h2d_async", _vp, _vp, _vp, _i64)
 _sig("fx_conv2d_tune_f32", _vp, _int, *([_i64] * 11), _int, _int)
 _sig("fx_reduce_max_noalloc_f32", _vp, _vp, _vp, _vp, _i64, _i64, _i64)
 NOALLOC_SCRATCH_BYTES = 4 << 20
@@ -243,6 +254,27 @@ class Context:
         self.close()
 
     # ---- runtime ----
+    def graph_begin(self):
+        """Starts recording the calls made on this context into a graph (see fx_graph_begin in the header for the rules)."""
+        check(lib.fx_graph_begin(self.h))
+
+    def graph_end(self):
+        """Ends the recording; returns the graph handle for graph_launch / graph_info / graph_destroy."""
+        g = _vp()
+        check(lib.fx_graph_end(self.h, C.byref(g)))
+        return g
+
+    def graph_launch(self, g):
+        check(lib.fx_graph_launch(self.h, g))
+
+    def graph_info(self, g):
+        n, k, h = _i64(0), _i64(0), _i64(0)
+        check(lib.fx_graph_info(g, C.byref(n), C.byref(k), C.byref(h)))
+        return {"nodes": n.value, "kernel_nodes": k.value, "held_blocks": h.value}
+
+    def graph_destroy(self, g):
+        check(lib.fx_graph_destroy(self.h, g))
+
     def sync(self):
         check(lib.fx_sync(self.h))
 

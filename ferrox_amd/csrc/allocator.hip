@@ -45,6 +45,7 @@ struct Pool {
     int literal_ids = 0;
     int best_fit = 0;
     hipStream_t stream = nullptr;  // work that may still touch a block is queued here
+    const bool* recording = nullptr;  // the owning context's flag: nothing is evicted (it would wait for the stream) while it is set
     std::vector<Bucket> buckets;
     std::unordered_map<uint64_t, int> active;         // allocation id -> bucket index
     struct Live { i64 elems; bool held; };            // held: handed to a caller (not sitting in a bucket)
@@ -75,7 +76,7 @@ static void device_free(Pool* p, const Block& b, bool& drained) {
 static void bucket_return(Pool* p, Bucket& b, Block blk) {
     const i64 cur = (i64)b.blocks.size();
     bool drained = false;
-    if (cur >= b.cfg.max_blocks) {
+    if (cur >= b.cfg.max_blocks && !(p->recording && *p->recording)) {
         if (b.cfg.eviction_threshold_ms >= 0) {  // evict_older_than, mod.rs:307-320
             const uint64_t now = now_ms();
             std::vector<Block> keep;
@@ -103,10 +104,11 @@ static void bucket_return(Pool* p, Bucket& b, Block blk) {
     b.blocks.push_back(blk);
 }
 
-Pool* pool_create(const fx_pool_config* cfg, int elem_size, hipStream_t stream) {
+Pool* pool_create(const fx_pool_config* cfg, int elem_size, hipStream_t stream, const bool* recording) {
     Pool* p = new Pool();
     p->elem_size = elem_size;
     p->stream = stream;
+    p->recording = recording;
     fx_pool_config def{};
     if (!cfg || cfg->n_buckets == 0) {
         // The four size classes of PoolConfig::default (mod.rs:50-82) with block counts sized for 288 GB of HBM:
@@ -204,7 +206,7 @@ int fx_alloc(fx_ctx* c, int dtype, int64_t n, void** ptr, int64_t* granted, uint
     }
     void* d = nullptr;
     hipError_t e = hipMalloc(&d, (size_t)n * (size_t)p->elem_size);
-    if (e != hipSuccess) {
+    if (e != hipSuccess && !c->capturing) {
         // one retry after releasing everything cached
         bool drained = false;
         for (auto& bk : p->buckets) { for (auto& x : bk.blocks) device_free(p, x, drained); bk.blocks.clear(); }
@@ -236,6 +238,13 @@ int fx_free(fx_ctx* c, int dtype, void* ptr, uint64_t id) {
     auto lv = p->live.find(ptr);
     FX_REQUIRE(lv != p->live.end(), "fx_free: pointer %p is not owned by this pool", ptr);
     FX_REQUIRE(lv->second.held, "fx_free: pointer %p was already released", ptr);
+    if (c->capturing) {
+        // the graph being recorded will use this address at every launch: the block goes back to the pool when the graph
+        // is destroyed (fx_graph_destroy), not now
+        for (const auto& h : c->capture_held) FX_REQUIRE(h.ptr != ptr, "fx_free: pointer %p was already released", ptr);
+        c->capture_held.push_back(fx_ctx::Held{dtype, ptr, id});
+        return FX_OK;
+    }
     lv->second.held = false;
     const i64 elems = lv->second.elems;
     p->st.bytes_in_use -= elems * p->elem_size;
@@ -259,6 +268,7 @@ int fx_free(fx_ctx* c, int dtype, void* ptr, uint64_t id) {
 
 int fx_pool_cleanup(fx_ctx* c, int dtype) {  // cuda.rs:113-119
     FX_CHECK_CTX(c);
+    FX_NOT_RECORDING(c, "fx_pool_cleanup");
     Pool* p = get_pool(c, dtype);
     FX_REQUIRE(p != nullptr, "fx_pool_cleanup: unknown dtype %d", dtype);
     FX_HIP_CHECK(hipStreamSynchronize(c->stream));
@@ -270,6 +280,7 @@ int fx_pool_cleanup(fx_ctx* c, int dtype) {  // cuda.rs:113-119
 
 int fx_pool_reset(fx_ctx* c, int dtype) {  // cuda.rs:125-133
     FX_CHECK_CTX(c);
+    FX_NOT_RECORDING(c, "fx_pool_reset");
     Pool* p = get_pool(c, dtype);
     FX_REQUIRE(p != nullptr, "fx_pool_reset: unknown dtype %d", dtype);
     FX_HIP_CHECK(hipStreamSynchronize(c->stream));

@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include "../../include/ferrox_hip.h"
 
@@ -45,6 +46,11 @@ int bind_device(int device);  // runtime.hip
     } while (0)
 
 // Checks the launch itself (bad configuration shows up here, not at the next sync).
+// Calls that wait for the stream refuse to run while it records a graph (the wait would invalidate the recording).
+#define FX_NOT_RECORDING(c, what)                                                                           \
+    FX_REQUIRE(!(c)->capturing, "%s waits for the stream, which is recording a graph (fx_graph_begin): call it before "  \
+               "fx_graph_begin or after fx_graph_end", what)
+
 #define FX_LAUNCH_CHECK()                                                                                   \
     do {                                                                                                    \
         hipError_t _e = hipGetLastError();                                                                  \
@@ -73,6 +79,11 @@ struct fx_ctx {
     // tile shape that measured fastest per convolution layer shape (conv_patch.hpp); used under launch_mutex
     std::map<std::array<i64, 14>, int> conv_tile_cache;
     bool conv_retune = false;  // set by fx_conv2d_tune around its call: time the shapes again even when the cache has an entry
+    // Between fx_graph_begin and fx_graph_end the stream records instead of running: blocks released meanwhile stay out of
+    // the pool (the graph keeps using their addresses at every launch) and nothing may wait for the stream.
+    bool capturing = false;
+    struct Held { int dtype; void* ptr; uint64_t id; };
+    std::vector<Held> capture_held;
     hipEvent_t ev_tune[2] = {nullptr, nullptr};
     // returns a scratch region of at least `bytes` (256-byte aligned); nullptr + error on failure
     void* get_scratch(i64 bytes);

@@ -416,6 +416,7 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
         T* col = (T*)ws;
         bool own = false;
         if (!col) {
+            FX_NOT_RECORDING(c, "a convolution call without a caller-supplied workspace");
             FX_HIP_CHECK(hipMalloc((void**)&col, (size_t)need));
             own = true;
         }
@@ -527,6 +528,7 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
         // the slices' results is allocated and released here)
         const i64 nchunks = fx::ceil_div(B, d.bc), nw = Cout * Cin * kh * kw;
         T* tmp = nullptr;
+        FX_NOT_RECORDING(c, "a convolution call without a caller-supplied workspace");
         FX_HIP_CHECK(hipMalloc((void**)&tmp, (size_t)(nchunks * nw) * sizeof(T)));
         int rc = FX_OK;
         for (i64 i = 0; i < nchunks && !rc; ++i) {

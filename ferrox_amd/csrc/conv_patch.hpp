@@ -810,6 +810,9 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
     static const bool tune = [] { const char* v = getenv("FX_CONV_TUNE"); return !(v && atoi(v) == 0); }();
     if (!tune || pl.nimg) return launch_plan(c, pl, x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu);
     const std::array<i64, 14> key = {flip, batch_class(B), C, H, W, M, OH, OW, sh, sw, ph, pw, bias ? 1 : 0, relu};
+    // a stream that is recording a graph cannot be timed: a layer shape first met there runs with the modelled tile
+    if (c->capturing && c->conv_tile_cache.find(key) == c->conv_tile_cache.end())
+        return launch_plan(c, pl, x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu);
     Plan cand[MAX_CAND];
     const int n = candidates(cand, c->num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw);
     auto it = c->conv_tile_cache.find(key);

@@ -313,6 +313,7 @@ int softmax_ce_bwd(fx_ctx* c, const T* probs, const T* targets, const T* gup, T*
 template <typename T> struct OptHyper {
     T lr, beta1, beta2, eps, wd, bc1, bc2;  // SGD: beta1 = momentum
     int flag;                               // Adam: amsgrad; SGD: nesterov
+    const T* bc_dev = nullptr;              // Adam: when set, {bc1, bc2} are read from device memory instead
 };
 
 template <typename T>
@@ -368,8 +369,14 @@ __global__ __launch_bounds__(256) void multi_step_kernel(const MultiTensors<T> t
     while (t + 1 < tt.count && blockIdx.x >= tt.first[t + 1]) ++t;  // wave-uniform
     const i64 i = (i64)(blockIdx.x - tt.first[t]) * 256 + threadIdx.x;
     if (i >= tt.n[t]) return;
-    if (ADAM) adam_element<T>(tt.p[t], tt.g[t], tt.m[t], tt.v[t], tt.x[t], i, h);
-    else sgd_element<T>(tt.p[t], tt.g[t], tt.m[t], i, h);
+    if (ADAM) {
+        if (h.bc_dev) {  // the step-dependent scalars of a recorded step: a graph repeats the kernel with the arguments of the recording
+            OptHyper<T> hs = h;
+            hs.bc1 = h.bc_dev[0];
+            hs.bc2 = h.bc_dev[1];
+            adam_element<T>(tt.p[t], tt.g[t], tt.m[t], tt.v[t], tt.x[t], i, hs);
+        } else adam_element<T>(tt.p[t], tt.g[t], tt.m[t], tt.v[t], tt.x[t], i, h);
+    } else sgd_element<T>(tt.p[t], tt.g[t], tt.m[t], i, h);
 }
 
 // m / v / x: tables that may be null as a whole (SGD without momentum; Adam without AMSGrad)
@@ -476,6 +483,15 @@ int sgd_step(fx_ctx* c, T* p, const T* g, T* buf, i64 n, T lr, T momentum, T wd,
         OptHyper<T> h;                                                                                                 \
         adam_hyper(h, lr, beta1, beta2, eps, wd, bc1, bc2, 0);                                                         \
         return multi_step<T, true>(c, count, p, g, m, v, nullptr, n, h, "fx_adam_step_multi");                         \
+    }                                                                                                                  \
+    extern "C" int fx_adam_step_multi_bc_##S(fx_ctx* c, int count, T* const* p, const T* const* g, T* const* m,        \
+                                              T* const* v, T* const* vmax, const int64_t* n, T lr, T beta1, T beta2,    \
+                                              T eps, T wd, const T* bc) {                                              \
+        FX_REQUIRE(bc != nullptr, "fx_adam_step_multi_bc: null bias-correction pointer");                             \
+        OptHyper<T> h;                                                                                                 \
+        adam_hyper(h, lr, beta1, beta2, eps, wd, T(1), T(1), vmax != nullptr);                                         \
+        h.bc_dev = bc;                                                                                                 \
+        return multi_step<T, true>(c, count, p, g, m, v, vmax, n, h, "fx_adam_step_multi_bc");                         \
     }                                                                                                                  \
     extern "C" int fx_adam_amsgrad_step_multi_##S(fx_ctx* c, int count, T* const* p, const T* const* g, T* const* m,   \
                                                   T* const* v, T* const* vmax, const int64_t* n, T lr, T beta1,        \

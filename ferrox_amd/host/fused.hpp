@@ -32,6 +32,10 @@ template <typename T> struct FusedApi;
                               T eps, T wd, T bc1, T bc2) {                                                             \
             return fx_adam_step_multi_##S(c, k, p, g, m, v, n, lr, b1, b2, eps, wd, bc1, bc2);                         \
         }                                                                                                              \
+        static int adam_multi_bc(fx_ctx* c, int k, T* const* p, const T* const* g, T* const* m, T* const* v, T* const* x, const int64_t* n, T lr, \
+                                 T b1, T b2, T eps, T wd, const T* bc) {                                                \
+            return fx_adam_step_multi_bc_##S(c, k, p, g, m, v, x, n, lr, b1, b2, eps, wd, bc);                         \
+        }                                                                                                              \
         static int sgd_multi(fx_ctx* c, int k, T* const* p, const T* const* g, const int64_t* n, T lr) { return fx_sgd_step_multi_##S(c, k, p, g, n, lr); } \
         static int sgd_momentum_multi(fx_ctx* c, int k, T* const* p, const T* const* g, T* const* b, const int64_t* n, T lr, T mom, T wd, int nes) { \
             return fx_sgd_momentum_step_multi_##S(c, k, p, g, b, n, lr, mom, wd, nes);                                 \
@@ -390,10 +394,38 @@ template <typename T> struct SGDFused : SGD<T> {
 // Adam with every parameter of a group updated in one launch (fx_adam_step_multi / fx_adam_amsgrad_step_multi)
 template <typename T> struct AdamFused : Adam<T> {
     AdamFused(T lr_, T b1, T b2, T eps_, T wd, bool amsgrad_ = false) : Adam<T>(lr_, b1, b2, eps_, wd, amsgrad_) {}
+    ~AdamFused() override {
+        if (bc_host) (void)fx_host_free(fused_ctx(), bc_host);
+    }
+    // Steps that are recorded once and replayed (Model::enable_graph): the bias corrections are the only scalars of the
+    // step that change, so they travel through device memory.  The host keeps them in page-locked memory, every step
+    // queues a copy from there to bc_dev (a recorded copy reads the same host address at every replay) and the kernel
+    // reads bc_dev.
+    bool device_bc = false;
+    T* bc_host = nullptr;
+    Tensor<T> bc_dev;
+    void use_device_bias_corrections() {
+        if (device_bc) return;
+        void* h = nullptr;
+        fx_ok(fx_host_alloc(fused_ctx(), (int64_t)(2 * sizeof(T)), &h));
+        bc_host = static_cast<T*>(h);
+        bc_dev = HipStorage<T>::zeros({2});
+        device_bc = true;
+    }
+    // the host half of a step whose device half is a graph launch: the caller launches the graph afterwards
+    void advance_for_replay() {
+        this->step_count += 1;
+        adam_bias_corrections(this->beta1, this->beta2, this->step_count, bc_host[0], bc_host[1]);
+    }
     void step(AutoFerroxEngine<T>& g) override {
         this->step_count += 1;
         T bc1, bc2;
         adam_bias_corrections(this->beta1, this->beta2, this->step_count, bc1, bc2);
+        if (device_bc) {
+            bc_host[0] = bc1;
+            bc_host[1] = bc2;
+            fx_ok(fx_h2d_async(fused_ctx(), bc_dev->data(), bc_host, (int64_t)(2 * sizeof(T))));
+        }
         for (const auto& group : this->param_groups) {
             const T glr = group.lr.value_or(this->lr), gwd = group.weight_decay.value_or(this->weight_decay);
             std::vector<T*> ps, ms, vs, xs;
@@ -418,7 +450,10 @@ template <typename T> struct AdamFused : Adam<T> {
                 ns.push_back((int64_t)w->size());
             }
             if (ps.empty()) continue;
-            if (this->amsgrad)
+            if (device_bc)
+                fx_ok(FusedApi<T>::adam_multi_bc(fused_ctx(), (int)ps.size(), ps.data(), gs.data(), ms.data(), vs.data(), this->amsgrad ? xs.data() : nullptr,
+                                                 ns.data(), glr, this->beta1, this->beta2, this->eps, gwd, bc_dev->data()));
+            else if (this->amsgrad)
                 fx_ok(FusedApi<T>::adam_amsgrad_multi(fused_ctx(), (int)ps.size(), ps.data(), gs.data(), ms.data(), vs.data(), xs.data(), ns.data(), glr,
                                                       this->beta1, this->beta2, this->eps, gwd, bc1, bc2));
             else

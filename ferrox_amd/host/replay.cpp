@@ -35,6 +35,8 @@ struct ModelBase {
     virtual void get_state(int i, void* host) const = 0;
     virtual std::vector<uint8_t> optimizer_state() const = 0;
     virtual void load_optimizer_state(const uint8_t* data, size_t n) = 0;
+    virtual void enable_graph(bool on) = 0;
+    virtual void graph_info(int64_t* nodes, int64_t* kernels, int64_t* held) const = 0;
 };
 
 std::vector<std::string> split(const std::string& s, char sep) {
@@ -63,6 +65,40 @@ template <typename T> struct Model : ModelBase {
     bool input_requires_grad = false;
     bool have_input_node = false;
     NodeId input_node = 0;
+
+    // Recorded steps (enable_graph): after two eager steps on the same batch shape -- the pool then serves every request of
+    // a step from its buckets, the scratch region has its size, the conv tiles are timed -- the next step is recorded into a
+    // graph once and every later one is a single launch of it.  The recorded step is the eager one call for call, so the
+    // results have the same bits.  Only the fused engine is recorded: its optimizers update the parameters in place and
+    // its loss is read after the step, whereas the op-by-op engines put every updated parameter into a NEW tensor (a replay
+    // would keep reading the old one), read the loss in the middle of a step (training.rs:60-64) and pass Adam's bias
+    // corrections as scalar arguments of a dozen elementwise kernels.  Also left eager: models with a Dropout layer (a new
+    // mask per step, seeded on the host) and a batch that enters as a leaf with a gradient.
+    bool graph_on = false, has_dropout = false;
+    fx_graph* step_graph = nullptr;
+    bool graph_with_update = true;  // the recorded step includes the optimizer step
+    Tensor<T> graph_loss;           // where the recorded step leaves its loss
+    int warm_steps = 0;
+    ~Model() override { drop_graph(); }
+    void drop_graph() {
+        if (step_graph) (void)fx_graph_destroy(BackendManager::get().ctx(), step_graph);
+        step_graph = nullptr;
+        graph_loss.reset();
+        warm_steps = 0;
+    }
+    bool graph_supported() const {
+        return fused && !has_dropout && !input_requires_grad;
+    }
+    void enable_graph(bool on) override {
+        if (on && !graph_on)
+            if (auto* a = dynamic_cast<AdamFused<T>*>(opt.get())) a->use_device_bias_corrections();
+        if (!on) drop_graph();
+        graph_on = on;
+    }
+    void graph_info(int64_t* nodes, int64_t* kernels, int64_t* held) const override {
+        *nodes = *kernels = *held = 0;
+        if (step_graph) fx_ok(fx_graph_info(step_graph, nodes, kernels, held));
+    }
 
     // engine: 0 = reference op sequence without the per-node deep clones, 1 = reference op sequence as is,
     //         2 = fused layers / loss / optimizers
@@ -122,6 +158,7 @@ template <typename T> struct Model : ModelBase {
                 double p = 0.5;
                 uint64_t seed = 0;
                 ss >> p >> seed;
+                has_dropout = true;
                 if (engine == 1) layers.push_back(std::make_unique<Dropout<T>>(p, seed));
                 else layers.push_back(std::make_unique<DropoutFused<T>>(p, seed));
             } else if (kind == "relu") layers.push_back(std::make_unique<ReLU<T>>());
@@ -183,6 +220,13 @@ template <typename T> struct Model : ModelBase {
     int num_params() const override { return (int)params.size(); }
     int64_t param_numel(int i) const override { return (int64_t)graph.get_tensor(params.at(i))->size(); }
     void set_batch(const void* xv, const Shape& xs, const void* yv, const Shape& ys) override {
+        if (graph_on && x && y && x->shape() == xs && y->shape() == ys) {
+            // a recorded step reads the batch at the addresses it was recorded with: new data goes there
+            fx_ok(fx_h2d(BackendManager::get().ctx(), x->data(), xv, (int64_t)(x->size() * sizeof(T))));
+            fx_ok(fx_h2d(BackendManager::get().ctx(), y->data(), yv, (int64_t)(y->size() * sizeof(T))));
+            return;
+        }
+        drop_graph();
         x = HipStorage<T>::from_vec(static_cast<const T*>(xv), xs);
         y = HipStorage<T>::from_vec(static_cast<const T*>(yv), ys);
         if (have_input_node) graph.update_parameter(input_node, x->clone_storage());
@@ -203,8 +247,53 @@ template <typename T> struct Model : ModelBase {
         for (auto& l : layers) in = l->forward(graph, in);
         return in;
     }
+    // zero_gradients -> forward -> loss -> copy of the loss -> backward -> update, nothing read back: the form a step is
+    // recorded in
+    Tensor<T> step_body(bool optimizer_step) {
+        graph.zero_gradients();
+        const NodeId xin = graph.create_variable(fused ? HipStorage<T>::borrow(*x) : x->clone_storage(), false);
+        const NodeId pred = forward(xin);
+        NodeId loss;
+        if (loss_kind == 1) loss = graph.apply_operation(std::make_unique<Sum<T>>(false), {pred});
+        else {
+            const NodeId yin = graph.create_variable(fused ? HipStorage<T>::borrow(*y) : y->clone_storage(), false);
+            loss = fused ? cce_loss_fused<T>(graph, pred, yin) : cce_loss<T>(graph, pred, yin);
+        }
+        Tensor<T> lcopy = graph.get_tensor(loss)->clone_storage();
+        graph.backward(loss);
+        if (optimizer_step) opt->step(graph);
+        return lcopy;
+    }
     double train_step(bool optimizer_step) override {
         if (!x || !y) throw Error("set_batch was not called");
+        if (graph_on && graph_supported()) {
+            fx_ctx* c = BackendManager::get().ctx();
+            if (step_graph && graph_with_update != optimizer_step) drop_graph();
+            if (step_graph) {
+                if (optimizer_step)
+                    if (auto* a = dynamic_cast<AdamFused<T>*>(opt.get())) a->advance_for_replay();
+                fx_ok(fx_graph_launch(c, step_graph));
+                return (double)graph_loss->first();
+            }
+            if (warm_steps >= 2) {
+                fx_ok(fx_graph_begin(c));
+                Tensor<T> l;
+                try {
+                    l = step_body(optimizer_step);
+                } catch (...) {
+                    fx_graph* g = nullptr;
+                    if (fx_graph_end(c, &g) == FX_OK && g) (void)fx_graph_destroy(c, g);
+                    graph_on = false;  // the step was neither run nor recorded: the caller sees the error, later steps run eagerly
+                    throw;
+                }
+                fx_ok(fx_graph_end(c, &step_graph));
+                graph_loss = std::move(l);
+                graph_with_update = optimizer_step;
+                fx_ok(fx_graph_launch(c, step_graph));
+                return (double)graph_loss->first();
+            }
+            ++warm_steps;
+        }
         graph.zero_gradients();
         NodeId xin;
         if (input_requires_grad) {
@@ -332,6 +421,14 @@ int fxh_model_get_input_grad(void* m, void* host) {
     return guarded([&] { static_cast<ModelBase*>(m)->get_input_grad(host); });
 }
 // n steps back to back; wall time covers forward + backward + optimizer step of every step and one final sync
+// Later steps are recorded once and replayed as one graph launch where the model allows it (see Model::graph_on).
+int fxh_model_enable_graph(void* m, int on) {
+    return guarded([&] { static_cast<ModelBase*>(m)->enable_graph(on != 0); });
+}
+// nodes / kernel nodes / pool blocks of the recorded step (zeros while there is none)
+int fxh_model_graph_info(void* m, int64_t* nodes, int64_t* kernels, int64_t* held) {
+    return guarded([&] { static_cast<ModelBase*>(m)->graph_info(nodes, kernels, held); });
+}
 int fxh_model_train_steps(void* m, int n, double* last_loss, double* total_ms) {
     return guarded([&] {
         fx_ok(fx_sync(BackendManager::get().ctx()));

@@ -46,6 +46,8 @@ lib.fxh_free.restype = None
 lib.fxh_model_load_optimizer_state.argtypes = [C.c_void_p, C.c_char_p, C.c_int64]
 lib.fxh_set_conv_grad_mode.argtypes = [C.c_int]
 lib.fxh_model_configure.argtypes = [C.c_void_p, C.c_int, C.c_int]
+lib.fxh_model_enable_graph.argtypes = [C.c_void_p, C.c_int]
+lib.fxh_model_graph_info.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
 lib.fxh_model_backward.argtypes = [C.c_void_p, C.POINTER(C.c_double)]
 lib.fxh_model_add_param_group.argtypes = [C.c_void_p, C.POINTER(C.c_int), C.c_int, C.c_double, C.c_double, C.c_double]
 lib.fxh_model_input_numel.argtypes = [C.c_void_p]
@@ -137,6 +139,16 @@ class Model:
         assert out.size == lib.fxh_model_input_numel(self.h)
         _check(lib.fxh_model_get_input_grad(self.h, out.ctypes.data))
         return out
+
+    def enable_graph(self, on=True):
+        """Later train steps are recorded once (after two eager ones) and replayed as one graph launch where the model
+        allows it: fused engine, no Dropout layer, no gradient for the batch.  Same results, bit for bit."""
+        _check(lib.fxh_model_enable_graph(self.h, int(on)))
+
+    def graph_info(self):
+        n, k, h = C.c_int64(0), C.c_int64(0), C.c_int64(0)
+        _check(lib.fxh_model_graph_info(self.h, C.byref(n), C.byref(k), C.byref(h)))
+        return {"nodes": n.value, "kernel_nodes": k.value, "held_blocks": h.value}
 
     def train_steps(self, n):
         loss, ms = C.c_double(0), C.c_double(0)

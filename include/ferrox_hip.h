@@ -341,12 +341,48 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
     int fx_adam_amsgrad_step_multi_##S(fx_ctx* ctx, int count, T* const* p, const T* const* g, T* const* m,            \
                                        T* const* v, T* const* vmax, const int64_t* n, T lr, T beta1, T beta2, T eps,   \
                                        T weight_decay, T bc1, T bc2);                                                  \
+    /* The multi-tensor Adam step for recorded steps (fx_graph_*): the bias corrections, the only scalars of a step    \
+       that change from one step to the next, are read from DEVICE memory, bc = {bc1, bc2}; vmax may be NULL (no       \
+       AMSGrad).  Same arithmetic and bits as the calls above. */                                                      \
+    int fx_adam_step_multi_bc_##S(fx_ctx* ctx, int count, T* const* p, const T* const* g, T* const* m, T* const* v,    \
+                                  T* const* vmax, const int64_t* n, T lr, T beta1, T beta2, T eps, T weight_decay,     \
+                                  const T* bc);                                                                        \
     int fx_sgd_step_multi_##S(fx_ctx* ctx, int count, T* const* p, const T* const* g, const int64_t* n, T lr);         \
     int fx_sgd_momentum_step_multi_##S(fx_ctx* ctx, int count, T* const* p, const T* const* g, T* const* buf,          \
                                        const int64_t* n, T lr, T momentum, T weight_decay, int nesterov);
 
 FX_DECLARE_KERNELS(float, f32)
 FX_DECLARE_KERNELS(double, f64)
+
+/* ---- recorded steps (HIP graphs) -------------------------------------------------------------------------------
+ * No counterpart in the reference, which launches every kernel of a training step from the host
+ * (examples/common/training.rs:105-160; about 230 launches in the CNN configuration, 3.4 us each, more than the kernels
+ * themselves take).  Between fx_graph_begin and fx_graph_end the context's stream RECORDS the calls made on this
+ * context instead of running them; fx_graph_launch then replays the recording as one submission, with the pointer and
+ * scalar arguments of the recording.  Rules for the recorded region:
+ *   - run the same calls once eagerly first: the pool then serves every request from its buckets, the library's
+ *     scratch region has its final size and the convolution tile shapes are timed (none of this can happen while
+ *     recording: fx_alloc may still fall through to hipMalloc, but a call that waits for the stream -- fx_sync,
+ *     fx_h2d, fx_d2h, fx_timer_stop, fx_pool_cleanup, the tile timing -- makes fx_graph_end fail);
+ *   - blocks released with fx_free while recording stay out of the pool: they are the graph's temporaries, used at the
+ *     same addresses by every launch, and go back to the pool in fx_graph_destroy;
+ *   - what a launch reads from outside (the batch) must sit at the recorded addresses: copy new data there;
+ *   - scalars that change per step must come from device memory: fx_adam_step_multi_bc reads its bias corrections
+ *     there, and fx_h2d_async from fx_host_alloc'ed memory is recorded as "copy from this host address", so the
+ *     host rewrites the values between launches.
+ * A launch is stream-ordered like any other call; results are bit-identical to the eager calls (same kernels, same
+ * arguments). */
+typedef struct fx_graph fx_graph;
+int fx_graph_begin(fx_ctx* ctx);
+int fx_graph_end(fx_ctx* ctx, fx_graph** out);
+int fx_graph_launch(fx_ctx* ctx, fx_graph* graph);
+/* number of nodes, of kernel nodes, and of pool blocks the graph keeps (any pointer may be NULL) */
+int fx_graph_info(fx_graph* graph, int64_t* nodes, int64_t* kernel_nodes, int64_t* held_blocks);
+int fx_graph_destroy(fx_ctx* ctx, fx_graph* graph);
+/* Page-locked host memory and an upload from it that does not wait (fx_h2d waits for the copy). */
+int fx_host_alloc(fx_ctx* ctx, int64_t bytes, void** out);
+int fx_host_free(fx_ctx* ctx, void* ptr);
+int fx_h2d_async(fx_ctx* ctx, void* dst, const void* src_pinned, int64_t bytes);
 
 /* ---- an entry point that allocates nothing ---------------------------------------------------------------
  * No counterpart in the reference.  It is for callers that cannot allocate device memory at the time of the call:
