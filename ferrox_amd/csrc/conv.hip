@@ -16,6 +16,7 @@
 #include "wgrad_patch.hpp"
 #include "conv_smallc.hpp"
 #include "conv_patch.hpp"
+#include "conv_patch_f64.hpp"
 
 namespace fx {
 int col2im_f32(fx_ctx*, const float*, float*, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, int);
@@ -149,11 +150,30 @@ cpk::Plan dgrad_patch_plan(fx_ctx* c, const Dims& d, int mode) {
     return cpk::Plan();
 }
 
+// f64: the same structure on the 16x16x4 MFMA (conv_patch_f64.hpp)
+template <typename T>
+cpd::Plan fwd_patch64_plan(fx_ctx* c, const Dims& d) {
+    if constexpr (sizeof(T) == 8) {
+        if (!generic_only()) return cpd::make_plan(c ? c->num_cus : 256, d.B, d.Cin, d.H, d.W, d.Cout, d.oh, d.ow, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
+    }
+    return cpd::Plan();
+}
+template <typename T>
+cpd::Plan dgrad_patch64_plan(fx_ctx* c, const Dims& d, int mode) {
+    if constexpr (sizeof(T) == 8) {
+        if (mode == 0 && !generic_only() && d.sh == 1 && d.sw == 1 && d.ph <= 2 && d.pw <= 2)
+            return cpd::make_plan(c ? c->num_cus : 256, d.B, d.Cout, d.oh, d.ow, d.Cin, d.H, d.W, d.kh, d.kw, 1, 1, 2 - d.ph, 2 - d.pw);
+    }
+    return cpd::Plan();
+}
+
 template <typename T>
 i64 fwd_ws_bytes(fx_ctx* c, const Dims& d) {
     // enough for either kernel: a misaligned tensor sends a patch-kernel shape to the implicit GEMM
     const cpk::Plan pl = fwd_patch_plan<T>(c, d);
     const i64 generic = d.Cin % CONV_BK == 0 ? d.Cin * d.Cout * d.kh * d.kw * (i64)sizeof(T) : 0;
+    const cpd::Plan pd = fwd_patch64_plan<T>(c, d);
+    if (pd.ok) return std::max(generic, cpd::workspace_bytes(pd));
     return pl.ok ? std::max(generic, cpk::workspace_bytes(pl, d.Cout)) : generic;
 }
 
@@ -185,6 +205,14 @@ int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64
             float* wimg = (float*)(ws ? ws : c->get_scratch(need));
             if (!wimg) return FX_ERR_OOM;
             return cpk::run(c, pl, x, w, y, wimg, 0, Cout, Cin, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw, bias, relu);
+        }
+    }
+    if constexpr (sizeof(T) == 8) {
+        const cpd::Plan pd = fwd_patch64_plan<T>(c, d);
+        if (pd.ok && aligned16(x, ws) && aligned16(y, y)) {
+            double* wimg = (double*)(ws ? ws : c->get_scratch(need));
+            if (!wimg) return FX_ERR_OOM;
+            return cpd::run(c, pd, x, w, y, wimg, 0, Cout, Cin, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw, bias, relu);
         }
     }
     if (d.Cin % CONV_BK == 0) {
@@ -383,6 +411,8 @@ i64 dgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     if (mode == 1) return d.Cin * d.kh * d.kw * d.B * d.oh * d.ow * (i64)sizeof(T);
     const cpk::Plan pl = dgrad_patch_plan<T>(c, d, mode);
     const i64 generic = d.Cin * d.Cout * d.kh * d.kw * (i64)sizeof(T);
+    const cpd::Plan pd = dgrad_patch64_plan<T>(c, d, mode);
+    if (pd.ok) return std::max(generic, cpd::workspace_bytes(pd));
     return pl.ok ? std::max(generic, cpk::workspace_bytes(pl, d.Cin)) : generic;
 }
 
@@ -435,6 +465,10 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
     if constexpr (sizeof(T) == 4) {
         const cpk::Plan pl = dgrad_patch_plan<T>(c, d, mode);
         if (pl.ok && aligned16(g, wt)) return cpk::run(c, pl, g, w, dx, wt, 1, Cout, Cin, B, Cout, d.oh, d.ow, Cin, H, W, 1, 1, 2 - ph, 2 - pw);
+    }
+    if constexpr (sizeof(T) == 8) {
+        const cpd::Plan pd = dgrad_patch64_plan<T>(c, d, mode);
+        if (pd.ok && aligned16(g, wt) && aligned16(dx, dx)) return cpd::run(c, pd, g, w, dx, wt, 1, Cout, Cin, B, Cout, d.oh, d.ow, Cin, H, W, 1, 1, 2 - ph, 2 - pw);
     }
     if (dgrad_classes_ok<T>(d)) return dgrad_classes<T>(c, g, w, dx, wt, d);
     if (Cout % CONV_BK == 0) {

@@ -554,6 +554,61 @@ def test_conv2d_patch_kernel_shapes(ctx, orc):
             assert np.array_equal(out.numpy(), ref), (kind, case)
 
 
+# f64 on the 16x16x4 MFMA patch kernel (conv_patch_f64.hpp: 3x3, channels % 8 == 0, even rows of up to 64 doubles, at most 8 patch
+# rows under a tile, at least 32 output channels and 64 pixels): every tile width, two channel tiles, ragged channel counts,
+# tiles that end inside a row, paddings 0 / 1 / 2, a strided forward pass, bias + ReLU in the store.
+CONV_F64_PATCH_CASES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw)
+    (2, 64, 56, 56, 128, (1, 1), (1, 1)), (3, 8, 6, 12, 60, (1, 1), (1, 1)), (3, 16, 8, 36, 120, (1, 1), (0, 0)), (2, 24, 10, 16, 104, (1, 1), (2, 2)),
+    (1, 8, 64, 64, 52, (1, 1), (1, 1)), (2, 16, 9, 62, 64, (2, 1), (1, 1)), (5, 32, 32, 32, 64, (1, 1), (1, 1)), (3, 8, 14, 28, 72, (1, 1), (1, 1)),
+    (2, 8, 9, 30, 128, (1, 1), (0, 0)), (2, 32, 28, 28, 33, (1, 1), (1, 1)),
+]
+
+
+def test_conv2d_f64_patch_kernel_shapes(ctx, orc):
+    import torch
+    import torch.nn.functional as F
+    from ferrox_amd import capi
+    rng = np.random.default_rng(61)
+    tol = TOL[np.dtype(np.float64)]
+    for (B, Cin, H, W, Cout, st, pd) in CONV_F64_PATCH_CASES:
+        case = (B, Cin, H, W, Cout, st, pd)
+        x = rng.uniform(-1, 1, (B, Cin, H, W))
+        w = rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9))
+        bias = rng.standard_normal(Cout)
+        oh, ow = orc.out_hw(H, W, 3, 3, st[0], st[1], pd[0], pd[1])
+        g = rng.standard_normal((B, Cout, oh, ow))
+        dx_, dw_, dg_, db_ = ctx.upload(x), ctx.upload(w), ctx.upload(g), ctx.upload(bias)
+        y = ctx.conv2d_fwd(dx_, dw_, st, pd).numpy()
+        dxg = ctx.conv2d_dgrad(dg_, dw_, x.shape, st, pd, 0).numpy()
+        tx = torch.from_numpy(x).to(torch.float64).requires_grad_(True)
+        tw = torch.from_numpy(w).to(torch.float64)
+        ty = F.conv2d(tx, tw, stride=st, padding=pd)
+        ty.backward(torch.from_numpy(g))
+        ay = F.conv2d(tx.detach().abs(), tw.abs(), stride=st, padding=pd).max().item()
+        assert np.abs(y - ty.detach().numpy()).max() <= tol * ay, ("fwd", case)
+        assert rel_err(dxg, tx.grad.numpy()) <= tol * 8, ("dgrad", case)
+        assert rel_err(y, orc.conv2d_fwd(x, w, st, pd)) <= tol * 8, ("fwd vs oracle", case)
+        assert rel_err(dxg, orc.conv2d_dgrad(g, w, x.shape, st, pd, 0)) <= tol * 8, ("dgrad vs oracle", case)
+        # bias + ReLU in the store of the kernel = the forward pass followed by fx_bias_act, bit for bit
+        dims = (B, Cin, H, W, Cout, 3, 3, st[0], st[1], pd[0], pd[1])
+        fused = ctx.empty(y.shape, np.float64)
+        capi.check(capi.lib.fx_conv2d_fwd_bias_act_f64(ctx.h, dx_.ptr, dw_.ptr, db_.ptr, fused.ptr, *dims, 1, None, 0))
+        two = ctx.conv2d_fwd(dx_, dw_, st, pd)
+        capi.check(capi.lib.fx_bias_act_f64(ctx.h, two.ptr, db_.ptr, B, Cout, oh * ow, 1))
+        assert np.array_equal(fused.numpy(), two.numpy()), ("bias + relu", case)
+        # caller-provided workspaces of exactly the advertised size give the same bits
+        for kind, fn, a, b_, ref, shape in (
+                (capi.CONV_FWD, capi.lib.fx_conv2d_fwd_f64, dx_, dw_, y, y.shape),
+                (capi.CONV_DGRAD, capi.lib.fx_conv2d_dgrad_f64, dg_, dw_, dxg, x.shape)):
+            need = capi.lib.fx_conv2d_workspace_bytes(kind, capi.FX_F64, 0, *dims)
+            assert need >= 0, case
+            ws = ctx.empty((max(need, 8) // 8,), np.float64)
+            out = ctx.empty(shape, np.float64)
+            extra = () if kind == capi.CONV_FWD else (0,)
+            capi.check(fn(ctx.h, a.ptr, b_.ptr, out.ptr, *dims, *extra, ws.ptr, need))
+            assert np.array_equal(out.numpy(), ref), (kind, case)
+
+
 # Image layers (at most 4 input channels forward, 3 for the weight gradient; W % 4 == 0): the LDS-patch kernels for
 # few channels.  Ragged Cout, tiles that end inside a row, strides, wide rows, padding 0 and 2, one-channel MNIST shape.
 SMALLC_CASES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw)

@@ -440,3 +440,90 @@ def test_forward_patch_kernel_loads_stay_inside_the_tensors(case):
     if st == (1, 1):  # the data gradient runs the same kernel over grad_out with padding 2 - p and channels swapped
         OH, OW = H + 2 * pd[0] - 2, W + 2 * pd[1] - 2
         fwd_loads_in_bounds(B, M, OH, OW, C, 1, 1, 2 - pd[0], 2 - pd[1])
+
+
+# ---- conv_patch_f64.hpp: the f64 twin of the persistent forward / data-gradient kernel ---------------------------------------
+D_PPLANE, D_NXP, D_LPR = 573, 8, 32
+def f64_plans(B, C, H, W, M, OH, OW, kh, kw, sh, sw, ph, pw):
+    """cpd::make_plan's candidates (tile widths 8, 7, 5), or [] when the layer stays on the implicit GEMM."""
+    L = OH * OW
+    if kh != 3 or kw != 3 or C % CC or W < 2 or W % 2 or W > 2 * D_LPR or sh > 8 or sw > 8 or L < 64 or M < 32: return []
+    plans = []
+    for tn in (8, 7, 5):
+        np_ = 16 * tn
+        tiles, mtiles = _ceil_div(L, np_), _ceil_div(M, 64)
+        rows = min(OH, np_ // OW if np_ % OW == 0 else (np_ - 1) // OW + 2); PR = (rows - 1) * sh + 3
+        if PR > D_NXP or mtiles * 64 > M * 2 or tiles * np_ > L * 2: continue
+        pw2 = W + 2 * pw
+        if sw == 1:
+            padded = pw2
+            while (sh * padded - OW) % 16: padded += 1
+            if PR * padded <= D_PPLANE: pw2 = padded
+        if PR * pw2 > D_PPLANE: continue
+        plans.append(dict(TN=tn, PR=PR, PW=pw2, tpi=tiles, mtiles=mtiles, nchunks=C // CC, NPIX=np_))
+    return plans
+def f64_walk(pl, B, C, H, W, M, OH, OW, sh, sw, ph, pw, num_cus=256):
+    """Every tile is visited exactly once; weight-image, input and output addresses and the LDS offsets stay inside their buffers;
+    every 16-byte load is 16-byte aligned."""
+    PW, PLANE, bufsz, L, NPIX = pl["PW"], D_PPLANE, CC * D_PPLANE + 16, OH * OW, pl["NPIX"]
+    assert PLANE >= pl["PR"] * PW and PW >= W + 2 * pw and pl["PR"] <= D_NXP
+    assert 2 * bufsz * 8 <= 72 * 1024 and (bufsz + 4 * PLANE + 2) * 8 < 65536
+    bt = B * pl["tpi"]; ntiles = bt * pl["mtiles"]
+    nblk = min(ntiles, 2 * num_cus); chunk = 0
+    if ntiles % 8 == 0 and nblk >= 8:
+        nblk -= nblk % 8; chunk = ntiles // 8
+    seen = [0] * ntiles
+    for bid in range(nblk):
+        if chunk: x = bid & 7; q, step, end = x * chunk + (bid >> 3), nblk >> 3, (x + 1) * chunk
+        else: q, step, end = bid, nblk, ntiles
+        while q < end:
+            seen[q] += 1; q += step
+    assert all(v == 1 for v in seen)
+    wbuf = pl["mtiles"] * 4 * pl["nchunks"] * KK * 64 * 2          # doubles written by cpd::wimg_kernel = the workspace asked for
+    xsize, ysize = B * C * H * W, B * M * L
+    for q in sorted({0, 1, pl["tpi"] - 1, pl["tpi"], bt - 1, ntiles - 1, ntiles // 2} & set(range(ntiles))):
+        mt, rem = divmod(q, bt); b, t = divmod(rem, pl["tpi"])
+        pix0 = t * NPIX; py0 = pix0 // OW; iy_base = py0 * sh - ph; m0 = mt * 64
+        for wave in range(4):
+            for ch in (0, pl["nchunks"] - 1):
+                a = ((mt * 4 + wave) * pl["nchunks"] + ch) * KK * 128 + 8 * 128 + 63 * 2
+                assert a + 2 <= wbuf and a % 2 == 0, ("A", a, wbuf)
+        for ch in (0, pl["nchunks"] - 1):
+            for tid in range(NT):
+                pq, xc = tid & 31, tid >> 5
+                lane_in = pq < ((W + 1) >> 1); xcol = min(2 * pq, W - 2)
+                for u in range(D_NXP):
+                    iy = iy_base + u
+                    if u < pl["PR"] and 0 <= iy < H:
+                        a = ((b * C + ch * CC) * H + iy) * W + ((xc * H * W + xcol) if lane_in else 0)
+                        assert 0 <= a and a + 2 <= xsize and a % 2 == 0, ("x", a, xsize)
+                    if u < pl["PR"] and lane_in:
+                        d = xc * PLANE + pw + xcol + u * PW
+                        assert 0 <= d and d + 2 <= CC * PLANE, ("park", d)
+        for pi in range(pix0, pix0 + NPIX):
+            if pi >= L: continue
+            py, px = divmod(pi, OW)
+            off = (py - py0) * sh * PW + px * sw + 7 * PLANE + 2 * PW + 2   # last channel, last tap
+            assert 0 <= (py - py0) * sh + 2 < pl["PR"] and px * sw + 2 < PW and off < CC * PLANE, ("B read", off)
+            assert (b * M + min(M, m0 + 64) - 1) * L + pi < ysize
+    return "f64 x%d ok" % pl["TN"]
+
+
+F64_SHAPES = [  # B, C, H, W, M, (sh, sw), (ph, pw)
+    (2, 64, 56, 56, 128, (1, 1), (1, 1)), (128, 64, 56, 56, 128, (1, 1), (1, 1)), (2, 8, 6, 12, 60, (1, 1), (1, 1)), (3, 16, 8, 36, 120, (1, 1), (0, 0)),
+    (2, 24, 10, 16, 104, (1, 1), (2, 2)), (1, 8, 64, 64, 52, (1, 1), (1, 1)), (2, 16, 9, 62, 60, (2, 1), (1, 1)), (4, 32, 32, 32, 64, (1, 1), (1, 1)),
+    (2, 8, 9, 64, 128, (2, 1), (1, 1)), (3, 8, 14, 28, 64, (1, 1), (1, 1)), (2, 8, 9, 30, 128, (1, 1), (0, 0)), (2, 32, 28, 28, 33, (1, 1), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", F64_SHAPES, ids=str)
+def test_f64_patch_kernel_loads_stay_inside_the_tensors(case):
+    B, C, H, W, M, st, pd = case
+    OH, OW = (H + 2 * pd[0] - 3) // st[0] + 1, (W + 2 * pd[1] - 3) // st[1] + 1
+    plans = f64_plans(B, C, H, W, M, OH, OW, 3, 3, st[0], st[1], pd[0], pd[1])
+    assert plans, "the shape must exercise the f64 patch kernel"
+    for pl in plans:
+        f64_walk(pl, min(B, 3), C, H, W, M, OH, OW, st[0], st[1], pd[0], pd[1])
+    if st == (1, 1) and M % CC == 0 and OW % 2 == 0:  # the data gradient: a forward pass over grad_out, channels swapped, padding 2 - p
+        for pl in f64_plans(B, M, OH, OW, C, H, W, 3, 3, 1, 1, 2 - pd[0], 2 - pd[1]):
+            f64_walk(pl, min(B, 3), M, OH, OW, C, H, W, 1, 1, 2 - pd[0], 2 - pd[1])
