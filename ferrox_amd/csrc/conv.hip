@@ -17,6 +17,7 @@
 #include "conv_smallc.hpp"
 #include "conv_patch.hpp"
 #include "conv_patch_f64.hpp"
+#include "wgrad_patch_f64.hpp"
 
 namespace fx {
 int col2im_f32(fx_ctx*, const float*, float*, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, int);
@@ -531,6 +532,15 @@ wgp::Plan patch_plan(fx_ctx* c, const Dims& d, int mode) {
 }
 
 template <typename T>
+wgd::Plan patch64_plan(fx_ctx* c, const Dims& d, int mode) {
+    if constexpr (sizeof(T) == 8) {
+        if (mode == 0 && !generic_only())
+            return wgd::make_plan(c ? c->num_cus : 256, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
+    }
+    return wgd::Plan();
+}
+
+template <typename T>
 i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     const wgp::Plan pl = patch_plan<T>(c, d, mode);
     int splits, kps;
@@ -542,6 +552,8 @@ i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
         const csc::Plan sp = smallc_plan<T>(c, d, true);
         if (sp.ok) generic = std::max(generic, csc::wgrad_workspace_bytes(sp, d.Cout, d.Cin));
     }
+    const wgd::Plan pd = patch64_plan<T>(c, d, mode);
+    if (pd.ok) generic = std::max(generic, wgd::workspace_bytes(pd, d.Cout, d.Cin));
     return pl.ok ? std::max(generic, wgp::workspace_bytes(pl, d.Cout, d.Cin)) : generic;
 }
 
@@ -597,6 +609,14 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
             float* part = (float*)(ws ? ws : c->get_scratch(need));
             if (!part) return FX_ERR_OOM;
             return wgp::run(c, pl, x, g, dw, part, Cin, H, W, Cout, sh, sw, ph, pw, d.oh, d.ow);
+        }
+    }
+    if constexpr (sizeof(T) == 8) {
+        const wgd::Plan pd = patch64_plan<T>(c, d, mode);
+        if (pd.ok && aligned16(x, g) && aligned16(ws, ws)) {
+            double* part = (double*)(ws ? ws : c->get_scratch(need));
+            if (!part) return FX_ERR_OOM;
+            return wgd::run(c, pd, x, g, dw, part, Cin, H, W, Cout, sh, ph, pw, d.oh, d.ow);
         }
     }
     if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64) return wgrad_tile<T, TileM128>(c, x, g, dw, d, mode, ws);

@@ -609,6 +609,43 @@ def test_conv2d_f64_patch_kernel_shapes(ctx, orc):
             assert np.array_equal(out.numpy(), ref), (kind, case)
 
 
+# f64 weight gradient on the 16x16x4 MFMA patch kernel (wgrad_patch_f64.hpp: 3x3, unit column stride, rows of 24 / 32 / 56 / 64
+# pixels, Cin % 16 == 0, Cout % 64 == 0): every row length, several channel tiles, paddings 0 / 1 / 2, a row stride of 2, a batch
+# that does not fill the splits evenly.
+CONV_F64_WGRAD_CASES = [  # B, Cin, H, W, Cout, sh, (ph, pw)
+    (2, 64, 56, 56, 128, 1, (1, 1)), (3, 16, 32, 32, 64, 1, (1, 1)), (2, 32, 26, 26, 64, 1, (0, 0)), (2, 16, 24, 62, 128, 1, (2, 2)),
+    (2, 48, 47, 24, 64, 2, (1, 1)), (5, 16, 8, 64, 64, 1, (1, 1)), (37, 16, 9, 32, 64, 1, (1, 1)),
+]
+
+
+def test_conv2d_f64_wgrad_patch_kernel_shapes(ctx, orc):
+    import torch
+    import torch.nn.functional as F
+    from ferrox_amd import capi
+    rng = np.random.default_rng(62)
+    tol = TOL[np.dtype(np.float64)]
+    for (B, Cin, H, W, Cout, sh, pd) in CONV_F64_WGRAD_CASES:
+        case = (B, Cin, H, W, Cout, sh, pd)
+        st = (sh, 1)
+        x = rng.uniform(-1, 1, (B, Cin, H, W))
+        oh, ow = orc.out_hw(H, W, 3, 3, st[0], st[1], pd[0], pd[1])
+        g = rng.standard_normal((B, Cout, oh, ow))
+        dx_, dg_ = ctx.upload(x), ctx.upload(g)
+        dwg = ctx.conv2d_wgrad(dx_, dg_, (Cout, Cin, 3, 3), st, pd, 0).numpy()
+        tw = torch.zeros((Cout, Cin, 3, 3), dtype=torch.float64, requires_grad=True)
+        F.conv2d(torch.from_numpy(x), tw, stride=st, padding=pd).backward(torch.from_numpy(g))
+        assert rel_err(dwg, tw.grad.numpy()) <= tol * 8, ("wgrad", case)
+        if B * Cout * oh * ow <= 1 << 20:
+            assert rel_err(dwg, orc.conv2d_wgrad(x, g, (Cout, Cin, 3, 3), st, pd, 0)) <= tol * 8, ("wgrad vs oracle", case)
+        # a caller-provided workspace of exactly the advertised size gives the same bits
+        dims = (B, Cin, H, W, Cout, 3, 3, st[0], st[1], pd[0], pd[1])
+        need = capi.lib.fx_conv2d_workspace_bytes(capi.CONV_WGRAD, capi.FX_F64, 0, *dims)
+        ws = ctx.empty((max(need, 8) // 8,), np.float64)
+        out = ctx.empty((Cout, Cin, 3, 3), np.float64)
+        capi.check(capi.lib.fx_conv2d_wgrad_f64(ctx.h, dx_.ptr, dg_.ptr, out.ptr, *dims, 0, ws.ptr, need))
+        assert np.array_equal(out.numpy(), dwg), case
+
+
 # Image layers (at most 4 input channels forward, 3 for the weight gradient; W % 4 == 0): the LDS-patch kernels for
 # few channels.  Ragged Cout, tiles that end inside a row, strides, wide rows, padding 0 and 2, one-channel MNIST shape.
 SMALLC_CASES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw)

@@ -527,3 +527,67 @@ def test_f64_patch_kernel_loads_stay_inside_the_tensors(case):
     if st == (1, 1) and M % CC == 0 and OW % 2 == 0:  # the data gradient: a forward pass over grad_out, channels swapped, padding 2 - p
         for pl in f64_plans(B, M, OH, OW, C, H, W, 3, 3, 1, 1, 2 - pd[0], 2 - pd[1]):
             f64_walk(pl, min(B, 3), M, OH, OW, C, H, W, 1, 1, 2 - pd[0], 2 - pd[1])
+
+
+# ---- wgrad_patch_f64.hpp: the f64 weight gradient -------------------------------------------------------------------------------
+def wgd_plan(B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, oh, ow, num_cus=256):
+    if (kh != 3 or kw != 3 or sw != 1 or sh > 8 or Cin % 16 or Cout % 64 or W % 2 or W > 64 or ow % 8 or ow < 24 or ow > 64
+            or ow // 8 not in (3, 4, 7, 8)): return None
+    PW = W + 2 * pw; PLANE = (3 * PW) | 1; GP = ow | 1
+    smem = max((64 * GP + 16 * PLANE + 16) * 8, 2 * 4 * 64 * 8)
+    if smem > 72 * 1024: return None
+    stages = B * oh; tiles = (Cin // 16) * (Cout // 64)
+    splits = max(1, min(num_cus * 2 // tiles, max(1, stages // 4)))
+    sps = _ceil_div(stages, splits)
+    return dict(PW=PW, PLANE=PLANE, GP=GP, NK=ow // 8, stages=stages, sps=sps, splits=_ceil_div(stages, sps), smem=smem)
+def wgd_walk(pl, B, Cin, H, W, Cout, sh, ph, pw, oh, ow):
+    L, PW, PLANE, GP, NK = oh * ow, pl["PW"], pl["PLANE"], pl["GP"], pl["NK"]
+    gsize, xsize = B * Cout * L, B * Cin * H * W
+    covered = set()
+    for z in range(pl["splits"]):
+        covered |= set(range(z * pl["sps"], min(pl["stages"], (z + 1) * pl["sps"])))
+    assert covered == set(range(pl["stages"]))
+    assert PW == ow + 2 and PLANE >= 3 * PW and GP >= ow
+    for s in (0, 1, oh - 1, oh, pl["stages"] - 1):
+        if not 0 <= s < pl["stages"]: continue
+        b, oy = divmod(s, oh); iy0 = oy * sh - ph
+        for c0 in (0, Cin - 16):
+            for oc0 in (0, Cout - 64):
+                for tid in range(NT):
+                    pq, prow = tid & 31, tid >> 5
+                    if pq < ow // 2:
+                        for u in range(8):
+                            a = ((b * Cout + oc0 + prow + 8 * u) * L) + oy * ow + 2 * pq
+                            assert 0 <= a and a + 2 <= gsize and a % 2 == 0, ("g", a)
+                            d = (prow + 8 * u) * GP + 2 * pq
+                            assert d + 2 <= 64 * GP
+                    if pq < W // 2:
+                        for r in range(3):
+                            iy = iy0 + r
+                            for cu in range(2):
+                                if 0 <= iy < H:
+                                    a = ((b * Cin + c0 + prow + 8 * cu) * H + iy) * W + 2 * pq
+                                    assert 0 <= a and a + 2 <= xsize and a % 2 == 0, ("x", a)
+                                d = (prow + 8 * cu) * PLANE + r * PW + pw + 2 * pq
+                                assert d + 2 <= 16 * PLANE
+    for wk in range(2):   # operand reads of the last pixel group
+        pix = wk * 4 * NK + 4 * (NK - 1) + 3
+        assert pix < ow and 63 * GP + pix < 64 * GP and 15 * PLANE + 2 * PW + pix + 2 < 16 * PLANE
+    assert pl["splits"] * Cout * Cin * 9 * 8 > 0
+    return "wgd ok"
+
+
+WGD_SHAPES = [  # B, Cin, H, W, Cout, sh, (ph, pw)
+    (128, 64, 56, 56, 128, 1, (1, 1)), (3, 16, 32, 32, 64, 1, (1, 1)), (2, 32, 26, 26, 64, 1, (0, 0)), (2, 16, 24, 62, 128, 1, (2, 2)),
+    (2, 48, 47, 24, 64, 2, (1, 1)), (5, 16, 8, 64, 64, 1, (1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", WGD_SHAPES, ids=str)
+def test_f64_weight_gradient_patch_kernel_loads_stay_inside_the_tensors(case):
+    B, Cin, H, W, Cout, sh, pd = case
+    oh, ow = (H + 2 * pd[0] - 3) // sh + 1, W + 2 * pd[1] - 2
+    B = min(B, 3)  # the first and the last images are the ones at the tensor ends
+    pl = wgd_plan(B, Cin, H, W, Cout, 3, 3, sh, 1, pd[0], pd[1], oh, ow)
+    assert pl is not None, "the shape must exercise the f64 weight-gradient patch kernel"
+    wgd_walk(pl, B, Cin, H, W, Cout, sh, pd[0], pd[1], oh, ow)
