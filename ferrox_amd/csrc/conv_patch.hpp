@@ -164,7 +164,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
             const int idx = wd + u * NT;
             if ((u + 1) * NT <= WIMG / 4 || idx < WIMG / 4) *reinterpret_cast<float4*>(Ws + 4 * idx) = wv[u];
         }
-        if (x_lane && !(p.relu & 4096)) {
+        if (x_lane) {
 #pragma unroll
             for (int u = 0; u < NXP; ++u) {
                 const int r = 2 * u + rp;

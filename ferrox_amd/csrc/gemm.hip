@@ -34,12 +34,14 @@ int run(fx_ctx* c, i64 M, i64 N, i64 K, const T* A, const T* B, T* C, const T* b
         MatStore<T> ep{C, N, 0, (int)M, (int)N};
         return launch<T, Cfg>(c, al, bl, ep, M, N, K, 1, kps);
     }
-    *bias_pending = bias != nullptr;  // split-K: the caller adds the bias after the ordered sum
+    // split-K: the bias (and ReLU) ride in the ordered sum's store where its indices fit 32 bits, else the caller adds them after it
+    const bool in_sum = bias != nullptr && M * N <= 0x7fffffff;
+    *bias_pending = bias != nullptr && !in_sum;
     T* part = (T*)c->get_scratch((i64)splits * M * N * (i64)sizeof(T));
     if (!part) return FX_ERR_OOM;
     MatStore<T> ep{part, N, M * N, (int)M, (int)N};
     if (int rc = launch<T, Cfg>(c, al, bl, ep, M, N, K, splits, kps)) return rc;
-    return launch_splitk_reduce<T>(c, part, C, M * N, splits);
+    return launch_splitk_reduce<T>(c, part, C, M * N, splits, in_sum ? bias : nullptr, N, relu);
 }
 
 template <typename T, class Cfg>

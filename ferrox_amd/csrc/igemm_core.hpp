@@ -587,8 +587,25 @@ __global__ __launch_bounds__(Cfg::NT) void igemm_multi_kernel(const MultiProblem
 }
 
 // Sums split-K partials in split order (deterministic) into the final buffer; 8 independent loads in flight.
+// Optional epilogue of the sums below: + bias[column] (row-major [rows][ncols] outputs), then ReLU -- the operations of
+// fx_bias_act in its order, so the bits are those of the sum followed by that call.
+template <typename T> struct SumEpilogue {
+    const T* bias = nullptr;
+    FastDiv div_cols;
+    int ncols = 1, relu = 0;
+    __device__ __forceinline__ T apply(T s, i64 i) const {
+        if (bias) {
+            const uint32_t r = div_cols.div((uint32_t)i);
+            s = s + bias[(uint32_t)i - r * (uint32_t)ncols];
+            if (relu) s = s > T(0) ? s : T(0);
+        }
+        return s;
+    }
+};
+
 template <typename T>
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(const T* __restrict__ part, T* __restrict__ out, i64 n, int splits) {
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const T* __restrict__ part, T* __restrict__ out, i64 n, int splits,
+                                                            const SumEpilogue<T> ep = SumEpilogue<T>()) {
     const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     T s = T(0);
@@ -601,7 +618,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const T* __restrict_
         for (int u = 0; u < 8; ++u) s = s + v[u];
     }
     for (; z < splits; ++z) s = s + part[(i64)z * n + i];
-    out[i] = s;
+    out[i] = ep.apply(s, i);
 }
 
 template <typename T, class Cfg, class AL, class BL, class EP>
@@ -633,7 +650,8 @@ int launch_multi(fx_ctx* c, const MultiProblem<AL, BL, EP, NP>& mp, int count) {
 // order, then the G partial sums are added in order of g.  The grouping depends only on (n, splits), so the
 // result is reproducible run to run; it differs from the single-chain order by rounding only.
 template <typename T, int G>
-__global__ __launch_bounds__(256) void splitk_reduce_grouped_kernel(const T* __restrict__ part, T* __restrict__ out, i64 n, int splits) {
+__global__ __launch_bounds__(256) void splitk_reduce_grouped_kernel(const T* __restrict__ part, T* __restrict__ out, i64 n, int splits,
+                                                                    const SumEpilogue<T> ep = SumEpilogue<T>()) {
     constexpr int COLS = 256 / G;
     __shared__ T sm[G][COLS];
     const int col = threadIdx.x % COLS, g = threadIdx.x / COLS;
@@ -656,18 +674,24 @@ __global__ __launch_bounds__(256) void splitk_reduce_grouped_kernel(const T* __r
         T t = sm[0][col];
 #pragma unroll
         for (int u = 1; u < G; ++u) t = t + sm[u][col];
-        out[i] = t;
+        out[i] = ep.apply(t, i);
     }
 }
 
+// bias (with ncols, relu): the epilogue above; n must then fit 32 bits
 template <typename T>
-int launch_splitk_reduce(fx_ctx* c, const T* part, T* out, i64 n, int splits) {
+int launch_splitk_reduce(fx_ctx* c, const T* part, T* out, i64 n, int splits, const T* bias = nullptr, i64 ncols = 1, int relu = 0) {
+    SumEpilogue<T> ep;
+    if (bias) {
+        FX_REQUIRE(n <= 0x7fffffff && ncols >= 1 && ncols <= 0x7fffffff, "split-K sum with bias: %lld outputs exceed 2^31", (long long)n);
+        ep.bias = bias; ep.ncols = (int)ncols; ep.relu = relu; ep.div_cols = FastDiv((uint32_t)ncols);
+    }
     if (splits >= 128 && n <= (1 << 16))
-        splitk_reduce_grouped_kernel<T, 16><<<dim3((unsigned)fx::ceil_div(n, 16)), dim3(256), 0, c->stream>>>(part, out, n, splits);
+        splitk_reduce_grouped_kernel<T, 16><<<dim3((unsigned)fx::ceil_div(n, 16)), dim3(256), 0, c->stream>>>(part, out, n, splits, ep);
     else if (splits >= 32 && n <= (1 << 18))
-        splitk_reduce_grouped_kernel<T, 4><<<dim3((unsigned)fx::ceil_div(n, 64)), dim3(256), 0, c->stream>>>(part, out, n, splits);
+        splitk_reduce_grouped_kernel<T, 4><<<dim3((unsigned)fx::ceil_div(n, 64)), dim3(256), 0, c->stream>>>(part, out, n, splits, ep);
     else
-        splitk_reduce_kernel<T><<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(part, out, n, splits);
+        splitk_reduce_kernel<T><<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(part, out, n, splits, ep);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

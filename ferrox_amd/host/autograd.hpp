@@ -480,14 +480,27 @@ template <typename T> class AutoFerroxEngine {
         if (!it->second.is_parameter()) throw Error("Can only update parameter nodes (leaf nodes with requires_grad)");
         it->second.tensor = std::move(t);
     }
-    void backward(NodeId loss_id) {  // :700-733
+    // keep_loss: receives the loss tensor itself before the graph is cleaned up (the fused training loop reads it after the
+    // step instead of cloning it).  With reuse_unit_seed set, a one-element loss is seeded from a tensor of one 1.0 that is
+    // filled once and only ever read, instead of a fresh ones() per step (same value, one kernel fewer).
+    bool reuse_unit_seed = false;
+    void backward(NodeId loss_id, Tensor<T>* keep_loss = nullptr) {  // :700-733
         const HipStorage<T>* loss = get_tensor(loss_id);
         if (!loss) throw Error("Loss node not found");
-        grads_[loss_id] = HipStorage<T>::ones(loss->shape());
+        if (reuse_unit_seed && loss->size() == 1) {
+            if (!unit_seed_) unit_seed_ = HipStorage<T>::ones({1});
+            Tensor<T> seed = HipStorage<T>::borrow(*unit_seed_);
+            seed->reshape(loss->shape());
+            grads_[loss_id] = std::move(seed);
+        } else grads_[loss_id] = HipStorage<T>::ones(loss->shape());
         std::set<NodeId> visited;
         std::vector<NodeId> topo;
         topological_sort(loss_id, visited, topo);
         for (auto it = topo.rbegin(); it != topo.rend(); ++it) backward_node(*it);
+        if (keep_loss) {
+            auto it = nodes_.find(loss_id);
+            if (it != nodes_.end()) *keep_loss = std::move(it->second.tensor);
+        }
         cleanup();
     }
     size_t num_nodes() const { return nodes_.size(); }
@@ -544,6 +557,7 @@ template <typename T> class AutoFerroxEngine {
     }
 
     bool literal_;
+    Tensor<T> unit_seed_;
     NodeId next_id_ = 0;
     std::map<NodeId, Node> nodes_;
     std::map<NodeId, Tensor<T>> grads_;

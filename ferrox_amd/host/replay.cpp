@@ -104,6 +104,7 @@ template <typename T> struct Model : ModelBase {
     //         2 = fused layers / loss / optimizers
     Model(const std::string& spec, const std::string& optspec, int engine, const void* const* pv, int np)
         : graph(engine == 1), fused(engine == 2) {
+        graph.reuse_unit_seed = fused;
         int pi = 0;
         auto next = [&]() -> const T* {
             if (pi >= np) throw Error("not enough parameter arrays for the layer spec");
@@ -247,8 +248,8 @@ template <typename T> struct Model : ModelBase {
         for (auto& l : layers) in = l->forward(graph, in);
         return in;
     }
-    // zero_gradients -> forward -> loss -> copy of the loss -> backward -> update, nothing read back: the form a step is
-    // recorded in
+    // zero_gradients -> forward -> loss -> backward -> update, nothing read back (the loss tensor is handed out): the form a
+    // step is recorded in
     Tensor<T> step_body(bool optimizer_step) {
         graph.zero_gradients();
         const NodeId xin = graph.create_variable(fused ? HipStorage<T>::borrow(*x) : x->clone_storage(), false);
@@ -259,10 +260,10 @@ template <typename T> struct Model : ModelBase {
             const NodeId yin = graph.create_variable(fused ? HipStorage<T>::borrow(*y) : y->clone_storage(), false);
             loss = fused ? cce_loss_fused<T>(graph, pred, yin) : cce_loss<T>(graph, pred, yin);
         }
-        Tensor<T> lcopy = graph.get_tensor(loss)->clone_storage();
-        graph.backward(loss);
+        Tensor<T> lval;
+        graph.backward(loss, &lval);
         if (optimizer_step) opt->step(graph);
-        return lcopy;
+        return lval;
     }
     double train_step(bool optimizer_step) override {
         if (!x || !y) throw Error("set_batch was not called");
@@ -319,12 +320,12 @@ template <typename T> struct Model : ModelBase {
             if (optimizer_step) opt->step(graph);
             return (double)lv;
         }
-        // fused engine: the loss is copied aside and read after the backward pass and the update are enqueued, so the
-        // device never waits for the host in the middle of a step
-        Tensor<T> lcopy = graph.get_tensor(loss)->clone_storage();
-        graph.backward(loss);
+        // fused engine: the loss tensor outlives the graph's clean-up and is read after the backward pass and the update are
+        // enqueued, so the device never waits for the host in the middle of a step
+        Tensor<T> lval;
+        graph.backward(loss, &lval);
         if (optimizer_step) opt->step(graph);
-        return (double)lcopy->first();
+        return (double)lval->first();
     }
     void get_param(int i, void* host) const override {
         std::vector<T> v = graph.get_tensor(params.at(i))->to_vec();
