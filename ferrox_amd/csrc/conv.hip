@@ -14,6 +14,7 @@
 
 #include "igemm_core.hpp"
 #include "wgrad_patch.hpp"
+#include "wgrad_patch_s2.hpp"
 #include "conv_smallc.hpp"
 #include "conv_patch.hpp"
 #include "conv_patch_f64.hpp"
@@ -532,6 +533,15 @@ wgp::Plan patch_plan(fx_ctx* c, const Dims& d, int mode) {
 }
 
 template <typename T>
+wg2::Plan patch_s2_plan(fx_ctx* c, const Dims& d, int mode) {
+    if constexpr (sizeof(T) == 4) {
+        if (mode == 0 && !generic_only())
+            return wg2::make_plan(c ? c->num_cus : 256, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
+    }
+    return wg2::Plan();
+}
+
+template <typename T>
 wgd::Plan patch64_plan(fx_ctx* c, const Dims& d, int mode) {
     if constexpr (sizeof(T) == 8) {
         if (mode == 0 && !generic_only())
@@ -554,6 +564,8 @@ i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     }
     const wgd::Plan pd = patch64_plan<T>(c, d, mode);
     if (pd.ok) generic = std::max(generic, wgd::workspace_bytes(pd, d.Cout, d.Cin));
+    const wg2::Plan p2 = patch_s2_plan<T>(c, d, mode);
+    if (p2.ok) generic = std::max(generic, wg2::workspace_bytes(p2, d.Cout, d.Cin));
     return pl.ok ? std::max(generic, wgp::workspace_bytes(pl, d.Cout, d.Cin)) : generic;
 }
 
@@ -603,6 +615,12 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
                 if (!part) return FX_ERR_OOM;
             }
             return csc::run_wgrad(c, sp, x, g, dw, part, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw);
+        }
+        const wg2::Plan p2 = patch_s2_plan<T>(c, d, mode);
+        if (p2.ok && aligned16(x, g) && aligned16(ws, ws)) {
+            float* part = (float*)(ws ? ws : c->get_scratch(need));
+            if (!part) return FX_ERR_OOM;
+            return wg2::run(c, p2, x, g, dw, part, Cin, H, Cout, ph, d.oh);
         }
         const wgp::Plan pl = patch_plan<T>(c, d, mode);
         if (pl.ok && aligned16(x, g) && aligned16(ws, ws)) {

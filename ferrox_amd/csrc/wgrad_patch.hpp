@@ -368,6 +368,43 @@ __global__ __launch_bounds__(256) void wgrad_patch_reduce_grouped_kernel(const f
     }
 }
 
+// The grouped sum over four adjacent outputs per thread (n and Cin multiples of 4, so the four share their output channel and
+// tap): 16-byte loads, a group's 16 threads cover 256 contiguous bytes of a partial.  Same grouping and order as above.
+template <int G>
+__global__ __launch_bounds__(256) void wgrad_patch_reduce_vec_kernel(const float* __restrict__ part, float* __restrict__ out, int n,
+                                                                     int splits, int Cin, FastDiv div_row, FastDiv div_cin) {
+    constexpr int COLS = 256 / G;
+    __shared__ float4 sm[G][COLS];
+    const int col = threadIdx.x % COLS, g = threadIdx.x / COLS;
+    const int j = (blockIdx.x * COLS + col) * 4;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (j < n) {
+        int z = g;
+        for (; z + 7 * G < splits; z += 8 * G) {
+            float4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(part + (i64)(z + u * G) * n + j);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) { s.x = s.x + v[u].x; s.y = s.y + v[u].y; s.z = s.z + v[u].z; s.w = s.w + v[u].w; }
+        }
+        for (; z < splits; z += G) {
+            const float4 v = *reinterpret_cast<const float4*>(part + (i64)z * n + j);
+            s.x = s.x + v.x; s.y = s.y + v.y; s.z = s.z + v.z; s.w = s.w + v.w;
+        }
+    }
+    sm[g][col] = s;
+    __syncthreads();
+    if (g == 0 && j < n) {
+        float4 t = sm[0][col];
+#pragma unroll
+        for (int u = 1; u < G; ++u) { const float4 v = sm[u][col]; t.x = t.x + v.x; t.y = t.y + v.y; t.z = t.z + v.z; t.w = t.w + v.w; }
+        const int oc = (int)div_row.div((uint32_t)j), rem = j - oc * (KK * Cin);
+        const int tap = (int)div_cin.div((uint32_t)rem), c = rem - tap * Cin;
+        float* o = out + ((i64)oc * Cin + c) * KK + tap;
+        o[0] = t.x; o[KK] = t.y; o[2 * KK] = t.z; o[3 * KK] = t.w;
+    }
+}
+
 struct Plan {
     bool ok = false;
     int R = 1, PR = 0, PW = 0, PLANE = 0, GP = 0, Kst = 0, splits = 1, sps = 1, stages = 0;

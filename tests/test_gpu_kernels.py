@@ -443,6 +443,11 @@ WGRAD_PATCH_CASES = [
     (1, 33, 8, 24, 16, (1, 1), (1, 1)), (2, 17, 6, 32, 32, (1, 1), (1, 1)), (3, 48, 8, 32, 64, (1, 1), (1, 1)),
     # 64-wide rows with 64 x 64 channels (the 64-plane layout exceeds the LDS budget)
     (2, 64, 8, 64, 64, (1, 1), (1, 1)), (2, 64, 8, 64, 32, (1, 1), (1, 1)),
+    # stride 2, padding 1 over maps 32 and 64 wide: the double-buffered stride-2 kernel in its three wave layouts, a top row
+    # without padding, an odd height (the last patch row is below the image), many splits
+    (3, 32, 32, 32, 64, (2, 2), (1, 1)), (2, 64, 8, 32, 128, (2, 2), (1, 1)), (5, 32, 16, 32, 32, (2, 2), (1, 1)), (2, 32, 8, 64, 64, (2, 2), (1, 1)),
+    (2, 64, 4, 64, 128, (2, 2), (1, 1)), (3, 32, 12, 64, 96, (2, 2), (1, 1)), (2, 32, 9, 32, 64, (2, 2), (0, 1)), (2, 32, 15, 32, 64, (2, 2), (1, 1)),
+    (40, 32, 8, 32, 64, (2, 2), (1, 1)),
     # narrow maps: one whole image per stage, (channel, row) pair staging
     (3, 64, 8, 8, 128, (1, 1), (1, 1)), (2, 32, 8, 8, 64, (1, 1), (1, 1)), (2, 96, 8, 8, 20, (1, 1), (1, 1)), (2, 32, 6, 8, 100, (1, 1), (1, 1)),
     (3, 64, 4, 16, 72, (1, 1), (1, 1)), (2, 48, 8, 8, 24, (1, 1), (1, 1)), (70, 128, 8, 8, 128, (1, 1), (1, 1)),

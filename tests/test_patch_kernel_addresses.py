@@ -591,3 +591,93 @@ def test_f64_weight_gradient_patch_kernel_loads_stay_inside_the_tensors(case):
     pl = wgd_plan(B, Cin, H, W, Cout, 3, 3, sh, 1, pd[0], pd[1], oh, ow)
     assert pl is not None, "the shape must exercise the f64 weight-gradient patch kernel"
     wgd_walk(pl, B, Cin, H, W, Cout, sh, pd[0], pd[1], oh, ow)
+
+
+# ---- f32 stride-2 weight gradient (wgrad_patch_s2.hpp) ----
+WG2_INSTANCES = [(1, 16, 4), (2, 16, 4), (4, 16, 4), (1, 32, 2), (2, 32, 2), (4, 32, 2)]
+def wg2_plan(B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, oh, ow, num_cus=256):
+    if kh != 3 or kw != 3 or sh != 2 or sw != 2 or pw != 1 or ph > 1 or W != 2 * ow or Cin % 32 or Cout % 32: return None
+    wmo = 4 if Cout % 128 == 0 else 2 if Cout % 64 == 0 else 1
+    pick = [(a, o, r) for (a, o, r) in WG2_INSTANCES if a == wmo and o == ow and oh % r == 0]
+    if not pick: return None
+    WMO, OW, R = pick[0]
+    stages = B * (oh // R); tiles = (Cin // 32) * (Cout // (32 * WMO))
+    splits = max(1, min(num_cus // tiles, max(1, stages // 2)))
+    sps = _ceil_div(stages, splits)
+    return dict(WMO=WMO, OW=OW, R=R, stages=stages, sps=sps, splits=_ceil_div(stages, sps))
+def wg2_walk(pl, B, Cin, H, Cout, ph, oh):
+    WMO, OW, R = pl["WMO"], pl["OW"], pl["R"]
+    WK, BM, W, PW, XR, KST = 4 // WMO, 32 * WMO, 2 * OW, 2 * OW + 2, 2 * R + 1, R * OW
+    GP, PLANE = _odd_pitch_w(KST), _odd_pitch_w(XR * PW)
+    XL = 8 if W <= 32 else 16
+    RX = NT // XL; NXP = XR * 32 // RX; NG = BM // 16
+    SEG = OW // WK; PAIRS = SEG // 2; BUF = BM * GP + 32 * PLANE
+    red = 4 * (9 - 9 // WK) * 16 * 64 * 4 if WK == 2 else 4 * 16 * 64 * 4   # the closing sum's LDS slots
+    assert XR * 32 % RX == 0 and max(2 * BUF * 4, red) <= 160 * 1024 and SEG % 2 == 0 and KST % 4 == 0 and KST <= 64
+    L, spi = oh * OW, oh // R
+    gsize, xsize = B * Cout * L, B * Cin * H * W
+    covered = set()
+    for z in range(pl["splits"]):
+        covered |= set(range(z * pl["sps"], min(pl["stages"], (z + 1) * pl["sps"])))
+    assert covered == set(range(pl["stages"]))
+    rows_parked = set()
+    for s in (0, 1, spi - 1, spi, pl["stages"] - 1):
+        if not 0 <= s < pl["stages"]: continue
+        b, k = divmod(s, spi); oy0 = k * R; iy0 = 2 * oy0 - ph
+        for c0 in (0, Cin - 32):
+            for oc0 in (0, Cout - BM):
+                for tid in range(NT):
+                    gq, grow, xq, xrow = tid & 15, tid >> 4, tid & (XL - 1), tid // XL
+                    g_lane, x_lane = gq < KST // 4, xq < W // 4
+                    for u in range(NG):
+                        a = (b * Cout + oc0 + 16 * u + grow) * L + oy0 * OW + (4 * gq if g_lane else 0)
+                        assert 0 <= a and a + 4 <= gsize and a % 4 == 0, ("g", a)
+                        if g_lane:
+                            d = (16 * u + grow) * GP + 4 * gq
+                            assert d + 4 <= BM * GP
+                    for u in range(NXP):
+                        r, cb = u * RX // 32, u * RX % 32
+                        iy = iy0 + r
+                        assert cb + xrow < 32 and r < XR
+                        if 0 <= iy < H:
+                            a = ((b * Cin + c0 + cb + xrow) * H + iy) * W + (4 * xq if x_lane else 0)
+                            assert 0 <= a and a + 4 <= xsize and a % 4 == 0, ("x", a)
+                        if x_lane:
+                            d = BM * GP + (cb + xrow) * PLANE + r * PW + 1 + 4 * xq
+                            assert BM * GP <= d and d + 4 <= BUF
+                            rows_parked.add((cb + xrow, r))
+    assert rows_parked == {(c, r) for c in range(32) for r in range(XR)}
+    # operand reads of every lane over the unrolled pixel loop stay inside the stage buffer, and the patch columns they touch are
+    # columns 0 .. W: the zero column on the left and the W staged ones
+    for wave in range(4):
+        wmo, wk = wave % WMO, wave // WMO
+        for lane in (0, 31, 32, 63):
+            half, l32 = lane >> 5, lane & 31
+            ga0 = (wmo * 32 + l32) * GP + wk * SEG + half
+            xb0 = BM * GP + l32 * PLANE + 2 * (wk * SEG + half)
+            for r in range(R):
+                for j in range(PAIRS):
+                    a = ga0 + r * OW + 2 * j
+                    assert a - (wmo * 32 + l32) * GP < KST
+                    for ky in range(3):
+                        for kx in range(3):
+                            d = xb0 + (2 * r + ky) * PW + 4 * j + kx
+                            col = d - BM * GP - l32 * PLANE - (2 * r + ky) * PW
+                            assert 0 <= col <= W and d < BUF
+    return "wg2 ok"
+
+
+WG2_SHAPES = [  # B, Cin, H, W, Cout, (ph, pw)
+    (256, 32, 32, 32, 64, (1, 1)), (2, 64, 8, 32, 128, (1, 1)), (5, 32, 16, 32, 32, (1, 1)), (2, 32, 8, 64, 64, (1, 1)), (2, 64, 4, 64, 128, (1, 1)),
+    (3, 32, 12, 64, 96, (1, 1)), (2, 32, 9, 32, 64, (0, 1)), (2, 32, 15, 32, 64, (1, 1)), (40, 32, 8, 32, 64, (1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", WG2_SHAPES, ids=str)
+def test_stride2_weight_gradient_patch_kernel_loads_stay_inside_the_tensors(case):
+    B, Cin, H, W, Cout, pd = case
+    oh, ow = (H + 2 * pd[0] - 3) // 2 + 1, (W + 2 * pd[1] - 3) // 2 + 1
+    B = min(B, 3)
+    pl = wg2_plan(B, Cin, H, W, Cout, 3, 3, 2, 2, pd[0], pd[1], oh, ow)
+    assert pl is not None, "the shape must exercise the stride-2 weight-gradient patch kernel"
+    assert wg2_walk(pl, B, Cin, H, Cout, pd[0], oh) == "wg2 ok"
