@@ -15,6 +15,7 @@
 #include "igemm_core.hpp"
 #include "wgrad_patch.hpp"
 #include "wgrad_patch_s2.hpp"
+#include "dgrad_patch_s2.hpp"
 #include "conv_smallc.hpp"
 #include "conv_patch.hpp"
 #include "conv_patch_f64.hpp"
@@ -462,6 +463,12 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
     }
     if (dgrad_small_cin_ok<T>(d)) return dgrad_small_cin<T>(c, g, w, dx, d);
     std::lock_guard<std::mutex> lk(c->launch_mutex);
+    if constexpr (sizeof(T) == 4) {
+        if (!generic_only()) {
+            const dg2::Plan p2 = dg2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
+            if (p2.ok && aligned16(g, w) && aligned16(dx, dx)) return dg2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh);
+        }
+    }
     T* wt = (T*)(ws ? ws : c->get_scratch(need));
     if (!wt) return FX_ERR_OOM;
     if constexpr (sizeof(T) == 4) {

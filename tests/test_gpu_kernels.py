@@ -770,6 +770,10 @@ STRIDED_DGRAD_CASES = [
     (2, 3, 8, 8, 16, (2, 2), (2, 2), (0, 0)), (2, 70, 10, 9, 48, (3, 3), (3, 3), (1, 1)), (1, 8, 12, 12, 16, (5, 5), (2, 2), (2, 2)),
     (2, 4, 1, 9, 16, (3, 3), (2, 2), (1, 1)), (2, 130, 7, 6, 32, (3, 3), (1, 2), (0, 1)), (2, 6, 9, 9, 24, (3, 3), (2, 2), (1, 1)),
     (1, 2, 5, 5, 16, (3, 3), (2, 2), (0, 0)),
+    # stride 2, padding 1, maps 32 and 64 wide: the parity-class patch kernel (one and several tiles per image, channel tiles,
+    # one to eight output-channel chunks)
+    (3, 32, 32, 32, 64, (3, 3), (2, 2), (1, 1)), (2, 64, 32, 32, 128, (3, 3), (2, 2), (1, 1)), (2, 32, 64, 64, 32, (3, 3), (2, 2), (1, 1)),
+    (2, 64, 16, 64, 64, (3, 3), (2, 2), (1, 1)), (2, 32, 32, 32, 48, (3, 3), (2, 2), (1, 1)), (1, 96, 64, 32, 16, (3, 3), (2, 2), (1, 1)),
 ]
 
 

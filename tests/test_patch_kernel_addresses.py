@@ -681,3 +681,91 @@ def test_stride2_weight_gradient_patch_kernel_loads_stay_inside_the_tensors(case
     pl = wg2_plan(B, Cin, H, W, Cout, 3, 3, 2, 2, pd[0], pd[1], oh, ow)
     assert pl is not None, "the shape must exercise the stride-2 weight-gradient patch kernel"
     assert wg2_walk(pl, B, Cin, H, Cout, pd[0], oh) == "wg2 ok"
+
+
+# ---- f32 stride-2 data gradient (dgrad_patch_s2.hpp) ----
+DG2_INSTANCES = [(16, 16), (32, 16)]
+def dg2_plan(B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, oh, ow):
+    if kh != 3 or kw != 3 or sh != 2 or sw != 2 or ph != 1 or pw != 1 or W != 2 * ow or H != 2 * oh or Cin % 32: return None
+    pick = [(o, c) for (o, c) in DG2_INSTANCES if ow == o and Cout % c == 0 and oh % (256 // o) == 0]
+    return dict(OW=pick[0][0], OCC=pick[0][1]) if pick else None
+def dg2_walk(pl, B, Cin, Cout, oh):
+    OW, OCC = pl["OW"], pl["OCC"]
+    NTD, TR, PC = 512, 256 // OW, OW + 1
+    PR = TR + 1; GPL = (PR * PC) | 1; KS = OCC // 2
+    WCH, GCH = KS * 9 * 64, OCC * GPL; BUF = WCH + GCH
+    W4 = OCC * 72; NWP = _ceil_div(W4, NTD); NGP = OCC * 64 // NTD; X4 = OCC * OW // 4
+    assert 2 * BUF * 4 <= 160 * 1024 and OCC * 64 % NTD == 0 and X4 <= NTD
+    L, H, W, tpi, nct = oh * OW, 2 * oh, 2 * OW, oh // TR, Cin // 32
+    gsize, wsize, xsize = B * Cout * L, Cout * Cin * 9, B * Cin * H * W
+    w_written, g_written = set(), set()
+    for blk in sorted({0, 1, nct - 1, nct, B * tpi * nct - 1}):
+        if not 0 <= blk < B * tpi * nct: continue
+        bt, ct = divmod(blk, nct); b, tile = divmod(bt, tpi)
+        c0, i0 = ct * 32, tile * TR
+        next_row = i0 + TR < oh
+        for k in (0, Cout // OCC - 1):
+            oc0 = k * OCC
+            first = blk == 0 and k == 0
+            for tid in range(NTD):
+                for u in range(NWP):
+                    f = u * NTD + tid
+                    ok = f < W4
+                    ocl, q = divmod(f, 72)
+                    a = c0 * 9 + oc0 * Cin * 9 + ((ocl * Cin * 9 + 4 * q) if ok else 0)
+                    assert 0 <= a and a + 4 <= wsize and a % 4 == 0, ("w", a)
+                    if ok and first:
+                        for i in range(4):
+                            c, t = divmod(4 * q + i, 9)
+                            d = ((ocl >> 1) * 9 + t) * 64 + (ocl & 1) * 32 + c
+                            assert 0 <= d < WCH
+                            w_written.add(d)
+                gq, goc = tid & 63, tid >> 6
+                for u in range(NGP):
+                    a = (b * Cout * oh + i0) * OW + (oc0 + 8 * u + goc) * L + 4 * gq
+                    assert 0 <= a and a + 4 <= gsize and a % 4 == 0, ("g", a)
+                    d = (8 * u + goc) * GPL + (gq // (OW // 4)) * PC + (gq % (OW // 4)) * 4
+                    assert d + 4 <= GCH
+                    if first: g_written.update(range(d, d + 4))
+                xoc, xq = divmod(tid, OW // 4)
+                if next_row:
+                    a = (b * Cout * oh + i0) * OW + oc0 * L + ((xoc * L + TR * OW + 4 * xq) if tid < X4 else 0)
+                    assert 0 <= a and a + 4 <= gsize and a % 4 == 0, ("g row", a)
+                if tid < X4:
+                    d = xoc * GPL + TR * PC + 4 * xq
+                    assert d + 4 <= GCH
+                    if first: g_written.update(range(d, d + 4))
+        # stores: the pair of lane (cell, half) for accumulator element e and row class py
+        for wave in range(8):
+            for lane in (0, 15, 16, 31, 32, 63):
+                half, l32 = lane >> 5, lane & 31
+                crow, ccol = divmod(wave * 32 + l32, OW)
+                for e in (0, 15):
+                    c = 8 * (e >> 2) + 4 * half + (e & 3)
+                    for py in range(2):
+                        a = (((b * Cin + c0 + c) * H) + 2 * (i0 + crow) + py) * W + 2 * ccol
+                        assert 0 <= a and a + 2 <= xsize and a % 2 == 0
+                # operand reads: plane of oc = 2 ks + half, rows crow .. crow + 1, columns ccol .. ccol + 1
+                for ks in (0, KS - 1):
+                    d = (2 * ks + half) * GPL + (crow + 1) * PC + ccol + 1
+                    assert d < GCH and crow + 1 < PR and ccol + 1 < PC
+    assert w_written == set(range(WCH))
+    # every patch element that the MFMA loop reads is staged or zeroed: all rows 0 .. TR, columns 0 .. OW - 1 staged, column OW zeroed
+    need = {oc * GPL + r * PC + c for oc in range(OCC) for r in range(PR) for c in range(OW)}
+    assert need <= g_written
+    return "dg2 ok"
+
+
+DG2_SHAPES = [  # B, Cin, H, W, Cout
+    (256, 32, 32, 32, 64), (2, 64, 32, 32, 128), (2, 32, 64, 64, 32), (2, 64, 16, 64, 64), (2, 32, 32, 32, 48), (1, 96, 64, 32, 16),
+]
+
+
+@pytest.mark.parametrize("case", DG2_SHAPES, ids=str)
+def test_stride2_data_gradient_patch_kernel_accesses_stay_inside_the_tensors(case):
+    B, Cin, H, W, Cout = case
+    oh, ow = H // 2, W // 2
+    B = min(B, 3)
+    pl = dg2_plan(B, Cin, H, W, Cout, 3, 3, 2, 2, 1, 1, oh, ow)
+    assert pl is not None, "the shape must exercise the stride-2 data-gradient patch kernel"
+    assert dg2_walk(pl, B, Cin, Cout, oh) == "dg2 ok"
