@@ -317,6 +317,34 @@ template <typename T> struct GlobalAvgPoolFused : Module<T> {
     }
 };
 
+// Flatten as a view: the reshaped tensor aliases its input's memory (the graph keeps the input alive until its clean-up)
+// instead of the copy that Reshape makes (src/ops/reshape.rs:4-55 clones the tensor first).  Same values, no kernel.
+template <typename T> struct ReshapeViewOp : Operator<T> {
+    Shape new_shape;
+    explicit ReshapeViewOp(Shape s) : new_shape(std::move(s)) {}
+    Tensor<T> compute(const TensorRefs<T>& in) const override {
+        Tensor<T> r = HipStorage<T>::borrow(*in[0]);
+        r->reshape(new_shape);
+        return r;
+    }
+    std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
+        g->reshape(in[0]->shape());
+        std::vector<Tensor<T>> r;
+        r.push_back(std::move(g));
+        return r;
+    }
+    size_t num_inputs() const override { return 1; }
+    const char* name() const override { return "ReshapeView"; }
+};
+template <typename T> struct FlattenFused : Module<T> {  // src/nn/layers/pooling.rs:100-140 (batch-first)
+    NodeId forward(AutoFerroxEngine<T>& g, NodeId input) override {
+        const Shape& s = g.get_tensor(input)->shape();
+        size_t rest = 1;
+        for (size_t i = 1; i < s.size(); ++i) rest *= s[i];
+        return g.apply_operation(std::make_unique<ReshapeViewOp<T>>(Shape{s[0], rest}), {input});
+    }
+};
+
 // Dropout with the mask drawn on the device (same stream as the host-built mask of Dropout)
 template <typename T> struct DropoutFusedOp : Operator<T> {
     double p;

@@ -163,7 +163,10 @@ template <typename T> struct Model : ModelBase {
                 if (engine == 1) layers.push_back(std::make_unique<Dropout<T>>(p, seed));
                 else layers.push_back(std::make_unique<DropoutFused<T>>(p, seed));
             } else if (kind == "relu") layers.push_back(std::make_unique<ReLU<T>>());
-            else if (kind == "flatten") layers.push_back(std::make_unique<Flatten<T>>());
+            else if (kind == "flatten") {
+                if (fused) layers.push_back(std::make_unique<FlattenFused<T>>());
+                else layers.push_back(std::make_unique<Flatten<T>>());
+            }
             else throw Error("unknown layer '" + kind + "'");
             for (NodeId p : layers.back()->parameters()) params.push_back(p);
         }
