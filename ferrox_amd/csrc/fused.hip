@@ -249,12 +249,53 @@ __global__ __launch_bounds__(256) void mean_rows_kernel(const T* __restrict__ ro
     if (threadIdx.x == 0) loss[0] = sm[0] * inv;
 }
 
+// Both steps in one block for small problems (up to 1024 rows and 16384 logits): thread t takes rows t, t + 256, ... -- the rows and the order in which
+// mean_rows_kernel's thread t adds them -- and the same tree follows, so the loss has the bits of the two-kernel path.
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_ce_small_kernel(const T* __restrict__ x, const T* __restrict__ y, T* __restrict__ probs,
+                                                               T* __restrict__ loss, i64 B, i64 C, T lo, T hi, T inv) {
+    __shared__ T sm[256];
+    T tot = T(0);
+    for (i64 b = threadIdx.x; b < B; b += 256) {
+        const T* xr = x + b * C;
+        const T* yr = y + b * C;
+        T* pr = probs + b * C;
+        T m = lowest<T>();
+        for (i64 k = 0; k < C; ++k) { const T v = xr[k]; if (v > m) m = v; }
+        T s = T(0);
+        for (i64 k = 0; k < C; ++k) { const T e = dev_exp<T>(xr[k] - m); pr[k] = e; s = s + e; }
+        T acc = T(0);
+        for (i64 k = 0; k < C; ++k) {
+            const T smx = pr[k] / s;
+            pr[k] = smx;
+            T p = smx;
+            if (p < lo) p = lo;
+            if (p > hi) p = hi;
+            acc = acc + yr[k] * dev_log<T>(p);
+        }
+        tot = tot + (-acc);
+    }
+    sm[threadIdx.x] = tot;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) sm[threadIdx.x] = sm[threadIdx.x] + sm[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) loss[0] = sm[0] * inv;
+}
+
 template <typename T>
 int softmax_ce_fwd(fx_ctx* c, const T* logits, const T* targets, T* probs, T* loss, i64 B, i64 C) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(B >= 1 && C >= 1, "fx_softmax_ce_fwd: bad shape");
     FX_REQUIRE(logits && targets && probs && loss, "fx_softmax_ce_fwd: null pointer");
     std::lock_guard<std::mutex> lk(c->launch_mutex);
+    if (B <= 1024 && B * C <= 16384) {  // little work: one launch instead of two
+        softmax_ce_small_kernel<T><<<dim3(1), dim3(256), 0, c->stream>>>(logits, targets, probs, loss, B, C, (T)1e-8, (T)(1.0 - 1e-8),
+                                                                         (T)(1.0 / (double)B));
+        FX_LAUNCH_CHECK();
+        return FX_OK;
+    }
     T* rowloss = (T*)c->get_scratch(B * (i64)sizeof(T));
     if (!rowloss) return FX_ERR_OOM;
     softmax_ce_rows_kernel<T><<<dim3((unsigned)fx::ceil_div(B, (i64)256)), dim3(256), 0, c->stream>>>(
