@@ -5,6 +5,7 @@
 #include <cstdlib>
 
 #include "gemm_lds.hpp"
+#include "gemm_thin.hpp"
 
 extern "C" int fx_bias_act_f32(fx_ctx*, float*, const float*, int64_t, int64_t, int64_t, int);
 extern "C" int fx_bias_act_f64(fx_ctx*, double*, const double*, int64_t, int64_t, int64_t, int);
@@ -71,6 +72,10 @@ int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B,
             const glk::Plan pl = glk::make_plan(c->num_cus, ta != 0, tb != 0, M, N, K, ta ? M : K, tb ? K : N);
             lds_path = pl.ok && !generic_only && fx::aligned16(A) && fx::aligned16(B) && fx::aligned16(C);
             if (lds_path) rc = glk::run(c, pl, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu);
+            else if (!generic_only && gthin::eligible(c->num_cus, ta != 0, tb != 0, M, N, K)) {
+                lds_path = true;
+                rc = gthin::run(c, M, N, K, A, B, C, bias, relu);
+            }
         }
         if (lds_path) {
         } else if (K == 0) {  // empty sum

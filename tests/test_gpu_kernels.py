@@ -336,6 +336,8 @@ GEMM_THIN_SHAPES = [
     ("n", 256, 10, 16384), ("n", 37, 1, 1024), ("n", 130, 16, 2052), ("n", 2050, 7, 1536), ("n", 16, 13, 4096),
     ("k", 256, 16384, 10), ("k", 19, 1028, 1), ("k", 300, 4096, 16), ("k", 17, 2052, 7),
     ("m", 10, 16384, 256), ("m", 1, 1024, 16), ("m", 16, 1028, 1000), ("m", 7, 2052, 33), ("m", 13, 65536, 40),
+    # wide enough for the one-launch thin kernel (f32): ragged N, odd K, K past one round of loads, all 32 rows
+    ("m", 32, 9000, 100), ("m", 7, 8200, 131), ("m", 1, 8192, 33), ("m", 10, 8192, 1000),
 ]
 
 
