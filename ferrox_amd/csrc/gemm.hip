@@ -6,6 +6,7 @@
 
 #include "gemm_lds.hpp"
 #include "gemm_thin.hpp"
+#include "gemm_small.hpp"
 
 extern "C" int fx_bias_act_f32(fx_ctx*, float*, const float*, int64_t, int64_t, int64_t, int);
 extern "C" int fx_bias_act_f64(fx_ctx*, double*, const double*, int64_t, int64_t, int64_t, int);
@@ -75,6 +76,9 @@ int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B,
             else if (!generic_only && gthin::eligible(c->num_cus, ta != 0, tb != 0, M, N, K)) {
                 lds_path = true;
                 rc = gthin::run(c, M, N, K, A, B, C, bias, relu);
+            } else if (!generic_only && gsmall::eligible(c->num_cus, ta != 0, tb != 0, M, N, K, A, B)) {
+                lds_path = true;
+                rc = gsmall::run(c, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu);
             }
         }
         if (lds_path) {

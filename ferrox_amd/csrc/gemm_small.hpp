@@ -1,0 +1,125 @@
+// C[M,N] = op(A) . op(B) for small products (f32) in one launch: the layers of a multilayer perceptron at batch 256
+// (MatMul::compute / MatMul::gradient, src/ops/matrix.rs:17-55, in the three layouts Linear's forward and backward produce).
+//
+// The general tiles give such a product too few blocks to fill the chip unless K is split over blocks, and then a second
+// kernel adds the partial sums: two launches of 5 to 14 us for a few hundred kFLOP per CU.  Here a block (8 waves) owns a
+// 32 x 32 tile of C and splits K over its waves instead: every wave loads its slice of both operands straight from global
+// memory into the MFMA operand registers, all loads of the slice in flight at once, and the eight sums are added through LDS in
+// wave order -- no LDS staging, no partial sums in memory, one launch.
+//
+// Operand registers: a group of 8 consecutive k feeds 4 MFMAs; lane l = (i = l % 32, h = l / 32) holds, for MFMA j of the
+// group, the element with k = 8 g + 4 h + j of row (column) i.  An operand stored k-contiguous gets that as one 16-byte load,
+// one stored row/column-contiguous as four 4-byte loads that run along 128-byte lines.  Both operands use the same assignment,
+// so any mix of layouts works.  Elements past K are zeroed in both operands after the load (their addresses are clamped
+// into the matrix).
+#pragma once
+#include <cstdlib>
+
+#include "igemm_core.hpp"
+
+namespace gsmall {
+using igemm::f32x16;
+
+constexpr int NT = 512, WAVES = 8, MAXG = 16;  // groups of 8 k per wave: K <= 8 * 8 * 16
+
+struct Params {
+    const float* A;
+    const float* B;
+    float* C;
+    const float* bias;  // over n, or null
+    int relu;
+    int M, N, K;
+    int G;  // groups per wave
+};
+
+// KC: the operand is stored [rows][K] (k contiguous, K % 4 == 0, 16-byte aligned); else [K][rows].
+template <bool KC>
+__device__ __forceinline__ void load_group(const float* __restrict__ base, int row, int rows, int K, int k, float (&v)[4]) {
+    if constexpr (KC) {
+        const int kc = min(k, K - 4);
+        const float4 q = *reinterpret_cast<const float4*>(base + (i64)row * K + kc);
+        v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = base[(i64)min(k + j, K - 1) * rows + row];
+    }
+}
+
+template <bool AKC, bool BKC>
+__global__ __launch_bounds__(NT) void small_kernel(const Params p) {
+    __shared__ float red[WAVES * 16 * 64];
+    const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, l32 = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int am = min(m0 + l32, p.M - 1), bn = min(n0 + l32, p.N - 1);  // past the edge: a valid row / column, result unused
+    const int g0 = wave * p.G;
+
+    float a[MAXG][4], b[MAXG][4];
+#pragma unroll
+    for (int g = 0; g < MAXG; ++g) {
+        if (g < p.G) {  // scalar
+            const int k = 8 * (g0 + g) + 4 * h;
+            load_group<AKC>(p.A, am, p.M, p.K, k, a[g]);
+            load_group<BKC>(p.B, bn, p.N, p.K, k, b[g]);
+        }
+    }
+    f32x16 acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+#pragma unroll
+    for (int g = 0; g < MAXG; ++g) {
+        if (g < p.G) {
+            const int k = 8 * (g0 + g) + 4 * h;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool in = k + j < p.K;
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(in ? a[g][j] : 0.f, in ? b[g][j] : 0.f, acc, 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) red[(wave * 16 + e) * 64 + lane] = acc[e];
+    __syncthreads();
+    // wave w finishes accumulator elements 2 w and 2 w + 1: the eight sums in wave order, then the bias kernel's operations
+    const int n = n0 + l32;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const int e = 2 * wave + u;
+        float v = red[e * 64 + lane];
+#pragma unroll
+        for (int q = 1; q < WAVES; ++q) v = v + red[(q * 16 + e) * 64 + lane];
+        const int m = m0 + 8 * (e >> 2) + 4 * h + (e & 3);
+        if (m < p.M && n < p.N) {
+            if (p.bias) {
+                v = v + p.bias[n];
+                if (p.relu) v = v > 0.f ? v : 0.f;
+            }
+            p.C[(i64)m * p.N + n] = v;
+        }
+    }
+}
+
+// A is k-contiguous unless ta, B is k-contiguous when tb.
+inline bool eligible(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, const float* A, const float* B) {
+    static const bool off = [] { const char* v = getenv("FX_GEMM_SMALL"); return v && atoi(v) == 0; }();
+    if (off || K < 32 || K > 8 * WAVES * MAXG || M < 1 || N < 1) return false;
+    if (!ta && (K % 4 != 0 || !fx::aligned16(A))) return false;
+    if (tb && (K % 4 != 0 || !fx::aligned16(B))) return false;
+    const i64 blocks = fx::ceil_div(M, (i64)32) * fx::ceil_div(N, (i64)32);
+    // a 32 x 32 tile re-reads each operand once per tile row / column: M N K / 4 bytes through L2, kept under 32 MB
+    return blocks <= 2 * (i64)num_cus && M * N * K <= (1ll << 27);
+}
+
+inline int run(fx_ctx* c, bool ta, bool tb, i64 M, i64 N, i64 K, const float* A, const float* B, float* C, const float* bias, int relu) {
+    Params p{A, B, C, bias, relu, (int)M, (int)N, (int)K, 0};
+    p.G = (int)fx::ceil_div(fx::ceil_div(K, (i64)8), (i64)WAVES);
+    const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32));
+    if (!ta && !tb) small_kernel<true, false><<<grid, dim3(NT), 0, c->stream>>>(p);
+    else if (!ta && tb) small_kernel<true, true><<<grid, dim3(NT), 0, c->stream>>>(p);
+    else if (ta && !tb) small_kernel<false, false><<<grid, dim3(NT), 0, c->stream>>>(p);
+    else small_kernel<false, true><<<grid, dim3(NT), 0, c->stream>>>(p);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+}  // namespace gsmall
