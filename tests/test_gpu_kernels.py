@@ -367,6 +367,48 @@ def test_gemm_with_one_thin_dimension(ctx, dtype):
         assert np.array_equal(fused.numpy(), got.numpy()), (kind, M, N, K)
 
 
+# small f32 products take a one-launch kernel (32 x 32 tile per block, K split over the block's waves): every layout, ragged
+# tile edges, K with half a group of eight left over, the longest K it takes, and K not a multiple of 4 for each layout (only the
+# row/column-contiguous loads take that; the others fall back to the general tiles)
+GEMM_SMALL_SHAPES = [(33, 65, 36), (256, 512, 784), (100, 31, 1024), (1, 1, 32), (64, 64, 44), (32, 96, 250), (70, 200, 127)]
+
+
+def test_gemm_small_products_all_layouts(ctx):
+    from ferrox_amd import capi
+    rng = np.random.default_rng(47)
+    tol = TOL[np.dtype(np.float32)]
+    for (M, N, K) in GEMM_SMALL_SHAPES:
+        a = rng.standard_normal((M, K)).astype(np.float32)
+        b = rng.standard_normal((K, N)).astype(np.float32)
+        truth = a.astype(np.float64) @ b.astype(np.float64)
+        scale = (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)).max()
+        bias = rng.standard_normal(N).astype(np.float32)
+        dbias = ctx.upload(bias)
+        for ta in (False, True):
+            for tb in (False, True):
+                da = ctx.upload(np.ascontiguousarray(a.T) if ta else a)
+                db = ctx.upload(np.ascontiguousarray(b.T) if tb else b)
+                got = ctx.gemm(da, db, ta, tb)
+                case = (M, N, K, ta, tb)
+                assert np.abs(got.numpy() - truth).max() <= tol * scale, case
+                assert np.array_equal(ctx.gemm(da, db, ta, tb).numpy(), got.numpy()), case
+                fused = ctx.empty((M, N), np.float32)
+                capi.check(capi.lib.fx_gemm_bias_act_f32(ctx.h, int(ta), int(tb), M, N, K, da.ptr, db.ptr, dbias.ptr, fused.ptr, 1))
+                ctx.bias_act(got, dbias, M, N, 1, act=1)
+                assert np.array_equal(fused.numpy(), got.numpy()), case
+    # an infinity in the last row of K must not leak into other outputs through the clamped re-reads past K
+    M, N, K = 40, 40, 36
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    b = rng.standard_normal((K, N)).astype(np.float32)
+    b[K - 1, 3] = np.inf
+    a[5, K - 1] = 0.0
+    got = ctx.gemm(ctx.upload(np.ascontiguousarray(a.T)), ctx.upload(b), True, False).numpy()
+    with np.errstate(invalid="ignore"):
+        ref = a.astype(np.float64) @ b.astype(np.float64)
+    assert np.isnan(got[5, 3]) and np.isnan(ref[5, 3])
+    assert np.array_equal(np.isinf(got), np.isinf(ref)) and np.array_equal(np.isnan(got), np.isnan(ref))
+
+
 def test_gemm_shape_mismatch_message(ctx):
     from ferrox_amd.capi import FerroxHipError
     a = ctx.upload(np.zeros((2, 3), np.float32))
