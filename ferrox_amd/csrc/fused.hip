@@ -256,6 +256,38 @@ __global__ __launch_bounds__(256) void softmax_ce_small_kernel(const T* __restri
                                                                T* __restrict__ loss, i64 B, i64 C, T lo, T hi, T inv) {
     __shared__ T sm[256];
     T tot = T(0);
+    if (C <= 16) {
+        // a row fits the registers: all of its loads are in flight together instead of one dependent access after the other
+        // (the arithmetic and its order are those of the general loop below)
+        const int c = (int)C;
+        for (i64 b = threadIdx.x; b < B; b += 256) {
+            T xv[16], yv[16], pv[16];
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {
+                xv[k] = k < c ? x[b * C + k] : T(0);
+                yv[k] = k < c ? y[b * C + k] : T(0);
+            }
+            T m = lowest<T>();
+#pragma unroll
+            for (int k = 0; k < 16; ++k) if (k < c && xv[k] > m) m = xv[k];
+            T s = T(0);
+#pragma unroll
+            for (int k = 0; k < 16; ++k) if (k < c) { pv[k] = dev_exp<T>(xv[k] - m); s = s + pv[k]; }
+            T acc = T(0);
+#pragma unroll
+            for (int k = 0; k < 16; ++k) if (k < c) {
+                const T smx = pv[k] / s;
+                pv[k] = smx;
+                T p = smx;
+                if (p < lo) p = lo;
+                if (p > hi) p = hi;
+                acc = acc + yv[k] * dev_log<T>(p);
+            }
+#pragma unroll
+            for (int k = 0; k < 16; ++k) if (k < c) probs[b * C + k] = pv[k];
+            tot = tot + (-acc);
+        }
+    } else
     for (i64 b = threadIdx.x; b < B; b += 256) {
         const T* xr = x + b * C;
         const T* yr = y + b * C;
@@ -319,6 +351,29 @@ __global__ __launch_bounds__(256) void softmax_ce_bwd_kernel(const T* __restrict
     T* dr = dx + b * C;
     const T dtl = -(gup[0] * inv);
     T dot = T(0);
+    if (C <= 16) {  // the row in registers, loads in flight together; same arithmetic in the same order as below
+        const int c = (int)C;
+        T sv[16], yv[16], dv[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            sv[k] = k < c ? sr[k] : T(0);
+            yv[k] = k < c ? yr[k] : T(0);
+        }
+#pragma unroll
+        for (int k = 0; k < 16; ++k) if (k < c) {
+            const T s = sv[k];
+            T p = s;
+            if (p < lo) p = lo;
+            if (p > hi) p = hi;
+            const T dp = (dtl * yv[k]) / p;
+            const T ds = (dp * (s >= lo ? T(1) : T(0))) * (s <= hi ? T(1) : T(0));
+            dv[k] = ds;
+            dot = dot + ds * s;
+        }
+#pragma unroll
+        for (int k = 0; k < 16; ++k) if (k < c) dr[k] = sv[k] * (dv[k] - dot);
+        return;
+    }
     for (i64 k = 0; k < C; ++k) {
         const T s = sr[k];
         T p = s;
