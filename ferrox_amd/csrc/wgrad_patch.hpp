@@ -564,9 +564,14 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
     FX_LAUNCH_CHECK();
     const int n = (int)p.part_stride;
     const FastDiv div_row((uint32_t)(KK * Cin)), div_cin((uint32_t)Cin);
-    // measured: with 256 partials of 73 728 outputs the single chain per output is the faster one (0.095 vs 0.106 ms for the
-    // whole pass at [64,128,28,28] -> 64); with 1024 partials of 18 432 outputs the grouped sum wins (0.118 vs 0.141 ms)
-    if (pl.partials() >= 512 && n <= (1 << 17))
+    // the two 4-byte kernels serve partial sums that are not 16-byte addressable; between them, measured: with 256 partials of
+    // 73 728 outputs the single chain per output is the faster one (0.095 vs 0.106 ms for the whole pass at [64,128,28,28] -> 64),
+    // with 1024 partials of 18 432 outputs the grouped sum wins (0.118 vs 0.141 ms)
+    // measured: the 16-byte grouped sum beats both kernels below wherever it applies (0.4845 -> 0.4786 ms for the whole pass at
+    // [128,64,56,56] -> 128 with 256 partials, 0.1996 -> 0.188 ms at [256,64,32,32] -> 64)
+    if (n % 4 == 0 && Cin % 4 == 0 && fx::aligned16(part)) {
+        wgrad_patch_reduce_vec_kernel<16><<<dim3((unsigned)fx::ceil_div((i64)n, 64)), dim3(256), 0, c->stream>>>(part, dw, n, pl.partials(), (int)Cin, div_row, div_cin);
+    } else if (pl.partials() >= 512 && n <= (1 << 17))
         wgrad_patch_reduce_grouped_kernel<16><<<dim3((unsigned)fx::ceil_div((i64)n, 16)), dim3(256), 0, c->stream>>>(part, dw, n, pl.partials(), (int)Cin, div_row, div_cin);
     else
         wgrad_patch_reduce_kernel<<<dim3((unsigned)fx::ceil_div((i64)n, 256)), dim3(256), 0, c->stream>>>(part, dw, n, pl.partials(), (int)Cin, div_row, div_cin);
