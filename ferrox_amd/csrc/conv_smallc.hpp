@@ -37,6 +37,7 @@ struct FwdParams {
     float* y;
     const float* bias;
     int relu;
+    int ntiles;  // B * tiles per image
     Geometry g;
 };
 
@@ -72,18 +73,20 @@ __device__ __forceinline__ int tap_offset(const Geometry& g, int k) {
     return c * g.PLANE + ky * g.PW + kx;
 }
 
-// KS = ceil(Cin * 9 / 2) MFMA steps.  grid = (B * tiles per image, ceil(Cout / 32)).
+// KS = ceil(Cin * 9 / 2) MFMA steps.  grid = (blocks, ceil(Cout / 32)); block x takes the (image, tile) pairs x, x + blocks, ...
+// The patch of the next pair is loaded into registers before the MFMAs and stores of the current one (at most NPV float4 per
+// thread), so a block's loads, MFMAs and stores overlap from its second tile on.
+constexpr int NPV = 4;
 template <int KS, bool BIAS>
 __global__ __launch_bounds__(NT) void fwd_kernel(const FwdParams p) {
     extern __shared__ __align__(16) float patch[];
     const Geometry& g = p.g;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
-    const int b = (int)g.div_tpi.div(blockIdx.x), tile = (int)blockIdx.x - b * g.tpi;
+    const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int m0 = blockIdx.y * 32;
     const int L = g.OH * g.OW, K = g.C * KK;
-    const int pix0 = tile * NPIX, py0 = (int)g.div_ow.div((uint32_t)pix0), iy0 = py0 * g.sh - g.ph;
 
-    // the weight loads are in flight while the patch is staged; they are first used after the second barrier
+    // the weight loads are in flight while the first patch is staged; they are first used after the second barrier
     float wraw[KS];
     int koff[KS];
     const bool m_ok = m0 + l32 < g.Cout;
@@ -94,38 +97,79 @@ __global__ __launch_bounds__(NT) void fwd_kernel(const FwdParams p) {
         wraw[s] = wrow[k < K ? k : 0];
         koff[s] = tap_offset(g, k);
     }
-    for (int i = tid; i < g.C * g.PLANE; i += NT) patch[i] = 0.f;
-    __syncthreads();
-    stage_patch(g, p.x, patch, b, iy0, tid);
-    __syncthreads();
+    // per-thread constants of the staging: patch items tid + NT v (see stage_patch for the item -> (channel, row, vector) map)
+    const int W4 = (g.W + 3) >> 2, items = g.C * g.PR * W4;
+    int p_src[NPV], p_dst[NPV], p_row[NPV];
+#pragma unroll
+    for (int v = 0; v < NPV; ++v) {
+        const int i = min(tid + v * NT, items - 1);
+        const int rc = (int)g.div_w4.div((uint32_t)i), q = min(4 * (i - rc * W4), g.W - 4);
+        const int c = (int)g.div_pr.div((uint32_t)rc), r = rc - c * g.PR;
+        p_src[v] = c * g.H * g.W + q;
+        p_dst[v] = c * g.PLANE + r * g.PW + g.pw + q;
+        p_row[v] = r;
+    }
+    float4 pv[NPV];
+    auto prefetch = [&](int t) __attribute__((always_inline)) {
+        const int b = (int)g.div_tpi.div((uint32_t)t), tile = t - b * g.tpi;
+        const int iy0 = (int)g.div_ow.div((uint32_t)(tile * NPIX)) * g.sh - g.ph;
+#pragma unroll
+        for (int v = 0; v < NPV; ++v) {
+            if (v * NT >= items) break;  // block-uniform
+            const int iy = iy0 + p_row[v];
+            const bool ok = iy >= 0 && iy < g.H;
+            pv[v] = *reinterpret_cast<const float4*>(p.x + (i64)b * g.C * g.H * g.W + p_src[v] + (ok ? iy : 0) * g.W);
+            if (!ok) pv[v] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    const int ntiles = p.ntiles;
+    int t = blockIdx.x;
+    if (t < ntiles) prefetch(t);
+    for (int i = tid; i < g.C * g.PLANE; i += NT) patch[i] = 0.f;  // the padding columns stay zero from here on
     float wreg[KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) wreg[s] = m_ok && 2 * s + half < K ? wraw[s] : 0.f;
 
-    float* yb = p.y + (i64)b * g.Cout * L;
+    for (; t < ntiles; t += gridDim.x) {
+        const int b = (int)g.div_tpi.div((uint32_t)t), tile = t - b * g.tpi;
+        const int pix0 = tile * NPIX, py0 = (int)g.div_ow.div((uint32_t)pix0);
+        __syncthreads();  // the previous tile's reads are done (and the zero fill before the first)
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk) {
-        const int pbase = pix0 + (wave * 2 + blk) * 32;
-        if (pbase >= L) break;  // wave-uniform
-        const int pp = pbase + l32, pc = min(pp, L - 1);
-        const int oy = (int)g.div_ow.div((uint32_t)pc), ox = pc - oy * g.OW;
-        const float* src = patch + (oy - py0) * g.sh * g.PW + ox * g.sw;
-        f32x16 acc;
+        for (int v = 0; v < NPV; ++v) {
+            if (v * NT >= items) break;
+            if (tid + v * NT < items) {
+                float* d = patch + p_dst[v];
+                d[0] = pv[v].x; d[1] = pv[v].y; d[2] = pv[v].z; d[3] = pv[v].w;
+            }
+        }
+        __syncthreads();
+        if (t + (int)gridDim.x < ntiles) prefetch(t + gridDim.x);
+
+        float* yb = p.y + (i64)b * g.Cout * L;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+        for (int blk = 0; blk < 2; ++blk) {
+            const int pbase = pix0 + (wave * 2 + blk) * 32;
+            if (pbase >= L) break;  // wave-uniform
+            const int pp = pbase + l32, pc = min(pp, L - 1);
+            const int oy = (int)g.div_ow.div((uint32_t)pc), ox = pc - oy * g.OW;
+            const float* src = patch + (oy - py0) * g.sh * g.PW + ox * g.sw;
+            f32x16 acc;
 #pragma unroll
-        for (int s = 0; s < KS; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wreg[s], src[koff[s]], acc, 0, 0, 0);
-        if (pp < L) {
+            for (int e = 0; e < 16; ++e) acc[e] = 0.f;
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int ch = m0 + igemm::Mfma<float>::row(e, lane);
-                if (ch < g.Cout) {
-                    float v = acc[e];
-                    if constexpr (BIAS) {
-                        v += p.bias[ch];
-                        if (p.relu) v = v > 0.f ? v : 0.f;
+            for (int s = 0; s < KS; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wreg[s], src[koff[s]], acc, 0, 0, 0);
+            if (pp < L) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int ch = m0 + igemm::Mfma<float>::row(e, lane);
+                    if (ch < g.Cout) {
+                        float v = acc[e];
+                        if constexpr (BIAS) {
+                            v += p.bias[ch];
+                            if (p.relu) v = v > 0.f ? v : 0.f;
+                        }
+                        yb[(i64)ch * L + pp] = v;
                     }
-                    yb[(i64)ch * L + pp] = v;
                 }
             }
         }
@@ -213,6 +257,7 @@ inline Plan make_plan(int num_cus, bool wgrad, i64 B, i64 C, i64 H, i64 W, i64 C
     pl.tpi = (int)fx::ceil_div(L, (i64)NPIX);
     pl.smem = ((size_t)C * pl.PLANE + (wgrad ? (size_t)32 * GP : 0)) * sizeof(float);
     if (pl.smem > LDS_LIMIT || B * pl.tpi > 0x7fffffff) return pl;
+    if (!wgrad && C * pl.PR * ((W + 3) / 4) > NPV * NT) return pl;  // the patch items one thread keeps in flight
     if (wgrad) {
         pl.stages = (int)(B * pl.tpi);
         const i64 mblocks = fx::ceil_div(Cout, (i64)32);
@@ -245,7 +290,14 @@ inline int run_fwd(fx_ctx* c, const Plan& pl, const float* x, const float* w, fl
     FwdParams p;
     p.x = x; p.w = w; p.y = y; p.bias = bias; p.relu = relu;
     p.g = make_geometry(pl, C, H, W, Cout, OH, OW, sh, sw, ph, pw);
-    const dim3 grid((unsigned)(B * pl.tpi), (unsigned)fx::ceil_div(Cout, (i64)32));
+    p.ntiles = (int)(B * pl.tpi);
+    // two blocks per CU for every row of 32 output channels, every block with the same number of tiles (measured at
+    // [256,3,32,32]: -> 32 13.9 us one tile per block, 14.0 / 12.7 / 13.6 us at one / two / four blocks per CU; -> 64 20.9 one tile
+    // per block, 21.2 / 20.7 at two / four blocks per CU over both rows)
+    const i64 mblocks = fx::ceil_div(Cout, (i64)32);
+    const i64 want = std::max<i64>(1, 2 * (i64)c->num_cus);
+    const i64 per_block = fx::ceil_div((i64)p.ntiles, want);
+    const dim3 grid((unsigned)fx::ceil_div((i64)p.ntiles, per_block), (unsigned)mblocks);
 #define FX_CSC_FWD(KSV)                                                                                 \
     do {                                                                                                \
         if (bias) fwd_kernel<KSV, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                     \

@@ -287,6 +287,7 @@ def smallc_plan(wgrad, B, C, H, W, Cout, sh, sw, ph, pw, OH, OW, num_cus=256):
     if OW > 64 or PR * OW > 2 * SC_NPIX * sh: return None
     pl = dict(PR=PR, PW=PW, PLANE=PR * PW, tpi=_ceil_div(L, SC_NPIX))
     if (C * pl["PLANE"] + (32 * SC_GP if wgrad else 0)) * 4 > 60 * 1024: return None
+    if not wgrad and C * PR * ((W + 3) // 4) > 4 * 256: return None   # the patch items a thread of the forward kernel keeps in flight
     if wgrad:
         stages, mblocks = B * pl["tpi"], _ceil_div(Cout, 32)
         splits = max(1, min(stages, 4 * num_cus // mblocks))
