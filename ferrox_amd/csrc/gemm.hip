@@ -81,6 +81,13 @@ int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B,
                 rc = gsmall::run(c, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu);
             }
         }
+        if constexpr (sizeof(T) == 8) {
+            static const bool generic_only = std::getenv("FX_GEMM_GENERIC") != nullptr;
+            if (!generic_only && gsmall::eligible_f64(c->num_cus, ta != 0, tb != 0, M, N, K, A, B)) {
+                lds_path = true;
+                rc = gsmall::run_f64(c, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu);
+            }
+        }
         if (lds_path) {
         } else if (K == 0) {  // empty sum
             rc = launch_zero<T>(c, C, M * N);

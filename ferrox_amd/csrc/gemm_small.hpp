@@ -99,6 +99,128 @@ __global__ __launch_bounds__(NT) void small_kernel(const Params p) {
     }
 }
 
+// ---- f64 twin on v_mfma_f64_16x16x4_f64 -------------------------------------------------------------------------------------
+// The 32 x 32 tile is 2 x 2 MFMA blocks of 16 x 16; a group of 8 consecutive k feeds 2 MFMA steps of 4 k each.  Lane
+// l = (i = l % 16, q = l / 16) holds, for step j of the group, the element with k = 8 g + 2 q + j of rows (columns) i and i + 16:
+// one 16-byte load per row for a k-contiguous operand, two 8-byte loads along 128-byte lines otherwise.  A wave keeps at most
+// MAXG_D groups in flight (128 registers) and walks its slice of K in batches of that size.
+using igemm::f64x4;
+constexpr int MAXG_D = 8;
+
+struct ParamsD {
+    const double* A;
+    const double* B;
+    double* C;
+    const double* bias;
+    int relu;
+    int M, N, K;
+    int G;  // groups per wave
+};
+
+template <bool KC>
+__device__ __forceinline__ void load_group_d(const double* __restrict__ base, int row, int rows, int K, int k, double (&v)[2]) {
+    if constexpr (KC) {
+        typedef double d2 __attribute__((ext_vector_type(2)));
+        const d2 q = *reinterpret_cast<const d2*>(base + (i64)row * K + min(k, K - 2));
+        v[0] = q.x; v[1] = q.y;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) v[j] = base[(i64)min(k + j, K - 1) * rows + row];
+    }
+}
+
+template <bool AKC, bool BKC>
+__global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
+    extern __shared__ __align__(16) double red_d[];  // [8 waves][16 elements][64 lanes]
+    const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, l16 = lane & 15;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int am0 = min(m0 + l16, p.M - 1), am1 = min(m0 + 16 + l16, p.M - 1);  // past the edge: a valid row / column, result unused
+    const int bn0 = min(n0 + l16, p.N - 1), bn1 = min(n0 + 16 + l16, p.N - 1);
+    const int g0 = wave * p.G;
+    f64x4 acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[a][b][e] = 0.;
+    for (int gb = 0; gb < p.G; gb += MAXG_D) {  // scalar loop: batches of MAXG_D groups
+        double a0[MAXG_D][2], a1[MAXG_D][2], b0[MAXG_D][2], b1[MAXG_D][2];
+#pragma unroll
+        for (int g = 0; g < MAXG_D; ++g) {
+            if (gb + g < p.G) {
+                const int k = 8 * (g0 + gb + g) + 2 * q;
+                load_group_d<AKC>(p.A, am0, p.M, p.K, k, a0[g]);
+                load_group_d<AKC>(p.A, am1, p.M, p.K, k, a1[g]);
+                load_group_d<BKC>(p.B, bn0, p.N, p.K, k, b0[g]);
+                load_group_d<BKC>(p.B, bn1, p.N, p.K, k, b1[g]);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < MAXG_D; ++g) {
+            if (gb + g < p.G) {
+                const int k = 8 * (g0 + gb + g) + 2 * q;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const bool in = k + j < p.K;  // past K: zeros in both operands, whatever the clamped loads returned
+                    const double x0 = in ? a0[g][j] : 0., x1 = in ? a1[g][j] : 0., y0 = in ? b0[g][j] : 0., y1 = in ? b1[g][j] : 0.;
+                    acc[0][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(x0, y0, acc[0][0], 0, 0, 0);
+                    acc[0][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(x0, y1, acc[0][1], 0, 0, 0);
+                    acc[1][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(x1, y0, acc[1][0], 0, 0, 0);
+                    acc[1][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(x1, y1, acc[1][1], 0, 0, 0);
+                }
+            }
+        }
+    }
+    // element index 4 (2 a + b) + e of lane l is C[m0 + 16 a + 4 e + l / 16][n0 + 16 b + l % 16]
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) red_d[(wave * 16 + 4 * (2 * a + b) + e) * 64 + lane] = acc[a][b][e];
+    __syncthreads();
+    // wave w finishes elements 2 w and 2 w + 1: the eight sums in wave order, then the bias kernel's operations
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const int el = 2 * wave + u, blk = el >> 2, e = el & 3;
+        double v = red_d[el * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) v = v + red_d[(w * 16 + el) * 64 + lane];
+        const int m = m0 + 16 * (blk >> 1) + 4 * e + q, n = n0 + 16 * (blk & 1) + l16;
+        if (m < p.M && n < p.N) {
+            if (p.bias) {
+                v = v + p.bias[n];
+                if (p.relu) v = v > 0. ? v : 0.;
+            }
+            p.C[(i64)m * p.N + n] = v;
+        }
+    }
+}
+
+inline bool eligible_f64(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, const double* A, const double* B) {
+    static const bool off = [] { const char* v = getenv("FX_GEMM_SMALL"); return v && atoi(v) == 0; }();
+    if (off || K < 32 || K > 8 * WAVES * MAXG || M < 1 || N < 1) return false;
+    if (!ta && (K % 2 != 0 || !fx::aligned16(A))) return false;
+    if (tb && (K % 2 != 0 || !fx::aligned16(B))) return false;
+    const i64 blocks = fx::ceil_div(M, (i64)32) * fx::ceil_div(N, (i64)32);
+    return blocks <= 2 * (i64)num_cus && M * N * K <= (1ll << 27);  // M N K / 2 bytes through L2, under 64 MB
+}
+
+inline int run_f64(fx_ctx* c, bool ta, bool tb, i64 M, i64 N, i64 K, const double* A, const double* B, double* C, const double* bias, int relu) {
+    ParamsD p{A, B, C, bias, relu, (int)M, (int)N, (int)K, 0};
+    p.G = (int)fx::ceil_div(fx::ceil_div(K, (i64)8), (i64)WAVES);
+    const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32));
+    const size_t lds = (size_t)WAVES * 16 * 64 * sizeof(double);
+    if (!ta && !tb) small_kernel_f64<true, false><<<grid, dim3(NT), lds, c->stream>>>(p);
+    else if (!ta && tb) small_kernel_f64<true, true><<<grid, dim3(NT), lds, c->stream>>>(p);
+    else if (ta && !tb) small_kernel_f64<false, false><<<grid, dim3(NT), lds, c->stream>>>(p);
+    else small_kernel_f64<false, true><<<grid, dim3(NT), lds, c->stream>>>(p);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
 // A is k-contiguous unless ta, B is k-contiguous when tb.
 inline bool eligible(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, const float* A, const float* B) {
     static const bool off = [] { const char* v = getenv("FX_GEMM_SMALL"); return v && atoi(v) == 0; }();

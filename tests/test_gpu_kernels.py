@@ -367,22 +367,24 @@ def test_gemm_with_one_thin_dimension(ctx, dtype):
         assert np.array_equal(fused.numpy(), got.numpy()), (kind, M, N, K)
 
 
-# small f32 products take a one-launch kernel (32 x 32 tile per block, K split over the block's waves): every layout, ragged
+# small products take a one-launch kernel (32 x 32 tile per block, K split over the block's waves): every layout, ragged
 # tile edges, K with half a group of eight left over, the longest K it takes, and K not a multiple of 4 for each layout (only the
 # row/column-contiguous loads take that; the others fall back to the general tiles)
 GEMM_SMALL_SHAPES = [(33, 65, 36), (256, 512, 784), (100, 31, 1024), (1, 1, 32), (64, 64, 44), (32, 96, 250), (70, 200, 127)]
 
 
-def test_gemm_small_products_all_layouts(ctx):
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_small_products_all_layouts(ctx, dtype):
     from ferrox_amd import capi
     rng = np.random.default_rng(47)
-    tol = TOL[np.dtype(np.float32)]
+    tol = TOL[np.dtype(dtype)]
+    sfx = "f32" if dtype == np.float32 else "f64"
     for (M, N, K) in GEMM_SMALL_SHAPES:
-        a = rng.standard_normal((M, K)).astype(np.float32)
-        b = rng.standard_normal((K, N)).astype(np.float32)
+        a = rng.standard_normal((M, K)).astype(dtype)
+        b = rng.standard_normal((K, N)).astype(dtype)
         truth = a.astype(np.float64) @ b.astype(np.float64)
         scale = (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)).max()
-        bias = rng.standard_normal(N).astype(np.float32)
+        bias = rng.standard_normal(N).astype(dtype)
         dbias = ctx.upload(bias)
         for ta in (False, True):
             for tb in (False, True):
@@ -392,14 +394,14 @@ def test_gemm_small_products_all_layouts(ctx):
                 case = (M, N, K, ta, tb)
                 assert np.abs(got.numpy() - truth).max() <= tol * scale, case
                 assert np.array_equal(ctx.gemm(da, db, ta, tb).numpy(), got.numpy()), case
-                fused = ctx.empty((M, N), np.float32)
-                capi.check(capi.lib.fx_gemm_bias_act_f32(ctx.h, int(ta), int(tb), M, N, K, da.ptr, db.ptr, dbias.ptr, fused.ptr, 1))
+                fused = ctx.empty((M, N), dtype)
+                capi.check(getattr(capi.lib, "fx_gemm_bias_act_" + sfx)(ctx.h, int(ta), int(tb), M, N, K, da.ptr, db.ptr, dbias.ptr, fused.ptr, 1))
                 ctx.bias_act(got, dbias, M, N, 1, act=1)
                 assert np.array_equal(fused.numpy(), got.numpy()), case
     # an infinity in the last row of K must not leak into other outputs through the clamped re-reads past K
     M, N, K = 40, 40, 36
-    a = rng.standard_normal((M, K)).astype(np.float32)
-    b = rng.standard_normal((K, N)).astype(np.float32)
+    a = rng.standard_normal((M, K)).astype(dtype)
+    b = rng.standard_normal((K, N)).astype(dtype)
     b[K - 1, 3] = np.inf
     a[5, K - 1] = 0.0
     got = ctx.gemm(ctx.upload(np.ascontiguousarray(a.T)), ctx.upload(b), True, False).numpy()
