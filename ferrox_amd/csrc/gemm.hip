@@ -54,6 +54,26 @@ int run_trans(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const 
     return run<T, Cfg, true, true>(c, M, N, K, A, B, C, bias, relu, pend);
 }
 
+// the one-launch small-product kernel; with K split over blocks, its partial results and their ordered sum (bias and ReLU in the sum's store)
+int small_launch(fx_ctx* c, const gsmall::Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K, const float* A, const float* B, float* C, const float* bias,
+                 int relu, float* part) {
+    return gsmall::run(c, pl, ta, tb, M, N, K, A, B, C, bias, relu, part);
+}
+int small_launch(fx_ctx* c, const gsmall::Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K, const double* A, const double* B, double* C,
+                 const double* bias, int relu, double* part) {
+    return gsmall::run_f64(c, pl, ta, tb, M, N, K, A, B, C, bias, relu, part);
+}
+template <typename T>
+int small_product(fx_ctx* c, const gsmall::Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K, const T* A, const T* B, T* C, const T* bias, int relu) {
+    T* part = nullptr;
+    if (pl.splits > 1) {
+        part = (T*)c->get_scratch(gsmall::workspace_bytes<T>(pl, M, N));
+        if (!part) return FX_ERR_OOM;
+    }
+    if (int rc = small_launch(c, pl, ta, tb, M, N, K, A, B, C, bias, relu, part)) return rc;
+    return pl.splits > 1 ? launch_splitk_reduce<T>(c, part, C, M * N, pl.splits, bias, N, relu) : FX_OK;
+}
+
 template <typename T>
 int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B, T* C, const T* bias = nullptr, int relu = 0) {
     FX_CHECK_CTX(c);
@@ -76,16 +96,22 @@ int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B,
             else if (!generic_only && gthin::eligible(c->num_cus, ta != 0, tb != 0, M, N, K)) {
                 lds_path = true;
                 rc = gthin::run(c, M, N, K, A, B, C, bias, relu);
-            } else if (!generic_only && gsmall::eligible(c->num_cus, ta != 0, tb != 0, M, N, K, A, B)) {
-                lds_path = true;
-                rc = gsmall::run(c, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu);
+            } else if (!generic_only) {
+                const gsmall::Plan sp = gsmall::make_plan<float>(c->num_cus, ta != 0, tb != 0, M, N, K, A, B);
+                if (sp.ok) {
+                    lds_path = true;
+                    rc = small_product<float>(c, sp, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu);
+                }
             }
         }
         if constexpr (sizeof(T) == 8) {
             static const bool generic_only = std::getenv("FX_GEMM_GENERIC") != nullptr;
-            if (!generic_only && gsmall::eligible_f64(c->num_cus, ta != 0, tb != 0, M, N, K, A, B)) {
-                lds_path = true;
-                rc = gsmall::run_f64(c, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu);
+            if (!generic_only) {
+                const gsmall::Plan sp = gsmall::make_plan<double>(c->num_cus, ta != 0, tb != 0, M, N, K, A, B);
+                if (sp.ok) {
+                    lds_path = true;
+                    rc = small_product<double>(c, sp, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu);
+                }
             }
         }
         if (lds_path) {

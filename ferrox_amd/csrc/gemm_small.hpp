@@ -29,7 +29,9 @@ struct Params {
     const float* bias;  // over n, or null
     int relu;
     int M, N, K;
-    int G;  // groups per wave
+    int G;       // groups per wave
+    int kz;      // K per block when the grid's z dimension splits K (a multiple of 8 * WAVES * G ... see run), else K
+    i64 zstride; // elements between the partial results of consecutive z (0 when K is not split)
 };
 
 // KC: the operand is stored [rows][K] (k contiguous, K % 4 == 0, 16-byte aligned); else [K][rows].
@@ -52,13 +54,14 @@ __global__ __launch_bounds__(NT) void small_kernel(const Params p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
     const int am = min(m0 + l32, p.M - 1), bn = min(n0 + l32, p.N - 1);  // past the edge: a valid row / column, result unused
+    const int kbase = blockIdx.z * p.kz, kend = min(p.K, kbase + p.kz);    // this block's range of K (all of it unless K is split over z)
     const int g0 = wave * p.G;
 
     float a[MAXG][4], b[MAXG][4];
 #pragma unroll
     for (int g = 0; g < MAXG; ++g) {
         if (g < p.G) {  // scalar
-            const int k = 8 * (g0 + g) + 4 * h;
+            const int k = kbase + 8 * (g0 + g) + 4 * h;
             load_group<AKC>(p.A, am, p.M, p.K, k, a[g]);
             load_group<BKC>(p.B, bn, p.N, p.K, k, b[g]);
         }
@@ -69,10 +72,10 @@ __global__ __launch_bounds__(NT) void small_kernel(const Params p) {
 #pragma unroll
     for (int g = 0; g < MAXG; ++g) {
         if (g < p.G) {
-            const int k = 8 * (g0 + g) + 4 * h;
+            const int k = kbase + 8 * (g0 + g) + 4 * h;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const bool in = k + j < p.K;
+                const bool in = k + j < kend;
                 acc = __builtin_amdgcn_mfma_f32_32x32x2f32(in ? a[g][j] : 0.f, in ? b[g][j] : 0.f, acc, 0, 0, 0);
             }
         }
@@ -94,7 +97,7 @@ __global__ __launch_bounds__(NT) void small_kernel(const Params p) {
                 v = v + p.bias[n];
                 if (p.relu) v = v > 0.f ? v : 0.f;
             }
-            p.C[(i64)m * p.N + n] = v;
+            p.C[(i64)blockIdx.z * p.zstride + (i64)m * p.N + n] = v;
         }
     }
 }
@@ -115,6 +118,8 @@ struct ParamsD {
     int relu;
     int M, N, K;
     int G;  // groups per wave
+    int kz;
+    i64 zstride;
 };
 
 template <bool KC>
@@ -137,6 +142,7 @@ __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
     const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
     const int am0 = min(m0 + l16, p.M - 1), am1 = min(m0 + 16 + l16, p.M - 1);  // past the edge: a valid row / column, result unused
     const int bn0 = min(n0 + l16, p.N - 1), bn1 = min(n0 + 16 + l16, p.N - 1);
+    const int kbase = blockIdx.z * p.kz, kend = min(p.K, kbase + p.kz);
     const int g0 = wave * p.G;
     f64x4 acc[2][2];
 #pragma unroll
@@ -150,7 +156,7 @@ __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
 #pragma unroll
         for (int g = 0; g < MAXG_D; ++g) {
             if (gb + g < p.G) {
-                const int k = 8 * (g0 + gb + g) + 2 * q;
+                const int k = kbase + 8 * (g0 + gb + g) + 2 * q;
                 load_group_d<AKC>(p.A, am0, p.M, p.K, k, a0[g]);
                 load_group_d<AKC>(p.A, am1, p.M, p.K, k, a1[g]);
                 load_group_d<BKC>(p.B, bn0, p.N, p.K, k, b0[g]);
@@ -160,10 +166,10 @@ __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
 #pragma unroll
         for (int g = 0; g < MAXG_D; ++g) {
             if (gb + g < p.G) {
-                const int k = 8 * (g0 + gb + g) + 2 * q;
+                const int k = kbase + 8 * (g0 + gb + g) + 2 * q;
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
-                    const bool in = k + j < p.K;  // past K: zeros in both operands, whatever the clamped loads returned
+                    const bool in = k + j < kend;  // past K: zeros in both operands, whatever the clamped loads returned
                     const double x0 = in ? a0[g][j] : 0., x1 = in ? a1[g][j] : 0., y0 = in ? b0[g][j] : 0., y1 = in ? b1[g][j] : 0.;
                     acc[0][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(x0, y0, acc[0][0], 0, 0, 0);
                     acc[0][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(x0, y1, acc[0][1], 0, 0, 0);
@@ -194,24 +200,57 @@ __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
                 v = v + p.bias[n];
                 if (p.relu) v = v > 0. ? v : 0.;
             }
-            p.C[(i64)m * p.N + n] = v;
+            p.C[(i64)blockIdx.z * p.zstride + (i64)m * p.N + n] = v;
         }
     }
 }
 
-inline bool eligible_f64(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, const double* A, const double* B) {
+// How a product runs here: K in one block (splits == 1), or split over the grid's z dimension into `splits` ranges of kz whose
+// partial results the caller adds in order (igemm::launch_splitk_reduce) -- long reductions with few tiles, the forward product of
+// a classifier head ([256,16384] x [16384,10]).
+struct Plan {
+    bool ok = false;
+    int G = 0, kz = 0, splits = 1;
+};
+
+template <typename T>
+inline Plan make_plan(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, const T* A, const T* B) {
+    Plan pl;
     static const bool off = [] { const char* v = getenv("FX_GEMM_SMALL"); return v && atoi(v) == 0; }();
-    if (off || K < 32 || K > 8 * WAVES * MAXG || M < 1 || N < 1) return false;
-    if (!ta && (K % 2 != 0 || !fx::aligned16(A))) return false;
-    if (tb && (K % 2 != 0 || !fx::aligned16(B))) return false;
-    const i64 blocks = fx::ceil_div(M, (i64)32) * fx::ceil_div(N, (i64)32);
-    return blocks <= 2 * (i64)num_cus && M * N * K <= (1ll << 27);  // M N K / 2 bytes through L2, under 64 MB
+    constexpr int KV = 16 / (int)sizeof(T);  // elements per 16-byte load of a k-contiguous operand
+    if (off || K < 32 || M < 1 || N < 1 || K >= (1ll << 30)) return pl;
+    if (!ta && (K % KV != 0 || !fx::aligned16(A))) return pl;
+    if (tb && (K % KV != 0 || !fx::aligned16(B))) return pl;
+    const i64 tiles = fx::ceil_div(M, (i64)32) * fx::ceil_div(N, (i64)32);
+    // a 32 x 32 tile re-reads each operand once per tile row / column: M N K sizeof(T) / 16 bytes through L2, kept under 32 MB (f32) / 64 MB (f64)
+    if (tiles > 2 * (i64)num_cus || M * N * K > (1ll << 27)) return pl;
+    const i64 kmax = 8 * WAVES * MAXG;  // the most one block takes
+    if (K <= kmax) {
+        pl.G = (int)fx::ceil_div(fx::ceil_div(K, (i64)8), (i64)WAVES);
+        pl.kz = (int)K;
+    } else {
+        // split K over blocks: about 2 blocks per CU, each at least 256 deep, ranges a multiple of 8 * WAVES
+        if (M * N > (1 << 18)) return pl;  // the partial sums stay small
+        i64 splits = std::max<i64>(fx::ceil_div(K, kmax), std::min<i64>(2 * (i64)num_cus / tiles, K / 256));
+        i64 kz = fx::ceil_div(fx::ceil_div(K, splits), (i64)(8 * WAVES)) * (8 * WAVES);
+        splits = fx::ceil_div(K, kz);
+        if (kz > kmax || splits > 65535) return pl;
+        pl.G = (int)(kz / (8 * WAVES));
+        pl.kz = (int)kz;
+        pl.splits = (int)splits;
+    }
+    pl.ok = true;
+    return pl;
 }
 
-inline int run_f64(fx_ctx* c, bool ta, bool tb, i64 M, i64 N, i64 K, const double* A, const double* B, double* C, const double* bias, int relu) {
-    ParamsD p{A, B, C, bias, relu, (int)M, (int)N, (int)K, 0};
-    p.G = (int)fx::ceil_div(fx::ceil_div(K, (i64)8), (i64)WAVES);
-    const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32));
+template <typename T> inline i64 workspace_bytes(const Plan& pl, i64 M, i64 N) { return pl.splits > 1 ? (i64)pl.splits * M * N * (i64)sizeof(T) : 0; }
+
+// part: workspace_bytes() of scratch when pl.splits > 1 (the caller then adds the partial results, with the bias)
+inline int run_f64(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K, const double* A, const double* B, double* C, const double* bias,
+                   int relu, double* part) {
+    const bool split = pl.splits > 1;
+    ParamsD p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0};
+    const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32), (unsigned)pl.splits);
     const size_t lds = (size_t)WAVES * 16 * 64 * sizeof(double);
     if (!ta && !tb) small_kernel_f64<true, false><<<grid, dim3(NT), lds, c->stream>>>(p);
     else if (!ta && tb) small_kernel_f64<true, true><<<grid, dim3(NT), lds, c->stream>>>(p);
@@ -221,21 +260,11 @@ inline int run_f64(fx_ctx* c, bool ta, bool tb, i64 M, i64 N, i64 K, const doubl
     return FX_OK;
 }
 
-// A is k-contiguous unless ta, B is k-contiguous when tb.
-inline bool eligible(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, const float* A, const float* B) {
-    static const bool off = [] { const char* v = getenv("FX_GEMM_SMALL"); return v && atoi(v) == 0; }();
-    if (off || K < 32 || K > 8 * WAVES * MAXG || M < 1 || N < 1) return false;
-    if (!ta && (K % 4 != 0 || !fx::aligned16(A))) return false;
-    if (tb && (K % 4 != 0 || !fx::aligned16(B))) return false;
-    const i64 blocks = fx::ceil_div(M, (i64)32) * fx::ceil_div(N, (i64)32);
-    // a 32 x 32 tile re-reads each operand once per tile row / column: M N K / 4 bytes through L2, kept under 32 MB
-    return blocks <= 2 * (i64)num_cus && M * N * K <= (1ll << 27);
-}
-
-inline int run(fx_ctx* c, bool ta, bool tb, i64 M, i64 N, i64 K, const float* A, const float* B, float* C, const float* bias, int relu) {
-    Params p{A, B, C, bias, relu, (int)M, (int)N, (int)K, 0};
-    p.G = (int)fx::ceil_div(fx::ceil_div(K, (i64)8), (i64)WAVES);
-    const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32));
+inline int run(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K, const float* A, const float* B, float* C, const float* bias, int relu,
+               float* part) {
+    const bool split = pl.splits > 1;
+    Params p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0};
+    const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32), (unsigned)pl.splits);
     if (!ta && !tb) small_kernel<true, false><<<grid, dim3(NT), 0, c->stream>>>(p);
     else if (!ta && tb) small_kernel<true, true><<<grid, dim3(NT), 0, c->stream>>>(p);
     else if (ta && !tb) small_kernel<false, false><<<grid, dim3(NT), 0, c->stream>>>(p);
