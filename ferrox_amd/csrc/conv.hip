@@ -16,6 +16,7 @@
 #include "wgrad_patch.hpp"
 #include "wgrad_patch_s2.hpp"
 #include "dgrad_patch_s2.hpp"
+#include "fwd_patch_s2.hpp"
 #include "conv_smallc.hpp"
 #include "conv_patch.hpp"
 #include "conv_patch_f64.hpp"
@@ -203,6 +204,10 @@ int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64
     if constexpr (sizeof(T) == 4) {
         const csc::Plan sp = smallc_plan<T>(c, d, false);
         if (sp.ok && aligned16(x, x)) return csc::run_fwd(c, sp, x, w, y, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw, bias, relu);
+        if (!generic_only()) {
+            const fw2::Plan f2 = fw2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
+            if (f2.ok && aligned16(x, w) && aligned16(y, y)) return fw2::run(c, f2, x, w, y, B, Cin, H, Cout, d.oh, bias, relu);
+        }
         const cpk::Plan pl = fwd_patch_plan<T>(c, d);
         if (pl.ok && aligned16(x, ws)) {
             float* wimg = (float*)(ws ? ws : c->get_scratch(need));

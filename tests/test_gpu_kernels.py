@@ -564,6 +564,10 @@ CONV_PATCH_CASES = [
     # maps of at most 64 pixels: whole images stacked in one tile (odd batches: the last tile holds one image)
     (5, 16, 8, 8, 128, (1, 1), (1, 1)), (3, 8, 7, 7, 64, (1, 1), (1, 1)), (7, 8, 6, 6, 40, (1, 1), (1, 1)), (4, 8, 6, 10, 200, (1, 1), (0, 1)),
     (33, 64, 8, 8, 64, (1, 1), (1, 1)), (9, 16, 8, 8, 100, (1, 1), (0, 0)),
+    # stride 2 over maps 32 and 64 wide (fwd_patch_s2.hpp): 32 or 64 output channels per block, one to five chunks of 8 input
+    # channels, one to four tiles of 256 pixels per image
+    (2, 8, 32, 32, 32, (2, 2), (1, 1)), (2, 16, 64, 64, 64, (2, 2), (1, 1)), (2, 24, 16, 64, 32, (2, 2), (1, 1)),
+    (3, 40, 64, 32, 32, (2, 2), (1, 1)), (5, 8, 32, 32, 64, (2, 2), (1, 1)), (1, 8, 128, 64, 32, (2, 2), (1, 1)),
 ]
 
 
@@ -591,8 +595,15 @@ def test_conv2d_patch_kernel_shapes(ctx, orc):
         assert rel_err(dxg, tx.grad.numpy()) <= tol * 8, ("dgrad", case)
         assert rel_err(y, orc.conv2d_fwd(x, w, st, pd)) <= tol * 8, ("fwd vs oracle", case)
         assert rel_err(dxg, orc.conv2d_dgrad(g, w, x.shape, st, pd, 0)) <= tol * 8, ("dgrad vs oracle", case)
-        # caller-provided workspaces of exactly the advertised size give the same bits
         dims = (B, Cin, H, W, Cout, 3, 3, st[0], st[1], pd[0], pd[1])
+        # bias + ReLU in the store of the kernel = the forward pass followed by fx_bias_act, bit for bit
+        db_ = ctx.upload(rng.standard_normal(Cout).astype(np.float32))
+        fused = ctx.empty(y.shape, np.float32)
+        capi.check(capi.lib.fx_conv2d_fwd_bias_act_f32(ctx.h, dx_.ptr, dw_.ptr, db_.ptr, fused.ptr, *dims, 1, None, 0))
+        two = ctx.conv2d_fwd(dx_, dw_, st, pd)
+        ctx.bias_act(two, db_, B, Cout, oh * ow, act=1)
+        assert np.array_equal(fused.numpy(), two.numpy()), ("bias+relu", case)
+        # caller-provided workspaces of exactly the advertised size give the same bits
         for kind, fn, a, b_, ref, shape in (
                 (capi.CONV_FWD, capi.lib.fx_conv2d_fwd_f32, dx_, dw_, y, y.shape),
                 (capi.CONV_DGRAD, capi.lib.fx_conv2d_dgrad_f32, dg_, dw_, dxg, x.shape)):

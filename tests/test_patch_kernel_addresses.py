@@ -770,3 +770,107 @@ def test_stride2_data_gradient_patch_kernel_accesses_stay_inside_the_tensors(cas
     pl = dg2_plan(B, Cin, H, W, Cout, 3, 3, 2, 2, 1, 1, oh, ow)
     assert pl is not None, "the shape must exercise the stride-2 data-gradient patch kernel"
     assert dg2_walk(pl, B, Cin, Cout, oh) == "dg2 ok"
+
+
+# ---- f32 stride-2 forward pass (fwd_patch_s2.hpp) ----
+FW2_INSTANCES = [(16, 2), (16, 1), (32, 2), (32, 1)]
+def fw2_plan(B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, oh, ow):
+    if kh != 3 or kw != 3 or sh != 2 or sw != 2 or ph != 1 or pw != 1 or W != 2 * ow or H != 2 * oh or Cin % 8 or Cout % 32: return None
+    if not (Cout == 32 or (Cout == 64 and Cin <= 16)): return None
+    mb = 2 if Cout % 64 == 0 else 1
+    pick = [(o, m) for (o, m) in FW2_INSTANCES if ow == o and mb == m and oh % (256 // o) == 0]
+    return dict(OW=pick[0][0], MB=pick[0][1]) if pick else None
+def fw2_walk(pl, B, Cin, Cout, oh):
+    OW, MB = pl["OW"], pl["MB"]
+    NTF, CC, TR, HALF = 512, 8, 256 // OW, OW + 1
+    PR, W, H = 2 * TR + 1, 2 * OW, 2 * oh
+    RP = 40 if OW == 16 else 2 * HALF
+    PLANE = (PR * RP) | 1
+    WCH, XCH = (CC // 2) * 9 * MB * 64, CC * PLANE; BUF = WCH + XCH
+    W4, X4 = MB * 32 * CC * 9 // 4, CC * PR * (W // 4)
+    NWP, NXP = _ceil_div(W4, NTF), _ceil_div(X4, NTF)
+    assert 2 * BUF * 4 <= 160 * 1024 and 2 * HALF <= RP
+    L, tpi, nmt = oh * OW, oh // TR, Cout // (32 * MB)
+    xsize, wsize, ysize = B * Cin * H * W, Cout * Cin * 9, B * Cout * L
+    nblk = B * tpi * nmt
+    w_written, x_written = set(), set()
+    for blk in sorted({0, 1, nmt - 1, nmt, nblk - 1}):
+        if not 0 <= blk < nblk: continue
+        bt, mt = divmod(blk, nmt); b, tile = divmod(bt, tpi)
+        oc0, oy0 = mt * 32 * MB, tile * TR
+        iy0 = 2 * oy0 - 1
+        for k in sorted({0, Cin // CC - 1}):
+            c0 = k * CC
+            first = blk == 0 and k == 0
+            for tid in range(NTF):
+                for u in range(NWP):
+                    f = u * NTF + tid
+                    ok = f < W4
+                    ocl, q = divmod(f, 18)
+                    a = oc0 * Cin * 9 + c0 * 9 + ((ocl * Cin * 9 + 4 * q) if ok else 0)
+                    assert 0 <= a and a + 4 <= wsize and a % 4 == 0, ("w", a)
+                    if ok and first:
+                        for i in range(4):
+                            cl, t = divmod(4 * q + i, 9)
+                            d = (((cl >> 1) * 9 + t) * MB + (ocl >> 5)) * 64 + (cl & 1) * 32 + (ocl & 31)
+                            assert 0 <= d < WCH and d not in w_written
+                            w_written.add(d)
+                for u in range(NXP):
+                    f = u * NTF + tid
+                    inside = f < X4
+                    cr, q = divmod(f, W // 4); c, r = divmod(cr, PR)
+                    iy = iy0 + r
+                    ok = inside and 0 <= iy < H
+                    a = b * Cin * H * W + c0 * H * W + (((c * H + iy) * W + 4 * q) if ok else 0)
+                    assert 0 <= a and a + 4 <= xsize and a % 4 == 0, ("x", a)
+                    if inside:
+                        d = c * PLANE + r * RP + 2 * q
+                        for o in (HALF, 1, HALF + 1, 2):
+                            assert 0 <= d + o < XCH and (not first or d + o not in x_written)
+                            if first: x_written.add(d + o)
+        # the zero column, operand reads and stores of the corner lanes
+        if blk == 0:
+            for i in range(2 * CC * PR):
+                buf, rem = divmod(i, CC * PR); c, r = divmod(rem, PR)
+                assert buf < 2
+                d = c * PLANE + r * RP
+                assert d not in x_written or buf == 1
+                if buf == 0: x_written.add(d)
+        for wave in range(8):
+            for lane in (0, 15, 16, 31, 32, 47, 63):
+                half, l32 = lane >> 5, lane & 31
+                pix = wave * 32 + l32
+                prow, pcol = divmod(pix, OW)
+                for cp in (0, CC // 2 - 1):
+                    for t in range(9):
+                        ky, kx = divmod(t, 3)
+                        d = (half + 2 * cp) * PLANE + (2 * prow + ky) * RP + pcol + (HALF if kx == 1 else 0) + (1 if kx == 2 else 0)
+                        # the word holds patch row 2 prow + ky, patch column 2 pcol + kx of channel 2 cp + half
+                        c, rem = divmod(d, PLANE); r, o = divmod(rem, RP)
+                        assert c == 2 * cp + half and r == 2 * prow + ky and r < PR
+                        pc = 2 * o if o < HALF else 2 * (o - HALF) + 1
+                        assert o < 2 * HALF and pc == 2 * pcol + kx
+                        assert blk != 0 or d in x_written
+                        for m in range(MB):
+                            assert ((cp * 9 + t) * MB + m) * 64 + lane < WCH
+                for m in range(MB):
+                    for e in (0, 15):
+                        oc = m * 32 + 8 * (e >> 2) + 4 * half + (e & 3)
+                        a = (b * Cout + oc0 + oc) * L + oy0 * OW + pix
+                        assert 0 <= a < ysize and oc0 + oc < Cout and oy0 * OW + pix < L
+    assert w_written == set(range(WCH))
+    return "fw2 ok"
+
+FW2_SHAPES = [  # B, Cin, H, W, Cout
+    (256, 32, 32, 32, 32), (2, 8, 32, 32, 32), (2, 16, 64, 64, 64), (2, 24, 16, 64, 32), (3, 40, 64, 32, 32), (2, 8, 32, 32, 64),
+]
+
+
+@pytest.mark.parametrize("case", FW2_SHAPES, ids=str)
+def test_stride2_forward_patch_kernel_accesses_stay_inside_the_tensors(case):
+    B, Cin, H, W, Cout = case
+    oh, ow = H // 2, W // 2
+    B = min(B, 3)
+    pl = fw2_plan(B, Cin, H, W, Cout, 3, 3, 2, 2, 1, 1, oh, ow)
+    assert pl is not None, "the shape must exercise the stride-2 forward patch kernel"
+    assert fw2_walk(pl, B, Cin, Cout, oh) == "fw2 ok"
