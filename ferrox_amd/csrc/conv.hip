@@ -16,11 +16,13 @@
 #include "wgrad_patch.hpp"
 #include "wgrad_patch_s2.hpp"
 #include "dgrad_patch_s2.hpp"
+#include "dgrad_patch_s2_f64.hpp"
 #include "fwd_patch_s2.hpp"
 #include "conv_smallc.hpp"
 #include "conv_patch.hpp"
 #include "conv_patch_f64.hpp"
 #include "wgrad_patch_f64.hpp"
+#include "wgrad_patch_s2_f64.hpp"
 
 namespace fx {
 int col2im_f32(fx_ctx*, const float*, float*, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, int);
@@ -473,6 +475,11 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
             const dg2::Plan p2 = dg2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
             if (p2.ok && aligned16(g, w) && aligned16(dx, dx)) return dg2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh);
         }
+    } else {
+        if (!generic_only()) {
+            const dgd2::Plan p2 = dgd2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
+            if (p2.ok && aligned16(g, w) && aligned16(dx, dx)) return dgd2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh);
+        }
     }
     T* wt = (T*)(ws ? ws : c->get_scratch(need));
     if (!wt) return FX_ERR_OOM;
@@ -563,6 +570,15 @@ wgd::Plan patch64_plan(fx_ctx* c, const Dims& d, int mode) {
 }
 
 template <typename T>
+wgd2::Plan patch64_s2_plan(fx_ctx* c, const Dims& d, int mode) {
+    if constexpr (sizeof(T) == 8) {
+        if (mode == 0 && !generic_only())
+            return wgd2::make_plan(c ? c->num_cus : 256, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
+    }
+    return wgd2::Plan();
+}
+
+template <typename T>
 i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     const wgp::Plan pl = patch_plan<T>(c, d, mode);
     int splits, kps;
@@ -578,6 +594,8 @@ i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     if (pd.ok) generic = std::max(generic, wgd::workspace_bytes(pd, d.Cout, d.Cin));
     const wg2::Plan p2 = patch_s2_plan<T>(c, d, mode);
     if (p2.ok) generic = std::max(generic, wg2::workspace_bytes(p2, d.Cout, d.Cin));
+    const wgd2::Plan q2 = patch64_s2_plan<T>(c, d, mode);
+    if (q2.ok) generic = std::max(generic, wgd2::workspace_bytes(q2, d.Cout, d.Cin));
     return pl.ok ? std::max(generic, wgp::workspace_bytes(pl, d.Cout, d.Cin)) : generic;
 }
 
@@ -642,6 +660,12 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
         }
     }
     if constexpr (sizeof(T) == 8) {
+        const wgd2::Plan q2 = patch64_s2_plan<T>(c, d, mode);
+        if (q2.ok && aligned16(x, g) && aligned16(ws, ws)) {
+            double* part = (double*)(ws ? ws : c->get_scratch(need));
+            if (!part) return FX_ERR_OOM;
+            return wgd2::run(c, q2, x, g, dw, part, Cin, H, Cout, ph, d.oh);
+        }
         const wgd::Plan pd = patch64_plan<T>(c, d, mode);
         if (pd.ok && aligned16(x, g) && aligned16(ws, ws)) {
             double* part = (double*)(ws ? ws : c->get_scratch(need));

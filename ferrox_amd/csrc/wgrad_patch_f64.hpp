@@ -234,6 +234,44 @@ __global__ __launch_bounds__(256) void wgrad_f64_reduce_kernel(const double* __r
     out[((i64)oc * Cin + c) * KK + t] = s;
 }
 
+// The same sum for many partials of a small output (n and Cin even): the splits are dealt to G groups of threads (group g adds
+// splits g, g + G, ... in order), the groups' sums are added in group order through LDS; two adjacent outputs per thread, so a
+// group's 16 threads read 256 contiguous bytes of a partial with 16-byte loads.
+template <int G>
+__global__ __launch_bounds__(256) void wgrad_f64_reduce_vec_kernel(const double* __restrict__ part, double* __restrict__ out, int n, int splits,
+                                                                   int Cin, FastDiv div_row, FastDiv div_cin) {
+    constexpr int COLS = 256 / G;
+    __shared__ double2 sm[G][COLS];
+    const int col = threadIdx.x % COLS, g = threadIdx.x / COLS;
+    const int j = (blockIdx.x * COLS + col) * 2;
+    double2 s = make_double2(0., 0.);
+    if (j < n) {
+        int z = g;
+        for (; z + 7 * G < splits; z += 8 * G) {
+            double2 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const double2*>(part + (i64)(z + u * G) * n + j);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) { s.x = s.x + v[u].x; s.y = s.y + v[u].y; }
+        }
+        for (; z < splits; z += G) {
+            const double2 v = *reinterpret_cast<const double2*>(part + (i64)z * n + j);
+            s.x = s.x + v.x; s.y = s.y + v.y;
+        }
+    }
+    sm[g][col] = s;
+    __syncthreads();
+    if (g == 0 && j < n) {
+        double2 t = sm[0][col];
+#pragma unroll
+        for (int u = 1; u < G; ++u) { const double2 v = sm[u][col]; t.x = t.x + v.x; t.y = t.y + v.y; }
+        const int oc = (int)div_row.div((uint32_t)j), rem = j - oc * (KK * Cin);
+        const int tap = (int)div_cin.div((uint32_t)rem), c = rem - tap * Cin;
+        double* o = out + ((i64)oc * Cin + c) * KK + tap;
+        o[0] = t.x; o[KK] = t.y;
+    }
+}
+
 struct Plan {
     bool ok = false;
     int PW = 0, PLANE = 0, GP = 0, NK = 0, splits = 1, sps = 1, stages = 0;

@@ -677,6 +677,10 @@ def test_conv2d_f64_patch_kernel_shapes(ctx, orc):
 CONV_F64_WGRAD_CASES = [  # B, Cin, H, W, Cout, sh, (ph, pw)
     (2, 64, 56, 56, 128, 1, (1, 1)), (3, 16, 32, 32, 64, 1, (1, 1)), (2, 32, 26, 26, 64, 1, (0, 0)), (2, 16, 24, 62, 128, 1, (2, 2)),
     (2, 48, 47, 24, 64, 2, (1, 1)), (5, 16, 8, 64, 64, 1, (1, 1)), (37, 16, 9, 32, 64, 1, (1, 1)),
+    # stride 2 in both directions over maps 32 and 64 wide (wgrad_patch_s2_f64.hpp): one and several tiles, an odd height, a top
+    # row without padding, stage ranges that do not divide evenly
+    (3, 32, 32, 32, 64, (2, 2), (1, 1)), (2, 64, 16, 64, 128, (2, 2), (1, 1)), (5, 32, 31, 32, 64, (2, 2), (1, 1)),
+    (2, 32, 33, 32, 64, (2, 2), (0, 1)), (70, 32, 32, 32, 64, (2, 2), (1, 1)), (3, 64, 6, 64, 192, (2, 2), (1, 1)),
 ]
 
 
@@ -688,7 +692,7 @@ def test_conv2d_f64_wgrad_patch_kernel_shapes(ctx, orc):
     tol = TOL[np.dtype(np.float64)]
     for (B, Cin, H, W, Cout, sh, pd) in CONV_F64_WGRAD_CASES:
         case = (B, Cin, H, W, Cout, sh, pd)
-        st = (sh, 1)
+        st = sh if isinstance(sh, tuple) else (sh, 1)
         x = rng.uniform(-1, 1, (B, Cin, H, W))
         oh, ow = orc.out_hw(H, W, 3, 3, st[0], st[1], pd[0], pd[1])
         g = rng.standard_normal((B, Cout, oh, ow))
@@ -831,6 +835,8 @@ STRIDED_DGRAD_CASES = [
     # one to eight output-channel chunks)
     (3, 32, 32, 32, 64, (3, 3), (2, 2), (1, 1)), (2, 64, 32, 32, 128, (3, 3), (2, 2), (1, 1)), (2, 32, 64, 64, 32, (3, 3), (2, 2), (1, 1)),
     (2, 64, 16, 64, 64, (3, 3), (2, 2), (1, 1)), (2, 32, 32, 32, 48, (3, 3), (2, 2), (1, 1)), (1, 96, 64, 32, 16, (3, 3), (2, 2), (1, 1)),
+    # output channels in chunks of 8 (the f64 kernel): one chunk, three chunks
+    (1, 32, 32, 32, 8, (3, 3), (2, 2), (1, 1)), (2, 32, 32, 64, 24, (3, 3), (2, 2), (1, 1)),
 ]
 
 

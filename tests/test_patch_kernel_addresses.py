@@ -772,6 +772,190 @@ def test_stride2_data_gradient_patch_kernel_accesses_stay_inside_the_tensors(cas
     assert dg2_walk(pl, B, Cin, Cout, oh) == "dg2 ok"
 
 
+# ---- f64 stride-2 data gradient (dgrad_patch_s2_f64.hpp) ----
+DGD2_INSTANCES = [(16, 8), (32, 8)]
+def dgd2_plan(B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, oh, ow):
+    if kh != 3 or kw != 3 or sh != 2 or sw != 2 or ph != 1 or pw != 1 or W != 2 * ow or H != 2 * oh or Cin % 32: return None
+    pick = [(o, c) for (o, c) in DGD2_INSTANCES if ow == o and Cout % c == 0 and oh % (256 // o) == 0]
+    return dict(OW=pick[0][0], OCC=pick[0][1]) if pick else None
+def dgd2_walk(pl, B, Cin, Cout, oh):
+    """Offsets in doubles; 16-byte loads and stores must sit on even offsets."""
+    OW, OCC = pl["OW"], pl["OCC"]
+    NTD, TR, PC = 512, 256 // OW, OW + 1
+    PR = TR + 1; GPL = (PR * PC) | 1; KS = OCC // 4
+    WCH, GCH = KS * 9 * 2 * 64, OCC * GPL; BUF = WCH + GCH
+    W2 = OCC * 144; NWP = _ceil_div(W2, NTD); NGP = OCC * 128 // NTD; X2 = OCC * OW // 2
+    assert 2 * BUF * 8 <= 160 * 1024 and OCC * 128 % NTD == 0 and X2 <= NTD
+    L, H, W, tpi, nct = oh * OW, 2 * oh, 2 * OW, oh // TR, Cin // 32
+    gsize, wsize, xsize = B * Cout * L, Cout * Cin * 9, B * Cin * H * W
+    w_written, g_written = set(), set()
+    for blk in sorted({0, 1, nct - 1, nct, B * tpi * nct - 1}):
+        if not 0 <= blk < B * tpi * nct: continue
+        bt, ct = divmod(blk, nct); b, tile = divmod(bt, tpi)
+        c0, i0 = ct * 32, tile * TR
+        next_row = i0 + TR < oh
+        for k in sorted({0, Cout // OCC - 1}):
+            oc0 = k * OCC
+            first = blk == 0 and k == 0
+            for tid in range(NTD):
+                for u in range(NWP):
+                    f = u * NTD + tid
+                    ok = f < W2
+                    ocl, q = divmod(f, 144)
+                    a = c0 * 9 + oc0 * Cin * 9 + ((ocl * Cin * 9 + 2 * q) if ok else 0)
+                    assert 0 <= a and a + 2 <= wsize and a % 2 == 0, ("w", a)
+                    if ok and first:
+                        for i in range(2):
+                            c, t = divmod(2 * q + i, 9)
+                            d = (((ocl >> 2) * 9 + t) * 2 + (c >> 4)) * 64 + (ocl & 3) * 16 + (c & 15)
+                            assert 0 <= d < WCH and d not in w_written
+                            w_written.add(d)
+                gq, goc = tid & 127, tid >> 7
+                for u in range(NGP):
+                    a = (b * Cout * oh + i0) * OW + (oc0 + 4 * u + goc) * L + 2 * gq
+                    assert 0 <= a and a + 2 <= gsize and a % 2 == 0, ("g", a)
+                    d = (4 * u + goc) * GPL + (gq // (OW // 2)) * PC + (gq % (OW // 2)) * 2
+                    assert d + 2 <= GCH
+                    if first: g_written.update(range(d, d + 2))
+                xoc, xq = divmod(tid, OW // 2)
+                if next_row:
+                    a = (b * Cout * oh + i0) * OW + oc0 * L + ((xoc * L + TR * OW + 2 * xq) if tid < X2 else 0)
+                    assert 0 <= a and a + 2 <= gsize and a % 2 == 0, ("g row", a)
+                if tid < X2:
+                    d = xoc * GPL + TR * PC + 2 * xq
+                    assert d + 2 <= GCH and xoc < OCC
+                    if first: g_written.update(range(d, d + 2))
+        # stores and operand reads of the corner lanes: lane l holds rows 4 e + l / 16 of a 16 x 16 block, column l % 16
+        for wave in range(8):
+            for lane in (0, 15, 16, 47, 48, 63):
+                kq, l16 = lane >> 4, lane & 15
+                for h in range(2):
+                    crow, ccol = divmod(wave * 32 + 16 * h + l16, OW)
+                    for ch in range(2):
+                        for e in (0, 3):
+                            c = 16 * ch + 4 * e + kq
+                            for py in range(2):
+                                a = (((b * Cin + c0 + c) * H) + 2 * (i0 + crow) + py) * W + 2 * ccol
+                                assert 0 <= a and a + 2 <= xsize and a % 2 == 0 and c0 + c < Cin
+                    for ks in (0, KS - 1):
+                        d = (4 * ks + kq) * GPL + (crow + 1) * PC + ccol + 1
+                        assert d < GCH and crow + 1 < PR and ccol + 1 < PC
+                        for t in range(9):
+                            for ch in range(2):
+                                assert ((ks * 9 + t) * 2 + ch) * 64 + lane < WCH
+    assert w_written == set(range(WCH))
+    need = {oc * GPL + r * PC + c for oc in range(OCC) for r in range(PR) for c in range(OW)}
+    assert need <= g_written
+    return "dgd2 ok"
+
+DGD2_SHAPES = [  # B, Cin, H, W, Cout
+    (256, 32, 32, 32, 64), (2, 64, 32, 32, 128), (2, 32, 64, 64, 32), (2, 64, 16, 64, 64), (2, 32, 32, 32, 8), (1, 96, 64, 32, 24),
+]
+
+
+@pytest.mark.parametrize("case", DGD2_SHAPES, ids=str)
+def test_stride2_f64_data_gradient_patch_kernel_accesses_stay_inside_the_tensors(case):
+    B, Cin, H, W, Cout = case
+    oh, ow = H // 2, W // 2
+    B = min(B, 3)
+    pl = dgd2_plan(B, Cin, H, W, Cout, 3, 3, 2, 2, 1, 1, oh, ow)
+    assert pl is not None, "the shape must exercise the f64 stride-2 data-gradient patch kernel"
+    assert dgd2_walk(pl, B, Cin, Cout, oh) == "dgd2 ok"
+
+
+# ---- f64 stride-2 weight gradient (wgrad_patch_s2_f64.hpp) ----
+WGD2_INSTANCES = [(16, 2), (32, 1)]
+def wgd2_plan(B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, oh, ow, num_cus=256):
+    if kh != 3 or kw != 3 or sh != 2 or sw != 2 or pw != 1 or ph > 1 or W != 2 * ow or Cin % 32 or Cout % 64: return None
+    pick = [(o, r) for (o, r) in WGD2_INSTANCES if o == ow and oh % r == 0]
+    if not pick: return None
+    OW, R = pick[0]
+    stages = B * (oh // R); tiles = (Cin // 32) * (Cout // 64)
+    splits = max(1, min(num_cus // tiles, max(1, stages // 2)))
+    sps = _ceil_div(stages, splits)
+    return dict(OW=OW, R=R, stages=stages, sps=sps, splits=_ceil_div(stages, sps))
+def wgd2_walk(pl, B, Cin, H, Cout, ph, oh):
+    """Offsets in doubles; 16-byte loads must sit on even offsets."""
+    OW, R = pl["OW"], pl["R"]
+    NTW, BM, W, PW, XR, KST = 256, 64, 2 * OW, 2 * OW + 2, 2 * R + 1, R * OW
+    GP, PLANE = KST | 1, (XR * PW) | 1
+    XL, GL = W // 2, KST // 2
+    RX, GR = NTW // XL, NTW // GL
+    NXP, NG = XR * 32 // RX, BM // GR
+    GROUPS, GPR, BUF = KST // 4, OW // 4, BM * GP + 32 * PLANE
+    assert NTW % XL == 0 and 32 % RX == 0 and NTW % GL == 0 and BM % GR == 0 and 2 * BUF * 8 <= 160 * 1024
+    L, spi = oh * OW, oh // R
+    gsize, xsize = B * Cout * L, B * Cin * H * W
+    covered = set()
+    for z in range(pl["splits"]):
+        covered |= set(range(z * pl["sps"], min(pl["stages"], (z + 1) * pl["sps"])))
+    assert covered == set(range(pl["stages"]))
+    rows_parked, g_parked = set(), set()
+    for s in (0, 1, spi - 1, spi, pl["stages"] - 1):
+        if not 0 <= s < pl["stages"]: continue
+        b, k = divmod(s, spi); oy0 = k * R; iy0 = 2 * oy0 - ph
+        for c0 in (0, Cin - 32):
+            for oc0 in (0, Cout - BM):
+                for tid in range(NTW):
+                    gq, grow, xq, xrow = tid % GL, tid // GL, tid % XL, tid // XL
+                    for u in range(NG):
+                        a = (b * Cout + oc0 + GR * u + grow) * L + oy0 * OW + 2 * gq
+                        assert 0 <= a and a + 2 <= gsize and a % 2 == 0, ("g", a)
+                        d = (GR * u + grow) * GP + 2 * gq
+                        assert d + 2 <= BM * GP and 2 * gq + 2 <= KST
+                        g_parked.update((GR * u + grow, 2 * gq + i) for i in range(2))
+                    for u in range(NXP):
+                        r, cb = u * RX // 32, u * RX % 32
+                        iy = iy0 + r
+                        assert cb + xrow < 32 and r < XR
+                        if 0 <= iy < H:
+                            a = ((b * Cin + c0 + cb + xrow) * H + iy) * W + 2 * xq
+                            assert 0 <= a and a + 2 <= xsize and a % 2 == 0, ("x", a)
+                        d = BM * GP + (cb + xrow) * PLANE + r * PW + 1 + 2 * xq
+                        assert BM * GP <= d and d + 2 <= BUF and 1 + 2 * xq + 2 <= W + 1
+                        rows_parked.update((cb + xrow, r, 1 + 2 * xq + i) for i in range(2))
+    assert rows_parked == {(c, r, col) for c in range(32) for r in range(XR) for col in range(1, W + 1)}
+    assert g_parked == {(oc, px) for oc in range(BM) for px in range(KST)}
+    # operand reads of the corner lanes over the unrolled pixel loop: pixels inside the stage, patch columns 0 .. W
+    for wave in range(4):
+        wmo, wc = wave & 1, wave >> 1
+        for lane in (0, 15, 16, 47, 48, 63):
+            kq, l16 = lane >> 4, lane & 15
+            ga0 = (wmo * 32 + l16) * GP + kq
+            xb0 = BM * GP + (wc * 16 + l16) * PLANE + 2 * kq
+            for u in range(GROUPS):
+                r, j = divmod(u, GPR)
+                for o in range(2):
+                    a = ga0 + 16 * o * GP + r * OW + 4 * j
+                    assert a - (wmo * 32 + 16 * o + l16) * GP < KST and a < BM * GP
+                for ky in range(3):
+                    for kx in range(3):
+                        d = xb0 + (2 * r + ky) * PW + 8 * j + kx
+                        col = d - BM * GP - (wc * 16 + l16) * PLANE - (2 * r + ky) * PW
+                        assert 0 <= col <= W and d < BUF and 2 * r + ky < XR
+                        assert col == 2 * (4 * j + kq) + kx
+            for o in range(2):
+                for e in (0, 3):
+                    oc = wmo * 32 + o * 16 + 4 * e + kq
+                    assert oc < BM and wc * 16 + l16 < 32
+    return "wgd2 ok"
+
+WGD2_SHAPES = [  # B, Cin, H, W, Cout, (ph, pw)
+    (256, 32, 32, 32, 64, (1, 1)), (2, 64, 8, 32, 128, (1, 1)), (2, 32, 8, 64, 64, (1, 1)), (2, 64, 4, 64, 128, (1, 1)),
+    (2, 32, 33, 32, 64, (0, 1)), (2, 32, 31, 32, 64, (1, 1)), (40, 32, 8, 32, 64, (1, 1)), (3, 32, 6, 64, 192, (1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", WGD2_SHAPES, ids=str)
+def test_stride2_f64_weight_gradient_patch_kernel_accesses_stay_inside_the_tensors(case):
+    B, Cin, H, W, Cout, pd = case
+    oh, ow = (H + 2 * pd[0] - 3) // 2 + 1, (W + 2 * pd[1] - 3) // 2 + 1
+    B = min(B, 41)
+    pl = wgd2_plan(B, Cin, H, W, Cout, 3, 3, 2, 2, pd[0], pd[1], oh, ow)
+    assert pl is not None, "the shape must exercise the f64 stride-2 weight-gradient patch kernel"
+    assert wgd2_walk(pl, B, Cin, H, Cout, pd[0], oh) == "wgd2 ok"
+
+
 # ---- f32 stride-2 forward pass (fwd_patch_s2.hpp) ----
 FW2_INSTANCES = [(16, 2), (16, 1), (32, 2), (32, 1)]
 def fw2_plan(B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, oh, ow):
