@@ -767,6 +767,34 @@ def test_conv2d_image_layer_kernels(ctx, orc):
         assert np.array_equal(out.numpy(), gw), case
 
 
+def test_conv2d_f64_image_layer_forward(ctx, orc):
+    """Image layers in f64 (1 to 4 input channels, K = Cin * 9 below two slabs of the implicit GEMM): forward, bias + ReLU in the store."""
+    import torch
+    import torch.nn.functional as F
+    from ferrox_amd import capi
+    rng = np.random.default_rng(63)
+    tol = TOL[np.dtype(np.float64)]
+    for (B, Cin, H, W, Cout, st, pd) in SMALLC_CASES:
+        case = (B, Cin, H, W, Cout, st, pd)
+        x = rng.uniform(-1, 1, (B, Cin, H, W))
+        w = rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9))
+        bias = rng.standard_normal(Cout)
+        oh, ow = orc.out_hw(H, W, 3, 3, st[0], st[1], pd[0], pd[1])
+        dx_, dw_, db_ = ctx.upload(x), ctx.upload(w), ctx.upload(bias)
+        y = ctx.conv2d_fwd(dx_, dw_, st, pd).numpy()
+        ty = F.conv2d(torch.from_numpy(x), torch.from_numpy(w), stride=st, padding=pd).numpy()
+        ay = F.conv2d(torch.from_numpy(np.abs(x)), torch.from_numpy(np.abs(w)), stride=st, padding=pd).max().item()
+        assert np.abs(y - ty).max() <= tol * ay, ("fwd", case)
+        assert rel_err(y, orc.conv2d_fwd(x, w, st, pd)) <= tol * 8, ("fwd vs oracle", case)
+        assert np.array_equal(ctx.conv2d_fwd(dx_, dw_, st, pd).numpy(), y), case
+        dims = (B, Cin, H, W, Cout, 3, 3, st[0], st[1], pd[0], pd[1])
+        fused = ctx.empty(y.shape, np.float64)
+        capi.check(capi.lib.fx_conv2d_fwd_bias_act_f64(ctx.h, dx_.ptr, dw_.ptr, db_.ptr, fused.ptr, *dims, 1, None, 0))
+        two = ctx.conv2d_fwd(dx_, dw_, st, pd)
+        capi.check(capi.lib.fx_bias_act_f64(ctx.h, two.ptr, db_.ptr, B, Cout, oh * ow, 1))
+        assert np.array_equal(fused.numpy(), two.numpy()), ("bias+relu", case)
+
+
 def test_conv2d_tune_up_front_and_ragged_batch(ctx, orc):
     """fx_conv2d_tune_f32 pays the tile timing for a layer before its first use; a ragged batch of the same size class and
     one of another class run afterwards, all against the oracle.  An output that overlaps an operand is not timed."""
