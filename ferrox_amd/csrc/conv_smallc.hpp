@@ -122,6 +122,13 @@ __global__ __launch_bounds__(NT) void fwd_kernel(const FwdParams p) {
             if (!ok) pv[v] = make_float4(0.f, 0.f, 0.f, 0.f);
         }
     };
+    // the bias of this lane's 16 output rows, loaded once (a load per tile in the store loop puts its latency on every tile)
+    float bv[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const int ch = m0 + igemm::Mfma<float>::row(e, lane);
+        bv[e] = BIAS ? p.bias[ch < g.Cout ? ch : g.Cout - 1] : 0.f;
+    }
     const int ntiles = p.ntiles;
     int t = blockIdx.x;
     if (t < ntiles) prefetch(t);
@@ -165,7 +172,7 @@ __global__ __launch_bounds__(NT) void fwd_kernel(const FwdParams p) {
                     if (ch < g.Cout) {
                         float v = acc[e];
                         if constexpr (BIAS) {
-                            v += p.bias[ch];
+                            v += bv[e];
                             if (p.relu) v = v > 0.f ? v : 0.f;
                         }
                         yb[(i64)ch * L + pp] = v;

@@ -56,6 +56,7 @@ __global__ __launch_bounds__(NT) void small_kernel(const Params p) {
     const int am = min(m0 + l32, p.M - 1), bn = min(n0 + l32, p.N - 1);  // past the edge: a valid row / column, result unused
     const int kbase = blockIdx.z * p.kz, kend = min(p.K, kbase + p.kz);    // this block's range of K (all of it unless K is split over z)
     const int g0 = wave * p.G;
+    const float bias_n = p.bias ? p.bias[bn] : 0.f;  // loaded up front: its latency stays off the closing sum
 
     float a[MAXG][4], b[MAXG][4];
 #pragma unroll
@@ -94,7 +95,7 @@ __global__ __launch_bounds__(NT) void small_kernel(const Params p) {
         const int m = m0 + 8 * (e >> 2) + 4 * h + (e & 3);
         if (m < p.M && n < p.N) {
             if (p.bias) {
-                v = v + p.bias[n];
+                v = v + bias_n;
                 if (p.relu) v = v > 0.f ? v : 0.f;
             }
             p.C[(i64)blockIdx.z * p.zstride + (i64)m * p.N + n] = v;
@@ -144,6 +145,8 @@ __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
     const int bn0 = min(n0 + l16, p.N - 1), bn1 = min(n0 + 16 + l16, p.N - 1);
     const int kbase = blockIdx.z * p.kz, kend = min(p.K, kbase + p.kz);
     const int g0 = wave * p.G;
+    // this wave finishes the column block (wave / 2) % 2 in the closing sum; its bias is loaded up front
+    const double bias_n = p.bias ? p.bias[(wave >> 1) & 1 ? bn1 : bn0] : 0.;
     f64x4 acc[2][2];
 #pragma unroll
     for (int a = 0; a < 2; ++a)
@@ -197,7 +200,7 @@ __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
         const int m = m0 + 16 * (blk >> 1) + 4 * e + q, n = n0 + 16 * (blk & 1) + l16;
         if (m < p.M && n < p.N) {
             if (p.bias) {
-                v = v + p.bias[n];
+                v = v + bias_n;
                 if (p.relu) v = v > 0. ? v : 0.;
             }
             p.C[(i64)blockIdx.z * p.zstride + (i64)m * p.N + n] = v;
