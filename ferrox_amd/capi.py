@@ -137,6 +137,7 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_relu_bwd_bias_grad_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64)
     _sig(f"fx_softmax_ce_fwd_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64)
     _sig(f"fx_softmax_ce_bwd_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64)
+    _sig(f"fx_softmax_ce_fwd_unit_grad_{_s}", _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64)
     _sig(f"fx_adam_step_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, *([_ct] * 7))
     _sig(f"fx_sgd_step_{_s}", _vp, _vp, _vp, _i64, _ct)
     _sig(f"fx_adam_step_multi_{_s}", _vp, _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_i64),
@@ -559,6 +560,12 @@ class Context:
         probs, loss = self.empty((B, Cc), logits.dtype), self.empty((1,), logits.dtype)
         check(self._fn("softmax_ce_fwd", logits.dtype)(self.h, logits.ptr, targets.ptr, probs.ptr, loss.ptr, B, Cc))
         return probs, loss
+
+    def softmax_ce_fwd_unit_grad(self, logits, targets):
+        B, Cc = logits.shape
+        probs, loss, d = self.empty((B, Cc), logits.dtype), self.empty((1,), logits.dtype), self.empty((B, Cc), logits.dtype)
+        check(self._fn("softmax_ce_fwd_unit_grad", logits.dtype)(self.h, logits.ptr, targets.ptr, probs.ptr, loss.ptr, d.ptr, B, Cc))
+        return probs, loss, d
 
     def softmax_ce_bwd(self, probs, targets, grad_loss):
         B, Cc = probs.shape

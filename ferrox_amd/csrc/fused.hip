@@ -251,11 +251,14 @@ __global__ __launch_bounds__(256) void mean_rows_kernel(const T* __restrict__ ro
 
 // Both steps in one block for small problems (up to 1024 rows and 16384 logits): thread t takes rows t, t + 256, ... -- the rows and the order in which
 // mean_rows_kernel's thread t adds them -- and the same tree follows, so the loss has the bits of the two-kernel path.
+// With dx != null the block also writes d loss / d logits for an upstream gradient of exactly 1 -- the operations of
+// softmax_ce_bwd_kernel on the row it has just finished, in their order, so dx has that kernel's bits.
 template <typename T>
 __global__ __launch_bounds__(256) void softmax_ce_small_kernel(const T* __restrict__ x, const T* __restrict__ y, T* __restrict__ probs,
-                                                               T* __restrict__ loss, i64 B, i64 C, T lo, T hi, T inv) {
+                                                               T* __restrict__ loss, T* __restrict__ dx, i64 B, i64 C, T lo, T hi, T inv) {
     __shared__ T sm[256];
     T tot = T(0);
+    const T dtl = -(T(1) * inv);
     if (C <= 16) {
         // a row fits the registers: all of its loads are in flight together instead of one dependent access after the other
         // (the arithmetic and its order are those of the general loop below)
@@ -286,6 +289,22 @@ __global__ __launch_bounds__(256) void softmax_ce_small_kernel(const T* __restri
 #pragma unroll
             for (int k = 0; k < 16; ++k) if (k < c) probs[b * C + k] = pv[k];
             tot = tot + (-acc);
+            if (dx) {
+                T dv[16], dot = T(0);
+#pragma unroll
+                for (int k = 0; k < 16; ++k) if (k < c) {
+                    const T sv = pv[k];
+                    T p = sv;
+                    if (p < lo) p = lo;
+                    if (p > hi) p = hi;
+                    const T dp = (dtl * yv[k]) / p;
+                    const T ds = (dp * (sv >= lo ? T(1) : T(0))) * (sv <= hi ? T(1) : T(0));
+                    dv[k] = ds;
+                    dot = dot + ds * sv;
+                }
+#pragma unroll
+                for (int k = 0; k < 16; ++k) if (k < c) dx[b * C + k] = pv[k] * (dv[k] - dot);
+            }
         }
     } else
     for (i64 b = threadIdx.x; b < B; b += 256) {
@@ -306,6 +325,21 @@ __global__ __launch_bounds__(256) void softmax_ce_small_kernel(const T* __restri
             acc = acc + yr[k] * dev_log<T>(p);
         }
         tot = tot + (-acc);
+        if (dx) {
+            T* dr = dx + b * C;
+            T dot = T(0);
+            for (i64 k = 0; k < C; ++k) {
+                const T sv = pr[k];
+                T p = sv;
+                if (p < lo) p = lo;
+                if (p > hi) p = hi;
+                const T dp = (dtl * yr[k]) / p;
+                const T ds = (dp * (sv >= lo ? T(1) : T(0))) * (sv <= hi ? T(1) : T(0));
+                dr[k] = ds;
+                dot = dot + ds * sv;
+            }
+            for (i64 k = 0; k < C; ++k) dr[k] = pr[k] * (dr[k] - dot);
+        }
     }
     sm[threadIdx.x] = tot;
     __syncthreads();
@@ -317,17 +351,23 @@ __global__ __launch_bounds__(256) void softmax_ce_small_kernel(const T* __restri
 }
 
 template <typename T>
-int softmax_ce_fwd(fx_ctx* c, const T* logits, const T* targets, T* probs, T* loss, i64 B, i64 C) {
+__global__ __launch_bounds__(256) void softmax_ce_bwd_kernel(const T* __restrict__ probs, const T* __restrict__ y, const T* __restrict__ gup,
+                                                             T gval, T* __restrict__ dx, i64 B, i64 C, T inv, T lo, T hi);
+
+// dlogits (optional): d loss / d logits for an upstream gradient of 1, with the bits of softmax_ce_bwd on a device 1.
+template <typename T>
+int softmax_ce_fwd(fx_ctx* c, const T* logits, const T* targets, T* probs, T* loss, i64 B, i64 C, T* dlogits = nullptr) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(B >= 1 && C >= 1, "fx_softmax_ce_fwd: bad shape");
     FX_REQUIRE(logits && targets && probs && loss, "fx_softmax_ce_fwd: null pointer");
     std::lock_guard<std::mutex> lk(c->launch_mutex);
-    if (B <= 1024 && B * C <= 16384) {  // little work: one launch instead of two
-        softmax_ce_small_kernel<T><<<dim3(1), dim3(256), 0, c->stream>>>(logits, targets, probs, loss, B, C, (T)1e-8, (T)(1.0 - 1e-8),
-                                                                         (T)(1.0 / (double)B));
+    if (B <= 1024 && B * C <= 16384) {  // little work: one launch instead of two (or three)
+        softmax_ce_small_kernel<T><<<dim3(1), dim3(256), 0, c->stream>>>(logits, targets, probs, loss, dlogits, B, C, (T)1e-8,
+                                                                         (T)(1.0 - 1e-8), (T)(1.0 / (double)B));
         FX_LAUNCH_CHECK();
         return FX_OK;
     }
+
     T* rowloss = (T*)c->get_scratch(B * (i64)sizeof(T));
     if (!rowloss) return FX_ERR_OOM;
     softmax_ce_rows_kernel<T><<<dim3((unsigned)fx::ceil_div(B, (i64)256)), dim3(256), 0, c->stream>>>(
@@ -335,21 +375,27 @@ int softmax_ce_fwd(fx_ctx* c, const T* logits, const T* targets, T* probs, T* lo
     FX_LAUNCH_CHECK();
     mean_rows_kernel<T><<<dim3(1), dim3(256), 0, c->stream>>>(rowloss, loss, B, (T)(1.0 / (double)B));
     FX_LAUNCH_CHECK();
+    if (dlogits) {
+        softmax_ce_bwd_kernel<T><<<dim3((unsigned)fx::ceil_div(B, (i64)256)), dim3(256), 0, c->stream>>>(
+            probs, targets, nullptr, T(1), dlogits, B, C, (T)(1.0 / (double)B), (T)1e-8, (T)(1.0 - 1e-8));
+        FX_LAUNCH_CHECK();
+    }
     return FX_OK;
 }
 
 // backward: upstream g (one element on the device) -> d logits, the composed chain evaluated per row:
 //   d_tl = (-(g * (1/B)));  d_logp = d_tl * y;  d_p = d_logp / p;  d_s = d_p * (s >= lo) * (s <= hi);
 //   d_x = s * (d_s - sum_c(d_s * s))
+// The upstream gradient is gup[0], or gval where gup is null.
 template <typename T>
-__global__ __launch_bounds__(256) void softmax_ce_bwd_kernel(const T* __restrict__ probs, const T* __restrict__ y,
-                                                             const T* __restrict__ gup, T* __restrict__ dx, i64 B, i64 C, T inv, T lo, T hi) {
+__global__ __launch_bounds__(256) void softmax_ce_bwd_kernel(const T* __restrict__ probs, const T* __restrict__ y, const T* __restrict__ gup,
+                                                             T gval, T* __restrict__ dx, i64 B, i64 C, T inv, T lo, T hi) {
     const i64 b = (i64)blockIdx.x * 256 + threadIdx.x;
     if (b >= B) return;
     const T* sr = probs + b * C;
     const T* yr = y + b * C;
     T* dr = dx + b * C;
-    const T dtl = -(gup[0] * inv);
+    const T dtl = -((gup ? gup[0] : gval) * inv);
     T dot = T(0);
     if (C <= 16) {  // the row in registers, loads in flight together; same arithmetic in the same order as below
         const int c = (int)C;
@@ -393,7 +439,7 @@ int softmax_ce_bwd(fx_ctx* c, const T* probs, const T* targets, const T* gup, T*
     FX_REQUIRE(B >= 1 && C >= 1, "fx_softmax_ce_bwd: bad shape");
     FX_REQUIRE(probs && targets && gup && dlogits, "fx_softmax_ce_bwd: null pointer");
     softmax_ce_bwd_kernel<T><<<dim3((unsigned)fx::ceil_div(B, (i64)256)), dim3(256), 0, c->stream>>>(
-        probs, targets, gup, dlogits, B, C, (T)(1.0 / (double)B), (T)1e-8, (T)(1.0 - 1e-8));
+        probs, targets, gup, T(0), dlogits, B, C, (T)(1.0 / (double)B), (T)1e-8, (T)(1.0 - 1e-8));
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
@@ -549,6 +595,11 @@ int sgd_step(fx_ctx* c, T* p, const T* g, T* buf, i64 n, T lr, T momentum, T wd,
     extern "C" int fx_softmax_ce_fwd_##S(fx_ctx* c, const T* logits, const T* targets, T* probs, T* loss, int64_t B,   \
                                          int64_t C) {                                                                  \
         return softmax_ce_fwd<T>(c, logits, targets, probs, loss, B, C);                                               \
+    }                                                                                                                  \
+    extern "C" int fx_softmax_ce_fwd_unit_grad_##S(fx_ctx* c, const T* logits, const T* targets, T* probs, T* loss,    \
+                                                   T* dlogits, int64_t B, int64_t C) {                                  \
+        FX_REQUIRE(dlogits, "fx_softmax_ce_fwd_unit_grad: null pointer");                                              \
+        return softmax_ce_fwd<T>(c, logits, targets, probs, loss, B, C, dlogits);                                      \
     }                                                                                                                  \
     extern "C" int fx_softmax_ce_bwd_##S(fx_ctx* c, const T* probs, const T* targets, const T* gup, T* dlogits,        \
                                          int64_t B, int64_t C) {                                                       \

@@ -484,6 +484,7 @@ template <typename T> class AutoFerroxEngine {
     // step instead of cloning it).  With reuse_unit_seed set, a one-element loss is seeded from a tensor of one 1.0 that is
     // filled once and only ever read, instead of a fresh ones() per step (same value, one kernel fewer).
     bool reuse_unit_seed = false;
+    const T* unit_seed_data() const { return unit_seed_ ? unit_seed_->data() : nullptr; }  // null before the first backward()
     void backward(NodeId loss_id, Tensor<T>* keep_loss = nullptr) {  // :700-733
         const HipStorage<T>* loss = get_tensor(loss_id);
         if (!loss) throw Error("Loss node not found");

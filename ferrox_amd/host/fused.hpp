@@ -24,6 +24,9 @@ template <typename T> struct FusedApi;
         static int bias_grad(fx_ctx* c, const T* g, T* out, int64_t o, int64_t C, int64_t i) { return fx_bias_grad_##S(c, g, out, o, C, i); } \
         static int sce_fwd(fx_ctx* c, const T* x, const T* y, T* p, T* l, int64_t B, int64_t C) { return fx_softmax_ce_fwd_##S(c, x, y, p, l, B, C); } \
         static int sce_bwd(fx_ctx* c, const T* p, const T* y, const T* g, T* d, int64_t B, int64_t C) { return fx_softmax_ce_bwd_##S(c, p, y, g, d, B, C); } \
+        static int sce_fwd_unit(fx_ctx* c, const T* x, const T* y, T* p, T* l, T* d, int64_t B, int64_t C) {            \
+            return fx_softmax_ce_fwd_unit_grad_##S(c, x, y, p, l, d, B, C);                                            \
+        }                                                                                                              \
         static int adam(fx_ctx* c, T* p, const T* g, T* m, T* v, int64_t n, T lr, T b1, T b2, T eps, T wd, T bc1, T bc2) { \
             return fx_adam_step_##S(c, p, g, m, v, n, lr, b1, b2, eps, wd, bc1, bc2);                                  \
         }                                                                                                              \
@@ -154,18 +157,36 @@ template <typename T> struct Conv2dFusedOp : Operator<T> {  // inputs: x [B,Cin,
 };
 
 template <typename T> struct SoftmaxCEOp : Operator<T> {  // inputs: logits [B,C], targets [B,C]; output: scalar loss
-    mutable Tensor<T> probs;  // kept for the backward pass
+    mutable Tensor<T> probs;        // kept for the backward pass
+    mutable Tensor<T> unit_grad;    // d logits for an upstream gradient of 1, written by the forward launch (see below)
+    const AutoFerroxEngine<T>* eng;  // or null
+    // On an engine that seeds backward() from its one shared tensor of 1.0 (reuse_unit_seed) the loss is normally the root of
+    // the tape and its upstream gradient that very tensor: the forward launch then also writes d logits for a gradient of 1,
+    // and gradient() hands them out without a launch when the upstream gradient is that tensor (else it runs the kernel).
+    explicit SoftmaxCEOp(const AutoFerroxEngine<T>* e = nullptr) : eng(e) {}
     Tensor<T> compute(const TensorRefs<T>& in) const override {
         const Shape& s = in[0]->shape();
         if (s.size() != 2 || in[1]->shape() != s) throw Error("CCELoss: predictions " + fmt_shape(s) + " vs targets " + fmt_shape(in[1]->shape()));
         probs = HipStorage<T>::alloc(s);
         Tensor<T> loss = HipStorage<T>::alloc({});
-        fx_ok(FusedApi<T>::sce_fwd(fused_ctx(), in[0]->data(), in[1]->data(), probs->data(), loss->data(), (int64_t)s[0], (int64_t)s[1]));
+        if (eng && eng->reuse_unit_seed) {
+            unit_grad = HipStorage<T>::alloc(s);
+            fx_ok(FusedApi<T>::sce_fwd_unit(fused_ctx(), in[0]->data(), in[1]->data(), probs->data(), loss->data(), unit_grad->data(),
+                                            (int64_t)s[0], (int64_t)s[1]));
+        } else {
+            unit_grad.reset();
+            fx_ok(FusedApi<T>::sce_fwd(fused_ctx(), in[0]->data(), in[1]->data(), probs->data(), loss->data(), (int64_t)s[0], (int64_t)s[1]));
+        }
         return loss;
     }
     std::vector<Tensor<T>> gradient(Tensor<T> g, const TensorRefs<T>& in, const HipStorage<T>*) const override {
         const Shape& s = in[0]->shape();
         std::vector<Tensor<T>> r(2);
+        if (unit_grad && eng && eng->unit_seed_data() && g->data() == eng->unit_seed_data()) {
+            r[0] = std::move(unit_grad);
+            return r;
+        }
+        unit_grad.reset();
         r[0] = HipStorage<T>::alloc(s);
         fx_ok(FusedApi<T>::sce_bwd(fused_ctx(), probs->data(), in[1]->data(), g->data(), r[0]->data(), (int64_t)s[0], (int64_t)s[1]));
         return r;  // no gradient for the targets
@@ -381,7 +402,7 @@ template <typename T> struct DropoutFused : Module<T> {
 };
 
 template <typename T> NodeId cce_loss_fused(AutoFerroxEngine<T>& g, NodeId predictions, NodeId targets) {
-    return g.apply_operation(std::make_unique<SoftmaxCEOp<T>>(), {predictions, targets});
+    return g.apply_operation(std::make_unique<SoftmaxCEOp<T>>(&g), {predictions, targets});
 }
 
 // SGD with every parameter of a group updated in one launch (fx_sgd_step_multi / fx_sgd_momentum_step_multi); same

@@ -315,6 +315,11 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
     int fx_softmax_ce_fwd_##S(fx_ctx* ctx, const T* logits, const T* targets, T* probs, T* loss, int64_t B, int64_t C); \
     int fx_softmax_ce_bwd_##S(fx_ctx* ctx, const T* probs, const T* targets, const T* grad_loss, T* dlogits, int64_t B, \
                               int64_t C);                                                                              \
+    /* The forward pass plus d logits for an upstream gradient of exactly 1 -- what backward() seeds a scalar loss     \
+       with (src/graph/mod.rs:700-733) -- in the same launch(es): probs and loss have the bits of fx_softmax_ce_fwd,   \
+       dlogits those of fx_softmax_ce_bwd on a device 1.  For a training step whose loss is the root of the tape. */   \
+    int fx_softmax_ce_fwd_unit_grad_##S(fx_ctx* ctx, const T* logits, const T* targets, T* probs, T* loss, T* dlogits, \
+                                        int64_t B, int64_t C);                                                         \
     /* Adam::step for one parameter, in place on p, m, v (src/nn/optim/adam.rs:288-358, no amsgrad):                   \
        m = m*b1 + g*(1-b1); v = v*b2 + (g*g)*(1-b2); p = p - ((m/bc1)/(sqrt(v/bc2)+eps))*lr [- p*(wd*lr)], with        \
        bc1 = 1-max(b1^t,1e-8), bc2 = 1-max(b2^t,1e-8) computed by the caller (adam.rs:110-126).  Same operations in    \

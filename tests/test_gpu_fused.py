@@ -82,6 +82,10 @@ def test_softmax_ce_fwd_bwd_vs_oracle(ctx, train, dtype):
         d = ctx.softmax_ce_bwd(probs, ctx.upload(y), ctx.upload(gl)).numpy()
         od = train.softmax_ce_backward(probs.numpy(), y, gl[0])
         assert np.abs(d - od).max() <= 8 * tol * max(np.abs(od).max(), 1e-30), (B, C)
+        # forward + gradient for a unit upstream gradient in one call: the bits of the two calls
+        p1, l1, d1 = ctx.softmax_ce_fwd_unit_grad(ctx.upload(x), ctx.upload(y))
+        assert np.array_equal(p1.numpy(), probs.numpy()) and np.array_equal(l1.numpy(), loss.numpy()), (B, C)
+        assert np.array_equal(d1.numpy(), ctx.softmax_ce_bwd(probs, ctx.upload(y), ctx.upload(np.array([1.0], dtype))).numpy()), (B, C)
         # textbook check where the clamp is inactive: torch log_softmax in float64
         if C > 1 and B < 3:
             tx = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
