@@ -63,19 +63,26 @@ __device__ __forceinline__ double shfl_down_t(double v, int d) { return __shfl_d
 __device__ __forceinline__ float shfl_down_t(float v, int d) { return __shfl_down(v, d, 64); }
 
 // Accumulator: value (+ index for the extrema).  IS_MAX: 0 = sum (ignores idx), 1 = maximum, 2 = minimum,
-// 3 = product (ignores idx; kernels/reduction.cu:232-301 starts from 1 and multiplies).
+// 3 = product (ignores idx; kernels/reduction.cu:232-301 starts from 1 and multiplies), 4 / 5 = maximum / minimum whose
+// position nobody asked for: the same comparisons on the values, without the 64-bit index that rides along in 1 / 2
+// (three more selects and a 64-bit add per element: 48.7 against 45.4 us for the sum over 2^26 floats).
 #define EXTREMUM(M) ((M) == 1 || (M) == 2)
 // The extrema start from the lowest / highest finite T and take strictly greater / smaller values
 // (cpu.rs:1231-1234, 1240-1252), so the first position attaining the extremum wins.
 template <typename T, int IS_MAX> struct Acc {
     T v;
     i64 i;
-    __device__ __forceinline__ void init() { v = IS_MAX == 1 ? lowest<T>() : IS_MAX == 2 ? -lowest<T>() : IS_MAX == 3 ? T(1) : T(0); i = NO_INDEX; }
+    __device__ __forceinline__ void init() {
+        v = (IS_MAX == 1 || IS_MAX == 4) ? lowest<T>() : (IS_MAX == 2 || IS_MAX == 5) ? -lowest<T>() : IS_MAX == 3 ? T(1) : T(0);
+        i = NO_INDEX;
+    }
     // element x at axis position p, visited in increasing p by this thread
     __device__ __forceinline__ void take(T x, i64 p) {
         if (IS_MAX == 1) { if (x > v) { v = x; i = p; } }
         else if (IS_MAX == 2) { if (x < v) { v = x; i = p; } }
         else if (IS_MAX == 3) v = v * x;
+        else if (IS_MAX == 4) { if (x > v) v = x; }
+        else if (IS_MAX == 5) { if (x < v) v = x; }
         else v = v + x;
     }
     // merge another accumulator (any order): ties go to the smaller index
@@ -83,6 +90,8 @@ template <typename T, int IS_MAX> struct Acc {
         if (IS_MAX == 1) { if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; } }
         else if (IS_MAX == 2) { if (ov < v || (ov == v && oi < i)) { v = ov; i = oi; } }
         else if (IS_MAX == 3) v = v * ov;
+        else if (IS_MAX == 4) { if (ov > v) v = ov; }
+        else if (IS_MAX == 5) { if (ov < v) v = ov; }
         else v = v + ov;
     }
 };
@@ -300,6 +309,10 @@ struct PartialSpace {
 template <typename T, int IS_MAX>
 int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i64 inner, T scale, const char* what,
            const PartialSpace& space = PartialSpace()) {
+    if constexpr (IS_MAX == 1 || IS_MAX == 2) {
+        // no position wanted: the value-only accumulator (same values; the scale of an extremum is 1)
+        if (idx_out == nullptr) return reduce<T, IS_MAX + 3>(c, in, out, nullptr, outer, axis, inner, T(1), what, space);
+    }
     FX_CHECK_CTX(c);
     FX_REQUIRE(outer >= 0 && axis >= 1 && inner >= 0, "%s: bad view [%lld, %lld, %lld]", what, (long long)outer,
                (long long)axis, (long long)inner);

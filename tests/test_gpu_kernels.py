@@ -222,6 +222,11 @@ def test_reduce_every_axis(ctx, orc, dtype):
             rv, ri = orc.reduce_axis("max", x, axis, want_idx=True)
             assert np.array_equal(v.numpy(), rv), ("max", shape, axis)
             assert np.array_equal(i, ri) and np.array_equal(i, np.argmax(x, axis=axis)), ("argmax", shape, axis)
+            # without the positions (the value-only accumulator): the same values, and the minimum likewise
+            assert np.array_equal(ctx.reduce("max", dx, axis).numpy(), rv), ("max, no index", shape, axis)
+            mv, mi = ctx.reduce("min", dx, axis, want_idx=True)
+            assert np.array_equal(mv.numpy(), x.min(axis=axis)) and np.array_equal(mi, np.argmin(x, axis=axis)), ("min", shape, axis)
+            assert np.array_equal(ctx.reduce("min", dx, axis).numpy(), x.min(axis=axis)), ("min, no index", shape, axis)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -247,6 +252,7 @@ def test_reduce_max_identity_and_nan(ctx, orc):
     rv, ri = orc.reduce_axis("max", x, 1, want_idx=True)
     assert np.array_equal(v.numpy(), rv) and np.array_equal(i, ri)
     assert v.numpy()[0] == lowest and i[0] == 0 and i[1] == 2
+    assert np.array_equal(ctx.reduce("max", ctx.upload(x), 1).numpy(), rv)  # value-only accumulator: same identity, NaN never taken
 
 
 def test_reference_reduction_vectors(ctx, golden):

@@ -46,6 +46,10 @@ def test_noalloc_reduce_max_refuses_oversized_partials():
         outer, axis, inner = 1, 32768, 512
         a = ctx.fill((outer * axis * inner,), 1.0, np.float32)
         out = ctx.empty((outer * inner,), np.float32)
+        idx = capi._RawI64(ctx, outer * inner)
         with pytest.raises(capi.FerroxHipError) as e:
-            capi.check(capi.lib.fx_reduce_max_noalloc_f32(ctx.h, a.ptr, out.ptr, None, outer, axis, inner))
+            capi.check(capi.lib.fx_reduce_max_noalloc_f32(ctx.h, a.ptr, out.ptr, idx.ptr, outer, axis, inner))
         assert e.value.code == 4 and "fixed scratch" in e.value.message
+        # without the positions the partials are the values alone (2.1 MB): they fit, and the maxima come out
+        capi.check(capi.lib.fx_reduce_max_noalloc_f32(ctx.h, a.ptr, out.ptr, None, outer, axis, inner))
+        np.testing.assert_array_equal(out.numpy(), np.ones(outer * inner, np.float32))
