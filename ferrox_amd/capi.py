@@ -133,6 +133,7 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_bias_act_{_s}", _vp, _vp, _vp, _i64, _i64, _i64, _int)
     _sig(f"fx_conv2d_fwd_bias_act_{_s}", _vp, _vp, _vp, _vp, _vp, *_CONV_INTS, _int, _vp, _i64)
     _sig(f"fx_gemm_bias_act_{_s}", _vp, _int, _int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _int)
+    _sig(f"fx_gemm_tn_colsum_{_s}", _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp)
     _sig(f"fx_bias_grad_{_s}", _vp, _vp, _vp, _i64, _i64, _i64)
     _sig(f"fx_relu_bwd_bias_grad_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64)
     _sig(f"fx_softmax_ce_fwd_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64)
@@ -455,6 +456,16 @@ class Context:
         o = out or self.empty((M, N), a.dtype)
         check(self._fn("gemm", a.dtype)(self.h, int(ta), int(tb), M, N, K, a.ptr, b.ptr, o.ptr))
         return o
+
+    def gemm_tn_colsum(self, a, b):
+        """a stored [K, M], b stored [K, N]: (a^T . b, column sums of a)."""
+        K, M = a.shape
+        if b.shape[0] != K:
+            raise FerroxHipError(1, f"Matrix multiplication shape mismatch: ({M}, {K}) @ ({b.shape[0]}, {b.shape[1]})")
+        N = b.shape[1]
+        o, s = self.empty((M, N), a.dtype), self.empty((M,), a.dtype)
+        check(self._fn("gemm_tn_colsum", a.dtype)(self.h, M, N, K, a.ptr, b.ptr, o.ptr, s.ptr))
+        return o, s
 
     def im2col(self, x, kernel, stride, padding):
         B, Cc, H, W = x.shape

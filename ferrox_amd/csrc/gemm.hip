@@ -16,6 +16,9 @@ using namespace igemm;
 
 int bias_act_t(fx_ctx* c, float* y, const float* b, i64 rows, i64 cols, int act) { return fx_bias_act_f32(c, y, b, rows, cols, 1, act); }
 int bias_act_t(fx_ctx* c, double* y, const double* b, i64 rows, i64 cols, int act) { return fx_bias_act_f64(c, y, b, rows, cols, 1, act); }
+// out[m] = sum over k of a[k][m] for a stored [K, M]
+int col_sum_t(fx_ctx* c, const float* a, float* out, i64 K, i64 M) { return fx_bias_grad_f32(c, a, out, K, M, 1); }
+int col_sum_t(fx_ctx* c, const double* a, double* out, i64 K, i64 M) { return fx_bias_grad_f64(c, a, out, K, M, 1); }
 
 typedef Tile<128, 128, 16, 64, 64> TileBig;    // 4 waves, 64x64 each
 typedef Tile<64, 64, 16, 32, 32> TileSmall;    // 4 waves, 32x32 each
@@ -56,26 +59,30 @@ int run_trans(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const 
 
 // the one-launch small-product kernel; with K split over blocks, its partial results and their ordered sum (bias and ReLU in the sum's store)
 int small_launch(fx_ctx* c, const gsmall::Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K, const float* A, const float* B, float* C, const float* bias,
-                 int relu, float* part) {
-    return gsmall::run(c, pl, ta, tb, M, N, K, A, B, C, bias, relu, part);
+                 int relu, float* part, float* asum) {
+    return gsmall::run(c, pl, ta, tb, M, N, K, A, B, C, bias, relu, part, asum);
 }
 int small_launch(fx_ctx* c, const gsmall::Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K, const double* A, const double* B, double* C,
-                 const double* bias, int relu, double* part) {
-    return gsmall::run_f64(c, pl, ta, tb, M, N, K, A, B, C, bias, relu, part);
+                 const double* bias, int relu, double* part, double* asum) {
+    return gsmall::run_f64(c, pl, ta, tb, M, N, K, A, B, C, bias, relu, part, asum);
 }
+// asum (optional, only with an unsplit reduction): the row sums of op(A) from the same launch
 template <typename T>
-int small_product(fx_ctx* c, const gsmall::Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K, const T* A, const T* B, T* C, const T* bias, int relu) {
+int small_product(fx_ctx* c, const gsmall::Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K, const T* A, const T* B, T* C, const T* bias, int relu,
+                  T* asum = nullptr) {
     T* part = nullptr;
     if (pl.splits > 1) {
         part = (T*)c->get_scratch(gsmall::workspace_bytes<T>(pl, M, N));
         if (!part) return FX_ERR_OOM;
     }
-    if (int rc = small_launch(c, pl, ta, tb, M, N, K, A, B, C, bias, relu, part)) return rc;
+    if (int rc = small_launch(c, pl, ta, tb, M, N, K, A, B, C, bias, relu, part, asum)) return rc;
     return pl.splits > 1 ? launch_splitk_reduce<T>(c, part, C, M * N, pl.splits, bias, N, relu) : FX_OK;
 }
 
+// asum_done (optional): with asum != null, set when the launch that computed C also wrote asum[m] = sum over k of op(A)[m][k]
 template <typename T>
-int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B, T* C, const T* bias = nullptr, int relu = 0) {
+int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B, T* C, const T* bias = nullptr, int relu = 0, T* asum = nullptr,
+         bool* asum_done = nullptr) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(M >= 0 && N >= 0 && K >= 0, "fx_gemm: negative dimension");
     if (M == 0 || N == 0) return FX_OK;
@@ -95,12 +102,15 @@ int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B,
             if (lds_path) rc = glk::run(c, pl, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu);
             else if (!generic_only && gthin::eligible(c->num_cus, ta != 0, tb != 0, M, N, K)) {
                 lds_path = true;
-                rc = gthin::run(c, M, N, K, A, B, C, bias, relu);
+                rc = gthin::run(c, M, N, K, A, B, C, bias, relu, asum);
+                if (asum) *asum_done = true;
             } else if (!generic_only) {
                 const gsmall::Plan sp = gsmall::make_plan<float>(c->num_cus, ta != 0, tb != 0, M, N, K, A, B);
                 if (sp.ok) {
                     lds_path = true;
-                    rc = small_product<float>(c, sp, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu);
+                    const bool with_sum = asum != nullptr && sp.splits == 1;
+                    rc = small_product<float>(c, sp, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu, with_sum ? asum : nullptr);
+                    if (with_sum) *asum_done = true;
                 }
             }
         }
@@ -110,7 +120,9 @@ int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B,
                 const gsmall::Plan sp = gsmall::make_plan<double>(c->num_cus, ta != 0, tb != 0, M, N, K, A, B);
                 if (sp.ok) {
                     lds_path = true;
-                    rc = small_product<double>(c, sp, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu);
+                    const bool with_sum = asum != nullptr && sp.splits == 1;
+                    rc = small_product<double>(c, sp, ta != 0, tb != 0, M, N, K, A, B, C, bias, relu, with_sum ? asum : nullptr);
+                    if (with_sum) *asum_done = true;
                 }
             }
         }
@@ -126,6 +138,23 @@ int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B,
 }
 }  // namespace
 
+// C[M,N] = A^T . B for A stored [K, M] and B stored [K, N], plus colsum[m] = sum over k of A[k][m]: the weight and the bias
+// gradient of a Linear layer from its upstream gradient A = dY [batch, out] and its input B = X [batch, in].  Small and thin
+// products compute the sums in the product's launch; the others run the bias-gradient kernel after it.
+template <typename T>
+int gemm_tn_colsum(fx_ctx* c, i64 M, i64 N, i64 K, const T* A, const T* B, T* C, T* colsum) {
+    FX_REQUIRE(colsum != nullptr, "fx_gemm_tn_colsum: null pointer");
+    FX_REQUIRE(M >= 1 && N >= 1 && K >= 1, "fx_gemm_tn_colsum: empty dimension");
+    bool done = false;
+    if (int rc = gemm<T>(c, 1, 0, M, N, K, A, B, C, nullptr, 0, colsum, &done)) return rc;
+    return done ? FX_OK : col_sum_t(c, A, colsum, K, M);
+}
+extern "C" int fx_gemm_tn_colsum_f32(fx_ctx* c, int64_t M, int64_t N, int64_t K, const float* A, const float* B, float* C, float* colsum) {
+    return gemm_tn_colsum<float>(c, M, N, K, A, B, C, colsum);
+}
+extern "C" int fx_gemm_tn_colsum_f64(fx_ctx* c, int64_t M, int64_t N, int64_t K, const double* A, const double* B, double* C, double* colsum) {
+    return gemm_tn_colsum<double>(c, M, N, K, A, B, C, colsum);
+}
 extern "C" int fx_gemm_f32(fx_ctx* c, int ta, int tb, int64_t M, int64_t N, int64_t K, const float* A, const float* B, float* C) {
     return gemm<float>(c, ta, tb, M, N, K, A, B, C);
 }

@@ -32,6 +32,7 @@ struct Params {
     int G;       // groups per wave
     int kz;      // K per block when the grid's z dimension splits K (a multiple of 8 * WAVES * G ... see run), else K
     i64 zstride; // elements between the partial results of consecutive z (0 when K is not split)
+    float* asum; // optional (K not split): asum[m] = sum over k of op(A)[m][k], written by the first block of every tile row
 };
 
 // KC: the operand is stored [rows][K] (k contiguous, K % 4 == 0, 16-byte aligned); else [K][rows].
@@ -50,6 +51,7 @@ __device__ __forceinline__ void load_group(const float* __restrict__ base, int r
 template <bool AKC, bool BKC>
 __global__ __launch_bounds__(NT) void small_kernel(const Params p) {
     __shared__ float red[WAVES * 16 * 64];
+    __shared__ float rsum[WAVES * 64];
     const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, l32 = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
@@ -70,6 +72,8 @@ __global__ __launch_bounds__(NT) void small_kernel(const Params p) {
     f32x16 acc;
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+    const bool want_asum = p.asum != nullptr && blockIdx.x == 0;  // block-uniform
+    float srow = 0.f;  // this lane's share of the sum of row am of op(A): its k in increasing order
 #pragma unroll
     for (int g = 0; g < MAXG; ++g) {
         if (g < p.G) {
@@ -78,12 +82,24 @@ __global__ __launch_bounds__(NT) void small_kernel(const Params p) {
             for (int j = 0; j < 4; ++j) {
                 const bool in = k + j < kend;
                 acc = __builtin_amdgcn_mfma_f32_32x32x2f32(in ? a[g][j] : 0.f, in ? b[g][j] : 0.f, acc, 0, 0, 0);
+                if (want_asum) srow = srow + (in ? a[g][j] : 0.f);
             }
         }
     }
 #pragma unroll
     for (int e = 0; e < 16; ++e) red[(wave * 16 + e) * 64 + lane] = acc[e];
+    if (want_asum) rsum[wave * 64 + lane] = srow;
     __syncthreads();
+    if (want_asum && wave == WAVES - 1 && h == 0 && m0 + l32 < p.M) {  // the 16 shares of a row in (wave, half) order
+        float v = rsum[l32];
+        v = v + rsum[32 + l32];
+#pragma unroll
+        for (int q = 1; q < WAVES; ++q) {
+            v = v + rsum[q * 64 + l32];
+            v = v + rsum[q * 64 + 32 + l32];
+        }
+        p.asum[m0 + l32] = v;
+    }
     // wave w finishes accumulator elements 2 w and 2 w + 1: the eight sums in wave order, then the bias kernel's operations
     const int n = n0 + l32;
 #pragma unroll
@@ -121,6 +137,7 @@ struct ParamsD {
     int G;  // groups per wave
     int kz;
     i64 zstride;
+    double* asum;  // optional, as in Params
 };
 
 template <bool KC>
@@ -154,6 +171,8 @@ __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
         for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[a][b][e] = 0.;
+    const bool want_asum = p.asum != nullptr && blockIdx.x == 0;  // block-uniform
+    double srow0 = 0., srow1 = 0.;  // this lane's shares of the sums of rows am0 and am1 of op(A): its k in increasing order
     for (int gb = 0; gb < p.G; gb += MAXG_D) {  // scalar loop: batches of MAXG_D groups
         double a0[MAXG_D][2], a1[MAXG_D][2], b0[MAXG_D][2], b1[MAXG_D][2];
 #pragma unroll
@@ -178,6 +197,7 @@ __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
                     acc[0][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(x0, y1, acc[0][1], 0, 0, 0);
                     acc[1][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(x1, y0, acc[1][0], 0, 0, 0);
                     acc[1][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(x1, y1, acc[1][1], 0, 0, 0);
+                    if (want_asum) { srow0 = srow0 + x0; srow1 = srow1 + x1; }
                 }
             }
         }
@@ -204,6 +224,24 @@ __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
                 if (p.relu) v = v > 0. ? v : 0.;
             }
             p.C[(i64)blockIdx.z * p.zstride + (i64)m * p.N + n] = v;
+        }
+    }
+    if (want_asum) {  // block-uniform: the row sums go through the same LDS once the closing sum has read it
+        __syncthreads();
+        red_d[(wave * 2 + 0) * 64 + lane] = srow0;
+        red_d[(wave * 2 + 1) * 64 + lane] = srow1;
+        __syncthreads();
+        if (wave == WAVES - 1 && lane < 32 && m0 + lane < p.M) {  // row m0 + lane: its 32 shares in (wave, quarter) order
+            const int r = lane >> 4, i = lane & 15;
+            double v = 0.;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w)
+#pragma unroll
+                for (int qq = 0; qq < 4; ++qq) {
+                    const double t = red_d[(w * 2 + r) * 64 + qq * 16 + i];
+                    v = (w == 0 && qq == 0) ? t : v + t;
+                }
+            p.asum[m0 + lane] = v;
         }
     }
 }
@@ -249,10 +287,12 @@ inline Plan make_plan(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, const 
 template <typename T> inline i64 workspace_bytes(const Plan& pl, i64 M, i64 N) { return pl.splits > 1 ? (i64)pl.splits * M * N * (i64)sizeof(T) : 0; }
 
 // part: workspace_bytes() of scratch when pl.splits > 1 (the caller then adds the partial results, with the bias)
+// asum (optional, only with pl.splits == 1): receives the row sums of op(A)
 inline int run_f64(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K, const double* A, const double* B, double* C, const double* bias,
-                   int relu, double* part) {
+                   int relu, double* part, double* asum = nullptr) {
     const bool split = pl.splits > 1;
-    ParamsD p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0};
+    FX_REQUIRE(!(split && asum), "small product: row sums need an unsplit reduction");
+    ParamsD p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0, asum};
     const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32), (unsigned)pl.splits);
     const size_t lds = (size_t)WAVES * 16 * 64 * sizeof(double);
     if (!ta && !tb) small_kernel_f64<true, false><<<grid, dim3(NT), lds, c->stream>>>(p);
@@ -264,9 +304,10 @@ inline int run_f64(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i6
 }
 
 inline int run(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K, const float* A, const float* B, float* C, const float* bias, int relu,
-               float* part) {
+               float* part, float* asum = nullptr) {
     const bool split = pl.splits > 1;
-    Params p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0};
+    FX_REQUIRE(!(split && asum), "small product: row sums need an unsplit reduction");
+    Params p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0, asum};
     const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32), (unsigned)pl.splits);
     if (!ta && !tb) small_kernel<true, false><<<grid, dim3(NT), 0, c->stream>>>(p);
     else if (!ta && tb) small_kernel<true, true><<<grid, dim3(NT), 0, c->stream>>>(p);

@@ -28,6 +28,7 @@ struct Params {
     int relu;
     int M, N, K;
     int as_rows;  // rows of A in LDS: the rows of K, zero padded to what the padded rounds of the last quarter index
+    float* asum;  // optional: asum[m] = sum over k of A[k][m], written by the first block
 };
 
 __global__ __launch_bounds__(NT) void thin_tn_kernel(const Params p) {
@@ -69,6 +70,14 @@ __global__ __launch_bounds__(NT) void thin_tn_kernel(const Params p) {
             if (i0 + j * NT < total) As[i0 + j * NT] = v[j];
     }
     __syncthreads();
+    const bool want_asum = p.asum != nullptr && blockIdx.x == 0;  // block-uniform
+    float* rs = As + p.as_rows * 32;                              // [16 parts][32 columns]
+    if (want_asum) {  // column m of A from LDS: part q adds rows q, q + 16, ... (rows past K are zero)
+        const int m = tid & 31, part = tid >> 5;
+        float v = 0.f;
+        for (int k = part; k < p.as_rows; k += 16) v = v + As[k * 32 + m];
+        rs[part * 32 + m] = v;
+    }
 
     f32x16 acc;
 #pragma unroll
@@ -97,6 +106,12 @@ __global__ __launch_bounds__(NT) void thin_tn_kernel(const Params p) {
         for (int e = 0; e < 16; ++e) red[(((kq - 1) * 2 + cs) * 16 + e) * 64 + lane] = acc[e];
     }
     __syncthreads();
+    if (want_asum && wave == 7 && lane < p.M) {  // the 16 parts in order
+        float v = rs[lane];
+#pragma unroll
+        for (int q = 1; q < 16; ++q) v = v + rs[q * 32 + lane];
+        p.asum[lane] = v;
+    }
     if (kq == 0 && n < p.N) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
@@ -119,7 +134,7 @@ inline int as_rows(i64 K) {
     const i64 pairs = (K + 1) / 2, pq = (pairs + KQ - 1) / KQ;
     return (int)(2 * ((KQ - 1) * pq + (pq + 2 * U - 1) / (2 * U) * (2 * U)));
 }
-inline size_t lds_bytes(i64 K) { return ((size_t)as_rows(K) * 32 + (KQ - 1) * 2 * 16 * 64) * sizeof(float); }
+inline size_t lds_bytes(i64 K) { return ((size_t)as_rows(K) * 32 + (KQ - 1) * 2 * 16 * 64 + 16 * 32) * sizeof(float); }
 
 // TN products this kernel takes: the general path needs two launches (split K) and stages B in 64-byte pieces.
 inline bool eligible(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K) {
@@ -128,8 +143,8 @@ inline bool eligible(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K) {
            N < (1ll << 31) - BN;
 }
 
-inline int run(fx_ctx* c, i64 M, i64 N, i64 K, const float* A, const float* B, float* C, const float* bias, int relu) {
-    Params p{A, B, C, bias, relu, (int)M, (int)N, (int)K, as_rows(K)};
+inline int run(fx_ctx* c, i64 M, i64 N, i64 K, const float* A, const float* B, float* C, const float* bias, int relu, float* asum = nullptr) {
+    Params p{A, B, C, bias, relu, (int)M, (int)N, (int)K, as_rows(K), asum};
     static const hipError_t attr = hipFuncSetAttribute((const void*)thin_tn_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT);
     FX_HIP_CHECK(attr);
     thin_tn_kernel<<<dim3((unsigned)fx::ceil_div(N, (i64)BN)), dim3(NT), lds_bytes(K), c->stream>>>(p);

@@ -278,6 +278,12 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
                                    int64_t ph, int64_t pw, int act, void* workspace, int64_t ws_bytes);                \
     int fx_gemm_bias_act_##S(fx_ctx* ctx, int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const T* A,       \
                              const T* B, const T* bias, T* C, int act);                                                \
+    /* Linear's weight and bias gradient in one call (nn/layers/linear.rs:152-308: MatMul::gradient, ops/matrix.rs:     \
+       34-55, and reduce_gradient_for_broadcasting, ops/basic.rs:10-53): C[M,N] = A^T . B for A = dY stored [K, M] and  \
+       B = X stored [K, N] -- the values of fx_gemm(1, 0, ...) -- and colsum[m] = sum over k of A[k][m], summed in a    \
+       fixed order of its own (equal to fx_bias_grad(A, K, M, 1) up to rounding).  Small and thin products write the    \
+       sums from the product's launch; the others run the bias-gradient kernel after it. */                            \
+    int fx_gemm_tn_colsum_##S(fx_ctx* ctx, int64_t M, int64_t N, int64_t K, const T* A, const T* B, T* C, T* colsum);  \
     /* BatchNorm, src/nn/layers/norm.rs:127-336, on x viewed as [outer, C, inner] ([N,C,H,W]: outer = N, inner = H*W;   \
        [N,F]: C = F, inner = 1).  stats: mean[C] and biased variance[C] of every channel in one read of x (the         \
        reference's Mean, Sub, Mul, Mean chain), and, when the pointers are not NULL, the running update                \

@@ -417,6 +417,27 @@ def test_gemm_small_products_all_layouts(ctx, dtype):
     assert np.array_equal(np.isinf(got), np.isinf(ref)) and np.array_equal(np.isnan(got), np.isnan(ref))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_tn_with_column_sums(ctx, dtype):
+    """Linear's weight + bias gradient in one call: the product has the bits of fx_gemm(1, 0), the column sums of dY are exact to
+    rounding (one-launch small and thin products, a K that is split over blocks, the general tiles with the sums in a second launch)."""
+    rng = np.random.default_rng(57)
+    tol = TOL[np.dtype(dtype)]
+    # K (batch), M (out), N (in)
+    for (K, M, N) in [(256, 10, 128), (256, 10, 16384), (256, 128, 256), (256, 256, 784), (64, 3, 40), (100, 33, 70), (37, 5, 9),
+                      (2048, 10, 64), (512, 600, 520), (256, 40, 16384)]:
+        a = rng.standard_normal((K, M)).astype(dtype)
+        b = rng.standard_normal((K, N)).astype(dtype)
+        da, db = ctx.upload(a), ctx.upload(b)
+        c, s = ctx.gemm_tn_colsum(da, db)
+        assert np.array_equal(c.numpy(), ctx.gemm(da, db, ta=True).numpy()), (K, M, N)
+        truth = a.astype(np.longdouble).sum(axis=0)
+        bound = tol * np.abs(a).astype(np.float64).sum(axis=0).max()
+        assert np.abs(s.numpy() - truth).max() <= bound, (K, M, N)
+        c2, s2 = ctx.gemm_tn_colsum(da, db)  # the same bits on a second run
+        assert np.array_equal(c2.numpy(), c.numpy()) and np.array_equal(s2.numpy(), s.numpy()), (K, M, N)
+
+
 def test_gemm_shape_mismatch_message(ctx):
     from ferrox_amd.capi import FerroxHipError
     a = ctx.upload(np.zeros((2, 3), np.float32))
