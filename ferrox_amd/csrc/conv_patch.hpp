@@ -427,18 +427,22 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_persist_kernel(const Params 
     };
     // The stores of a tile: a scalar base per accumulator row (SALU) and one 32-bit lane offset per pixel block, so that
     // a store costs no vector ALU work; tiles that reach past the last output channel or pixel take the checked path.
+    // The bias of the 16 output rows this lane stores, loaded at the start of a tile's last stage: in flight under that stage's
+    // MFMAs instead of between them and the stores (where every wave of the block would wait for it at the same time).
+    float bv[16];
+    auto load_bias = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int m = m0 + wm * 32 + igemm::Mfma<float>::row(e, lane);
+            bv[e] = BIAS ? p.bias[m < p.M ? m : p.M - 1] : 0.f;
+        }
+    };
     auto store_tile = [&]() __attribute__((always_inline)) {
         typedef __attribute__((address_space(1))) char gchar;
         typedef __attribute__((address_space(1))) float gfloat;
         const int mw = m0 + wm * 32;  // scalar
         float* const out = p.y + ((i64)b * p.M + mw) * p.L;
         const int wpix0 = pix0 + wn * 32 * TN;
-        float bv[16];
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const int m = mw + igemm::Mfma<float>::row(e, lane);
-            bv[e] = BIAS ? p.bias[m < p.M ? m : p.M - 1] : 0.f;
-        }
         auto rows = [&](auto checked_c) __attribute__((always_inline)) {
             constexpr bool CHECKED = decltype(checked_c)::value;
 #pragma unroll
@@ -484,6 +488,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_persist_kernel(const Params 
         const bool more = nq < qend;
         // the finished tile's coordinates are needed by its stores after the next tile's have been formed for the loads
         const int cb = b, cm0 = m0, cpix0 = pix0;
+        if (BIAS && last_ch) load_bias();
         if (more) {
             if (last_ch) geo(nq);
             prefetch(std::integral_constant<int, SET ^ 1>(), nch);

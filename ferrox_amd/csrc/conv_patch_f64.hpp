@@ -193,17 +193,22 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_f64_kernel(const Params p) {
         }
     };
     // The stores of a tile: a scalar base per accumulator row group (SALU) and one 32-bit lane offset per pixel block.
+    // The bias of the 4 output rows this lane stores, loaded at the start of a tile's last stage: in flight under that stage's
+    // MFMAs instead of between them and the stores (where every wave of the block would wait for it at the same time).
+    double bv[4];
+    auto load_bias = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int m = m0 + wave * 16 + 4 * e + kq;
+            bv[e] = BIAS ? p.bias[m < p.M ? m : p.M - 1] : 0.;
+        }
+    };
     auto store_tile = [&]() __attribute__((always_inline)) {
         typedef __attribute__((address_space(1))) char gchar;
         typedef __attribute__((address_space(1))) double gdouble;
         const int mw = m0 + wave * 16;  // scalar
         double* const out = p.y + ((i64)b * p.M + mw) * p.L;
-        double bv[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int m = mw + 4 * e + kq;
-            bv[e] = BIAS ? p.bias[m < p.M ? m : p.M - 1] : 0.;
-        }
+        if (BIAS && TN >= 8) load_bias();
         auto rows = [&](auto checked_c) __attribute__((always_inline)) {
             constexpr bool CHECKED = decltype(checked_c)::value;
 #pragma unroll
@@ -247,6 +252,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_f64_kernel(const Params p) {
         const bool more = nq < qend;
         // the finished tile's coordinates are needed by its stores after the next tile's have been formed for the loads
         const int cb = b, cm0 = m0, cpix0 = pix0;
+        if (BIAS && last_ch && TN < 8) load_bias();  // the widest tile has no registers to spare during the stage
         if (more) {
             if (last_ch) geo(nq);
             prefetch(std::integral_constant<int, SET ^ 1>(), nch);
