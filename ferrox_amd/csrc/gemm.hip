@@ -149,6 +149,41 @@ int gemm_tn_colsum(fx_ctx* c, i64 M, i64 N, i64 K, const T* A, const T* B, T* C,
     if (int rc = gemm<T>(c, 1, 0, M, N, K, A, B, C, nullptr, 0, colsum, &done)) return rc;
     return done ? FX_OK : col_sum_t(c, A, colsum, K, M);
 }
+// Linear's backward products in one call: dX[B, in] = dY[B, out] . W[out, in], dW[out, in] = dY^T . X[B, in] and (optionally)
+// db[out] = the column sums of dY.  Where both products are small ones (each would run the one-launch small-product kernel on its
+// own) they share a launch; the results have the bits of the separate calls either way.
+template <typename T>
+int linear_bwd(fx_ctx* c, i64 Bn, i64 I, i64 O, const T* g, const T* W, const T* X, T* dX, T* dW, T* db) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(g && W && X && dX && dW, "fx_linear_bwd: null pointer");
+    FX_REQUIRE(Bn >= 1 && I >= 1 && O >= 1 && Bn < (1ll << 31) && I < (1ll << 31) && O < (1ll << 31), "fx_linear_bwd: bad dimensions");
+    static const bool generic_only = std::getenv("FX_GEMM_GENERIC") != nullptr;
+    if (!generic_only) {
+        bool other = false;  // a product that gemm() would give to the slab or the thin kernel
+        if constexpr (sizeof(T) == 4) {
+            other = glk::make_plan(c->num_cus, false, false, Bn, I, O, O, I).ok || glk::make_plan(c->num_cus, true, false, O, I, Bn, O, I).ok ||
+                    gthin::eligible(c->num_cus, false, false, Bn, I, O) || gthin::eligible(c->num_cus, true, false, O, I, Bn);
+        }
+        if (!other) {
+            const gsmall::Plan p0 = gsmall::make_plan<T>(c->num_cus, false, false, Bn, I, O, g, W);
+            const gsmall::Plan p1 = gsmall::make_plan<T>(c->num_cus, true, false, O, I, Bn, g, X);
+            if (p0.ok && p1.ok && p0.splits == 1 && p1.splits == 1) {
+                std::lock_guard<std::mutex> lk(c->launch_mutex);
+                return gsmall::run_pair(c, p0, p1, Bn, I, O, g, W, dX, O, I, Bn, g, X, dW, db);
+            }
+        }
+    }
+    if (int rc = gemm<T>(c, 0, 0, Bn, I, O, g, W, dX)) return rc;
+    return db ? gemm_tn_colsum<T>(c, O, I, Bn, g, X, dW, db) : gemm<T>(c, 1, 0, O, I, Bn, g, X, dW);
+}
+extern "C" int fx_linear_bwd_f32(fx_ctx* c, int64_t B, int64_t in, int64_t out, const float* dY, const float* W, const float* X, float* dX,
+                                 float* dW, float* db) {
+    return linear_bwd<float>(c, B, in, out, dY, W, X, dX, dW, db);
+}
+extern "C" int fx_linear_bwd_f64(fx_ctx* c, int64_t B, int64_t in, int64_t out, const double* dY, const double* W, const double* X, double* dX,
+                                 double* dW, double* db) {
+    return linear_bwd<double>(c, B, in, out, dY, W, X, dX, dW, db);
+}
 extern "C" int fx_gemm_tn_colsum_f32(fx_ctx* c, int64_t M, int64_t N, int64_t K, const float* A, const float* B, float* C, float* colsum) {
     return gemm_tn_colsum<float>(c, M, N, K, A, B, C, colsum);
 }

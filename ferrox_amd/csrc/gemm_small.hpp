@@ -48,15 +48,14 @@ __device__ __forceinline__ void load_group(const float* __restrict__ base, int r
     }
 }
 
+// The work of one block: tile (bx, by) of the product, range bz of K.  red: WAVES * 16 * 64 floats of LDS, rsum: WAVES * 64.
 template <bool AKC, bool BKC>
-__global__ __launch_bounds__(NT) void small_kernel(const Params p) {
-    __shared__ float red[WAVES * 16 * 64];
-    __shared__ float rsum[WAVES * 64];
+__device__ __forceinline__ void small_body(const Params& p, float* red, float* rsum, int bx, int by, int bz) {
     const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, l32 = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int m0 = by * 32, n0 = bx * 32;
     const int am = min(m0 + l32, p.M - 1), bn = min(n0 + l32, p.N - 1);  // past the edge: a valid row / column, result unused
-    const int kbase = blockIdx.z * p.kz, kend = min(p.K, kbase + p.kz);    // this block's range of K (all of it unless K is split over z)
+    const int kbase = bz * p.kz, kend = min(p.K, kbase + p.kz);            // this block's range of K (all of it unless K is split over z)
     const int g0 = wave * p.G;
     const float bias_n = p.bias ? p.bias[bn] : 0.f;  // loaded up front: its latency stays off the closing sum
 
@@ -72,7 +71,7 @@ __global__ __launch_bounds__(NT) void small_kernel(const Params p) {
     f32x16 acc;
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] = 0.f;
-    const bool want_asum = p.asum != nullptr && blockIdx.x == 0;  // block-uniform
+    const bool want_asum = p.asum != nullptr && bx == 0;  // block-uniform
     float srow = 0.f;  // this lane's share of the sum of row am of op(A): its k in increasing order
 #pragma unroll
     for (int g = 0; g < MAXG; ++g) {
@@ -114,8 +113,29 @@ __global__ __launch_bounds__(NT) void small_kernel(const Params p) {
                 v = v + bias_n;
                 if (p.relu) v = v > 0.f ? v : 0.f;
             }
-            p.C[(i64)blockIdx.z * p.zstride + (i64)m * p.N + n] = v;
+            p.C[(i64)bz * p.zstride + (i64)m * p.N + n] = v;
         }
+    }
+}
+
+template <bool AKC, bool BKC>
+__global__ __launch_bounds__(NT) void small_kernel(const Params p) {
+    __shared__ float red[WAVES * 16 * 64];
+    __shared__ float rsum[WAVES * 64];
+    small_body<AKC, BKC>(p, red, rsum, blockIdx.x, blockIdx.y, blockIdx.z);
+}
+
+// Two independent products in one launch, blockIdx.z picks the product (neither splits K): the data and the weight gradient of a
+// Linear layer, dX = dY . W (both operands as stored: A k-contiguous) and dW = dY^T . X (A stored [K, M]).  A block outside its
+// product's tile range leaves at once.
+__global__ __launch_bounds__(NT) void small_pair_kernel(const Params p0, const Params p1) {
+    __shared__ float red[WAVES * 16 * 64];
+    __shared__ float rsum[WAVES * 64];
+    const int bx = blockIdx.x, by = blockIdx.y;
+    if (blockIdx.z == 0) {
+        if (bx * 32 < p0.N && by * 32 < p0.M) small_body<true, false>(p0, red, rsum, bx, by, 0);
+    } else {
+        if (bx * 32 < p1.N && by * 32 < p1.M) small_body<false, false>(p1, red, rsum, bx, by, 0);
     }
 }
 
@@ -152,15 +172,15 @@ __device__ __forceinline__ void load_group_d(const double* __restrict__ base, in
     }
 }
 
+// red_d: [8 waves][16 elements][64 lanes] doubles of LDS
 template <bool AKC, bool BKC>
-__global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
-    extern __shared__ __align__(16) double red_d[];  // [8 waves][16 elements][64 lanes]
+__device__ __forceinline__ void small_body_f64(const ParamsD& p, double* red_d, int bx, int by, int bz) {
     const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, l16 = lane & 15;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int m0 = by * 32, n0 = bx * 32;
     const int am0 = min(m0 + l16, p.M - 1), am1 = min(m0 + 16 + l16, p.M - 1);  // past the edge: a valid row / column, result unused
     const int bn0 = min(n0 + l16, p.N - 1), bn1 = min(n0 + 16 + l16, p.N - 1);
-    const int kbase = blockIdx.z * p.kz, kend = min(p.K, kbase + p.kz);
+    const int kbase = bz * p.kz, kend = min(p.K, kbase + p.kz);
     const int g0 = wave * p.G;
     // this wave finishes the column block (wave / 2) % 2 in the closing sum; its bias is loaded up front
     const double bias_n = p.bias ? p.bias[(wave >> 1) & 1 ? bn1 : bn0] : 0.;
@@ -171,7 +191,7 @@ __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
         for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[a][b][e] = 0.;
-    const bool want_asum = p.asum != nullptr && blockIdx.x == 0;  // block-uniform
+    const bool want_asum = p.asum != nullptr && bx == 0;  // block-uniform
     double srow0 = 0., srow1 = 0.;  // this lane's shares of the sums of rows am0 and am1 of op(A): its k in increasing order
     for (int gb = 0; gb < p.G; gb += MAXG_D) {  // scalar loop: batches of MAXG_D groups
         double a0[MAXG_D][2], a1[MAXG_D][2], b0[MAXG_D][2], b1[MAXG_D][2];
@@ -223,7 +243,7 @@ __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
                 v = v + bias_n;
                 if (p.relu) v = v > 0. ? v : 0.;
             }
-            p.C[(i64)blockIdx.z * p.zstride + (i64)m * p.N + n] = v;
+            p.C[(i64)bz * p.zstride + (i64)m * p.N + n] = v;
         }
     }
     if (want_asum) {  // block-uniform: the row sums go through the same LDS once the closing sum has read it
@@ -243,6 +263,22 @@ __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
                 }
             p.asum[m0 + lane] = v;
         }
+    }
+}
+
+template <bool AKC, bool BKC>
+__global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
+    extern __shared__ __align__(16) double red_d[];
+    small_body_f64<AKC, BKC>(p, red_d, blockIdx.x, blockIdx.y, blockIdx.z);
+}
+
+__global__ __launch_bounds__(NT) void small_pair_kernel_f64(const ParamsD p0, const ParamsD p1) {  // as small_pair_kernel
+    extern __shared__ __align__(16) double red_d[];
+    const int bx = blockIdx.x, by = blockIdx.y;
+    if (blockIdx.z == 0) {
+        if (bx * 32 < p0.N && by * 32 < p0.M) small_body_f64<true, false>(p0, red_d, bx, by, 0);
+    } else {
+        if (bx * 32 < p1.N && by * 32 < p1.M) small_body_f64<false, false>(p1, red_d, bx, by, 0);
     }
 }
 
@@ -313,6 +349,29 @@ inline int run(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K,
     else if (!ta && tb) small_kernel<true, true><<<grid, dim3(NT), 0, c->stream>>>(p);
     else if (ta && !tb) small_kernel<false, false><<<grid, dim3(NT), 0, c->stream>>>(p);
     else small_kernel<false, true><<<grid, dim3(NT), 0, c->stream>>>(p);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
+// dX[M0,N0] = A0 . B0 (A0 stored [M0,K0], B0 stored [K0,N0]) and dW[M1,N1] = A1^T . B1 (A1 stored [K1,M1], B1 stored [K1,N1]) in one
+// launch; both plans unsplit.  asum1 (optional): the row sums of A1^T, i.e. the column sums of A1.
+inline int run_pair(fx_ctx* c, const Plan& p0, const Plan& p1, i64 M0, i64 N0, i64 K0, const float* A0, const float* B0, float* C0, i64 M1, i64 N1,
+                    i64 K1, const float* A1, const float* B1, float* C1, float* asum1) {
+    FX_REQUIRE(p0.splits == 1 && p1.splits == 1, "small product pair: unsplit reductions only");
+    Params a{A0, B0, C0, nullptr, 0, (int)M0, (int)N0, (int)K0, p0.G, p0.kz, 0, nullptr};
+    Params b{A1, B1, C1, nullptr, 0, (int)M1, (int)N1, (int)K1, p1.G, p1.kz, 0, asum1};
+    const dim3 grid((unsigned)fx::ceil_div(std::max(N0, N1), (i64)32), (unsigned)fx::ceil_div(std::max(M0, M1), (i64)32), 2);
+    small_pair_kernel<<<grid, dim3(NT), 0, c->stream>>>(a, b);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+inline int run_pair(fx_ctx* c, const Plan& p0, const Plan& p1, i64 M0, i64 N0, i64 K0, const double* A0, const double* B0, double* C0, i64 M1,
+                    i64 N1, i64 K1, const double* A1, const double* B1, double* C1, double* asum1) {
+    FX_REQUIRE(p0.splits == 1 && p1.splits == 1, "small product pair: unsplit reductions only");
+    ParamsD a{A0, B0, C0, nullptr, 0, (int)M0, (int)N0, (int)K0, p0.G, p0.kz, 0, nullptr};
+    ParamsD b{A1, B1, C1, nullptr, 0, (int)M1, (int)N1, (int)K1, p1.G, p1.kz, 0, asum1};
+    const dim3 grid((unsigned)fx::ceil_div(std::max(N0, N1), (i64)32), (unsigned)fx::ceil_div(std::max(M0, M1), (i64)32), 2);
+    small_pair_kernel_f64<<<grid, dim3(NT), (size_t)WAVES * 16 * 64 * sizeof(double), c->stream>>>(a, b);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

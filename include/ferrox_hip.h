@@ -284,6 +284,12 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
        fixed order of its own (equal to fx_bias_grad(A, K, M, 1) up to rounding).  Small and thin products write the    \
        sums from the product's launch; the others run the bias-gradient kernel after it. */                            \
     int fx_gemm_tn_colsum_##S(fx_ctx* ctx, int64_t M, int64_t N, int64_t K, const T* A, const T* B, T* C, T* colsum);  \
+    /* Linear's backward products in one call (nn/layers/linear.rs:152-308, MatMul::gradient ops/matrix.rs:34-55):      \
+       dX[B, in] = dY[B, out] . W[out, in], dW[out, in] = dY^T . X[B, in] and, with db != NULL, db[out] = the column    \
+       sums of dY.  dX and dW have the bits of fx_gemm(0, 0, ...) and fx_gemm(1, 0, ...), db those of                   \
+       fx_gemm_tn_colsum; two small products share one launch. */                                                      \
+    int fx_linear_bwd_##S(fx_ctx* ctx, int64_t B, int64_t in, int64_t out, const T* dY, const T* W, const T* X, T* dX, \
+                          T* dW, T* db);                                                                               \
     /* BatchNorm, src/nn/layers/norm.rs:127-336, on x viewed as [outer, C, inner] ([N,C,H,W]: outer = N, inner = H*W;   \
        [N,F]: C = F, inner = 1).  stats: mean[C] and biased variance[C] of every channel in one read of x (the         \
        reference's Mean, Sub, Mul, Mean chain), and, when the pointers are not NULL, the running update                \

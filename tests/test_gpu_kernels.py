@@ -438,6 +438,26 @@ def test_gemm_tn_with_column_sums(ctx, dtype):
         assert np.array_equal(c2.numpy(), c.numpy()) and np.array_equal(s2.numpy(), s.numpy()), (K, M, N)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_linear_backward_products_in_one_call(ctx, dtype):
+    """fx_linear_bwd: the bits of the separate calls, whether the two products share a launch (both small), or one of them is a thin /
+    large / split product and they run one after the other; with and without the bias gradient."""
+    rng = np.random.default_rng(56)
+    # B, in, out
+    for (Bn, I, O) in [(256, 256, 128), (256, 784, 256), (256, 128, 10), (256, 16384, 10), (64, 40, 33), (37, 9, 50), (512, 512, 512),
+                       (256, 64, 96), (2048, 100, 64)]:
+        dy = rng.standard_normal((Bn, O)).astype(dtype)
+        w = rng.standard_normal((O, I)).astype(dtype)
+        x = rng.standard_normal((Bn, I)).astype(dtype)
+        ddy, dw_, dx_ = ctx.upload(dy), ctx.upload(w), ctx.upload(x)
+        gx, gw, gb = ctx.linear_bwd(ddy, dw_, dx_)
+        assert np.array_equal(gx.numpy(), ctx.gemm(ddy, dw_).numpy()), ("dX", Bn, I, O)
+        rw, rb = ctx.gemm_tn_colsum(ddy, dx_)
+        assert np.array_equal(gw.numpy(), rw.numpy()) and np.array_equal(gb.numpy(), rb.numpy()), ("dW, db", Bn, I, O)
+        gx2, gw2, _ = ctx.linear_bwd(ddy, dw_, dx_, want_db=False)
+        assert np.array_equal(gx2.numpy(), gx.numpy()) and np.array_equal(gw2.numpy(), gw.numpy()), ("no db", Bn, I, O)
+
+
 def test_gemm_shape_mismatch_message(ctx):
     from ferrox_amd.capi import FerroxHipError
     a = ctx.upload(np.zeros((2, 3), np.float32))
