@@ -35,13 +35,17 @@ struct Params {
     float* asum; // optional (K not split): asum[m] = sum over k of op(A)[m][k], written by the first block of every tile row
 };
 
-// KC: the operand is stored [rows][K] (k contiguous, K % 4 == 0, 16-byte aligned); else [K][rows].
-template <bool KC>
+// KC: 1 = the operand is stored [rows][K] (k contiguous, K % 4 == 0, 16-byte aligned); 2 = the same layout read element by element
+// (any K and alignment: the short reductions of a classifier head's data gradient); 0 = stored [K][rows].
+template <int KC>
 __device__ __forceinline__ void load_group(const float* __restrict__ base, int row, int rows, int K, int k, float (&v)[4]) {
-    if constexpr (KC) {
+    if constexpr (KC == 1) {
         const int kc = min(k, K - 4);
         const float4 q = *reinterpret_cast<const float4*>(base + (i64)row * K + kc);
         v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+    } else if constexpr (KC == 2) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = base[(i64)row * K + min(k + j, K - 1)];
     } else {
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = base[(i64)min(k + j, K - 1) * rows + row];
@@ -49,7 +53,7 @@ __device__ __forceinline__ void load_group(const float* __restrict__ base, int r
 }
 
 // The work of one block: tile (bx, by) of the product, range bz of K.  red: WAVES * 16 * 64 floats of LDS, rsum: WAVES * 64.
-template <bool AKC, bool BKC>
+template <int AKC, int BKC>
 __device__ __forceinline__ void small_body(const Params& p, float* red, float* rsum, int bx, int by, int bz) {
     const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, l32 = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -118,7 +122,7 @@ __device__ __forceinline__ void small_body(const Params& p, float* red, float* r
     }
 }
 
-template <bool AKC, bool BKC>
+template <int AKC, int BKC>
 __global__ __launch_bounds__(NT) void small_kernel(const Params p) {
     __shared__ float red[WAVES * 16 * 64];
     __shared__ float rsum[WAVES * 64];
@@ -128,14 +132,15 @@ __global__ __launch_bounds__(NT) void small_kernel(const Params p) {
 // Two independent products in one launch, blockIdx.z picks the product (neither splits K): the data and the weight gradient of a
 // Linear layer, dX = dY . W (both operands as stored: A k-contiguous) and dW = dY^T . X (A stored [K, M]).  A block outside its
 // product's tile range leaves at once.
+template <int A0>  // how the first product reads its A: 1 or 2
 __global__ __launch_bounds__(NT) void small_pair_kernel(const Params p0, const Params p1) {
     __shared__ float red[WAVES * 16 * 64];
     __shared__ float rsum[WAVES * 64];
     const int bx = blockIdx.x, by = blockIdx.y;
     if (blockIdx.z == 0) {
-        if (bx * 32 < p0.N && by * 32 < p0.M) small_body<true, false>(p0, red, rsum, bx, by, 0);
+        if (bx * 32 < p0.N && by * 32 < p0.M) small_body<A0, 0>(p0, red, rsum, bx, by, 0);
     } else {
-        if (bx * 32 < p1.N && by * 32 < p1.M) small_body<false, false>(p1, red, rsum, bx, by, 0);
+        if (bx * 32 < p1.N && by * 32 < p1.M) small_body<0, 0>(p1, red, rsum, bx, by, 0);
     }
 }
 
@@ -160,12 +165,15 @@ struct ParamsD {
     double* asum;  // optional, as in Params
 };
 
-template <bool KC>
+template <int KC>
 __device__ __forceinline__ void load_group_d(const double* __restrict__ base, int row, int rows, int K, int k, double (&v)[2]) {
-    if constexpr (KC) {
+    if constexpr (KC == 1) {
         typedef double d2 __attribute__((ext_vector_type(2)));
         const d2 q = *reinterpret_cast<const d2*>(base + (i64)row * K + min(k, K - 2));
         v[0] = q.x; v[1] = q.y;
+    } else if constexpr (KC == 2) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) v[j] = base[(i64)row * K + min(k + j, K - 1)];
     } else {
 #pragma unroll
         for (int j = 0; j < 2; ++j) v[j] = base[(i64)min(k + j, K - 1) * rows + row];
@@ -173,7 +181,7 @@ __device__ __forceinline__ void load_group_d(const double* __restrict__ base, in
 }
 
 // red_d: [8 waves][16 elements][64 lanes] doubles of LDS
-template <bool AKC, bool BKC>
+template <int AKC, int BKC>
 __device__ __forceinline__ void small_body_f64(const ParamsD& p, double* red_d, int bx, int by, int bz) {
     const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, l16 = lane & 15;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -266,19 +274,20 @@ __device__ __forceinline__ void small_body_f64(const ParamsD& p, double* red_d, 
     }
 }
 
-template <bool AKC, bool BKC>
+template <int AKC, int BKC>
 __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
     extern __shared__ __align__(16) double red_d[];
     small_body_f64<AKC, BKC>(p, red_d, blockIdx.x, blockIdx.y, blockIdx.z);
 }
 
+template <int A0>
 __global__ __launch_bounds__(NT) void small_pair_kernel_f64(const ParamsD p0, const ParamsD p1) {  // as small_pair_kernel
     extern __shared__ __align__(16) double red_d[];
     const int bx = blockIdx.x, by = blockIdx.y;
     if (blockIdx.z == 0) {
-        if (bx * 32 < p0.N && by * 32 < p0.M) small_body_f64<true, false>(p0, red_d, bx, by, 0);
+        if (bx * 32 < p0.N && by * 32 < p0.M) small_body_f64<A0, 0>(p0, red_d, bx, by, 0);
     } else {
-        if (bx * 32 < p1.N && by * 32 < p1.M) small_body_f64<false, false>(p1, red_d, bx, by, 0);
+        if (bx * 32 < p1.N && by * 32 < p1.M) small_body_f64<0, 0>(p1, red_d, bx, by, 0);
     }
 }
 
@@ -288,6 +297,7 @@ __global__ __launch_bounds__(NT) void small_pair_kernel_f64(const ParamsD p0, co
 struct Plan {
     bool ok = false;
     int G = 0, kz = 0, splits = 1;
+    bool a_elems = false;  // A is k-contiguous but not readable in 16-byte pieces (K % 4, alignment): element loads
 };
 
 template <typename T>
@@ -295,8 +305,9 @@ inline Plan make_plan(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, const 
     Plan pl;
     static const bool off = [] { const char* v = getenv("FX_GEMM_SMALL"); return v && atoi(v) == 0; }();
     constexpr int KV = 16 / (int)sizeof(T);  // elements per 16-byte load of a k-contiguous operand
-    if (off || K < 32 || M < 1 || N < 1 || K >= (1ll << 30)) return pl;
-    if (!ta && (K % KV != 0 || !fx::aligned16(A))) return pl;
+    if (off || K < 1 || M < 1 || N < 1 || K >= (1ll << 30)) return pl;
+    if (K < 32 && ta) return pl;  // short reductions: only with a k-contiguous A, read element by element (the general tiles serve the others)
+    if (!ta && (K % KV != 0 || !fx::aligned16(A) || K < 32)) pl.a_elems = true;
     if (tb && (K % KV != 0 || !fx::aligned16(B))) return pl;
     const i64 tiles = fx::ceil_div(M, (i64)32) * fx::ceil_div(N, (i64)32);
     // a 32 x 32 tile re-reads each operand once per tile row / column: M N K sizeof(T) / 16 bytes through L2, kept under 32 MB (f32) / 64 MB (f64)
@@ -331,10 +342,12 @@ inline int run_f64(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i6
     ParamsD p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0, asum};
     const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32), (unsigned)pl.splits);
     const size_t lds = (size_t)WAVES * 16 * 64 * sizeof(double);
-    if (!ta && !tb) small_kernel_f64<true, false><<<grid, dim3(NT), lds, c->stream>>>(p);
-    else if (!ta && tb) small_kernel_f64<true, true><<<grid, dim3(NT), lds, c->stream>>>(p);
-    else if (ta && !tb) small_kernel_f64<false, false><<<grid, dim3(NT), lds, c->stream>>>(p);
-    else small_kernel_f64<false, true><<<grid, dim3(NT), lds, c->stream>>>(p);
+    if (!ta && pl.a_elems && !tb) small_kernel_f64<2, 0><<<grid, dim3(NT), lds, c->stream>>>(p);
+    else if (!ta && pl.a_elems) small_kernel_f64<2, 1><<<grid, dim3(NT), lds, c->stream>>>(p);
+    else if (!ta && !tb) small_kernel_f64<1, 0><<<grid, dim3(NT), lds, c->stream>>>(p);
+    else if (!ta && tb) small_kernel_f64<1, 1><<<grid, dim3(NT), lds, c->stream>>>(p);
+    else if (ta && !tb) small_kernel_f64<0, 0><<<grid, dim3(NT), lds, c->stream>>>(p);
+    else small_kernel_f64<0, 1><<<grid, dim3(NT), lds, c->stream>>>(p);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
@@ -345,10 +358,12 @@ inline int run(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K,
     FX_REQUIRE(!(split && asum), "small product: row sums need an unsplit reduction");
     Params p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0, asum};
     const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32), (unsigned)pl.splits);
-    if (!ta && !tb) small_kernel<true, false><<<grid, dim3(NT), 0, c->stream>>>(p);
-    else if (!ta && tb) small_kernel<true, true><<<grid, dim3(NT), 0, c->stream>>>(p);
-    else if (ta && !tb) small_kernel<false, false><<<grid, dim3(NT), 0, c->stream>>>(p);
-    else small_kernel<false, true><<<grid, dim3(NT), 0, c->stream>>>(p);
+    if (!ta && pl.a_elems && !tb) small_kernel<2, 0><<<grid, dim3(NT), 0, c->stream>>>(p);
+    else if (!ta && pl.a_elems) small_kernel<2, 1><<<grid, dim3(NT), 0, c->stream>>>(p);
+    else if (!ta && !tb) small_kernel<1, 0><<<grid, dim3(NT), 0, c->stream>>>(p);
+    else if (!ta && tb) small_kernel<1, 1><<<grid, dim3(NT), 0, c->stream>>>(p);
+    else if (ta && !tb) small_kernel<0, 0><<<grid, dim3(NT), 0, c->stream>>>(p);
+    else small_kernel<0, 1><<<grid, dim3(NT), 0, c->stream>>>(p);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
@@ -361,7 +376,8 @@ inline int run_pair(fx_ctx* c, const Plan& p0, const Plan& p1, i64 M0, i64 N0, i
     Params a{A0, B0, C0, nullptr, 0, (int)M0, (int)N0, (int)K0, p0.G, p0.kz, 0, nullptr};
     Params b{A1, B1, C1, nullptr, 0, (int)M1, (int)N1, (int)K1, p1.G, p1.kz, 0, asum1};
     const dim3 grid((unsigned)fx::ceil_div(std::max(N0, N1), (i64)32), (unsigned)fx::ceil_div(std::max(M0, M1), (i64)32), 2);
-    small_pair_kernel<<<grid, dim3(NT), 0, c->stream>>>(a, b);
+    if (p0.a_elems) small_pair_kernel<2><<<grid, dim3(NT), 0, c->stream>>>(a, b);
+    else small_pair_kernel<1><<<grid, dim3(NT), 0, c->stream>>>(a, b);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
@@ -371,7 +387,9 @@ inline int run_pair(fx_ctx* c, const Plan& p0, const Plan& p1, i64 M0, i64 N0, i
     ParamsD a{A0, B0, C0, nullptr, 0, (int)M0, (int)N0, (int)K0, p0.G, p0.kz, 0, nullptr};
     ParamsD b{A1, B1, C1, nullptr, 0, (int)M1, (int)N1, (int)K1, p1.G, p1.kz, 0, asum1};
     const dim3 grid((unsigned)fx::ceil_div(std::max(N0, N1), (i64)32), (unsigned)fx::ceil_div(std::max(M0, M1), (i64)32), 2);
-    small_pair_kernel_f64<<<grid, dim3(NT), (size_t)WAVES * 16 * 64 * sizeof(double), c->stream>>>(a, b);
+    const size_t lds = (size_t)WAVES * 16 * 64 * sizeof(double);
+    if (p0.a_elems) small_pair_kernel_f64<2><<<grid, dim3(NT), lds, c->stream>>>(a, b);
+    else small_pair_kernel_f64<1><<<grid, dim3(NT), lds, c->stream>>>(a, b);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

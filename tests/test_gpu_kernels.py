@@ -376,7 +376,9 @@ def test_gemm_with_one_thin_dimension(ctx, dtype):
 # small products take a one-launch kernel (32 x 32 tile per block, K split over the block's waves): every layout, ragged
 # tile edges, K with half a group of eight left over, the longest K it takes, and K not a multiple of 4 for each layout (only the
 # row/column-contiguous loads take that; the others fall back to the general tiles)
-GEMM_SMALL_SHAPES = [(33, 65, 36), (256, 512, 784), (100, 31, 1024), (1, 1, 32), (64, 64, 44), (32, 96, 250), (70, 200, 127)]
+GEMM_SMALL_SHAPES = [(33, 65, 36), (256, 512, 784), (100, 31, 1024), (1, 1, 32), (64, 64, 44), (32, 96, 250), (70, 200, 127),
+                     # short and odd reductions: a k-contiguous A read element by element (K = 10: a classifier head's data gradient)
+                     (256, 128, 10), (40, 70, 1), (65, 33, 31), (256, 256, 45)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -445,7 +447,7 @@ def test_linear_backward_products_in_one_call(ctx, dtype):
     rng = np.random.default_rng(56)
     # B, in, out
     for (Bn, I, O) in [(256, 256, 128), (256, 784, 256), (256, 128, 10), (256, 16384, 10), (64, 40, 33), (37, 9, 50), (512, 512, 512),
-                       (256, 64, 96), (2048, 100, 64)]:
+                       (256, 64, 96), (2048, 100, 64), (256, 128, 7), (100, 60, 3)]:
         dy = rng.standard_normal((Bn, O)).astype(dtype)
         w = rng.standard_normal((O, I)).astype(dtype)
         x = rng.standard_normal((Bn, I)).astype(dtype)
