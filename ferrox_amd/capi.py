@@ -134,7 +134,7 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_conv2d_fwd_bias_act_{_s}", _vp, _vp, _vp, _vp, _vp, *_CONV_INTS, _int, _vp, _i64)
     _sig(f"fx_gemm_bias_act_{_s}", _vp, _int, _int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _int)
     _sig(f"fx_gemm_tn_colsum_{_s}", _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp)
-    _sig(f"fx_linear_bwd_{_s}", _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp)
+    _sig(f"fx_linear_bwd_{_s}", _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _int)
     _sig(f"fx_bias_grad_{_s}", _vp, _vp, _vp, _i64, _i64, _i64)
     _sig(f"fx_relu_bwd_bias_grad_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64)
     _sig(f"fx_softmax_ce_fwd_{_s}", _vp, _vp, _vp, _vp, _vp, _i64, _i64)
@@ -468,13 +468,14 @@ class Context:
         check(self._fn("gemm_tn_colsum", a.dtype)(self.h, M, N, K, a.ptr, b.ptr, o.ptr, s.ptr))
         return o, s
 
-    def linear_bwd(self, dy, w, x, want_db=True):
-        """dy [B, out], w [out, in], x [B, in] -> (dx [B, in], dw [out, in], db [out] or None)."""
+    def linear_bwd(self, dy, w, x, want_db=True, relu_below=False):
+        """dy [B, out], w [out, in], x [B, in] -> (dx [B, in], dw [out, in], db [out] or None); relu_below: dx times (x > 0)."""
         Bn, O = dy.shape
         I = w.shape[1]
         dx, dw = self.empty((Bn, I), dy.dtype), self.empty((O, I), dy.dtype)
         db = self.empty((O,), dy.dtype) if want_db else None
-        check(self._fn("linear_bwd", dy.dtype)(self.h, Bn, I, O, dy.ptr, w.ptr, x.ptr, dx.ptr, dw.ptr, db.ptr if want_db else None))
+        check(self._fn("linear_bwd", dy.dtype)(self.h, Bn, I, O, dy.ptr, w.ptr, x.ptr, dx.ptr, dw.ptr, db.ptr if want_db else None,
+                                               int(relu_below)))
         return dx, dw, db
 
     def im2col(self, x, kernel, stride, padding):

@@ -19,6 +19,8 @@ int bias_act_t(fx_ctx* c, double* y, const double* b, i64 rows, i64 cols, int ac
 // out[m] = sum over k of a[k][m] for a stored [K, M]
 int col_sum_t(fx_ctx* c, const float* a, float* out, i64 K, i64 M) { return fx_bias_grad_f32(c, a, out, K, M, 1); }
 int col_sum_t(fx_ctx* c, const double* a, double* out, i64 K, i64 M) { return fx_bias_grad_f64(c, a, out, K, M, 1); }
+int relu_bwd_t(fx_ctx* c, const float* g, const float* x, float* o, i64 n) { return fx_relu_bwd_f32(c, g, x, o, n); }
+int relu_bwd_t(fx_ctx* c, const double* g, const double* x, double* o, i64 n) { return fx_relu_bwd_f64(c, g, x, o, n); }
 
 typedef Tile<128, 128, 16, 64, 64> TileBig;    // 4 waves, 64x64 each
 typedef Tile<64, 64, 16, 32, 32> TileSmall;    // 4 waves, 32x32 each
@@ -152,8 +154,10 @@ int gemm_tn_colsum(fx_ctx* c, i64 M, i64 N, i64 K, const T* A, const T* B, T* C,
 // Linear's backward products in one call: dX[B, in] = dY[B, out] . W[out, in], dW[out, in] = dY^T . X[B, in] and (optionally)
 // db[out] = the column sums of dY.  Where both products are small ones (each would run the one-launch small-product kernel on its
 // own) they share a launch; the results have the bits of the separate calls either way.
+// relu_below: X is the output of a ReLU, and dX comes out as the gradient of that ReLU's input, (dY . W) * (X > 0 ? 1 : 0) --
+// fx_relu_bwd's operation, in the store of the product where the two share a launch, as a pass over dX otherwise.
 template <typename T>
-int linear_bwd(fx_ctx* c, i64 Bn, i64 I, i64 O, const T* g, const T* W, const T* X, T* dX, T* dW, T* db) {
+int linear_bwd(fx_ctx* c, i64 Bn, i64 I, i64 O, const T* g, const T* W, const T* X, T* dX, T* dW, T* db, int relu_below) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(g && W && X && dX && dW, "fx_linear_bwd: null pointer");
     FX_REQUIRE(Bn >= 1 && I >= 1 && O >= 1 && Bn < (1ll << 31) && I < (1ll << 31) && O < (1ll << 31), "fx_linear_bwd: bad dimensions");
@@ -169,20 +173,23 @@ int linear_bwd(fx_ctx* c, i64 Bn, i64 I, i64 O, const T* g, const T* W, const T*
             const gsmall::Plan p1 = gsmall::make_plan<T>(c->num_cus, true, false, O, I, Bn, g, X);
             if (p0.ok && p1.ok && p0.splits == 1 && p1.splits == 1) {
                 std::lock_guard<std::mutex> lk(c->launch_mutex);
-                return gsmall::run_pair(c, p0, p1, Bn, I, O, g, W, dX, O, I, Bn, g, X, dW, db);
+                return gsmall::run_pair(c, p0, p1, Bn, I, O, g, W, dX, O, I, Bn, g, X, dW, db, relu_below ? X : nullptr);
             }
         }
     }
     if (int rc = gemm<T>(c, 0, 0, Bn, I, O, g, W, dX)) return rc;
+    if (relu_below) {
+        if (int rc = relu_bwd_t(c, dX, X, dX, Bn * I)) return rc;
+    }
     return db ? gemm_tn_colsum<T>(c, O, I, Bn, g, X, dW, db) : gemm<T>(c, 1, 0, O, I, Bn, g, X, dW);
 }
 extern "C" int fx_linear_bwd_f32(fx_ctx* c, int64_t B, int64_t in, int64_t out, const float* dY, const float* W, const float* X, float* dX,
-                                 float* dW, float* db) {
-    return linear_bwd<float>(c, B, in, out, dY, W, X, dX, dW, db);
+                                 float* dW, float* db, int relu_below) {
+    return linear_bwd<float>(c, B, in, out, dY, W, X, dX, dW, db, relu_below);
 }
 extern "C" int fx_linear_bwd_f64(fx_ctx* c, int64_t B, int64_t in, int64_t out, const double* dY, const double* W, const double* X, double* dX,
-                                 double* dW, double* db) {
-    return linear_bwd<double>(c, B, in, out, dY, W, X, dX, dW, db);
+                                 double* dW, double* db, int relu_below) {
+    return linear_bwd<double>(c, B, in, out, dY, W, X, dX, dW, db, relu_below);
 }
 extern "C" int fx_gemm_tn_colsum_f32(fx_ctx* c, int64_t M, int64_t N, int64_t K, const float* A, const float* B, float* C, float* colsum) {
     return gemm_tn_colsum<float>(c, M, N, K, A, B, C, colsum);

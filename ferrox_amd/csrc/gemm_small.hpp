@@ -33,6 +33,7 @@ struct Params {
     int kz;      // K per block when the grid's z dimension splits K (a multiple of 8 * WAVES * G ... see run), else K
     i64 zstride; // elements between the partial results of consecutive z (0 when K is not split)
     float* asum; // optional (K not split): asum[m] = sum over k of op(A)[m][k], written by the first block of every tile row
+    const float* mask;  // optional, [M][N] like C (K not split, no bias): C = (op(A) . op(B)) * (mask > 0 ? 1 : 0), fx_relu_bwd's operation
 };
 
 // KC: 1 = the operand is stored [rows][K] (k contiguous, K % 4 == 0, 16-byte aligned); 2 = the same layout read element by element
@@ -62,6 +63,14 @@ __device__ __forceinline__ void small_body(const Params& p, float* red, float* r
     const int kbase = bz * p.kz, kend = min(p.K, kbase + p.kz);            // this block's range of K (all of it unless K is split over z)
     const int g0 = wave * p.G;
     const float bias_n = p.bias ? p.bias[bn] : 0.f;  // loaded up front: its latency stays off the closing sum
+    float mk[2] = {1.f, 1.f};                        // likewise the mask values of the two elements this lane stores
+    if (p.mask) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int e = 2 * wave + u, m = min(m0 + 8 * (e >> 2) + 4 * h + (e & 3), p.M - 1);
+            mk[u] = p.mask[(i64)m * p.N + bn];
+        }
+    }
 
     float a[MAXG][4], b[MAXG][4];
 #pragma unroll
@@ -117,6 +126,7 @@ __device__ __forceinline__ void small_body(const Params& p, float* red, float* r
                 v = v + bias_n;
                 if (p.relu) v = v > 0.f ? v : 0.f;
             }
+            if (p.mask) v = v * (mk[u] > 0.f ? 1.f : 0.f);
             p.C[(i64)bz * p.zstride + (i64)m * p.N + n] = v;
         }
     }
@@ -162,7 +172,8 @@ struct ParamsD {
     int G;  // groups per wave
     int kz;
     i64 zstride;
-    double* asum;  // optional, as in Params
+    double* asum;        // optional, as in Params
+    const double* mask;  // optional, as in Params
 };
 
 template <int KC>
@@ -192,6 +203,15 @@ __device__ __forceinline__ void small_body_f64(const ParamsD& p, double* red_d, 
     const int g0 = wave * p.G;
     // this wave finishes the column block (wave / 2) % 2 in the closing sum; its bias is loaded up front
     const double bias_n = p.bias ? p.bias[(wave >> 1) & 1 ? bn1 : bn0] : 0.;
+    double mk[2] = {1., 1.};  // the mask values of the two elements this lane stores
+    if (p.mask) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int el = 2 * wave + u, blk = el >> 2, e = el & 3;
+            const int m = min(m0 + 16 * (blk >> 1) + 4 * e + q, p.M - 1);
+            mk[u] = p.mask[(i64)m * p.N + ((blk & 1) ? bn1 : bn0)];
+        }
+    }
     f64x4 acc[2][2];
 #pragma unroll
     for (int a = 0; a < 2; ++a)
@@ -251,6 +271,7 @@ __device__ __forceinline__ void small_body_f64(const ParamsD& p, double* red_d, 
                 v = v + bias_n;
                 if (p.relu) v = v > 0. ? v : 0.;
             }
+            if (p.mask) v = v * (mk[u] > 0. ? 1. : 0.);
             p.C[(i64)bz * p.zstride + (i64)m * p.N + n] = v;
         }
     }
@@ -339,7 +360,7 @@ inline int run_f64(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i6
                    int relu, double* part, double* asum = nullptr) {
     const bool split = pl.splits > 1;
     FX_REQUIRE(!(split && asum), "small product: row sums need an unsplit reduction");
-    ParamsD p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0, asum};
+    ParamsD p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0, asum, nullptr};
     const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32), (unsigned)pl.splits);
     const size_t lds = (size_t)WAVES * 16 * 64 * sizeof(double);
     if (!ta && pl.a_elems && !tb) small_kernel_f64<2, 0><<<grid, dim3(NT), lds, c->stream>>>(p);
@@ -356,7 +377,7 @@ inline int run(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K,
                float* part, float* asum = nullptr) {
     const bool split = pl.splits > 1;
     FX_REQUIRE(!(split && asum), "small product: row sums need an unsplit reduction");
-    Params p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0, asum};
+    Params p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0, asum, nullptr};
     const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32), (unsigned)pl.splits);
     if (!ta && pl.a_elems && !tb) small_kernel<2, 0><<<grid, dim3(NT), 0, c->stream>>>(p);
     else if (!ta && pl.a_elems) small_kernel<2, 1><<<grid, dim3(NT), 0, c->stream>>>(p);
@@ -370,11 +391,12 @@ inline int run(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K,
 
 // dX[M0,N0] = A0 . B0 (A0 stored [M0,K0], B0 stored [K0,N0]) and dW[M1,N1] = A1^T . B1 (A1 stored [K1,M1], B1 stored [K1,N1]) in one
 // launch; both plans unsplit.  asum1 (optional): the row sums of A1^T, i.e. the column sums of A1.
+// mask0 (optional, [M0][N0]): the first product is stored times (mask0 > 0 ? 1 : 0).
 inline int run_pair(fx_ctx* c, const Plan& p0, const Plan& p1, i64 M0, i64 N0, i64 K0, const float* A0, const float* B0, float* C0, i64 M1, i64 N1,
-                    i64 K1, const float* A1, const float* B1, float* C1, float* asum1) {
+                    i64 K1, const float* A1, const float* B1, float* C1, float* asum1, const float* mask0) {
     FX_REQUIRE(p0.splits == 1 && p1.splits == 1, "small product pair: unsplit reductions only");
-    Params a{A0, B0, C0, nullptr, 0, (int)M0, (int)N0, (int)K0, p0.G, p0.kz, 0, nullptr};
-    Params b{A1, B1, C1, nullptr, 0, (int)M1, (int)N1, (int)K1, p1.G, p1.kz, 0, asum1};
+    Params a{A0, B0, C0, nullptr, 0, (int)M0, (int)N0, (int)K0, p0.G, p0.kz, 0, nullptr, mask0};
+    Params b{A1, B1, C1, nullptr, 0, (int)M1, (int)N1, (int)K1, p1.G, p1.kz, 0, asum1, nullptr};
     const dim3 grid((unsigned)fx::ceil_div(std::max(N0, N1), (i64)32), (unsigned)fx::ceil_div(std::max(M0, M1), (i64)32), 2);
     if (p0.a_elems) small_pair_kernel<2><<<grid, dim3(NT), 0, c->stream>>>(a, b);
     else small_pair_kernel<1><<<grid, dim3(NT), 0, c->stream>>>(a, b);
@@ -382,10 +404,10 @@ inline int run_pair(fx_ctx* c, const Plan& p0, const Plan& p1, i64 M0, i64 N0, i
     return FX_OK;
 }
 inline int run_pair(fx_ctx* c, const Plan& p0, const Plan& p1, i64 M0, i64 N0, i64 K0, const double* A0, const double* B0, double* C0, i64 M1,
-                    i64 N1, i64 K1, const double* A1, const double* B1, double* C1, double* asum1) {
+                    i64 N1, i64 K1, const double* A1, const double* B1, double* C1, double* asum1, const double* mask0) {
     FX_REQUIRE(p0.splits == 1 && p1.splits == 1, "small product pair: unsplit reductions only");
-    ParamsD a{A0, B0, C0, nullptr, 0, (int)M0, (int)N0, (int)K0, p0.G, p0.kz, 0, nullptr};
-    ParamsD b{A1, B1, C1, nullptr, 0, (int)M1, (int)N1, (int)K1, p1.G, p1.kz, 0, asum1};
+    ParamsD a{A0, B0, C0, nullptr, 0, (int)M0, (int)N0, (int)K0, p0.G, p0.kz, 0, nullptr, mask0};
+    ParamsD b{A1, B1, C1, nullptr, 0, (int)M1, (int)N1, (int)K1, p1.G, p1.kz, 0, asum1, nullptr};
     const dim3 grid((unsigned)fx::ceil_div(std::max(N0, N1), (i64)32), (unsigned)fx::ceil_div(std::max(M0, M1), (i64)32), 2);
     const size_t lds = (size_t)WAVES * 16 * 64 * sizeof(double);
     if (p0.a_elems) small_pair_kernel_f64<2><<<grid, dim3(NT), lds, c->stream>>>(a, b);

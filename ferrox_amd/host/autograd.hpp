@@ -37,6 +37,11 @@ template <typename T> struct Operator {
     virtual size_t num_inputs() const = 0;
     virtual bool cache_output() const { return false; }
     virtual const char* name() const = 0;
+    // Fused operators only.  output_is_relu(): the output went through a ReLU inside the operator.  The engine sets
+    // input0_is_relu_output before it asks for gradients when input 0 is the output of such an operator: the gradient of input 0
+    // may then be handed back already multiplied by the ReLU's mask (input 0 > 0), marked with HipStorage::relu_masked_by.
+    virtual bool output_is_relu() const { return false; }
+    mutable bool input0_is_relu_output = false;
 };
 
 // reduce_gradient_for_broadcasting, src/ops/basic.rs:10-53
@@ -539,6 +544,10 @@ template <typename T> class AutoFerroxEngine {
         TensorRefs<T> in = collect(node.inputs);
         std::vector<bool> needs;
         for (NodeId i : node.inputs) needs.push_back(nodes_.at(i).requires_grad);
+        {
+            auto pit = node.inputs.empty() ? nodes_.end() : nodes_.find(node.inputs[0]);
+            node.op->input0_is_relu_output = pit != nodes_.end() && pit->second.op && pit->second.op->output_is_relu();
+        }
         std::vector<Tensor<T>> gs = node.op->gradient_needs(std::move(grad_output), in, node.tensor.get(), needs);
         for (size_t i = 0; i < node.inputs.size(); ++i)
             if (gs[i]) accumulate_gradient(node.inputs[i], std::move(gs[i]));

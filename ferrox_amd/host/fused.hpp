@@ -51,8 +51,8 @@ template <typename T> struct FusedApi;
         static int relu_bias_grad(fx_ctx* c, const T* g, const T* y, T* gm, T* db, int64_t o, int64_t C, int64_t i) {  \
             return fx_relu_bwd_bias_grad_##S(c, g, y, gm, db, o, C, i);                                                \
         }                                                                                                              \
-        static int linear_bwd(fx_ctx* c, int64_t B, int64_t I, int64_t O, const T* g, const T* W, const T* X, T* dX, T* dW, T* db) { \
-            return fx_linear_bwd_##S(c, B, I, O, g, W, X, dX, dW, db);                                                 \
+        static int linear_bwd(fx_ctx* c, int64_t B, int64_t I, int64_t O, const T* g, const T* W, const T* X, T* dX, T* dW, T* db, int rb) { \
+            return fx_linear_bwd_##S(c, B, I, O, g, W, X, dX, dW, db, rb);                                             \
         }                                                                                                              \
         static int gemm_tn_colsum(fx_ctx* c, int64_t M, int64_t N, int64_t K, const T* A, const T* B, T* C, T* s) {      \
             return fx_gemm_tn_colsum_##S(c, M, N, K, A, B, C, s);                                                      \
@@ -109,22 +109,28 @@ template <typename T> struct LinearFusedOp : Operator<T> {  // inputs: x [B, in]
         const int64_t B = (int64_t)xs[0], I = (int64_t)xs[1], O = (int64_t)ws[0];
         std::vector<Tensor<T>> r(3);
         r[2] = HipStorage<T>::alloc({ws[0]});
-        if (relu) {  // mask and bias gradient in one pass over g
+        // the layer above may have handed g over already multiplied by this layer's ReLU mask (in the store of its data gradient)
+        const bool premasked = relu && g->relu_masked_by == static_cast<const void*>(out);
+        if (relu && !premasked) {  // mask and bias gradient in one pass over g
             Tensor<T> gm = HipStorage<T>::alloc(g->shape());
             fx_ok(FusedApi<T>::relu_bias_grad(fused_ctx(), g->data(), out->data(), gm->data(), r[2]->data(), B, O, 1));
             g = std::move(gm);
         }
         r[1] = HipStorage<T>::alloc(ws);
-        // without a ReLU the bias gradient (the column sums of g) comes out of the weight gradient's launch
-        T* db = relu ? nullptr : r[2]->data();
+        // where no pass over g has produced it, the bias gradient (the column sums of g) comes out of the weight gradient's launch
+        T* db = relu && !premasked ? nullptr : r[2]->data();
         if (needs[0]) {  // both products in one call (one launch where both are small)
+            const bool below = this->input0_is_relu_output;  // x is the output of a ReLU: dX comes out times that ReLU's mask
             r[0] = HipStorage<T>::alloc(xs);
-            fx_ok(FusedApi<T>::linear_bwd(fused_ctx(), B, I, O, g->data(), in[1]->data(), in[0]->data(), r[0]->data(), r[1]->data(), db));
+            fx_ok(FusedApi<T>::linear_bwd(fused_ctx(), B, I, O, g->data(), in[1]->data(), in[0]->data(), r[0]->data(), r[1]->data(), db,
+                                          below ? 1 : 0));
+            if (below) r[0]->relu_masked_by = static_cast<const void*>(in[0]);
         } else if (db) fx_ok(FusedApi<T>::gemm_tn_colsum(fused_ctx(), O, I, B, g->data(), in[0]->data(), r[1]->data(), db));
         else fx_ok(Api<T>::gemm(fused_ctx(), 1, 0, O, I, B, g->data(), in[0]->data(), r[1]->data()));
         return r;
     }
     size_t num_inputs() const override { return 3; }
+    bool output_is_relu() const override { return relu; }
     const char* name() const override { return "LinearFused"; }
 };
 

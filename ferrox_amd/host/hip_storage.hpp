@@ -120,6 +120,11 @@ template <typename T> class HipStorage {
     HipStorage& operator=(const HipStorage&) = delete;
     ~HipStorage() { release(); }
 
+    // Set on a gradient that its producer already multiplied by a ReLU's mask: the activation tensor whose (value > 0) was
+    // applied.  The operator that owns that activation then skips its own masking.  Never copied: any tensor made from this one
+    // (a sum of gradients, a clone) starts without the mark, and is masked again where it matters (the mask is idempotent).
+    const void* relu_masked_by = nullptr;
+
     // ---- factories: BackendManager::{zeros, ones, full, from_vec}, manager.rs:131-339 ------------------------
     // CudaOps::get_tensor (cuda/ops.rs:121-133): output buffers come from the pool and are not cleared.
     static Ptr alloc(const Shape& shape) {

@@ -287,9 +287,11 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
     /* Linear's backward products in one call (nn/layers/linear.rs:152-308, MatMul::gradient ops/matrix.rs:34-55):      \
        dX[B, in] = dY[B, out] . W[out, in], dW[out, in] = dY^T . X[B, in] and, with db != NULL, db[out] = the column    \
        sums of dY.  dX and dW have the bits of fx_gemm(0, 0, ...) and fx_gemm(1, 0, ...), db those of                   \
-       fx_gemm_tn_colsum; two small products share one launch. */                                                      \
+       fx_gemm_tn_colsum; two small products share one launch.  relu_below != 0: X is the output of a ReLU (the layer  \
+       below ends in one) and dX is the gradient of that ReLU's input, fx_relu_bwd(dY . W, X) (ReLU::gradient,          \
+       ops/unary.rs:358-375), bit for bit -- in the product's store where the products share a launch. */               \
     int fx_linear_bwd_##S(fx_ctx* ctx, int64_t B, int64_t in, int64_t out, const T* dY, const T* W, const T* X, T* dX, \
-                          T* dW, T* db);                                                                               \
+                          T* dW, T* db, int relu_below);                                                               \
     /* BatchNorm, src/nn/layers/norm.rs:127-336, on x viewed as [outer, C, inner] ([N,C,H,W]: outer = N, inner = H*W;   \
        [N,F]: C = F, inner = 1).  stats: mean[C] and biased variance[C] of every channel in one read of x (the         \
        reference's Mean, Sub, Mul, Mean chain), and, when the pointers are not NULL, the running update                \

@@ -458,6 +458,13 @@ def test_linear_backward_products_in_one_call(ctx, dtype):
         assert np.array_equal(gw.numpy(), rw.numpy()) and np.array_equal(gb.numpy(), rb.numpy()), ("dW, db", Bn, I, O)
         gx2, gw2, _ = ctx.linear_bwd(ddy, dw_, dx_, want_db=False)
         assert np.array_equal(gx2.numpy(), gx.numpy()) and np.array_equal(gw2.numpy(), gw.numpy()), ("no db", Bn, I, O)
+        # x as the output of a ReLU (zeros where it clipped): dX times the ReLU's mask, the bits of fx_relu_bwd on the product
+        xr = np.maximum(x, 0)
+        dxr = ctx.upload(xr)
+        gx3, gw3, gb3 = ctx.linear_bwd(ddy, dw_, dxr, relu_below=True)
+        assert np.array_equal(gx3.numpy(), ctx.relu_bwd(ctx.gemm(ddy, dw_), dxr).numpy()), ("masked dX", Bn, I, O)
+        rw3, rb3 = ctx.gemm_tn_colsum(ddy, dxr)
+        assert np.array_equal(gw3.numpy(), rw3.numpy()) and np.array_equal(gb3.numpy(), rb3.numpy()), ("dW, db with relu below", Bn, I, O)
 
 
 def test_gemm_shape_mismatch_message(ctx):
