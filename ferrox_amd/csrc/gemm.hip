@@ -107,7 +107,7 @@ int gemm(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const T* A, const T* B,
                 rc = gthin::run(c, M, N, K, A, B, C, bias, relu, asum);
                 if (asum) *asum_done = true;
             } else if (!generic_only) {
-                const gsmall::Plan sp = gsmall::make_plan<float>(c->num_cus, ta != 0, tb != 0, M, N, K, A, B);
+                const gsmall::Plan sp = gsmall::make_plan<float>(c->num_cus, ta != 0, tb != 0, M, N, K, A, B, asum == nullptr);
                 if (sp.ok) {
                     lds_path = true;
                     const bool with_sum = asum != nullptr && sp.splits == 1;

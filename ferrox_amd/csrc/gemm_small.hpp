@@ -154,6 +154,66 @@ __global__ __launch_bounds__(NT) void small_pair_kernel(const Params p0, const P
     }
 }
 
+// ---- 16 x 16 tiles (f32) on v_mfma_f32_16x16x4_f32 -----------------------------------------------------------------------------
+// A product of a few dozen 32 x 32 tiles leaves most of the chip idle and every block with a long operand read ([256,784] x
+// [784,256]: 64 blocks of 200 KB each).  With 16 x 16 tiles there are four times the blocks at half the bytes each.  A group of
+// 16 consecutive k feeds 4 MFMAs; lane l = (i = l % 16, q = l / 16) holds, for MFMA j of the group, the element with
+// k = 16 g + 4 q + j of row (column) i -- the same 16-byte load per lane as in the 32 x 32 kernel -- and 4 of the 256 sums
+// (row 4 q + e, column i).  K is split over the 8 waves and added through LDS in wave order as above.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int MAXG16 = 16;  // groups of 16 k per wave: K <= 16 * 8 * 16
+
+template <int AKC, int BKC>
+__global__ __launch_bounds__(NT) void small16_kernel(const Params p) {
+    __shared__ float red[WAVES * 4 * 64];
+    const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, i = lane & 15;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m0 = blockIdx.y * 16, n0 = blockIdx.x * 16;
+    const int am = min(m0 + i, p.M - 1), bn = min(n0 + i, p.N - 1);  // past the edge: a valid row / column, result unused
+    const int g0 = wave * p.G;
+    const float bias_n = p.bias ? p.bias[bn] : 0.f;
+
+    float a[MAXG16][4], b[MAXG16][4];
+#pragma unroll
+    for (int g = 0; g < MAXG16; ++g) {
+        if (g < p.G) {  // scalar
+            const int k = 16 * (g0 + g) + 4 * q;
+            load_group<AKC>(p.A, am, p.M, p.K, k, a[g]);
+            load_group<BKC>(p.B, bn, p.N, p.K, k, b[g]);
+        }
+    }
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int g = 0; g < MAXG16; ++g) {
+        if (g < p.G) {
+            const int k = 16 * (g0 + g) + 4 * q;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool in = k + j < p.K;
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(in ? a[g][j] : 0.f, in ? b[g][j] : 0.f, acc, 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) red[(wave * 4 + e) * 64 + lane] = acc[e];
+    __syncthreads();
+    // waves 0 .. 3 finish accumulator element `wave`: the eight sums in wave order, then the bias kernel's operations
+    if (wave < 4) {
+        const int e = wave;
+        float v = red[e * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) v = v + red[(w * 4 + e) * 64 + lane];
+        const int m = m0 + 4 * q + e, n = n0 + i;
+        if (m < p.M && n < p.N) {
+            if (p.bias) {
+                v = v + bias_n;
+                if (p.relu) v = v > 0.f ? v : 0.f;
+            }
+            p.C[(i64)m * p.N + n] = v;
+        }
+    }
+}
+
 // ---- f64 twin on v_mfma_f64_16x16x4_f64 -------------------------------------------------------------------------------------
 // The 32 x 32 tile is 2 x 2 MFMA blocks of 16 x 16; a group of 8 consecutive k feeds 2 MFMA steps of 4 k each.  Lane
 // l = (i = l % 16, q = l / 16) holds, for step j of the group, the element with k = 8 g + 2 q + j of rows (columns) i and i + 16:
@@ -319,10 +379,12 @@ struct Plan {
     bool ok = false;
     int G = 0, kz = 0, splits = 1;
     bool a_elems = false;  // A is k-contiguous but not readable in 16-byte pieces (K % 4, alignment): element loads
+    bool tile16 = false;   // f32: 16 x 16 tiles (few 32 x 32 tiles and a long enough reduction); no row sums or mask in this form
 };
 
+// allow16: the caller wants neither row sums nor a mask nor a pair launch (those exist for 32 x 32 tiles only)
 template <typename T>
-inline Plan make_plan(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, const T* A, const T* B) {
+inline Plan make_plan(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, const T* A, const T* B, bool allow16 = false) {
     Plan pl;
     static const bool off = [] { const char* v = getenv("FX_GEMM_SMALL"); return v && atoi(v) == 0; }();
     constexpr int KV = 16 / (int)sizeof(T);  // elements per 16-byte load of a k-contiguous operand
@@ -337,6 +399,15 @@ inline Plan make_plan(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, const 
     if (K <= kmax) {
         pl.G = (int)fx::ceil_div(fx::ceil_div(K, (i64)8), (i64)WAVES);
         pl.kz = (int)K;
+        if constexpr (sizeof(T) == 4) {
+            // fewer 32 x 32 tiles than half the CUs, each reading K >= 128 deep: 16 x 16 tiles fill more of the chip
+            const i64 tiles16 = fx::ceil_div(M, (i64)16) * fx::ceil_div(N, (i64)16);
+            static const bool off16 = [] { const char* v = getenv("FX_GEMM_SMALL16"); return v && atoi(v) == 0; }();
+            if (!off16 && allow16 && !pl.a_elems && 2 * tiles < (i64)num_cus && tiles16 <= 2 * (i64)num_cus && K >= 128 && N >= 16) {
+                pl.tile16 = true;
+                pl.G = (int)fx::ceil_div(fx::ceil_div(K, (i64)16), (i64)WAVES);
+            }
+        }
     } else {
         // split K over blocks: about 2 blocks per CU, each at least 256 deep, ranges a multiple of 8 * WAVES
         if (M * N > (1 << 18)) return pl;  // the partial sums stay small
@@ -378,6 +449,16 @@ inline int run(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K,
     const bool split = pl.splits > 1;
     FX_REQUIRE(!(split && asum), "small product: row sums need an unsplit reduction");
     Params p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0, asum, nullptr};
+    if (pl.tile16) {
+        FX_REQUIRE(!split && !asum && !pl.a_elems, "small product: 16 x 16 tiles take neither a split K nor row sums");
+        const dim3 grid16((unsigned)fx::ceil_div(N, (i64)16), (unsigned)fx::ceil_div(M, (i64)16));
+        if (!ta && !tb) small16_kernel<1, 0><<<grid16, dim3(NT), 0, c->stream>>>(p);
+        else if (!ta && tb) small16_kernel<1, 1><<<grid16, dim3(NT), 0, c->stream>>>(p);
+        else if (ta && !tb) small16_kernel<0, 0><<<grid16, dim3(NT), 0, c->stream>>>(p);
+        else small16_kernel<0, 1><<<grid16, dim3(NT), 0, c->stream>>>(p);
+        FX_LAUNCH_CHECK();
+        return FX_OK;
+    }
     const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32), (unsigned)pl.splits);
     if (!ta && pl.a_elems && !tb) small_kernel<2, 0><<<grid, dim3(NT), 0, c->stream>>>(p);
     else if (!ta && pl.a_elems) small_kernel<2, 1><<<grid, dim3(NT), 0, c->stream>>>(p);

@@ -278,18 +278,19 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
                                    int64_t ph, int64_t pw, int act, void* workspace, int64_t ws_bytes);                \
     int fx_gemm_bias_act_##S(fx_ctx* ctx, int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const T* A,       \
                              const T* B, const T* bias, T* C, int act);                                                \
-    /* Linear's weight and bias gradient in one call (nn/layers/linear.rs:152-308: MatMul::gradient, ops/matrix.rs:     \
-       34-55, and reduce_gradient_for_broadcasting, ops/basic.rs:10-53): C[M,N] = A^T . B for A = dY stored [K, M] and  \
-       B = X stored [K, N] -- the values of fx_gemm(1, 0, ...) -- and colsum[m] = sum over k of A[k][m], summed in a    \
-       fixed order of its own (equal to fx_bias_grad(A, K, M, 1) up to rounding).  Small and thin products write the    \
-       sums from the product's launch; the others run the bias-gradient kernel after it. */                            \
+    /* Linear's weight and bias gradient in one call (nn/layers/linear.rs:152-308: MatMul::gradient, ops/matrix.rs:    \
+       34-55, and reduce_gradient_for_broadcasting, ops/basic.rs:10-53): C[M,N] = A^T . B for A = dY stored [K, M] and \
+       B = X stored [K, N] -- fx_gemm(1, 0, ...) up to the order of summation -- and colsum[m] = sum over k of         \
+       A[k][m], in a fixed order of its own (equal to fx_bias_grad(A, K, M, 1) up to rounding).  Small and thin        \
+       products write the sums from the product's launch; the others run the bias-gradient kernel after it. */         \
     int fx_gemm_tn_colsum_##S(fx_ctx* ctx, int64_t M, int64_t N, int64_t K, const T* A, const T* B, T* C, T* colsum);  \
-    /* Linear's backward products in one call (nn/layers/linear.rs:152-308, MatMul::gradient ops/matrix.rs:34-55):      \
-       dX[B, in] = dY[B, out] . W[out, in], dW[out, in] = dY^T . X[B, in] and, with db != NULL, db[out] = the column    \
-       sums of dY.  dX and dW have the bits of fx_gemm(0, 0, ...) and fx_gemm(1, 0, ...), db those of                   \
-       fx_gemm_tn_colsum; two small products share one launch.  relu_below != 0: X is the output of a ReLU (the layer  \
-       below ends in one) and dX is the gradient of that ReLU's input, fx_relu_bwd(dY . W, X) (ReLU::gradient,          \
-       ops/unary.rs:358-375), bit for bit -- in the product's store where the products share a launch. */               \
+    /* Linear's backward products in one call (nn/layers/linear.rs:152-308, MatMul::gradient ops/matrix.rs:34-55):     \
+       dX[B, in] = dY[B, out] . W[out, in], dW[out, in] = dY^T . X[B, in] and, with db != NULL, db[out] = the column   \
+       sums of dY.  dX and dW are fx_gemm(0, 0, ...) and fx_gemm(1, 0, ...) up to the order of summation (a fixed one  \
+       per shape), dW and db have the bits of fx_gemm_tn_colsum; two small products share one launch.                  \
+       relu_below != 0: X is the output of a ReLU (the layer below ends in one) and dX is the gradient of that ReLU's  \
+       input, fx_relu_bwd(dY . W, X) (ReLU::gradient, ops/unary.rs:358-375) -- in the product's store where the        \
+       products share a launch. */                                                                                     \
     int fx_linear_bwd_##S(fx_ctx* ctx, int64_t B, int64_t in, int64_t out, const T* dY, const T* W, const T* X, T* dX, \
                           T* dW, T* db, int relu_below);                                                               \
     /* BatchNorm, src/nn/layers/norm.rs:127-336, on x viewed as [outer, C, inner] ([N,C,H,W]: outer = N, inner = H*W;   \
