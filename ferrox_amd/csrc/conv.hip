@@ -18,6 +18,7 @@
 #include "dgrad_patch_s2.hpp"
 #include "dgrad_patch_s2_f64.hpp"
 #include "fwd_patch_s2.hpp"
+#include "fwd_patch_s2_f64.hpp"
 #include "conv_smallc.hpp"
 #include "conv_patch.hpp"
 #include "conv_patch_f64.hpp"
@@ -218,6 +219,10 @@ int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64
         }
     }
     if constexpr (sizeof(T) == 8) {
+        if (!generic_only()) {
+            const fwd2::Plan f2 = fwd2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
+            if (f2.ok && aligned16(x, w) && aligned16(y, y)) return fwd2::run(c, f2, x, w, y, B, Cin, H, Cout, d.oh, bias, relu);
+        }
         const cpd::Plan pd = fwd_patch64_plan<T>(c, d);
         if (pd.ok && aligned16(x, ws) && aligned16(y, y)) {
             double* wimg = (double*)(ws ? ws : c->get_scratch(need));

@@ -683,6 +683,10 @@ CONV_F64_PATCH_CASES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw)
     (2, 64, 56, 56, 128, (1, 1), (1, 1)), (3, 8, 6, 12, 60, (1, 1), (1, 1)), (3, 16, 8, 36, 120, (1, 1), (0, 0)), (2, 24, 10, 16, 104, (1, 1), (2, 2)),
     (1, 8, 64, 64, 52, (1, 1), (1, 1)), (2, 16, 9, 62, 64, (2, 1), (1, 1)), (5, 32, 32, 32, 64, (1, 1), (1, 1)), (3, 8, 14, 28, 72, (1, 1), (1, 1)),
     (2, 8, 9, 30, 128, (1, 1), (0, 0)), (2, 32, 28, 28, 33, (1, 1), (1, 1)),
+    # stride 2 over maps 32 and 64 wide (fwd_patch_s2_f64.hpp; the data gradient runs dgrad_patch_s2_f64.hpp where Cin % 32 == 0): 32 and
+    # 64 output channels per block, one to eight chunks of 4 input channels, one to four tiles per image
+    (3, 32, 32, 32, 64, (2, 2), (1, 1)), (2, 4, 32, 32, 32, (2, 2), (1, 1)), (2, 16, 64, 64, 64, (2, 2), (1, 1)), (2, 12, 16, 64, 32, (2, 2), (1, 1)),
+    (1, 8, 128, 64, 64, (2, 2), (1, 1)),
 ]
 
 

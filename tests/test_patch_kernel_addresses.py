@@ -1058,3 +1058,102 @@ def test_stride2_forward_patch_kernel_accesses_stay_inside_the_tensors(case):
     pl = fw2_plan(B, Cin, H, W, Cout, 3, 3, 2, 2, 1, 1, oh, ow)
     assert pl is not None, "the shape must exercise the stride-2 forward patch kernel"
     assert fw2_walk(pl, B, Cin, Cout, oh) == "fw2 ok"
+
+
+# ---- f64 stride-2 forward pass (fwd_patch_s2_f64.hpp) ----
+def fwd2_plan(B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, oh, ow):
+    if kh != 3 or kw != 3 or sh != 2 or sw != 2 or ph != 1 or pw != 1 or W != 2 * ow or H != 2 * oh or Cin % 4 or Cout not in (32, 64): return None
+    mb = 2 if Cout % 64 == 0 else 1
+    pick = [(o, m) for (o, m) in FW2_INSTANCES if ow == o and mb == m and oh % (256 // o) == 0]
+    return dict(OW=pick[0][0], MB=pick[0][1]) if pick else None
+def fwd2_walk(pl, B, Cin, Cout, oh):
+    """Offsets in doubles; 16-byte loads must sit on even offsets."""
+    OW, MB = pl["OW"], pl["MB"]
+    NTF, CC, TR, HALF, NB = 512, 4, 256 // OW, OW + 1, 2 * MB
+    PR, W, H = 2 * TR + 1, 2 * OW, 2 * oh
+    RP = 40 if OW == 16 else 2 * HALF
+    PLANE = (PR * RP) | 1
+    WCH, XCH = 9 * NB * 64, CC * PLANE; BUF = WCH + XCH
+    W2, X2 = MB * 32 * CC * 9 // 2, CC * PR * (W // 2)
+    NWP, NXP = _ceil_div(W2, NTF), _ceil_div(X2, NTF)
+    assert 2 * BUF * 8 <= 160 * 1024 and 2 * HALF <= RP
+    L, tpi, nmt = oh * OW, oh // TR, Cout // (32 * MB)
+    xsize, wsize, ysize = B * Cin * H * W, Cout * Cin * 9, B * Cout * L
+    nblk = B * tpi * nmt
+    w_written, x_written = set(), set()
+    for blk in sorted({0, 1, nmt - 1, nmt, nblk - 1}):
+        if not 0 <= blk < nblk: continue
+        bt, mt = divmod(blk, nmt); b, tile = divmod(bt, tpi)
+        oc0, oy0 = mt * 32 * MB, tile * TR
+        iy0 = 2 * oy0 - 1
+        for k in sorted({0, Cin // CC - 1}):
+            c0 = k * CC
+            first = blk == 0 and k == 0
+            for tid in range(NTF):
+                for u in range(NWP):
+                    f = u * NTF + tid
+                    ok = f < W2
+                    ocl, q = divmod(f, 18)
+                    a = oc0 * Cin * 9 + c0 * 9 + ((ocl * Cin * 9 + 2 * q) if ok else 0)
+                    assert 0 <= a and a + 2 <= wsize and a % 2 == 0, ("w", a)
+                    if ok and first:
+                        for i in range(2):
+                            cl, t = divmod(2 * q + i, 9)
+                            d = (t * NB + (ocl >> 4)) * 64 + cl * 16 + (ocl & 15)
+                            assert 0 <= d < WCH and d not in w_written
+                            w_written.add(d)
+                for u in range(NXP):
+                    f = u * NTF + tid
+                    inside = f < X2
+                    cr, q = divmod(f, W // 2); c, r = divmod(cr, PR)
+                    iy = iy0 + r
+                    ok = inside and 0 <= iy < H
+                    a = b * Cin * H * W + c0 * H * W + (((c * H + iy) * W + 2 * q) if ok else 0)
+                    assert 0 <= a and a + 2 <= xsize and a % 2 == 0, ("x", a)
+                    if inside:
+                        d = c * PLANE + r * RP + q
+                        for o in (HALF, 1):
+                            assert 0 <= d + o < XCH and (not first or d + o not in x_written)
+                            if first: x_written.add(d + o)
+        if blk == 0:
+            for i in range(2 * CC * PR):
+                buf, rem = divmod(i, CC * PR); c, r = divmod(rem, PR)
+                d = c * PLANE + r * RP
+                assert buf < 2 and (d not in x_written or buf == 1)
+                if buf == 0: x_written.add(d)
+        for wave in range(8):
+            for lane in (0, 15, 16, 47, 48, 63):
+                kq, l16 = lane >> 4, lane & 15
+                for h in range(2):
+                    pix = wave * 32 + 16 * h + l16
+                    prow, pcol = divmod(pix, OW)
+                    for t in range(9):
+                        ky, kx = divmod(t, 3)
+                        d = kq * PLANE + (2 * prow + ky) * RP + pcol + (HALF if kx == 1 else 0) + (1 if kx == 2 else 0)
+                        c, rem = divmod(d, PLANE); r, o = divmod(rem, RP)
+                        assert c == kq and r == 2 * prow + ky and r < PR and o < 2 * HALF
+                        pc = 2 * o if o < HALF else 2 * (o - HALF) + 1
+                        assert pc == 2 * pcol + kx and (blk != 0 or d in x_written)
+                        for m in range(NB):
+                            assert (t * NB + m) * 64 + lane < WCH
+                    for m in range(NB):
+                        for e in (0, 3):
+                            oc = 16 * m + 4 * e + kq
+                            a = (b * Cout + oc0 + oc) * L + oy0 * OW + pix
+                            assert 0 <= a < ysize and oc0 + oc < Cout and oy0 * OW + pix < L
+    assert w_written == set(range(WCH))
+    return "fwd2 ok"
+
+FWD2_SHAPES = [  # B, Cin, H, W, Cout
+    (256, 32, 32, 32, 64), (2, 4, 32, 32, 32), (2, 16, 64, 64, 64), (2, 12, 16, 64, 32), (3, 40, 64, 32, 64),
+]
+
+
+@pytest.mark.parametrize("case", FWD2_SHAPES, ids=str)
+def test_stride2_f64_forward_patch_kernel_accesses_stay_inside_the_tensors(case):
+    B, Cin, H, W, Cout = case
+    oh, ow = H // 2, W // 2
+    B = min(B, 3)
+    pl = fwd2_plan(B, Cin, H, W, Cout, 3, 3, 2, 2, 1, 1, oh, ow)
+    assert pl is not None, "the shape must exercise the f64 stride-2 forward patch kernel"
+    assert fwd2_walk(pl, B, Cin, Cout, oh) == "fwd2 ok"
