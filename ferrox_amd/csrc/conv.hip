@@ -20,6 +20,7 @@
 #include "fwd_patch_s2.hpp"
 #include "fwd_patch_s2_f64.hpp"
 #include "conv_smallc.hpp"
+#include "conv_image_f64.hpp"
 #include "conv_patch.hpp"
 #include "conv_patch_f64.hpp"
 #include "wgrad_patch_f64.hpp"
@@ -219,6 +220,8 @@ int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64
         }
     }
     if constexpr (sizeof(T) == 8) {
+        if (!generic_only() && cim::eligible(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw) && aligned16(x, x) && aligned16(y, y))
+            return cim::run(c, x, w, y, B, Cin, H, Cout, bias, relu);
         if (!generic_only()) {
             const fwd2::Plan f2 = fwd2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
             if (f2.ok && aligned16(x, w) && aligned16(y, y)) return fwd2::run(c, f2, x, w, y, B, Cin, H, Cout, d.oh, bias, relu);

@@ -838,7 +838,11 @@ def test_conv2d_f64_image_layer_forward(ctx, orc):
     from ferrox_amd import capi
     rng = np.random.default_rng(63)
     tol = TOL[np.dtype(np.float64)]
-    for (B, Cin, H, W, Cout, st, pd) in SMALLC_CASES:
+    # maps 32 wide, heights a multiple of 8, output channels a multiple of 32: the image-layer kernel of conv_image_f64.hpp (1 to 4
+    # channels, one to five tiles per image, one to three blocks of output channels)
+    extra = [(3, 1, 8, 32, 64, (1, 1), (1, 1)), (2, 4, 40, 32, 96, (1, 1), (1, 1)), (5, 2, 24, 32, 32, (1, 1), (1, 1)),
+             (9, 3, 32, 32, 32, (1, 1), (1, 1))]
+    for (B, Cin, H, W, Cout, st, pd) in SMALLC_CASES + extra:
         case = (B, Cin, H, W, Cout, st, pd)
         x = rng.uniform(-1, 1, (B, Cin, H, W))
         w = rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9))
