@@ -604,6 +604,12 @@ i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     if (p2.ok) generic = std::max(generic, wg2::workspace_bytes(p2, d.Cout, d.Cin));
     const wgd2::Plan q2 = patch64_s2_plan<T>(c, d, mode);
     if (q2.ok) generic = std::max(generic, wgd2::workspace_bytes(q2, d.Cout, d.Cin));
+    if constexpr (sizeof(T) == 8) {
+        if (mode == 0 && !generic_only()) {
+            const cim::WPlan ip = cim::wgrad_plan(c ? c->num_cus : 256, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
+            if (ip.ok) generic = std::max(generic, cim::wgrad_workspace_bytes(ip, d.Cout, d.Cin));
+        }
+    }
     return pl.ok ? std::max(generic, wgp::workspace_bytes(pl, d.Cout, d.Cin)) : generic;
 }
 
@@ -668,6 +674,14 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
         }
     }
     if constexpr (sizeof(T) == 8) {
+        if (mode == 0 && !generic_only()) {
+            const cim::WPlan ip = cim::wgrad_plan(c->num_cus, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
+            if (ip.ok && aligned16(x, g) && aligned16(ws, ws)) {
+                double* part = (double*)(ws ? ws : c->get_scratch(need));
+                if (!part) return FX_ERR_OOM;
+                return cim::run_wgrad(c, ip, x, g, dw, part, Cin, H, Cout);
+            }
+        }
         const wgd2::Plan q2 = patch64_s2_plan<T>(c, d, mode);
         if (q2.ok && aligned16(x, g) && aligned16(ws, ws)) {
             double* part = (double*)(ws ? ws : c->get_scratch(need));

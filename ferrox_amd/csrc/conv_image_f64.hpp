@@ -160,4 +160,172 @@ inline int run(fx_ctx* c, const double* x, const double* w, double* y, i64 B, i6
     return FX_OK;
 }
 
+// ---- weight gradient of the same layer (1 to 3 channels: K = Cin * 9 <= 27 <= 32) -------------------------------------------
+//   dw[oc][c][ky][kx] = sum over (b, oy, ox) of g[b][oc][oy][ox] * x[b][c][oy + ky - 1][ox + kx - 1]
+// (grad_out_2d . im2col(x)^T, convolutions.rs:296-338).  The MFMA's 16 columns are (channel, tap) pairs -- two blocks of 16 hold
+// the K <= 27 of them -- its reduction runs over 4 pixels: lane l reads g[oc = l % 16 (+ 16)][pixel + l / 16] and
+// x[c][pixel + l / 16 shifted by the tap] for its pair (c, tap) = 16 block + l % 16, both from LDS, where a block has staged
+// 32 rows of g (256 pixels of one image, odd pitch) and the padded patch under them.  A wave takes one row of 32 pixels: 8 steps
+// of 4 MFMAs.  A block walks its range of tiles with the sums in registers, adds its eight waves' sums through LDS in wave
+// order and leaves one partial sum, laid out like dw; the ordered split sum adds the partials.  Bound by the one read of g.
+struct WParams {
+    const double* x;
+    const double* g;
+    double* part;  // [splits][Cout][Cin * 9]
+    int Cin, Cout, H, tpi;
+    int tiles, tps;  // B * tiles per image, tiles per split
+    FastDiv div_tpi;
+};
+
+constexpr int GPITCH = PIX + 1;
+
+__global__ __launch_bounds__(NT) void image_wgrad_f64_kernel(const WParams p) {
+    using S = Shape<32>;
+    constexpr int W = 32, TR = S::TR, PR = S::PR, PW = S::PW, PLANE = S::PLANE;
+    extern __shared__ __align__(16) double smem_w[];
+    double* Gs = smem_w;                   // [32 oc][GPITCH]
+    double* Xs = smem_w + 32 * GPITCH;     // [CP planes][PR][PW], odd plane pitch
+    const int tid = threadIdx.x, lane = tid & 63, kq = lane >> 4, l16 = lane & 15;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int oc0 = blockIdx.y * 32, L = p.H * W, K = p.Cin * KK;
+    const int t_beg = blockIdx.x * p.tps, t_end = min(p.tiles, t_beg + p.tps);
+
+    // this lane's (channel, tap) pairs: 16 nb + l16; pairs past K read a valid address and contribute zeros
+    int xoff[2];
+    bool pair_ok[2];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+        const int kp = 16 * nb + l16;
+        pair_ok[nb] = kp < K;
+        const int c = pair_ok[nb] ? kp / KK : 0, t = pair_ok[nb] ? kp % KK : 0;
+        xoff[nb] = c * PLANE + (wave + t / 3) * PW + t % 3 + kq;  // pixel (row wave, column 4 s + kq): + 4 s per step
+    }
+    const int goff = l16 * GPITCH + wave * W + kq;                // + 16 GPITCH for the second block of output channels
+
+    f64x4 acc[2][2];  // [oc block][pair block]
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[m][nb][e] = 0.;
+    // the zero columns left and right of the map stay zero over the tiles
+    for (int i = tid; i < CP * PR * 2; i += NT) {
+        const int cr = i >> 1;
+        Xs[(cr / PR) * PLANE + (cr % PR) * PW + (i & 1) * (W + 1)] = 0.;
+    }
+    for (int tl = t_beg; tl < t_end; ++tl) {
+        const int b = (int)p.div_tpi.div((uint32_t)tl), tile = tl - b * p.tpi;
+        const int oy0 = tile * TR, iy0 = oy0 - 1;
+        // g: 32 rows of 256 doubles, 8 double2 per thread
+        const double* gsrc = p.g + ((i64)b * p.Cout + oc0) * L + (i64)oy0 * W;
+        double2 gv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int f = u * NT + tid, row = f >> 7, q = f & 127;
+            gv[u] = *reinterpret_cast<const double2*>(gsrc + (i64)row * L + 2 * q);
+        }
+        const double* xsrc = p.x + (i64)b * p.Cin * L;
+        double2 xv[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int f = u * NT + tid;
+            xv[u] = make_double2(0., 0.);
+            if (f < S::X2) {
+                const int cr = f / (W / 2), q = f - cr * (W / 2), c = cr / PR, r = cr - c * PR;
+                const int iy = iy0 + r;
+                if (c < p.Cin && iy >= 0 && iy < p.H) xv[u] = *reinterpret_cast<const double2*>(xsrc + ((i64)c * p.H + iy) * W + 2 * q);
+            }
+        }
+        __syncthreads();  // the tile before has been read
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int f = u * NT + tid, row = f >> 7, q = f & 127;
+            double* d = Gs + row * GPITCH + 2 * q;
+            d[0] = gv[u].x;
+            d[1] = gv[u].y;
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int f = u * NT + tid;
+            if (f < S::X2) {
+                const int cr = f / (W / 2), q = f - cr * (W / 2), c = cr / PR, r = cr - c * PR;
+                double* d = Xs + c * PLANE + r * PW + 1 + 2 * q;
+                d[0] = xv[u].x;
+                d[1] = xv[u].y;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int s = 0; s < W / 4; ++s) {
+            const double a0 = Gs[goff + 4 * s], a1 = Gs[goff + 16 * GPITCH + 4 * s];
+            double b0 = Xs[xoff[0] + 4 * s], b1 = Xs[xoff[1] + 4 * s];
+            if (!pair_ok[0]) b0 = 0.;
+            if (!pair_ok[1]) b1 = 0.;
+            acc[0][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(a0, b0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(a0, b1, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(a1, b0, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(a1, b1, acc[1][1], 0, 0, 0);
+        }
+    }
+    // the eight waves' sums through LDS (the stage buffers are free after a barrier), added in wave order by waves 0 .. 3
+    __syncthreads();
+    double* red = smem_w;  // [8 waves][16 elements][64 lanes]
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) red[(wave * 16 + 4 * (2 * m + nb) + e) * 64 + lane] = acc[m][nb][e];
+    __syncthreads();
+    double* out = p.part + ((i64)blockIdx.x * p.Cout + oc0) * K;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const int el = 2 * wave + u, blk = el >> 2, e = el & 3;  // wave w finishes elements 2 w and 2 w + 1
+        double v = red[el * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < 8; ++w) v = v + red[(w * 16 + el) * 64 + lane];
+        const int oc = 16 * (blk >> 1) + 4 * e + kq, kp = 16 * (blk & 1) + l16;
+        if (kp < K) out[(i64)oc * K + kp] = v;
+    }
+}
+
+struct WPlan {
+    bool ok = false;
+    int splits = 1, tps = 1, tiles = 0;
+};
+
+inline WPlan wgrad_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw) {
+    WPlan pl;
+    static const bool off = [] { const char* v = getenv("FX_CIM"); return v && atoi(v) == 0; }();
+    if (off || kh != 3 || kw != 3 || sh != 1 || sw != 1 || ph != 1 || pw != 1 || Cin < 1 || Cin > 3 || W != 32 || H % (PIX / 32) != 0 || Cout % 32 != 0)
+        return pl;
+    const i64 tiles = B * (H / (PIX / 32)), rows = Cout / 32;
+    if (tiles > 0x7fffffff || rows > 65535) return pl;
+    // two blocks per CU (78 KB of LDS each); at least two tiles per block where there are that many
+    const i64 splits = std::max<i64>(1, std::min<i64>(2 * (i64)num_cus / rows, std::max<i64>(1, tiles / 2)));
+    pl.tps = (int)fx::ceil_div(tiles, splits);
+    pl.splits = (int)fx::ceil_div(tiles, (i64)pl.tps);
+    pl.tiles = (int)tiles;
+    pl.ok = true;
+    return pl;
+}
+inline i64 wgrad_workspace_bytes(const WPlan& pl, i64 Cout, i64 Cin) { return (i64)pl.splits * Cout * Cin * KK * (i64)sizeof(double); }
+
+// x, g and part must be 16-byte aligned.
+inline int run_wgrad(fx_ctx* c, const WPlan& pl, const double* x, const double* g, double* dw, double* part, i64 Cin, i64 H, i64 Cout) {
+    WParams p;
+    p.x = x; p.g = g; p.part = part;
+    p.Cin = (int)Cin; p.Cout = (int)Cout; p.H = (int)H;
+    p.tpi = (int)(H / (PIX / 32));
+    p.tiles = pl.tiles; p.tps = pl.tps;
+    p.div_tpi = FastDiv((uint32_t)p.tpi);
+    const size_t lds = std::max((size_t)(32 * GPITCH + Shape<32>::XCH), (size_t)8 * 16 * 64) * sizeof(double);
+    static const hipError_t attr = hipFuncSetAttribute((const void*)image_wgrad_f64_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    FX_HIP_CHECK(attr);
+    image_wgrad_f64_kernel<<<dim3((unsigned)pl.splits, (unsigned)(Cout / 32)), dim3(NT), lds, c->stream>>>(p);
+    FX_LAUNCH_CHECK();
+    return igemm::launch_splitk_reduce<double>(c, part, dw, Cout * Cin * KK, pl.splits);
+}
+
 }  // namespace cim

@@ -832,7 +832,8 @@ def test_conv2d_image_layer_kernels(ctx, orc):
 
 
 def test_conv2d_f64_image_layer_forward(ctx, orc):
-    """Image layers in f64 (1 to 4 input channels, K = Cin * 9 below two slabs of the implicit GEMM): forward, bias + ReLU in the store."""
+    """Image layers in f64 (1 to 4 input channels, K = Cin * 9 below two slabs of the implicit GEMM): forward, bias + ReLU in the store,
+    weight gradient."""
     import torch
     import torch.nn.functional as F
     from ferrox_amd import capi
@@ -841,7 +842,7 @@ def test_conv2d_f64_image_layer_forward(ctx, orc):
     # maps 32 wide, heights a multiple of 8, output channels a multiple of 32: the image-layer kernel of conv_image_f64.hpp (1 to 4
     # channels, one to five tiles per image, one to three blocks of output channels)
     extra = [(3, 1, 8, 32, 64, (1, 1), (1, 1)), (2, 4, 40, 32, 96, (1, 1), (1, 1)), (5, 2, 24, 32, 32, (1, 1), (1, 1)),
-             (9, 3, 32, 32, 32, (1, 1), (1, 1))]
+             (9, 3, 32, 32, 32, (1, 1), (1, 1)), (70, 3, 32, 32, 64, (1, 1), (1, 1))]
     for (B, Cin, H, W, Cout, st, pd) in SMALLC_CASES + extra:
         case = (B, Cin, H, W, Cout, st, pd)
         x = rng.uniform(-1, 1, (B, Cin, H, W))
@@ -861,6 +862,21 @@ def test_conv2d_f64_image_layer_forward(ctx, orc):
         two = ctx.conv2d_fwd(dx_, dw_, st, pd)
         capi.check(capi.lib.fx_bias_act_f64(ctx.h, two.ptr, db_.ptr, B, Cout, oh * ow, 1))
         assert np.array_equal(fused.numpy(), two.numpy()), ("bias+relu", case)
+        # the weight gradient of the layer (conv_image_f64.hpp for 1 to 3 channels on maps 32 wide, the implicit GEMM otherwise)
+        g = rng.standard_normal((B, Cout, oh, ow))
+        dg_ = ctx.upload(g)
+        gw = ctx.conv2d_wgrad(dx_, dg_, w.shape, st, pd, 0).numpy()
+        tw = torch.from_numpy(w).requires_grad_(True)
+        F.conv2d(torch.from_numpy(x), tw, stride=st, padding=pd).backward(torch.from_numpy(g))
+        assert rel_err(gw, tw.grad.numpy()) <= tol * 8, ("wgrad", case)
+        assert rel_err(gw, orc.conv2d_wgrad(x, g, w.shape, st, pd, 0)) <= tol * 8, ("wgrad vs oracle", case)
+        assert np.array_equal(ctx.conv2d_wgrad(dx_, dg_, w.shape, st, pd, 0).numpy(), gw), case
+        need = capi.lib.fx_conv2d_workspace_bytes(capi.CONV_WGRAD, capi.FX_F64, 0, *dims)
+        assert need >= 0
+        ws = ctx.empty((max(need, 8) // 8,), np.float64)
+        out = ctx.empty(w.shape, np.float64)
+        capi.check(capi.lib.fx_conv2d_wgrad_f64(ctx.h, dx_.ptr, dg_.ptr, out.ptr, *dims, 0, ws.ptr, need))
+        assert np.array_equal(out.numpy(), gw), case
 
 
 def test_conv2d_tune_up_front_and_ragged_batch(ctx, orc):
