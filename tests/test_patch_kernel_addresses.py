@@ -1157,3 +1157,114 @@ def test_stride2_f64_forward_patch_kernel_accesses_stay_inside_the_tensors(case)
     pl = fwd2_plan(B, Cin, H, W, Cout, 3, 3, 2, 2, 1, 1, oh, ow)
     assert pl is not None, "the shape must exercise the f64 stride-2 forward patch kernel"
     assert fwd2_walk(pl, B, Cin, Cout, oh) == "fwd2 ok"
+
+
+# ---- f64 image layer, forward and weight gradient (conv_image_f64.hpp) ----
+def cim_walk(B, Cin, H, Cout, wgrad, num_cus=256):
+    """Offsets in doubles; 16-byte loads must sit on even offsets."""
+    NTI, W, TR, CP = 512, 32, 8, 4
+    PR, PW = TR + 2, W + 2
+    PLANE = (PR * PW) | 1
+    X2 = CP * PR * (W // 2)
+    L, K, tpi = H * W, Cin * 9, H // TR
+    xsize, gsize = B * Cin * L, B * Cout * L
+    assert H % TR == 0 and Cout % 32 == 0 and 1 <= Cin <= (3 if wgrad else 4) and X2 <= 2 * NTI
+    tiles = B * tpi
+
+    def stage_patch(b, oy0):
+        cells = set()
+        for f in range(X2):
+            cr, q = divmod(f, W // 2); c, r = divmod(cr, PR)
+            iy = oy0 - 1 + r
+            if c < Cin and 0 <= iy < H:
+                a = b * Cin * L + (c * H + iy) * W + 2 * q
+                assert 0 <= a and a + 2 <= xsize and a % 2 == 0, ("x", a)
+            d = c * PLANE + r * PW + 1 + 2 * q
+            assert d + 2 <= CP * PLANE
+            cells.update((d, d + 1))
+        for i in range(CP * PR * 2):
+            cr = i >> 1
+            cells.add((cr // PR) * PLANE + (cr % PR) * PW + (i & 1) * (W + 1))
+        return cells
+
+    if not wgrad:
+        nmt = Cout // 32
+        for blk in sorted({0, nmt - 1, nmt, tiles * nmt - 1}):
+            bt, mt = divmod(blk, nmt); b, tile = divmod(bt, tpi)
+            oc0, oy0 = mt * 32, tile * TR
+            cells = stage_patch(b, oy0)
+            wcells = set()
+            for i in range(32 * CP * 9):
+                ocl, r = divmod(i, CP * 9); cl, t = divmod(r, 9)
+                if cl < Cin: assert (oc0 + ocl) * K + cl * 9 + t < Cout * K
+                wcells.add((t * 2 + (ocl >> 4)) * 64 + cl * 16 + (ocl & 15))
+            assert wcells == set(range(9 * 2 * 64))
+            for wave in range(8):
+                for lane in (0, 15, 16, 63):
+                    kq, l16 = lane >> 4, lane & 15
+                    for h in range(2):
+                        pix = wave * 32 + 16 * h + l16
+                        for t in range(9):
+                            d = kq * PLANE + (pix // W + t // 3) * PW + pix % W + t % 3
+                            assert d in cells
+                        for m in range(2):
+                            for e in (0, 3):
+                                a = (b * Cout + oc0 + 16 * m + 4 * e + kq) * L + oy0 * W + pix
+                                assert 0 <= a < gsize
+        return "cim fwd ok"
+    rows = Cout // 32
+    splits = max(1, min(2 * num_cus // rows, max(1, tiles // 2)))
+    tps = _ceil_div(tiles, splits); splits = _ceil_div(tiles, tps)
+    covered = set()
+    for z in range(splits): covered |= set(range(z * tps, min(tiles, (z + 1) * tps)))
+    assert covered == set(range(tiles))
+    GP = 257
+    assert (max(32 * GP + CP * PLANE, 8 * 16 * 64)) * 8 <= 96 * 1024
+    for tl in sorted({0, tpi - 1, tiles - 1}):
+        b, tile = divmod(tl, tpi); oy0 = tile * TR
+        cells = stage_patch(b, oy0)
+        for oc0 in (0, Cout - 32):
+            gcells = set()
+            for f in range(8 * NTI):
+                row, q = f >> 7, f & 127
+                a = (b * Cout + oc0 + row) * L + oy0 * W + 2 * q
+                assert 0 <= a and a + 2 <= gsize and a % 2 == 0, ("g", a)
+                gcells.update((row * GP + 2 * q, row * GP + 2 * q + 1))
+            for wave in range(8):
+                for lane in (0, 15, 16, 26, 63):
+                    kq, l16 = lane >> 4, lane & 15
+                    for s in range(W // 4):
+                        for m in range(2):
+                            assert (l16 + 16 * m) * GP + wave * W + kq + 4 * s in gcells
+                        for nb in range(2):
+                            kp = 16 * nb + l16
+                            c, t = divmod(kp, 9) if kp < K else (0, 0)
+                            d = c * PLANE + (wave + t // 3) * PW + t % 3 + kq + 4 * s
+                            assert d in cells
+                            # the word is pixel (row wave, column 4 s + kq) shifted by the tap
+                            assert d == c * PLANE + (wave + t // 3) * PW + (4 * s + kq) + t % 3
+    # partial sums: [splits][Cout][K], every (oc, pair < K) written once per split
+    for z in (0, splits - 1):
+        for oc0 in (0, Cout - 32):
+            seen = set()
+            for wave in range(8):
+                for u in range(2):
+                    el = 2 * wave + u; blk, e = el >> 2, el & 3
+                    for lane in range(64):
+                        kq, l16 = lane >> 4, lane & 15
+                        oc, kp = 16 * (blk >> 1) + 4 * e + kq, 16 * (blk & 1) + l16
+                        if kp < K:
+                            a = (z * Cout + oc0 + oc) * K + kp
+                            assert 0 <= a < splits * Cout * K and a not in seen
+                            seen.add(a)
+            assert len(seen) == 32 * K
+    return "cim wgrad ok"
+
+
+@pytest.mark.parametrize("case", [(256, 3, 32, 32), (2, 1, 8, 64), (3, 4, 40, 96), (5, 2, 24, 32)], ids=str)
+def test_f64_image_layer_kernels_accesses_stay_inside_the_tensors(case):
+    B, Cin, H, Cout = case
+    B = min(B, 9)
+    assert cim_walk(B, Cin, H, Cout, wgrad=False) == "cim fwd ok"
+    if Cin <= 3:
+        assert cim_walk(B, Cin, H, Cout, wgrad=True) == "cim wgrad ok"
