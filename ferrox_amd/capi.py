@@ -87,6 +87,8 @@ _sig("fx_pool_bucket_stats_get", _vp, _int, _int, C.POINTER(BucketStats))
 _sig("fx_h2d", _vp, _vp, _vp, _i64)
 _sig("fx_d2h", _vp, _vp, _vp, _i64)
 _sig("fx_d2d", _vp, _vp, _vp, _i64)
+_sig("fx_scratch_info", _vp, C.POINTER(_vp), C.POINTER(_i64), C.POINTER(_i64), C.POINTER(_i64))
+_sig("fx_device_mem_info", _vp, C.POINTER(_i64), C.POINTER(_i64))
 _sig("fx_conv2d_workspace_bytes", _int, _int, _int, *([_i64] * 11), restype=_i64)
 
 _CONV_INTS = [_i64] * 11
@@ -277,6 +279,17 @@ class Context:
 
     def graph_destroy(self, g):
         check(lib.fx_graph_destroy(self.h, g))
+
+    def scratch_info(self):
+        """The library's own scratch region: address, bytes, outgrown regions parked for live graphs, live graphs."""
+        cur, b, p, g = _vp(), _i64(0), _i64(0), _i64(0)
+        check(lib.fx_scratch_info(self.h, C.byref(cur), C.byref(b), C.byref(p), C.byref(g)))
+        return {"current": cur.value or 0, "bytes": b.value, "parked_regions": p.value, "live_graphs": g.value}
+
+    def device_mem_info(self):
+        f, t = _i64(0), _i64(0)
+        check(lib.fx_device_mem_info(self.h, C.byref(f), C.byref(t)))
+        return {"free": f.value, "total": t.value}
 
     def sync(self):
         check(lib.fx_sync(self.h))

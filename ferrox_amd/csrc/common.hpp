@@ -75,6 +75,11 @@ struct fx_ctx {
     // library-owned scratch (split-K partials, reduction partials, permuted weights); grows on demand
     void* scratch = nullptr;
     i64 scratch_bytes = 0;
+    // Recorded graphs keep the scratch address of their recording in their kernel arguments.  While any such graph is alive
+    // (fx_graph_end .. fx_graph_destroy) a region that has to grow is parked here instead of freed, so a later launch of the
+    // graph still finds its region; the parked regions are freed when the last graph is destroyed (or with the context).
+    int live_graphs = 0;
+    std::vector<void*> parked_scratch;
     std::mutex launch_mutex;
     // tile shape that measured fastest per convolution layer shape (conv_patch.hpp); used under launch_mutex
     std::map<std::array<i64, 14>, int> conv_tile_cache;

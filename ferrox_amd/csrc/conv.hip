@@ -734,6 +734,7 @@ extern "C" int64_t fx_conv2d_workspace_bytes(int kind, int dtype, int mode, int6
 extern "C" int fx_conv2d_tune_f32(fx_ctx* c, int kind, int64_t B, int64_t Cin, int64_t H, int64_t W, int64_t Cout, int64_t kh,
                                   int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw, int with_bias, int act) {
     FX_CHECK_CTX(c);
+    FX_NOT_RECORDING(c, "fx_conv2d_tune");
     FX_REQUIRE(kind == FX_CONV_FWD || kind == FX_CONV_DGRAD || kind == FX_CONV_WGRAD, "fx_conv2d_tune: unknown kind %d", kind);
     FX_REQUIRE(act == 0 || act == 1, "fx_conv2d_tune: act must be 0 (none) or 1 (relu)");
     Dims d;

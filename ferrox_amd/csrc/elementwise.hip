@@ -204,6 +204,9 @@ template <typename T> struct InRangeF {
     T lo, hi;
     __device__ __forceinline__ T operator()(T x, T) const { return (x >= lo && x <= hi) ? T(1) : T(0); }
 };
+template <typename T> struct CopyF {  // moves the bits: no arithmetic touches the value
+    __device__ __forceinline__ T operator()(T x, T) const { return x; }
+};
 template <typename T> struct FillF {
     T v;
     __device__ __forceinline__ T operator()(T, T) const { return v; }
@@ -649,3 +652,15 @@ int dropout(fx_ctx* c, const T* x, T* mask, T* y, i64 n, double p, uint64_t seed
 
 FX_DEFINE_EW(float, f32)
 FX_DEFINE_EW(double, f64)
+
+// Device-to-device copy of a small block as a streaming kernel on the context's stream.  A hipMemcpyAsync D2D of a few KB
+// to a few MB occupies the stream about twice as long as this kernel (a training step of the op-by-op engines issues dozens
+// of such clones).  4-byte granularity; returns FX_ERR_UNSUPPORTED for anything else so the caller can fall back.
+namespace fx {
+int copy_kernel(fx_ctx* c, void* dst, const void* src, i64 bytes) {
+    if ((bytes & 3) != 0 || (reinterpret_cast<uintptr_t>(dst) & 3u) != 0 || (reinterpret_cast<uintptr_t>(src) & 3u) != 0)
+        return FX_ERR_UNSUPPORTED;
+    return launch_ew<float, 1>(c, static_cast<const float*>(src), (const float*)nullptr, static_cast<float*>(dst), bytes / 4,
+                               CopyF<float>{}, "fx_d2d");
+}
+}  // namespace fx

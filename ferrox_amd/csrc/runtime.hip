@@ -2,6 +2,7 @@
 // Replaces CudaContextManager (src/backend/cuda/context.rs:30-175) and the named-stream StreamManager
 // (src/backend/cuda/stream_manager.rs:97-103): one compute stream, synchronous copies ordered on it.
 #include <cstdarg>
+#include <cstdlib>
 #include <cstring>
 
 #include "common.hpp"
@@ -22,6 +23,7 @@ int bind_device(int device) {
 }
 Pool* pool_create(const fx_pool_config* cfg, int elem_size, hipStream_t stream, const bool* recording);
 int static_scratch_init(int device);  // reduce.hip
+int copy_kernel(fx_ctx* c, void* dst, const void* src, i64 bytes);  // elementwise.hip
 void pool_destroy(Pool* p);
 }  // namespace fx
 
@@ -34,8 +36,12 @@ void* fx_ctx::get_scratch(i64 bytes) {
     }
     // Work already queued on the stream may still use the old region.
     if (scratch) {
-        if (hipStreamSynchronize(stream) != hipSuccess) return nullptr;
-        (void)hipFree(scratch);
+        if (live_graphs > 0) {
+            parked_scratch.push_back(scratch);  // a recorded graph still points into it
+        } else {
+            if (hipStreamSynchronize(stream) != hipSuccess) return nullptr;
+            (void)hipFree(scratch);
+        }
         scratch = nullptr;
         scratch_bytes = 0;
     }
@@ -99,6 +105,7 @@ int fx_destroy(fx_ctx* c) {
     fx::pool_destroy(c->pools[0]);
     fx::pool_destroy(c->pools[1]);
     if (c->scratch) (void)hipFree(c->scratch);
+    for (void* p : c->parked_scratch) (void)hipFree(p);
     (void)hipEventDestroy(c->ev_start);
     (void)hipEventDestroy(c->ev_stop);
     for (hipEvent_t e : c->ev_tune)
@@ -126,6 +133,7 @@ void* fx_stream(fx_ctx* c) { return c ? (void*)c->stream : nullptr; }
 
 int fx_timer_start(fx_ctx* c) {
     FX_CHECK_CTX(c);
+    FX_NOT_RECORDING(c, "fx_timer_start");
     FX_HIP_CHECK(hipEventRecord(c->ev_start, c->stream));
     return FX_OK;
 }
@@ -251,6 +259,7 @@ int fx_graph_end(fx_ctx* c, fx_graph** out) {
         fx::set_error("fx_graph_end: hipGraphInstantiate failed: %s", hipGetErrorString(ei));
         return FX_ERR_HIP;
     }
+    c->live_graphs += 1;
     *out = fg;
     return FX_OK;
 }
@@ -260,6 +269,24 @@ int fx_graph_launch(fx_ctx* c, fx_graph* g) {
     FX_REQUIRE(g && g->exec, "fx_graph_launch: null graph");
     FX_REQUIRE(!c->capturing, "fx_graph_launch: a graph is being recorded on this context");
     FX_HIP_CHECK(hipGraphLaunch(g->exec, c->stream));
+    return FX_OK;
+}
+
+int fx_scratch_info(fx_ctx* c, void** current, int64_t* bytes, int64_t* parked_regions, int64_t* live_graphs) {
+    FX_REQUIRE(c != nullptr, "null context");
+    if (current) *current = c->scratch;
+    if (bytes) *bytes = c->scratch_bytes;
+    if (parked_regions) *parked_regions = (int64_t)c->parked_scratch.size();
+    if (live_graphs) *live_graphs = c->live_graphs;
+    return FX_OK;
+}
+
+int fx_device_mem_info(fx_ctx* c, int64_t* free_bytes, int64_t* total_bytes) {
+    FX_CHECK_CTX(c);
+    size_t f = 0, t = 0;
+    FX_HIP_CHECK(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = (int64_t)f;
+    if (total_bytes) *total_bytes = (int64_t)t;
     return FX_OK;
 }
 
@@ -280,6 +307,11 @@ int fx_graph_destroy(fx_ctx* c, fx_graph* g) {
     if (g->graph) (void)hipGraphDestroy(g->graph);
     const int rc = release_held(c, g->held);
     delete g;
+    if (--c->live_graphs <= 0) {  // the stream is idle (synchronised above): nothing uses the parked regions any more
+        c->live_graphs = 0;
+        for (void* p : c->parked_scratch) (void)hipFree(p);
+        c->parked_scratch.clear();
+    }
     return rc;
 }
 
@@ -287,6 +319,13 @@ int fx_d2d(fx_ctx* c, void* dst, const void* src, int64_t bytes) {
     FX_CHECK_CTX(c);
     FX_REQUIRE(bytes >= 0 && (bytes == 0 || (dst && src)), "fx_d2d: bad arguments");
     if (bytes == 0) return FX_OK;
+    // blocks up to 32 MiB go through the library's own streaming kernel (half the stream time of a runtime copy at these
+    // sizes); larger ones and odd sizes / alignments through the runtime
+    static const bool use_kernel = !(getenv("FX_D2D_KERNEL") && atoi(getenv("FX_D2D_KERNEL")) == 0);
+    if (use_kernel && bytes <= (32ll << 20)) {
+        const int rc = fx::copy_kernel(c, dst, src, bytes);
+        if (rc != FX_ERR_UNSUPPORTED) return rc;
+    }
     FX_HIP_CHECK(hipMemcpyAsync(dst, src, (size_t)bytes, hipMemcpyDeviceToDevice, c->stream));
     return FX_OK;
 }

@@ -193,6 +193,7 @@ template <typename T> struct Model : ModelBase {
     // Moves the listed parameters (indices into the model's parameter list) out of their groups into a new group with
     // its own lr / weight decay / momentum (NaN = not set: the optimizer's value applies), ParameterGroup of optim/mod.rs:203-258.
     void add_param_group(const int* idx, int n, double lr, double wd, double mom) override {
+        drop_graph();  // lr / weight decay / momentum and the pointer tables are arguments of the recorded kernels
         ParameterGroup<T> group("group" + std::to_string(opt->param_groups.size()));
         for (int k = 0; k < n; ++k) {
             const NodeId id = params.at((size_t)idx[k]);
@@ -205,6 +206,7 @@ template <typename T> struct Model : ModelBase {
         opt->add_param_group(std::move(group));
     }
     void set_training(bool t) override {
+        drop_graph();  // batch statistics or running statistics: a different kernel sequence
         for (auto& l : layers) l->set_training(t);
     }
     std::vector<const HipStorage<T>*> all_state() const {
@@ -220,11 +222,14 @@ template <typename T> struct Model : ModelBase {
         std::memcpy(host, v.data(), v.size() * sizeof(T));
     }
     std::vector<uint8_t> optimizer_state() const override { return opt->state_dict().save_to_bytes(); }
-    void load_optimizer_state(const uint8_t* data, size_t n) override { opt->load_state_dict(OptimizerStateDict::load_from_bytes(data, n)); }
+    void load_optimizer_state(const uint8_t* data, size_t n) override {
+        drop_graph();  // the moments move to new tensors: a recording made before would keep updating the old addresses
+        opt->load_state_dict(OptimizerStateDict::load_from_bytes(data, n));
+    }
     int num_params() const override { return (int)params.size(); }
     int64_t param_numel(int i) const override { return (int64_t)graph.get_tensor(params.at(i))->size(); }
     void set_batch(const void* xv, const Shape& xs, const void* yv, const Shape& ys) override {
-        if (graph_on && x && y && x->shape() == xs && y->shape() == ys) {
+        if (graph_on && graph_supported() && x && y && x->shape() == xs && y->shape() == ys) {
             // a recorded step reads the batch at the addresses it was recorded with: new data goes there
             fx_ok(fx_h2d(BackendManager::get().ctx(), x->data(), xv, (int64_t)(x->size() * sizeof(T))));
             fx_ok(fx_h2d(BackendManager::get().ctx(), y->data(), yv, (int64_t)(y->size() * sizeof(T))));
@@ -237,6 +242,7 @@ template <typename T> struct Model : ModelBase {
     }
     void configure(int kind, bool in_grad) override {
         if (kind != 0 && kind != 1) throw Error("unknown loss kind");
+        drop_graph();  // another loss or another kind of input leaf: another step
         loss_kind = kind;
         input_requires_grad = in_grad;
     }

@@ -399,6 +399,16 @@ int fx_graph_launch(fx_ctx* ctx, fx_graph* graph);
 /* number of nodes, of kernel nodes, and of pool blocks the graph keeps (any pointer may be NULL) */
 int fx_graph_info(fx_graph* graph, int64_t* nodes, int64_t* kernel_nodes, int64_t* held_blocks);
 int fx_graph_destroy(fx_ctx* ctx, fx_graph* graph);
+/* The library's own scratch region (split-K partials, weight images, reduction partials): its address and size, the
+ * number of outgrown regions kept alive for recorded graphs, and the number of live graphs (any pointer may be NULL).
+ * A recorded graph holds the scratch address of its recording.  While a graph made by fx_graph_end has not been
+ * destroyed, a later eager call that needs a larger region allocates a new one and PARKS the old one (it stays valid
+ * for the graph's launches) instead of freeing it; parked regions are freed when the last graph is destroyed or with
+ * the context.  Host-only query: it never touches the stream. */
+int fx_scratch_info(fx_ctx* ctx, void** current, int64_t* bytes, int64_t* parked_regions, int64_t* live_graphs);
+/* Free and total device memory as the driver reports it (hipMemGetInfo); either pointer may be NULL.  No counterpart
+ * in the reference: callers use it to check that a call allocated nothing. */
+int fx_device_mem_info(fx_ctx* ctx, int64_t* free_bytes, int64_t* total_bytes);
 /* Page-locked host memory and an upload from it that does not wait (fx_h2d waits for the copy). */
 int fx_host_alloc(fx_ctx* ctx, int64_t bytes, void** out);
 int fx_host_free(fx_ctx* ctx, void* ptr);

@@ -17,3 +17,8 @@ def golden():
     import json
     with open(os.path.join(ROOT, "tests", "golden", "reference_vectors.json")) as f:
         return json.load(f)
+
+
+def pytest_sessionfinish(session, exitstatus):
+    import parity
+    parity.dump(ROOT)

@@ -122,3 +122,24 @@ def test_pooling_reference_vectors(ctx, golden):
         x, want = (np.array(v, np.float32) for v in golden[key]["arrays"])
         got = ctx.pool2d(ctx.upload(x.reshape(shape)), k, k, (0, 0), is_max).numpy()
         assert np.array_equal(got.ravel(), want), key
+
+
+def test_device_to_device_copy_moves_every_bit_pattern(ctx):
+    """fx_d2d: small blocks run as a copy kernel, large / odd ones through the runtime; random 32-bit patterns (NaN payloads,
+    denormals, both zeros) must arrive unchanged at every size and alignment."""
+    import ctypes as C
+    from ferrox_amd.capi import check, lib
+    rng = np.random.default_rng(77)
+    n = (40 << 20) // 4 + 3
+    bits = rng.integers(0, 2 ** 32, n, dtype=np.uint32)
+    bits[:4] = [0x7FC00001, 0x7F800001, 0x80000000, 0x00000001]   # quiet NaN with payload, signalling NaN, -0, denormal
+    src = ctx.upload(bits.view(np.float32))
+    dst = ctx.fill((n + 8,), 0.0, np.float32)
+    for off_src, off_dst, nbytes in [(0, 0, 4), (0, 0, 16), (4, 8, 4 * 1027), (0, 4, 1 << 20), (12, 0, (1 << 20) + 4), (0, 0, 3),
+                                     (1, 2, 1001), (0, 0, 32 << 20), (0, 0, (32 << 20) + 4), (4, 4, 40 << 20), (0, 0, 0)]:
+        check(lib.fx_fill_f32(ctx.h, dst.ptr, C.c_float(0.0), n + 8))
+        check(lib.fx_d2d(ctx.h, dst.ptr + off_dst, src.ptr + off_src, nbytes))
+        got = dst.numpy().view(np.uint8)
+        want = np.zeros((n + 8) * 4, np.uint8)
+        want[off_dst:off_dst + nbytes] = bits.view(np.uint8)[off_src:off_src + nbytes]
+        assert np.array_equal(got, want), (off_src, off_dst, nbytes)

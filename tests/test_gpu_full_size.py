@@ -47,20 +47,31 @@ def test_c3_convolution_full_size(ctx):
     # sampled entries of each pass, corners and edges included, against float64 sums; tolerance 1e-5 of sum |terms|
     pts = [(0, 0, 0, 0), (B - 1, Cout - 1, H - 1, W - 1), (5, 7, 0, W - 1), (9, 3, H - 1, 0)]
     pts += [tuple(int(v) for v in (rng.integers(B), rng.integers(Cout), rng.integers(H), rng.integers(W))) for _ in range(600)]
+    import parity
+    got_s, ref_s = [], []
     for (b, oc, oy, ox) in pts:
         patch = xp[b, :, oy:oy + 3, ox:ox + 3].astype(np.float64)
         ref, mag = (patch * w64[oc]).sum(), np.abs(patch * w64[oc]).sum()
         assert abs(y[b, oc, oy, ox] - ref) <= 1e-5 * mag, ("fwd", b, oc, oy, ox)
+        got_s.append(y[b, oc, oy, ox]); ref_s.append(ref)
+    # and the contract's own form on the sample: max |got - truth| within 1e-5 of max |truth|
+    parity.check("C3 full size fwd (604 sampled outputs)", np.array(got_s), np.array(ref_s), np.float32, case=(B, Cin, H, W, Cout))
+    got_s, ref_s = [], []
     for _ in range(600):
         b, c, yy, xx = (int(v) for v in (rng.integers(B), rng.integers(Cin), rng.integers(H), rng.integers(W)))
         # dx[b,c,y,x] = sum_{oc,ky,kx} g[b,oc,y+1-ky,x+1-kx] * w[oc,c,ky,kx]
         patch = gp[b, :, yy:yy + 3, xx:xx + 3][:, ::-1, ::-1].astype(np.float64)
         terms = patch * w64[:, c]
         assert abs(gx[b, c, yy, xx] - terms.sum()) <= 1e-5 * np.abs(terms).sum(), ("dgrad", b, c, yy, xx)
+        got_s.append(gx[b, c, yy, xx]); ref_s.append(terms.sum())
+    parity.check("C3 full size dgrad (600 sampled outputs)", np.array(got_s), np.array(ref_s), np.float32, case=(B, Cin, H, W, Cout))
+    got_s, ref_s = [], []
     for _ in range(40):
         oc, c, ky, kx = (int(v) for v in (rng.integers(Cout), rng.integers(Cin), rng.integers(3), rng.integers(3)))
         terms = g[:, oc].astype(np.float64) * xp[:, c, ky:ky + H, kx:kx + W]
         assert abs(gw[oc, c, ky, kx] - terms.sum()) <= 1e-5 * np.abs(terms).sum(), ("wgrad", oc, c, ky, kx)
+        got_s.append(gw[oc, c, ky, kx]); ref_s.append(terms.sum())
+    parity.check("C3 full size wgrad (40 sampled outputs)", np.array(got_s), np.array(ref_s), np.float32, case=(B, Cin, H, W, Cout))
     # adjoint identity: <conv(x, w), g> = <x, dgrad(g, w)> = <w, wgrad(x, g)>
     a, mag = dot64(y, g)
     b_, _ = dot64(x, gx)

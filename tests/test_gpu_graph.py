@@ -179,3 +179,114 @@ def test_models_that_cannot_be_recorded_stay_eager(host):
             assert np.array_equal(models[0].param(i), models[1].param(i))
         for m in models:
             m.close()
+
+
+def test_input_leaf_with_gradient_follows_the_batch_with_graphs_enabled(host):
+    """A model whose batch enters as a leaf with a gradient is never recorded; with graphs enabled it must still read each
+    new batch (not the copy of the first one) and hand out the gradient of that batch."""
+    spec, in_shape = MLP_SMALL, (9, 20)
+    params, x, y = kaiming_uniform_problem(spec, in_shape, 5, 9, np.float32)
+    rng = np.random.default_rng(21)
+    models = [host.Model(spec, params, "sgd 0.05", np.float32, literal_engine=False, fused=True) for _ in range(2)]
+    for m in models:
+        m.configure("cce", input_requires_grad=True)
+    models[1].enable_graph()
+    for step in range(4):
+        bx = rng.standard_normal(in_shape).astype(np.float32)
+        losses, grads = [], []
+        for m in models:
+            m.set_batch(bx, y)
+            losses.append(m.train_step())
+            grads.append(m.input_grad(in_shape))
+        assert losses[0] == losses[1], step
+        assert np.array_equal(grads[0], grads[1]), step
+        if step:
+            assert losses[0] != first  # the batch did change what the model saw
+        first = losses[0]
+    assert models[1].graph_info()["kernel_nodes"] == 0
+    for m in models:
+        m.close()
+
+
+@pytest.mark.parametrize("optspec", ["adam 0.001 0.9 0.999 1e-08 0.01 1", "sgd 0.05 0.9 0.0005 1"])
+def test_a_recording_is_dropped_when_the_state_it_holds_changes(host, optspec):
+    """Loading optimizer state, adding a parameter group, switching the training mode or the loss after a step was recorded:
+    the recording holds the old moment buffers, learning rates and kernel sequence, so the model must record again.  Checked
+    against an eager model that gets the same calls: losses, parameters, gradients and the saved optimizer state stay equal."""
+    spec, in_shape, ncls = CNN_SMALL, (5, 3, 8, 8), 5
+    params, x, y = kaiming_uniform_problem(spec, in_shape, ncls, 7, np.float32)
+    rng = np.random.default_rng(31)
+    models = [host.Model(spec, params, optspec, np.float32, literal_engine=False, fused=True) for _ in range(2)]
+    models[1].enable_graph()
+
+    def steps(n):
+        for _ in range(n):
+            bx = rng.standard_normal(in_shape).astype(np.float32)
+            by = np.eye(ncls, dtype=np.float32)[rng.integers(0, ncls, in_shape[0])]
+            losses = []
+            for m in models:
+                m.set_batch(bx, by)
+                losses.append(m.train_step())
+            assert losses[0] == losses[1]
+        for i in range(len(params)):
+            assert np.array_equal(models[0].param(i), models[1].param(i)), i
+            assert np.array_equal(models[0].grad(i), models[1].grad(i)), i
+        assert models[0].optimizer_state() == models[1].optimizer_state()
+
+    steps(4)
+    assert models[1].graph_info()["kernel_nodes"] > 0
+    saved = models[0].optimizer_state()
+    steps(2)
+    for m in models:
+        m.load_optimizer_state(saved)          # moments back to the state two steps ago, in new tensors
+    assert models[1].graph_info()["kernel_nodes"] == 0
+    steps(4)
+    assert models[1].graph_info()["kernel_nodes"] > 0
+    for m in models:
+        m.add_param_group([0, 1], lr=0.01, weight_decay=0.0)
+    assert models[1].graph_info()["kernel_nodes"] == 0
+    steps(4)
+    assert models[1].graph_info()["kernel_nodes"] > 0
+    for m in models:
+        m.set_training(False)
+    assert models[1].graph_info()["kernel_nodes"] == 0
+    for m in models:
+        m.set_training(True)
+    steps(3)
+    for m in models:
+        m.close()
+
+
+def test_scratch_that_grows_after_a_recording_is_parked_not_freed(ctx):
+    """A recorded split reduction keeps the scratch address of its recording.  A later, larger eager request must leave
+    that region alive (parked) until the graph is destroyed; the replay after the growth still gives the eager bits.
+    Host-side checks of the region bookkeeping; every kernel runs on valid memory either way."""
+    rng = np.random.default_rng(5)
+    a = ctx.upload(rng.standard_normal((64, 70000)).astype(np.float32))
+    out = ctx.empty((70000,), np.float32)
+    ctx.reduce("sum", a, 0, out=out)            # eager once: sizes the scratch region for this call
+    ref = out.numpy().copy()
+    before = ctx.scratch_info()
+    ctx.graph_begin()
+    ctx.reduce("sum", a, 0, out=out)
+    g = ctx.graph_end()
+    assert ctx.scratch_info()["live_graphs"] == before["live_graphs"] + 1
+    # a larger request: maxima with positions along axis 0 of [64, 100000 * k] leave 2 slices x 12 bytes per column
+    k = 1
+    while 2 * 100000 * k * 12 <= before["bytes"]:
+        k *= 2
+    big = ctx.fill((64, 100000 * k), 1.0, np.float32)
+    need_more, _ = ctx.reduce("max", big, 0, want_idx=True)
+    grown = ctx.scratch_info()
+    assert grown["bytes"] > before["bytes"]
+    assert grown["parked_regions"] == before["parked_regions"] + 1 and grown["current"] != before["current"]
+    ctx.unary("neg", out, out=out)
+    ctx.graph_launch(g)
+    assert np.array_equal(out.numpy(), ref)
+    ctx.graph_destroy(g)
+    after = ctx.scratch_info()
+    assert after["live_graphs"] == before["live_graphs"]
+    if after["live_graphs"] == 0:
+        assert after["parked_regions"] == 0
+    assert np.array_equal(need_more.numpy(), np.ones(big.shape[1], np.float32))
+    big.free()

@@ -6,8 +6,10 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
+import parity
+from parity import TOL
+
 DTYPES = [np.float32, np.float64]
-TOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float64): 1e-12}
 
 
 @pytest.fixture(scope="module")
@@ -79,10 +81,10 @@ def test_unary_ops(ctx, orc, dtype):
             ref = orc.unary(op, a.astype(np.float64)).astype(dtype)  # overflow to inf exactly where T overflows
         # tanh's exp-based formula (cpu.rs:1120-1146) cancels near 0 in T on CPU and GPU alike: allow a few ulp of 1.0
         atol = 4 * np.finfo(dtype).eps if op == "tanh" else 0
-        np.testing.assert_allclose(ctx.unary(op, da).numpy(), ref, rtol=TOL[np.dtype(dtype)] * 4, atol=atol, err_msg=op)
+        np.testing.assert_allclose(ctx.unary(op, da).numpy(), ref, rtol=TOL[np.dtype(dtype)], atol=atol, err_msg=op)
     for op in ("sqrt", "log", "reciprocal"):
         ref = orc.unary(op, (np.abs(a) + dtype(1e-3)).astype(np.float64))
-        assert rel_err(ctx.unary(op, pos).numpy(), ref) <= TOL[np.dtype(dtype)] * 4, op
+        parity.check("unary " + op, ctx.unary(op, pos).numpy(), ref)
     # saturation like the CPU backend (tensor.rs:2667-2729): exactly +-1 beyond |x| > 20, sigmoid -> 0 / 1
     t = ctx.unary("tanh", da).numpy()
     assert t[2] == 1.0 and t[3] == -1.0 and t[4] == 1.0 and t[5] == -1.0
@@ -205,19 +207,18 @@ RED_SHAPES = [(2, 2), (7, 13), (256, 10), (64, 1000), (3, 5, 7), (16, 32, 8, 8),
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_reduce_every_axis(ctx, orc, dtype):
     rng = np.random.default_rng(30)
-    tol = TOL[np.dtype(dtype)]
     for shape in RED_SHAPES:
         x = rng.standard_normal(shape).astype(dtype)
         dx = ctx.upload(x)
         for axis in range(len(shape)):
             truth = x.astype(np.longdouble).sum(axis=axis)
-            bound = tol * np.abs(x).astype(np.float64).sum(axis=axis).max()
+            terms = np.abs(x).astype(np.float64).sum(axis=axis).max()
             got = ctx.reduce("sum", dx, axis).numpy()
-            assert np.abs(got - truth).max() <= bound, ("sum", shape, axis)
-            # and against the oracle's CPU summation order, relative to the same scale
-            assert np.abs(got - orc.reduce_axis("sum", x, axis)).max() <= 2 * bound
+            # the GPU's summation order and the oracle's CPU order, each against the long double sum
+            parity.check("reduce sum", got, truth, oracle=orc.reduce_axis("sum", x, axis), case=(shape, axis), terms=terms)
             got = ctx.reduce("mean", dx, axis).numpy()
-            assert np.abs(got - truth / shape[axis]).max() <= bound / shape[axis] + tol * np.abs(truth / shape[axis]).max()
+            parity.check("reduce mean", got, truth / shape[axis], oracle=orc.reduce_axis("mean", x, axis), case=(shape, axis),
+                         terms=terms / shape[axis])
             v, i = ctx.reduce("max", dx, axis, want_idx=True)
             rv, ri = orc.reduce_axis("max", x, axis, want_idx=True)
             assert np.array_equal(v.numpy(), rv), ("max", shape, axis)
@@ -272,7 +273,7 @@ def test_softmax_axis(ctx, orc, golden, dtype):
     for shape, axis in (((256, 10), 1), ((4, 7, 5), 1), ((6, 9), 0)):
         x = (rng.standard_normal(shape) * 3).astype(dtype)
         got = ctx.softmax_axis(ctx.upload(x), axis).numpy()
-        assert rel_err(got, orc.softmax_axis(x.astype(np.float64), axis)) <= TOL[np.dtype(dtype)] * 4
+        parity.check("softmax_axis", got, orc.softmax_axis(x.astype(np.float64), axis), oracle=orc.softmax_axis(x, axis), case=(shape, axis))
     for key, shape, axis in (("softmax_axis1", (2, 3), 1), ("softmax_axis0", (2, 2), 0)):
         x, y = (np.array(v, dtype) for v in golden[key]["arrays"])
         got = ctx.softmax_axis(ctx.upload(x.reshape(shape)), axis).numpy().ravel()
@@ -287,7 +288,6 @@ GEMM_SHAPES = [(2, 2, 2), (1, 1, 1), (5, 7, 3), (64, 64, 64), (128, 128, 16), (1
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gemm_all_transposes(ctx, orc, golden, dtype):
     rng = np.random.default_rng(40)
-    tol = TOL[np.dtype(dtype)]
     for (M, N, K) in GEMM_SHAPES:
         a = rng.standard_normal((M, K)).astype(dtype)
         b = rng.standard_normal((K, N)).astype(dtype)
@@ -298,7 +298,7 @@ def test_gemm_all_transposes(ctx, orc, golden, dtype):
                 da = ctx.upload(a.T if ta else a)
                 db = ctx.upload(b.T if tb else b)
                 got = ctx.gemm(da, db, ta, tb).numpy()
-                assert np.abs(got - truth).max() <= tol * scale, (M, N, K, ta, tb)
+                parity.check("gemm", got, truth, case=(M, N, K, ta, tb), terms=scale)
     a, b, c = (np.array(v, dtype).reshape(2, 2) for v in golden["matmul"]["arrays"])
     assert np.array_equal(ctx.gemm(ctx.upload(a), ctx.upload(b)).numpy(), c)
     got = ctx.gemm(ctx.upload(rng.standard_normal((64, 64)).astype(dtype)), ctx.upload(np.eye(64, dtype=dtype))).numpy()
@@ -313,7 +313,6 @@ GEMM_LDS_SHAPES = [(2560, 2560, 128), (2500, 2436, 192), (4096, 3200, 64 * 3), (
 def test_gemm_lds_kernel_shapes_all_transposes_and_bias(ctx):
     from ferrox_amd import capi
     rng = np.random.default_rng(41)
-    tol = TOL[np.dtype(np.float32)]
     for (M, N, K) in GEMM_LDS_SHAPES:
         a = rng.standard_normal((M, K)).astype(np.float32)
         b = rng.standard_normal((K, N)).astype(np.float32)
@@ -326,7 +325,7 @@ def test_gemm_lds_kernel_shapes_all_transposes_and_bias(ctx):
                 da = ctx.upload(np.ascontiguousarray(a.T) if ta else a)
                 db = ctx.upload(np.ascontiguousarray(b.T) if tb else b)
                 got = ctx.gemm(da, db, ta, tb)
-                assert np.abs(got.numpy() - truth).max() <= tol * scale, (M, N, K, ta, tb)
+                parity.check("gemm lds", got.numpy(), truth, case=(M, N, K, ta, tb), terms=scale)
                 # same bits run to run, and the bias (+ReLU) epilogue equals the two-call sequence
                 assert np.array_equal(ctx.gemm(da, db, ta, tb).numpy(), got.numpy()), (M, N, K, ta, tb)
                 fused = ctx.empty((M, N), np.float32)
@@ -351,7 +350,6 @@ GEMM_THIN_SHAPES = [
 def test_gemm_with_one_thin_dimension(ctx, dtype):
     from ferrox_amd import capi
     rng = np.random.default_rng(43)
-    tol = TOL[np.dtype(dtype)]
     sfx = "f32" if dtype == np.float32 else "f64"
     for (kind, M, N, K) in GEMM_THIN_SHAPES:
         ta, tb = kind == "m", kind == "n"
@@ -362,7 +360,7 @@ def test_gemm_with_one_thin_dimension(ctx, dtype):
         da = ctx.upload(np.ascontiguousarray(a.T) if ta else a)
         db = ctx.upload(np.ascontiguousarray(b.T) if tb else b)
         got = ctx.gemm(da, db, ta, tb)
-        assert np.abs(got.numpy() - truth).max() <= tol * scale, (kind, M, N, K)
+        parity.check("gemm thin", got.numpy(), truth, case=(kind, M, N, K), terms=scale)
         assert np.array_equal(ctx.gemm(da, db, ta, tb).numpy(), got.numpy()), (kind, M, N, K)
         bias = rng.standard_normal(N).astype(dtype)
         dbias = ctx.upload(bias)
@@ -385,7 +383,6 @@ GEMM_SMALL_SHAPES = [(33, 65, 36), (256, 512, 784), (100, 31, 1024), (1, 1, 32),
 def test_gemm_small_products_all_layouts(ctx, dtype):
     from ferrox_amd import capi
     rng = np.random.default_rng(47)
-    tol = TOL[np.dtype(dtype)]
     sfx = "f32" if dtype == np.float32 else "f64"
     for (M, N, K) in GEMM_SMALL_SHAPES:
         a = rng.standard_normal((M, K)).astype(dtype)
@@ -400,7 +397,7 @@ def test_gemm_small_products_all_layouts(ctx, dtype):
                 db = ctx.upload(np.ascontiguousarray(b.T) if tb else b)
                 got = ctx.gemm(da, db, ta, tb)
                 case = (M, N, K, ta, tb)
-                assert np.abs(got.numpy() - truth).max() <= tol * scale, case
+                parity.check("gemm small", got.numpy(), truth, case=case, terms=scale)
                 assert np.array_equal(ctx.gemm(da, db, ta, tb).numpy(), got.numpy()), case
                 fused = ctx.empty((M, N), dtype)
                 capi.check(getattr(capi.lib, "fx_gemm_bias_act_" + sfx)(ctx.h, int(ta), int(tb), M, N, K, da.ptr, db.ptr, dbias.ptr, fused.ptr, 1))
@@ -424,7 +421,6 @@ def test_gemm_tn_with_column_sums(ctx, dtype):
     """Linear's weight + bias gradient in one call: the product and the column sums of dY to rounding, the same bits run to run
     (one-launch small and thin products, a K that is split over blocks, the general tiles with the sums in a second launch)."""
     rng = np.random.default_rng(57)
-    tol = TOL[np.dtype(dtype)]
     # K (batch), M (out), N (in)
     for (K, M, N) in [(256, 10, 128), (256, 10, 16384), (256, 128, 256), (256, 256, 784), (64, 3, 40), (100, 33, 70), (37, 5, 9),
                       (2048, 10, 64), (512, 600, 520), (256, 40, 16384)]:
@@ -433,10 +429,9 @@ def test_gemm_tn_with_column_sums(ctx, dtype):
         da, db = ctx.upload(a), ctx.upload(b)
         c, s = ctx.gemm_tn_colsum(da, db)
         scale = (np.abs(a.T).astype(np.float64) @ np.abs(b).astype(np.float64)).max()
-        assert np.abs(c.numpy() - a.T.astype(np.float64) @ b.astype(np.float64)).max() <= tol * scale, (K, M, N)
-        truth = a.astype(np.longdouble).sum(axis=0)
-        bound = tol * np.abs(a).astype(np.float64).sum(axis=0).max()
-        assert np.abs(s.numpy() - truth).max() <= bound, (K, M, N)
+        parity.check("gemm tn + colsum: product", c.numpy(), a.T.astype(np.float64) @ b.astype(np.float64), case=(K, M, N), terms=scale)
+        parity.check("gemm tn + colsum: sums", s.numpy(), a.astype(np.longdouble).sum(axis=0), case=(K, M, N),
+                     terms=np.abs(a).astype(np.float64).sum(axis=0).max())
         c2, s2 = ctx.gemm_tn_colsum(da, db)  # the same bits on a second run
         assert np.array_equal(c2.numpy(), c.numpy()) and np.array_equal(s2.numpy(), s.numpy()), (K, M, N)
 
@@ -457,7 +452,7 @@ def test_linear_backward_products_in_one_call(ctx, dtype):
         gx, gw, gb = ctx.linear_bwd(ddy, dw_, dx_)
         # dX: the product (the separate call may run another tile shape, i.e. another summation order)
         scale = (np.abs(dy).astype(np.float64) @ np.abs(w).astype(np.float64)).max()
-        assert np.abs(gx.numpy() - dy.astype(np.float64) @ w.astype(np.float64)).max() <= TOL[np.dtype(dtype)] * scale, ("dX", Bn, I, O)
+        parity.check("linear bwd dX", gx.numpy(), dy.astype(np.float64) @ w.astype(np.float64), case=(Bn, I, O), terms=scale)
         rw, rb = ctx.gemm_tn_colsum(ddy, dx_)
         assert np.array_equal(gw.numpy(), rw.numpy()) and np.array_equal(gb.numpy(), rb.numpy()), ("dW, db", Bn, I, O)
         gx2, gw2, _ = ctx.linear_bwd(ddy, dw_, dx_, want_db=False)
@@ -492,7 +487,6 @@ def test_conv2d_fwd_dgrad_wgrad_vs_oracle(ctx, orc, dtype):
     import torch
     import torch.nn.functional as F
     rng = np.random.default_rng(50)
-    tol = TOL[np.dtype(dtype)]
     for (B, Cin, H, W, Cout, k, s, p) in CONV_CASES:
         x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(dtype)
         w = (rng.standard_normal((Cout, Cin, k, k)) * np.sqrt(2.0 / (Cin * k * k))).astype(dtype)
@@ -509,18 +503,20 @@ def test_conv2d_fwd_dgrad_wgrad_vs_oracle(ctx, orc, dtype):
         ty.backward(torch.from_numpy(g).double())
         ay = F.conv2d(tx.detach().abs(), tw.detach().abs(), stride=s, padding=p).max().item()
         case = (B, Cin, H, W, Cout, k, s, p)
-        assert np.abs(y - ty.detach().numpy()).max() <= tol * ay, ("fwd", case)
-        assert rel_err(dxg, tx.grad.numpy()) <= tol * 8, ("dgrad", case)
-        assert rel_err(dwg, tw.grad.numpy()) <= tol * 8, ("wgrad", case)
-        # and against the CPU oracle (restated reference algorithm), both gradient modes
-        assert rel_err(y, orc.conv2d_fwd(x, w, (s, s), (p, p))) <= tol * 8
-        assert rel_err(dxg, orc.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), 0)) <= tol * 8
-        assert rel_err(dwg, orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 0)) <= tol * 8
-        if True:  # the CPU backend's literal gradients at every shape
-            lit_dx = ctx.conv2d_dgrad(dg_, dw_, x.shape, (s, s), (p, p), 1).numpy()
-            lit_dw = ctx.conv2d_wgrad(dx_, dg_, w.shape, (s, s), (p, p), 1).numpy()
-            assert rel_err(lit_dx, orc.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), 1)) <= tol * 8, ("literal dgrad", case)
-            assert rel_err(lit_dw, orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 1)) <= tol * 8, ("literal wgrad", case)
+        # the GPU result and the CPU oracle's (restated reference algorithm) on the same inputs, each within the stated
+        # tolerance of the float64 truth
+        parity.check("conv fwd", y, ty.detach().numpy(), oracle=orc.conv2d_fwd(x, w, (s, s), (p, p)), case=case, terms=ay)
+        parity.check("conv dgrad", dxg, tx.grad.numpy(), oracle=orc.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), 0), case=case)
+        parity.check("conv wgrad", dwg, tw.grad.numpy(), oracle=orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 0), case=case)
+        # the CPU backend's literal gradients at every shape: truth = the oracle's literal arithmetic carried out in float64
+        # (for f64 results the f64 oracle itself: two f64 summation orders differ by ~1e-15, far inside 1e-12)
+        lit_dx = ctx.conv2d_dgrad(dg_, dw_, x.shape, (s, s), (p, p), 1).numpy()
+        lit_dw = ctx.conv2d_wgrad(dx_, dg_, w.shape, (s, s), (p, p), 1).numpy()
+        x64, w64, g64 = x.astype(np.float64), w.astype(np.float64), g.astype(np.float64)
+        parity.check("conv dgrad literal", lit_dx, orc.conv2d_dgrad(g64, w64, x.shape, (s, s), (p, p), 1),
+                     oracle=orc.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), 1), case=case)
+        parity.check("conv wgrad literal", lit_dw, orc.conv2d_wgrad(x64, g64, w.shape, (s, s), (p, p), 1),
+                     oracle=orc.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 1), case=case)
 
 
 # 3x3 weight gradients around the LDS-patch kernel (taken when Cin % 32 == 0, Cout > 32, W % 4 == 0, W <= 64, even
@@ -568,7 +564,6 @@ def test_conv2d_wgrad_patch_kernel_shapes(ctx, orc):
     from ferrox_amd import capi
     import torch.nn.functional as F
     rng = np.random.default_rng(57)
-    tol = TOL[np.dtype(np.float32)]
     for (B, Cin, H, W, Cout, st, pd) in WGRAD_PATCH_CASES:
         x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(np.float32)
         oh, ow = orc.out_hw(H, W, 3, 3, st[0], st[1], pd[0], pd[1])
@@ -578,8 +573,7 @@ def test_conv2d_wgrad_patch_kernel_shapes(ctx, orc):
         tw = torch.zeros((Cout, Cin, 3, 3), dtype=torch.float64, requires_grad=True)
         F.conv2d(torch.from_numpy(x).double(), tw, stride=st, padding=pd).backward(torch.from_numpy(g).double())
         case = (B, Cin, H, W, Cout, st, pd)
-        assert rel_err(dw, tw.grad.numpy()) <= tol * 8, case
-        assert rel_err(dw, orc.conv2d_wgrad(x, g, (Cout, Cin, 3, 3), st, pd, 0)) <= tol * 8, case
+        parity.check("wgrad patch kernels", dw, tw.grad.numpy(), oracle=orc.conv2d_wgrad(x, g, (Cout, Cin, 3, 3), st, pd, 0), case=case)
         # same bits on a second run and with a caller-provided workspace of exactly the advertised size
         assert np.array_equal(dw, ctx.conv2d_wgrad(dx_, dg_, (Cout, Cin, 3, 3), st, pd, 0).numpy()), case
         need = capi.lib.fx_conv2d_workspace_bytes(capi.CONV_WGRAD, capi.FX_F32, 0, B, Cin, H, W, Cout, 3, 3, st[0], st[1], pd[0], pd[1])
@@ -636,7 +630,6 @@ def test_conv2d_patch_kernel_shapes(ctx, orc):
     import torch.nn.functional as F
     from ferrox_amd import capi
     rng = np.random.default_rng(58)
-    tol = TOL[np.dtype(np.float32)]
     for (B, Cin, H, W, Cout, st, pd) in CONV_PATCH_CASES:
         case = (B, Cin, H, W, Cout, st, pd)
         x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(np.float32)
@@ -651,10 +644,8 @@ def test_conv2d_patch_kernel_shapes(ctx, orc):
         ty = F.conv2d(tx, tw, stride=st, padding=pd)
         ty.backward(torch.from_numpy(g).double())
         ay = F.conv2d(tx.detach().abs(), tw.abs(), stride=st, padding=pd).max().item()
-        assert np.abs(y - ty.detach().numpy()).max() <= tol * ay, ("fwd", case)
-        assert rel_err(dxg, tx.grad.numpy()) <= tol * 8, ("dgrad", case)
-        assert rel_err(y, orc.conv2d_fwd(x, w, st, pd)) <= tol * 8, ("fwd vs oracle", case)
-        assert rel_err(dxg, orc.conv2d_dgrad(g, w, x.shape, st, pd, 0)) <= tol * 8, ("dgrad vs oracle", case)
+        parity.check("patch kernels fwd", y, ty.detach().numpy(), oracle=orc.conv2d_fwd(x, w, st, pd), case=case, terms=ay)
+        parity.check("patch kernels dgrad", dxg, tx.grad.numpy(), oracle=orc.conv2d_dgrad(g, w, x.shape, st, pd, 0), case=case)
         dims = (B, Cin, H, W, Cout, 3, 3, st[0], st[1], pd[0], pd[1])
         # bias + ReLU in the store of the kernel = the forward pass followed by fx_bias_act, bit for bit
         db_ = ctx.upload(rng.standard_normal(Cout).astype(np.float32))
@@ -695,7 +686,6 @@ def test_conv2d_f64_patch_kernel_shapes(ctx, orc):
     import torch.nn.functional as F
     from ferrox_amd import capi
     rng = np.random.default_rng(61)
-    tol = TOL[np.dtype(np.float64)]
     for (B, Cin, H, W, Cout, st, pd) in CONV_F64_PATCH_CASES:
         case = (B, Cin, H, W, Cout, st, pd)
         x = rng.uniform(-1, 1, (B, Cin, H, W))
@@ -711,10 +701,8 @@ def test_conv2d_f64_patch_kernel_shapes(ctx, orc):
         ty = F.conv2d(tx, tw, stride=st, padding=pd)
         ty.backward(torch.from_numpy(g))
         ay = F.conv2d(tx.detach().abs(), tw.abs(), stride=st, padding=pd).max().item()
-        assert np.abs(y - ty.detach().numpy()).max() <= tol * ay, ("fwd", case)
-        assert rel_err(dxg, tx.grad.numpy()) <= tol * 8, ("dgrad", case)
-        assert rel_err(y, orc.conv2d_fwd(x, w, st, pd)) <= tol * 8, ("fwd vs oracle", case)
-        assert rel_err(dxg, orc.conv2d_dgrad(g, w, x.shape, st, pd, 0)) <= tol * 8, ("dgrad vs oracle", case)
+        parity.check("patch kernels fwd", y, ty.detach().numpy(), oracle=orc.conv2d_fwd(x, w, st, pd), case=case, terms=ay)
+        parity.check("patch kernels dgrad", dxg, tx.grad.numpy(), oracle=orc.conv2d_dgrad(g, w, x.shape, st, pd, 0), case=case)
         # bias + ReLU in the store of the kernel = the forward pass followed by fx_bias_act, bit for bit
         dims = (B, Cin, H, W, Cout, 3, 3, st[0], st[1], pd[0], pd[1])
         fused = ctx.empty(y.shape, np.float64)
@@ -753,7 +741,6 @@ def test_conv2d_f64_wgrad_patch_kernel_shapes(ctx, orc):
     import torch.nn.functional as F
     from ferrox_amd import capi
     rng = np.random.default_rng(62)
-    tol = TOL[np.dtype(np.float64)]
     for (B, Cin, H, W, Cout, sh, pd) in CONV_F64_WGRAD_CASES:
         case = (B, Cin, H, W, Cout, sh, pd)
         st = sh if isinstance(sh, tuple) else (sh, 1)
@@ -764,9 +751,8 @@ def test_conv2d_f64_wgrad_patch_kernel_shapes(ctx, orc):
         dwg = ctx.conv2d_wgrad(dx_, dg_, (Cout, Cin, 3, 3), st, pd, 0).numpy()
         tw = torch.zeros((Cout, Cin, 3, 3), dtype=torch.float64, requires_grad=True)
         F.conv2d(torch.from_numpy(x), tw, stride=st, padding=pd).backward(torch.from_numpy(g))
-        assert rel_err(dwg, tw.grad.numpy()) <= tol * 8, ("wgrad", case)
-        if B * Cout * oh * ow <= 1 << 20:
-            assert rel_err(dwg, orc.conv2d_wgrad(x, g, (Cout, Cin, 3, 3), st, pd, 0)) <= tol * 8, ("wgrad vs oracle", case)
+        orc_dw = orc.conv2d_wgrad(x, g, (Cout, Cin, 3, 3), st, pd, 0) if B * Cout * oh * ow <= 1 << 20 else None
+        parity.check("wgrad patch kernels f64", dwg, tw.grad.numpy(), oracle=orc_dw, case=case)
         # a caller-provided workspace of exactly the advertised size gives the same bits
         dims = (B, Cin, H, W, Cout, 3, 3, st[0], st[1], pd[0], pd[1])
         need = capi.lib.fx_conv2d_workspace_bytes(capi.CONV_WGRAD, capi.FX_F64, 0, *dims)
@@ -793,7 +779,6 @@ def test_conv2d_image_layer_kernels(ctx, orc):
     import torch.nn.functional as F
     from ferrox_amd import capi
     rng = np.random.default_rng(59)
-    tol = TOL[np.dtype(np.float32)]
     for (B, Cin, H, W, Cout, st, pd) in SMALLC_CASES:
         case = (B, Cin, H, W, Cout, st, pd)
         x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(np.float32)
@@ -809,10 +794,8 @@ def test_conv2d_image_layer_kernels(ctx, orc):
         ty = F.conv2d(tx, tw, stride=st, padding=pd)
         ty.backward(torch.from_numpy(g).double())
         ay = F.conv2d(tx.abs(), tw.detach().abs(), stride=st, padding=pd).max().item()
-        assert np.abs(y - ty.detach().numpy()).max() <= tol * ay, ("fwd", case)
-        assert rel_err(gw, tw.grad.numpy()) <= tol * 8, ("wgrad", case)
-        assert rel_err(y, orc.conv2d_fwd(x, w, st, pd)) <= tol * 8, ("fwd vs oracle", case)
-        assert rel_err(gw, orc.conv2d_wgrad(x, g, w.shape, st, pd, 0)) <= tol * 8, ("wgrad vs oracle", case)
+        parity.check("image layers fwd", y, ty.detach().numpy(), oracle=orc.conv2d_fwd(x, w, st, pd), case=case, terms=ay)
+        parity.check("image layers wgrad", gw, tw.grad.numpy(), oracle=orc.conv2d_wgrad(x, g, w.shape, st, pd, 0), case=case)
         # same bits on a second run; bias + ReLU in the store equals the separate pass
         assert np.array_equal(ctx.conv2d_fwd(dx_, dw_, st, pd).numpy(), y), case
         assert np.array_equal(ctx.conv2d_wgrad(dx_, dg_, w.shape, st, pd, 0).numpy(), gw), case
@@ -838,7 +821,6 @@ def test_conv2d_f64_image_layer_forward(ctx, orc):
     import torch.nn.functional as F
     from ferrox_amd import capi
     rng = np.random.default_rng(63)
-    tol = TOL[np.dtype(np.float64)]
     # maps 32 wide, heights a multiple of 8, output channels a multiple of 32: the image-layer kernel of conv_image_f64.hpp (1 to 4
     # channels, one to five tiles per image, one to three blocks of output channels)
     extra = [(3, 1, 8, 32, 64, (1, 1), (1, 1)), (2, 4, 40, 32, 96, (1, 1), (1, 1)), (5, 2, 24, 32, 32, (1, 1), (1, 1)),
@@ -853,8 +835,7 @@ def test_conv2d_f64_image_layer_forward(ctx, orc):
         y = ctx.conv2d_fwd(dx_, dw_, st, pd).numpy()
         ty = F.conv2d(torch.from_numpy(x), torch.from_numpy(w), stride=st, padding=pd).numpy()
         ay = F.conv2d(torch.from_numpy(np.abs(x)), torch.from_numpy(np.abs(w)), stride=st, padding=pd).max().item()
-        assert np.abs(y - ty).max() <= tol * ay, ("fwd", case)
-        assert rel_err(y, orc.conv2d_fwd(x, w, st, pd)) <= tol * 8, ("fwd vs oracle", case)
+        parity.check("image layers fwd f64", y, ty, oracle=orc.conv2d_fwd(x, w, st, pd), case=case, terms=ay)
         assert np.array_equal(ctx.conv2d_fwd(dx_, dw_, st, pd).numpy(), y), case
         dims = (B, Cin, H, W, Cout, 3, 3, st[0], st[1], pd[0], pd[1])
         fused = ctx.empty(y.shape, np.float64)
@@ -868,8 +849,7 @@ def test_conv2d_f64_image_layer_forward(ctx, orc):
         gw = ctx.conv2d_wgrad(dx_, dg_, w.shape, st, pd, 0).numpy()
         tw = torch.from_numpy(w).requires_grad_(True)
         F.conv2d(torch.from_numpy(x), tw, stride=st, padding=pd).backward(torch.from_numpy(g))
-        assert rel_err(gw, tw.grad.numpy()) <= tol * 8, ("wgrad", case)
-        assert rel_err(gw, orc.conv2d_wgrad(x, g, w.shape, st, pd, 0)) <= tol * 8, ("wgrad vs oracle", case)
+        parity.check("image layers wgrad f64", gw, tw.grad.numpy(), oracle=orc.conv2d_wgrad(x, g, w.shape, st, pd, 0), case=case)
         assert np.array_equal(ctx.conv2d_wgrad(dx_, dg_, w.shape, st, pd, 0).numpy(), gw), case
         need = capi.lib.fx_conv2d_workspace_bytes(capi.CONV_WGRAD, capi.FX_F64, 0, *dims)
         assert need >= 0
@@ -957,7 +937,6 @@ def test_conv2d_strided_dgrad_vs_torch_and_oracle(ctx, orc, dtype):
     import torch
     import torch.nn.functional as F
     rng = np.random.default_rng(60)
-    tol = TOL[np.dtype(dtype)]
     for (B, Cin, H, W, Cout, k, st, pd) in STRIDED_DGRAD_CASES:
         case = (B, Cin, H, W, Cout, k, st, pd)
         oh, ow = orc.out_hw(H, W, k[0], k[1], st[0], st[1], pd[0], pd[1])
@@ -966,8 +945,7 @@ def test_conv2d_strided_dgrad_vs_torch_and_oracle(ctx, orc, dtype):
         dx = ctx.conv2d_dgrad(ctx.upload(g), ctx.upload(w), (B, Cin, H, W), st, pd, 0).numpy()
         tx = torch.zeros((B, Cin, H, W), dtype=torch.float64, requires_grad=True)
         F.conv2d(tx, torch.from_numpy(w).double(), stride=st, padding=pd).backward(torch.from_numpy(g).double())
-        assert rel_err(dx, tx.grad.numpy()) <= tol * 8, case
-        assert rel_err(dx, orc.conv2d_dgrad(g, w, (B, Cin, H, W), st, pd, 0)) <= tol * 8, case
+        parity.check("strided dgrad", dx, tx.grad.numpy(), oracle=orc.conv2d_dgrad(g, w, (B, Cin, H, W), st, pd, 0), case=case)
 
 
 @pytest.mark.parametrize("seed,dtype", [(61, np.float32), (62, np.float32), (63, np.float32), (64, np.float32), (65, np.float64), (66, np.float64)])
@@ -978,7 +956,6 @@ def test_conv2d_random_shapes_all_paths_vs_torch(ctx, seed, dtype):
     import torch
     import torch.nn.functional as F
     rng = np.random.default_rng(seed)
-    tol = TOL[np.dtype(dtype)] * 8
     chans = [1, 3, 4, 8, 16, 24, 32, 40, 64, 65, 72, 96, 128, 136]
     widths = [4, 6, 8, 12, 14, 16, 20, 28, 30, 32, 36, 56, 60, 64, 66, 68]
     for it in range(70):
@@ -1002,9 +979,9 @@ def test_conv2d_random_shapes_all_paths_vs_torch(ctx, seed, dtype):
         dx_, dw_, dg_ = ctx.upload(x), ctx.upload(w), ctx.upload(g)
         y = ctx.conv2d_fwd(dx_, dw_, (sh, sw), (ph, pw)).numpy()
         ay = F.conv2d(tx.detach().abs(), tw.detach().abs(), stride=(sh, sw), padding=(ph, pw)).max().item()
-        assert np.abs(y - ty.detach().numpy()).max() <= tol * max(ay, 1e-30), ("fwd", case)
-        assert rel_err(ctx.conv2d_dgrad(dg_, dw_, x.shape, (sh, sw), (ph, pw), 0).numpy(), tx.grad.numpy()) <= tol, ("dgrad", case)
-        assert rel_err(ctx.conv2d_wgrad(dx_, dg_, w.shape, (sh, sw), (ph, pw), 0).numpy(), tw.grad.numpy()) <= tol, ("wgrad", case)
+        parity.check("random shapes fwd", y, ty.detach().numpy(), case=case, terms=max(ay, 1e-30))
+        parity.check("random shapes dgrad", ctx.conv2d_dgrad(dg_, dw_, x.shape, (sh, sw), (ph, pw), 0).numpy(), tx.grad.numpy(), case=case)
+        parity.check("random shapes wgrad", ctx.conv2d_wgrad(dx_, dg_, w.shape, (sh, sw), (ph, pw), 0).numpy(), tw.grad.numpy(), case=case)
 
 
 def test_conv2d_misaligned_tensors_match_aligned(ctx):
@@ -1028,10 +1005,16 @@ def test_conv2d_misaligned_tensors_match_aligned(ctx):
     capi.check(capi.lib.fx_conv2d_fwd_f32(ctx.h, xp, dw_.ptr, y.ptr, *dims, None, 0))
     capi.check(capi.lib.fx_conv2d_dgrad_f32(ctx.h, gp, dw_.ptr, dx.ptr, *dims, 0, None, 0))
     capi.check(capi.lib.fx_conv2d_wgrad_f32(ctx.h, xp, gp, dwt.ptr, *dims, 0, None, 0))
-    tol = TOL[np.dtype(np.float32)] * 8
-    assert rel_err(y.numpy(), ctx.conv2d_fwd(dx_al, dw_, (1, 1), (1, 1)).numpy()) <= tol
-    assert rel_err(dx.numpy(), ctx.conv2d_dgrad(dg_al, dw_, x.shape, (1, 1), (1, 1), 0).numpy()) <= tol
-    assert rel_err(dwt.numpy(), ctx.conv2d_wgrad(dx_al, dg_al, w.shape, (1, 1), (1, 1), 0).numpy()) <= tol
+    import torch
+    import torch.nn.functional as F
+    tx = torch.from_numpy(x).double().requires_grad_(True)
+    tw = torch.from_numpy(w).double().requires_grad_(True)
+    ty = F.conv2d(tx, tw, stride=1, padding=1)
+    ty.backward(torch.from_numpy(g).double())
+    # the fallback kernels (misaligned) and the aligned ones, each against the float64 truth
+    parity.check("misaligned fwd", y.numpy(), ty.detach().numpy(), oracle=ctx.conv2d_fwd(dx_al, dw_, (1, 1), (1, 1)).numpy())
+    parity.check("misaligned dgrad", dx.numpy(), tx.grad.numpy(), oracle=ctx.conv2d_dgrad(dg_al, dw_, x.shape, (1, 1), (1, 1), 0).numpy())
+    parity.check("misaligned wgrad", dwt.numpy(), tw.grad.numpy(), oracle=ctx.conv2d_wgrad(dx_al, dg_al, w.shape, (1, 1), (1, 1), 0).numpy())
     del xb, gb
 
 

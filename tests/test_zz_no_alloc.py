@@ -39,6 +39,36 @@ def test_noalloc_reduce_max_two_calls_second_smaller():
         _both(ctx, small, 1)
 
 
+def test_noalloc_reduce_max_allocates_nothing_on_a_fresh_context():
+    """On a context that has never run a split reduction the library's growing scratch region does not exist yet: the
+    no-alloc call must leave it that way (its partials go to the fixed array), take nothing from the driver and nothing new
+    from the pool; the ordinary entry point on the same shape then does create the region."""
+    rng = np.random.default_rng(12)
+    a_host = rng.standard_normal((2048, 4096)).astype(np.float32)
+    with capi.Context(0) as ctx:
+        a = ctx.upload(a_host)
+        out = ctx.empty((4096,), np.float32)
+        idx = capi._RawI64(ctx, 4096)
+        ctx.sync()
+        assert ctx.scratch_info()["bytes"] == 0
+        pool_before, mem_before = ctx.pool_stats(np.float32), ctx.device_mem_info()["free"]
+        ctx.reduce_max_noalloc(a, 0, out, idx)             # 24 slices of partials: a split reduction
+        ctx.reduce_max_noalloc(a.reshape(a.size), 0, out, idx)  # one long run: 768 slices
+        ctx.sync()
+        pool_after, mem_after = ctx.pool_stats(np.float32), ctx.device_mem_info()["free"]
+        assert ctx.scratch_info()["bytes"] == 0 and ctx.scratch_info()["current"] == 0
+        assert mem_after == mem_before
+        for key in ("device_allocs", "active_allocations", "total_allocations"):
+            if key in pool_before:
+                assert pool_after[key] == pool_before[key], key
+        ctx.reduce_max_noalloc(a, 0, out, idx)
+        np.testing.assert_array_equal(out.numpy(), a_host.max(axis=0))
+        np.testing.assert_array_equal(idx.numpy(), a_host.argmax(axis=0))
+        ref, _ = ctx.reduce("max", a, 0, want_idx=True)    # the ordinary entry point grows the context's region
+        assert ctx.scratch_info()["bytes"] > 0
+        np.testing.assert_array_equal(ref.numpy(), a_host.max(axis=0))
+
+
 def test_noalloc_reduce_max_refuses_oversized_partials():
     with capi.Context(0) as ctx:
         # [32768, 512] along axis 0: two column tiles, so the axis is split into 1024 slices whose partials
