@@ -89,6 +89,7 @@ _sig("fx_d2h", _vp, _vp, _vp, _i64)
 _sig("fx_d2d", _vp, _vp, _vp, _i64)
 _sig("fx_scratch_info", _vp, C.POINTER(_vp), C.POINTER(_i64), C.POINTER(_i64), C.POINTER(_i64))
 _sig("fx_device_mem_info", _vp, C.POINTER(_i64), C.POINTER(_i64))
+_sig("fx_conv2d_bwd_relu_supported", _vp, _int, _int, *([_i64] * 11))
 _sig("fx_conv2d_workspace_bytes", _int, _int, _int, *([_i64] * 11), restype=_i64)
 
 _CONV_INTS = [_i64] * 11
@@ -132,6 +133,8 @@ for _s, _ct in (("f32", C.c_float), ("f64", C.c_double)):
     _sig(f"fx_conv2d_fwd_{_s}", _vp, _vp, _vp, _vp, *_CONV_INTS, _vp, _i64)
     _sig(f"fx_conv2d_dgrad_{_s}", _vp, _vp, _vp, _vp, *_CONV_INTS, _int, _vp, _i64)
     _sig(f"fx_conv2d_wgrad_{_s}", _vp, _vp, _vp, _vp, *_CONV_INTS, _int, _vp, _i64)
+    _sig(f"fx_conv2d_wgrad_relu_bias_{_s}", _vp, _vp, _vp, _vp, _vp, _vp, *_CONV_INTS, _vp, _i64)
+    _sig(f"fx_conv2d_dgrad_relu_{_s}", _vp, _vp, _vp, _vp, _vp, *_CONV_INTS)
     _sig(f"fx_bias_act_{_s}", _vp, _vp, _vp, _i64, _i64, _i64, _int)
     _sig(f"fx_conv2d_fwd_bias_act_{_s}", _vp, _vp, _vp, _vp, _vp, *_CONV_INTS, _int, _vp, _i64)
     _sig(f"fx_gemm_bias_act_{_s}", _vp, _int, _int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _int)
@@ -637,6 +640,27 @@ class Context:
 
     def sgd_step(self, p, g, lr):
         check(self._fn("sgd_step", p.dtype)(self.h, p.ptr, g.ptr, p.size, lr))
+
+    def conv2d_bwd_relu_supported(self, kind, dtype, x_shape, w_shape, stride, padding):
+        B, Cin, H, W = x_shape
+        Cout, _, kh, kw = w_shape
+        return bool(lib.fx_conv2d_bwd_relu_supported(self.h, kind, dtype_code(dtype)[0], B, Cin, H, W, Cout, kh, kw, *stride, *padding))
+
+    def conv2d_wgrad_relu_bias(self, x, g, act, w_shape, stride, padding):
+        """(dw, db) of a conv + ReLU layer from the unmasked upstream gradient g and the layer's activation."""
+        B, Cin, H, W = x.shape
+        Cout, _, kh, kw = w_shape
+        dw, db = self.empty(w_shape, x.dtype), self.empty((Cout,), x.dtype)
+        check(self._fn("conv2d_wgrad_relu_bias", x.dtype)(self.h, x.ptr, g.ptr, act.ptr, dw.ptr, db.ptr, B, Cin, H, W, Cout, kh, kw,
+                                                          *stride, *padding, None, 0))
+        return dw, db
+
+    def conv2d_dgrad_relu(self, g, act, w, x_shape, stride, padding):
+        B, Cin, H, W = x_shape
+        Cout, _, kh, kw = w.shape
+        dx = self.empty(x_shape, g.dtype)
+        check(self._fn("conv2d_dgrad_relu", g.dtype)(self.h, g.ptr, act.ptr, w.ptr, dx.ptr, B, Cin, H, W, Cout, kh, kw, *stride, *padding))
+        return dx
 
     def conv2d_wgrad(self, x, g, w_shape, stride, padding, mode=0, out=None):
         B, Cin, H, W = x.shape

@@ -596,12 +596,12 @@ i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     i64 generic = splits > 1 ? (i64)splits * d.Cout * d.Cin * d.kh * d.kw * (i64)sizeof(T) : 0;
     if (mode == 0) {
         const csc::Plan sp = smallc_plan<T>(c, d, true);
-        if (sp.ok) generic = std::max(generic, csc::wgrad_workspace_bytes(sp, d.Cout, d.Cin));
+        if (sp.ok) generic = std::max(generic, csc::wgrad_workspace_bytes(sp, d.Cout, d.Cin, true));  // covers the masked variant too
     }
     const wgd::Plan pd = patch64_plan<T>(c, d, mode);
     if (pd.ok) generic = std::max(generic, wgd::workspace_bytes(pd, d.Cout, d.Cin));
     const wg2::Plan p2 = patch_s2_plan<T>(c, d, mode);
-    if (p2.ok) generic = std::max(generic, wg2::workspace_bytes(p2, d.Cout, d.Cin));
+    if (p2.ok) generic = std::max(generic, wg2::workspace_bytes(p2, d.Cout, d.Cin, true));
     const wgd2::Plan q2 = patch64_s2_plan<T>(c, d, mode);
     if (q2.ok) generic = std::max(generic, wgd2::workspace_bytes(q2, d.Cout, d.Cin));
     if constexpr (sizeof(T) == 8) {
@@ -700,7 +700,87 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
     return wgrad_tile<T, TileSmall>(c, x, g, dw, d, mode, ws);
 }
 
+// ---- backward of conv + ReLU from the UNMASKED upstream gradient --------------------------------------------------------
+// The layer's ReLU gradient g * (act > 0) is applied while the consumer kernels stage g, and the weight-gradient kernel
+// also leaves the bias gradient (the sums of the masked g per output channel): no masked copy of g is written or re-read
+// and the separate mask + bias pass (fx_relu_bwd_bias_grad) disappears.  Kernels: the image-layer weight gradient
+// (conv_smallc.hpp) and the stride-2 pair (wgrad_patch_s2.hpp, dgrad_patch_s2.hpp), f32.
+template <typename T>
+bool bwd_relu_supported(int num_cus, int kind, const Dims& d) {
+    if constexpr (sizeof(T) == 4) {
+        if (generic_only() || d.B > d.bc) return false;
+        if (kind == FX_CONV_WGRAD) {
+            if (csc::make_plan(num_cus, true, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow).ok) return true;
+            return wg2::make_plan(num_cus, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow).ok;
+        }
+        if (kind == FX_CONV_DGRAD)
+            return !dgrad_small_cin_ok<T>(d) && dg2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow).ok;
+    }
+    return false;
+}
+
+template <typename T>
+int conv_wgrad_relu_bias(fx_ctx* c, const T* x, const T* g, const T* act, T* dw, T* db, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh,
+                         i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, void* ws, i64 ws_bytes) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(x && g && act && dw && db, "fx_conv2d_wgrad_relu_bias: null pointer");
+    Dims d;
+    if (int rc = check_dims<T>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_wgrad_relu_bias")) return rc;
+    if constexpr (sizeof(T) == 4) {
+        if (bwd_relu_supported<T>(c->num_cus, FX_CONV_WGRAD, d) && aligned16(x, g) && aligned16(act, ws)) {
+            const i64 need = wgrad_ws_bytes<T>(c, d, 0);
+            FX_REQUIRE(ws == nullptr || ws_bytes >= need, "fx_conv2d_wgrad_relu_bias: workspace of %lld bytes is smaller than the %lld needed",
+                       (long long)ws_bytes, (long long)need);
+            std::lock_guard<std::mutex> lk(c->launch_mutex);
+            const csc::Plan sp = smallc_plan<T>(c, d, true);
+            if (sp.ok) {
+                float* part = nullptr;
+                if (sp.splits > 1) {
+                    part = (float*)(ws ? ws : c->get_scratch(need));
+                    if (!part) return FX_ERR_OOM;
+                }
+                return csc::run_wgrad(c, sp, x, g, dw, part, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw, act, db);
+            }
+            const wg2::Plan p2 = patch_s2_plan<T>(c, d, 0);
+            if (p2.ok) {
+                float* part = (float*)(ws ? ws : c->get_scratch(need));
+                if (!part) return FX_ERR_OOM;
+                return wg2::run(c, p2, x, g, dw, part, Cin, H, Cout, ph, d.oh, act, db);
+            }
+        }
+    }
+    fx::set_error("fx_conv2d_wgrad_relu_bias: no fused kernel for this shape, dtype or alignment (ask fx_conv2d_bwd_relu_supported; use "
+                  "fx_relu_bwd_bias_grad + fx_conv2d_wgrad)");
+    return FX_ERR_UNSUPPORTED;
+}
+
+template <typename T>
+int conv_dgrad_relu(fx_ctx* c, const T* g, const T* act, const T* w, T* dx, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh,
+                    i64 sw, i64 ph, i64 pw) {
+    FX_CHECK_CTX(c);
+    FX_REQUIRE(g && act && w && dx, "fx_conv2d_dgrad_relu: null pointer");
+    Dims d;
+    if (int rc = check_dims<T>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_dgrad_relu")) return rc;
+    if constexpr (sizeof(T) == 4) {
+        if (bwd_relu_supported<T>(c->num_cus, FX_CONV_DGRAD, d) && aligned16(g, w) && aligned16(dx, act)) {
+            std::lock_guard<std::mutex> lk(c->launch_mutex);
+            const dg2::Plan p2 = dg2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
+            return dg2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh, act);
+        }
+    }
+    fx::set_error("fx_conv2d_dgrad_relu: no fused kernel for this shape, dtype or alignment (ask fx_conv2d_bwd_relu_supported; use "
+                  "fx_relu_bwd + fx_conv2d_dgrad)");
+    return FX_ERR_UNSUPPORTED;
+}
+
 }  // namespace
+
+extern "C" int fx_conv2d_bwd_relu_supported(fx_ctx* c, int kind, int dtype, int64_t B, int64_t Cin, int64_t H, int64_t W, int64_t Cout,
+                                            int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw) {
+    Dims d;
+    if (dtype != FX_F32 || check_dims<float>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_bwd_relu_supported")) return 0;
+    return bwd_relu_supported<float>(c ? c->num_cus : 256, kind, d) ? 1 : 0;
+}
 
 extern "C" int64_t fx_conv2d_workspace_bytes(int kind, int dtype, int mode, int64_t B, int64_t Cin, int64_t H, int64_t W,
                                              int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw) {
@@ -793,6 +873,16 @@ extern "C" int fx_conv2d_tune_f32(fx_ctx* c, int kind, int64_t B, int64_t Cin, i
                                        int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,   \
                                        int mode, void* ws, int64_t ws_bytes) {                                         \
         return conv_wgrad<T>(c, x, g, dw, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, mode, ws, ws_bytes);             \
+    }                                                                                                                  \
+    extern "C" int fx_conv2d_wgrad_relu_bias_##S(fx_ctx* c, const T* x, const T* g, const T* act, T* dw, T* db, int64_t B,   \
+                                                 int64_t Cin, int64_t H, int64_t W, int64_t Cout, int64_t kh, int64_t kw,  \
+                                                 int64_t sh, int64_t sw, int64_t ph, int64_t pw, void* ws, int64_t ws_bytes) { \
+        return conv_wgrad_relu_bias<T>(c, x, g, act, dw, db, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, ws, ws_bytes); \
+    }                                                                                                                  \
+    extern "C" int fx_conv2d_dgrad_relu_##S(fx_ctx* c, const T* g, const T* act, const T* w, T* dx, int64_t B, int64_t Cin,   \
+                                            int64_t H, int64_t W, int64_t Cout, int64_t kh, int64_t kw, int64_t sh,   \
+                                            int64_t sw, int64_t ph, int64_t pw) {                                      \
+        return conv_dgrad_relu<T>(c, g, act, w, dx, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw);                       \
     }
 
 FX_DEFINE_CONV(float, f32)

@@ -44,9 +44,11 @@ struct FwdParams {
 struct WgradParams {
     const float* x;
     const float* g;
+    const float* act;    // MASK: the layer's ReLU output; g is used as g * (act > 0)
     float* part;
+    float* bpart;        // MASK: per-split sums of the masked g over the split's pixels, [Cout] (the bias gradient)
     int stages, sps;     // B * tpi, stages per block
-    i64 part_stride;     // Cout * C * 9
+    i64 part_stride;     // floats between the partial sums of two splits (dw and bias alike)
     Geometry q;
 };
 
@@ -185,6 +187,10 @@ __global__ __launch_bounds__(NT) void fwd_kernel(const FwdParams p) {
 
 // grid = (splits, ceil(Cout / 32)); block z takes stages [z * sps, (z + 1) * sps), a stage being one tile of one image.
 // Needs C * 9 <= 32 and (OH * OW) % 4 == 0.
+// MASK: the gradient arrives unmasked from the layer above and the ReLU of this layer is applied while it is staged
+// (g * (act > 0), the bits of fx_relu_bwd); reduction column K = C * 9 <= 27 of the 32 is free, and with a B operand of 1.0
+// there the MFMA leaves sum over pixels of the masked g in it: the bias gradient, at no extra instruction.
+template <bool MASK>
 __global__ __launch_bounds__(NT, 2) void wgrad_kernel(const WgradParams p) {
     extern __shared__ __align__(16) float smem[];
     const Geometry& g = p.q;
@@ -194,6 +200,7 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(const WgradParams p) {
     const int m0 = blockIdx.y * 32, z = blockIdx.x;
     const int L = g.OH * g.OW, K = g.C * KK;
     const int toff = tap_offset(g, l32);
+    const bool ones = MASK && l32 == K;
     f32x16 acc;
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] = 0.f;
@@ -210,7 +217,13 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(const WgradParams p) {
         for (int u = 0; u < 8; ++u) {
             const int row = gr + 4 * u;
             const bool ok = col_ok && m0 + row < g.Cout;
-            const float4 v = *reinterpret_cast<const float4*>(p.g + ((i64)b * g.Cout + (ok ? m0 + row : 0)) * L + (ok ? pix0 + 4 * gq : 0));
+            const i64 goff = ((i64)b * g.Cout + (ok ? m0 + row : 0)) * L + (ok ? pix0 + 4 * gq : 0);
+            float4 v = *reinterpret_cast<const float4*>(p.g + goff);
+            if constexpr (MASK) {
+                const float4 a = *reinterpret_cast<const float4*>(p.act + goff);
+                v.x = v.x * (a.x > 0.f ? 1.f : 0.f); v.y = v.y * (a.y > 0.f ? 1.f : 0.f);
+                v.z = v.z * (a.z > 0.f ? 1.f : 0.f); v.w = v.w * (a.w > 0.f ? 1.f : 0.f);
+            }
             float* d = Gs + row * GP + 4 * gq;
             d[0] = ok ? v.x : 0.f; d[1] = ok ? v.y : 0.f; d[2] = ok ? v.z : 0.f; d[3] = ok ? v.w : 0.f;
         }
@@ -222,7 +235,8 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(const WgradParams p) {
         for (int st = 0; st < 32; ++st) {
             const int pc = min(pw0 + 2 * st, L - 1);  // past the end g is zero; the patch read only has to be in range
             const int oy = (int)g.div_ow.div((uint32_t)pc), ox = pc - oy * g.OW;
-            const float bv = patch[(oy - py0) * g.sh * g.PW + ox * g.sw + toff];
+            float bv = patch[(oy - py0) * g.sh * g.PW + ox * g.sw + toff];
+            if (MASK && ones) bv = 1.f;
             acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ga[2 * st], bv, acc, 0, 0, 0);
         }
     }
@@ -238,6 +252,7 @@ __global__ __launch_bounds__(NT, 2) void wgrad_kernel(const WgradParams p) {
         const float v = ((red[i] + red[1024 + i]) + red[2048 + i]) + red[3072 + i];
         const int m = m0 + igemm::Mfma<float>::row(e, ln), n = ln & 31;
         if (m < g.Cout && n < K) out[(i64)m * K + n] = v;
+        if (MASK && m < g.Cout && n == K) p.bpart[(i64)z * p.part_stride + m] = v;
     }
 }
 
@@ -279,7 +294,10 @@ inline Plan make_plan(int num_cus, bool wgrad, i64 B, i64 C, i64 H, i64 W, i64 C
     return pl;
 }
 
-inline i64 wgrad_workspace_bytes(const Plan& pl, i64 Cout, i64 C) { return pl.splits > 1 ? (i64)pl.splits * Cout * C * KK * (i64)sizeof(float) : 0; }
+// the masked variant keeps [Cout] bias sums behind every split's [Cout][C*9] partial
+inline i64 wgrad_workspace_bytes(const Plan& pl, i64 Cout, i64 C, bool with_bias = false) {
+    return pl.splits > 1 ? (i64)pl.splits * (Cout * C * KK + (with_bias ? Cout : 0)) * (i64)sizeof(float) : 0;
+}
 
 inline Geometry make_geometry(const Plan& pl, i64 C, i64 H, i64 W, i64 Cout, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw) {
     Geometry g;
@@ -322,16 +340,24 @@ inline int run_fwd(fx_ctx* c, const Plan& pl, const float* x, const float* w, fl
 }
 
 // x, g and part 16-byte aligned.  part holds splits x [Cout][C*9] partial sums (unused when splits == 1).
+// act / db non-null: the masked variant (g * (act > 0) staged, db = its sums per output channel), act 16-byte aligned too.
 inline int run_wgrad(fx_ctx* c, const Plan& pl, const float* x, const float* g, float* dw, float* part, i64 C, i64 H, i64 W, i64 Cout,
-                     i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw) {
+                     i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw, const float* act = nullptr, float* db = nullptr) {
     WgradParams p;
-    p.x = x; p.g = g; p.part = pl.splits > 1 ? part : dw;
-    p.stages = pl.stages; p.sps = pl.sps; p.part_stride = Cout * C * KK;
+    const i64 n = Cout * C * KK;
+    p.x = x; p.g = g; p.act = act;
+    p.part = pl.splits > 1 ? part : dw;
+    p.bpart = pl.splits > 1 ? part + n : db;
+    p.stages = pl.stages; p.sps = pl.sps; p.part_stride = n + (act ? Cout : 0);
     p.q = make_geometry(pl, C, H, W, Cout, OH, OW, sh, sw, ph, pw);
     const dim3 grid((unsigned)pl.splits, (unsigned)fx::ceil_div(Cout, (i64)32));
-    wgrad_kernel<<<grid, dim3(NT), pl.smem, c->stream>>>(p);
+    if (act) wgrad_kernel<true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);
+    else wgrad_kernel<false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);
     FX_LAUNCH_CHECK();
-    if (pl.splits > 1) return igemm::launch_splitk_reduce<float>(c, part, dw, p.part_stride, pl.splits);
+    if (pl.splits > 1) {
+        if (act) return igemm::launch_splitk_reduce_pair<float>(c, part, p.part_stride, pl.splits, dw, n, db, Cout);
+        return igemm::launch_splitk_reduce<float>(c, part, dw, n, pl.splits);
+    }
     return FX_OK;
 }
 

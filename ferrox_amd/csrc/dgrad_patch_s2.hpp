@@ -31,6 +31,7 @@ constexpr size_t LDS_LIMIT = 160 * 1024;
 
 struct Params {
     const float* g;
+    const float* act;  // MASK: the ReLU output of the layer whose gradient g is; g is staged as g * (act > 0)
     const float* w;
     float* dx;
     int Cin, Cout, oh, tpi, nct;  // tiles per image, channel tiles
@@ -51,7 +52,8 @@ struct Shape {
     static_assert(CELLS % OW == 0 && OW % 4 == 0 && OCC % 8 == 0 && OCC * (CELLS / 4) % NT == 0 && X4 <= NT && LDS <= LDS_LIMIT, "shape");
 };
 
-template <int OW, int OCC>
+// MASK: grad_out arrives unmasked and the layer's ReLU is applied to the staged patch (g * (act > 0), the bits of fx_relu_bwd).
+template <int OW, int OCC, bool MASK>
 __global__ __launch_bounds__(NT, 1) void dgrad_s2_kernel(const Params p) {
     using S = Shape<OW, OCC>;
     constexpr int TR = S::TR, PC = S::PC, GPL = S::GPL, KS = S::KS, WCH = S::WCH, BUF = S::BUF;
@@ -66,9 +68,15 @@ __global__ __launch_bounds__(NT, 1) void dgrad_s2_kernel(const Params p) {
 
     // staging maps (constant over the chunks)
     const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    float4 wv[S::NWP], gv[S::NGP], xv;
+    float4 wv[S::NWP], gv[S::NGP], xv, av[MASK ? S::NGP : 1], axv;
     const float* wsrc = p.w + (i64)c0 * KK;
     const float* gsrc = p.g + ((i64)b * p.Cout * p.oh + i0) * OW;
+    const float* asrc = MASK ? p.act + ((i64)b * p.Cout * p.oh + i0) * OW : nullptr;
+    auto masked = [](float4 v, const float4& a) __attribute__((always_inline)) {
+        v.x = v.x * (a.x > 0.f ? 1.f : 0.f); v.y = v.y * (a.y > 0.f ? 1.f : 0.f);
+        v.z = v.z * (a.z > 0.f ? 1.f : 0.f); v.w = v.w * (a.w > 0.f ? 1.f : 0.f);
+        return v;
+    };
     const int gq = tid & 63, goc = tid >> 6;                    // float4 of the tile's TR * OW floats, oc within a pass of 8
     const int g_dst = goc * GPL + (gq / (OW / 4)) * PC + (gq % (OW / 4)) * 4;
     const uint32_t g_off = (uint32_t)(goc * L + 4 * gq) * 4u;
@@ -88,6 +96,12 @@ __global__ __launch_bounds__(NT, 1) void dgrad_s2_kernel(const Params p) {
         for (int u = 0; u < S::NGP; ++u) gv[u] = ldg4(gsrc + (i64)(oc0 + 8 * u) * L, g_off);
         if (next_row) xv = ldg4(gsrc + (i64)oc0 * L, x_off);
         else xv = zero4;
+        if constexpr (MASK) {
+#pragma unroll
+            for (int u = 0; u < S::NGP; ++u) av[u] = ldg4(asrc + (i64)(oc0 + 8 * u) * L, g_off);
+            if (next_row) axv = ldg4(asrc + (i64)oc0 * L, x_off);
+            else axv = zero4;
+        }
     };
     auto park = [&](int buf) __attribute__((always_inline)) {
         float* Ws = smem + buf * BUF;
@@ -108,10 +122,12 @@ __global__ __launch_bounds__(NT, 1) void dgrad_s2_kernel(const Params p) {
 #pragma unroll
         for (int u = 0; u < S::NGP; ++u) {
             float* d = Gs + g_dst + 8 * u * GPL;
+            if constexpr (MASK) gv[u] = masked(gv[u], av[u]);
             d[0] = gv[u].x; d[1] = gv[u].y; d[2] = gv[u].z; d[3] = gv[u].w;
         }
         if (x_lane) {
             float* d = Gs + xoc * GPL + TR * PC + 4 * xq;
+            if constexpr (MASK) xv = masked(xv, axv);
             d[0] = xv.x; d[1] = xv.y; d[2] = xv.z; d[3] = xv.w;
         }
     };
@@ -215,9 +231,11 @@ inline Plan make_plan(i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i6
 }
 
 // g, w and dx must be 16-byte aligned (dx for its 8-byte pairs).
-inline int run(fx_ctx* c, const Plan& pl, const float* g, const float* w, float* dx, i64 B, i64 Cin, i64 Cout, i64 oh) {
+// act non-null: the masked variant (act 16-byte aligned as well).
+inline int run(fx_ctx* c, const Plan& pl, const float* g, const float* w, float* dx, i64 B, i64 Cin, i64 Cout, i64 oh,
+               const float* act = nullptr) {
     Params p;
-    p.g = g; p.w = w; p.dx = dx;
+    p.g = g; p.w = w; p.dx = dx; p.act = act;
     p.Cin = (int)Cin; p.Cout = (int)Cout; p.oh = (int)oh;
     p.tpi = (int)(oh / (CELLS / pl.OW));
     p.nct = (int)(Cin / CT);
@@ -227,10 +245,14 @@ inline int run(fx_ctx* c, const Plan& pl, const float* g, const float* w, float*
     bool launched = false;
 #define FX_DG2_LAUNCH(O, C_)                                                                                           \
     if (!launched && pl.OW == O && pl.OCC == C_) {                                                                     \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)dgrad_s2_kernel<O, C_>,                        \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)dgrad_s2_kernel<O, C_, false>,                 \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
+        static const hipError_t attr_m = hipFuncSetAttribute((const void*)dgrad_s2_kernel<O, C_, true>,                \
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
         FX_HIP_CHECK(attr);                                                                                            \
-        dgrad_s2_kernel<O, C_><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                                             \
+        FX_HIP_CHECK(attr_m);                                                                                          \
+        if (act) dgrad_s2_kernel<O, C_, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                              \
+        else dgrad_s2_kernel<O, C_, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                                 \
         launched = true;                                                                                               \
     }
     FX_DG2_SHAPES(FX_DG2_LAUNCH)

@@ -696,6 +696,58 @@ int launch_splitk_reduce(fx_ctx* c, const T* part, T* out, i64 n, int splits, co
     return FX_OK;
 }
 
+// Partial sums that carry a second, short result behind the first ([n1] then [n2] floats per split, `stride` apart): both are
+// added over the splits and go to their own tensors.  G threads share an output (thread g adds partials g, g + G, ... in order,
+// then the G sums are added in order of g; G = 1: one chain): the orders of splitk_reduce_kernel / splitk_reduce_grouped_kernel,
+// chosen by the same rule, so the first result has the bits launch_splitk_reduce gives it.
+template <typename T, int G>
+__global__ __launch_bounds__(256) void splitk_reduce_pair_kernel(const T* __restrict__ part, i64 stride, int splits, T* __restrict__ out1,
+                                                                 i64 n1, T* __restrict__ out2, i64 n2) {
+    constexpr int COLS = 256 / G;
+    __shared__ T sm[G][COLS];
+    const int col = threadIdx.x % COLS, g = threadIdx.x / COLS;
+    const i64 i = (i64)blockIdx.x * COLS + col;
+    T s = T(0);
+    if (i < n1 + n2) {
+        int z = g;
+        for (; z + 7 * G < splits; z += 8 * G) {
+            T v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = part[(i64)(z + u * G) * stride + i];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s = s + v[u];
+        }
+        for (; z < splits; z += G) s = s + part[(i64)z * stride + i];
+    }
+    if (G > 1) {
+        sm[g][col] = s;
+        __syncthreads();
+    }
+    if (g == 0 && i < n1 + n2) {
+        T t = s;
+        if (G > 1) {
+            t = sm[0][col];
+#pragma unroll
+            for (int u = 1; u < G; ++u) t = t + sm[u][col];
+        }
+        if (i < n1) out1[i] = t;
+        else out2[i - n1] = t;
+    }
+}
+template <typename T>
+int launch_splitk_reduce_pair(fx_ctx* c, const T* part, i64 stride, int splits, T* out1, i64 n1, T* out2, i64 n2) {
+    const i64 n = n1 + n2;
+    FX_REQUIRE(stride >= n && n <= 0x7fffffffll, "split-K pair sum: bad sizes");
+    if (splits >= 128 && n1 <= (1 << 16))
+        splitk_reduce_pair_kernel<T, 16><<<dim3((unsigned)fx::ceil_div(n, (i64)16)), dim3(256), 0, c->stream>>>(part, stride, splits, out1, n1, out2, n2);
+    else if (splits >= 32 && n1 <= (1 << 18))
+        splitk_reduce_pair_kernel<T, 4><<<dim3((unsigned)fx::ceil_div(n, (i64)64)), dim3(256), 0, c->stream>>>(part, stride, splits, out1, n1, out2, n2);
+    else
+        splitk_reduce_pair_kernel<T, 1><<<dim3((unsigned)fx::ceil_div(n, (i64)256)), dim3(256), 0, c->stream>>>(part, stride, splits, out1, n1, out2, n2);
+    FX_LAUNCH_CHECK();
+    return FX_OK;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void zero_kernel(T* __restrict__ out, i64 n) {
     const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;

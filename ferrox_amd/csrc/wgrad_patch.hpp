@@ -315,9 +315,41 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
         }
 }
 
+// A second, short result behind every partial (the bias sums of the masked kernels: nb floats at offset n of each split,
+// splits `stride` floats apart; stride 0 = the partials are n apart and there is no tail).  The blocks past the main ones
+// of a reduce launch add it over the splits, G threads per output like the main sum.
+struct ReduceTail {
+    i64 stride = 0;
+    float* db = nullptr;
+    int nb = 0;
+};
+inline i64 tail_blocks(const ReduceTail& t, int outputs_per_block) { return t.db ? fx::ceil_div((i64)t.nb, (i64)outputs_per_block) : 0; }
+template <int G>
+__device__ __forceinline__ void reduce_tail(const float* __restrict__ part, int n, int splits, const ReduceTail& t, int block) {
+    constexpr int COLS = 256 / G;
+    __shared__ float smt[G][COLS];
+    const int col = threadIdx.x % COLS, g = threadIdx.x / COLS;
+    const int i = block * COLS + col;
+    float s = 0.f;
+    if (i < t.nb)
+        for (int z = g; z < splits; z += G) s = s + part[(i64)z * t.stride + n + i];
+    smt[g][col] = s;
+    __syncthreads();
+    if (g == 0 && i < t.nb) {
+        float v = smt[0][col];
+#pragma unroll
+        for (int u = 1; u < G; ++u) v = v + smt[u][col];
+        t.db[i] = v;
+    }
+}
+
 // out[(oc*Cin + c)*KK + t] = sum_z part[z][oc][t][c], splits added in order.
 __global__ __launch_bounds__(256) void wgrad_patch_reduce_kernel(const float* __restrict__ part, float* __restrict__ out, int n,
-                                                                 int splits, int Cin, FastDiv div_row, FastDiv div_cin) {
+                                                                 int splits, int Cin, FastDiv div_row, FastDiv div_cin,
+                                                                 const ReduceTail tail = ReduceTail()) {
+    const int main_blocks = (n + 255) / 256;
+    if ((int)blockIdx.x >= main_blocks) { reduce_tail<1>(part, n, splits, tail, blockIdx.x - main_blocks); return; }
+    const i64 ps = tail.stride ? tail.stride : n;
     const int j = blockIdx.x * 256 + threadIdx.x;
     if (j >= n) return;
     float s = 0.f;
@@ -325,11 +357,11 @@ __global__ __launch_bounds__(256) void wgrad_patch_reduce_kernel(const float* __
     for (; z + 8 <= splits; z += 8) {
         float v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = part[(i64)(z + u) * n + j];
+        for (int u = 0; u < 8; ++u) v[u] = part[(i64)(z + u) * ps + j];
 #pragma unroll
         for (int u = 0; u < 8; ++u) s = s + v[u];
     }
-    for (; z < splits; ++z) s = s + part[(i64)z * n + j];
+    for (; z < splits; ++z) s = s + part[(i64)z * ps + j];
     const int oc = (int)div_row.div((uint32_t)j), rem = j - oc * (KK * Cin);
     const int t = (int)div_cin.div((uint32_t)rem), c = rem - t * Cin;
     out[((i64)oc * Cin + c) * KK + t] = s;
@@ -339,8 +371,12 @@ __global__ __launch_bounds__(256) void wgrad_patch_reduce_kernel(const float* __
 // order, then the G sums are added in order of g (fixed grouping: reproducible run to run).
 template <int G>
 __global__ __launch_bounds__(256) void wgrad_patch_reduce_grouped_kernel(const float* __restrict__ part, float* __restrict__ out, int n,
-                                                                         int splits, int Cin, FastDiv div_row, FastDiv div_cin) {
+                                                                         int splits, int Cin, FastDiv div_row, FastDiv div_cin,
+                                                                         const ReduceTail tail = ReduceTail()) {
     constexpr int COLS = 256 / G;
+    const int main_blocks = (n + COLS - 1) / COLS;
+    if ((int)blockIdx.x >= main_blocks) { reduce_tail<G>(part, n, splits, tail, blockIdx.x - main_blocks); return; }
+    const i64 ps = tail.stride ? tail.stride : n;
     __shared__ float sm[G][COLS];
     const int col = threadIdx.x % COLS, g = threadIdx.x / COLS;
     const int j = blockIdx.x * COLS + col;
@@ -350,11 +386,11 @@ __global__ __launch_bounds__(256) void wgrad_patch_reduce_grouped_kernel(const f
         for (; z + 7 * G < splits; z += 8 * G) {
             float v[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = part[(i64)(z + u * G) * n + j];
+            for (int u = 0; u < 8; ++u) v[u] = part[(i64)(z + u * G) * ps + j];
 #pragma unroll
             for (int u = 0; u < 8; ++u) s = s + v[u];
         }
-        for (; z < splits; z += G) s = s + part[(i64)z * n + j];
+        for (; z < splits; z += G) s = s + part[(i64)z * ps + j];
     }
     sm[g][col] = s;
     __syncthreads();
@@ -372,8 +408,12 @@ __global__ __launch_bounds__(256) void wgrad_patch_reduce_grouped_kernel(const f
 // tap): 16-byte loads, a group's 16 threads cover 256 contiguous bytes of a partial.  Same grouping and order as above.
 template <int G>
 __global__ __launch_bounds__(256) void wgrad_patch_reduce_vec_kernel(const float* __restrict__ part, float* __restrict__ out, int n,
-                                                                     int splits, int Cin, FastDiv div_row, FastDiv div_cin) {
+                                                                     int splits, int Cin, FastDiv div_row, FastDiv div_cin,
+                                                                     const ReduceTail tail = ReduceTail()) {
     constexpr int COLS = 256 / G;
+    const int main_blocks = (n + 4 * COLS - 1) / (4 * COLS);
+    if ((int)blockIdx.x >= main_blocks) { reduce_tail<G>(part, n, splits, tail, blockIdx.x - main_blocks); return; }
+    const i64 ps = tail.stride ? tail.stride : n;
     __shared__ float4 sm[G][COLS];
     const int col = threadIdx.x % COLS, g = threadIdx.x / COLS;
     const int j = (blockIdx.x * COLS + col) * 4;
@@ -383,12 +423,12 @@ __global__ __launch_bounds__(256) void wgrad_patch_reduce_vec_kernel(const float
         for (; z + 7 * G < splits; z += 8 * G) {
             float4 v[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(part + (i64)(z + u * G) * n + j);
+            for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(part + (i64)(z + u * G) * ps + j);
 #pragma unroll
             for (int u = 0; u < 8; ++u) { s.x = s.x + v[u].x; s.y = s.y + v[u].y; s.z = s.z + v[u].z; s.w = s.w + v[u].w; }
         }
         for (; z < splits; z += G) {
-            const float4 v = *reinterpret_cast<const float4*>(part + (i64)z * n + j);
+            const float4 v = *reinterpret_cast<const float4*>(part + (i64)z * ps + j);
             s.x = s.x + v.x; s.y = s.y + v.y; s.z = s.z + v.z; s.w = s.w + v.w;
         }
     }

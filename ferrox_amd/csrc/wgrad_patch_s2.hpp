@@ -39,7 +39,9 @@ constexpr int slot(int t, int q, int wk) {
 struct Params {
     const float* x;
     const float* g;
+    const float* act;  // MASK: the layer's ReLU output; g is staged as g * (act > 0)
     float* part;
+    float* bpart;      // MASK: per-split sums of the masked g per output channel ([Cout], part_stride apart): the bias gradient
     int Cin, H, Cout, oh, ph;
     int stages, sps, spi;  // all stages, stages per split, stages per image
     int xcd_chunk;         // blocks / 8 when that divides, else 0
@@ -65,7 +67,10 @@ struct Shape {
     static_assert(XR * CT % RX == 0 && LDS <= LDS_LIMIT, "staging");
 };
 
-template <int WMO, int OW, int R>
+// MASK: the gradient arrives unmasked from the layer above; the ReLU of this layer is applied to the staged rows of g
+// (g * (act > 0), the bits of fx_relu_bwd) and the blocks of the first channel tile also leave the sums of the masked rows
+// over their stages -- the bias gradient -- so no masked copy of g and no separate bias pass exist.
+template <int WMO, int OW, int R, bool MASK>
 __global__ __launch_bounds__(NT, 1) void wgrad_s2_kernel(const Params p) {
     using S = Shape<WMO, OW, R>;
     constexpr int WK = S::WK, BM = S::BM, W = S::W, PW = S::PW, GP = S::GP, PLANE = S::PLANE, BUF = S::BUF;
@@ -102,7 +107,10 @@ __global__ __launch_bounds__(NT, 1) void wgrad_s2_kernel(const Params p) {
     // row-major, q = 32 r + c; thread t owns float4 column t % XL of pairs t / XL + RX u, so the patch row of a pass is a
     // compile-time constant and its validity a scalar.
     const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    float4 gv[S::NG], xv[S::NXP];
+    float4 gv[S::NG], xv[S::NXP], av[MASK ? S::NG : 1];
+    float bsum[S::NG];
+#pragma unroll
+    for (int u = 0; u < S::NG; ++u) bsum[u] = 0.f;
     const int gq = tid & 15, grow = tid >> 4;
     const int xq = tid & (S::XL - 1), xrow = tid / S::XL;
     const bool g_lane = gq < S::KST / 4, x_lane = xq < W / 4;
@@ -118,6 +126,11 @@ __global__ __launch_bounds__(NT, 1) void wgrad_s2_kernel(const Params p) {
         const float* xsrc = p.x + ((i64)b * p.Cin + c0) * p.H * W;
 #pragma unroll
         for (int u = 0; u < S::NG; ++u) gv[u] = ldg4(gsrc + (i64)u * 16 * L, g_off);
+        if constexpr (MASK) {
+            const float* asrc = p.act + ((i64)b * p.Cout + oc0) * L + (i64)oy0 * OW;
+#pragma unroll
+            for (int u = 0; u < S::NG; ++u) av[u] = ldg4(asrc + (i64)u * 16 * L, g_off);
+        }
 #pragma unroll
         for (int u = 0; u < S::NXP; ++u) {
             const int r = u * S::RX / CT, cb = u * S::RX % CT;  // patch row and first channel of this pass
@@ -133,6 +146,11 @@ __global__ __launch_bounds__(NT, 1) void wgrad_s2_kernel(const Params p) {
 #pragma unroll
             for (int u = 0; u < S::NG; ++u) {
                 float* d = smem + gd + u * 16 * GP;
+                if constexpr (MASK) {
+                    gv[u].x = gv[u].x * (av[u].x > 0.f ? 1.f : 0.f); gv[u].y = gv[u].y * (av[u].y > 0.f ? 1.f : 0.f);
+                    gv[u].z = gv[u].z * (av[u].z > 0.f ? 1.f : 0.f); gv[u].w = gv[u].w * (av[u].w > 0.f ? 1.f : 0.f);
+                    bsum[u] = bsum[u] + ((gv[u].x + gv[u].y) + (gv[u].z + gv[u].w));
+                }
                 d[0] = gv[u].x; d[1] = gv[u].y; d[2] = gv[u].z; d[3] = gv[u].w;
             }
         }
@@ -195,6 +213,20 @@ __global__ __launch_bounds__(NT, 1) void wgrad_s2_kernel(const Params p) {
         cur ^= 1;
     }
 
+    if constexpr (MASK) {
+        // bias gradient of this block's stages: the 16 lanes that share a row of g add their sums in a fixed butterfly order
+        if (bxi == 0) {
+#pragma unroll
+            for (int u = 0; u < S::NG; ++u) {
+                float v = bsum[u];
+                v = v + __shfl_xor(v, 8, 64);
+                v = v + __shfl_xor(v, 4, 64);
+                v = v + __shfl_xor(v, 2, 64);
+                v = v + __shfl_xor(v, 1, 64);
+                if (gq == 0) p.bpart[(i64)bzi * p.part_stride + oc0 + grow + 16 * u] = v;
+            }
+        }
+    }
     // The WK waves that split the pixel rows hold partial sums of the same outputs, added here through LDS (the stage buffers
     // are free after the loop's last barrier) in order of the segment, so a block leaves one partial sum.
     float* out = p.part + (i64)bzi * p.part_stride;
@@ -304,40 +336,51 @@ inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 k
     return pl;
 }
 
-inline i64 workspace_bytes(const Plan& pl, i64 Cout, i64 Cin) { return (i64)pl.splits * Cout * Cin * KK * (i64)sizeof(float); }
+// the masked variant keeps [Cout] bias sums behind every split's partial
+inline i64 workspace_bytes(const Plan& pl, i64 Cout, i64 Cin, bool with_bias = false) {
+    return (i64)pl.splits * (Cout * Cin * KK + (with_bias ? Cout : 0)) * (i64)sizeof(float);
+}
 
 // x, g and part must be 16-byte aligned.
-inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float* dw, float* part, i64 Cin, i64 H, i64 Cout, i64 ph, i64 oh) {
+// act / db non-null: the masked variant (act 16-byte aligned as well).
+inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float* dw, float* part, i64 Cin, i64 H, i64 Cout, i64 ph, i64 oh,
+               const float* act = nullptr, float* db = nullptr) {
     Params p;
-    p.x = x; p.g = g; p.part = part;
+    p.x = x; p.g = g; p.part = part; p.act = act; p.bpart = part + Cout * Cin * KK;
     p.Cin = (int)Cin; p.H = (int)H; p.Cout = (int)Cout; p.oh = (int)oh; p.ph = (int)ph;
     p.stages = pl.stages; p.sps = pl.sps; p.spi = (int)(oh / pl.R);
     p.div_spi = FastDiv((uint32_t)p.spi);
-    p.part_stride = Cout * Cin * KK;
+    p.part_stride = Cout * Cin * KK + (act ? Cout : 0);
     const dim3 grid((unsigned)(Cin / CT), (unsigned)(Cout / (32 * pl.WMO)), (unsigned)pl.splits);
     const i64 blocks = (i64)grid.x * grid.y * grid.z;
     p.xcd_chunk = blocks % 8 == 0 && blocks <= 0x7fffffff ? (int)(blocks / 8) : 0;
     bool launched = false;
 #define FX_WG2_LAUNCH(A, O, RR)                                                                                        \
     if (!launched && pl.WMO == A && pl.OW == O && pl.R == RR) {                                                        \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_s2_kernel<A, O, RR>,                     \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_s2_kernel<A, O, RR, false>,              \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
+        static const hipError_t attr_m = hipFuncSetAttribute((const void*)wgrad_s2_kernel<A, O, RR, true>,             \
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
         FX_HIP_CHECK(attr);                                                                                            \
-        wgrad_s2_kernel<A, O, RR><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                                          \
+        FX_HIP_CHECK(attr_m);                                                                                          \
+        if (act) wgrad_s2_kernel<A, O, RR, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                           \
+        else wgrad_s2_kernel<A, O, RR, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                              \
         launched = true;                                                                                               \
     }
     FX_WG2_SHAPES(FX_WG2_LAUNCH)
 #undef FX_WG2_LAUNCH
     FX_REQUIRE(launched, "wgrad stride-2 patch kernel: unexpected shape (%d, %d, %d)", pl.WMO, pl.OW, pl.R);
     FX_LAUNCH_CHECK();
-    const int n = (int)p.part_stride;
+    const int n = (int)(Cout * Cin * KK);
+    const wgp::ReduceTail tail{p.part_stride, act ? db : nullptr, act ? (int)Cout : 0};
     const FastDiv div_row((uint32_t)(KK * Cin)), div_cin((uint32_t)Cin);
+    // (with the bias sums behind each partial the stride stays a multiple of 4 floats: Cout % 32 == 0)
     if (pl.splits >= 128 && n <= (1 << 17) && n % 4 == 0 && Cin % 4 == 0 && fx::aligned16(part))
-        wgp::wgrad_patch_reduce_vec_kernel<16><<<dim3((unsigned)fx::ceil_div((i64)n, 64)), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin);
+        wgp::wgrad_patch_reduce_vec_kernel<16><<<dim3((unsigned)(fx::ceil_div((i64)n, 64) + wgp::tail_blocks(tail, 16))), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail);
     else if (pl.splits >= 128 && n <= (1 << 17))
-        wgp::wgrad_patch_reduce_grouped_kernel<16><<<dim3((unsigned)fx::ceil_div((i64)n, 16)), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin);
+        wgp::wgrad_patch_reduce_grouped_kernel<16><<<dim3((unsigned)(fx::ceil_div((i64)n, 16) + wgp::tail_blocks(tail, 16))), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail);
     else
-        wgp::wgrad_patch_reduce_kernel<<<dim3((unsigned)fx::ceil_div((i64)n, 256)), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin);
+        wgp::wgrad_patch_reduce_kernel<<<dim3((unsigned)(fx::ceil_div((i64)n, 256) + wgp::tail_blocks(tail, 256))), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

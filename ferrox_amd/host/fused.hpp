@@ -63,6 +63,15 @@ template <typename T> struct FusedApi;
         static int conv_bias(fx_ctx* c, const T* x, const T* w, const T* b, T* y, const int64_t* d, int act) {         \
             return fx_conv2d_fwd_bias_act_##S(c, x, w, b, y, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9], d[10], act, nullptr, 0); \
         }                                                                                                              \
+        static int conv_bwd_relu_supported(fx_ctx* c, int kind, const int64_t* d) {                                    \
+            return fx_conv2d_bwd_relu_supported(c, kind, sizeof(T) == 8 ? FX_F64 : FX_F32, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9], d[10]); \
+        }                                                                                                              \
+        static int conv_wgrad_relu_bias(fx_ctx* c, const T* x, const T* g, const T* act, T* dw, T* db, const int64_t* d) { \
+            return fx_conv2d_wgrad_relu_bias_##S(c, x, g, act, dw, db, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9], d[10], nullptr, 0); \
+        }                                                                                                              \
+        static int conv_dgrad_relu(fx_ctx* c, const T* g, const T* act, const T* w, T* dx, const int64_t* d) {         \
+            return fx_conv2d_dgrad_relu_##S(c, g, act, w, dx, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], d[9], d[10]); \
+        }                                                                                                              \
         static int bn_stats(fx_ctx* c, const T* x, T* m, T* v, T* rm, T* rv, double mom, int64_t o, int64_t C, int64_t i) { \
             return fx_batchnorm_stats_##S(c, x, m, v, rm, rv, mom, o, C, i);                                           \
         }                                                                                                              \
@@ -156,6 +165,28 @@ template <typename T> struct Conv2dFusedOp : Operator<T> {  // inputs: x [B,Cin,
         const Shape gs = g->shape();
         std::vector<Tensor<T>> r(3);
         r[2] = HipStorage<T>::alloc({gs[1]});
+        if (relu && BackendManager::get().conv_grad_mode == 0) {
+            // The consumers of the masked gradient apply the mask themselves while they stage g, and the weight-gradient kernel
+            // leaves the bias gradient: no masked copy of g, no separate pass (where both kernels the layer needs exist).
+            const Shape &xs = in[0]->shape(), &ws = in[1]->shape();
+            const int64_t d[11] = {(int64_t)xs[0], (int64_t)xs[1], (int64_t)xs[2], (int64_t)xs[3], (int64_t)ws[0], (int64_t)ws[2], (int64_t)ws[3],
+                                   (int64_t)stride.first, (int64_t)stride.second, (int64_t)padding.first, (int64_t)padding.second};
+            static const bool off = [] { const char* v = getenv("FX_CONV_BWD_FUSED"); return v && atoi(v) == 0; }();
+            if (!off && FusedApi<T>::conv_bwd_relu_supported(fused_ctx(), FX_CONV_WGRAD, d) &&
+                (!needs[0] || FusedApi<T>::conv_bwd_relu_supported(fused_ctx(), FX_CONV_DGRAD, d))) {
+                r[1] = HipStorage<T>::alloc(ws);
+                const int rc = FusedApi<T>::conv_wgrad_relu_bias(fused_ctx(), in[0]->data(), g->data(), out->data(), r[1]->data(), r[2]->data(), d);
+                if (rc == FX_OK) {
+                    if (needs[0]) {
+                        r[0] = HipStorage<T>::alloc(xs);
+                        fx_ok(FusedApi<T>::conv_dgrad_relu(fused_ctx(), g->data(), out->data(), in[1]->data(), r[0]->data(), d));
+                    }
+                    return r;
+                }
+                if (rc != FX_ERR_UNSUPPORTED) fx_ok(rc);  // a misaligned tensor: the separate passes below
+                r[1].reset();
+            }
+        }
         if (relu) {  // mask and bias gradient in one pass over g
             Tensor<T> gm = HipStorage<T>::alloc(gs);
             fx_ok(FusedApi<T>::relu_bias_grad(fused_ctx(), g->data(), out->data(), gm->data(), r[2]->data(), (int64_t)gs[0], (int64_t)gs[1],

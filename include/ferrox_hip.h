@@ -278,6 +278,24 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
                                    int64_t ph, int64_t pw, int act, void* workspace, int64_t ws_bytes);                \
     int fx_gemm_bias_act_##S(fx_ctx* ctx, int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const T* A,       \
                              const T* B, const T* bias, T* C, int act);                                                \
+    /* Backward of a convolution whose output went through a ReLU (Conv2dOp::gradient, src/ops/batched.rs:194-217,     \
+       after ReLU::gradient, src/ops/unary.rs:358-375, and the bias reduction of src/ops/basic.rs:10-53), from the     \
+       UNMASKED upstream gradient g and the layer's activation act = relu(conv(x) + b), both [B,Cout,oh,ow]:           \
+         wgrad_relu_bias: dw = fx_conv2d_wgrad(x, g'), db[oc] = sum over (b, pixel) of g'      with g' = g*(act > 0)   \
+         dgrad_relu:      dx = fx_conv2d_dgrad(g', w)                                                                   \
+       g' is formed while the kernels stage g (the bits of fx_relu_bwd) and is never written: the separate mask +      \
+       bias pass and its read-back disappear.  Gradient mode 0 only.  dw and dx have the bits of the two-call          \
+       sequences; db is summed in the kernel's own fixed order (equal to fx_bias_grad up to rounding).  Served for     \
+       the shapes fx_conv2d_bwd_relu_supported reports (f32: 3x3 image layers of at most 3 channels; 3x3 stride-2      \
+       padding-1 layers over even maps 32 or 64 wide); any other call returns FX_ERR_UNSUPPORTED and changes nothing.  \
+       workspace as for fx_conv2d_wgrad (fx_conv2d_workspace_bytes(FX_CONV_WGRAD, ...) covers it). */                  \
+    int fx_conv2d_wgrad_relu_bias_##S(fx_ctx* ctx, const T* x, const T* g, const T* act, T* dw, T* db, int64_t B,      \
+                                      int64_t Cin, int64_t H, int64_t W, int64_t Cout, int64_t kh, int64_t kw,         \
+                                      int64_t sh, int64_t sw, int64_t ph, int64_t pw, void* workspace,                 \
+                                      int64_t ws_bytes);                                                               \
+    int fx_conv2d_dgrad_relu_##S(fx_ctx* ctx, const T* g, const T* act, const T* w, T* dx, int64_t B, int64_t Cin,     \
+                                 int64_t H, int64_t W, int64_t Cout, int64_t kh, int64_t kw, int64_t sh, int64_t sw,   \
+                                 int64_t ph, int64_t pw);                                                              \
     /* Linear's weight and bias gradient in one call (nn/layers/linear.rs:152-308: MatMul::gradient, ops/matrix.rs:    \
        34-55, and reduce_gradient_for_broadcasting, ops/basic.rs:10-53): C[M,N] = A^T . B for A = dY stored [K, M] and \
        B = X stored [K, N] -- fx_gemm(1, 0, ...) up to the order of summation -- and colsum[m] = sum over k of         \
@@ -392,6 +410,11 @@ FX_DECLARE_KERNELS(double, f64)
  *     host rewrites the values between launches.
  * A launch is stream-ordered like any other call; results are bit-identical to the eager calls (same kernels, same
  * arguments). */
+/* 1 when fx_conv2d_wgrad_relu_bias (kind FX_CONV_WGRAD) / fx_conv2d_dgrad_relu (kind FX_CONV_DGRAD) has a fused kernel
+ * for this dtype and shape on this context's device (16-byte aligned tensors assumed), else 0. */
+int fx_conv2d_bwd_relu_supported(fx_ctx* ctx, int kind, int dtype, int64_t B, int64_t Cin, int64_t H, int64_t W, int64_t Cout,
+                                 int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw);
+
 typedef struct fx_graph fx_graph;
 int fx_graph_begin(fx_ctx* ctx);
 int fx_graph_end(fx_ctx* ctx, fx_graph** out);
