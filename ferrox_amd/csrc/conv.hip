@@ -603,11 +603,11 @@ i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     const wg2::Plan p2 = patch_s2_plan<T>(c, d, mode);
     if (p2.ok) generic = std::max(generic, wg2::workspace_bytes(p2, d.Cout, d.Cin, true));
     const wgd2::Plan q2 = patch64_s2_plan<T>(c, d, mode);
-    if (q2.ok) generic = std::max(generic, wgd2::workspace_bytes(q2, d.Cout, d.Cin));
+    if (q2.ok) generic = std::max(generic, wgd2::workspace_bytes(q2, d.Cout, d.Cin, true));
     if constexpr (sizeof(T) == 8) {
         if (mode == 0 && !generic_only()) {
             const cim::WPlan ip = cim::wgrad_plan(c ? c->num_cus : 256, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
-            if (ip.ok) generic = std::max(generic, cim::wgrad_workspace_bytes(ip, d.Cout, d.Cin));
+            if (ip.ok) generic = std::max(generic, cim::wgrad_workspace_bytes(ip, d.Cout, d.Cin, true));
         }
     }
     return pl.ok ? std::max(generic, wgp::workspace_bytes(pl, d.Cout, d.Cin)) : generic;
@@ -715,6 +715,14 @@ bool bwd_relu_supported(int num_cus, int kind, const Dims& d) {
         }
         if (kind == FX_CONV_DGRAD)
             return !dgrad_small_cin_ok<T>(d) && dg2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow).ok;
+    } else {
+        if (generic_only() || d.B > d.bc) return false;
+        if (kind == FX_CONV_WGRAD) {
+            if (cim::wgrad_plan(num_cus, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw).ok) return true;
+            return wgd2::make_plan(num_cus, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow).ok;
+        }
+        if (kind == FX_CONV_DGRAD)
+            return !dgrad_small_cin_ok<T>(d) && dgd2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow).ok;
     }
     return false;
 }
@@ -748,6 +756,19 @@ int conv_wgrad_relu_bias(fx_ctx* c, const T* x, const T* g, const T* act, T* dw,
                 return wg2::run(c, p2, x, g, dw, part, Cin, H, Cout, ph, d.oh, act, db);
             }
         }
+    } else {
+        if (bwd_relu_supported<T>(c->num_cus, FX_CONV_WGRAD, d) && aligned16(x, g) && aligned16(act, ws)) {
+            const i64 need = wgrad_ws_bytes<T>(c, d, 0);
+            FX_REQUIRE(ws == nullptr || ws_bytes >= need, "fx_conv2d_wgrad_relu_bias: workspace of %lld bytes is smaller than the %lld needed",
+                       (long long)ws_bytes, (long long)need);
+            std::lock_guard<std::mutex> lk(c->launch_mutex);
+            double* part = (double*)(ws ? ws : c->get_scratch(need));
+            if (!part) return FX_ERR_OOM;
+            const cim::WPlan ip = cim::wgrad_plan(c->num_cus, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
+            if (ip.ok) return cim::run_wgrad(c, ip, x, g, dw, part, Cin, H, Cout, act, db);
+            const wgd2::Plan q2 = patch64_s2_plan<T>(c, d, 0);
+            if (q2.ok) return wgd2::run(c, q2, x, g, dw, part, Cin, H, Cout, ph, d.oh, act, db);
+        }
     }
     fx::set_error("fx_conv2d_wgrad_relu_bias: no fused kernel for this shape, dtype or alignment (ask fx_conv2d_bwd_relu_supported; use "
                   "fx_relu_bwd_bias_grad + fx_conv2d_wgrad)");
@@ -767,6 +788,12 @@ int conv_dgrad_relu(fx_ctx* c, const T* g, const T* act, const T* w, T* dx, i64 
             const dg2::Plan p2 = dg2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
             return dg2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh, act);
         }
+    } else {
+        if (bwd_relu_supported<T>(c->num_cus, FX_CONV_DGRAD, d) && aligned16(g, w) && aligned16(dx, act)) {
+            std::lock_guard<std::mutex> lk(c->launch_mutex);
+            const dgd2::Plan p2 = dgd2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
+            return dgd2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh, act);
+        }
     }
     fx::set_error("fx_conv2d_dgrad_relu: no fused kernel for this shape, dtype or alignment (ask fx_conv2d_bwd_relu_supported; use "
                   "fx_relu_bwd + fx_conv2d_dgrad)");
@@ -778,6 +805,10 @@ int conv_dgrad_relu(fx_ctx* c, const T* g, const T* act, const T* w, T* dx, i64 
 extern "C" int fx_conv2d_bwd_relu_supported(fx_ctx* c, int kind, int dtype, int64_t B, int64_t Cin, int64_t H, int64_t W, int64_t Cout,
                                             int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw) {
     Dims d;
+    if (dtype == FX_F64) {
+        if (check_dims<double>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_bwd_relu_supported")) return 0;
+        return bwd_relu_supported<double>(c ? c->num_cus : 256, kind, d) ? 1 : 0;
+    }
     if (dtype != FX_F32 || check_dims<float>(d, B, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, "fx_conv2d_bwd_relu_supported")) return 0;
     return bwd_relu_supported<float>(c ? c->num_cus : 256, kind, d) ? 1 : 0;
 }

@@ -171,7 +171,9 @@ inline int run(fx_ctx* c, const double* x, const double* w, double* y, i64 B, i6
 struct WParams {
     const double* x;
     const double* g;
-    double* part;  // [splits][Cout][Cin * 9]
+    const double* act;  // MASK: the layer's ReLU output; g is staged as g * (act > 0)
+    double* part;       // [splits][Cout][Cin * 9] (MASK: + [Cout] sums of the masked g behind each: the bias gradient)
+    i64 part_stride;    // doubles between the partial sums of two splits
     int Cin, Cout, H, tpi;
     int tiles, tps;  // B * tiles per image, tiles per split
     FastDiv div_tpi;
@@ -179,6 +181,10 @@ struct WParams {
 
 constexpr int GPITCH = PIX + 1;
 
+// MASK: the gradient arrives unmasked and this layer's ReLU is applied while g is staged (g * (act > 0), the bits of
+// fx_relu_bwd); pair index K <= 27 of the 32 is free, and with an operand of 1.0 there the MFMA leaves the sums of the masked g
+// over the pixels in it: the bias gradient.
+template <bool MASK>
 __global__ __launch_bounds__(NT) void image_wgrad_f64_kernel(const WParams p) {
     using S = Shape<32>;
     constexpr int W = 32, TR = S::TR, PR = S::PR, PW = S::PW, PLANE = S::PLANE;
@@ -192,11 +198,12 @@ __global__ __launch_bounds__(NT) void image_wgrad_f64_kernel(const WParams p) {
 
     // this lane's (channel, tap) pairs: 16 nb + l16; pairs past K read a valid address and contribute zeros
     int xoff[2];
-    bool pair_ok[2];
+    bool pair_ok[2], pair_one[2];
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
         const int kp = 16 * nb + l16;
         pair_ok[nb] = kp < K;
+        pair_one[nb] = MASK && kp == K;
         const int c = pair_ok[nb] ? kp / KK : 0, t = pair_ok[nb] ? kp % KK : 0;
         xoff[nb] = c * PLANE + (wave + t / 3) * PW + t % 3 + kq;  // pixel (row wave, column 4 s + kq): + 4 s per step
     }
@@ -224,6 +231,11 @@ __global__ __launch_bounds__(NT) void image_wgrad_f64_kernel(const WParams p) {
         for (int u = 0; u < 8; ++u) {
             const int f = u * NT + tid, row = f >> 7, q = f & 127;
             gv[u] = *reinterpret_cast<const double2*>(gsrc + (i64)row * L + 2 * q);
+            if constexpr (MASK) {
+                const double2 a = *reinterpret_cast<const double2*>(p.act + (gsrc - p.g) + (i64)row * L + 2 * q);
+                gv[u].x = gv[u].x * (a.x > 0. ? 1. : 0.);
+                gv[u].y = gv[u].y * (a.y > 0. ? 1. : 0.);
+            }
         }
         const double* xsrc = p.x + (i64)b * p.Cin * L;
         double2 xv[2];
@@ -260,8 +272,8 @@ __global__ __launch_bounds__(NT) void image_wgrad_f64_kernel(const WParams p) {
         for (int s = 0; s < W / 4; ++s) {
             const double a0 = Gs[goff + 4 * s], a1 = Gs[goff + 16 * GPITCH + 4 * s];
             double b0 = Xs[xoff[0] + 4 * s], b1 = Xs[xoff[1] + 4 * s];
-            if (!pair_ok[0]) b0 = 0.;
-            if (!pair_ok[1]) b1 = 0.;
+            if (!pair_ok[0]) b0 = pair_one[0] ? 1. : 0.;
+            if (!pair_ok[1]) b1 = pair_one[1] ? 1. : 0.;
             acc[0][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(a0, b0, acc[0][0], 0, 0, 0);
             acc[0][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(a0, b1, acc[0][1], 0, 0, 0);
             acc[1][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(a1, b0, acc[1][0], 0, 0, 0);
@@ -278,7 +290,8 @@ __global__ __launch_bounds__(NT) void image_wgrad_f64_kernel(const WParams p) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) red[(wave * 16 + 4 * (2 * m + nb) + e) * 64 + lane] = acc[m][nb][e];
     __syncthreads();
-    double* out = p.part + ((i64)blockIdx.x * p.Cout + oc0) * K;
+    double* out = p.part + (i64)blockIdx.x * p.part_stride + (i64)oc0 * K;
+    double* bout = p.part + (i64)blockIdx.x * p.part_stride + (i64)p.Cout * K + oc0;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
         const int el = 2 * wave + u, blk = el >> 2, e = el & 3;  // wave w finishes elements 2 w and 2 w + 1
@@ -287,6 +300,7 @@ __global__ __launch_bounds__(NT) void image_wgrad_f64_kernel(const WParams p) {
         for (int w = 1; w < 8; ++w) v = v + red[(w * 16 + el) * 64 + lane];
         const int oc = 16 * (blk >> 1) + 4 * e + kq, kp = 16 * (blk & 1) + l16;
         if (kp < K) out[(i64)oc * K + kp] = v;
+        if (MASK && kp == K) bout[oc] = v;
     }
 }
 
@@ -310,21 +324,32 @@ inline WPlan wgrad_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64
     pl.ok = true;
     return pl;
 }
-inline i64 wgrad_workspace_bytes(const WPlan& pl, i64 Cout, i64 Cin) { return (i64)pl.splits * Cout * Cin * KK * (i64)sizeof(double); }
+// the masked variant keeps [Cout] bias sums behind every split's partial
+inline i64 wgrad_workspace_bytes(const WPlan& pl, i64 Cout, i64 Cin, bool with_bias = false) {
+    return (i64)pl.splits * (Cout * Cin * KK + (with_bias ? Cout : 0)) * (i64)sizeof(double);
+}
 
 // x, g and part must be 16-byte aligned.
-inline int run_wgrad(fx_ctx* c, const WPlan& pl, const double* x, const double* g, double* dw, double* part, i64 Cin, i64 H, i64 Cout) {
+// act / db non-null: the masked variant (act 16-byte aligned as well).
+inline int run_wgrad(fx_ctx* c, const WPlan& pl, const double* x, const double* g, double* dw, double* part, i64 Cin, i64 H, i64 Cout,
+                     const double* act = nullptr, double* db = nullptr) {
     WParams p;
-    p.x = x; p.g = g; p.part = part;
+    p.x = x; p.g = g; p.part = part; p.act = act;
+    p.part_stride = Cout * Cin * KK + (act ? Cout : 0);
     p.Cin = (int)Cin; p.Cout = (int)Cout; p.H = (int)H;
     p.tpi = (int)(H / (PIX / 32));
     p.tiles = pl.tiles; p.tps = pl.tps;
     p.div_tpi = FastDiv((uint32_t)p.tpi);
     const size_t lds = std::max((size_t)(32 * GPITCH + Shape<32>::XCH), (size_t)8 * 16 * 64) * sizeof(double);
-    static const hipError_t attr = hipFuncSetAttribute((const void*)image_wgrad_f64_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    static const hipError_t attr = hipFuncSetAttribute((const void*)image_wgrad_f64_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    static const hipError_t attr_m = hipFuncSetAttribute((const void*)image_wgrad_f64_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
     FX_HIP_CHECK(attr);
-    image_wgrad_f64_kernel<<<dim3((unsigned)pl.splits, (unsigned)(Cout / 32)), dim3(NT), lds, c->stream>>>(p);
+    FX_HIP_CHECK(attr_m);
+    const dim3 grid((unsigned)pl.splits, (unsigned)(Cout / 32));
+    if (act) image_wgrad_f64_kernel<true><<<grid, dim3(NT), lds, c->stream>>>(p);
+    else image_wgrad_f64_kernel<false><<<grid, dim3(NT), lds, c->stream>>>(p);
     FX_LAUNCH_CHECK();
+    if (act) return igemm::launch_splitk_reduce_pair<double>(c, part, p.part_stride, pl.splits, dw, Cout * Cin * KK, db, Cout);
     return igemm::launch_splitk_reduce<double>(c, part, dw, Cout * Cin * KK, pl.splits);
 }
 

@@ -30,6 +30,7 @@ constexpr size_t LDS_LIMIT = 160 * 1024;
 
 struct Params {
     const double* g;
+    const double* act;  // MASK: the ReLU output of the layer whose gradient g is; g is staged as g * (act > 0)
     const double* w;
     double* dx;
     int Cin, Cout, oh, tpi, nct;  // tiles per image, channel tiles
@@ -58,7 +59,8 @@ struct Shape {
     static_assert(CELLS % OW == 0 && OW % 16 == 0 && OCC % 4 == 0 && OCC * (CELLS / 2) % NT == 0 && X2 <= NT && LDS <= LDS_LIMIT, "shape");
 };
 
-template <int OW, int OCC>
+// MASK: grad_out arrives unmasked and the layer's ReLU is applied to the staged patch (g * (act > 0), the bits of fx_relu_bwd).
+template <int OW, int OCC, bool MASK>
 __global__ __launch_bounds__(NT, 1) void dgrad_s2_f64_kernel(const Params p) {
     using S = Shape<OW, OCC>;
     constexpr int TR = S::TR, PC = S::PC, GPL = S::GPL, KS = S::KS, WCH = S::WCH, BUF = S::BUF;
@@ -74,9 +76,15 @@ __global__ __launch_bounds__(NT, 1) void dgrad_s2_f64_kernel(const Params p) {
 
     // staging maps (constant over the chunks)
     const double2 zero2 = make_double2(0., 0.);
-    double2 wv[S::NWP], gv[S::NGP], xv;
+    double2 wv[S::NWP], gv[S::NGP], xv, av[MASK ? S::NGP : 1], axv;
     const double* wsrc = p.w + (i64)c0 * KK;
     const double* gsrc = p.g + ((i64)b * p.Cout * p.oh + i0) * OW;
+    const double* asrc = MASK ? p.act + ((i64)b * p.Cout * p.oh + i0) * OW : nullptr;
+    auto masked = [](double2 v, const double2& a) __attribute__((always_inline)) {
+        v.x = v.x * (a.x > 0. ? 1. : 0.);
+        v.y = v.y * (a.y > 0. ? 1. : 0.);
+        return v;
+    };
     const int gq = tid & 127, goc = tid >> 7;                   // double2 of the tile's TR * OW doubles, oc within a pass of 4
     const int g_dst = goc * GPL + (gq / (OW / 2)) * PC + (gq % (OW / 2)) * 2;
     const uint32_t g_off = (uint32_t)(goc * L + 2 * gq) * 8u;
@@ -96,6 +104,12 @@ __global__ __launch_bounds__(NT, 1) void dgrad_s2_f64_kernel(const Params p) {
         for (int u = 0; u < S::NGP; ++u) gv[u] = ldg2(gsrc + (i64)(oc0 + 4 * u) * L, g_off);
         if (next_row) xv = ldg2(gsrc + (i64)oc0 * L, x_off);
         else xv = zero2;
+        if constexpr (MASK) {
+#pragma unroll
+            for (int u = 0; u < S::NGP; ++u) av[u] = ldg2(asrc + (i64)(oc0 + 4 * u) * L, g_off);
+            if (next_row) axv = ldg2(asrc + (i64)oc0 * L, x_off);
+            else axv = zero2;
+        }
     };
     auto park = [&](int buf) __attribute__((always_inline)) {
         double* Ws = smem + buf * BUF;
@@ -116,10 +130,12 @@ __global__ __launch_bounds__(NT, 1) void dgrad_s2_f64_kernel(const Params p) {
 #pragma unroll
         for (int u = 0; u < S::NGP; ++u) {
             double* d = Gs + g_dst + 4 * u * GPL;
+            if constexpr (MASK) gv[u] = masked(gv[u], av[u]);
             d[0] = gv[u].x; d[1] = gv[u].y;
         }
         if (x_lane) {
             double* d = Gs + xoc * GPL + TR * PC + 2 * xq;
+            if constexpr (MASK) xv = masked(xv, axv);
             d[0] = xv.x; d[1] = xv.y;
         }
     };
@@ -238,9 +254,11 @@ inline Plan make_plan(i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i6
 }
 
 // g, w and dx must be 16-byte aligned.
-inline int run(fx_ctx* c, const Plan& pl, const double* g, const double* w, double* dx, i64 B, i64 Cin, i64 Cout, i64 oh) {
+// act non-null: the masked variant (act 16-byte aligned as well).
+inline int run(fx_ctx* c, const Plan& pl, const double* g, const double* w, double* dx, i64 B, i64 Cin, i64 Cout, i64 oh,
+               const double* act = nullptr) {
     Params p;
-    p.g = g; p.w = w; p.dx = dx;
+    p.g = g; p.w = w; p.dx = dx; p.act = act;
     p.Cin = (int)Cin; p.Cout = (int)Cout; p.oh = (int)oh;
     p.tpi = (int)(oh / (CELLS / pl.OW));
     p.nct = (int)(Cin / CT);
@@ -250,10 +268,14 @@ inline int run(fx_ctx* c, const Plan& pl, const double* g, const double* w, doub
     bool launched = false;
 #define FX_DGD2_LAUNCH(O, C_)                                                                                          \
     if (!launched && pl.OW == O && pl.OCC == C_) {                                                                     \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)dgrad_s2_f64_kernel<O, C_>,                    \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)dgrad_s2_f64_kernel<O, C_, false>,             \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
+        static const hipError_t attr_m = hipFuncSetAttribute((const void*)dgrad_s2_f64_kernel<O, C_, true>,            \
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
         FX_HIP_CHECK(attr);                                                                                            \
-        dgrad_s2_f64_kernel<O, C_><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                                         \
+        FX_HIP_CHECK(attr_m);                                                                                          \
+        if (act) dgrad_s2_f64_kernel<O, C_, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                          \
+        else dgrad_s2_f64_kernel<O, C_, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                             \
         launched = true;                                                                                               \
     }
     FX_DGD2_SHAPES(FX_DGD2_LAUNCH)

@@ -331,8 +331,17 @@ __device__ __forceinline__ void reduce_tail(const float* __restrict__ part, int 
     const int col = threadIdx.x % COLS, g = threadIdx.x / COLS;
     const int i = block * COLS + col;
     float s = 0.f;
-    if (i < t.nb)
-        for (int z = g; z < splits; z += G) s = s + part[(i64)z * t.stride + n + i];
+    if (i < t.nb) {
+        int z = g;
+        for (; z + 7 * G < splits; z += 8 * G) {  // eight loads in flight, added in order
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = part[(i64)(z + u * G) * t.stride + n + i];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s = s + v[u];
+        }
+        for (; z < splits; z += G) s = s + part[(i64)z * t.stride + n + i];
+    }
     smt[g][col] = s;
     __syncthreads();
     if (g == 0 && i < t.nb) {

@@ -214,9 +214,49 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_f64_kernel(const Params p) 
             }
 }
 
+// A second, short result behind every partial (the bias sums of the masked kernels: nb doubles at offset n of each split,
+// splits `stride` doubles apart; stride 0 = the partials are n apart and there is no tail).  The blocks past the main ones
+// of a reduce launch add it over the splits, G threads per output like the main sum.
+struct ReduceTail {
+    i64 stride = 0;
+    double* db = nullptr;
+    int nb = 0;
+};
+inline i64 tail_blocks(const ReduceTail& t, int outputs_per_block) { return t.db ? fx::ceil_div((i64)t.nb, (i64)outputs_per_block) : 0; }
+template <int G>
+__device__ __forceinline__ void reduce_tail(const double* __restrict__ part, int n, int splits, const ReduceTail& t, int block) {
+    constexpr int COLS = 256 / G;
+    __shared__ double smt[G][COLS];
+    const int col = threadIdx.x % COLS, g = threadIdx.x / COLS;
+    const int i = block * COLS + col;
+    double s = 0.;
+    if (i < t.nb) {
+        int z = g;
+        for (; z + 7 * G < splits; z += 8 * G) {  // eight loads in flight, added in order
+            double v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = part[(i64)(z + u * G) * t.stride + n + i];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s = s + v[u];
+        }
+        for (; z < splits; z += G) s = s + part[(i64)z * t.stride + n + i];
+    }
+    smt[g][col] = s;
+    __syncthreads();
+    if (g == 0 && i < t.nb) {
+        double v = smt[0][col];
+#pragma unroll
+        for (int u = 1; u < G; ++u) v = v + smt[u][col];
+        t.db[i] = v;
+    }
+}
+
 // out[(oc*Cin + c)*KK + t] = sum_z part[z][oc][t][c], splits added in order.
 __global__ __launch_bounds__(256) void wgrad_f64_reduce_kernel(const double* __restrict__ part, double* __restrict__ out, int n, int splits,
-                                                               int Cin, FastDiv div_row, FastDiv div_cin) {
+                                                               int Cin, FastDiv div_row, FastDiv div_cin, const ReduceTail tail = ReduceTail()) {
+    const int main_blocks = (n + 255) / 256;
+    if ((int)blockIdx.x >= main_blocks) { reduce_tail<1>(part, n, splits, tail, blockIdx.x - main_blocks); return; }
+    const i64 ps = tail.stride ? tail.stride : n;
     const int j = blockIdx.x * 256 + threadIdx.x;
     if (j >= n) return;
     double s = 0.;
@@ -224,11 +264,11 @@ __global__ __launch_bounds__(256) void wgrad_f64_reduce_kernel(const double* __r
     for (; z + 8 <= splits; z += 8) {
         double v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = part[(i64)(z + u) * n + j];
+        for (int u = 0; u < 8; ++u) v[u] = part[(i64)(z + u) * ps + j];
 #pragma unroll
         for (int u = 0; u < 8; ++u) s = s + v[u];
     }
-    for (; z < splits; ++z) s = s + part[(i64)z * n + j];
+    for (; z < splits; ++z) s = s + part[(i64)z * ps + j];
     const int oc = (int)div_row.div((uint32_t)j), rem = j - oc * (KK * Cin);
     const int t = (int)div_cin.div((uint32_t)rem), c = rem - t * Cin;
     out[((i64)oc * Cin + c) * KK + t] = s;
@@ -239,8 +279,11 @@ __global__ __launch_bounds__(256) void wgrad_f64_reduce_kernel(const double* __r
 // group's 16 threads read 256 contiguous bytes of a partial with 16-byte loads.
 template <int G>
 __global__ __launch_bounds__(256) void wgrad_f64_reduce_vec_kernel(const double* __restrict__ part, double* __restrict__ out, int n, int splits,
-                                                                   int Cin, FastDiv div_row, FastDiv div_cin) {
+                                                                   int Cin, FastDiv div_row, FastDiv div_cin, const ReduceTail tail = ReduceTail()) {
     constexpr int COLS = 256 / G;
+    const int main_blocks = (n + 2 * COLS - 1) / (2 * COLS);
+    if ((int)blockIdx.x >= main_blocks) { reduce_tail<G>(part, n, splits, tail, blockIdx.x - main_blocks); return; }
+    const i64 ps = tail.stride ? tail.stride : n;
     __shared__ double2 sm[G][COLS];
     const int col = threadIdx.x % COLS, g = threadIdx.x / COLS;
     const int j = (blockIdx.x * COLS + col) * 2;
@@ -250,12 +293,12 @@ __global__ __launch_bounds__(256) void wgrad_f64_reduce_vec_kernel(const double*
         for (; z + 7 * G < splits; z += 8 * G) {
             double2 v[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const double2*>(part + (i64)(z + u * G) * n + j);
+            for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const double2*>(part + (i64)(z + u * G) * ps + j);
 #pragma unroll
             for (int u = 0; u < 8; ++u) { s.x = s.x + v[u].x; s.y = s.y + v[u].y; }
         }
         for (; z < splits; z += G) {
-            const double2 v = *reinterpret_cast<const double2*>(part + (i64)z * n + j);
+            const double2 v = *reinterpret_cast<const double2*>(part + (i64)z * ps + j);
             s.x = s.x + v.x; s.y = s.y + v.y;
         }
     }

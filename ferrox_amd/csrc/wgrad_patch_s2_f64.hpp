@@ -30,7 +30,9 @@ constexpr size_t LDS_LIMIT = 160 * 1024;
 struct Params {
     const double* x;
     const double* g;
+    const double* act;  // MASK: the layer's ReLU output; g is staged as g * (act > 0)
     double* part;
+    double* bpart;      // MASK: per-split sums of the masked g per output channel ([Cout], part_stride apart): the bias gradient
     int Cin, H, Cout, oh, ph;
     int stages, sps, spi;  // all stages, stages per split, stages per image
     int xcd_chunk;         // blocks / 8 when that divides, else 0
@@ -51,9 +53,13 @@ struct Shape {
     static constexpr int BUF = BM * GP + CT * PLANE;                      // doubles per stage buffer
     static constexpr size_t LDS = 2 * (size_t)BUF * sizeof(double);
     static_assert(OW % 4 == 0 && NT % XL == 0 && CT % RX == 0 && XR * CT % RX == 0 && NT % GL == 0 && BM % GR == 0 && LDS <= LDS_LIMIT, "shape");
+    static_assert(GL == 16, "the bias sums of the masked variant are added over the 16 lanes of a row");
 };
 
-template <int OW, int R>
+// MASK: the gradient arrives unmasked from the layer above; the ReLU of this layer is applied to the staged rows of g
+// (g * (act > 0), the bits of fx_relu_bwd) and the blocks of the first channel tile also leave the sums of the masked rows
+// over their stages: the bias gradient.
+template <int OW, int R, bool MASK>
 __global__ __launch_bounds__(NT, 1) void wgrad_s2_f64_kernel(const Params p) {
     using S = Shape<OW, R>;
     constexpr int W = S::W, PW = S::PW, GP = S::GP, PLANE = S::PLANE, BUF = S::BUF;
@@ -93,7 +99,10 @@ __global__ __launch_bounds__(NT, 1) void wgrad_s2_f64_kernel(const Params p) {
     // row-major, q = 32 r + c; thread t owns double2 column t % XL of pairs t / XL + RX u, so the patch row of a pass is a
     // compile-time constant and its validity a scalar.
     const double2 zero2 = make_double2(0., 0.);
-    double2 gv[S::NG], xv[S::NXP];
+    double2 gv[S::NG], xv[S::NXP], av[MASK ? S::NG : 1];
+    double bsum[S::NG];
+#pragma unroll
+    for (int u = 0; u < S::NG; ++u) bsum[u] = 0.;
     const int gq = tid % S::GL, grow = tid / S::GL;
     const int xq = tid % S::XL, xrow = tid / S::XL;
     const uint32_t g_off = (uint32_t)(grow * L + 2 * gq) * 8u;
@@ -108,6 +117,11 @@ __global__ __launch_bounds__(NT, 1) void wgrad_s2_f64_kernel(const Params p) {
         const double* xsrc = p.x + ((i64)b * p.Cin + c0) * p.H * W;
 #pragma unroll
         for (int u = 0; u < S::NG; ++u) gv[u] = ldg2(gsrc + (i64)u * S::GR * L, g_off);
+        if constexpr (MASK) {
+            const double* asrc = p.act + ((i64)b * p.Cout + oc0) * L + (i64)oy0 * OW;
+#pragma unroll
+            for (int u = 0; u < S::NG; ++u) av[u] = ldg2(asrc + (i64)u * S::GR * L, g_off);
+        }
 #pragma unroll
         for (int u = 0; u < S::NXP; ++u) {
             const int r = u * S::RX / CT, cb = u * S::RX % CT;  // patch row and first channel of this pass
@@ -122,6 +136,11 @@ __global__ __launch_bounds__(NT, 1) void wgrad_s2_f64_kernel(const Params p) {
 #pragma unroll
         for (int u = 0; u < S::NG; ++u) {
             double* d = smem + gd + u * S::GR * GP;
+            if constexpr (MASK) {
+                gv[u].x = gv[u].x * (av[u].x > 0. ? 1. : 0.);
+                gv[u].y = gv[u].y * (av[u].y > 0. ? 1. : 0.);
+                bsum[u] = bsum[u] + (gv[u].x + gv[u].y);
+            }
             d[0] = gv[u].x; d[1] = gv[u].y;
         }
 #pragma unroll
@@ -184,6 +203,20 @@ __global__ __launch_bounds__(NT, 1) void wgrad_s2_f64_kernel(const Params p) {
         cur ^= 1;
     }
 
+    if constexpr (MASK) {
+        // bias gradient of this block's stages: the 16 lanes that share a row of g add their sums in a fixed butterfly order
+        if (bxi == 0) {
+#pragma unroll
+            for (int u = 0; u < S::NG; ++u) {
+                double v = bsum[u];
+                v = v + __shfl_xor(v, 8, 64);
+                v = v + __shfl_xor(v, 4, 64);
+                v = v + __shfl_xor(v, 2, 64);
+                v = v + __shfl_xor(v, 1, 64);
+                if (gq == 0) p.bpart[(i64)bzi * p.part_stride + oc0 + grow + S::GR * u] = v;
+            }
+        }
+    }
     double* out = p.part + (i64)bzi * p.part_stride;
     const int ldo = KK * p.Cin;
 #pragma unroll
@@ -231,39 +264,49 @@ inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 k
     return pl;
 }
 
-inline i64 workspace_bytes(const Plan& pl, i64 Cout, i64 Cin) { return (i64)pl.splits * Cout * Cin * KK * (i64)sizeof(double); }
+// the masked variant keeps [Cout] bias sums behind every split's partial
+inline i64 workspace_bytes(const Plan& pl, i64 Cout, i64 Cin, bool with_bias = false) {
+    return (i64)pl.splits * (Cout * Cin * KK + (with_bias ? Cout : 0)) * (i64)sizeof(double);
+}
 
 // x, g and part must be 16-byte aligned.
-inline int run(fx_ctx* c, const Plan& pl, const double* x, const double* g, double* dw, double* part, i64 Cin, i64 H, i64 Cout, i64 ph, i64 oh) {
+// act / db non-null: the masked variant (act 16-byte aligned as well).
+inline int run(fx_ctx* c, const Plan& pl, const double* x, const double* g, double* dw, double* part, i64 Cin, i64 H, i64 Cout, i64 ph, i64 oh,
+               const double* act = nullptr, double* db = nullptr) {
     Params p;
-    p.x = x; p.g = g; p.part = part;
+    p.x = x; p.g = g; p.part = part; p.act = act; p.bpart = part + Cout * Cin * KK;
     p.Cin = (int)Cin; p.H = (int)H; p.Cout = (int)Cout; p.oh = (int)oh; p.ph = (int)ph;
     p.stages = pl.stages; p.sps = pl.sps; p.spi = (int)(oh / pl.R);
     p.div_spi = FastDiv((uint32_t)p.spi);
-    p.part_stride = Cout * Cin * KK;
+    p.part_stride = Cout * Cin * KK + (act ? Cout : 0);
     const dim3 grid((unsigned)(Cin / CT), (unsigned)(Cout / BM), (unsigned)pl.splits);
     const i64 blocks = (i64)grid.x * grid.y * grid.z;
     p.xcd_chunk = blocks % 8 == 0 && blocks <= 0x7fffffff ? (int)(blocks / 8) : 0;
     bool launched = false;
 #define FX_WGD2_LAUNCH(O, RR)                                                                                          \
     if (!launched && pl.OW == O && pl.R == RR) {                                                                       \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_s2_f64_kernel<O, RR>,                    \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_s2_f64_kernel<O, RR, false>,             \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
+        static const hipError_t attr_m = hipFuncSetAttribute((const void*)wgrad_s2_f64_kernel<O, RR, true>,            \
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
         FX_HIP_CHECK(attr);                                                                                            \
-        wgrad_s2_f64_kernel<O, RR><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                                         \
+        FX_HIP_CHECK(attr_m);                                                                                          \
+        if (act) wgrad_s2_f64_kernel<O, RR, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                          \
+        else wgrad_s2_f64_kernel<O, RR, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                             \
         launched = true;                                                                                               \
     }
     FX_WGD2_SHAPES(FX_WGD2_LAUNCH)
 #undef FX_WGD2_LAUNCH
     FX_REQUIRE(launched, "wgrad stride-2 patch kernel (f64): unexpected shape (%d, %d)", pl.OW, pl.R);
     FX_LAUNCH_CHECK();
-    const int n = (int)p.part_stride;
+    const int n = (int)(Cout * Cin * KK);
+    const wgd::ReduceTail tail{p.part_stride, act ? db : nullptr, act ? (int)Cout : 0};
     const FastDiv div_row((uint32_t)(KK * Cin)), div_cin((uint32_t)Cin);
-    // many partials of a small output: the grouped 16-byte sum (n and Cin are even here, part is 16-byte aligned)
+    // many partials of a small output: the grouped 16-byte sum (n, Cin and the stride are even here, part is 16-byte aligned)
     if (pl.splits >= 64 && n <= (1 << 18))
-        wgd::wgrad_f64_reduce_vec_kernel<16><<<dim3((unsigned)fx::ceil_div((i64)n, 32)), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin);
+        wgd::wgrad_f64_reduce_vec_kernel<16><<<dim3((unsigned)(fx::ceil_div((i64)n, 32) + wgd::tail_blocks(tail, 16))), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail);
     else
-        wgd::wgrad_f64_reduce_kernel<<<dim3((unsigned)fx::ceil_div((i64)n, 256)), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin);
+        wgd::wgrad_f64_reduce_kernel<<<dim3((unsigned)(fx::ceil_div((i64)n, 256) + wgd::tail_blocks(tail, 256))), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

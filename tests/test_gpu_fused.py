@@ -254,51 +254,59 @@ def test_conv_and_gemm_with_bias_epilogue_equal_two_call_sequence(ctx, dtype):
 
 # layers whose backward has the fused kernels: (B, Cin, H, W, Cout, stride, padding); the first group are image layers (weight
 # gradient only, as for a network's first layer), the second the stride-2 pair (weight and data gradient)
-CONV_BWD_RELU_CASES = [
-    (256, 3, 32, 32, 32, (1, 1), (1, 1)), (5, 1, 28, 28, 8, (1, 1), (1, 1)), (3, 3, 12, 16, 40, (1, 1), (1, 1)), (2, 2, 20, 8, 33, (2, 2), (1, 1)),
-    (256, 32, 32, 32, 64, (2, 2), (1, 1)), (3, 32, 32, 32, 32, (2, 2), (1, 1)), (2, 64, 64, 64, 128, (2, 2), (1, 1)), (2, 32, 16, 32, 96, (2, 2), (1, 1)),
-    (1, 96, 64, 64, 64, (2, 2), (1, 1)),
-]
+CONV_BWD_RELU_CASES = {
+    np.float32: [
+        (256, 3, 32, 32, 32, (1, 1), (1, 1)), (5, 1, 28, 28, 8, (1, 1), (1, 1)), (3, 3, 12, 16, 40, (1, 1), (1, 1)), (2, 2, 20, 8, 33, (2, 2), (1, 1)),
+        (256, 32, 32, 32, 64, (2, 2), (1, 1)), (3, 32, 32, 32, 32, (2, 2), (1, 1)), (2, 64, 64, 64, 128, (2, 2), (1, 1)), (2, 32, 16, 32, 96, (2, 2), (1, 1)),
+        (1, 96, 64, 64, 64, (2, 2), (1, 1))],
+    np.float64: [
+        (256, 3, 32, 32, 32, (1, 1), (1, 1)), (5, 1, 8, 32, 64, (1, 1), (1, 1)), (3, 2, 24, 32, 96, (1, 1), (1, 1)),
+        (256, 32, 32, 32, 64, (2, 2), (1, 1)), (3, 32, 32, 32, 64, (2, 2), (1, 1)), (2, 64, 64, 64, 128, (2, 2), (1, 1)), (2, 32, 16, 32, 64, (2, 2), (1, 1)),
+        (1, 96, 64, 64, 64, (2, 2), (1, 1))],
+}
 
 
-def test_conv_backward_from_the_unmasked_gradient(ctx):
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_conv_backward_from_the_unmasked_gradient(ctx, dtype):
     """fx_conv2d_wgrad_relu_bias / fx_conv2d_dgrad_relu: the ReLU mask applied while the kernels stage g.  dw and dx have the
-    bits of fx_relu_bwd followed by fx_conv2d_wgrad / fx_conv2d_dgrad; db agrees with the float64 sums of the masked gradient
+    bits of fx_relu_bwd followed by fx_conv2d_wgrad / fx_conv2d_dgrad; db agrees with the long double sums of the masked gradient
     to the stated tolerance; a second run gives the same bits; shapes without a fused kernel are refused."""
     import parity
     from ferrox_amd import capi
     rng = np.random.default_rng(91)
     served = 0
-    for (B, Cin, H, W, Cout, st, pd) in CONV_BWD_RELU_CASES:
+    for (B, Cin, H, W, Cout, st, pd) in CONV_BWD_RELU_CASES[dtype]:
         case = (B, Cin, H, W, Cout, st, pd)
         oh, ow = (H + 2 * pd[0] - 3) // st[0] + 1, (W + 2 * pd[1] - 3) // st[1] + 1
-        x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(np.float32)
-        w = (rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9))).astype(np.float32)
-        g = rng.standard_normal((B, Cout, oh, ow)).astype(np.float32)
-        act = np.maximum(rng.standard_normal((B, Cout, oh, ow)), 0).astype(np.float32)
+        x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(dtype)
+        w = (rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9))).astype(dtype)
+        g = rng.standard_normal((B, Cout, oh, ow)).astype(dtype)
+        act = np.maximum(rng.standard_normal((B, Cout, oh, ow)), 0).astype(dtype)
         dx_, dw_, dg_, da_ = ctx.upload(x), ctx.upload(w), ctx.upload(g), ctx.upload(act)
-        assert ctx.conv2d_bwd_relu_supported(capi.CONV_WGRAD, np.float32, x.shape, w.shape, st, pd), case
+        assert ctx.conv2d_bwd_relu_supported(capi.CONV_WGRAD, dtype, x.shape, w.shape, st, pd), case
         gm = ctx.relu_bwd(dg_, da_)
         want_dw = ctx.conv2d_wgrad(dx_, gm, w.shape, st, pd).numpy()
         dw, db = ctx.conv2d_wgrad_relu_bias(dx_, dg_, da_, w.shape, st, pd)
         assert np.array_equal(dw.numpy(), want_dw), ("dw", case)
-        masked = g.astype(np.float64) * (act > 0)
+        masked = g.astype(np.longdouble) * (act > 0)
         parity.check("conv bwd from unmasked g: bias grad", db.numpy(), masked.sum(axis=(0, 2, 3)), case=case,
-                     oracle=ctx.bias_grad(gm, B, Cout, oh * ow).numpy(), terms=np.abs(masked).sum(axis=(0, 2, 3)).max())
+                     oracle=ctx.bias_grad(gm, B, Cout, oh * ow).numpy(), terms=float(np.abs(masked).sum(axis=(0, 2, 3)).max()))
         dw2, db2 = ctx.conv2d_wgrad_relu_bias(dx_, dg_, da_, w.shape, st, pd)
         assert np.array_equal(dw2.numpy(), dw.numpy()) and np.array_equal(db2.numpy(), db.numpy()), ("rerun", case)
-        if ctx.conv2d_bwd_relu_supported(capi.CONV_DGRAD, np.float32, x.shape, w.shape, st, pd):
+        if ctx.conv2d_bwd_relu_supported(capi.CONV_DGRAD, dtype, x.shape, w.shape, st, pd):
             served += 1
             want_dx = ctx.conv2d_dgrad(gm, dw_, x.shape, st, pd).numpy()
             got_dx = ctx.conv2d_dgrad_relu(dg_, da_, dw_, x.shape, st, pd).numpy()
             assert np.array_equal(got_dx, want_dx), ("dx", case)
     assert served >= 4
-    # no fused kernel: a stride-1 layer over many channels, and f64
+    # no fused kernel: a stride-1 layer over many channels
     x_shape, w_shape = (2, 64, 16, 16), (64, 64, 3, 3)
-    assert not ctx.conv2d_bwd_relu_supported(capi.CONV_WGRAD, np.float32, x_shape, w_shape, (1, 1), (1, 1))
-    assert not ctx.conv2d_bwd_relu_supported(capi.CONV_WGRAD, np.float64, (256, 3, 32, 32), (32, 3, 3, 3), (1, 1), (1, 1))
-    z = ctx.fill(x_shape, 0.0)
-    zg = ctx.fill((2, 64, 16, 16), 0.0)
+    assert not ctx.conv2d_bwd_relu_supported(capi.CONV_WGRAD, dtype, x_shape, w_shape, (1, 1), (1, 1))
+    assert not ctx.conv2d_bwd_relu_supported(capi.CONV_DGRAD, dtype, x_shape, w_shape, (1, 1), (1, 1))
+    z = ctx.fill(x_shape, 0.0, dtype)
     with pytest.raises(capi.FerroxHipError) as e:
-        ctx.conv2d_wgrad_relu_bias(z, zg, zg, w_shape, (1, 1), (1, 1))
+        ctx.conv2d_wgrad_relu_bias(z, z, z, w_shape, (1, 1), (1, 1))
+    assert e.value.code == 4
+    with pytest.raises(capi.FerroxHipError) as e:
+        ctx.conv2d_dgrad_relu(z, z, ctx.fill(w_shape, 0.0, dtype), x_shape, (1, 1), (1, 1))
     assert e.value.code == 4
