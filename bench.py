@@ -383,6 +383,118 @@ def c5_step_flop(batch=256):
     return 2 * conv1 + 3 * conv2 + 3 * fc
 
 
+def train_step_roofline(name, batch, itemsize):
+    """Per-kernel algorithmic work of the fused training step of config C5 (the CNN) or C2 (the perceptron): (label, FLOP, HBM
+    bytes) for every launch group, each tensor counted once per kernel that must read or write it.  The time the step would take
+    with every kernel at its own roofline is the sum over kernels of max(FLOP / MFMA peak, bytes / HBM peak)."""
+    e = itemsize
+    if name == "C5_cnn":
+        a1 = batch * 32 * 32 * 32 * e      # conv1 activation [B,32,32,32]
+        a2 = batch * 64 * 16 * 16 * e      # conv2 activation [B,64,16,16]
+        x0 = batch * 3 * 32 * 32 * e
+        w1, w2, w3 = 32 * 27 * e, 64 * 288 * e, 10 * 16384 * e
+        f1, f2, f3 = 2.0 * 32 * 27 * batch * 1024, 2.0 * 64 * 288 * batch * 256, 2.0 * batch * 10 * 16384
+        nparam = 32 * 27 + 32 + 64 * 288 + 64 + 10 * 16384 + 10
+        return [
+            ("conv1 fwd + bias + relu", f1, x0 + w1 + a1),
+            ("conv2 fwd + bias + relu (stride 2)", f2, a1 + w2 + a2),
+            ("head fwd + bias", f3, a2 + w3),
+            ("softmax-CE loss + gradient", 0.0, 4 * batch * 10 * e),
+            ("head dX", f3, w3 + a2),
+            ("head dW + db", f3, a2 + w3),
+            ("conv2 dgrad, relu mask in staging", f2, 2 * a2 + w2 + a1),
+            ("conv2 wgrad + bias grad, relu mask in staging", f2, a1 + 2 * a2 + w2),
+            ("conv1 wgrad + bias grad, relu mask in staging", f1, 2 * a1 + x0 + w1),
+            ("Adam, all parameters in one launch", 0.0, 7 * nparam * e),
+        ]
+    if name == "C2_mlp":
+        dims = [(784, 256), (256, 128), (128, 10)]
+        rows = []
+        for li, (i, o) in enumerate(dims):
+            rows.append((f"fc{li + 1} fwd", 2.0 * batch * i * o, (batch * i + i * o + batch * o) * e))
+        rows.append(("softmax-CE loss + gradient", 0.0, 4 * batch * 10 * e))
+        for li, (i, o) in reversed(list(enumerate(dims))):
+            if li > 0:
+                rows.append((f"fc{li + 1} dX", 2.0 * batch * i * o, (batch * o + i * o + batch * i) * e))
+            rows.append((f"fc{li + 1} dW + db", 2.0 * batch * i * o, (batch * o + batch * i + i * o) * e))
+        nparam = sum(i * o + o for i, o in dims)
+        rows.append(("SGD, all parameters in one launch", 0.0, 3 * nparam * e))
+        return rows
+    return None
+
+
+def train_step_roofline_summary(name, dtype_name, step_ms, batch=256):
+    itemsize = 8 if dtype_name == "float64" else 4
+    rows = train_step_roofline(name, batch, itemsize)
+    if not rows:
+        return None
+    peak = (PEAK_F64_MFMA_TFLOPS if itemsize == 8 else PEAK_F32_MFMA_TFLOPS) * 1e12
+    t = [max(f / peak, b / (PEAK_HBM_GBS * 1e9)) for _, f, b in rows]
+    total = sum(t)
+    return {"bound": "mixed (per kernel: mfma or hbm, whichever is slower)", "time_at_roofline_ms": total * 1e3,
+            "measured_ms": step_ms, "frac": total * 1e3 / step_ms,
+            "algorithmic_flop": sum(f for _, f, _ in rows), "algorithmic_bytes": sum(b for _, _, b in rows),
+            "kernels": [{"kernel": lab, "flop": f, "bytes": b, "us_at_roofline": ti * 1e6, "bound": "mfma" if f / peak >= b / (PEAK_HBM_GBS * 1e9) else "hbm"}
+                        for (lab, f, b), ti in zip(rows, t)]}
+
+
+def bench_reference_microbench(ctx):
+    """The shapes of the reference's own kernel benchmark (kernels/benchmark.cu:21-25, 820-870): elementwise and activations on
+    2^26 elements, reductions over 2^20 elements (all, and the [1000, 1024, 1] axis view), a 1024^3 product and the
+    1 x 3 x 128 x 128 -> 32 convolution (forward, data gradient, weight gradient), f32 and f64."""
+    from ferrox_amd import capi
+    out = {}
+    n = 1 << 26
+    for dtype in (np.float32, np.float64):
+        sfx = capi.dtype_code(dtype)[1]
+        e = np.dtype(dtype).itemsize
+        a = ctx.uniform((n,), 41, -4.0, 4.0, dtype)
+        b = ctx.uniform((n,), 42, 0.5, 4.0, dtype)
+        o = ctx.empty((n,), dtype)
+        ew = {"add": (3, lambda: ctx.binary("add", a, b, out=o)), "mul": (3, lambda: ctx.binary("mul", a, b, out=o)),
+              "div": (3, lambda: ctx.binary("div", a, b, out=o)), "relu": (2, lambda: ctx.unary("relu", a, out=o)),
+              "sigmoid": (2, lambda: ctx.unary("sigmoid", a, out=o)), "tanh": (2, lambda: ctx.unary("tanh", a, out=o)),
+              "exp": (2, lambda: ctx.unary("exp", a, out=o)), "sqrt": (2, lambda: ctx.unary("sqrt", b, out=o))}
+        for name, (arrays, fn) in ew.items():
+            ms = time_stream(ctx, fn, 10, 2)
+            gbs = arrays * e * n / ms / 1e6
+            out[f"elementwise_2^26_{name}_{sfx}"] = {"us": ms * 1e3, "GBps": gbs, "frac_hbm": gbs / PEAK_HBM_GBS}
+        del a, b, o
+        nr = 1 << 20
+        r = ctx.normal((nr,), 43, 0.0, 1.0, dtype)
+        res = ctx.empty((1024,), dtype)
+        for kind in ("sum", "max", "min", "prod"):
+            for label, view in (("all", (1, nr, 1)), ("axis_1000x1024", (1000, 1024, 1))):
+                f = getattr(capi.lib, f"fx_reduce_{kind}_{sfx}")
+                if kind in ("max", "min"):
+                    fn = lambda f=f, view=view: capi.check(f(ctx.h, r.ptr, res.ptr, None, *view))  # noqa: E731
+                else:
+                    fn = lambda f=f, view=view: capi.check(f(ctx.h, r.ptr, res.ptr, *view))  # noqa: E731
+                ms = time_stream(ctx, fn, 20, 3)
+                nbytes = e * view[0] * view[1]
+                out[f"reduce_2^20_{kind}_{label}_{sfx}"] = {"us": ms * 1e3, "GBps": nbytes / ms / 1e6}
+        del r, res
+        M = 1024
+        ma, mb, mc = ctx.uniform((M, M), 44, -1.0, 1.0, dtype), ctx.uniform((M, M), 45, -1.0, 1.0, dtype), ctx.empty((M, M), dtype)
+        fn = lambda: capi.check(getattr(capi.lib, f"fx_gemm_{sfx}")(ctx.h, 0, 0, M, M, M, ma.ptr, mb.ptr, mc.ptr))  # noqa: E731
+        ms = time_stream(ctx, fn, 20, 3)
+        peak = PEAK_F32_MFMA_TFLOPS if dtype == np.float32 else PEAK_F64_MFMA_TFLOPS
+        out[f"matmul_1024_{sfx}"] = {"us": ms * 1e3, "tflops": 2.0 * M ** 3 / ms / 1e9, "frac_mfma": 2.0 * M ** 3 / ms / 1e9 / peak}
+        del ma, mb, mc
+        x = ctx.uniform((1, 3, 128, 128), 46, -1.0, 1.0, dtype)
+        w = ctx.normal((32, 3, 3, 3), 47, 0.0, 0.27, dtype)
+        g = ctx.normal((1, 32, 128, 128), 48, 0.0, 1.0, dtype)
+        y, dx, dw = ctx.empty(g.shape, dtype), ctx.empty(x.shape, dtype), ctx.empty(w.shape, dtype)
+        flop = 2.0 * 32 * 27 * 128 * 128
+        for name, fn in (("conv2d_forward", lambda: ctx.conv2d_fwd(x, w, (1, 1), (1, 1), out=y)),
+                         ("deconv2d", lambda: ctx.conv2d_dgrad(g, w, x.shape, (1, 1), (1, 1), 0, out=dx)),
+                         ("cross_correlation2d", lambda: ctx.conv2d_wgrad(x, g, w.shape, (1, 1), (1, 1), 0, out=dw))):
+            ms = time_stream(ctx, fn, 20, 3)
+            out[f"conv_1x3x128x128_to_32_{name}_{sfx}"] = {"us": ms * 1e3, "tflops": flop / ms / 1e9}
+        del x, w, g, y, dx, dw
+    return out
+
+
 def reference_pool_config():
     """PoolConfig::default() of the reference (src/backend/memory/mod.rs:50-82) with its allocation policy."""
     from ferrox_amd import capi
@@ -602,7 +714,10 @@ def main():
         "roofline": {"bound": "mfma", "kernel": CONV_KERNELS[dominant], "achieved": dom["tflops"],
                      "peak": PEAK_F32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": dom["tflops"] / PEAK_F32_MFMA_TFLOPS,
                      "traffic": traffic, "traffic_unit": "bytes per launch", "traffic_source": traffic_src,
-                     "algorithmic_bytes": 308.6e6, "avg_launch_ms": dom["ms"]},
+                     "algorithmic_bytes": 308.6e6, "avg_launch_ms": dom["ms"],
+                     # the other two metrics of the baseline: filled in below (slowest bandwidth kernel of config C4; the CNN
+                     # training step of config C5 against the sum of its kernels' rooflines)
+                     "others": {}},
         "conv_passes": {k: {"ms": v["ms"], "tflops": v["tflops"], "frac_mfma_f32": v["tflops"] / PEAK_F32_MFMA_TFLOPS}
                         for k, v in conv["per_pass"].items()},
         "conv_fwd_bias_relu": conv.get("fwd_bias_relu"),
@@ -619,10 +734,15 @@ def main():
                                  if "frac_hbm" in kv[1]], key=lambda kv: kv[1]["frac_hbm"])
         w_traffic, w_src = profile_traffic(C4_TRAFFIC_FILE, worst_name)
         w_ms = worst["us"] / 1e3 if "us" in worst else worst["ms"]
-        result["also"]["roofline_c4_worst"] = {
+        result["roofline"]["others"]["c4_worst"] = {
             "bound": "hbm", "kernel": worst_name, "achieved": worst["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
             "frac": worst["frac_hbm"], "traffic": w_traffic, "traffic_unit": "bytes per launch", "traffic_source": w_src,
             "algorithmic_bytes": worst["algorithmic_bytes"], "avg_launch_ms": w_ms}
+        # every C4 case in one compact table: name -> [microseconds per call, fraction of the HBM peak]
+        result["roofline"]["others"]["c4_cases_us_frac"] = {
+            k: [round(v["us"] if "us" in v else v["ms"] * 1e3, 1), round(v["frac_hbm"], 3)]
+            for k, v in list(result["also"]["reductions"].items()) + list(result["also"]["elementwise"].items()) if "frac_hbm" in v}
+        result["also"]["reference_microbench"] = bench_reference_microbench(ctx)
     ctx.close()
     if not args.skip_also and not args.skip_train:
         result["also"]["train_step"] = bench_train_steps(cpu=not args.skip_cpu)
@@ -636,10 +756,19 @@ def main():
         if c5:
             flop = c5_step_flop()
             tfl = flop / (c5["ms_per_step"] * 1e-3) / 1e12
-            result["also"]["roofline_c5_train_step"] = {
-                "bound": "mfma", "kernel": "C5 CNN train step, %s (all kernels of the step)" % c5_name, "achieved": tfl,
-                "peak": PEAK_F32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": tfl / PEAK_F32_MFMA_TFLOPS, "traffic": None,
-                "algorithmic_flop": flop, "avg_launch_ms": c5["ms_per_step"], "imgs_per_s": c5["imgs_per_s"]}
+            rf = train_step_roofline_summary("C5_cnn", "float32", c5["ms_per_step"])
+            rf.update({"kernel": "C5 CNN train step, %s (all kernels of the step)" % c5_name, "imgs_per_s": c5["imgs_per_s"],
+                       "mfma_only": {"achieved": tfl, "peak": PEAK_F32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": tfl / PEAK_F32_MFMA_TFLOPS},
+                       "traffic": None, "counters": "profiles/train_step_c5_f32_engine_fused_counters.txt"})
+            result["roofline"]["others"]["c5_train_step"] = rf
+        for key, cfg_name, dt in (("c5_train_step_f64", "C5_cnn", "float64"), ("c2_train_step", "C2_mlp", "float32")):
+            eng = result["also"]["train_step"].get(f"{cfg_name}_{dt}", {})
+            best = min((e for e in ("engine_fused", "engine_fused_graph") if e in eng), key=lambda e: eng[e]["ms_per_step"], default=None)
+            if best:
+                rf = train_step_roofline_summary(cfg_name, dt, eng[best]["ms_per_step"])
+                rf.pop("kernels")
+                rf.update({"kernel": f"{cfg_name} {dt} train step, {best}", "imgs_per_s": eng[best]["imgs_per_s"]})
+                result["roofline"]["others"][key] = rf
     if not args.skip_cpu:
         result["cpu_baseline"] = cpu_baseline_conv()
     print(json.dumps(result))

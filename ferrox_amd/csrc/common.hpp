@@ -60,6 +60,28 @@ int bind_device(int device);  // runtime.hip
         }                                                                                                   \
     } while (0)
 
+// Kernel launch, dynamic LDS and register-pinning statements go through these macros so that the same sources also build as
+// plain host C++ (FX_HOST_EMULATION, with a stand-in for <hip/hip_runtime.h>): a test harness then runs every thread of every
+// block of a launch on the CPU, with the tensors and the LDS between guard pages, and an access outside them faults there.
+#ifndef FX_HOST_EMULATION
+// FX_LAUNCH(grid, block, dynamic LDS bytes, stream, (arguments), kernel<template arguments>)
+#define FX_LAUNCH(grid, block, smem, stream, args, ...) __VA_ARGS__<<<(grid), (block), (smem), (stream)>>> args
+#define FX_DYNAMIC_SMEM(T, name) extern __shared__ __align__(16) T name[]
+// empty asm statements that make the compiler re-form a value at this point (vector / scalar register) instead of keeping
+// it alive, and that touch the accumulation registers
+#define FX_PIN_VGPR(a) asm volatile("" : "+v"(a))
+#define FX_PIN_VGPR2(a, b) asm volatile("" : "+v"(a), "+v"(b))
+#define FX_PIN_SGPR(a) asm volatile("" : "+s"(a))
+#define FX_TOUCH_AGPR(z) asm volatile("; accumulators in AGPRs %0" : "+a"(z))
+#else
+#define FX_LAUNCH(grid, block, smem, stream, args, ...) fxemu::launch((grid), (block), (size_t)(smem), [&] { __VA_ARGS__ args; })
+#define FX_DYNAMIC_SMEM(T, name) T* name = reinterpret_cast<T*>(fxemu::dynamic_smem())
+#define FX_PIN_VGPR(a) ((void)(a))
+#define FX_PIN_VGPR2(a, b) ((void)(a), (void)(b))
+#define FX_PIN_SGPR(a) ((void)(a))
+#define FX_TOUCH_AGPR(z) ((void)(z))
+#endif
+
 inline i64 ceil_div(i64 a, i64 b) { return (a + b - 1) / b; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -95,7 +95,7 @@ __global__ __launch_bounds__(256) void permute_weights_kernel(const T* __restric
 template <typename T>
 int permute_weights(fx_ctx* c, const T* w, T* out, const Dims& d, int mode) {
     const i64 nw = d.Cin * d.Cout * d.kh * d.kw;
-    permute_weights_kernel<T><<<dim3((unsigned)fx::ceil_div(nw, 256)), dim3(256), 0, c->stream>>>(w, out, (int)d.Cout, (int)d.Cin, (int)(d.kh * d.kw), mode);
+    FX_LAUNCH(dim3((unsigned)fx::ceil_div(nw, 256)), dim3(256), 0, c->stream, (w, out, (int)d.Cout, (int)d.Cin, (int)(d.kh * d.kw), mode), permute_weights_kernel<T>);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
@@ -308,8 +308,8 @@ int dgrad_classes_tile(fx_ctx* c, const T* g, const T* w, T* dx, T* wt, const Di
     i64 woff = 0, max_n = 0;
     auto flush = [&]() -> int {
         if (count == 0) return FX_OK;
-        permute_weights_class_kernel<T><<<dim3((unsigned)fx::ceil_div(max_n, 256), (unsigned)count), dim3(256), 0, c->stream>>>(
-            w, wt, (int)d.Cout, (int)d.Cin, (int)d.kh, (int)d.kw, (int)d.sh, (int)d.sw, cp);
+        FX_LAUNCH(dim3((unsigned)fx::ceil_div(max_n, 256), (unsigned)count), dim3(256), 0, c->stream, (
+            w, wt, (int)d.Cout, (int)d.Cin, (int)d.kh, (int)d.kw, (int)d.sh, (int)d.sw, cp), permute_weights_class_kernel<T>);
         FX_LAUNCH_CHECK();
         const int rc = igemm::launch_multi<T, Cfg>(c, mp, count);
         count = 0;
@@ -370,7 +370,7 @@ int dgrad_classes(fx_ctx* c, const T* g, const T* w, T* dx, T* wt, const Dims& d
 template <typename T>
 __global__ __launch_bounds__(256) void dgrad_small_cin_kernel(const T* __restrict__ g, const T* __restrict__ w, T* __restrict__ dx,
                                                               ConvShape s, int npix) {
-    extern __shared__ __align__(16) unsigned char smem_raw[];
+    FX_DYNAMIC_SMEM(unsigned char, smem_raw);
     T* wl = reinterpret_cast<T*>(smem_raw);
     const int KK = s.kh * s.kw;
     for (int i = threadIdx.x; i < KK * s.Cout * 4; i += 256) {
@@ -419,7 +419,7 @@ int dgrad_small_cin(fx_ctx* c, const T* g, const T* w, T* dx, const Dims& d) {
     const ConvShape s = make_shape(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
     const i64 npix = d.B * d.H * d.W;
     const size_t smem = (size_t)(d.kh * d.kw * d.Cout * 4) * sizeof(T);
-    dgrad_small_cin_kernel<T><<<dim3((unsigned)fx::ceil_div(npix, 256)), dim3(256), smem, c->stream>>>(g, w, dx, s, (int)npix);
+    FX_LAUNCH(dim3((unsigned)fx::ceil_div(npix, 256)), dim3(256), smem, c->stream, (g, w, dx, s, (int)npix), dgrad_small_cin_kernel<T>);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

@@ -154,8 +154,8 @@ inline int run(fx_ctx* c, const double* x, const double* w, double* y, i64 B, i6
     p.div_nmt = FastDiv((uint32_t)p.nmt);
     p.div_tpi = FastDiv((uint32_t)p.tpi);
     const dim3 grid((unsigned)(B * p.tpi * p.nmt));
-    if (bias) image_fwd_f64_kernel<32, true><<<grid, dim3(NT), 0, c->stream>>>(p);
-    else image_fwd_f64_kernel<32, false><<<grid, dim3(NT), 0, c->stream>>>(p);
+    if (bias) FX_LAUNCH(grid, dim3(NT), 0, c->stream, (p), image_fwd_f64_kernel<32, true>);
+    else FX_LAUNCH(grid, dim3(NT), 0, c->stream, (p), image_fwd_f64_kernel<32, false>);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
@@ -188,7 +188,7 @@ template <bool MASK>
 __global__ __launch_bounds__(NT) void image_wgrad_f64_kernel(const WParams p) {
     using S = Shape<32>;
     constexpr int W = 32, TR = S::TR, PR = S::PR, PW = S::PW, PLANE = S::PLANE;
-    extern __shared__ __align__(16) double smem_w[];
+    FX_DYNAMIC_SMEM(double, smem_w);
     double* Gs = smem_w;                   // [32 oc][GPITCH]
     double* Xs = smem_w + 32 * GPITCH;     // [CP planes][PR][PW], odd plane pitch
     const int tid = threadIdx.x, lane = tid & 63, kq = lane >> 4, l16 = lane & 15;
@@ -346,8 +346,8 @@ inline int run_wgrad(fx_ctx* c, const WPlan& pl, const double* x, const double* 
     FX_HIP_CHECK(attr);
     FX_HIP_CHECK(attr_m);
     const dim3 grid((unsigned)pl.splits, (unsigned)(Cout / 32));
-    if (act) image_wgrad_f64_kernel<true><<<grid, dim3(NT), lds, c->stream>>>(p);
-    else image_wgrad_f64_kernel<false><<<grid, dim3(NT), lds, c->stream>>>(p);
+    if (act) FX_LAUNCH(grid, dim3(NT), lds, c->stream, (p), image_wgrad_f64_kernel<true>);
+    else FX_LAUNCH(grid, dim3(NT), lds, c->stream, (p), image_wgrad_f64_kernel<false>);
     FX_LAUNCH_CHECK();
     if (act) return igemm::launch_splitk_reduce_pair<double>(c, part, p.part_stride, pl.splits, dw, Cout * Cin * KK, db, Cout);
     return igemm::launch_splitk_reduce<double>(c, part, dw, Cout * Cin * KK, pl.splits);

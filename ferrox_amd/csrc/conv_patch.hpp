@@ -83,7 +83,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
     constexpr int BM = 32 * WM, WN = 4 / WM, NPIX = 32 * TN * WN;
     constexpr int WIMG = BM * WPITCH;             // floats in one weight image
     constexpr int NW = (WIMG / 4 + NT - 1) / NT;  // float4 of the image per thread (the last one only partly used)
-    extern __shared__ __align__(16) float smem[];
+    FX_DYNAMIC_SMEM(float, smem);
     float* Ws = smem;
     float* Xs = smem + WIMG;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
     };
     auto park = [&]() {
         int xd = x_dst0, wd = tid;
-        asm volatile("" : "+v"(xd), "+v"(wd));  // recompute the addresses here instead of keeping them alive
+        FX_PIN_VGPR2(xd, wd);  // recompute the addresses here instead of keeping them alive
 #pragma unroll
         for (int u = 0; u < NW; ++u) {
             const int idx = wd + u * NT;
@@ -184,7 +184,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
         float a0, b0[TN], a1, b1[TN];
         const float* xrow[3] = {Xs, Xs + p.PW, Xs + 2 * p.PW};
 #pragma unroll
-        for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(boff[j]));  // form the 12 x TN read addresses per stage, not once
+        for (int j = 0; j < TN; ++j) FX_PIN_VGPR(boff[j]);  // form the 12 x TN read addresses per stage, not once
         auto rd = [&](float& a, float (&bv)[TN], int step) {
             const int t = step >> 2, cp = step & 3, ky = t / 3, kx = t % 3;
             a = wa[t * CC + 2 * cp];
@@ -303,7 +303,7 @@ template <int WM, int TN, bool BIAS>
 __global__ __launch_bounds__(NT, 2) void conv_patch_persist_kernel(const Params p) {
     constexpr int BM = 32 * WM, WN = 4 / WM, NPIX = 32 * TN * WN, NXP = NXP_PERSIST;
     constexpr int AIMG = KK * 64 * 4;  // floats of one (32-row block, chunk) weight image
-    extern __shared__ __align__(16) float smem[];
+    FX_DYNAMIC_SMEM(float, smem);
     const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
     // in a scalar register: what derives from the wave index (rows, pointers, tests) stays on the scalar unit
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -381,7 +381,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_persist_kernel(const Params 
     };
     auto park = [&](int buf) __attribute__((always_inline)) {
         int xd = x_dst0 + buf * PBUF;
-        asm volatile("" : "+v"(xd));
+        FX_PIN_VGPR(xd);
         if (x_lane) {
 #pragma unroll
             for (int u = 0; u < NXP; ++u) {
@@ -402,7 +402,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_persist_kernel(const Params 
 #pragma unroll
         for (int ky = 0; ky < 3; ++ky)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(boff[ky][j]));
+            for (int j = 0; j < TN; ++j) FX_PIN_VGPR(boff[ky][j]);
         auto rd = [&](float (&bv)[TN], int step) __attribute__((always_inline)) {
             const int t = step >> 2, cp = step & 3, ky = t / 3, kx = t % 3;
             const int imm = (SET * PBUF + 2 * cp * PPLANE + kx) * 4;
@@ -460,7 +460,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_persist_kernel(const Params 
                                 if (p.relu) v = v > 0.f ? v : 0.f;
                             }
                             float* rowp = out + (i64)ru * p.L;
-                            asm volatile("" : "+s"(rowp));  // keeps the row base apart from the lane offset: scalar base + 32-bit offset
+                            FX_PIN_SGPR(rowp);  // keeps the row base apart from the lane offset: scalar base + 32-bit offset
                             *(gfloat*)((gchar*)rowp + lo) = v;
                         }
                     }
@@ -672,7 +672,7 @@ inline int launch_persist(fx_ctx* c, const Plan& pl, const float* x, const float
                           i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw, const float* bias, int relu) {
     const i64 mblocks = (i64)pl.mtiles * pl.WM;
     const i64 n = mblocks * pl.nchunks * KK * 64 * 4;
-    wimg2_kernel<<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(w, wimg, (int)Cout, (int)Cin, (int)M, pl.nchunks, flip, n);
+    FX_LAUNCH(dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream, (w, wimg, (int)Cout, (int)Cin, (int)M, pl.nchunks, flip, n), wimg2_kernel);
     FX_LAUNCH_CHECK();
     Params p;
     p.x = x; p.wimg = wimg; p.y = y; p.bias = bias; p.relu = relu;
@@ -701,8 +701,8 @@ inline int launch_persist(fx_ctx* c, const Plan& pl, const float* x, const float
                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)PP_LDS); \
         FX_HIP_CHECK(attr0);                                                                                          \
         FX_HIP_CHECK(attr1);                                                                                          \
-        if (bias) conv_patch_persist_kernel<WMV, TNV, true><<<grid, dim3(NT), PP_LDS, c->stream>>>(p);                  \
-        else conv_patch_persist_kernel<WMV, TNV, false><<<grid, dim3(NT), PP_LDS, c->stream>>>(p);                      \
+        if (bias) FX_LAUNCH(grid, dim3(NT), PP_LDS, c->stream, (p), conv_patch_persist_kernel<WMV, TNV, true>);                  \
+        else FX_LAUNCH(grid, dim3(NT), PP_LDS, c->stream, (p), conv_patch_persist_kernel<WMV, TNV, false>);                      \
     } break;
     switch (pl.WM * 16 + pl.TN) {
         FX_CPK_PERSIST(4, 5)
@@ -721,8 +721,8 @@ inline int launch_plan(fx_ctx* c, const Plan& pl, const float* x, const float* w
                        i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw, const float* bias, int relu) {
     if (pl.persist) return launch_persist(c, pl, x, w, y, wimg, flip, Cout, Cin, B, C, H, W, M, OH, OW, sh, sw, ph, pw, bias, relu);
     const i64 n = (i64)pl.mtiles * pl.nchunks * pl.wimg();
-    wimg_kernel<<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(w, wimg, (int)Cout, (int)Cin, (int)M, pl.bm(),
-                                                                                  pl.nchunks, flip, n);
+    FX_LAUNCH(dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream, (w, wimg, (int)Cout, (int)Cin, (int)M, pl.bm(),
+                                                                                  pl.nchunks, flip, n), wimg_kernel);
     FX_LAUNCH_CHECK();
     Params p;
     p.x = x; p.wimg = wimg; p.y = y; p.bias = bias; p.relu = relu;
@@ -746,8 +746,8 @@ inline int launch_plan(fx_ctx* c, const Plan& pl, const float* x, const float* w
                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
         FX_HIP_CHECK(attr0);                                                                                          \
         FX_HIP_CHECK(attr1);                                                                                          \
-        if (bias) conv_patch_kernel<WMV, TNV, true, NXP_TALL, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);       \
-        else conv_patch_kernel<WMV, TNV, false, NXP_TALL, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);           \
+        if (bias) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), conv_patch_kernel<WMV, TNV, true, NXP_TALL, true>);       \
+        else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), conv_patch_kernel<WMV, TNV, false, NXP_TALL, true>);           \
     }
         if (pl.WM == 4) FX_CPK_LAUNCH_MULTI(4, 4) else FX_CPK_LAUNCH_MULTI(2, 2)
 #undef FX_CPK_LAUNCH_MULTI
@@ -762,8 +762,8 @@ inline int launch_plan(fx_ctx* c, const Plan& pl, const float* x, const float* w
                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
         FX_HIP_CHECK(attr0);                                                                                          \
         FX_HIP_CHECK(attr1);                                                                                          \
-        if (bias) conv_patch_kernel<WMV, TNV, true, NXPV><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                 \
-        else conv_patch_kernel<WMV, TNV, false, NXPV><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                     \
+        if (bias) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), conv_patch_kernel<WMV, TNV, true, NXPV>);                 \
+        else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), conv_patch_kernel<WMV, TNV, false, NXPV>);                     \
     }
 #define FX_CPK_LAUNCH(WMV, TNV)                                                                                       \
     case WMV * 16 + TNV:                                                                                              \

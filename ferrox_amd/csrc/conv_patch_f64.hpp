@@ -77,7 +77,7 @@ __device__ __forceinline__ double2 ldg2(const double* base, uint32_t byteoff) {
 template <int TN, bool BIAS>
 __global__ __launch_bounds__(NT, 2) void conv_patch_f64_kernel(const Params p) {
     constexpr int BM = 64, NPIX = 16 * TN;
-    extern __shared__ __align__(16) double smem[];
+    FX_DYNAMIC_SMEM(double, smem);
     const int tid = threadIdx.x, lane = tid & 63, kq = lane >> 4, l16 = lane & 15;
     // in a scalar register: what derives from the wave index (rows, pointers, tests) stays on the scalar unit
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_f64_kernel(const Params p) {
     };
     auto park = [&](int buf) __attribute__((always_inline)) {
         int xd = x_dst0 + buf * PBUF;
-        asm volatile("" : "+v"(xd));
+        FX_PIN_VGPR(xd);
         if (x_lane) {
 #pragma unroll
             for (int u = 0; u < NXP; ++u) {
@@ -169,7 +169,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_f64_kernel(const Params p) {
 #pragma unroll
         for (int ky = 0; ky < 3; ++ky)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(boff[ky][j]));
+            for (int j = 0; j < TN; ++j) FX_PIN_VGPR(boff[ky][j]);
         auto rd = [&](double (&bv)[TN], int step) __attribute__((always_inline)) {
             const int t = step >> 1, cp = step & 1, ky = t / 3, kx = t % 3;
             const int imm = (SET * PBUF + 4 * cp * PPLANE + kx) * 8;
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_f64_kernel(const Params p) {
                                 if (p.relu) v = v > 0. ? v : 0.;
                             }
                             double* rowp = out + (i64)(4 * e) * p.L;
-                            asm volatile("" : "+s"(rowp));  // keeps the row base apart from the lane offset: scalar base + 32-bit offset
+                            FX_PIN_SGPR(rowp);  // keeps the row base apart from the lane offset: scalar base + 32-bit offset
                             *(gdouble*)((gchar*)rowp + lo) = v;
                         }
                     }
@@ -331,7 +331,7 @@ inline i64 workspace_bytes(const Plan& pl) { return (i64)pl.mtiles * 4 * pl.nchu
 inline int run(fx_ctx* c, const Plan& pl, const double* x, const double* w, double* y, double* wimg, int flip, i64 Cout, i64 Cin, i64 B, i64 C,
                i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph, i64 pw, const double* bias = nullptr, int relu = 0) {
     const i64 n = (i64)pl.mtiles * 4 * pl.nchunks * AIMG;
-    wimg_kernel<<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(w, wimg, (int)Cout, (int)Cin, (int)M, pl.nchunks, flip, n);
+    FX_LAUNCH(dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream, (w, wimg, (int)Cout, (int)Cin, (int)M, pl.nchunks, flip, n), wimg_kernel);
     FX_LAUNCH_CHECK();
     Params p;
     p.x = x; p.wimg = wimg; p.y = y; p.bias = bias; p.relu = relu;
@@ -358,8 +358,8 @@ inline int run(fx_ctx* c, const Plan& pl, const double* x, const double* w, doub
                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES); \
         FX_HIP_CHECK(attr0);                                                                                           \
         FX_HIP_CHECK(attr1);                                                                                           \
-        if (bias) conv_patch_f64_kernel<TNV, true><<<grid, dim3(NT), LDS_BYTES, c->stream>>>(p);                       \
-        else conv_patch_f64_kernel<TNV, false><<<grid, dim3(NT), LDS_BYTES, c->stream>>>(p);                           \
+        if (bias) FX_LAUNCH(grid, dim3(NT), LDS_BYTES, c->stream, (p), conv_patch_f64_kernel<TNV, true>);                       \
+        else FX_LAUNCH(grid, dim3(NT), LDS_BYTES, c->stream, (p), conv_patch_f64_kernel<TNV, false>);                           \
     } break;
     switch (pl.TN) {
         FX_CPD_LAUNCH(8)

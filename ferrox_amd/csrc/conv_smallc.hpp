@@ -81,7 +81,7 @@ __device__ __forceinline__ int tap_offset(const Geometry& g, int k) {
 constexpr int NPV = 4;
 template <int KS, bool BIAS>
 __global__ __launch_bounds__(NT) void fwd_kernel(const FwdParams p) {
-    extern __shared__ __align__(16) float patch[];
+    FX_DYNAMIC_SMEM(float, patch);
     const Geometry& g = p.g;
     const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -192,7 +192,7 @@ __global__ __launch_bounds__(NT) void fwd_kernel(const FwdParams p) {
 // there the MFMA leaves sum over pixels of the masked g in it: the bias gradient, at no extra instruction.
 template <bool MASK>
 __global__ __launch_bounds__(NT, 2) void wgrad_kernel(const WgradParams p) {
-    extern __shared__ __align__(16) float smem[];
+    FX_DYNAMIC_SMEM(float, smem);
     const Geometry& g = p.q;
     float* Gs = smem;                 // [32][GP]
     float* patch = smem + 32 * GP;    // [C][PR][PW]
@@ -325,8 +325,8 @@ inline int run_fwd(fx_ctx* c, const Plan& pl, const float* x, const float* w, fl
     const dim3 grid((unsigned)fx::ceil_div((i64)p.ntiles, per_block), (unsigned)mblocks);
 #define FX_CSC_FWD(KSV)                                                                                 \
     do {                                                                                                \
-        if (bias) fwd_kernel<KSV, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                     \
-        else fwd_kernel<KSV, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                         \
+        if (bias) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), fwd_kernel<KSV, true>);                     \
+        else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), fwd_kernel<KSV, false>);                         \
     } while (0)
     switch ((int)C) {
         case 1: FX_CSC_FWD(5); break;
@@ -351,8 +351,8 @@ inline int run_wgrad(fx_ctx* c, const Plan& pl, const float* x, const float* g, 
     p.stages = pl.stages; p.sps = pl.sps; p.part_stride = n + (act ? Cout : 0);
     p.q = make_geometry(pl, C, H, W, Cout, OH, OW, sh, sw, ph, pw);
     const dim3 grid((unsigned)pl.splits, (unsigned)fx::ceil_div(Cout, (i64)32));
-    if (act) wgrad_kernel<true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);
-    else wgrad_kernel<false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);
+    if (act) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), wgrad_kernel<true>);
+    else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), wgrad_kernel<false>);
     FX_LAUNCH_CHECK();
     if (pl.splits > 1) {
         if (act) return igemm::launch_splitk_reduce_pair<float>(c, part, p.part_stride, pl.splits, dw, n, db, Cout);

@@ -57,7 +57,7 @@ template <int OW, int OCC, bool MASK>
 __global__ __launch_bounds__(NT, 1) void dgrad_s2_kernel(const Params p) {
     using S = Shape<OW, OCC>;
     constexpr int TR = S::TR, PC = S::PC, GPL = S::GPL, KS = S::KS, WCH = S::WCH, BUF = S::BUF;
-    extern __shared__ __align__(16) float smem[];
+    FX_DYNAMIC_SMEM(float, smem);
     const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int bt = (int)p.div_nct.div(blockIdx.x), ct = (int)blockIdx.x - bt * p.nct;
@@ -251,8 +251,8 @@ inline int run(fx_ctx* c, const Plan& pl, const float* g, const float* w, float*
                                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
         FX_HIP_CHECK(attr);                                                                                            \
         FX_HIP_CHECK(attr_m);                                                                                          \
-        if (act) dgrad_s2_kernel<O, C_, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                              \
-        else dgrad_s2_kernel<O, C_, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                                 \
+        if (act) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), dgrad_s2_kernel<O, C_, true>);                              \
+        else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), dgrad_s2_kernel<O, C_, false>);                                 \
         launched = true;                                                                                               \
     }
     FX_DG2_SHAPES(FX_DG2_LAUNCH)

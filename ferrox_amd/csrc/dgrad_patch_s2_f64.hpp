@@ -64,7 +64,7 @@ template <int OW, int OCC, bool MASK>
 __global__ __launch_bounds__(NT, 1) void dgrad_s2_f64_kernel(const Params p) {
     using S = Shape<OW, OCC>;
     constexpr int TR = S::TR, PC = S::PC, GPL = S::GPL, KS = S::KS, WCH = S::WCH, BUF = S::BUF;
-    extern __shared__ __align__(16) double smem_d[];
+    FX_DYNAMIC_SMEM(double, smem_d);
     double* smem = smem_d;
     const int tid = threadIdx.x, lane = tid & 63, kq = lane >> 4, l16 = lane & 15;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -274,8 +274,8 @@ inline int run(fx_ctx* c, const Plan& pl, const double* g, const double* w, doub
                                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
         FX_HIP_CHECK(attr);                                                                                            \
         FX_HIP_CHECK(attr_m);                                                                                          \
-        if (act) dgrad_s2_f64_kernel<O, C_, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                          \
-        else dgrad_s2_f64_kernel<O, C_, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                             \
+        if (act) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), dgrad_s2_f64_kernel<O, C_, true>);                          \
+        else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), dgrad_s2_f64_kernel<O, C_, false>);                             \
         launched = true;                                                                                               \
     }
     FX_DGD2_SHAPES(FX_DGD2_LAUNCH)

@@ -57,7 +57,7 @@ template <int OW, int MB, bool BIAS>
 __global__ __launch_bounds__(NT, 1) void fwd_s2_kernel(const Params p) {
     using S = Shape<OW, MB>;
     constexpr int TR = S::TR, PR = S::PR, W = S::W, RP = S::RP, PLANE = S::PLANE, WCH = S::WCH, BUF = S::BUF, HALF = S::HALF;
-    extern __shared__ __align__(16) float smem[];
+    FX_DYNAMIC_SMEM(float, smem);
     const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int bt = (int)p.div_nmt.div(blockIdx.x), mt = (int)blockIdx.x - bt * p.nmt;
@@ -241,8 +241,8 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* w, float*
                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
         FX_HIP_CHECK(attr0);                                                                                           \
         FX_HIP_CHECK(attr1);                                                                                           \
-        if (bias) fwd_s2_kernel<O, M_, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                               \
-        else fwd_s2_kernel<O, M_, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                                   \
+        if (bias) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), fwd_s2_kernel<O, M_, true>);                               \
+        else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), fwd_s2_kernel<O, M_, false>);                                   \
         launched = true;                                                                                               \
     }
     FX_FW2_SHAPES(FX_FW2_LAUNCH)

@@ -62,7 +62,7 @@ template <int OW, int MB, bool BIAS>
 __global__ __launch_bounds__(NT, 1) void fwd_s2_f64_kernel(const Params p) {
     using S = Shape<OW, MB>;
     constexpr int TR = S::TR, PR = S::PR, W = S::W, RP = S::RP, PLANE = S::PLANE, WCH = S::WCH, BUF = S::BUF, HALF = S::HALF, NB = S::NB;
-    extern __shared__ __align__(16) double smem_fwd2[];
+    FX_DYNAMIC_SMEM(double, smem_fwd2);
     double* smem = smem_fwd2;
     const int tid = threadIdx.x, lane = tid & 63, kq = lane >> 4, l16 = lane & 15;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -248,8 +248,8 @@ inline int run(fx_ctx* c, const Plan& pl, const double* x, const double* w, doub
                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
         FX_HIP_CHECK(attr0);                                                                                           \
         FX_HIP_CHECK(attr1);                                                                                           \
-        if (bias) fwd_s2_f64_kernel<O, M_, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                           \
-        else fwd_s2_f64_kernel<O, M_, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                               \
+        if (bias) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), fwd_s2_f64_kernel<O, M_, true>);                           \
+        else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), fwd_s2_f64_kernel<O, M_, false>);                               \
         launched = true;                                                                                               \
     }
     FX_FWD2_SHAPES(FX_FWD2_LAUNCH)

@@ -626,8 +626,8 @@ int launch(fx_ctx* c, const AL& al, const BL& bl, const EP& ep, i64 M, i64 N, i6
     const i64 gx = fx::ceil_div(N, Cfg::BN), gy = fx::ceil_div(M, Cfg::BM);
     FX_REQUIRE(gx <= 0x7fffffff && gy <= 65535 && splits >= 1 && splits <= 65535, "implicit GEMM grid out of range");
     FX_REQUIRE(K >= 1, "implicit GEMM needs K >= 1");
-    igemm_kernel<T, Cfg, AL, BL, EP><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)splits), dim3(Cfg::NT), 0, c->stream>>>(
-        al, bl, ep, (int)K, kps);
+    FX_LAUNCH(dim3((unsigned)gx, (unsigned)gy, (unsigned)splits), dim3(Cfg::NT), 0, c->stream, (
+        al, bl, ep, (int)K, kps), igemm_kernel<T, Cfg, AL, BL, EP>);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
@@ -641,7 +641,7 @@ int launch_multi(fx_ctx* c, const MultiProblem<AL, BL, EP, NP>& mp, int count) {
         gy = std::max(gy, mp.tiles_m[z]);
     }
     FX_REQUIRE(count >= 1 && count <= NP && gx >= 1 && gy >= 1 && gy <= 65535, "implicit GEMM grid out of range");
-    igemm_multi_kernel<T, Cfg, AL, BL, EP, NP><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)count), dim3(Cfg::NT), 0, c->stream>>>(mp);
+    FX_LAUNCH(dim3((unsigned)gx, (unsigned)gy, (unsigned)count), dim3(Cfg::NT), 0, c->stream, (mp), igemm_multi_kernel<T, Cfg, AL, BL, EP, NP>);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
@@ -687,11 +687,11 @@ int launch_splitk_reduce(fx_ctx* c, const T* part, T* out, i64 n, int splits, co
         ep.bias = bias; ep.ncols = (int)ncols; ep.relu = relu; ep.div_cols = FastDiv((uint32_t)ncols);
     }
     if (splits >= 128 && n <= (1 << 16))
-        splitk_reduce_grouped_kernel<T, 16><<<dim3((unsigned)fx::ceil_div(n, 16)), dim3(256), 0, c->stream>>>(part, out, n, splits, ep);
+        FX_LAUNCH(dim3((unsigned)fx::ceil_div(n, 16)), dim3(256), 0, c->stream, (part, out, n, splits, ep), splitk_reduce_grouped_kernel<T, 16>);
     else if (splits >= 32 && n <= (1 << 18))
-        splitk_reduce_grouped_kernel<T, 4><<<dim3((unsigned)fx::ceil_div(n, 64)), dim3(256), 0, c->stream>>>(part, out, n, splits, ep);
+        FX_LAUNCH(dim3((unsigned)fx::ceil_div(n, 64)), dim3(256), 0, c->stream, (part, out, n, splits, ep), splitk_reduce_grouped_kernel<T, 4>);
     else
-        splitk_reduce_kernel<T><<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(part, out, n, splits, ep);
+        FX_LAUNCH(dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream, (part, out, n, splits, ep), splitk_reduce_kernel<T>);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
@@ -739,11 +739,11 @@ int launch_splitk_reduce_pair(fx_ctx* c, const T* part, i64 stride, int splits, 
     const i64 n = n1 + n2;
     FX_REQUIRE(stride >= n && n <= 0x7fffffffll, "split-K pair sum: bad sizes");
     if (splits >= 128 && n1 <= (1 << 16))
-        splitk_reduce_pair_kernel<T, 16><<<dim3((unsigned)fx::ceil_div(n, (i64)16)), dim3(256), 0, c->stream>>>(part, stride, splits, out1, n1, out2, n2);
+        FX_LAUNCH(dim3((unsigned)fx::ceil_div(n, (i64)16)), dim3(256), 0, c->stream, (part, stride, splits, out1, n1, out2, n2), splitk_reduce_pair_kernel<T, 16>);
     else if (splits >= 32 && n1 <= (1 << 18))
-        splitk_reduce_pair_kernel<T, 4><<<dim3((unsigned)fx::ceil_div(n, (i64)64)), dim3(256), 0, c->stream>>>(part, stride, splits, out1, n1, out2, n2);
+        FX_LAUNCH(dim3((unsigned)fx::ceil_div(n, (i64)64)), dim3(256), 0, c->stream, (part, stride, splits, out1, n1, out2, n2), splitk_reduce_pair_kernel<T, 4>);
     else
-        splitk_reduce_pair_kernel<T, 1><<<dim3((unsigned)fx::ceil_div(n, (i64)256)), dim3(256), 0, c->stream>>>(part, stride, splits, out1, n1, out2, n2);
+        FX_LAUNCH(dim3((unsigned)fx::ceil_div(n, (i64)256)), dim3(256), 0, c->stream, (part, stride, splits, out1, n1, out2, n2), splitk_reduce_pair_kernel<T, 1>);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
@@ -756,7 +756,7 @@ __global__ __launch_bounds__(256) void zero_kernel(T* __restrict__ out, i64 n) {
 template <typename T>
 int launch_zero(fx_ctx* c, T* out, i64 n) {
     if (n == 0) return FX_OK;
-    zero_kernel<T><<<dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream>>>(out, n);
+    FX_LAUNCH(dim3((unsigned)fx::ceil_div(n, 256)), dim3(256), 0, c->stream, (out, n), zero_kernel<T>);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

@@ -63,7 +63,7 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
     constexpr int NG = BM / RPP, NXC = CT / RPP;
     constexpr int NXN = 5;  // NARROW: passes of 64 (channel, row) pairs; 32 channels x at most 10 rows
     constexpr int NX = NARROW ? NXN : NXC * XR;
-    extern __shared__ __align__(16) float smem[];
+    FX_DYNAMIC_SMEM(float, smem);
     float* Gs = smem;
     float* Xs = smem + BM * p.GP;
     const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
@@ -150,7 +150,7 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
     };
     auto park = [&]() {
         int gd = g_dst0, xd = x_dst0;
-        asm volatile("" : "+v"(gd), "+v"(xd));  // recompute the row addresses here instead of keeping 14 of them alive
+        FX_PIN_VGPR2(gd, xd);  // recompute the row addresses here instead of keeping 14 of them alive
         if (g_lane) {
 #pragma unroll
             for (int u = 0; u < NG; ++u) {
@@ -572,7 +572,7 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
         static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_patch_kernel<XRV, A, B_, C_>,           \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
         FX_HIP_CHECK(attr);                                                                                           \
-        wgrad_patch_kernel<XRV, A, B_, C_><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                                \
+        FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), wgrad_patch_kernel<XRV, A, B_, C_>);                                \
     } while (0)
     const int layout = pl.WMO * 100 + pl.WC * 10 + pl.WK;
     // pixel pairs of a wave's row segment when the unrolled pixel loop applies (unit column stride), else 0
@@ -582,14 +582,14 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
         static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_patch_kernel<XRV, A, B_, C_, false, PV>, \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
         FX_HIP_CHECK(attr);                                                                                           \
-        wgrad_patch_kernel<XRV, A, B_, C_, false, PV><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                     \
+        FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), wgrad_patch_kernel<XRV, A, B_, C_, false, PV>);                     \
     } while (0)
 #define FX_WGP_LAUNCH_NARROW(A, C_)                                                                                   \
     do {                                                                                                              \
         static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_patch_kernel<0, A, 1, C_, true>,        \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
         FX_HIP_CHECK(attr);                                                                                           \
-        wgrad_patch_kernel<0, A, 1, C_, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                             \
+        FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), wgrad_patch_kernel<0, A, 1, C_, true>);                             \
     } while (0)
     if (pl.narrow && layout == 411) FX_WGP_LAUNCH_NARROW(4, 1);
     else if (pl.narrow && layout == 212) FX_WGP_LAUNCH_NARROW(2, 2);
@@ -619,11 +619,11 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
     // measured: the 16-byte grouped sum beats both kernels below wherever it applies (0.4845 -> 0.4786 ms for the whole pass at
     // [128,64,56,56] -> 128 with 256 partials, 0.1996 -> 0.188 ms at [256,64,32,32] -> 64)
     if (n % 4 == 0 && Cin % 4 == 0 && fx::aligned16(part)) {
-        wgrad_patch_reduce_vec_kernel<16><<<dim3((unsigned)fx::ceil_div((i64)n, 64)), dim3(256), 0, c->stream>>>(part, dw, n, pl.partials(), (int)Cin, div_row, div_cin);
+        FX_LAUNCH(dim3((unsigned)fx::ceil_div((i64)n, 64)), dim3(256), 0, c->stream, (part, dw, n, pl.partials(), (int)Cin, div_row, div_cin), wgrad_patch_reduce_vec_kernel<16>);
     } else if (pl.partials() >= 512 && n <= (1 << 17))
-        wgrad_patch_reduce_grouped_kernel<16><<<dim3((unsigned)fx::ceil_div((i64)n, 16)), dim3(256), 0, c->stream>>>(part, dw, n, pl.partials(), (int)Cin, div_row, div_cin);
+        FX_LAUNCH(dim3((unsigned)fx::ceil_div((i64)n, 16)), dim3(256), 0, c->stream, (part, dw, n, pl.partials(), (int)Cin, div_row, div_cin), wgrad_patch_reduce_grouped_kernel<16>);
     else
-        wgrad_patch_reduce_kernel<<<dim3((unsigned)fx::ceil_div((i64)n, 256)), dim3(256), 0, c->stream>>>(part, dw, n, pl.partials(), (int)Cin, div_row, div_cin);
+        FX_LAUNCH(dim3((unsigned)fx::ceil_div((i64)n, 256)), dim3(256), 0, c->stream, (part, dw, n, pl.partials(), (int)Cin, div_row, div_cin), wgrad_patch_reduce_kernel);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

@@ -51,7 +51,7 @@ __device__ __forceinline__ double2 ldg2(const double* base, uint32_t byteoff) {
 template <int NK>
 __global__ __launch_bounds__(NT, 2) void wgrad_patch_f64_kernel(const Params p) {
     constexpr int NG = BM / 8, NXC = CT / 8, XR = 3;
-    extern __shared__ __align__(16) double smem[];
+    FX_DYNAMIC_SMEM(double, smem);
     double* Gs = smem;
     double* Xs = smem + BM * p.GP;
     const int tid = threadIdx.x, lane = tid & 63, kq = lane >> 4, l16 = lane & 15;
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_f64_kernel(const Params p) 
     };
     auto park = [&]() __attribute__((always_inline)) {
         int gd = g_dst0, xd = x_dst0;
-        asm volatile("" : "+v"(gd), "+v"(xd));  // recompute the row addresses here instead of keeping them alive
+        FX_PIN_VGPR2(gd, xd);  // recompute the row addresses here instead of keeping them alive
         if (g_lane) {
 #pragma unroll
             for (int u = 0; u < NG; ++u) {
@@ -368,7 +368,7 @@ inline int run(fx_ctx* c, const Plan& pl, const double* x, const double* g, doub
         static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_patch_f64_kernel<NKV>,                   \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
         FX_HIP_CHECK(attr);                                                                                            \
-        wgrad_patch_f64_kernel<NKV><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                                        \
+        FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), wgrad_patch_f64_kernel<NKV>);                                        \
     } break;
     switch (pl.NK) {
         FX_WGD_LAUNCH(3)
@@ -381,7 +381,7 @@ inline int run(fx_ctx* c, const Plan& pl, const double* x, const double* g, doub
     FX_LAUNCH_CHECK();
     const int n = (int)p.part_stride;
     const FastDiv div_row((uint32_t)(KK * Cin)), div_cin((uint32_t)Cin);
-    wgrad_f64_reduce_kernel<<<dim3((unsigned)fx::ceil_div((i64)n, 256)), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin);
+    FX_LAUNCH(dim3((unsigned)fx::ceil_div((i64)n, 256)), dim3(256), 0, c->stream, (part, dw, n, pl.splits, (int)Cin, div_row, div_cin), wgrad_f64_reduce_kernel);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

@@ -74,7 +74,7 @@ template <int WMO, int OW, int R, bool MASK>
 __global__ __launch_bounds__(NT, 1) void wgrad_s2_kernel(const Params p) {
     using S = Shape<WMO, OW, R>;
     constexpr int WK = S::WK, BM = S::BM, W = S::W, PW = S::PW, GP = S::GP, PLANE = S::PLANE, BUF = S::BUF;
-    extern __shared__ __align__(16) float smem[];
+    FX_DYNAMIC_SMEM(float, smem);
     const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wmo = wave % WMO, wk = wave / WMO;
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(NT, 1) void wgrad_s2_kernel(const Params p) {
         // one wave per SIMD owns all 512 registers of a lane: once a function touches the accumulation registers the compiler
         // splits them 256 + 256 and keeps the MFMA accumulators there
         int z = 0;
-        asm volatile("; accumulators in AGPRs %0" : "+a"(z));
+        FX_TOUCH_AGPR(z);
     }
     f32x16 acc[KK];
 #pragma unroll
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(NT, 1) void wgrad_s2_kernel(const Params p) {
     };
     auto park = [&](int buf) __attribute__((always_inline)) {
         int gd = g_dst0 + buf * BUF, xd = x_dst0 + buf * BUF;
-        asm volatile("" : "+v"(gd), "+v"(xd));
+        FX_PIN_VGPR2(gd, xd);
         if (g_lane) {
 #pragma unroll
             for (int u = 0; u < S::NG; ++u) {
@@ -363,8 +363,8 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
                                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
         FX_HIP_CHECK(attr);                                                                                            \
         FX_HIP_CHECK(attr_m);                                                                                          \
-        if (act) wgrad_s2_kernel<A, O, RR, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                           \
-        else wgrad_s2_kernel<A, O, RR, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                              \
+        if (act) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), wgrad_s2_kernel<A, O, RR, true>);                           \
+        else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), wgrad_s2_kernel<A, O, RR, false>);                              \
         launched = true;                                                                                               \
     }
     FX_WG2_SHAPES(FX_WG2_LAUNCH)
@@ -376,11 +376,11 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
     const FastDiv div_row((uint32_t)(KK * Cin)), div_cin((uint32_t)Cin);
     // (with the bias sums behind each partial the stride stays a multiple of 4 floats: Cout % 32 == 0)
     if (pl.splits >= 128 && n <= (1 << 17) && n % 4 == 0 && Cin % 4 == 0 && fx::aligned16(part))
-        wgp::wgrad_patch_reduce_vec_kernel<16><<<dim3((unsigned)(fx::ceil_div((i64)n, 64) + wgp::tail_blocks(tail, 16))), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail);
+        FX_LAUNCH(dim3((unsigned)(fx::ceil_div((i64)n, 64) + wgp::tail_blocks(tail, 16))), dim3(256), 0, c->stream, (part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail), wgp::wgrad_patch_reduce_vec_kernel<16>);
     else if (pl.splits >= 128 && n <= (1 << 17))
-        wgp::wgrad_patch_reduce_grouped_kernel<16><<<dim3((unsigned)(fx::ceil_div((i64)n, 16) + wgp::tail_blocks(tail, 16))), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail);
+        FX_LAUNCH(dim3((unsigned)(fx::ceil_div((i64)n, 16) + wgp::tail_blocks(tail, 16))), dim3(256), 0, c->stream, (part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail), wgp::wgrad_patch_reduce_grouped_kernel<16>);
     else
-        wgp::wgrad_patch_reduce_kernel<<<dim3((unsigned)(fx::ceil_div((i64)n, 256) + wgp::tail_blocks(tail, 256))), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail);
+        FX_LAUNCH(dim3((unsigned)(fx::ceil_div((i64)n, 256) + wgp::tail_blocks(tail, 256))), dim3(256), 0, c->stream, (part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail), wgp::wgrad_patch_reduce_kernel);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

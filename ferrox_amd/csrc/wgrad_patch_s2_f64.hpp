@@ -63,7 +63,7 @@ template <int OW, int R, bool MASK>
 __global__ __launch_bounds__(NT, 1) void wgrad_s2_f64_kernel(const Params p) {
     using S = Shape<OW, R>;
     constexpr int W = S::W, PW = S::PW, GP = S::GP, PLANE = S::PLANE, BUF = S::BUF;
-    extern __shared__ __align__(16) double smem_wgd2[];
+    FX_DYNAMIC_SMEM(double, smem_wgd2);
     double* smem = smem_wgd2;
     const int tid = threadIdx.x, lane = tid & 63, kq = lane >> 4, l16 = lane & 15;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(NT, 1) void wgrad_s2_f64_kernel(const Params p) {
         // one wave per SIMD owns all 512 registers of a lane: once a function touches the accumulation registers the compiler
         // splits them 256 + 256 and keeps the MFMA accumulators there
         int z = 0;
-        asm volatile("; accumulators in AGPRs %0" : "+a"(z));
+        FX_TOUCH_AGPR(z);
     }
     f64x4 acc[2][KK];
 #pragma unroll
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(NT, 1) void wgrad_s2_f64_kernel(const Params p) {
     };
     auto park = [&](int buf) __attribute__((always_inline)) {
         int gd = g_dst0 + buf * BUF, xd = x_dst0 + buf * BUF;
-        asm volatile("" : "+v"(gd), "+v"(xd));
+        FX_PIN_VGPR2(gd, xd);
 #pragma unroll
         for (int u = 0; u < S::NG; ++u) {
             double* d = smem + gd + u * S::GR * GP;
@@ -291,8 +291,8 @@ inline int run(fx_ctx* c, const Plan& pl, const double* x, const double* g, doub
                                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT); \
         FX_HIP_CHECK(attr);                                                                                            \
         FX_HIP_CHECK(attr_m);                                                                                          \
-        if (act) wgrad_s2_f64_kernel<O, RR, true><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                          \
-        else wgrad_s2_f64_kernel<O, RR, false><<<grid, dim3(NT), pl.smem, c->stream>>>(p);                             \
+        if (act) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), wgrad_s2_f64_kernel<O, RR, true>);                          \
+        else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), wgrad_s2_f64_kernel<O, RR, false>);                             \
         launched = true;                                                                                               \
     }
     FX_WGD2_SHAPES(FX_WGD2_LAUNCH)
@@ -304,9 +304,9 @@ inline int run(fx_ctx* c, const Plan& pl, const double* x, const double* g, doub
     const FastDiv div_row((uint32_t)(KK * Cin)), div_cin((uint32_t)Cin);
     // many partials of a small output: the grouped 16-byte sum (n, Cin and the stride are even here, part is 16-byte aligned)
     if (pl.splits >= 64 && n <= (1 << 18))
-        wgd::wgrad_f64_reduce_vec_kernel<16><<<dim3((unsigned)(fx::ceil_div((i64)n, 32) + wgd::tail_blocks(tail, 16))), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail);
+        FX_LAUNCH(dim3((unsigned)(fx::ceil_div((i64)n, 32) + wgd::tail_blocks(tail, 16))), dim3(256), 0, c->stream, (part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail), wgd::wgrad_f64_reduce_vec_kernel<16>);
     else
-        wgd::wgrad_f64_reduce_kernel<<<dim3((unsigned)(fx::ceil_div((i64)n, 256) + wgd::tail_blocks(tail, 256))), dim3(256), 0, c->stream>>>(part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail);
+        FX_LAUNCH(dim3((unsigned)(fx::ceil_div((i64)n, 256) + wgd::tail_blocks(tail, 256))), dim3(256), 0, c->stream, (part, dw, n, pl.splits, (int)Cin, div_row, div_cin, tail), wgd::wgrad_f64_reduce_kernel);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
