@@ -273,7 +273,8 @@ inline Plan make_plan(int num_cus, bool wgrad, i64 B, i64 C, i64 H, i64 W, i64 C
     pl.PR = (int)((rows - 1) * sh + 3);
     // wide images: a tile of 256 pixels covers about one output row and would stage five or seven input rows (measured
     // at 3 x 224 x 224 -> 64: 0.300 ms here against 0.245 ms for the implicit GEMM, 0.074 against 0.059 ms at stride 2)
-    if (OW > 64 || (i64)pl.PR * OW > 2 * (i64)NPIX * sh) return pl;
+    // (rows up to 256 floats that divide the tile -- 128: two rows per tile -- stage four rows for two and stay ahead of it)
+    if ((OW > 64 && (OW > NPIX || NPIX % OW != 0)) || (i64)pl.PR * OW > 2 * (i64)NPIX * sh) return pl;
     pl.PW = (int)(W + 2 * pw);
     pl.PLANE = pl.PR * pl.PW;
     pl.tpi = (int)fx::ceil_div(L, (i64)NPIX);

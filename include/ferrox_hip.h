@@ -381,8 +381,10 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
                                        T* const* v, T* const* vmax, const int64_t* n, T lr, T beta1, T beta2, T eps,   \
                                        T weight_decay, T bc1, T bc2);                                                  \
     /* The multi-tensor Adam step for recorded steps (fx_graph_*): the bias corrections, the only scalars of a step    \
-       that change from one step to the next, are read from DEVICE memory, bc = {bc1, bc2}; vmax may be NULL (no       \
-       AMSGrad).  Same arithmetic and bits as the calls above. */                                                      \
+       that change from one step to the next, are read from memory the device can address, bc = {bc1, bc2}: device    \
+       memory, or page-locked host memory from fx_host_alloc, which the kernel reads in place (the host then rewrites  \
+       the two values between launches, once the launch before has finished).  vmax may be NULL (no AMSGrad).  Same    \
+       arithmetic and bits as the calls above. */                                                                      \
     int fx_adam_step_multi_bc_##S(fx_ctx* ctx, int count, T* const* p, const T* const* g, T* const* m, T* const* v,    \
                                   T* const* vmax, const int64_t* n, T lr, T beta1, T beta2, T eps, T weight_decay,     \
                                   const T* bc);                                                                        \
@@ -406,9 +408,9 @@ FX_DECLARE_KERNELS(double, f64)
  *   - blocks released with fx_free while recording stay out of the pool: they are the graph's temporaries, used at the
  *     same addresses by every launch, and go back to the pool in fx_graph_destroy;
  *   - what a launch reads from outside (the batch) must sit at the recorded addresses: copy new data there;
- *   - scalars that change per step must come from device memory: fx_adam_step_multi_bc reads its bias corrections
- *     there, and fx_h2d_async from fx_host_alloc'ed memory is recorded as "copy from this host address", so the
- *     host rewrites the values between launches.
+ *   - scalars that change per step must come from memory: fx_adam_step_multi_bc reads its bias corrections through a
+ *     pointer, which may be page-locked host memory (fx_host_alloc) that the host rewrites between launches; an
+ *     fx_h2d_async from such memory is recorded as "copy from this host address" and serves larger data the same way.
  * A launch is stream-ordered like any other call; results are bit-identical to the eager calls (same kernels, same
  * arguments). */
 /* 1 when fx_conv2d_wgrad_relu_bias (kind FX_CONV_WGRAD) / fx_conv2d_dgrad_relu (kind FX_CONV_DGRAD) has a fused kernel

@@ -307,7 +307,9 @@ def test_gemm_all_transposes(ctx, orc, golden, dtype):
 
 # Products large enough for the LDS-slab f32 kernel on a 256-CU device (at least 384 tiles of 128 x 128, K % 64 == 0):
 # exact tiles, ragged M and N (rows / columns past the matrix are re-read, never stored), N below one tile.
-GEMM_LDS_SHAPES = [(2560, 2560, 128), (2500, 2436, 192), (4096, 3200, 64 * 3), (49152, 100, 128), (128 * 50, 1024 + 4, 256)]
+GEMM_LDS_SHAPES = [(2560, 2560, 128), (2500, 2436, 192), (4096, 3200, 64 * 3), (49152, 100, 128), (128 * 50, 1024 + 4, 256),
+                   # too few 128-row tiles to fill the chip: 64 x 64 and 64 x 128 tiles (exact, ragged rows and columns, M below 128)
+                   (1024, 1024, 1024), (1000, 1100, 192), (1280, 832, 128), (2048, 512, 256), (100, 16384, 128), (1988, 724, 320)]
 
 
 def test_gemm_lds_kernel_shapes_all_transposes_and_bias(ctx):
@@ -771,6 +773,8 @@ SMALLC_CASES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw)
     (1, 3, 20, 224, 16, (2, 2), (1, 1)), (1, 4, 10, 64, 16, (1, 2), (2, 0)), (3, 3, 9, 12, 40, (1, 1), (0, 0)), (37, 3, 16, 16, 32, (1, 1), (1, 1)),
     # row lengths that are not multiples of four floats
     (2, 3, 14, 14, 32, (1, 1), (1, 1)), (2, 1, 9, 7, 16, (1, 1), (1, 1)), (2, 3, 12, 30, 8, (1, 1), (1, 1)), (3, 1, 8, 5, 8, (1, 1), (1, 1)),
+    # rows of 128 floats (two per tile): the reference's own benchmark layer (kernels/benchmark.cu:856-860) and neighbours
+    (1, 3, 128, 128, 32, (1, 1), (1, 1)), (2, 1, 6, 128, 40, (1, 1), (1, 1)), (1, 2, 7, 256, 8, (2, 2), (1, 1)), (2, 3, 5, 128, 16, (1, 1), (0, 0)),
 ]
 
 
