@@ -13,6 +13,7 @@
 #include <cstdlib>
 
 #include "igemm_core.hpp"
+#include "gemm_lds.hpp"
 #include "wgrad_patch.hpp"
 #include "wgrad_patch_s2.hpp"
 #include "dgrad_patch_s2.hpp"
@@ -175,6 +176,31 @@ cpd::Plan dgrad_patch64_plan(fx_ctx* c, const Dims& d, int mode) {
     return cpd::Plan();
 }
 
+// 1x1 filters at unit stride without padding (f32): the convolution of one image is a plain product over the channels,
+//   fwd    Y_b [Cout, L]  = W [Cout, Cin] . X_b [Cin, L]
+//   dgrad  dX_b [Cin, L]  = W^T . G_b [Cout, L]
+//   wgrad  dW [Cout, Cin] = sum over b of G_b [Cout, L] . X_b^T
+// with every operand already laid out as the LDS-slab GEMM wants it (gemm_lds.hpp), so the whole batch runs as one launch of
+// that kernel (blockIdx.y = image); the weight gradient leaves one partial product per image and the ordered sum adds them.
+// kind: FX_CONV_FWD / FX_CONV_DGRAD / FX_CONV_WGRAD.
+template <typename T>
+glk::Plan pointwise_plan(fx_ctx* c, const Dims& d, int kind) {
+    if constexpr (sizeof(T) == 4) {
+        static const bool off = [] { const char* v = getenv("FX_CONV_1X1"); return v && atoi(v) == 0; }();
+        if (off || generic_only() || d.kh != 1 || d.kw != 1 || d.sh != 1 || d.sw != 1 || d.ph != 0 || d.pw != 0 || d.B > 65535) return glk::Plan();
+        const int cus = c ? c->num_cus : 256;
+        const i64 L = d.H * d.W;
+        glk::Plan pl;
+        if (kind == FX_CONV_FWD) pl = glk::make_plan(cus, false, false, d.Cout, L, d.Cin, d.Cin, L, d.B);
+        else if (kind == FX_CONV_DGRAD) pl = glk::make_plan(cus, true, false, d.Cin, L, d.Cout, d.Cin, L, d.B);
+        else if (d.B * d.Cout * d.Cin <= 0x7fffffff) pl = glk::make_plan(cus, false, true, d.Cout, d.Cin, L, L, L, d.B);
+        // only with the 128-row tiles: the 64-row ones measured below the implicit GEMM here ([32,256,56,56] -> 64: 55 against
+        // 63 TFLOP/s forward), the 128-row ones above it (-> 256: 92 against 86; [16,256,16,16] -> 1024: 94 against 64)
+        return pl.ok && pl.WM == 4 ? pl : glk::Plan();
+    }
+    return glk::Plan();
+}
+
 template <typename T>
 i64 fwd_ws_bytes(fx_ctx* c, const Dims& d) {
     // enough for either kernel: a misaligned tensor sends a patch-kernel shape to the implicit GEMM
@@ -211,6 +237,11 @@ int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64
         if (!generic_only()) {
             const fw2::Plan f2 = fw2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
             if (f2.ok && aligned16(x, w) && aligned16(y, y)) return fw2::run(c, f2, x, w, y, B, Cin, H, Cout, d.oh, bias, relu);
+        }
+        const glk::Plan pp = pointwise_plan<T>(c, d, FX_CONV_FWD);
+        if (pp.ok && aligned16(x, w) && aligned16(y, y)) {
+            const i64 L = d.H * d.W;
+            return glk::run(c, pp, false, false, Cout, L, Cin, w, x, y, bias, relu, B, 0, Cin * L, Cout * L, 1);
         }
         const cpk::Plan pl = fwd_patch_plan<T>(c, d);
         if (pl.ok && aligned16(x, ws)) {
@@ -482,6 +513,11 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
         if (!generic_only()) {
             const dg2::Plan p2 = dg2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
             if (p2.ok && aligned16(g, w) && aligned16(dx, dx)) return dg2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh);
+            const glk::Plan pp = pointwise_plan<T>(c, d, FX_CONV_DGRAD);
+            if (pp.ok && aligned16(g, w) && aligned16(dx, dx)) {
+                const i64 L = d.H * d.W;
+                return glk::run(c, pp, true, false, Cin, L, Cout, w, g, dx, nullptr, 0, B, 0, Cout * L, Cin * L);
+            }
         }
     } else {
         if (!generic_only()) {
@@ -604,6 +640,7 @@ i64 wgrad_ws_bytes(fx_ctx* c, const Dims& d, int mode) {
     if (p2.ok) generic = std::max(generic, wg2::workspace_bytes(p2, d.Cout, d.Cin, true));
     const wgd2::Plan q2 = patch64_s2_plan<T>(c, d, mode);
     if (q2.ok) generic = std::max(generic, wgd2::workspace_bytes(q2, d.Cout, d.Cin, true));
+    if (mode == 0 && pointwise_plan<T>(c, d, FX_CONV_WGRAD).ok) generic = std::max(generic, d.B * d.Cout * d.Cin * (i64)sizeof(T));
     if constexpr (sizeof(T) == 8) {
         if (mode == 0 && !generic_only()) {
             const cim::WPlan ip = cim::wgrad_plan(c ? c->num_cus : 256, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
@@ -665,6 +702,15 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
             float* part = (float*)(ws ? ws : c->get_scratch(need));
             if (!part) return FX_ERR_OOM;
             return wg2::run(c, p2, x, g, dw, part, Cin, H, Cout, ph, d.oh);
+        }
+        const glk::Plan pp = mode == 0 ? pointwise_plan<T>(c, d, FX_CONV_WGRAD) : glk::Plan();
+        if (pp.ok && aligned16(x, g) && aligned16(ws, dw)) {
+            const i64 L = d.H * d.W, n = Cout * Cin;
+            if (B == 1) return glk::run(c, pp, false, true, Cout, Cin, L, g, x, dw, nullptr, 0);
+            float* part = (float*)(ws ? ws : c->get_scratch(need));
+            if (!part) return FX_ERR_OOM;
+            if (int rc = glk::run(c, pp, false, true, Cout, Cin, L, g, x, part, nullptr, 0, B, Cout * L, Cin * L, n)) return rc;
+            return launch_splitk_reduce<T>(c, part, dw, n, (int)B);
         }
         const wgp::Plan pl = patch_plan<T>(c, d, mode);
         if (pl.ok && aligned16(x, g) && aligned16(ws, ws)) {

@@ -952,6 +952,54 @@ def test_conv2d_strided_dgrad_vs_torch_and_oracle(ctx, orc, dtype):
         parity.check("strided dgrad", dx, tx.grad.numpy(), oracle=orc.conv2d_dgrad(g, w, (B, Cin, H, W), st, pd, 0), case=case)
 
 
+# 1x1 filters at unit stride without padding: one launch of the batched LDS-slab product where the channel counts allow it
+# (channels reduced in slabs of 64, at least 128 of them; rows of H*W floats a multiple of four), the implicit GEMM otherwise.
+# B, Cin, H, W, Cout
+POINTWISE_CASES = [(3, 128, 16, 16, 256), (4, 256, 8, 8, 128), (2, 192, 12, 20, 96), (70, 128, 8, 8, 64), (1, 512, 32, 32, 128),
+                   (2, 64, 16, 16, 64), (3, 130, 8, 8, 70), (2, 128, 7, 9, 256), (5, 256, 16, 16, 256)]
+
+
+def test_conv2d_pointwise_layers(ctx, orc):
+    import torch
+    import torch.nn.functional as F
+    from ferrox_amd import capi
+    rng = np.random.default_rng(64)
+    for (B, Cin, H, W, Cout) in POINTWISE_CASES:
+        case = (B, Cin, H, W, Cout)
+        x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(np.float32)
+        w = (rng.standard_normal((Cout, Cin, 1, 1)) * np.sqrt(2.0 / Cin)).astype(np.float32)
+        g = rng.standard_normal((B, Cout, H, W)).astype(np.float32)
+        bias = rng.standard_normal(Cout).astype(np.float32)
+        dx_, dw_, dg_, db_ = ctx.upload(x), ctx.upload(w), ctx.upload(g), ctx.upload(bias)
+        y = ctx.conv2d_fwd(dx_, dw_, (1, 1), (0, 0)).numpy()
+        gx = ctx.conv2d_dgrad(dg_, dw_, x.shape, (1, 1), (0, 0), 0).numpy()
+        gw = ctx.conv2d_wgrad(dx_, dg_, w.shape, (1, 1), (0, 0), 0).numpy()
+        tx = torch.from_numpy(x).double().requires_grad_(True)
+        tw = torch.from_numpy(w).double().requires_grad_(True)
+        ty = F.conv2d(tx, tw)
+        ty.backward(torch.from_numpy(g).double())
+        ay = F.conv2d(tx.detach().abs(), tw.detach().abs()).max().item()
+        small = B * Cout * H * W * Cin <= 1 << 27  # the oracle's explicit column matrix stays small
+        parity.check("pointwise fwd", y, ty.detach().numpy(), oracle=orc.conv2d_fwd(x, w, (1, 1), (0, 0)) if small else None, case=case, terms=ay)
+        parity.check("pointwise dgrad", gx, tx.grad.numpy(), oracle=orc.conv2d_dgrad(g, w, x.shape, (1, 1), (0, 0), 0) if small else None, case=case)
+        parity.check("pointwise wgrad", gw, tw.grad.numpy(), oracle=orc.conv2d_wgrad(x, g, w.shape, (1, 1), (0, 0), 0) if small else None, case=case)
+        # same bits on a second run; bias + ReLU in the store equals the separate pass
+        assert np.array_equal(ctx.conv2d_fwd(dx_, dw_, (1, 1), (0, 0)).numpy(), y), case
+        assert np.array_equal(ctx.conv2d_wgrad(dx_, dg_, w.shape, (1, 1), (0, 0), 0).numpy(), gw), case
+        dims = (B, Cin, H, W, Cout, 1, 1, 1, 1, 0, 0)
+        fused = ctx.empty(y.shape, np.float32)
+        capi.check(capi.lib.fx_conv2d_fwd_bias_act_f32(ctx.h, dx_.ptr, dw_.ptr, db_.ptr, fused.ptr, *dims, 1, None, 0))
+        two = ctx.conv2d_fwd(dx_, dw_, (1, 1), (0, 0))
+        capi.check(capi.lib.fx_bias_act_f32(ctx.h, two.ptr, db_.ptr, B, Cout, H * W, 1))
+        assert np.array_equal(fused.numpy(), two.numpy()), ("bias+relu", case)
+        # a caller workspace of exactly the advertised size for the weight gradient
+        need = capi.lib.fx_conv2d_workspace_bytes(capi.CONV_WGRAD, capi.FX_F32, 0, *dims)
+        ws = ctx.empty((max(need, 4) // 4,), np.float32)
+        out = ctx.empty(w.shape, np.float32)
+        capi.check(capi.lib.fx_conv2d_wgrad_f32(ctx.h, dx_.ptr, dg_.ptr, out.ptr, *dims, 0, ws.ptr, need))
+        assert np.array_equal(out.numpy(), gw), case
+
+
 @pytest.mark.parametrize("seed,dtype", [(61, np.float32), (62, np.float32), (63, np.float32), (64, np.float32), (65, np.float64), (66, np.float64)])
 def test_conv2d_random_shapes_all_paths_vs_torch(ctx, seed, dtype):
     """Seeded random 3x3 / 1x1 / 5x5 shapes biased towards the dispatch boundaries of the conv kernels (channel counts

@@ -21,7 +21,7 @@ CLANG = os.environ.get("FX_WALK_CXX", "/opt/rocm/lib/llvm/bin/clang++")
 
 def _sources():
     files = [os.path.join(WALK_DIR, "walk.cpp"), os.path.join(WALK_DIR, "hip", "hip_runtime.h"), os.path.join(ROOT, "include", "ferrox_hip.h")]
-    files += sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp") or f == "conv.hip")
+    files += sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp") or f == "conv.hip")  # gemm_lds.hpp included
     return files
 
 
@@ -87,6 +87,8 @@ def gpu_test_cases():
     for (B, Cin, H, W, Cout, st, pd) in tk.SMALLC_CASES:
         for dt in ("f32", "f64"):
             add("image_layer", dt, B, Cin, H, W, Cout, 3, st, pd)
+    for (B, Cin, H, W, Cout) in tk.POINTWISE_CASES:
+        add("pointwise", "f32", B, Cin, H, W, Cout, 1, 1, 0)
     for (B, Cin, H, W, Cout, k, st, pd) in tk.STRIDED_DGRAD_CASES:
         for dt in ("f32", "f64"):
             add("strided", dt, B, Cin, H, W, Cout, k, st, pd)
