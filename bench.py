@@ -667,6 +667,10 @@ def main():
     ap.add_argument("--train-only", nargs="?", const="all", default=None, metavar="CONFIG,DTYPE,ENGINE",
                     help="run only the train-step section and print it (profiler runs); optional filter such as "
                          "C5_cnn,float32,engine_fused")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="with --train-only: first run a streaming add over 2^26 floats four times (reads 2 x 256 MiB, writes "
+                         "256 MiB per call): the kernel of known traffic that FETCH_SIZE / WRITE_SIZE readings of the same "
+                         "profiler run are scaled by")
     ap.add_argument("--c4-profile", action="store_true",
                     help="run only the C4 bandwidth kernels, 4 calls each on rotating inputs with marker dispatches between "
                          "the cases, and print the case order (for rocprofv3 counter runs)")
@@ -685,6 +689,15 @@ def main():
             print(json.dumps({"c4_profile_order": bench_c4_profile(ctx)}))
         return
     if args.train_only:
+        if args.calibrate:
+            from ferrox_amd import capi
+            with capi.Context(0) as cctx:
+                n = 1 << 26
+                a, b, o = cctx.uniform((n,), 1, -1.0, 1.0), cctx.uniform((n,), 2, -1.0, 1.0), cctx.empty((n,))
+                for _ in range(4):
+                    cctx.binary("add", a, b, out=o)
+                cctx.sync()
+                del a, b, o
         only = None if args.train_only == "all" else tuple(args.train_only.split(","))
         print(json.dumps({"train_step": bench_train_steps(cpu=False, only=only)}))
         return
