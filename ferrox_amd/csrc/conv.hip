@@ -186,8 +186,7 @@ cpd::Plan dgrad_patch64_plan(fx_ctx* c, const Dims& d, int mode) {
 template <typename T>
 glk::Plan pointwise_plan(fx_ctx* c, const Dims& d, int kind) {
     if constexpr (sizeof(T) == 4) {
-        static const bool off = [] { const char* v = getenv("FX_CONV_1X1"); return v && atoi(v) == 0; }();
-        if (off || generic_only() || d.kh != 1 || d.kw != 1 || d.sh != 1 || d.sw != 1 || d.ph != 0 || d.pw != 0 || d.B > 65535) return glk::Plan();
+        if (generic_only() || d.kh != 1 || d.kw != 1 || d.sh != 1 || d.sw != 1 || d.ph != 0 || d.pw != 0 || d.B > 65535) return glk::Plan();
         const int cus = c ? c->num_cus : 256;
         const i64 L = d.H * d.W;
         glk::Plan pl;

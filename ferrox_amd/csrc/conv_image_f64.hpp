@@ -139,8 +139,7 @@ __global__ __launch_bounds__(NT) void image_fwd_f64_kernel(const Params p) {
 
 // Maps 32 wide (8 rows per tile), heights a multiple of 8, output channels a multiple of 32.
 inline bool eligible(i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw) {
-    static const bool off = [] { const char* v = getenv("FX_CIM"); return v && atoi(v) == 0; }();
-    return !off && kh == 3 && kw == 3 && sh == 1 && sw == 1 && ph == 1 && pw == 1 && Cin >= 1 && Cin <= CP && W == 32 && H % (PIX / 32) == 0 &&
+    return kh == 3 && kw == 3 && sh == 1 && sw == 1 && ph == 1 && pw == 1 && Cin >= 1 && Cin <= CP && W == 32 && H % (PIX / 32) == 0 &&
            Cout % 32 == 0 && B * (H / (PIX / 32)) * (Cout / 32) <= 0x7fffffff;
 }
 
@@ -311,8 +310,7 @@ struct WPlan {
 
 inline WPlan wgrad_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw) {
     WPlan pl;
-    static const bool off = [] { const char* v = getenv("FX_CIM"); return v && atoi(v) == 0; }();
-    if (off || kh != 3 || kw != 3 || sh != 1 || sw != 1 || ph != 1 || pw != 1 || Cin < 1 || Cin > 3 || W != 32 || H % (PIX / 32) != 0 || Cout % 32 != 0)
+    if (kh != 3 || kw != 3 || sh != 1 || sw != 1 || ph != 1 || pw != 1 || Cin < 1 || Cin > 3 || W != 32 || H % (PIX / 32) != 0 || Cout % 32 != 0)
         return pl;
     const i64 tiles = B * (H / (PIX / 32)), rows = Cout / 32;
     if (tiles > 0x7fffffff || rows > 65535) return pl;

@@ -562,17 +562,13 @@ inline bool shape_plan(Plan& pl, int wm, int tn, int num_cus, i64 B, i64 C, i64 
 // Tile shapes of the persistent variant (wm x tn).
 constexpr int N_PSHAPES = 5;
 static const int PSHAPES[N_PSHAPES][2] = {{4, 5}, {4, 4}, {2, 5}, {2, 4}, {2, 3}};
-inline bool persist_enabled() {
-    static const bool off = [] { const char* v = getenv("FX_CPK_PERSIST"); return v && atoi(v) == 0; }();
-    return !off;
-}
 // The plan of the persistent variant for one tile shape; false when the shape does not fit this layer.
 inline bool persist_plan(Plan& pl, int wm, int tn, int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 sh, i64 sw, i64 ph,
                          i64 pw) {
     const i64 L = OH * OW, slots = 2 * (i64)std::max(1, num_cus);
     const i64 bm = 32 * wm, np = 32 * tn * (4 / wm), tiles = fx::ceil_div(L, np), mtiles = fx::ceil_div(M, bm);
     const i64 rows = std::min<i64>(OH, np % OW == 0 ? np / OW : (np - 1) / OW + 2), PR = (rows - 1) * sh + 3;
-    if (!persist_enabled() || PR > 2 * NXP_PERSIST || mtiles * bm > M * 2 || tiles * np > L * 2 || B * tiles * mtiles > 0x7fffffff) return false;
+    if (PR > 2 * NXP_PERSIST || mtiles * bm > M * 2 || tiles * np > L * 2 || B * tiles * mtiles > 0x7fffffff) return false;
     // patch row pitch: with unit column stride a run of 32 pixels that wraps to the next output row must continue 32
     // words further on (sh * pitch - OW a multiple of 32), else two of its lanes share a bank; the plain pitch when that
     // does not fit the plane.

@@ -316,8 +316,7 @@ inline bool shape_plan(Plan& pl, int tn, int num_cus, i64 B, i64 C, i64 H, i64 W
 // C input channels of H x W, M output channels of OH x OW (already the dimensions of the pass that runs).
 inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw) {
     Plan best;
-    static const bool off = [] { const char* v = getenv("FX_CPD"); return v && atoi(v) == 0; }();
-    if (off || kh != 3 || kw != 3 || C % CC != 0 || W < 2 || W % 2 != 0 || W > 2 * LPR || sh > 8 || sw > 8 || OH * OW < 64 || M < 32) return best;
+    if (kh != 3 || kw != 3 || C % CC != 0 || W < 2 || W % 2 != 0 || W > 2 * LPR || sh > 8 || sw > 8 || OH * OW < 64 || M < 32) return best;
     for (int tn : SHAPES) {
         Plan q;
         if (shape_plan(q, tn, num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw) && (!best.ok || q.cost < best.cost)) best = q;

@@ -218,8 +218,7 @@ struct Plan {
 
 inline Plan make_plan(i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, i64 oh, i64 ow) {
     Plan pl;
-    static const bool off = [] { const char* v = getenv("FX_DG2"); return v && atoi(v) == 0; }();
-    if (off || kh != 3 || kw != 3 || sh != 2 || sw != 2 || ph != 1 || pw != 1 || W != 2 * ow || H != 2 * oh || Cin % CT != 0) return pl;
+    if (kh != 3 || kw != 3 || sh != 2 || sw != 2 || ph != 1 || pw != 1 || W != 2 * ow || H != 2 * oh || Cin % CT != 0) return pl;
     if (Cout * oh * ow * 4 > 0x7fffffff || Cout * Cin * KK * 4 > 0x7fffffff || B * (Cin / CT) * oh > 0x7fffffff) return pl;
 #define FX_DG2_PICK(O, C_)                                                                   \
     if (!pl.ok && ow == O && Cout % C_ == 0 && oh % (CELLS / O) == 0) {                      \

@@ -203,8 +203,7 @@ struct Plan {
 
 inline Plan make_plan(i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, i64 oh, i64 ow) {
     Plan pl;
-    static const bool off = [] { const char* v = getenv("FX_FW2"); return v && atoi(v) == 0; }();
-    if (off || kh != 3 || kw != 3 || sh != 2 || sw != 2 || ph != 1 || pw != 1 || W != 2 * ow || H != 2 * oh || Cin % CC != 0 || Cout % 32 != 0) return pl;
+    if (kh != 3 || kw != 3 || sh != 2 || sw != 2 || ph != 1 || pw != 1 || W != 2 * ow || H != 2 * oh || Cin % CC != 0 || Cout % 32 != 0) return pl;
     if (Cin * H * W * 4 > 0x7fffffff || Cout * Cin * KK * 4 > 0x7fffffff || B * oh * (Cout / 32) > 0x7fffffff) return pl;
     // Measured against the tall-patch instantiation of the stride-1 kernel (256 images, 32x32 maps): 20.5 against 30.0 us at
     // 32 -> 32 channels, 7.4 against 12.3 us at 8 -> 32, 11.3 against 13.5 us at 8 -> 64, level at 16 -> 64 and 32 -> 64, and

@@ -269,7 +269,6 @@ struct Plan {
 // products of this shape that share the launch (their tiles count towards filling the chip).
 inline Plan make_plan(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, i64 lda, i64 ldb, i64 batch = 1) {
     Plan pl;
-    static const bool mid_off = [] { const char* v = getenv("FX_GEMM_MID"); return v && atoi(v) == 0; }();
     if (K < 2 * KC || K % KC != 0 || lda % 4 != 0 || ldb % 4 != 0 || M < 64 || N < 64) return pl;
     if ((ta && M % 4 != 0) || (!tb && N % 4 != 0)) return pl;
     // tile shape: the one with the least (rounds of co-resident blocks) x (work of a block); a nearly empty last round
@@ -280,7 +279,7 @@ inline Plan make_plan(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, i64 ld
     i64 best = -1, tiles = 0;
     for (const auto& sh : shapes) {
         const int wmv = sh[0], tn = sh[1], bm = 32 * wmv, bn = 32 * tn * (4 / wmv);
-        if (M < bm || (wmv == 2 && mid_off)) continue;
+        if (M < bm) continue;
         const i64 t = fx::ceil_div(M, (i64)bm) * fx::ceil_div(N, (i64)bn) * batch;
         // fewer tiles than 3/4 of the block slots: a smaller tile, or (below half a block per CU even with the smallest)
         // the generic kernel's K split

@@ -386,9 +386,8 @@ struct Plan {
 template <typename T>
 inline Plan make_plan(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, const T* A, const T* B, bool allow16 = false) {
     Plan pl;
-    static const bool off = [] { const char* v = getenv("FX_GEMM_SMALL"); return v && atoi(v) == 0; }();
     constexpr int KV = 16 / (int)sizeof(T);  // elements per 16-byte load of a k-contiguous operand
-    if (off || K < 1 || M < 1 || N < 1 || K >= (1ll << 30)) return pl;
+    if (K < 1 || M < 1 || N < 1 || K >= (1ll << 30)) return pl;
     if (K < 32 && ta) return pl;  // short reductions: only with a k-contiguous A, read element by element (the general tiles serve the others)
     if (!ta && (K % KV != 0 || !fx::aligned16(A) || K < 32)) pl.a_elems = true;
     if (tb && (K % KV != 0 || !fx::aligned16(B))) return pl;
@@ -402,8 +401,7 @@ inline Plan make_plan(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, const 
         if constexpr (sizeof(T) == 4) {
             // fewer 32 x 32 tiles than half the CUs, each reading K >= 128 deep: 16 x 16 tiles fill more of the chip
             const i64 tiles16 = fx::ceil_div(M, (i64)16) * fx::ceil_div(N, (i64)16);
-            static const bool off16 = [] { const char* v = getenv("FX_GEMM_SMALL16"); return v && atoi(v) == 0; }();
-            if (!off16 && allow16 && !pl.a_elems && 2 * tiles < (i64)num_cus && tiles16 <= 2 * (i64)num_cus && K >= 128 && N >= 16) {
+            if (allow16 && !pl.a_elems && 2 * tiles < (i64)num_cus && tiles16 <= 2 * (i64)num_cus && K >= 128 && N >= 16) {
                 pl.tile16 = true;
                 pl.G = (int)fx::ceil_div(fx::ceil_div(K, (i64)16), (i64)WAVES);
             }

@@ -138,8 +138,7 @@ inline size_t lds_bytes(i64 K) { return ((size_t)as_rows(K) * 32 + (KQ - 1) * 2 
 
 // TN products this kernel takes: the general path needs two launches (split K) and stages B in 64-byte pieces.
 inline bool eligible(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K) {
-    static const bool off = [] { const char* v = getenv("FX_GEMM_THIN"); return v && atoi(v) == 0; }();
-    return !off && ta && !tb && M >= 1 && M <= 32 && K >= 32 && K <= 2048 && lds_bytes(K) <= LDS_LIMIT && N >= 32 * (i64)num_cus &&
+    return ta && !tb && M >= 1 && M <= 32 && K >= 32 && K <= 2048 && lds_bytes(K) <= LDS_LIMIT && N >= 32 * (i64)num_cus &&
            N < (1ll << 31) - BN;
 }
 

@@ -321,8 +321,7 @@ int fx_d2d(fx_ctx* c, void* dst, const void* src, int64_t bytes) {
     if (bytes == 0) return FX_OK;
     // blocks up to 32 MiB go through the library's own streaming kernel (half the stream time of a runtime copy at these
     // sizes); larger ones and odd sizes / alignments through the runtime
-    static const bool use_kernel = !(getenv("FX_D2D_KERNEL") && atoi(getenv("FX_D2D_KERNEL")) == 0);
-    if (use_kernel && bytes <= (32ll << 20)) {
+    if (bytes <= (32ll << 20)) {
         const int rc = fx::copy_kernel(c, dst, src, bytes);
         if (rc != FX_ERR_UNSUPPORTED) return rc;
     }

@@ -325,8 +325,7 @@ inline int odd(int n) { return n | 1; }
 
 inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, i64 oh, i64 ow) {
     Plan pl;
-    static const bool off = [] { const char* v = getenv("FX_WGD"); return v && atoi(v) == 0; }();
-    if (off || kh != 3 || kw != 3 || sw != 1 || sh > 8 || Cin % CT != 0 || Cout % BM != 0 || W % 2 != 0 || W > 64 || ow % 8 != 0 || ow < 24 ||
+    if (kh != 3 || kw != 3 || sw != 1 || sh > 8 || Cin % CT != 0 || Cout % BM != 0 || W % 2 != 0 || W > 64 || ow % 8 != 0 || ow < 24 ||
         ow > 64 || Cout * Cin * KK > 0x7fffffff || B * oh > 0x7fffffff)
         return pl;
     pl.NK = (int)(ow / 8);

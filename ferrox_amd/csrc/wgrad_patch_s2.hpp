@@ -312,8 +312,7 @@ struct Plan {
 
 inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, i64 oh, i64 ow) {
     Plan pl;
-    static const bool off = [] { const char* v = getenv("FX_WG2"); return v && atoi(v) == 0; }();
-    if (off || kh != 3 || kw != 3 || sh != 2 || sw != 2 || pw != 1 || ph > 1 || W != 2 * ow || Cin % CT != 0 || Cout % 32 != 0) return pl;
+    if (kh != 3 || kw != 3 || sh != 2 || sw != 2 || pw != 1 || ph > 1 || W != 2 * ow || Cin % CT != 0 || Cout % 32 != 0) return pl;
     if (Cout * Cin * KK > 0x7fffffff || 32 * H * W * 4 > 0x7fffffff || Cout * oh * ow * 4 > 0x7fffffff) return pl;
     const int wmo = Cout % 128 == 0 ? 4 : Cout % 64 == 0 ? 2 : 1;
 #define FX_WG2_PICK(A, O, RR)                                            \

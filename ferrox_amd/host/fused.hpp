@@ -171,8 +171,7 @@ template <typename T> struct Conv2dFusedOp : Operator<T> {  // inputs: x [B,Cin,
             const Shape &xs = in[0]->shape(), &ws = in[1]->shape();
             const int64_t d[11] = {(int64_t)xs[0], (int64_t)xs[1], (int64_t)xs[2], (int64_t)xs[3], (int64_t)ws[0], (int64_t)ws[2], (int64_t)ws[3],
                                    (int64_t)stride.first, (int64_t)stride.second, (int64_t)padding.first, (int64_t)padding.second};
-            static const bool off = [] { const char* v = getenv("FX_CONV_BWD_FUSED"); return v && atoi(v) == 0; }();
-            if (!off && FusedApi<T>::conv_bwd_relu_supported(fused_ctx(), FX_CONV_WGRAD, d) &&
+            if (FusedApi<T>::conv_bwd_relu_supported(fused_ctx(), FX_CONV_WGRAD, d) &&
                 (!needs[0] || FusedApi<T>::conv_bwd_relu_supported(fused_ctx(), FX_CONV_DGRAD, d))) {
                 r[1] = HipStorage<T>::alloc(ws);
                 const int rc = FusedApi<T>::conv_wgrad_relu_bias(fused_ctx(), in[0]->data(), g->data(), out->data(), r[1]->data(), r[2]->data(), d);
