@@ -524,10 +524,14 @@ def bench_train_steps(steps=30, warmup=5, cpu=True, reference_pool=False, only=N
             # engine_literal: the reference's op sequence as is; engine_without_node_clones: the same minus the
             # engine's per-node deep clones; engine_fused: fused layers, loss and optimizer (extra entry points)
             # engine_fused_graph: the fused step recorded once into a HIP graph and replayed (one submission per step)
-            for label, literal, fused in (("engine_literal", True, False), ("engine_without_node_clones", False, False),
+            # engine_literal_copying_clones: engine_literal with every clone_storage() as the device copy the reference's CUDA
+            # backend makes; the other op-by-op lines share the block between a tensor and its clones
+            for label, literal, fused in (("engine_literal", True, False), ("engine_literal_copying_clones", True, False),
+                                          ("engine_without_node_clones", False, False),
                                           ("engine_fused", False, True), ("engine_fused_graph", False, True)):
                 if (fused and reference_pool) or (only and only[2] != label):
                     continue
+                host_api.set_share_clones(label != "engine_literal_copying_clones")
                 m = host_api.Model(cfg["spec"], params, cfg["opt"], dtype, literal_engine=literal, fused=fused)
                 if label == "engine_fused_graph":
                     m.enable_graph()
@@ -545,6 +549,7 @@ def bench_train_steps(steps=30, warmup=5, cpu=True, reference_pool=False, only=N
                 if label == "engine_fused_graph":
                     out[key][label]["graph"] = m.graph_info()  # kernel_nodes 0: the model has a Dropout layer and stayed eager
                 m.close()
+                host_api.set_share_clones(True)
             if cpu:
                 from oracle import train as otrain
                 ref = otrain.Sequential(cfg["spec"], params, dtype)

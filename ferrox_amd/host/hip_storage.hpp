@@ -63,6 +63,11 @@ class BackendManager {
     }
     // 0: mathematical conv gradients (the reference's GPU semantics); 1: the CPU backend's literal arithmetic
     int conv_grad_mode = 0;
+    // clone_storage() as a second owner of the same device block instead of a device-to-device copy.  Nothing reachable through
+    // the storage trait writes device memory in place (every op returns new storage, the &mut methods of storage/mod.rs:246-269
+    // change the view and materialise into a NEW block), so a shared clone cannot be told from a copied one.  Off for callers
+    // that do update tensors in place (the fused optimizers, a recorded step's batch).
+    bool share_clones = false;
 
   private:
     fx_ctx* ctx_ = nullptr;
@@ -168,6 +173,21 @@ template <typename T> class HipStorage {
     T* data() { return ptr_; }
     [[noreturn]] void cpu_data() const { throw Error("GPU storage has no CPU data. Use to_cpu() first"); }  // storage/cuda.rs:56-62
     Ptr clone_storage() const {  // CudaTensor::clone, context.rs:744-763
+        if (BackendManager::get().share_clones && ptr_ && !borrowed_) {
+            if (!owner_) {  // first clone: the block moves to a counted owner, which returns it to the pool when the last storage lets go
+                const uint64_t id = id_;
+                owner_ = std::shared_ptr<void>(static_cast<void*>(ptr_), [id](void* q) {
+                    if (BackendManager::get().has_hip()) fx_free(BackendManager::get().ctx(), Api<T>::dtype, q, id);
+                });
+            }
+            Ptr s(new HipStorage());
+            s->shape_ = shape_;
+            s->ptr_ = ptr_;
+            s->id_ = id_;
+            s->granted_ = granted_;
+            s->owner_ = owner_;
+            return s;
+        }
         Ptr s = alloc(shape_);
         fx_ok(fx_d2d(ctx(), s->ptr_, ptr_, (int64_t)(size() * sizeof(T))));
         return s;
@@ -421,7 +441,8 @@ template <typename T> class HipStorage {
     HipStorage() = default;
     static fx_ctx* ctx() { return BackendManager::get().ctx(); }
     void release() {
-        if (ptr_ && !borrowed_ && BackendManager::get().has_hip()) fx_free(ctx(), Api<T>::dtype, ptr_, id_);
+        if (owner_) owner_.reset();
+        else if (ptr_ && !borrowed_ && BackendManager::get().has_hip()) fx_free(ctx(), Api<T>::dtype, ptr_, id_);
         ptr_ = nullptr;
     }
     static void oai(const Shape& s, size_t axis, int64_t& outer, int64_t& ax, int64_t& inner) {
@@ -458,6 +479,7 @@ template <typename T> class HipStorage {
         std::swap(id_, r->id_);
         std::swap(granted_, r->granted_);
         std::swap(borrowed_, r->borrowed_);
+        std::swap(owner_, r->owner_);
         shape_ = ns;
     }
     Ptr pool2d(bool is_max, size_t k, size_t s, size_t p, const char* what) const {
@@ -533,6 +555,7 @@ template <typename T> class HipStorage {
     uint64_t id_ = 0;
     int64_t granted_ = 0;
     bool borrowed_ = false;
+    mutable std::shared_ptr<void> owner_;  // set once the block has more than one owner (share_clones)
 };
 
 // Tensor<T> (src/backend/tensor.rs:20-26) is a device tag plus a boxed storage; every method forwards to the

@@ -14,6 +14,8 @@ using namespace ferrox;
 
 namespace {
 thread_local std::string g_err;
+// clone_storage() of the op-by-op engines as a second owner of the block (default) or as the device copy the reference makes
+bool g_share_clones = true;
 
 struct ModelBase {
     virtual ~ModelBase() = default;
@@ -193,6 +195,7 @@ template <typename T> struct Model : ModelBase {
     // Moves the listed parameters (indices into the model's parameter list) out of their groups into a new group with
     // its own lr / weight decay / momentum (NaN = not set: the optimizer's value applies), ParameterGroup of optim/mod.rs:203-258.
     void add_param_group(const int* idx, int n, double lr, double wd, double mom) override {
+        enter();
         drop_graph();  // lr / weight decay / momentum and the pointer tables are arguments of the recorded kernels
         ParameterGroup<T> group("group" + std::to_string(opt->param_groups.size()));
         for (int k = 0; k < n; ++k) {
@@ -223,12 +226,14 @@ template <typename T> struct Model : ModelBase {
     }
     std::vector<uint8_t> optimizer_state() const override { return opt->state_dict().save_to_bytes(); }
     void load_optimizer_state(const uint8_t* data, size_t n) override {
+        enter();
         drop_graph();  // the moments move to new tensors: a recording made before would keep updating the old addresses
         opt->load_state_dict(OptimizerStateDict::load_from_bytes(data, n));
     }
     int num_params() const override { return (int)params.size(); }
     int64_t param_numel(int i) const override { return (int64_t)graph.get_tensor(params.at(i))->size(); }
     void set_batch(const void* xv, const Shape& xs, const void* yv, const Shape& ys) override {
+        enter();
         if (graph_on && graph_supported() && x && y && x->shape() == xs && y->shape() == ys) {
             // a recorded step reads the batch at the addresses it was recorded with: new data goes there
             fx_ok(fx_h2d(BackendManager::get().ctx(), x->data(), xv, (int64_t)(x->size() * sizeof(T))));
@@ -253,6 +258,9 @@ template <typename T> struct Model : ModelBase {
         std::vector<T> v = g->to_vec();
         std::memcpy(host, v.data(), v.size() * sizeof(T));
     }
+    // The fused engine updates parameters, moments and the batch in place, so its clones must stay copies; the op-by-op engines
+    // only ever create new storage, so theirs may share the block (hip_storage.hpp, share_clones).
+    void enter() const { BackendManager::get().share_clones = !fused && g_share_clones; }
     NodeId forward(NodeId in) {
         for (auto& l : layers) in = l->forward(graph, in);
         return in;
@@ -275,6 +283,7 @@ template <typename T> struct Model : ModelBase {
         return lval;
     }
     double train_step(bool optimizer_step) override {
+        enter();
         if (!x || !y) throw Error("set_batch was not called");
         if (graph_on && graph_supported()) {
             fx_ctx* c = BackendManager::get().ctx();
@@ -347,11 +356,13 @@ template <typename T> struct Model : ModelBase {
         std::memcpy(host, v.data(), v.size() * sizeof(T));
     }
     int64_t output_numel() override {
+        enter();
         const NodeId xin = graph.create_variable(x->clone_storage(), false);
         const NodeId pred = forward(xin);
         return (int64_t)graph.get_tensor(pred)->size();
     }
     void forward_only(void* host_out) override {
+        enter();
         const NodeId xin = graph.create_variable(x->clone_storage(), false);
         const NodeId pred = forward(xin);
         std::vector<T> v = graph.get_tensor(pred)->to_vec();
@@ -382,6 +393,8 @@ int fxh_init(int device, int conv_grad_mode, const fx_pool_config* cfg) {
 }
 void fxh_shutdown(void) { BackendManager::get().shutdown(); }
 // 0 = mathematical conv gradients, 1 = the CPU backend's literal arithmetic; read by every later deconv2d / cross_correlation2d
+// 1 (default): clones made by the op-by-op engines share their block; 0: they are device-to-device copies as in the reference
+void fxh_set_share_clones(int on) { g_share_clones = on != 0; }
 int fxh_set_conv_grad_mode(int mode) {
     return guarded([&] {
         if (mode != 0 && mode != 1) throw Error("conv gradient mode must be 0 or 1");

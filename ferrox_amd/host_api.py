@@ -45,6 +45,8 @@ lib.fxh_free.argtypes = [C.c_void_p]
 lib.fxh_free.restype = None
 lib.fxh_model_load_optimizer_state.argtypes = [C.c_void_p, C.c_char_p, C.c_int64]
 lib.fxh_set_conv_grad_mode.argtypes = [C.c_int]
+lib.fxh_set_share_clones.argtypes = [C.c_int]
+lib.fxh_set_share_clones.restype = None
 lib.fxh_model_configure.argtypes = [C.c_void_p, C.c_int, C.c_int]
 lib.fxh_model_enable_graph.argtypes = [C.c_void_p, C.c_int]
 lib.fxh_model_graph_info.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
@@ -67,6 +69,13 @@ def _check(rc):
 
 def init(device=0, conv_grad_mode=0, pool_config=None):
     _check(lib.fxh_init(device, conv_grad_mode, C.byref(pool_config) if pool_config is not None else None))
+
+
+def set_share_clones(on):
+    """True (default): clone_storage() in the op-by-op engines is a second owner of the same device block (nothing reachable
+    through the storage trait writes device memory in place, so it cannot be told from a copy); False: a device-to-device copy
+    per clone, as the reference's CUDA backend makes (cuda/context.rs:744-763)."""
+    lib.fxh_set_share_clones(1 if on else 0)
 
 
 def set_conv_grad_mode(mode):

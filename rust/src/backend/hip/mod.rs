@@ -10,7 +10,7 @@ use crate::backend::memory::PoolConfig;
 use ferrox_hip_sys as sys;
 use ndarray::ArrayD;
 use std::os::raw::{c_int, c_void};
-use std::sync::OnceLock;
+use std::sync::{Arc, OnceLock};
 
 /// Element types the library has kernels for.  `unsafe`: the implementor promises that `DTYPE` names its own layout.
 pub unsafe trait HipRepr: Copy + Send + Sync + 'static {
@@ -177,17 +177,34 @@ pub fn with_hip<R>(f: impl FnOnce(&HipContext) -> Result<R, String>) -> Result<R
     f(hip_context()?)
 }
 
-/// One pool block plus a shape: the device half of a tensor.  Always contiguous (views are materialised eagerly, like
-/// CUDAStorage does, storage/cuda.rs:795-911).
+/// One block of the pool.  It goes back to the pool when its last owner lets go (CudaTensor::drop, cuda/context.rs:726-742).
 #[derive(Debug)]
-pub struct HipTensor<T: HipRepr> {
+struct HipBlock<T: HipRepr> {
     ptr: *mut T,
     granted: i64,
     id: u64,
+}
+unsafe impl<T: HipRepr> Send for HipBlock<T> {}
+unsafe impl<T: HipRepr> Sync for HipBlock<T> {}
+
+impl<T: HipRepr> Drop for HipBlock<T> {
+    /// A failure is ignored, as in the reference.
+    fn drop(&mut self) {
+        if let Ok(ctx) = hip_context() {
+            unsafe { sys::fx_free(ctx.raw(), T::DTYPE, self.block.ptr as *mut c_void, self.id) };
+        }
+    }
+}
+
+/// A counted reference to a pool block plus a shape: the device half of a tensor.  Always contiguous (views are materialised
+/// eagerly, like CUDAStorage does, storage/cuda.rs:795-911).  No method of the storage trait writes a block after the call that
+/// produced it has returned (every op returns new storage; the `&mut self` view methods, storage/mod.rs:246-269, materialise into a
+/// new block), so `share()` -- a second owner of the same block -- cannot be told from the device copy of `try_clone()`.
+#[derive(Debug)]
+pub struct HipTensor<T: HipRepr> {
+    block: Arc<HipBlock<T>>,
     shape: Vec<usize>,
 }
-unsafe impl<T: HipRepr> Send for HipTensor<T> {}
-unsafe impl<T: HipRepr> Sync for HipTensor<T> {}
 
 impl<T: HipRepr> HipTensor<T> {
     /// CudaOps::get_tensor (cuda/ops.rs:121-133): the block comes from the pool and is NOT cleared.
@@ -196,11 +213,11 @@ impl<T: HipRepr> HipTensor<T> {
         let ctx = hip_context()?;
         let (mut p, mut granted, mut id) = (std::ptr::null_mut::<c_void>(), 0i64, 0u64);
         sys::check(unsafe { sys::fx_alloc(ctx.raw(), T::DTYPE, n as i64, &mut p, &mut granted, &mut id) })?;
-        Ok(HipTensor { ptr: p as *mut T, granted, id, shape: shape.to_vec() })
+        Ok(HipTensor { block: Arc::new(HipBlock { ptr: p as *mut T, granted, id }), shape: shape.to_vec() })
     }
     pub fn full(shape: &[usize], value: T) -> Result<Self, String> {
         let t = Self::alloc(shape)?;
-        sys::check(unsafe { T::fx_fill(hip_context()?.raw(), t.ptr, value, t.size() as i64) })?;
+        sys::check(unsafe { T::fx_fill(hip_context()?.raw(), t.block.ptr, value, t.size() as i64) })?;
         Ok(t)
     }
     /// host_to_device, cuda/context.rs:81-97
@@ -210,7 +227,7 @@ impl<T: HipRepr> HipTensor<T> {
             return Err(format!("Data length {} doesn't match shape {:?}", data.len(), shape));
         }
         let bytes = (data.len() * std::mem::size_of::<T>()) as i64;
-        sys::check(unsafe { sys::fx_h2d(hip_context()?.raw(), t.ptr as *mut c_void, data.as_ptr() as *const c_void, bytes) })?;
+        sys::check(unsafe { sys::fx_h2d(hip_context()?.raw(), t.block.ptr as *mut c_void, data.as_ptr() as *const c_void, bytes) })?;
         Ok(t)
     }
     /// CudaTensor::from_cpu_array, cuda/context.rs:330-351
@@ -230,7 +247,7 @@ impl<T: HipRepr> HipTensor<T> {
         let n = self.size();
         let mut v = Vec::<T>::with_capacity(n);
         let bytes = (n * std::mem::size_of::<T>()) as i64;
-        sys::check(unsafe { sys::fx_d2h(hip_context()?.raw(), v.as_mut_ptr() as *mut c_void, self.ptr as *const c_void, bytes) })?;
+        sys::check(unsafe { sys::fx_d2h(hip_context()?.raw(), v.as_mut_ptr() as *mut c_void, self.block.ptr as *const c_void, bytes) })?;
         unsafe { v.set_len(n) };
         Ok(v)
     }
@@ -238,15 +255,21 @@ impl<T: HipRepr> HipTensor<T> {
     pub fn try_clone(&self) -> Result<Self, String> {
         let t = Self::alloc(&self.shape)?;
         let bytes = (self.size() * std::mem::size_of::<T>()) as i64;
-        sys::check(unsafe { sys::fx_d2d(hip_context()?.raw(), t.ptr as *mut c_void, self.ptr as *const c_void, bytes) })?;
+        sys::check(unsafe { sys::fx_d2d(hip_context()?.raw(), t.block.ptr as *mut c_void, self.block.ptr as *const c_void, bytes) })?;
         Ok(t)
+    }
+    /// A second owner of the same block (what `clone_storage` hands out: 61 device copies per CNN training step become
+    /// reference-count bumps).  Callers that do write blocks in place (fused optimizer steps, a recorded step's batch) must use
+    /// `try_clone()` for anything that has to keep its old value.
+    pub fn share(&self) -> Self {
+        HipTensor { block: Arc::clone(&self.block), shape: self.shape.clone() }
     }
     pub fn shape(&self) -> &[usize] { &self.shape }
     pub fn size(&self) -> usize { self.shape.iter().product() }
     pub fn ndim(&self) -> usize { self.shape.len() }
-    pub fn ptr(&self) -> *const T { self.ptr }
-    pub fn ptr_mut(&self) -> *mut T { self.ptr }
-    pub fn granted_elems(&self) -> i64 { self.granted }
+    pub fn ptr(&self) -> *const T { self.block.ptr }
+    pub fn ptr_mut(&self) -> *mut T { self.block.ptr }
+    pub fn granted_elems(&self) -> i64 { self.block.granted }
     /// Metadata-only reshape (the storage is contiguous).
     pub fn set_shape(&mut self, shape: Vec<usize>) { self.shape = shape; }
 }
@@ -255,11 +278,3 @@ impl<T: HipRepr> Clone for HipTensor<T> {
     fn clone(&self) -> Self { self.try_clone().expect("device-to-device copy failed") }
 }
 
-impl<T: HipRepr> Drop for HipTensor<T> {
-    /// CudaTensor::drop, cuda/context.rs:726-742: the block goes back to the pool; a failure is ignored like there.
-    fn drop(&mut self) {
-        if let Ok(ctx) = hip_context() {
-            unsafe { sys::fx_free(ctx.raw(), T::DTYPE, self.ptr as *mut c_void, self.id) };
-        }
-    }
-}

@@ -228,8 +228,11 @@ where
     fn owns_data(&self) -> bool {
         true
     }
+    /// CudaTensor::clone (cuda/context.rs:744-763) is a device-to-device copy; here the clone is a second owner of the same
+    /// block, which the trait cannot tell apart (see HipTensor::share) and which takes the reference's per-node deep clones
+    /// (graph/mod.rs:735-751) and `Tensor::clone` (tensor.rs:34-48) out of the training step's device time.
     fn clone_storage(&self) -> Boxed<T> {
-        Self::boxed(self.hip_data.try_clone()?)
+        Self::boxed(self.hip_data.share())
     }
 
     // ---- elementwise (storage/cuda.rs:74-319): a CPU operand is uploaded first ----

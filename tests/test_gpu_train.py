@@ -155,6 +155,41 @@ def test_train_step_matches_oracle(host, case, dtype, engine):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("case", [c for c in CASES if c[0] in ("cnn_small", "cnn_cls_small", "mlp_small_momentum", "cnn_small_amsgrad_wd")],
+                         ids=["cnn_small", "cnn_cls_small", "mlp_small_momentum", "cnn_small_amsgrad_wd"])
+@pytest.mark.parametrize("engine", ["literal", "lean"])
+def test_shared_clones_cannot_be_told_from_copied_ones(host, case, dtype, engine):
+    """clone_storage() as a second owner of the block (the default of the op-by-op engines) against the device copy the
+    reference makes: loss, every gradient, every parameter and the optimizer's moments after several steps, bit for bit; and the
+    shared form asks the pool for fewer blocks."""
+    name, spec, in_shape, ncls, optspec, steps = case
+    params, x, y = kaiming_uniform_problem(spec, in_shape, ncls, 11, dtype)
+    runs = {}
+    try:
+        for share in (True, False):
+            host.set_share_clones(share)
+            model = host.Model(spec, params, optspec, dtype, literal_engine=engine == "literal", fused=False)
+            try:
+                model.set_batch(x, y)
+                st0 = host.pool_stats(dtype)
+                losses = [model.train_step() for _ in range(steps + 1)]
+                st1 = host.pool_stats(dtype)
+                runs[share] = (losses, [model.grad(i).copy() for i in range(len(params))], [model.param(i).copy() for i in range(len(params))],
+                               [s.copy() for s in model.state()] + [np.frombuffer(model.optimizer_state(), np.uint8).copy()], (st1["pool_hits"] + st1["pool_misses"]) - (st0["pool_hits"] + st0["pool_misses"]))
+            finally:
+                model.close()
+    finally:
+        host.set_share_clones(True)
+    a, b = runs[True], runs[False]
+    assert a[0] == b[0], (name, "loss", a[0], b[0])
+    for k in (1, 2, 3):
+        assert len(a[k]) == len(b[k])
+        for i, (u, v) in enumerate(zip(a[k], b[k])):
+            assert np.array_equal(u, v), (name, ("grad", "param", "state")[k - 1], i)
+    assert a[4] < b[4], (name, "pool requests", a[4], b[4])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("case", [c for c in CASES if c[0] in ("cnn_small", "cnn_c5")], ids=["cnn_small", "cnn_c5"])
 @pytest.mark.parametrize("engine", ["literal", "lean", "fused"])
 def test_train_step_with_cpu_literal_conv_gradients(host, case, dtype, engine):
