@@ -643,7 +643,7 @@ def bench_conv_sweep():
         return ctx.timer_stop() / runs
 
     out = {}
-    for hw, batch in ((64, 64), (32, 128), (16, 256), (8, 512)):
+    for hw, batch in ((128, 16), (112, 16), (64, 64), (32, 128), (16, 256), (8, 512)):
         for cin in (32, 64, 128, 256):
             for cout in (32, 64, 128, 256):
                 x = ctx.uniform((batch, cin, hw, hw), 1, -1.0, 1.0)

@@ -28,7 +28,8 @@ constexpr int CC = 8, NT = 256, KK = 9;
 constexpr int WPITCH = KK * CC + 1;         // 73
 constexpr int NXP_SHORT = 4, NXP_TALL = 10;  // patch rows are staged two per pass: up to 8 rows, or 20 (strided layers)
 constexpr int NXP_PERSIST = 5;              // persistent variant: up to 10 patch rows
-constexpr int LPR = 16;                     // lanes per patch row: W <= 64
+constexpr int NXP_WIDE = 6, NXP_WIDE2 = 8;  // persistent variant, rows of 65 to 128 floats: up to 6 patch rows; 129 to 256: 8 passes = 4 rows
+constexpr int LPR = 16;                     // lanes per patch row: W <= 64 (the persistent variant also takes 32: W <= 128)
 constexpr int SLACK = 16;
 constexpr size_t LDS_BUDGET = 72 * 1024;
 // persistent variant: fixed plane pitch (1 mod 4) and buffer size, so that buffer, channel pair and tap column are all
@@ -299,9 +300,13 @@ __global__ __launch_bounds__(256) void wimg2_kernel(const float* __restrict__ w,
 
 __device__ __forceinline__ float f4sel(const float4& v, int e) { return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w; }
 
-template <int WM, int TN, bool BIAS>
+// WIDE 1: rows of 65 to 128 floats.  A staging pass is then one patch row of the 8 channels (32 lanes per row) instead of two
+// (16 lanes per row), up to NXP_WIDE rows.  WIDE 2: rows of 129 to 256 floats, 64 lanes per row: a pass is one patch row of four
+// channels (a wave each), two passes per row, up to 4 rows.  Nothing else differs.
+template <int WM, int TN, bool BIAS, int WIDE = 0>
 __global__ __launch_bounds__(NT, 2) void conv_patch_persist_kernel(const Params p) {
-    constexpr int BM = 32 * WM, WN = 4 / WM, NPIX = 32 * TN * WN, NXP = NXP_PERSIST;
+    constexpr int BM = 32 * WM, WN = 4 / WM, NPIX = 32 * TN * WN, NXP = WIDE == 2 ? NXP_WIDE2 : WIDE ? NXP_WIDE : NXP_PERSIST;
+    constexpr int LPRK = LPR << WIDE;  // lanes per patch row
     constexpr int AIMG = KK * 64 * 4;  // floats of one (32-row block, chunk) weight image
     FX_DYNAMIC_SMEM(float, smem);
     const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
@@ -358,8 +363,12 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_persist_kernel(const Params 
     };
 
     // staging: thread t owns float4 column t % 16 of patch rows 2u + rp of channel (t / 16) % 8, rp = t / 128
+    // (WIDE 1: column t % 32 of patch row u of channel t / 32; WIDE 2: column t % 64 of patch row u / 2 of channel 4 (u % 2) + t / 64)
     const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    const int pq = tid & (LPR - 1), xc = (tid >> 4) & (CC - 1), rp = wave >> 1;  // rp scalar: row tests and row pointers stay on the SALU
+    const int pq = tid & (LPRK - 1), xc = WIDE == 2 ? wave : (tid / LPRK) & (CC - 1), rp = WIDE ? 0 : wave >> 1;  // rp, and with WIDE 2 xc, scalar: row tests and row pointers stay on the SALU
+    // patch row and additional channels of staging pass u
+    auto pass_row = [&](int u) __attribute__((always_inline)) { return WIDE == 2 ? u >> 1 : WIDE == 1 ? u : 2 * u + rp; };
+    auto pass_ch = [&](int u) __attribute__((always_inline)) { return WIDE == 2 ? 4 * (u & 1) : 0; };
     const bool x_lane = pq < ((p.W + 3) >> 2);
     const int xcol = min(4 * pq, p.W - 4);
     const uint32_t x_off = x_lane ? (uint32_t)(xc * p.H * p.W + xcol) * 4u : 0u;
@@ -374,8 +383,8 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_persist_kernel(const Params 
         const float* xsrc = p.x + ((i64)b * p.C + (i64)ch * CC) * p.H * p.W;
 #pragma unroll
         for (int u = 0; u < NXP; ++u) {
-            const int r = 2 * u + rp, iy = iy_base + r;
-            if (r < p.PR && iy >= 0 && iy < p.H) xv[u] = ldg4(xsrc + (i64)iy * p.W, x_off);  // scalar test
+            const int r = pass_row(u), iy = iy_base + r;
+            if (r < p.PR && iy >= 0 && iy < p.H) xv[u] = ldg4(xsrc + ((i64)pass_ch(u) * p.H + iy) * p.W, x_off);  // scalar test
             else xv[u] = zero4;
         }
     };
@@ -385,10 +394,10 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_persist_kernel(const Params 
         if (x_lane) {
 #pragma unroll
             for (int u = 0; u < NXP; ++u) {
-                const int r = 2 * u + rp;
+                const int r = pass_row(u);
                 if (r < p.PR) {  // scalar test
                     const float4 v = xv[u];
-                    float* d = smem + xd + r * p.PW;
+                    float* d = smem + xd + pass_ch(u) * PPLANE + r * p.PW;
                     d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
                 }
             }
@@ -529,6 +538,7 @@ struct Plan {
     i64 cost = 0;           // modelled cost: rounds of co-resident blocks x MFMA work of a block
     size_t smem = 0;
     bool persist = false;  // a plan for conv_patch_persist_kernel (persist_plan); PW is then its padded row pitch
+    int wide = 0;          // its instantiation for rows of 65 to 128 floats (1) or 129 to 256 (2)
     int bm() const { return 32 * WM; }
     int npix() const { return 32 * TN * (4 / WM); }
     i64 wimg() const { return (i64)bm() * WPITCH; }
@@ -568,7 +578,9 @@ inline bool persist_plan(Plan& pl, int wm, int tn, int num_cus, i64 B, i64 C, i6
     const i64 L = OH * OW, slots = 2 * (i64)std::max(1, num_cus);
     const i64 bm = 32 * wm, np = 32 * tn * (4 / wm), tiles = fx::ceil_div(L, np), mtiles = fx::ceil_div(M, bm);
     const i64 rows = std::min<i64>(OH, np % OW == 0 ? np / OW : (np - 1) / OW + 2), PR = (rows - 1) * sh + 3;
-    if (PR > 2 * NXP_PERSIST || mtiles * bm > M * 2 || tiles * np > L * 2 || B * tiles * mtiles > 0x7fffffff) return false;
+    const int wide = W > 8 * LPR ? 2 : W > 4 * LPR ? 1 : 0;  // wide rows: fewer patch rows, and a register budget without the fifth accumulator block
+    if (PR > (wide == 2 ? NXP_WIDE2 / 2 : wide ? NXP_WIDE : 2 * NXP_PERSIST) || (wide && tn > 4) || mtiles * bm > M * 2 || tiles * np > L * 2 || B * tiles * mtiles > 0x7fffffff)
+        return false;
     // patch row pitch: with unit column stride a run of 32 pixels that wraps to the next output row must continue 32
     // words further on (sh * pitch - OW a multiple of 32), else two of its lanes share a bank; the plain pitch when that
     // does not fit the plane.
@@ -581,6 +593,7 @@ inline bool persist_plan(Plan& pl, int wm, int tn, int num_cus, i64 B, i64 C, i6
     if (PR * pw2 > PPLANE) return false;
     pl = Plan();
     pl.persist = true;
+    pl.wide = wide;
     pl.WM = wm; pl.TN = tn; pl.PR = (int)PR; pl.tpi = (int)tiles; pl.PW = (int)pw2; pl.PLANE = PPLANE;
     pl.mtiles = (int)mtiles;
     pl.nchunks = (int)(C / CC);
@@ -596,7 +609,7 @@ inline bool persist_plan(Plan& pl, int wm, int tn, int num_cus, i64 B, i64 C, i6
 inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i64 OW, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph,
                       i64 pw) {
     Plan pl;
-    if (kh != 3 || kw != 3 || C % CC != 0 || W < 4 || W > 4 * LPR || sh > 8 || sw > 8) return pl;
+    if (kh != 3 || kw != 3 || C % CC != 0 || W < 4 || W > 16 * LPR || sh > 8 || sw > 8) return pl;
     const i64 L = OH * OW;
     // Maps of at most 64 pixels: a 128-pixel tile takes as many whole images as fit its pixels and the 20 patch rows
     // (8 x 8 and 7 x 7 maps: two images), provided that fills at least half of the tile.
@@ -628,7 +641,7 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
     }
     for (const auto& sp : shapes) {
         Plan q;
-        if (shape_plan(q, sp[0], sp[1], num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw) && (!best.ok || q.cost < best.cost)) best = q;
+        if (W <= 4 * LPR && shape_plan(q, sp[0], sp[1], num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw) && (!best.ok || q.cost < best.cost)) best = q;
     }
     return best;
 }
@@ -648,7 +661,7 @@ inline int candidates(Plan (&out)[MAX_CAND], int num_cus, i64 B, i64 C, i64 H, i
             ++n;
         }
     for (const auto& sp : shapes)
-        if (shape_plan(all[n], sp[0], sp[1], num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw)) {
+        if (W <= 4 * LPR && shape_plan(all[n], sp[0], sp[1], num_cus, B, C, H, W, M, OH, OW, sh, sw, ph, pw)) {
             if (best < 0 || all[n].cost < best) best = all[n].cost;
             ++n;
         }
@@ -689,23 +702,29 @@ inline int launch_persist(fx_ctx* c, const Plan& pl, const float* x, const float
         p.xcd_chunk = p.ntiles / 8;
     }
     const dim3 grid((unsigned)nblk);
-#define FX_CPK_PERSIST(WMV, TNV)                                                                                      \
-    case WMV * 16 + TNV: {                                                                                            \
-        static const hipError_t attr0 = hipFuncSetAttribute((const void*)conv_patch_persist_kernel<WMV, TNV, false>,  \
-                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)PP_LDS); \
-        static const hipError_t attr1 = hipFuncSetAttribute((const void*)conv_patch_persist_kernel<WMV, TNV, true>,   \
-                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)PP_LDS); \
-        FX_HIP_CHECK(attr0);                                                                                          \
-        FX_HIP_CHECK(attr1);                                                                                          \
-        if (bias) FX_LAUNCH(grid, dim3(NT), PP_LDS, c->stream, (p), conv_patch_persist_kernel<WMV, TNV, true>);                  \
-        else FX_LAUNCH(grid, dim3(NT), PP_LDS, c->stream, (p), conv_patch_persist_kernel<WMV, TNV, false>);                      \
+#define FX_CPK_PERSIST(WMV, TNV, WIDEV)                                                                                    \
+    case WIDEV * 256 + WMV * 16 + TNV: {                                                                                \
+        static const hipError_t attr0 = hipFuncSetAttribute((const void*)conv_patch_persist_kernel<WMV, TNV, false, WIDEV>,   \
+                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)PP_LDS);         \
+        static const hipError_t attr1 = hipFuncSetAttribute((const void*)conv_patch_persist_kernel<WMV, TNV, true, WIDEV>,    \
+                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)PP_LDS);         \
+        FX_HIP_CHECK(attr0);                                                                                                  \
+        FX_HIP_CHECK(attr1);                                                                                                  \
+        if (bias) FX_LAUNCH(grid, dim3(NT), PP_LDS, c->stream, (p), conv_patch_persist_kernel<WMV, TNV, true, WIDEV>);        \
+        else FX_LAUNCH(grid, dim3(NT), PP_LDS, c->stream, (p), conv_patch_persist_kernel<WMV, TNV, false, WIDEV>);            \
     } break;
-    switch (pl.WM * 16 + pl.TN) {
-        FX_CPK_PERSIST(4, 5)
-        FX_CPK_PERSIST(4, 4)
-        FX_CPK_PERSIST(2, 5)
-        FX_CPK_PERSIST(2, 4)
-        FX_CPK_PERSIST(2, 3)
+    switch (pl.wide * 256 + pl.WM * 16 + pl.TN) {
+        FX_CPK_PERSIST(4, 5, 0)
+        FX_CPK_PERSIST(4, 4, 0)
+        FX_CPK_PERSIST(2, 5, 0)
+        FX_CPK_PERSIST(2, 4, 0)
+        FX_CPK_PERSIST(2, 3, 0)
+        FX_CPK_PERSIST(4, 4, 1)
+        FX_CPK_PERSIST(2, 4, 1)
+        FX_CPK_PERSIST(2, 3, 1)
+        FX_CPK_PERSIST(4, 4, 2)
+        FX_CPK_PERSIST(2, 4, 2)
+        FX_CPK_PERSIST(2, 3, 2)
         default: FX_REQUIRE(false, "conv patch kernel (persistent): unexpected tile %d x %d", pl.WM, pl.TN);
     }
 #undef FX_CPK_PERSIST

@@ -46,7 +46,8 @@ struct Params {
     int stages, sps, spi;       // all stages, stages per split, stages per image
     int xcd_chunk;              // blocks / 8 when that divides (see the kernel), else 0
     int XRn;                    // NARROW kernels: patch rows per stage (a whole image)
-    FastDiv div_spi, div_xr;
+    int segw, nseg;             // SEG kernels: pixels per row segment, segments per row
+    FastDiv div_spi, div_xr, div_nseg;
     i64 part_stride;
 };
 
@@ -55,9 +56,14 @@ struct Params {
 // staged by (channel, row) pairs, 4 lanes per row and 64 pairs per pass, instead of 16 lanes per row: with 8-float rows
 // the regular map would leave 14 of 16 lanes idle and could hold only 4 of the image's 10 patch rows.
 // PAIRS > 0 (unit column stride, a wave's row segment = 2 PAIRS pixels): the pixel loop of a row is unrolled, see compute.
-template <int XR, int WMO, int WC, int WK, bool NARROW = false, int PAIRS = 0>
+// SEG (rows of more than 64 floats; unit column stride, padding 1, XR = 3): a stage is one SEGMENT of segw pixels of one output
+// row.  The patch under it is staged with four columns of halo on either side, taken from the neighbouring segments or zero
+// past the ends of the row: thread column q holds image columns sg * segw - 4 + 4q .. + 3, so LDS column j of a patch row is
+// image column sg * segw - 4 + j and every column of the patch is rewritten by every stage.
+template <int XR, int WMO, int WC, int WK, bool NARROW = false, int PAIRS = 0, bool SEG = false>
 __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
     static_assert(WMO * WC * WK == 4, "four waves");
+    static_assert(!SEG || (!NARROW && XR == 3), "segment stages: one output row, three patch rows");
     static_assert(!NARROW || WC == 1, "narrow staging holds 32 channel planes");
     constexpr int BM = 32 * WMO, CT = 32 * WC;
     constexpr int NG = BM / RPP, NXC = CT / RPP;
@@ -81,7 +87,7 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
     }
     const int c0 = bxi * CT, oc0 = byi * BM;
     const int L = p.oh * p.ow;
-    const int k4 = p.Kst >> 2, w4 = p.W >> 2;
+    const int k4 = p.Kst >> 2, w4 = SEG ? (p.segw >> 2) + 2 : p.W >> 2;
 
     for (int i = tid; i < CT * p.PLANE + SLACK; i += NT) Xs[i] = 0.f;  // the padding columns stay zero from here on
     f32x16 acc[KK];
@@ -98,23 +104,33 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
     const bool g_lane = pq < k4, x_lane = pq < w4;
     const bool full_m = oc0 + BM <= p.Cout;
     const uint32_t g_off = g_lane ? (uint32_t)(prow * L + 4 * pq) * 4u : 0u;
-    const uint32_t x_off = x_lane ? (uint32_t)(prow * p.H * p.W + 4 * pq) * 4u : 0u;
-    const uint32_t x_off0 = x_lane ? (uint32_t)(4 * pq) * 4u : 0u;  // the same columns in the first plane of a pass
+    uint32_t x_off = x_lane ? (uint32_t)(prow * p.H * p.W + 4 * pq) * 4u : 0u;
+    uint32_t x_off0 = x_lane ? (uint32_t)(4 * pq) * 4u : 0u;  // the same columns in the first plane of a pass
+    bool col_zero = false;  // SEG: this thread's columns of the stage in flight lie past an end of the row
     // ragged input-channel counts come only with the 1 x 1 x 4 layout; elsewhere this folds to a constant and the
     // staging code carries no channel tests (they cost the 128-row layout a fifth of its speed in registers)
     constexpr bool RAGGED_C = WMO == 1 && WC == 1;  // 1 x 1 x 4: the only layout the planner gives ragged counts to
     const bool full_c = !RAGGED_C || c0 + CT <= p.Cin;
     const int g_dst0 = prow * p.GP + 4 * pq;
-    const int x_dst0 = BM * p.GP + prow * p.PLANE + p.pw + 4 * pq;
+    const int x_dst0 = BM * p.GP + prow * p.PLANE + (SEG ? 0 : p.pw) + 4 * pq;
     // NARROW: float4 column and first (channel, row) pair of this thread
     const int npq = tid & 3, npp = tid >> 2;
     const bool nx_lane = npq < ((p.W + 3) >> 2);
     const int nxcol = min(4 * npq, p.W - 4), npairs = CT * p.XRn;
     auto prefetch = [&](int s) {
         const int b = (int)p.div_spi.div((uint32_t)s);
-        const int oy0 = (s - b * p.spi) * p.R;
+        int oy0 = (s - b * p.spi) * p.R, sg = 0;
+        if constexpr (SEG) {
+            const int rest = s - b * p.spi;
+            oy0 = (int)p.div_nseg.div((uint32_t)rest);
+            sg = rest - oy0 * p.nseg;
+            const int cx = sg * p.segw - 4 + 4 * pq;  // first image column of this thread's four
+            col_zero = cx < 0 || cx >= p.W;
+            x_off = x_lane && !col_zero ? (uint32_t)(prow * p.H * p.W + cx) * 4u : 0u;
+            x_off0 = x_lane && !col_zero ? (uint32_t)cx * 4u : 0u;
+        }
         const int iy0 = oy0 * p.sh - p.ph;
-        const float* gsrc = p.g + ((i64)b * p.Cout + oc0) * L + (i64)oy0 * p.ow;
+        const float* gsrc = p.g + ((i64)b * p.Cout + oc0) * L + (i64)oy0 * p.ow + sg * (SEG ? p.segw : 0);
         const float* xsrc = p.x + ((i64)b * p.Cin + c0) * p.H * p.W;
 #pragma unroll
         for (int u = 0; u < NG; ++u) {
@@ -180,7 +196,7 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
 #pragma unroll
                 for (int cu = 0; cu < NXC; ++cu) {
                     if (!(full_c || c0 + prow + cu * RPP < p.Cin)) continue;
-                    const float4 v = xv[r * NXC + cu];
+                    const float4 v = SEG && col_zero ? zero4 : xv[r * NXC + cu];
                     float* d = smem + xd + cu * RPP * p.PLANE + r * p.PW;
                     d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
                 }
@@ -188,9 +204,9 @@ __global__ __launch_bounds__(NT, 2) void wgrad_patch_kernel(const Params p) {
     };
 
     const int wmo = wave % WMO, wc = (wave / WMO) % WC, wk = wave / (WMO * WC);
-    const int seg = p.ow / WK;  // pixels of a row that this wave covers (a multiple of 2)
+    const int seg = (SEG ? p.segw : p.ow) / WK;  // pixels of a row that this wave covers (a multiple of 2)
     const float* ga = Gs + (wmo * 32 + l32) * p.GP + half + wk * seg;
-    const float* xb = Xs + (wc * 32 + l32) * p.PLANE + (half + wk * seg) * p.sw;
+    const float* xb = Xs + (wc * 32 + l32) * p.PLANE + (half + wk * seg) * p.sw + (SEG ? 4 - p.pw : 0);
     const int sw2 = 2 * p.sw;
     // One stage of MFMA work.  Two register sets alternate: while the MFMAs of one pixel pair run, the operands of
     // the next pair are read from LDS into the other set.  The reads past the end of a row land in the pitch
@@ -459,6 +475,7 @@ struct Plan {
     int R = 1, PR = 0, PW = 0, PLANE = 0, GP = 0, Kst = 0, splits = 1, sps = 1, stages = 0;
     int WMO = 4, WC = 1, WK = 1;  // wave layout
     bool narrow = false;          // whole-image stages with the (channel, row) pair staging
+    int segw = 0, nseg = 0;       // rows of more than 64 floats: pixels per row segment, segments per row (SEG kernels)
     size_t smem = 0;
     int bm() const { return 32 * WMO; }
     int ct() const { return 32 * WC; }
@@ -474,7 +491,16 @@ inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 k
     // output channels the padded block loses ([256,16,32,32] -> 64 0.098 -> 0.113 ms, [128,48,56,56] -> 128 0.549 -> 0.594 ms).
     const bool ragged_c = Cin % 32 != 0;
     if (ragged_c && (Cout > 32 || fx::ceil_div(Cin, (i64)32) * 32 > 2 * Cin)) return pl;
-    if (kh != KH || kw != KW || ow % 2 != 0 || W % 4 != 0 || W > 4 * LPR || sh > 8 || sw > 8) return pl;
+    if (kh != KH || kw != KW || ow % 2 != 0 || W % 4 != 0 || sh > 8 || sw > 8) return pl;
+    // Rows of more than 64 floats are walked in segments: the largest divisor of the row that is a multiple of 4 within 24 .. 56
+    // pixels (with its two halo vectors a staged patch row then fits the 16 lanes of a staging row).
+    i64 segw = 0;
+    if (W > 4 * LPR) {
+        if (sw != 1 || pw != 1 || ow != W) return pl;
+        for (i64 k = 56; k >= 24 && !segw; k -= 4)
+            if (ow % k == 0) segw = k;
+        if (!segw) return pl;
+    }
     // Wave layouts that fit the channel counts, the preferred one first.  Up to 32 output channels: one block of them, the
     // four waves split the input channels and / or the rows; up to 64: two blocks, the other two waves take more input
     // channels or split the rows.  A layout with 64 input channels per block holds only 3 patch rows (64 channel planes x
@@ -482,12 +508,13 @@ inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 k
     // next layout is tried.
     int cand[2][3], ncand = 0;
     auto add = [&](int a, int b, int c) { cand[ncand][0] = a; cand[ncand][1] = b; cand[ncand][2] = c; ++ncand; };
+    const i64 rowlen = segw ? segw : ow;  // pixels of a row in one stage
     if (Cout <= 32) {
-        if (Cin % 64 == 0 && ow % 4 == 0) add(1, 2, 2);
-        if (ow % 8 == 0) add(1, 1, 4);
+        if (Cin % 64 == 0 && rowlen % 4 == 0) add(1, 2, 2);
+        if (rowlen % 8 == 0) add(1, 1, 4);
     } else if (Cout <= 64) {
         if (Cin % 64 == 0) add(2, 2, 1);
-        if (ow % 4 == 0) add(2, 1, 2);
+        if (rowlen % 4 == 0) add(2, 1, 2);
     } else {
         add(4, 1, 1);
     }
@@ -495,24 +522,29 @@ inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 k
     for (int k = 0; k < ncand && !best; ++k) {
         pl.WMO = cand[k][0]; pl.WC = cand[k][1]; pl.WK = cand[k][2];
         const i64 max_pr = pl.WC == 2 ? 3 : 4;
-        for (int R = 1; R <= oh; ++R) {
-            if (oh % R || R * ow > 4 * LPR || (R - 1) * sh + kh > max_pr) continue;
-            if ((R * ow) % 4 == 0) best = R;
+        for (int R = 1; R <= (segw ? 1 : oh); ++R) {
+            if (oh % R || R * rowlen > 4 * LPR || (R - 1) * sh + kh > max_pr) continue;
+            if ((R * rowlen) % 4 == 0) best = R;
         }
         // measured at [256,32,32,32] -> 64, stride 2 (16 pixels per stage): 0.063 ms here against 0.050 ms for the implicit GEMM
         // (and with two output rows over five patch rows per stage: 0.063 against 0.053 ms there, 0.192 against 0.156 ms at
         // [128,64,56,56] -> 128 stride 2: a strided patch stages four input values per output pixel)
-        if (best * ow < 24) best = 0;
+        if (best * rowlen < 24) best = 0;
         if (!best) continue;
         pl.R = best;
         pl.PR = (int)((best - 1) * sh + kh);
-        pl.PW = (int)(W + 2 * pw);
+        pl.PW = (int)(segw ? segw + 8 : W + 2 * pw);
         pl.PLANE = odd_pitch(pl.PR * pl.PW);
-        pl.Kst = (int)(best * ow);
+        pl.Kst = (int)(best * rowlen);
         pl.GP = odd_pitch(pl.Kst);
         pl.smem = ((size_t)pl.bm() * pl.GP + (size_t)pl.ct() * pl.PLANE + SLACK) * sizeof(float);
         if (pl.WK > 1) pl.smem = std::max<size_t>(pl.smem, 4 * 16 * 64 * sizeof(float));  // the closing sum over the row segments
         if (pl.smem > LDS_BUDGET) best = 0;  // 64 planes of 3 x 66 floats: the next layout holds 32 planes
+    }
+    if (!best && segw) return pl;
+    if (segw) {
+        pl.segw = (int)segw;
+        pl.nseg = (int)(ow / segw);
     }
     if (!best) {
         // maps of at most 64 pixels with rows of at most 16 floats: one whole image per stage (NARROW kernels)
@@ -536,7 +568,8 @@ inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 k
         if (pl.smem > LDS_BUDGET) return pl;
     }
     const i64 BM = pl.bm(), CT = pl.ct();
-    pl.stages = (int)(B * (oh / best));
+    if (B * (oh / best) * std::max(1, pl.nseg) > 0x7fffffff) return pl;
+    pl.stages = (int)(B * (oh / best) * std::max(1, pl.nseg));
     const i64 tiles = fx::ceil_div(Cin, CT) * fx::ceil_div(Cout, BM);
     const i64 want = (i64)num_cus * 2;
     // at least four stages per block where there are that many: a block's partial sum (and its closing sum over the row
@@ -559,7 +592,9 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
     p.Cin = (int)Cin; p.H = (int)H; p.W = (int)W; p.Cout = (int)Cout; p.oh = (int)oh; p.ow = (int)ow;
     p.sh = (int)sh; p.sw = (int)sw; p.ph = (int)ph; p.pw = (int)pw;
     p.R = pl.R; p.PW = pl.PW; p.PLANE = pl.PLANE; p.GP = pl.GP; p.Kst = pl.Kst;
-    p.stages = pl.stages; p.sps = pl.sps; p.spi = (int)(oh / pl.R);
+    p.stages = pl.stages; p.sps = pl.sps; p.spi = (int)(oh / pl.R) * std::max(1, pl.nseg);
+    p.segw = pl.segw; p.nseg = std::max(1, pl.nseg);
+    p.div_nseg = FastDiv((uint32_t)p.nseg);
     p.div_spi = FastDiv((uint32_t)p.spi);
     p.XRn = pl.PR;
     p.div_xr = FastDiv((uint32_t)pl.PR);
@@ -576,7 +611,8 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
     } while (0)
     const int layout = pl.WMO * 100 + pl.WC * 10 + pl.WK;
     // pixel pairs of a wave's row segment when the unrolled pixel loop applies (unit column stride), else 0
-    const int pairs = sw == 1 && !pl.narrow && (ow / pl.WK) % 2 == 0 ? (int)(ow / pl.WK / 2) : 0;
+    const i64 rowlen = pl.segw ? pl.segw : ow;
+    const int pairs = sw == 1 && !pl.narrow && (rowlen / pl.WK) % 2 == 0 ? (int)(rowlen / pl.WK / 2) : 0;
 #define FX_WGP_LAUNCH_PAIRS(XRV, A, B_, C_, PV)                                                                       \
     do {                                                                                                              \
         static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_patch_kernel<XRV, A, B_, C_, false, PV>, \
@@ -591,7 +627,26 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
         FX_HIP_CHECK(attr);                                                                                           \
         FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), wgrad_patch_kernel<0, A, 1, C_, true>);                             \
     } while (0)
-    if (pl.narrow && layout == 411) FX_WGP_LAUNCH_NARROW(4, 1);
+#define FX_WGP_LAUNCH_SEG(A, B_, C_, PV)                                                                              \
+    do {                                                                                                              \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)wgrad_patch_kernel<3, A, B_, C_, false, PV, true>, \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
+        FX_HIP_CHECK(attr);                                                                                           \
+        FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), wgrad_patch_kernel<3, A, B_, C_, false, PV, true>);        \
+    } while (0)
+    if (pl.segw) {
+        FX_REQUIRE(pl.PR == 3, "wgrad patch kernel: segment stages hold three patch rows");
+        if (layout == 411 && pairs == 28) FX_WGP_LAUNCH_SEG(4, 1, 1, 28);
+        else if (layout == 411 && pairs == 16) FX_WGP_LAUNCH_SEG(4, 1, 1, 16);
+        else if (layout == 411) FX_WGP_LAUNCH_SEG(4, 1, 1, 0);
+        else if (layout == 221 && pairs == 28) FX_WGP_LAUNCH_SEG(2, 2, 1, 28);
+        else if (layout == 221 && pairs == 16) FX_WGP_LAUNCH_SEG(2, 2, 1, 16);
+        else if (layout == 221) FX_WGP_LAUNCH_SEG(2, 2, 1, 0);
+        else if (layout == 212) FX_WGP_LAUNCH_SEG(2, 1, 2, 0);
+        else if (layout == 122) FX_WGP_LAUNCH_SEG(1, 2, 2, 0);
+        else if (layout == 114) FX_WGP_LAUNCH_SEG(1, 1, 4, 0);
+        else FX_REQUIRE(false, "wgrad patch kernel: unexpected wave layout %d", layout);
+    } else if (pl.narrow && layout == 411) FX_WGP_LAUNCH_NARROW(4, 1);
     else if (pl.narrow && layout == 212) FX_WGP_LAUNCH_NARROW(2, 2);
     else if (pl.narrow && layout == 114) FX_WGP_LAUNCH_NARROW(1, 4);
     else if (pl.narrow) FX_REQUIRE(false, "wgrad patch kernel: unexpected narrow layout %d", layout);
@@ -610,6 +665,7 @@ inline int run(fx_ctx* c, const Plan& pl, const float* x, const float* g, float*
 #undef FX_WGP_LAUNCH
 #undef FX_WGP_LAUNCH_PAIRS
 #undef FX_WGP_LAUNCH_NARROW
+#undef FX_WGP_LAUNCH_SEG
     FX_LAUNCH_CHECK();
     const int n = (int)p.part_stride;
     const FastDiv div_row((uint32_t)(KK * Cin)), div_cin((uint32_t)Cin);

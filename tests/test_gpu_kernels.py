@@ -558,6 +558,11 @@ WGRAD_PATCH_CASES = [
     # strided layers (implicit GEMM)
     (3, 32, 32, 32, 64, (2, 2), (1, 1)), (2, 64, 56, 56, 128, (2, 2), (1, 1)), (2, 32, 16, 24, 70, (2, 1), (1, 1)),
     (2, 32, 13, 32, 48, (2, 2), (0, 1)),
+    # rows of more than 64 floats, walked in segments of 24 to 56 pixels with halo columns from the neighbouring segments: every
+    # wave layout, unrolled and plain pixel loops, two to seven segments per row, ragged channel counts, a row stride
+    (2, 32, 6, 112, 128, (1, 1), (1, 1)), (1, 64, 5, 128, 64, (1, 1), (1, 1)), (1, 32, 4, 224, 40, (1, 1), (1, 1)),
+    (2, 64, 3, 96, 32, (1, 1), (1, 1)), (1, 32, 4, 80, 20, (1, 1), (1, 1)), (1, 32, 3, 72, 130, (1, 1), (1, 1)),
+    (1, 16, 4, 112, 32, (1, 1), (1, 1)), (1, 64, 7, 128, 200, (2, 1), (1, 1)), (1, 128, 2, 256, 64, (1, 1), (1, 1)),
 ]
 
 
@@ -624,6 +629,13 @@ CONV_PATCH_CASES = [
     # channels, one to four tiles of 256 pixels per image
     (2, 8, 32, 32, 32, (2, 2), (1, 1)), (2, 16, 64, 64, 64, (2, 2), (1, 1)), (2, 24, 16, 64, 32, (2, 2), (1, 1)),
     (3, 40, 64, 32, 32, (2, 2), (1, 1)), (5, 8, 32, 32, 64, (2, 2), (1, 1)), (1, 8, 128, 64, 32, (2, 2), (1, 1)),
+    # rows of 65 to 128 floats (one patch row per staging pass): tiles 4x4, 2x4, 2x3, ragged channels and pixels, a row length that
+    # is not a multiple of four floats, no padding, two row strides
+    (2, 8, 10, 112, 128, (1, 1), (1, 1)), (1, 16, 6, 128, 64, (1, 1), (1, 1)), (2, 8, 7, 100, 40, (1, 1), (1, 1)), (1, 8, 9, 127, 72, (1, 1), (0, 0)),
+    (2, 24, 5, 66, 200, (1, 1), (1, 1)), (1, 8, 12, 96, 64, (2, 1), (1, 1)), (3, 8, 4, 128, 120, (1, 1), (1, 2)), (1, 16, 33, 80, 32, (1, 1), (1, 1)),
+    # rows of 129 to 256 floats (two staging passes per patch row)
+    (1, 8, 5, 224, 64, (1, 1), (1, 1)), (1, 16, 4, 256, 128, (1, 1), (1, 1)), (2, 8, 6, 160, 40, (1, 1), (1, 1)), (1, 8, 7, 130, 72, (1, 1), (0, 0)),
+    (1, 24, 3, 255, 200, (1, 1), (1, 1)),
 ]
 
 
