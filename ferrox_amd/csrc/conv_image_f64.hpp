@@ -159,43 +159,41 @@ inline int run(fx_ctx* c, const double* x, const double* w, double* y, i64 B, i6
     return FX_OK;
 }
 
-// ---- weight gradient of the same layer (1 to 3 channels: K = Cin * 9 <= 27 <= 32) -------------------------------------------
+// ---- weight gradient of the same layer (1 to 3 channels: K = Cin * 9 <= 27 <= 32), by row bands ---------------------------------
 //   dw[oc][c][ky][kx] = sum over (b, oy, ox) of g[b][oc][oy][ox] * x[b][c][oy + ky - 1][ox + kx - 1]
 // (grad_out_2d . im2col(x)^T, convolutions.rs:296-338).  The MFMA's 16 columns are (channel, tap) pairs -- two blocks of 16 hold
-// the K <= 27 of them -- its reduction runs over 4 pixels: lane l reads g[oc = l % 16 (+ 16)][pixel + l / 16] and
-// x[c][pixel + l / 16 shifted by the tap] for its pair (c, tap) = 16 block + l % 16, both from LDS, where a block has staged
-// 32 rows of g (256 pixels of one image, odd pitch) and the padded patch under them.  A wave takes one row of 32 pixels: 8 steps
-// of 4 MFMAs.  A block walks its range of tiles with the sums in registers, adds its eight waves' sums through LDS in wave
-// order and leaves one partial sum, laid out like dw; the ordered split sum adds the partials.  Bound by the one read of g.
-struct WParams {
-    const double* x;
-    const double* g;
-    const double* act;  // MASK: the layer's ReLU output; g is staged as g * (act > 0)
-    double* part;       // [splits][Cout][Cin * 9] (MASK: + [Cout] sums of the masked g behind each: the bias gradient)
-    i64 part_stride;    // doubles between the partial sums of two splits
-    int Cin, Cout, H, tpi;
-    int tiles, tps;  // B * tiles per image, tiles per split
-    FastDiv div_tpi;
-};
-
-constexpr int GPITCH = PIX + 1;
-
-// MASK: the gradient arrives unmasked and this layer's ReLU is applied while g is staged (g * (act > 0), the bits of
+// the K <= 27 of them -- and its reduction runs over 4 pixels.  Every WAVE is on its own: it takes a band of rb output rows of one
+// image, copies the rb + 2 input rows under it into its private piece of LDS, and feeds g to the MFMA straight from global memory
+// -- which pixel goes to which reduction step is free as long as both operands agree: lane (m = l % 16, q = l / 16) takes the 8
+// pixels 8 q .. 8 q + 7 of a row as four 16-byte loads per block of 16 output channels, two rows of loads in flight.  No block
+// barrier before the closing sum of the four waves (wave order, through LDS); one partial sum per block, laid out like dw, added by
+// the ordered split sum.  Bound by the one read of g.  (A block-tile form -- 256 pixels of g staged through LDS behind two barriers
+// per tile, blocks in lockstep -- ran [256,3,32,32] -> 32 in 24.7 us, with mask and bias sums 42.3 us; this one 20.7 / 27.0 us.)
+// MASK: the gradient arrives unmasked and this layer's ReLU is applied to g as it is loaded (g * (act > 0), the bits of
 // fx_relu_bwd); pair index K <= 27 of the 32 is free, and with an operand of 1.0 there the MFMA leaves the sums of the masked g
 // over the pixels in it: the bias gradient.
+struct RowWParams {
+    const double* x;
+    const double* g;
+    const double* act;
+    double* part;
+    i64 part_stride;
+    int Cin, Cout, H, B;
+    int rb, bands, ntasks;
+    int PLANE, wave_doubles;  // (rb + 2) * 34 doubles per channel plane; doubles of LDS per wave
+    FastDiv div_bands, div_pr;
+};
+constexpr int NTR = 256, ROW_NPV = 8;  // threads per block; double2 of the patch one lane keeps in flight
+
 template <bool MASK>
-__global__ __launch_bounds__(NT) void image_wgrad_f64_kernel(const WParams p) {
-    using S = Shape<32>;
-    constexpr int W = 32, TR = S::TR, PR = S::PR, PW = S::PW, PLANE = S::PLANE;
-    FX_DYNAMIC_SMEM(double, smem_w);
-    double* Gs = smem_w;                   // [32 oc][GPITCH]
-    double* Xs = smem_w + 32 * GPITCH;     // [CP planes][PR][PW], odd plane pitch
+__global__ __launch_bounds__(NTR) void image_wgrad_rows_f64_kernel(const RowWParams p) {
+    constexpr int W = 32, PW = W + 2, W2 = W / 2;
+    FX_DYNAMIC_SMEM(double, smem_r);
     const int tid = threadIdx.x, lane = tid & 63, kq = lane >> 4, l16 = lane & 15;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int task = blockIdx.x * 4 + wave;
+    double* patch = smem_r + wave * p.wave_doubles;
     const int oc0 = blockIdx.y * 32, L = p.H * W, K = p.Cin * KK;
-    const int t_beg = blockIdx.x * p.tps, t_end = min(p.tiles, t_beg + p.tps);
-
-    // this lane's (channel, tap) pairs: 16 nb + l16; pairs past K read a valid address and contribute zeros
     int xoff[2];
     bool pair_ok[2], pair_one[2];
 #pragma unroll
@@ -204,10 +202,8 @@ __global__ __launch_bounds__(NT) void image_wgrad_f64_kernel(const WParams p) {
         pair_ok[nb] = kp < K;
         pair_one[nb] = MASK && kp == K;
         const int c = pair_ok[nb] ? kp / KK : 0, t = pair_ok[nb] ? kp % KK : 0;
-        xoff[nb] = c * PLANE + (wave + t / 3) * PW + t % 3 + kq;  // pixel (row wave, column 4 s + kq): + 4 s per step
+        xoff[nb] = c * p.PLANE + (t / 3) * PW + t % 3 + 8 * kq;  // pixel (row 0, column 8 q): + PW per row, + j per step
     }
-    const int goff = l16 * GPITCH + wave * W + kq;                // + 16 GPITCH for the second block of output channels
-
     f64x4 acc[2][2];  // [oc block][pair block]
 #pragma unroll
     for (int m = 0; m < 2; ++m)
@@ -215,73 +211,87 @@ __global__ __launch_bounds__(NT) void image_wgrad_f64_kernel(const WParams p) {
         for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[m][nb][e] = 0.;
-    // the zero columns left and right of the map stay zero over the tiles
-    for (int i = tid; i < CP * PR * 2; i += NT) {
-        const int cr = i >> 1;
-        Xs[(cr / PR) * PLANE + (cr % PR) * PW + (i & 1) * (W + 1)] = 0.;
+    if (task < p.ntasks) {  // wave-uniform
+        const int b = (int)p.div_bands.div((uint32_t)task), oy0 = (task - b * p.bands) * p.rb;
+        const int nr = min(p.rb, p.H - oy0);
+        // lane's 8 pixels of output channel oc0 + 16 m + l16, row oy0 + r: four double2 per m
+        const i64 grow = ((i64)b * p.Cout + oc0 + l16) * L + (i64)oy0 * W + 8 * kq;
+        double2 gv[2][8], av[2][8];
+        auto load = [&](int set, int r) __attribute__((always_inline)) {
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const i64 off = grow + (i64)m * 16 * L + (i64)r * W + 2 * u;
+                    gv[set][4 * m + u] = *reinterpret_cast<const double2*>(p.g + off);
+                    if constexpr (MASK) av[set][4 * m + u] = *reinterpret_cast<const double2*>(p.act + off);
+                }
+        };
+        auto mul = [&](int set, int r) __attribute__((always_inline)) {
+            const double* src = patch + r * PW;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                double2 g0 = gv[set][u], g1 = gv[set][4 + u];
+                if constexpr (MASK) {
+                    const double2 a0 = av[set][u], a1 = av[set][4 + u];
+                    g0.x = g0.x * (a0.x > 0. ? 1. : 0.); g0.y = g0.y * (a0.y > 0. ? 1. : 0.);
+                    g1.x = g1.x * (a1.x > 0. ? 1. : 0.); g1.y = g1.y * (a1.y > 0. ? 1. : 0.);
+                }
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const double a0 = j ? g0.y : g0.x, a1 = j ? g1.y : g1.x;
+                    double b0 = src[xoff[0] + 2 * u + j], b1 = src[xoff[1] + 2 * u + j];
+                    if (!pair_ok[0]) b0 = pair_one[0] ? 1. : 0.;
+                    if (!pair_ok[1]) b1 = pair_one[1] ? 1. : 0.;
+                    acc[0][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(a0, b0, acc[0][0], 0, 0, 0);
+                    acc[0][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(a0, b1, acc[0][1], 0, 0, 0);
+                    acc[1][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(a1, b0, acc[1][0], 0, 0, 0);
+                    acc[1][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(a1, b1, acc[1][1], 0, 0, 0);
+                }
+            }
+        };
+        load(0, 0);
+        // the rows [oy0 - 1, oy0 + rb] of the Cin planes into the wave's patch, zero above and below the image and in columns 0 and 33
+        {
+            const int PR = p.rb + 2, items = p.Cin * PR * W2;
+            const double* xsrc = p.x + (i64)b * p.Cin * L;
+            double2 v[ROW_NPV];
+            int dst[ROW_NPV];
+#pragma unroll
+            for (int u = 0; u < ROW_NPV; ++u) {
+                const int i = min(lane + 64 * u, items - 1);
+                const int rc = i / W2, q2 = i - rc * W2;
+                const int c = (int)p.div_pr.div((uint32_t)rc), r = rc - c * PR;
+                const int iy = oy0 - 1 + r;
+                const bool ok = iy >= 0 && iy < p.H;
+                v[u] = *reinterpret_cast<const double2*>(xsrc + ((i64)c * p.H + (ok ? iy : 0)) * W + 2 * q2);
+                if (!ok) v[u] = make_double2(0., 0.);
+                dst[u] = c * p.PLANE + r * PW + 1 + 2 * q2;
+            }
+            for (int i = lane; i < p.Cin * PR; i += 64) {
+                const int c = (int)p.div_pr.div((uint32_t)i), r = i - c * PR;
+                patch[c * p.PLANE + r * PW] = 0.;
+                patch[c * p.PLANE + r * PW + W + 1] = 0.;
+            }
+#pragma unroll
+            for (int u = 0; u < ROW_NPV; ++u)
+                if (lane + 64 * u < items) {
+                    double* d = patch + dst[u];
+                    d[0] = v[u].x;
+                    d[1] = v[u].y;
+                }
+            __builtin_amdgcn_wave_barrier();  // one wave: its LDS accesses complete in program order, so this is a scheduling fence only
+        }
+        for (int r = 0; r < nr; r += 2) {
+            if (r + 1 < nr) load(1, r + 1);
+            mul(0, r);
+            if (r + 2 < nr) load(0, r + 2);
+            if (r + 1 < nr) mul(1, r + 1);
+        }
     }
-    for (int tl = t_beg; tl < t_end; ++tl) {
-        const int b = (int)p.div_tpi.div((uint32_t)tl), tile = tl - b * p.tpi;
-        const int oy0 = tile * TR, iy0 = oy0 - 1;
-        // g: 32 rows of 256 doubles, 8 double2 per thread
-        const double* gsrc = p.g + ((i64)b * p.Cout + oc0) * L + (i64)oy0 * W;
-        double2 gv[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int f = u * NT + tid, row = f >> 7, q = f & 127;
-            gv[u] = *reinterpret_cast<const double2*>(gsrc + (i64)row * L + 2 * q);
-            if constexpr (MASK) {
-                const double2 a = *reinterpret_cast<const double2*>(p.act + (gsrc - p.g) + (i64)row * L + 2 * q);
-                gv[u].x = gv[u].x * (a.x > 0. ? 1. : 0.);
-                gv[u].y = gv[u].y * (a.y > 0. ? 1. : 0.);
-            }
-        }
-        const double* xsrc = p.x + (i64)b * p.Cin * L;
-        double2 xv[2];
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int f = u * NT + tid;
-            xv[u] = make_double2(0., 0.);
-            if (f < S::X2) {
-                const int cr = f / (W / 2), q = f - cr * (W / 2), c = cr / PR, r = cr - c * PR;
-                const int iy = iy0 + r;
-                if (c < p.Cin && iy >= 0 && iy < p.H) xv[u] = *reinterpret_cast<const double2*>(xsrc + ((i64)c * p.H + iy) * W + 2 * q);
-            }
-        }
-        __syncthreads();  // the tile before has been read
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int f = u * NT + tid, row = f >> 7, q = f & 127;
-            double* d = Gs + row * GPITCH + 2 * q;
-            d[0] = gv[u].x;
-            d[1] = gv[u].y;
-        }
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int f = u * NT + tid;
-            if (f < S::X2) {
-                const int cr = f / (W / 2), q = f - cr * (W / 2), c = cr / PR, r = cr - c * PR;
-                double* d = Xs + c * PLANE + r * PW + 1 + 2 * q;
-                d[0] = xv[u].x;
-                d[1] = xv[u].y;
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int s = 0; s < W / 4; ++s) {
-            const double a0 = Gs[goff + 4 * s], a1 = Gs[goff + 16 * GPITCH + 4 * s];
-            double b0 = Xs[xoff[0] + 4 * s], b1 = Xs[xoff[1] + 4 * s];
-            if (!pair_ok[0]) b0 = pair_one[0] ? 1. : 0.;
-            if (!pair_ok[1]) b1 = pair_one[1] ? 1. : 0.;
-            acc[0][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(a0, b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(a0, b1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(a1, b0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(a1, b1, acc[1][1], 0, 0, 0);
-        }
-    }
-    // the eight waves' sums through LDS (the stage buffers are free after a barrier), added in wave order by waves 0 .. 3
+    // the four waves hold sums over different bands: added in wave order (the patches are dead after the barrier)
     __syncthreads();
-    double* red = smem_w;  // [8 waves][16 elements][64 lanes]
+    double* red = smem_r;  // [4 waves][16 elements][64 lanes]
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
@@ -292,11 +302,9 @@ __global__ __launch_bounds__(NT) void image_wgrad_f64_kernel(const WParams p) {
     double* out = p.part + (i64)blockIdx.x * p.part_stride + (i64)oc0 * K;
     double* bout = p.part + (i64)blockIdx.x * p.part_stride + (i64)p.Cout * K + oc0;
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-        const int el = 2 * wave + u, blk = el >> 2, e = el & 3;  // wave w finishes elements 2 w and 2 w + 1
-        double v = red[el * 64 + lane];
-#pragma unroll
-        for (int w = 1; w < 8; ++w) v = v + red[(w * 16 + el) * 64 + lane];
+    for (int u = 0; u < 4; ++u) {
+        const int el = 4 * wave + u, blk = el >> 2, e = el & 3;  // wave w finishes elements 4 w .. 4 w + 3
+        const double v = ((red[el * 64 + lane] + red[(16 + el) * 64 + lane]) + red[(32 + el) * 64 + lane]) + red[(48 + el) * 64 + lane];
         const int oc = 16 * (blk >> 1) + 4 * e + kq, kp = 16 * (blk & 1) + l16;
         if (kp < K) out[(i64)oc * K + kp] = v;
         if (MASK && kp == K) bout[oc] = v;
@@ -305,20 +313,25 @@ __global__ __launch_bounds__(NT) void image_wgrad_f64_kernel(const WParams p) {
 
 struct WPlan {
     bool ok = false;
-    int splits = 1, tps = 1, tiles = 0;
+    int rb = 0, tasks = 0, splits = 1;  // rows per band, bands in all, blocks (= partial sums)
+    i64 B = 0;
 };
 
 inline WPlan wgrad_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw) {
     WPlan pl;
-    if (kh != 3 || kw != 3 || sh != 1 || sw != 1 || ph != 1 || pw != 1 || Cin < 1 || Cin > 3 || W != 32 || H % (PIX / 32) != 0 || Cout % 32 != 0)
+    if (kh != 3 || kw != 3 || sh != 1 || sw != 1 || ph != 1 || pw != 1 || Cin < 1 || Cin > 3 || W != 32 || Cout % 32 != 0)
         return pl;
-    const i64 tiles = B * (H / (PIX / 32)), rows = Cout / 32;
-    if (tiles > 0x7fffffff || rows > 65535) return pl;
-    // two blocks per CU (78 KB of LDS each); at least two tiles per block where there are that many
-    const i64 splits = std::max<i64>(1, std::min<i64>(2 * (i64)num_cus / rows, std::max<i64>(1, tiles / 2)));
-    pl.tps = (int)fx::ceil_div(tiles, splits);
-    pl.splits = (int)fx::ceil_div(tiles, (i64)pl.tps);
-    pl.tiles = (int)tiles;
+    const i64 rows = Cout / 32;
+    if (rows > 65535 || B * H > 0x3fffffff) return pl;
+    pl.B = B;
+    // about one wave per SIMD (measured for the f32 twin of this kernel, conv_smallc.hpp), within what a lane stages
+    i64 rb = std::max<i64>(2, std::min<i64>(8, B * H / (4 * (i64)std::max(1, num_cus))));
+    rb = std::min<i64>(rb, H);
+    while (rb > 1 && Cin * (rb + 2) * 16 > ROW_NPV * 64) --rb;
+    if (Cin * (rb + 2) * 16 > ROW_NPV * 64) return pl;
+    pl.rb = (int)rb;
+    pl.tasks = (int)(B * fx::ceil_div(H, rb));
+    pl.splits = (int)fx::ceil_div((i64)pl.tasks, (i64)4);
     pl.ok = true;
     return pl;
 }
@@ -331,23 +344,20 @@ inline i64 wgrad_workspace_bytes(const WPlan& pl, i64 Cout, i64 Cin, bool with_b
 // act / db non-null: the masked variant (act 16-byte aligned as well).
 inline int run_wgrad(fx_ctx* c, const WPlan& pl, const double* x, const double* g, double* dw, double* part, i64 Cin, i64 H, i64 Cout,
                      const double* act = nullptr, double* db = nullptr) {
-    WParams p;
-    p.x = x; p.g = g; p.part = part; p.act = act;
-    p.part_stride = Cout * Cin * KK + (act ? Cout : 0);
-    p.Cin = (int)Cin; p.Cout = (int)Cout; p.H = (int)H;
-    p.tpi = (int)(H / (PIX / 32));
-    p.tiles = pl.tiles; p.tps = pl.tps;
-    p.div_tpi = FastDiv((uint32_t)p.tpi);
-    const size_t lds = std::max((size_t)(32 * GPITCH + Shape<32>::XCH), (size_t)8 * 16 * 64) * sizeof(double);
-    static const hipError_t attr = hipFuncSetAttribute((const void*)image_wgrad_f64_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-    static const hipError_t attr_m = hipFuncSetAttribute((const void*)image_wgrad_f64_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-    FX_HIP_CHECK(attr);
-    FX_HIP_CHECK(attr_m);
+    RowWParams q;
+    q.x = x; q.g = g; q.act = act; q.part = part;
+    q.part_stride = Cout * Cin * KK + (act ? Cout : 0);
+    q.Cin = (int)Cin; q.Cout = (int)Cout; q.H = (int)H; q.B = (int)pl.B;
+    q.rb = pl.rb; q.bands = (int)fx::ceil_div(H, (i64)pl.rb); q.ntasks = pl.tasks;
+    q.PLANE = (pl.rb + 2) * 34;
+    q.wave_doubles = (int)Cin * q.PLANE;
+    q.div_bands = FastDiv((uint32_t)q.bands); q.div_pr = FastDiv((uint32_t)(pl.rb + 2));
+    const size_t lds = std::max((size_t)4 * q.wave_doubles, (size_t)4 * 16 * 64) * sizeof(double);
     const dim3 grid((unsigned)pl.splits, (unsigned)(Cout / 32));
-    if (act) FX_LAUNCH(grid, dim3(NT), lds, c->stream, (p), image_wgrad_f64_kernel<true>);
-    else FX_LAUNCH(grid, dim3(NT), lds, c->stream, (p), image_wgrad_f64_kernel<false>);
+    if (act) FX_LAUNCH(grid, dim3(NTR), lds, c->stream, (q), image_wgrad_rows_f64_kernel<true>);
+    else FX_LAUNCH(grid, dim3(NTR), lds, c->stream, (q), image_wgrad_rows_f64_kernel<false>);
     FX_LAUNCH_CHECK();
-    if (act) return igemm::launch_splitk_reduce_pair<double>(c, part, p.part_stride, pl.splits, dw, Cout * Cin * KK, db, Cout);
+    if (act) return igemm::launch_splitk_reduce_pair<double>(c, part, q.part_stride, pl.splits, dw, Cout * Cin * KK, db, Cout);
     return igemm::launch_splitk_reduce<double>(c, part, dw, Cout * Cin * KK, pl.splits);
 }
 

@@ -579,6 +579,9 @@ inline bool persist_plan(Plan& pl, int wm, int tn, int num_cus, i64 B, i64 C, i6
     const i64 bm = 32 * wm, np = 32 * tn * (4 / wm), tiles = fx::ceil_div(L, np), mtiles = fx::ceil_div(M, bm);
     const i64 rows = std::min<i64>(OH, np % OW == 0 ? np / OW : (np - 1) / OW + 2), PR = (rows - 1) * sh + 3;
     const int wide = W > 8 * LPR ? 2 : W > 4 * LPR ? 1 : 0;  // wide rows: fewer patch rows, and a register budget without the fifth accumulator block
+    // wide rows have no 32-row tile: a 64-row tile over 32 channels measured 48 against 67 TFLOP/s for the implicit GEMM
+    // ([16,64,112,112] <- 32 data gradient), so at most a third of the rows may be padding there
+    if (wide && mtiles * bm * 2 > M * 3) return false;
     if (PR > (wide == 2 ? NXP_WIDE2 / 2 : wide ? NXP_WIDE : 2 * NXP_PERSIST) || (wide && tn > 4) || mtiles * bm > M * 2 || tiles * np > L * 2 || B * tiles * mtiles > 0x7fffffff)
         return false;
     // patch row pitch: with unit column stride a run of 32 pixels that wraps to the next output row must continue 32

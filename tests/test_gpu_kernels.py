@@ -787,6 +787,8 @@ SMALLC_CASES = [  # B, Cin, H, W, Cout, (sh, sw), (ph, pw)
     (2, 3, 14, 14, 32, (1, 1), (1, 1)), (2, 1, 9, 7, 16, (1, 1), (1, 1)), (2, 3, 12, 30, 8, (1, 1), (1, 1)), (3, 1, 8, 5, 8, (1, 1), (1, 1)),
     # rows of 128 floats (two per tile): the reference's own benchmark layer (kernels/benchmark.cu:856-860) and neighbours
     (1, 3, 128, 128, 32, (1, 1), (1, 1)), (2, 1, 6, 128, 40, (1, 1), (1, 1)), (1, 2, 7, 256, 8, (2, 2), (1, 1)), (2, 3, 5, 128, 16, (1, 1), (0, 0)),
+    # row-band weight gradient: bands of 4 and 8 rows that do not divide the height, two blocks of 32 pixels per row, ragged Cout
+    (130, 2, 33, 32, 40, (1, 1), (1, 1)), (300, 1, 30, 32, 32, (1, 1), (1, 1)), (70, 3, 30, 64, 8, (1, 1), (1, 1)),
 ]
 
 
@@ -830,6 +832,16 @@ def test_conv2d_image_layer_kernels(ctx, orc):
         assert np.array_equal(out.numpy(), gw), case
 
 
+# maps 32 wide, heights a multiple of 8, output channels a multiple of 32: the image-layer kernel of conv_image_f64.hpp (1 to 4
+# channels, one to five tiles per image, one to three blocks of output channels)
+IMAGE_F64_EXTRA = [
+    (3, 1, 8, 32, 64, (1, 1), (1, 1)), (2, 4, 40, 32, 96, (1, 1), (1, 1)), (5, 2, 24, 32, 32, (1, 1), (1, 1)),
+    (9, 3, 32, 32, 32, (1, 1), (1, 1)), (70, 3, 32, 32, 64, (1, 1), (1, 1)),
+    # row-band weight gradient: heights that are not multiples of 8 or of the band, bands of 4 and 8 rows
+    (9, 3, 33, 32, 32, (1, 1), (1, 1)), (140, 2, 30, 32, 32, (1, 1), (1, 1)), (300, 1, 30, 32, 64, (1, 1), (1, 1)),
+]
+
+
 def test_conv2d_f64_image_layer_forward(ctx, orc):
     """Image layers in f64 (1 to 4 input channels, K = Cin * 9 below two slabs of the implicit GEMM): forward, bias + ReLU in the store,
     weight gradient."""
@@ -837,11 +849,7 @@ def test_conv2d_f64_image_layer_forward(ctx, orc):
     import torch.nn.functional as F
     from ferrox_amd import capi
     rng = np.random.default_rng(63)
-    # maps 32 wide, heights a multiple of 8, output channels a multiple of 32: the image-layer kernel of conv_image_f64.hpp (1 to 4
-    # channels, one to five tiles per image, one to three blocks of output channels)
-    extra = [(3, 1, 8, 32, 64, (1, 1), (1, 1)), (2, 4, 40, 32, 96, (1, 1), (1, 1)), (5, 2, 24, 32, 32, (1, 1), (1, 1)),
-             (9, 3, 32, 32, 32, (1, 1), (1, 1)), (70, 3, 32, 32, 64, (1, 1), (1, 1))]
-    for (B, Cin, H, W, Cout, st, pd) in SMALLC_CASES + extra:
+    for (B, Cin, H, W, Cout, st, pd) in SMALLC_CASES + IMAGE_F64_EXTRA:
         case = (B, Cin, H, W, Cout, st, pd)
         x = rng.uniform(-1, 1, (B, Cin, H, W))
         w = rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9))

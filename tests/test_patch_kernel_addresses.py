@@ -87,6 +87,8 @@ def gpu_test_cases():
     for (B, Cin, H, W, Cout, st, pd) in tk.SMALLC_CASES:
         for dt in ("f32", "f64"):
             add("image_layer", dt, B, Cin, H, W, Cout, 3, st, pd)
+    for (B, Cin, H, W, Cout, st, pd) in tk.IMAGE_F64_EXTRA:
+        add("image_layer_f64", "f64", B, Cin, H, W, Cout, 3, st, pd)
     for (B, Cin, H, W, Cout) in tk.POINTWISE_CASES:
         add("pointwise", "f32", B, Cin, H, W, Cout, 1, 1, 0)
     for (B, Cin, H, W, Cout, k, st, pd) in tk.STRIDED_DGRAD_CASES:
