@@ -12,6 +12,7 @@
 #include <cstdint>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <numeric>
 #include <sstream>
 #include <stdexcept>
@@ -174,6 +175,8 @@ template <typename T> class HipStorage {
     [[noreturn]] void cpu_data() const { throw Error("GPU storage has no CPU data. Use to_cpu() first"); }  // storage/cuda.rs:56-62
     Ptr clone_storage() const {  // CudaTensor::clone, context.rs:744-763
         if (BackendManager::get().share_clones && ptr_ && !borrowed_) {
+            static std::mutex first_clone;  // two threads may clone one storage through const references at the same time
+            std::lock_guard<std::mutex> lk(first_clone);
             if (!owner_) {  // first clone: the block moves to a counted owner, which returns it to the pool when the last storage lets go
                 const uint64_t id = id_;
                 owner_ = std::shared_ptr<void>(static_cast<void*>(ptr_), [id](void* q) {
