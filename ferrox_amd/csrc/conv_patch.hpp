@@ -617,7 +617,7 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
     // Maps of at most 64 pixels: a 128-pixel tile takes as many whole images as fit its pixels and the 20 patch rows
     // (8 x 8 and 7 x 7 maps: two images), provided that fills at least half of the tile.
     const i64 RPI = (OH - 1) * sh + 3;
-    if (L <= 64 && B >= 2) {
+    if (L <= 64 && B >= 2 && W <= 4 * LPR) {  // (its staging covers rows of at most 64 floats)
         const i64 nimg = std::min<i64>(std::min<i64>(128 / L, 2 * NXP_TALL / RPI), B);
         const int wm = M > 64 ? 4 : 2;
         const i64 bm = 32 * wm, mtiles = fx::ceil_div(M, bm);

@@ -1020,27 +1020,41 @@ def test_conv2d_pointwise_layers(ctx, orc):
         assert np.array_equal(out.numpy(), gw), case
 
 
-@pytest.mark.parametrize("seed,dtype", [(61, np.float32), (62, np.float32), (63, np.float32), (64, np.float32), (65, np.float64), (66, np.float64)])
-def test_conv2d_random_shapes_all_paths_vs_torch(ctx, seed, dtype):
-    """Seeded random 3x3 / 1x1 / 5x5 shapes biased towards the dispatch boundaries of the conv kernels (channel counts
-    around multiples of 8 / 16 / 32 / 64, widths around 64 and multiples of 4, strides 1-3, paddings 0-2): forward,
-    data gradient and weight gradient against torch in float64."""
-    import torch
-    import torch.nn.functional as F
+RANDOM_CONV_SEEDS = [(61, np.float32), (62, np.float32), (63, np.float32), (64, np.float32), (65, np.float64), (66, np.float64),
+                     (67, np.float32), (68, np.float32), (69, np.float64)]
+
+
+def random_conv_shapes(seed):
+    """Seeded random 3x3 / 1x1 / 5x5 layer shapes biased towards the dispatch boundaries of the conv kernels (channel counts around
+    multiples of 8 / 16 / 32 / 64, widths around 64 and multiples of 4, strides 1-3, paddings 0-2); seeds from 67 on draw rows of
+    72 to 256 floats (the wide-row paths of the patch kernels).  Also walked on the CPU before they run on a GPU."""
     rng = np.random.default_rng(seed)
     chans = [1, 3, 4, 8, 16, 24, 32, 40, 64, 65, 72, 96, 128, 136]
-    widths = [4, 6, 8, 12, 14, 16, 20, 28, 30, 32, 36, 56, 60, 64, 66, 68]
-    for it in range(70):
+    widths = [4, 6, 8, 12, 14, 16, 20, 28, 30, 32, 36, 56, 60, 64, 66, 68] if seed < 67 else [72, 80, 96, 100, 112, 126, 128, 130, 160, 192, 224, 256]
+    heights = [1, 2, 3, 5, 8, 9, 14, 28] if seed < 67 else [1, 2, 3, 4, 5, 7]
+    out = []
+    for it in range(70 if seed < 67 else 40):
         Cin, Cout = int(rng.choice(chans)), int(rng.choice(chans))
         k = int(rng.choice([3, 3, 3, 3, 1, 5]))
         sh, sw = int(rng.choice([1, 1, 1, 2, 3])), int(rng.choice([1, 1, 1, 2, 3]))
         ph, pw = int(rng.integers(0, 3)), int(rng.integers(0, 3))
         W = int(rng.choice(widths))
-        H = int(rng.choice([1, 2, 3, 5, 8, 9, 14, 28])) if rng.random() < 0.7 else W
+        H = int(rng.choice(heights)) if seed >= 67 or rng.random() < 0.7 else W
         B = int(rng.choice([1, 2, 3, 5]))
         if H + 2 * ph < k or W + 2 * pw < k or B * Cin * H * W > 1_500_000 or B * Cout * H * W > 3_000_000:
             continue
-        case = (it, B, Cin, H, W, Cout, k, (sh, sw), (ph, pw))
+        out.append((it, B, Cin, H, W, Cout, k, (sh, sw), (ph, pw)))
+    return out
+
+
+@pytest.mark.parametrize("seed,dtype", RANDOM_CONV_SEEDS)
+def test_conv2d_random_shapes_all_paths_vs_torch(ctx, seed, dtype):
+    """Forward, data gradient and weight gradient of random_conv_shapes(seed) against torch in float64."""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(seed + 1000)
+    for case in random_conv_shapes(seed):
+        it, B, Cin, H, W, Cout, k, (sh, sw), (ph, pw) = case
         x = rng.uniform(-1, 1, (B, Cin, H, W)).astype(dtype)
         w = (rng.standard_normal((Cout, Cin, k, k)) * np.sqrt(2.0 / (Cin * k * k))).astype(dtype)
         tx = torch.from_numpy(x).double().requires_grad_(True)
