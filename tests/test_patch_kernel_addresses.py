@@ -127,8 +127,8 @@ def test_the_walk_faults_when_a_buffer_is_16_bytes_short(walk_binary, which):
     code is entitled to, the walk of layers that use it must end in a fault that names the case."""
     cases = [("cnn_conv1", "f32", (3, 3, 32, 32, 32, 3, 3, 1, 1, 1, 1)), ("cnn_conv2", "f32", (3, 32, 32, 32, 64, 3, 3, 2, 2, 1, 1)),
              ("stride1", "f32", (2, 64, 16, 16, 128, 3, 3, 1, 1, 1, 1)), ("cnn_conv2", "f64", (3, 32, 32, 32, 64, 3, 3, 2, 2, 1, 1))]
-    if which == "ws":  # a layer whose weight gradient fills the advertised workspace to the last byte (256 partial sums)
-        cases.append(("roofline_layer_slice", "f32", (2, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1)))
+    if which == "ws":  # layers on the implicit GEMM, whose ordered K split fills the advertised workspace to the last byte
+        cases += [("five_by_five", "f32", (4, 16, 12, 12, 32, 5, 5, 1, 1, 2, 2)), ("strided_14", "f32", (8, 32, 14, 14, 64, 3, 3, 2, 2, 1, 1))]
     if which == "act":  # only layers with a fused conv + ReLU backward read the activation
         cases = [c for c in cases if c[0] != "stride1"]
     faults = 0
