@@ -90,6 +90,7 @@ _sig("fx_d2d", _vp, _vp, _vp, _i64)
 _sig("fx_scratch_info", _vp, C.POINTER(_vp), C.POINTER(_i64), C.POINTER(_i64), C.POINTER(_i64))
 _sig("fx_device_mem_info", _vp, C.POINTER(_i64), C.POINTER(_i64))
 _sig("fx_conv2d_bwd_relu_supported", _vp, _int, _int, *([_i64] * 11))
+_sig("fx_conv2d_last_path", _vp, restype=C.c_char_p)
 _sig("fx_conv2d_workspace_bytes", _int, _int, _int, *([_i64] * 11), restype=_i64)
 
 _CONV_INTS = [_i64] * 11
@@ -640,6 +641,10 @@ class Context:
 
     def sgd_step(self, p, g, lr):
         check(self._fn("sgd_step", p.dtype)(self.h, p.ptr, g.ptr, p.size, lr))
+
+    def conv2d_last_path(self):
+        """The kernel family the last convolution call on this context ran (a fixed string per dispatch branch)."""
+        return lib.fx_conv2d_last_path(self.h).decode()
 
     def conv2d_bwd_relu_supported(self, kind, dtype, x_shape, w_shape, stride, padding):
         B, Cin, H, W = x_shape

@@ -100,6 +100,7 @@ struct fx_ctx {
     // Recorded graphs keep the scratch address of their recording in their kernel arguments.  While any such graph is alive
     // (fx_graph_end .. fx_graph_destroy) a region that has to grow is parked here instead of freed, so a later launch of the
     // graph still finds its region; the parked regions are freed when the last graph is destroyed (or with the context).
+    const char* last_conv_path = "";  // which kernel family the last convolution call took (fx_conv2d_last_path)
     int live_graphs = 0;
     std::vector<void*> parked_scratch;
     std::mutex launch_mutex;

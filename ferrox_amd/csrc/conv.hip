@@ -43,6 +43,8 @@ typedef Tile<32, 256, 16, 32, 64> TileM32;    // 4 waves as 1x4, 32x64 each
 typedef Tile<64, 64, 16, 32, 32> TileSmall;   // 4 waves as 2x2, 32x32 each
 typedef Tile<32, 32, 16, 32, 32> TileTiny;    // one wave: first-layer weight gradients (Cout <= 32, Cin*kh*kw <= 32)
 // FX_CONV_GENERIC=1 in the environment sends every shape to the implicit-GEMM kernels (A/B timing, debugging).
+// What the last convolution call on this context ran (fx_conv2d_last_path): a fixed string per dispatch branch.
+#define FX_TAKES(c, name) ((c)->last_conv_path = (name))
 static bool generic_only() { const char* v = getenv("FX_CONV_GENERIC"); return v && atoi(v) != 0; }
 
 int gemm_t(fx_ctx* c, int ta, int tb, i64 M, i64 N, i64 K, const float* A, const float* B, float* C) { return fx_gemm_f32(c, ta, tb, M, N, K, A, B, C); }
@@ -232,37 +234,38 @@ int conv_fwd(fx_ctx* c, const T* x, const T* w, T* y, i64 B, i64 Cin, i64 H, i64
     std::lock_guard<std::mutex> lk(c->launch_mutex);
     if constexpr (sizeof(T) == 4) {
         const csc::Plan sp = smallc_plan<T>(c, d, false);
-        if (sp.ok && aligned16(x, x)) return csc::run_fwd(c, sp, x, w, y, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw, bias, relu);
+        if (sp.ok && aligned16(x, x)) return FX_TAKES(c, "image layer, tiles (csc)"), csc::run_fwd(c, sp, x, w, y, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw, bias, relu);
         if (!generic_only()) {
             const fw2::Plan f2 = fw2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
-            if (f2.ok && aligned16(x, w) && aligned16(y, y)) return fw2::run(c, f2, x, w, y, B, Cin, H, Cout, d.oh, bias, relu);
+            if (f2.ok && aligned16(x, w) && aligned16(y, y)) return FX_TAKES(c, "stride-2 patch (fw2)"), fw2::run(c, f2, x, w, y, B, Cin, H, Cout, d.oh, bias, relu);
         }
         const glk::Plan pp = pointwise_plan<T>(c, d, FX_CONV_FWD);
         if (pp.ok && aligned16(x, w) && aligned16(y, y)) {
             const i64 L = d.H * d.W;
-            return glk::run(c, pp, false, false, Cout, L, Cin, w, x, y, bias, relu, B, 0, Cin * L, Cout * L, 1);
+            return FX_TAKES(c, "1x1 as batched slab GEMM (glk)"), glk::run(c, pp, false, false, Cout, L, Cin, w, x, y, bias, relu, B, 0, Cin * L, Cout * L, 1);
         }
         const cpk::Plan pl = fwd_patch_plan<T>(c, d);
         if (pl.ok && aligned16(x, ws)) {
             float* wimg = (float*)(ws ? ws : c->get_scratch(need));
             if (!wimg) return FX_ERR_OOM;
-            return cpk::run(c, pl, x, w, y, wimg, 0, Cout, Cin, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw, bias, relu);
+            return FX_TAKES(c, "LDS patch (cpk)"), cpk::run(c, pl, x, w, y, wimg, 0, Cout, Cin, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw, bias, relu);
         }
     }
     if constexpr (sizeof(T) == 8) {
         if (!generic_only() && cim::eligible(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw) && aligned16(x, x) && aligned16(y, y))
-            return cim::run(c, x, w, y, B, Cin, H, Cout, bias, relu);
+            return FX_TAKES(c, "image layer (cim)"), cim::run(c, x, w, y, B, Cin, H, Cout, bias, relu);
         if (!generic_only()) {
             const fwd2::Plan f2 = fwd2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
-            if (f2.ok && aligned16(x, w) && aligned16(y, y)) return fwd2::run(c, f2, x, w, y, B, Cin, H, Cout, d.oh, bias, relu);
+            if (f2.ok && aligned16(x, w) && aligned16(y, y)) return FX_TAKES(c, "stride-2 patch (fwd2)"), fwd2::run(c, f2, x, w, y, B, Cin, H, Cout, d.oh, bias, relu);
         }
         const cpd::Plan pd = fwd_patch64_plan<T>(c, d);
         if (pd.ok && aligned16(x, ws) && aligned16(y, y)) {
             double* wimg = (double*)(ws ? ws : c->get_scratch(need));
             if (!wimg) return FX_ERR_OOM;
-            return cpd::run(c, pd, x, w, y, wimg, 0, Cout, Cin, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw, bias, relu);
+            return FX_TAKES(c, "LDS patch (cpd)"), cpd::run(c, pd, x, w, y, wimg, 0, Cout, Cin, B, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw, bias, relu);
         }
     }
+    FX_TAKES(c, "implicit GEMM");
     if (d.Cin % CONV_BK == 0) {
         T* wp = (T*)(ws ? ws : c->get_scratch(need));
         if (!wp) return FX_ERR_OOM;
@@ -498,6 +501,7 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
             FX_HIP_CHECK(hipMalloc((void**)&col, (size_t)need));
             own = true;
         }
+        FX_TAKES(c, "explicit GEMM + col2im (CPU-literal mode)");
         int rc = gemm_t(c, 1, 0, K, N, Cout, w, g, col);
         if (!rc) rc = col2im_t(c, col, dx, B, Cin, H, W, kh, kw, sh, sw, ph, pw, 1);
         if (own) {
@@ -506,35 +510,36 @@ int conv_dgrad(fx_ctx* c, const T* g, const T* w, T* dx, i64 B, i64 Cin, i64 H, 
         }
         return rc;
     }
-    if (dgrad_small_cin_ok<T>(d)) return dgrad_small_cin<T>(c, g, w, dx, d);
+    if (dgrad_small_cin_ok<T>(d)) return FX_TAKES(c, "direct gather, few input channels"), dgrad_small_cin<T>(c, g, w, dx, d);
     std::lock_guard<std::mutex> lk(c->launch_mutex);
     if constexpr (sizeof(T) == 4) {
         if (!generic_only()) {
             const dg2::Plan p2 = dg2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
-            if (p2.ok && aligned16(g, w) && aligned16(dx, dx)) return dg2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh);
+            if (p2.ok && aligned16(g, w) && aligned16(dx, dx)) return FX_TAKES(c, "stride-2 patch (dg2)"), dg2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh);
             const glk::Plan pp = pointwise_plan<T>(c, d, FX_CONV_DGRAD);
             if (pp.ok && aligned16(g, w) && aligned16(dx, dx)) {
                 const i64 L = d.H * d.W;
-                return glk::run(c, pp, true, false, Cin, L, Cout, w, g, dx, nullptr, 0, B, 0, Cout * L, Cin * L);
+                return FX_TAKES(c, "1x1 as batched slab GEMM (glk)"), glk::run(c, pp, true, false, Cin, L, Cout, w, g, dx, nullptr, 0, B, 0, Cout * L, Cin * L);
             }
         }
     } else {
         if (!generic_only()) {
             const dgd2::Plan p2 = dgd2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
-            if (p2.ok && aligned16(g, w) && aligned16(dx, dx)) return dgd2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh);
+            if (p2.ok && aligned16(g, w) && aligned16(dx, dx)) return FX_TAKES(c, "stride-2 patch (dgd2)"), dgd2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh);
         }
     }
     T* wt = (T*)(ws ? ws : c->get_scratch(need));
     if (!wt) return FX_ERR_OOM;
     if constexpr (sizeof(T) == 4) {
         const cpk::Plan pl = dgrad_patch_plan<T>(c, d, mode);
-        if (pl.ok && aligned16(g, wt)) return cpk::run(c, pl, g, w, dx, wt, 1, Cout, Cin, B, Cout, d.oh, d.ow, Cin, H, W, 1, 1, 2 - ph, 2 - pw);
+        if (pl.ok && aligned16(g, wt)) return FX_TAKES(c, "LDS patch (cpk)"), cpk::run(c, pl, g, w, dx, wt, 1, Cout, Cin, B, Cout, d.oh, d.ow, Cin, H, W, 1, 1, 2 - ph, 2 - pw);
     }
     if constexpr (sizeof(T) == 8) {
         const cpd::Plan pd = dgrad_patch64_plan<T>(c, d, mode);
-        if (pd.ok && aligned16(g, wt) && aligned16(dx, dx)) return cpd::run(c, pd, g, w, dx, wt, 1, Cout, Cin, B, Cout, d.oh, d.ow, Cin, H, W, 1, 1, 2 - ph, 2 - pw);
+        if (pd.ok && aligned16(g, wt) && aligned16(dx, dx)) return FX_TAKES(c, "LDS patch (cpd)"), cpd::run(c, pd, g, w, dx, wt, 1, Cout, Cin, B, Cout, d.oh, d.ow, Cin, H, W, 1, 1, 2 - ph, 2 - pw);
     }
-    if (dgrad_classes_ok<T>(d)) return dgrad_classes<T>(c, g, w, dx, wt, d);
+    if (dgrad_classes_ok<T>(d)) return FX_TAKES(c, "implicit GEMM by pixel classes"), dgrad_classes<T>(c, g, w, dx, wt, d);
+    FX_TAKES(c, "implicit GEMM");
     if (Cout % CONV_BK == 0) {
         if (int rc = permute_weights<T>(c, w, wt, d, 2)) return rc;
         switch (pick_tile(c, Cin, B * H * W)) {
@@ -694,17 +699,19 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
                 part = (float*)(ws ? ws : c->get_scratch(need));
                 if (!part) return FX_ERR_OOM;
             }
+            FX_TAKES(c, sp.rb ? "image layer, row bands (csc)" : "image layer, tiles (csc)");
             return csc::run_wgrad(c, sp, x, g, dw, part, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw);
         }
         const wg2::Plan p2 = patch_s2_plan<T>(c, d, mode);
         if (p2.ok && aligned16(x, g) && aligned16(ws, ws)) {
             float* part = (float*)(ws ? ws : c->get_scratch(need));
             if (!part) return FX_ERR_OOM;
-            return wg2::run(c, p2, x, g, dw, part, Cin, H, Cout, ph, d.oh);
+            return FX_TAKES(c, "stride-2 patch (wg2)"), wg2::run(c, p2, x, g, dw, part, Cin, H, Cout, ph, d.oh);
         }
         const glk::Plan pp = mode == 0 ? pointwise_plan<T>(c, d, FX_CONV_WGRAD) : glk::Plan();
         if (pp.ok && aligned16(x, g) && aligned16(ws, dw)) {
             const i64 L = d.H * d.W, n = Cout * Cin;
+            FX_TAKES(c, "1x1 as batched slab GEMM (glk)");
             if (B == 1) return glk::run(c, pp, false, true, Cout, Cin, L, g, x, dw, nullptr, 0);
             float* part = (float*)(ws ? ws : c->get_scratch(need));
             if (!part) return FX_ERR_OOM;
@@ -715,6 +722,7 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
         if (pl.ok && aligned16(x, g) && aligned16(ws, ws)) {
             float* part = (float*)(ws ? ws : c->get_scratch(need));
             if (!part) return FX_ERR_OOM;
+            FX_TAKES(c, pl.segw ? "LDS patch, row segments (wgp)" : "LDS patch (wgp)");
             return wgp::run(c, pl, x, g, dw, part, Cin, H, W, Cout, sh, sw, ph, pw, d.oh, d.ow);
         }
     }
@@ -724,22 +732,23 @@ int conv_wgrad(fx_ctx* c, const T* x, const T* g, T* dw, i64 B, i64 Cin, i64 H, 
             if (ip.ok && aligned16(x, g) && aligned16(ws, ws)) {
                 double* part = (double*)(ws ? ws : c->get_scratch(need));
                 if (!part) return FX_ERR_OOM;
-                return cim::run_wgrad(c, ip, x, g, dw, part, Cin, H, Cout);
+                return FX_TAKES(c, "image layer, row bands (cim)"), cim::run_wgrad(c, ip, x, g, dw, part, Cin, H, Cout);
             }
         }
         const wgd2::Plan q2 = patch64_s2_plan<T>(c, d, mode);
         if (q2.ok && aligned16(x, g) && aligned16(ws, ws)) {
             double* part = (double*)(ws ? ws : c->get_scratch(need));
             if (!part) return FX_ERR_OOM;
-            return wgd2::run(c, q2, x, g, dw, part, Cin, H, Cout, ph, d.oh);
+            return FX_TAKES(c, "stride-2 patch (wgd2)"), wgd2::run(c, q2, x, g, dw, part, Cin, H, Cout, ph, d.oh);
         }
         const wgd::Plan pd = patch64_plan<T>(c, d, mode);
         if (pd.ok && aligned16(x, g) && aligned16(ws, ws)) {
             double* part = (double*)(ws ? ws : c->get_scratch(need));
             if (!part) return FX_ERR_OOM;
-            return wgd::run(c, pd, x, g, dw, part, Cin, H, W, Cout, sh, ph, pw, d.oh, d.ow);
+            return FX_TAKES(c, "LDS patch (wgd)"), wgd::run(c, pd, x, g, dw, part, Cin, H, W, Cout, sh, ph, pw, d.oh, d.ow);
         }
     }
+    FX_TAKES(c, mode == 0 ? "implicit GEMM" : "implicit GEMM (CPU-literal mode)");
     if (d.Cout > 64 && d.Cin * d.kh * d.kw > 64) return wgrad_tile<T, TileM128>(c, x, g, dw, d, mode, ws);
     if (d.Cout <= 32 && d.Cin * d.kh * d.kw <= 32) return wgrad_tile<T, TileTiny>(c, x, g, dw, d, mode, ws);
     return wgrad_tile<T, TileSmall>(c, x, g, dw, d, mode, ws);
@@ -792,13 +801,14 @@ int conv_wgrad_relu_bias(fx_ctx* c, const T* x, const T* g, const T* act, T* dw,
                     part = (float*)(ws ? ws : c->get_scratch(need));
                     if (!part) return FX_ERR_OOM;
                 }
+                FX_TAKES(c, sp.rb ? "image layer, row bands (csc), ReLU mask and bias sums inside" : "image layer, tiles (csc), ReLU mask and bias sums inside");
                 return csc::run_wgrad(c, sp, x, g, dw, part, Cin, H, W, Cout, d.oh, d.ow, sh, sw, ph, pw, act, db);
             }
             const wg2::Plan p2 = patch_s2_plan<T>(c, d, 0);
             if (p2.ok) {
                 float* part = (float*)(ws ? ws : c->get_scratch(need));
                 if (!part) return FX_ERR_OOM;
-                return wg2::run(c, p2, x, g, dw, part, Cin, H, Cout, ph, d.oh, act, db);
+                return FX_TAKES(c, "stride-2 patch (wg2), ReLU mask and bias sums inside"), wg2::run(c, p2, x, g, dw, part, Cin, H, Cout, ph, d.oh, act, db);
             }
         }
     } else {
@@ -810,9 +820,9 @@ int conv_wgrad_relu_bias(fx_ctx* c, const T* x, const T* g, const T* act, T* dw,
             double* part = (double*)(ws ? ws : c->get_scratch(need));
             if (!part) return FX_ERR_OOM;
             const cim::WPlan ip = cim::wgrad_plan(c->num_cus, d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
-            if (ip.ok) return cim::run_wgrad(c, ip, x, g, dw, part, Cin, H, Cout, act, db);
+            if (ip.ok) return FX_TAKES(c, "image layer, row bands (cim), ReLU mask and bias sums inside"), cim::run_wgrad(c, ip, x, g, dw, part, Cin, H, Cout, act, db);
             const wgd2::Plan q2 = patch64_s2_plan<T>(c, d, 0);
-            if (q2.ok) return wgd2::run(c, q2, x, g, dw, part, Cin, H, Cout, ph, d.oh, act, db);
+            if (q2.ok) return FX_TAKES(c, "stride-2 patch (wgd2), ReLU mask and bias sums inside"), wgd2::run(c, q2, x, g, dw, part, Cin, H, Cout, ph, d.oh, act, db);
         }
     }
     fx::set_error("fx_conv2d_wgrad_relu_bias: no fused kernel for this shape, dtype or alignment (ask fx_conv2d_bwd_relu_supported; use "
@@ -831,13 +841,13 @@ int conv_dgrad_relu(fx_ctx* c, const T* g, const T* act, const T* w, T* dx, i64 
         if (bwd_relu_supported<T>(c->num_cus, FX_CONV_DGRAD, d) && aligned16(g, w) && aligned16(dx, act)) {
             std::lock_guard<std::mutex> lk(c->launch_mutex);
             const dg2::Plan p2 = dg2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
-            return dg2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh, act);
+            return FX_TAKES(c, "stride-2 patch (dg2), ReLU mask inside"), dg2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh, act);
         }
     } else {
         if (bwd_relu_supported<T>(c->num_cus, FX_CONV_DGRAD, d) && aligned16(g, w) && aligned16(dx, act)) {
             std::lock_guard<std::mutex> lk(c->launch_mutex);
             const dgd2::Plan p2 = dgd2::make_plan(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw, d.oh, d.ow);
-            return dgd2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh, act);
+            return FX_TAKES(c, "stride-2 patch (dgd2), ReLU mask inside"), dgd2::run(c, p2, g, w, dx, B, Cin, Cout, d.oh, act);
         }
     }
     fx::set_error("fx_conv2d_dgrad_relu: no fused kernel for this shape, dtype or alignment (ask fx_conv2d_bwd_relu_supported; use "
@@ -846,6 +856,8 @@ int conv_dgrad_relu(fx_ctx* c, const T* g, const T* act, const T* w, T* dx, i64 
 }
 
 }  // namespace
+
+extern "C" const char* fx_conv2d_last_path(fx_ctx* c) { return c ? c->last_conv_path : ""; }
 
 extern "C" int fx_conv2d_bwd_relu_supported(fx_ctx* c, int kind, int dtype, int64_t B, int64_t Cin, int64_t H, int64_t W, int64_t Cout,
                                             int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw) {

@@ -413,6 +413,12 @@ FX_DECLARE_KERNELS(double, f64)
  *     fx_h2d_async from such memory is recorded as "copy from this host address" and serves larger data the same way.
  * A launch is stream-ordered like any other call; results are bit-identical to the eager calls (same kernels, same
  * arguments). */
+/* Which kernel family the last convolution call on this context ran, as a fixed string: "LDS patch (cpk)", "LDS patch, row
+ * segments (wgp)", "image layer, row bands (csc)", "stride-2 patch (dg2)", "1x1 as batched slab GEMM (glk)", "implicit GEMM",
+ * "implicit GEMM by pixel classes", "explicit GEMM + col2im (CPU-literal mode)", ...  A call that returned an error leaves the
+ * previous value.  No counterpart in the reference (KernelManager looks kernels up by name, src/backend/cuda/kernels.rs:223-292):
+ * it lets a caller see when a layer shape falls off the specialised kernels onto the implicit GEMM. */
+const char* fx_conv2d_last_path(fx_ctx* ctx);
 /* 1 when fx_conv2d_wgrad_relu_bias (kind FX_CONV_WGRAD) / fx_conv2d_dgrad_relu (kind FX_CONV_DGRAD) has a fused kernel
  * for this dtype and shape on this context's device (16-byte aligned tensors assumed), else 0. */
 int fx_conv2d_bwd_relu_supported(fx_ctx* ctx, int kind, int dtype, int64_t B, int64_t Cin, int64_t H, int64_t W, int64_t Cout,

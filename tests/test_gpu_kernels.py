@@ -1020,6 +1020,40 @@ def test_conv2d_pointwise_layers(ctx, orc):
         assert np.array_equal(out.numpy(), gw), case
 
 
+EXPECTED_PATHS = [  # (B, Cin, H, W, Cout, k, stride, padding, dtype) -> kernel family of forward, data gradient, weight gradient
+    ((8, 64, 56, 56, 128, 3, 1, 1, np.float32), ("LDS patch (cpk)", "LDS patch (cpk)", "LDS patch (wgp)")),                       # the roofline layer
+    ((8, 64, 56, 56, 128, 3, 1, 1, np.float64), ("LDS patch (cpd)", "LDS patch (cpd)", "LDS patch (wgd)")),
+    ((16, 3, 32, 32, 32, 3, 1, 1, np.float32), ("image layer, tiles (csc)", "direct gather, few input channels", "image layer, row bands (csc)")),
+    ((16, 3, 32, 32, 32, 3, 1, 1, np.float64), ("image layer (cim)", "direct gather, few input channels", "image layer, row bands (cim)")),
+    ((16, 32, 32, 32, 64, 3, 2, 1, np.float32), ("LDS patch (cpk)", "stride-2 patch (dg2)", "stride-2 patch (wg2)")),
+    ((16, 32, 32, 32, 64, 3, 2, 1, np.float64), ("stride-2 patch (fwd2)", "stride-2 patch (dgd2)", "stride-2 patch (wgd2)")),
+    ((2, 64, 12, 112, 128, 3, 1, 1, np.float32), ("LDS patch (cpk)", "LDS patch (cpk)", "LDS patch, row segments (wgp)")),       # rows of 112 floats
+    ((1, 64, 6, 224, 64, 3, 1, 1, np.float32), ("LDS patch (cpk)", "LDS patch (cpk)", "LDS patch, row segments (wgp)")),         # rows of 224 floats
+    ((1, 3, 128, 128, 32, 3, 1, 1, np.float32), ("image layer, tiles (csc)", "direct gather, few input channels", "image layer, tiles (csc)")),  # the reference's benchmark layer
+    ((64, 256, 32, 32, 256, 1, 1, 0, np.float32), ("1x1 as batched slab GEMM (glk)",) * 3),                                     # enough tiles to fill the chip
+    ((4, 32, 20, 20, 64, 5, 1, 2, np.float32), ("implicit GEMM",) * 3),                                                          # no 5 x 5 kernels
+    ((4, 64, 56, 56, 128, 3, 2, 1, np.float32), ("LDS patch (cpk)", "implicit GEMM by pixel classes", "LDS patch (wgp)")),        # stride 2 off the 32 / 64 wide maps
+]
+
+
+def test_layers_take_the_kernels_written_for_them(ctx):
+    """A parity test passes on the implicit GEMM as well: this one asks the library which kernel family each call ran, for the
+    baseline layers and for one layer per specialised path, so that a planner that silently starts refusing a shape fails here."""
+    for (B, Cin, H, W, Cout, k, s, p, dtype), want in EXPECTED_PATHS:
+        oh, ow = (H + 2 * p - k) // s + 1, (W + 2 * p - k) // s + 1
+        x, w, g = ctx.uniform((B, Cin, H, W), 1, -1.0, 1.0, dtype), ctx.normal((Cout, Cin, k, k), 2, 0.0, 0.1, dtype), ctx.normal((B, Cout, oh, ow), 3, 0.0, 1.0, dtype)
+        got = []
+        ctx.conv2d_fwd(x, w, (s, s), (p, p)).free()
+        got.append(ctx.conv2d_last_path())
+        ctx.conv2d_dgrad(g, w, x.shape, (s, s), (p, p), 0).free()
+        got.append(ctx.conv2d_last_path())
+        ctx.conv2d_wgrad(x, g, w.shape, (s, s), (p, p), 0).free()
+        got.append(ctx.conv2d_last_path())
+        for a in (x, w, g):
+            a.free()
+        assert tuple(got) == want, ((B, Cin, H, W, Cout, k, s, p, np.dtype(dtype).name), got, want)
+
+
 RANDOM_CONV_SEEDS = [(61, np.float32), (62, np.float32), (63, np.float32), (64, np.float32), (65, np.float64), (66, np.float64),
                      (67, np.float32), (68, np.float32), (69, np.float64)]
 

@@ -97,6 +97,8 @@ def gpu_test_cases():
     for np_dt, dt in ((np.float32, "f32"), (np.float64, "f64")):
         for (B, Cin, H, W, Cout, st, pd) in tf.CONV_BWD_RELU_CASES[np_dt]:
             add("bwd_relu", dt, B, Cin, H, W, Cout, 3, st, pd)
+    for (B, Cin, H, W, Cout, k, st, pd, np_dt), _ in tk.EXPECTED_PATHS:
+        add("path", "f32" if np_dt == np.float32 else "f64", B, Cin, H, W, Cout, k, st, pd)
     for seed, np_dt in tk.RANDOM_CONV_SEEDS:
         for (it, B, Cin, H, W, Cout, k, st, pd) in tk.random_conv_shapes(seed):
             add("random_%d" % seed, "f32" if np_dt == np.float32 else "f64", B, Cin, H, W, Cout, k, st, pd)
