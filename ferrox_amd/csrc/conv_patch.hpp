@@ -12,6 +12,7 @@
 // test is left in the MFMA loop.  Ws arrives as a ready-made image (built once per call by wimg_kernel), so its
 // staging is a straight 16-byte copy; the patch rows use the regular thread-to-row map of the weight-gradient
 // kernel.  The next stage's global loads are issued before the MFMA loop of the current one.
+// Rows of up to 64 floats; the persistent variant further down also takes rows of up to 256 (its WIDE staging maps).
 #pragma once
 #include <array>
 #include <cstdio>

@@ -11,7 +11,7 @@
 //   wgrad     dw[oc][k] = sum_pixel g[oc][pixel] * patch(pixel, k)     A = g staged as Gs[oc][pixel] (odd pitch),
 //             B = patch with n = k; each wave reduces a quarter of the tile's pixels into one 32 x 32 accumulator, the
 //             four are added through LDS at the end, blocks over disjoint pixel ranges leave partial sums that
-//             the split-K reduction adds in order.
+//             the split-K reduction adds in order.  (Stride 1 / padding 1 layers take the row-band form further down.)
 // Both are bound by the activation tensor they write / read (33.5 MB at [256,32,32,32]), not by the MFMA pipe.
 #pragma once
 #include "igemm_core.hpp"

@@ -20,8 +20,9 @@
 //
 // Staging: thread t owns float4 column t % 16 of rows t/16 + 16u of either operand, so every address is a
 // per-thread constant plus a wave-uniform step.  The next stage's global loads are issued before the MFMA loop of
-// the current stage and held in registers until that loop is done.  That fixes the shapes served here (rows of at
-// most 64 floats, 3 or 4 patch rows); the implicit-GEMM kernel takes the rest.
+// the current stage and held in registers until that loop is done.  That fixes the shapes served here (stages of at
+// most 64 pixels over 3 or 4 patch rows: rows of at most 64 floats, or segments of wider rows, see SEG below); the
+// implicit-GEMM kernel takes the rest.
 #pragma once
 #include "igemm_core.hpp"
 

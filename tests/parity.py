@@ -15,7 +15,7 @@ rounding of zero: its mask flips, and one flipped position moves a first-layer w
 against the oracle in its own dtype, at the same 1x tolerance; such rows are recorded with bound = "oracle (relu kink)".
 
 Every check appends a row (label, case, dtype, err_gpu, err_oracle, bound); at the end of a GPU session the rows are
-written to gpurun_out/parity_errors.json (scratch output, used to build the error table of the design notes).
+written to parity_errors.json in the run's scratch output folder (the source of the achieved-error table).
 """
 import json
 import os
