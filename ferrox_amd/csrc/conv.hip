@@ -194,7 +194,10 @@ glk::Plan pointwise_plan(fx_ctx* c, const Dims& d, int kind) {
         glk::Plan pl;
         if (kind == FX_CONV_FWD) pl = glk::make_plan(cus, false, false, d.Cout, L, d.Cin, d.Cin, L, d.B);
         else if (kind == FX_CONV_DGRAD) pl = glk::make_plan(cus, true, false, d.Cin, L, d.Cout, d.Cin, L, d.B);
-        else if (d.B * d.Cout * d.Cin <= 0x7fffffff) pl = glk::make_plan(cus, false, true, d.Cout, d.Cin, L, L, L, d.B);
+        // (one partial result per image: where those outweigh the operands -- small maps under many channels -- the implicit GEMM's
+        // K split over the whole batch moves less; measured at [64,1024,14,14] -> 256: 63 against 66 TFLOP/s, at [64,256,14,14] -> 256: 46 against 31)
+        else if (d.B * d.Cout * d.Cin <= 0x7fffffff && 5 * d.Cout * d.Cin <= 4 * (d.Cout + d.Cin) * L)
+            pl = glk::make_plan(cus, false, true, d.Cout, d.Cin, L, L, L, d.B);
         // only with the 128-row tiles: the 64-row ones measured below the implicit GEMM here ([32,256,56,56] -> 64: 55 against
         // 63 TFLOP/s forward), the 128-row ones above it (-> 256: 92 against 86; [16,256,16,16] -> 1024: 94 against 64)
         return pl.ok && pl.WM == 4 ? pl : glk::Plan();

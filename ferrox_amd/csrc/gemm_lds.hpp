@@ -44,8 +44,11 @@ struct Params {
 };
 
 // TA: A is stored [K, M] (m contiguous); TB: B is stored [N, K] (k contiguous).
-template <int TN, int WM, bool TA, bool TB, bool BIAS>
+// KT (both operands k-contiguous only): K need not be a multiple of the stage depth -- the last stage loads what is left of the rows
+// (K a multiple of 4: a 16-byte vector is inside a row or past it) and parks zeros behind it.
+template <int TN, int WM, bool TA, bool TB, bool BIAS, bool KT = false>
 __global__ __launch_bounds__(NT, 2) void gemm_lds_kernel(const Params p) {
+    static_assert(!KT || (!TA && TB), "the K tail is handled for k-contiguous operands");
     constexpr int WN = 4 / WM, BM = 32 * WM, BN = 32 * TN * WN;
     constexpr int NACC = TN == 1 ? 2 : TN;  // accumulator blocks of a wave (TN == 1: even and odd MFMA steps apart)
     // The 128-row tiles keep one stage in LDS and rely on the CU's second block to cover staging; the 64-row tiles run where
@@ -105,19 +108,33 @@ __global__ __launch_bounds__(NT, 2) void gemm_lds_kernel(const Params p) {
         for (int u = 0; u < NB; ++u) b_off[u] = (uint32_t)((i64)(tid / Q + RS * u) * p.ldb + c4) * 4u;
     }
     float4 av[NA], bv[NB];
+    bool dead = false;  // KT: this thread's four k of the stage in flight lie past K (its loads re-read the stage's first vector)
     auto prefetch = [&](int k0) {
         const float* a = TA ? Ab + (i64)k0 * p.lda : Ab + k0;
         const float* b = TB ? Bb + k0 : Bb + (i64)k0 * p.ldb;
+        uint32_t back = 0;
+        if constexpr (KT) {
+            dead = k0 + 4 * (tid & 15) >= p.K;
+            back = dead ? 16u * (tid & 15) : 0u;
+        }
 #pragma unroll
-        for (int u = 0; u < NA; ++u) av[u] = ldg4(a, a_off[u]);
+        for (int u = 0; u < NA; ++u) av[u] = ldg4(a, a_off[u] - back);
 #pragma unroll
-        for (int u = 0; u < NB; ++u) bv[u] = ldg4(b, b_off[u]);
+        for (int u = 0; u < NB; ++u) bv[u] = ldg4(b, b_off[u] - back);
     };
     auto park = [&](int buf) {
         int t = tid;
         FX_PIN_VGPR(t);  // recompute the LDS addresses here instead of keeping them alive over the MFMA loop
         float* const As = smem + buf * (ASZ + BSZ);
         float* const Bs = As + ASZ;
+        if constexpr (KT) {
+            if (dead) {
+#pragma unroll
+                for (int u = 0; u < NA; ++u) av[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int u = 0; u < NB; ++u) bv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
         if (!TA) {
 #pragma unroll
             for (int u = 0; u < NA; ++u) {
@@ -269,7 +286,8 @@ struct Plan {
 // products of this shape that share the launch (their tiles count towards filling the chip).
 inline Plan make_plan(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, i64 lda, i64 ldb, i64 batch = 1) {
     Plan pl;
-    if (K < 2 * KC || K % KC != 0 || lda % 4 != 0 || ldb % 4 != 0 || M < 64 || N < 64) return pl;
+    // (a K that is no multiple of the stage depth: only with both operands k-contiguous, see KT in the kernel)
+    if (K < 2 * KC || (K % KC != 0 && !(K % 4 == 0 && !ta && tb)) || lda % 4 != 0 || ldb % 4 != 0 || M < 64 || N < 64) return pl;
     if ((ta && M % 4 != 0) || (!tb && N % 4 != 0)) return pl;
     // tile shape: the one with the least (rounds of co-resident blocks) x (work of a block); a nearly empty last round
     // costs as much as a full one (3072 x 3072: 576 tiles of 128 x 128 take two rounds, 1152 of 128 x 64 take 2.25).  The
@@ -303,17 +321,20 @@ inline Plan make_plan(int num_cus, bool ta, bool tb, i64 M, i64 N, i64 K, i64 ld
     return pl;
 }
 
-template <int TN, int WM, bool TA, bool TB>
+template <int TN, int WM, bool TA, bool TB, bool KT = false>
 inline int launch(fx_ctx* c, const Plan& pl, const Params& p, int batch) {
     const dim3 grid((unsigned)p.tiles, (unsigned)batch), blk(NT);
-    static const hipError_t attr0 = hipFuncSetAttribute((const void*)gemm_lds_kernel<TN, WM, TA, TB, false>,
+    if constexpr (!KT && !TA && TB) {
+        if (p.K % KC != 0) return launch<TN, WM, TA, TB, true>(c, pl, p, batch);
+    }
+    static const hipError_t attr0 = hipFuncSetAttribute((const void*)gemm_lds_kernel<TN, WM, TA, TB, false, KT>,
                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)(WM == 2 ? LDS_BUDGET_MID : LDS_BUDGET));
-    static const hipError_t attr1 = hipFuncSetAttribute((const void*)gemm_lds_kernel<TN, WM, TA, TB, true>,
+    static const hipError_t attr1 = hipFuncSetAttribute((const void*)gemm_lds_kernel<TN, WM, TA, TB, true, KT>,
                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)(WM == 2 ? LDS_BUDGET_MID : LDS_BUDGET));
     FX_HIP_CHECK(attr0);
     FX_HIP_CHECK(attr1);
-    if (p.bias) FX_LAUNCH(grid, blk, pl.smem, c->stream, (p), gemm_lds_kernel<TN, WM, TA, TB, true>);
-    else FX_LAUNCH(grid, blk, pl.smem, c->stream, (p), gemm_lds_kernel<TN, WM, TA, TB, false>);
+    if (p.bias) FX_LAUNCH(grid, blk, pl.smem, c->stream, (p), gemm_lds_kernel<TN, WM, TA, TB, true, KT>);
+    else FX_LAUNCH(grid, blk, pl.smem, c->stream, (p), gemm_lds_kernel<TN, WM, TA, TB, false, KT>);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
