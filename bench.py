@@ -115,7 +115,7 @@ def bench_conv(ctx, steps, warmup, dtype=np.float32, B=None):
     per_pass = {}
     for name, fn in passes.items():
         ms = time_stream(ctx, fn, steps, warmup)
-        per_pass[name] = {"ms": ms, "tflops": flop / ms / 1e9}
+        per_pass[name] = {"ms": ms, "tflops": flop / ms / 1e9, "kernel_family": ctx.conv2d_last_path()}
     res = {"flop_per_pass": flop, "per_pass": per_pass, "ms_per_step": wall_ms, "tflops": 3 * flop / wall_ms / 1e9}
     if dtype == np.float32 and B == C3["B"]:
         # forward + bias + ReLU: in the conv kernel's store (one pass over y) vs conv, then an in-place bias/ReLU pass
@@ -736,14 +736,14 @@ def main():
                      # the other two metrics of the baseline: filled in below (slowest bandwidth kernel of config C4; the CNN
                      # training step of config C5 against the sum of its kernels' rooflines)
                      "others": {}},
-        "conv_passes": {k: {"ms": v["ms"], "tflops": v["tflops"], "frac_mfma_f32": v["tflops"] / PEAK_F32_MFMA_TFLOPS}
+        "conv_passes": {k: {"ms": v["ms"], "tflops": v["tflops"], "frac_mfma_f32": v["tflops"] / PEAK_F32_MFMA_TFLOPS, "kernel_family": v["kernel_family"]}
                         for k, v in conv["per_pass"].items()},
         "conv_fwd_bias_relu": conv.get("fwd_bias_relu"),
     }
     if not args.skip_also:
         c64 = bench_conv(ctx, max(3, args.steps // 4), 1, np.float64, B=C3["B"])
         result["also"] = {
-            "conv_f64": {k: {"ms": v["ms"], "tflops": v["tflops"], "frac_mfma_f64": v["tflops"] / PEAK_F64_MFMA_TFLOPS}
+            "conv_f64": {k: {"ms": v["ms"], "tflops": v["tflops"], "frac_mfma_f64": v["tflops"] / PEAK_F64_MFMA_TFLOPS, "kernel_family": v["kernel_family"]}
                          for k, v in c64["per_pass"].items()},
         }
         result["also"].update(bench_bandwidth(ctx))
