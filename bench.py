@@ -651,10 +651,15 @@ def bench_conv_sweep():
                 w = ctx.normal((cout, cin, 3, 3), 3, 0.0, 0.05)
                 y, dx, dw = ctx.empty(g.shape), ctx.empty(x.shape), ctx.empty(w.shape)
                 gflop = 2.0 * cout * cin * 9 * batch * hw * hw / 1e9
-                ms = (timed(lambda: ctx.conv2d_fwd(x, w, (1, 1), (1, 1), out=y)),
-                      timed(lambda: ctx.conv2d_dgrad(g, w, x.shape, (1, 1), (1, 1), 0, out=dx)),
-                      timed(lambda: ctx.conv2d_wgrad(x, g, w.shape, (1, 1), (1, 1), 0, out=dw)))
+                ms, fam = [], []
+                for fn in (lambda: ctx.conv2d_fwd(x, w, (1, 1), (1, 1), out=y),
+                           lambda: ctx.conv2d_dgrad(g, w, x.shape, (1, 1), (1, 1), 0, out=dx),
+                           lambda: ctx.conv2d_wgrad(x, g, w.shape, (1, 1), (1, 1), 0, out=dw)):
+                    ms.append(timed(fn))
+                    fam.append(ctx.conv2d_last_path())
                 out[f"B{batch}_{cin}to{cout}_{hw}x{hw}"] = [round(gflop / m, 1) for m in ms]
+                if any("implicit" in f for f in fam):  # layers that fall off the specialised kernels say so
+                    out[f"B{batch}_{cin}to{cout}_{hw}x{hw}_kernel_families"] = fam
                 for a in (x, g, w, y, dx, dw):
                     a.free()
     ctx.close()
