@@ -1060,7 +1060,7 @@ def test_layers_take_the_kernels_written_for_them(ctx):
 
 
 RANDOM_CONV_SEEDS = [(61, np.float32), (62, np.float32), (63, np.float32), (64, np.float32), (65, np.float64), (66, np.float64),
-                     (67, np.float32), (68, np.float32), (69, np.float64)]
+                     (67, np.float32), (68, np.float32), (69, np.float64), (70, np.float32), (71, np.float64)]
 
 
 def random_conv_shapes(seed):
