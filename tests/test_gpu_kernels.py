@@ -312,7 +312,9 @@ GEMM_LDS_SHAPES = [(2560, 2560, 128), (2500, 2436, 192), (4096, 3200, 64 * 3), (
                    (1024, 1024, 1024), (1000, 1100, 192), (1280, 832, 128), (2048, 512, 256), (100, 16384, 128), (1988, 724, 320),
                    # K that is no multiple of the 64-deep stage (served for A . B^T with both operands k-contiguous; the other forms take
                    # the general tiles): a tail of 4, 40 and 60 values
-                   (2560, 2560, 132), (2048, 1536, 1000), (1024, 1024, 252)]
+                   (2560, 2560, 132), (2048, 1536, 1000), (1024, 1024, 252),
+                   # about one 64-row tile per CU (ragged rows and columns too)
+                   (1000, 1000, 384), (640, 1100, 512), (1024, 960, 256)]
 
 
 def test_gemm_lds_kernel_shapes_all_transposes_and_bias(ctx):
@@ -981,7 +983,9 @@ def test_conv2d_strided_dgrad_vs_torch_and_oracle(ctx, orc, dtype):
 POINTWISE_CASES = [(3, 128, 16, 16, 256), (4, 256, 8, 8, 128), (2, 192, 12, 20, 96), (70, 128, 8, 8, 64), (1, 512, 32, 32, 128),
                    (2, 64, 16, 16, 64), (3, 130, 8, 8, 70), (2, 128, 7, 9, 256), (5, 256, 16, 16, 256),
                    # maps whose pixel count is no multiple of 64 (the weight gradient's reduction length): 14 x 14, 28 x 28, 10 x 10
-                   (64, 256, 14, 14, 256), (16, 128, 28, 28, 256), (96, 128, 10, 10, 128)]
+                   (64, 256, 14, 14, 256), (16, 128, 28, 28, 256), (96, 128, 10, 10, 128),
+                   # about one 64-row tile per CU
+                   (4, 512, 28, 28, 256), (2, 256, 32, 32, 512)]
 
 
 def test_conv2d_pointwise_layers(ctx, orc):
