@@ -628,8 +628,8 @@ def _cpu_model():
 
 
 def bench_conv_sweep():
-    """3x3, stride 1, padding 1, f32: TFLOP/s of the three passes over channel counts and map sizes (batch sized to a few
-    GFLOP per pass).  Timed with the library's event timer on its own stream, 20 runs after 3 warm-up runs each."""
+    """3x3, padding 1, f32: TFLOP/s of the three passes over channel counts and map sizes at stride 1, and over the
+    channel-doubling layers at stride 2 (batch sized to a few GFLOP per pass).  Timed with the library's event timer on its own stream, 20 runs after 3 warm-up runs each."""
     from ferrox_amd import capi
     ctx = capi.Context(0)
 
@@ -643,25 +643,36 @@ def bench_conv_sweep():
         return ctx.timer_stop() / runs
 
     out = {}
+
+    def layer(key, batch, cin, hw, cout, stride, always_name):
+        oh = (hw + 2 - 3) // stride + 1
+        x = ctx.uniform((batch, cin, hw, hw), 1, -1.0, 1.0)
+        g = ctx.normal((batch, cout, oh, oh), 2, 0.0, 1.0)
+        w = ctx.normal((cout, cin, 3, 3), 3, 0.0, 0.05)
+        y, dx, dw = ctx.empty(g.shape), ctx.empty(x.shape), ctx.empty(w.shape)
+        gflop = 2.0 * cout * cin * 9 * batch * oh * oh / 1e9
+        st = (stride, stride)
+        ms, fam = [], []
+        for fn in (lambda: ctx.conv2d_fwd(x, w, st, (1, 1), out=y),
+                   lambda: ctx.conv2d_dgrad(g, w, x.shape, st, (1, 1), 0, out=dx),
+                   lambda: ctx.conv2d_wgrad(x, g, w.shape, st, (1, 1), 0, out=dw)):
+            ms.append(timed(fn))
+            fam.append(ctx.conv2d_last_path())
+        out[key] = [round(gflop / m, 1) for m in ms]
+        if always_name or any("implicit" in f for f in fam):  # layers that fall off the specialised kernels say so
+            out[key + "_kernel_families"] = fam
+        for a in (x, g, w, y, dx, dw):
+            a.free()
+
     for hw, batch in ((128, 16), (112, 16), (64, 64), (32, 128), (16, 256), (8, 512)):
         for cin in (32, 64, 128, 256):
             for cout in (32, 64, 128, 256):
-                x = ctx.uniform((batch, cin, hw, hw), 1, -1.0, 1.0)
-                g = ctx.normal((batch, cout, hw, hw), 2, 0.0, 1.0)
-                w = ctx.normal((cout, cin, 3, 3), 3, 0.0, 0.05)
-                y, dx, dw = ctx.empty(g.shape), ctx.empty(x.shape), ctx.empty(w.shape)
-                gflop = 2.0 * cout * cin * 9 * batch * hw * hw / 1e9
-                ms, fam = [], []
-                for fn in (lambda: ctx.conv2d_fwd(x, w, (1, 1), (1, 1), out=y),
-                           lambda: ctx.conv2d_dgrad(g, w, x.shape, (1, 1), (1, 1), 0, out=dx),
-                           lambda: ctx.conv2d_wgrad(x, g, w.shape, (1, 1), (1, 1), 0, out=dw)):
-                    ms.append(timed(fn))
-                    fam.append(ctx.conv2d_last_path())
-                out[f"B{batch}_{cin}to{cout}_{hw}x{hw}"] = [round(gflop / m, 1) for m in ms]
-                if any("implicit" in f for f in fam):  # layers that fall off the specialised kernels say so
-                    out[f"B{batch}_{cin}to{cout}_{hw}x{hw}_kernel_families"] = fam
-                for a in (x, g, w, y, dx, dw):
-                    a.free()
+                layer(f"B{batch}_{cin}to{cout}_{hw}x{hw}", batch, cin, hw, cout, 1, False)
+    # stride 2 (padding 1), the channel-doubling layers between the stages of a residual network and the two of the CNN
+    # example: which kernel family takes each pass is part of the figure
+    for hw, batch in ((64, 128), (56, 128), (32, 256), (28, 256), (16, 512), (14, 512)):
+        for cin, cout in ((32, 64), (64, 128), (128, 256)):
+            layer(f"stride2_B{batch}_{cin}to{cout}_{hw}x{hw}", batch, cin, hw, cout, 2, True)
     ctx.close()
     return out
 
@@ -685,8 +696,8 @@ def main():
                     help="run only the C4 bandwidth kernels, 4 calls each on rotating inputs with marker dispatches between "
                          "the cases, and print the case order (for rocprofv3 counter runs)")
     ap.add_argument("--conv-sweep", action="store_true",
-                    help="run only a sweep of 3x3 stride-1 f32 layer shapes (Cin, Cout in 32..256; 8x8..64x64 maps) and print "
-                         "TFLOP/s per pass as one JSON line")
+                    help="run only a sweep of 3x3 f32 layer shapes (stride 1: Cin, Cout in 32..256 over 8x8..128x128 maps; stride 2: "
+                         "channel-doubling layers over 14x14..64x64 maps) and print TFLOP/s per pass as one JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the hot path has no cross-GPU exchange built); use --gpus 1")

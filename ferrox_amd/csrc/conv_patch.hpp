@@ -80,9 +80,12 @@ __global__ __launch_bounds__(256) void wimg_kernel(const float* __restrict__ w, 
 
 // MULTI: maps of at most 64 pixels.  A tile is then nimg whole images stacked in the patch, each with its own zero
 // rows above and below, so that the 128 pixels of the smallest tile are not mostly padding.
-template <int WM, int TN, bool BIAS, int NXP, bool MULTI = false>
+// NARROW: rows of at most 32 floats are staged by 8 lanes each, four patch rows per pass instead of two (strided layers over
+// narrow maps need more patch rows than pixels' worth: a 128-pixel tile of a 14-wide output at stride 2 sits on 23 rows).
+template <int WM, int TN, bool BIAS, int NXP, bool MULTI = false, bool NARROW = false>
 __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
     constexpr int BM = 32 * WM, WN = 4 / WM, NPIX = 32 * TN * WN;
+    constexpr int LPRN = NARROW ? LPR / 2 : LPR, RPP = NT / (LPRN * CC);  // lanes per patch row, rows per pass
     constexpr int WIMG = BM * WPITCH;             // floats in one weight image
     constexpr int NW = (WIMG / 4 + NT - 1) / NT;  // float4 of the image per thread (the last one only partly used)
     FX_DYNAMIC_SMEM(float, smem);
@@ -124,9 +127,10 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
     __syncthreads();
 
     // staging: thread t copies float4 t + 256u of the weight image and owns float4 column t % 16 of patch rows
-    // 2u + rp of channel (t / 16) % 8, where rp = t / 128 is uniform over a wave.
+    // 2u + rp of channel (t / 16) % 8, where rp = t / 128 is uniform over a wave (NARROW: column t % 8 of rows 4u + rp,
+    // channel (t / 8) % 8, rp = t / 64).
     const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    const int pq = tid & (LPR - 1), xc = (tid >> 4) & (CC - 1), rp = tid >> 7;
+    const int pq = tid & (LPRN - 1), xc = (tid / LPRN) & (CC - 1), rp = tid / (LPRN * CC);
     // A row of W floats is covered by ceil(W / 4) vectors; the last one is moved back to end at the row's end (it then
     // overlaps its neighbour, which parks the same values), so no load crosses into the next row or past the tensor.
     const bool x_lane = pq < ((p.W + 3) >> 2);
@@ -146,7 +150,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
         const float* xsrc = xsrc0 + (i64)ch * CC * p.H * p.W;
 #pragma unroll
         for (int u = 0; u < NXP; ++u) {
-            const int r = 2 * u + rp;
+            const int r = RPP * u + rp;
             if constexpr (MULTI) {
                 const int img = (int)p.div_rpi.div((uint32_t)r), iy = r - img * p.RPI - p.ph;
                 if (r < p.PR && iy >= 0 && iy < p.H && b + img < p.B) xv[u] = ldg4(xsrc + ((i64)img * p.C * p.H + iy) * p.W, x_off);
@@ -169,7 +173,7 @@ __global__ __launch_bounds__(NT, 2) void conv_patch_kernel(const Params p) {
         if (x_lane) {
 #pragma unroll
             for (int u = 0; u < NXP; ++u) {
-                const int r = 2 * u + rp;
+                const int r = RPP * u + rp;
                 if (r < p.PR) {  // wave-uniform
                     const float4 v = xv[u];
                     float* d = smem + xd + r * p.PW;
@@ -535,6 +539,7 @@ struct Plan {
     bool ok = false;
     int WM = 4, TN = 0, PR = 0, PW = 0, PLANE = 0, tpi = 0, mtiles = 0, nchunks = 0;
     bool tall = false;  // more than 8 patch rows: the NXP_TALL instantiation
+    bool narrow = false;  // more than 20 patch rows of at most 32 floats: the NARROW instantiation
     int nimg = 0, RPI = 0;  // small maps: images per tile and patch rows per image (0: one image per tile)
     i64 cost = 0;           // modelled cost: rounds of co-resident blocks x MFMA work of a block
     size_t smem = 0;
@@ -553,13 +558,18 @@ inline bool shape_plan(Plan& pl, int wm, int tn, int num_cus, i64 B, i64 C, i64 
     // output rows under a tile: tiles that start on a row boundary cover exactly np / OW rows
     const i64 rows = std::min<i64>(OH, np % OW == 0 ? np / OW : (np - 1) / OW + 2), PR = (rows - 1) * sh + 3;
     const bool tall_ok = wm <= 2 || tn <= 6;  // instantiated tall variants
+    const bool narrow_ok = W <= 2 * LPR && wm >= 2 && tall_ok;  // 21 to 40 patch rows: rows of at most 32 floats, four per staging pass
     // at most half of the channel rows and half of the pixels of an image's tiles may be padding (measured at 7 x 7 maps,
     // 49 pixels under a 128-pixel tile: 0.084 ms against 0.061 ms for the implicit GEMM at [256,128,7,7] -> 128)
-    if (PR > 2 * NXP_TALL || (PR > 2 * NXP_SHORT && !tall_ok) || mtiles * bm > M * 2 || tiles * np > L * 2) return false;
+    if (PR > (narrow_ok ? 4 : 2) * NXP_TALL || (PR > 2 * NXP_SHORT && !tall_ok) || mtiles * bm > M * 2 || tiles * np > L * 2) return false;
+    // strided layers, whose patch is four times the tile: at most a third of the pixels may be padding (16 x 16 maps at stride 2,
+    // 64 pixels under a 128-pixel tile: 57 and 62 against 68 and 95 TFLOP/s for the implicit GEMM at 64 -> 128 and 128 -> 256)
+    if ((sh > 1 || sw > 1) && tiles * np * 2 > L * 3) return false;
     pl = Plan();
     pl.WM = wm; pl.TN = tn; pl.PR = (int)PR; pl.tpi = (int)tiles;
     pl.cost = fx::ceil_div(B * tiles * mtiles, slots) * np * bm;
     pl.tall = pl.PR > 2 * NXP_SHORT;
+    pl.narrow = pl.PR > 2 * NXP_TALL;
     pl.PW = (int)(W + 2 * pw);
     pl.PLANE = wgp::odd_pitch(pl.PR * pl.PW);
     pl.smem = ((size_t)pl.wimg() + (size_t)CC * pl.PLANE + SLACK) * sizeof(float);
@@ -619,7 +629,11 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
     // (8 x 8 and 7 x 7 maps: two images), provided that fills at least half of the tile.
     const i64 RPI = (OH - 1) * sh + 3;
     if (L <= 64 && B >= 2 && W <= 4 * LPR) {  // (its staging covers rows of at most 64 floats)
-        const i64 nimg = std::min<i64>(std::min<i64>(128 / L, 2 * NXP_TALL / RPI), B);
+        // up to 40 patch rows where the NARROW staging pays: strided layers, and rows of at least two vectors (5 x 5 and 6 x 6 maps
+        // at stride 1, five and three images per tile: 79-100 and 71-97 TFLOP/s against 66-85 and 72-104 for the implicit GEMM over
+        // 64 to 256 channels; 4 x 4 maps, one vector per row in eight lanes: 48-65 against 59-104, left to the implicit GEMM)
+        const bool narrow_rows = W <= 2 * LPR && (sh > 1 || sw > 1 || W >= 5);
+        const i64 nimg = std::min<i64>(std::min<i64>(128 / L, (narrow_rows ? 4 : 2) * NXP_TALL / RPI), B);
         const int wm = M > 64 ? 4 : 2;
         const i64 bm = 32 * wm, mtiles = fx::ceil_div(M, bm);
         if (nimg >= 2 && nimg * L >= 64 && mtiles * bm <= M * 2 && mtiles <= 65535) {
@@ -627,6 +641,7 @@ inline Plan make_plan(int num_cus, i64 B, i64 C, i64 H, i64 W, i64 M, i64 OH, i6
             pl.nimg = (int)nimg; pl.RPI = (int)RPI;
             pl.PR = (int)(nimg * RPI);
             pl.tall = true;
+            pl.narrow = pl.PR > 2 * NXP_TALL;
             pl.tpi = 1;
             pl.PW = (int)(W + 2 * pw);
             pl.PLANE = wgp::odd_pitch(pl.PR * pl.PW);
@@ -757,41 +772,52 @@ inline int launch_plan(fx_ctx* c, const Plan& pl, const float* x, const float* w
     const dim3 grid((unsigned)gx, (unsigned)pl.mtiles);
     p.xcd_chunk = gx % 8 == 0 ? (int)(gx / 8) : 0;
     if (pl.nimg) {
-#define FX_CPK_LAUNCH_MULTI(WMV, TNV)                                                                                \
+#define FX_CPK_LAUNCH_MULTI(WMV, TNV, NARROWV)                                                                       \
     {                                                                                                                 \
-        static const hipError_t attr0 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, false, NXP_TALL, true>, \
+        static const hipError_t attr0 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, false, NXP_TALL, true, NARROWV>, \
                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
-        static const hipError_t attr1 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, true, NXP_TALL, true>, \
+        static const hipError_t attr1 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, true, NXP_TALL, true, NARROWV>, \
                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
         FX_HIP_CHECK(attr0);                                                                                          \
         FX_HIP_CHECK(attr1);                                                                                          \
-        if (bias) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), conv_patch_kernel<WMV, TNV, true, NXP_TALL, true>);       \
-        else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), conv_patch_kernel<WMV, TNV, false, NXP_TALL, true>);           \
+        if (bias) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), conv_patch_kernel<WMV, TNV, true, NXP_TALL, true, NARROWV>);  \
+        else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), conv_patch_kernel<WMV, TNV, false, NXP_TALL, true, NARROWV>);      \
     }
-        if (pl.WM == 4) FX_CPK_LAUNCH_MULTI(4, 4) else FX_CPK_LAUNCH_MULTI(2, 2)
+        if (pl.narrow) {
+            if (pl.WM == 4) FX_CPK_LAUNCH_MULTI(4, 4, true) else FX_CPK_LAUNCH_MULTI(2, 2, true)
+        } else {
+            if (pl.WM == 4) FX_CPK_LAUNCH_MULTI(4, 4, false) else FX_CPK_LAUNCH_MULTI(2, 2, false)
+        }
 #undef FX_CPK_LAUNCH_MULTI
         FX_LAUNCH_CHECK();
         return FX_OK;
     }
-#define FX_CPK_LAUNCH_N(WMV, TNV, NXPV)                                                                              \
+#define FX_CPK_LAUNCH_N(WMV, TNV, NXPV, NARROWV)                                                                     \
     {                                                                                                                 \
-        static const hipError_t attr0 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, false, NXPV>,    \
+        static const hipError_t attr0 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, false, NXPV, false, NARROWV>, \
                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
-        static const hipError_t attr1 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, true, NXPV>,     \
+        static const hipError_t attr1 = hipFuncSetAttribute((const void*)conv_patch_kernel<WMV, TNV, true, NXPV, false, NARROWV>, \
                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BUDGET); \
         FX_HIP_CHECK(attr0);                                                                                          \
         FX_HIP_CHECK(attr1);                                                                                          \
-        if (bias) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), conv_patch_kernel<WMV, TNV, true, NXPV>);                 \
-        else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), conv_patch_kernel<WMV, TNV, false, NXPV>);                     \
+        if (bias) FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), conv_patch_kernel<WMV, TNV, true, NXPV, false, NARROWV>);  \
+        else FX_LAUNCH(grid, dim3(NT), pl.smem, c->stream, (p), conv_patch_kernel<WMV, TNV, false, NXPV, false, NARROWV>);      \
     }
 #define FX_CPK_LAUNCH(WMV, TNV)                                                                                       \
     case WMV * 16 + TNV:                                                                                              \
-        if (pl.tall) FX_CPK_LAUNCH_N(WMV, TNV, NXP_TALL) else FX_CPK_LAUNCH_N(WMV, TNV, NXP_SHORT)                    \
+        if (pl.narrow) FX_CPK_LAUNCH_N(WMV, TNV, NXP_TALL, true)                                                      \
+        else if (pl.tall) FX_CPK_LAUNCH_N(WMV, TNV, NXP_TALL, false)                                                  \
+        else FX_CPK_LAUNCH_N(WMV, TNV, NXP_SHORT, false)                                                              \
+        break;
+#define FX_CPK_LAUNCH_WIDE_TILE(WMV, TNV) /* one block of channels: no NARROW instantiation */                       \
+    case WMV * 16 + TNV:                                                                                              \
+        FX_REQUIRE(!pl.narrow, "conv patch kernel: no narrow-row variant of tile %d x %d", WMV, TNV);                \
+        if (pl.tall) FX_CPK_LAUNCH_N(WMV, TNV, NXP_TALL, false) else FX_CPK_LAUNCH_N(WMV, TNV, NXP_SHORT, false)      \
         break;
 #define FX_CPK_LAUNCH_SHORT(WMV, TNV)                                                                                 \
     case WMV * 16 + TNV:                                                                                              \
         FX_REQUIRE(!pl.tall, "conv patch kernel: no tall variant of tile %d x %d", WMV, TNV);                        \
-        FX_CPK_LAUNCH_N(WMV, TNV, NXP_SHORT)                                                                          \
+        FX_CPK_LAUNCH_N(WMV, TNV, NXP_SHORT, false)                                                                   \
         break;
     switch (pl.WM * 16 + pl.TN) {
         FX_CPK_LAUNCH(4, 4)
@@ -802,12 +828,13 @@ inline int launch_plan(fx_ctx* c, const Plan& pl, const float* x, const float* w
         FX_CPK_LAUNCH(2, 2)
         FX_CPK_LAUNCH(2, 3)
         FX_CPK_LAUNCH(2, 4)
-        FX_CPK_LAUNCH(1, 2)
-        FX_CPK_LAUNCH(1, 3)
-        FX_CPK_LAUNCH(1, 4)
+        FX_CPK_LAUNCH_WIDE_TILE(1, 2)
+        FX_CPK_LAUNCH_WIDE_TILE(1, 3)
+        FX_CPK_LAUNCH_WIDE_TILE(1, 4)
         default: FX_REQUIRE(false, "conv patch kernel: unexpected tile %d x %d", pl.WM, pl.TN);
     }
 #undef FX_CPK_LAUNCH_N
+#undef FX_CPK_LAUNCH_WIDE_TILE
 #undef FX_CPK_LAUNCH_SHORT
 #undef FX_CPK_LAUNCH
     FX_LAUNCH_CHECK();

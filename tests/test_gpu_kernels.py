@@ -618,6 +618,12 @@ CONV_PATCH_CASES = [
     # strided layers: up to 20 patch rows under a tile
     (8, 32, 32, 32, 64, (2, 2), (1, 1)), (4, 64, 56, 56, 128, (2, 2), (1, 1)), (2, 16, 30, 40, 60, (2, 1), (1, 1)),
     (2, 8, 16, 34, 128, (3, 3), (1, 1)), (64, 16, 28, 28, 128, (2, 2), (1, 1)),
+    # 21 to 40 patch rows of at most 32 floats (four rows per staging pass): stride 2 over 28- and 14-wide maps (one tile of two
+    # images at 14 x 14, odd batch), no padding, a row length that is no multiple of four floats, 64- and 128-row tiles; stacked
+    # images of 5 x 5 and 6 x 6 maps at stride 1 (4 x 4 maps stay on the implicit GEMM)
+    (4, 16, 28, 28, 128, (2, 2), (1, 1)), (3, 8, 28, 28, 64, (2, 2), (1, 1)), (5, 16, 14, 14, 128, (2, 2), (1, 1)), (6, 8, 14, 14, 64, (2, 2), (1, 1)),
+    (2, 8, 30, 30, 40, (2, 2), (0, 0)), (2, 8, 27, 31, 64, (2, 2), (1, 1)), (9, 16, 5, 5, 64, (1, 1), (1, 1)), (13, 8, 4, 4, 128, (1, 1), (1, 1)),
+    (3, 8, 20, 24, 200, (3, 2), (1, 1)),
     # 32 channels out (forward) or in (data gradient): one block of channels, four waves along the pixels (1x2, 1x3, 1x4)
     (64, 64, 32, 32, 32, (1, 1), (1, 1)), (3, 16, 9, 20, 30, (1, 1), (1, 1)), (64, 8, 16, 32, 32, (2, 1), (1, 1)),
     (2, 8, 18, 10, 27, (1, 1), (0, 0)), (64, 32, 32, 32, 64, (1, 1), (1, 1)), (40, 32, 16, 16, 24, (1, 1), (1, 1)),
@@ -1042,6 +1048,8 @@ EXPECTED_PATHS = [  # (B, Cin, H, W, Cout, k, stride, padding, dtype) -> kernel 
     ((64, 256, 32, 32, 256, 1, 1, 0, np.float32), ("1x1 as batched slab GEMM (glk)",) * 3),                                     # enough tiles to fill the chip
     ((4, 32, 20, 20, 64, 5, 1, 2, np.float32), ("implicit GEMM",) * 3),                                                          # no 5 x 5 kernels
     ((4, 64, 56, 56, 128, 3, 2, 1, np.float32), ("LDS patch (cpk)", "implicit GEMM by pixel classes", "LDS patch (wgp)")),        # stride 2 off the 32 / 64 wide maps
+    ((8, 64, 28, 28, 128, 3, 2, 1, np.float32), ("LDS patch (cpk)", "implicit GEMM by pixel classes", "implicit GEMM")),          # 23 patch rows under a tile
+    ((8, 64, 14, 14, 128, 3, 2, 1, np.float32), ("LDS patch (cpk)", "implicit GEMM by pixel classes", "implicit GEMM")),          # two 7 x 7 outputs per tile
 ]
 
 
