@@ -307,8 +307,9 @@ struct Plan {
     size_t smem = 0;
 };
 
-// Instantiated (WMO, OW, R): rows of 16 and 32 pixels (maps 32 and 64 wide).
-#define FX_WG2_SHAPES(X) X(1, 16, 4) X(2, 16, 4) X(4, 16, 4) X(1, 32, 2) X(2, 32, 2) X(4, 32, 2)
+// Instantiated (WMO, OW, R): rows of 16 and 32 pixels (maps 32 and 64 wide); of 28 pixels (56 wide; a segment of 7 pixels cannot be
+// walked in pairs, so no layout with four row segments); of 8 pixels, a whole 8 x 8 output per stage (16 wide).
+#define FX_WG2_SHAPES(X) X(1, 16, 4) X(2, 16, 4) X(4, 16, 4) X(1, 32, 2) X(2, 32, 2) X(4, 32, 2) X(2, 28, 2) X(4, 28, 2) X(1, 8, 8) X(2, 8, 8) X(4, 8, 8) X(4, 14, 2)
 
 inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, i64 oh, i64 ow) {
     Plan pl;

@@ -237,7 +237,7 @@ struct Plan {
 };
 
 // Instantiated (OW, R): rows of 16 and 32 pixels (maps 32 and 64 wide), 32 pixels per stage.
-#define FX_WGD2_SHAPES(X) X(16, 2) X(32, 1)
+#define FX_WGD2_SHAPES(X) X(16, 2) X(32, 1) X(8, 4)
 
 inline Plan make_plan(int num_cus, i64 B, i64 Cin, i64 H, i64 W, i64 Cout, i64 kh, i64 kw, i64 sh, i64 sw, i64 ph, i64 pw, i64 oh, i64 ow) {
     Plan pl;

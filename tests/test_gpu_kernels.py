@@ -557,6 +557,13 @@ WGRAD_PATCH_CASES = [
     (3, 32, 32, 32, 64, (2, 2), (1, 1)), (2, 64, 8, 32, 128, (2, 2), (1, 1)), (5, 32, 16, 32, 32, (2, 2), (1, 1)), (2, 32, 8, 64, 64, (2, 2), (1, 1)),
     (2, 64, 4, 64, 128, (2, 2), (1, 1)), (3, 32, 12, 64, 96, (2, 2), (1, 1)), (2, 32, 9, 32, 64, (2, 2), (0, 1)), (2, 32, 15, 32, 64, (2, 2), (1, 1)),
     (40, 32, 8, 32, 64, (2, 2), (1, 1)),
+    # the same kernel over maps 56 wide (rows of 28 pixels: two and one row segments) and 16 wide (a whole 8 x 8 output per stage:
+    # one, two and four row segments) and 28 wide (two of 14 output rows per stage, 128 output channels per block), a top row without
+    # padding, an odd height, many splits
+    (2, 32, 56, 56, 64, (2, 2), (1, 1)), (2, 64, 8, 56, 128, (2, 2), (1, 1)), (3, 32, 12, 56, 192, (2, 2), (1, 1)), (2, 32, 9, 56, 64, (2, 2), (0, 1)),
+    (3, 32, 16, 16, 32, (2, 2), (1, 1)), (5, 64, 16, 16, 64, (2, 2), (1, 1)), (2, 32, 16, 16, 128, (2, 2), (1, 1)), (2, 32, 15, 16, 64, (2, 2), (1, 1)),
+    (2, 32, 17, 16, 96, (2, 2), (0, 1)), (70, 32, 16, 16, 64, (2, 2), (1, 1)), (33, 32, 4, 56, 128, (2, 2), (1, 1)),
+    (3, 32, 28, 28, 128, (2, 2), (1, 1)), (2, 64, 12, 28, 256, (2, 2), (1, 1)), (2, 32, 27, 28, 128, (2, 2), (1, 1)),
     # narrow maps: one whole image per stage, (channel, row) pair staging
     (3, 64, 8, 8, 128, (1, 1), (1, 1)), (2, 32, 8, 8, 64, (1, 1), (1, 1)), (2, 96, 8, 8, 20, (1, 1), (1, 1)), (2, 32, 6, 8, 100, (1, 1), (1, 1)),
     (3, 64, 4, 16, 72, (1, 1), (1, 1)), (2, 48, 8, 8, 24, (1, 1), (1, 1)), (70, 128, 8, 8, 128, (1, 1), (1, 1)),
@@ -758,6 +765,9 @@ CONV_F64_WGRAD_CASES = [  # B, Cin, H, W, Cout, sh, (ph, pw)
     # row without padding, stage ranges that do not divide evenly
     (3, 32, 32, 32, 64, (2, 2), (1, 1)), (2, 64, 16, 64, 128, (2, 2), (1, 1)), (5, 32, 31, 32, 64, (2, 2), (1, 1)),
     (2, 32, 33, 32, 64, (2, 2), (0, 1)), (70, 32, 32, 32, 64, (2, 2), (1, 1)), (3, 64, 6, 64, 192, (2, 2), (1, 1)),
+    # ... and 16 wide (half of an 8 x 8 output per stage)
+    (3, 32, 16, 16, 64, (2, 2), (1, 1)), (2, 64, 16, 16, 128, (2, 2), (1, 1)), (5, 32, 15, 16, 64, (2, 2), (1, 1)), (2, 32, 17, 16, 64, (2, 2), (0, 1)),
+    (70, 32, 8, 16, 64, (2, 2), (1, 1)),
 ]
 
 
@@ -1042,13 +1052,15 @@ EXPECTED_PATHS = [  # (B, Cin, H, W, Cout, k, stride, padding, dtype) -> kernel 
     ((16, 3, 32, 32, 32, 3, 1, 1, np.float64), ("image layer (cim)", "direct gather, few input channels", "image layer, row bands (cim)")),
     ((16, 32, 32, 32, 64, 3, 2, 1, np.float32), ("LDS patch (cpk)", "stride-2 patch (dg2)", "stride-2 patch (wg2)")),
     ((16, 32, 32, 32, 64, 3, 2, 1, np.float64), ("stride-2 patch (fwd2)", "stride-2 patch (dgd2)", "stride-2 patch (wgd2)")),
+    ((16, 32, 16, 16, 64, 3, 2, 1, np.float64), ("implicit GEMM", "implicit GEMM by pixel classes", "stride-2 patch (wgd2)")),
     ((2, 64, 12, 112, 128, 3, 1, 1, np.float32), ("LDS patch (cpk)", "LDS patch (cpk)", "LDS patch, row segments (wgp)")),       # rows of 112 floats
     ((1, 64, 6, 224, 64, 3, 1, 1, np.float32), ("LDS patch (cpk)", "LDS patch (cpk)", "LDS patch, row segments (wgp)")),         # rows of 224 floats
     ((1, 3, 128, 128, 32, 3, 1, 1, np.float32), ("image layer, tiles (csc)", "direct gather, few input channels", "image layer, tiles (csc)")),  # the reference's benchmark layer
     ((64, 256, 32, 32, 256, 1, 1, 0, np.float32), ("1x1 as batched slab GEMM (glk)",) * 3),                                     # enough tiles to fill the chip
     ((4, 32, 20, 20, 64, 5, 1, 2, np.float32), ("implicit GEMM",) * 3),                                                          # no 5 x 5 kernels
-    ((4, 64, 56, 56, 128, 3, 2, 1, np.float32), ("LDS patch (cpk)", "implicit GEMM by pixel classes", "LDS patch (wgp)")),        # stride 2 off the 32 / 64 wide maps
-    ((8, 64, 28, 28, 128, 3, 2, 1, np.float32), ("LDS patch (cpk)", "implicit GEMM by pixel classes", "implicit GEMM")),          # 23 patch rows under a tile
+    ((4, 64, 56, 56, 128, 3, 2, 1, np.float32), ("LDS patch (cpk)", "implicit GEMM by pixel classes", "stride-2 patch (wg2)")),   # stride 2 over a 56-wide map
+    ((8, 64, 16, 16, 128, 3, 2, 1, np.float32), ("LDS patch (cpk)", "implicit GEMM by pixel classes", "stride-2 patch (wg2)")),   # ... and a 16-wide one
+    ((8, 64, 28, 28, 128, 3, 2, 1, np.float32), ("LDS patch (cpk)", "implicit GEMM by pixel classes", "stride-2 patch (wg2)")),   # 23 patch rows under a tile
     ((8, 64, 14, 14, 128, 3, 2, 1, np.float32), ("LDS patch (cpk)", "implicit GEMM by pixel classes", "implicit GEMM")),          # two 7 x 7 outputs per tile
 ]
 
