@@ -445,6 +445,102 @@ __global__ __launch_bounds__(256) void dgrad_small_cin_kernel(const T* __restric
     for (int c = 0; c < s.Cin; ++c) o[(i64)c * s.H * s.W] = acc[c];
 }
 
+// The same for 3 x 3 filters at unit stride and padding 1 over rows that are whole 16-byte vectors: a thread owns four consecutive
+// input pixels of a row and reads the four grad_out values above them as one vector -- the two neighbours come from the adjacent
+// lanes -- so one coalesced load feeds 3 x 4 x CIN FMAs (the kernel above: one load per CIN).  The output channels are split over
+// the four waves of a block (wave q takes every fourth one), so four waves per SIMD hide the load latency; their sums are added
+// through LDS in wave order.  A block covers 64 pixel groups.
+// Measured on [256,3,32,32] <- 32 channels: 17.4 us against 31.1 us with the kernel above; with four pixels per thread read as six
+// scalar loads (lanes 16 bytes apart: four times the cache lines per load) 38.0 us.
+__device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void load4(const double* p, double (&v)[4]) {
+    const double2 t0 = *reinterpret_cast<const double2*>(p), t1 = *reinterpret_cast<const double2*>(p + 2);
+    v[0] = t0.x; v[1] = t0.y; v[2] = t1.x; v[3] = t1.y;
+}
+template <typename T, int CIN>
+__global__ __launch_bounds__(256) void dgrad_small_cin_s1_kernel(const T* __restrict__ g, const T* __restrict__ w, T* __restrict__ dx,
+                                                                 ConvShape s, int ngroups, int WQ, igemm::FastDiv div_wq) {
+    constexpr int KW = 3, PX = 4;
+    FX_DYNAMIC_SMEM(unsigned char, smem_raw);
+    T* wl = reinterpret_cast<T*>(smem_raw);  // [tap][oc][4]; afterwards the sums of waves 1 .. 3: [3][PX * CIN][64]
+    const int KK = 3 * KW;
+    for (int i = threadIdx.x; i < KK * s.Cout * 4; i += 256) {
+        const int c = i & 3, oc = (i >> 2) % s.Cout, t = (i >> 2) / s.Cout;
+        wl[i] = c < s.Cin ? w[((i64)oc * s.Cin + c) * KK + t] : T(0);
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
+    const int n = blockIdx.x * 64 + lane;
+    const bool live = n < ngroups;
+    const uint32_t nn = live ? (uint32_t)n : 0u;
+    const uint32_t row = div_wq.div(nn), xq = nn - row * WQ;  // row = b * H + y
+    const uint32_t b = row / (uint32_t)s.H;
+    const int y = (int)(row - b * s.H), x0 = (int)xq * PX;
+    const int L = s.H * s.W;  // the output map has the size of the input
+    const T* gb = g + (i64)b * s.Cout * L + x0;
+    // the values left and right of the vector: from the neighbouring lane when it holds the same row, else (a row that continues
+    // in another wave) loaded by this lane; zero outside the row
+    const bool has_left = xq > 0, has_right = (int)xq < WQ - 1;
+    const bool left_far = live && has_left && lane == 0, right_far = live && has_right && (lane == 63 || n + 1 >= ngroups);
+    T acc[PX][CIN];
+#pragma unroll
+    for (int j = 0; j < PX; ++j)
+#pragma unroll
+        for (int c = 0; c < CIN; ++c) acc[j][c] = T(0);
+    for (int ky = 0; ky < 3; ++ky) {
+        const int oy = y + 1 - ky;
+        if (oy < 0 || oy >= s.H) continue;
+        const T* grow = gb + (i64)oy * s.W;
+        const T* wrow = wl + ky * KW * s.Cout * 4;
+#pragma unroll 2
+        for (int oc = q; oc < s.Cout; oc += 4) {
+            T gv[KW + PX - 1], mid[4];
+            const T* gp = grow + (i64)oc * L;
+            if (live) load4(gp, mid);
+            else mid[0] = mid[1] = mid[2] = mid[3] = T(0);
+            T lv = __shfl_up(mid[3], 1, 64), rv = __shfl_down(mid[0], 1, 64);
+            if (left_far) lv = gp[-1];
+            if (right_far) rv = gp[4];
+            gv[0] = has_left ? lv : T(0);
+            gv[1] = mid[0]; gv[2] = mid[1]; gv[3] = mid[2]; gv[4] = mid[3];
+            gv[5] = has_right ? rv : T(0);
+#pragma unroll
+            for (int kx = 0; kx < KW; ++kx) {
+                const T* wt = wrow + (kx * s.Cout + oc) * 4;
+#pragma unroll
+                for (int c = 0; c < CIN; ++c) {
+                    const T wv = wt[c];
+#pragma unroll
+                    for (int j = 0; j < PX; ++j) acc[j][c] += gv[j + KW - 1 - kx] * wv;  // grad_out column x0 + j + 1 - kx
+                }
+            }
+        }
+    }
+    __syncthreads();  // every wave is done with the filters
+    T* red = wl;
+    if (q != 0) {
+#pragma unroll
+        for (int j = 0; j < PX; ++j)
+#pragma unroll
+            for (int c = 0; c < CIN; ++c) red[((q - 1) * PX * CIN + j * CIN + c) * 64 + lane] = acc[j][c];
+    }
+    __syncthreads();
+    if (q != 0 || !live) return;
+    T* o = dx + ((i64)b * s.Cin * s.H + y) * s.W + x0;
+#pragma unroll
+    for (int c = 0; c < CIN; ++c)
+#pragma unroll
+        for (int j = 0; j < PX; ++j) {
+            T v = acc[j][c];
+#pragma unroll
+            for (int r = 0; r < 3; ++r) v += red[(r * PX * CIN + j * CIN + c) * 64 + lane];
+            o[(i64)c * s.H * s.W + j] = v;
+        }
+}
+
 template <typename T>
 bool dgrad_small_cin_ok(const Dims& d) {
     return d.Cin <= 4 && d.kh * d.kw * d.Cout * 4 * (i64)sizeof(T) <= 48 * 1024 && !generic_only();
@@ -455,6 +551,18 @@ int dgrad_small_cin(fx_ctx* c, const T* g, const T* w, T* dx, const Dims& d) {
     const ConvShape s = make_shape(d.B, d.Cin, d.H, d.W, d.Cout, d.kh, d.kw, d.sh, d.sw, d.ph, d.pw);
     const i64 npix = d.B * d.H * d.W;
     const size_t smem = (size_t)(d.kh * d.kw * d.Cout * 4) * sizeof(T);
+    // (f64: level with the one-pixel kernel, 30.8 against 34.6 us on that layer and 242 against 210 us on [16,4,224,224] <- 64)
+    if (sizeof(T) == 4 && d.sh == 1 && d.sw == 1 && d.kh == 3 && d.kw == 3 && d.ph == 1 && d.pw == 1 && d.W % 4 == 0 && d.Cin >= 3 &&
+        fx::aligned16(g) && d.B * d.H * d.W < (1ll << 31)) {
+        const i64 WQ = fx::ceil_div(d.W, (i64)4), ngroups = d.B * d.H * WQ;
+        const size_t need = std::max(smem, (size_t)3 * 4 * d.Cin * 64 * sizeof(T));
+        const dim3 grid((unsigned)fx::ceil_div(ngroups, (i64)64));
+        const igemm::FastDiv div_wq((uint32_t)WQ);
+        if (d.Cin == 3) FX_LAUNCH(grid, dim3(256), need, c->stream, (g, w, dx, s, (int)ngroups, (int)WQ, div_wq), dgrad_small_cin_s1_kernel<T, 3>);
+        else FX_LAUNCH(grid, dim3(256), need, c->stream, (g, w, dx, s, (int)ngroups, (int)WQ, div_wq), dgrad_small_cin_s1_kernel<T, 4>);
+        FX_LAUNCH_CHECK();
+        return FX_OK;
+    }
     FX_LAUNCH(dim3((unsigned)fx::ceil_div(npix, 256)), dim3(256), smem, c->stream, (g, w, dx, s, (int)npix), dgrad_small_cin_kernel<T>);
     FX_LAUNCH_CHECK();
     return FX_OK;

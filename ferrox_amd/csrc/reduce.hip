@@ -202,6 +202,47 @@ __global__ __launch_bounds__(256) void short_row_reduce_kernel(const T* __restri
     }
 }
 
+// Short rows whose length is a multiple of the 16-byte vector (rows of up to 64 vectors): a lane takes one vector of a row, GV =
+// power of two >= vectors per row lanes share a row, and a thread keeps the vectors of U rows in flight (a block reads U
+// contiguous stretches of 4 KiB when the row length is a power of two).  One element per lane, as above, left a [256,32,32,32]
+// sum over the last axis at 24 us for 33.5 MB.
+template <typename T, int IS_MAX>
+__global__ __launch_bounds__(256) void short_row_vec_kernel(const T* __restrict__ in, T* __restrict__ out, i64* __restrict__ idx_out,
+                                                            i64 outer, int axis_v, int GV, T scale) {
+    constexpr int N = Vec16<T>::N, U = 4;
+    typedef typename Vec16<T>::type V;
+    const int lane = threadIdx.x & 63;
+    const int a = threadIdx.x % GV;
+    const i64 rows_per_pass = 256 / GV;
+    const i64 row0 = (i64)blockIdx.x * U * rows_per_pass + threadIdx.x / GV;
+    V v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const i64 o = row0 + u * rows_per_pass;
+        if (o < outer && a < axis_v) v[u] = ld16<false>(reinterpret_cast<const V*>(in + o * axis_v * N) + a);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const i64 o = row0 + u * rows_per_pass;
+        Acc<T, IS_MAX> acc;
+        acc.init();
+        if (o < outer && a < axis_v) {
+#pragma unroll
+            for (int e = 0; e < N; ++e) acc.take(vget<T>(v[u], e), a * N + e);
+        }
+        for (int d = GV >> 1; d >= 1; d >>= 1) {
+            const T ov = shfl_down_t(acc.v, d);
+            i64 oi = NO_INDEX;
+            if (EXTREMUM(IS_MAX)) oi = shfl_down_i64(acc.i, d);
+            if ((lane % GV) + d < GV) acc.merge(ov, oi);
+        }
+        if (a == 0 && o < outer) {
+            out[o] = EXTREMUM(IS_MAX) ? acc.v : acc.v * scale;
+            if (EXTREMUM(IS_MAX) && idx_out) idx_out[o] = acc.i == NO_INDEX ? 0 : acc.i;
+        }
+    }
+}
+
 // Combine S slice partials per output: one 256-thread block per output element, slices merged with the tie rule.
 template <typename T, int IS_MAX>
 __global__ __launch_bounds__(256) void combine_rows_kernel(const T* __restrict__ pv, const i64* __restrict__ pi, T* __restrict__ out,
@@ -345,6 +386,16 @@ int reduce(fx_ctx* c, const T* in, T* out, i64* idx_out, i64 outer, i64 axis, i6
     const i64 target_blocks = (i64)c->num_cus * 8;
 
     if (inner == 1) {
+        if (axis % N == 0 && axis / N <= 64 && fx::aligned16(in)) {
+            const int axis_v = (int)(axis / N);
+            int GV = 1;
+            while (GV < axis_v) GV <<= 1;
+            const i64 blocks = fx::ceil_div(outer, (i64)4 * (256 / GV));
+            FX_REQUIRE(blocks <= 0x7fffffff, "%s: too many rows", what);
+            short_row_vec_kernel<T, IS_MAX><<<dim3((unsigned)blocks), dim3(256), 0, c->stream>>>(in, out, idx_out, outer, axis_v, GV, scale);
+            FX_LAUNCH_CHECK();
+            return FX_OK;
+        }
         if (axis <= 64 && outer >= 1) {
             int G = 1;
             while (G < axis) G <<= 1;

@@ -77,6 +77,7 @@ inline void __syncthreads() {}
 #define __builtin_amdgcn_readfirstlane(x) (x)
 template <typename T> inline T __shfl_xor(T v, int, int = 64) { return v; }
 template <typename T> inline T __shfl_down(T v, int, int = 64) { return v; }
+template <typename T> inline T __shfl_up(T v, int, int = 64) { return v; }
 template <typename T> inline T __shfl(T v, int, int = 64) { return v; }
 inline uint32_t __umulhi(uint32_t a, uint32_t b) { return (uint32_t)(((uint64_t)a * b) >> 32); }
 template <typename V> inline V fxemu_mfma(double a, double b, V c) { c[0] += (decltype(c[0] + 0))(a * b); return c; }

@@ -201,7 +201,10 @@ def test_im2col_rectangular(ctx, orc):
 
 
 # ------------------------------------------------------------------------------------------ reductions
-RED_SHAPES = [(2, 2), (7, 13), (256, 10), (64, 1000), (3, 5, 7), (16, 32, 8, 8), (1, 70001), (5000, 33), (300, 4100), (2049, 515)]
+RED_SHAPES = [(2, 2), (7, 13), (256, 10), (64, 1000), (3, 5, 7), (16, 32, 8, 8), (1, 70001), (5000, 33), (300, 4100), (2049, 515),
+              # short last axes that are whole 16-byte vectors (one vector per lane, several rows per thread): 1 to 64 vectors per row,
+              # row counts that end inside a block's pass, more rows than one grid dimension holds
+              (37, 4), (1029, 12), (8, 32, 32), (515, 36), (100, 64), (77, 100), (33, 128), (9, 256), (70001, 8), (3, 2)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -828,13 +831,17 @@ def test_conv2d_image_layer_kernels(ctx, orc):
         dx_, dw_, dg_, db_ = ctx.upload(x), ctx.upload(w), ctx.upload(g), ctx.upload(bias)
         y = ctx.conv2d_fwd(dx_, dw_, st, pd).numpy()
         gw = ctx.conv2d_wgrad(dx_, dg_, w.shape, st, pd, 0).numpy()
-        tx = torch.from_numpy(x).double()
+        gx = ctx.conv2d_dgrad(dg_, dw_, x.shape, st, pd, 0).numpy()
+        tx = torch.from_numpy(x).double().requires_grad_(True)
         tw = torch.from_numpy(w).double().requires_grad_(True)
         ty = F.conv2d(tx, tw, stride=st, padding=pd)
         ty.backward(torch.from_numpy(g).double())
-        ay = F.conv2d(tx.abs(), tw.detach().abs(), stride=st, padding=pd).max().item()
+        ay = F.conv2d(tx.detach().abs(), tw.detach().abs(), stride=st, padding=pd).max().item()
         parity.check("image layers fwd", y, ty.detach().numpy(), oracle=orc.conv2d_fwd(x, w, st, pd), case=case, terms=ay)
         parity.check("image layers wgrad", gw, tw.grad.numpy(), oracle=orc.conv2d_wgrad(x, g, w.shape, st, pd, 0), case=case)
+        # the data gradient of a layer of few input channels (a gather per input pixel, four pixels per thread at unit stride)
+        parity.check("image layers dgrad", gx, tx.grad.numpy(), oracle=orc.conv2d_dgrad(g, w, x.shape, st, pd, 0), case=case)
+        assert np.array_equal(ctx.conv2d_dgrad(dg_, dw_, x.shape, st, pd, 0).numpy(), gx), case
         # same bits on a second run; bias + ReLU in the store equals the separate pass
         assert np.array_equal(ctx.conv2d_fwd(dx_, dw_, st, pd).numpy(), y), case
         assert np.array_equal(ctx.conv2d_wgrad(dx_, dg_, w.shape, st, pd, 0).numpy(), gw), case
