@@ -287,8 +287,8 @@ enum fx_scalar_op { FX_ADD_SCALAR = 0, FX_SUB_SCALAR = 1, FX_MUL_SCALAR = 2, FX_
        bias pass and its read-back disappear.  Gradient mode 0 only.  dw and dx have the bits of the two-call          \
        sequences; db is summed in the kernel's own fixed order (equal to fx_bias_grad up to rounding).  Served for     \
        the shapes fx_conv2d_bwd_relu_supported reports (3x3 image layers of at most 3 channels -- f64: maps 32 wide --  \
-       and 3x3 stride-2 padding-1 layers over even maps 32 or 64 wide); any other call returns FX_ERR_UNSUPPORTED and  \
-       changes nothing.                                                                                                \
+       and 3x3 stride-2 padding-1 layers over even maps 32 or 64 wide; the weight gradient also over maps 56, 28 and   \
+       16 wide); any other call returns FX_ERR_UNSUPPORTED and changes nothing.                                        \
        workspace as for fx_conv2d_wgrad (fx_conv2d_workspace_bytes(FX_CONV_WGRAD, ...) covers it). */                  \
     int fx_conv2d_wgrad_relu_bias_##S(fx_ctx* ctx, const T* x, const T* g, const T* act, T* dw, T* db, int64_t B,      \
                                       int64_t Cin, int64_t H, int64_t W, int64_t Cout, int64_t kh, int64_t kw,         \

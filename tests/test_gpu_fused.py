@@ -258,11 +258,15 @@ CONV_BWD_RELU_CASES = {
     np.float32: [
         (256, 3, 32, 32, 32, (1, 1), (1, 1)), (5, 1, 28, 28, 8, (1, 1), (1, 1)), (3, 3, 12, 16, 40, (1, 1), (1, 1)), (2, 2, 20, 8, 33, (2, 2), (1, 1)),
         (256, 32, 32, 32, 64, (2, 2), (1, 1)), (3, 32, 32, 32, 32, (2, 2), (1, 1)), (2, 64, 64, 64, 128, (2, 2), (1, 1)), (2, 32, 16, 32, 96, (2, 2), (1, 1)),
-        (1, 96, 64, 64, 64, (2, 2), (1, 1))],
+        (1, 96, 64, 64, 64, (2, 2), (1, 1)),
+        # weight gradient only: the stride-2 kernel over maps 56, 28 and 16 wide
+        (2, 32, 56, 56, 64, (2, 2), (1, 1)), (3, 64, 12, 56, 128, (2, 2), (1, 1)), (3, 32, 28, 28, 128, (2, 2), (1, 1)),
+        (5, 32, 16, 16, 32, (2, 2), (1, 1)), (3, 64, 16, 16, 64, (2, 2), (1, 1)), (70, 32, 16, 16, 128, (2, 2), (1, 1))],
     np.float64: [
         (256, 3, 32, 32, 32, (1, 1), (1, 1)), (5, 1, 8, 32, 64, (1, 1), (1, 1)), (3, 2, 24, 32, 96, (1, 1), (1, 1)),
         (256, 32, 32, 32, 64, (2, 2), (1, 1)), (3, 32, 32, 32, 64, (2, 2), (1, 1)), (2, 64, 64, 64, 128, (2, 2), (1, 1)), (2, 32, 16, 32, 64, (2, 2), (1, 1)),
-        (1, 96, 64, 64, 64, (2, 2), (1, 1))],
+        (1, 96, 64, 64, 64, (2, 2), (1, 1)),
+        (5, 32, 16, 16, 64, (2, 2), (1, 1)), (70, 64, 16, 16, 128, (2, 2), (1, 1))],
 }
 
 
