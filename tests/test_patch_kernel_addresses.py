@@ -117,10 +117,16 @@ BASELINE_LAYERS = [
 
 
 def test_every_access_of_the_convolution_path_stays_inside_its_buffers(walk_binary):
+    from concurrent.futures import ThreadPoolExecutor
     cases = gpu_test_cases() + BASELINE_LAYERS
-    r = run_walk(walk_binary, cases)
-    assert r.returncode == 0, (r.stdout[-600:], r.stderr[-1500:])
-    assert "walked %d cases" % len(cases) in r.stdout, r.stdout[-300:]
+    # the cases are independent: interleaved shares of the list run as separate processes side by side
+    shares = max(1, min(6, (os.cpu_count() or 2) - 1))
+    parts = [cases[i::shares] for i in range(shares)]
+    with ThreadPoolExecutor(shares) as pool:
+        results = list(pool.map(lambda part: run_walk(walk_binary, part), parts))
+    for part, r in zip(parts, results):
+        assert r.returncode == 0, (r.stdout[-600:], r.stderr[-1500:])
+        assert "walked %d cases" % len(part) in r.stdout, r.stdout[-300:]
 
 
 @pytest.mark.parametrize("which", ["x", "w", "y", "g", "dx", "dw", "act", "ws", "lds"])
