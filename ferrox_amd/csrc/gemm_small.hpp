@@ -357,13 +357,13 @@ __device__ __forceinline__ void small_body_f64(const ParamsD& p, double* red_d, 
 
 template <int AKC, int BKC>
 __global__ __launch_bounds__(NT) void small_kernel_f64(const ParamsD p) {
-    extern __shared__ __align__(16) double red_d[];
+    FX_DYNAMIC_SMEM(double, red_d);
     small_body_f64<AKC, BKC>(p, red_d, blockIdx.x, blockIdx.y, blockIdx.z);
 }
 
 template <int A0>
 __global__ __launch_bounds__(NT) void small_pair_kernel_f64(const ParamsD p0, const ParamsD p1) {  // as small_pair_kernel
-    extern __shared__ __align__(16) double red_d[];
+    FX_DYNAMIC_SMEM(double, red_d);
     const int bx = blockIdx.x, by = blockIdx.y;
     if (blockIdx.z == 0) {
         if (bx * 32 < p0.N && by * 32 < p0.M) small_body_f64<A0, 0>(p0, red_d, bx, by, 0);
@@ -432,12 +432,12 @@ inline int run_f64(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i6
     ParamsD p{A, B, split ? part : C, split ? nullptr : bias, relu, (int)M, (int)N, (int)K, pl.G, pl.kz, split ? M * N : 0, asum, nullptr};
     const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32), (unsigned)pl.splits);
     const size_t lds = (size_t)WAVES * 16 * 64 * sizeof(double);
-    if (!ta && pl.a_elems && !tb) small_kernel_f64<2, 0><<<grid, dim3(NT), lds, c->stream>>>(p);
-    else if (!ta && pl.a_elems) small_kernel_f64<2, 1><<<grid, dim3(NT), lds, c->stream>>>(p);
-    else if (!ta && !tb) small_kernel_f64<1, 0><<<grid, dim3(NT), lds, c->stream>>>(p);
-    else if (!ta && tb) small_kernel_f64<1, 1><<<grid, dim3(NT), lds, c->stream>>>(p);
-    else if (ta && !tb) small_kernel_f64<0, 0><<<grid, dim3(NT), lds, c->stream>>>(p);
-    else small_kernel_f64<0, 1><<<grid, dim3(NT), lds, c->stream>>>(p);
+    if (!ta && pl.a_elems && !tb) FX_LAUNCH(grid, dim3(NT), lds, c->stream, (p), small_kernel_f64<2, 0>);
+    else if (!ta && pl.a_elems) FX_LAUNCH(grid, dim3(NT), lds, c->stream, (p), small_kernel_f64<2, 1>);
+    else if (!ta && !tb) FX_LAUNCH(grid, dim3(NT), lds, c->stream, (p), small_kernel_f64<1, 0>);
+    else if (!ta && tb) FX_LAUNCH(grid, dim3(NT), lds, c->stream, (p), small_kernel_f64<1, 1>);
+    else if (ta && !tb) FX_LAUNCH(grid, dim3(NT), lds, c->stream, (p), small_kernel_f64<0, 0>);
+    else FX_LAUNCH(grid, dim3(NT), lds, c->stream, (p), small_kernel_f64<0, 1>);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
@@ -450,20 +450,20 @@ inline int run(fx_ctx* c, const Plan& pl, bool ta, bool tb, i64 M, i64 N, i64 K,
     if (pl.tile16) {
         FX_REQUIRE(!split && !asum && !pl.a_elems, "small product: 16 x 16 tiles take neither a split K nor row sums");
         const dim3 grid16((unsigned)fx::ceil_div(N, (i64)16), (unsigned)fx::ceil_div(M, (i64)16));
-        if (!ta && !tb) small16_kernel<1, 0><<<grid16, dim3(NT), 0, c->stream>>>(p);
-        else if (!ta && tb) small16_kernel<1, 1><<<grid16, dim3(NT), 0, c->stream>>>(p);
-        else if (ta && !tb) small16_kernel<0, 0><<<grid16, dim3(NT), 0, c->stream>>>(p);
-        else small16_kernel<0, 1><<<grid16, dim3(NT), 0, c->stream>>>(p);
+        if (!ta && !tb) FX_LAUNCH(grid16, dim3(NT), 0, c->stream, (p), small16_kernel<1, 0>);
+        else if (!ta && tb) FX_LAUNCH(grid16, dim3(NT), 0, c->stream, (p), small16_kernel<1, 1>);
+        else if (ta && !tb) FX_LAUNCH(grid16, dim3(NT), 0, c->stream, (p), small16_kernel<0, 0>);
+        else FX_LAUNCH(grid16, dim3(NT), 0, c->stream, (p), small16_kernel<0, 1>);
         FX_LAUNCH_CHECK();
         return FX_OK;
     }
     const dim3 grid((unsigned)fx::ceil_div(N, (i64)32), (unsigned)fx::ceil_div(M, (i64)32), (unsigned)pl.splits);
-    if (!ta && pl.a_elems && !tb) small_kernel<2, 0><<<grid, dim3(NT), 0, c->stream>>>(p);
-    else if (!ta && pl.a_elems) small_kernel<2, 1><<<grid, dim3(NT), 0, c->stream>>>(p);
-    else if (!ta && !tb) small_kernel<1, 0><<<grid, dim3(NT), 0, c->stream>>>(p);
-    else if (!ta && tb) small_kernel<1, 1><<<grid, dim3(NT), 0, c->stream>>>(p);
-    else if (ta && !tb) small_kernel<0, 0><<<grid, dim3(NT), 0, c->stream>>>(p);
-    else small_kernel<0, 1><<<grid, dim3(NT), 0, c->stream>>>(p);
+    if (!ta && pl.a_elems && !tb) FX_LAUNCH(grid, dim3(NT), 0, c->stream, (p), small_kernel<2, 0>);
+    else if (!ta && pl.a_elems) FX_LAUNCH(grid, dim3(NT), 0, c->stream, (p), small_kernel<2, 1>);
+    else if (!ta && !tb) FX_LAUNCH(grid, dim3(NT), 0, c->stream, (p), small_kernel<1, 0>);
+    else if (!ta && tb) FX_LAUNCH(grid, dim3(NT), 0, c->stream, (p), small_kernel<1, 1>);
+    else if (ta && !tb) FX_LAUNCH(grid, dim3(NT), 0, c->stream, (p), small_kernel<0, 0>);
+    else FX_LAUNCH(grid, dim3(NT), 0, c->stream, (p), small_kernel<0, 1>);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
@@ -477,8 +477,8 @@ inline int run_pair(fx_ctx* c, const Plan& p0, const Plan& p1, i64 M0, i64 N0, i
     Params a{A0, B0, C0, nullptr, 0, (int)M0, (int)N0, (int)K0, p0.G, p0.kz, 0, nullptr, mask0};
     Params b{A1, B1, C1, nullptr, 0, (int)M1, (int)N1, (int)K1, p1.G, p1.kz, 0, asum1, nullptr};
     const dim3 grid((unsigned)fx::ceil_div(std::max(N0, N1), (i64)32), (unsigned)fx::ceil_div(std::max(M0, M1), (i64)32), 2);
-    if (p0.a_elems) small_pair_kernel<2><<<grid, dim3(NT), 0, c->stream>>>(a, b);
-    else small_pair_kernel<1><<<grid, dim3(NT), 0, c->stream>>>(a, b);
+    if (p0.a_elems) FX_LAUNCH(grid, dim3(NT), 0, c->stream, (a, b), small_pair_kernel<2>);
+    else FX_LAUNCH(grid, dim3(NT), 0, c->stream, (a, b), small_pair_kernel<1>);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }
@@ -489,8 +489,8 @@ inline int run_pair(fx_ctx* c, const Plan& p0, const Plan& p1, i64 M0, i64 N0, i
     ParamsD b{A1, B1, C1, nullptr, 0, (int)M1, (int)N1, (int)K1, p1.G, p1.kz, 0, asum1, nullptr};
     const dim3 grid((unsigned)fx::ceil_div(std::max(N0, N1), (i64)32), (unsigned)fx::ceil_div(std::max(M0, M1), (i64)32), 2);
     const size_t lds = (size_t)WAVES * 16 * 64 * sizeof(double);
-    if (p0.a_elems) small_pair_kernel_f64<2><<<grid, dim3(NT), lds, c->stream>>>(a, b);
-    else small_pair_kernel_f64<1><<<grid, dim3(NT), lds, c->stream>>>(a, b);
+    if (p0.a_elems) FX_LAUNCH(grid, dim3(NT), lds, c->stream, (a, b), small_pair_kernel_f64<2>);
+    else FX_LAUNCH(grid, dim3(NT), lds, c->stream, (a, b), small_pair_kernel_f64<1>);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

@@ -32,7 +32,7 @@ struct Params {
 };
 
 __global__ __launch_bounds__(NT) void thin_tn_kernel(const Params p) {
-    extern __shared__ __align__(16) float smem[];
+    FX_DYNAMIC_SMEM(float, smem);
     float* red = smem;                          // [3 quarters][2 column slabs][16][64]
     float* As = smem + (KQ - 1) * 2 * 16 * 64;  // [as_rows][32]: A[k][m], zero for m >= M and k >= K
     const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
@@ -146,7 +146,7 @@ inline int run(fx_ctx* c, i64 M, i64 N, i64 K, const float* A, const float* B, f
     Params p{A, B, C, bias, relu, (int)M, (int)N, (int)K, as_rows(K), asum};
     static const hipError_t attr = hipFuncSetAttribute((const void*)thin_tn_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT);
     FX_HIP_CHECK(attr);
-    thin_tn_kernel<<<dim3((unsigned)fx::ceil_div(N, (i64)BN)), dim3(NT), lds_bytes(K), c->stream>>>(p);
+    FX_LAUNCH(dim3((unsigned)fx::ceil_div(N, (i64)BN)), dim3(NT), lds_bytes(K), c->stream, (p), thin_tn_kernel);
     FX_LAUNCH_CHECK();
     return FX_OK;
 }

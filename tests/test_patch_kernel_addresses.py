@@ -1,4 +1,6 @@
-"""Bounds check of the convolution path on the CPU (no GPU): the library's own conv.hip -- dispatch, planners and every
+"""Bounds check of the convolution and matrix-product paths on the CPU (no GPU): the library's own conv.hip and gemm.hip --
+dispatch, planners and every kernel they launch -- are compiled as host C++ (second half of this file: the products).
+The convolution path: conv.hip -- dispatch, planners and every
 patch / image-layer / stride-2 / implicit-GEMM kernel it launches -- is compiled as host C++ against a stand-in HIP header
 (tests/kernel_walk/) and every thread of every block of every launch is run on the CPU with each tensor, the workspace and the
 dynamic LDS between inaccessible pages.  What runs is the kernels' own address arithmetic, not a restatement of it: an
@@ -20,24 +22,24 @@ CLANG = os.environ.get("FX_WALK_CXX", "/opt/rocm/lib/llvm/bin/clang++")
 
 
 def _sources():
-    files = [os.path.join(WALK_DIR, "walk.cpp"), os.path.join(WALK_DIR, "hip", "hip_runtime.h"), os.path.join(ROOT, "include", "ferrox_hip.h")]
-    files += sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp") or f == "conv.hip")  # gemm_lds.hpp included
+    files = [os.path.join(WALK_DIR, "walk.cpp"), os.path.join(WALK_DIR, "walk_gemm.cpp"), os.path.join(WALK_DIR, "hip", "hip_runtime.h"),
+             os.path.join(ROOT, "include", "ferrox_hip.h")]
+    files += sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp") or f in ("conv.hip", "gemm.hip"))
     return files
 
 
-@pytest.fixture(scope="module")
-def walk_binary():
-    """Builds tests/kernel_walk/build/walk (kept until a source it includes changes)."""
+def _build_walk(name):
+    """Builds tests/kernel_walk/build/<name> from tests/kernel_walk/<name>.cpp (kept until a source it includes changes)."""
     if not os.path.exists(CLANG):
         pytest.skip("no clang++ to build the host emulation with")
     out_dir = os.path.join(WALK_DIR, "build")
     os.makedirs(out_dir, exist_ok=True)
-    exe, stamp = os.path.join(out_dir, "walk"), os.path.join(out_dir, "walk.sha1")
+    exe, stamp = os.path.join(out_dir, name), os.path.join(out_dir, name + ".sha1")
     # the index arithmetic also runs under the integer checks of the undefined-behaviour sanitizer (overflow, shifts,
     # static array bounds: the statically sized LDS arrays), any finding ends the walk
     cmd = [CLANG, "-x", "c++", "-std=c++17", "-O1", "-g", "-I", WALK_DIR, "-DFX_HOST_EMULATION=1", "-Wno-unknown-attributes",
            "-Wno-unused-value", "-Wno-psabi", "-fsanitize=signed-integer-overflow,shift,bounds,integer-divide-by-zero",
-           "-fno-sanitize-recover=all", "-o", exe, os.path.join(WALK_DIR, "walk.cpp")]
+           "-fno-sanitize-recover=all", "-o", exe, os.path.join(WALK_DIR, name + ".cpp")]
     h = hashlib.sha1(" ".join(cmd).encode())
     for f in _sources():
         h.update(open(f, "rb").read())
@@ -46,6 +48,16 @@ def walk_binary():
         assert r.returncode == 0, r.stderr[-4000:]
         open(stamp, "w").write(h.hexdigest())
     return exe
+
+
+@pytest.fixture(scope="module")
+def walk_binary():
+    return _build_walk("walk")
+
+
+@pytest.fixture(scope="module")
+def gemm_walk_binary():
+    return _build_walk("walk_gemm")
 
 
 def run_walk(exe, cases, env=None, timeout=900):
@@ -149,3 +161,40 @@ def test_the_walk_faults_when_a_buffer_is_16_bytes_short(walk_binary, which):
         assert faulted or which == "ws", (which, case, "did not fault")
         faults += faulted
     assert faults >= 1, which
+
+
+# ------------------------------------------------------------------------------------------ matrix products
+def gemm_cases():
+    """(name, dtype, (M, N, K)) for every product shape of the GPU tests, both types, plus the products of the baseline
+    configurations; walk_gemm runs all four transpose forms with and without the bias epilogue on each."""
+    import test_gpu_kernels as tk
+    shapes = list(tk.GEMM_SHAPES) + list(tk.GEMM_LDS_SHAPES) + list(tk.GEMM_SMALL_SHAPES) + [(M, N, K) for (_, M, N, K) in tk.GEMM_THIN_SHAPES]
+    # classifier head of the CNN step and its gradients, the MLP layers, the reference's benchmark product, a product of full tiles
+    shapes += [(256, 10, 16384), (256, 16384, 10), (10, 16384, 256), (256, 256, 784), (256, 128, 256), (256, 10, 128), (784, 256, 256),
+               (1024, 1024, 1024), (2048, 2048, 512)]
+    cases = []
+    for (M, N, K) in shapes:
+        for dt in ("f32", "f64"):
+            cases.append(("gemm_%d" % len(cases), dt, (M, N, K)))
+    return cases
+
+
+def test_every_access_of_the_matrix_product_path_stays_inside_its_buffers(gemm_walk_binary):
+    from concurrent.futures import ThreadPoolExecutor
+    cases = gemm_cases()
+    shares = max(1, min(6, (os.cpu_count() or 2) - 1))
+    parts = [cases[i::shares] for i in range(shares)]
+    with ThreadPoolExecutor(shares) as pool:
+        results = list(pool.map(lambda part: run_walk(gemm_walk_binary, part), parts))
+    for part, r in zip(parts, results):
+        assert r.returncode == 0, (r.stdout[-600:], r.stderr[-1500:])
+        assert "walked %d cases" % len(part) in r.stdout, r.stdout[-300:]
+
+
+@pytest.mark.parametrize("which", ["a", "b", "c"])
+def test_the_product_walk_faults_when_a_matrix_is_16_bytes_short(gemm_walk_binary, which):
+    """The detector's own test, as for the convolution walk: with A, B or C 16 bytes shorter than its shape the walk must end in a
+    fault that names the case, on the slab kernel, the small-product kernel and the general tiles alike."""
+    for case in [("slab", "f32", (2560, 2560, 128)), ("small", "f32", (33, 65, 36)), ("general", "f64", (130, 257, 75))]:
+        r = run_walk(gemm_walk_binary, [case], env={"FX_WALK_SHRINK": which})
+        assert r.returncode == 3 and "FAULT" in r.stderr and case[0] in r.stderr, (which, case, r.returncode, r.stderr[-500:])
