@@ -51,13 +51,24 @@ def _build_walk(name):
 
 
 @pytest.fixture(scope="module")
-def walk_binary():
-    return _build_walk("walk")
+def walk_binaries():
+    """Both harnesses, compiled side by side."""
+    if not os.path.exists(CLANG):
+        pytest.skip("no clang++ to build the host emulation with")
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(2) as pool:
+        conv, gemm = pool.map(_build_walk, ("walk", "walk_gemm"))
+    return {"walk": conv, "walk_gemm": gemm}
 
 
 @pytest.fixture(scope="module")
-def gemm_walk_binary():
-    return _build_walk("walk_gemm")
+def walk_binary(walk_binaries):
+    return walk_binaries["walk"]
+
+
+@pytest.fixture(scope="module")
+def gemm_walk_binary(walk_binaries):
+    return walk_binaries["walk_gemm"]
 
 
 def run_walk(exe, cases, env=None, timeout=900):
